@@ -1,0 +1,139 @@
+/*
+ * phx_qconv.h -- C ABI of the MI355X (gfx950) quaternion Conv2D / Dense engine.
+ *
+ * Plain C: pointers, sizes and POD structs only.  Every entry point enqueues work on the given
+ * HIP stream and returns without synchronising; tensors live in device memory owned by the caller.
+ * A non-zero return value is an error (see phx_status_string); nothing has been enqueued then.
+ *
+ * Tensor layout (identical to the reference engine's, src/backend/tensor.hpp:527-535 and
+ * src/conv2d.hpp:169): activations are NCHW with the four quaternion components stacked on the
+ * batch axis, x[4*n, ci, h, w] with component p in rows [p*n, (p+1)*n); filters carry the
+ * component outermost, w[4, co, ci, kh, kw] (OIHW) or w[4, co, kh, kw, ci] (OHWI); bias is
+ * [4, co].  Dense: x[4*n, ni], w[4, ni, no] (layout IO), bias[4, no].
+ *
+ * Product convention: y = x (x) w, input on the left (src/algebras.cc:28-49).
+ */
+#ifndef PHX_QCONV_H
+#define PHX_QCONV_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* phx_stream_t; /* a hipStream_t; NULL is the default stream */
+
+enum phx_status {
+    PHX_OK = 0,
+    PHX_ERR_INVALID_ARGUMENT = 1, /* malformed descriptor or null pointer */
+    PHX_ERR_NOT_SUPPORTED = 2,    /* valid request outside what the kernels cover */
+    PHX_ERR_WORKSPACE = 3,        /* workspace smaller than phx_*_workspace_bytes() */
+    PHX_ERR_RUNTIME = 4           /* HIP runtime reported an error */
+};
+
+enum phx_dtype { PHX_F32 = 0, PHX_F16 = 1 };
+
+enum phx_filter_layout { PHX_OIHW = 0, PHX_OHWI = 1 };
+
+/* Which Hamilton-product formulation runs.
+ * Mirrors Context::preferSpeedToMemory() (src/backend/backend.hpp:58): the reference's default is
+ * the factorized 8-product path (src/conv2d.hpp:167-234), UPSTRIDE_MEMORY_OPTIMIZED=1 selects the
+ * 16-product path (src/conv2d.hpp:237-275). */
+enum phx_product_mode { PHX_PRODUCT_16 = 16, PHX_PRODUCT_8 = 8 };
+
+/* UPSTRIDE_CONV_FP16_POLICY (src/backend/backend.cc:35-42, src/backend/backend.hpp:60-66).
+ * Applies to PHX_F16 tensors only; accumulation is fp32 under every policy.
+ *   FULL32      fp32 MFMA in every pass (operands widened while staged)
+ *   BACKWARD32  fp16 MFMA forward, fp32 MFMA backward
+ *   FULL16      fp16 MFMA in every pass */
+enum phx_fp16_policy { PHX_FP16_FULL32 = 0, PHX_FP16_BACKWARD32 = 1, PHX_FP16_FULL16 = 2 };
+
+enum phx_pass { PHX_PASS_FWD = 0, PHX_PASS_BWD_DATA = 1, PHX_PASS_BWD_WEIGHTS = 2 };
+
+/* Quaternion Conv2D geometry; replaces the per-call arguments the reference passes to
+ * UpstrideConv2DFunctor / UpstrideConv2DGradFunctor (src/conv2d.hpp:40-58, 72-79, 297-316,
+ * 331-339) after Conv2DDescriptor has resolved the padding (src/backend/conv2d_descriptor.hpp:132-174). */
+typedef struct phx_qconv_desc {
+    int32_t dtype;         /* phx_dtype of every tensor of the call */
+    int32_t n;             /* images; activation tensors have 4*n batch rows */
+    int32_t ci, co;        /* quaternion channels in / out */
+    int32_t h, w;          /* input spatial size */
+    int32_t kh, kw;        /* filter size */
+    int32_t stride_h, stride_w;
+    int32_t dilation_h, dilation_w;
+    int32_t pad_top, pad_left, pad_bottom, pad_right;
+    int32_t filter_layout; /* phx_filter_layout */
+    int32_t product_mode;  /* phx_product_mode */
+    int32_t fp16_policy;   /* phx_fp16_policy */
+    int32_t has_bias;      /* forward only: bias pointer must be non-null when set */
+} phx_qconv_desc;
+
+/* Quaternion Dense geometry (src/backend/dense_descriptor.hpp:11-59); filter layout is IO. */
+typedef struct phx_qdense_desc {
+    int32_t dtype;
+    int32_t n;             /* batch; activation tensors have 4*n rows */
+    int32_t ni, no;        /* quaternion features in / out */
+    int32_t product_mode;
+    int32_t fp16_policy;
+    int32_t has_bias;
+} phx_qdense_desc;
+
+const char* phx_status_string(int status);
+
+/* Output spatial size for the descriptor's explicit padding (src/utils.cc:42-51). */
+int phx_qconv2d_output_hw(const phx_qconv_desc* desc, int32_t* ho, int32_t* wo);
+
+/* Scratch bytes one call of the given pass needs (packed filters, split-K partial sums). */
+size_t phx_qconv2d_workspace_bytes(const phx_qconv_desc* desc, int pass);
+size_t phx_qdense_workspace_bytes(const phx_qdense_desc* desc, int pass);
+
+/* y = x (x) w (+ bias).  Replaces UpstrideConv2DFunctor<Device,T>::operator() for the quaternion
+ * algebra (src/conv2d.hpp:72-95, 167-275) and the forward custom-kernel hook
+ * QuatKernelPointwiseConvForwardFunctor::operator() (src/backend/backend.hpp:163-185). */
+int phx_qconv2d_fwd(const phx_qconv_desc* desc, phx_stream_t stream, const void* x, const void* w,
+                    const void* bias_or_null, void* y, void* workspace, size_t workspace_bytes);
+
+/* dx = g (x) conj(w), spatially transposed.  Replaces the input-gradient half of
+ * UpstrideConv2DGradFunctor<Device,T>::operator() (src/conv2d.hpp:331-357, 433-562) and of
+ * QuatKernelPointwiseConvBackwardFunctor::operator() (src/backend/backend.hpp:196-220). */
+int phx_qconv2d_bwd_data(const phx_qconv_desc* desc, phx_stream_t stream, const void* grad, const void* w,
+                         void* dx, void* workspace, size_t workspace_bytes);
+
+/* dw = conj(x) (x) g, reduced over batch and space.  Replaces the filter-gradient half of the
+ * same two reference operators. */
+int phx_qconv2d_bwd_weights(const phx_qconv_desc* desc, phx_stream_t stream, const void* x, const void* grad,
+                            void* dw, void* workspace, size_t workspace_bytes);
+
+/* Dense trio.  Replaces UpstrideDenseFunctor / UpstrideDenseGradFunctor for the quaternion
+ * algebra (src/dense.hpp:52-62, 77-180, 223-237, 252-377). */
+int phx_qdense_fwd(const phx_qdense_desc* desc, phx_stream_t stream, const void* x, const void* w,
+                   const void* bias_or_null, void* y, void* workspace, size_t workspace_bytes);
+int phx_qdense_bwd_data(const phx_qdense_desc* desc, phx_stream_t stream, const void* grad, const void* w,
+                        void* dx, void* workspace, size_t workspace_bytes);
+int phx_qdense_bwd_weights(const phx_qdense_desc* desc, phx_stream_t stream, const void* x, const void* grad,
+                           void* dw, void* workspace, size_t workspace_bytes);
+
+/* Device plumbing for hosts that do not link the HIP runtime themselves.  Replaces what
+ * device::CUDA does for the reference (src/backend/cudnn/device.hpp:13-229: malloc/free on the
+ * device, the stream the operations are enqueued on) and the host<->device copies of
+ * TensorManipulations<device::CUDA> (src/backend/cudnn/tensor.hpp:19-111). */
+int phx_device_count(int32_t* count);
+int phx_device_malloc(void** ptr, size_t bytes);
+int phx_device_free(void* ptr);
+int phx_memcpy_h2d(void* dst, const void* src, size_t bytes, phx_stream_t stream);
+int phx_memcpy_d2h(void* dst, const void* src, size_t bytes, phx_stream_t stream);
+int phx_memset_zero(void* dst, size_t bytes, phx_stream_t stream);
+int phx_stream_create(phx_stream_t* stream);
+int phx_stream_destroy(phx_stream_t stream);
+int phx_stream_synchronize(phx_stream_t stream);
+
+/* Name of the kernel variant the last successful call on this thread dispatched to (for
+ * profiling and tests); a static string. */
+const char* phx_last_kernel_name(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,7 @@
+"""phoenix_core_amd -- MI355X (gfx950) quaternion Conv2D / Dense engine.
+
+The arithmetic lives in hand-written HIP kernels (csrc/) behind a C ABI (include/phx_qconv.h);
+`ops` is the Python host mirror of the reference's operator interface for this path."""
+from . import capi  # noqa: F401
+from .ops import (Context, Conv2DDescriptor, DenseDescriptor, conv2d_bwd, conv2d_fwd, default_context,  # noqa: F401
+                  dense_bwd, dense_fwd, windowed_output_size_and_padding)

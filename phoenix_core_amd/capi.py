@@ -1,0 +1,94 @@
+"""ctypes binding of the engine's C ABI (include/phx_qconv.h).
+
+Loads phoenix_core_amd/lib/libphx_qconv.so and fails loudly when it is missing: there is no
+fallback path, CPU or otherwise."""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libphx_qconv.so")
+
+PHX_OK = 0
+PHX_F32, PHX_F16 = 0, 1
+PHX_OIHW, PHX_OHWI = 0, 1
+PHX_PRODUCT_16, PHX_PRODUCT_8 = 16, 8
+PHX_FP16_FULL32, PHX_FP16_BACKWARD32, PHX_FP16_FULL16 = 0, 1, 2
+PHX_PASS_FWD, PHX_PASS_BWD_DATA, PHX_PASS_BWD_WEIGHTS = 0, 1, 2
+
+# every symbol include/phx_qconv.h declares
+EXPORTS = (
+    "phx_status_string", "phx_qconv2d_output_hw", "phx_qconv2d_workspace_bytes", "phx_qdense_workspace_bytes",
+    "phx_qconv2d_fwd", "phx_qconv2d_bwd_data", "phx_qconv2d_bwd_weights",
+    "phx_qdense_fwd", "phx_qdense_bwd_data", "phx_qdense_bwd_weights",
+    "phx_device_count", "phx_device_malloc", "phx_device_free", "phx_memcpy_h2d", "phx_memcpy_d2h",
+    "phx_memset_zero", "phx_stream_create", "phx_stream_destroy", "phx_stream_synchronize",
+    "phx_last_kernel_name",
+)
+
+
+class QConvDesc(ctypes.Structure):
+    _fields_ = [(k, ctypes.c_int32) for k in (
+        "dtype", "n", "ci", "co", "h", "w", "kh", "kw", "stride_h", "stride_w", "dilation_h", "dilation_w",
+        "pad_top", "pad_left", "pad_bottom", "pad_right", "filter_layout", "product_mode", "fp16_policy", "has_bias")]
+
+
+class QDenseDesc(ctypes.Structure):
+    _fields_ = [(k, ctypes.c_int32) for k in ("dtype", "n", "ni", "no", "product_mode", "fp16_policy", "has_bias")]
+
+
+class PhxError(RuntimeError):
+    def __init__(self, status, what):
+        self.status = status
+        super().__init__("%s: %s" % (what, status_string(status)))
+
+
+_lib = None
+
+
+def lib():
+    """The loaded shared library; raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.isfile(LIB_PATH):
+            raise ImportError("%s is missing: build it with `python -m phoenix_core_amd.build`" % LIB_PATH)
+        L = ctypes.CDLL(LIB_PATH)
+        vp, sz, i32p = ctypes.c_void_p, ctypes.c_size_t, ctypes.POINTER(ctypes.c_int32)
+        cd, dd = ctypes.POINTER(QConvDesc), ctypes.POINTER(QDenseDesc)
+        L.phx_status_string.restype = ctypes.c_char_p
+        L.phx_status_string.argtypes = [ctypes.c_int]
+        L.phx_last_kernel_name.restype = ctypes.c_char_p
+        L.phx_qconv2d_output_hw.argtypes = [cd, i32p, i32p]
+        L.phx_qconv2d_workspace_bytes.restype = sz
+        L.phx_qconv2d_workspace_bytes.argtypes = [cd, ctypes.c_int]
+        L.phx_qdense_workspace_bytes.restype = sz
+        L.phx_qdense_workspace_bytes.argtypes = [dd, ctypes.c_int]
+        L.phx_qconv2d_fwd.argtypes = [cd, vp, vp, vp, vp, vp, vp, sz]
+        L.phx_qconv2d_bwd_data.argtypes = [cd, vp, vp, vp, vp, vp, sz]
+        L.phx_qconv2d_bwd_weights.argtypes = [cd, vp, vp, vp, vp, vp, sz]
+        L.phx_qdense_fwd.argtypes = [dd, vp, vp, vp, vp, vp, vp, sz]
+        L.phx_qdense_bwd_data.argtypes = [dd, vp, vp, vp, vp, vp, sz]
+        L.phx_qdense_bwd_weights.argtypes = [dd, vp, vp, vp, vp, vp, sz]
+        L.phx_device_count.argtypes = [i32p]
+        L.phx_device_malloc.argtypes = [ctypes.POINTER(vp), sz]
+        L.phx_device_free.argtypes = [vp]
+        L.phx_memcpy_h2d.argtypes = [vp, vp, sz, vp]
+        L.phx_memcpy_d2h.argtypes = [vp, vp, sz, vp]
+        L.phx_memset_zero.argtypes = [vp, sz, vp]
+        L.phx_stream_create.argtypes = [ctypes.POINTER(vp)]
+        L.phx_stream_destroy.argtypes = [vp]
+        L.phx_stream_synchronize.argtypes = [vp]
+        _lib = L
+    return _lib
+
+
+def status_string(status):
+    return lib().phx_status_string(int(status)).decode()
+
+
+def last_kernel_name():
+    return lib().phx_last_kernel_name().decode()
+
+
+def check(status, what):
+    if status != PHX_OK:
+        raise PhxError(status, what)

@@ -1,0 +1,396 @@
+// fp32-MFMA kernels (v_mfma_f32_32x32x2_f32): quaternion convolution forward / input-gradient
+// (one kernel, two lane maps) and filter-gradient, in the 16-product and the factorized 8-product
+// formulation.  Storage type TS is float or _Float16 (operands widened while staged into LDS).
+#pragma once
+
+#include "phx_device.h"
+
+namespace phx {
+
+enum { MAP_FWD = 0, MAP_DGRAD = 1 };
+
+constexpr int F32_CK = 8;  // input channels staged per K chunk (4 MFMA k-pairs)
+
+struct ConvArgs {
+    TileSrc in;         // x (forward) or the output gradient (input-gradient pass)
+    const float* wpk;   // packed filters, see pack_filters_f32
+    const void* bias;   // [4][Cout] in storage type or null
+    void* out;
+    long out_cs;        // elements between output components
+    int Cout, Hout, Wout;
+    int taps, Kw;       // filter taps (Kh*Kw) and filter width
+    int dh, dw, sh, sw; // dilation and stride of the correlation
+    int pt, pl;         // virtual input row of output row 0, tap 0, is -pt (same for columns)
+    int NB, TH, TW;     // output pixels per workgroup tile: images x rows x columns
+    int HTH, HTW, HPp;  // halo window and LDS pitch per staged channel
+    int lpr_log2;       // lanes per staged row (log2)
+    int tiles_n, tiles_h, tiles_w, co_tiles;
+    int nchunks;        // ceil(Cin / F32_CK)
+};
+
+// Forward / input-gradient kernel.
+//   workgroup = 4 waves = WCO filter sub-tiles (32 output channels each) x 4/WCO pixel ranges,
+//   each wave owns NTW MFMA column tiles of 32 output pixels and all four output components.
+//   A operand = packed filters straight from global memory (L2 resident, one 16/32-byte load per
+//   lane and K step, prefetched one step ahead); B operand = activations from the LDS halo window.
+//   MODE 16: acc[q] += W_{p^q} * (+-x_p), 16 MFMAs per K step, filters reused across the 4x4 block.
+//   MODE 8 : acc[i] += R_i * L_i with the 8 lanes L_i formed in registers, 8 MFMAs per K step.
+template <typename TS, int MODE, int MAP, int WCO, int NTW>
+__global__ void __launch_bounds__(WG_THREADS) qconv_fwd_f32_kernel(const ConvArgs P) {
+    constexpr int CK = F32_CK;
+    constexpr int WPX = 4 / WCO;
+    constexpr int NACC = (MODE == 16) ? 4 : 8;
+    constexpr int WC = (MODE == 16) ? 4 : 8;  // packed filter values per lane and K step
+    extern __shared__ float lds[];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wco = wave % WCO, wpx = wave / WCO;
+    const int j = lane & 31, kk = lane >> 5;
+
+    int bid = xcd_remap(blockIdx.x, gridDim.x);
+    const int ct = bid % P.co_tiles;
+    bid /= P.co_tiles;
+    const int tw = bid % P.tiles_w;
+    bid /= P.tiles_w;
+    const int th = bid % P.tiles_h;
+    const int tn = bid / P.tiles_h;
+    const int n0 = tn * P.NB, ho0 = th * P.TH, wo0 = tw * P.TW;
+    const int h0 = ho0 * P.sh - P.pt, w0 = wo0 * P.sw - P.pl;
+
+    int poff[NTW];
+    long oaddr[NTW];
+    bool pvalid[NTW];
+    const int thw = P.TH * P.TW;
+#pragma unroll
+    for (int t = 0; t < NTW; ++t) {
+        const int pix = (wpx * NTW + t) * 32 + j;
+        const int nb = pix / thw, rem = pix - nb * thw;
+        const int r = rem / P.TW, c = rem - r * P.TW;
+        pvalid[t] = nb < P.NB && (n0 + nb) < P.in.N && (ho0 + r) < P.Hout && (wo0 + c) < P.Wout;
+        poff[t] = pvalid[t] ? (nb * P.HTH + r * P.sh) * P.HTW + c * P.sw : 0;
+        oaddr[t] = ((long)(n0 + nb) * P.Cout * P.Hout + (ho0 + r)) * P.Wout + (wo0 + c);
+    }
+
+    f32x16 acc[NTW][NACC];
+#pragma unroll
+    for (int t = 0; t < NTW; ++t)
+#pragma unroll
+        for (int a = 0; a < NACC; ++a)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[t][a][r] = 0.f;
+
+    const int steps_per_chunk = P.taps * (CK / 2);
+    const long nsteps = (long)P.nchunks * steps_per_chunk;
+    const float* wptr = P.wpk + ((long)(ct * WCO + wco) * nsteps * 64 + lane) * WC;
+    f32x4 wcur[WC / 4], wnext[WC / 4];
+#pragma unroll
+    for (int v = 0; v < WC / 4; ++v) wcur[v] = *reinterpret_cast<const f32x4*>(wptr + 4 * v);
+
+    long step = 0;
+    const long cpitch = (long)CK * P.HPp;  // LDS floats between components
+    for (int chunk = 0; chunk < P.nchunks; ++chunk) {
+        __syncthreads();
+        stage_window<TS, CK, float>(lds, P.in, n0, chunk * CK, h0, w0, P.NB, P.HTH, P.HTW, P.HPp, P.lpr_log2);
+        __syncthreads();
+        int kh = 0, kw = 0;
+        for (int tap = 0; tap < P.taps; ++tap) {
+            const int tapoff = kh * P.dh * P.HTW + kw * P.dw;
+#pragma unroll
+            for (int cp = 0; cp < CK / 2; ++cp) {
+                const long nxt = (step + 1 < nsteps) ? step + 1 : step;
+#pragma unroll
+                for (int v = 0; v < WC / 4; ++v)
+                    wnext[v] = *reinterpret_cast<const f32x4*>(wptr + nxt * (64 * WC) + 4 * v);
+                const float* xb = lds + (2 * cp + kk) * P.HPp + tapoff;
+#pragma unroll
+                for (int t = 0; t < NTW; ++t) {
+                    float x[4];
+#pragma unroll
+                    for (int p = 0; p < 4; ++p) x[p] = xb[p * cpitch + poff[t]];
+                    if constexpr (MODE == 16) {
+                        float nx[4];
+#pragma unroll
+                        for (int p = 0; p < 4; ++p) nx[p] = -x[p];
+#pragma unroll
+                        for (int p = 0; p < 4; ++p)
+#pragma unroll
+                            for (int q = 0; q < 4; ++q)
+                                acc[t][q] = __builtin_amdgcn_mfma_f32_32x32x2f32(wcur[0][p ^ q], qneg(p, q) ? nx[p] : x[p],
+                                                                                 acc[t][q], 0, 0, 0);
+                    } else {
+                        float L[8];
+                        if constexpr (MAP == MAP_FWD) lanes_left(x, L);
+                        else lanes_grad(x, L, 0.5f);
+#pragma unroll
+                        for (int i = 0; i < 8; ++i)
+                            acc[t][i] = __builtin_amdgcn_mfma_f32_32x32x2f32(wcur[i >> 2][i & 3], L[i], acc[t][i], 0, 0, 0);
+                    }
+                }
+#pragma unroll
+                for (int v = 0; v < WC / 4; ++v) wcur[v] = wnext[v];
+                ++step;
+            }
+            if (++kw == P.Kw) { kw = 0; ++kh; }
+        }
+    }
+
+    // epilogue: fold lanes (8-product), add bias, store NCHW with components on the batch axis
+    TS* out = static_cast<TS*>(P.out);
+    const TS* bias = static_cast<const TS*>(P.bias);
+    const long plane = (long)P.Hout * P.Wout;
+    const int co_base = (ct * WCO + wco) * 32 + 4 * kk;
+#pragma unroll
+    for (int t = 0; t < NTW; ++t) {
+        f32x16 y[4];
+        if constexpr (MODE == 16) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) y[q] = acc[t][q];
+        } else if constexpr (MAP == MAP_FWD) {
+            merge_output(acc[t], y);
+        } else {
+            merge_left_grad(acc[t], y);
+        }
+        if (!pvalid[t]) continue;
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int co = co_base + 8 * (r >> 2) + (r & 3);
+                if (co < P.Cout) {
+                    float v = y[q][r];
+                    if (bias) v += ldf<TS>(bias + q * P.Cout + co);
+                    stf<TS>(out + q * P.out_cs + oaddr[t] + co * plane, v);
+                }
+            }
+    }
+}
+
+// Filter packing for the kernel above.  One value group per (32-channel filter tile, K step, lane):
+//   lane = (row = lane % 32, kk = lane / 32), output channel = tile*32 + row,
+//   K step = ((chunk * taps) + tap) * 4 + cp, input channel = chunk*8 + 2*cp + kk.
+//   MODE 16: the four filter components; MODE 8: the eight right-operand lanes R_i.
+//   MAP_DGRAD swaps the channel roles, mirrors the taps and (MODE 16) conjugates the filter, so
+//   that dx = g (x) conj(w) runs through the forward kernel.
+// Filter element (r, o, i, kh, kw) lives at r*wcs + o*so + i*si + kh*skh + kw*skw.
+struct PackArgs {
+    const void* w;
+    float* out;
+    long wcs, so, si, skh, skw;
+    int Co, Ci;       // filter dims of the convolution (not of the correlation being run)
+    int Kh, Kw;
+    int rows, red;    // correlation: output channels (rows) and reduced channels
+    int row_tiles, nchunks;
+};
+
+template <typename TS, int MODE, int MAP>
+__global__ void __launch_bounds__(WG_THREADS) pack_filters_f32_kernel(const PackArgs P) {
+    constexpr int WC = (MODE == 16) ? 4 : 8;
+    const int taps = P.Kh * P.Kw;
+    const long total = (long)P.row_tiles * P.nchunks * taps * 4 * 64;
+    const TS* w = static_cast<const TS*>(P.w);
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
+        const int lane = idx & 63;
+        long s = idx >> 6;
+        const int cp = s & 3;
+        s >>= 2;
+        const int tap = s % taps;
+        s /= taps;
+        const int chunk = s % P.nchunks;
+        const int tile = s / P.nchunks;
+        const int row = tile * 32 + (lane & 31);
+        const int red = chunk * F32_CK + 2 * cp + (lane >> 5);
+        int kh = tap / P.Kw, kw = tap - kh * P.Kw;
+        float wv[4] = {0.f, 0.f, 0.f, 0.f};
+        if (row < P.rows && red < P.red) {
+            int o = row, i = red;
+            if (MAP == MAP_DGRAD) {
+                o = red;
+                i = row;
+                kh = P.Kh - 1 - kh;
+                kw = P.Kw - 1 - kw;
+            }
+            const long off = o * P.so + i * P.si + kh * P.skh + kw * P.skw;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) wv[r] = ldf<TS>(w + r * P.wcs + off);
+        }
+        float* dst = P.out + idx * WC;
+        if constexpr (MODE == 16) {
+            const float sgn = (MAP == MAP_DGRAD) ? -1.f : 1.f;
+            dst[0] = wv[0];
+            dst[1] = sgn * wv[1];
+            dst[2] = sgn * wv[2];
+            dst[3] = sgn * wv[3];
+        } else {
+            float R[8];
+            lanes_right(wv, R);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) dst[i] = R[i];
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Filter gradient.  GEMM view: rows = output channels (A operand = output gradient), columns =
+// input channels (B operand = shifted input), reduction over batch and output pixels.
+//   grid.x = (64-channel row tile, 64-channel column tile), grid.y = tap group (one filter row kh
+//   and up to TPW adjacent kw), grid.z = split of the reduction; each workgroup walks its share of
+//   the pixel tiles, stages gradient and input windows in LDS and accumulates in registers.
+//   wave = (32 rows) x (32 columns) x TPW taps x 4 components (MODE 16) or 8 lanes (MODE 8).
+//   Partial sums go to workspace[z] and are summed in a fixed order by reduce_wgrad_kernel.
+// ---------------------------------------------------------------------------------------------
+struct WgradArgs {
+    TileSrc x, g;
+    float* partial;     // [Z][taps][4][CoP][CiP]
+    int Kh, Kw, sh, sw, dh, dw, pt, pl;
+    int NB, TH, TW;     // reduction tile: images x output rows x output columns
+    int KP, KPp, HPp;   // pixels per tile (even), LDS pitches (odd) of gradient / input windows
+    int HTH, HTWmax;
+    int lpr_g, lpr_x;   // log2 lanes per staged row
+    int tiles_n, tiles_h, tiles_w;
+    int co_tiles, ci_tiles, CoP, CiP;
+    int groups_per_row; // tap groups per filter row
+};
+
+template <typename TS, int MODE, int TPW>
+__global__ void __launch_bounds__(WG_THREADS) qconv_wgrad_f32_kernel(const WgradArgs P) {
+    constexpr int CT = 64;
+    constexpr int NACC = (MODE == 16) ? 4 : 8;
+    extern __shared__ float lds[];
+    float* gl = lds;                           // [4][CT][KPp]
+    float* xl = lds + 4 * CT * P.KPp;          // [4][CT][HPp]
+    int* poff = reinterpret_cast<int*>(xl + 4 * CT * P.HPp);  // [KP]
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wco = wave & 1, wci = wave >> 1;
+    const int m = lane & 31, kk = lane >> 5;
+    const int cot = blockIdx.x % P.co_tiles, cit = blockIdx.x / P.co_tiles;
+    const int kh = blockIdx.y / P.groups_per_row;
+    const int kw0 = (blockIdx.y % P.groups_per_row) * TPW;
+    const int nkw = (P.Kw - kw0 < TPW) ? P.Kw - kw0 : TPW;
+    const int HTW = (P.TW - 1) * P.sw + (nkw - 1) * P.dw + 1;
+
+    const int thw = P.TH * P.TW;
+    for (int k = tid; k < P.KP; k += WG_THREADS) {
+        const int nb = k / thw, rem = k - nb * thw;
+        const int r = rem / P.TW, c = rem - r * P.TW;
+        poff[k] = (nb < P.NB) ? (nb * P.HTH + r * P.sh) * HTW + c * P.sw : 0;
+    }
+
+    f32x16 acc[TPW][NACC];
+#pragma unroll
+    for (int t = 0; t < TPW; ++t)
+#pragma unroll
+        for (int a = 0; a < NACC; ++a)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[t][a][r] = 0.f;
+
+    const int ntiles = P.tiles_n * P.tiles_h * P.tiles_w;
+    const long gcp = (long)CT * P.KPp, xcp = (long)CT * P.HPp;
+    for (int tile = blockIdx.z; tile < ntiles; tile += gridDim.z) {
+        const int tw = tile % P.tiles_w;
+        const int th = (tile / P.tiles_w) % P.tiles_h;
+        const int tn = tile / (P.tiles_w * P.tiles_h);
+        const int n0 = tn * P.NB, ho0 = th * P.TH, wo0 = tw * P.TW;
+        __syncthreads();
+        // gradient window: TH x TW output pixels, no halo; pixels beyond the tensor are zero and
+        // therefore contribute nothing whatever the input window holds there
+        stage_window<TS, CT, float>(gl, P.g, n0, cot * CT, ho0, wo0, P.NB, P.TH, P.TW, P.KPp, P.lpr_g);
+        stage_window<TS, CT, float>(xl, P.x, n0, cit * CT, ho0 * P.sh - P.pt + kh * P.dh,
+                                    wo0 * P.sw - P.pl + kw0 * P.dw, P.NB, P.HTH, HTW, P.HPp, P.lpr_x);
+        if (P.KP != P.NB * thw)  // odd pixel count: the padding column of the gradient window must be zero
+            for (int c = tid; c < 4 * CT; c += WG_THREADS) gl[c * P.KPp + P.KP - 1] = 0.f;
+        __syncthreads();
+        const float* ga = gl + (wco * 32 + m) * P.KPp + kk;
+        const float* xb = xl + (wci * 32 + m) * P.HPp;
+        for (int ks = 0; ks < P.KP; ks += 2) {
+            float g[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) g[q] = ga[q * gcp + ks];
+            const int po = poff[ks + kk];
+            float G[8];
+            if constexpr (MODE == 8) lanes_grad(g, G, 0.5f);
+#pragma unroll
+            for (int t = 0; t < TPW; ++t) {
+                if (t < nkw) {
+                    float x[4];
+#pragma unroll
+                    for (int p = 0; p < 4; ++p) x[p] = xb[p * xcp + po + t * P.dw];
+                    if constexpr (MODE == 16) {
+                        float nx[4];
+#pragma unroll
+                        for (int p = 0; p < 4; ++p) nx[p] = -x[p];
+#pragma unroll
+                        for (int p = 0; p < 4; ++p)
+#pragma unroll
+                            for (int q = 0; q < 4; ++q)
+                                acc[t][p ^ q] = __builtin_amdgcn_mfma_f32_32x32x2f32(g[q], qneg(p, q) ? nx[p] : x[p],
+                                                                                     acc[t][p ^ q], 0, 0, 0);
+                    } else {
+                        float L[8];
+                        lanes_left(x, L);
+#pragma unroll
+                        for (int i = 0; i < 8; ++i)
+                            acc[t][i] = __builtin_amdgcn_mfma_f32_32x32x2f32(G[i], L[i], acc[t][i], 0, 0, 0);
+                    }
+                }
+            }
+        }
+    }
+
+    // partial[z][tap][r][co][ci]
+    const int taps = P.Kh * P.Kw;
+    const long tap_stride = 4L * P.CoP * P.CiP;
+    float* dst = P.partial + (long)blockIdx.z * taps * tap_stride;
+    const int ci = cit * CT + wci * 32 + m;
+    const int co_base = cot * CT + wco * 32 + 4 * kk;
+#pragma unroll
+    for (int t = 0; t < TPW; ++t) {
+        if (t >= nkw) continue;
+        f32x16 y[4];
+        if constexpr (MODE == 16) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) y[r] = acc[t][r];
+        } else {
+            merge_right_grad(acc[t], y);
+        }
+        float* d = dst + (long)(kh * P.Kw + kw0 + t) * tap_stride;
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int co = co_base + 8 * (e >> 2) + (e & 3);
+                d[((long)r * P.CoP + co) * P.CiP + ci] = y[r][e];
+            }
+    }
+}
+
+struct ReduceArgs {
+    const float* partial;
+    void* dw;
+    long wcs, so, si, skh, skw;
+    int Z, Co, Ci, Kh, Kw, CoP, CiP;
+};
+
+// dw(r, co, ci, kh, kw) = sum_z partial[z][tap][r][co][ci], in increasing z (deterministic)
+template <typename TS>
+__global__ void __launch_bounds__(WG_THREADS) reduce_wgrad_kernel(const ReduceArgs P) {
+    const int taps = P.Kh * P.Kw;
+    const long total = 4L * taps * P.Co * P.Ci;
+    const long zstride = 4L * taps * P.CoP * P.CiP;
+    TS* dw = static_cast<TS*>(P.dw);
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
+        const int ci = idx % P.Ci;
+        long s = idx / P.Ci;
+        const int co = s % P.Co;
+        s /= P.Co;
+        const int r = s & 3;
+        const int tap = s >> 2;
+        const float* src = P.partial + (((long)tap * 4 + r) * P.CoP + co) * P.CiP + ci;
+        float sum = 0.f;
+        for (int z = 0; z < P.Z; ++z) sum += src[z * zstride];
+        const int kh = tap / P.Kw, kw = tap - kh * P.Kw;
+        stf<TS>(dw + r * P.wcs + co * P.so + ci * P.si + kh * P.skh + kw * P.skw, sum);
+    }
+}
+
+}  // namespace phx

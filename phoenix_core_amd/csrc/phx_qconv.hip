@@ -1,0 +1,532 @@
+// C ABI of the gfx950 quaternion Conv2D / Dense engine: descriptor checks, tile planning, filter
+// packing and kernel dispatch.  See include/phx_qconv.h for the contract.
+#include "../../include/phx_qconv.h"
+
+#include <algorithm>
+#include <cstdio>
+#include <cstring>
+
+#include "phx_kernels_f32.h"
+
+namespace phx {
+
+static thread_local const char* g_last_kernel = "";
+static thread_local char g_name_buf[128];
+
+#define PHX_HIP(call)                                              \
+    do {                                                           \
+        hipError_t e_ = (call);                                    \
+        if (e_ != hipSuccess) { (void)hipGetLastError(); return PHX_ERR_RUNTIME; } \
+    } while (0)
+
+static inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+static inline int cdiv(int a, int b) { return (a + b - 1) / b; }
+
+// Filter addressing: element (r, o, i, kh, kw) at r*wcs + o*so + i*si + kh*skh + kw*skw
+struct FilterStrides {
+    long wcs, so, si, skh, skw;
+};
+
+// One quaternion correlation problem in the engine's internal terms
+struct Problem {
+    int dtype, mode, policy;
+    int n, ci, co, h, w, kh, kw, sh, sw, dh, dw, pt, pl, pb, pr, ho, wo;
+    FilterStrides fs;
+    bool has_bias;
+};
+
+static int out_size(int in, int k, int d, int s, int before, int after) {
+    const int eff = (k - 1) * d + 1;
+    return (in + before + after - eff + s) / s;
+}
+
+static int problem_from_conv(const phx_qconv_desc* d, Problem& p) {
+    if (!d) return PHX_ERR_INVALID_ARGUMENT;
+    if (d->dtype != PHX_F32 && d->dtype != PHX_F16) return PHX_ERR_INVALID_ARGUMENT;
+    if (d->product_mode != PHX_PRODUCT_16 && d->product_mode != PHX_PRODUCT_8) return PHX_ERR_INVALID_ARGUMENT;
+    if (d->fp16_policy < PHX_FP16_FULL32 || d->fp16_policy > PHX_FP16_FULL16) return PHX_ERR_INVALID_ARGUMENT;
+    if (d->filter_layout != PHX_OIHW && d->filter_layout != PHX_OHWI) return PHX_ERR_INVALID_ARGUMENT;
+    if (d->n < 0 || d->ci <= 0 || d->co <= 0 || d->h < 0 || d->w < 0 || d->kh <= 0 || d->kw <= 0)
+        return PHX_ERR_INVALID_ARGUMENT;
+    if (d->stride_h <= 0 || d->stride_w <= 0 || d->dilation_h <= 0 || d->dilation_w <= 0)
+        return PHX_ERR_INVALID_ARGUMENT;
+    if (d->pad_top < 0 || d->pad_left < 0 || d->pad_bottom < 0 || d->pad_right < 0) return PHX_ERR_INVALID_ARGUMENT;
+    p.dtype = d->dtype;
+    p.mode = d->product_mode;
+    p.policy = d->fp16_policy;
+    p.n = d->n; p.ci = d->ci; p.co = d->co; p.h = d->h; p.w = d->w; p.kh = d->kh; p.kw = d->kw;
+    p.sh = d->stride_h; p.sw = d->stride_w; p.dh = d->dilation_h; p.dw = d->dilation_w;
+    p.pt = d->pad_top; p.pl = d->pad_left; p.pb = d->pad_bottom; p.pr = d->pad_right;
+    p.ho = out_size(p.h, p.kh, p.dh, p.sh, p.pt, p.pb);
+    p.wo = out_size(p.w, p.kw, p.dw, p.sw, p.pl, p.pr);
+    if ((p.h > 0 && p.ho <= 0) || (p.w > 0 && p.wo <= 0)) return PHX_ERR_INVALID_ARGUMENT;
+    const long taps = (long)p.kh * p.kw;
+    p.fs.wcs = (long)p.co * p.ci * taps;
+    if (d->filter_layout == PHX_OIHW) {
+        p.fs.so = p.ci * taps; p.fs.si = taps; p.fs.skh = p.kw; p.fs.skw = 1;
+    } else {  // OHWI
+        p.fs.so = taps * p.ci; p.fs.si = 1; p.fs.skh = (long)p.kw * p.ci; p.fs.skw = p.ci;
+    }
+    p.has_bias = d->has_bias != 0;
+    return PHX_OK;
+}
+
+static int problem_from_dense(const phx_qdense_desc* d, Problem& p) {
+    if (!d) return PHX_ERR_INVALID_ARGUMENT;
+    if (d->dtype != PHX_F32 && d->dtype != PHX_F16) return PHX_ERR_INVALID_ARGUMENT;
+    if (d->product_mode != PHX_PRODUCT_16 && d->product_mode != PHX_PRODUCT_8) return PHX_ERR_INVALID_ARGUMENT;
+    if (d->fp16_policy < PHX_FP16_FULL32 || d->fp16_policy > PHX_FP16_FULL16) return PHX_ERR_INVALID_ARGUMENT;
+    if (d->n < 0 || d->ni <= 0 || d->no <= 0) return PHX_ERR_INVALID_ARGUMENT;
+    p.dtype = d->dtype; p.mode = d->product_mode; p.policy = d->fp16_policy;
+    p.n = d->n; p.ci = d->ni; p.co = d->no; p.h = p.w = 1; p.kh = p.kw = 1;
+    p.sh = p.sw = p.dh = p.dw = 1; p.pt = p.pl = p.pb = p.pr = 0; p.ho = p.wo = 1;
+    // layout IO: w[r][i][o]
+    p.fs.wcs = (long)p.ci * p.co; p.fs.so = 1; p.fs.si = p.co; p.fs.skh = 0; p.fs.skw = 0;
+    p.has_bias = d->has_bias != 0;
+    return PHX_OK;
+}
+
+static bool is_empty(const Problem& p) { return p.n == 0 || p.h == 0 || p.w == 0; }
+
+static bool is_pointwise_unit(const Problem& p) {
+    return p.kh == 1 && p.kw == 1 && p.sh == 1 && p.sw == 1 && !p.pt && !p.pl && !p.pb && !p.pr;
+}
+
+// A pointwise, unit-stride, unpadded convolution sees each image plane as one long row
+static Problem flatten_pointwise(const Problem& p) {
+    Problem f = p;
+    if (is_pointwise_unit(p)) {
+        f.w = p.h * p.w; f.h = 1;
+        f.wo = p.ho * p.wo; f.ho = 1;
+    }
+    return f;
+}
+
+// -------------------------------------------------------------------------------------------
+// Correlation view shared by forward and input-gradient: out[N][Cout][Hout][Wout] from
+// in[N][Cin][Hin][Win] (seen through zero insertion uh, uw), unit stride unless forward.
+// -------------------------------------------------------------------------------------------
+struct Corr {
+    int N, Cin, Hin, Win, Cout, Hout, Wout;
+    int Kh, Kw, sh, sw, dh, dw, pt, pl, uh, uw;
+};
+
+static Corr corr_forward(const Problem& p) {
+    Corr c{p.n, p.ci, p.h, p.w, p.co, p.ho, p.wo, p.kh, p.kw, p.sh, p.sw, p.dh, p.dw, p.pt, p.pl, 1, 1};
+    if (p.kh == 1 && p.kw == 1 && p.sh == 1 && p.sw == 1 && !p.pt && !p.pl && !p.pb && !p.pr) {
+        c.Win = p.h * p.w; c.Hin = 1; c.Wout = p.ho * p.wo; c.Hout = 1;  // pointwise: one long row per image
+    }
+    return c;
+}
+
+static Corr corr_dgrad(const Problem& p) {
+    Corr c{p.n, p.co, p.ho, p.wo, p.ci, p.h, p.w, p.kh, p.kw, 1, 1, p.dh, p.dw,
+           (p.kh - 1) * p.dh - p.pt, (p.kw - 1) * p.dw - p.pl, p.sh, p.sw};
+    if (p.kh == 1 && p.kw == 1 && p.sh == 1 && p.sw == 1 && !p.pt && !p.pl && !p.pb && !p.pr) {
+        c.Win = p.ho * p.wo; c.Hin = 1; c.Wout = p.h * p.w; c.Hout = 1;
+    }
+    return c;
+}
+
+struct FwdPlan {
+    int WCO, NTW, BN;
+    int NB, TH, TW, HTH, HTW, HPp, lpr_log2;
+    int tiles_n, tiles_h, tiles_w, co_tiles, nchunks;
+    size_t lds_bytes, wpk_bytes;
+    int wgs;
+};
+
+static int lpr_for(int row_len) {
+    int l = 3;
+    while (l < 6 && (1 << l) < row_len) ++l;
+    return l;
+}
+
+constexpr int LDS_FLOATS_MAX = 16384;  // 64 KiB: two workgroups per CU
+
+static bool plan_forward(const Corr& c, int mode, FwdPlan& best) {
+    double best_score = -1.0;
+    const int wcos[3] = {1, 2, 4};
+    for (int wi = 0; wi < 3; ++wi) {
+        const int WCO = wcos[wi];
+        if (WCO > 1 && 32 * WCO > ((c.Cout + 31) / 32) * 32) continue;
+        for (int NTW = 1; NTW <= 2; ++NTW) {
+            const int BN = (4 / WCO) * NTW * 32;
+            int cand[16];
+            int nc = 0;
+            for (int k = 1; k <= 8; ++k) cand[nc++] = cdiv(c.Wout, k);
+            cand[nc++] = 8; cand[nc++] = 16; cand[nc++] = 32; cand[nc++] = BN;
+            for (int a = 0; a < nc; ++a) {
+                const int TW = std::min(cand[a], std::min(c.Wout, BN));
+                if (TW <= 0) continue;
+                for (int TH = 1; TH <= std::min(c.Hout, BN / TW); ++TH) {
+                    int NB = 1;
+                    if (TH == c.Hout && TW == c.Wout) NB = std::max(1, std::min(c.N, BN / (TH * TW)));
+                    const int HTH = (TH - 1) * c.sh + (c.Kh - 1) * c.dh + 1;
+                    const int HTW = (TW - 1) * c.sw + (c.Kw - 1) * c.dw + 1;
+                    const int HP = NB * HTH * HTW;
+                    const int HPp = HP;
+                    if (4 * F32_CK * HPp > LDS_FLOATS_MAX) continue;
+                    const int tn = cdiv(c.N, NB), th = cdiv(c.Hout, TH), tw = cdiv(c.Wout, TW);
+                    const int cot = cdiv(c.Cout, 32 * WCO);
+                    const long wgs = (long)tn * th * tw * cot;
+                    const double eff = ((double)c.N * c.Hout * c.Wout * c.Cout) / ((double)wgs * BN * 32 * WCO);
+                    const double fill = (double)wgs / ((double)cdiv((int)std::min<long>(wgs, 1 << 30), 512) * 512);
+                    const double halo = (double)(NB * TH * TW) / HP;  // staged data actually used
+                    const double score = eff * (0.25 + 0.75 * fill) * (0.9 + 0.1 * halo) * (NTW == 2 ? 1.02 : 1.0);
+                    if (score > best_score) {
+                        best_score = score;
+                        best = FwdPlan{WCO, NTW, BN, NB, TH, TW, HTH, HTW, HPp, lpr_for(HTW), tn, th, tw, cot,
+                                       cdiv(c.Cin, F32_CK), (size_t)4 * F32_CK * HPp * sizeof(float), 0, (int)wgs};
+                    }
+                }
+            }
+        }
+    }
+    if (best_score < 0) return false;
+    const int WC = (mode == 16) ? 4 : 8;
+    best.wpk_bytes = (size_t)best.co_tiles * best.WCO * best.nchunks * c.Kh * c.Kw * 4 * 64 * WC * sizeof(float);
+    return true;
+}
+
+template <typename TS, int MODE, int MAP>
+static int launch_fwd_variant(const FwdPlan& pl, const ConvArgs& a, hipStream_t st) {
+#define PHX_CASE(WCO_, NTW_)                                                                                     \
+    if (pl.WCO == WCO_ && pl.NTW == NTW_) {                                                                      \
+        hipLaunchKernelGGL((qconv_fwd_f32_kernel<TS, MODE, MAP, WCO_, NTW_>), dim3(pl.wgs), dim3(WG_THREADS),    \
+                           pl.lds_bytes, st, a);                                                                 \
+        return PHX_OK;                                                                                           \
+    }
+    PHX_CASE(1, 1) PHX_CASE(1, 2) PHX_CASE(2, 1) PHX_CASE(2, 2) PHX_CASE(4, 1) PHX_CASE(4, 2)
+#undef PHX_CASE
+    return PHX_ERR_NOT_SUPPORTED;
+}
+
+template <typename TS>
+static int run_corr(const Problem& p, const Corr& c, int map, hipStream_t st, const void* in, const void* w,
+                    const void* bias, void* out, void* ws, size_t ws_bytes) {
+    FwdPlan pl;
+    if (!plan_forward(c, p.mode, pl)) return PHX_ERR_NOT_SUPPORTED;
+    if (ws_bytes < pl.wpk_bytes || !ws) return PHX_ERR_WORKSPACE;
+    float* wpk = static_cast<float*>(ws);
+
+    PackArgs pa;
+    pa.w = w; pa.out = wpk;
+    pa.wcs = p.fs.wcs; pa.so = p.fs.so; pa.si = p.fs.si; pa.skh = p.fs.skh; pa.skw = p.fs.skw;
+    pa.Co = p.co; pa.Ci = p.ci; pa.Kh = p.kh; pa.Kw = p.kw;
+    pa.rows = c.Cout; pa.red = c.Cin; pa.row_tiles = pl.co_tiles * pl.WCO; pa.nchunks = pl.nchunks;
+    const long pack_items = (long)pa.row_tiles * pa.nchunks * p.kh * p.kw * 4 * 64;
+    const int pack_blocks = (int)std::min<long>((pack_items + WG_THREADS - 1) / WG_THREADS, 4096);
+
+    ConvArgs a;
+    a.in.base = in; a.in.comp_stride = (long)c.N * c.Cin * c.Hin * c.Win;
+    a.in.N = c.N; a.in.C = c.Cin; a.in.Hd = c.Hin; a.in.Wd = c.Win; a.in.uh = c.uh; a.in.uw = c.uw;
+    a.wpk = wpk; a.bias = bias; a.out = out;
+    a.out_cs = (long)c.N * c.Cout * c.Hout * c.Wout;
+    a.Cout = c.Cout; a.Hout = c.Hout; a.Wout = c.Wout;
+    a.taps = c.Kh * c.Kw; a.Kw = c.Kw; a.dh = c.dh; a.dw = c.dw; a.sh = c.sh; a.sw = c.sw; a.pt = c.pt; a.pl = c.pl;
+    a.NB = pl.NB; a.TH = pl.TH; a.TW = pl.TW; a.HTH = pl.HTH; a.HTW = pl.HTW; a.HPp = pl.HPp;
+    a.lpr_log2 = pl.lpr_log2;
+    a.tiles_n = pl.tiles_n; a.tiles_h = pl.tiles_h; a.tiles_w = pl.tiles_w; a.co_tiles = pl.co_tiles;
+    a.nchunks = pl.nchunks;
+
+    int rc;
+    if (p.mode == 16) {
+        if (map == MAP_FWD)
+            hipLaunchKernelGGL((pack_filters_f32_kernel<TS, 16, MAP_FWD>), dim3(pack_blocks), dim3(WG_THREADS), 0, st, pa);
+        else
+            hipLaunchKernelGGL((pack_filters_f32_kernel<TS, 16, MAP_DGRAD>), dim3(pack_blocks), dim3(WG_THREADS), 0, st, pa);
+        rc = launch_fwd_variant<TS, 16, MAP_FWD>(pl, a, st);  // conjugation lives in the packing
+    } else if (map == MAP_FWD) {
+        hipLaunchKernelGGL((pack_filters_f32_kernel<TS, 8, MAP_FWD>), dim3(pack_blocks), dim3(WG_THREADS), 0, st, pa);
+        rc = launch_fwd_variant<TS, 8, MAP_FWD>(pl, a, st);
+    } else {
+        hipLaunchKernelGGL((pack_filters_f32_kernel<TS, 8, MAP_DGRAD>), dim3(pack_blocks), dim3(WG_THREADS), 0, st, pa);
+        rc = launch_fwd_variant<TS, 8, MAP_DGRAD>(pl, a, st);
+    }
+    if (rc != PHX_OK) return rc;
+    PHX_HIP(hipGetLastError());
+    snprintf(g_name_buf, sizeof(g_name_buf), "qconv_%s_f32mfma_p%d_%s_wco%d_ntw%d_tile%dx%dx%d",
+             map == MAP_FWD ? "fwd" : "dgrad", p.mode, sizeof(TS) == 4 ? "f32" : "f16", pl.WCO, pl.NTW, pl.NB, pl.TH,
+             pl.TW);
+    g_last_kernel = g_name_buf;
+    return PHX_OK;
+}
+
+// -------------------------------------------------------------------------------------------
+// Filter gradient
+// -------------------------------------------------------------------------------------------
+struct WgPlan {
+    int TPW, NB, TH, TW, KP, KPp, HPp, HTH, HTWmax, lpr_g, lpr_x;
+    int tiles_n, tiles_h, tiles_w, co_tiles, ci_tiles, CoP, CiP, groups_per_row, Z;
+    size_t lds_bytes, partial_bytes;
+};
+
+static bool plan_wgrad(const Problem& p, WgPlan& best) {
+    const int TPW = (p.mode == 16) ? 3 : 1;
+    const int nkw = std::min(TPW, p.kw);
+    double best_score = -1.0;
+    const int budget = LDS_FLOATS_MAX / (4 * 64);  // KPp + HPp (+ offsets) per staged channel
+    for (int TW = 1; TW <= std::min(p.wo, 64); ++TW) {
+        for (int TH = 1; TH <= p.ho; ++TH) {
+            for (int NB = 1; NB <= p.n; ++NB) {
+                if (NB > 1 && !(TH == p.ho && TW == p.wo)) break;
+                const int pix = NB * TH * TW;
+                const int KP = (pix + 1) & ~1;
+                const int HTH = (TH - 1) * p.sh + 1;
+                const int HTW = (TW - 1) * p.sw + (nkw - 1) * p.dw + 1;
+                const int KPp = KP | 1, HPp = (NB * HTH * HTW) | 1;
+                if (KPp + HPp + (KP + 255) / 256 > budget) break;
+                const int tn = cdiv(p.n, NB), th = cdiv(p.ho, TH), tw = cdiv(p.wo, TW);
+                const double eff = ((double)p.n * p.ho * p.wo) / ((double)tn * th * tw * KP);
+                const double score = eff * (1.0 + 0.002 * KP);
+                if (score > best_score) {
+                    best_score = score;
+                    best.TPW = TPW; best.NB = NB; best.TH = TH; best.TW = TW; best.KP = KP; best.KPp = KPp;
+                    best.HPp = HPp; best.HTH = HTH; best.HTWmax = HTW;
+                    best.lpr_g = lpr_for(TW); best.lpr_x = lpr_for(HTW);
+                    best.tiles_n = tn; best.tiles_h = th; best.tiles_w = tw;
+                }
+            }
+        }
+    }
+    if (best_score < 0) return false;
+    best.co_tiles = cdiv(p.co, 64); best.ci_tiles = cdiv(p.ci, 64);
+    best.CoP = best.co_tiles * 64; best.CiP = best.ci_tiles * 64;
+    best.groups_per_row = cdiv(p.kw, TPW);
+    const int xy = best.co_tiles * best.ci_tiles * best.groups_per_row * p.kh;
+    const int ntiles = best.tiles_n * best.tiles_h * best.tiles_w;
+    best.Z = std::max(1, std::min(ntiles, 512 / std::max(1, xy)));
+    best.lds_bytes = ((size_t)4 * 64 * (best.KPp + best.HPp) + best.KP) * sizeof(float);
+    best.partial_bytes = (size_t)best.Z * p.kh * p.kw * 4 * best.CoP * best.CiP * sizeof(float);
+    return true;
+}
+
+template <typename TS>
+static int run_wgrad(const Problem& p, hipStream_t st, const void* x, const void* g, void* dw, void* ws,
+                     size_t ws_bytes) {
+    WgPlan pl;
+    if (!plan_wgrad(p, pl)) return PHX_ERR_NOT_SUPPORTED;
+    if (ws_bytes < pl.partial_bytes || !ws) return PHX_ERR_WORKSPACE;
+    WgradArgs a;
+    a.x.base = x; a.x.comp_stride = (long)p.n * p.ci * p.h * p.w; a.x.N = p.n; a.x.C = p.ci; a.x.Hd = p.h; a.x.Wd = p.w;
+    a.x.uh = a.x.uw = 1;
+    a.g.base = g; a.g.comp_stride = (long)p.n * p.co * p.ho * p.wo; a.g.N = p.n; a.g.C = p.co; a.g.Hd = p.ho; a.g.Wd = p.wo;
+    a.g.uh = a.g.uw = 1;
+    a.partial = static_cast<float*>(ws);
+    a.Kh = p.kh; a.Kw = p.kw; a.sh = p.sh; a.sw = p.sw; a.dh = p.dh; a.dw = p.dw; a.pt = p.pt; a.pl = p.pl;
+    a.NB = pl.NB; a.TH = pl.TH; a.TW = pl.TW; a.KP = pl.KP; a.KPp = pl.KPp; a.HPp = pl.HPp; a.HTH = pl.HTH;
+    a.HTWmax = pl.HTWmax; a.lpr_g = pl.lpr_g; a.lpr_x = pl.lpr_x;
+    a.tiles_n = pl.tiles_n; a.tiles_h = pl.tiles_h; a.tiles_w = pl.tiles_w;
+    a.co_tiles = pl.co_tiles; a.ci_tiles = pl.ci_tiles; a.CoP = pl.CoP; a.CiP = pl.CiP;
+    a.groups_per_row = pl.groups_per_row;
+    const dim3 grid(pl.co_tiles * pl.ci_tiles, pl.groups_per_row * p.kh, pl.Z);
+    if (p.mode == 16)
+        hipLaunchKernelGGL((qconv_wgrad_f32_kernel<TS, 16, 3>), grid, dim3(WG_THREADS), pl.lds_bytes, st, a);
+    else
+        hipLaunchKernelGGL((qconv_wgrad_f32_kernel<TS, 8, 1>), grid, dim3(WG_THREADS), pl.lds_bytes, st, a);
+    PHX_HIP(hipGetLastError());
+    ReduceArgs r;
+    r.partial = a.partial; r.dw = dw;
+    r.wcs = p.fs.wcs; r.so = p.fs.so; r.si = p.fs.si; r.skh = p.fs.skh; r.skw = p.fs.skw;
+    r.Z = pl.Z; r.Co = p.co; r.Ci = p.ci; r.Kh = p.kh; r.Kw = p.kw; r.CoP = pl.CoP; r.CiP = pl.CiP;
+    const long items = 4L * p.kh * p.kw * p.co * p.ci;
+    const int blocks = (int)std::min<long>((items + WG_THREADS - 1) / WG_THREADS, 8192);
+    hipLaunchKernelGGL((reduce_wgrad_kernel<TS>), dim3(blocks), dim3(WG_THREADS), 0, st, r);
+    PHX_HIP(hipGetLastError());
+    snprintf(g_name_buf, sizeof(g_name_buf), "qconv_wgrad_f32mfma_p%d_%s_tile%dx%dx%d_z%d", p.mode,
+             sizeof(TS) == 4 ? "f32" : "f16", pl.NB, pl.TH, pl.TW, pl.Z);
+    g_last_kernel = g_name_buf;
+    return PHX_OK;
+}
+
+static size_t workspace_for(const Problem& p, int pass) {
+    if (is_empty(p)) return 0;
+    if (pass == PHX_PASS_BWD_WEIGHTS) {
+        WgPlan pl;
+        return plan_wgrad(flatten_pointwise(p), pl) ? align_up(pl.partial_bytes, 256) : 0;
+    }
+    const Corr c = (pass == PHX_PASS_FWD) ? corr_forward(p) : corr_dgrad(p);
+    FwdPlan pl;
+    return plan_forward(c, p.mode, pl) ? align_up(pl.wpk_bytes, 256) : 0;
+}
+
+static int do_fwd(const Problem& p, hipStream_t st, const void* x, const void* w, const void* bias, void* y, void* ws,
+                  size_t wsb) {
+    if (is_empty(p)) return PHX_OK;  // the reference returns silently on empty input (src/conv2d.hpp:81-82)
+    if (!x || !w || !y || (p.has_bias && !bias)) return PHX_ERR_INVALID_ARGUMENT;
+    const Corr c = corr_forward(p);
+    const void* b = p.has_bias ? bias : nullptr;
+    return p.dtype == PHX_F32 ? run_corr<float>(p, c, MAP_FWD, st, x, w, b, y, ws, wsb)
+                              : run_corr<_Float16>(p, c, MAP_FWD, st, x, w, b, y, ws, wsb);
+}
+
+static int do_bwd_data(const Problem& p, hipStream_t st, const void* g, const void* w, void* dx, void* ws, size_t wsb) {
+    if (is_empty(p)) return PHX_OK;
+    if (!g || !w || !dx) return PHX_ERR_INVALID_ARGUMENT;
+    const Corr c = corr_dgrad(p);
+    return p.dtype == PHX_F32 ? run_corr<float>(p, c, MAP_DGRAD, st, g, w, nullptr, dx, ws, wsb)
+                              : run_corr<_Float16>(p, c, MAP_DGRAD, st, g, w, nullptr, dx, ws, wsb);
+}
+
+static int do_bwd_weights(const Problem& p, hipStream_t st, const void* x, const void* g, void* dw, void* ws,
+                          size_t wsb) {
+    if (!dw) return PHX_ERR_INVALID_ARGUMENT;
+    if (is_empty(p)) {  // the reference zeroes the filter gradient on empty input (src/conv2d.hpp:341-344)
+        const size_t bytes = (size_t)4 * p.fs.wcs * (p.dtype == PHX_F32 ? 4 : 2);
+        PHX_HIP(hipMemsetAsync(dw, 0, bytes, st));
+        return PHX_OK;
+    }
+    if (!x || !g) return PHX_ERR_INVALID_ARGUMENT;
+    const Problem f = flatten_pointwise(p);
+    return p.dtype == PHX_F32 ? run_wgrad<float>(f, st, x, g, dw, ws, wsb)
+                              : run_wgrad<_Float16>(f, st, x, g, dw, ws, wsb);
+}
+
+}  // namespace phx
+
+using namespace phx;
+
+extern "C" {
+
+const char* phx_status_string(int status) {
+    switch (status) {
+        case PHX_OK: return "ok";
+        case PHX_ERR_INVALID_ARGUMENT: return "invalid argument";
+        case PHX_ERR_NOT_SUPPORTED: return "not supported";
+        case PHX_ERR_WORKSPACE: return "workspace too small";
+        case PHX_ERR_RUNTIME: return "HIP runtime error";
+    }
+    return "unknown status";
+}
+
+const char* phx_last_kernel_name(void) { return g_last_kernel; }
+
+int phx_qconv2d_output_hw(const phx_qconv_desc* desc, int32_t* ho, int32_t* wo) {
+    Problem p;
+    const int rc = problem_from_conv(desc, p);
+    if (rc != PHX_OK) return rc;
+    if (ho) *ho = p.ho;
+    if (wo) *wo = p.wo;
+    return PHX_OK;
+}
+
+size_t phx_qconv2d_workspace_bytes(const phx_qconv_desc* desc, int pass) {
+    Problem p;
+    if (problem_from_conv(desc, p) != PHX_OK) return 0;
+    return workspace_for(p, pass);
+}
+
+size_t phx_qdense_workspace_bytes(const phx_qdense_desc* desc, int pass) {
+    Problem p;
+    if (problem_from_dense(desc, p) != PHX_OK) return 0;
+    return workspace_for(p, pass);
+}
+
+int phx_qconv2d_fwd(const phx_qconv_desc* desc, phx_stream_t stream, const void* x, const void* w,
+                    const void* bias_or_null, void* y, void* workspace, size_t workspace_bytes) {
+    Problem p;
+    const int rc = problem_from_conv(desc, p);
+    if (rc != PHX_OK) return rc;
+    return do_fwd(p, static_cast<hipStream_t>(stream), x, w, bias_or_null, y, workspace, workspace_bytes);
+}
+
+int phx_qconv2d_bwd_data(const phx_qconv_desc* desc, phx_stream_t stream, const void* grad, const void* w, void* dx,
+                         void* workspace, size_t workspace_bytes) {
+    Problem p;
+    const int rc = problem_from_conv(desc, p);
+    if (rc != PHX_OK) return rc;
+    return do_bwd_data(p, static_cast<hipStream_t>(stream), grad, w, dx, workspace, workspace_bytes);
+}
+
+int phx_qconv2d_bwd_weights(const phx_qconv_desc* desc, phx_stream_t stream, const void* x, const void* grad, void* dw,
+                            void* workspace, size_t workspace_bytes) {
+    Problem p;
+    const int rc = problem_from_conv(desc, p);
+    if (rc != PHX_OK) return rc;
+    return do_bwd_weights(p, static_cast<hipStream_t>(stream), x, grad, dw, workspace, workspace_bytes);
+}
+
+int phx_qdense_fwd(const phx_qdense_desc* desc, phx_stream_t stream, const void* x, const void* w,
+                   const void* bias_or_null, void* y, void* workspace, size_t workspace_bytes) {
+    Problem p;
+    const int rc = problem_from_dense(desc, p);
+    if (rc != PHX_OK) return rc;
+    return do_fwd(p, static_cast<hipStream_t>(stream), x, w, bias_or_null, y, workspace, workspace_bytes);
+}
+
+int phx_qdense_bwd_data(const phx_qdense_desc* desc, phx_stream_t stream, const void* grad, const void* w, void* dx,
+                        void* workspace, size_t workspace_bytes) {
+    Problem p;
+    const int rc = problem_from_dense(desc, p);
+    if (rc != PHX_OK) return rc;
+    return do_bwd_data(p, static_cast<hipStream_t>(stream), grad, w, dx, workspace, workspace_bytes);
+}
+
+int phx_qdense_bwd_weights(const phx_qdense_desc* desc, phx_stream_t stream, const void* x, const void* grad, void* dw,
+                           void* workspace, size_t workspace_bytes) {
+    Problem p;
+    const int rc = problem_from_dense(desc, p);
+    if (rc != PHX_OK) return rc;
+    return do_bwd_weights(p, static_cast<hipStream_t>(stream), x, grad, dw, workspace, workspace_bytes);
+}
+
+int phx_device_count(int32_t* count) {
+    int c = 0;
+    if (hipGetDeviceCount(&c) != hipSuccess) { (void)hipGetLastError(); c = 0; }
+    if (count) *count = c;
+    return PHX_OK;
+}
+
+int phx_device_malloc(void** ptr, size_t bytes) {
+    if (!ptr) return PHX_ERR_INVALID_ARGUMENT;
+    *ptr = nullptr;
+    if (bytes == 0) return PHX_OK;
+    PHX_HIP(hipMalloc(ptr, bytes));
+    return PHX_OK;
+}
+
+int phx_device_free(void* ptr) {
+    if (ptr) PHX_HIP(hipFree(ptr));
+    return PHX_OK;
+}
+
+int phx_memcpy_h2d(void* dst, const void* src, size_t bytes, phx_stream_t stream) {
+    if (bytes == 0) return PHX_OK;
+    PHX_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, static_cast<hipStream_t>(stream)));
+    PHX_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+    return PHX_OK;
+}
+
+int phx_memcpy_d2h(void* dst, const void* src, size_t bytes, phx_stream_t stream) {
+    if (bytes == 0) return PHX_OK;
+    PHX_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, static_cast<hipStream_t>(stream)));
+    PHX_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+    return PHX_OK;
+}
+
+int phx_memset_zero(void* dst, size_t bytes, phx_stream_t stream) {
+    if (bytes == 0) return PHX_OK;
+    PHX_HIP(hipMemsetAsync(dst, 0, bytes, static_cast<hipStream_t>(stream)));
+    return PHX_OK;
+}
+
+int phx_stream_create(phx_stream_t* stream) {
+    if (!stream) return PHX_ERR_INVALID_ARGUMENT;
+    hipStream_t s;
+    PHX_HIP(hipStreamCreate(&s));
+    *stream = s;
+    return PHX_OK;
+}
+
+int phx_stream_destroy(phx_stream_t stream) {
+    if (stream) PHX_HIP(hipStreamDestroy(static_cast<hipStream_t>(stream)));
+    return PHX_OK;
+}
+
+int phx_stream_synchronize(phx_stream_t stream) {
+    PHX_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+    return PHX_OK;
+}
+
+}  // extern "C"
