@@ -1,0 +1,182 @@
+#!/usr/bin/env python3
+"""Benchmark of the quaternion Conv2D hot path on one MI355X.
+
+A step is one pass of the hot path over one batch of synthetic input: forward, input-gradient and
+filter-gradient of one quaternion convolution, inputs resident in HBM.  The default workload is the
+pointwise fp32 configuration (N=32, 64->64 quaternion channels, 56x56); --workload selects the
+others.  Prints ONE JSON line: real-equivalent TFLOP/s (16 real multiply-adds per quaternion
+multiply-add, for either product mode), the roofline of the dominant kernel and the reference's CPU
+algorithm timed on the host cores of the same box.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+METRIC = "quaternion conv TFLOP/s (real-equiv, % MFMA peak) + q-ResNet-50 fwd+bwd img/s"
+PEAK_TFLOPS = {"f32": 157.3, "f16": 2500.0}  # MI355X dense MFMA peaks
+
+WORKLOADS = {
+    # name: (n, ci, co, h, w, k, padding, dtype, policy)
+    "c2_pw_f32": (32, 64, 64, 56, 56, 1, "VALID", "f32", "fp32"),
+    "c3_k3_f32": (64, 64, 64, 56, 56, 3, "SAME", "f32", "fp32"),
+    "c4_k3_f16_128_28": (128, 128, 128, 28, 28, 3, "SAME", "f16", "full16"),
+    "c4_k3_f16_256_14": (128, 256, 256, 14, 14, 3, "SAME", "f16", "full16"),
+    "c4_pw_f16_128_28": (128, 128, 128, 28, 28, 1, "VALID", "f16", "full16"),
+    "c4_pw_f16_256_14": (128, 256, 256, 14, 14, 1, "VALID", "f16", "full16"),
+}
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="c2_pw_f32", choices=sorted(WORKLOADS))
+    ap.add_argument("--mode", type=int, default=0, choices=[0, 8, 16],
+                    help="product formulation; 0 = from UPSTRIDE_MEMORY_OPTIMIZED like the reference (default 8)")
+    ap.add_argument("--policy", default=None, help="override UPSTRIDE_CONV_FP16_POLICY for fp16 workloads")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU time budget of the cpu_baseline leg")
+    return ap.parse_args()
+
+
+def cpu_baseline(cfg, mode, seconds):
+    """The reference's CPU algorithm (lane decomposition + scalar oneDNN convolutions through
+    torch's CPU backend) on a bounded sample of the same workload."""
+    import torch
+    import oracle
+    from oracle import torch_cpu_path as tcp
+    n, ci, co, h, w, k, padding, _, _ = cfg
+    threads = min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(threads)
+    n_s = max(1, n // 8)
+    g = oracle.make_geom(n_s, ci, co, h, w, k, k, 1, 1, padding)
+    gen = torch.Generator().manual_seed(0x5EED)
+    x = torch.randn(4 * n_s, ci, h, w, generator=gen)
+    wt = torch.randn(4, co, ci, k, k, generator=gen) * (2.0 / (ci * k * k)) ** 0.5
+    gr = torch.randn(4 * n_s, co, g.ho, g.wo, generator=gen)
+    name = "factorized" if mode == 8 else "generic"
+    flops = 3 * 2 * 16 * n_s * co * ci * g.ho * g.wo * k * k
+
+    def step():
+        tcp.conv2d_fwd(g, x, wt, None, name)
+        tcp.conv2d_bwd(g, x, wt, gr, name)
+
+    step()  # warm-up (primitive creation)
+    times = []
+    t_end = time.perf_counter() + seconds
+    while len(times) < 3 or (time.perf_counter() < t_end and len(times) < 50):
+        t0 = time.perf_counter()
+        step()
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    med = times[len(times) // 2]
+    return {
+        "value": flops / med / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+        "sample": "%d of %d images of the same workload, fwd+dgrad+wgrad, %s path, scalar convs by torch %s CPU "
+                  "(oneDNN), fp32, median of %d runs" % (n_s, n, name, torch.__version__, len(times)),
+        "ms_per_step_sample": med * 1e3,
+    }
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (--gpus %d refused)" % args.gpus,
+              file=sys.stderr)
+        return 2
+
+    import torch
+    import phoenix_core_amd as phx
+    from phoenix_core_amd import capi
+
+    cfg = WORKLOADS[args.workload]
+    n, ci, co, h, w, k, padding, dt, policy = cfg
+    if args.policy:
+        policy = args.policy
+    env = {"UPSTRIDE_CONV_FP16_POLICY": policy}
+    if args.mode == 16 or (args.mode == 0 and phx.Context().memory_optimized):
+        env["UPSTRIDE_MEMORY_OPTIMIZED"] = "1"
+    ctx = phx.Context(env)
+    mode = 16 if ctx.memory_optimized else 8
+    dtype = torch.float32 if dt == "f32" else torch.float16
+
+    dev = torch.device("cuda:0")
+    torch.manual_seed(0x5EED + sorted(WORKLOADS).index(args.workload))
+    scale = 1.0 if dt == "f32" else 0.5
+    x = (scale * torch.randn(4 * n, ci, h, w, device=dev)).to(dtype)
+    wt = (scale * torch.randn(4, co, ci, k, k, device=dev) * (2.0 / (ci * k * k)) ** 0.5).to(dtype)
+    desc = phx.Conv2DDescriptor(x.shape, wt.shape, 1, 1, padding, dtype=dtype, context=ctx)
+    gr = (scale * torch.randn(desc.output_shape, device=dev)).to(dtype)
+    ho, wo = desc.output_shape[2:]
+    y = torch.empty(desc.output_shape, dtype=dtype, device=dev)
+    dx = torch.empty_like(x)
+    dw = torch.empty_like(wt)
+    L = capi.lib()
+    sizes = [desc.workspace_bytes(p) for p in (capi.PHX_PASS_FWD, capi.PHX_PASS_BWD_DATA, capi.PHX_PASS_BWD_WEIGHTS)]
+    ws = torch.empty(max(sizes), dtype=torch.uint8, device=dev)
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+    d = ctypes.byref(desc.c)
+    names = {}
+
+    def step():
+        capi.check(L.phx_qconv2d_fwd(d, stream, P(x), P(wt), None, P(y), P(ws), sizes[0]), "fwd")
+        names.setdefault("fwd", capi.last_kernel_name())
+        capi.check(L.phx_qconv2d_bwd_data(d, stream, P(gr), P(wt), P(dx), P(ws), sizes[1]), "bwd_data")
+        names.setdefault("bwd_data", capi.last_kernel_name())
+        capi.check(L.phx_qconv2d_bwd_weights(d, stream, P(x), P(gr), P(dw), P(ws), sizes[2]), "bwd_weights")
+        names.setdefault("bwd_weights", capi.last_kernel_name())
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    capi.profile_enable(3 * args.steps)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    kernel_ms = capi.profile_collect(3 * args.steps)
+    capi.profile_enable(0)
+
+    flops_pass = 2.0 * 16 * n * co * ci * ho * wo * k * k
+    ms_per_step = elapsed / args.steps * 1e3
+    value = 3 * flops_pass / (ms_per_step * 1e-3) / 1e12
+    per_pass = {}
+    for i, key in enumerate(("fwd", "bwd_data", "bwd_weights")):
+        vals = kernel_ms[i::3]
+        per_pass[key] = sum(vals) / max(1, len(vals))
+    dominant = max(per_pass, key=per_pass.get)
+    compute = "f32" if (dt == "f32" or policy == "fp32" or (policy == "backward32" and dominant != "fwd")) else "f16"
+    achieved = flops_pass / (per_pass[dominant] * 1e-3) / 1e12
+    out = {
+        "metric": METRIC, "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": dt, "data": "synthetic",
+        "config": {"workload": "%s: quaternion conv %dx%d stride 1, N=%d (4N=%d rows), %d->%d q-channels, %dx%d, "
+                               "fwd+input-grad+filter-grad" % (args.workload, k, k, n, 4 * n, ci, co, h, w),
+                   "product_mode": mode, "fp16_policy": policy, "padding": padding},
+        "images_per_s": n / (ms_per_step * 1e-3),
+        "frac_of_mfma_peak": value / PEAK_TFLOPS[compute],
+        "executed_tflops": value * (0.5 if mode == 8 else 1.0),
+        "kernel_ms": per_pass, "kernels": names,
+        "roofline": {"bound": "mfma", "kernel": names[dominant], "achieved": achieved, "peak": PEAK_TFLOPS[compute],
+                     "unit": "TFLOP/s", "frac": achieved / PEAK_TFLOPS[compute], "traffic": None,
+                     "executed": achieved * (0.5 if mode == 8 else 1.0)},
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(cfg, mode, args.cpu_seconds)
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -129,6 +129,17 @@ int phx_stream_create(phx_stream_t* stream);
 int phx_stream_destroy(phx_stream_t stream);
 int phx_stream_synchronize(phx_stream_t stream);
 
+/* Kernel timing for benchmarks.  phx_profile_enable(capacity > 0) allocates `capacity` HIP event
+ * pairs for the calling thread; from then on every compute entry point called by that thread
+ * brackets its dominant kernel (the MFMA kernel, not the filter packing or the split-K reduction)
+ * with the next pair, recorded on the call's stream, until the pairs run out.  Nothing
+ * synchronises while recording.  phx_profile_collect() waits for the recorded pairs, writes their
+ * elapsed times in call order, returns how many there were through `count` and rearms the pairs.
+ * phx_profile_enable(0) stops recording.  No counterpart in the reference, whose profiler
+ * (src/backend/cudnn/kernels.cc:54-85) times candidate launch configurations instead. */
+int phx_profile_enable(int capacity);
+int phx_profile_collect(float* milliseconds, int max_count, int* count);
+
 /* Name of the kernel variant the last successful call on this thread dispatched to (for
  * profiling and tests); a static string. */
 const char* phx_last_kernel_name(void);

@@ -22,7 +22,7 @@ EXPORTS = (
     "phx_qdense_fwd", "phx_qdense_bwd_data", "phx_qdense_bwd_weights",
     "phx_device_count", "phx_device_malloc", "phx_device_free", "phx_memcpy_h2d", "phx_memcpy_d2h",
     "phx_memset_zero", "phx_stream_create", "phx_stream_destroy", "phx_stream_synchronize",
-    "phx_last_kernel_name",
+    "phx_last_kernel_name", "phx_profile_enable", "phx_profile_collect",
 )
 
 
@@ -77,6 +77,8 @@ def lib():
         L.phx_stream_create.argtypes = [ctypes.POINTER(vp)]
         L.phx_stream_destroy.argtypes = [vp]
         L.phx_stream_synchronize.argtypes = [vp]
+        L.phx_profile_enable.argtypes = [ctypes.c_int]
+        L.phx_profile_collect.argtypes = [ctypes.POINTER(ctypes.c_float), ctypes.c_int, i32p]
         _lib = L
     return _lib
 
@@ -92,3 +94,16 @@ def last_kernel_name():
 def check(status, what):
     if status != PHX_OK:
         raise PhxError(status, what)
+
+
+def profile_enable(capacity):
+    """Start (capacity > 0) or stop (0) timing the dominant kernel of each call of this thread."""
+    check(lib().phx_profile_enable(int(capacity)), "phx_profile_enable")
+
+
+def profile_collect(max_count=4096):
+    """Elapsed milliseconds of the kernels timed since the last collect, in call order."""
+    buf = (ctypes.c_float * max_count)()
+    n = ctypes.c_int32(0)
+    check(lib().phx_profile_collect(buf, max_count, ctypes.byref(n)), "phx_profile_collect")
+    return [buf[i] for i in range(n.value)]

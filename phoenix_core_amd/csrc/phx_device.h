@@ -125,51 +125,66 @@ struct TileSrc {
     int uh, uw;        // zero-insertion factors (1 = none)
 };
 
-// Copies the window [n0, n0+NB) x [c0, c0+NCH) x [h0, h0+HTH) x [w0, w0+HTW) of all four
-// components into LDS as dst[(p*NCH + c)*pitch + (nb*HTH + hr)*HTW + hc], zero-filling whatever
-// falls outside the tensor.  Rows are dealt to groups of `lpr` adjacent lanes so that global
-// reads run along W.
-template <typename TS, int NCH, typename TD>
-__device__ __forceinline__ void stage_window(TD* dst, const TileSrc& s, int n0, int c0, int h0, int w0, int NB,
-                                             int HTH, int HTW, int pitch, int lpr_log2) {
-    const TS* base = static_cast<const TS*>(s.base);
-    const int lpr = 1 << lpr_log2;
-    const int rl = threadIdx.x & (lpr - 1);
-    const int worker = threadIdx.x >> lpr_log2;
-    const int workers = WG_THREADS >> lpr_log2;
-    const int rows_per_c = NB * HTH;
-    const int rows = 4 * NCH * rows_per_c;
+// Window staging, split so that global loads can be in flight while the previous chunk is being
+// multiplied: each thread owns ONE position of the window [n0, n0+NB) x [h0, h0+HTH) x [w0, w0+HTW)
+// (decoded once, it does not depend on the channel) and walks over the (component, channel) planes
+// of a chunk.  The 256 threads form G = 256 >> P2LOG groups of 2^P2LOG positions; group g loads
+// planes g, g+G, ...  Loads are unconditional (out-of-tensor positions read the tensor's first
+// element and are zeroed by a select) so that the staged values stay plain registers.
+struct StagePos {
+    long goff;   // offset of this thread's position from the start of component 0, channel 0
+    int pos;     // position inside the window, < 2^P2LOG
+    int group;   // which plane subset this thread loads
+    bool valid;  // position lies inside the tensor (otherwise it is staged as zero)
+};
+
+template <int P2LOG>
+__device__ __forceinline__ StagePos make_stage_pos(const TileSrc& s, int n0, int h0, int w0, int NB, int HTH, int HTW) {
+    StagePos sp;
+    sp.pos = threadIdx.x & ((1 << P2LOG) - 1);
+    sp.group = threadIdx.x >> P2LOG;
+    const int hw = HTH * HTW;
+    const int nb = sp.pos / hw, rem = sp.pos - nb * hw;
+    const int hr = rem / HTW, hc = rem - hr * HTW;
+    int vh = h0 + hr, vw = w0 + hc;
+    bool ok = nb < NB && (n0 + nb) < s.N && vh >= 0 && vw >= 0;
+    if (s.uh > 1) { ok = ok && (vh % s.uh == 0); vh /= s.uh; }
+    if (s.uw > 1) { ok = ok && (vw % s.uw == 0); vw /= s.uw; }
+    ok = ok && vh < s.Hd && vw < s.Wd;
+    sp.valid = ok;
+    sp.goff = ok ? ((long)(n0 + nb) * s.C * s.Hd + vh) * s.Wd + vw : 0;
+    return sp;
+}
+
+// Issues the loads of one chunk: NCH channels starting at c0, all four components.
+// v[e] receives plane pc = e*G + group, pc = p*NCH + c.
+template <typename TS, int NCH, int P2LOG>
+__device__ __forceinline__ void stage_load(float (&v)[(4 * NCH) >> (8 - P2LOG)], const TileSrc& s, const StagePos& sp,
+                                           int c0) {
+    constexpr int G = WG_THREADS >> P2LOG;
+    constexpr int E = (4 * NCH) / G;
+    const TS* origin = static_cast<const TS*>(s.base);
     const long plane = (long)s.Hd * s.Wd;
-    for (int row = worker; row < rows; row += workers) {
-        const int pc = row / rows_per_c;
-        const int rr = row - pc * rows_per_c;
-        const int nb = rr / HTH;
-        const int hr = rr - nb * HTH;
-        const int p = pc / NCH, c = pc - p * NCH;
-        int vh = h0 + hr;
-        bool ok = (c0 + c < s.C) && (n0 + nb < s.N) && vh >= 0;
-        if (s.uh > 1) {
-            ok = ok && (vh % s.uh == 0);
-            vh /= s.uh;
-        }
-        ok = ok && vh < s.Hd;
-        const TS* src = base + p * s.comp_stride + ((long)(n0 + nb) * s.C + c0 + c) * plane + (long)vh * s.Wd;
-        TD* out = dst + (long)pc * pitch + rr * HTW;
-        if (s.uw == 1) {
-            for (int hc = rl; hc < HTW; hc += lpr) {
-                const int vw = w0 + hc;
-                float v = 0.f;
-                if (ok && vw >= 0 && vw < s.Wd) v = ldf<TS>(src + vw);
-                out[hc] = (TD)v;
-            }
-        } else {
-            for (int hc = rl; hc < HTW; hc += lpr) {
-                const int vw = w0 + hc;
-                float v = 0.f;
-                if (ok && vw >= 0 && (vw % s.uw == 0) && (vw / s.uw) < s.Wd) v = ldf<TS>(src + vw / s.uw);
-                out[hc] = (TD)v;
-            }
-        }
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+        const int pc = e * G + sp.group;
+        const int p = pc / NCH, c = pc % NCH;
+        const bool ok = sp.valid && (c0 + c) < s.C;
+        const TS* ptr = ok ? origin + sp.goff + p * s.comp_stride + (long)(c0 + c) * plane : origin;
+        const float t = ldf<TS>(ptr);
+        v[e] = ok ? t : 0.f;
+    }
+}
+
+// Writes the staged chunk as dst[pc*pitch + pos]
+template <int NCH, int P2LOG, typename TD>
+__device__ __forceinline__ void stage_store(TD* dst, const float (&v)[(4 * NCH) >> (8 - P2LOG)], const StagePos& sp,
+                                            int HP, int pitch) {
+    constexpr int G = WG_THREADS >> P2LOG;
+    constexpr int E = (4 * NCH) / G;
+    if (sp.pos < HP) {
+#pragma unroll
+        for (int e = 0; e < E; ++e) dst[(e * G + sp.group) * pitch + sp.pos] = (TD)v[e];
     }
 }
 

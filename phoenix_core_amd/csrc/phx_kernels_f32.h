@@ -22,8 +22,7 @@ struct ConvArgs {
     int dh, dw, sh, sw; // dilation and stride of the correlation
     int pt, pl;         // virtual input row of output row 0, tap 0, is -pt (same for columns)
     int NB, TH, TW;     // output pixels per workgroup tile: images x rows x columns
-    int HTH, HTW, HPp;  // halo window and LDS pitch per staged channel
-    int lpr_log2;       // lanes per staged row (log2)
+    int HTH, HTW, HP, HPp;  // halo window, its size and the LDS pitch per staged channel
     int tiles_n, tiles_h, tiles_w, co_tiles;
     int nchunks;        // ceil(Cin / F32_CK)
 };
@@ -88,10 +87,16 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_fwd_f32_kernel(const ConvArg
 
     long step = 0;
     const long cpitch = (long)CK * P.HPp;  // LDS floats between components
+    constexpr int P2LOG = 8;  // one window position per thread, every thread walks all 32 planes
+    const StagePos sp = make_stage_pos<P2LOG>(P.in, n0, h0, w0, P.NB, P.HTH, P.HTW);
+    float stage[4 * CK];
+    stage_load<TS, CK, P2LOG>(stage, P.in, sp, 0);
     for (int chunk = 0; chunk < P.nchunks; ++chunk) {
         __syncthreads();
-        stage_window<TS, CK, float>(lds, P.in, n0, chunk * CK, h0, w0, P.NB, P.HTH, P.HTW, P.HPp, P.lpr_log2);
+        stage_store<CK, P2LOG, float>(lds, stage, sp, P.HP, P.HPp);
         __syncthreads();
+        // next chunk's global loads fly while this chunk is multiplied
+        if (chunk + 1 < P.nchunks) stage_load<TS, CK, P2LOG>(stage, P.in, sp, (chunk + 1) * CK);
         int kh = 0, kw = 0;
         for (int tap = 0; tap < P.taps; ++tap) {
             const int tapoff = kh * P.dh * P.HTW + kw * P.dw;
@@ -141,27 +146,30 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_fwd_f32_kernel(const ConvArg
     const int co_base = (ct * WCO + wco) * 32 + 4 * kk;
 #pragma unroll
     for (int t = 0; t < NTW; ++t) {
-        f32x16 y[4];
-        if constexpr (MODE == 16) {
-#pragma unroll
-            for (int q = 0; q < 4; ++q) y[q] = acc[t][q];
-        } else if constexpr (MAP == MAP_FWD) {
-            merge_output(acc[t], y);
-        } else {
-            merge_left_grad(acc[t], y);
-        }
         if (!pvalid[t]) continue;
 #pragma unroll
-        for (int q = 0; q < 4; ++q)
+        for (int r = 0; r < 16; ++r) {
+            const int co = co_base + 8 * (r >> 2) + (r & 3);
+            float y[4];
+            if constexpr (MODE == 16) {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int co = co_base + 8 * (r >> 2) + (r & 3);
-                if (co < P.Cout) {
-                    float v = y[q][r];
+                for (int q = 0; q < 4; ++q) y[q] = acc[t][q][r];
+            } else {
+                float l[8];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) l[i] = acc[t][i][r];
+                if constexpr (MAP == MAP_FWD) merge_output(l, y);
+                else merge_left_grad(l, y);
+            }
+            if (co < P.Cout) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    float v = y[q];
                     if (bias) v += ldf<TS>(bias + q * P.Cout + co);
                     stf<TS>(out + q * P.out_cs + oaddr[t] + co * plane, v);
                 }
             }
+        }
     }
 }
 
@@ -245,7 +253,7 @@ struct WgradArgs {
     int NB, TH, TW;     // reduction tile: images x output rows x output columns
     int KP, KPp, HPp;   // pixels per tile (even), LDS pitches (odd) of gradient / input windows
     int HTH, HTWmax;
-    int lpr_g, lpr_x;   // log2 lanes per staged row
+    int HPx;            // input window size for a full tap group (<= 32, like KP)
     int tiles_n, tiles_h, tiles_w;
     int co_tiles, ci_tiles, CoP, CiP;
     int groups_per_row; // tap groups per filter row
@@ -286,20 +294,32 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_wgrad_f32_kernel(const Wgrad
 
     const int ntiles = P.tiles_n * P.tiles_h * P.tiles_w;
     const long gcp = (long)CT * P.KPp, xcp = (long)CT * P.HPp;
-    for (int tile = blockIdx.z; tile < ntiles; tile += gridDim.z) {
+    constexpr int P2LOG = 5;  // 32 window positions x 8 plane groups
+    float sg[32], sx[32];
+    StagePos spg, spx;
+    auto issue = [&](int tile) {
         const int tw = tile % P.tiles_w;
         const int th = (tile / P.tiles_w) % P.tiles_h;
         const int tn = tile / (P.tiles_w * P.tiles_h);
         const int n0 = tn * P.NB, ho0 = th * P.TH, wo0 = tw * P.TW;
-        __syncthreads();
         // gradient window: TH x TW output pixels, no halo; pixels beyond the tensor are zero and
         // therefore contribute nothing whatever the input window holds there
-        stage_window<TS, CT, float>(gl, P.g, n0, cot * CT, ho0, wo0, P.NB, P.TH, P.TW, P.KPp, P.lpr_g);
-        stage_window<TS, CT, float>(xl, P.x, n0, cit * CT, ho0 * P.sh - P.pt + kh * P.dh,
-                                    wo0 * P.sw - P.pl + kw0 * P.dw, P.NB, P.HTH, HTW, P.HPp, P.lpr_x);
+        spg = make_stage_pos<P2LOG>(P.g, n0, ho0, wo0, P.NB, P.TH, P.TW);
+        spx = make_stage_pos<P2LOG>(P.x, n0, ho0 * P.sh - P.pt + kh * P.dh, wo0 * P.sw - P.pl + kw0 * P.dw, P.NB, P.HTH,
+                                    HTW);
+        stage_load<TS, CT, P2LOG>(sg, P.g, spg, cot * CT);
+        stage_load<TS, CT, P2LOG>(sx, P.x, spx, cit * CT);
+    };
+    const int HPx = P.NB * P.HTH * HTW;
+    if ((int)blockIdx.z < ntiles) issue(blockIdx.z);
+    for (int tile = blockIdx.z; tile < ntiles; tile += gridDim.z) {
+        __syncthreads();
+        stage_store<CT, P2LOG, float>(gl, sg, spg, P.NB * thw, P.KPp);
+        stage_store<CT, P2LOG, float>(xl, sx, spx, HPx, P.HPp);
         if (P.KP != P.NB * thw)  // odd pixel count: the padding column of the gradient window must be zero
             for (int c = tid; c < 4 * CT; c += WG_THREADS) gl[c * P.KPp + P.KP - 1] = 0.f;
         __syncthreads();
+        if (tile + (int)gridDim.z < ntiles) issue(tile + gridDim.z);
         const float* ga = gl + (wco * 32 + m) * P.KPp + kk;
         const float* xb = xl + (wci * 32 + m) * P.HPp;
         for (int ks = 0; ks < P.KP; ks += 2) {
@@ -346,21 +366,23 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_wgrad_f32_kernel(const Wgrad
 #pragma unroll
     for (int t = 0; t < TPW; ++t) {
         if (t >= nkw) continue;
-        f32x16 y[4];
-        if constexpr (MODE == 16) {
-#pragma unroll
-            for (int r = 0; r < 4; ++r) y[r] = acc[t][r];
-        } else {
-            merge_right_grad(acc[t], y);
-        }
         float* d = dst + (long)(kh * P.Kw + kw0 + t) * tap_stride;
 #pragma unroll
-        for (int r = 0; r < 4; ++r)
+        for (int e = 0; e < 16; ++e) {
+            const int co = co_base + 8 * (e >> 2) + (e & 3);
+            float y[4];
+            if constexpr (MODE == 16) {
 #pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                const int co = co_base + 8 * (e >> 2) + (e & 3);
-                d[((long)r * P.CoP + co) * P.CiP + ci] = y[r][e];
+                for (int r = 0; r < 4; ++r) y[r] = acc[t][r][e];
+            } else {
+                float l[8];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) l[i] = acc[t][i][e];
+                merge_right_grad(l, y);
             }
+#pragma unroll
+            for (int r = 0; r < 4; ++r) d[((long)r * P.CoP + co) * P.CiP + ci] = y[r];
+        }
     }
 }
 

@@ -5,6 +5,7 @@
 #include <algorithm>
 #include <cstdio>
 #include <cstring>
+#include <vector>
 
 #include "phx_kernels_f32.h"
 
@@ -12,6 +13,28 @@ namespace phx {
 
 static thread_local const char* g_last_kernel = "";
 static thread_local char g_name_buf[128];
+
+// optional event pairs around the dominant kernel of each call (see phx_profile_enable)
+struct ProfileState {
+    std::vector<hipEvent_t> ev;  // 2 per slot
+    int used = 0;
+    bool on = false;
+};
+static thread_local ProfileState g_prof;
+
+struct KernelTimer {
+    hipStream_t st;
+    int slot;
+    explicit KernelTimer(hipStream_t s) : st(s), slot(-1) {
+        if (g_prof.on && 2 * (g_prof.used + 1) <= (int)g_prof.ev.size()) {
+            slot = g_prof.used++;
+            (void)hipEventRecord(g_prof.ev[2 * slot], st);
+        }
+    }
+    ~KernelTimer() {
+        if (slot >= 0) (void)hipEventRecord(g_prof.ev[2 * slot + 1], st);
+    }
+};
 
 #define PHX_HIP(call)                                              \
     do {                                                           \
@@ -130,17 +153,12 @@ static Corr corr_dgrad(const Problem& p) {
 
 struct FwdPlan {
     int WCO, NTW, BN;
-    int NB, TH, TW, HTH, HTW, HPp, lpr_log2;
+    int NB, TH, TW, HTH, HTW, HP, HPp;
     int tiles_n, tiles_h, tiles_w, co_tiles, nchunks;
     size_t lds_bytes, wpk_bytes;
     int wgs;
 };
 
-static int lpr_for(int row_len) {
-    int l = 3;
-    while (l < 6 && (1 << l) < row_len) ++l;
-    return l;
-}
 
 constexpr int LDS_FLOATS_MAX = 16384;  // 64 KiB: two workgroups per CU
 
@@ -150,7 +168,7 @@ static bool plan_forward(const Corr& c, int mode, FwdPlan& best) {
     for (int wi = 0; wi < 3; ++wi) {
         const int WCO = wcos[wi];
         if (WCO > 1 && 32 * WCO > ((c.Cout + 31) / 32) * 32) continue;
-        for (int NTW = 1; NTW <= 2; ++NTW) {
+        for (int NTW = 1; NTW <= (mode == 16 ? 2 : 1); ++NTW) {  // 8 lanes x 2 column tiles would spill
             const int BN = (4 / WCO) * NTW * 32;
             int cand[16];
             int nc = 0;
@@ -166,7 +184,7 @@ static bool plan_forward(const Corr& c, int mode, FwdPlan& best) {
                     const int HTW = (TW - 1) * c.sw + (c.Kw - 1) * c.dw + 1;
                     const int HP = NB * HTH * HTW;
                     const int HPp = HP;
-                    if (4 * F32_CK * HPp > LDS_FLOATS_MAX) continue;
+                    if (HP > 256) continue;  // one staging position per thread
                     const int tn = cdiv(c.N, NB), th = cdiv(c.Hout, TH), tw = cdiv(c.Wout, TW);
                     const int cot = cdiv(c.Cout, 32 * WCO);
                     const long wgs = (long)tn * th * tw * cot;
@@ -176,7 +194,7 @@ static bool plan_forward(const Corr& c, int mode, FwdPlan& best) {
                     const double score = eff * (0.25 + 0.75 * fill) * (0.9 + 0.1 * halo) * (NTW == 2 ? 1.02 : 1.0);
                     if (score > best_score) {
                         best_score = score;
-                        best = FwdPlan{WCO, NTW, BN, NB, TH, TW, HTH, HTW, HPp, lpr_for(HTW), tn, th, tw, cot,
+                        best = FwdPlan{WCO, NTW, BN, NB, TH, TW, HTH, HTW, HP, HPp, tn, th, tw, cot,
                                        cdiv(c.Cin, F32_CK), (size_t)4 * F32_CK * HPp * sizeof(float), 0, (int)wgs};
                     }
                 }
@@ -197,7 +215,10 @@ static int launch_fwd_variant(const FwdPlan& pl, const ConvArgs& a, hipStream_t 
                            pl.lds_bytes, st, a);                                                                 \
         return PHX_OK;                                                                                           \
     }
-    PHX_CASE(1, 1) PHX_CASE(1, 2) PHX_CASE(2, 1) PHX_CASE(2, 2) PHX_CASE(4, 1) PHX_CASE(4, 2)
+    PHX_CASE(1, 1) PHX_CASE(2, 1) PHX_CASE(4, 1)
+    if constexpr (MODE == 16) {
+        PHX_CASE(1, 2) PHX_CASE(2, 2) PHX_CASE(4, 2)
+    }
 #undef PHX_CASE
     return PHX_ERR_NOT_SUPPORTED;
 }
@@ -225,8 +246,7 @@ static int run_corr(const Problem& p, const Corr& c, int map, hipStream_t st, co
     a.out_cs = (long)c.N * c.Cout * c.Hout * c.Wout;
     a.Cout = c.Cout; a.Hout = c.Hout; a.Wout = c.Wout;
     a.taps = c.Kh * c.Kw; a.Kw = c.Kw; a.dh = c.dh; a.dw = c.dw; a.sh = c.sh; a.sw = c.sw; a.pt = c.pt; a.pl = c.pl;
-    a.NB = pl.NB; a.TH = pl.TH; a.TW = pl.TW; a.HTH = pl.HTH; a.HTW = pl.HTW; a.HPp = pl.HPp;
-    a.lpr_log2 = pl.lpr_log2;
+    a.NB = pl.NB; a.TH = pl.TH; a.TW = pl.TW; a.HTH = pl.HTH; a.HTW = pl.HTW; a.HP = pl.HP; a.HPp = pl.HPp;
     a.tiles_n = pl.tiles_n; a.tiles_h = pl.tiles_h; a.tiles_w = pl.tiles_w; a.co_tiles = pl.co_tiles;
     a.nchunks = pl.nchunks;
 
@@ -236,12 +256,15 @@ static int run_corr(const Problem& p, const Corr& c, int map, hipStream_t st, co
             hipLaunchKernelGGL((pack_filters_f32_kernel<TS, 16, MAP_FWD>), dim3(pack_blocks), dim3(WG_THREADS), 0, st, pa);
         else
             hipLaunchKernelGGL((pack_filters_f32_kernel<TS, 16, MAP_DGRAD>), dim3(pack_blocks), dim3(WG_THREADS), 0, st, pa);
+        KernelTimer timer(st);
         rc = launch_fwd_variant<TS, 16, MAP_FWD>(pl, a, st);  // conjugation lives in the packing
     } else if (map == MAP_FWD) {
         hipLaunchKernelGGL((pack_filters_f32_kernel<TS, 8, MAP_FWD>), dim3(pack_blocks), dim3(WG_THREADS), 0, st, pa);
+        KernelTimer timer(st);
         rc = launch_fwd_variant<TS, 8, MAP_FWD>(pl, a, st);
     } else {
         hipLaunchKernelGGL((pack_filters_f32_kernel<TS, 8, MAP_DGRAD>), dim3(pack_blocks), dim3(WG_THREADS), 0, st, pa);
+        KernelTimer timer(st);
         rc = launch_fwd_variant<TS, 8, MAP_DGRAD>(pl, a, st);
     }
     if (rc != PHX_OK) return rc;
@@ -257,7 +280,7 @@ static int run_corr(const Problem& p, const Corr& c, int map, hipStream_t st, co
 // Filter gradient
 // -------------------------------------------------------------------------------------------
 struct WgPlan {
-    int TPW, NB, TH, TW, KP, KPp, HPp, HTH, HTWmax, lpr_g, lpr_x;
+    int TPW, NB, TH, TW, KP, KPp, HPp, HPx, HTH, HTWmax;
     int tiles_n, tiles_h, tiles_w, co_tiles, ci_tiles, CoP, CiP, groups_per_row, Z;
     size_t lds_bytes, partial_bytes;
 };
@@ -275,16 +298,15 @@ static bool plan_wgrad(const Problem& p, WgPlan& best) {
                 const int KP = (pix + 1) & ~1;
                 const int HTH = (TH - 1) * p.sh + 1;
                 const int HTW = (TW - 1) * p.sw + (nkw - 1) * p.dw + 1;
-                const int KPp = KP | 1, HPp = (NB * HTH * HTW) | 1;
-                if (KPp + HPp + (KP + 255) / 256 > budget) break;
+                const int KPp = KP | 1, HPx = NB * HTH * HTW, HPp = HPx | 1;
+                if (KPp + HPp + (KP + 255) / 256 > budget || KP > 32 || HPx > 32) break;
                 const int tn = cdiv(p.n, NB), th = cdiv(p.ho, TH), tw = cdiv(p.wo, TW);
                 const double eff = ((double)p.n * p.ho * p.wo) / ((double)tn * th * tw * KP);
-                const double score = eff * (1.0 + 0.002 * KP);
+                const double score = eff * (1.0 + 0.002 * KP) * (TW >= std::min(p.wo, 8) ? 1.0 : 0.5);
                 if (score > best_score) {
                     best_score = score;
                     best.TPW = TPW; best.NB = NB; best.TH = TH; best.TW = TW; best.KP = KP; best.KPp = KPp;
-                    best.HPp = HPp; best.HTH = HTH; best.HTWmax = HTW;
-                    best.lpr_g = lpr_for(TW); best.lpr_x = lpr_for(HTW);
+                    best.HPp = HPp; best.HPx = HPx; best.HTH = HTH; best.HTWmax = HTW;
                     best.tiles_n = tn; best.tiles_h = th; best.tiles_w = tw;
                 }
             }
@@ -316,15 +338,18 @@ static int run_wgrad(const Problem& p, hipStream_t st, const void* x, const void
     a.partial = static_cast<float*>(ws);
     a.Kh = p.kh; a.Kw = p.kw; a.sh = p.sh; a.sw = p.sw; a.dh = p.dh; a.dw = p.dw; a.pt = p.pt; a.pl = p.pl;
     a.NB = pl.NB; a.TH = pl.TH; a.TW = pl.TW; a.KP = pl.KP; a.KPp = pl.KPp; a.HPp = pl.HPp; a.HTH = pl.HTH;
-    a.HTWmax = pl.HTWmax; a.lpr_g = pl.lpr_g; a.lpr_x = pl.lpr_x;
+    a.HTWmax = pl.HTWmax; a.HPx = pl.HPx;
     a.tiles_n = pl.tiles_n; a.tiles_h = pl.tiles_h; a.tiles_w = pl.tiles_w;
     a.co_tiles = pl.co_tiles; a.ci_tiles = pl.ci_tiles; a.CoP = pl.CoP; a.CiP = pl.CiP;
     a.groups_per_row = pl.groups_per_row;
     const dim3 grid(pl.co_tiles * pl.ci_tiles, pl.groups_per_row * p.kh, pl.Z);
-    if (p.mode == 16)
-        hipLaunchKernelGGL((qconv_wgrad_f32_kernel<TS, 16, 3>), grid, dim3(WG_THREADS), pl.lds_bytes, st, a);
-    else
-        hipLaunchKernelGGL((qconv_wgrad_f32_kernel<TS, 8, 1>), grid, dim3(WG_THREADS), pl.lds_bytes, st, a);
+    {
+        KernelTimer timer(st);
+        if (p.mode == 16)
+            hipLaunchKernelGGL((qconv_wgrad_f32_kernel<TS, 16, 3>), grid, dim3(WG_THREADS), pl.lds_bytes, st, a);
+        else
+            hipLaunchKernelGGL((qconv_wgrad_f32_kernel<TS, 8, 1>), grid, dim3(WG_THREADS), pl.lds_bytes, st, a);
+    }
     PHX_HIP(hipGetLastError());
     ReduceArgs r;
     r.partial = a.partial; r.dw = dw;
@@ -401,6 +426,31 @@ const char* phx_status_string(int status) {
 }
 
 const char* phx_last_kernel_name(void) { return g_last_kernel; }
+
+int phx_profile_enable(int capacity) {
+    g_prof.on = false;
+    g_prof.used = 0;
+    if (capacity <= 0) return PHX_OK;
+    while ((int)g_prof.ev.size() < 2 * capacity) {
+        hipEvent_t e;
+        PHX_HIP(hipEventCreate(&e));
+        g_prof.ev.push_back(e);
+    }
+    g_prof.on = true;
+    return PHX_OK;
+}
+
+int phx_profile_collect(float* milliseconds, int max_count, int* count) {
+    if (!count || (max_count > 0 && !milliseconds)) return PHX_ERR_INVALID_ARGUMENT;
+    const int n = std::min(g_prof.used, max_count);
+    for (int i = 0; i < n; ++i) {
+        PHX_HIP(hipEventSynchronize(g_prof.ev[2 * i + 1]));
+        PHX_HIP(hipEventElapsedTime(&milliseconds[i], g_prof.ev[2 * i], g_prof.ev[2 * i + 1]));
+    }
+    *count = n;
+    g_prof.used = 0;
+    return PHX_OK;
+}
 
 int phx_qconv2d_output_hw(const phx_qconv_desc* desc, int32_t* ho, int32_t* wo) {
     Problem p;
