@@ -24,7 +24,7 @@ struct ConvArgs {
     int NB, TH, TW;     // output pixels per workgroup tile: images x rows x columns
     int HTH, HTW, HP, HPp;  // halo window, its size and the LDS pitch per staged channel
     int tiles_n, tiles_h, tiles_w, co_tiles;
-    int nchunks;        // ceil(Cin / F32_CK)
+    int nchunks;        // ceil(Cin / CK) for the kernel's chunk size CK
 };
 
 // Forward / input-gradient kernel.
@@ -34,9 +34,8 @@ struct ConvArgs {
 //   lane and K step, prefetched one step ahead); B operand = activations from the LDS halo window.
 //   MODE 16: acc[q] += W_{p^q} * (+-x_p), 16 MFMAs per K step, filters reused across the 4x4 block.
 //   MODE 8 : acc[i] += R_i * L_i with the 8 lanes L_i formed in registers, 8 MFMAs per K step.
-template <typename TS, int MODE, int MAP, int WCO, int NTW>
-__global__ void __launch_bounds__(WG_THREADS) qconv_fwd_f32_kernel(const ConvArgs P) {
-    constexpr int CK = F32_CK;
+template <typename TS, int MODE, int MAP, int WCO, int NTW, int CK, int P2LOG>
+__global__ void __launch_bounds__(WG_THREADS, (MODE == 8 || NTW == 1) ? 2 : 1) qconv_fwd_f32_kernel(const ConvArgs P) {
     constexpr int WPX = 4 / WCO;
     constexpr int NACC = (MODE == 16) ? 4 : 8;
     constexpr int WC = (MODE == 16) ? 4 : 8;  // packed filter values per lane and K step
@@ -87,9 +86,9 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_fwd_f32_kernel(const ConvArg
 
     long step = 0;
     const long cpitch = (long)CK * P.HPp;  // LDS floats between components
-    constexpr int P2LOG = 8;  // one window position per thread, every thread walks all 32 planes
+    // 2^P2LOG window positions, 256 >> P2LOG thread groups sharing the 4*CK planes of a chunk
     const StagePos sp = make_stage_pos<P2LOG>(P.in, n0, h0, w0, P.NB, P.HTH, P.HTW);
-    float stage[4 * CK];
+    float stage[(4 * CK) >> (8 - P2LOG)];
     stage_load<TS, CK, P2LOG>(stage, P.in, sp, 0);
     for (int chunk = 0; chunk < P.nchunks; ++chunk) {
         __syncthreads();
@@ -393,25 +392,47 @@ struct ReduceArgs {
     int Z, Co, Ci, Kh, Kw, CoP, CiP;
 };
 
-// dw(r, co, ci, kh, kw) = sum_z partial[z][tap][r][co][ci], in increasing z (deterministic)
+// dw(r, co, ci, kh, kw) = sum_z partial[z][tap][r][co][ci].  A workgroup owns 32 consecutive
+// outputs; its 8 z-slices each add every 8th partial, then the slices are added in a fixed order,
+// so the result does not depend on scheduling.
 template <typename TS>
 __global__ void __launch_bounds__(WG_THREADS) reduce_wgrad_kernel(const ReduceArgs P) {
+    __shared__ float part[8][33];
     const int taps = P.Kh * P.Kw;
     const long total = 4L * taps * P.Co * P.Ci;
     const long zstride = 4L * taps * P.CoP * P.CiP;
     TS* dw = static_cast<TS*>(P.dw);
-    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
-        const int ci = idx % P.Ci;
-        long s = idx / P.Ci;
-        const int co = s % P.Co;
-        s /= P.Co;
-        const int r = s & 3;
-        const int tap = s >> 2;
+    const int lane = threadIdx.x & 31, slice = threadIdx.x >> 5;
+    const long idx = (long)blockIdx.x * 32 + lane;
+    float sum = 0.f;
+    int ci = 0, co = 0, r = 0, tap = 0;
+    if (idx < total) {
+        ci = idx % P.Ci;
+        long t = idx / P.Ci;
+        co = t % P.Co;
+        t /= P.Co;
+        r = t & 3;
+        tap = t >> 2;
         const float* src = P.partial + (((long)tap * 4 + r) * P.CoP + co) * P.CiP + ci;
-        float sum = 0.f;
-        for (int z = 0; z < P.Z; ++z) sum += src[z * zstride];
+        float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+        int z = slice;
+        for (; z + 24 < P.Z; z += 32) {
+            s0 += src[(long)z * zstride];
+            s1 += src[(long)(z + 8) * zstride];
+            s2 += src[(long)(z + 16) * zstride];
+            s3 += src[(long)(z + 24) * zstride];
+        }
+        for (; z < P.Z; z += 8) s0 += src[(long)z * zstride];
+        sum = (s0 + s1) + (s2 + s3);
+    }
+    part[slice][lane] = sum;
+    __syncthreads();
+    if (slice == 0 && idx < total) {
+        float v = part[0][lane];
+#pragma unroll
+        for (int k = 1; k < 8; ++k) v += part[k][lane];
         const int kh = tap / P.Kw, kw = tap - kh * P.Kw;
-        stf<TS>(dw + r * P.wcs + co * P.so + ci * P.si + kh * P.skh + kw * P.skw, sum);
+        stf<TS>(dw + r * P.wcs + co * P.so + ci * P.si + kh * P.skh + kw * P.skw, v);
     }
 }
 

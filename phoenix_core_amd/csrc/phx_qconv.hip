@@ -153,6 +153,7 @@ static Corr corr_dgrad(const Problem& p) {
 
 struct FwdPlan {
     int WCO, NTW, BN;
+    int CK, P2LOG;           // channels per chunk and log2 staging positions of the kernel variant
     int NB, TH, TW, HTH, HTW, HP, HPp;
     int tiles_n, tiles_h, tiles_w, co_tiles, nchunks;
     size_t lds_bytes, wpk_bytes;
@@ -194,31 +195,47 @@ static bool plan_forward(const Corr& c, int mode, FwdPlan& best) {
                     const double score = eff * (0.25 + 0.75 * fill) * (0.9 + 0.1 * halo) * (NTW == 2 ? 1.02 : 1.0);
                     if (score > best_score) {
                         best_score = score;
-                        best = FwdPlan{WCO, NTW, BN, NB, TH, TW, HTH, HTW, HP, HPp, tn, th, tw, cot,
-                                       cdiv(c.Cin, F32_CK), (size_t)4 * F32_CK * HPp * sizeof(float), 0, (int)wgs};
+                        best.WCO = WCO; best.NTW = NTW; best.BN = BN;
+                        best.NB = NB; best.TH = TH; best.TW = TW; best.HTH = HTH; best.HTW = HTW;
+                        best.HP = HP; best.HPp = HPp;
+                        best.tiles_n = tn; best.tiles_h = th; best.tiles_w = tw; best.co_tiles = cot;
+                        best.wgs = (int)wgs;
                     }
                 }
             }
         }
     }
     if (best_score < 0) return false;
+    // kernel variant: pointwise problems are bandwidth/latency bound and take as many channels per
+    // chunk as 32 staging registers per thread allow; everything else uses 8-channel chunks
+    best.CK = F32_CK; best.P2LOG = 8;
+    if (c.Kh == 1 && c.Kw == 1 && c.Cin >= 32) {
+        if (best.HP <= 64) { best.CK = 32; best.P2LOG = 6; }
+        else if (best.HP <= 128) { best.CK = 16; best.P2LOG = 7; }
+    }
+    best.nchunks = cdiv(c.Cin, best.CK);
+    best.lds_bytes = (size_t)4 * best.CK * best.HPp * sizeof(float);
     const int WC = (mode == 16) ? 4 : 8;
-    best.wpk_bytes = (size_t)best.co_tiles * best.WCO * best.nchunks * c.Kh * c.Kw * 4 * 64 * WC * sizeof(float);
+    // packed in 8-channel groups: nchunks * CK/8 groups per filter tile
+    best.wpk_bytes = (size_t)best.co_tiles * best.WCO * best.nchunks * (best.CK / F32_CK) * c.Kh * c.Kw * 4 * 64 * WC *
+                     sizeof(float);
     return true;
 }
 
 template <typename TS, int MODE, int MAP>
 static int launch_fwd_variant(const FwdPlan& pl, const ConvArgs& a, hipStream_t st) {
-#define PHX_CASE(WCO_, NTW_)                                                                                     \
-    if (pl.WCO == WCO_ && pl.NTW == NTW_) {                                                                      \
-        hipLaunchKernelGGL((qconv_fwd_f32_kernel<TS, MODE, MAP, WCO_, NTW_>), dim3(pl.wgs), dim3(WG_THREADS),    \
-                           pl.lds_bytes, st, a);                                                                 \
+#define PHX_CASE(WCO_, NTW_, CK_, P2_)                                                                           \
+    if (pl.WCO == WCO_ && pl.NTW == NTW_ && pl.CK == CK_ && pl.P2LOG == P2_) {                                   \
+        hipLaunchKernelGGL((qconv_fwd_f32_kernel<TS, MODE, MAP, WCO_, NTW_, CK_, P2_>), dim3(pl.wgs),            \
+                           dim3(WG_THREADS), pl.lds_bytes, st, a);                                               \
         return PHX_OK;                                                                                           \
     }
-    PHX_CASE(1, 1) PHX_CASE(2, 1) PHX_CASE(4, 1)
+#define PHX_CASES(WCO_, NTW_) PHX_CASE(WCO_, NTW_, 8, 8) PHX_CASE(WCO_, NTW_, 16, 7) PHX_CASE(WCO_, NTW_, 32, 6)
+    PHX_CASES(1, 1) PHX_CASES(2, 1) PHX_CASES(4, 1)
     if constexpr (MODE == 16) {
-        PHX_CASE(1, 2) PHX_CASE(2, 2) PHX_CASE(4, 2)
+        PHX_CASES(1, 2) PHX_CASES(2, 2) PHX_CASES(4, 2)
     }
+#undef PHX_CASES
 #undef PHX_CASE
     return PHX_ERR_NOT_SUPPORTED;
 }
@@ -235,7 +252,7 @@ static int run_corr(const Problem& p, const Corr& c, int map, hipStream_t st, co
     pa.w = w; pa.out = wpk;
     pa.wcs = p.fs.wcs; pa.so = p.fs.so; pa.si = p.fs.si; pa.skh = p.fs.skh; pa.skw = p.fs.skw;
     pa.Co = p.co; pa.Ci = p.ci; pa.Kh = p.kh; pa.Kw = p.kw;
-    pa.rows = c.Cout; pa.red = c.Cin; pa.row_tiles = pl.co_tiles * pl.WCO; pa.nchunks = pl.nchunks;
+    pa.rows = c.Cout; pa.red = c.Cin; pa.row_tiles = pl.co_tiles * pl.WCO; pa.nchunks = pl.nchunks * (pl.CK / F32_CK);
     const long pack_items = (long)pa.row_tiles * pa.nchunks * p.kh * p.kw * 4 * 64;
     const int pack_blocks = (int)std::min<long>((pack_items + WG_THREADS - 1) / WG_THREADS, 4096);
 
@@ -269,9 +286,9 @@ static int run_corr(const Problem& p, const Corr& c, int map, hipStream_t st, co
     }
     if (rc != PHX_OK) return rc;
     PHX_HIP(hipGetLastError());
-    snprintf(g_name_buf, sizeof(g_name_buf), "qconv_%s_f32mfma_p%d_%s_wco%d_ntw%d_tile%dx%dx%d",
-             map == MAP_FWD ? "fwd" : "dgrad", p.mode, sizeof(TS) == 4 ? "f32" : "f16", pl.WCO, pl.NTW, pl.NB, pl.TH,
-             pl.TW);
+    snprintf(g_name_buf, sizeof(g_name_buf), "qconv_%s_f32mfma_p%d_%s_wco%d_ntw%d_ck%d_tile%dx%dx%d",
+             map == MAP_FWD ? "fwd" : "dgrad", p.mode, sizeof(TS) == 4 ? "f32" : "f16", pl.WCO, pl.NTW, pl.CK, pl.NB,
+             pl.TH, pl.TW);
     g_last_kernel = g_name_buf;
     return PHX_OK;
 }
@@ -356,7 +373,7 @@ static int run_wgrad(const Problem& p, hipStream_t st, const void* x, const void
     r.wcs = p.fs.wcs; r.so = p.fs.so; r.si = p.fs.si; r.skh = p.fs.skh; r.skw = p.fs.skw;
     r.Z = pl.Z; r.Co = p.co; r.Ci = p.ci; r.Kh = p.kh; r.Kw = p.kw; r.CoP = pl.CoP; r.CiP = pl.CiP;
     const long items = 4L * p.kh * p.kw * p.co * p.ci;
-    const int blocks = (int)std::min<long>((items + WG_THREADS - 1) / WG_THREADS, 8192);
+    const int blocks = (int)((items + 31) / 32);
     hipLaunchKernelGGL((reduce_wgrad_kernel<TS>), dim3(blocks), dim3(WG_THREADS), 0, st, r);
     PHX_HIP(hipGetLastError());
     snprintf(g_name_buf, sizeof(g_name_buf), "qconv_wgrad_f32mfma_p%d_%s_tile%dx%dx%d_z%d", p.mode,
