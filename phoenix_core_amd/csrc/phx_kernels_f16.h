@@ -1,0 +1,237 @@
+// fp16-MFMA kernels (v_mfma_f32_32x32x16_f16, fp32 accumulation) for fp16 tensors: quaternion
+// convolution forward / input-gradient in the 16-product and the factorized 8-product formulation.
+#pragma once
+
+#include "phx_kernels_f32.h"
+
+namespace phx {
+
+// Staged layout: unit u = p*2 + kp (component p, 8-channel pack kp) holds one 16-byte entry per
+// window position, lds[u*pitch + pos] = {x_p[c0 + kp*8 + 0..7]} at that position.  NCHW keeps the
+// channels of one pixel HW elements apart, so the transposition happens here: every thread gathers
+// the 8 channels of a pack for its own position and writes them with one 16-byte LDS store; the
+// MFMA B operand (lane = pixel, 8 consecutive K values) is then a single aligned 16-byte LDS read.
+template <int P2LOG>
+__device__ __forceinline__ void stage_load16(f16x8 (&v)[8 >> (8 - P2LOG)], const TileSrc& s, const StagePos& sp,
+                                             int c0) {
+    constexpr int G = WG_THREADS >> P2LOG;
+    constexpr int E = 8 / G;
+    const _Float16* origin = static_cast<const _Float16*>(s.base);
+    const long plane = (long)s.Hd * s.Wd;
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+        const int u = e * G + sp.group;
+        const int p = u >> 1, kp = u & 1;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int c = c0 + kp * 8 + i;
+            const bool ok = sp.valid && c < s.C;
+            const _Float16* ptr = ok ? origin + sp.goff + p * s.comp_stride + (long)c * plane : origin;
+            const _Float16 t = *ptr;
+            v[e][i] = ok ? t : (_Float16)0;
+        }
+    }
+}
+
+template <int P2LOG>
+__device__ __forceinline__ void stage_store16(f16x8* dst, const f16x8 (&v)[8 >> (8 - P2LOG)], const StagePos& sp,
+                                              int HP, int pitch) {
+    constexpr int G = WG_THREADS >> P2LOG;
+    constexpr int E = 8 / G;
+    if (sp.pos < HP) {
+#pragma unroll
+        for (int e = 0; e < E; ++e) dst[(e * G + sp.group) * pitch + sp.pos] = v[e];
+    }
+}
+
+// Same tiling as qconv_fwd_f32_kernel: 4 waves = WCO filter sub-tiles (32 output channels) x
+// 4/WCO pixel ranges, NTW column tiles of 32 pixels per wave, all four output components per wave.
+// One K step is a whole 16-channel chunk at one filter tap.
+//   MODE 16: 16 MFMAs per step and column tile, the four filter components reused across the
+//            4x4 block, negative entries by flipping the sign bits of the activation operand.
+//   MODE 8 : 8 MFMAs per step and column tile on lanes formed with packed fp16 adds.
+template <int MODE, int MAP, int WCO, int NTW, int P2LOG>
+__global__ void __launch_bounds__(WG_THREADS, (MODE == 8 || NTW == 1) ? 2 : 1) qconv_fwd_f16_kernel(const ConvArgs P) {
+    constexpr int CK = F16_CK;
+    constexpr int WPX = 4 / WCO;
+    constexpr int NACC = (MODE == 16) ? 4 : 8;
+    constexpr int WC = (MODE == 16) ? 4 : 8;  // packed 16-byte filter vectors per lane and K step
+    extern __shared__ f16x8 lds16[];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wco = wave % WCO, wpx = wave / WCO;
+    const int j = lane & 31, kk = lane >> 5;
+
+    int bid = xcd_remap(blockIdx.x, gridDim.x);
+    const int ct = bid % P.co_tiles;
+    bid /= P.co_tiles;
+    const int tw = bid % P.tiles_w;
+    bid /= P.tiles_w;
+    const int th = bid % P.tiles_h;
+    const int tn = bid / P.tiles_h;
+    const int n0 = tn * P.NB, ho0 = th * P.TH, wo0 = tw * P.TW;
+    const int h0 = ho0 * P.sh - P.pt, w0 = wo0 * P.sw - P.pl;
+
+    int poff[NTW];
+    long oaddr[NTW];
+    bool pvalid[NTW];
+    const int thw = P.TH * P.TW;
+#pragma unroll
+    for (int t = 0; t < NTW; ++t) {
+        const int pix = (wpx * NTW + t) * 32 + j;
+        const int nb = pix / thw, rem = pix - nb * thw;
+        const int r = rem / P.TW, c = rem - r * P.TW;
+        pvalid[t] = nb < P.NB && (n0 + nb) < P.in.N && (ho0 + r) < P.Hout && (wo0 + c) < P.Wout;
+        poff[t] = pvalid[t] ? (nb * P.HTH + r * P.sh) * P.HTW + c * P.sw : 0;
+        oaddr[t] = ((long)(n0 + nb) * P.Cout * P.Hout + (ho0 + r)) * P.Wout + (wo0 + c);
+    }
+
+    f32x16 acc[NTW][NACC];
+#pragma unroll
+    for (int t = 0; t < NTW; ++t)
+#pragma unroll
+        for (int a = 0; a < NACC; ++a)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[t][a][r] = 0.f;
+
+    const long nsteps = (long)P.nchunks * P.taps;
+    const f16x8* wptr = static_cast<const f16x8*>(P.wpk) + ((long)(ct * WCO + wco) * nsteps * 64 + lane) * WC;
+    f16x8 wcur[WC], wnext[WC];
+#pragma unroll
+    for (int v = 0; v < WC; ++v) wcur[v] = wptr[v];
+
+    long step = 0;
+    const StagePos sp = make_stage_pos<P2LOG>(P.in, n0, h0, w0, P.NB, P.HTH, P.HTW);
+    f16x8 stage[8 >> (8 - P2LOG)];
+    stage_load16<P2LOG>(stage, P.in, sp, 0);
+    for (int chunk = 0; chunk < P.nchunks; ++chunk) {
+        __syncthreads();
+        stage_store16<P2LOG>(lds16, stage, sp, P.HP, P.HPp);
+        __syncthreads();
+        if (chunk + 1 < P.nchunks) stage_load16<P2LOG>(stage, P.in, sp, (chunk + 1) * CK);
+        int kh = 0, kw = 0;
+        for (int tap = 0; tap < P.taps; ++tap) {
+            const int tapoff = kh * P.dh * P.HTW + kw * P.dw;
+            const long nxt = (step + 1 < nsteps) ? step + 1 : step;
+#pragma unroll
+            for (int v = 0; v < WC; ++v) wnext[v] = wptr[nxt * (64 * WC) + v];
+            const f16x8* xb = lds16 + kk * P.HPp + tapoff;
+#pragma unroll
+            for (int t = 0; t < NTW; ++t) {
+                f16x8 x[4];
+#pragma unroll
+                for (int p = 0; p < 4; ++p) x[p] = xb[p * 2 * P.HPp + poff[t]];
+                if constexpr (MODE == 16) {
+                    f16x8 nx[4];
+#pragma unroll
+                    for (int p = 0; p < 4; ++p) nx[p] = -x[p];
+#pragma unroll
+                    for (int p = 0; p < 4; ++p)
+#pragma unroll
+                        for (int q = 0; q < 4; ++q)
+                            acc[t][q] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wcur[p ^ q], qneg(p, q) ? nx[p] : x[p],
+                                                                               acc[t][q], 0, 0, 0);
+                } else {
+                    f16x8 L[8];
+                    if constexpr (MAP == MAP_FWD) lanes_left(x, L);
+                    else lanes_grad(x, L, (_Float16)0.5f);
+#pragma unroll
+                    for (int i = 0; i < 8; ++i)
+                        acc[t][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wcur[i], L[i], acc[t][i], 0, 0, 0);
+                }
+            }
+#pragma unroll
+            for (int v = 0; v < WC; ++v) wcur[v] = wnext[v];
+            ++step;
+            if (++kw == P.Kw) { kw = 0; ++kh; }
+        }
+    }
+
+    _Float16* out = static_cast<_Float16*>(P.out);
+    const _Float16* bias = static_cast<const _Float16*>(P.bias);
+    const long plane = (long)P.Hout * P.Wout;
+    const int co_base = (ct * WCO + wco) * 32 + 4 * kk;
+#pragma unroll
+    for (int t = 0; t < NTW; ++t) {
+        if (!pvalid[t]) continue;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int co = co_base + 8 * (r >> 2) + (r & 3);
+            float y[4];
+            if constexpr (MODE == 16) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) y[q] = acc[t][q][r];
+            } else {
+                float l[8];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) l[i] = acc[t][i][r];
+                if constexpr (MAP == MAP_FWD) merge_output(l, y);
+                else merge_left_grad(l, y);
+            }
+            if (co < P.Cout) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    float v = y[q];
+                    if (bias) v += (float)bias[q * P.Cout + co];
+                    out[q * P.out_cs + oaddr[t] + co * plane] = (_Float16)v;
+                }
+            }
+        }
+    }
+}
+
+// Filter packing for the kernel above: one group of WC 16-byte vectors per (32-channel filter
+// tile, K step, lane); lane = (row = lane % 32, kk = lane / 32), K step = chunk*taps + tap,
+// vector element i = reduced channel chunk*16 + kk*8 + i.  MODE 16: the four filter components
+// (conjugated for MAP_DGRAD); MODE 8: the eight right-operand lanes, formed in fp32 and rounded once.
+template <int MODE, int MAP>
+__global__ void __launch_bounds__(WG_THREADS) pack_filters_f16_kernel(const PackArgs P) {
+    constexpr int WC = (MODE == 16) ? 4 : 8;
+    const int taps = P.Kh * P.Kw;
+    const long total = (long)P.row_tiles * P.nchunks * taps * 64;
+    const _Float16* w = static_cast<const _Float16*>(P.w);
+    f16x8* outv = reinterpret_cast<f16x8*>(P.out);
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
+        const int lane = idx & 63;
+        long s = idx >> 6;
+        const int tap = s % taps;
+        s /= taps;
+        const int chunk = s % P.nchunks;
+        const int tile = s / P.nchunks;
+        const int row = tile * 32 + (lane & 31);
+        int kh = tap / P.Kw, kw = tap - kh * P.Kw;
+        if (MAP == MAP_DGRAD) {
+            kh = P.Kh - 1 - kh;
+            kw = P.Kw - 1 - kw;
+        }
+        f16x8 vec[WC];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int red = chunk * F16_CK + (lane >> 5) * 8 + i;
+            float wv[4] = {0.f, 0.f, 0.f, 0.f};
+            if (row < P.rows && red < P.red) {
+                const int o = (MAP == MAP_DGRAD) ? red : row;
+                const int in = (MAP == MAP_DGRAD) ? row : red;
+                const long off = o * P.so + in * P.si + kh * P.skh + kw * P.skw;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) wv[r] = (float)w[r * P.wcs + off];
+            }
+            if constexpr (MODE == 16) {
+                const float sgn = (MAP == MAP_DGRAD) ? -1.f : 1.f;
+                vec[0][i] = (_Float16)wv[0];
+                vec[1][i] = (_Float16)(sgn * wv[1]);
+                vec[2][i] = (_Float16)(sgn * wv[2]);
+                vec[3][i] = (_Float16)(sgn * wv[3]);
+            } else {
+                float R[8];
+                lanes_right(wv, R);
+#pragma unroll
+                for (int l = 0; l < 8; ++l) vec[l][i] = (_Float16)R[l];
+            }
+        }
+#pragma unroll
+        for (int v = 0; v < WC; ++v) outv[idx * WC + v] = vec[v];
+    }
+}
+
+}  // namespace phx

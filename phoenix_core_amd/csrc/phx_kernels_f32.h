@@ -9,11 +9,12 @@ namespace phx {
 
 enum { MAP_FWD = 0, MAP_DGRAD = 1 };
 
-constexpr int F32_CK = 8;  // input channels staged per K chunk (4 MFMA k-pairs)
+constexpr int F32_CK = 8;   // fp32 MFMA: input channels per K chunk (4 MFMA k-pairs)
+constexpr int F16_CK = 16;  // fp16 MFMA: input channels per K chunk = one MFMA K step (two 8-channel packs)
 
 struct ConvArgs {
     TileSrc in;         // x (forward) or the output gradient (input-gradient pass)
-    const float* wpk;   // packed filters, see pack_filters_f32
+    const void* wpk;    // packed filters (see the pack_filters kernels), in the MFMA operand type
     const void* bias;   // [4][Cout] in storage type or null
     void* out;
     long out_cs;        // elements between output components
@@ -79,7 +80,7 @@ __global__ void __launch_bounds__(WG_THREADS, (MODE == 8 || NTW == 1) ? 2 : 1) q
 
     const int steps_per_chunk = P.taps * (CK / 2);
     const long nsteps = (long)P.nchunks * steps_per_chunk;
-    const float* wptr = P.wpk + ((long)(ct * WCO + wco) * nsteps * 64 + lane) * WC;
+    const float* wptr = static_cast<const float*>(P.wpk) + ((long)(ct * WCO + wco) * nsteps * 64 + lane) * WC;
     f32x4 wcur[WC / 4], wnext[WC / 4];
 #pragma unroll
     for (int v = 0; v < WC / 4; ++v) wcur[v] = *reinterpret_cast<const f32x4*>(wptr + 4 * v);
@@ -181,7 +182,7 @@ __global__ void __launch_bounds__(WG_THREADS, (MODE == 8 || NTW == 1) ? 2 : 1) q
 // Filter element (r, o, i, kh, kw) lives at r*wcs + o*so + i*si + kh*skh + kw*skw.
 struct PackArgs {
     const void* w;
-    float* out;
+    void* out;
     long wcs, so, si, skh, skw;
     int Co, Ci;       // filter dims of the convolution (not of the correlation being run)
     int Kh, Kw;
@@ -220,7 +221,7 @@ __global__ void __launch_bounds__(WG_THREADS) pack_filters_f32_kernel(const Pack
 #pragma unroll
             for (int r = 0; r < 4; ++r) wv[r] = ldf<TS>(w + r * P.wcs + off);
         }
-        float* dst = P.out + idx * WC;
+        float* dst = static_cast<float*>(P.out) + idx * WC;
         if constexpr (MODE == 16) {
             const float sgn = (MAP == MAP_DGRAD) ? -1.f : 1.f;
             dst[0] = wv[0];

@@ -1,0 +1,27 @@
+// Host-side launch interface between the C ABI translation unit and the translation units that
+// instantiate the kernel templates (split so that they compile in parallel).
+#pragma once
+
+#include "phx_kernels_f32.h"
+
+namespace phx {
+
+// which instantiation of the forward / input-gradient kernel to run
+struct FwdVariant {
+    bool half_storage;  // tensors are fp16 (else fp32)
+    bool f16_mfma;      // fp16 matrix-core arithmetic (else fp32)
+    int mode, map;      // 16 / 8, MAP_FWD / MAP_DGRAD
+    int WCO, NTW, CK, P2LOG;
+    int wgs;
+    size_t lds_bytes;
+};
+
+int launch_pack_filters(const FwdVariant& v, const PackArgs& a, int blocks, hipStream_t st);
+int launch_fwd_f32(const FwdVariant& v, const ConvArgs& a, hipStream_t st);
+int launch_fwd_f16(const FwdVariant& v, const ConvArgs& a, hipStream_t st);
+int launch_pack_filters_f16(const FwdVariant& v, const PackArgs& a, int blocks, hipStream_t st);
+
+int launch_wgrad_f32(bool half_storage, int mode, const WgradArgs& a, dim3 grid, size_t lds_bytes, hipStream_t st);
+int launch_reduce_wgrad(bool half_storage, const ReduceArgs& a, int blocks, hipStream_t st);
+
+}  // namespace phx

@@ -1,0 +1,40 @@
+// Instantiations of the fp16-MFMA forward / input-gradient kernels and their filter packing.
+#include "phx_kernels_f16.h"
+#include "phx_launch.h"
+
+namespace phx {
+
+template <int MODE, int MAP>
+static int launch_variant16(const FwdVariant& v, const ConvArgs& a, hipStream_t st) {
+#define PHX_CASE(WCO_, NTW_, P2_)                                                                             \
+    if (v.WCO == WCO_ && v.NTW == NTW_ && v.P2LOG == P2_) {                                                   \
+        hipLaunchKernelGGL((qconv_fwd_f16_kernel<MODE, MAP, WCO_, NTW_, P2_>), dim3(v.wgs), dim3(WG_THREADS), \
+                           v.lds_bytes, st, a);                                                               \
+        return 0;                                                                                             \
+    }
+#define PHX_CASES(WCO_, NTW_) PHX_CASE(WCO_, NTW_, 8) PHX_CASE(WCO_, NTW_, 7)
+    PHX_CASES(1, 1) PHX_CASES(2, 1) PHX_CASES(4, 1)
+    if constexpr (MODE == 16) {
+        PHX_CASES(1, 2) PHX_CASES(2, 2) PHX_CASES(4, 2)
+    }
+#undef PHX_CASES
+#undef PHX_CASE
+    return -1;
+}
+
+int launch_fwd_f16(const FwdVariant& v, const ConvArgs& a, hipStream_t st) {
+    if (v.mode == 16) return launch_variant16<16, MAP_FWD>(v, a, st);
+    if (v.map == MAP_FWD) return launch_variant16<8, MAP_FWD>(v, a, st);
+    return launch_variant16<8, MAP_DGRAD>(v, a, st);
+}
+
+int launch_pack_filters_f16(const FwdVariant& v, const PackArgs& a, int blocks, hipStream_t st) {
+    const dim3 g(blocks), b(WG_THREADS);
+    if (v.mode == 16 && v.map == MAP_FWD) hipLaunchKernelGGL((pack_filters_f16_kernel<16, MAP_FWD>), g, b, 0, st, a);
+    else if (v.mode == 16) hipLaunchKernelGGL((pack_filters_f16_kernel<16, MAP_DGRAD>), g, b, 0, st, a);
+    else if (v.map == MAP_FWD) hipLaunchKernelGGL((pack_filters_f16_kernel<8, MAP_FWD>), g, b, 0, st, a);
+    else hipLaunchKernelGGL((pack_filters_f16_kernel<8, MAP_DGRAD>), g, b, 0, st, a);
+    return 0;
+}
+
+}  // namespace phx

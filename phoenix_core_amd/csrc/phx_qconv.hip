@@ -7,7 +7,7 @@
 #include <cstring>
 #include <vector>
 
-#include "phx_kernels_f32.h"
+#include "phx_launch.h"
 
 namespace phx {
 
@@ -163,7 +163,7 @@ struct FwdPlan {
 
 constexpr int LDS_FLOATS_MAX = 16384;  // 64 KiB: two workgroups per CU
 
-static bool plan_forward(const Corr& c, int mode, FwdPlan& best) {
+static bool plan_forward(const Corr& c, int mode, bool f16mfma, FwdPlan& best) {
     double best_score = -1.0;
     const int wcos[3] = {1, 2, 4};
     for (int wi = 0; wi < 3; ++wi) {
@@ -206,60 +206,64 @@ static bool plan_forward(const Corr& c, int mode, FwdPlan& best) {
         }
     }
     if (best_score < 0) return false;
-    // kernel variant: pointwise problems are bandwidth/latency bound and take as many channels per
+    const int WC = (mode == 16) ? 4 : 8;
+    const int taps = c.Kh * c.Kw;
+    if (f16mfma) {
+        // fp16 MFMA: 16-channel chunks, one 16-byte LDS entry per (component, 8-channel pack, position)
+        best.CK = F16_CK;
+        best.P2LOG = best.HP <= 128 ? 7 : 8;
+        best.nchunks = cdiv(c.Cin, best.CK);
+        best.lds_bytes = (size_t)8 * best.HPp * 16;
+        best.wpk_bytes = (size_t)best.co_tiles * best.WCO * best.nchunks * taps * 64 * WC * 16;
+        return true;
+    }
+    // fp32 MFMA: pointwise problems are bandwidth/latency bound and take as many channels per
     // chunk as 32 staging registers per thread allow; everything else uses 8-channel chunks
     best.CK = F32_CK; best.P2LOG = 8;
-    if (c.Kh == 1 && c.Kw == 1 && c.Cin >= 32) {
+    if (taps == 1 && c.Cin >= 32) {
         if (best.HP <= 64) { best.CK = 32; best.P2LOG = 6; }
         else if (best.HP <= 128) { best.CK = 16; best.P2LOG = 7; }
     }
     best.nchunks = cdiv(c.Cin, best.CK);
     best.lds_bytes = (size_t)4 * best.CK * best.HPp * sizeof(float);
-    const int WC = (mode == 16) ? 4 : 8;
     // packed in 8-channel groups: nchunks * CK/8 groups per filter tile
-    best.wpk_bytes = (size_t)best.co_tiles * best.WCO * best.nchunks * (best.CK / F32_CK) * c.Kh * c.Kw * 4 * 64 * WC *
+    best.wpk_bytes = (size_t)best.co_tiles * best.WCO * best.nchunks * (best.CK / F32_CK) * taps * 4 * 64 * WC *
                      sizeof(float);
     return true;
 }
 
-template <typename TS, int MODE, int MAP>
-static int launch_fwd_variant(const FwdPlan& pl, const ConvArgs& a, hipStream_t st) {
-#define PHX_CASE(WCO_, NTW_, CK_, P2_)                                                                           \
-    if (pl.WCO == WCO_ && pl.NTW == NTW_ && pl.CK == CK_ && pl.P2LOG == P2_) {                                   \
-        hipLaunchKernelGGL((qconv_fwd_f32_kernel<TS, MODE, MAP, WCO_, NTW_, CK_, P2_>), dim3(pl.wgs),            \
-                           dim3(WG_THREADS), pl.lds_bytes, st, a);                                               \
-        return PHX_OK;                                                                                           \
-    }
-#define PHX_CASES(WCO_, NTW_) PHX_CASE(WCO_, NTW_, 8, 8) PHX_CASE(WCO_, NTW_, 16, 7) PHX_CASE(WCO_, NTW_, 32, 6)
-    PHX_CASES(1, 1) PHX_CASES(2, 1) PHX_CASES(4, 1)
-    if constexpr (MODE == 16) {
-        PHX_CASES(1, 2) PHX_CASES(2, 2) PHX_CASES(4, 2)
-    }
-#undef PHX_CASES
-#undef PHX_CASE
-    return PHX_ERR_NOT_SUPPORTED;
+// fp16 tensors use fp16 matrix-core arithmetic where UPSTRIDE_CONV_FP16_POLICY allows it for the
+// pass (forward: full16 or backward32; backward: full16 only), fp32 arithmetic otherwise
+static bool use_f16_mfma(const Problem& p, int pass) {
+    if (p.dtype != PHX_F16) return false;
+    if (pass == PHX_PASS_FWD) return p.policy == PHX_FP16_FULL16 || p.policy == PHX_FP16_BACKWARD32;
+    return p.policy == PHX_FP16_FULL16;
 }
 
-template <typename TS>
 static int run_corr(const Problem& p, const Corr& c, int map, hipStream_t st, const void* in, const void* w,
                     const void* bias, void* out, void* ws, size_t ws_bytes) {
+    const bool f16 = use_f16_mfma(p, map == MAP_FWD ? PHX_PASS_FWD : PHX_PASS_BWD_DATA);
     FwdPlan pl;
-    if (!plan_forward(c, p.mode, pl)) return PHX_ERR_NOT_SUPPORTED;
+    if (!plan_forward(c, p.mode, f16, pl)) return PHX_ERR_NOT_SUPPORTED;
     if (ws_bytes < pl.wpk_bytes || !ws) return PHX_ERR_WORKSPACE;
-    float* wpk = static_cast<float*>(ws);
+
+    FwdVariant v;
+    v.half_storage = p.dtype == PHX_F16; v.f16_mfma = f16; v.mode = p.mode; v.map = map;
+    v.WCO = pl.WCO; v.NTW = pl.NTW; v.CK = pl.CK; v.P2LOG = pl.P2LOG; v.wgs = pl.wgs; v.lds_bytes = pl.lds_bytes;
 
     PackArgs pa;
-    pa.w = w; pa.out = wpk;
+    pa.w = w; pa.out = ws;
     pa.wcs = p.fs.wcs; pa.so = p.fs.so; pa.si = p.fs.si; pa.skh = p.fs.skh; pa.skw = p.fs.skw;
     pa.Co = p.co; pa.Ci = p.ci; pa.Kh = p.kh; pa.Kw = p.kw;
-    pa.rows = c.Cout; pa.red = c.Cin; pa.row_tiles = pl.co_tiles * pl.WCO; pa.nchunks = pl.nchunks * (pl.CK / F32_CK);
-    const long pack_items = (long)pa.row_tiles * pa.nchunks * p.kh * p.kw * 4 * 64;
+    pa.rows = c.Cout; pa.red = c.Cin; pa.row_tiles = pl.co_tiles * pl.WCO;
+    pa.nchunks = f16 ? pl.nchunks : pl.nchunks * (pl.CK / F32_CK);
+    const long pack_items = (long)pa.row_tiles * pa.nchunks * p.kh * p.kw * (f16 ? 1 : 4) * 64;
     const int pack_blocks = (int)std::min<long>((pack_items + WG_THREADS - 1) / WG_THREADS, 4096);
 
     ConvArgs a;
     a.in.base = in; a.in.comp_stride = (long)c.N * c.Cin * c.Hin * c.Win;
     a.in.N = c.N; a.in.C = c.Cin; a.in.Hd = c.Hin; a.in.Wd = c.Win; a.in.uh = c.uh; a.in.uw = c.uw;
-    a.wpk = wpk; a.bias = bias; a.out = out;
+    a.wpk = ws; a.bias = bias; a.out = out;
     a.out_cs = (long)c.N * c.Cout * c.Hout * c.Wout;
     a.Cout = c.Cout; a.Hout = c.Hout; a.Wout = c.Wout;
     a.taps = c.Kh * c.Kw; a.Kw = c.Kw; a.dh = c.dh; a.dw = c.dw; a.sh = c.sh; a.sw = c.sw; a.pt = c.pt; a.pl = c.pl;
@@ -267,28 +271,17 @@ static int run_corr(const Problem& p, const Corr& c, int map, hipStream_t st, co
     a.tiles_n = pl.tiles_n; a.tiles_h = pl.tiles_h; a.tiles_w = pl.tiles_w; a.co_tiles = pl.co_tiles;
     a.nchunks = pl.nchunks;
 
-    int rc;
-    if (p.mode == 16) {
-        if (map == MAP_FWD)
-            hipLaunchKernelGGL((pack_filters_f32_kernel<TS, 16, MAP_FWD>), dim3(pack_blocks), dim3(WG_THREADS), 0, st, pa);
-        else
-            hipLaunchKernelGGL((pack_filters_f32_kernel<TS, 16, MAP_DGRAD>), dim3(pack_blocks), dim3(WG_THREADS), 0, st, pa);
+    int rc = f16 ? launch_pack_filters_f16(v, pa, pack_blocks, st) : launch_pack_filters(v, pa, pack_blocks, st);
+    if (rc != 0) return PHX_ERR_NOT_SUPPORTED;
+    {
         KernelTimer timer(st);
-        rc = launch_fwd_variant<TS, 16, MAP_FWD>(pl, a, st);  // conjugation lives in the packing
-    } else if (map == MAP_FWD) {
-        hipLaunchKernelGGL((pack_filters_f32_kernel<TS, 8, MAP_FWD>), dim3(pack_blocks), dim3(WG_THREADS), 0, st, pa);
-        KernelTimer timer(st);
-        rc = launch_fwd_variant<TS, 8, MAP_FWD>(pl, a, st);
-    } else {
-        hipLaunchKernelGGL((pack_filters_f32_kernel<TS, 8, MAP_DGRAD>), dim3(pack_blocks), dim3(WG_THREADS), 0, st, pa);
-        KernelTimer timer(st);
-        rc = launch_fwd_variant<TS, 8, MAP_DGRAD>(pl, a, st);
+        rc = f16 ? launch_fwd_f16(v, a, st) : launch_fwd_f32(v, a, st);
     }
-    if (rc != PHX_OK) return rc;
+    if (rc != 0) return PHX_ERR_NOT_SUPPORTED;
     PHX_HIP(hipGetLastError());
-    snprintf(g_name_buf, sizeof(g_name_buf), "qconv_%s_f32mfma_p%d_%s_wco%d_ntw%d_ck%d_tile%dx%dx%d",
-             map == MAP_FWD ? "fwd" : "dgrad", p.mode, sizeof(TS) == 4 ? "f32" : "f16", pl.WCO, pl.NTW, pl.CK, pl.NB,
-             pl.TH, pl.TW);
+    snprintf(g_name_buf, sizeof(g_name_buf), "qconv_%s_%smfma_p%d_%s_wco%d_ntw%d_ck%d_tile%dx%dx%d",
+             map == MAP_FWD ? "fwd" : "dgrad", f16 ? "f16" : "f32", p.mode, p.dtype == PHX_F32 ? "f32" : "f16", pl.WCO,
+             pl.NTW, pl.CK, pl.NB, pl.TH, pl.TW);
     g_last_kernel = g_name_buf;
     return PHX_OK;
 }
@@ -341,7 +334,6 @@ static bool plan_wgrad(const Problem& p, WgPlan& best) {
     return true;
 }
 
-template <typename TS>
 static int run_wgrad(const Problem& p, hipStream_t st, const void* x, const void* g, void* dw, void* ws,
                      size_t ws_bytes) {
     WgPlan pl;
@@ -360,12 +352,10 @@ static int run_wgrad(const Problem& p, hipStream_t st, const void* x, const void
     a.co_tiles = pl.co_tiles; a.ci_tiles = pl.ci_tiles; a.CoP = pl.CoP; a.CiP = pl.CiP;
     a.groups_per_row = pl.groups_per_row;
     const dim3 grid(pl.co_tiles * pl.ci_tiles, pl.groups_per_row * p.kh, pl.Z);
+    const bool half_storage = p.dtype == PHX_F16;
     {
         KernelTimer timer(st);
-        if (p.mode == 16)
-            hipLaunchKernelGGL((qconv_wgrad_f32_kernel<TS, 16, 3>), grid, dim3(WG_THREADS), pl.lds_bytes, st, a);
-        else
-            hipLaunchKernelGGL((qconv_wgrad_f32_kernel<TS, 8, 1>), grid, dim3(WG_THREADS), pl.lds_bytes, st, a);
+        launch_wgrad_f32(half_storage, p.mode, a, grid, pl.lds_bytes, st);
     }
     PHX_HIP(hipGetLastError());
     ReduceArgs r;
@@ -374,10 +364,10 @@ static int run_wgrad(const Problem& p, hipStream_t st, const void* x, const void
     r.Z = pl.Z; r.Co = p.co; r.Ci = p.ci; r.Kh = p.kh; r.Kw = p.kw; r.CoP = pl.CoP; r.CiP = pl.CiP;
     const long items = 4L * p.kh * p.kw * p.co * p.ci;
     const int blocks = (int)((items + 31) / 32);
-    hipLaunchKernelGGL((reduce_wgrad_kernel<TS>), dim3(blocks), dim3(WG_THREADS), 0, st, r);
+    launch_reduce_wgrad(half_storage, r, blocks, st);
     PHX_HIP(hipGetLastError());
     snprintf(g_name_buf, sizeof(g_name_buf), "qconv_wgrad_f32mfma_p%d_%s_tile%dx%dx%d_z%d", p.mode,
-             sizeof(TS) == 4 ? "f32" : "f16", pl.NB, pl.TH, pl.TW, pl.Z);
+             p.dtype == PHX_F32 ? "f32" : "f16", pl.NB, pl.TH, pl.TW, pl.Z);
     g_last_kernel = g_name_buf;
     return PHX_OK;
 }
@@ -390,7 +380,7 @@ static size_t workspace_for(const Problem& p, int pass) {
     }
     const Corr c = (pass == PHX_PASS_FWD) ? corr_forward(p) : corr_dgrad(p);
     FwdPlan pl;
-    return plan_forward(c, p.mode, pl) ? align_up(pl.wpk_bytes, 256) : 0;
+    return plan_forward(c, p.mode, use_f16_mfma(p, pass), pl) ? align_up(pl.wpk_bytes, 256) : 0;
 }
 
 static int do_fwd(const Problem& p, hipStream_t st, const void* x, const void* w, const void* bias, void* y, void* ws,
@@ -399,16 +389,14 @@ static int do_fwd(const Problem& p, hipStream_t st, const void* x, const void* w
     if (!x || !w || !y || (p.has_bias && !bias)) return PHX_ERR_INVALID_ARGUMENT;
     const Corr c = corr_forward(p);
     const void* b = p.has_bias ? bias : nullptr;
-    return p.dtype == PHX_F32 ? run_corr<float>(p, c, MAP_FWD, st, x, w, b, y, ws, wsb)
-                              : run_corr<_Float16>(p, c, MAP_FWD, st, x, w, b, y, ws, wsb);
+    return run_corr(p, c, MAP_FWD, st, x, w, b, y, ws, wsb);
 }
 
 static int do_bwd_data(const Problem& p, hipStream_t st, const void* g, const void* w, void* dx, void* ws, size_t wsb) {
     if (is_empty(p)) return PHX_OK;
     if (!g || !w || !dx) return PHX_ERR_INVALID_ARGUMENT;
     const Corr c = corr_dgrad(p);
-    return p.dtype == PHX_F32 ? run_corr<float>(p, c, MAP_DGRAD, st, g, w, nullptr, dx, ws, wsb)
-                              : run_corr<_Float16>(p, c, MAP_DGRAD, st, g, w, nullptr, dx, ws, wsb);
+    return run_corr(p, c, MAP_DGRAD, st, g, w, nullptr, dx, ws, wsb);
 }
 
 static int do_bwd_weights(const Problem& p, hipStream_t st, const void* x, const void* g, void* dw, void* ws,
@@ -421,8 +409,7 @@ static int do_bwd_weights(const Problem& p, hipStream_t st, const void* x, const
     }
     if (!x || !g) return PHX_ERR_INVALID_ARGUMENT;
     const Problem f = flatten_pointwise(p);
-    return p.dtype == PHX_F32 ? run_wgrad<float>(f, st, x, g, dw, ws, wsb)
-                              : run_wgrad<_Float16>(f, st, x, g, dw, ws, wsb);
+    return run_wgrad(f, st, x, g, dw, ws, wsb);
 }
 
 }  // namespace phx

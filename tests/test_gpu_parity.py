@@ -148,3 +148,58 @@ def test_empty_input_is_a_no_op_and_zeroes_dw():
     assert y.shape == (0, 3, 5, 5)
     dw, dx = phx.conv2d_bwd(x, w, torch.empty(0, 3, 5, 5, device="cuda"), desc)
     assert torch.count_nonzero(dw).item() == 0 and dx.shape == x.shape
+
+
+FP16_CASES = [c for c in CONV_CASES if c[0] in ("pw_64", "pw_ragged", "pw_7x7img", "k3_same", "k3_same_56", "k3_ragged",
+                                                "k3_s2", "k7_s2", "k32_asym", "co_gt_128")] + [
+    ("k3_128_28", 2, 128, 128, 28, 28, 3, 3, 1, 1, "SAME"),
+    ("pw_256_14", 3, 256, 256, 14, 14, 1, 1, 1, 1, "VALID"),
+]
+
+
+@pytest.mark.parametrize("policy", ["full16", "backward32", "fp32"])
+@pytest.mark.parametrize("mode", [16, 8])
+@pytest.mark.parametrize("case", FP16_CASES, ids=[c[0] for c in FP16_CASES])
+def test_conv_fp16(case, mode, policy):
+    """fp16 tensors N(0,1)*0.5 under the three UPSTRIDE_CONV_FP16_POLICY values; the yardstick is the
+    fp64 closed form on the fp16-rounded inputs (the reference's CPU backend is float-only)."""
+    name, n, ci, co, h, w, kh, kw, stride, dilation, padding = case
+    dtype = torch.float16
+    g, x, wt, b, gr = make_inputs(hash(name) % 1000 + 1, n, ci, co, h, w, kh, kw, stride, dilation, padding, dtype, 0.5)
+    print("case", name, "mode", mode, "policy", policy, flush=True)
+    desc = phx.Conv2DDescriptor(x.shape, wt.shape, stride, dilation, padding, use_bias=True, dtype=dtype,
+                                context=Ctx(mode, policy))
+    xd, wd, bd, gd = (torch.from_numpy(a).cuda() for a in (x, wt, b, gr))
+    y = phx.conv2d_fwd(xd, wd, bd, desc)
+    k_fwd = capi.last_kernel_name()
+    dw, dx = phx.conv2d_bwd(xd, wd, gd, desc)
+    k_bwd = capi.last_kernel_name()  # the input-gradient kernel runs last
+    torch.cuda.synchronize()
+    assert ("f16mfma" in k_fwd) == (policy in ("full16", "backward32")), k_fwd
+    assert ("f16mfma" in k_bwd) == (policy == "full16"), k_bwd
+    x64, w64, b64, g64 = (a.astype(np.float64) for a in (x, wt, b, gr))
+    want_y = oracle.conv2d_fwd(g, x64, w64, b64, "hamilton")
+    want_dw, want_dx = oracle.conv2d_bwd(g, x64, w64, g64, "hamilton")
+    assert_close(y.cpu().numpy(), want_y, dtype, "fwd " + k_fwd)
+    assert_close(dx.cpu().numpy(), want_dx, dtype, "dgrad " + k_bwd)
+    assert_close(dw.cpu().numpy(), want_dw, dtype, "wgrad " + name)
+
+
+@pytest.mark.parametrize("policy", ["full16", "fp32"])
+@pytest.mark.parametrize("mode", [16, 8])
+def test_dense_fp16(mode, policy):
+    n, ni, no = 16, 96, 40
+    r = np.random.default_rng(5)
+    x = (0.5 * r.standard_normal((4 * n, ni))).astype(np.float16)
+    w = (0.5 * r.standard_normal((4, ni, no)) * np.sqrt(2.0 / ni)).astype(np.float16)
+    b = (0.5 * r.standard_normal((4, no))).astype(np.float16)
+    gr = (0.5 * r.standard_normal((4 * n, no))).astype(np.float16)
+    desc = phx.DenseDescriptor(x.shape, w.shape, use_bias=True, dtype=torch.float16, context=Ctx(mode, policy))
+    xd, wd, bd, gd = (torch.from_numpy(a).cuda() for a in (x, w, b, gr))
+    y = phx.dense_fwd(xd, wd, bd, desc)
+    dw, dx = phx.dense_bwd(xd, wd, gd, desc)
+    x64, w64, b64, g64 = (a.astype(np.float64) for a in (x, w, b, gr))
+    assert_close(y.cpu().numpy(), oracle.dense_fwd(x64, w64, b64, "generic"), torch.float16, "dense fwd")
+    want_dw, want_dx = oracle.dense_bwd(x64, w64, g64, "generic")
+    assert_close(dx.cpu().numpy(), want_dx, torch.float16, "dense dgrad")
+    assert_close(dw.cpu().numpy(), want_dw, torch.float16, "dense wgrad")
