@@ -42,6 +42,8 @@ def parse():
                     help="product formulation; 0 = from UPSTRIDE_MEMORY_OPTIMIZED like the reference (default 8)")
     ap.add_argument("--policy", default=None, help="override UPSTRIDE_CONV_FP16_POLICY for fp16 workloads")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also launch a plain 256 MiB device copy (untimed), the yardstick for HBM byte counters")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU time budget of the cpu_baseline leg")
     return ap.parse_args()
 
@@ -134,6 +136,12 @@ def main():
         capi.check(L.phx_qconv2d_bwd_weights(d, stream, P(x), P(gr), P(dw), P(ws), sizes[2]), "bwd_weights")
         names.setdefault("bwd_weights", capi.last_kernel_name())
 
+    if args.copy_calibration:
+        src = torch.empty(64 << 20, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)  # reads 256 MiB, writes 256 MiB
+        del src, dst
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()

@@ -1,0 +1,921 @@
+// C++ host layer of the MI355X quaternion engine: the reference engine's operator interface for
+// the quaternion Conv2D / Dense path, re-implemented on top of the C ABI in include/phx_qconv.h.
+//
+// A program written against the reference's API (namespace upstride: Shape, Tensor, descriptors,
+// Context, conv2DFwd / conv2DBwd / denseFwd / denseBwd) compiles against this header with
+// Device = upstride::device::HIP.  Header-only, plain C++14, no HIP headers needed: every device
+// operation goes through libphx_qconv.so.
+//
+// Reference files mirrored (interfaces only, the implementation is new):
+//   src/algebras.hpp, src/backend/types.hpp, src/backend/tensor.hpp, src/utils.{hpp,cc},
+//   src/backend/conv2d_descriptor.hpp, src/backend/dense_descriptor.hpp, src/backend/backend.{hpp,cc},
+//   src/backend/memory_request.hpp, src/backend/operation.hpp, src/backend/device.hpp,
+//   src/backend/op_collections.hpp, src/conv2d.hpp, src/dense.hpp, src/upstride.hpp
+#pragma once
+
+#include <algorithm>
+#include <array>
+#include <cstdint>
+#include <cstdlib>
+#include <cstring>
+#include <initializer_list>
+#include <list>
+#include <map>
+#include <memory>
+#include <mutex>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "phx_qconv.h"
+
+namespace upstride {
+
+// ---------------------------------------------------------------------------------------------
+// Algebras (src/algebras.hpp:17-27, 176-188)
+// ---------------------------------------------------------------------------------------------
+enum Algebra { REAL, COMPLEX, QUATERNION, GA_300 };
+
+static const int MULTIVECTOR_DIM[] = {1, 2, 4, 8};
+
+inline Algebra getAlgebraFromType(int uptype) {
+    if (uptype < 0 || uptype > 3) throw std::invalid_argument("Invalid datatype index: " + std::to_string(uptype));
+    return static_cast<Algebra>(uptype);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Basic types (src/backend/types.hpp)
+// ---------------------------------------------------------------------------------------------
+typedef std::vector<int32_t> IntTuple;
+
+class IntPair {
+   public:
+    int x, y;  // x: height axis, y: width axis (src/backend/conv2d_descriptor.hpp:165-173)
+    IntPair() : x(0), y(0) {}
+    IntPair(int val) : x(val), y(val) {}
+    IntPair(int x, int y) : x(x), y(y) {}
+    IntPair(const IntTuple& tuple) {
+        if (tuple.size() == 1) x = y = tuple[0];
+        else if (tuple.size() == 2) { x = tuple[0]; y = tuple[1]; }
+        else throw std::invalid_argument("Cannot construct an integer pair from a tuple of " +
+                                         std::to_string(tuple.size()) + " elements");
+    }
+    IntPair operator+(const IntPair& o) const { return IntPair(x + o.x, y + o.y); }
+    IntPair operator-(const IntPair& o) const { return IntPair(x - o.x, y - o.y); }
+    IntPair operator*(const IntPair& o) const { return IntPair(x * o.x, y * o.y); }
+    IntPair operator/(const IntPair& o) const { return IntPair(x / o.x, y / o.y); }
+    bool operator==(const IntPair& o) const { return x == o.x && y == o.y; }
+    bool operator!=(const IntPair& o) const { return !(*this == o); }
+    bool operator<(const IntPair& o) const { return x < o.x || (x == o.x && y < o.y); }
+    static IntPair zeros() { return IntPair(0, 0); }
+    static IntPair ones() { return IntPair(1, 1); }
+};
+
+enum class Padding { SAME, VALID, EXPLICIT };
+enum class DataFormat { NCHW, NHWC, NC };
+enum class FilterLayout { OIHW, OHWI, HWIO, IO, OI };
+
+inline Padding paddingFromString(const std::string& s) {
+    if (s == "SAME") return Padding::SAME;
+    if (s == "VALID") return Padding::VALID;
+    if (s == "EXPLICIT") return Padding::EXPLICIT;
+    throw std::invalid_argument("Invalid padding encountered: " + s);
+}
+
+inline DataFormat dataFormatFromString(const std::string& s) {
+    if (s == "NHWC") return DataFormat::NHWC;
+    if (s == "NCHW") return DataFormat::NCHW;
+    throw std::invalid_argument("Invalid data format encountered: " + s);
+}
+
+inline const char* dataFormatToString(DataFormat f) {
+    return f == DataFormat::NCHW ? "NCHW" : f == DataFormat::NHWC ? "NHWC" : "";
+}
+
+inline FilterLayout filterLayoutFromString(const std::string& s) {
+    static const char* names[] = {"OIHW", "OHWI", "HWIO", "IO", "OI"};
+    for (int i = 0; i < 5; ++i)
+        if (s == names[i]) return static_cast<FilterLayout>(i);
+    throw std::invalid_argument("Invalid filter layout encountered: " + s);
+}
+
+inline const char* filterLayoutToString(FilterLayout f) {
+    static const char* names[] = {"OIHW", "OHWI", "HWIO", "IO", "OI"};
+    return names[static_cast<int>(f)];
+}
+
+// 16-bit float storage type for host code; arithmetic happens on the device only
+struct half {
+    uint16_t bits;
+};
+
+template <typename T> struct PhxDtype;
+template <> struct PhxDtype<float> { static const int value = PHX_F32; };
+template <> struct PhxDtype<half> { static const int value = PHX_F16; };
+
+// ---------------------------------------------------------------------------------------------
+// Shape (src/backend/tensor.hpp:35-276)
+// ---------------------------------------------------------------------------------------------
+inline int getWidthDimensionNumber(DataFormat f) { return f == DataFormat::NCHW ? 3 : 2; }
+inline int getHeightDimensionNumber(DataFormat f) { return f == DataFormat::NCHW ? 2 : 1; }
+inline int getDepthDimensionNumber(DataFormat f) { return f == DataFormat::NCHW ? 1 : 3; }
+
+class Shape {
+    std::vector<int> dims;
+
+   public:
+    Shape() {}
+    template <typename numeric>
+    Shape(std::initializer_list<numeric> list) {
+        for (auto v : list) dims.push_back(static_cast<int>(v));
+    }
+    Shape(int s, const int* values) : dims(values, values + s) {}
+    explicit Shape(int s) : dims(s, 0) {}
+
+    static const Shape& empty_shape() { static const Shape e; return e; }
+
+    uint8_t getSize() const { return static_cast<uint8_t>(dims.size()); }
+    const int* getShapePtr() const { return dims.data(); }
+    bool empty() const {  // no dimensions, or any dimension of extent zero
+        return dims.empty() || std::find(dims.begin(), dims.end(), 0) != dims.end();
+    }
+    int operator[](int i) const { return dims[i]; }
+    int& operator[](int i) { return dims[i]; }
+    bool operator==(const Shape& o) const { return dims == o.dims; }
+    bool operator!=(const Shape& o) const { return dims != o.dims; }
+    int compare(const Shape& o) const {  // shorter first, then lexicographic
+        if (dims.size() != o.dims.size()) return dims.size() < o.dims.size() ? -1 : +1;
+        for (size_t i = 0; i < dims.size(); ++i)
+            if (dims[i] != o.dims[i]) return dims[i] < o.dims[i] ? -1 : +1;
+        return 0;
+    }
+    bool operator<(const Shape& o) const { return compare(o) < 0; }
+    int& width(DataFormat f) { return dims[getWidthDimensionNumber(f)]; }
+    int width(DataFormat f) const { return dims[getWidthDimensionNumber(f)]; }
+    int& height(DataFormat f) { return dims[getHeightDimensionNumber(f)]; }
+    int height(DataFormat f) const { return dims[getHeightDimensionNumber(f)]; }
+    int& depth(DataFormat f) { return dims[getDepthDimensionNumber(f)]; }
+    int depth(DataFormat f) const { return dims[getDepthDimensionNumber(f)]; }
+    int64_t numel() const {
+        if (dims.empty()) return 0;
+        int64_t n = 1;
+        for (int d : dims) n *= d;
+        return n;
+    }
+    Shape expandDim(int dim = 0) const {
+        Shape r(*this);
+        r.dims.insert(r.dims.begin() + dim, 1);
+        return r;
+    }
+    // Pythonic slice; unlike the reference, slicing an empty shape is an error, not a wild read
+    Shape slice(int from, int to = 0) const {
+        const int n = static_cast<int>(dims.size());
+        if (from < 0) from += n;
+        if (to <= 0) to += n;
+        if (from >= 0 && from < to && to <= n) return Shape(to - from, dims.data() + from);
+        throw std::invalid_argument("Slice is out of range: " + std::to_string(from) + ":" + std::to_string(to));
+    }
+    Shape split(int numParts) const {
+        if (dims.empty() || dims[0] % numParts != 0)
+            throw std::invalid_argument("Cannot split " + std::to_string(dims.empty() ? 0 : dims[0]) + " onto " +
+                                        std::to_string(numParts) + " parts");
+        Shape r(*this);
+        r.dims[0] /= numParts;
+        return r;
+    }
+};
+
+// ---------------------------------------------------------------------------------------------
+// Windowed output size and padding (src/utils.cc:10-51)
+// ---------------------------------------------------------------------------------------------
+inline int computeWindowedOutputSizeAndPadding(int inputSize, int filterSize, int dilation, int stride, Padding padding,
+                                               int& paddingBefore, int& paddingAfter) {
+    const int effective = (filterSize - 1) * dilation + 1;
+    if (padding == Padding::VALID) {
+        paddingBefore = paddingAfter = 0;
+        return (inputSize - effective + stride) / stride;
+    }
+    if (padding == Padding::SAME) {
+        const int out = (inputSize + stride - 1) / stride;
+        const int needed = std::max(0, (out - 1) * stride + effective - inputSize);
+        paddingBefore = needed / 2;
+        paddingAfter = needed - paddingBefore;
+        return out;
+    }
+    throw std::invalid_argument("Invalid padding");
+}
+
+inline int computeWindowedOutputSizeAndPadding(int inputSize, int filterSize, int dilation, int stride,
+                                               int paddingBefore, int paddingAfter) {
+    const int effective = (filterSize - 1) * dilation + 1;
+    return (inputSize + paddingBefore + paddingAfter - effective + stride) / stride;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Context: environment switches, read once (src/backend/backend.hpp:36-74, backend.cc:17-57)
+// ---------------------------------------------------------------------------------------------
+enum class ConvFp16ComputePolicy { FULL_16, FORWARD_16_BACKWARD_32, FULL_32 };
+
+class Context {
+    bool envOptimizeMemoryUse;
+    ConvFp16ComputePolicy convFp16ComputePolicy;
+
+   public:
+    Context() {
+        const char* mem = std::getenv("UPSTRIDE_MEMORY_OPTIMIZED");
+        envOptimizeMemoryUse = mem && std::strtol(mem, nullptr, 10) > 0;
+        const char* pol = std::getenv("UPSTRIDE_CONV_FP16_POLICY");
+        const std::string p(pol ? pol : "");
+        convFp16ComputePolicy = p == "full16" ? ConvFp16ComputePolicy::FULL_16
+                                : p == "backward32" ? ConvFp16ComputePolicy::FORWARD_16_BACKWARD_32
+                                                    : ConvFp16ComputePolicy::FULL_32;
+    }
+    virtual ~Context() {}
+    bool preferSpeedToMemory() const { return !envOptimizeMemoryUse; }
+    bool isFp16ConvForwardAllowed() const { return convFp16ComputePolicy != ConvFp16ComputePolicy::FULL_32; }
+    bool isFp16ConvBackwardAllowed() const { return convFp16ComputePolicy == ConvFp16ComputePolicy::FULL_16; }
+    virtual void cleanUp() {}
+
+    int phxProductMode() const { return preferSpeedToMemory() ? PHX_PRODUCT_8 : PHX_PRODUCT_16; }
+    int phxFp16Policy() const {
+        return convFp16ComputePolicy == ConvFp16ComputePolicy::FULL_16 ? PHX_FP16_FULL16
+               : convFp16ComputePolicy == ConvFp16ComputePolicy::FORWARD_16_BACKWARD_32 ? PHX_FP16_BACKWARD32
+                                                                                        : PHX_FP16_FULL32;
+    }
+};
+
+// ---------------------------------------------------------------------------------------------
+// Temporary memory (src/backend/memory_request.hpp:15-29, src/backend/operation.hpp)
+// ---------------------------------------------------------------------------------------------
+class Allocator {
+   public:
+    virtual ~Allocator() {}
+    virtual void* mallocTemp(size_t size) = 0;  // valid until the operation returns
+    virtual size_t getAlignmentConstraint() const = 0;
+};
+
+class Operation {
+    size_t memoryNeeds = 0;
+
+   public:
+    virtual ~Operation() {}
+    void updateMemoryNeeds(size_t v) { memoryNeeds = std::max(memoryNeeds, v); }
+    size_t getMemoryNeeds() const { return memoryNeeds; }
+};
+
+inline void phxCheck(int status, const char* what) {
+    if (status == PHX_OK) return;
+    const std::string msg = std::string(what) + ": " + phx_status_string(status);
+    if (status == PHX_ERR_INVALID_ARGUMENT) throw std::invalid_argument(msg);
+    throw std::runtime_error(msg);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Descriptors (src/backend/conv2d_descriptor.hpp, src/backend/dense_descriptor.hpp)
+// ---------------------------------------------------------------------------------------------
+class Conv2DFilterLayout {
+    int o, i, h, w;
+
+   public:
+    Conv2DFilterLayout(FilterLayout layout, Algebra algebra = Algebra::REAL) {
+        switch (layout) {
+            case FilterLayout::OIHW: o = 0; i = 1; h = 2; w = 3; break;
+            case FilterLayout::OHWI: o = 0; h = 1; w = 2; i = 3; break;
+            case FilterLayout::HWIO: h = 0; w = 1; i = 2; o = 3; break;
+            default: throw std::invalid_argument("Unsupported Conv2D filter layout");
+        }
+        if (algebra != Algebra::REAL) { ++o; ++i; ++h; ++w; }  // blade dimension goes outermost
+    }
+    static int rank(Algebra algebra) { return algebra == Algebra::REAL ? 4 : 5; }
+    int numOutputChannelsDim() const { return o; }
+    int numInputChannelsDim() const { return i; }
+    int heightDim() const { return h; }
+    int widthDim() const { return w; }
+    int numOutputChannels(const Shape& s) const { return s[o]; }
+    int numInputChannels(const Shape& s) const { return s[i]; }
+    int height(const Shape& s) const { return s[h]; }
+    int width(const Shape& s) const { return s[w]; }
+};
+
+class Conv2DDescriptor {
+   protected:
+    Shape inputShape, filterShape;
+    IntPair stride, dilation;
+    int groups;
+    Algebra algebra;
+    DataFormat dataFormat;
+    FilterLayout filterLayout;
+    bool realValuedInput;
+    IntPair padBefore, padAfter;
+
+    template <class D>
+    static int compareCommon(const D& a, const D& b) {
+        int c = a.inputShape.compare(b.inputShape);
+        if (c) return c;
+        c = a.filterShape.compare(b.filterShape);
+        if (c) return c;
+#define PHX_CMP(field) if (a.field < b.field) return -1; if (b.field < a.field) return +1;
+        PHX_CMP(stride) PHX_CMP(dilation) PHX_CMP(groups) PHX_CMP(algebra) PHX_CMP(dataFormat) PHX_CMP(filterLayout)
+        PHX_CMP(realValuedInput) PHX_CMP(padBefore) PHX_CMP(padAfter)
+#undef PHX_CMP
+        return 0;
+    }
+
+   public:
+    Conv2DDescriptor(const Shape& inputShape, const Shape& filterShape, IntPair stride, IntPair dilation,
+                     Padding paddingPreset, const IntTuple& explicitPadding, int groups, Algebra algebra,
+                     DataFormat dataFormat, FilterLayout filterLayout, bool realValuedInput = false)
+        : inputShape(inputShape), filterShape(filterShape), stride(stride), dilation(dilation), groups(groups),
+          algebra(algebra), dataFormat(dataFormat), filterLayout(filterLayout), realValuedInput(realValuedInput) {
+        if (inputShape.getSize() != 4) throw std::invalid_argument("Four-dimensional input tensor expected");
+        if (algebra != Algebra::REAL) {
+            if (filterShape.getSize() != 5) throw std::invalid_argument("Five-dimensional filter tensor expected");
+            if (filterShape[0] != MULTIVECTOR_DIM[algebra])
+                throw std::invalid_argument("First filter dimension mismatch, got " + std::to_string(filterShape[0]));
+        } else if (filterShape.getSize() != 4) {
+            throw std::invalid_argument("Four-dimensional filter tensor expected");
+        }
+        Conv2DFilterLayout filter(filterLayout, algebra);
+        if (paddingPreset == Padding::EXPLICIT) {
+            // the reference parses EXPLICIT but then rejects it; here it works: (top, left, bottom, right)
+            if (explicitPadding.size() != 4) throw std::invalid_argument("Explicit padding needs four values");
+            padBefore = IntPair(explicitPadding[0], explicitPadding[1]);
+            padAfter = IntPair(explicitPadding[2], explicitPadding[3]);
+        } else {
+            computeWindowedOutputSizeAndPadding(inputShape.height(dataFormat), filter.height(filterShape), dilation.x,
+                                                stride.x, paddingPreset, padBefore.x, padAfter.x);
+            computeWindowedOutputSizeAndPadding(inputShape.width(dataFormat), filter.width(filterShape), dilation.y,
+                                                stride.y, paddingPreset, padBefore.y, padAfter.y);
+        }
+    }
+
+    Shape getOutputShape() const {
+        Conv2DFilterLayout filter(filterLayout, algebra);
+        Shape out(4);
+        out[0] = inputShape[0] * (realValuedInput ? MULTIVECTOR_DIM[algebra] : 1);
+        out.depth(dataFormat) = filter.numOutputChannels(filterShape);
+        out.height(dataFormat) = computeWindowedOutputSizeAndPadding(
+            inputShape.height(dataFormat), filter.height(filterShape), dilation.x, stride.x, padBefore.x, padAfter.x);
+        out.width(dataFormat) = computeWindowedOutputSizeAndPadding(
+            inputShape.width(dataFormat), filter.width(filterShape), dilation.y, stride.y, padBefore.y, padAfter.y);
+        return out;
+    }
+
+    const Shape& getInputShape() const { return inputShape; }
+    const Shape& getFilterShape() const { return filterShape; }
+    const IntPair& getStride() const { return stride; }
+    const IntPair& getDilation() const { return dilation; }
+    int getGroups() const { return groups; }
+    Algebra getAlgebra() const { return algebra; }
+    DataFormat getDataFormat() const { return dataFormat; }
+    FilterLayout getFilterLayout() const { return filterLayout; }
+    bool isRealValuedInput() const { return realValuedInput; }
+    IntPair getPaddingBefore() const { return padBefore; }
+    IntPair getPaddingAfter() const { return padAfter; }
+};
+
+class Conv2DFwdDescriptor : public Conv2DDescriptor {
+    bool useBias;
+
+   public:
+    Conv2DFwdDescriptor(const Shape& inputShape, const Shape& filterShape, IntPair stride, IntPair dilation,
+                        Padding paddingPreset, const IntTuple& explicitPadding, int groups, Algebra algebra,
+                        DataFormat dataFormat, FilterLayout filterLayout, bool useBias, bool realValuedInput = false)
+        : Conv2DDescriptor(inputShape, filterShape, stride, dilation, paddingPreset, explicitPadding, groups, algebra,
+                           dataFormat, filterLayout, realValuedInput),
+          useBias(useBias) {}
+    bool operator<(const Conv2DFwdDescriptor& o) const {
+        const int c = compareCommon(*this, o);
+        return c ? c < 0 : useBias < o.useBias;
+    }
+    bool operator==(const Conv2DFwdDescriptor& o) const { return !(*this < o) && !(o < *this); }
+    bool isBiasUsed() const { return useBias; }
+    Shape getBiasShape() const {
+        if (!useBias) return Shape();
+        Conv2DFilterLayout filter(filterLayout, algebra);
+        const int channels = filter.numOutputChannels(filterShape);
+        if (algebra == Algebra::REAL) return Shape{channels};
+        return Shape{MULTIVECTOR_DIM[algebra], channels};
+    }
+};
+
+class Conv2DBwdDescriptor : public Conv2DDescriptor {
+    bool requireInputGrad;
+
+   public:
+    Conv2DBwdDescriptor(const Shape& inputShape, const Shape& filterShape, IntPair stride, IntPair dilation,
+                        Padding paddingPreset, const IntTuple& explicitPadding, int groups, Algebra algebra,
+                        DataFormat dataFormat, FilterLayout filterLayout, bool requireInputGrad = true,
+                        bool realValuedInput = false)
+        : Conv2DDescriptor(inputShape, filterShape, stride, dilation, paddingPreset, explicitPadding, groups, algebra,
+                           dataFormat, filterLayout, realValuedInput),
+          requireInputGrad(requireInputGrad) {}
+    bool operator<(const Conv2DBwdDescriptor& o) const {
+        const int c = compareCommon(*this, o);
+        return c ? c < 0 : requireInputGrad < o.requireInputGrad;
+    }
+    bool operator==(const Conv2DBwdDescriptor& o) const { return !(*this < o) && !(o < *this); }
+    bool isInputGradientRequired() const { return requireInputGrad; }
+};
+
+class DenseDescriptor {
+   protected:
+    Shape inputShape, filterShape;
+    Algebra algebra;
+    FilterLayout filterLayout;
+
+    int compareCommon(const DenseDescriptor& o) const {
+        int c = inputShape.compare(o.inputShape);
+        if (c) return c;
+        c = filterShape.compare(o.filterShape);
+        if (c) return c;
+        if (algebra != o.algebra) return algebra < o.algebra ? -1 : +1;
+        if (filterLayout != o.filterLayout) return filterLayout < o.filterLayout ? -1 : +1;
+        return 0;
+    }
+
+   public:
+    DenseDescriptor(const Shape& inputShape, const Shape& filterShape, Algebra algebra, FilterLayout filterLayout)
+        : inputShape(inputShape), filterShape(filterShape), algebra(algebra), filterLayout(filterLayout) {
+        if (filterLayout != FilterLayout::IO && filterLayout != FilterLayout::OI)
+            throw std::invalid_argument("Dense filters are IO or OI");
+    }
+    int getOutputChannels() const {
+        const int idx = algebra == Algebra::REAL ? 0 : 1;
+        return filterLayout == FilterLayout::IO ? filterShape[idx + 1] : filterShape[idx];
+    }
+    Shape getInputShape() const { return inputShape; }
+    Shape getFilterShape() const { return filterShape; }
+    Shape getOutputShape() const { return Shape{inputShape[0], getOutputChannels()}; }
+    Shape getBiasShape() const {
+        if (algebra == Algebra::REAL) return Shape{getOutputChannels()};
+        return Shape{MULTIVECTOR_DIM[algebra], getOutputChannels()};
+    }
+    Algebra getAlgebra() const { return algebra; }
+    FilterLayout getFilterLayout() const { return filterLayout; }
+};
+
+class DenseFwdDescriptor : public DenseDescriptor {
+    bool useBias;
+
+   public:
+    DenseFwdDescriptor(const Shape& in, const Shape& filter, Algebra algebra, FilterLayout layout, bool useBias)
+        : DenseDescriptor(in, filter, algebra, layout), useBias(useBias) {}
+    bool operator<(const DenseFwdDescriptor& o) const {  // a strict weak order, unlike the reference's
+        const int c = compareCommon(o);
+        return c ? c < 0 : useBias < o.useBias;
+    }
+    bool isBiasUsed() const { return useBias; }
+};
+
+class DenseBwdDescriptor : public DenseDescriptor {
+    bool requireInputGrad;
+
+   public:
+    DenseBwdDescriptor(const Shape& in, const Shape& filter, Algebra algebra, FilterLayout layout, bool requireInputGrad)
+        : DenseDescriptor(in, filter, algebra, layout), requireInputGrad(requireInputGrad) {}
+    bool operator<(const DenseBwdDescriptor& o) const {
+        const int c = compareCommon(o);
+        return c ? c < 0 : requireInputGrad < o.requireInputGrad;
+    }
+    bool isInputGradientRequired() const { return requireInputGrad; }
+};
+
+// ---------------------------------------------------------------------------------------------
+// Operation cache: descriptor -> operation, most recently used first, trimmed to the 100 most
+// recent once more than 200 exist (src/backend/op_collections.hpp:121-144, op_collections.cc:6-64)
+// ---------------------------------------------------------------------------------------------
+template <class Descriptor>
+class OpCollection {
+    struct Entry {
+        Descriptor descriptor;
+        std::unique_ptr<Operation> op;
+    };
+    std::list<Entry> lru;
+    std::map<Descriptor, typename std::list<Entry>::iterator> index;
+
+   public:
+    static const size_t GC_THRESHOLD = 200, GC_KEEP = 100;
+
+    template <class Device, class OpClass>
+    OpClass& get(Device& device, const Descriptor& descriptor) {
+        auto it = index.find(descriptor);
+        if (it != index.end()) {
+            lru.splice(lru.begin(), lru, it->second);
+            return static_cast<OpClass&>(*it->second->op);
+        }
+        if (lru.size() > GC_THRESHOLD)
+            while (lru.size() > GC_KEEP) {
+                index.erase(lru.back().descriptor);
+                lru.pop_back();
+            }
+        lru.push_front(Entry{descriptor, std::unique_ptr<Operation>(new OpClass(device, descriptor))});
+        index.emplace(descriptor, lru.begin());
+        return static_cast<OpClass&>(*lru.front().op);
+    }
+    size_t size() const { return lru.size(); }
+};
+
+// ---------------------------------------------------------------------------------------------
+// Device (src/backend/device.hpp:12-110) and its HIP specialisation
+// ---------------------------------------------------------------------------------------------
+class Device : public Allocator {
+    Device(const Device&) = delete;
+    Context& context;
+    OpCollection<Conv2DFwdDescriptor> conv2dFwdOps;
+    OpCollection<Conv2DBwdDescriptor> conv2dBwdOps;
+    OpCollection<DenseFwdDescriptor> denseFwdOps;
+    OpCollection<DenseBwdDescriptor> denseBwdOps;
+    std::mutex accessControl;
+    void* workspace = nullptr;
+    size_t workspaceSize = 0;
+
+    virtual void* malloc(size_t size) = 0;
+    virtual void free(void* memory) = 0;
+
+   public:
+    explicit Device(Context& context) : context(context) {}
+    virtual ~Device() {}
+    Context& getContext() { return context; }
+    std::mutex& getAccessControl() { return accessControl; }
+
+    template <class DeviceClass, class OperationClass>
+    OperationClass& getConv2DFwdOperation(const Conv2DFwdDescriptor& d) {
+        return conv2dFwdOps.get<DeviceClass, OperationClass>(static_cast<DeviceClass&>(*this), d);
+    }
+    template <class DeviceClass, class OperationClass>
+    OperationClass& getConv2DBwdOperation(const Conv2DBwdDescriptor& d) {
+        return conv2dBwdOps.get<DeviceClass, OperationClass>(static_cast<DeviceClass&>(*this), d);
+    }
+    template <class DeviceClass, class OperationClass>
+    OperationClass& getDenseFwdOperation(const DenseFwdDescriptor& d) {
+        return denseFwdOps.get<DeviceClass, OperationClass>(static_cast<DeviceClass&>(*this), d);
+    }
+    template <class DeviceClass, class OperationClass>
+    OperationClass& getDenseBwdOperation(const DenseBwdDescriptor& d) {
+        return denseBwdOps.get<DeviceClass, OperationClass>(static_cast<DeviceClass&>(*this), d);
+    }
+
+    // grow-only workspace shared by all operations of the device
+    void* requestWorkspaceMemory(size_t size) {
+        if (size > workspaceSize) {
+            free(workspace);
+            workspace = malloc(size);
+            workspaceSize = size;
+        }
+        return workspace;
+    }
+    void freeWorkspaceMemory() {
+        free(workspace);
+        workspace = nullptr;
+        workspaceSize = 0;
+    }
+    size_t getWorkspaceSize() const { return workspaceSize; }
+    void* mallocTemp(size_t size) override { return requestWorkspaceMemory(size); }
+    size_t getAlignmentConstraint() const override { return 256; }
+};
+
+namespace device {
+
+// One HIP stream per device object; operations are enqueued asynchronously on it
+class HIP : public Device {
+    phx_stream_t hipStream;
+    bool ownsStream;
+
+    void* malloc(size_t size) override {
+        void* p = nullptr;
+        phxCheck(phx_device_malloc(&p, size), "device malloc");
+        return p;
+    }
+    void free(void* memory) override {
+        if (!memory) return;
+        phx_stream_synchronize(hipStream);
+        phx_device_free(memory);
+    }
+
+   public:
+    explicit HIP(Context& context) : Device(context), hipStream(nullptr), ownsStream(true) {
+        phxCheck(phx_stream_create(&hipStream), "stream create");
+    }
+    HIP(Context& context, phx_stream_t stream) : Device(context), hipStream(stream), ownsStream(false) {}
+    ~HIP() {
+        freeWorkspaceMemory();
+        if (ownsStream) phx_stream_destroy(hipStream);
+    }
+    phx_stream_t stream() const { return hipStream; }
+    void synchronize() { phxCheck(phx_stream_synchronize(hipStream), "stream synchronize"); }
+    static int count() {
+        int32_t n = 0;
+        phx_device_count(&n);
+        return n;
+    }
+};
+
+}  // namespace device
+
+// ---------------------------------------------------------------------------------------------
+// Tensors (src/backend/tensor.hpp:387-581), device = HIP
+// ---------------------------------------------------------------------------------------------
+template <typename Device, typename T>
+class Tensor {
+    Tensor(const Tensor&) = delete;
+
+   protected:
+    Device& device;
+    Shape shape;
+    T* tensor;
+
+   public:
+    Tensor(Device& device, const Shape& sh, T* t) : device(device), shape(sh), tensor(t) {}
+    T* getDataPtr() { return tensor; }
+    const T* getDataPtr() const { return tensor; }
+    const Shape& getShape() const { return shape; }
+    Device& getDevice() { return device; }
+    const Device& getDevice() const { return device; }
+
+    void zero() {
+        phxCheck(phx_memset_zero(tensor, shape.numel() * sizeof(T), device.stream()), "tensor zero");
+    }
+    Tensor& operator=(const std::vector<typename std::remove_const<T>::type>& contents) {
+        if (static_cast<int64_t>(contents.size()) != shape.numel())
+            throw std::invalid_argument("Cannot assign tensor contents: size mismatch");
+        phxCheck(phx_memcpy_h2d(tensor, contents.data(), contents.size() * sizeof(T), device.stream()), "tensor upload");
+        return *this;
+    }
+    template <typename vector_t>
+    operator std::vector<vector_t>() const {
+        static_assert(sizeof(vector_t) == sizeof(T), "Scalar datatype mismatch when copying a tensor into a vector");
+        std::vector<vector_t> contents(shape.numel());
+        phxCheck(phx_memcpy_d2h(contents.data(), tensor, contents.size() * sizeof(T),
+                                const_cast<Device&>(device).stream()), "tensor download");
+        return contents;
+    }
+    operator Tensor<Device, const T>&() { return reinterpret_cast<Tensor<Device, const T>&>(*this); }
+};
+
+template <typename Device, typename T>
+class AllocatedTensor : public Tensor<Device, T> {
+   public:
+    using Tensor<Device, T>::operator=;
+    AllocatedTensor(Device& device, const Shape& shape) : Tensor<Device, T>(device, shape, nullptr) {
+        void* p = nullptr;
+        phxCheck(phx_device_malloc(&p, shape.numel() * sizeof(T)), "tensor allocation");
+        this->tensor = static_cast<T*>(p);
+    }
+    ~AllocatedTensor() {
+        phx_stream_synchronize(this->device.stream());
+        phx_device_free(this->tensor);
+    }
+};
+
+// Zero-copy split along the outermost dimension
+template <typename Device, typename T, const int PARTS>
+class TensorSplit {
+    std::vector<std::unique_ptr<Tensor<Device, T>>> parts;
+    Shape partShape;
+
+   public:
+    TensorSplit(Tensor<Device, T>& input, bool keepOuterDimension = true) {
+        const Shape& s = input.getShape();
+        if (keepOuterDimension) {
+            if (s.getSize() == 0 || s[0] % PARTS != 0)
+                throw std::invalid_argument("Cannot split " + std::to_string(s.getSize() ? s[0] : 0) +
+                                            " entries in outer dimension onto " + std::to_string(PARTS) + " parts");
+            partShape = s.split(PARTS);
+        } else {
+            if (s.getSize() == 0 || s[0] != PARTS)
+                throw std::invalid_argument("Expected a tensor of " + std::to_string(PARTS) +
+                                            " entries in outer dimension, but got " +
+                                            std::to_string(s.getSize() ? s[0] : 0));
+            partShape = s.slice(1);
+        }
+        T* ptr = input.getDataPtr();
+        const int64_t step = partShape.numel();
+        for (int i = 0; i < PARTS; ++i, ptr += step)
+            parts.emplace_back(new Tensor<Device, T>(input.getDevice(), partShape, ptr));
+    }
+    const Tensor<Device, T>& operator[](int i) const { return *parts[i]; }
+    Tensor<Device, T>& operator[](int i) { return *parts[i]; }
+    constexpr int numParts() const { return PARTS; }
+    const Shape& shape() const { return partShape; }
+};
+
+// ---------------------------------------------------------------------------------------------
+// Operators (src/conv2d.hpp, src/dense.hpp).  The quaternion algebra runs on the fused HIP
+// kernels -- the seat the reference gives its custom quaternion kernels ahead of the factorized
+// and generic branches (src/conv2d.hpp:117-119, 380-382) -- with UPSTRIDE_MEMORY_OPTIMIZED
+// choosing the 8- or 16-product formulation inside them.  Other algebras are not built here.
+// ---------------------------------------------------------------------------------------------
+namespace detail {
+
+inline phx_qconv_desc makeConvDesc(const Conv2DDescriptor& d, Context& ctx, int dtype, bool useBias) {
+    if (d.getAlgebra() != Algebra::QUATERNION)
+        throw std::runtime_error("Only the quaternion algebra is built for device::HIP");
+    if (d.isRealValuedInput()) throw std::runtime_error("Real-valued input is not built for device::HIP");
+    if (d.getDataFormat() != DataFormat::NCHW) throw std::runtime_error("device::HIP runs NCHW tensors only");
+    if (d.getGroups() != 1) throw std::runtime_error("Grouped quaternion convolution is not built for device::HIP");
+    const FilterLayout fl = d.getFilterLayout();
+    if (fl != FilterLayout::OIHW && fl != FilterLayout::OHWI)
+        throw std::runtime_error("device::HIP takes OIHW or OHWI filters");
+    Conv2DFilterLayout filter(fl, Algebra::QUATERNION);
+    const Shape& in = d.getInputShape();
+    const Shape& w = d.getFilterShape();
+    phx_qconv_desc c;
+    c.dtype = dtype;
+    c.n = in[0] / 4;
+    c.ci = filter.numInputChannels(w);
+    c.co = filter.numOutputChannels(w);
+    c.h = in[2];
+    c.w = in[3];
+    c.kh = filter.height(w);
+    c.kw = filter.width(w);
+    c.stride_h = d.getStride().x; c.stride_w = d.getStride().y;
+    c.dilation_h = d.getDilation().x; c.dilation_w = d.getDilation().y;
+    c.pad_top = d.getPaddingBefore().x; c.pad_left = d.getPaddingBefore().y;
+    c.pad_bottom = d.getPaddingAfter().x; c.pad_right = d.getPaddingAfter().y;
+    c.filter_layout = fl == FilterLayout::OIHW ? PHX_OIHW : PHX_OHWI;
+    c.product_mode = ctx.phxProductMode();
+    c.fp16_policy = ctx.phxFp16Policy();
+    c.has_bias = useBias ? 1 : 0;
+    if (in[0] % 4 != 0) throw std::invalid_argument("Cannot split " + std::to_string(in[0]) + " onto 4 parts");
+    if (in[1] != c.ci) throw std::invalid_argument("Input channels do not match the filter");
+    return c;
+}
+
+inline phx_qdense_desc makeDenseDesc(const DenseDescriptor& d, Context& ctx, int dtype, bool useBias) {
+    if (d.getAlgebra() != Algebra::QUATERNION)
+        throw std::runtime_error("Only the quaternion algebra is built for device::HIP");
+    if (d.getFilterLayout() != FilterLayout::IO) throw std::runtime_error("device::HIP takes dense filters in IO layout");
+    const Shape in = d.getInputShape(), w = d.getFilterShape();
+    if (in.getSize() != 2 || w.getSize() != 3 || w[0] != 4 || in[0] % 4 != 0 || in[1] != w[1])
+        throw std::invalid_argument("Dense expects input [4n, in] and filter [4, in, out]");
+    phx_qdense_desc c;
+    c.dtype = dtype; c.n = in[0] / 4; c.ni = w[1]; c.no = w[2];
+    c.product_mode = ctx.phxProductMode(); c.fp16_policy = ctx.phxFp16Policy(); c.has_bias = useBias ? 1 : 0;
+    return c;
+}
+
+}  // namespace detail
+
+template <typename Device, typename T>
+class UpstrideConv2DFunctor : public Operation {
+    Device& device;
+    phx_qconv_desc desc;
+
+   public:
+    UpstrideConv2DFunctor(Device& device, const Conv2DFwdDescriptor& descriptor)
+        : device(device),
+          desc(detail::makeConvDesc(descriptor, device.getContext(), PhxDtype<T>::value, descriptor.isBiasUsed())) {}
+
+    void operator()(Allocator& allocator, const Tensor<Device, const T>& inputTensor,
+                    const Tensor<Device, const T>& kernelTensor, const Tensor<Device, const T>* biasTensor,
+                    Tensor<Device, T>& outputTensor, const IntPair& /*padBefore*/, const IntPair& /*padAfter*/,
+                    int /*groups*/ = 1) {
+        if (inputTensor.getShape().empty()) return;
+        if (desc.has_bias && !biasTensor)
+            throw std::invalid_argument("Bias application is configured but no bias tensor is given");
+        const size_t bytes = phx_qconv2d_workspace_bytes(&desc, PHX_PASS_FWD);
+        updateMemoryNeeds(bytes);
+        void* ws = bytes ? allocator.mallocTemp(bytes) : nullptr;
+        phx_qconv_desc d = desc;
+        d.has_bias = biasTensor ? 1 : 0;
+        phxCheck(phx_qconv2d_fwd(&d, device.stream(), inputTensor.getDataPtr(), kernelTensor.getDataPtr(),
+                                 biasTensor ? biasTensor->getDataPtr() : nullptr, outputTensor.getDataPtr(), ws, bytes),
+                 "conv2d forward");
+    }
+};
+
+template <typename Device, typename T>
+class UpstrideConv2DGradFunctor : public Operation {
+    Device& device;
+    phx_qconv_desc desc;
+    bool requireInputGrad;
+
+   public:
+    UpstrideConv2DGradFunctor(Device& device, const Conv2DBwdDescriptor& descriptor)
+        : device(device), desc(detail::makeConvDesc(descriptor, device.getContext(), PhxDtype<T>::value, false)),
+          requireInputGrad(descriptor.isInputGradientRequired()) {}
+
+    void operator()(Allocator& allocator, const Tensor<Device, const T>& inputTensor,
+                    const Tensor<Device, const T>& kernelTensor, const Tensor<Device, const T>& gradTensor,
+                    Tensor<Device, T>& kernelGradTensor, Tensor<Device, T>& inputGradTensor, const IntPair&,
+                    const IntPair&, int = 1) {
+        if (inputTensor.getShape().empty()) {
+            kernelGradTensor.zero();
+            return;
+        }
+        const size_t bw = phx_qconv2d_workspace_bytes(&desc, PHX_PASS_BWD_WEIGHTS);
+        const size_t bd = requireInputGrad ? phx_qconv2d_workspace_bytes(&desc, PHX_PASS_BWD_DATA) : 0;
+        const size_t bytes = std::max(bw, bd);
+        updateMemoryNeeds(bytes);
+        void* ws = bytes ? allocator.mallocTemp(bytes) : nullptr;
+        phxCheck(phx_qconv2d_bwd_weights(&desc, device.stream(), inputTensor.getDataPtr(), gradTensor.getDataPtr(),
+                                         kernelGradTensor.getDataPtr(), ws, bytes), "conv2d filter gradient");
+        // the input gradient is left untouched when not required (the reference's factorized path
+        // recomposes it from lanes it never wrote in that case)
+        if (requireInputGrad)
+            phxCheck(phx_qconv2d_bwd_data(&desc, device.stream(), gradTensor.getDataPtr(), kernelTensor.getDataPtr(),
+                                          inputGradTensor.getDataPtr(), ws, bytes), "conv2d input gradient");
+    }
+};
+
+template <typename Device, typename T>
+class UpstrideDenseFunctor : public Operation {
+    Device& device;
+    phx_qdense_desc desc;
+
+   public:
+    UpstrideDenseFunctor(Device& device, const DenseFwdDescriptor& descriptor)
+        : device(device),
+          desc(detail::makeDenseDesc(descriptor, device.getContext(), PhxDtype<T>::value, descriptor.isBiasUsed())) {}
+
+    void operator()(Allocator& allocator, const Tensor<Device, const T>& inputTensor,
+                    const Tensor<Device, const T>& kernelTensor, const Tensor<Device, const T>* biasTensor,
+                    Tensor<Device, T>& outputTensor) {
+        if (inputTensor.getShape().empty()) return;
+        const size_t bytes = phx_qdense_workspace_bytes(&desc, PHX_PASS_FWD);
+        updateMemoryNeeds(bytes);
+        void* ws = bytes ? allocator.mallocTemp(bytes) : nullptr;
+        phx_qdense_desc d = desc;
+        d.has_bias = biasTensor ? 1 : 0;
+        phxCheck(phx_qdense_fwd(&d, device.stream(), inputTensor.getDataPtr(), kernelTensor.getDataPtr(),
+                                biasTensor ? biasTensor->getDataPtr() : nullptr, outputTensor.getDataPtr(), ws, bytes),
+                 "dense forward");
+    }
+};
+
+template <typename Device, typename T>
+class UpstrideDenseGradFunctor : public Operation {
+    Device& device;
+    phx_qdense_desc desc;
+    bool requireInputGrad;
+
+   public:
+    UpstrideDenseGradFunctor(Device& device, const DenseBwdDescriptor& descriptor)
+        : device(device), desc(detail::makeDenseDesc(descriptor, device.getContext(), PhxDtype<T>::value, false)),
+          requireInputGrad(descriptor.isInputGradientRequired()) {}
+
+    void operator()(Allocator& allocator, const Tensor<Device, const T>& inputTensor,
+                    const Tensor<Device, const T>& kernelTensor, const Tensor<Device, const T>& gradTensor,
+                    Tensor<Device, T>& kernelGradTensor, Tensor<Device, T>& inputGradTensor) {
+        if (inputTensor.getShape().empty()) {
+            kernelGradTensor.zero();
+            return;
+        }
+        const size_t bw = phx_qdense_workspace_bytes(&desc, PHX_PASS_BWD_WEIGHTS);
+        const size_t bd = requireInputGrad ? phx_qdense_workspace_bytes(&desc, PHX_PASS_BWD_DATA) : 0;
+        const size_t bytes = std::max(bw, bd);
+        updateMemoryNeeds(bytes);
+        void* ws = bytes ? allocator.mallocTemp(bytes) : nullptr;
+        phxCheck(phx_qdense_bwd_weights(&desc, device.stream(), inputTensor.getDataPtr(), gradTensor.getDataPtr(),
+                                        kernelGradTensor.getDataPtr(), ws, bytes), "dense filter gradient");
+        if (requireInputGrad)
+            phxCheck(phx_qdense_bwd_data(&desc, device.stream(), gradTensor.getDataPtr(), kernelTensor.getDataPtr(),
+                                         inputGradTensor.getDataPtr(), ws, bytes), "dense input gradient");
+    }
+};
+
+// ---------------------------------------------------------------------------------------------
+// Entry points (src/upstride.hpp:18-86): lock the device, fetch the cached operation, run it
+// ---------------------------------------------------------------------------------------------
+template <typename Device, typename T>
+void conv2DFwd(Device& device, Allocator& allocator, const Tensor<Device, const T>& inputTensor,
+               const Tensor<Device, const T>& filterTensor, const Tensor<Device, const T>* biasTensor,
+               Tensor<Device, T>& outputTensor, const Conv2DFwdDescriptor& descriptor) {
+    std::lock_guard<std::mutex> lock(device.getAccessControl());
+    auto& op = device.template getConv2DFwdOperation<Device, UpstrideConv2DFunctor<Device, T>>(descriptor);
+    op(allocator, inputTensor, filterTensor, biasTensor, outputTensor, descriptor.getPaddingBefore(),
+       descriptor.getPaddingAfter(), descriptor.getGroups());
+}
+
+template <typename Device, typename T>
+void conv2DBwd(Device& device, Allocator& allocator, const Tensor<Device, const T>& inputTensor,
+               const Tensor<Device, const T>& filterTensor, const Tensor<Device, const T>& gradTensor,
+               Tensor<Device, T>& filterGradTensor, Tensor<Device, T>& inputGradTensor,
+               const Conv2DBwdDescriptor& descriptor) {
+    std::lock_guard<std::mutex> lock(device.getAccessControl());
+    auto& op = device.template getConv2DBwdOperation<Device, UpstrideConv2DGradFunctor<Device, T>>(descriptor);
+    op(allocator, inputTensor, filterTensor, gradTensor, filterGradTensor, inputGradTensor,
+       descriptor.getPaddingBefore(), descriptor.getPaddingAfter(), descriptor.getGroups());
+}
+
+template <typename Device, typename T>
+void denseFwd(Device& device, Allocator& allocator, const Tensor<Device, const T>& inputTensor,
+              const Tensor<Device, const T>& filterTensor, const Tensor<Device, const T>* biasTensor,
+              Tensor<Device, T>& outputTensor, const DenseFwdDescriptor& descriptor) {
+    std::lock_guard<std::mutex> lock(device.getAccessControl());
+    auto& op = device.template getDenseFwdOperation<Device, UpstrideDenseFunctor<Device, T>>(descriptor);
+    op(allocator, inputTensor, filterTensor, biasTensor, outputTensor);
+}
+
+template <typename Device, typename T>
+void denseBwd(Device& device, Allocator& allocator, const Tensor<Device, const T>& inputTensor,
+              const Tensor<Device, const T>& filterTensor, const Tensor<Device, const T>& gradTensor,
+              Tensor<Device, T>& filterGradTensor, Tensor<Device, T>& inputGradTensor,
+              const DenseBwdDescriptor& descriptor) {
+    std::lock_guard<std::mutex> lock(device.getAccessControl());
+    auto& op = device.template getDenseBwdOperation<Device, UpstrideDenseGradFunctor<Device, T>>(descriptor);
+    op(allocator, inputTensor, filterTensor, gradTensor, filterGradTensor, inputGradTensor);
+}
+
+}  // namespace upstride

@@ -1,0 +1,62 @@
+"""The C-ABI library loads without a GPU and exports every symbol include/phx_qconv.h declares;
+descriptor validation and workspace sizing (host-only code paths) behave."""
+import ctypes
+import os
+import re
+
+import phoenix_core_amd as phx
+from phoenix_core_amd import capi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_every_declared_symbol_is_exported():
+    header = open(os.path.join(ROOT, "include", "phx_qconv.h")).read()
+    declared = set(re.findall(r"\b(phx_[a-z0-9_]+)\s*\(", header))
+    lib = capi.lib()
+    assert declared, "no declarations found"
+    missing = [s for s in sorted(declared) if not hasattr(lib, s)]
+    assert not missing, missing
+    assert declared == set(capi.EXPORTS)
+
+
+def test_status_strings_and_descriptor_validation():
+    assert capi.status_string(0) == "ok"
+    assert "workspace" in capi.status_string(3)
+    bad = capi.QConvDesc(0, 1, 0, 4, 8, 8, 3, 3, 1, 1, 1, 1, 0, 0, 0, 0, 0, 8, 0, 0)  # zero input channels
+    ho, wo = ctypes.c_int32(), ctypes.c_int32()
+    assert capi.lib().phx_qconv2d_output_hw(ctypes.byref(bad), ctypes.byref(ho), ctypes.byref(wo)) == 1
+    assert capi.lib().phx_qconv2d_workspace_bytes(ctypes.byref(bad), 0) == 0
+    good = capi.QConvDesc(0, 2, 4, 4, 9, 8, 3, 3, 2, 2, 1, 1, 1, 0, 1, 1, 0, 8, 0, 0)
+    assert capi.lib().phx_qconv2d_output_hw(ctypes.byref(good), ctypes.byref(ho), ctypes.byref(wo)) == 0
+    assert (ho.value, wo.value) == (5, 4)
+    for which in (0, 1, 2):
+        assert capi.lib().phx_qconv2d_workspace_bytes(ctypes.byref(good), which) > 0
+
+
+def test_python_descriptor_matches_oracle_padding():
+    import oracle
+    import torch
+    for (h, w, k, s, d, pad) in [(56, 56, 3, 1, 1, "SAME"), (15, 14, 3, 2, 1, "SAME"), (224, 224, 7, 2, 1, "SAME"),
+                                 (9, 9, 3, 1, 2, "VALID"), (28, 28, 1, 2, 1, "VALID")]:
+        desc = phx.Conv2DDescriptor((8, 3, h, w), (4, 5, 3, k, k), s, d, pad, dtype=torch.float32,
+                                    context=phx.Context({}))
+        g = oracle.make_geom(2, 3, 5, h, w, k, k, s, d, pad)
+        assert desc.output_shape == (8, 5, g.ho, g.wo)
+        assert desc.pad_before == (g.pt, g.pl) and desc.pad_after == (g.pb, g.pr)
+
+
+def test_python_context_matches_oracle_env_rules():
+    import oracle
+    for mem in (None, "", "0", "1", "2", "-1", "yes", "1x", " 3"):
+        for pol in (None, "", "full16", "backward32", "fp32", "FULL16"):
+            env = {}
+            if mem is not None:
+                env["UPSTRIDE_MEMORY_OPTIMIZED"] = mem
+            if pol is not None:
+                env["UPSTRIDE_CONV_FP16_POLICY"] = pol
+            ctx = phx.Context(env)
+            assert ctx.memory_optimized == oracle.env_memory_optimized(mem), (mem, pol)
+            want = oracle.env_fp16_policy(pol)
+            assert ctx.is_fp16_conv_forward_allowed() == (want in ("full16", "backward32"))
+            assert ctx.is_fp16_conv_backward_allowed() == (want == "full16")
