@@ -234,4 +234,180 @@ __global__ void __launch_bounds__(WG_THREADS) pack_filters_f16_kernel(const Pack
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Filter gradient on fp16 MFMA.  Same decomposition as qconv_wgrad_f32_kernel (64x64 channel tile,
+// tap group = one filter row with up to TPW taps, split-K over pixel tiles, fp32 partial sums
+// reduced by reduce_wgrad_kernel); the reduction index (pixels) is contiguous in NCHW, so both
+// windows are staged as they lie.  One K step = 16 pixels = two 8-pixel packs:
+//   A operand (output gradient): 8 consecutive tile pixels = one aligned 16-byte LDS read;
+//   B operand (input, shifted by the tap): the 8 pixels' window offsets come from a per-tile
+//   table, the 8 halves are gathered with 16-bit LDS reads (any stride / dilation / padding).
+// ---------------------------------------------------------------------------------------------
+template <int P2LOG>
+__device__ __forceinline__ void stage_load_h2(f16x2 (&v)[(128) >> (8 - P2LOG)], const TileSrc& s, const StagePos& sp,
+                                              int c0) {
+    // 256 planes (4 components x 64 channels), G = 256 >> P2LOG groups, 256/G planes per thread, two per register
+    constexpr int G = WG_THREADS >> P2LOG;
+    constexpr int E = 256 / G;
+    const _Float16* origin = static_cast<const _Float16*>(s.base);
+    const long plane = (long)s.Hd * s.Wd;
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+        const int pc = e * G + sp.group;
+        const int p = pc >> 6, c = pc & 63;
+        const bool ok = sp.valid && (c0 + c) < s.C;
+        const _Float16* ptr = ok ? origin + sp.goff + p * s.comp_stride + (long)(c0 + c) * plane : origin;
+        const _Float16 t = *ptr;
+        v[e >> 1][e & 1] = ok ? t : (_Float16)0;
+    }
+}
+
+template <int P2LOG>
+__device__ __forceinline__ void stage_store_h2(_Float16* dst, const f16x2 (&v)[(128) >> (8 - P2LOG)],
+                                               const StagePos& sp, int HP, int pitch) {
+    constexpr int G = WG_THREADS >> P2LOG;
+    constexpr int E = 256 / G;
+    if (sp.pos < HP) {
+#pragma unroll
+        for (int e = 0; e < E; ++e) dst[(e * G + sp.group) * pitch + sp.pos] = v[e >> 1][e & 1];
+    }
+}
+
+template <int MODE, int TPW>
+__global__ void __launch_bounds__(WG_THREADS) qconv_wgrad_f16_kernel(const WgradArgs P) {
+    constexpr int CT = 64;
+    constexpr int NACC = (MODE == 16) ? 4 : 8;
+    constexpr int P2LOG = 6;  // 64 window positions x 4 plane groups
+    extern __shared__ f16x8 lds16[];
+    _Float16* gl = reinterpret_cast<_Float16*>(lds16);   // [4][CT][KPp], KPp multiple of 8 (16-byte rows)
+    _Float16* xl = gl + 4 * CT * P.KPp;                    // [4][CT][HPp]
+    int* poff = reinterpret_cast<int*>(xl + 4 * CT * P.HPp);  // [KP], 16-byte aligned
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wco = wave & 1, wci = wave >> 1;
+    const int m = lane & 31, kk = lane >> 5;
+    const int cot = blockIdx.x % P.co_tiles, cit = blockIdx.x / P.co_tiles;
+    const int kh = blockIdx.y / P.groups_per_row;
+    const int kw0 = (blockIdx.y % P.groups_per_row) * TPW;
+    const int nkw = (P.Kw - kw0 < TPW) ? P.Kw - kw0 : TPW;
+    const int HTW = (P.TW - 1) * P.sw + (nkw - 1) * P.dw + 1;
+    const int thw = P.TH * P.TW;
+    const int npix = P.NB * thw;
+
+    for (int k = tid; k < P.KP; k += WG_THREADS) {
+        const int nb = k / thw, rem = k - nb * thw;
+        const int r = rem / P.TW, c = rem - r * P.TW;
+        poff[k] = (k < npix) ? (nb * P.HTH + r * P.sh) * HTW + c * P.sw : 0;
+    }
+
+    f32x16 acc[TPW][NACC];
+#pragma unroll
+    for (int t = 0; t < TPW; ++t)
+#pragma unroll
+        for (int a = 0; a < NACC; ++a)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[t][a][r] = 0.f;
+
+    const int ntiles = P.tiles_n * P.tiles_h * P.tiles_w;
+    const long gcp = (long)CT * P.KPp, xcp = (long)CT * P.HPp;
+    f16x2 sg[32], sx[32];
+    StagePos spg, spx;
+    auto issue = [&](int tile) {
+        const int tw = tile % P.tiles_w;
+        const int th = (tile / P.tiles_w) % P.tiles_h;
+        const int tn = tile / (P.tiles_w * P.tiles_h);
+        const int n0 = tn * P.NB, ho0 = th * P.TH, wo0 = tw * P.TW;
+        spg = make_stage_pos<P2LOG>(P.g, n0, ho0, wo0, P.NB, P.TH, P.TW);
+        spx = make_stage_pos<P2LOG>(P.x, n0, ho0 * P.sh - P.pt + kh * P.dh, wo0 * P.sw - P.pl + kw0 * P.dw, P.NB, P.HTH,
+                                    HTW);
+        stage_load_h2<P2LOG>(sg, P.g, spg, cot * CT);
+        stage_load_h2<P2LOG>(sx, P.x, spx, cit * CT);
+    };
+    const int HPx = P.NB * P.HTH * HTW;
+    if ((int)blockIdx.z < ntiles) issue(blockIdx.z);
+    for (int tile = blockIdx.z; tile < ntiles; tile += gridDim.z) {
+        __syncthreads();
+        stage_store_h2<P2LOG>(gl, sg, spg, npix, P.KPp);
+        stage_store_h2<P2LOG>(xl, sx, spx, HPx, P.HPp);
+        // reduction indices beyond the tile's pixels must contribute zero
+        for (int i = tid; i < 4 * CT * (P.KP - npix); i += WG_THREADS) {
+            const int c = i / (P.KP - npix), k = npix + i % (P.KP - npix);
+            gl[c * P.KPp + k] = (_Float16)0;
+        }
+        __syncthreads();
+        if (tile + (int)gridDim.z < ntiles) issue(tile + gridDim.z);
+
+        const _Float16* ga = gl + (wco * 32 + m) * P.KPp + kk * 8;
+        const _Float16* xb = xl + (wci * 32 + m) * P.HPp;
+        for (int ks = 0; ks < P.KP; ks += 16) {
+            f16x8 g[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) g[q] = *reinterpret_cast<const f16x8*>(ga + q * gcp + ks);
+            int po[8];
+            {
+                const int4 a = *reinterpret_cast<const int4*>(poff + ks + kk * 8);
+                const int4 b = *reinterpret_cast<const int4*>(poff + ks + kk * 8 + 4);
+                po[0] = a.x; po[1] = a.y; po[2] = a.z; po[3] = a.w;
+                po[4] = b.x; po[5] = b.y; po[6] = b.z; po[7] = b.w;
+            }
+            f16x8 G[8];
+            if constexpr (MODE == 8) lanes_grad(g, G, (_Float16)0.5f);
+#pragma unroll
+            for (int t = 0; t < TPW; ++t) {
+                if (t < nkw) {
+                    f16x8 x[4];
+#pragma unroll
+                    for (int p = 0; p < 4; ++p)
+#pragma unroll
+                        for (int i = 0; i < 8; ++i) x[p][i] = xb[p * xcp + po[i] + t * P.dw];
+                    if constexpr (MODE == 16) {
+                        f16x8 nx[4];
+#pragma unroll
+                        for (int p = 0; p < 4; ++p) nx[p] = -x[p];
+#pragma unroll
+                        for (int p = 0; p < 4; ++p)
+#pragma unroll
+                            for (int q = 0; q < 4; ++q)
+                                acc[t][p ^ q] = __builtin_amdgcn_mfma_f32_32x32x16_f16(g[q], qneg(p, q) ? nx[p] : x[p],
+                                                                                       acc[t][p ^ q], 0, 0, 0);
+                    } else {
+                        f16x8 L[8];
+                        lanes_left(x, L);
+#pragma unroll
+                        for (int i = 0; i < 8; ++i)
+                            acc[t][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(G[i], L[i], acc[t][i], 0, 0, 0);
+                    }
+                }
+            }
+        }
+    }
+
+    const int taps = P.Kh * P.Kw;
+    const long tap_stride = 4L * P.CoP * P.CiP;
+    float* dst = P.partial + (long)blockIdx.z * taps * tap_stride;
+    const int ci = cit * CT + wci * 32 + m;
+    const int co_base = cot * CT + wco * 32 + 4 * kk;
+#pragma unroll
+    for (int t = 0; t < TPW; ++t) {
+        if (t >= nkw) continue;
+        float* d = dst + (long)(kh * P.Kw + kw0 + t) * tap_stride;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            const int co = co_base + 8 * (e >> 2) + (e & 3);
+            float y[4];
+            if constexpr (MODE == 16) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) y[r] = acc[t][r][e];
+            } else {
+                float l[8];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) l[i] = acc[t][i][e];
+                merge_right_grad(l, y);
+            }
+#pragma unroll
+            for (int r = 0; r < 4; ++r) d[((long)r * P.CoP + co) * P.CiP + ci] = y[r];
+        }
+    }
+}
+
 }  // namespace phx

@@ -22,6 +22,7 @@ int launch_fwd_f16(const FwdVariant& v, const ConvArgs& a, hipStream_t st);
 int launch_pack_filters_f16(const FwdVariant& v, const PackArgs& a, int blocks, hipStream_t st);
 
 int launch_wgrad_f32(bool half_storage, int mode, const WgradArgs& a, dim3 grid, size_t lds_bytes, hipStream_t st);
+int launch_wgrad_f16(int mode, const WgradArgs& a, dim3 grid, size_t lds_bytes, hipStream_t st);
 int launch_reduce_wgrad(bool half_storage, const ReduceArgs& a, int blocks, hipStream_t st);
 
 }  // namespace phx

@@ -295,21 +295,25 @@ struct WgPlan {
     size_t lds_bytes, partial_bytes;
 };
 
-static bool plan_wgrad(const Problem& p, WgPlan& best) {
+static bool plan_wgrad(const Problem& p, bool f16mfma, WgPlan& best) {
     const int TPW = (p.mode == 16) ? 3 : 1;
     const int nkw = std::min(TPW, p.kw);
     double best_score = -1.0;
     const int budget = LDS_FLOATS_MAX / (4 * 64);  // KPp + HPp (+ offsets) per staged channel
+    const int maxpos = f16mfma ? 64 : 32;  // staging positions per window
     for (int TW = 1; TW <= std::min(p.wo, 64); ++TW) {
         for (int TH = 1; TH <= p.ho; ++TH) {
             for (int NB = 1; NB <= p.n; ++NB) {
                 if (NB > 1 && !(TH == p.ho && TW == p.wo)) break;
                 const int pix = NB * TH * TW;
-                const int KP = (pix + 1) & ~1;
+                const int KP = f16mfma ? (pix + 15) & ~15 : (pix + 1) & ~1;
                 const int HTH = (TH - 1) * p.sh + 1;
                 const int HTW = (TW - 1) * p.sw + (nkw - 1) * p.dw + 1;
-                const int KPp = KP | 1, HPx = NB * HTH * HTW, HPp = HPx | 1;
-                if (KPp + HPp + (KP + 255) / 256 > budget || KP > 32 || HPx > 32) break;
+                const int HPx = NB * HTH * HTW;
+                // fp32: odd pitches (bank-conflict-free 4-byte reads); fp16: 16-byte rows plus one 16-byte skew
+                const int KPp = f16mfma ? KP + 8 : KP | 1, HPp = f16mfma ? ((HPx + 7) & ~7) + 8 : HPx | 1;
+                if (pix > maxpos || HPx > maxpos) break;
+                if (!f16mfma && KPp + HPp + (KP + 255) / 256 > budget) break;
                 const int tn = cdiv(p.n, NB), th = cdiv(p.ho, TH), tw = cdiv(p.wo, TW);
                 const double eff = ((double)p.n * p.ho * p.wo) / ((double)tn * th * tw * KP);
                 const double score = eff * (1.0 + 0.002 * KP) * (TW >= std::min(p.wo, 8) ? 1.0 : 0.5);
@@ -329,15 +333,17 @@ static bool plan_wgrad(const Problem& p, WgPlan& best) {
     const int xy = best.co_tiles * best.ci_tiles * best.groups_per_row * p.kh;
     const int ntiles = best.tiles_n * best.tiles_h * best.tiles_w;
     best.Z = std::max(1, std::min(ntiles, 512 / std::max(1, xy)));
-    best.lds_bytes = ((size_t)4 * 64 * (best.KPp + best.HPp) + best.KP) * sizeof(float);
+    best.lds_bytes = f16mfma ? (size_t)4 * 64 * (best.KPp + best.HPp) * 2 + (size_t)best.KP * 4 + 16
+                             : ((size_t)4 * 64 * (best.KPp + best.HPp) + best.KP) * sizeof(float);
     best.partial_bytes = (size_t)best.Z * p.kh * p.kw * 4 * best.CoP * best.CiP * sizeof(float);
     return true;
 }
 
 static int run_wgrad(const Problem& p, hipStream_t st, const void* x, const void* g, void* dw, void* ws,
                      size_t ws_bytes) {
+    const bool f16 = use_f16_mfma(p, PHX_PASS_BWD_WEIGHTS);
     WgPlan pl;
-    if (!plan_wgrad(p, pl)) return PHX_ERR_NOT_SUPPORTED;
+    if (!plan_wgrad(p, f16, pl)) return PHX_ERR_NOT_SUPPORTED;
     if (ws_bytes < pl.partial_bytes || !ws) return PHX_ERR_WORKSPACE;
     WgradArgs a;
     a.x.base = x; a.x.comp_stride = (long)p.n * p.ci * p.h * p.w; a.x.N = p.n; a.x.C = p.ci; a.x.Hd = p.h; a.x.Wd = p.w;
@@ -355,7 +361,8 @@ static int run_wgrad(const Problem& p, hipStream_t st, const void* x, const void
     const bool half_storage = p.dtype == PHX_F16;
     {
         KernelTimer timer(st);
-        launch_wgrad_f32(half_storage, p.mode, a, grid, pl.lds_bytes, st);
+        if (f16) launch_wgrad_f16(p.mode, a, grid, pl.lds_bytes, st);
+        else launch_wgrad_f32(half_storage, p.mode, a, grid, pl.lds_bytes, st);
     }
     PHX_HIP(hipGetLastError());
     ReduceArgs r;
@@ -366,7 +373,7 @@ static int run_wgrad(const Problem& p, hipStream_t st, const void* x, const void
     const int blocks = (int)((items + 31) / 32);
     launch_reduce_wgrad(half_storage, r, blocks, st);
     PHX_HIP(hipGetLastError());
-    snprintf(g_name_buf, sizeof(g_name_buf), "qconv_wgrad_f32mfma_p%d_%s_tile%dx%dx%d_z%d", p.mode,
+    snprintf(g_name_buf, sizeof(g_name_buf), "qconv_wgrad_%smfma_p%d_%s_tile%dx%dx%d_z%d", f16 ? "f16" : "f32", p.mode,
              p.dtype == PHX_F32 ? "f32" : "f16", pl.NB, pl.TH, pl.TW, pl.Z);
     g_last_kernel = g_name_buf;
     return PHX_OK;
@@ -376,7 +383,7 @@ static size_t workspace_for(const Problem& p, int pass) {
     if (is_empty(p)) return 0;
     if (pass == PHX_PASS_BWD_WEIGHTS) {
         WgPlan pl;
-        return plan_wgrad(flatten_pointwise(p), pl) ? align_up(pl.partial_bytes, 256) : 0;
+        return plan_wgrad(flatten_pointwise(p), use_f16_mfma(p, pass), pl) ? align_up(pl.partial_bytes, 256) : 0;
     }
     const Corr c = (pass == PHX_PASS_FWD) ? corr_forward(p) : corr_dgrad(p);
     FwdPlan pl;

@@ -172,9 +172,14 @@ def test_conv_fp16(case, mode, policy):
     xd, wd, bd, gd = (torch.from_numpy(a).cuda() for a in (x, wt, b, gr))
     y = phx.conv2d_fwd(xd, wd, bd, desc)
     k_fwd = capi.last_kernel_name()
-    dw, dx = phx.conv2d_bwd(xd, wd, gd, desc)
+    dw, _ = phx.conv2d_bwd(xd, wd, gd, phx.Conv2DDescriptor(x.shape, wt.shape, stride, dilation, padding, dtype=dtype,
+                                                           context=Ctx(mode, policy), require_input_grad=False))
+    k_wg = capi.last_kernel_name()
+    assert _ is None and ("f16mfma" in k_wg) == (policy == "full16"), k_wg
+    dw2, dx = phx.conv2d_bwd(xd, wd, gd, desc)
     k_bwd = capi.last_kernel_name()  # the input-gradient kernel runs last
     torch.cuda.synchronize()
+    assert torch.equal(dw, dw2)  # deterministic reduction
     assert ("f16mfma" in k_fwd) == (policy in ("full16", "backward32")), k_fwd
     assert ("f16mfma" in k_bwd) == (policy == "full16"), k_bwd
     x64, w64, b64, g64 = (a.astype(np.float64) for a in (x, wt, b, gr))
