@@ -37,6 +37,14 @@ __device__ __forceinline__ void stf<float>(float* p, float v) { *p = v; }
 template <>
 __device__ __forceinline__ void stf<_Float16>(_Float16* p, float v) { *p = (_Float16)v; }
 
+// -v for eight packed halves: flip the sign bits with four integer XORs (the generic vector negate
+// lowers to three instructions per register)
+__device__ __forceinline__ f16x8 neg8(const f16x8 v) {
+    typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+    const u32x4 m = {0x80008000u, 0x80008000u, 0x80008000u, 0x80008000u};
+    return __builtin_bit_cast(f16x8, __builtin_bit_cast(u32x4, v) ^ m);
+}
+
 // Lane maps of the factorized (8-product) Hamilton product.  Same arithmetic as the reference's
 // TensorManipulations lane maps (src/backend/onednn/tensor.hpp:61-170), applied to registers.
 template <typename V>
@@ -116,6 +124,15 @@ __device__ __forceinline__ int xcd_remap(int hw_id, int total) {
     return xcd * base + (xcd < rem ? xcd : rem) + slot;
 }
 
+// Sixteen zero bytes in device memory: out-of-tensor staging positions load from here, which keeps
+// the staging loads unconditional and free of selects.
+static __device__ __attribute__((aligned(16))) const unsigned int phx_zero_block[4] = {0u, 0u, 0u, 0u};
+
+template <typename T>
+__device__ __forceinline__ const T* zero_ptr() {
+    return reinterpret_cast<const T*>(phx_zero_block);
+}
+
 // A rectangular window of a component-stacked NCHW tensor t[4][N][C][Hd][Wd], seen through an
 // optional zero-insertion (virtual coordinate v maps to stored v/u when v % u == 0, else zero).
 struct TileSrc {
@@ -129,8 +146,8 @@ struct TileSrc {
 // multiplied: each thread owns ONE position of the window [n0, n0+NB) x [h0, h0+HTH) x [w0, w0+HTW)
 // (decoded once, it does not depend on the channel) and walks over the (component, channel) planes
 // of a chunk.  The 256 threads form G = 256 >> P2LOG groups of 2^P2LOG positions; group g loads
-// planes g, g+G, ...  Loads are unconditional (out-of-tensor positions read the tensor's first
-// element and are zeroed by a select) so that the staged values stay plain registers.
+// planes g, g+G, ...  Loads are unconditional (out-of-tensor positions read a block of zeros) so
+// that the staged values stay plain registers.
 struct StagePos {
     long goff;   // offset of this thread's position from the start of component 0, channel 0
     int pos;     // position inside the window, < 2^P2LOG
@@ -170,9 +187,8 @@ __device__ __forceinline__ void stage_load(float (&v)[(4 * NCH) >> (8 - P2LOG)],
         const int pc = e * G + sp.group;
         const int p = pc / NCH, c = pc % NCH;
         const bool ok = sp.valid && (c0 + c) < s.C;
-        const TS* ptr = ok ? origin + sp.goff + p * s.comp_stride + (long)(c0 + c) * plane : origin;
-        const float t = ldf<TS>(ptr);
-        v[e] = ok ? t : 0.f;
+        const TS* ptr = ok ? origin + sp.goff + p * s.comp_stride + (long)(c0 + c) * plane : zero_ptr<TS>();
+        v[e] = ldf<TS>(ptr);
     }
 }
 

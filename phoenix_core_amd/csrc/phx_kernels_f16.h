@@ -26,9 +26,8 @@ __device__ __forceinline__ void stage_load16(f16x8 (&v)[8 >> (8 - P2LOG)], const
         for (int i = 0; i < 8; ++i) {
             const int c = c0 + kp * 8 + i;
             const bool ok = sp.valid && c < s.C;
-            const _Float16* ptr = ok ? origin + sp.goff + p * s.comp_stride + (long)c * plane : origin;
-            const _Float16 t = *ptr;
-            v[e][i] = ok ? t : (_Float16)0;
+            const _Float16* ptr = ok ? origin + sp.goff + p * s.comp_stride + (long)c * plane : zero_ptr<_Float16>();
+            v[e][i] = *ptr;
         }
     }
 }
@@ -41,6 +40,74 @@ __device__ __forceinline__ void stage_store16(f16x8* dst, const f16x8 (&v)[8 >> 
     if (sp.pos < HP) {
 #pragma unroll
         for (int e = 0; e < E; ++e) dst[(e * G + sp.group) * pitch + sp.pos] = v[e];
+    }
+}
+
+// Pair staging: when image rows have an even length (and no zero insertion is in play) the window
+// is widened to start at an even column, so that two horizontally adjacent positions are one aligned
+// 32-bit word in every channel plane.  A thread then gathers the 8 channels of a pack for TWO
+// positions with 8 dword loads, splits low/high halves with 8 byte-permutes and writes two 16-byte
+// LDS entries: half the load instructions, each twice as wide.  128 pair positions x 2 thread
+// groups; a group walks 4 of the 8 (component, pack) units.
+struct StagePairPos {
+    long goff;   // element offset of the pair's first position (even)
+    int pos;     // window position of the pair's first element
+    int group;
+    bool valid, inwin;
+};
+
+__device__ __forceinline__ StagePairPos make_stage_pairpos(const TileSrc& s, int n0, int h0, int w0e, int NB, int HTH,
+                                                           int HTWe) {
+    StagePairPos sp;
+    const int pp = threadIdx.x & 127;
+    sp.group = threadIdx.x >> 7;
+    const int rowpairs = HTWe >> 1;
+    const int hw = HTH * rowpairs;
+    const int nb = pp / hw, rem = pp - nb * hw;
+    const int hr = rem / rowpairs, hcp = rem - hr * rowpairs;
+    const int vh = h0 + hr, vw = w0e + 2 * hcp;
+    sp.inwin = nb < NB;
+    sp.pos = (nb * HTH + hr) * HTWe + 2 * hcp;
+    const bool ok = sp.inwin && (n0 + nb) < s.N && vh >= 0 && vh < s.Hd && vw >= 0 && vw + 1 < s.Wd;
+    sp.valid = ok;
+    sp.goff = ok ? ((long)(n0 + nb) * s.C * s.Hd + vh) * s.Wd + vw : 0;
+    return sp;
+}
+
+__device__ __forceinline__ void stage_load16_pairs(unsigned int (&d)[4][8], const TileSrc& s, const StagePairPos& sp,
+                                                   int c0) {
+    const _Float16* origin = static_cast<const _Float16*>(s.base);
+    const long plane = (long)s.Hd * s.Wd;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const int u = e * 2 + sp.group;
+        const int p = u >> 1, kp = u & 1;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int c = c0 + kp * 8 + i;
+            const bool ok = sp.valid && c < s.C;
+            const _Float16* ptr = ok ? origin + sp.goff + p * s.comp_stride + (long)c * plane : zero_ptr<_Float16>();
+            d[e][i] = *reinterpret_cast<const unsigned int*>(ptr);
+        }
+    }
+}
+
+__device__ __forceinline__ void stage_store16_pairs(f16x8* dst, const unsigned int (&d)[4][8], const StagePairPos& sp,
+                                                    int pitch) {
+    typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+    if (sp.inwin) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            u32x4 lo, hi;
+#pragma unroll
+            for (int m = 0; m < 4; ++m) {
+                lo[m] = __builtin_amdgcn_perm(d[e][2 * m + 1], d[e][2 * m], 0x05040100u);
+                hi[m] = __builtin_amdgcn_perm(d[e][2 * m + 1], d[e][2 * m], 0x07060302u);
+            }
+            f16x8* q = dst + (e * 2 + sp.group) * pitch + sp.pos;
+            q[0] = __builtin_bit_cast(f16x8, lo);
+            q[1] = __builtin_bit_cast(f16x8, hi);
+        }
     }
 }
 
@@ -124,7 +191,7 @@ __global__ void __launch_bounds__(WG_THREADS, (MODE == 8 || NTW == 1) ? 2 : 1) q
                 if constexpr (MODE == 16) {
                     f16x8 nx[4];
 #pragma unroll
-                    for (int p = 0; p < 4; ++p) nx[p] = -x[p];
+                    for (int p = 0; p < 4; ++p) nx[p] = neg8(x[p]);
 #pragma unroll
                     for (int p = 0; p < 4; ++p)
 #pragma unroll
@@ -235,6 +302,214 @@ __global__ void __launch_bounds__(WG_THREADS) pack_filters_f16_kernel(const Pack
 }
 
 // ---------------------------------------------------------------------------------------------
+// Forward / input-gradient, 16-product, both operands through LDS.
+// The K loop runs over steps (16-channel chunk, tap).  Filters are packed per call into the exact
+// LDS image of a group of TG consecutive steps of one chunk and copied global->LDS by the direct
+// (register-less) load path, double buffered: the copy of group i+1 is issued before group i is
+// multiplied.  Activations are staged per chunk as in qconv_fwd_f16_kernel, their global loads
+// issued one chunk ahead into registers.  The inner loop therefore holds only LDS reads and MFMAs.
+//   packed filters: [filter tile of WCO*32 channels][group][tap in group][wco][component][lane] x 16 bytes
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ void lds_dma_16(const void* gsrc, void* ldst) {
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)gsrc,
+                                     (__attribute__((address_space(3))) void*)ldst, 16, 0, 0);
+}
+
+__device__ __forceinline__ void wait_vmem_all() { __builtin_amdgcn_s_waitcnt(0x0F70); }  // vmcnt(0)
+
+template <int WCO, int NTW, int P2LOG, bool PAIRS>
+__global__ void __launch_bounds__(WG_THREADS, 2) qconv_fwd_f16_lds_kernel(const ConvArgs P) {
+    constexpr int CK = F16_CK;
+    constexpr int WPX = 4 / WCO;
+    constexpr int TG = F16_TG;
+    constexpr int WIMG = TG * WCO * 4 * 64;  // 16-byte vectors per filter group image
+    extern __shared__ f16x8 lds16[];
+    f16x8* xl = lds16;                    // [8 units][HPp]
+    f16x8* wl = lds16 + 8 * P.HPp;        // [2][WIMG]
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wco = wave % WCO, wpx = wave / WCO;
+    const int j = lane & 31, kk = lane >> 5;
+
+    int bid = xcd_remap(blockIdx.x, gridDim.x);
+    const int ct = bid % P.co_tiles;
+    bid /= P.co_tiles;
+    const int tw = bid % P.tiles_w;
+    bid /= P.tiles_w;
+    const int th = bid % P.tiles_h;
+    const int tn = bid / P.tiles_h;
+    const int n0 = tn * P.NB, ho0 = th * P.TH, wo0 = tw * P.TW;
+    const int h0 = ho0 * P.sh - P.pt, w0 = wo0 * P.sw - P.pl;
+    const int w0e = PAIRS ? (w0 & ~1) : w0;  // pair staging starts the window at an even column
+    const int colshift = w0 - w0e;
+
+    int poff[NTW];
+    long oaddr[NTW];
+    bool pvalid[NTW];
+    const int thw = P.TH * P.TW;
+#pragma unroll
+    for (int t = 0; t < NTW; ++t) {
+        const int pix = (wpx * NTW + t) * 32 + j;
+        const int nb = pix / thw, rem = pix - nb * thw;
+        const int r = rem / P.TW, c = rem - r * P.TW;
+        pvalid[t] = nb < P.NB && (n0 + nb) < P.in.N && (ho0 + r) < P.Hout && (wo0 + c) < P.Wout;
+        poff[t] = pvalid[t] ? (nb * P.HTH + r * P.sh) * P.HTW + c * P.sw + colshift : colshift;
+        oaddr[t] = ((long)(n0 + nb) * P.Cout * P.Hout + (ho0 + r)) * P.Wout + (wo0 + c);
+    }
+
+    f32x16 acc[NTW][4];
+#pragma unroll
+    for (int t = 0; t < NTW; ++t)
+#pragma unroll
+        for (int a = 0; a < 4; ++a)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[t][a][r] = 0.f;
+
+    const int ngroups = (P.taps + TG - 1) / TG;          // per chunk
+    const int total_groups = P.nchunks * ngroups;
+    const f16x8* wsrc = static_cast<const f16x8*>(P.wpk) + (long)ct * total_groups * WIMG;
+    // filter group image -> LDS buffer: TG*WCO*4 slices of 64 vectors, dealt round-robin to the waves
+    auto copy_group = [&](int gs) {
+        const f16x8* src = wsrc + (long)gs * WIMG;
+        f16x8* dst = wl + (gs & 1) * WIMG;
+#pragma unroll
+        for (int s = 0; s < TG * WCO; ++s) {
+            const int slice = s * 4 + wave;
+            lds_dma_16(src + slice * 64 + lane, dst + slice * 64);
+        }
+    };
+
+    const StagePos sp = make_stage_pos<P2LOG>(P.in, n0, h0, w0, P.NB, P.HTH, P.HTW);
+    const StagePairPos spp = make_stage_pairpos(P.in, n0, h0, w0e, P.NB, P.HTH, P.HTW);
+    f16x8 stage[PAIRS ? 1 : (8 >> (8 - P2LOG))];
+    unsigned int stagep[PAIRS ? 4 : 1][8];
+    auto load_chunk = [&](int c0) {
+        if constexpr (PAIRS) stage_load16_pairs(stagep, P.in, spp, c0);
+        else stage_load16<P2LOG>(stage, P.in, sp, c0);
+    };
+    auto store_chunk = [&]() {
+        if constexpr (PAIRS) stage_store16_pairs(xl, stagep, spp, P.HPp);
+        else stage_store16<P2LOG>(xl, stage, sp, P.HP, P.HPp);
+    };
+    load_chunk(0);
+    copy_group(0);
+
+    int gs = 0;
+    for (int chunk = 0; chunk < P.nchunks; ++chunk) {
+        __syncthreads();  // every wave is done reading the previous chunk's activations
+        store_chunk();
+        int tap = 0, kh = 0, kw = 0;
+        for (int g = 0; g < ngroups; ++g, ++gs) {
+            wait_vmem_all();   // this group's filters have landed in LDS
+            __syncthreads();   // ... for every wave; activations of this chunk are visible
+            if (gs + 1 < total_groups) copy_group(gs + 1);
+            if (g == 0 && chunk + 1 < P.nchunks) load_chunk((chunk + 1) * CK);
+            const f16x8* wb = wl + (gs & 1) * WIMG + wco * 256 + lane;
+#pragma unroll
+            for (int tg = 0; tg < TG; ++tg) {
+                if (tap < P.taps) {
+                    const int tapoff = kh * P.dh * P.HTW + kw * P.dw;
+                    // negative blocks of the Hamilton matrix only ever use -w1, -w2, -w3: flip the
+                    // filter operand once per step instead of the activation operand per column tile
+                    f16x8 w[4], nw[4];
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        w[r] = wb[(tg * WCO * 4 + r) * 64];
+                        nw[r] = neg8(w[r]);
+                    }
+                    const f16x8* xb = xl + kk * P.HPp + tapoff;
+#pragma unroll
+                    for (int t = 0; t < NTW; ++t) {
+                        f16x8 x[4];
+#pragma unroll
+                        for (int p = 0; p < 4; ++p) x[p] = xb[p * 2 * P.HPp + poff[t]];
+#pragma unroll
+                        for (int p = 0; p < 4; ++p)
+#pragma unroll
+                            for (int q = 0; q < 4; ++q)
+                                acc[t][q] = __builtin_amdgcn_mfma_f32_32x32x16_f16(qneg(p, q) ? nw[p ^ q] : w[p ^ q], x[p],
+                                                                                   acc[t][q], 0, 0, 0);
+                    }
+                    ++tap;
+                    if (++kw == P.Kw) { kw = 0; ++kh; }
+                }
+            }
+        }
+    }
+
+    _Float16* out = static_cast<_Float16*>(P.out);
+    const _Float16* bias = static_cast<const _Float16*>(P.bias);
+    const long plane = (long)P.Hout * P.Wout;
+    const int co_base = (ct * WCO + wco) * 32 + 4 * kk;
+#pragma unroll
+    for (int t = 0; t < NTW; ++t) {
+        if (!pvalid[t]) continue;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int co = co_base + 8 * (r >> 2) + (r & 3);
+            if (co < P.Cout) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    float v = acc[t][q][r];
+                    if (bias) v += (float)bias[q * P.Cout + co];
+                    out[q * P.out_cs + oaddr[t] + co * plane] = (_Float16)v;
+                }
+            }
+        }
+    }
+}
+
+// Filter packing for qconv_fwd_f16_lds_kernel (16-product only; conjugated / mirrored / transposed
+// for MAP_DGRAD).  One thread per 16-byte vector of the image described above; taps beyond the
+// filter (last group of a chunk) and channels beyond the tensor are zero.
+struct PackLdsArgs {
+    PackArgs base;
+    int WCO;       // filter sub-tiles per workgroup tile
+    int ngroups;   // tap groups per chunk
+};
+
+template <int MAP>
+__global__ void __launch_bounds__(WG_THREADS) pack_filters_f16_lds_kernel(const PackLdsArgs A) {
+    const PackArgs& P = A.base;
+    constexpr int TG = F16_TG;
+    const int taps = P.Kh * P.Kw;
+    // index = ((((tile*nchunks + chunk)*ngroups + g)*TG + tg)*WCO + wco)*4 + r)*64 + lane
+    const long total = (long)P.row_tiles * P.nchunks * A.ngroups * TG * A.WCO * 4 * 64;
+    const _Float16* w = static_cast<const _Float16*>(P.w);
+    f16x8* outv = reinterpret_cast<f16x8*>(P.out);
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
+        const int lane = idx & 63;
+        long s = idx >> 6;
+        const int r = s & 3; s >>= 2;
+        const int wco = s % A.WCO; s /= A.WCO;
+        const int tg = s % TG; s /= TG;
+        const int g = s % A.ngroups; s /= A.ngroups;
+        const int chunk = s % P.nchunks;
+        const int tile = s / P.nchunks;
+        const int tap = g * TG + tg;
+        const int row = (tile * A.WCO + wco) * 32 + (lane & 31);
+        f16x8 vec;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) vec[i] = (_Float16)0;
+        if (tap < taps && row < P.rows) {
+            int kh = tap / P.Kw, kw = tap - kh * P.Kw;
+            if (MAP == MAP_DGRAD) { kh = P.Kh - 1 - kh; kw = P.Kw - 1 - kw; }
+            const float sgn = (MAP == MAP_DGRAD && r > 0) ? -1.f : 1.f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int red = chunk * F16_CK + (lane >> 5) * 8 + i;
+                if (red < P.red) {
+                    const int o = (MAP == MAP_DGRAD) ? red : row;
+                    const int in = (MAP == MAP_DGRAD) ? row : red;
+                    vec[i] = (_Float16)(sgn * (float)w[r * P.wcs + o * P.so + in * P.si + kh * P.skh + kw * P.skw]);
+                }
+            }
+        }
+        outv[idx] = vec;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
 // Filter gradient on fp16 MFMA.  Same decomposition as qconv_wgrad_f32_kernel (64x64 channel tile,
 // tap group = one filter row with up to TPW taps, split-K over pixel tiles, fp32 partial sums
 // reduced by reduce_wgrad_kernel); the reduction index (pixels) is contiguous in NCHW, so both
@@ -256,9 +531,8 @@ __device__ __forceinline__ void stage_load_h2(f16x2 (&v)[(128) >> (8 - P2LOG)], 
         const int pc = e * G + sp.group;
         const int p = pc >> 6, c = pc & 63;
         const bool ok = sp.valid && (c0 + c) < s.C;
-        const _Float16* ptr = ok ? origin + sp.goff + p * s.comp_stride + (long)(c0 + c) * plane : origin;
-        const _Float16 t = *ptr;
-        v[e >> 1][e & 1] = ok ? t : (_Float16)0;
+        const _Float16* ptr = ok ? origin + sp.goff + p * s.comp_stride + (long)(c0 + c) * plane : zero_ptr<_Float16>();
+        v[e >> 1][e & 1] = *ptr;
     }
 }
 
@@ -363,7 +637,7 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_wgrad_f16_kernel(const Wgrad
                     if constexpr (MODE == 16) {
                         f16x8 nx[4];
 #pragma unroll
-                        for (int p = 0; p < 4; ++p) nx[p] = -x[p];
+                        for (int p = 0; p < 4; ++p) nx[p] = neg8(x[p]);
 #pragma unroll
                         for (int p = 0; p < 4; ++p)
 #pragma unroll

@@ -12,6 +12,9 @@ struct FwdVariant {
     bool f16_mfma;      // fp16 matrix-core arithmetic (else fp32)
     int mode, map;      // 16 / 8, MAP_FWD / MAP_DGRAD
     int WCO, NTW, CK, P2LOG;
+    bool lds_filters;   // fp16 MFMA only: filters staged through LDS (qconv_fwd_f16_lds_kernel)
+    int ngroups;        // tap groups per chunk for that kernel
+    bool pairs;         // fp16 MFMA: activations staged as aligned position pairs
     int wgs;
     size_t lds_bytes;
 };

@@ -22,7 +22,24 @@ static int launch_variant16(const FwdVariant& v, const ConvArgs& a, hipStream_t 
     return -1;
 }
 
+template <bool PAIRS>
+static int launch_lds16(const FwdVariant& v, const ConvArgs& a, hipStream_t st) {
+    constexpr int P2A = 8, P2B = PAIRS ? 8 : 7;  // the pair path has a single staging shape
+#define PHX_CASE(WCO_, NTW_, P2_)                                                                             \
+    if (v.WCO == WCO_ && v.NTW == NTW_ && (PAIRS || v.P2LOG == P2_)) {                                        \
+        hipLaunchKernelGGL((qconv_fwd_f16_lds_kernel<WCO_, NTW_, P2_, PAIRS>), dim3(v.wgs), dim3(WG_THREADS), \
+                           v.lds_bytes, st, a);                                                               \
+        return 0;                                                                                             \
+    }
+    PHX_CASE(1, 1, P2A) PHX_CASE(1, 1, P2B) PHX_CASE(1, 2, P2A) PHX_CASE(1, 2, P2B)
+    PHX_CASE(2, 1, P2A) PHX_CASE(2, 1, P2B) PHX_CASE(2, 2, P2A) PHX_CASE(2, 2, P2B)
+    PHX_CASE(4, 1, P2A) PHX_CASE(4, 1, P2B) PHX_CASE(4, 2, P2A) PHX_CASE(4, 2, P2B)
+#undef PHX_CASE
+    return -1;
+}
+
 int launch_fwd_f16(const FwdVariant& v, const ConvArgs& a, hipStream_t st) {
+    if (v.lds_filters) return v.pairs ? launch_lds16<true>(v, a, st) : launch_lds16<false>(v, a, st);
     if (v.mode == 16) return launch_variant16<16, MAP_FWD>(v, a, st);
     if (v.map == MAP_FWD) return launch_variant16<8, MAP_FWD>(v, a, st);
     return launch_variant16<8, MAP_DGRAD>(v, a, st);
@@ -30,6 +47,12 @@ int launch_fwd_f16(const FwdVariant& v, const ConvArgs& a, hipStream_t st) {
 
 int launch_pack_filters_f16(const FwdVariant& v, const PackArgs& a, int blocks, hipStream_t st) {
     const dim3 g(blocks), b(WG_THREADS);
+    if (v.lds_filters) {
+        PackLdsArgs la{a, v.WCO, v.ngroups};
+        if (v.map == MAP_FWD) hipLaunchKernelGGL((pack_filters_f16_lds_kernel<MAP_FWD>), g, b, 0, st, la);
+        else hipLaunchKernelGGL((pack_filters_f16_lds_kernel<MAP_DGRAD>), g, b, 0, st, la);
+        return 0;
+    }
     if (v.mode == 16 && v.map == MAP_FWD) hipLaunchKernelGGL((pack_filters_f16_kernel<16, MAP_FWD>), g, b, 0, st, a);
     else if (v.mode == 16) hipLaunchKernelGGL((pack_filters_f16_kernel<16, MAP_DGRAD>), g, b, 0, st, a);
     else if (v.map == MAP_FWD) hipLaunchKernelGGL((pack_filters_f16_kernel<8, MAP_FWD>), g, b, 0, st, a);

@@ -4,6 +4,7 @@
 
 #include <algorithm>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <vector>
 
@@ -154,6 +155,9 @@ static Corr corr_dgrad(const Problem& p) {
 struct FwdPlan {
     int WCO, NTW, BN;
     int CK, P2LOG;           // channels per chunk and log2 staging positions of the kernel variant
+    bool lds_filters;        // fp16 MFMA, 16-product, more than one tap: filters go through LDS
+    int ngroups;             // tap groups per chunk in that case
+    bool pairs;              // fp16 MFMA: window rows widened to even columns, staged as position pairs
     int NB, TH, TW, HTH, HTW, HP, HPp;
     int tiles_n, tiles_h, tiles_w, co_tiles, nchunks;
     size_t lds_bytes, wpk_bytes;
@@ -165,11 +169,19 @@ constexpr int LDS_FLOATS_MAX = 16384;  // 64 KiB: two workgroups per CU
 
 static bool plan_forward(const Corr& c, int mode, bool f16mfma, FwdPlan& best) {
     double best_score = -1.0;
+    // fp16 MFMA with filters in LDS: stage activations as aligned pairs when rows are even
+    const bool pairs = f16mfma && mode == 16 && c.Kh * c.Kw > 1 && (c.Win % 2 == 0) && c.uw == 1;
+    best.pairs = pairs;
     const int wcos[3] = {1, 2, 4};
+    // PHX_TUNE_TILE="wco,ntw" pins the workgroup shape (kernel tuning experiments)
+    int force_wco = 0, force_ntw = 0;
+    if (const char* t = std::getenv("PHX_TUNE_TILE")) sscanf(t, "%d,%d", &force_wco, &force_ntw);
     for (int wi = 0; wi < 3; ++wi) {
         const int WCO = wcos[wi];
+        if (force_wco && WCO != force_wco) continue;
         if (WCO > 1 && 32 * WCO > ((c.Cout + 31) / 32) * 32) continue;
         for (int NTW = 1; NTW <= (mode == 16 ? 2 : 1); ++NTW) {  // 8 lanes x 2 column tiles would spill
+            if (force_ntw && NTW != force_ntw) continue;
             const int BN = (4 / WCO) * NTW * 32;
             int cand[16];
             int nc = 0;
@@ -182,7 +194,8 @@ static bool plan_forward(const Corr& c, int mode, bool f16mfma, FwdPlan& best) {
                     int NB = 1;
                     if (TH == c.Hout && TW == c.Wout) NB = std::max(1, std::min(c.N, BN / (TH * TW)));
                     const int HTH = (TH - 1) * c.sh + (c.Kh - 1) * c.dh + 1;
-                    const int HTW = (TW - 1) * c.sw + (c.Kw - 1) * c.dw + 1;
+                    int HTW = (TW - 1) * c.sw + (c.Kw - 1) * c.dw + 1;
+                    if (pairs) HTW = (HTW + 2) & ~1;  // room for the even start column, even pitch
                     const int HP = NB * HTH * HTW;
                     const int HPp = HP;
                     if (HP > 256) continue;  // one staging position per thread
@@ -192,7 +205,11 @@ static bool plan_forward(const Corr& c, int mode, bool f16mfma, FwdPlan& best) {
                     const double eff = ((double)c.N * c.Hout * c.Wout * c.Cout) / ((double)wgs * BN * 32 * WCO);
                     const double fill = (double)wgs / ((double)cdiv((int)std::min<long>(wgs, 1 << 30), 512) * 512);
                     const double halo = (double)(NB * TH * TW) / HP;  // staged data actually used
-                    const double score = eff * (0.25 + 0.75 * fill) * (0.9 + 0.1 * halo) * (NTW == 2 ? 1.02 : 1.0);
+                    double score = eff * (0.25 + 0.75 * fill) * (0.9 + 0.1 * halo) * (NTW == 2 ? 1.02 : 1.0);
+                    // fp16 MFMA is operand-bandwidth hungry: two column tiles per wave and two filter
+                    // sub-tiles per workgroup amortise LDS reads and activation staging (measured)
+                    if (pairs) score *= (NTW == 2 ? 1.25 : 1.0) * (WCO == 2 ? 1.08 : 1.0);
+                    else if (f16mfma && NTW == 2) score *= 0.8;  // that kernel drops to one workgroup per CU
                     if (score > best_score) {
                         best_score = score;
                         best.WCO = WCO; best.NTW = NTW; best.BN = BN;
@@ -215,11 +232,18 @@ static bool plan_forward(const Corr& c, int mode, bool f16mfma, FwdPlan& best) {
         best.nchunks = cdiv(c.Cin, best.CK);
         best.lds_bytes = (size_t)8 * best.HPp * 16;
         best.wpk_bytes = (size_t)best.co_tiles * best.WCO * best.nchunks * taps * 64 * WC * 16;
+        best.lds_filters = (mode == 16 && taps > 1);
+        best.ngroups = cdiv(taps, F16_TG);
+        if (best.lds_filters) {
+            const size_t wimg = (size_t)F16_TG * best.WCO * 4 * 64 * 16;  // one filter group image
+            best.lds_bytes += 2 * wimg;
+            best.wpk_bytes = (size_t)best.co_tiles * best.nchunks * best.ngroups * wimg;
+        }
         return true;
     }
     // fp32 MFMA: pointwise problems are bandwidth/latency bound and take as many channels per
     // chunk as 32 staging registers per thread allow; everything else uses 8-channel chunks
-    best.CK = F32_CK; best.P2LOG = 8;
+    best.CK = F32_CK; best.P2LOG = 8; best.lds_filters = false; best.ngroups = 0;
     if (taps == 1 && c.Cin >= 32) {
         if (best.HP <= 64) { best.CK = 32; best.P2LOG = 6; }
         else if (best.HP <= 128) { best.CK = 16; best.P2LOG = 7; }
@@ -250,6 +274,7 @@ static int run_corr(const Problem& p, const Corr& c, int map, hipStream_t st, co
     FwdVariant v;
     v.half_storage = p.dtype == PHX_F16; v.f16_mfma = f16; v.mode = p.mode; v.map = map;
     v.WCO = pl.WCO; v.NTW = pl.NTW; v.CK = pl.CK; v.P2LOG = pl.P2LOG; v.wgs = pl.wgs; v.lds_bytes = pl.lds_bytes;
+    v.lds_filters = pl.lds_filters; v.ngroups = pl.ngroups; v.pairs = pl.pairs;
 
     PackArgs pa;
     pa.w = w; pa.out = ws;
@@ -257,7 +282,9 @@ static int run_corr(const Problem& p, const Corr& c, int map, hipStream_t st, co
     pa.Co = p.co; pa.Ci = p.ci; pa.Kh = p.kh; pa.Kw = p.kw;
     pa.rows = c.Cout; pa.red = c.Cin; pa.row_tiles = pl.co_tiles * pl.WCO;
     pa.nchunks = f16 ? pl.nchunks : pl.nchunks * (pl.CK / F32_CK);
-    const long pack_items = (long)pa.row_tiles * pa.nchunks * p.kh * p.kw * (f16 ? 1 : 4) * 64;
+    const long pack_items = pl.lds_filters ? (long)(pl.wpk_bytes / 16)
+                                            : (long)pa.row_tiles * pa.nchunks * p.kh * p.kw * (f16 ? 1 : 4) * 64;
+    if (pl.lds_filters) pa.row_tiles = pl.co_tiles;  // packed per workgroup tile of WCO*32 channels
     const int pack_blocks = (int)std::min<long>((pack_items + WG_THREADS - 1) / WG_THREADS, 4096);
 
     ConvArgs a;
@@ -279,8 +306,8 @@ static int run_corr(const Problem& p, const Corr& c, int map, hipStream_t st, co
     }
     if (rc != 0) return PHX_ERR_NOT_SUPPORTED;
     PHX_HIP(hipGetLastError());
-    snprintf(g_name_buf, sizeof(g_name_buf), "qconv_%s_%smfma_p%d_%s_wco%d_ntw%d_ck%d_tile%dx%dx%d",
-             map == MAP_FWD ? "fwd" : "dgrad", f16 ? "f16" : "f32", p.mode, p.dtype == PHX_F32 ? "f32" : "f16", pl.WCO,
+    snprintf(g_name_buf, sizeof(g_name_buf), "qconv_%s_%smfma%s_p%d_%s_wco%d_ntw%d_ck%d_tile%dx%dx%d",
+             map == MAP_FWD ? "fwd" : "dgrad", f16 ? "f16" : "f32", pl.lds_filters ? (pl.pairs ? "ldsp" : "lds") : "", p.mode, p.dtype == PHX_F32 ? "f32" : "f16", pl.WCO,
              pl.NTW, pl.CK, pl.NB, pl.TH, pl.TW);
     g_last_kernel = g_name_buf;
     return PHX_OK;
