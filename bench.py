@@ -30,6 +30,7 @@ WORKLOADS = {
     "c4_pw_f16_128_28": (128, 128, 128, 28, 28, 1, "VALID", "f16", "full16"),
     "c4_pw_f16_256_14": (128, 256, 256, 14, 14, 1, "VALID", "f16", "full16"),
 }
+RESNET = "c5_qresnet50"  # quaternion ResNet-50 forward+backward, N=64, 224x224, fp16 full16 policy
 
 
 def parse():
@@ -37,10 +38,11 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="c2_pw_f32", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="c2_pw_f32", choices=sorted(WORKLOADS) + [RESNET])
     ap.add_argument("--mode", type=int, default=0, choices=[0, 8, 16],
                     help="product formulation; 0 = from UPSTRIDE_MEMORY_OPTIMIZED like the reference (default 8)")
     ap.add_argument("--policy", default=None, help="override UPSTRIDE_CONV_FP16_POLICY for fp16 workloads")
+    ap.add_argument("--batch", type=int, default=64, help="images per step of the ResNet workload")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch a plain 256 MiB device copy (untimed), the yardstick for HBM byte counters")
@@ -87,12 +89,91 @@ def cpu_baseline(cfg, mode, seconds):
     }
 
 
+def resnet_flops(n):
+    """Real-equivalent forward FLOPs of the 53 convolutions + head (2*16*N*Co*Ci*Ho*Wo*Kh*Kw each)."""
+    total, size = 0.0, 224
+    def conv(ci, co, k, s, hin):
+        ho = (hin + s - 1) // s
+        return 2.0 * 16 * n * co * ci * ho * ho * k * k, ho
+    f, size = conv(3, 16, 7, 2, size)
+    total += f
+    size = (size + 1) // 2  # max-pool
+    cin = 16
+    for width, cout, count, stride in ((16, 64, 3, 1), (32, 128, 4, 2), (64, 256, 6, 2), (128, 512, 3, 2)):
+        for i in range(count):
+            s = stride if i == 0 else 1
+            total += conv(cin, width, 1, 1, size)[0]
+            f, out = conv(width, width, 3, s, size)
+            total += f + conv(width, cout, 1, 1, out)[0]
+            if s != 1 or cin != cout:
+                total += conv(cin, cout, 1, s, size)[0]
+            size, cin = out, cout
+    return total + 2.0 * 16 * n * 250 * 512
+
+
+def bench_resnet(args):
+    import torch
+    import phoenix_core_amd as phx
+    from phoenix_core_amd import capi
+    policy = args.policy or "full16"
+    env = {"UPSTRIDE_CONV_FP16_POLICY": policy}
+    if args.mode == 16 or (args.mode == 0 and phx.Context().memory_optimized):
+        env["UPSTRIDE_MEMORY_OPTIMIZED"] = "1"
+    ctx = phx.Context(env)
+    mode = 16 if ctx.memory_optimized else 8
+    n = args.batch
+    dev = torch.device("cuda:0")
+    torch.manual_seed(0x5EED + 5)
+    model = phx.QResNet50(1000, dtype=torch.float16, context=ctx).to(dev).train()
+    images = torch.randn(n, 3, 224, 224, device=dev).half()
+    labels = torch.randint(0, 1000, (n,), device=dev)
+    xq = phx.QResNet50.lift(images)
+
+    def step():
+        model.zero_grad(set_to_none=True)
+        loss = torch.nn.functional.cross_entropy(model(xq).float(), labels)
+        loss.backward()
+        return loss
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    ncalls = 3 * 54
+    capi.profile_enable(ncalls * args.steps)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        loss = step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    kernel_ms = capi.profile_collect(ncalls * args.steps)
+    capi.profile_enable(0)
+    ms_per_step = elapsed / args.steps * 1e3
+    fwd_flops = resnet_flops(n)
+    conv_ms = sum(kernel_ms) / args.steps
+    out = {
+        "metric": METRIC, "value": n / (ms_per_step * 1e-3), "unit": "img/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "%s: quaternion ResNet-50 forward+backward (no optimizer step, as the metric names), "
+                               "N=%d (4N=%d rows), 224x224, 53 quaternion convs + quaternion dense head; batch-norm, "
+                               "ReLU, pooling and cross-entropy by PyTorch" % (RESNET, n, 4 * n),
+                   "product_mode": mode, "fp16_policy": policy},
+        "real_equiv_tflops": 3 * fwd_flops / (ms_per_step * 1e-3) / 1e12,
+        "quaternion_kernel_ms_per_step": conv_ms, "loss": float(loss.detach()),
+    }
+    print(json.dumps(out))
+    return 0
+
+
 def main():
     args = parse()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (--gpus %d refused)" % args.gpus,
               file=sys.stderr)
         return 2
+    if args.workload == RESNET:
+        return bench_resnet(args)
 
     import torch
     import phoenix_core_amd as phx

@@ -130,8 +130,7 @@ int phx_stream_destroy(phx_stream_t stream);
 int phx_stream_synchronize(phx_stream_t stream);
 
 /* Kernel timing for benchmarks.  phx_profile_enable(capacity > 0) allocates `capacity` HIP event
- * pairs for the calling thread; from then on every compute entry point called by that thread
- * brackets its dominant kernel (the MFMA kernel, not the filter packing or the split-K reduction)
+ * pairs for the process; from then on every compute entry point, from whatever thread, brackets its dominant kernel (the MFMA kernel, not the filter packing or the split-K reduction)
  * with the next pair, recorded on the call's stream, until the pairs run out.  Nothing
  * synchronises while recording.  phx_profile_collect() waits for the recorded pairs, writes their
  * elapsed times in call order, returns how many there were through `count` and rearms the pairs.

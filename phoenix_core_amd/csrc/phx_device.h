@@ -9,6 +9,7 @@
 
 namespace phx {
 
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
@@ -40,7 +41,6 @@ __device__ __forceinline__ void stf<_Float16>(_Float16* p, float v) { *p = (_Flo
 // -v for eight packed halves: flip the sign bits with four integer XORs (the generic vector negate
 // lowers to three instructions per register)
 __device__ __forceinline__ f16x8 neg8(const f16x8 v) {
-    typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
     const u32x4 m = {0x80008000u, 0x80008000u, 0x80008000u, 0x80008000u};
     return __builtin_bit_cast(f16x8, __builtin_bit_cast(u32x4, v) ^ m);
 }
@@ -124,9 +124,9 @@ __device__ __forceinline__ int xcd_remap(int hw_id, int total) {
     return xcd * base + (xcd < rem ? xcd : rem) + slot;
 }
 
-// Sixteen zero bytes in device memory: out-of-tensor staging positions load from here, which keeps
-// the staging loads unconditional and free of selects.
-static __device__ __attribute__((aligned(16))) const unsigned int phx_zero_block[4] = {0u, 0u, 0u, 0u};
+// Sixty-four zero bytes in device memory: out-of-tensor staging positions load from here, which
+// keeps the staging loads unconditional and free of selects.
+static __device__ __attribute__((aligned(16))) const unsigned int phx_zero_block[16] = {};
 
 template <typename T>
 __device__ __forceinline__ const T* zero_ptr() {

@@ -94,7 +94,6 @@ __device__ __forceinline__ void stage_load16_pairs(unsigned int (&d)[4][8], cons
 
 __device__ __forceinline__ void stage_store16_pairs(f16x8* dst, const unsigned int (&d)[4][8], const StagePairPos& sp,
                                                     int pitch) {
-    typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
     if (sp.inwin) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
@@ -117,7 +116,7 @@ __device__ __forceinline__ void stage_store16_pairs(f16x8* dst, const unsigned i
 //   MODE 16: 16 MFMAs per step and column tile, the four filter components reused across the
 //            4x4 block, negative entries by flipping the sign bits of the activation operand.
 //   MODE 8 : 8 MFMAs per step and column tile on lanes formed with packed fp16 adds.
-template <int MODE, int MAP, int WCO, int NTW, int P2LOG>
+template <int MODE, int MAP, int WCO, int NTW, int P2LOG, bool PAIRS>
 __global__ void __launch_bounds__(WG_THREADS, (MODE == 8 || NTW == 1) ? 2 : 1) qconv_fwd_f16_kernel(const ConvArgs P) {
     constexpr int CK = F16_CK;
     constexpr int WPX = 4 / WCO;
@@ -138,6 +137,8 @@ __global__ void __launch_bounds__(WG_THREADS, (MODE == 8 || NTW == 1) ? 2 : 1) q
     const int tn = bid / P.tiles_h;
     const int n0 = tn * P.NB, ho0 = th * P.TH, wo0 = tw * P.TW;
     const int h0 = ho0 * P.sh - P.pt, w0 = wo0 * P.sw - P.pl;
+    const int w0e = PAIRS ? (w0 & ~1) : w0;  // pair staging starts the window at an even column
+    const int colshift = w0 - w0e;
 
     int poff[NTW];
     long oaddr[NTW];
@@ -149,7 +150,7 @@ __global__ void __launch_bounds__(WG_THREADS, (MODE == 8 || NTW == 1) ? 2 : 1) q
         const int nb = pix / thw, rem = pix - nb * thw;
         const int r = rem / P.TW, c = rem - r * P.TW;
         pvalid[t] = nb < P.NB && (n0 + nb) < P.in.N && (ho0 + r) < P.Hout && (wo0 + c) < P.Wout;
-        poff[t] = pvalid[t] ? (nb * P.HTH + r * P.sh) * P.HTW + c * P.sw : 0;
+        poff[t] = pvalid[t] ? (nb * P.HTH + r * P.sh) * P.HTW + c * P.sw + colshift : colshift;
         oaddr[t] = ((long)(n0 + nb) * P.Cout * P.Hout + (ho0 + r)) * P.Wout + (wo0 + c);
     }
 
@@ -169,13 +170,23 @@ __global__ void __launch_bounds__(WG_THREADS, (MODE == 8 || NTW == 1) ? 2 : 1) q
 
     long step = 0;
     const StagePos sp = make_stage_pos<P2LOG>(P.in, n0, h0, w0, P.NB, P.HTH, P.HTW);
-    f16x8 stage[8 >> (8 - P2LOG)];
-    stage_load16<P2LOG>(stage, P.in, sp, 0);
+    const StagePairPos spp = make_stage_pairpos(P.in, n0, h0, w0e, P.NB, P.HTH, P.HTW);
+    f16x8 stage[PAIRS ? 1 : (8 >> (8 - P2LOG))];
+    unsigned int stagep[PAIRS ? 4 : 1][8];
+    auto load_chunk = [&](int c0) {
+        if constexpr (PAIRS) stage_load16_pairs(stagep, P.in, spp, c0);
+        else stage_load16<P2LOG>(stage, P.in, sp, c0);
+    };
+    auto store_chunk = [&]() {
+        if constexpr (PAIRS) stage_store16_pairs(lds16, stagep, spp, P.HPp);
+        else stage_store16<P2LOG>(lds16, stage, sp, P.HP, P.HPp);
+    };
+    load_chunk(0);
     for (int chunk = 0; chunk < P.nchunks; ++chunk) {
         __syncthreads();
-        stage_store16<P2LOG>(lds16, stage, sp, P.HP, P.HPp);
+        store_chunk();
         __syncthreads();
-        if (chunk + 1 < P.nchunks) stage_load16<P2LOG>(stage, P.in, sp, (chunk + 1) * CK);
+        if (chunk + 1 < P.nchunks) load_chunk((chunk + 1) * CK);
         int kh = 0, kw = 0;
         for (int tap = 0; tap < P.taps; ++tap) {
             const int tapoff = kh * P.dh * P.HTW + kw * P.dw;
@@ -510,177 +521,316 @@ __global__ void __launch_bounds__(WG_THREADS) pack_filters_f16_lds_kernel(const 
 }
 
 // ---------------------------------------------------------------------------------------------
-// Filter gradient on fp16 MFMA.  Same decomposition as qconv_wgrad_f32_kernel (64x64 channel tile,
-// tap group = one filter row with up to TPW taps, split-K over pixel tiles, fp32 partial sums
-// reduced by reduce_wgrad_kernel); the reduction index (pixels) is contiguous in NCHW, so both
-// windows are staged as they lie.  One K step = 16 pixels = two 8-pixel packs:
-//   A operand (output gradient): 8 consecutive tile pixels = one aligned 16-byte LDS read;
-//   B operand (input, shifted by the tap): the 8 pixels' window offsets come from a per-tile
-//   table, the 8 halves are gathered with 16-bit LDS reads (any stride / dilation / padding).
+// Filter gradient on fp16 MFMA (v_mfma_f32_16x16x32_f16).  GEMM view per tap: rows = output
+// channels (A operand = output gradient), columns = input channels (B operand = input shifted by
+// the tap), reduction over batch x output pixels -- the contiguous index of NCHW, so both operands
+// are staged as they lie: 16-byte chunks of 8 consecutive pixels of one row.
+//   Reduction space: every output row (n, ho) is cut into ceil(Wo/8) chunks of 8 pixels; a pixel
+//   tile is any 8 consecutive chunks of that list (64 reduction indices, two K steps of 32).
+//   Elements past the row end, padding columns and padding rows are cleared with a per-chunk bit
+//   mask after the (unconditional) load, so the loads themselves are plain 16-byte global loads
+//   at 2-byte alignment.  The few chunks whose load would reach outside the tensor allocation
+//   (first / last rows of the first / last plane) are filled element by element instead.
+//   One workgroup = (CoT x CiT channel tile) x (one filter row kh, TPW adjacent kw) x (slice of
+//   the reduction); CoT = 32*MT, CiT = 32*NT, the 4 waves form a 2x2 grid, each owning MT x NT
+//   MFMA tiles of 16x16 channels for every tap of the group and all four components (16-product:
+//   signs folded into a negated copy of the gradient operand) or all eight lanes (8-product).
+//   TPW == 3 (unit stride and dilation along W): one 10-pixel load per input chunk yields the
+//   three copies shifted by 0/1/2 pixels with byte-align operations; each copy is written to its
+//   own LDS plane so every MFMA operand is one aligned 16-byte LDS read.
+//   SW == 2: the input chunk is 16 consecutive pixels of which the even ones are kept.
+//   Partial sums go to workspace[z]; reduce_wgrad_kernel adds them in a fixed order.
 // ---------------------------------------------------------------------------------------------
-template <int P2LOG>
-__device__ __forceinline__ void stage_load_h2(f16x2 (&v)[(128) >> (8 - P2LOG)], const TileSrc& s, const StagePos& sp,
-                                              int c0) {
-    // 256 planes (4 components x 64 channels), G = 256 >> P2LOG groups, 256/G planes per thread, two per register
-    constexpr int G = WG_THREADS >> P2LOG;
-    constexpr int E = 256 / G;
-    const _Float16* origin = static_cast<const _Float16*>(s.base);
-    const long plane = (long)s.Hd * s.Wd;
-#pragma unroll
-    for (int e = 0; e < E; ++e) {
-        const int pc = e * G + sp.group;
-        const int p = pc >> 6, c = pc & 63;
-        const bool ok = sp.valid && (c0 + c) < s.C;
-        const _Float16* ptr = ok ? origin + sp.goff + p * s.comp_stride + (long)(c0 + c) * plane : zero_ptr<_Float16>();
-        v[e >> 1][e & 1] = *ptr;
-    }
+constexpr int WG16_KP = 64;         // reduction indices per pixel tile
+constexpr int WG16_PITCH = 64 + 8;  // LDS halves per staged channel row (16-byte skew against bank conflicts)
+
+typedef u32x4 u32x4_a2 __attribute__((aligned(2)));
+typedef unsigned int u32_a2 __attribute__((aligned(2)));
+
+__device__ __forceinline__ u32x4 load16_a2(const _Float16* p) {
+    return *reinterpret_cast<const __attribute__((address_space(1))) u32x4_a2*>(
+        (const __attribute__((address_space(1))) _Float16*)p);
+}
+__device__ __forceinline__ unsigned int load4_a2(const _Float16* p) {
+    return *reinterpret_cast<const __attribute__((address_space(1))) u32_a2*>(
+        (const __attribute__((address_space(1))) _Float16*)p);
 }
 
-template <int P2LOG>
-__device__ __forceinline__ void stage_store_h2(_Float16* dst, const f16x2 (&v)[(128) >> (8 - P2LOG)],
-                                               const StagePos& sp, int HP, int pitch) {
-    constexpr int G = WG_THREADS >> P2LOG;
-    constexpr int E = 256 / G;
-    if (sp.pos < HP) {
+// bit i of `bits` set <=> half i of the chunk is kept
+__device__ __forceinline__ u32x4 expand_half_mask(unsigned int bits) {
+    u32x4 mk;
 #pragma unroll
-        for (int e = 0; e < E; ++e) dst[(e * G + sp.group) * pitch + sp.pos] = v[e >> 1][e & 1];
+    for (int d = 0; d < 4; ++d) {
+        const unsigned int lo = (unsigned int)((int)(bits << (31 - 2 * d)) >> 31);
+        const unsigned int hi = (unsigned int)((int)(bits << (30 - 2 * d)) >> 31);
+        mk[d] = (lo & 0x0000FFFFu) | (hi & 0xFFFF0000u);
     }
+    return mk;
 }
 
-template <int MODE, int TPW>
+// bits [lo, hi) set, both clamped to [0, 8]
+__device__ __forceinline__ unsigned int interval_bits(int lo, int hi) {
+    lo = lo < 0 ? 0 : lo;
+    hi = hi > 8 ? 8 : hi;
+    return hi > lo ? ((1u << hi) - (1u << lo)) : 0u;
+}
+
+struct WgChunk {  // where one 8-pixel chunk of the reduction space lies
+    bool live;    // inside the reduction space
+    int n, ho, wo0;
+};
+
+__device__ __forceinline__ WgChunk wg_chunk(const WgradArgs& P, int tile, int j) {
+    WgChunk c;
+    const int gi = tile * 8 + j;
+    c.live = gi < P.nchunks;
+    const int row = gi / P.cpr;
+    c.wo0 = (gi - row * P.cpr) * 8;
+    c.n = row / P.g.Hd;
+    c.ho = row - c.n * P.g.Hd;
+    return c;
+}
+
+template <int MODE, int MT, int NT, int TPW, int SW>
 __global__ void __launch_bounds__(WG_THREADS) qconv_wgrad_f16_kernel(const WgradArgs P) {
-    constexpr int CT = 64;
-    constexpr int NACC = (MODE == 16) ? 4 : 8;
-    constexpr int P2LOG = 6;  // 64 window positions x 4 plane groups
+    static_assert(TPW == 1 || (TPW == 3 && SW == 1), "shifted copies need unit stride");
+    constexpr int CoT = 32 * MT, CiT = 32 * NT;
+    constexpr int NL = (MODE == 16) ? 4 : 8;  // accumulators per (tap, tile): components or lanes
+    constexpr int KPp = WG16_PITCH;
+    constexpr int GE = 4 * MT, XE = 4 * NT;                  // chunks per thread and tile: gradient / input planes
+    constexpr int XR = (TPW == 3) ? 5 : (SW == 2 ? 8 : 4);   // dwords loaded per input chunk
     extern __shared__ f16x8 lds16[];
-    _Float16* gl = reinterpret_cast<_Float16*>(lds16);   // [4][CT][KPp], KPp multiple of 8 (16-byte rows)
-    _Float16* xl = gl + 4 * CT * P.KPp;                    // [4][CT][HPp]
-    int* poff = reinterpret_cast<int*>(xl + 4 * CT * P.HPp);  // [KP], 16-byte aligned
+    _Float16* gl = reinterpret_cast<_Float16*>(lds16);  // [4][CoT][KPp]
+    _Float16* xl = gl + 4 * CoT * KPp;                   // [TPW][4][CiT][KPp]
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wco = wave & 1, wci = wave >> 1;
-    const int m = lane & 31, kk = lane >> 5;
-    const int cot = blockIdx.x % P.co_tiles, cit = blockIdx.x / P.co_tiles;
-    const int kh = blockIdx.y / P.groups_per_row;
-    const int kw0 = (blockIdx.y % P.groups_per_row) * TPW;
+    const int wm = wave & 1, wn = wave >> 1;
+    const int m = lane & 15, kb = lane >> 4;
+    // workgroups that share a reduction slice read the same gradient / input rows: keep them on one XCD
+    int bid = xcd_remap(blockIdx.x, gridDim.x);
+    const int cot = bid % P.co_tiles;  bid /= P.co_tiles;
+    const int cit = bid % P.ci_tiles;  bid /= P.ci_tiles;
+    const int ngroups = P.groups_per_row * P.Kh;
+    const int grp = bid % ngroups;
+    const int zi = bid / ngroups;
+    const int kh = grp / P.groups_per_row;
+    const int kw0 = (grp % P.groups_per_row) * TPW;
     const int nkw = (P.Kw - kw0 < TPW) ? P.Kw - kw0 : TPW;
-    const int HTW = (P.TW - 1) * P.sw + (nkw - 1) * P.dw + 1;
-    const int thw = P.TH * P.TW;
-    const int npix = P.NB * thw;
 
-    for (int k = tid; k < P.KP; k += WG_THREADS) {
-        const int nb = k / thw, rem = k - nb * thw;
-        const int r = rem / P.TW, c = rem - r * P.TW;
-        poff[k] = (k < npix) ? (nb * P.HTH + r * P.sh) * HTW + c * P.sw : 0;
-    }
+    // staging role: chunk j of the tile, planes pg + 32*i of every component
+    const int j = tid & 7, pg = tid >> 3;
+    const int Ho = P.g.Hd, Wo = P.g.Wd, H = P.x.Hd, W = P.x.Wd;
+    const long gplane = (long)Ho * Wo, xplane = (long)H * W;
+    const _Float16* gbase = static_cast<const _Float16*>(P.g.base);
+    const _Float16* xbase = static_cast<const _Float16*>(P.x.base);
+    const _Float16* gend = gbase + 3 * P.g.comp_stride + (long)P.g.N * P.g.C * gplane;
+    const _Float16* xend = xbase + 3 * P.x.comp_stride + (long)P.x.N * P.x.C * xplane;
+    const int co_first = cot * CoT + pg, ci_first = cit * CiT + pg;
 
-    f32x16 acc[TPW][NACC];
+    f32x4 acc[TPW][MT][NT][NL];
 #pragma unroll
     for (int t = 0; t < TPW; ++t)
 #pragma unroll
-        for (int a = 0; a < NACC; ++a)
+        for (int i = 0; i < MT; ++i)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) acc[t][a][r] = 0.f;
+            for (int jn = 0; jn < NT; ++jn)
+#pragma unroll
+                for (int a = 0; a < NL; ++a) acc[t][i][jn][a] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    const int ntiles = P.tiles_n * P.tiles_h * P.tiles_w;
-    const long gcp = (long)CT * P.KPp, xcp = (long)CT * P.HPp;
-    f16x2 sg[32], sx[32];
-    StagePos spg, spx;
+    u32x4 sg[GE];
+    unsigned int sx[XE][XR];
+    unsigned int gbits = 0, xbits[TPW];
+    bool careful = false;  // this thread's chunk of the tile in flight is filled element by element
+
+    auto xcol0 = [&](const WgChunk& c) { return c.wo0 * SW + kw0 * P.dw - P.pl; };
+    auto xrow = [&](const WgChunk& c) { return c.ho * P.sh + kh * P.dh - P.pt; };
+
     auto issue = [&](int tile) {
-        const int tw = tile % P.tiles_w;
-        const int th = (tile / P.tiles_w) % P.tiles_h;
-        const int tn = tile / (P.tiles_w * P.tiles_h);
-        const int n0 = tn * P.NB, ho0 = th * P.TH, wo0 = tw * P.TW;
-        spg = make_stage_pos<P2LOG>(P.g, n0, ho0, wo0, P.NB, P.TH, P.TW);
-        spx = make_stage_pos<P2LOG>(P.x, n0, ho0 * P.sh - P.pt + kh * P.dh, wo0 * P.sw - P.pl + kw0 * P.dw, P.NB, P.HTH,
-                                    HTW);
-        stage_load_h2<P2LOG>(sg, P.g, spg, cot * CT);
-        stage_load_h2<P2LOG>(sx, P.x, spx, cit * CT);
-    };
-    const int HPx = P.NB * P.HTH * HTW;
-    if ((int)blockIdx.z < ntiles) issue(blockIdx.z);
-    for (int tile = blockIdx.z; tile < ntiles; tile += gridDim.z) {
-        __syncthreads();
-        stage_store_h2<P2LOG>(gl, sg, spg, npix, P.KPp);
-        stage_store_h2<P2LOG>(xl, sx, spx, HPx, P.HPp);
-        // reduction indices beyond the tile's pixels must contribute zero
-        for (int i = tid; i < 4 * CT * (P.KP - npix); i += WG_THREADS) {
-            const int c = i / (P.KP - npix), k = npix + i % (P.KP - npix);
-            gl[c * P.KPp + k] = (_Float16)0;
-        }
-        __syncthreads();
-        if (tile + (int)gridDim.z < ntiles) issue(tile + gridDim.z);
-
-        const _Float16* ga = gl + (wco * 32 + m) * P.KPp + kk * 8;
-        const _Float16* xb = xl + (wci * 32 + m) * P.HPp;
-        for (int ks = 0; ks < P.KP; ks += 16) {
-            f16x8 g[4];
+        const WgChunk c = wg_chunk(P, tile, j);
+        const int left = Wo - c.wo0;  // pixels of the row from the chunk start
+        gbits = c.live ? interval_bits(0, left) : 0u;
+        const int hi = xrow(c), wi0 = xcol0(c);
+        const bool rowok = c.live && hi >= 0 && hi < H;
 #pragma unroll
-            for (int q = 0; q < 4; ++q) g[q] = *reinterpret_cast<const f16x8*>(ga + q * gcp + ks);
-            int po[8];
-            {
-                const int4 a = *reinterpret_cast<const int4*>(poff + ks + kk * 8);
-                const int4 b = *reinterpret_cast<const int4*>(poff + ks + kk * 8 + 4);
-                po[0] = a.x; po[1] = a.y; po[2] = a.z; po[3] = a.w;
-                po[4] = b.x; po[5] = b.y; po[6] = b.z; po[7] = b.w;
+        for (int t = 0; t < TPW; ++t) {
+            const int c0 = wi0 + t * P.dw;  // input column of the chunk's first pixel for tap t
+            const int lo = SW == 1 ? -c0 : (1 - c0) >> 1;
+            const int up = SW == 1 ? W - c0 : (W - c0 + 1) >> 1;
+            xbits[t] = (rowok && t < nkw) ? (interval_bits(lo, up < left ? up : left)) : 0u;
+        }
+        const _Float16* gp = gbase + ((long)c.n * P.g.C * Ho + c.ho) * Wo + c.wo0 + (long)co_first * gplane;
+        const _Float16* xp = xbase + ((long)c.n * P.x.C * H + hi) * W + wi0 + (long)ci_first * xplane;
+        // would any of this thread's vector loads leave the tensors?
+        const _Float16* gmax = gp + 3 * P.g.comp_stride + (long)(32 * (MT - 1)) * gplane + 8;
+        const _Float16* xmax = xp + 3 * P.x.comp_stride + (long)(32 * (NT - 1)) * xplane + 2 * XR;
+        careful = (c.live && gmax > gend) || (rowok && (xp < xbase || xmax > xend));
+        const bool gok = c.live && !careful, xok = rowok && !careful;
+#pragma unroll
+        for (int e = 0; e < GE; ++e) {
+            const int q = e / MT, cc = (e % MT) * 32;
+            const bool ok = gok && co_first + cc < P.g.C;
+            sg[e] = load16_a2(ok ? gp + q * P.g.comp_stride + cc * gplane : zero_ptr<_Float16>());
+        }
+#pragma unroll
+        for (int e = 0; e < XE; ++e) {
+            const int q = e / NT, cc = (e % NT) * 32;
+            const bool ok = xok && ci_first + cc < P.x.C;
+            const _Float16* ptr = ok ? xp + q * P.x.comp_stride + cc * xplane : zero_ptr<_Float16>();
+            const u32x4 a = load16_a2(ptr);
+            sx[e][0] = a[0]; sx[e][1] = a[1]; sx[e][2] = a[2]; sx[e][3] = a[3];
+            if constexpr (XR == 5) sx[e][4] = load4_a2(ptr + 8);
+            if constexpr (XR == 8) {
+                const u32x4 b = load16_a2(ptr + 8);
+                sx[e][4] = b[0]; sx[e][5] = b[1]; sx[e][6] = b[2]; sx[e][7] = b[3];
             }
-            f16x8 G[8];
-            if constexpr (MODE == 8) lanes_grad(g, G, (_Float16)0.5f);
+        }
+    };
+
+    // element-wise fill of this thread's chunk (cold: only next to the ends of the tensors)
+    auto fill_careful = [&](int tile) {
+        const WgChunk c = wg_chunk(P, tile, j);
+        const int hi = xrow(c), wi0 = xcol0(c);
+        const bool rowok = c.live && hi >= 0 && hi < H;
+#pragma unroll 1
+        for (int e = 0; e < GE; ++e) {
+            const int q = e / MT, cc = (e % MT) * 32;
+            const _Float16* src = gbase + q * P.g.comp_stride + (((long)c.n * P.g.C + co_first + cc) * Ho + c.ho) * Wo + c.wo0;
+#pragma unroll 1
+            for (int i = 0; i < 8; ++i) {
+                const bool ok = c.live && co_first + cc < P.g.C && c.wo0 + i < Wo;
+                gl[(q * CoT + cc + pg) * KPp + j * 8 + i] = ok ? src[i] : (_Float16)0;
+            }
+        }
+#pragma unroll 1
+        for (int t = 0; t < nkw; ++t)
+#pragma unroll 1
+            for (int e = 0; e < XE; ++e) {
+                const int q = e / NT, cc = (e % NT) * 32;
+                const _Float16* src = xbase + q * P.x.comp_stride + (((long)c.n * P.x.C + ci_first + cc) * H + hi) * W;
+#pragma unroll 1
+                for (int i = 0; i < 8; ++i) {
+                    const int col = wi0 + t * P.dw + i * SW;
+                    const bool ok = rowok && ci_first + cc < P.x.C && c.wo0 + i < Wo && col >= 0 && col < W;
+                    xl[((t * 4 + q) * CiT + cc + pg) * KPp + j * 8 + i] = ok ? src[col] : (_Float16)0;
+                }
+            }
+    };
+
+    const int ntiles = P.ntiles;
+    if (zi < ntiles) issue(zi);
+    for (int tile = zi; tile < ntiles; tile += P.zsplit) {
+        __syncthreads();
+        {
+            const u32x4 mg = expand_half_mask(gbits);
+#pragma unroll
+            for (int e = 0; e < GE; ++e) {
+                const int q = e / MT, cc = (e % MT) * 32;
+                *reinterpret_cast<u32x4*>(gl + (q * CoT + cc + pg) * KPp + j * 8) = sg[e] & mg;
+            }
 #pragma unroll
             for (int t = 0; t < TPW; ++t) {
                 if (t < nkw) {
-                    f16x8 x[4];
+                    const u32x4 mx = expand_half_mask(xbits[t]);
 #pragma unroll
-                    for (int p = 0; p < 4; ++p)
+                    for (int e = 0; e < XE; ++e) {
+                        const int q = e / NT, cc = (e % NT) * 32;
+                        u32x4 v;
+                        if constexpr (XR == 8) {
 #pragma unroll
-                        for (int i = 0; i < 8; ++i) x[p][i] = xb[p * xcp + po[i] + t * P.dw];
-                    if constexpr (MODE == 16) {
-                        f16x8 nx[4];
+                            for (int d = 0; d < 4; ++d) v[d] = __builtin_amdgcn_perm(sx[e][2 * d + 1], sx[e][2 * d], 0x05040100u);
+                        } else if (t == 1) {
 #pragma unroll
-                        for (int p = 0; p < 4; ++p) nx[p] = neg8(x[p]);
+                            for (int d = 0; d < 4; ++d) v[d] = __builtin_amdgcn_alignbyte(sx[e][(d + 1) % XR], sx[e][d], 2);
+                        } else {
+#pragma unroll
+                            for (int d = 0; d < 4; ++d) v[d] = sx[e][(d + (t >> 1)) % XR];
+                        }
+                        *reinterpret_cast<u32x4*>(xl + ((t * 4 + q) * CiT + cc + pg) * KPp + j * 8) = v & mx;
+                    }
+                }
+            }
+            if (careful) fill_careful(tile);
+        }
+        __syncthreads();
+        if (tile + P.zsplit < ntiles) issue(tile + P.zsplit);
+
+#pragma unroll
+        for (int ks = 0; ks < WG16_KP; ks += 32) {
+            f16x8 g[MT][4], ng[MT][4];
+#pragma unroll
+            for (int i = 0; i < MT; ++i)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    g[i][q] = *reinterpret_cast<const f16x8*>(gl + (q * CoT + (wm * MT + i) * 16 + m) * KPp + ks + kb * 8);
+                    if constexpr (MODE == 16) ng[i][q] = neg8(g[i][q]);
+                }
+#pragma unroll
+            for (int t = 0; t < TPW; ++t) {
+                if (t < nkw) {
+#pragma unroll
+                    for (int jn = 0; jn < NT; ++jn) {
+                        f16x8 x[4];
 #pragma unroll
                         for (int p = 0; p < 4; ++p)
+                            x[p] = *reinterpret_cast<const f16x8*>(xl + ((t * 4 + p) * CiT + (wn * NT + jn) * 16 + m) * KPp +
+                                                                   ks + kb * 8);
+                        if constexpr (MODE == 16) {
 #pragma unroll
-                            for (int q = 0; q < 4; ++q)
-                                acc[t][p ^ q] = __builtin_amdgcn_mfma_f32_32x32x16_f16(g[q], qneg(p, q) ? nx[p] : x[p],
-                                                                                       acc[t][p ^ q], 0, 0, 0);
-                    } else {
-                        f16x8 L[8];
-                        lanes_left(x, L);
+                            for (int i = 0; i < MT; ++i)
 #pragma unroll
-                        for (int i = 0; i < 8; ++i)
-                            acc[t][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(G[i], L[i], acc[t][i], 0, 0, 0);
+                                for (int p = 0; p < 4; ++p)
+#pragma unroll
+                                    for (int q = 0; q < 4; ++q)
+                                        acc[t][i][jn][p ^ q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                                            qneg(p, q) ? ng[i][q] : g[i][q], x[p], acc[t][i][jn][p ^ q], 0, 0, 0);
+                        } else {
+                            f16x8 L[8];
+                            lanes_left(x, L);
+#pragma unroll
+                            for (int i = 0; i < MT; ++i) {
+                                f16x8 Gl[8];
+                                lanes_grad(g[i], Gl, (_Float16)0.5f);
+#pragma unroll
+                                for (int l = 0; l < 8; ++l)
+                                    acc[t][i][jn][l] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Gl[l], L[l], acc[t][i][jn][l], 0, 0, 0);
+                            }
+                        }
                     }
                 }
             }
         }
     }
 
+    // partial[z][tap][r][co][ci]; D tile: lane holds column ci = lane % 16, rows co = 4*(lane/16) + 0..3
     const int taps = P.Kh * P.Kw;
     const long tap_stride = 4L * P.CoP * P.CiP;
-    float* dst = P.partial + (long)blockIdx.z * taps * tap_stride;
-    const int ci = cit * CT + wci * 32 + m;
-    const int co_base = cot * CT + wco * 32 + 4 * kk;
+    float* dst = P.partial + (long)zi * taps * tap_stride;
 #pragma unroll
     for (int t = 0; t < TPW; ++t) {
         if (t >= nkw) continue;
         float* d = dst + (long)(kh * P.Kw + kw0 + t) * tap_stride;
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-            const int co = co_base + 8 * (e >> 2) + (e & 3);
-            float y[4];
-            if constexpr (MODE == 16) {
+        for (int i = 0; i < MT; ++i)
 #pragma unroll
-                for (int r = 0; r < 4; ++r) y[r] = acc[t][r][e];
-            } else {
-                float l[8];
+            for (int jn = 0; jn < NT; ++jn) {
+                const int ci = cit * CiT + (wn * NT + jn) * 16 + m;
+                const int co_base = cot * CoT + (wm * MT + i) * 16 + 4 * kb;
 #pragma unroll
-                for (int i = 0; i < 8; ++i) l[i] = acc[t][i][e];
-                merge_right_grad(l, y);
+                for (int e = 0; e < 4; ++e) {
+                    float y[4];
+                    if constexpr (MODE == 16) {
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) y[r] = acc[t][i][jn][r][e];
+                    } else {
+                        float l[8];
+#pragma unroll
+                        for (int a = 0; a < 8; ++a) l[a] = acc[t][i][jn][a][e];
+                        merge_right_grad(l, y);
+                    }
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) d[((long)r * P.CoP + co_base + e) * P.CiP + ci] = y[r];
+                }
             }
-#pragma unroll
-            for (int r = 0; r < 4; ++r) d[((long)r * P.CoP + co) * P.CiP + ci] = y[r];
-        }
     }
 }
 

@@ -258,6 +258,7 @@ struct WgradArgs {
     int tiles_n, tiles_h, tiles_w;
     int co_tiles, ci_tiles, CoP, CiP;
     int groups_per_row; // tap groups per filter row
+    int cpr, nchunks, ntiles, zsplit;  // fp16 kernel: 8-pixel chunks per output row / in total, pixel tiles, reduction slices
 };
 
 template <typename TS, int MODE, int TPW>

@@ -4,15 +4,16 @@
 
 namespace phx {
 
-template <int MODE, int MAP>
+template <int MODE, int MAP, bool PAIRS>
 static int launch_variant16(const FwdVariant& v, const ConvArgs& a, hipStream_t st) {
+    constexpr int P2A = 8, P2B = PAIRS ? 8 : 7;  // the pair path has a single staging shape
 #define PHX_CASE(WCO_, NTW_, P2_)                                                                             \
-    if (v.WCO == WCO_ && v.NTW == NTW_ && v.P2LOG == P2_) {                                                   \
-        hipLaunchKernelGGL((qconv_fwd_f16_kernel<MODE, MAP, WCO_, NTW_, P2_>), dim3(v.wgs), dim3(WG_THREADS), \
-                           v.lds_bytes, st, a);                                                               \
+    if (v.WCO == WCO_ && v.NTW == NTW_ && (PAIRS || v.P2LOG == P2_)) {                                        \
+        hipLaunchKernelGGL((qconv_fwd_f16_kernel<MODE, MAP, WCO_, NTW_, P2_, PAIRS>), dim3(v.wgs),            \
+                           dim3(WG_THREADS), v.lds_bytes, st, a);                                             \
         return 0;                                                                                             \
     }
-#define PHX_CASES(WCO_, NTW_) PHX_CASE(WCO_, NTW_, 8) PHX_CASE(WCO_, NTW_, 7)
+#define PHX_CASES(WCO_, NTW_) PHX_CASE(WCO_, NTW_, P2A) PHX_CASE(WCO_, NTW_, P2B)
     PHX_CASES(1, 1) PHX_CASES(2, 1) PHX_CASES(4, 1)
     if constexpr (MODE == 16) {
         PHX_CASES(1, 2) PHX_CASES(2, 2) PHX_CASES(4, 2)
@@ -20,6 +21,13 @@ static int launch_variant16(const FwdVariant& v, const ConvArgs& a, hipStream_t 
 #undef PHX_CASES
 #undef PHX_CASE
     return -1;
+}
+
+template <bool PAIRS>
+static int launch_v1(const FwdVariant& v, const ConvArgs& a, hipStream_t st) {
+    if (v.mode == 16) return launch_variant16<16, MAP_FWD, PAIRS>(v, a, st);
+    if (v.map == MAP_FWD) return launch_variant16<8, MAP_FWD, PAIRS>(v, a, st);
+    return launch_variant16<8, MAP_DGRAD, PAIRS>(v, a, st);
 }
 
 template <bool PAIRS>
@@ -40,9 +48,7 @@ static int launch_lds16(const FwdVariant& v, const ConvArgs& a, hipStream_t st) 
 
 int launch_fwd_f16(const FwdVariant& v, const ConvArgs& a, hipStream_t st) {
     if (v.lds_filters) return v.pairs ? launch_lds16<true>(v, a, st) : launch_lds16<false>(v, a, st);
-    if (v.mode == 16) return launch_variant16<16, MAP_FWD>(v, a, st);
-    if (v.map == MAP_FWD) return launch_variant16<8, MAP_FWD>(v, a, st);
-    return launch_variant16<8, MAP_DGRAD>(v, a, st);
+    return v.pairs ? launch_v1<true>(v, a, st) : launch_v1<false>(v, a, st);
 }
 
 int launch_pack_filters_f16(const FwdVariant& v, const PackArgs& a, int blocks, hipStream_t st) {

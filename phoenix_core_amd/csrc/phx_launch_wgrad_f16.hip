@@ -1,14 +1,39 @@
-// Instantiations of the fp16-MFMA filter-gradient kernels.
+// fp16-MFMA filter-gradient kernels, 16-product, three taps per workgroup; dispatch over all variants.
 #include "phx_kernels_f16.h"
 #include "phx_launch.h"
 
 namespace phx {
 
-int launch_wgrad_f16(int mode, const WgradArgs& a, dim3 grid, size_t lds_bytes, hipStream_t st) {
-    const dim3 b(WG_THREADS);
-    if (mode == 16) hipLaunchKernelGGL((qconv_wgrad_f16_kernel<16, 3>), grid, b, lds_bytes, st, a);
-    else hipLaunchKernelGGL((qconv_wgrad_f16_kernel<8, 1>), grid, b, lds_bytes, st, a);
+template <int MODE, int MT, int NT, int TPW, int SW>
+static int launch_one(const WgradArgs& a, int nblocks, size_t lds_bytes, hipStream_t st) {
+    auto kernel = qconv_wgrad_f16_kernel<MODE, MT, NT, TPW, SW>;
+    static bool raised = false;  // dynamic LDS above the default 64 KiB needs an explicit opt-in
+    if (!raised && lds_bytes > 64 * 1024) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                160 * 1024) != hipSuccess) {
+            (void)hipGetLastError();
+            return -1;
+        }
+        raised = true;
+    }
+    hipLaunchKernelGGL(kernel, dim3(nblocks), dim3(WG_THREADS), lds_bytes, st, a);
     return 0;
+}
+
+int launch_wgrad_f16_p16t3(int MT, int NT, const WgradArgs& a, int nblocks, size_t lds_bytes, hipStream_t st) {
+#define PHX_CASE(MT_, NT_) \
+    if (MT == MT_ && NT == NT_) return launch_one<16, MT_, NT_, 3, 1>(a, nblocks, lds_bytes, st);
+    PHX_CASE(1, 1) PHX_CASE(1, 2) PHX_CASE(2, 1) PHX_CASE(2, 2)
+#undef PHX_CASE
+    return -1;
+}
+
+int launch_wgrad_f16(int mode, int MT, int NT, int TPW, int SW, const WgradArgs& a, int nblocks, size_t lds_bytes,
+                     hipStream_t st) {
+    if (mode == 16 && TPW == 3 && SW == 1) return launch_wgrad_f16_p16t3(MT, NT, a, nblocks, lds_bytes, st);
+    if (TPW != 1) return -1;
+    return mode == 16 ? launch_wgrad_f16_p16(MT, NT, 1, SW, a, nblocks, lds_bytes, st)
+                      : launch_wgrad_f16_p8(MT, NT, SW, a, nblocks, lds_bytes, st);
 }
 
 }  // namespace phx

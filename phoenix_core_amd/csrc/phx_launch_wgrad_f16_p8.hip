@@ -1,0 +1,33 @@
+// fp16-MFMA filter-gradient kernels, 8-product.
+#include "phx_kernels_f16.h"
+#include "phx_launch.h"
+
+namespace phx {
+
+template <int MODE, int MT, int NT, int TPW, int SW>
+static int launch_one(const WgradArgs& a, int nblocks, size_t lds_bytes, hipStream_t st) {
+    auto kernel = qconv_wgrad_f16_kernel<MODE, MT, NT, TPW, SW>;
+    static bool raised = false;  // dynamic LDS above the default 64 KiB needs an explicit opt-in
+    if (!raised && lds_bytes > 64 * 1024) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                160 * 1024) != hipSuccess) {
+            (void)hipGetLastError();
+            return -1;
+        }
+        raised = true;
+    }
+    hipLaunchKernelGGL(kernel, dim3(nblocks), dim3(WG_THREADS), lds_bytes, st, a);
+    return 0;
+}
+
+int launch_wgrad_f16_p8(int MT, int NT, int SW, const WgradArgs& a, int nblocks, size_t lds_bytes, hipStream_t st) {
+#define PHX_CASE(MT_, NT_)                                                                     \
+    if (MT == MT_ && NT == NT_)                                                                \
+        return SW == 1 ? launch_one<8, MT_, NT_, 1, 1>(a, nblocks, lds_bytes, st)              \
+                       : launch_one<8, MT_, NT_, 1, 2>(a, nblocks, lds_bytes, st);
+    PHX_CASE(1, 1) PHX_CASE(1, 2) PHX_CASE(2, 1) PHX_CASE(2, 2)
+#undef PHX_CASE
+    return -1;
+}
+
+}  // namespace phx

@@ -6,6 +6,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <vector>
 
 #include "phx_launch.h"
@@ -21,13 +22,16 @@ struct ProfileState {
     int used = 0;
     bool on = false;
 };
-static thread_local ProfileState g_prof;
+static ProfileState g_prof;  // process-wide: frameworks run backward passes on their own threads
+static std::mutex g_prof_mutex;
 
 struct KernelTimer {
     hipStream_t st;
     int slot;
     explicit KernelTimer(hipStream_t s) : st(s), slot(-1) {
-        if (g_prof.on && 2 * (g_prof.used + 1) <= (int)g_prof.ev.size()) {
+        if (!g_prof.on) return;
+        std::lock_guard<std::mutex> lock(g_prof_mutex);
+        if (2 * (g_prof.used + 1) <= (int)g_prof.ev.size()) {
             slot = g_prof.used++;
             (void)hipEventRecord(g_prof.ev[2 * slot], st);
         }
@@ -170,7 +174,8 @@ constexpr int LDS_FLOATS_MAX = 16384;  // 64 KiB: two workgroups per CU
 static bool plan_forward(const Corr& c, int mode, bool f16mfma, FwdPlan& best) {
     double best_score = -1.0;
     // fp16 MFMA with filters in LDS: stage activations as aligned pairs when rows are even
-    const bool pairs = f16mfma && mode == 16 && c.Kh * c.Kw > 1 && (c.Win % 2 == 0) && c.uw == 1;
+    const bool pairs = f16mfma && (c.Win % 2 == 0) && c.uw == 1;
+    const bool ldsk = f16mfma && mode == 16 && c.Kh * c.Kw > 1;  // filters through LDS
     best.pairs = pairs;
     const int wcos[3] = {1, 2, 4};
     // PHX_TUNE_TILE="wco,ntw" pins the workgroup shape (kernel tuning experiments)
@@ -208,7 +213,7 @@ static bool plan_forward(const Corr& c, int mode, bool f16mfma, FwdPlan& best) {
                     double score = eff * (0.25 + 0.75 * fill) * (0.9 + 0.1 * halo) * (NTW == 2 ? 1.02 : 1.0);
                     // fp16 MFMA is operand-bandwidth hungry: two column tiles per wave and two filter
                     // sub-tiles per workgroup amortise LDS reads and activation staging (measured)
-                    if (pairs) score *= (NTW == 2 ? 1.25 : 1.0) * (WCO == 2 ? 1.08 : 1.0);
+                    if (ldsk) score *= (NTW == 2 ? 1.25 : 1.0) * (WCO == 2 ? 1.08 : 1.0);
                     else if (f16mfma && NTW == 2) score *= 0.8;  // that kernel drops to one workgroup per CU
                     if (score > best_score) {
                         best_score = score;
@@ -232,7 +237,7 @@ static bool plan_forward(const Corr& c, int mode, bool f16mfma, FwdPlan& best) {
         best.nchunks = cdiv(c.Cin, best.CK);
         best.lds_bytes = (size_t)8 * best.HPp * 16;
         best.wpk_bytes = (size_t)best.co_tiles * best.WCO * best.nchunks * taps * 64 * WC * 16;
-        best.lds_filters = (mode == 16 && taps > 1);
+        best.lds_filters = ldsk;
         best.ngroups = cdiv(taps, F16_TG);
         if (best.lds_filters) {
             const size_t wimg = (size_t)F16_TG * best.WCO * 4 * 64 * 16;  // one filter group image
@@ -319,28 +324,39 @@ static int run_corr(const Problem& p, const Corr& c, int map, hipStream_t st, co
 struct WgPlan {
     int TPW, NB, TH, TW, KP, KPp, HPp, HPx, HTH, HTWmax;
     int tiles_n, tiles_h, tiles_w, co_tiles, ci_tiles, CoP, CiP, groups_per_row, Z;
+    int MT, NT;  // fp16 kernel: 32*MT x 32*NT channel tile
+    int SW, cpr, nchunks, ntiles;  // fp16 kernel: stride along W, 8-pixel chunks per output row / in total, pixel tiles
     size_t lds_bytes, partial_bytes;
 };
 
-static bool plan_wgrad(const Problem& p, bool f16mfma, WgPlan& best) {
+static void finish_wgrad_plan(const Problem& p, int CoT, int CiT, WgPlan& best) {
+    best.co_tiles = cdiv(p.co, CoT); best.ci_tiles = cdiv(p.ci, CiT);
+    best.CoP = best.co_tiles * CoT; best.CiP = best.ci_tiles * CiT;
+    best.groups_per_row = cdiv(p.kw, best.TPW);
+    const int xy = best.co_tiles * best.ci_tiles * best.groups_per_row * p.kh;
+    const int ntiles = best.tiles_n * best.tiles_h * best.tiles_w;
+    best.Z = std::max(1, std::min(ntiles, 1024 / std::max(1, xy)));
+    best.partial_bytes = (size_t)best.Z * p.kh * p.kw * 4 * best.CoP * best.CiP * sizeof(float);
+}
+
+// fp32-MFMA kernel: 64x64 channel tiles, pixel tile and input window of at most 32 positions
+static bool plan_wgrad_f32(const Problem& p, WgPlan& best) {
     const int TPW = (p.mode == 16) ? 3 : 1;
     const int nkw = std::min(TPW, p.kw);
     double best_score = -1.0;
     const int budget = LDS_FLOATS_MAX / (4 * 64);  // KPp + HPp (+ offsets) per staged channel
-    const int maxpos = f16mfma ? 64 : 32;  // staging positions per window
     for (int TW = 1; TW <= std::min(p.wo, 64); ++TW) {
         for (int TH = 1; TH <= p.ho; ++TH) {
             for (int NB = 1; NB <= p.n; ++NB) {
                 if (NB > 1 && !(TH == p.ho && TW == p.wo)) break;
                 const int pix = NB * TH * TW;
-                const int KP = f16mfma ? (pix + 15) & ~15 : (pix + 1) & ~1;
+                const int KP = (pix + 1) & ~1;
                 const int HTH = (TH - 1) * p.sh + 1;
                 const int HTW = (TW - 1) * p.sw + (nkw - 1) * p.dw + 1;
                 const int HPx = NB * HTH * HTW;
-                // fp32: odd pitches (bank-conflict-free 4-byte reads); fp16: 16-byte rows plus one 16-byte skew
-                const int KPp = f16mfma ? KP + 8 : KP | 1, HPp = f16mfma ? ((HPx + 7) & ~7) + 8 : HPx | 1;
-                if (pix > maxpos || HPx > maxpos) break;
-                if (!f16mfma && KPp + HPp + (KP + 255) / 256 > budget) break;
+                const int KPp = KP | 1, HPp = HPx | 1;  // odd pitches: bank-conflict-free 4-byte reads
+                if (pix > 32 || HPx > 32) break;
+                if (KPp + HPp + (KP + 255) / 256 > budget) break;
                 const int tn = cdiv(p.n, NB), th = cdiv(p.ho, TH), tw = cdiv(p.wo, TW);
                 const double eff = ((double)p.n * p.ho * p.wo) / ((double)tn * th * tw * KP);
                 const double score = eff * (1.0 + 0.002 * KP) * (TW >= std::min(p.wo, 8) ? 1.0 : 0.5);
@@ -354,21 +370,48 @@ static bool plan_wgrad(const Problem& p, bool f16mfma, WgPlan& best) {
         }
     }
     if (best_score < 0) return false;
-    best.co_tiles = cdiv(p.co, 64); best.ci_tiles = cdiv(p.ci, 64);
-    best.CoP = best.co_tiles * 64; best.CiP = best.ci_tiles * 64;
-    best.groups_per_row = cdiv(p.kw, TPW);
-    const int xy = best.co_tiles * best.ci_tiles * best.groups_per_row * p.kh;
-    const int ntiles = best.tiles_n * best.tiles_h * best.tiles_w;
-    best.Z = std::max(1, std::min(ntiles, 512 / std::max(1, xy)));
-    best.lds_bytes = f16mfma ? (size_t)4 * 64 * (best.KPp + best.HPp) * 2 + (size_t)best.KP * 4 + 16
-                             : ((size_t)4 * 64 * (best.KPp + best.HPp) + best.KP) * sizeof(float);
-    best.partial_bytes = (size_t)best.Z * p.kh * p.kw * 4 * best.CoP * best.CiP * sizeof(float);
+    best.MT = best.NT = 2;
+    finish_wgrad_plan(p, 64, 64, best);
+    best.lds_bytes = ((size_t)4 * 64 * (best.KPp + best.HPp) + best.KP) * sizeof(float);
     return true;
+}
+
+// fp16-MFMA kernel: 32*MT x 32*NT channel tiles; reduction over 8-pixel chunks of the output rows, 8 chunks per tile
+static bool plan_wgrad_f16(const Problem& p, WgPlan& best) {
+    best = WgPlan{};
+    best.SW = p.sw;
+    best.TPW = (p.mode == 16 && p.kw > 1 && p.sw == 1 && p.dw == 1) ? 3 : 1;
+    best.MT = p.co > 32 ? 2 : 1;
+    best.NT = p.ci > 32 ? 2 : 1;
+    if (const char* e = getenv("PHX_TUNE_WG")) sscanf(e, "%d,%d", &best.MT, &best.NT);
+    const int CoT = 32 * best.MT, CiT = 32 * best.NT;
+    best.cpr = cdiv(p.wo, 8);
+    const long nchunks = (long)p.n * p.ho * best.cpr;
+    if (nchunks > (1L << 28)) return false;
+    best.nchunks = (int)nchunks;
+    best.ntiles = cdiv(best.nchunks, 8);
+    best.co_tiles = cdiv(p.co, CoT); best.ci_tiles = cdiv(p.ci, CiT);
+    best.CoP = best.co_tiles * CoT; best.CiP = best.ci_tiles * CiT;
+    best.groups_per_row = cdiv(p.kw, best.TPW);
+    const int xy = best.co_tiles * best.ci_tiles * best.groups_per_row * p.kh;
+    best.Z = std::max(1, std::min(best.ntiles, 1024 / std::max(1, xy)));
+    best.partial_bytes = (size_t)best.Z * p.kh * p.kw * 4 * best.CoP * best.CiP * sizeof(float);
+    best.lds_bytes = (size_t)(4 * CoT + best.TPW * 4 * CiT) * 72 * 2;
+    return true;
+}
+
+// strides along W other than 1 and 2 have no fp16-MFMA filter-gradient kernel: fp32 arithmetic serves them
+static bool wgrad_on_f16_mfma(const Problem& p) {
+    return use_f16_mfma(p, PHX_PASS_BWD_WEIGHTS) && (p.sw == 1 || p.sw == 2);
+}
+
+static bool plan_wgrad(const Problem& p, bool f16mfma, WgPlan& best) {
+    return f16mfma ? plan_wgrad_f16(p, best) : plan_wgrad_f32(p, best);
 }
 
 static int run_wgrad(const Problem& p, hipStream_t st, const void* x, const void* g, void* dw, void* ws,
                      size_t ws_bytes) {
-    const bool f16 = use_f16_mfma(p, PHX_PASS_BWD_WEIGHTS);
+    const bool f16 = wgrad_on_f16_mfma(p);
     WgPlan pl;
     if (!plan_wgrad(p, f16, pl)) return PHX_ERR_NOT_SUPPORTED;
     if (ws_bytes < pl.partial_bytes || !ws) return PHX_ERR_WORKSPACE;
@@ -384,12 +427,18 @@ static int run_wgrad(const Problem& p, hipStream_t st, const void* x, const void
     a.tiles_n = pl.tiles_n; a.tiles_h = pl.tiles_h; a.tiles_w = pl.tiles_w;
     a.co_tiles = pl.co_tiles; a.ci_tiles = pl.ci_tiles; a.CoP = pl.CoP; a.CiP = pl.CiP;
     a.groups_per_row = pl.groups_per_row;
+    a.cpr = pl.cpr; a.nchunks = pl.nchunks; a.ntiles = pl.ntiles; a.zsplit = pl.Z;
+    const int nblocks16 = pl.co_tiles * pl.ci_tiles * pl.groups_per_row * p.kh * pl.Z;
     const dim3 grid(pl.co_tiles * pl.ci_tiles, pl.groups_per_row * p.kh, pl.Z);
     const bool half_storage = p.dtype == PHX_F16;
     {
         KernelTimer timer(st);
-        if (f16) launch_wgrad_f16(p.mode, a, grid, pl.lds_bytes, st);
-        else launch_wgrad_f32(half_storage, p.mode, a, grid, pl.lds_bytes, st);
+        if (f16) {
+            if (launch_wgrad_f16(p.mode, pl.MT, pl.NT, pl.TPW, pl.SW, a, nblocks16, pl.lds_bytes, st) != 0)
+                return PHX_ERR_RUNTIME;
+        } else {
+            launch_wgrad_f32(half_storage, p.mode, a, grid, pl.lds_bytes, st);
+        }
     }
     PHX_HIP(hipGetLastError());
     ReduceArgs r;
@@ -400,8 +449,12 @@ static int run_wgrad(const Problem& p, hipStream_t st, const void* x, const void
     const int blocks = (int)((items + 31) / 32);
     launch_reduce_wgrad(half_storage, r, blocks, st);
     PHX_HIP(hipGetLastError());
-    snprintf(g_name_buf, sizeof(g_name_buf), "qconv_wgrad_%smfma_p%d_%s_tile%dx%dx%d_z%d", f16 ? "f16" : "f32", p.mode,
-             p.dtype == PHX_F32 ? "f32" : "f16", pl.NB, pl.TH, pl.TW, pl.Z);
+    if (f16)
+        snprintf(g_name_buf, sizeof(g_name_buf), "qconv_wgrad_f16mfma_p%d_f16_ch%dx%d_taps%d_sw%d_z%d", p.mode, 32 * pl.MT,
+                 32 * pl.NT, pl.TPW, pl.SW, pl.Z);
+    else
+        snprintf(g_name_buf, sizeof(g_name_buf), "qconv_wgrad_f32mfma_p%d_%s_tile%dx%dx%d_z%d", p.mode,
+                 p.dtype == PHX_F32 ? "f32" : "f16", pl.NB, pl.TH, pl.TW, pl.Z);
     g_last_kernel = g_name_buf;
     return PHX_OK;
 }
@@ -410,7 +463,7 @@ static size_t workspace_for(const Problem& p, int pass) {
     if (is_empty(p)) return 0;
     if (pass == PHX_PASS_BWD_WEIGHTS) {
         WgPlan pl;
-        return plan_wgrad(flatten_pointwise(p), use_f16_mfma(p, pass), pl) ? align_up(pl.partial_bytes, 256) : 0;
+        return plan_wgrad(flatten_pointwise(p), wgrad_on_f16_mfma(p), pl) ? align_up(pl.partial_bytes, 256) : 0;
     }
     const Corr c = (pass == PHX_PASS_FWD) ? corr_forward(p) : corr_dgrad(p);
     FwdPlan pl;
@@ -466,6 +519,7 @@ const char* phx_status_string(int status) {
 const char* phx_last_kernel_name(void) { return g_last_kernel; }
 
 int phx_profile_enable(int capacity) {
+    std::lock_guard<std::mutex> lock(g_prof_mutex);
     g_prof.on = false;
     g_prof.used = 0;
     if (capacity <= 0) return PHX_OK;
@@ -480,6 +534,7 @@ int phx_profile_enable(int capacity) {
 
 int phx_profile_collect(float* milliseconds, int max_count, int* count) {
     if (!count || (max_count > 0 && !milliseconds)) return PHX_ERR_INVALID_ARGUMENT;
+    std::lock_guard<std::mutex> lock(g_prof_mutex);
     const int n = std::min(g_prof.used, max_count);
     for (int i = 0; i < n; ++i) {
         PHX_HIP(hipEventSynchronize(g_prof.ev[2 * i + 1]));

@@ -1,0 +1,167 @@
+"""torch.autograd wrappers over the quaternion operators and a quaternion ResNet-50.
+
+The reference engine was consumed by an external framework plugin that registered its operators
+with gradients; this module plays that role for PyTorch.  QConv2d / QLinear hold the reference's
+tensor layouts (components stacked on the batch axis, filters [4, Co, Ci, Kh, Kw], dense filters
+[4, I, O]); every forward / backward call goes through the HIP library.  The ResNet-50 below is
+the standard bottleneck stack with every channel count divided by four (quaternion channels);
+batch-norm, ReLU, pooling and the loss are plain PyTorch (the reference has no model code).
+"""
+import math
+
+import torch
+from torch import nn
+
+from . import ops
+
+
+class _QConv2dFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, w, bias, fdesc, bdesc):
+        ctx.save_for_backward(x, w)
+        ctx.bdesc = bdesc
+        ctx.has_bias = bias is not None
+        return ops.conv2d_fwd(x, w, bias, fdesc)
+
+    @staticmethod
+    def backward(ctx, grad):
+        x, w = ctx.saved_tensors
+        grad = grad.contiguous()
+        dw, dx = ops.conv2d_bwd(x, w, grad, ctx.bdesc)
+        db = None
+        if ctx.has_bias:  # bias enters every output component once: plain reduction
+            n = grad.shape[0] // 4
+            db = grad.view(4, n, grad.shape[1], -1).float().sum(dim=(1, 3)).to(grad.dtype)
+        return dx, dw, db, None, None
+
+
+class _QLinearFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, w, bias, fdesc, bdesc):
+        ctx.save_for_backward(x, w)
+        ctx.bdesc = bdesc
+        ctx.has_bias = bias is not None
+        return ops.dense_fwd(x, w, bias, fdesc)
+
+    @staticmethod
+    def backward(ctx, grad):
+        x, w = ctx.saved_tensors
+        grad = grad.contiguous()
+        dw, dx = ops.dense_bwd(x, w, grad, ctx.bdesc)
+        db = None
+        if ctx.has_bias:
+            n = grad.shape[0] // 4
+            db = grad.view(4, n, -1).float().sum(dim=1).to(grad.dtype)
+        return dx, dw, db, None, None
+
+
+class QConv2d(nn.Module):
+    """Quaternion Conv2D: x [4N, Ci, H, W] -> y [4N, Co, Ho, Wo]; padding 'SAME' / 'VALID' as in
+    the reference's descriptors (src/backend/conv2d_descriptor.hpp:132-174)."""
+
+    def __init__(self, in_channels, out_channels, kernel_size, stride=1, padding="SAME", dilation=1, bias=False,
+                 dtype=torch.float32, context=None, input_requires_grad=True):
+        super().__init__()
+        k = (kernel_size, kernel_size) if isinstance(kernel_size, int) else tuple(kernel_size)
+        self.stride, self.padding, self.dilation = stride, padding, dilation
+        self.context = context
+        self.input_requires_grad = input_requires_grad
+        fan_in = in_channels * k[0] * k[1]
+        w = torch.randn(4, out_channels, in_channels, k[0], k[1]) * math.sqrt(2.0 / fan_in)  # He-normal per component
+        self.weight = nn.Parameter(w.to(dtype))
+        self.bias = nn.Parameter(torch.zeros(4, out_channels, dtype=dtype)) if bias else None
+        self._descs = {}
+
+    def _descriptors(self, x):
+        key = (tuple(x.shape), x.dtype)
+        if key not in self._descs:
+            common = dict(stride=self.stride, dilation=self.dilation, padding=self.padding, dtype=x.dtype,
+                          context=self.context)
+            fwd = ops.Conv2DDescriptor(x.shape, self.weight.shape, use_bias=self.bias is not None, **common)
+            bwd = ops.Conv2DDescriptor(x.shape, self.weight.shape, require_input_grad=self.input_requires_grad, **common)
+            self._descs[key] = (fwd, bwd)
+        return self._descs[key]
+
+    def forward(self, x):
+        fwd, bwd = self._descriptors(x)
+        return _QConv2dFn.apply(x.contiguous(), self.weight, self.bias, fwd, bwd)
+
+
+class QLinear(nn.Module):
+    """Quaternion Dense: x [4N, I] -> y [4N, O], filter layout IO."""
+
+    def __init__(self, in_features, out_features, bias=True, dtype=torch.float32, context=None):
+        super().__init__()
+        lim = math.sqrt(6.0 / (in_features + out_features))  # Glorot-uniform per component
+        self.weight = nn.Parameter(torch.empty(4, in_features, out_features).uniform_(-lim, lim).to(dtype))
+        self.bias = nn.Parameter(torch.zeros(4, out_features, dtype=dtype)) if bias else None
+        self.context = context
+        self._descs = {}
+
+    def forward(self, x):
+        key = (tuple(x.shape), x.dtype)
+        if key not in self._descs:
+            fwd = ops.DenseDescriptor(x.shape, self.weight.shape, use_bias=self.bias is not None, dtype=x.dtype,
+                                      context=self.context)
+            bwd = ops.DenseDescriptor(x.shape, self.weight.shape, dtype=x.dtype, context=self.context)
+            self._descs[key] = (fwd, bwd)
+        fwd, bwd = self._descs[key]
+        return _QLinearFn.apply(x.contiguous(), self.weight, self.bias, fwd, bwd)
+
+
+class _Bottleneck(nn.Module):
+    def __init__(self, cin, width, cout, stride, dtype, context):
+        super().__init__()
+        mk = lambda ci, co, k, s: QConv2d(ci, co, k, stride=s, padding="SAME", dtype=dtype, context=context)
+        self.conv1, self.bn1 = mk(cin, width, 1, 1), nn.BatchNorm2d(width)
+        self.conv2, self.bn2 = mk(width, width, 3, stride), nn.BatchNorm2d(width)
+        self.conv3, self.bn3 = mk(width, cout, 1, 1), nn.BatchNorm2d(cout)
+        self.down = None
+        if stride != 1 or cin != cout:
+            self.down = nn.Sequential(mk(cin, cout, 1, stride), nn.BatchNorm2d(cout))
+        self.relu = nn.ReLU(inplace=True)
+
+    def forward(self, x):
+        idt = x if self.down is None else self.down(x)
+        y = self.relu(self.bn1(self.conv1(x)))
+        y = self.relu(self.bn2(self.conv2(y)))
+        y = self.bn3(self.conv3(y))
+        return self.relu(y + idt)
+
+
+class QResNet50(nn.Module):
+    """ResNet-50 with quaternion channels = real channels / 4: stem 3->16 (7x7 s2), stages of
+    (3, 4, 6, 3) bottlenecks with widths 16/32/64/128 and outputs 64/128/256/512, head = quaternion
+    Dense 512 -> 250 units (= 1000 logits).  53 convolutions."""
+
+    def __init__(self, num_classes=1000, dtype=torch.float32, context=None):
+        super().__init__()
+        assert num_classes % 4 == 0
+        self.stem = QConv2d(3, 16, 7, stride=2, padding="SAME", dtype=dtype, context=context, input_requires_grad=False)
+        self.bn = nn.BatchNorm2d(16)
+        self.relu = nn.ReLU(inplace=True)
+        self.pool = nn.MaxPool2d(3, 2, 1)
+        blocks, cin = [], 16
+        for width, cout, count, stride in ((16, 64, 3, 1), (32, 128, 4, 2), (64, 256, 6, 2), (128, 512, 3, 2)):
+            for i in range(count):
+                blocks.append(_Bottleneck(cin, width, cout, stride if i == 0 else 1, dtype, context))
+                cin = cout
+        self.blocks = nn.Sequential(*blocks)
+        self.head = QLinear(512, num_classes // 4, bias=True, dtype=dtype, context=context)
+
+    @staticmethod
+    def lift(images):
+        """Real images [N, 3, H, W] -> quaternion input [4N, 3, H, W]: real part = image, imaginary parts zero."""
+        z = torch.zeros_like(images)
+        return torch.cat([images, z, z, z], dim=0)
+
+    def forward(self, xq):
+        y = self.pool(self.relu(self.bn(self.stem(xq))))
+        y = self.blocks(y)
+        y = y.float().mean(dim=(2, 3)).to(xq.dtype)           # [4N, 512]
+        y = self.head(y)                                      # [4N, 250]
+        n = y.shape[0] // 4
+        return y.view(4, n, -1).permute(1, 0, 2).reshape(n, -1)  # [N, 1000]: the four components side by side
+
+    def conv_layers(self):
+        return [m for m in self.modules() if isinstance(m, QConv2d)]
