@@ -568,17 +568,46 @@ __device__ __forceinline__ u32x4 expand_half_mask(unsigned int bits) {
     return mk;
 }
 
-// bits [lo, hi) set, both clamped to [0, 8]
+// bits [lo, hi) set, both clamped to [0, MAXB]
+template <int MAXB = 8>
 __device__ __forceinline__ unsigned int interval_bits(int lo, int hi) {
     lo = lo < 0 ? 0 : lo;
-    hi = hi > 8 ? 8 : hi;
+    hi = hi > MAXB ? MAXB : hi;
     return hi > lo ? ((1u << hi) - (1u << lo)) : 0u;
 }
 
 struct WgChunk {  // where one 8-pixel chunk of the reduction space lies
     bool live;    // inside the reduction space
     int n, ho, wo0;
+    int gi;       // index in the chunk list
 };
+
+struct WgStep {   // advance of a thread's chunk from one of its tiles to the next (uniform)
+    int dgi, dwo, dho, dn;
+};
+
+__device__ __forceinline__ WgStep wg_step(const WgradArgs& P) {
+    WgStep s;
+    s.dgi = 8 * P.zsplit;
+    const int drow = s.dgi / P.cpr;
+    s.dwo = (s.dgi - drow * P.cpr) * 8;
+    s.dn = drow / P.g.Hd;
+    s.dho = drow - s.dn * P.g.Hd;
+    return s;
+}
+
+// the same chunk position one tile step later, without divisions
+__device__ __forceinline__ void wg_advance(WgChunk& c, const WgStep& s, const WgradArgs& P) {
+    c.gi += s.dgi;
+    c.live = c.gi < P.nchunks;
+    c.wo0 += s.dwo;
+    const bool c1 = c.wo0 >= P.cpr * 8;
+    c.wo0 -= c1 ? P.cpr * 8 : 0;
+    c.ho += s.dho + (c1 ? 1 : 0);
+    const bool c2 = c.ho >= P.g.Hd;
+    c.ho -= c2 ? P.g.Hd : 0;
+    c.n += s.dn + (c2 ? 1 : 0);
+}
 
 __device__ __forceinline__ WgChunk wg_chunk(const WgradArgs& P, int tile, int j) {
     WgChunk c;
@@ -588,6 +617,7 @@ __device__ __forceinline__ WgChunk wg_chunk(const WgradArgs& P, int tile, int j)
     c.wo0 = (gi - row * P.cpr) * 8;
     c.n = row / P.g.Hd;
     c.ho = row - c.n * P.g.Hd;
+    c.gi = gi;
     return c;
 }
 
@@ -615,7 +645,7 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_wgrad_f16_kernel(const Wgrad
     const int zi = bid / ngroups;
     const int kh = grp / P.groups_per_row;
     const int kw0 = (grp % P.groups_per_row) * TPW;
-    const int nkw = (P.Kw - kw0 < TPW) ? P.Kw - kw0 : TPW;
+    constexpr int nkw = TPW;  // tap groups are always full
 
     // staging role: chunk j of the tile, planes pg + 32*i of every component
     const int j = tid & 7, pg = tid >> 3;
@@ -623,214 +653,357 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_wgrad_f16_kernel(const Wgrad
     const long gplane = (long)Ho * Wo, xplane = (long)H * W;
     const _Float16* gbase = static_cast<const _Float16*>(P.g.base);
     const _Float16* xbase = static_cast<const _Float16*>(P.x.base);
-    const _Float16* gend = gbase + 3 * P.g.comp_stride + (long)P.g.N * P.g.C * gplane;
-    const _Float16* xend = xbase + 3 * P.x.comp_stride + (long)P.x.N * P.x.C * xplane;
     const int co_first = cot * CoT + pg, ci_first = cit * CiT + pg;
 
-    f32x4 acc[TPW][MT][NT][NL];
+    // 64x64 channel tiles: one 32x32 MFMA tile per wave (v_mfma_f32_32x32x16_f16 sustains its full rate from a
+    // single wave per SIMD, the 16x16 shape does not); smaller tiles: MT x NT tiles of 16x16 per wave
+    constexpr bool BIG = (MT == 2 && NT == 2);
+    f32x4 acc[BIG ? 1 : TPW][MT][NT][NL];
+    f32x16 accb[BIG ? TPW : 1][NL];
 #pragma unroll
-    for (int t = 0; t < TPW; ++t)
+    for (int t = 0; t < (BIG ? 1 : TPW); ++t)
 #pragma unroll
         for (int i = 0; i < MT; ++i)
 #pragma unroll
             for (int jn = 0; jn < NT; ++jn)
 #pragma unroll
                 for (int a = 0; a < NL; ++a) acc[t][i][jn][a] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int t = 0; t < (BIG ? TPW : 1); ++t)
+#pragma unroll
+        for (int a = 0; a < NL; ++a)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) accb[t][a][r] = 0.f;
 
     u32x4 sg[GE];
     unsigned int sx[XE][XR];
-    unsigned int gbits = 0, xbits[TPW];
-    bool careful = false;  // this thread's chunk of the tile in flight is filled element by element
+    u32x4 mg;                // keeps the gradient pixels that lie inside their row
+    unsigned int mx[XR];     // keeps the loaded input columns that lie inside the image
+    bool careful = false;    // this thread's chunk of the tile in flight is filled element by element
 
     auto xcol0 = [&](const WgChunk& c) { return c.wo0 * SW + kw0 * P.dw - P.pl; };
     auto xrow = [&](const WgChunk& c) { return c.ho * P.sh + kh * P.dh - P.pt; };
 
-    auto issue = [&](int tile) {
-        const WgChunk c = wg_chunk(P, tile, j);
-        const int left = Wo - c.wo0;  // pixels of the row from the chunk start
-        gbits = c.live ? interval_bits(0, left) : 0u;
+    // Loads of one tile: every address is (uniform component/plane-group base) + (one 32-bit element
+    // offset per thread), so a tile costs a handful of address instructions.  Chunks outside the
+    // reduction space or on padding rows load from offset 0 and are masked to zero; channels beyond
+    // the tensor re-read its last channel (their rows of the partial result are never reduced).
+    // 32-bit element offsets inside one component: the host guarantees they fit
+    const int gimg = P.g.C * (int)gplane, ximg = P.x.C * (int)xplane;
+    const int gcomp = P.g.N * gimg, xcomp = P.x.N * ximg;  // elements per component
+    int gch[MT], xch[NT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i) gch[i] = (co_first + 32 * i < P.g.C ? co_first + 32 * i : P.g.C - 1) * (int)gplane;
+#pragma unroll
+    for (int i = 0; i < NT; ++i) xch[i] = (ci_first + 32 * i < P.x.C ? ci_first + 32 * i : P.x.C - 1) * (int)xplane;
+
+    unsigned int lgoff[MT], lxoff[NT];  // load offsets of the tile being fetched
+    auto prep = [&](const WgChunk& c) {
         const int hi = xrow(c), wi0 = xcol0(c);
         const bool rowok = c.live && hi >= 0 && hi < H;
+        const int grow = c.n * gimg + c.ho * Wo + c.wo0;
+        const int xrow_off = c.n * ximg + hi * W + wi0;
+        int goff[MT], xoff[NT];
 #pragma unroll
-        for (int t = 0; t < TPW; ++t) {
-            const int c0 = wi0 + t * P.dw;  // input column of the chunk's first pixel for tap t
-            const int lo = SW == 1 ? -c0 : (1 - c0) >> 1;
-            const int up = SW == 1 ? W - c0 : (W - c0 + 1) >> 1;
-            xbits[t] = (rowok && t < nkw) ? (interval_bits(lo, up < left ? up : left)) : 0u;
-        }
-        const _Float16* gp = gbase + ((long)c.n * P.g.C * Ho + c.ho) * Wo + c.wo0 + (long)co_first * gplane;
-        const _Float16* xp = xbase + ((long)c.n * P.x.C * H + hi) * W + wi0 + (long)ci_first * xplane;
+        for (int i = 0; i < MT; ++i) goff[i] = grow + gch[i];
+#pragma unroll
+        for (int i = 0; i < NT; ++i) xoff[i] = xrow_off + xch[i];
         // would any of this thread's vector loads leave the tensors?
-        const _Float16* gmax = gp + 3 * P.g.comp_stride + (long)(32 * (MT - 1)) * gplane + 8;
-        const _Float16* xmax = xp + 3 * P.x.comp_stride + (long)(32 * (NT - 1)) * xplane + 2 * XR;
-        careful = (c.live && gmax > gend) || (rowok && (xp < xbase || xmax > xend));
+        careful = (c.live && goff[MT - 1] + 8 > gcomp) || (rowok && (xoff[0] < 0 || xoff[NT - 1] + 2 * XR > xcomp));
         const bool gok = c.live && !careful, xok = rowok && !careful;
+        mg = expand_half_mask(gok ? interval_bits(0, Wo - c.wo0) : 0u);
+        {
+            const unsigned int bits = xok ? interval_bits<2 * XR>(-wi0, W - wi0) : 0u;
 #pragma unroll
-        for (int e = 0; e < GE; ++e) {
-            const int q = e / MT, cc = (e % MT) * 32;
-            const bool ok = gok && co_first + cc < P.g.C;
-            sg[e] = load16_a2(ok ? gp + q * P.g.comp_stride + cc * gplane : zero_ptr<_Float16>());
+            for (int d = 0; d < XR; ++d) {
+                const unsigned int lo = (unsigned int)((int)(bits << (31 - 2 * d)) >> 31);
+                const unsigned int up = (unsigned int)((int)(bits << (30 - 2 * d)) >> 31);
+                mx[d] = (lo & 0x0000FFFFu) | (up & 0xFFFF0000u);
+            }
         }
 #pragma unroll
-        for (int e = 0; e < XE; ++e) {
-            const int q = e / NT, cc = (e % NT) * 32;
-            const bool ok = xok && ci_first + cc < P.x.C;
-            const _Float16* ptr = ok ? xp + q * P.x.comp_stride + cc * xplane : zero_ptr<_Float16>();
-            const u32x4 a = load16_a2(ptr);
-            sx[e][0] = a[0]; sx[e][1] = a[1]; sx[e][2] = a[2]; sx[e][3] = a[3];
-            if constexpr (XR == 5) sx[e][4] = load4_a2(ptr + 8);
-            if constexpr (XR == 8) {
+        for (int i = 0; i < MT; ++i) lgoff[i] = (unsigned int)(gok ? goff[i] : 0);
+#pragma unroll
+        for (int i = 0; i < NT; ++i) lxoff[i] = (unsigned int)(xok ? xoff[i] : 0);
+    };
+    // the load instructions of a tile, one "slot" each, so that they can be spread over the MFMA blocks:
+    // a wave that issues them back to back stalls until the memory pipeline has taken them all
+    constexpr int XL = (XR == 4) ? 1 : 2;          // load instructions per input chunk
+    constexpr int NLOADS = GE + XE * XL;
+    auto load_slot = [&](int sl) {
+        if (sl < GE) {
+            sg[sl] = load16_a2(gbase + (sl / MT) * P.g.comp_stride + lgoff[sl % MT]);
+        } else if (sl < NLOADS) {
+            const int e = (sl - GE) / XL, part = (sl - GE) % XL;
+            const _Float16* ptr = xbase + (e / NT) * P.x.comp_stride + lxoff[e % NT];
+            if (part == 0) {
+                const u32x4 a = load16_a2(ptr);
+                sx[e][0] = a[0]; sx[e][1] = a[1]; sx[e][2] = a[2]; sx[e][3] = a[3];
+            } else if constexpr (XR == 5) {
+                sx[e][4] = load4_a2(ptr + 8);
+            } else if constexpr (XR == 8) {
                 const u32x4 b = load16_a2(ptr + 8);
                 sx[e][4] = b[0]; sx[e][5] = b[1]; sx[e][6] = b[2]; sx[e][7] = b[3];
             }
         }
     };
 
-    // element-wise fill of this thread's chunk (cold: only next to the ends of the tensors)
+    // element-wise fill of this thread's chunk (only next to the ends of the tensors).  The loads of
+    // one plane are independent of each other, so their latencies overlap.
     auto fill_careful = [&](int tile) {
+        constexpr int NEL = 7 * SW + TPW;  // input columns one chunk touches over all taps of the group
         const WgChunk c = wg_chunk(P, tile, j);
         const int hi = xrow(c), wi0 = xcol0(c);
         const bool rowok = c.live && hi >= 0 && hi < H;
-#pragma unroll 1
+#pragma unroll 2
         for (int e = 0; e < GE; ++e) {
             const int q = e / MT, cc = (e % MT) * 32;
-            const _Float16* src = gbase + q * P.g.comp_stride + (((long)c.n * P.g.C + co_first + cc) * Ho + c.ho) * Wo + c.wo0;
-#pragma unroll 1
-            for (int i = 0; i < 8; ++i) {
-                const bool ok = c.live && co_first + cc < P.g.C && c.wo0 + i < Wo;
-                gl[(q * CoT + cc + pg) * KPp + j * 8 + i] = ok ? src[i] : (_Float16)0;
-            }
+            const int ch = co_first + cc < P.g.C ? co_first + cc : P.g.C - 1;
+            const _Float16* src = gbase + q * P.g.comp_stride + (((long)c.n * P.g.C + ch) * Ho + c.ho) * Wo + c.wo0;
+            _Float16 v[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[i] = (c.live && c.wo0 + i < Wo) ? src[i] : (_Float16)0;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) gl[(q * CoT + cc + pg) * KPp + j * 8 + i] = v[i];
         }
-#pragma unroll 1
-        for (int t = 0; t < nkw; ++t)
-#pragma unroll 1
-            for (int e = 0; e < XE; ++e) {
-                const int q = e / NT, cc = (e % NT) * 32;
-                const _Float16* src = xbase + q * P.x.comp_stride + (((long)c.n * P.x.C + ci_first + cc) * H + hi) * W;
-#pragma unroll 1
-                for (int i = 0; i < 8; ++i) {
-                    const int col = wi0 + t * P.dw + i * SW;
-                    const bool ok = rowok && ci_first + cc < P.x.C && c.wo0 + i < Wo && col >= 0 && col < W;
-                    xl[((t * 4 + q) * CiT + cc + pg) * KPp + j * 8 + i] = ok ? src[col] : (_Float16)0;
-                }
+#pragma unroll 2
+        for (int e = 0; e < XE; ++e) {
+            const int q = e / NT, cc = (e % NT) * 32;
+            const int ch = ci_first + cc < P.x.C ? ci_first + cc : P.x.C - 1;
+            const _Float16* src = xbase + q * P.x.comp_stride + (((long)c.n * P.x.C + ch) * H + hi) * W;
+            _Float16 w[NEL];
+#pragma unroll
+            for (int k = 0; k < NEL; ++k) {
+                const int col = wi0 + k;
+                w[k] = (rowok && col >= 0 && col < W) ? src[col] : (_Float16)0;
             }
+#pragma unroll
+            for (int t = 0; t < TPW; ++t)
+#pragma unroll
+                for (int i = 0; i < 8; ++i) xl[((t * 4 + q) * CiT + cc + pg) * KPp + j * 8 + i] = w[i * SW + t];
+        }
     };
 
     const int ntiles = P.ntiles;
-    if (zi < ntiles) issue(zi);
+    const WgStep step = wg_step(P);
+    WgChunk nextc = wg_chunk(P, zi, j);
+    prep(nextc);
+#pragma unroll
+    for (int sl = 0; sl < NLOADS; ++sl) load_slot(sl);
+#ifdef PHX_EXP_TIMING
+    long long tph[5] = {0, 0, 0, 0, 0};
+#define PHX_STAMP(i) { __builtin_amdgcn_sched_barrier(0); const long long now = clock64(); tph[i] += now - tlast; tlast = now; __builtin_amdgcn_sched_barrier(0); }
+    long long tlast = clock64();
+#else
+#define PHX_STAMP(i)
+#endif
     for (int tile = zi; tile < ntiles; tile += P.zsplit) {
         __syncthreads();
+        PHX_STAMP(0)
         {
-            const u32x4 mg = expand_half_mask(gbits);
 #pragma unroll
             for (int e = 0; e < GE; ++e) {
                 const int q = e / MT, cc = (e % MT) * 32;
                 *reinterpret_cast<u32x4*>(gl + (q * CoT + cc + pg) * KPp + j * 8) = sg[e] & mg;
             }
 #pragma unroll
-            for (int t = 0; t < TPW; ++t) {
-                if (t < nkw) {
-                    const u32x4 mx = expand_half_mask(xbits[t]);
+            for (int e = 0; e < XE; ++e) {
+                const int q = e / NT, cc = (e % NT) * 32;
+                unsigned int w[XR];
 #pragma unroll
-                    for (int e = 0; e < XE; ++e) {
-                        const int q = e / NT, cc = (e % NT) * 32;
-                        u32x4 v;
-                        if constexpr (XR == 8) {
+                for (int d = 0; d < XR; ++d) w[d] = sx[e][d] & mx[d];
 #pragma unroll
-                            for (int d = 0; d < 4; ++d) v[d] = __builtin_amdgcn_perm(sx[e][2 * d + 1], sx[e][2 * d], 0x05040100u);
-                        } else if (t == 1) {
+                for (int t = 0; t < TPW; ++t) {
+                    u32x4 v;
+                    if constexpr (XR == 8) {
 #pragma unroll
-                            for (int d = 0; d < 4; ++d) v[d] = __builtin_amdgcn_alignbyte(sx[e][(d + 1) % XR], sx[e][d], 2);
-                        } else {
+                        for (int d = 0; d < 4; ++d) v[d] = __builtin_amdgcn_perm(w[2 * d + 1], w[2 * d], 0x05040100u);
+                    } else if (t == 1) {
 #pragma unroll
-                            for (int d = 0; d < 4; ++d) v[d] = sx[e][(d + (t >> 1)) % XR];
-                        }
-                        *reinterpret_cast<u32x4*>(xl + ((t * 4 + q) * CiT + cc + pg) * KPp + j * 8) = v & mx;
+                        for (int d = 0; d < 4; ++d) v[d] = __builtin_amdgcn_alignbyte(w[(d + 1) % XR], w[d], 2);
+                    } else {
+#pragma unroll
+                        for (int d = 0; d < 4; ++d) v[d] = w[(d + (t >> 1)) % XR];
                     }
+                    *reinterpret_cast<u32x4*>(xl + ((t * 4 + q) * CiT + cc + pg) * KPp + j * 8) = v;
                 }
             }
             if (careful) fill_careful(tile);
         }
+        PHX_STAMP(1)
         __syncthreads();
-        if (tile + P.zsplit < ntiles) issue(tile + P.zsplit);
+        PHX_STAMP(2)
+        // the next tile's loads and masks are issued without a branch (past the end they turn into
+        // masked loads of offset 0), so that they interleave with the multiplications below
+        wg_advance(nextc, step, P);
+        prep(nextc);  // free to mix with the first MFMA block
+        PHX_STAMP(3)
 
+        if constexpr (BIG) {
+            // blocks b = (K step of 16, tap); lane = (channel row/column lane % 32, K half lane / 32)
+            constexpr int NBLK = (WG16_KP / 16) * TPW;
+            const int m32 = lane & 31, kb2 = lane >> 5;
+            f16x8 gf[2][4], xf[2][4];
+            auto read_g = [&](f16x8 (&g)[4], int ks) {
 #pragma unroll
-        for (int ks = 0; ks < WG16_KP; ks += 32) {
-            f16x8 g[MT][4], ng[MT][4];
+                for (int q = 0; q < 4; ++q)
+                    g[q] = *reinterpret_cast<const f16x8*>(gl + (q * CoT + wm * 32 + m32) * KPp + ks * 16 + kb2 * 8);
+            };
+            auto read_x = [&](f16x8 (&x)[4], int blk) {
+                const int ks = blk / TPW, t = blk % TPW;
+#pragma unroll
+                for (int p = 0; p < 4; ++p)
+                    x[p] = *reinterpret_cast<const f16x8*>(xl + ((t * 4 + p) * CiT + wn * 32 + m32) * KPp + ks * 16 + kb2 * 8);
+            };
+            read_g(gf[0], 0);
+            read_x(xf[0], 0);
+            constexpr int LPB = (NLOADS + NBLK - 1) / NBLK;  // global loads issued per block
+#pragma unroll
+            for (int blk = 0; blk < NBLK; ++blk) {
+                const int ks = blk / TPW, t = blk % TPW;
+#pragma unroll
+                for (int sl = blk * LPB; sl < (blk + 1) * LPB; ++sl) load_slot(sl);
+                if (blk + 1 < NBLK) {
+                    read_x(xf[(blk + 1) & 1], blk + 1);
+                    if ((blk + 1) % TPW == 0) read_g(gf[(ks + 1) & 1], ks + 1);
+                }
+                __builtin_amdgcn_sched_barrier(0);  // the reads of the next block stay ahead of this block's MFMAs
+                const f16x8(&x)[4] = xf[blk & 1];
+                const f16x8(&g)[4] = gf[ks & 1];
+                if constexpr (MODE == 16) {
+                    f16x8 nx[4];
+#pragma unroll
+                    for (int p = 0; p < 4; ++p) nx[p] = neg8(x[p]);
+#pragma unroll
+                    for (int p = 0; p < 4; ++p)
+#pragma unroll
+                        for (int q = 0; q < 4; ++q)
+                            accb[t][p ^ q] = __builtin_amdgcn_mfma_f32_32x32x16_f16(g[q], qneg(p, q) ? nx[p] : x[p],
+                                                                                   accb[t][p ^ q], 0, 0, 0);
+                } else {
+                    f16x8 L[8], Gl[8];
+                    lanes_left(x, L);
+                    lanes_grad(g, Gl, (_Float16)0.5f);
+#pragma unroll
+                    for (int l = 0; l < 8; ++l)
+                        accb[t][l] = __builtin_amdgcn_mfma_f32_32x32x16_f16(Gl[l], L[l], accb[t][l], 0, 0, 0);
+                }
+            }
+        } else {
+        // MFMA blocks b = (K step, tap, column tile); the operands of block b+1 are read from LDS while
+        // block b multiplies.  TPW is exact here (the host picks TPW == 3 only for Kw % 3 == 0).
+        constexpr int BPK = TPW * NT;               // blocks per K step
+        constexpr int NBLK = (WG16_KP / 32) * BPK;
+        f16x8 gf[2][MT][4], xf[2][4];
+        auto read_g = [&](f16x8 (&g)[MT][4], int ks) {
 #pragma unroll
             for (int i = 0; i < MT; ++i)
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    g[i][q] = *reinterpret_cast<const f16x8*>(gl + (q * CoT + (wm * MT + i) * 16 + m) * KPp + ks + kb * 8);
-                    if constexpr (MODE == 16) ng[i][q] = neg8(g[i][q]);
-                }
+                for (int q = 0; q < 4; ++q)
+                    g[i][q] = *reinterpret_cast<const f16x8*>(gl + (q * CoT + (wm * MT + i) * 16 + m) * KPp + ks * 32 + kb * 8);
+        };
+        auto read_x = [&](f16x8 (&x)[4], int blk) {
+            const int ks = blk / BPK, t = (blk % BPK) / NT, jn = blk % NT;
 #pragma unroll
-            for (int t = 0; t < TPW; ++t) {
-                if (t < nkw) {
+            for (int p = 0; p < 4; ++p)
+                x[p] = *reinterpret_cast<const f16x8*>(xl + ((t * 4 + p) * CiT + (wn * NT + jn) * 16 + m) * KPp + ks * 32 + kb * 8);
+        };
+        read_g(gf[0], 0);
+        read_x(xf[0], 0);
+        constexpr int LPB = (NLOADS + NBLK - 1) / NBLK;  // global loads issued per block
 #pragma unroll
-                    for (int jn = 0; jn < NT; ++jn) {
-                        f16x8 x[4];
+        for (int blk = 0; blk < NBLK; ++blk) {
+            const int ks = blk / BPK, t = (blk % BPK) / NT, jn = blk % NT;
 #pragma unroll
-                        for (int p = 0; p < 4; ++p)
-                            x[p] = *reinterpret_cast<const f16x8*>(xl + ((t * 4 + p) * CiT + (wn * NT + jn) * 16 + m) * KPp +
-                                                                   ks + kb * 8);
-                        if constexpr (MODE == 16) {
+            for (int sl = blk * LPB; sl < (blk + 1) * LPB; ++sl) load_slot(sl);
+            if (blk + 1 < NBLK) {
+                read_x(xf[(blk + 1) & 1], blk + 1);
+                if ((blk + 1) % BPK == 0) read_g(gf[(ks + 1) & 1], ks + 1);
+            }
+            const f16x8(&x)[4] = xf[blk & 1];
+            const f16x8(&g)[MT][4] = gf[ks & 1];
+            if constexpr (MODE == 16) {
+                f16x8 nx[4];
 #pragma unroll
-                            for (int i = 0; i < MT; ++i)
+                for (int p = 0; p < 4; ++p) nx[p] = neg8(x[p]);
 #pragma unroll
-                                for (int p = 0; p < 4; ++p)
+                for (int i = 0; i < MT; ++i)
 #pragma unroll
-                                    for (int q = 0; q < 4; ++q)
-                                        acc[t][i][jn][p ^ q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-                                            qneg(p, q) ? ng[i][q] : g[i][q], x[p], acc[t][i][jn][p ^ q], 0, 0, 0);
-                        } else {
-                            f16x8 L[8];
-                            lanes_left(x, L);
+                    for (int p = 0; p < 4; ++p)
 #pragma unroll
-                            for (int i = 0; i < MT; ++i) {
-                                f16x8 Gl[8];
-                                lanes_grad(g[i], Gl, (_Float16)0.5f);
+                        for (int q = 0; q < 4; ++q)
+                            acc[t][i][jn][p ^ q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                                g[i][q], qneg(p, q) ? nx[p] : x[p], acc[t][i][jn][p ^ q], 0, 0, 0);
+            } else {
+                f16x8 L[8];
+                lanes_left(x, L);
 #pragma unroll
-                                for (int l = 0; l < 8; ++l)
-                                    acc[t][i][jn][l] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Gl[l], L[l], acc[t][i][jn][l], 0, 0, 0);
-                            }
-                        }
-                    }
+                for (int i = 0; i < MT; ++i) {
+                    f16x8 Gl[8];
+                    lanes_grad(g[i], Gl, (_Float16)0.5f);
+#pragma unroll
+                    for (int l = 0; l < 8; ++l)
+                        acc[t][i][jn][l] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Gl[l], L[l], acc[t][i][jn][l], 0, 0, 0);
                 }
             }
         }
+            }
+        PHX_STAMP(4)
     }
 
-    // partial[z][tap][r][co][ci]; D tile: lane holds column ci = lane % 16, rows co = 4*(lane/16) + 0..3
+#ifdef PHX_EXP_TIMING
+    if ((blockIdx.x % 97) == 0 && lane == 0)
+        printf("wg %d wave %d: bar1 %lld store %lld bar2 %lld issue %lld mfma %lld (per tile, %d tiles)\n", (int)blockIdx.x, wave,
+               tph[0] / 21, tph[1] / 21, tph[2] / 21, tph[3] / 21, tph[4] / 21, (ntiles - zi + P.zsplit - 1) / P.zsplit);
+#endif
+    // partial[z][tap][r][co][ci]
     const int taps = P.Kh * P.Kw;
     const long tap_stride = 4L * P.CoP * P.CiP;
     float* dst = P.partial + (long)zi * taps * tap_stride;
+    auto merged = [&](const float (&l)[NL], float (&y)[4]) {
+        if constexpr (MODE == 16) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) y[r] = l[r];
+        } else {
+            merge_right_grad(l, y);
+        }
+    };
 #pragma unroll
     for (int t = 0; t < TPW; ++t) {
-        if (t >= nkw) continue;
         float* d = dst + (long)(kh * P.Kw + kw0 + t) * tap_stride;
+        if constexpr (BIG) {
+            // 32x32 D tile: lane holds column ci = lane % 32, register e holds row 8*(e/4) + 4*(lane/32) + e%4
+            const int ci = cit * CiT + wn * 32 + (lane & 31);
+            const int co_base = cot * CoT + wm * 32 + 4 * (lane >> 5);
 #pragma unroll
-        for (int i = 0; i < MT; ++i)
+            for (int e = 0; e < 16; ++e) {
+                float l[NL], y[4];
 #pragma unroll
-            for (int jn = 0; jn < NT; ++jn) {
-                const int ci = cit * CiT + (wn * NT + jn) * 16 + m;
-                const int co_base = cot * CoT + (wm * MT + i) * 16 + 4 * kb;
+                for (int a = 0; a < NL; ++a) l[a] = accb[t][a][e];
+                merged(l, y);
+                const int co = co_base + 8 * (e >> 2) + (e & 3);
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    float y[4];
-                    if constexpr (MODE == 16) {
-#pragma unroll
-                        for (int r = 0; r < 4; ++r) y[r] = acc[t][i][jn][r][e];
-                    } else {
-                        float l[8];
-#pragma unroll
-                        for (int a = 0; a < 8; ++a) l[a] = acc[t][i][jn][a][e];
-                        merge_right_grad(l, y);
-                    }
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) d[((long)r * P.CoP + co_base + e) * P.CiP + ci] = y[r];
-                }
+                for (int r = 0; r < 4; ++r) d[((long)r * P.CoP + co) * P.CiP + ci] = y[r];
             }
+        } else {
+            // 16x16 D tiles: lane holds column ci = lane % 16, rows co = 4*(lane/16) + 0..3
+#pragma unroll
+            for (int i = 0; i < MT; ++i)
+#pragma unroll
+                for (int jn = 0; jn < NT; ++jn) {
+                    const int ci = cit * CiT + (wn * NT + jn) * 16 + m;
+                    const int co_base = cot * CoT + (wm * MT + i) * 16 + 4 * kb;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        float l[NL], y[4];
+#pragma unroll
+                        for (int a = 0; a < NL; ++a) l[a] = acc[t][i][jn][a][e];
+                        merged(l, y);
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) d[((long)r * P.CoP + co_base + e) * P.CiP + ci] = y[r];
+                    }
+                }
+        }
     }
 }
 

@@ -380,7 +380,7 @@ static bool plan_wgrad_f32(const Problem& p, WgPlan& best) {
 static bool plan_wgrad_f16(const Problem& p, WgPlan& best) {
     best = WgPlan{};
     best.SW = p.sw;
-    best.TPW = (p.mode == 16 && p.kw > 1 && p.sw == 1 && p.dw == 1) ? 3 : 1;
+    best.TPW = (p.mode == 16 && p.kw % 3 == 0 && p.sw == 1 && p.dw == 1) ? 3 : 1;
     best.MT = p.co > 32 ? 2 : 1;
     best.NT = p.ci > 32 ? 2 : 1;
     if (const char* e = getenv("PHX_TUNE_WG")) sscanf(e, "%d,%d", &best.MT, &best.NT);
@@ -393,16 +393,24 @@ static bool plan_wgrad_f16(const Problem& p, WgPlan& best) {
     best.co_tiles = cdiv(p.co, CoT); best.ci_tiles = cdiv(p.ci, CiT);
     best.CoP = best.co_tiles * CoT; best.CiP = best.ci_tiles * CiT;
     best.groups_per_row = cdiv(p.kw, best.TPW);
-    const int xy = best.co_tiles * best.ci_tiles * best.groups_per_row * p.kh;
-    best.Z = std::max(1, std::min(best.ntiles, 1024 / std::max(1, xy)));
-    best.partial_bytes = (size_t)best.Z * p.kh * p.kw * 4 * best.CoP * best.CiP * sizeof(float);
     best.lds_bytes = (size_t)(4 * CoT + best.TPW * 4 * CiT) * 72 * 2;
+    // one round of workgroups: as many reduction slices as fill every CU once (twice where two workgroups fit),
+    // which keeps the partial sums small and lets no CU wait for a straggler round
+    const int xy = best.co_tiles * best.ci_tiles * best.groups_per_row * p.kh;
+    const int per_cu = best.lds_bytes <= 80 * 1024 ? 2 : 1;
+    int target = 256 * per_cu;
+    if (const char* e = getenv("PHX_TUNE_WGS")) target = atoi(e);
+    best.Z = std::max(1, std::min(best.ntiles, target / std::max(1, xy)));
+    best.partial_bytes = (size_t)best.Z * p.kh * p.kw * 4 * best.CoP * best.CiP * sizeof(float);
     return true;
 }
 
 // strides along W other than 1 and 2 have no fp16-MFMA filter-gradient kernel: fp32 arithmetic serves them
 static bool wgrad_on_f16_mfma(const Problem& p) {
-    return use_f16_mfma(p, PHX_PASS_BWD_WEIGHTS) && (p.sw == 1 || p.sw == 2);
+    // the kernel addresses one component with 32-bit element offsets
+    const long lim = (1L << 31) - 64;
+    return use_f16_mfma(p, PHX_PASS_BWD_WEIGHTS) && (p.sw == 1 || p.sw == 2) && (long)p.n * p.ci * p.h * p.w < lim &&
+           (long)p.n * p.co * p.ho * p.wo < lim;
 }
 
 static bool plan_wgrad(const Problem& p, bool f16mfma, WgPlan& best) {
