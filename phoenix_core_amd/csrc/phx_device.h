@@ -124,6 +124,63 @@ __device__ __forceinline__ int xcd_remap(int hw_id, int total) {
     return xcd * base + (xcd < rem ? xcd : rem) + slot;
 }
 
+// 16- and 4-byte global loads from addresses with only 2-byte alignment (one instruction each).
+typedef u32x4 u32x4_a2 __attribute__((aligned(2)));
+typedef unsigned int u32_a2 __attribute__((aligned(2)));
+
+__device__ __forceinline__ u32x4 load16_a2(const _Float16* p) {
+    return *reinterpret_cast<const __attribute__((address_space(1))) u32x4_a2*>(
+        (const __attribute__((address_space(1))) _Float16*)p);
+}
+__device__ __forceinline__ unsigned int load4_a2(const _Float16* p) {
+    return *reinterpret_cast<const __attribute__((address_space(1))) u32_a2*>(
+        (const __attribute__((address_space(1))) _Float16*)p);
+}
+
+// Bit masks over the eight fp16 values of a 16-byte chunk.
+// bit i of `bits` set <=> half i of the chunk is kept
+__device__ __forceinline__ u32x4 expand_half_mask(unsigned int bits) {
+    u32x4 mk;
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+        const unsigned int lo = (unsigned int)((int)(bits << (31 - 2 * d)) >> 31);
+        const unsigned int hi = (unsigned int)((int)(bits << (30 - 2 * d)) >> 31);
+        mk[d] = (lo & 0x0000FFFFu) | (hi & 0xFFFF0000u);
+    }
+    return mk;
+}
+
+// bits [lo, hi) set, both clamped to [0, MAXB]
+template <int MAXB = 8>
+__device__ __forceinline__ unsigned int interval_bits(int lo, int hi) {
+    lo = lo < 0 ? 0 : lo;
+    hi = hi > MAXB ? MAXB : hi;
+    return hi > lo ? ((1u << hi) - (1u << lo)) : 0u;
+}
+
+// Developer option -DPHX_PHASE_TIMING: a kernel brackets its phases with PHX_STAMP(i); the shader
+// clocks spent in each phase (at most six) are summed per wave and printed by lane 0 of every 97th workgroup.
+// Without the option the macros expand to nothing.
+#ifdef PHX_PHASE_TIMING
+#define PHX_PHASES_BEGIN(n) long long phx_tph[6] = {}; long long phx_tlast = clock64();
+#define PHX_STAMP(i)                                             \
+    {                                                            \
+        __builtin_amdgcn_sched_barrier(0);                       \
+        const long long phx_now = clock64();                     \
+        phx_tph[i] += phx_now - phx_tlast;                       \
+        phx_tlast = phx_now;                                     \
+        __builtin_amdgcn_sched_barrier(0);                       \
+    }
+#define PHX_PHASES_REPORT(what, n)                                                                           \
+    if ((blockIdx.x % 97) == 0 && (threadIdx.x & 63) == 0)                                                   \
+        printf("%s | wg %d wave %d: %lld %lld %lld %lld %lld %lld\n", what, (int)blockIdx.x,                 \
+               (int)(threadIdx.x >> 6), phx_tph[0], phx_tph[1], phx_tph[2], phx_tph[3], phx_tph[4], phx_tph[5]);
+#else
+#define PHX_PHASES_BEGIN(n)
+#define PHX_STAMP(i)
+#define PHX_PHASES_REPORT(what, n)
+#endif
+
 // Sixty-four zero bytes in device memory: out-of-tensor staging positions load from here, which
 // keeps the staging loads unconditional and free of selects.
 static __device__ __attribute__((aligned(16))) const unsigned int phx_zero_block[16] = {};

@@ -328,8 +328,90 @@ __device__ __forceinline__ void lds_dma_16(const void* gsrc, void* ldst) {
 
 __device__ __forceinline__ void wait_vmem_all() { __builtin_amdgcn_s_waitcnt(0x0F70); }  // vmcnt(0)
 
-template <int WCO, int NTW, int P2LOG, bool PAIRS>
-__global__ void __launch_bounds__(WG_THREADS, 2) qconv_fwd_f16_lds_kernel(const ConvArgs P) {
+// Chunk staging of the activation window (CHUNKS): the window is NB*HTH rows of HTW positions, HTW a
+// multiple of 8.  One task = (component, 8-channel pack, 8 consecutive positions of a row): eight
+// 16-byte loads (one per channel, 2-byte aligned), an 8x8 transpose with byte permutes, eight 16-byte
+// LDS entries.  A quarter of the load instructions of the pair staging, and no restriction on W.
+// Positions outside the image are cleared with a mask that is fixed per task; tasks whose loads
+// could leave the tensor (first / last rows of the first / last plane) load nothing and are filled
+// element by element.  Entries are swizzled inside aligned groups of 8 (entry ^ (entry/8)%8) so that
+// the eight stores of neighbouring tasks spread over all LDS banks.
+struct StageChunk {
+    const _Float16* ptr;  // channel 0 of the task's component at the task's first position
+    int ent;              // unit * pitch + first entry of the task
+    int swz;
+    unsigned int bits;    // positions inside the image
+    int kp;
+    bool task, live, careful;
+};
+
+__device__ __forceinline__ int swizzle_entry(int e) { return e ^ ((e >> 3) & 7); }
+
+__device__ __forceinline__ StageChunk make_stage_chunk(const TileSrc& s, int n0, int h0, int w0, int NB, int HTH, int HTW,
+                                                       int HPp) {
+    StageChunk sc;
+    const int cpr = HTW >> 3;
+    const int hp8 = NB * HTH * cpr;  // tasks per unit
+    const int u = threadIdx.x / hp8, ch = threadIdx.x - u * hp8;
+    sc.task = u < 8;
+    const int row = ch / cpr, cc = ch - row * cpr;
+    const int nb = row / HTH, hr = row - nb * HTH;
+    const int vh = h0 + hr, vw0 = w0 + cc * 8;
+    const int p = u >> 1;
+    sc.kp = u & 1;
+    sc.live = sc.task && (n0 + nb) < s.N && vh >= 0 && vh < s.Hd;
+    sc.bits = sc.live ? interval_bits(-vw0, s.Wd - vw0) : 0u;
+    const _Float16* base = static_cast<const _Float16*>(s.base);
+    const long plane = (long)s.Hd * s.Wd;
+    sc.ptr = base + p * s.comp_stride + ((long)(n0 + nb) * s.C * s.Hd + vh) * s.Wd + vw0;
+    const _Float16* end = base + 3 * s.comp_stride + (long)s.N * s.C * plane;
+    sc.careful = sc.live && (sc.ptr < base || sc.ptr + (long)(s.C - 1) * plane + 8 > end);
+    const int e0 = row * HTW + cc * 8;
+    sc.ent = (sc.task ? u : 0) * HPp + e0;
+    sc.swz = (e0 >> 3) & 7;
+    return sc;
+}
+
+__device__ __forceinline__ void stage_chunk_load(u32x4 (&r)[8], const TileSrc& s, const StageChunk& sc, int c0, int i) {
+    const long plane = (long)s.Hd * s.Wd;
+    const int c = c0 + sc.kp * 8 + i;
+    const int cl = c < s.C ? c : s.C - 1;  // the filters hold zeros for channels past the tensor
+    const _Float16* ptr = (sc.live && !sc.careful) ? sc.ptr + cl * plane : static_cast<const _Float16*>(s.base);
+    r[i] = load16_a2(ptr);
+}
+
+__device__ __forceinline__ void stage_chunk_store(f16x8* xl, const u32x4 (&r)[8], const TileSrc& s, const StageChunk& sc,
+                                                  int c0) {
+    if (!sc.task) return;
+    const u32x4 mk = expand_half_mask(sc.careful ? 0u : sc.bits);
+    u32x4 rm[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) rm[i] = r[i] & mk;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        u32x4 v;
+#pragma unroll
+        for (int m = 0; m < 4; ++m)
+            v[m] = __builtin_amdgcn_perm(rm[2 * m + 1][j >> 1], rm[2 * m][j >> 1], (j & 1) ? 0x07060302u : 0x05040100u);
+        xl[sc.ent + (j ^ sc.swz)] = __builtin_bit_cast(f16x8, v);
+    }
+    if (sc.careful) {
+        const long plane = (long)s.Hd * s.Wd;
+        _Float16* xh = reinterpret_cast<_Float16*>(xl);
+#pragma unroll 2
+        for (int i = 0; i < 8; ++i) {
+            const int c = c0 + sc.kp * 8 + i;
+            _Float16 v[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[j] = (c < s.C && ((sc.bits >> j) & 1)) ? sc.ptr[c * plane + j] : (_Float16)0;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) xh[(sc.ent + (j ^ sc.swz)) * 8 + i] = v[j];
+        }
+    }
+}
+
+template <int WCO, int NTW, int P2LOG, bool CHUNKS>
+__global__ void __launch_bounds__(WG_THREADS, NTW == 1 ? 2 : 1) qconv_fwd_f16_lds_kernel(const ConvArgs P) {
     constexpr int CK = F16_CK;
     constexpr int WPX = 4 / WCO;
     constexpr int TG = F16_TG;
@@ -351,8 +433,6 @@ __global__ void __launch_bounds__(WG_THREADS, 2) qconv_fwd_f16_lds_kernel(const 
     const int tn = bid / P.tiles_h;
     const int n0 = tn * P.NB, ho0 = th * P.TH, wo0 = tw * P.TW;
     const int h0 = ho0 * P.sh - P.pt, w0 = wo0 * P.sw - P.pl;
-    const int w0e = PAIRS ? (w0 & ~1) : w0;  // pair staging starts the window at an even column
-    const int colshift = w0 - w0e;
 
     int poff[NTW];
     long oaddr[NTW];
@@ -364,7 +444,7 @@ __global__ void __launch_bounds__(WG_THREADS, 2) qconv_fwd_f16_lds_kernel(const 
         const int nb = pix / thw, rem = pix - nb * thw;
         const int r = rem / P.TW, c = rem - r * P.TW;
         pvalid[t] = nb < P.NB && (n0 + nb) < P.in.N && (ho0 + r) < P.Hout && (wo0 + c) < P.Wout;
-        poff[t] = pvalid[t] ? (nb * P.HTH + r * P.sh) * P.HTW + c * P.sw + colshift : colshift;
+        poff[t] = pvalid[t] ? (nb * P.HTH + r * P.sh) * P.HTW + c * P.sw : 0;
         oaddr[t] = ((long)(n0 + nb) * P.Cout * P.Hout + (ho0 + r)) * P.Wout + (wo0 + c);
     }
 
@@ -379,73 +459,143 @@ __global__ void __launch_bounds__(WG_THREADS, 2) qconv_fwd_f16_lds_kernel(const 
     const int ngroups = (P.taps + TG - 1) / TG;          // per chunk
     const int total_groups = P.nchunks * ngroups;
     const f16x8* wsrc = static_cast<const f16x8*>(P.wpk) + (long)ct * total_groups * WIMG;
+
+    // activation staging, one chunk ahead in registers
+    const StagePos sp = make_stage_pos<P2LOG>(P.in, n0, h0, w0, P.NB, P.HTH, P.HTW);
+    const StageChunk sc = make_stage_chunk(P.in, n0, h0, w0, P.NB, P.HTH, P.HTW, P.HPp);
+    f16x8 stage[CHUNKS ? 1 : (8 >> (8 - P2LOG))];
+    u32x4 stagec[CHUNKS ? 8 : 1];
+    constexpr int XLOADS = CHUNKS ? 8 : 0;  // activation load instructions that can be dealt out one by one
+    auto store_chunk = [&](int c0) {
+        if constexpr (CHUNKS) stage_chunk_store(xl, stagec, P.in, sc, c0);
+        else stage_store16<P2LOG>(xl, stage, sp, P.HP, P.HPp);
+    };
+    if constexpr (CHUNKS) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) stage_chunk_load(stagec, P.in, sc, 0, i);
+    } else {
+        stage_load16<P2LOG>(stage, P.in, sp, 0);
+    }
     // filter group image -> LDS buffer: TG*WCO*4 slices of 64 vectors, dealt round-robin to the waves
-    auto copy_group = [&](int gs) {
-        const f16x8* src = wsrc + (long)gs * WIMG;
-        f16x8* dst = wl + (gs & 1) * WIMG;
+    {
 #pragma unroll
         for (int s = 0; s < TG * WCO; ++s) {
             const int slice = s * 4 + wave;
-            lds_dma_16(src + slice * 64 + lane, dst + slice * 64);
+            lds_dma_16(wsrc + slice * 64 + lane, wl + slice * 64);
         }
-    };
+    }
 
-    const StagePos sp = make_stage_pos<P2LOG>(P.in, n0, h0, w0, P.NB, P.HTH, P.HTW);
-    const StagePairPos spp = make_stage_pairpos(P.in, n0, h0, w0e, P.NB, P.HTH, P.HTW);
-    f16x8 stage[PAIRS ? 1 : (8 >> (8 - P2LOG))];
-    unsigned int stagep[PAIRS ? 4 : 1][8];
-    auto load_chunk = [&](int c0) {
-        if constexpr (PAIRS) stage_load16_pairs(stagep, P.in, spp, c0);
-        else stage_load16<P2LOG>(stage, P.in, sp, c0);
-    };
-    auto store_chunk = [&]() {
-        if constexpr (PAIRS) stage_store16_pairs(xl, stagep, spp, P.HPp);
-        else stage_store16<P2LOG>(xl, stage, sp, P.HP, P.HPp);
-    };
-    load_chunk(0);
-    copy_group(0);
-
-    int gs = 0;
-    for (int chunk = 0; chunk < P.nchunks; ++chunk) {
-        __syncthreads();  // every wave is done reading the previous chunk's activations
-        store_chunk();
-        int tap = 0, kh = 0, kw = 0;
-        for (int g = 0; g < ngroups; ++g, ++gs) {
-            wait_vmem_all();   // this group's filters have landed in LDS
+    PHX_PHASES_BEGIN(5)
+    bool x_in_flight = false;  // activation loads were issued after the latest filter copy
+    int chunk = 0, g = 0, tap = 0, kh = 0, kw = 0;
+    // one flat loop over (chunk, filter group) steps: a single loop keeps the accumulators in place
+    for (int gs = 0; gs < total_groups; ++gs) {
+        if (g == 0) {
+            __syncthreads();  // every wave is done reading the previous chunk's activations
+            PHX_STAMP(0)
+            store_chunk(chunk * CK);  // (waits for this chunk's activation loads)
+            PHX_STAMP(1)
+            tap = 0; kh = 0; kw = 0;
+        }
+        {
+            // this group's filters have landed in LDS; vmcnt counts in order, so activation loads issued
+            // after the filter copy may stay in flight
+            if (x_in_flight) __builtin_amdgcn_s_waitcnt(0x0F70 | XLOADS);
+            else wait_vmem_all();
             __syncthreads();   // ... for every wave; activations of this chunk are visible
-            if (gs + 1 < total_groups) copy_group(gs + 1);
-            if (g == 0 && chunk + 1 < P.nchunks) load_chunk((chunk + 1) * CK);
-            const f16x8* wb = wl + (gs & 1) * WIMG + wco * 256 + lane;
+            PHX_STAMP(2)
+            // The group is a fixed sequence of TG*NTW blocks of 16 MFMAs.  Taps past the end of the filter
+            // are packed as zeros, so they are multiplied like the others (against window offset 0).
+            // A wave that issues its global loads back to back stalls until the memory pipeline has taken
+            // them all; so the LDS copy of the next filter group is dealt out over the first half of the
+            // blocks and the activation loads of the next chunk (first group of a chunk) over the second half.
+            constexpr int NBLK = TG * NTW;
+            constexpr int DBLK = (NBLK + 1) / 2;                    // blocks that carry filter-copy slices
+            constexpr int DPB = (TG * WCO + DBLK - 1) / DBLK;
+            constexpr int XBLK = NBLK - DBLK;                       // blocks that carry activation loads
+            constexpr int XPB = XBLK ? (XLOADS + XBLK - 1) / XBLK : 0;
+            const bool more_groups = gs + 1 < total_groups;
+            const bool more_chunks = g == 0 && chunk + 1 < P.nchunks;
+            int tapoff[TG];
 #pragma unroll
             for (int tg = 0; tg < TG; ++tg) {
-                if (tap < P.taps) {
-                    const int tapoff = kh * P.dh * P.HTW + kw * P.dw;
-                    // negative blocks of the Hamilton matrix only ever use -w1, -w2, -w3: flip the
-                    // filter operand once per step instead of the activation operand per column tile
-                    f16x8 w[4], nw[4];
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        w[r] = wb[(tg * WCO * 4 + r) * 64];
-                        nw[r] = neg8(w[r]);
-                    }
-                    const f16x8* xb = xl + kk * P.HPp + tapoff;
-#pragma unroll
-                    for (int t = 0; t < NTW; ++t) {
-                        f16x8 x[4];
-#pragma unroll
-                        for (int p = 0; p < 4; ++p) x[p] = xb[p * 2 * P.HPp + poff[t]];
-#pragma unroll
-                        for (int p = 0; p < 4; ++p)
-#pragma unroll
-                            for (int q = 0; q < 4; ++q)
-                                acc[t][q] = __builtin_amdgcn_mfma_f32_32x32x16_f16(qneg(p, q) ? nw[p ^ q] : w[p ^ q], x[p],
-                                                                                   acc[t][q], 0, 0, 0);
-                    }
-                    ++tap;
-                    if (++kw == P.Kw) { kw = 0; ++kh; }
-                }
+                tapoff[tg] = tap < P.taps ? kh * P.dh * P.HTW + kw * P.dw : 0;
+                ++tap;
+                if (++kw == P.Kw) { kw = 0; ++kh; }
             }
+            const f16x8* wb = wl + (gs & 1) * WIMG + wco * 256 + lane;
+            const f16x8* wsrc_next = wsrc + (long)(gs + 1) * WIMG;
+            f16x8* wdst_next = wl + ((gs + 1) & 1) * WIMG;
+            f16x8 wf[2][4], xf[2][4];
+            auto read_w = [&](f16x8 (&w)[4], int tg) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) w[r] = wb[(tg * WCO * 4 + r) * 64];
+            };
+            auto read_x = [&](f16x8 (&x)[4], int blk) {
+                const int pos = tapoff[blk / NTW] + poff[blk % NTW];
+                const f16x8* xb = xl + kk * P.HPp + (CHUNKS ? swizzle_entry(pos) : pos);
+#pragma unroll
+                for (int p = 0; p < 4; ++p) x[p] = xb[p * 2 * P.HPp];
+            };
+            read_w(wf[0], 0);
+            read_x(xf[0], 0);
+            if constexpr (!CHUNKS) {
+                if (more_chunks) stage_load16<P2LOG>(stage, P.in, sp, (chunk + 1) * CK);
+            }
+            PHX_STAMP(3)
+#pragma unroll
+            for (int blk = 0; blk < NBLK; ++blk) {
+                const int tg = blk / NTW, t = blk % NTW;
+                if (blk < DBLK) {
+                    if (more_groups) {
+#pragma unroll
+                        for (int s = blk * DPB; s < (blk + 1) * DPB && s < TG * WCO; ++s) {
+                            const int slice = s * 4 + wave;
+                            lds_dma_16(wsrc_next + slice * 64 + lane, wdst_next + slice * 64);
+                        }
+                    }
+                } else if constexpr (CHUNKS) {
+                    if (more_chunks) {
+#pragma unroll
+                        for (int i = (blk - DBLK) * XPB; i < (blk - DBLK + 1) * XPB && i < 8; ++i)
+                            stage_chunk_load(stagec, P.in, sc, (chunk + 1) * CK, i);
+                    }
+                }
+                const f16x8(&w)[4] = wf[tg & 1];
+                const f16x8(&x)[4] = xf[blk & 1];
+                // negative blocks of the Hamilton matrix only ever use -w1, -w2, -w3
+                f16x8 nw[4];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) nw[r] = neg8(w[r]);
+#pragma unroll
+                for (int p = 0; p < 4; ++p) {
+#pragma unroll
+                    for (int q = 0; q < 4; ++q)
+                        acc[t][q] = __builtin_amdgcn_mfma_f32_32x32x16_f16(qneg(p, q) ? nw[p ^ q] : w[p ^ q], x[p], acc[t][q],
+                                                                           0, 0, 0);
+                    if (p == 0) {
+                        // the next block's operands are requested once this block is under way: everything
+                        // outstanding at the top of a block is then exactly what that block needs
+                        __builtin_amdgcn_sched_barrier(0);
+                        if (blk + 1 < NBLK) {
+                            read_x(xf[(blk + 1) & 1], blk + 1);
+                            if ((blk + 1) % NTW == 0) read_w(wf[(tg + 1) & 1], tg + 1);
+                        }
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                }
+                // pin the accumulators to the AGPR file: left alone, the allocator parks one column tile in
+                // VGPRs and copies 64 registers in and out around every block
+                if constexpr (NTW == 2) {  // (one workgroup per CU: 512 registers, MFMA in its AGPR form)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) asm volatile("" : "+a"(acc[t][q]));
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            x_in_flight = CHUNKS && more_chunks;
+            PHX_STAMP(4)
         }
+        if (++g == ngroups) { g = 0; ++chunk; }
     }
 
     _Float16* out = static_cast<_Float16*>(P.out);
@@ -468,6 +618,9 @@ __global__ void __launch_bounds__(WG_THREADS, 2) qconv_fwd_f16_lds_kernel(const 
             }
         }
     }
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    PHX_STAMP(5)
+    PHX_PHASES_REPORT("fwd_f16_lds: barrier / store / wait+barrier / prefetch / mfma / epilogue", 6)
 }
 
 // Filter packing for qconv_fwd_f16_lds_kernel (16-product only; conjugated / mirrored / transposed
@@ -543,38 +696,6 @@ __global__ void __launch_bounds__(WG_THREADS) pack_filters_f16_lds_kernel(const 
 // ---------------------------------------------------------------------------------------------
 constexpr int WG16_KP = 64;         // reduction indices per pixel tile
 constexpr int WG16_PITCH = 64 + 8;  // LDS halves per staged channel row (16-byte skew against bank conflicts)
-
-typedef u32x4 u32x4_a2 __attribute__((aligned(2)));
-typedef unsigned int u32_a2 __attribute__((aligned(2)));
-
-__device__ __forceinline__ u32x4 load16_a2(const _Float16* p) {
-    return *reinterpret_cast<const __attribute__((address_space(1))) u32x4_a2*>(
-        (const __attribute__((address_space(1))) _Float16*)p);
-}
-__device__ __forceinline__ unsigned int load4_a2(const _Float16* p) {
-    return *reinterpret_cast<const __attribute__((address_space(1))) u32_a2*>(
-        (const __attribute__((address_space(1))) _Float16*)p);
-}
-
-// bit i of `bits` set <=> half i of the chunk is kept
-__device__ __forceinline__ u32x4 expand_half_mask(unsigned int bits) {
-    u32x4 mk;
-#pragma unroll
-    for (int d = 0; d < 4; ++d) {
-        const unsigned int lo = (unsigned int)((int)(bits << (31 - 2 * d)) >> 31);
-        const unsigned int hi = (unsigned int)((int)(bits << (30 - 2 * d)) >> 31);
-        mk[d] = (lo & 0x0000FFFFu) | (hi & 0xFFFF0000u);
-    }
-    return mk;
-}
-
-// bits [lo, hi) set, both clamped to [0, MAXB]
-template <int MAXB = 8>
-__device__ __forceinline__ unsigned int interval_bits(int lo, int hi) {
-    lo = lo < 0 ? 0 : lo;
-    hi = hi > MAXB ? MAXB : hi;
-    return hi > lo ? ((1u << hi) - (1u << lo)) : 0u;
-}
 
 struct WgChunk {  // where one 8-pixel chunk of the reduction space lies
     bool live;    // inside the reduction space
@@ -790,13 +911,7 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_wgrad_f16_kernel(const Wgrad
     prep(nextc);
 #pragma unroll
     for (int sl = 0; sl < NLOADS; ++sl) load_slot(sl);
-#ifdef PHX_EXP_TIMING
-    long long tph[5] = {0, 0, 0, 0, 0};
-#define PHX_STAMP(i) { __builtin_amdgcn_sched_barrier(0); const long long now = clock64(); tph[i] += now - tlast; tlast = now; __builtin_amdgcn_sched_barrier(0); }
-    long long tlast = clock64();
-#else
-#define PHX_STAMP(i)
-#endif
+    PHX_PHASES_BEGIN(5)
     for (int tile = zi; tile < ntiles; tile += P.zsplit) {
         __syncthreads();
         PHX_STAMP(0)
@@ -951,11 +1066,7 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_wgrad_f16_kernel(const Wgrad
         PHX_STAMP(4)
     }
 
-#ifdef PHX_EXP_TIMING
-    if ((blockIdx.x % 97) == 0 && lane == 0)
-        printf("wg %d wave %d: bar1 %lld store %lld bar2 %lld issue %lld mfma %lld (per tile, %d tiles)\n", (int)blockIdx.x, wave,
-               tph[0] / 21, tph[1] / 21, tph[2] / 21, tph[3] / 21, tph[4] / 21, (ntiles - zi + P.zsplit - 1) / P.zsplit);
-#endif
+    PHX_PHASES_REPORT("wgrad_f16: barrier / store / barrier / prepare / mfma", 5)
     // partial[z][tap][r][co][ci]
     const int taps = P.Kh * P.Kw;
     const long tap_stride = 4L * P.CoP * P.CiP;

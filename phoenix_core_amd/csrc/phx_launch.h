@@ -15,6 +15,7 @@ struct FwdVariant {
     bool lds_filters;   // fp16 MFMA only: filters staged through LDS (qconv_fwd_f16_lds_kernel)
     int ngroups;        // tap groups per chunk for that kernel
     bool pairs;         // fp16 MFMA: activations staged as aligned position pairs
+    bool chunks;        // fp16 MFMA, filters in LDS: activations staged as 8-position chunks
     int wgs;
     size_t lds_bytes;
 };

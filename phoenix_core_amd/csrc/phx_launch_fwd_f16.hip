@@ -30,12 +30,12 @@ static int launch_v1(const FwdVariant& v, const ConvArgs& a, hipStream_t st) {
     return launch_variant16<8, MAP_DGRAD, PAIRS>(v, a, st);
 }
 
-template <bool PAIRS>
+template <bool CHUNKS>
 static int launch_lds16(const FwdVariant& v, const ConvArgs& a, hipStream_t st) {
-    constexpr int P2A = 8, P2B = PAIRS ? 8 : 7;  // the pair path has a single staging shape
+    constexpr int P2A = 8, P2B = CHUNKS ? 8 : 7;  // chunk staging has a single shape
 #define PHX_CASE(WCO_, NTW_, P2_)                                                                             \
-    if (v.WCO == WCO_ && v.NTW == NTW_ && (PAIRS || v.P2LOG == P2_)) {                                        \
-        hipLaunchKernelGGL((qconv_fwd_f16_lds_kernel<WCO_, NTW_, P2_, PAIRS>), dim3(v.wgs), dim3(WG_THREADS), \
+    if (v.WCO == WCO_ && v.NTW == NTW_ && (CHUNKS || v.P2LOG == P2_)) {                                        \
+        hipLaunchKernelGGL((qconv_fwd_f16_lds_kernel<WCO_, NTW_, P2_, CHUNKS>), dim3(v.wgs), dim3(WG_THREADS), \
                            v.lds_bytes, st, a);                                                               \
         return 0;                                                                                             \
     }
@@ -47,7 +47,7 @@ static int launch_lds16(const FwdVariant& v, const ConvArgs& a, hipStream_t st) 
 }
 
 int launch_fwd_f16(const FwdVariant& v, const ConvArgs& a, hipStream_t st) {
-    if (v.lds_filters) return v.pairs ? launch_lds16<true>(v, a, st) : launch_lds16<false>(v, a, st);
+    if (v.lds_filters) return v.chunks ? launch_lds16<true>(v, a, st) : launch_lds16<false>(v, a, st);
     return v.pairs ? launch_v1<true>(v, a, st) : launch_v1<false>(v, a, st);
 }
 

@@ -162,6 +162,7 @@ struct FwdPlan {
     bool lds_filters;        // fp16 MFMA, 16-product, more than one tap: filters go through LDS
     int ngroups;             // tap groups per chunk in that case
     bool pairs;              // fp16 MFMA: window rows widened to even columns, staged as position pairs
+    bool chunks;             // fp16 MFMA, filters in LDS: window rows widened to a multiple of 8, staged as chunks
     int NB, TH, TW, HTH, HTW, HP, HPp;
     int tiles_n, tiles_h, tiles_w, co_tiles, nchunks;
     size_t lds_bytes, wpk_bytes;
@@ -174,9 +175,10 @@ constexpr int LDS_FLOATS_MAX = 16384;  // 64 KiB: two workgroups per CU
 static bool plan_forward(const Corr& c, int mode, bool f16mfma, FwdPlan& best) {
     double best_score = -1.0;
     // fp16 MFMA with filters in LDS: stage activations as aligned pairs when rows are even
-    const bool pairs = f16mfma && (c.Win % 2 == 0) && c.uw == 1;
     const bool ldsk = f16mfma && mode == 16 && c.Kh * c.Kw > 1;  // filters through LDS
-    best.pairs = pairs;
+    const bool chunks = ldsk && c.uw == 1;
+    const bool pairs = f16mfma && !chunks && (c.Win % 2 == 0) && c.uw == 1;
+    best.pairs = pairs; best.chunks = chunks;
     const int wcos[3] = {1, 2, 4};
     // PHX_TUNE_TILE="wco,ntw" pins the workgroup shape (kernel tuning experiments)
     int force_wco = 0, force_ntw = 0;
@@ -201,6 +203,7 @@ static bool plan_forward(const Corr& c, int mode, bool f16mfma, FwdPlan& best) {
                     const int HTH = (TH - 1) * c.sh + (c.Kh - 1) * c.dh + 1;
                     int HTW = (TW - 1) * c.sw + (c.Kw - 1) * c.dw + 1;
                     if (pairs) HTW = (HTW + 2) & ~1;  // room for the even start column, even pitch
+                    if (chunks) HTW = (HTW + 7) & ~7;  // whole 8-position chunks
                     const int HP = NB * HTH * HTW;
                     const int HPp = HP;
                     if (HP > 256) continue;  // one staging position per thread
@@ -279,7 +282,7 @@ static int run_corr(const Problem& p, const Corr& c, int map, hipStream_t st, co
     FwdVariant v;
     v.half_storage = p.dtype == PHX_F16; v.f16_mfma = f16; v.mode = p.mode; v.map = map;
     v.WCO = pl.WCO; v.NTW = pl.NTW; v.CK = pl.CK; v.P2LOG = pl.P2LOG; v.wgs = pl.wgs; v.lds_bytes = pl.lds_bytes;
-    v.lds_filters = pl.lds_filters; v.ngroups = pl.ngroups; v.pairs = pl.pairs;
+    v.lds_filters = pl.lds_filters; v.ngroups = pl.ngroups; v.pairs = pl.pairs; v.chunks = pl.chunks;
 
     PackArgs pa;
     pa.w = w; pa.out = ws;
@@ -312,7 +315,7 @@ static int run_corr(const Problem& p, const Corr& c, int map, hipStream_t st, co
     if (rc != 0) return PHX_ERR_NOT_SUPPORTED;
     PHX_HIP(hipGetLastError());
     snprintf(g_name_buf, sizeof(g_name_buf), "qconv_%s_%smfma%s_p%d_%s_wco%d_ntw%d_ck%d_tile%dx%dx%d",
-             map == MAP_FWD ? "fwd" : "dgrad", f16 ? "f16" : "f32", pl.lds_filters ? (pl.pairs ? "ldsp" : "lds") : "", p.mode, p.dtype == PHX_F32 ? "f32" : "f16", pl.WCO,
+             map == MAP_FWD ? "fwd" : "dgrad", f16 ? "f16" : "f32", pl.lds_filters ? (pl.chunks ? "ldsc" : "lds") : "", p.mode, p.dtype == PHX_F32 ? "f32" : "f16", pl.WCO,
              pl.NTW, pl.CK, pl.NB, pl.TH, pl.TW);
     g_last_kernel = g_name_buf;
     return PHX_OK;
