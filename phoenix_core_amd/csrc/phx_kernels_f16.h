@@ -225,37 +225,7 @@ __global__ void __launch_bounds__(WG_THREADS, (MODE == 8 || NTW == 1) ? 2 : 1) q
         }
     }
 
-    _Float16* out = static_cast<_Float16*>(P.out);
-    const _Float16* bias = static_cast<const _Float16*>(P.bias);
-    const long plane = (long)P.Hout * P.Wout;
-    const int co_base = (ct * WCO + wco) * 32 + 4 * kk;
-#pragma unroll
-    for (int t = 0; t < NTW; ++t) {
-        if (!pvalid[t]) continue;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int co = co_base + 8 * (r >> 2) + (r & 3);
-            float y[4];
-            if constexpr (MODE == 16) {
-#pragma unroll
-                for (int q = 0; q < 4; ++q) y[q] = acc[t][q][r];
-            } else {
-                float l[8];
-#pragma unroll
-                for (int i = 0; i < 8; ++i) l[i] = acc[t][i][r];
-                if constexpr (MAP == MAP_FWD) merge_output(l, y);
-                else merge_left_grad(l, y);
-            }
-            if (co < P.Cout) {
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    float v = y[q];
-                    if (bias) v += (float)bias[q * P.Cout + co];
-                    out[q * P.out_cs + oaddr[t] + co * plane] = (_Float16)v;
-                }
-            }
-        }
-    }
+    conv_epilogue<_Float16, MODE, MAP, NTW, NACC>(P, acc, (ct * WCO + wco) * 32 + 4 * kk, oaddr, pvalid);
 }
 
 // Filter packing for the kernel above: one group of WC 16-byte vectors per (32-channel filter
@@ -410,12 +380,15 @@ __device__ __forceinline__ void stage_chunk_store(f16x8* xl, const u32x4 (&r)[8]
     }
 }
 
-template <int WCO, int NTW, int P2LOG, bool CHUNKS>
-__global__ void __launch_bounds__(WG_THREADS, NTW == 1 ? 2 : 1) qconv_fwd_f16_lds_kernel(const ConvArgs P) {
+template <int MODE, int MAP, int WCO, int NTW, int P2LOG, bool CHUNKS>
+__global__ void __launch_bounds__(WG_THREADS, (MODE == 16 && NTW == 1) ? 2 : 1) qconv_fwd_f16_lds_kernel(const ConvArgs P) {
     constexpr int CK = F16_CK;
     constexpr int WPX = 4 / WCO;
     constexpr int TG = F16_TG;
-    constexpr int WIMG = TG * WCO * 4 * 64;  // 16-byte vectors per filter group image
+    constexpr int NW = (MODE == 16) ? 4 : 8;   // filter operands per tap and sub-tile: components or right lanes
+    constexpr bool PIN = !(MODE == 16 && NTW == 1);  // one workgroup per CU: MFMA in its AGPR form
+    constexpr int WIMG = TG * WCO * NW * 64;   // 16-byte vectors per filter group image
+    constexpr int NSL = TG * WCO * NW / 4;     // 1 KiB slices of that image per wave
     extern __shared__ f16x8 lds16[];
     f16x8* xl = lds16;                    // [8 units][HPp]
     f16x8* wl = lds16 + 8 * P.HPp;        // [2][WIMG]
@@ -448,11 +421,11 @@ __global__ void __launch_bounds__(WG_THREADS, NTW == 1 ? 2 : 1) qconv_fwd_f16_ld
         oaddr[t] = ((long)(n0 + nb) * P.Cout * P.Hout + (ho0 + r)) * P.Wout + (wo0 + c);
     }
 
-    f32x16 acc[NTW][4];
+    f32x16 acc[NTW][NW];
 #pragma unroll
     for (int t = 0; t < NTW; ++t)
 #pragma unroll
-        for (int a = 0; a < 4; ++a)
+        for (int a = 0; a < NW; ++a)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[t][a][r] = 0.f;
 
@@ -476,10 +449,10 @@ __global__ void __launch_bounds__(WG_THREADS, NTW == 1 ? 2 : 1) qconv_fwd_f16_ld
     } else {
         stage_load16<P2LOG>(stage, P.in, sp, 0);
     }
-    // filter group image -> LDS buffer: TG*WCO*4 slices of 64 vectors, dealt round-robin to the waves
+    // filter group image -> LDS buffer: slices of 64 vectors, dealt round-robin to the waves
     {
 #pragma unroll
-        for (int s = 0; s < TG * WCO; ++s) {
+        for (int s = 0; s < NSL; ++s) {
             const int slice = s * 4 + wave;
             lds_dma_16(wsrc + slice * 64 + lane, wl + slice * 64);
         }
@@ -511,7 +484,7 @@ __global__ void __launch_bounds__(WG_THREADS, NTW == 1 ? 2 : 1) qconv_fwd_f16_ld
             // blocks and the activation loads of the next chunk (first group of a chunk) over the second half.
             constexpr int NBLK = TG * NTW;
             constexpr int DBLK = (NBLK + 1) / 2;                    // blocks that carry filter-copy slices
-            constexpr int DPB = (TG * WCO + DBLK - 1) / DBLK;
+            constexpr int DPB = (NSL + DBLK - 1) / DBLK;
             constexpr int XBLK = NBLK - DBLK;                       // blocks that carry activation loads
             constexpr int XPB = XBLK ? (XLOADS + XBLK - 1) / XBLK : 0;
             const bool more_groups = gs + 1 < total_groups;
@@ -523,13 +496,13 @@ __global__ void __launch_bounds__(WG_THREADS, NTW == 1 ? 2 : 1) qconv_fwd_f16_ld
                 ++tap;
                 if (++kw == P.Kw) { kw = 0; ++kh; }
             }
-            const f16x8* wb = wl + (gs & 1) * WIMG + wco * 256 + lane;
+            const f16x8* wb = wl + (gs & 1) * WIMG + wco * (NW * 64) + lane;
             const f16x8* wsrc_next = wsrc + (long)(gs + 1) * WIMG;
             f16x8* wdst_next = wl + ((gs + 1) & 1) * WIMG;
-            f16x8 wf[2][4], xf[2][4];
-            auto read_w = [&](f16x8 (&w)[4], int tg) {
+            f16x8 wf[2][NW], xf[2][4];
+            auto read_w = [&](f16x8 (&w)[NW], int tg) {
 #pragma unroll
-                for (int r = 0; r < 4; ++r) w[r] = wb[(tg * WCO * 4 + r) * 64];
+                for (int r = 0; r < NW; ++r) w[r] = wb[(tg * WCO * NW + r) * 64];
             };
             auto read_x = [&](f16x8 (&x)[4], int blk) {
                 const int pos = tapoff[blk / NTW] + poff[blk % NTW];
@@ -549,7 +522,7 @@ __global__ void __launch_bounds__(WG_THREADS, NTW == 1 ? 2 : 1) qconv_fwd_f16_ld
                 if (blk < DBLK) {
                     if (more_groups) {
 #pragma unroll
-                        for (int s = blk * DPB; s < (blk + 1) * DPB && s < TG * WCO; ++s) {
+                        for (int s = blk * DPB; s < (blk + 1) * DPB && s < NSL; ++s) {
                             const int slice = s * 4 + wave;
                             lds_dma_16(wsrc_next + slice * 64 + lane, wdst_next + slice * 64);
                         }
@@ -561,34 +534,48 @@ __global__ void __launch_bounds__(WG_THREADS, NTW == 1 ? 2 : 1) qconv_fwd_f16_ld
                             stage_chunk_load(stagec, P.in, sc, (chunk + 1) * CK, i);
                     }
                 }
-                const f16x8(&w)[4] = wf[tg & 1];
+                const f16x8(&w)[NW] = wf[tg & 1];
                 const f16x8(&x)[4] = xf[blk & 1];
-                // negative blocks of the Hamilton matrix only ever use -w1, -w2, -w3
-                f16x8 nw[4];
+                // the next block's operands are requested once this block is under way: everything
+                // outstanding at the top of a block is then exactly what that block needs
+                auto prefetch = [&]() {
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (blk + 1 < NBLK) {
+                        read_x(xf[(blk + 1) & 1], blk + 1);
+                        if ((blk + 1) % NTW == 0) read_w(wf[(tg + 1) & 1], tg + 1);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                };
+                if constexpr (MODE == 16) {
+                    // negative blocks of the Hamilton matrix only ever use -w1, -w2, -w3
+                    f16x8 nw[4];
 #pragma unroll
-                for (int r = 0; r < 4; ++r) nw[r] = neg8(w[r]);
+                    for (int r = 0; r < 4; ++r) nw[r] = neg8(w[r]);
 #pragma unroll
-                for (int p = 0; p < 4; ++p) {
+                    for (int p = 0; p < 4; ++p) {
 #pragma unroll
-                    for (int q = 0; q < 4; ++q)
-                        acc[t][q] = __builtin_amdgcn_mfma_f32_32x32x16_f16(qneg(p, q) ? nw[p ^ q] : w[p ^ q], x[p], acc[t][q],
-                                                                           0, 0, 0);
-                    if (p == 0) {
-                        // the next block's operands are requested once this block is under way: everything
-                        // outstanding at the top of a block is then exactly what that block needs
-                        __builtin_amdgcn_sched_barrier(0);
-                        if (blk + 1 < NBLK) {
-                            read_x(xf[(blk + 1) & 1], blk + 1);
-                            if ((blk + 1) % NTW == 0) read_w(wf[(tg + 1) & 1], tg + 1);
-                        }
-                        __builtin_amdgcn_sched_barrier(0);
+                        for (int q = 0; q < 4; ++q)
+                            acc[t][q] = __builtin_amdgcn_mfma_f32_32x32x16_f16(qneg(p, q) ? nw[p ^ q] : w[p ^ q], x[p],
+                                                                               acc[t][q], 0, 0, 0);
+                        if (p == 0) prefetch();
+                    }
+                } else {
+                    // factorized form: eight independent products of a left lane (formed here from the four
+                    // staged components) with a right lane (packed)
+                    f16x8 L[8];
+                    if constexpr (MAP == MAP_FWD) lanes_left(x, L);
+                    else lanes_grad(x, L, (_Float16)0.5f);
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) {
+                        acc[t][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(w[i], L[i], acc[t][i], 0, 0, 0);
+                        if (i == 1) prefetch();
                     }
                 }
                 // pin the accumulators to the AGPR file: left alone, the allocator parks one column tile in
                 // VGPRs and copies 64 registers in and out around every block
-                if constexpr (NTW == 2) {  // (one workgroup per CU: 512 registers, MFMA in its AGPR form)
+                if constexpr (PIN) {
 #pragma unroll
-                    for (int q = 0; q < 4; ++q) asm volatile("" : "+a"(acc[t][q]));
+                    for (int q = 0; q < NW; ++q) asm volatile("" : "+a"(acc[t][q]));
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -598,26 +585,7 @@ __global__ void __launch_bounds__(WG_THREADS, NTW == 1 ? 2 : 1) qconv_fwd_f16_ld
         if (++g == ngroups) { g = 0; ++chunk; }
     }
 
-    _Float16* out = static_cast<_Float16*>(P.out);
-    const _Float16* bias = static_cast<const _Float16*>(P.bias);
-    const long plane = (long)P.Hout * P.Wout;
-    const int co_base = (ct * WCO + wco) * 32 + 4 * kk;
-#pragma unroll
-    for (int t = 0; t < NTW; ++t) {
-        if (!pvalid[t]) continue;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int co = co_base + 8 * (r >> 2) + (r & 3);
-            if (co < P.Cout) {
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    float v = acc[t][q][r];
-                    if (bias) v += (float)bias[q * P.Cout + co];
-                    out[q * P.out_cs + oaddr[t] + co * plane] = (_Float16)v;
-                }
-            }
-        }
-    }
+    conv_epilogue<_Float16, MODE, MAP, NTW, NW>(P, acc, (ct * WCO + wco) * 32 + 4 * kk, oaddr, pvalid);
     __builtin_amdgcn_s_waitcnt(0x0F70);
     PHX_STAMP(5)
     PHX_PHASES_REPORT("fwd_f16_lds: barrier / store / wait+barrier / prefetch / mfma / epilogue", 6)
@@ -632,19 +600,20 @@ struct PackLdsArgs {
     int ngroups;   // tap groups per chunk
 };
 
-template <int MAP>
+template <int MODE, int MAP>
 __global__ void __launch_bounds__(WG_THREADS) pack_filters_f16_lds_kernel(const PackLdsArgs A) {
     const PackArgs& P = A.base;
     constexpr int TG = F16_TG;
+    constexpr int NW = (MODE == 16) ? 4 : 8;
     const int taps = P.Kh * P.Kw;
-    // index = ((((tile*nchunks + chunk)*ngroups + g)*TG + tg)*WCO + wco)*4 + r)*64 + lane
-    const long total = (long)P.row_tiles * P.nchunks * A.ngroups * TG * A.WCO * 4 * 64;
+    // index = ((((tile*nchunks + chunk)*ngroups + g)*TG + tg)*WCO + wco)*NW + r)*64 + lane
+    const long total = (long)P.row_tiles * P.nchunks * A.ngroups * TG * A.WCO * NW * 64;
     const _Float16* w = static_cast<const _Float16*>(P.w);
     f16x8* outv = reinterpret_cast<f16x8*>(P.out);
     for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
         const int lane = idx & 63;
         long s = idx >> 6;
-        const int r = s & 3; s >>= 2;
+        const int r = s % NW; s /= NW;
         const int wco = s % A.WCO; s /= A.WCO;
         const int tg = s % TG; s /= TG;
         const int g = s % A.ngroups; s /= A.ngroups;
@@ -658,14 +627,23 @@ __global__ void __launch_bounds__(WG_THREADS) pack_filters_f16_lds_kernel(const 
         if (tap < taps && row < P.rows) {
             int kh = tap / P.Kw, kw = tap - kh * P.Kw;
             if (MAP == MAP_DGRAD) { kh = P.Kh - 1 - kh; kw = P.Kw - 1 - kw; }
-            const float sgn = (MAP == MAP_DGRAD && r > 0) ? -1.f : 1.f;
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 const int red = chunk * F16_CK + (lane >> 5) * 8 + i;
                 if (red < P.red) {
                     const int o = (MAP == MAP_DGRAD) ? red : row;
                     const int in = (MAP == MAP_DGRAD) ? row : red;
-                    vec[i] = (_Float16)(sgn * (float)w[r * P.wcs + o * P.so + in * P.si + kh * P.skh + kw * P.skw]);
+                    const long off = o * P.so + in * P.si + kh * P.skh + kw * P.skw;
+                    if constexpr (MODE == 16) {
+                        const float sgn = (MAP == MAP_DGRAD && r > 0) ? -1.f : 1.f;  // conjugate
+                        vec[i] = (_Float16)(sgn * (float)w[r * P.wcs + off]);
+                    } else {
+                        float wv[4], R[8];
+#pragma unroll
+                        for (int c = 0; c < 4; ++c) wv[c] = (float)w[c * P.wcs + off];
+                        lanes_right(wv, R);  // formed in fp32, rounded once
+                        vec[i] = (_Float16)R[r];
+                    }
                 }
             }
         }

@@ -27,7 +27,129 @@ struct ConvArgs {
     int HTH, HTW, HP, HPp;  // halo window, its size and the LDS pitch per staged channel
     int tiles_n, tiles_h, tiles_w, co_tiles;
     int nchunks;        // ceil(Cin / CK) for the kernel's chunk size CK
+    int vec;            // output pixels a lane stores at once (4, 2 or 1): divides TW and Wout
 };
+
+// ---------------------------------------------------------------------------------------------
+// Epilogue shared by the forward / input-gradient kernels (32x32 MFMA tiles: a lane holds one pixel
+// column, register e the channel row 8*(e/4) + 4*(lane/32) + e%4).  Vector memory instructions are
+// accepted at a fixed rate per wave whatever their width, so 64 scalar stores per column tile are
+// the expensive way out.  Each group of four registers (four consecutive channels) is transposed
+// across the four lanes of a quad (four consecutive pixels) with DPP moves; a lane then owns one
+// channel x four pixels and stores them as one 8- or 16-byte word.  P.vec == 2 does the same with
+// lane pairs, P.vec == 1 is the scalar form for tiles whose rows do not divide.
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ float dpp_quad_xor1(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));
+}
+__device__ __forceinline__ float dpp_quad_xor2(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));
+}
+
+// a[k] = row k at this lane's column -> o[m] = row (lane & 1) + 2*h at columns (pair base + m), h = 0, 1
+__device__ __forceinline__ void pair_transpose(const float (&a)[4], float (&b)[2], float (&d)[2], bool odd) {
+    const float n0 = dpp_quad_xor1(a[0]), n1 = dpp_quad_xor1(a[1]), n2 = dpp_quad_xor1(a[2]), n3 = dpp_quad_xor1(a[3]);
+    b[0] = odd ? n1 : a[0];  b[1] = odd ? a[1] : n0;   // rows 0 / 1
+    d[0] = odd ? n3 : a[2];  d[1] = odd ? a[3] : n2;   // rows 2 / 3
+}
+
+// a[k] = row k at this lane's column -> o[m] = row (lane & 3) at columns (quad base + m)
+__device__ __forceinline__ void quad_transpose(const float (&a)[4], float (&o)[4], int ql) {
+    float b[2], d[2];
+    pair_transpose(a, b, d, ql & 1);
+    const bool hi = ql & 2;
+    const float s0 = hi ? b[0] : d[0], s1 = hi ? b[1] : d[1];
+    const float r0 = dpp_quad_xor2(s0), r1 = dpp_quad_xor2(s1);
+    o[0] = hi ? r0 : b[0];  o[1] = hi ? r1 : b[1];
+    o[2] = hi ? d[0] : r0;  o[3] = hi ? d[1] : r1;
+}
+
+template <typename TS, int V>
+__device__ __forceinline__ void store_pixels(TS* ptr, const float (&v)[V]) {
+    typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
+    if constexpr (sizeof(TS) == 4) {
+        typedef float fv __attribute__((ext_vector_type(V), aligned(4)));
+        fv w;
+#pragma unroll
+        for (int i = 0; i < V; ++i) w[i] = v[i];
+        *reinterpret_cast<fv*>(ptr) = w;
+    } else {
+        typedef _Float16 hv __attribute__((ext_vector_type(V), aligned(2)));
+        hv w;
+#pragma unroll
+        for (int i = 0; i < V; ++i) w[i] = (_Float16)v[i];
+        *reinterpret_cast<hv*>(ptr) = w;
+    }
+}
+
+template <typename TS, int MODE, int MAP, int NTW, int NACC>
+__device__ __forceinline__ void conv_epilogue(const ConvArgs& P, const f32x16 (&acc)[NTW][NACC], int co_base,
+                                              const long (&oaddr)[NTW], const bool (&pvalid)[NTW]) {
+    TS* out = static_cast<TS*>(P.out);
+    const TS* bias = static_cast<const TS*>(P.bias);
+    const long plane = (long)P.Hout * P.Wout;
+    const int ql = threadIdx.x & 3;
+    auto component_rows = [&](int t, int e, float (&y)[4]) {  // the four output components of register e
+        if constexpr (MODE == 16) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) y[q] = acc[t][q][e];
+        } else {
+            float l[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) l[i] = acc[t][i][e];
+            if constexpr (MAP == MAP_FWD) merge_output(l, y);
+            else merge_left_grad(l, y);
+        }
+    };
+#pragma unroll
+    for (int t = 0; t < NTW; ++t) {
+        if (!pvalid[t]) continue;  // uniform over a quad / pair when P.vec > 1
+#pragma unroll
+        for (int rq = 0; rq < 4; ++rq) {
+            float y[4][4];  // [row in group][component]
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                component_rows(t, rq * 4 + k, y[k]);
+                const int co = co_base + 8 * rq + k;
+                if (bias && co < P.Cout) {
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) y[k][q] += ldf<TS>(bias + q * P.Cout + co);
+                }
+            }
+            if (P.vec == 4) {
+                const int co = co_base + 8 * rq + ql;
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const float a[4] = {y[0][q], y[1][q], y[2][q], y[3][q]};
+                    float o[4];
+                    quad_transpose(a, o, ql);
+                    if (co < P.Cout) store_pixels<TS, 4>(out + q * P.out_cs + (oaddr[t] - ql) + co * plane, o);
+                }
+            } else if (P.vec == 2) {
+                const int odd = ql & 1;
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const float a[4] = {y[0][q], y[1][q], y[2][q], y[3][q]};
+                    float b[2], d[2];
+                    pair_transpose(a, b, d, odd);
+                    const int co = co_base + 8 * rq + odd;
+                    TS* dst = out + q * P.out_cs + (oaddr[t] - odd);
+                    if (co < P.Cout) store_pixels<TS, 2>(dst + co * plane, b);
+                    if (co + 2 < P.Cout) store_pixels<TS, 2>(dst + (co + 2) * plane, d);
+                }
+            } else {
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const int co = co_base + 8 * rq + k;
+                    if (co < P.Cout) {
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) stf<TS>(out + q * P.out_cs + oaddr[t] + co * plane, y[k][q]);
+                    }
+                }
+            }
+        }
+    }
+}
 
 // Forward / input-gradient kernel.
 //   workgroup = 4 waves = WCO filter sub-tiles (32 output channels each) x 4/WCO pixel ranges,
@@ -141,37 +263,7 @@ __global__ void __launch_bounds__(WG_THREADS, (MODE == 8 || NTW == 1) ? 2 : 1) q
     }
 
     // epilogue: fold lanes (8-product), add bias, store NCHW with components on the batch axis
-    TS* out = static_cast<TS*>(P.out);
-    const TS* bias = static_cast<const TS*>(P.bias);
-    const long plane = (long)P.Hout * P.Wout;
-    const int co_base = (ct * WCO + wco) * 32 + 4 * kk;
-#pragma unroll
-    for (int t = 0; t < NTW; ++t) {
-        if (!pvalid[t]) continue;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int co = co_base + 8 * (r >> 2) + (r & 3);
-            float y[4];
-            if constexpr (MODE == 16) {
-#pragma unroll
-                for (int q = 0; q < 4; ++q) y[q] = acc[t][q][r];
-            } else {
-                float l[8];
-#pragma unroll
-                for (int i = 0; i < 8; ++i) l[i] = acc[t][i][r];
-                if constexpr (MAP == MAP_FWD) merge_output(l, y);
-                else merge_left_grad(l, y);
-            }
-            if (co < P.Cout) {
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    float v = y[q];
-                    if (bias) v += ldf<TS>(bias + q * P.Cout + co);
-                    stf<TS>(out + q * P.out_cs + oaddr[t] + co * plane, v);
-                }
-            }
-        }
-    }
+    conv_epilogue<TS, MODE, MAP, NTW, NACC>(P, acc, (ct * WCO + wco) * 32 + 4 * kk, oaddr, pvalid);
 }
 
 // Filter packing for the kernel above.  One value group per (32-channel filter tile, K step, lane):

@@ -23,6 +23,7 @@ struct FwdVariant {
 int launch_pack_filters(const FwdVariant& v, const PackArgs& a, int blocks, hipStream_t st);
 int launch_fwd_f32(const FwdVariant& v, const ConvArgs& a, hipStream_t st);
 int launch_fwd_f16(const FwdVariant& v, const ConvArgs& a, hipStream_t st);
+int launch_fwd_f16_lds8(const FwdVariant& v, const ConvArgs& a, hipStream_t st);  // 8-product, filters through LDS
 int launch_pack_filters_f16(const FwdVariant& v, const PackArgs& a, int blocks, hipStream_t st);
 
 int launch_wgrad_f32(bool half_storage, int mode, const WgradArgs& a, dim3 grid, size_t lds_bytes, hipStream_t st);

@@ -35,7 +35,7 @@ static int launch_lds16(const FwdVariant& v, const ConvArgs& a, hipStream_t st) 
     constexpr int P2A = 8, P2B = CHUNKS ? 8 : 7;  // chunk staging has a single shape
 #define PHX_CASE(WCO_, NTW_, P2_)                                                                             \
     if (v.WCO == WCO_ && v.NTW == NTW_ && (CHUNKS || v.P2LOG == P2_)) {                                        \
-        hipLaunchKernelGGL((qconv_fwd_f16_lds_kernel<WCO_, NTW_, P2_, CHUNKS>), dim3(v.wgs), dim3(WG_THREADS), \
+        hipLaunchKernelGGL((qconv_fwd_f16_lds_kernel<16, MAP_FWD, WCO_, NTW_, P2_, CHUNKS>), dim3(v.wgs), dim3(WG_THREADS), \
                            v.lds_bytes, st, a);                                                               \
         return 0;                                                                                             \
     }
@@ -47,6 +47,7 @@ static int launch_lds16(const FwdVariant& v, const ConvArgs& a, hipStream_t st) 
 }
 
 int launch_fwd_f16(const FwdVariant& v, const ConvArgs& a, hipStream_t st) {
+    if (v.lds_filters && v.mode == 8) return launch_fwd_f16_lds8(v, a, st);
     if (v.lds_filters) return v.chunks ? launch_lds16<true>(v, a, st) : launch_lds16<false>(v, a, st);
     return v.pairs ? launch_v1<true>(v, a, st) : launch_v1<false>(v, a, st);
 }
@@ -55,8 +56,10 @@ int launch_pack_filters_f16(const FwdVariant& v, const PackArgs& a, int blocks, 
     const dim3 g(blocks), b(WG_THREADS);
     if (v.lds_filters) {
         PackLdsArgs la{a, v.WCO, v.ngroups};
-        if (v.map == MAP_FWD) hipLaunchKernelGGL((pack_filters_f16_lds_kernel<MAP_FWD>), g, b, 0, st, la);
-        else hipLaunchKernelGGL((pack_filters_f16_lds_kernel<MAP_DGRAD>), g, b, 0, st, la);
+        if (v.mode == 16 && v.map == MAP_FWD) hipLaunchKernelGGL((pack_filters_f16_lds_kernel<16, MAP_FWD>), g, b, 0, st, la);
+        else if (v.mode == 16) hipLaunchKernelGGL((pack_filters_f16_lds_kernel<16, MAP_DGRAD>), g, b, 0, st, la);
+        else if (v.map == MAP_FWD) hipLaunchKernelGGL((pack_filters_f16_lds_kernel<8, MAP_FWD>), g, b, 0, st, la);
+        else hipLaunchKernelGGL((pack_filters_f16_lds_kernel<8, MAP_DGRAD>), g, b, 0, st, la);
         return 0;
     }
     if (v.mode == 16 && v.map == MAP_FWD) hipLaunchKernelGGL((pack_filters_f16_kernel<16, MAP_FWD>), g, b, 0, st, a);

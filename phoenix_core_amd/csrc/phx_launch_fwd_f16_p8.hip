@@ -1,0 +1,33 @@
+// fp16-MFMA forward / input-gradient kernels with both operands through LDS, factorized 8-product form.
+#include "phx_kernels_f16.h"
+#include "phx_launch.h"
+
+namespace phx {
+
+template <int MAP>
+static int launch_lds8(const FwdVariant& v, const ConvArgs& a, hipStream_t st) {
+#define PHX_CASE(WCO_, NTW_)                                                                                       \
+    if (v.WCO == WCO_ && v.NTW == NTW_) {                                                                          \
+        auto kernel = qconv_fwd_f16_lds_kernel<8, MAP, WCO_, NTW_, 8, true>;                                       \
+        static bool raised = false; /* dynamic LDS above the default 64 KiB needs an explicit opt-in */           \
+        if (!raised && v.lds_bytes > 64 * 1024) {                                                                  \
+            if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, \
+                                    160 * 1024) != hipSuccess) {                                                   \
+                (void)hipGetLastError();                                                                           \
+                return -1;                                                                                         \
+            }                                                                                                      \
+            raised = true;                                                                                         \
+        }                                                                                                          \
+        hipLaunchKernelGGL(kernel, dim3(v.wgs), dim3(WG_THREADS), v.lds_bytes, st, a);                             \
+        return 0;                                                                                                  \
+    }
+    PHX_CASE(1, 1) PHX_CASE(1, 2) PHX_CASE(2, 1) PHX_CASE(2, 2)
+#undef PHX_CASE
+    return -1;
+}
+
+int launch_fwd_f16_lds8(const FwdVariant& v, const ConvArgs& a, hipStream_t st) {
+    return v.map == MAP_FWD ? launch_lds8<MAP_FWD>(v, a, st) : launch_lds8<MAP_DGRAD>(v, a, st);
+}
+
+}  // namespace phx

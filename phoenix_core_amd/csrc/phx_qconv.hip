@@ -175,7 +175,8 @@ constexpr int LDS_FLOATS_MAX = 16384;  // 64 KiB: two workgroups per CU
 static bool plan_forward(const Corr& c, int mode, bool f16mfma, FwdPlan& best) {
     double best_score = -1.0;
     // fp16 MFMA with filters in LDS: stage activations as aligned pairs when rows are even
-    const bool ldsk = f16mfma && mode == 16 && c.Kh * c.Kw > 1;  // filters through LDS
+    // filters through LDS: 16-product always, 8-product where the chunk staging applies
+    const bool ldsk = f16mfma && c.Kh * c.Kw > 1 && (mode == 16 || c.uw == 1);
     const bool chunks = ldsk && c.uw == 1;
     const bool pairs = f16mfma && !chunks && (c.Win % 2 == 0) && c.uw == 1;
     best.pairs = pairs; best.chunks = chunks;
@@ -187,7 +188,9 @@ static bool plan_forward(const Corr& c, int mode, bool f16mfma, FwdPlan& best) {
         const int WCO = wcos[wi];
         if (force_wco && WCO != force_wco) continue;
         if (WCO > 1 && 32 * WCO > ((c.Cout + 31) / 32) * 32) continue;
-        for (int NTW = 1; NTW <= (mode == 16 ? 2 : 1); ++NTW) {  // 8 lanes x 2 column tiles would spill
+        if (ldsk && mode == 8 && WCO > 2) continue;  // eight filter lanes: the LDS images of 4 sub-tiles do not fit
+        // 8 lanes x 2 column tiles fill the whole AGPR file: only the LDS kernel is built that way
+        for (int NTW = 1; NTW <= ((mode == 16 || ldsk) ? 2 : 1); ++NTW) {
             if (force_ntw && NTW != force_ntw) continue;
             const int BN = (4 / WCO) * NTW * 32;
             int cand[16];
@@ -243,7 +246,7 @@ static bool plan_forward(const Corr& c, int mode, bool f16mfma, FwdPlan& best) {
         best.lds_filters = ldsk;
         best.ngroups = cdiv(taps, F16_TG);
         if (best.lds_filters) {
-            const size_t wimg = (size_t)F16_TG * best.WCO * 4 * 64 * 16;  // one filter group image
+            const size_t wimg = (size_t)F16_TG * best.WCO * WC * 64 * 16;  // one filter group image
             best.lds_bytes += 2 * wimg;
             best.wpk_bytes = (size_t)best.co_tiles * best.nchunks * best.ngroups * wimg;
         }
@@ -305,6 +308,9 @@ static int run_corr(const Problem& p, const Corr& c, int map, hipStream_t st, co
     a.NB = pl.NB; a.TH = pl.TH; a.TW = pl.TW; a.HTH = pl.HTH; a.HTW = pl.HTW; a.HP = pl.HP; a.HPp = pl.HPp;
     a.tiles_n = pl.tiles_n; a.tiles_h = pl.tiles_h; a.tiles_w = pl.tiles_w; a.co_tiles = pl.co_tiles;
     a.nchunks = pl.nchunks;
+    // pixels a lane may store as one word: the groups must not straddle tile rows or the image edge
+    a.vec = (pl.TW % 4 == 0 && c.Wout % 4 == 0) ? 4 : (pl.TW % 2 == 0 && c.Wout % 2 == 0) ? 2 : 1;
+    if (const char* e = getenv("PHX_TUNE_VEC")) a.vec = std::min(a.vec, atoi(e));
 
     int rc = f16 ? launch_pack_filters_f16(v, pa, pack_blocks, st) : launch_pack_filters(v, pa, pack_blocks, st);
     if (rc != 0) return PHX_ERR_NOT_SUPPORTED;
