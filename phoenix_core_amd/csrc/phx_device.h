@@ -197,6 +197,7 @@ struct TileSrc {
     long comp_stride;  // elements between components
     int N, C, Hd, Wd;  // stored dims per component
     int uh, uw;        // zero-insertion factors (1 = none)
+    int pw;            // pointwise trick: window row r holds channels (chunk*pw + r)*16.. of the single image row (0 = off)
 };
 
 // Window staging, split so that global loads can be in flight while the previous chunk is being

@@ -312,6 +312,7 @@ struct StageChunk {
     int swz;
     unsigned int bits;    // positions inside the image
     int kp;
+    int sub;              // pointwise trick: 16-channel sub-chunk this window row stands for
     bool task, live, careful;
 };
 
@@ -326,10 +327,14 @@ __device__ __forceinline__ StageChunk make_stage_chunk(const TileSrc& s, int n0,
     sc.task = u < 8;
     const int row = ch / cpr, cc = ch - row * cpr;
     const int nb = row / HTH, hr = row - nb * HTH;
-    const int vh = h0 + hr, vw0 = w0 + cc * 8;
+    // pointwise trick (s.pw > 0): the window rows are not image rows but consecutive 16-channel
+    // sub-chunks of the one (flattened) image row, so that a "filter column" of s.pw taps walks over
+    // 16*s.pw channels per staged chunk
+    sc.sub = s.pw ? hr : 0;
+    const int vh = s.pw ? 0 : h0 + hr, vw0 = w0 + cc * 8;
     const int p = u >> 1;
     sc.kp = u & 1;
-    sc.live = sc.task && (n0 + nb) < s.N && vh >= 0 && vh < s.Hd;
+    sc.live = sc.task && nb < NB && (n0 + nb) < s.N && vh >= 0 && vh < s.Hd;
     sc.bits = sc.live ? interval_bits(-vw0, s.Wd - vw0) : 0u;
     const _Float16* base = static_cast<const _Float16*>(s.base);
     const long plane = (long)s.Hd * s.Wd;
@@ -344,9 +349,11 @@ __device__ __forceinline__ StageChunk make_stage_chunk(const TileSrc& s, int n0,
 
 __device__ __forceinline__ void stage_chunk_load(u32x4 (&r)[8], const TileSrc& s, const StageChunk& sc, int c0, int i) {
     const long plane = (long)s.Hd * s.Wd;
-    const int c = c0 + sc.kp * 8 + i;
-    const int cl = c < s.C ? c : s.C - 1;  // the filters hold zeros for channels past the tensor
-    const _Float16* ptr = (sc.live && !sc.careful) ? sc.ptr + cl * plane : static_cast<const _Float16*>(s.base);
+    const int cv = c0 + sc.kp * 8 + i;
+    const int c = s.pw ? ((cv >> 4) * s.pw + sc.sub) * 16 + (cv & 15) : cv;
+    // channels past the tensor meet zero filters: any finite value will do, the tensor's first bytes are safe
+    const _Float16* ptr =
+        (sc.live && !sc.careful && c < s.C) ? sc.ptr + c * plane : static_cast<const _Float16*>(s.base);
     r[i] = load16_a2(ptr);
 }
 
@@ -370,7 +377,8 @@ __device__ __forceinline__ void stage_chunk_store(f16x8* xl, const u32x4 (&r)[8]
         _Float16* xh = reinterpret_cast<_Float16*>(xl);
 #pragma unroll 2
         for (int i = 0; i < 8; ++i) {
-            const int c = c0 + sc.kp * 8 + i;
+            const int cv = c0 + sc.kp * 8 + i;
+            const int c = s.pw ? ((cv >> 4) * s.pw + sc.sub) * 16 + (cv & 15) : cv;
             _Float16 v[8];
 #pragma unroll
             for (int j = 0; j < 8; ++j) v[j] = (c < s.C && ((sc.bits >> j) & 1)) ? sc.ptr[c * plane + j] : (_Float16)0;
@@ -598,6 +606,7 @@ struct PackLdsArgs {
     PackArgs base;
     int WCO;       // filter sub-tiles per workgroup tile
     int ngroups;   // tap groups per chunk
+    int pw;        // pointwise trick: the taps of a group are pw consecutive 16-channel sub-chunks (0 = off)
 };
 
 template <int MODE, int MAP>
@@ -605,7 +614,7 @@ __global__ void __launch_bounds__(WG_THREADS) pack_filters_f16_lds_kernel(const 
     const PackArgs& P = A.base;
     constexpr int TG = F16_TG;
     constexpr int NW = (MODE == 16) ? 4 : 8;
-    const int taps = P.Kh * P.Kw;
+    const int taps = A.pw ? A.pw : P.Kh * P.Kw;
     // index = ((((tile*nchunks + chunk)*ngroups + g)*TG + tg)*WCO + wco)*NW + r)*64 + lane
     const long total = (long)P.row_tiles * P.nchunks * A.ngroups * TG * A.WCO * NW * 64;
     const _Float16* w = static_cast<const _Float16*>(P.w);
@@ -627,9 +636,11 @@ __global__ void __launch_bounds__(WG_THREADS) pack_filters_f16_lds_kernel(const 
         if (tap < taps && row < P.rows) {
             int kh = tap / P.Kw, kw = tap - kh * P.Kw;
             if (MAP == MAP_DGRAD) { kh = P.Kh - 1 - kh; kw = P.Kw - 1 - kw; }
+            if (A.pw) kh = kw = 0;  // the one real tap
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
-                const int red = chunk * F16_CK + (lane >> 5) * 8 + i;
+                const int k16 = (lane >> 5) * 8 + i;
+                const int red = A.pw ? (chunk * A.pw + tap) * 16 + k16 : chunk * F16_CK + k16;
                 if (red < P.red) {
                     const int o = (MAP == MAP_DGRAD) ? red : row;
                     const int in = (MAP == MAP_DGRAD) ? row : red;

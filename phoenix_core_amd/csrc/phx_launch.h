@@ -16,6 +16,7 @@ struct FwdVariant {
     int ngroups;        // tap groups per chunk for that kernel
     bool pairs;         // fp16 MFMA: activations staged as aligned position pairs
     bool chunks;        // fp16 MFMA, filters in LDS: activations staged as 8-position chunks
+    int pw;             // pointwise convolution run as a column of pw virtual taps over 16-channel sub-chunks (0 = off)
     int wgs;
     size_t lds_bytes;
 };

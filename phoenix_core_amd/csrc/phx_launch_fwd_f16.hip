@@ -55,7 +55,7 @@ int launch_fwd_f16(const FwdVariant& v, const ConvArgs& a, hipStream_t st) {
 int launch_pack_filters_f16(const FwdVariant& v, const PackArgs& a, int blocks, hipStream_t st) {
     const dim3 g(blocks), b(WG_THREADS);
     if (v.lds_filters) {
-        PackLdsArgs la{a, v.WCO, v.ngroups};
+        PackLdsArgs la{a, v.WCO, v.ngroups, v.pw};
         if (v.mode == 16 && v.map == MAP_FWD) hipLaunchKernelGGL((pack_filters_f16_lds_kernel<16, MAP_FWD>), g, b, 0, st, la);
         else if (v.mode == 16) hipLaunchKernelGGL((pack_filters_f16_lds_kernel<16, MAP_DGRAD>), g, b, 0, st, la);
         else if (v.map == MAP_FWD) hipLaunchKernelGGL((pack_filters_f16_lds_kernel<8, MAP_FWD>), g, b, 0, st, la);

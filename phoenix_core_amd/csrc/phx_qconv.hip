@@ -275,23 +275,52 @@ static bool use_f16_mfma(const Problem& p, int pass) {
     return p.policy == PHX_FP16_FULL16;
 }
 
-static int run_corr(const Problem& p, const Corr& c, int map, hipStream_t st, const void* in, const void* w,
+// A pointwise fp16 correlation on one long row per image has a single tap, which would leave the LDS
+// kernels one MFMA block per barrier.  It is run instead as a column of PW_TAPS virtual taps: window
+// row r of the staged tile holds the 16-channel sub-chunk r of a 48-channel chunk, and "tap" r of the
+// packed filters holds the matching filter slice.  Returns the virtual correlation (pw = its tap count).
+constexpr int PW_TAPS = F16_TG;
+static Corr virtual_pointwise(const Corr& c, bool f16mfma, int& pw) {
+    pw = 0;
+    if (!f16mfma || c.Kh * c.Kw != 1 || c.uh != 1 || c.uw != 1 || c.sh != 1 || c.sw != 1 || c.Hin != 1 || c.Hout != 1 ||
+        c.pt != 0 || c.pl != 0 || c.Win != c.Wout)
+        return c;
+    if (getenv("PHX_TUNE_NOPW")) return c;
+    pw = PW_TAPS;
+    Corr v = c;
+    v.Kh = PW_TAPS; v.Kw = 1; v.dh = 1;
+    v.Cin = 16 * cdiv(c.Cin, 16 * PW_TAPS);  // 16 virtual channels per 48-channel chunk
+    return v;
+}
+
+// plans the virtual-tap form of a pointwise correlation where it applies and fits, the plain form otherwise
+static bool plan_corr(const Corr& creal, int mode, bool f16mfma, Corr& c, FwdPlan& pl, int& pw) {
+    c = virtual_pointwise(creal, f16mfma, pw);
+    if (pw && plan_forward(c, mode, f16mfma, pl) && pl.lds_filters && pl.chunks) return true;
+    pw = 0;
+    c = creal;
+    return plan_forward(c, mode, f16mfma, pl);
+}
+
+static int run_corr(const Problem& p, const Corr& creal, int map, hipStream_t st, const void* in, const void* w,
                     const void* bias, void* out, void* ws, size_t ws_bytes) {
     const bool f16 = use_f16_mfma(p, map == MAP_FWD ? PHX_PASS_FWD : PHX_PASS_BWD_DATA);
+    int pw = 0;
+    Corr c;
     FwdPlan pl;
-    if (!plan_forward(c, p.mode, f16, pl)) return PHX_ERR_NOT_SUPPORTED;
+    if (!plan_corr(creal, p.mode, f16, c, pl, pw)) return PHX_ERR_NOT_SUPPORTED;
     if (ws_bytes < pl.wpk_bytes || !ws) return PHX_ERR_WORKSPACE;
 
     FwdVariant v;
     v.half_storage = p.dtype == PHX_F16; v.f16_mfma = f16; v.mode = p.mode; v.map = map;
     v.WCO = pl.WCO; v.NTW = pl.NTW; v.CK = pl.CK; v.P2LOG = pl.P2LOG; v.wgs = pl.wgs; v.lds_bytes = pl.lds_bytes;
-    v.lds_filters = pl.lds_filters; v.ngroups = pl.ngroups; v.pairs = pl.pairs; v.chunks = pl.chunks;
+    v.lds_filters = pl.lds_filters; v.ngroups = pl.ngroups; v.pairs = pl.pairs; v.chunks = pl.chunks; v.pw = pw;
 
     PackArgs pa;
     pa.w = w; pa.out = ws;
     pa.wcs = p.fs.wcs; pa.so = p.fs.so; pa.si = p.fs.si; pa.skh = p.fs.skh; pa.skw = p.fs.skw;
     pa.Co = p.co; pa.Ci = p.ci; pa.Kh = p.kh; pa.Kw = p.kw;
-    pa.rows = c.Cout; pa.red = c.Cin; pa.row_tiles = pl.co_tiles * pl.WCO;
+    pa.rows = c.Cout; pa.red = creal.Cin; pa.row_tiles = pl.co_tiles * pl.WCO;
     pa.nchunks = f16 ? pl.nchunks : pl.nchunks * (pl.CK / F32_CK);
     const long pack_items = pl.lds_filters ? (long)(pl.wpk_bytes / 16)
                                             : (long)pa.row_tiles * pa.nchunks * p.kh * p.kw * (f16 ? 1 : 4) * 64;
@@ -299,8 +328,8 @@ static int run_corr(const Problem& p, const Corr& c, int map, hipStream_t st, co
     const int pack_blocks = (int)std::min<long>((pack_items + WG_THREADS - 1) / WG_THREADS, 4096);
 
     ConvArgs a;
-    a.in.base = in; a.in.comp_stride = (long)c.N * c.Cin * c.Hin * c.Win;
-    a.in.N = c.N; a.in.C = c.Cin; a.in.Hd = c.Hin; a.in.Wd = c.Win; a.in.uh = c.uh; a.in.uw = c.uw;
+    a.in.base = in; a.in.comp_stride = (long)c.N * creal.Cin * c.Hin * c.Win;
+    a.in.N = c.N; a.in.C = creal.Cin; a.in.Hd = c.Hin; a.in.Wd = c.Win; a.in.uh = c.uh; a.in.uw = c.uw; a.in.pw = pw;
     a.wpk = ws; a.bias = bias; a.out = out;
     a.out_cs = (long)c.N * c.Cout * c.Hout * c.Wout;
     a.Cout = c.Cout; a.Hout = c.Hout; a.Wout = c.Wout;
@@ -321,7 +350,7 @@ static int run_corr(const Problem& p, const Corr& c, int map, hipStream_t st, co
     if (rc != 0) return PHX_ERR_NOT_SUPPORTED;
     PHX_HIP(hipGetLastError());
     snprintf(g_name_buf, sizeof(g_name_buf), "qconv_%s_%smfma%s_p%d_%s_wco%d_ntw%d_ck%d_tile%dx%dx%d",
-             map == MAP_FWD ? "fwd" : "dgrad", f16 ? "f16" : "f32", pl.lds_filters ? (pl.chunks ? "ldsc" : "lds") : "", p.mode, p.dtype == PHX_F32 ? "f32" : "f16", pl.WCO,
+             map == MAP_FWD ? "fwd" : "dgrad", f16 ? "f16" : "f32", pl.lds_filters ? (pw ? "ldspw" : pl.chunks ? "ldsc" : "lds") : "", p.mode, p.dtype == PHX_F32 ? "f32" : "f16", pl.WCO,
              pl.NTW, pl.CK, pl.NB, pl.TH, pl.TW);
     g_last_kernel = g_name_buf;
     return PHX_OK;
@@ -434,9 +463,9 @@ static int run_wgrad(const Problem& p, hipStream_t st, const void* x, const void
     if (ws_bytes < pl.partial_bytes || !ws) return PHX_ERR_WORKSPACE;
     WgradArgs a;
     a.x.base = x; a.x.comp_stride = (long)p.n * p.ci * p.h * p.w; a.x.N = p.n; a.x.C = p.ci; a.x.Hd = p.h; a.x.Wd = p.w;
-    a.x.uh = a.x.uw = 1;
+    a.x.uh = a.x.uw = 1; a.x.pw = 0;
     a.g.base = g; a.g.comp_stride = (long)p.n * p.co * p.ho * p.wo; a.g.N = p.n; a.g.C = p.co; a.g.Hd = p.ho; a.g.Wd = p.wo;
-    a.g.uh = a.g.uw = 1;
+    a.g.uh = a.g.uw = 1; a.g.pw = 0;
     a.partial = static_cast<float*>(ws);
     a.Kh = p.kh; a.Kw = p.kw; a.sh = p.sh; a.sw = p.sw; a.dh = p.dh; a.dw = p.dw; a.pt = p.pt; a.pl = p.pl;
     a.NB = pl.NB; a.TH = pl.TH; a.TW = pl.TW; a.KP = pl.KP; a.KPp = pl.KPp; a.HPp = pl.HPp; a.HTH = pl.HTH;
@@ -482,9 +511,12 @@ static size_t workspace_for(const Problem& p, int pass) {
         WgPlan pl;
         return plan_wgrad(flatten_pointwise(p), wgrad_on_f16_mfma(p), pl) ? align_up(pl.partial_bytes, 256) : 0;
     }
-    const Corr c = (pass == PHX_PASS_FWD) ? corr_forward(p) : corr_dgrad(p);
+    int pw = 0;
+    Corr c;
     FwdPlan pl;
-    return plan_forward(c, p.mode, use_f16_mfma(p, pass), pl) ? align_up(pl.wpk_bytes, 256) : 0;
+    return plan_corr((pass == PHX_PASS_FWD) ? corr_forward(p) : corr_dgrad(p), p.mode, use_f16_mfma(p, pass), c, pl, pw)
+               ? align_up(pl.wpk_bytes, 256)
+               : 0;
 }
 
 static int do_fwd(const Problem& p, hipStream_t st, const void* x, const void* w, const void* bias, void* y, void* ws,
