@@ -365,9 +365,15 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_wgrad_f32_kernel(const Wgrad
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wco = wave & 1, wci = wave >> 1;
     const int m = lane & 31, kk = lane >> 5;
-    const int cot = blockIdx.x % P.co_tiles, cit = blockIdx.x / P.co_tiles;
-    const int kh = blockIdx.y / P.groups_per_row;
-    const int kw0 = (blockIdx.y % P.groups_per_row) * TPW;
+    // workgroups that share a reduction slice read the same gradient / input tiles: keep them on one XCD
+    int bid = xcd_remap(blockIdx.x, gridDim.x);
+    const int cot = bid % P.co_tiles;  bid /= P.co_tiles;
+    const int cit = bid % P.ci_tiles;  bid /= P.ci_tiles;
+    const int ngroups = P.groups_per_row * P.Kh;
+    const int grp = bid % ngroups;
+    const int zi = bid / ngroups;
+    const int kh = grp / P.groups_per_row;
+    const int kw0 = (grp % P.groups_per_row) * TPW;
     const int nkw = (P.Kw - kw0 < TPW) ? P.Kw - kw0 : TPW;
     const int HTW = (P.TW - 1) * P.sw + (nkw - 1) * P.dw + 1;
 
@@ -405,15 +411,15 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_wgrad_f32_kernel(const Wgrad
         stage_load<TS, CT, P2LOG>(sx, P.x, spx, cit * CT);
     };
     const int HPx = P.NB * P.HTH * HTW;
-    if ((int)blockIdx.z < ntiles) issue(blockIdx.z);
-    for (int tile = blockIdx.z; tile < ntiles; tile += gridDim.z) {
+    if (zi < ntiles) issue(zi);
+    for (int tile = zi; tile < ntiles; tile += P.zsplit) {
         __syncthreads();
         stage_store<CT, P2LOG, float>(gl, sg, spg, P.NB * thw, P.KPp);
         stage_store<CT, P2LOG, float>(xl, sx, spx, HPx, P.HPp);
         if (P.KP != P.NB * thw)  // odd pixel count: the padding column of the gradient window must be zero
             for (int c = tid; c < 4 * CT; c += WG_THREADS) gl[c * P.KPp + P.KP - 1] = 0.f;
         __syncthreads();
-        if (tile + (int)gridDim.z < ntiles) issue(tile + gridDim.z);
+        if (tile + P.zsplit < ntiles) issue(tile + P.zsplit);
         const float* ga = gl + (wco * 32 + m) * P.KPp + kk;
         const float* xb = xl + (wci * 32 + m) * P.HPp;
         for (int ks = 0; ks < P.KP; ks += 2) {
@@ -454,7 +460,7 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_wgrad_f32_kernel(const Wgrad
     // partial[z][tap][r][co][ci]
     const int taps = P.Kh * P.Kw;
     const long tap_stride = 4L * P.CoP * P.CiP;
-    float* dst = P.partial + (long)blockIdx.z * taps * tap_stride;
+    float* dst = P.partial + (long)zi * taps * tap_stride;
     const int ci = cit * CT + wci * 32 + m;
     const int co_base = cot * CT + wco * 32 + 4 * kk;
 #pragma unroll

@@ -373,7 +373,9 @@ static void finish_wgrad_plan(const Problem& p, int CoT, int CiT, WgPlan& best) 
     best.groups_per_row = cdiv(p.kw, best.TPW);
     const int xy = best.co_tiles * best.ci_tiles * best.groups_per_row * p.kh;
     const int ntiles = best.tiles_n * best.tiles_h * best.tiles_w;
-    best.Z = std::max(1, std::min(ntiles, 1024 / std::max(1, xy)));
+    int target = 512;  // two workgroups per CU: one round
+    if (const char* e = getenv("PHX_TUNE_WGS")) target = atoi(e);
+    best.Z = std::max(1, std::min(ntiles, target / std::max(1, xy)));
     best.partial_bytes = (size_t)best.Z * p.kh * p.kw * 4 * best.CoP * best.CiP * sizeof(float);
 }
 
@@ -474,16 +476,15 @@ static int run_wgrad(const Problem& p, hipStream_t st, const void* x, const void
     a.co_tiles = pl.co_tiles; a.ci_tiles = pl.ci_tiles; a.CoP = pl.CoP; a.CiP = pl.CiP;
     a.groups_per_row = pl.groups_per_row;
     a.cpr = pl.cpr; a.nchunks = pl.nchunks; a.ntiles = pl.ntiles; a.zsplit = pl.Z;
-    const int nblocks16 = pl.co_tiles * pl.ci_tiles * pl.groups_per_row * p.kh * pl.Z;
-    const dim3 grid(pl.co_tiles * pl.ci_tiles, pl.groups_per_row * p.kh, pl.Z);
+    const int nblocks = pl.co_tiles * pl.ci_tiles * pl.groups_per_row * p.kh * pl.Z;
     const bool half_storage = p.dtype == PHX_F16;
     {
         KernelTimer timer(st);
         if (f16) {
-            if (launch_wgrad_f16(p.mode, pl.MT, pl.NT, pl.TPW, pl.SW, a, nblocks16, pl.lds_bytes, st) != 0)
+            if (launch_wgrad_f16(p.mode, pl.MT, pl.NT, pl.TPW, pl.SW, a, nblocks, pl.lds_bytes, st) != 0)
                 return PHX_ERR_RUNTIME;
         } else {
-            launch_wgrad_f32(half_storage, p.mode, a, grid, pl.lds_bytes, st);
+            launch_wgrad_f32(half_storage, p.mode, a, dim3(nblocks), pl.lds_bytes, st);
         }
     }
     PHX_HIP(hipGetLastError());
