@@ -32,6 +32,20 @@ WORKLOADS = {
 }
 RESNET = "c5_qresnet50"  # quaternion ResNet-50 forward+backward, N=64, 224x224, fp16 full16 policy
 
+# HBM bytes per launch of the main kernel of each pass, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
+# this script (summaries under profiles/): (FETCH_SIZE * 2 KiB + WRITE_SIZE * 1 KiB), the unit sizes being
+# what the same counters read for a plain 256 MiB device copy.  Configurations not profiled report null.
+KIB = 1024.0
+MEASURED_TRAFFIC = {
+    ("c2_pw_f32", 8): {"fwd": (67977.4 * 2 + 134848.0) * KIB, "bwd_data": (67929.3 * 2 + 134848.0) * KIB,
+                       "bwd_weights": (200924.6 * 2 + 32768.0) * KIB},
+    ("c3_k3_f32", 8): {"fwd": (144540.2 * 2 + 252797.4) * KIB, "bwd_data": (148207.4 * 2 + 260483.6) * KIB},
+    ("c4_k3_f16_128_28", 16): {"fwd": (83626.8 * 2 + 105457.0) * KIB, "bwd_data": (83626.8 * 2 + 105457.0) * KIB,
+                               "bwd_weights": (179973.6 * 2 + 48384.0) * KIB},
+    ("c4_k3_f16_128_28", 8): {"fwd": (119473.0 * 2 + 105540.2) * KIB, "bwd_data": (119625.7 * 2 + 104716.3) * KIB,
+                              "bwd_weights": (359772.5 * 2 + 32256.0) * KIB},
+}
+
 
 def parse():
     ap = argparse.ArgumentParser()
@@ -246,6 +260,14 @@ def main():
     dominant = max(per_pass, key=per_pass.get)
     compute = "f32" if (dt == "f32" or policy == "fp32" or (policy == "backward32" and dominant != "fwd")) else "f16"
     achieved = flops_pass / (per_pass[dominant] * 1e-3) / 1e12
+    esize = 4 if dt == "f32" else 2
+    # algorithmic bytes of a pass: read the activations (or the gradient), read the filters, write the result
+    bytes_pass = {
+        "fwd": esize * (x.numel() + wt.numel() + y.numel()),
+        "bwd_data": esize * (gr.numel() + wt.numel() + dx.numel()),
+        "bwd_weights": esize * (x.numel() + gr.numel() + dw.numel()),
+    }
+    traffic = MEASURED_TRAFFIC.get((args.workload, mode), {}).get(dominant)
     out = {
         "metric": METRIC, "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
@@ -257,8 +279,10 @@ def main():
         "frac_of_mfma_peak": value / PEAK_TFLOPS[compute],
         "executed_tflops": value * (0.5 if mode == 8 else 1.0),
         "kernel_ms": per_pass, "kernels": names,
+        "algorithmic_hbm_gb_s": {k: bytes_pass[k] / (per_pass[k] * 1e-3) / 1e9 for k in per_pass},
         "roofline": {"bound": "mfma", "kernel": names[dominant], "achieved": achieved, "peak": PEAK_TFLOPS[compute],
-                     "unit": "TFLOP/s", "frac": achieved / PEAK_TFLOPS[compute], "traffic": None,
+                     "unit": "TFLOP/s", "frac": achieved / PEAK_TFLOPS[compute], "traffic": traffic,
+                     "algorithmic_bytes": bytes_pass[dominant],
                      "executed": achieved * (0.5 if mode == 8 else 1.0)},
     }
     if not args.no_cpu_baseline:
