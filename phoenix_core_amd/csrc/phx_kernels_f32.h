@@ -151,6 +151,97 @@ __device__ __forceinline__ void conv_epilogue(const ConvArgs& P, const f32x16 (&
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Vector staging of the activation window for the fp32-MFMA kernels (VSTG): the LDS layout
+// [component][channel][position] is position-contiguous like NCHW itself, so staging is a plain
+// copy.  A thread owns one group of 4 consecutive positions of a window row (HTW is a multiple of 4)
+// and walks over the (component, channel) planes: one 16-byte (fp32) or 8-byte (fp16 storage) load
+// and one 16-byte LDS store per plane, a quarter of the instructions of the per-position form.
+// Positions outside the image are cleared with a mask that is fixed per thread; threads whose
+// loads could leave the tensor load nothing and fill their positions element by element.
+// 2^(P2LOG-2) position groups x (1024 >> P2LOG) thread groups; thread group g takes planes g, g+G4, ...
+// ---------------------------------------------------------------------------------------------
+struct StageVec {
+    long goff;           // element offset of the group's first position from component 0, channel 0
+    int lpos;            // first window position of the group
+    int group;
+    unsigned int bits;   // positions inside the image
+    bool live, careful;
+};
+
+template <typename TS, int P2LOG>
+__device__ __forceinline__ StageVec make_stage_vec(const TileSrc& s, int n0, int h0, int w0, int NB, int HTH, int HTW,
+                                                   int HP) {
+    StageVec sv;
+    constexpr int NPC = 1 << (P2LOG - 2);
+    const int pc = threadIdx.x & (NPC - 1);
+    sv.group = threadIdx.x >> (P2LOG - 2);
+    sv.lpos = pc * 4;
+    const int row = sv.lpos / HTW, col = sv.lpos - row * HTW;
+    const int nb = row / HTH, hr = row - nb * HTH;
+    const int vh = h0 + hr, vw0 = w0 + col;
+    sv.live = sv.lpos < HP && nb < NB && (n0 + nb) < s.N && vh >= 0 && vh < s.Hd;
+    sv.bits = sv.live ? interval_bits<4>(-vw0, s.Wd - vw0) : 0u;
+    sv.goff = ((long)(n0 + nb) * s.C * s.Hd + vh) * s.Wd + vw0;
+    const long plane = (long)s.Hd * s.Wd;
+    const long total = 3 * s.comp_stride + (long)s.N * s.C * plane;
+    sv.careful = sv.live && (sv.goff < 0 || sv.goff + 3 * s.comp_stride + (long)(s.C - 1) * plane + 4 > total);
+    return sv;
+}
+
+// plane index e*G4 + group -> (component, channel of the chunk)
+template <typename TS, int NCH, int P2LOG>
+__device__ __forceinline__ void stage_vec_load(f32x4 (&v)[(NCH << P2LOG) >> 8], const TileSrc& s, const StageVec& sv,
+                                               int c0, int e) {
+    constexpr int G4 = (4 * WG_THREADS) >> P2LOG;
+    const TS* origin = static_cast<const TS*>(s.base);
+    const long plane = (long)s.Hd * s.Wd;
+    const int pc = e * G4 + sv.group;
+    const int p = pc / NCH, c = c0 + pc % NCH;
+    // channels past the tensor meet zero filters: any finite value will do, the tensor's first bytes are safe
+    const TS* ptr = (sv.live && !sv.careful && c < s.C) ? origin + sv.goff + p * s.comp_stride + c * plane : origin;
+    if constexpr (sizeof(TS) == 4) {
+        typedef f32x4 f32x4_a4 __attribute__((aligned(4)));
+        v[e] = *reinterpret_cast<const f32x4_a4*>(ptr);
+    } else {
+        typedef _Float16 f16x4_a2 __attribute__((ext_vector_type(4), aligned(2)));
+        const f16x4_a2 h = *reinterpret_cast<const f16x4_a2*>(ptr);
+        v[e] = f32x4{(float)h[0], (float)h[1], (float)h[2], (float)h[3]};
+    }
+}
+
+template <typename TS, int NCH, int P2LOG>
+__device__ __forceinline__ void stage_vec_store(float* lds, const f32x4 (&v)[(NCH << P2LOG) >> 8], const TileSrc& s,
+                                                const StageVec& sv, int c0, int HP, int HPp) {
+    constexpr int G4 = (4 * WG_THREADS) >> P2LOG;
+    constexpr int E = (NCH << P2LOG) >> 8;
+    if (sv.lpos >= HP) return;
+    const unsigned int keep = sv.careful ? 0u : sv.bits;
+    u32x4 mk;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) mk[i] = (unsigned int)((int)(keep << (31 - i)) >> 31);
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+        const u32x4 w = __builtin_bit_cast(u32x4, v[e]) & mk;
+        *reinterpret_cast<u32x4*>(lds + (e * G4 + sv.group) * HPp + sv.lpos) = w;
+    }
+    if (sv.careful) {
+        const TS* origin = static_cast<const TS*>(s.base);
+        const long plane = (long)s.Hd * s.Wd;
+#pragma unroll 2
+        for (int e = 0; e < E; ++e) {
+            const int pc = e * G4 + sv.group;
+            const int p = pc / NCH, c = c0 + pc % NCH;
+            float t[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                t[i] = (c < s.C && ((sv.bits >> i) & 1)) ? ldf<TS>(origin + sv.goff + p * s.comp_stride + c * plane + i) : 0.f;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) lds[pc * HPp + sv.lpos + i] = t[i];
+        }
+    }
+}
+
 // Forward / input-gradient kernel.
 //   workgroup = 4 waves = WCO filter sub-tiles (32 output channels each) x 4/WCO pixel ranges,
 //   each wave owns NTW MFMA column tiles of 32 output pixels and all four output components.
@@ -158,7 +249,7 @@ __device__ __forceinline__ void conv_epilogue(const ConvArgs& P, const f32x16 (&
 //   lane and K step, prefetched one step ahead); B operand = activations from the LDS halo window.
 //   MODE 16: acc[q] += W_{p^q} * (+-x_p), 16 MFMAs per K step, filters reused across the 4x4 block.
 //   MODE 8 : acc[i] += R_i * L_i with the 8 lanes L_i formed in registers, 8 MFMAs per K step.
-template <typename TS, int MODE, int MAP, int WCO, int NTW, int CK, int P2LOG>
+template <typename TS, int MODE, int MAP, int WCO, int NTW, int CK, int P2LOG, bool VSTG>
 __global__ void __launch_bounds__(WG_THREADS, (MODE == 8 || NTW == 1) ? 2 : 1) qconv_fwd_f32_kernel(const ConvArgs P) {
     constexpr int WPX = 4 / WCO;
     constexpr int NACC = (MODE == 16) ? 4 : 8;
@@ -204,31 +295,61 @@ __global__ void __launch_bounds__(WG_THREADS, (MODE == 8 || NTW == 1) ? 2 : 1) q
     const int steps_per_chunk = P.taps * (CK / 2);
     const long nsteps = (long)P.nchunks * steps_per_chunk;
     const float* wptr = static_cast<const float*>(P.wpk) + ((long)(ct * WCO + wco) * nsteps * 64 + lane) * WC;
-    f32x4 wcur[WC / 4], wnext[WC / 4];
+    // packed filters: register pipeline two K steps deep (an L2 hit takes longer than one step's MFMAs)
+    f32x4 wcur[WC / 4], wnext[WC / 4], wnext2[WC / 4];
 #pragma unroll
-    for (int v = 0; v < WC / 4; ++v) wcur[v] = *reinterpret_cast<const f32x4*>(wptr + 4 * v);
+    for (int v = 0; v < WC / 4; ++v) {
+        wcur[v] = *reinterpret_cast<const f32x4*>(wptr + 4 * v);
+        wnext[v] = *reinterpret_cast<const f32x4*>(wptr + (nsteps > 1 ? 1 : 0) * (64 * WC) + 4 * v);
+    }
 
     long step = 0;
     const long cpitch = (long)CK * P.HPp;  // LDS floats between components
     // 2^P2LOG window positions, 256 >> P2LOG thread groups sharing the 4*CK planes of a chunk
     const StagePos sp = make_stage_pos<P2LOG>(P.in, n0, h0, w0, P.NB, P.HTH, P.HTW);
-    float stage[(4 * CK) >> (8 - P2LOG)];
-    stage_load<TS, CK, P2LOG>(stage, P.in, sp, 0);
+    const StageVec sv = make_stage_vec<TS, P2LOG>(P.in, n0, h0, w0, P.NB, P.HTH, P.HTW, P.HP);
+    constexpr int EV = (CK << P2LOG) >> 8;  // vector loads per thread and chunk
+    float stage[VSTG ? 1 : ((4 * CK) >> (8 - P2LOG))];
+    f32x4 stagev[VSTG ? EV : 1];
+    if constexpr (VSTG) {
+#pragma unroll
+        for (int e = 0; e < EV; ++e) stage_vec_load<TS, CK, P2LOG>(stagev, P.in, sv, 0, e);
+    } else {
+        stage_load<TS, CK, P2LOG>(stage, P.in, sp, 0);
+    }
+    PHX_PHASES_BEGIN(6)
     for (int chunk = 0; chunk < P.nchunks; ++chunk) {
         __syncthreads();
-        stage_store<CK, P2LOG, float>(lds, stage, sp, P.HP, P.HPp);
+        PHX_STAMP(0)
+        if constexpr (VSTG) stage_vec_store<TS, CK, P2LOG>(lds, stagev, P.in, sv, chunk * CK, P.HP, P.HPp);
+        else stage_store<CK, P2LOG, float>(lds, stage, sp, P.HP, P.HPp);
+        PHX_STAMP(1)
         __syncthreads();
-        // next chunk's global loads fly while this chunk is multiplied
-        if (chunk + 1 < P.nchunks) stage_load<TS, CK, P2LOG>(stage, P.in, sp, (chunk + 1) * CK);
+        PHX_STAMP(2)
+        // next chunk's global loads fly while this chunk is multiplied; the vector form deals them out over
+        // the K steps of the first tap (a wave that issues them back to back stalls until all are taken)
+        const bool more = chunk + 1 < P.nchunks;
+        if constexpr (!VSTG) {
+            if (more) stage_load<TS, CK, P2LOG>(stage, P.in, sp, (chunk + 1) * CK);
+        }
+        PHX_STAMP(3)
         int kh = 0, kw = 0;
         for (int tap = 0; tap < P.taps; ++tap) {
             const int tapoff = kh * P.dh * P.HTW + kw * P.dw;
 #pragma unroll
             for (int cp = 0; cp < CK / 2; ++cp) {
-                const long nxt = (step + 1 < nsteps) ? step + 1 : step;
+                if constexpr (VSTG) {
+                    constexpr int LPS = (EV + CK / 2 - 1) / (CK / 2);  // loads per K step
+                    if (more && tap == 0) {
+#pragma unroll
+                        for (int e = cp * LPS; e < (cp + 1) * LPS && e < EV; ++e)
+                            stage_vec_load<TS, CK, P2LOG>(stagev, P.in, sv, (chunk + 1) * CK, e);
+                    }
+                }
+                const long nxt = (step + 2 < nsteps) ? step + 2 : nsteps - 1;
 #pragma unroll
                 for (int v = 0; v < WC / 4; ++v)
-                    wnext[v] = *reinterpret_cast<const f32x4*>(wptr + nxt * (64 * WC) + 4 * v);
+                    wnext2[v] = *reinterpret_cast<const f32x4*>(wptr + nxt * (64 * WC) + 4 * v);
                 const float* xb = lds + (2 * cp + kk) * P.HPp + tapoff;
 #pragma unroll
                 for (int t = 0; t < NTW; ++t) {
@@ -255,15 +376,21 @@ __global__ void __launch_bounds__(WG_THREADS, (MODE == 8 || NTW == 1) ? 2 : 1) q
                     }
                 }
 #pragma unroll
-                for (int v = 0; v < WC / 4; ++v) wcur[v] = wnext[v];
+                for (int v = 0; v < WC / 4; ++v) {
+                    wcur[v] = wnext[v];
+                    wnext[v] = wnext2[v];
+                }
                 ++step;
             }
             if (++kw == P.Kw) { kw = 0; ++kh; }
         }
+        PHX_STAMP(4)
     }
 
     // epilogue: fold lanes (8-product), add bias, store NCHW with components on the batch axis
     conv_epilogue<TS, MODE, MAP, NTW, NACC>(P, acc, (ct * WCO + wco) * 32 + 4 * kk, oaddr, pvalid);
+    PHX_STAMP(5)
+    PHX_PHASES_REPORT("fwd_f32: barrier / store / barrier / load issue / mfma / epilogue", 6)
 }
 
 // Filter packing for the kernel above.  One value group per (32-channel filter tile, K step, lane):

@@ -14,6 +14,7 @@ struct FwdVariant {
     int WCO, NTW, CK, P2LOG;
     bool lds_filters;   // fp16 MFMA only: filters staged through LDS (qconv_fwd_f16_lds_kernel)
     int ngroups;        // tap groups per chunk for that kernel
+    bool vstage;        // fp32 MFMA: activations staged as groups of 4 positions (no zero insertion)
     bool pairs;         // fp16 MFMA: activations staged as aligned position pairs
     bool chunks;        // fp16 MFMA, filters in LDS: activations staged as 8-position chunks
     int pw;             // pointwise convolution run as a column of pw virtual taps over 16-channel sub-chunks (0 = off)

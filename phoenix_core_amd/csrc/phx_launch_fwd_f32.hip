@@ -5,13 +5,16 @@ namespace phx {
 
 template <typename TS, int MODE, int MAP>
 static int launch_variant(const FwdVariant& v, const ConvArgs& a, hipStream_t st) {
-#define PHX_CASE(WCO_, NTW_, CK_, P2_)                                                                        \
-    if (v.WCO == WCO_ && v.NTW == NTW_ && v.CK == CK_ && v.P2LOG == P2_) {                                    \
-        hipLaunchKernelGGL((qconv_fwd_f32_kernel<TS, MODE, MAP, WCO_, NTW_, CK_, P2_>), dim3(v.wgs),          \
+#define PHX_CASE(WCO_, NTW_, CK_, P2_, VS_)                                                                   \
+    if (v.WCO == WCO_ && v.NTW == NTW_ && v.CK == CK_ && v.P2LOG == P2_ && v.vstage == VS_) {                 \
+        hipLaunchKernelGGL((qconv_fwd_f32_kernel<TS, MODE, MAP, WCO_, NTW_, CK_, P2_, VS_>), dim3(v.wgs),     \
                            dim3(WG_THREADS), v.lds_bytes, st, a);                                             \
         return 0;                                                                                             \
     }
-#define PHX_CASES(WCO_, NTW_) PHX_CASE(WCO_, NTW_, 8, 8) PHX_CASE(WCO_, NTW_, 16, 7) PHX_CASE(WCO_, NTW_, 32, 6)
+    // vector staging for every window without zero insertion; the per-position form only in its general shape
+#define PHX_CASES(WCO_, NTW_)                                                                       \
+    PHX_CASE(WCO_, NTW_, 8, 8, true) PHX_CASE(WCO_, NTW_, 16, 7, true) PHX_CASE(WCO_, NTW_, 32, 6, true) \
+    PHX_CASE(WCO_, NTW_, 8, 8, false)
     PHX_CASES(1, 1) PHX_CASES(2, 1) PHX_CASES(4, 1)
     if constexpr (MODE == 16) {
         PHX_CASES(1, 2) PHX_CASES(2, 2) PHX_CASES(4, 2)

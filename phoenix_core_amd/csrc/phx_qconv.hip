@@ -161,6 +161,7 @@ struct FwdPlan {
     int CK, P2LOG;           // channels per chunk and log2 staging positions of the kernel variant
     bool lds_filters;        // fp16 MFMA, 16-product, more than one tap: filters go through LDS
     int ngroups;             // tap groups per chunk in that case
+    bool vstage;             // fp32 MFMA: window rows widened to a multiple of 4, staged as 4-position vectors
     bool pairs;              // fp16 MFMA: window rows widened to even columns, staged as position pairs
     bool chunks;             // fp16 MFMA, filters in LDS: window rows widened to a multiple of 8, staged as chunks
     int NB, TH, TW, HTH, HTW, HP, HPp;
@@ -179,7 +180,8 @@ static bool plan_forward(const Corr& c, int mode, bool f16mfma, FwdPlan& best) {
     const bool ldsk = f16mfma && c.Kh * c.Kw > 1 && (mode == 16 || c.uw == 1);
     const bool chunks = ldsk && c.uw == 1;
     const bool pairs = f16mfma && !chunks && (c.Win % 2 == 0) && c.uw == 1;
-    best.pairs = pairs; best.chunks = chunks;
+    const bool vstage = !f16mfma && c.uw == 1;
+    best.pairs = pairs; best.chunks = chunks; best.vstage = vstage;
     const int wcos[3] = {1, 2, 4};
     // PHX_TUNE_TILE="wco,ntw" pins the workgroup shape (kernel tuning experiments)
     int force_wco = 0, force_ntw = 0;
@@ -207,6 +209,7 @@ static bool plan_forward(const Corr& c, int mode, bool f16mfma, FwdPlan& best) {
                     int HTW = (TW - 1) * c.sw + (c.Kw - 1) * c.dw + 1;
                     if (pairs) HTW = (HTW + 2) & ~1;  // room for the even start column, even pitch
                     if (chunks) HTW = (HTW + 7) & ~7;  // whole 8-position chunks
+                    if (vstage) HTW = (HTW + 3) & ~3;  // whole 4-position groups
                     const int HP = NB * HTH * HTW;
                     const int HPp = HP;
                     if (HP > 256) continue;  // one staging position per thread
@@ -255,7 +258,8 @@ static bool plan_forward(const Corr& c, int mode, bool f16mfma, FwdPlan& best) {
     // fp32 MFMA: pointwise problems are bandwidth/latency bound and take as many channels per
     // chunk as 32 staging registers per thread allow; everything else uses 8-channel chunks
     best.CK = F32_CK; best.P2LOG = 8; best.lds_filters = false; best.ngroups = 0;
-    if (taps == 1 && c.Cin >= 32) {
+    if (vstage) best.HPp = (best.HP + 3) & ~3;  // 16-byte aligned LDS rows
+    if (taps == 1 && c.Cin >= 32 && vstage) {
         if (best.HP <= 64) { best.CK = 32; best.P2LOG = 6; }
         else if (best.HP <= 128) { best.CK = 16; best.P2LOG = 7; }
     }
@@ -314,7 +318,7 @@ static int run_corr(const Problem& p, const Corr& creal, int map, hipStream_t st
     FwdVariant v;
     v.half_storage = p.dtype == PHX_F16; v.f16_mfma = f16; v.mode = p.mode; v.map = map;
     v.WCO = pl.WCO; v.NTW = pl.NTW; v.CK = pl.CK; v.P2LOG = pl.P2LOG; v.wgs = pl.wgs; v.lds_bytes = pl.lds_bytes;
-    v.lds_filters = pl.lds_filters; v.ngroups = pl.ngroups; v.pairs = pl.pairs; v.chunks = pl.chunks; v.pw = pw;
+    v.lds_filters = pl.lds_filters; v.ngroups = pl.ngroups; v.pairs = pl.pairs; v.chunks = pl.chunks; v.pw = pw; v.vstage = pl.vstage;
 
     PackArgs pa;
     pa.w = w; pa.out = ws;
