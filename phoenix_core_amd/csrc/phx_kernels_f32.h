@@ -242,6 +242,37 @@ __device__ __forceinline__ void stage_vec_store(float* lds, const f32x4 (&v)[(NC
     }
 }
 
+// same, for LDS rows with an odd pitch (bank-conflict-free 4-byte reads down a column of rows): four 4-byte stores
+template <typename TS, int NCH, int P2LOG>
+__device__ __forceinline__ void stage_vec_store_scalar(float* lds, const f32x4 (&v)[(NCH << P2LOG) >> 8], const TileSrc& s,
+                                                       const StageVec& sv, int c0, int HP, int pitch) {
+    constexpr int G4 = (4 * WG_THREADS) >> P2LOG;
+    constexpr int E = (NCH << P2LOG) >> 8;
+    if (sv.lpos >= HP) return;
+    const unsigned int keep = sv.careful ? 0u : sv.bits;
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+        float* dst = lds + (e * G4 + sv.group) * pitch + sv.lpos;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) dst[i] = ((keep >> i) & 1) ? v[e][i] : 0.f;
+    }
+    if (sv.careful) {
+        const TS* origin = static_cast<const TS*>(s.base);
+        const long plane = (long)s.Hd * s.Wd;
+#pragma unroll 2
+        for (int e = 0; e < E; ++e) {
+            const int pc = e * G4 + sv.group;
+            const int p = pc / NCH, c = c0 + pc % NCH;
+            float t[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                t[i] = (c < s.C && ((sv.bits >> i) & 1)) ? ldf<TS>(origin + sv.goff + p * s.comp_stride + c * plane + i) : 0.f;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) lds[pc * pitch + sv.lpos + i] = t[i];
+        }
+    }
+}
+
 // Forward / input-gradient kernel.
 //   workgroup = 4 waves = WCO filter sub-tiles (32 output channels each) x 4/WCO pixel ranges,
 //   each wave owns NTW MFMA column tiles of 32 output pixels and all four output components.
@@ -480,7 +511,7 @@ struct WgradArgs {
     int cpr, nchunks, ntiles, zsplit;  // fp16 kernel: 8-pixel chunks per output row / in total, pixel tiles, reduction slices
 };
 
-template <typename TS, int MODE, int TPW>
+template <typename TS, int MODE, int TPW, bool VEC>
 __global__ void __launch_bounds__(WG_THREADS) qconv_wgrad_f32_kernel(const WgradArgs P) {
     constexpr int CT = 64;
     constexpr int NACC = (MODE == 16) ? 4 : 8;
@@ -502,7 +533,8 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_wgrad_f32_kernel(const Wgrad
     const int kh = grp / P.groups_per_row;
     const int kw0 = (grp % P.groups_per_row) * TPW;
     const int nkw = (P.Kw - kw0 < TPW) ? P.Kw - kw0 : TPW;
-    const int HTW = (P.TW - 1) * P.sw + (nkw - 1) * P.dw + 1;
+    const int HTWx = (P.TW - 1) * P.sw + (nkw - 1) * P.dw + 1;
+    const int HTW = VEC ? ((HTWx + 3) & ~3) : HTWx;  // vector staging: whole groups of 4 positions per window row
 
     const int thw = P.TH * P.TW;
     for (int k = tid; k < P.KP; k += WG_THREADS) {
@@ -521,63 +553,103 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_wgrad_f32_kernel(const Wgrad
 
     const int ntiles = P.tiles_n * P.tiles_h * P.tiles_w;
     const long gcp = (long)CT * P.KPp, xcp = (long)CT * P.HPp;
-    constexpr int P2LOG = 5;  // 32 window positions x 8 plane groups
-    float sg[32], sx[32];
+    constexpr int P2LOG = 5;  // 32 window positions x 8 plane groups (vector form: 8 groups of 4 x 32 plane groups)
+    float sg[VEC ? 1 : 32], sx[VEC ? 1 : 32];
+    f32x4 vg[VEC ? 8 : 1], vx[VEC ? 8 : 1];
     StagePos spg, spx;
-    auto issue = [&](int tile) {
+    StageVec svg, svx;
+    auto locate = [&](int tile) {
         const int tw = tile % P.tiles_w;
         const int th = (tile / P.tiles_w) % P.tiles_h;
         const int tn = tile / (P.tiles_w * P.tiles_h);
         const int n0 = tn * P.NB, ho0 = th * P.TH, wo0 = tw * P.TW;
+        const int h0x = ho0 * P.sh - P.pt + kh * P.dh, w0x = wo0 * P.sw - P.pl + kw0 * P.dw;
         // gradient window: TH x TW output pixels, no halo; pixels beyond the tensor are zero and
         // therefore contribute nothing whatever the input window holds there
-        spg = make_stage_pos<P2LOG>(P.g, n0, ho0, wo0, P.NB, P.TH, P.TW);
-        spx = make_stage_pos<P2LOG>(P.x, n0, ho0 * P.sh - P.pt + kh * P.dh, wo0 * P.sw - P.pl + kw0 * P.dw, P.NB, P.HTH,
-                                    HTW);
-        stage_load<TS, CT, P2LOG>(sg, P.g, spg, cot * CT);
-        stage_load<TS, CT, P2LOG>(sx, P.x, spx, cit * CT);
+        if constexpr (VEC) {
+            svg = make_stage_vec<TS, P2LOG>(P.g, n0, ho0, wo0, P.NB, P.TH, P.TW, P.NB * thw);
+            svx = make_stage_vec<TS, P2LOG>(P.x, n0, h0x, w0x, P.NB, P.HTH, HTW, P.NB * P.HTH * HTW);
+        } else {
+            spg = make_stage_pos<P2LOG>(P.g, n0, ho0, wo0, P.NB, P.TH, P.TW);
+            spx = make_stage_pos<P2LOG>(P.x, n0, h0x, w0x, P.NB, P.HTH, HTW);
+        }
+    };
+    auto issue = [&](int tile) {
+        locate(tile);
+        if constexpr (VEC) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                stage_vec_load<TS, CT, P2LOG>(vg, P.g, svg, cot * CT, e);
+                stage_vec_load<TS, CT, P2LOG>(vx, P.x, svx, cit * CT, e);
+            }
+        } else {
+            stage_load<TS, CT, P2LOG>(sg, P.g, spg, cot * CT);
+            stage_load<TS, CT, P2LOG>(sx, P.x, spx, cit * CT);
+        }
     };
     const int HPx = P.NB * P.HTH * HTW;
     if (zi < ntiles) issue(zi);
     for (int tile = zi; tile < ntiles; tile += P.zsplit) {
         __syncthreads();
-        stage_store<CT, P2LOG, float>(gl, sg, spg, P.NB * thw, P.KPp);
-        stage_store<CT, P2LOG, float>(xl, sx, spx, HPx, P.HPp);
+        if constexpr (VEC) {
+            stage_vec_store_scalar<TS, CT, P2LOG>(gl, vg, P.g, svg, cot * CT, P.NB * thw, P.KPp);
+            stage_vec_store_scalar<TS, CT, P2LOG>(xl, vx, P.x, svx, cit * CT, HPx, P.HPp);
+        } else {
+            stage_store<CT, P2LOG, float>(gl, sg, spg, P.NB * thw, P.KPp);
+            stage_store<CT, P2LOG, float>(xl, sx, spx, HPx, P.HPp);
+        }
         if (P.KP != P.NB * thw)  // odd pixel count: the padding column of the gradient window must be zero
             for (int c = tid; c < 4 * CT; c += WG_THREADS) gl[c * P.KPp + P.KP - 1] = 0.f;
         __syncthreads();
-        if (tile + P.zsplit < ntiles) issue(tile + P.zsplit);
+        const bool more = tile + P.zsplit < ntiles;
+        if constexpr (VEC) {
+            if (more) locate(tile + P.zsplit);
+        } else {
+            if (more) issue(tile + P.zsplit);
+        }
         const float* ga = gl + (wco * 32 + m) * P.KPp + kk;
         const float* xb = xl + (wci * 32 + m) * P.HPp;
-        for (int ks = 0; ks < P.KP; ks += 2) {
-            float g[4];
+        // (vector form: at most 16 K steps, unrolled, so that the next tile's loads can be dealt over them --
+        // a wave that issues them back to back stalls until the memory pipeline has taken them all)
 #pragma unroll
-            for (int q = 0; q < 4; ++q) g[q] = ga[q * gcp + ks];
-            const int po = poff[ks + kk];
-            float G[8];
-            if constexpr (MODE == 8) lanes_grad(g, G, 0.5f);
+        for (int ksi = 0; ksi < (VEC ? 16 : 1); ++ksi) {
+            if constexpr (VEC) {
+                if (more && ksi < 8) {
+                    stage_vec_load<TS, CT, P2LOG>(vg, P.g, svg, cot * CT, ksi);
+                    stage_vec_load<TS, CT, P2LOG>(vx, P.x, svx, cit * CT, ksi);
+                }
+                if (2 * ksi >= P.KP) continue;
+            }
+            for (int ks = VEC ? 2 * ksi : 0; ks < (VEC ? 2 * ksi + 2 : P.KP); ks += 2) {
+                float g[4];
 #pragma unroll
-            for (int t = 0; t < TPW; ++t) {
-                if (t < nkw) {
-                    float x[4];
+                for (int q = 0; q < 4; ++q) g[q] = ga[q * gcp + ks];
+                const int po = poff[ks + kk];
+                float G[8];
+                if constexpr (MODE == 8) lanes_grad(g, G, 0.5f);
 #pragma unroll
-                    for (int p = 0; p < 4; ++p) x[p] = xb[p * xcp + po + t * P.dw];
-                    if constexpr (MODE == 16) {
-                        float nx[4];
+                for (int t = 0; t < TPW; ++t) {
+                    if (t < nkw) {
+                        float x[4];
 #pragma unroll
-                        for (int p = 0; p < 4; ++p) nx[p] = -x[p];
+                        for (int p = 0; p < 4; ++p) x[p] = xb[p * xcp + po + t * P.dw];
+                        if constexpr (MODE == 16) {
+                            float nx[4];
 #pragma unroll
-                        for (int p = 0; p < 4; ++p)
+                            for (int p = 0; p < 4; ++p) nx[p] = -x[p];
 #pragma unroll
-                            for (int q = 0; q < 4; ++q)
-                                acc[t][p ^ q] = __builtin_amdgcn_mfma_f32_32x32x2f32(g[q], qneg(p, q) ? nx[p] : x[p],
-                                                                                     acc[t][p ^ q], 0, 0, 0);
-                    } else {
-                        float L[8];
-                        lanes_left(x, L);
+                            for (int p = 0; p < 4; ++p)
 #pragma unroll
-                        for (int i = 0; i < 8; ++i)
-                            acc[t][i] = __builtin_amdgcn_mfma_f32_32x32x2f32(G[i], L[i], acc[t][i], 0, 0, 0);
+                                for (int q = 0; q < 4; ++q)
+                                    acc[t][p ^ q] = __builtin_amdgcn_mfma_f32_32x32x2f32(g[q], qneg(p, q) ? nx[p] : x[p],
+                                                                                         acc[t][p ^ q], 0, 0, 0);
+                        } else {
+                            float L[8];
+                            lanes_left(x, L);
+#pragma unroll
+                            for (int i = 0; i < 8; ++i)
+                                acc[t][i] = __builtin_amdgcn_mfma_f32_32x32x2f32(G[i], L[i], acc[t][i], 0, 0, 0);
+                        }
                     }
                 }
             }

@@ -3,15 +3,17 @@
 
 namespace phx {
 
-int launch_wgrad_f32(bool half_storage, int mode, const WgradArgs& a, dim3 grid, size_t lds_bytes, hipStream_t st) {
+template <typename TS, bool VEC>
+static void launch_ts(int mode, const WgradArgs& a, dim3 grid, size_t lds_bytes, hipStream_t st) {
     const dim3 b(WG_THREADS);
-    if (half_storage) {
-        if (mode == 16) hipLaunchKernelGGL((qconv_wgrad_f32_kernel<_Float16, 16, 3>), grid, b, lds_bytes, st, a);
-        else hipLaunchKernelGGL((qconv_wgrad_f32_kernel<_Float16, 8, 1>), grid, b, lds_bytes, st, a);
-    } else {
-        if (mode == 16) hipLaunchKernelGGL((qconv_wgrad_f32_kernel<float, 16, 3>), grid, b, lds_bytes, st, a);
-        else hipLaunchKernelGGL((qconv_wgrad_f32_kernel<float, 8, 1>), grid, b, lds_bytes, st, a);
-    }
+    if (mode == 16) hipLaunchKernelGGL((qconv_wgrad_f32_kernel<TS, 16, 3, VEC>), grid, b, lds_bytes, st, a);
+    else hipLaunchKernelGGL((qconv_wgrad_f32_kernel<TS, 8, 1, VEC>), grid, b, lds_bytes, st, a);
+}
+
+int launch_wgrad_f32(bool half_storage, bool vec, int mode, const WgradArgs& a, dim3 grid, size_t lds_bytes,
+                     hipStream_t st) {
+    if (half_storage) vec ? launch_ts<_Float16, true>(mode, a, grid, lds_bytes, st) : launch_ts<_Float16, false>(mode, a, grid, lds_bytes, st);
+    else vec ? launch_ts<float, true>(mode, a, grid, lds_bytes, st) : launch_ts<float, false>(mode, a, grid, lds_bytes, st);
     return 0;
 }
 

@@ -367,6 +367,7 @@ struct WgPlan {
     int TPW, NB, TH, TW, KP, KPp, HPp, HPx, HTH, HTWmax;
     int tiles_n, tiles_h, tiles_w, co_tiles, ci_tiles, CoP, CiP, groups_per_row, Z;
     int MT, NT;  // fp16 kernel: 32*MT x 32*NT channel tile
+    bool vec;    // fp32 kernel: windows staged as groups of 4 positions
     int SW, cpr, nchunks, ntiles;  // fp16 kernel: stride along W, 8-pixel chunks per output row / in total, pixel tiles
     size_t lds_bytes, partial_bytes;
 };
@@ -389,26 +390,31 @@ static bool plan_wgrad_f32(const Problem& p, WgPlan& best) {
     const int nkw = std::min(TPW, p.kw);
     double best_score = -1.0;
     const int budget = LDS_FLOATS_MAX / (4 * 64);  // KPp + HPp (+ offsets) per staged channel
-    for (int TW = 1; TW <= std::min(p.wo, 64); ++TW) {
-        for (int TH = 1; TH <= p.ho; ++TH) {
-            for (int NB = 1; NB <= p.n; ++NB) {
-                if (NB > 1 && !(TH == p.ho && TW == p.wo)) break;
-                const int pix = NB * TH * TW;
-                const int KP = (pix + 1) & ~1;
-                const int HTH = (TH - 1) * p.sh + 1;
-                const int HTW = (TW - 1) * p.sw + (nkw - 1) * p.dw + 1;
-                const int HPx = NB * HTH * HTW;
-                const int KPp = KP | 1, HPp = HPx | 1;  // odd pitches: bank-conflict-free 4-byte reads
-                if (pix > 32 || HPx > 32) break;
-                if (KPp + HPp + (KP + 255) / 256 > budget) break;
-                const int tn = cdiv(p.n, NB), th = cdiv(p.ho, TH), tw = cdiv(p.wo, TW);
-                const double eff = ((double)p.n * p.ho * p.wo) / ((double)tn * th * tw * KP);
-                const double score = eff * (1.0 + 0.002 * KP) * (TW >= std::min(p.wo, 8) ? 1.0 : 0.5);
-                if (score > best_score) {
-                    best_score = score;
-                    best.TPW = TPW; best.NB = NB; best.TH = TH; best.TW = TW; best.KP = KP; best.KPp = KPp;
-                    best.HPp = HPp; best.HPx = HPx; best.HTH = HTH; best.HTWmax = HTW;
-                    best.tiles_n = tn; best.tiles_h = th; best.tiles_w = tw;
+    for (int vec = 0; vec < 2; ++vec) {  // vec: windows staged as groups of 4 positions (16-byte loads)
+        for (int TW = vec ? 4 : 1; TW <= std::min(p.wo, 64); TW += vec ? 4 : 1) {
+            for (int TH = 1; TH <= p.ho; ++TH) {
+                for (int NB = 1; NB <= p.n; ++NB) {
+                    if (NB > 1 && !(TH == p.ho && TW == p.wo)) break;
+                    const int pix = NB * TH * TW;
+                    const int KP = (pix + 1) & ~1;
+                    const int HTH = (TH - 1) * p.sh + 1;
+                    int HTW = (TW - 1) * p.sw + (nkw - 1) * p.dw + 1;
+                    if (vec) HTW = (HTW + 3) & ~3;
+                    const int HPx = NB * HTH * HTW;
+                    const int KPp = KP | 1, HPp = HPx | 1;  // odd pitches: bank-conflict-free 4-byte reads
+                    if (pix > 32 || HPx > 32) break;
+                    if (KPp + HPp + (KP + 255) / 256 > budget) break;
+                    const int tn = cdiv(p.n, NB), th = cdiv(p.ho, TH), tw = cdiv(p.wo, TW);
+                    const double eff = ((double)p.n * p.ho * p.wo) / ((double)tn * th * tw * KP);
+                    const double score =
+                        eff * (1.0 + 0.002 * KP) * (TW >= std::min(p.wo, 8) ? 1.0 : 0.5) * (vec ? 1.25 : 1.0);
+                    if (score > best_score) {
+                        best_score = score;
+                        best.vec = vec != 0;
+                        best.TPW = TPW; best.NB = NB; best.TH = TH; best.TW = TW; best.KP = KP; best.KPp = KPp;
+                        best.HPp = HPp; best.HPx = HPx; best.HTH = HTH; best.HTWmax = HTW;
+                        best.tiles_n = tn; best.tiles_h = th; best.tiles_w = tw;
+                    }
                 }
             }
         }
@@ -488,7 +494,7 @@ static int run_wgrad(const Problem& p, hipStream_t st, const void* x, const void
             if (launch_wgrad_f16(p.mode, pl.MT, pl.NT, pl.TPW, pl.SW, a, nblocks, pl.lds_bytes, st) != 0)
                 return PHX_ERR_RUNTIME;
         } else {
-            launch_wgrad_f32(half_storage, p.mode, a, dim3(nblocks), pl.lds_bytes, st);
+            launch_wgrad_f32(half_storage, pl.vec, p.mode, a, dim3(nblocks), pl.lds_bytes, st);
         }
     }
     PHX_HIP(hipGetLastError());
@@ -504,7 +510,7 @@ static int run_wgrad(const Problem& p, hipStream_t st, const void* x, const void
         snprintf(g_name_buf, sizeof(g_name_buf), "qconv_wgrad_f16mfma_p%d_f16_ch%dx%d_taps%d_sw%d_z%d", p.mode, 32 * pl.MT,
                  32 * pl.NT, pl.TPW, pl.SW, pl.Z);
     else
-        snprintf(g_name_buf, sizeof(g_name_buf), "qconv_wgrad_f32mfma_p%d_%s_tile%dx%dx%d_z%d", p.mode,
+        snprintf(g_name_buf, sizeof(g_name_buf), "qconv_wgrad_f32mfma%s_p%d_%s_tile%dx%dx%d_z%d", pl.vec ? "v" : "", p.mode,
                  p.dtype == PHX_F32 ? "f32" : "f16", pl.NB, pl.TH, pl.TW, pl.Z);
     g_last_kernel = g_name_buf;
     return PHX_OK;
