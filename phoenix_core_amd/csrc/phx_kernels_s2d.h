@@ -1,0 +1,89 @@
+// Space-to-depth rewriting of stride-2 convolutions with very few input channels (network stems).
+//   y[ho][wo] = sum_{kh,kw} x[2ho + kh - pt][2wo + kw - pl] * w[kh][kw]
+// With kh - pt = 2a + b (b in {0,1}) and x'[(c,bh,bw)][i][j] = x[c][2i + bh][2j + bw] this is a
+// unit-stride convolution of x' (4x the channels, half the extent) with
+//   w'[(c,bh,bw)][ah - amin][aw - amin] = w[c][2ah + bh + pt][2aw + bw + pl]   (zero outside the filter).
+// A 7x7 stride-2 stem on 3 channels becomes a 4x4 unit-stride convolution on 12 channels, which the
+// tiled kernels run at their usual efficiency; the strided form would stage a 4x larger halo window
+// for every output tile and pad 3 channels to a 16-channel K step.
+// The three kernels here are the elementwise rearrangements: activations, filters, filter gradient.
+#pragma once
+
+#include "phx_device.h"
+
+namespace phx {
+
+struct S2dArgs {
+    const void* src;
+    void* dst;
+    long planes;        // 4N * C image planes
+    int H, W, H2, W2;   // source extent, destination extent (ceil(H/2), ceil(W/2))
+};
+
+// one thread per (plane, destination row, 4 destination columns): reads 2 rows x 8 source columns
+template <typename TS>
+__global__ void __launch_bounds__(WG_THREADS) s2d_input_kernel(const S2dArgs A) {
+    const int wq = (A.W2 + 3) / 4;
+    const long total = A.planes * A.H2 * wq;
+    const TS* src = static_cast<const TS*>(A.src);
+    TS* dst = static_cast<TS*>(A.dst);
+    const long dplane = (long)A.H2 * A.W2;
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
+        const int jq = idx % wq;
+        const long rest = idx / wq;
+        const int i = rest % A.H2;
+        const long plane = rest / A.H2;
+        const int j0 = jq * 4;
+#pragma unroll
+        for (int bh = 0; bh < 2; ++bh) {
+            const int h = 2 * i + bh;
+            TS v[8];
+            const TS* row = src + (plane * A.H + h) * A.W + 2 * j0;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) v[k] = (h < A.H && 2 * j0 + k < A.W) ? row[k] : (TS)0;
+#pragma unroll
+            for (int bw = 0; bw < 2; ++bw) {
+                TS* out = dst + (plane * 4 + bh * 2 + bw) * dplane + (long)i * A.W2 + j0;
+#pragma unroll
+                for (int k = 0; k < 4; ++k)
+                    if (j0 + k < A.W2) out[k] = v[2 * k + bw];
+            }
+        }
+    }
+}
+
+struct S2dFilterArgs {
+    const void* w;      // caller's filters, element (r, o, i, kh, kw) at r*wcs + o*so + i*si + kh*skh + kw*skw
+    void* w2;           // rearranged filters [4][Co][4*Ci][K2h][K2w] (OIHW)
+    long wcs, so, si, skh, skw;
+    int Co, Ci, Kh, Kw, K2h, K2w;
+    int pt, pl, aminh, aminw;
+};
+
+// to_caller == false: w -> w2;  to_caller == true: dw2 -> dw (every caller element has exactly one image)
+template <typename TS>
+__global__ void __launch_bounds__(WG_THREADS) s2d_filter_kernel(const S2dFilterArgs A, bool to_caller) {
+    const TS* src = static_cast<const TS*>(to_caller ? A.w2 : A.w);
+    TS* dst = static_cast<TS*>(to_caller ? const_cast<void*>(A.w) : A.w2);
+    const int C2 = 4 * A.Ci;
+    const long total = 4L * A.Co * C2 * A.K2h * A.K2w;
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
+        long s = idx;
+        const int aw = s % A.K2w; s /= A.K2w;
+        const int ah = s % A.K2h; s /= A.K2h;
+        const int c2 = s % C2; s /= C2;
+        const int o = s % A.Co;
+        const int r = s / A.Co;
+        const int c = c2 >> 2, bh = (c2 >> 1) & 1, bw = c2 & 1;
+        const int kh = 2 * (ah + A.aminh) + bh + A.pt, kw = 2 * (aw + A.aminw) + bw + A.pl;
+        const bool inside = kh >= 0 && kh < A.Kh && kw >= 0 && kw < A.Kw;
+        const long off = r * A.wcs + o * A.so + c * A.si + kh * A.skh + kw * A.skw;
+        if (to_caller) {
+            if (inside) dst[off] = src[idx];
+        } else {
+            dst[idx] = inside ? src[off] : (TS)0;
+        }
+    }
+}
+
+}  // namespace phx

@@ -14,7 +14,8 @@
 namespace phx {
 
 static thread_local const char* g_last_kernel = "";
-static thread_local char g_name_buf[128];
+static thread_local char g_name_buf[160];
+static thread_local const char* g_name_prefix = "";  // "s2d_" while a rewritten problem runs
 
 // optional event pairs around the dominant kernel of each call (see phx_profile_enable)
 struct ProfileState {
@@ -353,7 +354,7 @@ static int run_corr(const Problem& p, const Corr& creal, int map, hipStream_t st
     }
     if (rc != 0) return PHX_ERR_NOT_SUPPORTED;
     PHX_HIP(hipGetLastError());
-    snprintf(g_name_buf, sizeof(g_name_buf), "qconv_%s_%smfma%s_p%d_%s_wco%d_ntw%d_ck%d_tile%dx%dx%d",
+    snprintf(g_name_buf, sizeof(g_name_buf), "%sqconv_%s_%smfma%s_p%d_%s_wco%d_ntw%d_ck%d_tile%dx%dx%d", g_name_prefix,
              map == MAP_FWD ? "fwd" : "dgrad", f16 ? "f16" : "f32", pl.lds_filters ? (pw ? "ldspw" : pl.chunks ? "ldsc" : "lds") : "", p.mode, p.dtype == PHX_F32 ? "f32" : "f16", pl.WCO,
              pl.NTW, pl.CK, pl.NB, pl.TH, pl.TW);
     g_last_kernel = g_name_buf;
@@ -507,16 +508,16 @@ static int run_wgrad(const Problem& p, hipStream_t st, const void* x, const void
     launch_reduce_wgrad(half_storage, r, blocks, st);
     PHX_HIP(hipGetLastError());
     if (f16)
-        snprintf(g_name_buf, sizeof(g_name_buf), "qconv_wgrad_f16mfma_p%d_f16_ch%dx%d_taps%d_sw%d_z%d", p.mode, 32 * pl.MT,
+        snprintf(g_name_buf, sizeof(g_name_buf), "%sqconv_wgrad_f16mfma_p%d_f16_ch%dx%d_taps%d_sw%d_z%d", g_name_prefix, p.mode, 32 * pl.MT,
                  32 * pl.NT, pl.TPW, pl.SW, pl.Z);
     else
-        snprintf(g_name_buf, sizeof(g_name_buf), "qconv_wgrad_f32mfma%s_p%d_%s_tile%dx%dx%d_z%d", pl.vec ? "v" : "", p.mode,
+        snprintf(g_name_buf, sizeof(g_name_buf), "%sqconv_wgrad_f32mfma%s_p%d_%s_tile%dx%dx%d_z%d", g_name_prefix, pl.vec ? "v" : "", p.mode,
                  p.dtype == PHX_F32 ? "f32" : "f16", pl.NB, pl.TH, pl.TW, pl.Z);
     g_last_kernel = g_name_buf;
     return PHX_OK;
 }
 
-static size_t workspace_for(const Problem& p, int pass) {
+static size_t workspace_plain(const Problem& p, int pass) {
     if (is_empty(p)) return 0;
     if (pass == PHX_PASS_BWD_WEIGHTS) {
         WgPlan pl;
@@ -530,12 +531,80 @@ static size_t workspace_for(const Problem& p, int pass) {
                : 0;
 }
 
+// Space-to-depth view of a stride-2 convolution with at most 4 input channels (see phx_kernels_s2d.h):
+// the unit-stride problem q on rearranged activations / filters, and the workspace the rearranged copies take.
+struct S2dView {
+    Problem q;
+    S2dFilterArgs fa;
+    size_t x2_bytes, w2_bytes;
+};
+
+static int floordiv(int a, int b) { return a >= 0 ? a / b : -((-a + b - 1) / b); }
+
+static bool s2d_view(const Problem& p, S2dView& v) {
+    if (p.sh != 2 || p.sw != 2 || p.dh != 1 || p.dw != 1 || p.ci > 4 || (p.kh < 3 && p.kw < 3) || is_empty(p)) return false;
+    if (getenv("PHX_TUNE_NOS2D")) return false;
+    const int aminh = floordiv(-p.pt, 2), amaxh = floordiv(p.kh - 1 - p.pt, 2);
+    const int aminw = floordiv(-p.pl, 2), amaxw = floordiv(p.kw - 1 - p.pl, 2);
+    Problem& q = v.q;
+    q = p;
+    q.ci = 4 * p.ci;
+    q.h = (p.h + 1) / 2; q.w = (p.w + 1) / 2;
+    q.kh = amaxh - aminh + 1; q.kw = amaxw - aminw + 1;
+    q.sh = q.sw = 1;
+    q.pt = -aminh; q.pl = -aminw;
+    q.pb = p.ho - q.h - q.pt + q.kh - 1;
+    q.pr = p.wo - q.w - q.pl + q.kw - 1;
+    if (q.pb < 0 || q.pr < 0) return false;
+    q.ho = out_size(q.h, q.kh, 1, 1, q.pt, q.pb);
+    q.wo = out_size(q.w, q.kw, 1, 1, q.pl, q.pr);
+    if (q.ho != p.ho || q.wo != p.wo) return false;
+    const long taps2 = (long)q.kh * q.kw;
+    q.fs.wcs = (long)q.co * q.ci * taps2; q.fs.so = q.ci * taps2; q.fs.si = taps2; q.fs.skh = q.kw; q.fs.skw = 1;
+    const size_t esize = p.dtype == PHX_F32 ? 4 : 2;
+    v.x2_bytes = align_up((size_t)4 * p.n * q.ci * q.h * q.w * esize, 256);
+    v.w2_bytes = align_up((size_t)4 * q.fs.wcs * esize, 256);
+    S2dFilterArgs& f = v.fa;
+    f.wcs = p.fs.wcs; f.so = p.fs.so; f.si = p.fs.si; f.skh = p.fs.skh; f.skw = p.fs.skw;
+    f.Co = p.co; f.Ci = p.ci; f.Kh = p.kh; f.Kw = p.kw; f.K2h = q.kh; f.K2w = q.kw;
+    f.pt = p.pt; f.pl = p.pl; f.aminh = aminh; f.aminw = aminw;
+    return true;
+}
+
+static size_t workspace_for(const Problem& p, int pass) {
+    S2dView v;
+    if (pass != PHX_PASS_BWD_DATA && s2d_view(p, v)) return v.x2_bytes + v.w2_bytes + workspace_plain(v.q, pass);
+    return workspace_plain(p, pass);
+}
+
+static void s2d_rearrange_input(const Problem& p, const S2dView& v, const void* x, void* x2, hipStream_t st) {
+    S2dArgs a;
+    a.src = x; a.dst = x2; a.planes = 4L * p.n * p.ci; a.H = p.h; a.W = p.w; a.H2 = v.q.h; a.W2 = v.q.w;
+    launch_s2d_input(p.dtype == PHX_F16, a, st);
+}
+
 static int do_fwd(const Problem& p, hipStream_t st, const void* x, const void* w, const void* bias, void* y, void* ws,
                   size_t wsb) {
     if (is_empty(p)) return PHX_OK;  // the reference returns silently on empty input (src/conv2d.hpp:81-82)
     if (!x || !w || !y || (p.has_bias && !bias)) return PHX_ERR_INVALID_ARGUMENT;
-    const Corr c = corr_forward(p);
     const void* b = p.has_bias ? bias : nullptr;
+    S2dView v;
+    if (s2d_view(p, v)) {
+        if (wsb < v.x2_bytes + v.w2_bytes || !ws) return PHX_ERR_WORKSPACE;
+        char* x2 = static_cast<char*>(ws);
+        char* w2 = x2 + v.x2_bytes;
+        s2d_rearrange_input(p, v, x, x2, st);
+        S2dFilterArgs fa = v.fa;
+        fa.w = w; fa.w2 = w2;
+        launch_s2d_filter(p.dtype == PHX_F16, fa, false, st);
+        PHX_HIP(hipGetLastError());
+        g_name_prefix = "s2d_";
+        const int rc = run_corr(v.q, corr_forward(v.q), MAP_FWD, st, x2, w2, b, y, w2 + v.w2_bytes,
+                                wsb - v.x2_bytes - v.w2_bytes);
+        g_name_prefix = "";
+        return rc;
+    }
+    const Corr c = corr_forward(p);
     return run_corr(p, c, MAP_FWD, st, x, w, b, y, ws, wsb);
 }
 
@@ -555,6 +624,22 @@ static int do_bwd_weights(const Problem& p, hipStream_t st, const void* x, const
         return PHX_OK;
     }
     if (!x || !g) return PHX_ERR_INVALID_ARGUMENT;
+    S2dView v;
+    if (s2d_view(p, v)) {
+        if (wsb < v.x2_bytes + v.w2_bytes || !ws) return PHX_ERR_WORKSPACE;
+        char* x2 = static_cast<char*>(ws);
+        char* dw2 = x2 + v.x2_bytes;
+        s2d_rearrange_input(p, v, x, x2, st);
+        g_name_prefix = "s2d_";
+        const int rc = run_wgrad(v.q, st, x2, g, dw2, dw2 + v.w2_bytes, wsb - v.x2_bytes - v.w2_bytes);
+        g_name_prefix = "";
+        if (rc != PHX_OK) return rc;
+        S2dFilterArgs fa = v.fa;
+        fa.w = dw; fa.w2 = dw2;
+        launch_s2d_filter(p.dtype == PHX_F16, fa, true, st);
+        PHX_HIP(hipGetLastError());
+        return PHX_OK;
+    }
     const Problem f = flatten_pointwise(p);
     return run_wgrad(f, st, x, g, dw, ws, wsb);
 }
