@@ -620,7 +620,8 @@ static int do_bwd_weights(const Problem& p, hipStream_t st, const void* x, const
     if (!dw) return PHX_ERR_INVALID_ARGUMENT;
     if (is_empty(p)) {  // the reference zeroes the filter gradient on empty input (src/conv2d.hpp:341-344)
         const size_t bytes = (size_t)4 * p.fs.wcs * (p.dtype == PHX_F32 ? 4 : 2);
-        PHX_HIP(hipMemsetAsync(dw, 0, bytes, st));
+        launch_fill_zero(dw, bytes, st);
+        PHX_HIP(hipGetLastError());
         return PHX_OK;
     }
     if (!x || !g) return PHX_ERR_INVALID_ARGUMENT;
@@ -795,7 +796,8 @@ int phx_memcpy_d2h(void* dst, const void* src, size_t bytes, phx_stream_t stream
 
 int phx_memset_zero(void* dst, size_t bytes, phx_stream_t stream) {
     if (bytes == 0) return PHX_OK;
-    PHX_HIP(hipMemsetAsync(dst, 0, bytes, static_cast<hipStream_t>(stream)));
+    launch_fill_zero(dst, bytes, static_cast<hipStream_t>(stream));
+    PHX_HIP(hipGetLastError());
     return PHX_OK;
 }
 
