@@ -141,11 +141,10 @@ def bench_resnet(args):
     model = phx.QResNet50(1000, dtype=torch.float16, context=ctx).to(dev).train()
     images = torch.randn(n, 3, 224, 224, device=dev).half()
     labels = torch.randint(0, 1000, (n,), device=dev)
-    xq = phx.QResNet50.lift(images)
 
     def step():
         model.zero_grad(set_to_none=True)
-        loss = torch.nn.functional.cross_entropy(model(xq).float(), labels)
+        loss = torch.nn.functional.cross_entropy(model(images).float(), labels)
         loss.backward()
         return loss
 
@@ -170,7 +169,8 @@ def bench_resnet(args):
         "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f16", "data": "synthetic",
         "config": {"workload": "%s: quaternion ResNet-50 forward+backward (no optimizer step, as the metric names), "
-                               "N=%d (4N=%d rows), 224x224, 53 quaternion convs + quaternion dense head; batch-norm, "
+                               "N=%d real images (4N=%d quaternion rows after the real-input stem), 224x224, 53 quaternion convs + "
+                               "quaternion dense head; batch-norm, "
                                "ReLU, pooling and cross-entropy by PyTorch" % (RESNET, n, 4 * n),
                    "product_mode": mode, "fp16_policy": policy},
         "real_equiv_tflops": 3 * fwd_flops / (ms_per_step * 1e-3) / 1e12,

@@ -68,6 +68,11 @@ typedef struct phx_qconv_desc {
     int32_t product_mode;  /* phx_product_mode */
     int32_t fp16_policy;   /* phx_fp16_policy */
     int32_t has_bias;      /* forward only: bias pointer must be non-null when set */
+    int32_t real_input;    /* real-valued input (realValuedInput, src/backend/conv2d_descriptor.hpp:262-278,
+                              src/conv2d.hpp:122-164, 384-430): 0 or 1; when set x is [n, ci, h, w] with no
+                              imaginary parts, filters, outputs and output gradients stay quaternion-valued, has_bias
+                              must be 0 (src/conv2d.hpp:125-127) and
+                              phx_qconv2d_bwd_data is refused as the reference refuses it (src/conv2d.hpp:394-398) */
 } phx_qconv_desc;
 
 /* Quaternion Dense geometry (src/backend/dense_descriptor.hpp:11-59); filter layout is IO. */

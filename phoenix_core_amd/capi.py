@@ -9,6 +9,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libphx_qconv.so")
 
 PHX_OK = 0
+PHX_ERR_INVALID_ARGUMENT, PHX_ERR_NOT_SUPPORTED, PHX_ERR_WORKSPACE, PHX_ERR_RUNTIME = 1, 2, 3, 4
 PHX_F32, PHX_F16 = 0, 1
 PHX_OIHW, PHX_OHWI = 0, 1
 PHX_PRODUCT_16, PHX_PRODUCT_8 = 16, 8
@@ -29,7 +30,8 @@ EXPORTS = (
 class QConvDesc(ctypes.Structure):
     _fields_ = [(k, ctypes.c_int32) for k in (
         "dtype", "n", "ci", "co", "h", "w", "kh", "kw", "stride_h", "stride_w", "dilation_h", "dilation_w",
-        "pad_top", "pad_left", "pad_bottom", "pad_right", "filter_layout", "product_mode", "fp16_policy", "has_bias")]
+        "pad_top", "pad_left", "pad_bottom", "pad_right", "filter_layout", "product_mode", "fp16_policy", "has_bias",
+        "real_input")]
 
 
 class QDenseDesc(ctypes.Structure):

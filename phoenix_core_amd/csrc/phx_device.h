@@ -197,6 +197,7 @@ struct TileSrc {
     long comp_stride;  // elements between components
     int N, C, Hd, Wd;  // stored dims per component
     int uh, uw;        // zero-insertion factors (1 = none)
+    int ncomp;         // components present in memory: 4, or 1 for a real-valued tensor (components 1..3 read as zero)
     int pw;            // pointwise trick: window row r holds channels (chunk*pw + r)*16.. of the single image row (0 = off)
 };
 
@@ -244,7 +245,7 @@ __device__ __forceinline__ void stage_load(float (&v)[(4 * NCH) >> (8 - P2LOG)],
     for (int e = 0; e < E; ++e) {
         const int pc = e * G + sp.group;
         const int p = pc / NCH, c = pc % NCH;
-        const bool ok = sp.valid && (c0 + c) < s.C;
+        const bool ok = sp.valid && (c0 + c) < s.C && p < s.ncomp;
         const TS* ptr = ok ? origin + sp.goff + p * s.comp_stride + (long)(c0 + c) * plane : zero_ptr<TS>();
         v[e] = ldf<TS>(ptr);
     }

@@ -25,7 +25,7 @@ __device__ __forceinline__ void stage_load16(f16x8 (&v)[8 >> (8 - P2LOG)], const
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             const int c = c0 + kp * 8 + i;
-            const bool ok = sp.valid && c < s.C;
+            const bool ok = sp.valid && c < s.C && p < s.ncomp;
             const _Float16* ptr = ok ? origin + sp.goff + p * s.comp_stride + (long)c * plane : zero_ptr<_Float16>();
             v[e][i] = *ptr;
         }
@@ -85,7 +85,7 @@ __device__ __forceinline__ void stage_load16_pairs(unsigned int (&d)[4][8], cons
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             const int c = c0 + kp * 8 + i;
-            const bool ok = sp.valid && c < s.C;
+            const bool ok = sp.valid && c < s.C && p < s.ncomp;
             const _Float16* ptr = ok ? origin + sp.goff + p * s.comp_stride + (long)c * plane : zero_ptr<_Float16>();
             d[e][i] = *reinterpret_cast<const unsigned int*>(ptr);
         }
@@ -334,12 +334,12 @@ __device__ __forceinline__ StageChunk make_stage_chunk(const TileSrc& s, int n0,
     const int vh = s.pw ? 0 : h0 + hr, vw0 = w0 + cc * 8;
     const int p = u >> 1;
     sc.kp = u & 1;
-    sc.live = sc.task && nb < NB && (n0 + nb) < s.N && vh >= 0 && vh < s.Hd;
+    sc.live = sc.task && p < s.ncomp && nb < NB && (n0 + nb) < s.N && vh >= 0 && vh < s.Hd;
     sc.bits = sc.live ? interval_bits(-vw0, s.Wd - vw0) : 0u;
     const _Float16* base = static_cast<const _Float16*>(s.base);
     const long plane = (long)s.Hd * s.Wd;
     sc.ptr = base + p * s.comp_stride + ((long)(n0 + nb) * s.C * s.Hd + vh) * s.Wd + vw0;
-    const _Float16* end = base + 3 * s.comp_stride + (long)s.N * s.C * plane;
+    const _Float16* end = base + (long)(s.ncomp - 1) * s.comp_stride + (long)s.N * s.C * plane;
     sc.careful = sc.live && (sc.ptr < base || sc.ptr + (long)(s.C - 1) * plane + 8 > end);
     const int e0 = row * HTW + cc * 8;
     sc.ent = (sc.task ? u : 0) * HPp + e0;
@@ -801,6 +801,7 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_wgrad_f16_kernel(const Wgrad
     // 32-bit element offsets inside one component: the host guarantees they fit
     const int gimg = P.g.C * (int)gplane, ximg = P.x.C * (int)xplane;
     const int gcomp = P.g.N * gimg, xcomp = P.x.N * ximg;  // elements per component
+    const int xnc = P.x.ncomp;                              // 1 for a real-valued input: components 1..3 are zero
     int gch[MT], xch[NT];
 #pragma unroll
     for (int i = 0; i < MT; ++i) gch[i] = (co_first + 32 * i < P.g.C ? co_first + 32 * i : P.g.C - 1) * (int)gplane;
@@ -845,7 +846,7 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_wgrad_f16_kernel(const Wgrad
             sg[sl] = load16_a2(gbase + (sl / MT) * P.g.comp_stride + lgoff[sl % MT]);
         } else if (sl < NLOADS) {
             const int e = (sl - GE) / XL, part = (sl - GE) % XL;
-            const _Float16* ptr = xbase + (e / NT) * P.x.comp_stride + lxoff[e % NT];
+            const _Float16* ptr = xbase + ((e / NT) < xnc ? (e / NT) * P.x.comp_stride + lxoff[e % NT] : 0);
             if (part == 0) {
                 const u32x4 a = load16_a2(ptr);
                 sx[e][0] = a[0]; sx[e][1] = a[1]; sx[e][2] = a[2]; sx[e][3] = a[3];
@@ -885,7 +886,7 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_wgrad_f16_kernel(const Wgrad
 #pragma unroll
             for (int k = 0; k < NEL; ++k) {
                 const int col = wi0 + k;
-                w[k] = (rowok && col >= 0 && col < W) ? src[col] : (_Float16)0;
+                w[k] = (rowok && q < xnc && col >= 0 && col < W) ? src[col] : (_Float16)0;
             }
 #pragma unroll
             for (int t = 0; t < TPW; ++t)
@@ -915,7 +916,7 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_wgrad_f16_kernel(const Wgrad
                 const int q = e / NT, cc = (e % NT) * 32;
                 unsigned int w[XR];
 #pragma unroll
-                for (int d = 0; d < XR; ++d) w[d] = sx[e][d] & mx[d];
+                for (int d = 0; d < XR; ++d) w[d] = q < xnc ? (sx[e][d] & mx[d]) : 0u;
 #pragma unroll
                 for (int t = 0; t < TPW; ++t) {
                     u32x4 v;

@@ -143,7 +143,8 @@ __device__ __forceinline__ void conv_epilogue(const ConvArgs& P, const f32x16 (&
                     const int co = co_base + 8 * rq + k;
                     if (co < P.Cout) {
 #pragma unroll
-                        for (int q = 0; q < 4; ++q) stf<TS>(out + q * P.out_cs + oaddr[t] + co * plane, y[k][q]);
+                        for (int q = 0; q < 4; ++q)
+                            stf<TS>(out + q * P.out_cs + oaddr[t] + co * plane, y[k][q]);
                     }
                 }
             }
@@ -184,8 +185,9 @@ __device__ __forceinline__ StageVec make_stage_vec(const TileSrc& s, int n0, int
     sv.bits = sv.live ? interval_bits<4>(-vw0, s.Wd - vw0) : 0u;
     sv.goff = ((long)(n0 + nb) * s.C * s.Hd + vh) * s.Wd + vw0;
     const long plane = (long)s.Hd * s.Wd;
-    const long total = 3 * s.comp_stride + (long)s.N * s.C * plane;
-    sv.careful = sv.live && (sv.goff < 0 || sv.goff + 3 * s.comp_stride + (long)(s.C - 1) * plane + 4 > total);
+    const long last = (long)(s.ncomp - 1) * s.comp_stride;  // offset of the last component in memory
+    const long total = last + (long)s.N * s.C * plane;
+    sv.careful = sv.live && (sv.goff < 0 || sv.goff + last + (long)(s.C - 1) * plane + 4 > total);
     return sv;
 }
 
@@ -199,7 +201,9 @@ __device__ __forceinline__ void stage_vec_load(f32x4 (&v)[(NCH << P2LOG) >> 8], 
     const int pc = e * G4 + sv.group;
     const int p = pc / NCH, c = c0 + pc % NCH;
     // channels past the tensor meet zero filters: any finite value will do, the tensor's first bytes are safe
-    const TS* ptr = (sv.live && !sv.careful && c < s.C) ? origin + sv.goff + p * s.comp_stride + c * plane : origin;
+    // (components a real-valued tensor does not have are masked to zero by the store)
+    const TS* ptr =
+        (sv.live && !sv.careful && c < s.C && p < s.ncomp) ? origin + sv.goff + p * s.comp_stride + c * plane : origin;
     if constexpr (sizeof(TS) == 4) {
         typedef f32x4 f32x4_a4 __attribute__((aligned(4)));
         v[e] = *reinterpret_cast<const f32x4_a4*>(ptr);
@@ -222,7 +226,8 @@ __device__ __forceinline__ void stage_vec_store(float* lds, const f32x4 (&v)[(NC
     for (int i = 0; i < 4; ++i) mk[i] = (unsigned int)((int)(keep << (31 - i)) >> 31);
 #pragma unroll
     for (int e = 0; e < E; ++e) {
-        const u32x4 w = __builtin_bit_cast(u32x4, v[e]) & mk;
+        const bool present = (e * G4 + sv.group) / NCH < s.ncomp;
+        const u32x4 w = present ? (__builtin_bit_cast(u32x4, v[e]) & mk) : u32x4{0u, 0u, 0u, 0u};
         *reinterpret_cast<u32x4*>(lds + (e * G4 + sv.group) * HPp + sv.lpos) = w;
     }
     if (sv.careful) {
@@ -235,7 +240,9 @@ __device__ __forceinline__ void stage_vec_store(float* lds, const f32x4 (&v)[(NC
             float t[4];
 #pragma unroll
             for (int i = 0; i < 4; ++i)
-                t[i] = (c < s.C && ((sv.bits >> i) & 1)) ? ldf<TS>(origin + sv.goff + p * s.comp_stride + c * plane + i) : 0.f;
+                t[i] = (c < s.C && p < s.ncomp && ((sv.bits >> i) & 1))
+                           ? ldf<TS>(origin + sv.goff + p * s.comp_stride + c * plane + i)
+                           : 0.f;
 #pragma unroll
             for (int i = 0; i < 4; ++i) lds[pc * HPp + sv.lpos + i] = t[i];
         }
@@ -253,8 +260,9 @@ __device__ __forceinline__ void stage_vec_store_scalar(float* lds, const f32x4 (
 #pragma unroll
     for (int e = 0; e < E; ++e) {
         float* dst = lds + (e * G4 + sv.group) * pitch + sv.lpos;
+        const bool present = (e * G4 + sv.group) / NCH < s.ncomp;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) dst[i] = ((keep >> i) & 1) ? v[e][i] : 0.f;
+        for (int i = 0; i < 4; ++i) dst[i] = (present && ((keep >> i) & 1)) ? v[e][i] : 0.f;
     }
     if (sv.careful) {
         const TS* origin = static_cast<const TS*>(s.base);
@@ -266,7 +274,9 @@ __device__ __forceinline__ void stage_vec_store_scalar(float* lds, const f32x4 (
             float t[4];
 #pragma unroll
             for (int i = 0; i < 4; ++i)
-                t[i] = (c < s.C && ((sv.bits >> i) & 1)) ? ldf<TS>(origin + sv.goff + p * s.comp_stride + c * plane + i) : 0.f;
+                t[i] = (c < s.C && p < s.ncomp && ((sv.bits >> i) & 1))
+                           ? ldf<TS>(origin + sv.goff + p * s.comp_stride + c * plane + i)
+                           : 0.f;
 #pragma unroll
             for (int i = 0; i < 4; ++i) lds[pc * pitch + sv.lpos + i] = t[i];
         }

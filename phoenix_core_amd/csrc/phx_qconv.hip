@@ -62,6 +62,7 @@ struct Problem {
     int n, ci, co, h, w, kh, kw, sh, sw, dh, dw, pt, pl, pb, pr, ho, wo;
     FilterStrides fs;
     bool has_bias;
+    bool real_input;  // x (and dx) are real-valued [n, ci, h, w]: imaginary components are zero and not stored
 };
 
 static int out_size(int in, int k, int d, int s, int before, int after) {
@@ -80,6 +81,9 @@ static int problem_from_conv(const phx_qconv_desc* d, Problem& p) {
     if (d->stride_h <= 0 || d->stride_w <= 0 || d->dilation_h <= 0 || d->dilation_w <= 0)
         return PHX_ERR_INVALID_ARGUMENT;
     if (d->pad_top < 0 || d->pad_left < 0 || d->pad_bottom < 0 || d->pad_right < 0) return PHX_ERR_INVALID_ARGUMENT;
+    if (d->real_input != 0 && d->real_input != 1) return PHX_ERR_INVALID_ARGUMENT;
+    // "Bias addition is not supported for type0 inputs" (src/conv2d.hpp:125-127)
+    if (d->real_input && d->has_bias) return PHX_ERR_INVALID_ARGUMENT;
     p.dtype = d->dtype;
     p.mode = d->product_mode;
     p.policy = d->fp16_policy;
@@ -97,6 +101,7 @@ static int problem_from_conv(const phx_qconv_desc* d, Problem& p) {
         p.fs.so = taps * p.ci; p.fs.si = 1; p.fs.skh = (long)p.kw * p.ci; p.fs.skw = p.ci;
     }
     p.has_bias = d->has_bias != 0;
+    p.real_input = d->real_input != 0;
     return PHX_OK;
 }
 
@@ -112,6 +117,7 @@ static int problem_from_dense(const phx_qdense_desc* d, Problem& p) {
     // layout IO: w[r][i][o]
     p.fs.wcs = (long)p.ci * p.co; p.fs.so = 1; p.fs.si = p.co; p.fs.skh = 0; p.fs.skw = 0;
     p.has_bias = d->has_bias != 0;
+    p.real_input = false;
     return PHX_OK;
 }
 
@@ -335,6 +341,8 @@ static int run_corr(const Problem& p, const Corr& creal, int map, hipStream_t st
     ConvArgs a;
     a.in.base = in; a.in.comp_stride = (long)c.N * creal.Cin * c.Hin * c.Win;
     a.in.N = c.N; a.in.C = creal.Cin; a.in.Hd = c.Hin; a.in.Wd = c.Win; a.in.uh = c.uh; a.in.uw = c.uw; a.in.pw = pw;
+    // real-valued input: the forward pass reads one component, the others are zero
+    a.in.ncomp = (p.real_input && map == MAP_FWD) ? 1 : 4;
     a.wpk = ws; a.bias = bias; a.out = out;
     a.out_cs = (long)c.N * c.Cout * c.Hout * c.Wout;
     a.Cout = c.Cout; a.Hout = c.Hout; a.Wout = c.Wout;
@@ -476,9 +484,9 @@ static int run_wgrad(const Problem& p, hipStream_t st, const void* x, const void
     if (ws_bytes < pl.partial_bytes || !ws) return PHX_ERR_WORKSPACE;
     WgradArgs a;
     a.x.base = x; a.x.comp_stride = (long)p.n * p.ci * p.h * p.w; a.x.N = p.n; a.x.C = p.ci; a.x.Hd = p.h; a.x.Wd = p.w;
-    a.x.uh = a.x.uw = 1; a.x.pw = 0;
+    a.x.uh = a.x.uw = 1; a.x.pw = 0; a.x.ncomp = p.real_input ? 1 : 4;
     a.g.base = g; a.g.comp_stride = (long)p.n * p.co * p.ho * p.wo; a.g.N = p.n; a.g.C = p.co; a.g.Hd = p.ho; a.g.Wd = p.wo;
-    a.g.uh = a.g.uw = 1; a.g.pw = 0;
+    a.g.uh = a.g.uw = 1; a.g.pw = 0; a.g.ncomp = 4;
     a.partial = static_cast<float*>(ws);
     a.Kh = p.kh; a.Kw = p.kw; a.sh = p.sh; a.sw = p.sw; a.dh = p.dh; a.dw = p.dw; a.pt = p.pt; a.pl = p.pl;
     a.NB = pl.NB; a.TH = pl.TH; a.TW = pl.TW; a.KP = pl.KP; a.KPp = pl.KPp; a.HPp = pl.HPp; a.HTH = pl.HTH;
@@ -562,7 +570,7 @@ static bool s2d_view(const Problem& p, S2dView& v) {
     const long taps2 = (long)q.kh * q.kw;
     q.fs.wcs = (long)q.co * q.ci * taps2; q.fs.so = q.ci * taps2; q.fs.si = taps2; q.fs.skh = q.kw; q.fs.skw = 1;
     const size_t esize = p.dtype == PHX_F32 ? 4 : 2;
-    v.x2_bytes = align_up((size_t)4 * p.n * q.ci * q.h * q.w * esize, 256);
+    v.x2_bytes = align_up((size_t)(p.real_input ? 1 : 4) * p.n * q.ci * q.h * q.w * esize, 256);
     v.w2_bytes = align_up((size_t)4 * q.fs.wcs * esize, 256);
     S2dFilterArgs& f = v.fa;
     f.wcs = p.fs.wcs; f.so = p.fs.so; f.si = p.fs.si; f.skh = p.fs.skh; f.skw = p.fs.skw;
@@ -579,7 +587,7 @@ static size_t workspace_for(const Problem& p, int pass) {
 
 static void s2d_rearrange_input(const Problem& p, const S2dView& v, const void* x, void* x2, hipStream_t st) {
     S2dArgs a;
-    a.src = x; a.dst = x2; a.planes = 4L * p.n * p.ci; a.H = p.h; a.W = p.w; a.H2 = v.q.h; a.W2 = v.q.w;
+    a.src = x; a.dst = x2; a.planes = (p.real_input ? 1L : 4L) * p.n * p.ci; a.H = p.h; a.W = p.w; a.H2 = v.q.h; a.W2 = v.q.w;
     launch_s2d_input(p.dtype == PHX_F16, a, st);
 }
 
@@ -725,6 +733,9 @@ int phx_qconv2d_bwd_data(const phx_qconv_desc* desc, phx_stream_t stream, const 
     Problem p;
     const int rc = problem_from_conv(desc, p);
     if (rc != PHX_OK) return rc;
+    // the gradient with respect to a real-valued input has imaginary parts that are stored nowhere;
+    // the reference refuses the request likewise (src/conv2d.hpp:394-398)
+    if (p.real_input) return PHX_ERR_INVALID_ARGUMENT;
     return do_bwd_data(p, static_cast<hipStream_t>(stream), grad, w, dx, workspace, workspace_bytes);
 }
 

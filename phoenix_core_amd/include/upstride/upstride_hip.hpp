@@ -711,7 +711,6 @@ namespace detail {
 inline phx_qconv_desc makeConvDesc(const Conv2DDescriptor& d, Context& ctx, int dtype, bool useBias) {
     if (d.getAlgebra() != Algebra::QUATERNION)
         throw std::runtime_error("Only the quaternion algebra is built for device::HIP");
-    if (d.isRealValuedInput()) throw std::runtime_error("Real-valued input is not built for device::HIP");
     if (d.getDataFormat() != DataFormat::NCHW) throw std::runtime_error("device::HIP runs NCHW tensors only");
     if (d.getGroups() != 1) throw std::runtime_error("Grouped quaternion convolution is not built for device::HIP");
     const FilterLayout fl = d.getFilterLayout();
@@ -722,7 +721,8 @@ inline phx_qconv_desc makeConvDesc(const Conv2DDescriptor& d, Context& ctx, int 
     const Shape& w = d.getFilterShape();
     phx_qconv_desc c;
     c.dtype = dtype;
-    c.n = in[0] / 4;
+    const bool real = d.isRealValuedInput();  // [n, ci, h, w] without imaginary components
+    c.n = real ? in[0] : in[0] / 4;
     c.ci = filter.numInputChannels(w);
     c.co = filter.numOutputChannels(w);
     c.h = in[2];
@@ -736,8 +736,9 @@ inline phx_qconv_desc makeConvDesc(const Conv2DDescriptor& d, Context& ctx, int 
     c.filter_layout = fl == FilterLayout::OIHW ? PHX_OIHW : PHX_OHWI;
     c.product_mode = ctx.phxProductMode();
     c.fp16_policy = ctx.phxFp16Policy();
-    c.has_bias = useBias ? 1 : 0;
-    if (in[0] % 4 != 0) throw std::invalid_argument("Cannot split " + std::to_string(in[0]) + " onto 4 parts");
+    c.has_bias = (useBias && !real) ? 1 : 0;  // a bias given with a real-valued input is refused at call time
+    c.real_input = real ? 1 : 0;
+    if (!real && in[0] % 4 != 0) throw std::invalid_argument("Cannot split " + std::to_string(in[0]) + " onto 4 parts");
     if (in[1] != c.ci) throw std::invalid_argument("Input channels do not match the filter");
     return c;
 }
@@ -774,6 +775,8 @@ class UpstrideConv2DFunctor : public Operation {
         if (inputTensor.getShape().empty()) return;
         if (desc.has_bias && !biasTensor)
             throw std::invalid_argument("Bias application is configured but no bias tensor is given");
+        if (desc.real_input && biasTensor)  // src/conv2d.hpp:125-127
+            throw std::runtime_error("Bias addition is not supported for type0 inputs");
         const size_t bytes = phx_qconv2d_workspace_bytes(&desc, PHX_PASS_FWD);
         updateMemoryNeeds(bytes);
         void* ws = bytes ? allocator.mallocTemp(bytes) : nullptr;
@@ -804,6 +807,10 @@ class UpstrideConv2DGradFunctor : public Operation {
             kernelGradTensor.zero();
             return;
         }
+        // the gradient of a quaternion output with respect to a real input has imaginary parts that
+        // are not stored anywhere (src/conv2d.hpp:394-398)
+        if (desc.real_input && requireInputGrad)
+            throw std::logic_error("Input gradient required for type0 input tensor");
         const size_t bw = phx_qconv2d_workspace_bytes(&desc, PHX_PASS_BWD_WEIGHTS);
         const size_t bd = requireInputGrad ? phx_qconv2d_workspace_bytes(&desc, PHX_PASS_BWD_DATA) : 0;
         const size_t bytes = std::max(bw, bd);

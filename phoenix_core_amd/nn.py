@@ -57,11 +57,15 @@ class _QLinearFn(torch.autograd.Function):
 
 class QConv2d(nn.Module):
     """Quaternion Conv2D: x [4N, Ci, H, W] -> y [4N, Co, Ho, Wo]; padding 'SAME' / 'VALID' as in
-    the reference's descriptors (src/backend/conv2d_descriptor.hpp:132-174)."""
+    the reference's descriptors (src/backend/conv2d_descriptor.hpp:132-174).  With real_input the
+    layer takes a real tensor [N, Ci, H, W] (realValuedInput of the reference) and, as there, gives
+    no gradient for it."""
 
     def __init__(self, in_channels, out_channels, kernel_size, stride=1, padding="SAME", dilation=1, bias=False,
-                 dtype=torch.float32, context=None, input_requires_grad=True):
+                 dtype=torch.float32, context=None, input_requires_grad=True, real_input=False):
         super().__init__()
+        self.real_input = real_input
+        input_requires_grad = input_requires_grad and not real_input
         k = (kernel_size, kernel_size) if isinstance(kernel_size, int) else tuple(kernel_size)
         self.stride, self.padding, self.dilation = stride, padding, dilation
         self.context = context
@@ -76,7 +80,7 @@ class QConv2d(nn.Module):
         key = (tuple(x.shape), x.dtype)
         if key not in self._descs:
             common = dict(stride=self.stride, dilation=self.dilation, padding=self.padding, dtype=x.dtype,
-                          context=self.context)
+                          context=self.context, real_valued_input=self.real_input)
             fwd = ops.Conv2DDescriptor(x.shape, self.weight.shape, use_bias=self.bias is not None, **common)
             bwd = ops.Conv2DDescriptor(x.shape, self.weight.shape, require_input_grad=self.input_requires_grad, **common)
             self._descs[key] = (fwd, bwd)
@@ -132,12 +136,14 @@ class _Bottleneck(nn.Module):
 class QResNet50(nn.Module):
     """ResNet-50 with quaternion channels = real channels / 4: stem 3->16 (7x7 s2), stages of
     (3, 4, 6, 3) bottlenecks with widths 16/32/64/128 and outputs 64/128/256/512, head = quaternion
-    Dense 512 -> 250 units (= 1000 logits).  53 convolutions."""
+    Dense 512 -> 250 units (= 1000 logits).  53 convolutions.  The stem takes the real images
+    [N, 3, H, W] directly (real_input=True) or, with real_input=False, their lift() to quaternions."""
 
-    def __init__(self, num_classes=1000, dtype=torch.float32, context=None):
+    def __init__(self, num_classes=1000, dtype=torch.float32, context=None, real_input=True):
         super().__init__()
         assert num_classes % 4 == 0
-        self.stem = QConv2d(3, 16, 7, stride=2, padding="SAME", dtype=dtype, context=context, input_requires_grad=False)
+        self.stem = QConv2d(3, 16, 7, stride=2, padding="SAME", dtype=dtype, context=context, input_requires_grad=False,
+                            real_input=real_input)
         self.bn = nn.BatchNorm2d(16)
         self.relu = nn.ReLU(inplace=True)
         self.pool = nn.MaxPool2d(3, 2, 1)
@@ -155,10 +161,10 @@ class QResNet50(nn.Module):
         z = torch.zeros_like(images)
         return torch.cat([images, z, z, z], dim=0)
 
-    def forward(self, xq):
-        y = self.pool(self.relu(self.bn(self.stem(xq))))
+    def forward(self, x):
+        y = self.pool(self.relu(self.bn(self.stem(x))))
         y = self.blocks(y)
-        y = y.float().mean(dim=(2, 3)).to(xq.dtype)           # [4N, 512]
+        y = y.float().mean(dim=(2, 3)).to(x.dtype)            # [4N, 512]
         y = self.head(y)                                      # [4N, 250]
         n = y.shape[0] // 4
         return y.view(4, n, -1).permute(1, 0, 2).reshape(n, -1)  # [N, 1000]: the four components side by side

@@ -86,7 +86,7 @@ class Conv2DDescriptor:
 
     def __init__(self, input_shape, filter_shape, stride=1, dilation=1, padding="VALID", groups=1,
                  algebra=QUATERNION, filter_layout="OIHW", use_bias=False, dtype=torch.float32, context=None,
-                 require_input_grad=True):
+                 require_input_grad=True, real_valued_input=False):
         if len(input_shape) != 4:
             raise ValueError("Four-dimensional input tensor expected")
         if algebra != QUATERNION:
@@ -97,7 +97,7 @@ class Conv2DDescriptor:
             raise ValueError("First filter dimension mismatch, got %d" % filter_shape[0])
         if groups != 1:
             raise NotImplementedError("grouped quaternion convolution is not built")
-        if input_shape[0] % 4:
+        if not real_valued_input and input_shape[0] % 4:
             raise ValueError("Cannot split %d onto 4 parts" % input_shape[0])
         if filter_layout == "OIHW":
             _, co, ci, kh, kw = filter_shape
@@ -115,7 +115,12 @@ class Conv2DDescriptor:
         self.use_bias = bool(use_bias)
         self.require_input_grad = bool(require_input_grad)
         self.dtype = dtype
+        # real-valued input (realValuedInput of the reference's descriptors): [n, ci, h, w] without imaginary
+        # parts; the output still has the four components stacked on the batch axis
+        self.real_valued_input = bool(real_valued_input)
         n4, _, h, w = input_shape
+        if self.real_valued_input:
+            n4 *= 4
         if isinstance(padding, str):
             ho, pt, pb = windowed_output_size_and_padding(h, kh, self.dilation[0], self.stride[0], padding)
             wo, pl, pr = windowed_output_size_and_padding(w, kw, self.dilation[1], self.stride[1], padding)
@@ -129,7 +134,8 @@ class Conv2DDescriptor:
         self.c = capi.QConvDesc(
             _DTYPES[dtype], n4 // 4, ci, co, h, w, kh, kw, self.stride[0], self.stride[1], self.dilation[0],
             self.dilation[1], pt, pl, pb, pr, capi.PHX_OIHW if filter_layout == "OIHW" else capi.PHX_OHWI,
-            self.context.product_mode, self.context.fp16_policy, int(self.use_bias))
+            self.context.product_mode, self.context.fp16_policy, int(self.use_bias and not self.real_valued_input),
+            int(self.real_valued_input))
 
     def workspace_bytes(self, which):
         return capi.lib().phx_qconv2d_workspace_bytes(ctypes.byref(self.c), which)
@@ -218,6 +224,8 @@ def conv2d_fwd(x, w, bias, desc, out=None):
         raise ValueError("tensor shapes / dtype do not match the descriptor")
     if desc.use_bias and (bias is None or tuple(bias.shape) != desc.bias_shape):
         raise ValueError("bias tensor missing or of wrong shape")
+    if desc.real_valued_input and desc.use_bias:  # src/conv2d.hpp:125-127
+        raise RuntimeError("Bias addition is not supported for type0 inputs")
     y = out if out is not None else torch.empty(desc.output_shape, dtype=desc.dtype, device=dev)
     nbytes = desc.workspace_bytes(capi.PHX_PASS_FWD)
     ws = _workspace.get(dev, nbytes)
@@ -241,6 +249,8 @@ def conv2d_bwd(x, w, grad, desc):
                                                   _ptr(ws), nbytes), "phx_qconv2d_bwd_weights")
     dx = None
     if desc.require_input_grad:
+        if desc.real_valued_input:  # src/conv2d.hpp:394-398
+            raise RuntimeError("Input gradient required for type0 input tensor")
         dx = torch.empty(desc.input_shape, dtype=desc.dtype, device=dev)
         nbytes = desc.workspace_bytes(capi.PHX_PASS_BWD_DATA)
         ws = _workspace.get(dev, nbytes)

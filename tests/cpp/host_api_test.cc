@@ -171,6 +171,39 @@ static void gpuQuaternionOnes(Context& context) {  // tests/tests.cpp:292-315
     CHECK(out[0] == -36.0f && out[1] == 36.0f && out[2] == 36.0f && out[3] == 36.0f);
 }
 
+static void gpuQuaternionRealInput(Context& context) {  // tests/tests.cpp:317-369
+    device::HIP device(context);
+    AllocatedTensor<device::HIP, float> input(device, {1, 3, 2, 2});
+    input = {0, 0, 0, 0,   -1, 0, 0, 0,   1, 2, 3, 4};
+    AllocatedTensor<device::HIP, float> kernel(device, {MULTIVECTOR_DIM[Algebra::QUATERNION], 2, 3, 1, 1});
+    kernel = {1, 1, 1,  0, 0, 2,    0, 0, 0,  -1, -1, -1,    0, 1, 2,  0, 2, 4,    -1, -2, -3,  0, 0, 1};
+    AllocatedTensor<device::HIP, float> output(device, {MULTIVECTOR_DIM[Algebra::QUATERNION], 2, 2, 2});
+    Conv2DFwdDescriptor descriptor(input.getShape(), kernel.getShape(), 1, 1, Padding::VALID, {}, 1, Algebra::QUATERNION,
+                                   DataFormat::NCHW, FilterLayout::OIHW, false, true);
+    CHECK(descriptor.getOutputShape() == Shape({4, 2, 2, 2}));
+    conv2DFwd<device::HIP, float>(device, device, input, kernel, nullptr, output, descriptor);
+    std::vector<float> got = output;
+    CHECK(equalVectors(got, std::vector<float>{0, 2, 3, 4,  2, 4, 6, 8,    0, 0, 0, 0,  0, -2, -3, -4,
+                                               1, 4, 6, 8,  2, 8, 12, 16,  -1, -6, -9, -12,  1, 2, 3, 4}));
+    // filter gradient for g = 1 in the real component of output channel 0: dw_r(0, c) = sum over pixels of x_c
+    // for r = 0 and 0 for the imaginary parts' own products with the zero imaginary input, i.e. conj(x) (x) g
+    AllocatedTensor<device::HIP, float> g(device, {4, 2, 2, 2}), dw(device, {4, 2, 3, 1, 1}), dx(device, {1, 3, 2, 2});
+    std::vector<float> gv(32, 0.f);
+    for (int i = 0; i < 4; ++i) gv[i] = 1.f;
+    g = gv;
+    Conv2DBwdDescriptor bd(input.getShape(), kernel.getShape(), 1, 1, Padding::VALID, {}, 1, Algebra::QUATERNION,
+                           DataFormat::NCHW, FilterLayout::OIHW, false, true);
+    conv2DBwd<device::HIP, float>(device, device, input, kernel, g, dw, dx, bd);
+    std::vector<float> gdw = dw;
+    std::vector<float> want(24, 0.f);
+    want[0] = 0.f; want[1] = -1.f; want[2] = 10.f;
+    CHECK(equalVectors(gdw, want, 1e-5f));
+    // the input gradient cannot be required (src/conv2d.hpp:394-398)
+    Conv2DBwdDescriptor need(input.getShape(), kernel.getShape(), 1, 1, Padding::VALID, {}, 1, Algebra::QUATERNION,
+                             DataFormat::NCHW, FilterLayout::OIHW, true, true);
+    CHECK_THROWS((conv2DBwd<device::HIP, float>(device, device, input, kernel, g, dw, dx, need)), std::logic_error);
+}
+
 static void gpuPointwiseKnownAnswer(Context& context) {
     // 2 pixels, 2 input channels, 1 output channel; y = sum_c x_c (x) w_c computed by hand:
     //   pixel 0: (1+2i)(3+k) + (j)(1-i)   = (3 + 6i - 2j + k) + (j + k)      = 3 + 6i - j + 2k
@@ -260,6 +293,7 @@ int main(int argc, char** argv) {
             if (pass) setenv("UPSTRIDE_MEMORY_OPTIMIZED", "1", 1); else unsetenv("UPSTRIDE_MEMORY_OPTIMIZED");
             Context context;
             gpuQuaternionOnes(context);
+            gpuQuaternionRealInput(context);
             gpuPointwiseKnownAnswer(context);
             gpuDenseAndEmpty(context);
             testTensorSplit(context);

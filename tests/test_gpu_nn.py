@@ -109,15 +109,18 @@ def _cpu_forward(model, xq):
     return logits, cpu_params
 
 
-def test_qresnet50_end_to_end_matches_cpu_restatement():
+@pytest.mark.parametrize("real_input", [True, False])
+def test_qresnet50_end_to_end_matches_cpu_restatement(real_input):
+    """The stem either takes the real images (real-valued input) or their lift to quaternions with zero
+    imaginary parts; the CPU restatement always runs on the lifted tensor."""
     torch.manual_seed(2)
-    model = phx.QResNet50(num_classes=1000, dtype=torch.float32, context=Ctx(8)).cuda().train()
+    model = phx.QResNet50(num_classes=1000, dtype=torch.float32, context=Ctx(8), real_input=real_input).cuda().train()
     convs = model.conv_layers()
     assert len(convs) == 53
     images = torch.randn(2, 3, 64, 64)
     labels = torch.tensor([3, 997])
     xq = phx.QResNet50.lift(images)
-    logits = model(xq.cuda())
+    logits = model(images.cuda() if real_input else xq.cuda())
     loss = torch.nn.functional.cross_entropy(logits, labels.cuda())
     loss.backward()
     cpu_logits, cpu_params = _cpu_forward(model, xq)

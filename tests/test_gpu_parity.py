@@ -2,6 +2,8 @@
 inputs.  Tolerances are the ones the task states: relative error (max-norm and L2) <= 1e-4 for
 fp32 tensors, <= 2e-2 for fp16 tensors under every fp16 policy; the yardstick is the oracle's
 fp64 closed-form quaternion convolution evaluated on the (fp16-rounded) inputs."""
+import ctypes
+
 import numpy as np
 import pytest
 import torch
@@ -116,6 +118,75 @@ def test_reference_kat_quaternion_ones():
         desc = phx.Conv2DDescriptor(x.shape, w.shape, 1, 1, "VALID", context=Ctx(mode))
         y = phx.conv2d_fwd(x, w, None, desc)
         assert y.flatten().tolist() == [-36.0, 36.0, 36.0, 36.0]
+
+
+def test_reference_kat_quaternion_real_input():
+    """tests/tests.cpp:317-369 of the reference: a real 3x2x2 image through a quaternion 1x1 filter with
+    two output channels, exact, on both product paths."""
+    x = [0, 0, 0, 0, -1, 0, 0, 0, 1, 2, 3, 4]
+    w = [1, 1, 1, 0, 0, 2, 0, 0, 0, -1, -1, -1, 0, 1, 2, 0, 2, 4, -1, -2, -3, 0, 0, 1]
+    want = [0, 2, 3, 4, 2, 4, 6, 8, 0, 0, 0, 0, 0, -2, -3, -4, 1, 4, 6, 8, 2, 8, 12, 16, -1, -6, -9, -12, 1, 2, 3, 4]
+    for mode in (8, 16):
+        for dtype in (torch.float32, torch.float16):
+            xd = torch.tensor(x, dtype=dtype, device="cuda").reshape(1, 3, 2, 2)
+            wd = torch.tensor(w, dtype=dtype, device="cuda").reshape(4, 2, 3, 1, 1)
+            desc = phx.Conv2DDescriptor(xd.shape, wd.shape, 1, 1, "VALID", dtype=dtype, context=Ctx(mode, "full16"),
+                                        real_valued_input=True)
+            assert desc.output_shape == (4, 2, 2, 2)
+            y = phx.conv2d_fwd(xd, wd, None, desc)
+            assert y.flatten().tolist() == [float(v) for v in want], (mode, dtype)
+
+
+REAL_INPUT_CASES = [c for c in CONV_CASES if c[0] in ("pw_ragged", "k3_same", "k3_ragged", "k3_s2", "k7_s2", "k3_s2_c4",
+                                                      "k32_asym", "pw_64")] + [
+    ("stem_7x7", 2, 3, 64, 64, 64, 7, 7, 2, 1, "SAME"),
+]
+
+
+@pytest.mark.parametrize("dtype,policy", [(torch.float32, "fp32"), (torch.float16, "full16"), (torch.float16, "fp32")],
+                         ids=["f32", "f16_full16", "f16_fp32"])
+@pytest.mark.parametrize("mode", [16, 8])
+@pytest.mark.parametrize("case", REAL_INPUT_CASES, ids=[c[0] for c in REAL_INPUT_CASES])
+def test_conv_real_valued_input(case, mode, dtype, policy):
+    """Real-valued input (realValuedInput of the reference's descriptors, src/conv2d.hpp:122-164 forward,
+    384-430 backward): x is [n, ci, h, w], the output and the filter gradient are quaternion-valued, and the
+    input gradient cannot be asked for.  The fp32 yardstick is the oracle's restatement of that branch; for
+    fp16 tensors it is the fp64 closed form on the input padded with zero imaginary parts."""
+    name, n, ci, co, h, w, kh, kw, stride, dilation, padding = case
+    scale = 1.0 if dtype == torch.float32 else 0.5
+    g, x, wt, b, gr = make_inputs(hash(name) % 1000 + 2, n, ci, co, h, w, kh, kw, stride, dilation, padding, dtype, scale)
+    x = np.ascontiguousarray(x[:n])
+    print("case", name, "mode", mode, dtype, policy, flush=True)
+    ctx = Ctx(mode, policy)
+    desc = phx.Conv2DDescriptor(x.shape, wt.shape, stride, dilation, padding, dtype=dtype, context=ctx,
+                                real_valued_input=True, require_input_grad=False)
+    assert desc.output_shape == (4 * n, co, g.ho, g.wo)
+    xd, wd, bd, gd = (torch.from_numpy(a).cuda() for a in (x, wt, b, gr))
+    y = phx.conv2d_fwd(xd, wd, None, desc)
+    k_fwd = capi.last_kernel_name()
+    dw, dx = phx.conv2d_bwd(xd, wd, gd, desc)
+    torch.cuda.synchronize()
+    assert dx is None
+    if dtype == torch.float32:
+        want_y = oracle.conv2d_fwd(g, x, wt, None, "generic", real_valued_input=True)
+        want_dw, _ = oracle.conv2d_bwd(g, x, wt, gr, "generic", real_valued_input=True)
+    else:
+        x4 = np.zeros((4 * n,) + x.shape[1:], np.float64)
+        x4[:n] = x
+        w64, b64, g64 = (a.astype(np.float64) for a in (wt, b, gr))
+        want_y = oracle.conv2d_fwd(g, x4, w64, None, "hamilton")
+        want_dw, _ = oracle.conv2d_bwd(g, x4, w64, g64, "hamilton")
+    assert_close(y.cpu().numpy(), want_y, dtype, "fwd " + k_fwd)
+    assert_close(dw.cpu().numpy(), want_dw, dtype, "wgrad " + capi.last_kernel_name())
+    # neither a bias nor the input gradient can be asked for, as in the reference (src/conv2d.hpp:125-127, 394-398)
+    with pytest.raises(RuntimeError):
+        phx.conv2d_fwd(xd, wd, bd, phx.Conv2DDescriptor(x.shape, wt.shape, stride, dilation, padding, use_bias=True,
+                                                        dtype=dtype, context=ctx, real_valued_input=True))
+    with pytest.raises(RuntimeError):
+        phx.conv2d_bwd(xd, wd, gd, phx.Conv2DDescriptor(x.shape, wt.shape, stride, dilation, padding, dtype=dtype,
+                                                        context=ctx, real_valued_input=True))
+    assert capi.lib().phx_qconv2d_bwd_data(ctypes.byref(desc.c), None, None, None, None, None, 0) == \
+        capi.PHX_ERR_INVALID_ARGUMENT
 
 
 @pytest.mark.parametrize("mode", [16, 8])
