@@ -388,6 +388,38 @@ __device__ __forceinline__ void stage_chunk_store(f16x8* xl, const u32x4 (&r)[8]
     }
 }
 
+// One eighth of the left-operand lane map of the factorized product: step i leaves lane i ready
+// (forward: lanes_left; input gradient: lanes_grad without the factor 1/2, which the packed filters
+// carry; T holds its four partial sums between steps).
+template <int MAP>
+__device__ __forceinline__ void lane_step(const f16x8 (&x)[4], f16x8 (&L)[8], f16x8 (&T)[4], int i) {
+    if constexpr (MAP == MAP_FWD) {
+        switch (i) {
+            case 0: L[0] = add8(x[3], x[1]); break;
+            case 1: L[1] = sub8(x[0], x[2]); break;
+            case 2: L[2] = add8(x[0], x[2]); break;
+            case 3: L[3] = sub8(x[3], x[1]); break;
+            case 4: L[4] = sub8(x[3], x[2]); break;
+            case 5: L[5] = add8(x[1], x[0]); break;
+            case 6: L[6] = sub8(x[0], x[1]); break;
+            default: L[7] = add8(x[3], x[2]); break;
+        }
+    } else {
+        // the plain copies (lanes 4..7) first: they free the component registers for the next request;
+        // T = {g0+g1, g2+g3, g0-g1, g2-g3}
+        switch (i) {
+            case 0: L[4] = x[0]; L[5] = x[1]; T[0] = add8(x[0], x[1]); break;
+            case 1: L[6] = x[2]; L[7] = x[3]; T[1] = add8(x[2], x[3]); break;
+            case 2: T[2] = sub8(x[0], x[1]); break;
+            case 3: T[3] = sub8(x[2], x[3]); break;
+            case 4: L[0] = sub8(T[1], T[0]); break;
+            case 5: L[1] = sub8(T[2], T[3]); break;
+            case 6: L[2] = add8(T[2], T[3]); break;
+            default: L[3] = add8(T[0], T[1]); break;
+        }
+    }
+}
+
 template <int MODE, int MAP, int WCO, int NTW, int P2LOG, bool CHUNKS>
 __global__ void __launch_bounds__(WG_THREADS, (MODE == 16 && NTW == 1) ? 2 : 1) qconv_fwd_f16_lds_kernel(const ConvArgs P) {
     constexpr int CK = F16_CK;
@@ -398,12 +430,16 @@ __global__ void __launch_bounds__(WG_THREADS, (MODE == 16 && NTW == 1) ? 2 : 1) 
     constexpr int WIMG = TG * WCO * NW * 64;   // 16-byte vectors per filter group image
     constexpr int NSL = TG * WCO * NW / 4;     // 1 KiB slices of that image per wave
     extern __shared__ f16x8 lds16[];
-    f16x8* xl = lds16;                    // [8 units][HPp]
-    f16x8* wl = lds16 + 8 * P.HPp;        // [2][WIMG]
+    // unit pitch of the staged window: fixed with chunk staging, so that the four component reads of an
+    // operand differ by immediate offsets only (the host sets HPp to the same value)
+    const int XP = CHUNKS ? F16_XPITCH : P.HPp;
+    f16x8* xl = lds16;                    // [8 units][XP]
+    f16x8* wl = lds16 + 8 * XP;           // [2][WIMG]
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wco = wave % WCO, wpx = wave / WCO;
     const int j = lane & 31, kk = lane >> 5;
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);  // (a scalar the compiler can address LDS copies with)
 
     int bid = xcd_remap(blockIdx.x, gridDim.x);
     const int ct = bid % P.co_tiles;
@@ -443,7 +479,7 @@ __global__ void __launch_bounds__(WG_THREADS, (MODE == 16 && NTW == 1) ? 2 : 1) 
 
     // activation staging, one chunk ahead in registers
     const StagePos sp = make_stage_pos<P2LOG>(P.in, n0, h0, w0, P.NB, P.HTH, P.HTW);
-    const StageChunk sc = make_stage_chunk(P.in, n0, h0, w0, P.NB, P.HTH, P.HTW, P.HPp);
+    const StageChunk sc = make_stage_chunk(P.in, n0, h0, w0, P.NB, P.HTH, P.HTW, XP);
     f16x8 stage[CHUNKS ? 1 : (8 >> (8 - P2LOG))];
     u32x4 stagec[CHUNKS ? 8 : 1];
     constexpr int XLOADS = CHUNKS ? 8 : 0;  // activation load instructions that can be dealt out one by one
@@ -457,18 +493,32 @@ __global__ void __launch_bounds__(WG_THREADS, (MODE == 16 && NTW == 1) ? 2 : 1) 
     } else {
         stage_load16<P2LOG>(stage, P.in, sp, 0);
     }
-    // filter group image -> LDS buffer: slices of 64 vectors, dealt round-robin to the waves
+    // filter group image -> LDS buffer: slices of 64 vectors, dealt round-robin to the waves.  Slice
+    // s * 4 + wave starts at vector s * 256 + wave * 64: a uniform base plus the thread index on the
+    // global side, a scalar address on the LDS side.
+    auto copy_slice = [&](const f16x8* src, f16x8* dst, int s) {
+        lds_dma_16(src + s * 256 + tid, dst + s * 256 + wave_u * 64);
+    };
     {
 #pragma unroll
-        for (int s = 0; s < NSL; ++s) {
-            const int slice = s * 4 + wave;
-            lds_dma_16(wsrc + slice * 64 + lane, wl + slice * 64);
-        }
+        for (int s = 0; s < NSL; ++s) copy_slice(wsrc, wl, s);
     }
 
     PHX_PHASES_BEGIN(5)
     bool x_in_flight = false;  // activation loads were issued after the latest filter copy
     int chunk = 0, g = 0, tap = 0, kh = 0, kw = 0;
+    // Factorized form: the left lanes of a block are formed from the four staged components while the
+    // previous block is being multiplied (one wave per SIMD: nothing else hides that arithmetic), from
+    // components requested a block earlier still.  Where the next group works on the same staged chunk
+    // that pipeline runs on across the group boundary (CARRY; it needs an even number of blocks per group
+    // so that the register double buffers keep their parity).
+#ifdef PHX_EXP_NOCARRY
+    constexpr bool CARRY = false;
+#else
+    constexpr bool CARRY = MODE == 8 && (TG * NTW) % 2 == 0;
+#endif
+    f16x8 xf[2][4], Lf[MODE == 8 ? 2 : 1][8], Lt[4];
+    bool carried = false;      // the previous group left this group's first lanes and components in registers
     // one flat loop over (chunk, filter group) steps: a single loop keeps the accumulators in place
     for (int gs = 0; gs < total_groups; ++gs) {
         if (g == 0) {
@@ -497,29 +547,52 @@ __global__ void __launch_bounds__(WG_THREADS, (MODE == 16 && NTW == 1) ? 2 : 1) 
             constexpr int XPB = XBLK ? (XLOADS + XBLK - 1) / XBLK : 0;
             const bool more_groups = gs + 1 < total_groups;
             const bool more_chunks = g == 0 && chunk + 1 < P.nchunks;
-            int tapoff[TG];
+            // window offsets of this group's taps and (CARRY) of the next group's
+            int tapoff[CARRY ? 2 * TG : TG];
 #pragma unroll
             for (int tg = 0; tg < TG; ++tg) {
                 tapoff[tg] = tap < P.taps ? kh * P.dh * P.HTW + kw * P.dw : 0;
                 ++tap;
                 if (++kw == P.Kw) { kw = 0; ++kh; }
             }
+            if constexpr (CARRY) {
+                int tap2 = tap, kh2 = kh, kw2 = kw;
+#pragma unroll
+                for (int tg = TG; tg < 2 * TG; ++tg) {
+                    tapoff[tg] = tap2 < P.taps ? kh2 * P.dh * P.HTW + kw2 * P.dw : 0;
+                    ++tap2;
+                    if (++kw2 == P.Kw) { kw2 = 0; ++kh2; }
+                }
+            }
+            const bool carry = CARRY && g + 1 < ngroups;  // the next group multiplies the same staged chunk
             const f16x8* wb = wl + (gs & 1) * WIMG + wco * (NW * 64) + lane;
             const f16x8* wsrc_next = wsrc + (long)(gs + 1) * WIMG;
             f16x8* wdst_next = wl + ((gs + 1) & 1) * WIMG;
-            f16x8 wf[2][NW], xf[2][4];
+            f16x8 wf[2][NW];
             auto read_w = [&](f16x8 (&w)[NW], int tg) {
 #pragma unroll
                 for (int r = 0; r < NW; ++r) w[r] = wb[(tg * WCO * NW + r) * 64];
             };
             auto read_x = [&](f16x8 (&x)[4], int blk) {
                 const int pos = tapoff[blk / NTW] + poff[blk % NTW];
-                const f16x8* xb = xl + kk * P.HPp + (CHUNKS ? swizzle_entry(pos) : pos);
+                const f16x8* xb = xl + kk * XP + (CHUNKS ? swizzle_entry(pos) : pos);
 #pragma unroll
-                for (int p = 0; p < 4; ++p) x[p] = xb[p * 2 * P.HPp];
+                for (int p = 0; p < 4; ++p) x[p] = xb[p * 2 * XP];
             };
             read_w(wf[0], 0);
-            read_x(xf[0], 0);
+            if constexpr (MODE == 16) {
+                read_x(xf[0], 0);
+            } else {
+                if (!carried) {
+                    read_x(xf[0], 0);
+                    if (NBLK > 1) read_x(xf[1], 1);
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) lane_step<MAP>(xf[0], Lf[0], Lt, i);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                if (NBLK > 2) read_x(xf[0], 2);
+                __builtin_amdgcn_sched_barrier(0);
+            }
             if constexpr (!CHUNKS) {
                 if (more_chunks) stage_load16<P2LOG>(stage, P.in, sp, (chunk + 1) * CK);
             }
@@ -529,17 +602,17 @@ __global__ void __launch_bounds__(WG_THREADS, (MODE == 16 && NTW == 1) ? 2 : 1) 
                 const int tg = blk / NTW, t = blk % NTW;
                 if (blk < DBLK) {
                     if (more_groups) {
+                        // (loops with constant bounds: they must unroll, the staging registers are indexed by them)
 #pragma unroll
-                        for (int s = blk * DPB; s < (blk + 1) * DPB && s < NSL; ++s) {
-                            const int slice = s * 4 + wave;
-                            lds_dma_16(wsrc_next + slice * 64 + lane, wdst_next + slice * 64);
+                        for (int s = 0; s < NSL; ++s) {
+                            if (s / DPB == blk) copy_slice(wsrc_next, wdst_next, s);
                         }
                     }
                 } else if constexpr (CHUNKS) {
                     if (more_chunks) {
 #pragma unroll
-                        for (int i = (blk - DBLK) * XPB; i < (blk - DBLK + 1) * XPB && i < 8; ++i)
-                            stage_chunk_load(stagec, P.in, sc, (chunk + 1) * CK, i);
+                        for (int i = 0; i < 8; ++i)
+                            if (i / XPB == blk - DBLK) stage_chunk_load(stagec, P.in, sc, (chunk + 1) * CK, i);
                     }
                 }
                 const f16x8(&w)[NW] = wf[tg & 1];
@@ -568,15 +641,26 @@ __global__ void __launch_bounds__(WG_THREADS, (MODE == 16 && NTW == 1) ? 2 : 1) 
                         if (p == 0) prefetch();
                     }
                 } else {
-                    // factorized form: eight independent products of a left lane (formed here from the four
-                    // staged components) with a right lane (packed)
-                    f16x8 L[8];
-                    if constexpr (MAP == MAP_FWD) lanes_left(x, L);
-                    else lanes_grad(x, L, (_Float16)0.5f);
+                    // factorized form: eight independent products of a left lane with a right lane (packed).
+                    // Each product is followed by the arithmetic for one lane of the next block; the
+                    // components of the block after that are requested as soon as their registers are free.
+                    __builtin_amdgcn_sched_barrier(0);
+                    // (block numbers from NBLK on are the next group's, reached only with carry; the third
+                    // block of the next group is requested at that group's start, once its first is consumed)
+                    // The requests go out after the first product: whatever the wait in front of that
+                    // product covers was requested a whole block ago.
 #pragma unroll
                     for (int i = 0; i < 8; ++i) {
-                        acc[t][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(w[i], L[i], acc[t][i], 0, 0, 0);
-                        if (i == 1) prefetch();
+                        acc[t][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(w[i], Lf[blk & 1][i], acc[t][i], 0, 0, 0);
+                        if (blk + 1 < NBLK || carry) lane_step<MAP>(xf[(blk + 1) & 1], Lf[(blk + 1) & 1], Lt, i);
+                        __builtin_amdgcn_sched_barrier(0);
+                        // (last block: after the lane arithmetic, whose waits sit behind run-time branches there
+                        // and are therefore complete ones)
+                        if (i == (blk == NBLK - 1 ? 7 : 0)) {
+                            if (blk > 0 && (blk + 2 < NBLK || carry)) read_x(xf[blk & 1], blk + 2);
+                            if (t == NTW - 1 && tg + 1 < TG) read_w(wf[(tg + 1) & 1], tg + 1);
+                            __builtin_amdgcn_sched_barrier(0);
+                        }
                     }
                 }
                 // pin the accumulators to the AGPR file: left alone, the allocator parks one column tile in
@@ -588,6 +672,7 @@ __global__ void __launch_bounds__(WG_THREADS, (MODE == 16 && NTW == 1) ? 2 : 1) 
                 __builtin_amdgcn_sched_barrier(0);
             }
             x_in_flight = CHUNKS && more_chunks;
+            carried = carry;
             PHX_STAMP(4)
         }
         if (++g == ngroups) { g = 0; ++chunk; }
@@ -653,7 +738,8 @@ __global__ void __launch_bounds__(WG_THREADS) pack_filters_f16_lds_kernel(const 
 #pragma unroll
                         for (int c = 0; c < 4; ++c) wv[c] = (float)w[c * P.wcs + off];
                         lanes_right(wv, R);  // formed in fp32, rounded once
-                        vec[i] = (_Float16)R[r];
+                        // input gradient: the kernel forms the gradient lanes 0..3 without their factor 1/2
+                        vec[i] = (_Float16)((MAP == MAP_DGRAD && r < 4) ? 0.5f * R[r] : R[r]);
                     }
                 }
             }

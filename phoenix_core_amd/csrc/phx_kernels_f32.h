@@ -12,6 +12,7 @@ enum { MAP_FWD = 0, MAP_DGRAD = 1 };
 constexpr int F32_CK = 8;   // fp32 MFMA: input channels per K chunk (4 MFMA k-pairs)
 constexpr int F16_CK = 16;  // fp16 MFMA: input channels per K chunk = one MFMA K step (two 8-channel packs)
 constexpr int F16_TG = 3;   // fp16 MFMA, LDS-staged filters: taps per filter group
+constexpr int F16_XPITCH = 256;  // fp16 LDS kernels with chunk staging: entries per unit of the staged window
 
 struct ConvArgs {
     TileSrc in;         // x (forward) or the output gradient (input-gradient pass)

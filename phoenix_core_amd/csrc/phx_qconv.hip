@@ -251,6 +251,7 @@ static bool plan_forward(const Corr& c, int mode, bool f16mfma, FwdPlan& best) {
         best.CK = F16_CK;
         best.P2LOG = best.HP <= 128 ? 7 : 8;
         best.nchunks = cdiv(c.Cin, best.CK);
+        if (chunks) best.HPp = F16_XPITCH;  // the chunk-staging kernels address the window with a fixed unit pitch
         best.lds_bytes = (size_t)8 * best.HPp * 16;
         best.wpk_bytes = (size_t)best.co_tiles * best.WCO * best.nchunks * taps * 64 * WC * 16;
         best.lds_filters = ldsk;
