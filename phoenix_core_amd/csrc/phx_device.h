@@ -85,23 +85,15 @@ __device__ __forceinline__ void lanes_grad(const V (&g)[4], V (&G)[8], S half) {
 }
 
 // The same lane maps on eight packed halves.  The compiler expands a vector subtraction of halves
-// into scalar operations (three instructions per register); a - b is issued here as one packed add
-// with the second operand negated.
-__device__ __forceinline__ f16x8 sub8(const f16x8 a, const f16x8 b) {
-    const u32x4 ua = __builtin_bit_cast(u32x4, a), ub = __builtin_bit_cast(u32x4, b);
-    u32x4 r;
-#pragma unroll
-    for (int m = 0; m < 4; ++m) {
-        unsigned int t;
-        asm("v_pk_add_f16 %0, %1, %2 neg_lo:[0,1] neg_hi:[0,1]" : "=v"(t) : "v"(ua[m]), "v"(ub[m]));
-        r[m] = t;
-    }
-    return __builtin_bit_cast(f16x8, r);
-}
+// into scalar operations (three instructions per register); a - b is written as a + (-b) with the
+// sign flipped by an integer XOR, which it cannot fold back into a subtraction: two instructions.
+__device__ __forceinline__ f16x8 sub8(const f16x8 a, const f16x8 b) { return a + neg8(b); }
 
-// a + b through the same route: unlike the plain operator it stays where it is written, between the
-// matrix instructions it is meant to overlap with
-__device__ __forceinline__ f16x8 add8(const f16x8 a, const f16x8 b) {
+// Single-instruction forms, a + b and a - b as one packed add (second operand negated).  The
+// instruction scheduler and the hazard logic of the compiler do not see through these: use them only
+// where the result is consumed many instructions later (lane_step in the LDS forward kernel), and
+// they then stay exactly where they are written, between the matrix instructions they overlap with.
+__device__ __forceinline__ f16x8 add8_pinned(const f16x8 a, const f16x8 b) {
     const u32x4 ua = __builtin_bit_cast(u32x4, a), ub = __builtin_bit_cast(u32x4, b);
     u32x4 r;
 #pragma unroll
@@ -113,22 +105,35 @@ __device__ __forceinline__ f16x8 add8(const f16x8 a, const f16x8 b) {
     return __builtin_bit_cast(f16x8, r);
 }
 
+__device__ __forceinline__ f16x8 sub8_pinned(const f16x8 a, const f16x8 b) {
+    const u32x4 ua = __builtin_bit_cast(u32x4, a), ub = __builtin_bit_cast(u32x4, b);
+    u32x4 r;
+#pragma unroll
+    for (int m = 0; m < 4; ++m) {
+        unsigned int t;
+        asm("v_pk_add_f16 %0, %1, %2 neg_lo:[0,1] neg_hi:[0,1]" : "=v"(t) : "v"(ua[m]), "v"(ub[m]));
+        r[m] = t;
+    }
+    return __builtin_bit_cast(f16x8, r);
+}
+
 __device__ __forceinline__ void lanes_left(const f16x8 (&x)[4], f16x8 (&L)[8]) {
+    const f16x8 n1 = neg8(x[1]), n2 = neg8(x[2]);
     L[0] = x[3] + x[1];
-    L[1] = sub8(x[0], x[2]);
+    L[1] = x[0] + n2;
     L[2] = x[0] + x[2];
-    L[3] = sub8(x[3], x[1]);
-    L[4] = sub8(x[3], x[2]);
+    L[3] = x[3] + n1;
+    L[4] = x[3] + n2;
     L[5] = x[1] + x[0];
-    L[6] = sub8(x[0], x[1]);
+    L[6] = x[0] + n1;
     L[7] = x[3] + x[2];
 }
 
 // lanes_grad without the factor 1/2 on lanes 0..3 (the caller folds it into the other operand)
 __device__ __forceinline__ void lanes_grad_unscaled(const f16x8 (&g)[4], f16x8 (&G)[8]) {
-    const f16x8 t1 = g[0] + g[1], t3 = sub8(g[0], g[1]), t2 = g[2] + g[3], t4 = sub8(g[2], g[3]);
-    G[0] = sub8(t2, t1);
-    G[1] = sub8(t3, t4);
+    const f16x8 t1 = g[0] + g[1], t3 = g[0] + neg8(g[1]), t2 = g[2] + g[3], t4 = g[2] + neg8(g[3]);
+    G[0] = t2 + neg8(t1);
+    G[1] = t3 + neg8(t4);
     G[2] = t3 + t4;
     G[3] = t1 + t2;
     G[4] = g[0];

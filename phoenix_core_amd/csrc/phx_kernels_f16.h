@@ -395,27 +395,27 @@ template <int MAP>
 __device__ __forceinline__ void lane_step(const f16x8 (&x)[4], f16x8 (&L)[8], f16x8 (&T)[4], int i) {
     if constexpr (MAP == MAP_FWD) {
         switch (i) {
-            case 0: L[0] = add8(x[3], x[1]); break;
-            case 1: L[1] = sub8(x[0], x[2]); break;
-            case 2: L[2] = add8(x[0], x[2]); break;
-            case 3: L[3] = sub8(x[3], x[1]); break;
-            case 4: L[4] = sub8(x[3], x[2]); break;
-            case 5: L[5] = add8(x[1], x[0]); break;
-            case 6: L[6] = sub8(x[0], x[1]); break;
-            default: L[7] = add8(x[3], x[2]); break;
+            case 0: L[0] = add8_pinned(x[3], x[1]); break;
+            case 1: L[1] = sub8_pinned(x[0], x[2]); break;
+            case 2: L[2] = add8_pinned(x[0], x[2]); break;
+            case 3: L[3] = sub8_pinned(x[3], x[1]); break;
+            case 4: L[4] = sub8_pinned(x[3], x[2]); break;
+            case 5: L[5] = add8_pinned(x[1], x[0]); break;
+            case 6: L[6] = sub8_pinned(x[0], x[1]); break;
+            default: L[7] = add8_pinned(x[3], x[2]); break;
         }
     } else {
         // the plain copies (lanes 4..7) first: they free the component registers for the next request;
         // T = {g0+g1, g2+g3, g0-g1, g2-g3}
         switch (i) {
-            case 0: L[4] = x[0]; L[5] = x[1]; T[0] = add8(x[0], x[1]); break;
-            case 1: L[6] = x[2]; L[7] = x[3]; T[1] = add8(x[2], x[3]); break;
-            case 2: T[2] = sub8(x[0], x[1]); break;
-            case 3: T[3] = sub8(x[2], x[3]); break;
-            case 4: L[0] = sub8(T[1], T[0]); break;
-            case 5: L[1] = sub8(T[2], T[3]); break;
-            case 6: L[2] = add8(T[2], T[3]); break;
-            default: L[3] = add8(T[0], T[1]); break;
+            case 0: L[4] = x[0]; L[5] = x[1]; T[0] = add8_pinned(x[0], x[1]); break;
+            case 1: L[6] = x[2]; L[7] = x[3]; T[1] = add8_pinned(x[2], x[3]); break;
+            case 2: T[2] = sub8_pinned(x[0], x[1]); break;
+            case 3: T[3] = sub8_pinned(x[2], x[3]); break;
+            case 4: L[0] = sub8_pinned(T[1], T[0]); break;
+            case 5: L[1] = sub8_pinned(T[2], T[3]); break;
+            case 6: L[2] = add8_pinned(T[2], T[3]); break;
+            default: L[3] = add8_pinned(T[0], T[1]); break;
         }
     }
 }
