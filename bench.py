@@ -37,13 +37,14 @@ RESNET = "c5_qresnet50"  # quaternion ResNet-50 forward+backward, N=64, 224x224,
 # what the same counters read for a plain 256 MiB device copy.  Configurations not profiled report null.
 KIB = 1024.0
 MEASURED_TRAFFIC = {
-    ("c2_pw_f32", 8): {"fwd": (67977.4 * 2 + 134848.0) * KIB, "bwd_data": (67929.3 * 2 + 134848.0) * KIB,
-                       "bwd_weights": (200924.6 * 2 + 32768.0) * KIB},
-    ("c3_k3_f32", 8): {"fwd": (144540.2 * 2 + 252797.4) * KIB, "bwd_data": (148207.4 * 2 + 260483.6) * KIB},
-    ("c4_k3_f16_128_28", 16): {"fwd": (83626.8 * 2 + 105457.0) * KIB, "bwd_data": (83626.8 * 2 + 105457.0) * KIB,
-                               "bwd_weights": (179973.6 * 2 + 48384.0) * KIB},
-    ("c4_k3_f16_128_28", 8): {"fwd": (119473.0 * 2 + 105540.2) * KIB, "bwd_data": (119625.7 * 2 + 104716.3) * KIB,
-                              "bwd_weights": (359772.5 * 2 + 32256.0) * KIB},
+    ("c2_pw_f32", 8): {"fwd": (66673.9 * 2 + 131712.0) * KIB, "bwd_data": (66610.1 * 2 + 131712.0) * KIB,
+                       "bwd_weights": (100555.4 * 2 + 32768.0) * KIB},
+    ("c3_k3_f32", 8): {"fwd": (150715.1 * 2 + 244946.0) * KIB, "bwd_data": (161077.9 * 2 + 246386.3) * KIB,
+                       "bwd_weights": (379051.4 * 2 + 32256.0) * KIB},
+    ("c4_k3_f16_128_28", 16): {"fwd": (83632.0 * 2 + 105213.6) * KIB, "bwd_data": (83632.0 * 2 + 105213.6) * KIB,
+                               "bwd_weights": (179991.1 * 2 + 48384.0) * KIB},
+    ("c4_k3_f16_128_28", 8): {"fwd": (119336.1 * 2 + 105641.7) * KIB, "bwd_data": (122965.9 * 2 + 116104.1) * KIB,
+                              "bwd_weights": (360865.7 * 2 + 32256.0) * KIB},
 }
 
 

@@ -180,7 +180,7 @@ struct FwdPlan {
 
 constexpr int LDS_FLOATS_MAX = 16384;  // 64 KiB: two workgroups per CU
 
-static bool plan_forward(const Corr& c, int mode, bool f16mfma, FwdPlan& best) {
+static bool plan_forward(const Corr& c, int mode, bool f16mfma, FwdPlan& best, bool pointwise = false) {
     double best_score = -1.0;
     // fp16 MFMA with filters in LDS: stage activations as aligned pairs when rows are even
     // filters through LDS: 16-product always, 8-product where the chunk staging applies
@@ -229,7 +229,10 @@ static bool plan_forward(const Corr& c, int mode, bool f16mfma, FwdPlan& best) {
                     double score = eff * (0.25 + 0.75 * fill) * (0.9 + 0.1 * halo) * (NTW == 2 ? 1.02 : 1.0);
                     // fp16 MFMA is operand-bandwidth hungry: two column tiles per wave and two filter
                     // sub-tiles per workgroup amortise LDS reads and activation staging (measured)
-                    if (ldsk) score *= (NTW == 2 ? 1.25 : 1.0) * (WCO == 2 ? 1.08 : 1.0);
+                    // (pointwise problems, 16-product: workgroups live for a few blocks only, and two of them
+                    // per CU -- one column tile per wave, two filter sub-tiles -- hide each other's start and end)
+                    if (ldsk && pointwise && mode == 16) score *= (NTW == 1 ? 1.25 : 1.0) * (WCO == 2 ? 1.2 : 1.0);
+                    else if (ldsk) score *= (NTW == 2 ? 1.25 : 1.0) * (WCO == 2 ? 1.08 : 1.0);
                     else if (f16mfma && NTW == 2) score *= 0.8;  // that kernel drops to one workgroup per CU
                     if (score > best_score) {
                         best_score = score;
@@ -308,7 +311,7 @@ static Corr virtual_pointwise(const Corr& c, bool f16mfma, int& pw) {
 // plans the virtual-tap form of a pointwise correlation where it applies and fits, the plain form otherwise
 static bool plan_corr(const Corr& creal, int mode, bool f16mfma, Corr& c, FwdPlan& pl, int& pw) {
     c = virtual_pointwise(creal, f16mfma, pw);
-    if (pw && plan_forward(c, mode, f16mfma, pl) && pl.lds_filters && pl.chunks) return true;
+    if (pw && plan_forward(c, mode, f16mfma, pl, true) && pl.lds_filters && pl.chunks) return true;
     pw = 0;
     c = creal;
     return plan_forward(c, mode, f16mfma, pl);
