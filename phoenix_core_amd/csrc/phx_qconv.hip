@@ -184,10 +184,12 @@ static bool plan_forward(const Corr& c, int mode, bool f16mfma, FwdPlan& best, b
     double best_score = -1.0;
     // fp16 MFMA with filters in LDS: stage activations as aligned pairs when rows are even
     // filters through LDS: 16-product always, 8-product where the chunk staging applies
-    const bool ldsk = f16mfma && c.Kh * c.Kw > 1 && (mode == 16 || c.uw == 1);
-    const bool chunks = ldsk && c.uw == 1;
-    const bool pairs = f16mfma && !chunks && (c.Win % 2 == 0) && c.uw == 1;
-    const bool vstage = !f16mfma && c.uw == 1;
+    // the vector staging forms copy runs of stored positions: no zero insertion along either axis
+    const bool dense_window = c.uh == 1 && c.uw == 1;
+    const bool ldsk = f16mfma && c.Kh * c.Kw > 1 && (mode == 16 || dense_window);
+    const bool chunks = ldsk && dense_window;
+    const bool pairs = f16mfma && !chunks && (c.Win % 2 == 0) && dense_window;
+    const bool vstage = !f16mfma && dense_window;
     best.pairs = pairs; best.chunks = chunks; best.vstage = vstage;
     const int wcos[3] = {1, 2, 4};
     // PHX_TUNE_TILE="wco,ntw" pins the workgroup shape (kernel tuning experiments)

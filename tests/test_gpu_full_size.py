@@ -1,0 +1,132 @@
+"""GPU parity at the benchmark's full sizes, where the CPU oracle cannot run the whole problem in seconds.
+
+Three size-independent checks per configuration, all through the C ABI on the full-size tensors:
+
+* crop parity: forward and input gradient are local, so a corner window of the first / last images of the
+  full-size result must equal the oracle's result on the cropped problem (same padding on the window's own
+  borders, interior pixels compared);
+* sparse-gradient parity: the filter gradient is a sum over all images and pixels; with an output gradient
+  that is zero outside a corner window of two images it must equal the oracle's filter gradient of the
+  cropped problem, while the kernel still walks the full-size reduction;
+* adjoint identities on dense random tensors: <conv(x, w), g> = <x, dgrad(g, w)> = <w, wgrad(x, g)>
+  (the backward passes are the transposes of the forward map), inner products accumulated in fp64.
+
+Tolerances: crops as in test_gpu_parity.py (1e-4 fp32, 2e-2 fp16, max-norm and L2, against the fp64 closed
+form); inner products within 1e-4 (fp32) / 2e-3 (fp16) of ||a||*||b||."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import phoenix_core_amd as phx
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.float32: 1e-4, torch.float16: 2e-2}
+DOT_TOL = {torch.float32: 1e-4, torch.float16: 2e-3}
+
+# name, n, ci, co, h, w, k, padding, dtype, policy  (BASELINE configurations C2, C3, C4)
+FULL = [
+    ("c2_pw_f32", 32, 64, 64, 56, 56, 1, "VALID", torch.float32, "fp32"),
+    ("c3_k3_f32", 64, 64, 64, 56, 56, 3, "SAME", torch.float32, "fp32"),
+    ("c4_k3_f16_128_28", 128, 128, 128, 28, 28, 3, "SAME", torch.float16, "full16"),
+    ("c4_k3_f16_256_14", 128, 256, 256, 14, 14, 3, "SAME", torch.float16, "full16"),
+    ("c4_pw_f16_128_28", 128, 128, 128, 28, 28, 1, "VALID", torch.float16, "full16"),
+    ("c4_pw_f16_256_14", 128, 256, 256, 14, 14, 1, "VALID", torch.float16, "backward32"),
+]
+
+
+class Ctx(phx.Context):
+    def __init__(self, mode, policy):
+        env = {"UPSTRIDE_CONV_FP16_POLICY": policy}
+        if mode == 16:
+            env["UPSTRIDE_MEMORY_OPTIMIZED"] = "1"
+        super().__init__(env)
+
+
+def close(got, want, dtype, what):
+    got = got.astype(np.float64)
+    d = np.abs(got - want)
+    e_max = d.max() / max(np.abs(want).max(), 1e-30)
+    e_l2 = np.sqrt((d ** 2).sum()) / max(np.sqrt((want ** 2).sum()), 1e-30)
+    assert np.isfinite(got).all(), what
+    assert e_max <= TOL[dtype] and e_l2 <= TOL[dtype], "%s: rel max %.3e, rel l2 %.3e" % (what, e_max, e_l2)
+
+
+def rows_of(images, n):
+    """Batch rows of the given images in the component-major layout [4n, ...]."""
+    return [p * n + i for p in range(4) for i in images]
+
+
+def dot(a, b):
+    return (a.double() * b.double()).sum().item()
+
+
+def norm(a):
+    return a.double().norm().item()
+
+
+@pytest.mark.parametrize("mode", [8, 16])
+@pytest.mark.parametrize("cfg", FULL, ids=[c[0] for c in FULL])
+def test_full_size(cfg, mode):
+    name, n, ci, co, h, w, k, padding, dtype, policy = cfg
+    print("config", name, "mode", mode, flush=True)
+    scale = 1.0 if dtype == torch.float32 else 0.5
+    gen = torch.Generator(device="cuda").manual_seed(0x5EED + len(name) + mode)
+    x = (scale * torch.randn(4 * n, ci, h, w, device="cuda", generator=gen)).to(dtype)
+    wt = (scale * np.sqrt(2.0 / (ci * k * k)) * torch.randn(4, co, ci, k, k, device="cuda", generator=gen)).to(dtype)
+    g = (scale * torch.randn(4 * n, co, h, w, device="cuda", generator=gen)).to(dtype)
+    desc = phx.Conv2DDescriptor(x.shape, wt.shape, 1, 1, padding, dtype=dtype, context=Ctx(mode, policy))
+    assert desc.output_shape == tuple(g.shape)
+    y = phx.conv2d_fwd(x, wt, None, desc)
+    dw, dx = phx.conv2d_bwd(x, wt, g, desc)
+
+    # adjoint identities on the dense tensors
+    yg, xdx, wdw = dot(y, g), dot(x, dx), dot(wt, dw)
+    tol = DOT_TOL[dtype]
+    assert abs(yg - xdx) <= tol * norm(y) * norm(g), (yg, xdx)
+    assert abs(yg - wdw) <= tol * norm(y) * norm(g), (yg, wdw)
+
+    # crop parity of forward / input gradient: top-left window of the first two images, bottom-right window
+    # of the last two; the outermost ring of the window next to the cut is left out (its halo is missing)
+    c = min(h, 12)
+    halo = (k - 1) // 2
+    w64 = wt.cpu().numpy().astype(np.float64)
+    for images, (h0, w0) in (((0, 1), (0, 0)), ((n - 2, n - 1), (h - c, w - c))):
+        rows = rows_of(images, n)
+        xc = x[rows][:, :, h0:h0 + c, w0:w0 + c].cpu().numpy().astype(np.float64)
+        gc = g[rows][:, :, h0:h0 + c, w0:w0 + c].cpu().numpy().astype(np.float64)
+        geom = oracle.make_geom(2, ci, co, c, c, k, k, 1, 1, padding)
+        want_y = oracle.conv2d_fwd(geom, xc, w64, None, "hamilton")
+        _, want_dx = oracle.conv2d_bwd(geom, xc, w64, gc, "hamilton")
+        # keep the pixels whose window lies inside the crop or in the image's true padding
+        lo_h = 0 if h0 == 0 else halo
+        hi_h = c if h0 + c == h and h0 != 0 else c - halo
+        lo_w = 0 if w0 == 0 else halo
+        hi_w = c if w0 + c == w and w0 != 0 else c - halo
+        if c == h:  # the crop is the whole plane
+            lo_h, hi_h, lo_w, hi_w = 0, c, 0, c
+        got_y = y[rows][:, :, h0:h0 + c, w0:w0 + c].cpu().numpy()
+        got_dx = dx[rows][:, :, h0:h0 + c, w0:w0 + c].cpu().numpy()
+        sl = (slice(None), slice(None), slice(lo_h, hi_h), slice(lo_w, hi_w))
+        close(got_y[sl], want_y[sl], dtype, "fwd crop %s" % (images,))
+        close(got_dx[sl], want_dx[sl], dtype, "dgrad crop %s" % (images,))
+
+    # sparse-gradient parity of the filter gradient: gradient confined to a window of two images; the window
+    # of x that can meet it is the same window grown by the halo, so crop x with the halo and use explicit
+    # padding for what lies outside the image
+    images, h0, w0 = (1, n - 1), h - c, 0
+    rows = rows_of(images, n)
+    gs = torch.zeros_like(g)
+    gs[rows, :, h0:h0 + c, w0:w0 + c] = g[rows][:, :, h0:h0 + c, w0:w0 + c]
+    dws, _ = phx.conv2d_bwd(x, wt, gs, phx.Conv2DDescriptor(x.shape, wt.shape, 1, 1, padding, dtype=dtype,
+                                                            context=Ctx(mode, policy), require_input_grad=False))
+    top, left = max(h0 - halo, 0), max(w0 - halo, 0)
+    bot, right = min(h0 + c + halo, h), min(w0 + c + halo, w)
+    xc = x[rows][:, :, top:bot, left:right].cpu().numpy().astype(np.float64)
+    gc = g[rows][:, :, h0:h0 + c, w0:w0 + c].cpu().numpy().astype(np.float64)
+    pads = (halo - (h0 - top), halo - (w0 - left), halo - (bot - (h0 + c)), halo - (right - (w0 + c)))
+    geom = oracle.make_geom(2, ci, co, bot - top, right - left, k, k, 1, 1, pads)
+    assert (geom.ho, geom.wo) == (c, c)
+    want_dw, _ = oracle.conv2d_bwd(geom, xc, w64, gc, "hamilton", need_dx=False)
+    close(dws.cpu().numpy(), want_dw, dtype, "wgrad of a sparse gradient")

@@ -65,6 +65,7 @@ CONV_CASES = [
     ("k3_s2_c4", 2, 4, 8, 15, 13, 3, 3, 2, 1, "SAME"),       # few input channels, stride 2: space-to-depth path
     ("k5_s2_valid", 1, 2, 8, 17, 16, 5, 5, 2, 1, "VALID"),
     ("k3_dil2", 1, 4, 6, 12, 12, 3, 3, 1, 2, "SAME"),
+    ("k32_s21", 2, 8, 8, 13, 19, 3, 2, (2, 1), 1, "SAME"),    # stride along H only: zero insertion in rows, dense columns
     ("k32_asym", 1, 4, 4, 8, 9, 3, 2, (1, 2), (2, 1), (2, 0, 1, 3)),
     ("single_pixel", 4, 6, 6, 1, 1, 1, 1, 1, 1, "VALID"),
     ("co_gt_128", 1, 8, 136, 7, 7, 1, 1, 1, 1, "VALID"),
@@ -224,7 +225,7 @@ def test_empty_input_is_a_no_op_and_zeroes_dw():
 
 
 FP16_CASES = [c for c in CONV_CASES if c[0] in ("pw_64", "pw_ragged", "pw_7x7img", "k3_same", "k3_same_56", "k3_ragged",
-                                                "k3_valid", "k3_s2", "pw_s2", "k7_s2", "k3_s2_c4", "k5_s2_valid", "k3_dil2", "k32_asym",
+                                                "k3_valid", "k3_s2", "pw_s2", "k7_s2", "k3_s2_c4", "k5_s2_valid", "k3_dil2", "k32_s21", "k32_asym",
                                                 "co_gt_128")] + [
     ("k3_s3", 2, 8, 8, 13, 13, 3, 3, 3, 1, "SAME"),
     ("k3_128_28", 2, 128, 128, 28, 28, 3, 3, 1, 1, "SAME"),
