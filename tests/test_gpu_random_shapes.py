@@ -104,3 +104,31 @@ def test_random_geometry_fp16(seed):
     policy = ["full16", "backward32", "fp32"][seed % 3]
     print("case", cfg, policy, flush=True)
     run_case(cfg, r, torch.float16, policy)
+
+
+@pytest.mark.parametrize("seed", range(48))
+def test_random_dense(seed):
+    """Quaternion Dense on random batch / feature counts, both tensor types, every mode and policy, in fp64
+    against the oracle's generic path."""
+    r = np.random.default_rng(9000 + seed)
+    n, ni, no = int(r.integers(1, 80)), int(r.integers(1, 200)), int(r.integers(1, 200))
+    dtype = [torch.float32, torch.float16][seed % 2]
+    mode, policy, bias = int(r.choice([8, 16])), str(r.choice(["full16", "backward32", "fp32"])), bool(r.random() < 0.5)
+    print("dense", n, ni, no, dtype, mode, policy, bias, flush=True)
+    npdt = np.float32 if dtype == torch.float32 else np.float16
+    scale = 1.0 if dtype == torch.float32 else 0.5
+    lim = np.sqrt(6.0 / (ni + no))
+    x = (scale * r.standard_normal((4 * n, ni))).astype(npdt)
+    w = r.uniform(-lim, lim, (4, ni, no)).astype(npdt)
+    b = (scale * r.standard_normal((4, no))).astype(npdt)
+    gr = (scale * r.standard_normal((4 * n, no))).astype(npdt)
+    desc = phx.DenseDescriptor(x.shape, w.shape, use_bias=bias, dtype=dtype, context=Ctx(mode, policy))
+    xd, wd, bd, gd = (torch.from_numpy(a).cuda() for a in (x, w, b, gr))
+    y = phx.dense_fwd(xd, wd, bd if bias else None, desc)
+    dw, dx = phx.dense_bwd(xd, wd, gd, desc)
+    x64, w64, b64, g64 = (a.astype(np.float64) for a in (x, w, b, gr))
+    want_y = oracle.dense_fwd(x64, w64, b64 if bias else None, "generic")
+    want_dw, want_dx = oracle.dense_bwd(x64, w64, g64, "generic")
+    close(y.cpu().numpy(), want_y, dtype, "dense fwd")
+    close(dx.cpu().numpy(), want_dx, dtype, "dense dgrad")
+    close(dw.cpu().numpy(), want_dw, dtype, "dense wgrad")
