@@ -165,6 +165,7 @@ static Corr corr_dgrad(const Problem& p) {
 
 struct FwdPlan {
     int WCO, NTW, BN;
+    int kmode;               // product formulation the kernel runs in (see plan_corr)
     int CK, P2LOG;           // channels per chunk and log2 staging positions of the kernel variant
     bool lds_filters;        // fp16 MFMA, 16-product, more than one tap: filters go through LDS
     int ngroups;             // tap groups per chunk in that case
@@ -311,11 +312,22 @@ static Corr virtual_pointwise(const Corr& c, bool f16mfma, int& pw) {
 }
 
 // plans the virtual-tap form of a pointwise correlation where it applies and fits, the plain form otherwise
+// pl.kmode is the product formulation the kernel runs in.  It is the mode asked for, except for pointwise
+// problems on fp16 matrix cores in 8-product mode: their workgroups live for two or three tap groups, where
+// the factorized kernel (one workgroup per CU, lane arithmetic in front of every block) loses to the
+// 16-product kernel with two workgroups per CU (128->128@28^2: 412 against 592 TFLOP/s real-equivalent; the
+// 16<->64-channel layers of a ResNet 37-75 against 64-112).  The 8-product mode means "prefer speed"
+// (src/backend/backend.hpp:36-66), so those problems run on the 16-product kernel; PHX_TUNE_PW8 keeps the
+// factorized one (tests exercise it).
 static bool plan_corr(const Corr& creal, int mode, bool f16mfma, Corr& c, FwdPlan& pl, int& pw) {
     c = virtual_pointwise(creal, f16mfma, pw);
-    if (pw && plan_forward(c, mode, f16mfma, pl, true) && pl.lds_filters && pl.chunks) return true;
+    if (pw) {
+        pl.kmode = (mode == 8 && !getenv("PHX_TUNE_PW8")) ? 16 : mode;
+        if (plan_forward(c, pl.kmode, f16mfma, pl, true) && pl.lds_filters && pl.chunks) return true;
+    }
     pw = 0;
     c = creal;
+    pl.kmode = mode;
     return plan_forward(c, mode, f16mfma, pl);
 }
 
@@ -329,7 +341,7 @@ static int run_corr(const Problem& p, const Corr& creal, int map, hipStream_t st
     if (ws_bytes < pl.wpk_bytes || !ws) return PHX_ERR_WORKSPACE;
 
     FwdVariant v;
-    v.half_storage = p.dtype == PHX_F16; v.f16_mfma = f16; v.mode = p.mode; v.map = map;
+    v.half_storage = p.dtype == PHX_F16; v.f16_mfma = f16; v.mode = pl.kmode; v.map = map;
     v.WCO = pl.WCO; v.NTW = pl.NTW; v.CK = pl.CK; v.P2LOG = pl.P2LOG; v.wgs = pl.wgs; v.lds_bytes = pl.lds_bytes;
     v.lds_filters = pl.lds_filters; v.ngroups = pl.ngroups; v.pairs = pl.pairs; v.chunks = pl.chunks; v.pw = pw; v.vstage = pl.vstage;
 
@@ -369,7 +381,7 @@ static int run_corr(const Problem& p, const Corr& creal, int map, hipStream_t st
     if (rc != 0) return PHX_ERR_NOT_SUPPORTED;
     PHX_HIP(hipGetLastError());
     snprintf(g_name_buf, sizeof(g_name_buf), "%sqconv_%s_%smfma%s_p%d_%s_wco%d_ntw%d_ck%d_tile%dx%dx%d", g_name_prefix,
-             map == MAP_FWD ? "fwd" : "dgrad", f16 ? "f16" : "f32", pl.lds_filters ? (pw ? "ldspw" : pl.chunks ? "ldsc" : "lds") : "", p.mode, p.dtype == PHX_F32 ? "f32" : "f16", pl.WCO,
+             map == MAP_FWD ? "fwd" : "dgrad", f16 ? "f16" : "f32", pl.lds_filters ? (pw ? "ldspw" : pl.chunks ? "ldsc" : "lds") : "", pl.kmode, p.dtype == PHX_F32 ? "f32" : "f16", pl.WCO,
              pl.NTW, pl.CK, pl.NB, pl.TH, pl.TW);
     g_last_kernel = g_name_buf;
     return PHX_OK;
@@ -382,6 +394,7 @@ struct WgPlan {
     int TPW, NB, TH, TW, KP, KPp, HPp, HPx, HTH, HTWmax;
     int tiles_n, tiles_h, tiles_w, co_tiles, ci_tiles, CoP, CiP, groups_per_row, Z;
     int MT, NT;  // fp16 kernel: 32*MT x 32*NT channel tile
+    int kmode;   // fp16 kernel: product formulation the kernel runs in (see wgrad_f16_formulation)
     bool vec;    // fp32 kernel: windows staged as groups of 4 positions
     int SW, cpr, nchunks, ntiles;  // fp16 kernel: stride along W, 8-pixel chunks per output row / in total, pixel tiles
     size_t lds_bytes, partial_bytes;
@@ -442,10 +455,22 @@ static bool plan_wgrad_f32(const Problem& p, WgPlan& best) {
 }
 
 // fp16-MFMA kernel: 32*MT x 32*NT channel tiles; reduction over 8-pixel chunks of the output rows, 8 chunks per tile
+// On fp16 matrix cores the filter gradient is faster in its 16-product form whatever the product mode asks
+// for: the factorized form halves the matrix instructions but must form lanes of BOTH operands with packed
+// vector adds in front of every block (80 vector instructions per 8 MFMAs), and its eight accumulator sets
+// leave no room to share a staged gradient tile between three taps (measured 128->128@28^2 3x3: 1016 against
+// 794 TFLOP/s real-equivalent, pointwise 780 against 700).  UPSTRIDE_MEMORY_OPTIMIZED unset means "prefer
+// speed" (src/backend/backend.hpp:36-66), so the 8-product mode runs this pass on the 16-product kernel;
+// PHX_TUNE_WG8 keeps the factorized kernel (tests exercise it).
+static int wgrad_f16_formulation(const Problem& p) {
+    return (p.mode == 8 && !getenv("PHX_TUNE_WG8")) ? 16 : p.mode;
+}
+
 static bool plan_wgrad_f16(const Problem& p, WgPlan& best) {
     best = WgPlan{};
     best.SW = p.sw;
-    best.TPW = (p.mode == 16 && p.kw % 3 == 0 && p.sw == 1 && p.dw == 1) ? 3 : 1;
+    best.kmode = wgrad_f16_formulation(p);
+    best.TPW = (best.kmode == 16 && p.kw % 3 == 0 && p.sw == 1 && p.dw == 1) ? 3 : 1;
     best.MT = p.co > 32 ? 2 : 1;
     best.NT = p.ci > 32 ? 2 : 1;
     if (const char* e = getenv("PHX_TUNE_WG")) sscanf(e, "%d,%d", &best.MT, &best.NT);
@@ -506,7 +531,7 @@ static int run_wgrad(const Problem& p, hipStream_t st, const void* x, const void
     {
         KernelTimer timer(st);
         if (f16) {
-            if (launch_wgrad_f16(p.mode, pl.MT, pl.NT, pl.TPW, pl.SW, a, nblocks, pl.lds_bytes, st) != 0)
+            if (launch_wgrad_f16(pl.kmode, pl.MT, pl.NT, pl.TPW, pl.SW, a, nblocks, pl.lds_bytes, st) != 0)
                 return PHX_ERR_RUNTIME;
         } else {
             launch_wgrad_f32(half_storage, pl.vec, p.mode, a, dim3(nblocks), pl.lds_bytes, st);
@@ -522,7 +547,7 @@ static int run_wgrad(const Problem& p, hipStream_t st, const void* x, const void
     launch_reduce_wgrad(half_storage, r, blocks, st);
     PHX_HIP(hipGetLastError());
     if (f16)
-        snprintf(g_name_buf, sizeof(g_name_buf), "%sqconv_wgrad_f16mfma_p%d_f16_ch%dx%d_taps%d_sw%d_z%d", g_name_prefix, p.mode, 32 * pl.MT,
+        snprintf(g_name_buf, sizeof(g_name_buf), "%sqconv_wgrad_f16mfma_p%d_f16_ch%dx%d_taps%d_sw%d_z%d", g_name_prefix, pl.kmode, 32 * pl.MT,
                  32 * pl.NT, pl.TPW, pl.SW, pl.Z);
     else
         snprintf(g_name_buf, sizeof(g_name_buf), "%sqconv_wgrad_f32mfma%s_p%d_%s_tile%dx%dx%d_z%d", g_name_prefix, pl.vec ? "v" : "", p.mode,

@@ -268,6 +268,54 @@ def test_conv_fp16(case, mode, policy):
     assert_close(dw.cpu().numpy(), want_dw, dtype, "wgrad " + name)
 
 
+@pytest.mark.parametrize("case", [c for c in FP16_CASES if c[0] in ("pw_64", "pw_ragged", "k3_same", "k3_ragged", "k3_s2",
+                                                                       "k7_s2", "k32_asym", "k3_128_28", "pw_256_14")],
+                         ids=lambda c: c[0])
+def test_factorized_filter_gradient_on_fp16_matrix_cores(case, monkeypatch):
+    """In 8-product mode the fp16 filter gradient runs on the 16-product kernel by default (it is the faster
+    one there); PHX_TUNE_WG8 selects the factorized 8-lane kernel, which must meet the same tolerance."""
+    name, n, ci, co, h, w, kh, kw, stride, dilation, padding = case
+    dtype = torch.float16
+    g, x, wt, b, gr = make_inputs(hash(name) % 1000 + 3, n, ci, co, h, w, kh, kw, stride, dilation, padding, dtype, 0.5)
+    xd, wd, gd = (torch.from_numpy(a).cuda() for a in (x, wt, gr))
+    desc = phx.Conv2DDescriptor(x.shape, wt.shape, stride, dilation, padding, dtype=dtype, context=Ctx(8, "full16"),
+                                require_input_grad=False)
+    dw16, _ = phx.conv2d_bwd(xd, wd, gd, desc)
+    assert "f16mfma_p16" in capi.last_kernel_name()
+    monkeypatch.setenv("PHX_TUNE_WG8", "1")
+    dw8, _ = phx.conv2d_bwd(xd, wd, gd, desc)
+    assert "f16mfma_p8" in capi.last_kernel_name()
+    want_dw, _ = oracle.conv2d_bwd(g, x.astype(np.float64), wt.astype(np.float64), gr.astype(np.float64), "hamilton",
+                                   need_dx=False)
+    assert_close(dw8.cpu().numpy(), want_dw, dtype, "8-product wgrad " + name)
+    assert_close(dw16.cpu().numpy(), want_dw, dtype, "16-product wgrad " + name)
+
+
+@pytest.mark.parametrize("case", [c for c in FP16_CASES if c[0] in ("pw_64", "pw_ragged", "pw_7x7img", "pw_256_14", "co_gt_128")],
+                         ids=lambda c: c[0])
+def test_factorized_pointwise_on_fp16_matrix_cores(case, monkeypatch):
+    """In 8-product mode pointwise fp16 problems run on the 16-product kernel by default (two workgroups per CU
+    beat the factorized kernel there); PHX_TUNE_PW8 selects the factorized kernel, same tolerance."""
+    name, n, ci, co, h, w, kh, kw, stride, dilation, padding = case
+    dtype = torch.float16
+    g, x, wt, b, gr = make_inputs(hash(name) % 1000 + 4, n, ci, co, h, w, kh, kw, stride, dilation, padding, dtype, 0.5)
+    xd, wd, bd, gd = (torch.from_numpy(a).cuda() for a in (x, wt, b, gr))
+    desc = phx.Conv2DDescriptor(x.shape, wt.shape, stride, dilation, padding, use_bias=True, dtype=dtype,
+                                context=Ctx(8, "full16"))
+    x64, w64, b64, g64 = (a.astype(np.float64) for a in (x, wt, b, gr))
+    want_y = oracle.conv2d_fwd(g, x64, w64, b64, "hamilton")
+    _, want_dx = oracle.conv2d_bwd(g, x64, w64, g64, "hamilton")
+    for forced, tag in ((False, "ldspw_p16"), (True, "ldspw_p8")):
+        if forced:
+            monkeypatch.setenv("PHX_TUNE_PW8", "1")
+        y = phx.conv2d_fwd(xd, wd, bd, desc)
+        assert tag in capi.last_kernel_name(), capi.last_kernel_name()
+        _, dx = phx.conv2d_bwd(xd, wd, gd, desc)
+        assert tag in capi.last_kernel_name(), capi.last_kernel_name()
+        assert_close(y.cpu().numpy(), want_y, dtype, "fwd " + tag)
+        assert_close(dx.cpu().numpy(), want_dx, dtype, "dgrad " + tag)
+
+
 @pytest.mark.parametrize("policy", ["full16", "fp32"])
 @pytest.mark.parametrize("mode", [16, 8])
 def test_dense_fp16(mode, policy):
