@@ -40,7 +40,11 @@ enum phx_filter_layout { PHX_OIHW = 0, PHX_OHWI = 1 };
 /* Which Hamilton-product formulation runs.
  * Mirrors Context::preferSpeedToMemory() (src/backend/backend.hpp:58): the reference's default is
  * the factorized 8-product path (src/conv2d.hpp:167-234), UPSTRIDE_MEMORY_OPTIMIZED=1 selects the
- * 16-product path (src/conv2d.hpp:237-275). */
+ * 16-product path (src/conv2d.hpp:237-275).
+ * PHX_PRODUCT_16 always runs the 16-product kernels.  PHX_PRODUCT_8 is the "prefer speed" setting: the
+ * factorized 8-product kernels run wherever they are the faster ones (every fp32 pass; fp16 forward and
+ * input gradient with more than one filter tap); the fp16-MFMA filter gradient and fp16-MFMA pointwise
+ * passes are faster in 16-product form and run that way (phx_last_kernel_name() tells which ran). */
 enum phx_product_mode { PHX_PRODUCT_16 = 16, PHX_PRODUCT_8 = 8 };
 
 /* UPSTRIDE_CONV_FP16_POLICY (src/backend/backend.cc:35-42, src/backend/backend.hpp:60-66).
