@@ -699,15 +699,20 @@ __global__ void __launch_bounds__(WG_THREADS) pack_filters_f16_lds_kernel(const 
     const PackArgs& P = A.base;
     constexpr int TG = F16_TG;
     constexpr int NW = (MODE == 16) ? 4 : 8;
+    // 16-product: one thread per 16-byte vector (one component).  8-product: one thread per group of the
+    // eight lane vectors of a (tap, sub-tile, lane) slot, which all derive from the same 8 x 4 filter values.
+    constexpr int PER = (MODE == 16) ? 1 : NW;
     const int taps = A.pw ? A.pw : P.Kh * P.Kw;
-    // index = ((((tile*nchunks + chunk)*ngroups + g)*TG + tg)*WCO + wco)*NW + r)*64 + lane
-    const long total = (long)P.row_tiles * P.nchunks * A.ngroups * TG * A.WCO * NW * 64;
+    // vector index = ((((tile*nchunks + chunk)*ngroups + g)*TG + tg)*WCO + wco)*NW + r)*64 + lane
+    const long total = (long)P.row_tiles * P.nchunks * A.ngroups * TG * A.WCO * (NW / PER) * 64;
     const _Float16* w = static_cast<const _Float16*>(P.w);
     f16x8* outv = reinterpret_cast<f16x8*>(P.out);
     for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
         const int lane = idx & 63;
         long s = idx >> 6;
-        const int r = s % NW; s /= NW;
+        int r = 0;
+        if constexpr (PER == 1) { r = s % NW; s /= NW; }
+        const long slot = s;  // (tile, chunk, g, tg, wco)
         const int wco = s % A.WCO; s /= A.WCO;
         const int tg = s % TG; s /= TG;
         const int g = s % A.ngroups; s /= A.ngroups;
@@ -715,9 +720,11 @@ __global__ void __launch_bounds__(WG_THREADS) pack_filters_f16_lds_kernel(const 
         const int tile = s / P.nchunks;
         const int tap = g * TG + tg;
         const int row = (tile * A.WCO + wco) * 32 + (lane & 31);
-        f16x8 vec;
+        f16x8 vec[PER];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) vec[i] = (_Float16)0;
+        for (int q = 0; q < PER; ++q)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) vec[q][i] = (_Float16)0;
         if (tap < taps && row < P.rows) {
             int kh = tap / P.Kw, kw = tap - kh * P.Kw;
             if (MAP == MAP_DGRAD) { kh = P.Kh - 1 - kh; kw = P.Kw - 1 - kw; }
@@ -732,19 +739,25 @@ __global__ void __launch_bounds__(WG_THREADS) pack_filters_f16_lds_kernel(const 
                     const long off = o * P.so + in * P.si + kh * P.skh + kw * P.skw;
                     if constexpr (MODE == 16) {
                         const float sgn = (MAP == MAP_DGRAD && r > 0) ? -1.f : 1.f;  // conjugate
-                        vec[i] = (_Float16)(sgn * (float)w[r * P.wcs + off]);
+                        vec[0][i] = (_Float16)(sgn * (float)w[r * P.wcs + off]);
                     } else {
                         float wv[4], R[8];
 #pragma unroll
                         for (int c = 0; c < 4; ++c) wv[c] = (float)w[c * P.wcs + off];
                         lanes_right(wv, R);  // formed in fp32, rounded once
                         // input gradient: the kernel forms the gradient lanes 0..3 without their factor 1/2
-                        vec[i] = (_Float16)((MAP == MAP_DGRAD && r < 4) ? 0.5f * R[r] : R[r]);
+#pragma unroll
+                        for (int q = 0; q < 8; ++q) vec[q][i] = (_Float16)((MAP == MAP_DGRAD && q < 4) ? 0.5f * R[q] : R[q]);
                     }
                 }
             }
         }
-        outv[idx] = vec;
+        if constexpr (PER == 1) {
+            outv[idx] = vec[0];
+        } else {
+#pragma unroll
+            for (int q = 0; q < PER; ++q) outv[(slot * NW + q) * 64 + lane] = vec[q];
+        }
     }
 }
 

@@ -351,7 +351,8 @@ static int run_corr(const Problem& p, const Corr& creal, int map, hipStream_t st
     pa.Co = p.co; pa.Ci = p.ci; pa.Kh = p.kh; pa.Kw = p.kw;
     pa.rows = c.Cout; pa.red = creal.Cin; pa.row_tiles = pl.co_tiles * pl.WCO;
     pa.nchunks = f16 ? pl.nchunks : pl.nchunks * (pl.CK / F32_CK);
-    const long pack_items = pl.lds_filters ? (long)(pl.wpk_bytes / 16)
+    // (LDS images: one thread per 16-byte vector, in 8-product form one thread per eight lane vectors)
+    const long pack_items = pl.lds_filters ? (long)(pl.wpk_bytes / 16) / (pl.kmode == 8 ? 8 : 1)
                                             : (long)pa.row_tiles * pa.nchunks * p.kh * p.kw * (f16 ? 1 : 4) * 64;
     if (pl.lds_filters) pa.row_tiles = pl.co_tiles;  // packed per workgroup tile of WCO*32 channels
     const int pack_blocks = (int)std::min<long>((pack_items + WG_THREADS - 1) / WG_THREADS, 4096);
