@@ -66,6 +66,8 @@ def parse():
                     help="product formulation; 0 = from UPSTRIDE_MEMORY_OPTIMIZED like the reference (default 8)")
     ap.add_argument("--policy", default=None, help="override UPSTRIDE_CONV_FP16_POLICY for fp16 workloads")
     ap.add_argument("--batch", type=int, default=64, help="images per step of the ResNet workload")
+    ap.add_argument("--torch-bn", action="store_true",
+                    help="ResNet workload: torch.nn.BatchNorm2d + ReLU (MIOpen) instead of the library's batch-norm kernels")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch a plain 256 MiB device copy (untimed), the yardstick for HBM byte counters")
@@ -147,7 +149,7 @@ def bench_resnet(args):
     n = args.batch
     dev = torch.device("cuda:0")
     torch.manual_seed(0x5EED + 5)
-    model = phx.QResNet50(1000, dtype=torch.float16, context=ctx).to(dev).train()
+    model = phx.QResNet50(1000, dtype=torch.float16, context=ctx, fused_bn=not args.torch_bn).to(dev).train()
     images = torch.randn(n, 3, 224, 224, device=dev).half()
     labels = torch.randint(0, 1000, (n,), device=dev)
 
@@ -179,9 +181,11 @@ def bench_resnet(args):
         "vs_baseline": None, "dtype": "f16", "data": "synthetic",
         "config": {"workload": "%s: quaternion ResNet-50 forward+backward (no optimizer step, as the metric names), "
                                "N=%d real images (4N=%d quaternion rows after the real-input stem), 224x224, 53 quaternion convs + "
-                               "quaternion dense head; batch-norm, "
-                               "ReLU, pooling and cross-entropy by PyTorch" % (RESNET, n, 4 * n),
-                   "product_mode": mode, "fp16_policy": policy},
+                               "quaternion dense head; batch-norm (with the ReLU behind it) by %s, residual add, "
+                               "pooling and cross-entropy by PyTorch"
+                               % (RESNET, n, 4 * n, "torch.nn.BatchNorm2d (MIOpen)" if args.torch_bn else
+                                  "the library's streaming kernels (include/phx_bn.h)"),
+                   "product_mode": mode, "fp16_policy": policy, "batch_norm": "torch" if args.torch_bn else "library"},
         "real_equiv_tflops": 3 * fwd_flops / (ms_per_step * 1e-3) / 1e12,
         "quaternion_kernel_ms_per_step": conv_ms, "loss": float(loss.detach()),
     }

@@ -27,6 +27,15 @@ EXPORTS = (
 )
 
 
+# every symbol include/phx_bn.h declares (batch normalisation for the ResNet harness)
+EXPORTS_BN = ("phx_bn_workspace_bytes", "phx_bn_fwd_train", "phx_bn_bwd")
+
+
+class BnDesc(ctypes.Structure):
+    _fields_ = [("dtype", ctypes.c_int32), ("rows", ctypes.c_int32), ("c", ctypes.c_int32), ("hw", ctypes.c_int32),
+                ("eps", ctypes.c_float), ("momentum", ctypes.c_float), ("relu", ctypes.c_int32)]
+
+
 class QConvDesc(ctypes.Structure):
     _fields_ = [(k, ctypes.c_int32) for k in (
         "dtype", "n", "ci", "co", "h", "w", "kh", "kw", "stride_h", "stride_w", "dilation_h", "dilation_w",
@@ -70,6 +79,11 @@ def lib():
         L.phx_qdense_fwd.argtypes = [dd, vp, vp, vp, vp, vp, vp, sz]
         L.phx_qdense_bwd_data.argtypes = [dd, vp, vp, vp, vp, vp, sz]
         L.phx_qdense_bwd_weights.argtypes = [dd, vp, vp, vp, vp, vp, sz]
+        bd = ctypes.POINTER(BnDesc)
+        L.phx_bn_workspace_bytes.restype = sz
+        L.phx_bn_workspace_bytes.argtypes = [bd]
+        L.phx_bn_fwd_train.argtypes = [bd, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, sz]
+        L.phx_bn_bwd.argtypes = [bd, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, sz]
         L.phx_device_count.argtypes = [i32p]
         L.phx_device_malloc.argtypes = [ctypes.POINTER(vp), sz]
         L.phx_device_free.argtypes = [vp]

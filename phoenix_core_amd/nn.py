@@ -113,22 +113,67 @@ class QLinear(nn.Module):
         return _QLinearFn.apply(x.contiguous(), self.weight, self.bias, fwd, bwd)
 
 
+class _QBatchNormFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, gamma, beta, running_mean, running_var, eps, momentum, relu):
+        y, mean, invstd = ops.batch_norm_fwd(x, gamma, beta, running_mean, running_var, eps, momentum, relu)
+        ctx.save_for_backward(x, gamma, beta, mean, invstd)
+        ctx.eps, ctx.relu = eps, relu
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, gamma, beta, mean, invstd = ctx.saved_tensors
+        dx, dgamma, dbeta = ops.batch_norm_bwd(x, dy.contiguous(), gamma, beta, mean, invstd, ctx.eps, ctx.relu)
+        return dx, dgamma, dbeta, None, None, None, None, None
+
+
+class QBatchNorm2d(nn.Module):
+    """torch.nn.BatchNorm2d semantics on [4N, C, H, W] (the four components of a quaternion channel share the
+    statistics of their channel), optionally followed by ReLU, on the library's streaming kernels in
+    training mode: a channel is spread over many workgroups, where one-workgroup-per-channel library kernels
+    leave a 16-channel layer on 16 of 256 CUs.  Parameters and statistics are fp32 whatever the tensor type.
+    Evaluation mode uses torch.nn.functional.batch_norm with the running statistics."""
+
+    def __init__(self, num_features, eps=1e-5, momentum=0.1, relu=False):
+        super().__init__()
+        self.eps, self.momentum, self.relu = eps, momentum, relu
+        self.weight = nn.Parameter(torch.ones(num_features))
+        self.bias = nn.Parameter(torch.zeros(num_features))
+        self.register_buffer("running_mean", torch.zeros(num_features))
+        self.register_buffer("running_var", torch.ones(num_features))
+
+    def forward(self, x):
+        if self.training:
+            return _QBatchNormFn.apply(x.contiguous(), self.weight, self.bias, self.running_mean, self.running_var,
+                                       self.eps, self.momentum, self.relu)
+        y = nn.functional.batch_norm(x, self.running_mean, self.running_var, self.weight, self.bias, False, 0.0, self.eps)
+        return torch.relu(y) if self.relu else y
+
+
 class _Bottleneck(nn.Module):
-    def __init__(self, cin, width, cout, stride, dtype, context):
+    def __init__(self, cin, width, cout, stride, dtype, context, fused_bn):
         super().__init__()
         mk = lambda ci, co, k, s: QConv2d(ci, co, k, stride=s, padding="SAME", dtype=dtype, context=context)
-        self.conv1, self.bn1 = mk(cin, width, 1, 1), nn.BatchNorm2d(width)
-        self.conv2, self.bn2 = mk(width, width, 3, stride), nn.BatchNorm2d(width)
-        self.conv3, self.bn3 = mk(width, cout, 1, 1), nn.BatchNorm2d(cout)
+        # fused_bn: batch-norm (+ the ReLU behind it) on the library's kernels; otherwise torch's modules
+        bn = (lambda c, relu: QBatchNorm2d(c, relu=relu)) if fused_bn else (lambda c, relu: nn.BatchNorm2d(c))
+        self.fused_bn = fused_bn
+        self.conv1, self.bn1 = mk(cin, width, 1, 1), bn(width, True)
+        self.conv2, self.bn2 = mk(width, width, 3, stride), bn(width, True)
+        self.conv3, self.bn3 = mk(width, cout, 1, 1), bn(cout, False)
         self.down = None
         if stride != 1 or cin != cout:
-            self.down = nn.Sequential(mk(cin, cout, 1, stride), nn.BatchNorm2d(cout))
+            self.down = nn.Sequential(mk(cin, cout, 1, stride), bn(cout, False))
         self.relu = nn.ReLU(inplace=True)
 
     def forward(self, x):
         idt = x if self.down is None else self.down(x)
-        y = self.relu(self.bn1(self.conv1(x)))
-        y = self.relu(self.bn2(self.conv2(y)))
+        if self.fused_bn:
+            y = self.bn1(self.conv1(x))
+            y = self.bn2(self.conv2(y))
+        else:
+            y = self.relu(self.bn1(self.conv1(x)))
+            y = self.relu(self.bn2(self.conv2(y)))
         y = self.bn3(self.conv3(y))
         return self.relu(y + idt)
 
@@ -136,21 +181,23 @@ class _Bottleneck(nn.Module):
 class QResNet50(nn.Module):
     """ResNet-50 with quaternion channels = real channels / 4: stem 3->16 (7x7 s2), stages of
     (3, 4, 6, 3) bottlenecks with widths 16/32/64/128 and outputs 64/128/256/512, head = quaternion
-    Dense 512 -> 250 units (= 1000 logits).  53 convolutions.  The stem takes the real images
+    Dense 512 -> 250 units (= 1000 logits).  53 convolutions.  Batch-norm (with the ReLU behind it) runs on the
+    library's kernels (fused_bn=True) or on torch's modules.  The stem takes the real images
     [N, 3, H, W] directly (real_input=True) or, with real_input=False, their lift() to quaternions."""
 
-    def __init__(self, num_classes=1000, dtype=torch.float32, context=None, real_input=True):
+    def __init__(self, num_classes=1000, dtype=torch.float32, context=None, real_input=True, fused_bn=True):
         super().__init__()
         assert num_classes % 4 == 0
         self.stem = QConv2d(3, 16, 7, stride=2, padding="SAME", dtype=dtype, context=context, input_requires_grad=False,
                             real_input=real_input)
-        self.bn = nn.BatchNorm2d(16)
+        self.fused_bn = fused_bn
+        self.bn = QBatchNorm2d(16, relu=True) if fused_bn else nn.BatchNorm2d(16)
         self.relu = nn.ReLU(inplace=True)
         self.pool = nn.MaxPool2d(3, 2, 1)
         blocks, cin = [], 16
         for width, cout, count, stride in ((16, 64, 3, 1), (32, 128, 4, 2), (64, 256, 6, 2), (128, 512, 3, 2)):
             for i in range(count):
-                blocks.append(_Bottleneck(cin, width, cout, stride if i == 0 else 1, dtype, context))
+                blocks.append(_Bottleneck(cin, width, cout, stride if i == 0 else 1, dtype, context, fused_bn))
                 cin = cout
         self.blocks = nn.Sequential(*blocks)
         self.head = QLinear(512, num_classes // 4, bias=True, dtype=dtype, context=context)
@@ -162,7 +209,8 @@ class QResNet50(nn.Module):
         return torch.cat([images, z, z, z], dim=0)
 
     def forward(self, x):
-        y = self.pool(self.relu(self.bn(self.stem(x))))
+        y = self.bn(self.stem(x))
+        y = self.pool(y if self.fused_bn else self.relu(y))
         y = self.blocks(y)
         y = y.float().mean(dim=(2, 3)).to(x.dtype)            # [4N, 512]
         y = self.head(y)                                      # [4N, 250]

@@ -20,6 +20,17 @@ def test_every_declared_symbol_is_exported():
     assert declared == set(capi.EXPORTS)
 
 
+def test_batch_norm_header_symbols_are_exported():
+    header = open(os.path.join(ROOT, "include", "phx_bn.h")).read()
+    declared = set(re.findall(r"\b(phx_bn_[a-z0-9_]+)\s*\(", header))
+    lib = capi.lib()
+    assert declared == set(capi.EXPORTS_BN)
+    assert all(hasattr(lib, s) for s in declared)
+    desc = capi.BnDesc(capi.PHX_F16, 256, 16, 3136, 1e-5, 0.1, 1)
+    assert lib.phx_bn_workspace_bytes(ctypes.byref(desc)) > 0
+    assert lib.phx_bn_workspace_bytes(ctypes.byref(capi.BnDesc(7, 1, 1, 1, 1e-5, 0.1, 0))) == 0
+
+
 def test_status_strings_and_descriptor_validation():
     assert capi.status_string(0) == "ok"
     assert "workspace" in capi.status_string(3)

@@ -1,0 +1,68 @@
+"""Batch normalisation (+ ReLU) kernels of include/phx_bn.h against torch's batch_norm evaluated in fp64 on
+the CPU from the same (fp16- or fp32-rounded) inputs: output, saved and running statistics, input gradient
+and parameter gradients.  Tolerance: 1e-4 (fp32 tensors) / 4e-3 (fp16 tensors, whose outputs are rounded to
+fp16) of the largest reference magnitude."""
+import numpy as np
+import pytest
+import torch
+
+import phoenix_core_amd as phx
+
+pytestmark = pytest.mark.gpu
+
+SHAPES = [(8, 16, 14, 14), (12, 5, 7, 7), (3, 130, 1, 1), (64, 33, 9, 5), (1, 4, 3, 3), (256, 16, 28, 28), (40, 512, 7, 7)]
+
+
+def close(got, want, tol, what):
+    got = got.detach().double().cpu()
+    err = (got - want).abs().max().item()
+    assert torch.isfinite(got).all(), what
+    assert err <= tol * max(want.abs().max().item(), 1e-6), "%s: abs err %.3e of max %.3e" % (what, err, want.abs().max().item())
+
+
+@pytest.mark.parametrize("relu", [False, True])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_batch_norm_matches_torch(shape, dtype, relu):
+    print("shape", shape, dtype, relu, flush=True)
+    gen = torch.Generator().manual_seed(sum(shape))
+    c = shape[1]
+    x = (torch.randn(shape, generator=gen) * 1.5 + 0.3).to(dtype)
+    dy = torch.randn(shape, generator=gen).to(dtype)
+    gamma = torch.rand(c, generator=gen) + 0.5
+    beta = torch.randn(c, generator=gen) * 0.3
+    mod = phx.QBatchNorm2d(c, relu=relu).cuda().train()
+    with torch.no_grad():
+        mod.weight.copy_(gamma)
+        mod.bias.copy_(beta)
+    xd = x.cuda().requires_grad_(True)
+    y = mod(xd)
+    y.backward(dy.cuda())
+
+    x64 = x.double().requires_grad_(True)
+    g64, b64 = gamma.double().requires_grad_(True), beta.double().requires_grad_(True)
+    rm, rv = torch.zeros(c, dtype=torch.float64), torch.ones(c, dtype=torch.float64)
+    ref = torch.nn.functional.batch_norm(x64, rm, rv, g64, b64, True, 0.1, 1e-5)
+    if relu:
+        ref = torch.relu(ref)
+    ref.backward(dy.double())
+    tol = 1e-4 if dtype == torch.float32 else 4e-3
+    assert y.dtype == dtype and y.shape == tuple(shape)
+    close(y, ref.detach(), tol, "y")
+    close(xd.grad, x64.grad, tol, "dx")
+    close(mod.weight.grad, g64.grad, tol, "dgamma")
+    close(mod.bias.grad, b64.grad, tol, "dbeta")
+    close(mod.running_mean, rm, 1e-4, "running mean")
+    close(mod.running_var, rv, 1e-4, "running var")
+
+
+def test_eval_mode_uses_running_statistics():
+    mod = phx.QBatchNorm2d(6, relu=True).cuda()
+    x = torch.randn(8, 6, 5, 5, device="cuda")
+    mod.train()
+    mod(x)
+    mod.eval()
+    y = mod(x)
+    want = torch.relu(torch.nn.functional.batch_norm(x, mod.running_mean, mod.running_var, mod.weight, mod.bias, False, 0.0,
+                                                     mod.eps))
+    assert torch.allclose(y, want)

@@ -87,7 +87,11 @@ def _cpu_forward(model, xq):
 
     cpu_params = {}
     import copy
-    bn = lambda m: copy.deepcopy(m).cpu().float().train()
+    def bn(m):  # torch's module with the same parameters and statistics, whichever module the model holds
+        t = torch.nn.BatchNorm2d(m.weight.numel(), eps=m.eps, momentum=m.momentum)
+        t.load_state_dict({k: v.detach().cpu().float() for k, v in m.state_dict().items() if k != "num_batches_tracked"},
+                          strict=False)
+        return t.train()
     y = model.pool(model.relu(bn(model.bn)(conv(model.stem, xq))))
     for b in model.blocks:
         idt = y if b.down is None else bn(b.down[1])(conv(b.down[0], y))
@@ -109,12 +113,13 @@ def _cpu_forward(model, xq):
     return logits, cpu_params
 
 
-@pytest.mark.parametrize("real_input", [True, False])
-def test_qresnet50_end_to_end_matches_cpu_restatement(real_input):
+@pytest.mark.parametrize("real_input,fused_bn", [(True, True), (False, False), (True, False)])
+def test_qresnet50_end_to_end_matches_cpu_restatement(real_input, fused_bn):
     """The stem either takes the real images (real-valued input) or their lift to quaternions with zero
     imaginary parts; the CPU restatement always runs on the lifted tensor."""
     torch.manual_seed(2)
-    model = phx.QResNet50(num_classes=1000, dtype=torch.float32, context=Ctx(8), real_input=real_input).cuda().train()
+    model = phx.QResNet50(num_classes=1000, dtype=torch.float32, context=Ctx(8), real_input=real_input,
+                          fused_bn=fused_bn).cuda().train()
     convs = model.conv_layers()
     assert len(convs) == 53
     images = torch.randn(2, 3, 64, 64)
