@@ -196,6 +196,12 @@ __device__ __forceinline__ u32x4 load16_a2(const _Float16* p) {
     return *reinterpret_cast<const __attribute__((address_space(1))) u32x4_a2*>(
         (const __attribute__((address_space(1))) _Float16*)p);
 }
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+typedef u32x2 u32x2_a2 __attribute__((aligned(2)));
+__device__ __forceinline__ u32x2 load8_a2(const _Float16* p) {
+    return *reinterpret_cast<const __attribute__((address_space(1))) u32x2_a2*>(
+        (const __attribute__((address_space(1))) _Float16*)p);
+}
 __device__ __forceinline__ unsigned int load4_a2(const _Float16* p) {
     return *reinterpret_cast<const __attribute__((address_space(1))) u32_a2*>(
         (const __attribute__((address_space(1))) _Float16*)p);

@@ -776,7 +776,7 @@ __global__ void __launch_bounds__(WG_THREADS) pack_filters_f16_lds_kernel(const 
 //   the reduction); CoT = 32*MT, CiT = 32*NT, the 4 waves form a 2x2 grid, each owning MT x NT
 //   MFMA tiles of 16x16 channels for every tap of the group and all four components (16-product:
 //   signs folded into a negated copy of the gradient operand) or all eight lanes (8-product).
-//   TPW == 3 (unit stride and dilation along W): one 10-pixel load per input chunk yields the
+//   TPW == 3 or 4 (unit stride and dilation along W): one 10- or 12-pixel load per input chunk yields the
 //   three copies shifted by 0/1/2 pixels with byte-align operations; each copy is written to its
 //   own LDS plane so every MFMA operand is one aligned 16-byte LDS read.
 //   SW == 2: the input chunk is 16 consecutive pixels of which the even ones are kept.
@@ -832,12 +832,12 @@ __device__ __forceinline__ WgChunk wg_chunk(const WgradArgs& P, int tile, int j)
 
 template <int MODE, int MT, int NT, int TPW, int SW>
 __global__ void __launch_bounds__(WG_THREADS) qconv_wgrad_f16_kernel(const WgradArgs P) {
-    static_assert(TPW == 1 || (TPW == 3 && SW == 1), "shifted copies need unit stride");
+    static_assert(TPW == 1 || ((TPW == 3 || TPW == 4) && SW == 1), "shifted copies need unit stride");
     constexpr int CoT = 32 * MT, CiT = 32 * NT;
     constexpr int NL = (MODE == 16) ? 4 : 8;  // accumulators per (tap, tile): components or lanes
     constexpr int KPp = WG16_PITCH;
     constexpr int GE = 4 * MT, XE = 4 * NT;                  // chunks per thread and tile: gradient / input planes
-    constexpr int XR = (TPW == 3) ? 5 : (SW == 2 ? 8 : 4);   // dwords loaded per input chunk
+    constexpr int XR = (TPW == 3) ? 5 : (TPW == 4) ? 6 : (SW == 2 ? 8 : 4);   // dwords loaded per input chunk
     extern __shared__ f16x8 lds16[];
     _Float16* gl = reinterpret_cast<_Float16*>(lds16);  // [4][CoT][KPp]
     _Float16* xl = gl + 4 * CoT * KPp;                   // [TPW][4][CiT][KPp]
@@ -951,6 +951,9 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_wgrad_f16_kernel(const Wgrad
                 sx[e][0] = a[0]; sx[e][1] = a[1]; sx[e][2] = a[2]; sx[e][3] = a[3];
             } else if constexpr (XR == 5) {
                 sx[e][4] = load4_a2(ptr + 8);
+            } else if constexpr (XR == 6) {
+                const u32x2 b = load8_a2(ptr + 8);
+                sx[e][4] = b[0]; sx[e][5] = b[1];
             } else if constexpr (XR == 8) {
                 const u32x4 b = load16_a2(ptr + 8);
                 sx[e][4] = b[0]; sx[e][5] = b[1]; sx[e][6] = b[2]; sx[e][7] = b[3];
@@ -1022,9 +1025,10 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_wgrad_f16_kernel(const Wgrad
                     if constexpr (XR == 8) {
 #pragma unroll
                         for (int d = 0; d < 4; ++d) v[d] = __builtin_amdgcn_perm(w[2 * d + 1], w[2 * d], 0x05040100u);
-                    } else if (t == 1) {
+                    } else if (t & 1) {  // shifted by an odd number of pixels: halves of two neighbouring dwords
 #pragma unroll
-                        for (int d = 0; d < 4; ++d) v[d] = __builtin_amdgcn_alignbyte(w[(d + 1) % XR], w[d], 2);
+                        for (int d = 0; d < 4; ++d)
+                            v[d] = __builtin_amdgcn_alignbyte(w[(d + (t >> 1) + 1) % XR], w[(d + (t >> 1)) % XR], 2);
                     } else {
 #pragma unroll
                         for (int d = 0; d < 4; ++d) v[d] = w[(d + (t >> 1)) % XR];
@@ -1133,11 +1137,13 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_wgrad_f16_kernel(const Wgrad
 #pragma unroll
                 for (int i = 0; i < MT; ++i)
 #pragma unroll
-                    for (int p = 0; p < 4; ++p)
+                    for (int p = 0; p < 4; ++p) {
+                        if (p >= xnc) continue;  // real-valued input: components 1..3 are zero, their products too
 #pragma unroll
                         for (int q = 0; q < 4; ++q)
                             acc[t][i][jn][p ^ q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
                                 g[i][q], qneg(p, q) ? nx[p] : x[p], acc[t][i][jn][p ^ q], 0, 0, 0);
+                    }
             } else {
                 f16x8 L[8];
                 lanes_left(x, L);

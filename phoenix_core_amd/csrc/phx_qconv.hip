@@ -471,10 +471,15 @@ static bool plan_wgrad_f16(const Problem& p, WgPlan& best) {
     best = WgPlan{};
     best.SW = p.sw;
     best.kmode = wgrad_f16_formulation(p);
-    best.TPW = (best.kmode == 16 && p.kw % 3 == 0 && p.sw == 1 && p.dw == 1) ? 3 : 1;
     best.MT = p.co > 32 ? 2 : 1;
     best.NT = p.ci > 32 ? 2 : 1;
     if (const char* e = getenv("PHX_TUNE_WG")) sscanf(e, "%d,%d", &best.MT, &best.NT);
+    // taps of one filter row that share a workgroup (and with it the staged gradient tile): three, or four
+    // where the row has a multiple of four taps and the channel tile leaves the registers for it
+    const bool shifts = best.kmode == 16 && p.sw == 1 && p.dw == 1;
+    best.TPW = (shifts && p.kw % 3 == 0) ? 3 : (shifts && p.kw % 4 == 0 && !(best.MT == 2 && best.NT == 2)) ? 4 : 1;
+    auto lds_need = [&](int tpw) { return (size_t)(4 * 32 * best.MT + tpw * 4 * 32 * best.NT) * 72 * 2; };
+    if (lds_need(best.TPW) > 160 * 1024) best.TPW = 1;  // (four shifted copies of a 64-channel input tile do not fit)
     const int CoT = 32 * best.MT, CiT = 32 * best.NT;
     best.cpr = cdiv(p.wo, 8);
     const long nchunks = (long)p.n * p.ho * best.cpr;

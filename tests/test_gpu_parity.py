@@ -228,6 +228,8 @@ FP16_CASES = [c for c in CONV_CASES if c[0] in ("pw_64", "pw_ragged", "pw_7x7img
                                                 "k3_valid", "k3_s2", "pw_s2", "k7_s2", "k3_s2_c4", "k5_s2_valid", "k3_dil2", "k32_s21", "k32_asym",
                                                 "co_gt_128")] + [
     ("k3_s3", 2, 8, 8, 13, 13, 3, 3, 3, 1, "SAME"),
+    ("k4_same", 2, 8, 16, 13, 15, 4, 4, 1, 1, "SAME"),        # four taps per filter row share a filter-gradient workgroup
+    ("k24_c40", 3, 40, 24, 9, 21, 2, 4, 1, 1, "VALID"),
     ("k3_128_28", 2, 128, 128, 28, 28, 3, 3, 1, 1, "SAME"),
     ("pw_256_14", 3, 256, 256, 14, 14, 1, 1, 1, 1, "VALID"),
 ]

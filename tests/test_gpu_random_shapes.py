@@ -37,7 +37,7 @@ def close(got, want, dtype, what):
 def draw(seed):
     r = np.random.default_rng(seed)
     while True:
-        kh, kw = (int(v) for v in r.choice([1, 1, 2, 3, 3, 5, 7], 2))
+        kh, kw = (int(v) for v in r.choice([1, 1, 2, 3, 3, 4, 5, 7], 2))
         if r.random() < 0.6:
             kw = kh
         stride = tuple(int(v) for v in r.choice([1, 1, 1, 2, 2, 3], 2))
