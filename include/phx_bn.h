@@ -33,17 +33,19 @@ typedef struct phx_bn_desc {
 
 size_t phx_bn_workspace_bytes(const phx_bn_desc* desc);
 
-/* y = gamma * (x - mean) / sqrt(var + eps) + beta with the batch statistics of x; save_mean and
- * save_invstd ([C] each) receive them for the backward pass; running_mean / running_var ([C]) are
- * updated when non-null. */
-int phx_bn_fwd_train(const phx_bn_desc* desc, phx_stream_t stream, const void* x, const float* gamma, const float* beta,
-                     void* y, float* save_mean, float* save_invstd, float* running_mean_or_null,
-                     float* running_var_or_null, void* workspace, size_t workspace_bytes);
+/* y = gamma * (x - mean) / sqrt(var + eps) + beta (+ residual) with the batch statistics of x, then the
+ * optional ReLU; save_mean and save_invstd ([C] each) receive the statistics for the backward pass;
+ * running_mean / running_var ([C]) are updated when non-null.  The residual (same shape as x, e.g. the
+ * identity branch of a bottleneck block) is added in front of the ReLU. */
+int phx_bn_fwd_train(const phx_bn_desc* desc, phx_stream_t stream, const void* x, const void* residual_or_null,
+                     const float* gamma, const float* beta, void* y, float* save_mean, float* save_invstd,
+                     float* running_mean_or_null, float* running_var_or_null, void* workspace, size_t workspace_bytes);
 
-/* dx, dgamma, dbeta from x, dy and the saved statistics (beta is read for the ReLU mask only). */
-int phx_bn_bwd(const phx_bn_desc* desc, phx_stream_t stream, const void* x, const void* dy, const float* gamma,
-               const float* beta, const float* save_mean, const float* save_invstd, void* dx, float* dgamma,
-               float* dbeta, void* workspace, size_t workspace_bytes);
+/* dx, dgamma, dbeta from x, dy and the saved statistics (beta and the residual are read for the ReLU mask
+ * only); with a residual (relu must be set), dresidual receives its gradient, dy behind the ReLU. */
+int phx_bn_bwd(const phx_bn_desc* desc, phx_stream_t stream, const void* x, const void* residual_or_null, const void* dy,
+               const float* gamma, const float* beta, const float* save_mean, const float* save_invstd, void* dx,
+               void* dresidual_or_null, float* dgamma, float* dbeta, void* workspace, size_t workspace_bytes);
 
 #ifdef __cplusplus
 }

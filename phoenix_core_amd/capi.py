@@ -82,8 +82,8 @@ def lib():
         bd = ctypes.POINTER(BnDesc)
         L.phx_bn_workspace_bytes.restype = sz
         L.phx_bn_workspace_bytes.argtypes = [bd]
-        L.phx_bn_fwd_train.argtypes = [bd, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, sz]
-        L.phx_bn_bwd.argtypes = [bd, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, sz]
+        L.phx_bn_fwd_train.argtypes = [bd, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, sz]
+        L.phx_bn_bwd.argtypes = [bd, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, sz]
         L.phx_device_count.argtypes = [i32p]
         L.phx_device_malloc.argtypes = [ctypes.POINTER(vp), sz]
         L.phx_device_free.argtypes = [vp]

@@ -13,7 +13,9 @@ namespace phx {
 struct BnArgs {
     const void* x;
     const void* dy;      // backward only
+    const void* res;     // optional residual added in front of the ReLU (null = none)
     void* out;           // y (forward) or dx (backward)
+    void* dres;          // backward with a residual: its gradient (the gradient behind the ReLU)
     const float* gamma;
     const float* beta;
     float* partial;      // [C][S][2]
@@ -121,6 +123,7 @@ __global__ void __launch_bounds__(256) bn_sums_kernel(const BnArgs P) {
     const int nb = min(P.rows_per_split, P.rows - b0);
     const TS* x = static_cast<const TS*>(P.x);
     const TS* dy = static_cast<const TS*>(P.dy);
+    const TS* res = static_cast<const TS*>(P.res);
     float mean = 0.f, invstd = 0.f, g = 0.f, be = 0.f;
     if constexpr (MODE == 1) { mean = P.save_mean[c]; invstd = P.save_invstd[c]; g = P.gamma[c]; be = P.beta[c]; }
     float a0 = 0.f, a1 = 0.f;
@@ -135,12 +138,13 @@ __global__ void __launch_bounds__(256) bn_sums_kernel(const BnArgs P) {
 #pragma unroll
             for (int i = 0; i < V; ++i) { a0 += xv[i]; a1 += xv[i] * xv[i]; }
         } else {
-            float dv[V];
+            float dv[V], rv[V];
             load_chunk<TS>(dy + off, n, dv);
+            if (res) load_chunk<TS>(res + off, n, rv);
 #pragma unroll
             for (int i = 0; i < V; ++i) {
                 const float xh = (xv[i] - mean) * invstd;
-                const float d = (P.relu && g * xh + be <= 0.f) ? 0.f : dv[i];
+                const float d = (P.relu && g * xh + be + (res ? rv[i] : 0.f) <= 0.f) ? 0.f : dv[i];
                 a0 += d;
                 a1 += d * xh;  // (elements past the plane carry dy = 0)
             }
@@ -185,18 +189,21 @@ __global__ void __launch_bounds__(256) bn_apply_kernel(const BnArgs P) {
     const float k0 = t0 / m, k1 = t1 / m, scale = g * invstd;
     const TS* x = static_cast<const TS*>(P.x);
     const TS* dy = static_cast<const TS*>(P.dy);
+    const TS* res = static_cast<const TS*>(P.res);
     TS* out = static_cast<TS*>(P.out);
+    TS* dres = static_cast<TS*>(P.dres);
     const int total = nb * P.nchunk;
     for (int idx = threadIdx.x; idx < total; idx += 256) {
         const int b = idx / P.nchunk, ch = idx - b * P.nchunk;
         const long off = ((long)(b0 + b) * P.C + c) * P.hw + ch * V;
         const int n = min(V, P.hw - ch * V);
-        float xv[V], ov[V];
+        float xv[V], ov[V], rv[V];
         load_chunk<TS>(x + off, n, xv);
+        if (res) load_chunk<TS>(res + off, n, rv);
         if constexpr (MODE == 0) {
 #pragma unroll
             for (int i = 0; i < V; ++i) {
-                const float y = scale * (xv[i] - mean) + be;
+                const float y = scale * (xv[i] - mean) + be + (res ? rv[i] : 0.f);
                 ov[i] = (P.relu && y < 0.f) ? 0.f : y;
             }
         } else {
@@ -205,9 +212,11 @@ __global__ void __launch_bounds__(256) bn_apply_kernel(const BnArgs P) {
 #pragma unroll
             for (int i = 0; i < V; ++i) {
                 const float xh = (xv[i] - mean) * invstd;
-                const float d = (P.relu && g * xh + be <= 0.f) ? 0.f : dv[i];
+                const float d = (P.relu && g * xh + be + (res ? rv[i] : 0.f) <= 0.f) ? 0.f : dv[i];
                 ov[i] = scale * (d - k0 - xh * k1);
+                dv[i] = d;
             }
+            if (dres) store_chunk<TS>(dres + off, n, dv);
         }
         store_chunk<TS>(out + off, n, ov);
     }
@@ -252,16 +261,16 @@ size_t phx_bn_workspace_bytes(const phx_bn_desc* desc) {
     return ((size_t)a.C * a.S * 2 * sizeof(float) + 255) / 256 * 256;
 }
 
-int phx_bn_fwd_train(const phx_bn_desc* desc, phx_stream_t stream, const void* x, const float* gamma, const float* beta,
-                     void* y, float* save_mean, float* save_invstd, float* running_mean_or_null,
-                     float* running_var_or_null, void* workspace, size_t workspace_bytes) {
+int phx_bn_fwd_train(const phx_bn_desc* desc, phx_stream_t stream, const void* x, const void* residual_or_null,
+                     const float* gamma, const float* beta, void* y, float* save_mean, float* save_invstd,
+                     float* running_mean_or_null, float* running_var_or_null, void* workspace, size_t workspace_bytes) {
     BnArgs a{};
     const int rc = plan(desc, a);
     if (rc != PHX_OK) return rc;
     if (desc->rows == 0 || desc->hw == 0) return PHX_OK;
     if (!x || !gamma || !beta || !y || !save_mean || !save_invstd) return PHX_ERR_INVALID_ARGUMENT;
     if (!workspace || workspace_bytes < (size_t)a.C * a.S * 2 * sizeof(float)) return PHX_ERR_WORKSPACE;
-    a.x = x; a.out = y; a.gamma = gamma; a.beta = beta; a.partial = static_cast<float*>(workspace);
+    a.x = x; a.res = residual_or_null; a.out = y; a.gamma = gamma; a.beta = beta; a.partial = static_cast<float*>(workspace);
     a.save_mean = save_mean; a.save_invstd = save_invstd; a.run_mean = running_mean_or_null; a.run_var = running_var_or_null;
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (desc->dtype == PHX_F16) launch_all<_Float16>(a, false, st);
@@ -270,9 +279,9 @@ int phx_bn_fwd_train(const phx_bn_desc* desc, phx_stream_t stream, const void* x
     return PHX_OK;
 }
 
-int phx_bn_bwd(const phx_bn_desc* desc, phx_stream_t stream, const void* x, const void* dy, const float* gamma,
-               const float* beta, const float* save_mean, const float* save_invstd, void* dx, float* dgamma,
-               float* dbeta, void* workspace, size_t workspace_bytes) {
+int phx_bn_bwd(const phx_bn_desc* desc, phx_stream_t stream, const void* x, const void* residual_or_null, const void* dy,
+               const float* gamma, const float* beta, const float* save_mean, const float* save_invstd, void* dx,
+               void* dresidual_or_null, float* dgamma, float* dbeta, void* workspace, size_t workspace_bytes) {
     BnArgs a{};
     const int rc = plan(desc, a);
     if (rc != PHX_OK) return rc;
@@ -280,7 +289,8 @@ int phx_bn_bwd(const phx_bn_desc* desc, phx_stream_t stream, const void* x, cons
     if (desc->rows == 0 || desc->hw == 0) return PHX_OK;
     if (!x || !dy || !gamma || !beta || !save_mean || !save_invstd || !dx) return PHX_ERR_INVALID_ARGUMENT;
     if (!workspace || workspace_bytes < (size_t)a.C * a.S * 2 * sizeof(float)) return PHX_ERR_WORKSPACE;
-    a.x = x; a.dy = dy; a.out = dx; a.gamma = gamma; a.beta = beta; a.partial = static_cast<float*>(workspace);
+    if (residual_or_null && !desc->relu) return PHX_ERR_INVALID_ARGUMENT;  // without the ReLU its gradient is dy itself
+    a.x = x; a.res = residual_or_null; a.dres = dresidual_or_null; a.dy = dy; a.out = dx; a.gamma = gamma; a.beta = beta; a.partial = static_cast<float*>(workspace);
     a.save_mean = const_cast<float*>(save_mean); a.save_invstd = const_cast<float*>(save_invstd);
     a.dgamma = dgamma; a.dbeta = dbeta;
     hipStream_t st = static_cast<hipStream_t>(stream);

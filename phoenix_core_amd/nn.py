@@ -115,17 +115,18 @@ class QLinear(nn.Module):
 
 class _QBatchNormFn(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, x, gamma, beta, running_mean, running_var, eps, momentum, relu):
-        y, mean, invstd = ops.batch_norm_fwd(x, gamma, beta, running_mean, running_var, eps, momentum, relu)
-        ctx.save_for_backward(x, gamma, beta, mean, invstd)
+    def forward(ctx, x, residual, gamma, beta, running_mean, running_var, eps, momentum, relu):
+        y, mean, invstd = ops.batch_norm_fwd(x, gamma, beta, running_mean, running_var, eps, momentum, relu, residual)
+        ctx.save_for_backward(x, residual, gamma, beta, mean, invstd)
         ctx.eps, ctx.relu = eps, relu
         return y
 
     @staticmethod
     def backward(ctx, dy):
-        x, gamma, beta, mean, invstd = ctx.saved_tensors
-        dx, dgamma, dbeta = ops.batch_norm_bwd(x, dy.contiguous(), gamma, beta, mean, invstd, ctx.eps, ctx.relu)
-        return dx, dgamma, dbeta, None, None, None, None, None
+        x, residual, gamma, beta, mean, invstd = ctx.saved_tensors
+        dx, dgamma, dbeta, dres = ops.batch_norm_bwd(x, dy.contiguous(), gamma, beta, mean, invstd, ctx.eps, ctx.relu,
+                                                     residual)
+        return dx, dres, dgamma, dbeta, None, None, None, None, None
 
 
 class QBatchNorm2d(nn.Module):
@@ -143,11 +144,17 @@ class QBatchNorm2d(nn.Module):
         self.register_buffer("running_mean", torch.zeros(num_features))
         self.register_buffer("running_var", torch.ones(num_features))
 
-    def forward(self, x):
+    def forward(self, x, residual=None):
+        """residual (relu=True only): added to the normalised tensor in front of the ReLU, as the identity branch
+        of a bottleneck block is."""
+        if residual is not None and not self.relu:
+            raise ValueError("a residual goes in front of the ReLU: construct the module with relu=True")
         if self.training:
-            return _QBatchNormFn.apply(x.contiguous(), self.weight, self.bias, self.running_mean, self.running_var,
-                                       self.eps, self.momentum, self.relu)
+            return _QBatchNormFn.apply(x.contiguous(), None if residual is None else residual.contiguous(), self.weight,
+                                       self.bias, self.running_mean, self.running_var, self.eps, self.momentum, self.relu)
         y = nn.functional.batch_norm(x, self.running_mean, self.running_var, self.weight, self.bias, False, 0.0, self.eps)
+        if residual is not None:
+            y = y + residual
         return torch.relu(y) if self.relu else y
 
 
@@ -160,7 +167,7 @@ class _Bottleneck(nn.Module):
         self.fused_bn = fused_bn
         self.conv1, self.bn1 = mk(cin, width, 1, 1), bn(width, True)
         self.conv2, self.bn2 = mk(width, width, 3, stride), bn(width, True)
-        self.conv3, self.bn3 = mk(width, cout, 1, 1), bn(cout, False)
+        self.conv3, self.bn3 = mk(width, cout, 1, 1), bn(cout, True)  # (fused: ReLU behind the residual add)
         self.down = None
         if stride != 1 or cin != cout:
             self.down = nn.Sequential(mk(cin, cout, 1, stride), bn(cout, False))
@@ -171,9 +178,9 @@ class _Bottleneck(nn.Module):
         if self.fused_bn:
             y = self.bn1(self.conv1(x))
             y = self.bn2(self.conv2(y))
-        else:
-            y = self.relu(self.bn1(self.conv1(x)))
-            y = self.relu(self.bn2(self.conv2(y)))
+            return self.bn3(self.conv3(y), idt)
+        y = self.relu(self.bn1(self.conv1(x)))
+        y = self.relu(self.bn2(self.conv2(y)))
         y = self.bn3(self.conv3(y))
         return self.relu(y + idt)
 

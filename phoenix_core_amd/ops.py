@@ -296,11 +296,13 @@ def dense_bwd(x, w, grad, desc):
     return dw, dx
 
 
-def batch_norm_fwd(x, gamma, beta, running_mean, running_var, eps, momentum, relu):
-    """Training-mode batch normalisation (+ ReLU) of [rows, C, H, W] (include/phx_bn.h; no counterpart in the
-    reference, which holds no model code).  Returns (y, save_mean, save_invstd); the running statistics are
+def batch_norm_fwd(x, gamma, beta, running_mean, running_var, eps, momentum, relu, residual=None):
+    """Training-mode batch normalisation (+ residual, + ReLU) of [rows, C, H, W] (include/phx_bn.h; no counterpart in
+    the reference, which holds no model code).  Returns (y, save_mean, save_invstd); the running statistics are
     updated in place when given."""
-    dev = _dev_check(x, gamma, beta, running_mean, running_var)
+    dev = _dev_check(x, gamma, beta, running_mean, running_var, residual)
+    if residual is not None and (residual.shape != x.shape or residual.dtype != x.dtype):
+        raise ValueError("the residual must have the shape and type of the input")
     rows, c = x.shape[0], x.shape[1]
     hw = x.numel() // max(rows * c, 1)
     desc = capi.BnDesc(_DTYPES[x.dtype], rows, c, hw, eps, momentum, int(relu))
@@ -309,23 +311,26 @@ def batch_norm_fwd(x, gamma, beta, running_mean, running_var, eps, momentum, rel
     invstd = torch.empty(c, dtype=torch.float32, device=dev)
     nbytes = capi.lib().phx_bn_workspace_bytes(ctypes.byref(desc))
     ws = _workspace.get(dev, nbytes)
-    capi.check(capi.lib().phx_bn_fwd_train(ctypes.byref(desc), _stream(), _ptr(x), _ptr(gamma), _ptr(beta), _ptr(y),
-                                           _ptr(mean), _ptr(invstd), _ptr(running_mean), _ptr(running_var), _ptr(ws),
-                                           nbytes), "phx_bn_fwd_train")
+    capi.check(capi.lib().phx_bn_fwd_train(ctypes.byref(desc), _stream(), _ptr(x), _ptr(residual), _ptr(gamma), _ptr(beta),
+                                           _ptr(y), _ptr(mean), _ptr(invstd), _ptr(running_mean), _ptr(running_var),
+                                           _ptr(ws), nbytes), "phx_bn_fwd_train")
     return y, mean, invstd
 
 
-def batch_norm_bwd(x, dy, gamma, beta, mean, invstd, eps, relu):
-    """Returns (dx, dgamma, dbeta) of batch_norm_fwd."""
-    dev = _dev_check(x, dy, gamma, beta, mean, invstd)
+def batch_norm_bwd(x, dy, gamma, beta, mean, invstd, eps, relu, residual=None):
+    """Returns (dx, dgamma, dbeta, dresidual) of batch_norm_fwd; dresidual is None without a residual."""
+    dev = _dev_check(x, dy, gamma, beta, mean, invstd, residual)
     rows, c = x.shape[0], x.shape[1]
     hw = x.numel() // max(rows * c, 1)
     desc = capi.BnDesc(_DTYPES[x.dtype], rows, c, hw, eps, 0.0, int(relu))
     dx = torch.empty_like(x)
-    dgamma = torch.zeros(c, dtype=torch.float32, device=dev)
-    dbeta = torch.zeros(c, dtype=torch.float32, device=dev)
+    dres = torch.empty_like(x) if residual is not None else None
+    empty = rows * hw == 0  # nothing is enqueued then: the parameter gradients are zero
+    dgamma = (torch.zeros if empty else torch.empty)(c, dtype=torch.float32, device=dev)
+    dbeta = (torch.zeros if empty else torch.empty)(c, dtype=torch.float32, device=dev)
     nbytes = capi.lib().phx_bn_workspace_bytes(ctypes.byref(desc))
     ws = _workspace.get(dev, nbytes)
-    capi.check(capi.lib().phx_bn_bwd(ctypes.byref(desc), _stream(), _ptr(x), _ptr(dy), _ptr(gamma), _ptr(beta), _ptr(mean),
-                                     _ptr(invstd), _ptr(dx), _ptr(dgamma), _ptr(dbeta), _ptr(ws), nbytes), "phx_bn_bwd")
-    return dx, dgamma, dbeta
+    capi.check(capi.lib().phx_bn_bwd(ctypes.byref(desc), _stream(), _ptr(x), _ptr(residual), _ptr(dy), _ptr(gamma),
+                                     _ptr(beta), _ptr(mean), _ptr(invstd), _ptr(dx), _ptr(dres), _ptr(dgamma), _ptr(dbeta),
+                                     _ptr(ws), nbytes), "phx_bn_bwd")
+    return dx, dgamma, dbeta, dres

@@ -20,11 +20,11 @@ def close(got, want, tol, what):
     assert err <= tol * max(want.abs().max().item(), 1e-6), "%s: abs err %.3e of max %.3e" % (what, err, want.abs().max().item())
 
 
-@pytest.mark.parametrize("relu", [False, True])
+@pytest.mark.parametrize("relu,residual", [(False, False), (True, False), (True, True)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
 @pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "x".join(map(str, s)))
-def test_batch_norm_matches_torch(shape, dtype, relu):
-    print("shape", shape, dtype, relu, flush=True)
+def test_batch_norm_matches_torch(shape, dtype, relu, residual):
+    print("shape", shape, dtype, relu, residual, flush=True)
     gen = torch.Generator().manual_seed(sum(shape))
     c = shape[1]
     x = (torch.randn(shape, generator=gen) * 1.5 + 0.3).to(dtype)
@@ -35,14 +35,19 @@ def test_batch_norm_matches_torch(shape, dtype, relu):
     with torch.no_grad():
         mod.weight.copy_(gamma)
         mod.bias.copy_(beta)
+    res = (torch.randn(shape, generator=gen) * 0.7).to(dtype) if residual else None
     xd = x.cuda().requires_grad_(True)
-    y = mod(xd)
+    rd = res.cuda().requires_grad_(True) if residual else None
+    y = mod(xd, rd) if residual else mod(xd)
     y.backward(dy.cuda())
 
     x64 = x.double().requires_grad_(True)
     g64, b64 = gamma.double().requires_grad_(True), beta.double().requires_grad_(True)
     rm, rv = torch.zeros(c, dtype=torch.float64), torch.ones(c, dtype=torch.float64)
     ref = torch.nn.functional.batch_norm(x64, rm, rv, g64, b64, True, 0.1, 1e-5)
+    r64 = res.double().requires_grad_(True) if residual else None
+    if residual:
+        ref = ref + r64
     if relu:
         ref = torch.relu(ref)
     ref.backward(dy.double())
@@ -50,6 +55,8 @@ def test_batch_norm_matches_torch(shape, dtype, relu):
     assert y.dtype == dtype and y.shape == tuple(shape)
     close(y, ref.detach(), tol, "y")
     close(xd.grad, x64.grad, tol, "dx")
+    if residual:
+        close(rd.grad, r64.grad, tol, "dresidual")
     close(mod.weight.grad, g64.grad, tol, "dgamma")
     close(mod.bias.grad, b64.grad, tol, "dbeta")
     close(mod.running_mean, rm, 1e-4, "running mean")
