@@ -205,10 +205,12 @@ static bool plan_forward(const Corr& c, int mode, bool f16mfma, FwdPlan& best, b
         for (int NTW = 1; NTW <= ((mode == 16 || ldsk) ? 2 : 1); ++NTW) {
             if (force_ntw && NTW != force_ntw) continue;
             const int BN = (4 / WCO) * NTW * 32;
-            int cand[16];
+            int cand[24];
             int nc = 0;
             for (int k = 1; k <= 8; ++k) cand[nc++] = cdiv(c.Wout, k);
             cand[nc++] = 8; cand[nc++] = 16; cand[nc++] = 32; cand[nc++] = BN;
+            // (long rows whose window must stay within the staging limit: fractions of the workgroup's pixels)
+            cand[nc++] = BN / 2; cand[nc++] = (3 * BN) / 4; cand[nc++] = 48; cand[nc++] = 80;
             for (int a = 0; a < nc; ++a) {
                 const int TW = std::min(cand[a], std::min(c.Wout, BN));
                 if (TW <= 0) continue;
