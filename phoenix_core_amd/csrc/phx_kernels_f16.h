@@ -249,8 +249,8 @@ __global__ void __launch_bounds__(WG_THREADS) pack_filters_f16_kernel(const Pack
         const int row = tile * 32 + (lane & 31);
         int kh = tap / P.Kw, kw = tap - kh * P.Kw;
         if (MAP == MAP_DGRAD) {
-            kh = P.Kh - 1 - kh;
-            kw = P.Kw - 1 - kw;
+            kh = P.khm - kh * P.khs;
+            kw = P.kwm - kw * P.kws;
         }
         f16x8 vec[WC];
 #pragma unroll
@@ -727,8 +727,11 @@ __global__ void __launch_bounds__(WG_THREADS) pack_filters_f16_lds_kernel(const 
             for (int i = 0; i < 8; ++i) vec[q][i] = (_Float16)0;
         if (tap < taps && row < P.rows) {
             int kh = tap / P.Kw, kw = tap - kh * P.Kw;
-            if (MAP == MAP_DGRAD) { kh = P.Kh - 1 - kh; kw = P.Kw - 1 - kw; }
-            if (A.pw) kh = kw = 0;  // the one real tap
+            if (MAP == MAP_DGRAD) { kh = P.khm - kh * P.khs; kw = P.kwm - kw * P.kws; }
+            if (A.pw) {  // the one real tap (of a strided convolution's phase: the filter tap that reaches it)
+                kh = (MAP == MAP_DGRAD) ? P.khm : 0;
+                kw = (MAP == MAP_DGRAD) ? P.kwm : 0;
+            }
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 const int k16 = (lane >> 5) * 8 + i;

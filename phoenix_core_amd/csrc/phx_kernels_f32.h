@@ -447,7 +447,8 @@ struct PackArgs {
     void* out;
     long wcs, so, si, skh, skw;
     int Co, Ci;       // filter dims of the convolution (not of the correlation being run)
-    int Kh, Kw;
+    int Kh, Kw;       // taps of the correlation being run
+    int khm, khs, kwm, kws;  // input gradient: tap (u, v) of the correlation is filter tap (khm - u*khs, kwm - v*kws)
     int rows, red;    // correlation: output channels (rows) and reduced channels
     int row_tiles, nchunks;
 };
@@ -476,8 +477,8 @@ __global__ void __launch_bounds__(WG_THREADS) pack_filters_f32_kernel(const Pack
             if (MAP == MAP_DGRAD) {
                 o = red;
                 i = row;
-                kh = P.Kh - 1 - kh;
-                kw = P.Kw - 1 - kw;
+                kh = P.khm - kh * P.khs;
+                kw = P.kwm - kw * P.kws;
             }
             const long off = o * P.so + i * P.si + kh * P.skh + kw * P.skw;
 #pragma unroll

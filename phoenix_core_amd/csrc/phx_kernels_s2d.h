@@ -86,4 +86,52 @@ __global__ void __launch_bounds__(WG_THREADS) s2d_filter_kernel(const S2dFilterA
     }
 }
 
+// Input gradient of a strided convolution, computed per phase: dx(h, w) with (h % sh, w % sw) = (a, b) is a
+// unit-stride correlation of the output gradient with the filter taps that can reach that phase.  The phases
+// are computed densely into buffers [4N*C][Hp][Wp] (phase (a, b) at ph[a*sw + b]; an offset of -1 marks a
+// phase no tap reaches, which is zero) and interleaved into dx here: coalesced writes, one pass.
+struct PhaseMergeArgs {
+    const void* buf;      // start of the phase buffers
+    void* dx;
+    long off[16];         // element offset of each phase buffer, -1 = all zero
+    long planes;          // 4N * C
+    int H, W, sh, sw;
+};
+
+// A thread per 16 bytes of a dx row: whole-word stores (rows start at element alignment only, which the store
+// tolerates), loads along the sw phase rows that feed the row.
+template <typename TS>
+__global__ void __launch_bounds__(WG_THREADS) phase_merge_kernel(const PhaseMergeArgs A) {
+    constexpr int V = 16 / sizeof(TS);
+    const TS* buf = static_cast<const TS*>(A.buf);
+    TS* dx = static_cast<TS*>(A.dx);
+    const int cpr = (A.W + V - 1) / V;  // 16-byte words per row
+    const long total = A.planes * A.H * cpr;
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
+        const long r = idx / cpr;
+        const int w0 = (int)(idx - r * cpr) * V;
+        const long plane = r / A.H;
+        const int h = (int)(r - plane * A.H);
+        const int a = h % A.sh, hp = h / A.sh;
+        const int Hp = (A.H - a + A.sh - 1) / A.sh;
+        TS v[V];
+#pragma unroll
+        for (int i = 0; i < V; ++i) {
+            const int w = w0 + i;
+            const int b = w % A.sw;
+            const long o = A.off[a * A.sw + b];
+            const int Wp = (A.W - b + A.sw - 1) / A.sw;
+            v[i] = (o >= 0 && w < A.W) ? buf[o + (plane * Hp + hp) * Wp + w / A.sw] : (TS)0;
+        }
+        TS* dst = dx + r * A.W + w0;
+        if (w0 + V <= A.W) {
+            u32x4 raw;
+            __builtin_memcpy(&raw, v, 16);
+            *reinterpret_cast<__attribute__((address_space(1))) u32x4_a2*>((__attribute__((address_space(1))) _Float16*)dst) = raw;
+        } else {
+            for (int i = 0; w0 + i < A.W; ++i) dst[i] = v[i];
+        }
+    }
+}
+
 }  // namespace phx

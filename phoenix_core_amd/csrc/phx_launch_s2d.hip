@@ -43,4 +43,12 @@ int launch_fill_zero(void* dst, size_t bytes, hipStream_t st) {
     return 0;
 }
 
+int launch_phase_merge(bool half_storage, const PhaseMergeArgs& a, hipStream_t st) {
+    const long items = a.planes * a.H * ((a.W + 3) / 4);  // at most: 16-byte words
+    if (items == 0) return 0;
+    if (half_storage) hipLaunchKernelGGL((phase_merge_kernel<_Float16>), dim3(blocks_for(items)), dim3(WG_THREADS), 0, st, a);
+    else hipLaunchKernelGGL((phase_merge_kernel<float>), dim3(blocks_for(items)), dim3(WG_THREADS), 0, st, a);
+    return 0;
+}
+
 }  // namespace phx

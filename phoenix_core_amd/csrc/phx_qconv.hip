@@ -144,10 +144,13 @@ static Problem flatten_pointwise(const Problem& p) {
 struct Corr {
     int N, Cin, Hin, Win, Cout, Hout, Wout;
     int Kh, Kw, sh, sw, dh, dw, pt, pl, uh, uw;
+    // input gradient: tap (u, v) of the correlation is filter tap (khm - u*khs, kwm - v*kws); the plain mirrored
+    // filter has khm = Kh-1, khs = 1
+    int khm, khs, kwm, kws;
 };
 
 static Corr corr_forward(const Problem& p) {
-    Corr c{p.n, p.ci, p.h, p.w, p.co, p.ho, p.wo, p.kh, p.kw, p.sh, p.sw, p.dh, p.dw, p.pt, p.pl, 1, 1};
+    Corr c{p.n, p.ci, p.h, p.w, p.co, p.ho, p.wo, p.kh, p.kw, p.sh, p.sw, p.dh, p.dw, p.pt, p.pl, 1, 1, p.kh - 1, 1, p.kw - 1, 1};
     if (p.kh == 1 && p.kw == 1 && p.sh == 1 && p.sw == 1 && !p.pt && !p.pl && !p.pb && !p.pr) {
         c.Win = p.h * p.w; c.Hin = 1; c.Wout = p.ho * p.wo; c.Hout = 1;  // pointwise: one long row per image
     }
@@ -156,7 +159,7 @@ static Corr corr_forward(const Problem& p) {
 
 static Corr corr_dgrad(const Problem& p) {
     Corr c{p.n, p.co, p.ho, p.wo, p.ci, p.h, p.w, p.kh, p.kw, 1, 1, p.dh, p.dw,
-           (p.kh - 1) * p.dh - p.pt, (p.kw - 1) * p.dw - p.pl, p.sh, p.sw};
+           (p.kh - 1) * p.dh - p.pt, (p.kw - 1) * p.dw - p.pl, p.sh, p.sw, p.kh - 1, 1, p.kw - 1, 1};
     if (p.kh == 1 && p.kw == 1 && p.sh == 1 && p.sw == 1 && !p.pt && !p.pl && !p.pb && !p.pr) {
         c.Win = p.ho * p.wo; c.Hin = 1; c.Wout = p.h * p.w; c.Hout = 1;
     }
@@ -329,8 +332,12 @@ static bool plan_corr(const Corr& creal, int mode, bool f16mfma, Corr& c, FwdPla
     }
     pw = 0;
     c = creal;
-    pl.kmode = mode;
-    return plan_forward(c, mode, f16mfma, pl);
+    // zero-inserted windows (input gradient of a strided convolution with several taps) on fp16 matrix cores:
+    // the factorized kernel has no LDS-filter form for them, the 16-product kernel has (3x3 stride 2 at
+    // 32-128 channels: 0.15-0.18 ms against 0.08-0.11 ms), so the 8-product mode takes that one here as well
+    const bool zero_inserted = c.uh > 1 || c.uw > 1;
+    pl.kmode = (f16mfma && mode == 8 && zero_inserted && c.Kh * c.Kw > 1 && !getenv("PHX_TUNE_ZI8")) ? 16 : mode;
+    return plan_forward(c, pl.kmode, f16mfma, pl);
 }
 
 static int run_corr(const Problem& p, const Corr& creal, int map, hipStream_t st, const void* in, const void* w,
@@ -350,12 +357,13 @@ static int run_corr(const Problem& p, const Corr& creal, int map, hipStream_t st
     PackArgs pa;
     pa.w = w; pa.out = ws;
     pa.wcs = p.fs.wcs; pa.so = p.fs.so; pa.si = p.fs.si; pa.skh = p.fs.skh; pa.skw = p.fs.skw;
-    pa.Co = p.co; pa.Ci = p.ci; pa.Kh = p.kh; pa.Kw = p.kw;
+    pa.Co = p.co; pa.Ci = p.ci; pa.Kh = creal.Kh; pa.Kw = creal.Kw;
+    pa.khm = creal.khm; pa.khs = creal.khs; pa.kwm = creal.kwm; pa.kws = creal.kws;
     pa.rows = c.Cout; pa.red = creal.Cin; pa.row_tiles = pl.co_tiles * pl.WCO;
     pa.nchunks = f16 ? pl.nchunks : pl.nchunks * (pl.CK / F32_CK);
     // (LDS images: one thread per 16-byte vector, in 8-product form one thread per eight lane vectors)
     const long pack_items = pl.lds_filters ? (long)(pl.wpk_bytes / 16) / (pl.kmode == 8 ? 8 : 1)
-                                            : (long)pa.row_tiles * pa.nchunks * p.kh * p.kw * (f16 ? 1 : 4) * 64;
+                                            : (long)pa.row_tiles * pa.nchunks * creal.Kh * creal.Kw * (f16 ? 1 : 4) * 64;
     if (pl.lds_filters) pa.row_tiles = pl.co_tiles;  // packed per workgroup tile of WCO*32 channels
     const int pack_blocks = (int)std::min<long>((pack_items + WG_THREADS - 1) / WG_THREADS, 4096);
 
@@ -564,6 +572,54 @@ static int run_wgrad(const Problem& p, hipStream_t st, const void* x, const void
     return PHX_OK;
 }
 
+// Input gradient of a strided convolution by phases (see phase_merge_kernel): the rows h = sh*i + a of dx
+// receive the filter rows kh with kh*dh = a + pt (mod sh), which form an arithmetic progression; row i of
+// the phase reads gradient row i + (a + pt - kh*dh)/sh.  Per axis that is a unit-stride correlation with
+// `taps` taps, dilation `dil` and `pad` rows of zero padding in front.
+struct PhaseAxis {
+    int taps, kmax, kstep, dil, pad, size;
+};
+
+static PhaseAxis phase_axis(int a, int extent, int k, int d, int s, int pad_before) {
+    PhaseAxis ax{0, 0, 1, 1, 0, a < extent ? (extent - a + s - 1) / s : 0};
+    int first = -1, second = -1;
+    for (int kk = 0; kk < k; ++kk) {
+        if ((a + pad_before - kk * d) % s != 0) continue;  // (C++ remainder: zero exactly for multiples, whatever the sign)
+        if (first < 0) first = kk;
+        else if (second < 0) second = kk;
+        ax.kmax = kk;
+        ++ax.taps;
+    }
+    if (ax.taps == 0) return ax;
+    ax.kstep = second >= 0 ? second - first : 1;
+    ax.dil = second >= 0 ? (ax.kstep * d) / s : 1;
+    // tap u is filter tap kmax - u*kstep and reads gradient row i + off(kmax) + u*dil
+    const int off_min = (a + pad_before - ax.kmax * d) / s;
+    ax.pad = -off_min;
+    return ax;
+}
+
+// Used for strided pointwise convolutions (one phase holds everything, the others are zero: 0.15 -> 0.08-0.11 ms
+// on the downsampling layers of a ResNet).  With more than one tap the phases are several small launches
+// each, and the zero-insertion form on the LDS kernel is the faster one at the sizes measured
+// (3x3 stride 2, 32-128 channels: 0.08-0.11 ms against 0.13-0.19 ms); PHX_TUNE_PHASE=1 sends every strided
+// input gradient through the phases, PHX_TUNE_PHASE=0 none.
+static bool dgrad_by_phases(const Problem& p) {
+    if ((p.sh == 1 && p.sw == 1) || p.sh * p.sw > 16 || is_empty(p)) return false;
+    if (const char* e = getenv("PHX_TUNE_PHASE")) return atoi(e) != 0;
+    return p.kh == 1 && p.kw == 1;
+}
+
+static Corr phase_corr(const Problem& p, const PhaseAxis& ah, const PhaseAxis& aw) {
+    Corr c{p.n, p.co, p.ho, p.wo, p.ci, ah.size, aw.size, ah.taps, aw.taps, 1, 1, ah.dil, aw.dil, ah.pad, aw.pad, 1, 1,
+           ah.kmax, ah.kstep, aw.kmax, aw.kstep};
+    // a single tap over the whole gradient plane (strided pointwise convolutions): one long row per image
+    if (ah.taps == 1 && aw.taps == 1 && !ah.pad && !aw.pad && ah.size == p.ho && aw.size == p.wo) {
+        c.Win = p.ho * p.wo; c.Hin = 1; c.Wout = c.Win; c.Hout = 1;
+    }
+    return c;
+}
+
 static size_t workspace_plain(const Problem& p, int pass) {
     if (is_empty(p)) return 0;
     if (pass == PHX_PASS_BWD_WEIGHTS) {
@@ -573,6 +629,20 @@ static size_t workspace_plain(const Problem& p, int pass) {
     int pw = 0;
     Corr c;
     FwdPlan pl;
+    if (pass == PHX_PASS_BWD_DATA && dgrad_by_phases(p)) {
+        // phase buffers (together the size of dx, each rounded up) + the largest packed sub-filter
+        const size_t esize = p.dtype == PHX_F32 ? 4 : 2;
+        size_t bufs = 0, wpk = 0;
+        for (int a = 0; a < p.sh; ++a)
+            for (int b = 0; b < p.sw; ++b) {
+                const PhaseAxis ah = phase_axis(a, p.h, p.kh, p.dh, p.sh, p.pt), aw = phase_axis(b, p.w, p.kw, p.dw, p.sw, p.pl);
+                if (!ah.taps || !aw.taps || !ah.size || !aw.size) continue;
+                bufs += align_up((size_t)4 * p.n * p.ci * ah.size * aw.size * esize, 256);
+                if (!plan_corr(phase_corr(p, ah, aw), p.mode, use_f16_mfma(p, pass), c, pl, pw)) return 0;
+                wpk = std::max(wpk, align_up(pl.wpk_bytes, 256));
+            }
+        return bufs + wpk;
+    }
     return plan_corr((pass == PHX_PASS_FWD) ? corr_forward(p) : corr_dgrad(p), p.mode, use_f16_mfma(p, pass), c, pl, pw)
                ? align_up(pl.wpk_bytes, 256)
                : 0;
@@ -658,6 +728,35 @@ static int do_fwd(const Problem& p, hipStream_t st, const void* x, const void* w
 static int do_bwd_data(const Problem& p, hipStream_t st, const void* g, const void* w, void* dx, void* ws, size_t wsb) {
     if (is_empty(p)) return PHX_OK;
     if (!g || !w || !dx) return PHX_ERR_INVALID_ARGUMENT;
+    if (dgrad_by_phases(p)) {
+        const size_t esize = p.dtype == PHX_F32 ? 4 : 2;
+        PhaseMergeArgs m;
+        m.buf = ws; m.dx = dx; m.planes = 4L * p.n * p.ci; m.H = p.h; m.W = p.w; m.sh = p.sh; m.sw = p.sw;
+        size_t bufs = 0;
+        for (int i = 0; i < 16; ++i) m.off[i] = -1;
+        for (int a = 0; a < p.sh; ++a)
+            for (int b = 0; b < p.sw; ++b) {
+                const PhaseAxis ah = phase_axis(a, p.h, p.kh, p.dh, p.sh, p.pt), aw = phase_axis(b, p.w, p.kw, p.dw, p.sw, p.pl);
+                if (!ah.taps || !aw.taps || !ah.size || !aw.size) continue;
+                m.off[a * p.sw + b] = (long)(bufs / esize);
+                bufs += align_up((size_t)4 * p.n * p.ci * ah.size * aw.size * esize, 256);
+            }
+        if (wsb < bufs || !ws) return PHX_ERR_WORKSPACE;
+        char* base = static_cast<char*>(ws);
+        g_name_prefix = "phase_";
+        for (int a = 0; a < p.sh; ++a)
+            for (int b = 0; b < p.sw; ++b) {
+                if (m.off[a * p.sw + b] < 0) continue;
+                const PhaseAxis ah = phase_axis(a, p.h, p.kh, p.dh, p.sh, p.pt), aw = phase_axis(b, p.w, p.kw, p.dw, p.sw, p.pl);
+                const int rc = run_corr(p, phase_corr(p, ah, aw), MAP_DGRAD, st, g, w, nullptr,
+                                        base + m.off[a * p.sw + b] * esize, base + bufs, wsb - bufs);
+                if (rc != PHX_OK) { g_name_prefix = ""; return rc; }
+            }
+        g_name_prefix = "";
+        launch_phase_merge(p.dtype == PHX_F16, m, st);
+        PHX_HIP(hipGetLastError());
+        return PHX_OK;
+    }
     const Corr c = corr_dgrad(p);
     return run_corr(p, c, MAP_DGRAD, st, g, w, nullptr, dx, ws, wsb);
 }

@@ -318,6 +318,32 @@ def test_factorized_pointwise_on_fp16_matrix_cores(case, monkeypatch):
         assert_close(dx.cpu().numpy(), want_dx, dtype, "dgrad " + tag)
 
 
+STRIDED = [c for c in FP16_CASES if c[0] in ("k3_s2", "pw_s2", "k7_s2", "k3_s2_c4", "k5_s2_valid", "k3_s3", "k32_s21")]
+
+
+@pytest.mark.parametrize("variant", ["phases", "zero_insertion", "zero_insertion_factorized"])
+@pytest.mark.parametrize("dtype,policy", [(torch.float32, "fp32"), (torch.float16, "full16")], ids=["f32", "f16"])
+@pytest.mark.parametrize("mode", [16, 8])
+@pytest.mark.parametrize("case", STRIDED, ids=lambda c: c[0])
+def test_strided_input_gradient_variants(case, mode, dtype, policy, variant, monkeypatch):
+    """The input gradient of a strided convolution has two implementations, per-phase dense correlations merged
+    into dx and zero insertion in the staged window (on fp16 matrix cores in 16-product form unless the
+    factorized one is forced); the planner picks by shape, the environment overrides select each."""
+    name, n, ci, co, h, w, kh, kw, stride, dilation, padding = case
+    scale = 1.0 if dtype == torch.float32 else 0.5
+    g, x, wt, b, gr = make_inputs(hash(name) % 1000 + 5, n, ci, co, h, w, kh, kw, stride, dilation, padding, dtype, scale)
+    monkeypatch.setenv("PHX_TUNE_PHASE", "1" if variant == "phases" else "0")
+    if variant == "zero_insertion_factorized":
+        monkeypatch.setenv("PHX_TUNE_ZI8", "1")
+    desc = phx.Conv2DDescriptor(x.shape, wt.shape, stride, dilation, padding, dtype=dtype, context=Ctx(mode, policy))
+    xd, wd, gd = (torch.from_numpy(a).cuda() for a in (x, wt, gr))
+    _, dx = phx.conv2d_bwd(xd, wd, gd, desc)
+    k = capi.last_kernel_name()
+    assert k.startswith("phase_") == (variant == "phases"), k
+    _, want_dx = oracle.conv2d_bwd(g, x.astype(np.float64), wt.astype(np.float64), gr.astype(np.float64), "hamilton")
+    assert_close(dx.cpu().numpy(), want_dx, dtype, "dgrad " + k)
+
+
 @pytest.mark.parametrize("policy", ["full16", "fp32"])
 @pytest.mark.parametrize("mode", [16, 8])
 def test_dense_fp16(mode, policy):
