@@ -512,11 +512,7 @@ __global__ void __launch_bounds__(WG_THREADS, (MODE == 16 && NTW == 1) ? 2 : 1) 
     // components requested a block earlier still.  Where the next group works on the same staged chunk
     // that pipeline runs on across the group boundary (CARRY; it needs an even number of blocks per group
     // so that the register double buffers keep their parity).
-#ifdef PHX_EXP_NOCARRY
-    constexpr bool CARRY = false;
-#else
     constexpr bool CARRY = MODE == 8 && (TG * NTW) % 2 == 0;
-#endif
     f16x8 xf[2][4], Lf[MODE == 8 ? 2 : 1][8], Lt[4];
     bool carried = false;      // the previous group left this group's first lanes and components in registers
     // one flat loop over (chunk, filter group) steps: a single loop keeps the accumulators in place
