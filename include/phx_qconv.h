@@ -77,6 +77,8 @@ typedef struct phx_qconv_desc {
                               imaginary parts, filters, outputs and output gradients stay quaternion-valued, has_bias
                               must be 0 (src/conv2d.hpp:125-127) and
                               phx_qconv2d_bwd_data is refused as the reference refuses it (src/conv2d.hpp:394-398) */
+    int32_t groups;        /* grouped convolution: ci and co are the totals, both multiples of groups; the filter is
+                              [4, co, ci/groups, kh, kw] (OHWI: [4, co, kh, kw, ci/groups]); 0 or 1 = ungrouped */
 } phx_qconv_desc;
 
 /* Quaternion Dense geometry (src/backend/dense_descriptor.hpp:11-59); filter layout is IO. */

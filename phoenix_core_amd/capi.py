@@ -40,7 +40,7 @@ class QConvDesc(ctypes.Structure):
     _fields_ = [(k, ctypes.c_int32) for k in (
         "dtype", "n", "ci", "co", "h", "w", "kh", "kw", "stride_h", "stride_w", "dilation_h", "dilation_w",
         "pad_top", "pad_left", "pad_bottom", "pad_right", "filter_layout", "product_mode", "fp16_policy", "has_bias",
-        "real_input")]
+        "real_input", "groups")]
 
 
 class QDenseDesc(ctypes.Structure):

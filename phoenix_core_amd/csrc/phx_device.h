@@ -266,6 +266,7 @@ struct TileSrc {
     const void* base;
     long comp_stride;  // elements between components
     int N, C, Hd, Wd;  // stored dims per component
+    int Cs;            // channels per image in memory (>= C: a grouped convolution sees a slice of C channels from base on)
     int uh, uw;        // zero-insertion factors (1 = none)
     int ncomp;         // components present in memory: 4, or 1 for a real-valued tensor (components 1..3 read as zero)
     int pw;            // pointwise trick: window row r holds channels (chunk*pw + r)*16.. of the single image row (0 = off)
@@ -298,7 +299,7 @@ __device__ __forceinline__ StagePos make_stage_pos(const TileSrc& s, int n0, int
     if (s.uw > 1) { ok = ok && (vw % s.uw == 0); vw /= s.uw; }
     ok = ok && vh < s.Hd && vw < s.Wd;
     sp.valid = ok;
-    sp.goff = ok ? ((long)(n0 + nb) * s.C * s.Hd + vh) * s.Wd + vw : 0;
+    sp.goff = ok ? ((long)(n0 + nb) * s.Cs * s.Hd + vh) * s.Wd + vw : 0;
     return sp;
 }
 

@@ -70,7 +70,7 @@ __device__ __forceinline__ StagePairPos make_stage_pairpos(const TileSrc& s, int
     sp.pos = (nb * HTH + hr) * HTWe + 2 * hcp;
     const bool ok = sp.inwin && (n0 + nb) < s.N && vh >= 0 && vh < s.Hd && vw >= 0 && vw + 1 < s.Wd;
     sp.valid = ok;
-    sp.goff = ok ? ((long)(n0 + nb) * s.C * s.Hd + vh) * s.Wd + vw : 0;
+    sp.goff = ok ? ((long)(n0 + nb) * s.Cs * s.Hd + vh) * s.Wd + vw : 0;
     return sp;
 }
 
@@ -151,7 +151,7 @@ __global__ void __launch_bounds__(WG_THREADS, (MODE == 8 || NTW == 1) ? 2 : 1) q
         const int r = rem / P.TW, c = rem - r * P.TW;
         pvalid[t] = nb < P.NB && (n0 + nb) < P.in.N && (ho0 + r) < P.Hout && (wo0 + c) < P.Wout;
         poff[t] = pvalid[t] ? (nb * P.HTH + r * P.sh) * P.HTW + c * P.sw + colshift : colshift;
-        oaddr[t] = ((long)(n0 + nb) * P.Cout * P.Hout + (ho0 + r)) * P.Wout + (wo0 + c);
+        oaddr[t] = ((long)(n0 + nb) * P.CoutS * P.Hout + (ho0 + r)) * P.Wout + (wo0 + c);
     }
 
     f32x16 acc[NTW][NACC];
@@ -338,8 +338,8 @@ __device__ __forceinline__ StageChunk make_stage_chunk(const TileSrc& s, int n0,
     sc.bits = sc.live ? interval_bits(-vw0, s.Wd - vw0) : 0u;
     const _Float16* base = static_cast<const _Float16*>(s.base);
     const long plane = (long)s.Hd * s.Wd;
-    sc.ptr = base + p * s.comp_stride + ((long)(n0 + nb) * s.C * s.Hd + vh) * s.Wd + vw0;
-    const _Float16* end = base + (long)(s.ncomp - 1) * s.comp_stride + (long)s.N * s.C * plane;
+    sc.ptr = base + p * s.comp_stride + ((long)(n0 + nb) * s.Cs * s.Hd + vh) * s.Wd + vw0;
+    const _Float16* end = base + (long)(s.ncomp - 1) * s.comp_stride + ((long)(s.N - 1) * s.Cs + s.C) * plane;
     sc.careful = sc.live && (sc.ptr < base || sc.ptr + (long)(s.C - 1) * plane + 8 > end);
     const int e0 = row * HTW + cc * 8;
     sc.ent = (sc.task ? u : 0) * HPp + e0;
@@ -462,7 +462,7 @@ __global__ void __launch_bounds__(WG_THREADS, (MODE == 16 && NTW == 1) ? 2 : 1) 
         const int r = rem / P.TW, c = rem - r * P.TW;
         pvalid[t] = nb < P.NB && (n0 + nb) < P.in.N && (ho0 + r) < P.Hout && (wo0 + c) < P.Wout;
         poff[t] = pvalid[t] ? (nb * P.HTH + r * P.sh) * P.HTW + c * P.sw : 0;
-        oaddr[t] = ((long)(n0 + nb) * P.Cout * P.Hout + (ho0 + r)) * P.Wout + (wo0 + c);
+        oaddr[t] = ((long)(n0 + nb) * P.CoutS * P.Hout + (ho0 + r)) * P.Wout + (wo0 + c);
     }
 
     f32x16 acc[NTW][NW];
@@ -897,8 +897,9 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_wgrad_f16_kernel(const Wgrad
     // reduction space or on padding rows load from offset 0 and are masked to zero; channels beyond
     // the tensor re-read its last channel (their rows of the partial result are never reduced).
     // 32-bit element offsets inside one component: the host guarantees they fit
-    const int gimg = P.g.C * (int)gplane, ximg = P.x.C * (int)xplane;
-    const int gcomp = P.g.N * gimg, xcomp = P.x.N * ximg;  // elements per component
+    const int gimg = P.g.Cs * (int)gplane, ximg = P.x.Cs * (int)xplane;
+    // elements from the base to the end of the last image's channels, per component
+    const int gcomp = (P.g.N - 1) * gimg + P.g.C * (int)gplane, xcomp = (P.x.N - 1) * ximg + P.x.C * (int)xplane;
     const int xnc = P.x.ncomp;                              // 1 for a real-valued input: components 1..3 are zero
     int gch[MT], xch[NT];
 #pragma unroll
@@ -971,7 +972,7 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_wgrad_f16_kernel(const Wgrad
         for (int e = 0; e < GE; ++e) {
             const int q = e / MT, cc = (e % MT) * 32;
             const int ch = co_first + cc < P.g.C ? co_first + cc : P.g.C - 1;
-            const _Float16* src = gbase + q * P.g.comp_stride + (((long)c.n * P.g.C + ch) * Ho + c.ho) * Wo + c.wo0;
+            const _Float16* src = gbase + q * P.g.comp_stride + (((long)c.n * P.g.Cs + ch) * Ho + c.ho) * Wo + c.wo0;
             _Float16 v[8];
 #pragma unroll
             for (int i = 0; i < 8; ++i) v[i] = (c.live && c.wo0 + i < Wo) ? src[i] : (_Float16)0;
@@ -982,7 +983,7 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_wgrad_f16_kernel(const Wgrad
         for (int e = 0; e < XE; ++e) {
             const int q = e / NT, cc = (e % NT) * 32;
             const int ch = ci_first + cc < P.x.C ? ci_first + cc : P.x.C - 1;
-            const _Float16* src = xbase + q * P.x.comp_stride + (((long)c.n * P.x.C + ch) * H + hi) * W;
+            const _Float16* src = xbase + q * P.x.comp_stride + (((long)c.n * P.x.Cs + ch) * H + hi) * W;
             _Float16 w[NEL];
 #pragma unroll
             for (int k = 0; k < NEL; ++k) {

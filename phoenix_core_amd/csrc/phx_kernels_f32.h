@@ -21,6 +21,7 @@ struct ConvArgs {
     void* out;
     long out_cs;        // elements between output components
     int Cout, Hout, Wout;
+    int CoutS;          // output channels per image in memory (>= Cout: grouped convolutions write a slice); also the bias stride
     int taps, Kw;       // filter taps (Kh*Kw) and filter width
     int dh, dw, sh, sw; // dilation and stride of the correlation
     int pt, pl;         // virtual input row of output row 0, tap 0, is -pt (same for columns)
@@ -114,7 +115,7 @@ __device__ __forceinline__ void conv_epilogue(const ConvArgs& P, const f32x16 (&
                 const int co = co_base + 8 * rq + k;
                 if (bias && co < P.Cout) {
 #pragma unroll
-                    for (int q = 0; q < 4; ++q) y[k][q] += ldf<TS>(bias + q * P.Cout + co);
+                    for (int q = 0; q < 4; ++q) y[k][q] += ldf<TS>(bias + q * P.CoutS + co);
                 }
             }
             if (P.vec == 4) {
@@ -184,10 +185,10 @@ __device__ __forceinline__ StageVec make_stage_vec(const TileSrc& s, int n0, int
     const int vh = h0 + hr, vw0 = w0 + col;
     sv.live = sv.lpos < HP && nb < NB && (n0 + nb) < s.N && vh >= 0 && vh < s.Hd;
     sv.bits = sv.live ? interval_bits<4>(-vw0, s.Wd - vw0) : 0u;
-    sv.goff = ((long)(n0 + nb) * s.C * s.Hd + vh) * s.Wd + vw0;
+    sv.goff = ((long)(n0 + nb) * s.Cs * s.Hd + vh) * s.Wd + vw0;
     const long plane = (long)s.Hd * s.Wd;
     const long last = (long)(s.ncomp - 1) * s.comp_stride;  // offset of the last component in memory
-    const long total = last + (long)s.N * s.C * plane;
+    const long total = last + ((long)(s.N - 1) * s.Cs + s.C) * plane;
     sv.careful = sv.live && (sv.goff < 0 || sv.goff + last + (long)(s.C - 1) * plane + 4 > total);
     return sv;
 }
@@ -323,7 +324,7 @@ __global__ void __launch_bounds__(WG_THREADS, (MODE == 8 || NTW == 1) ? 2 : 1) q
         const int r = rem / P.TW, c = rem - r * P.TW;
         pvalid[t] = nb < P.NB && (n0 + nb) < P.in.N && (ho0 + r) < P.Hout && (wo0 + c) < P.Wout;
         poff[t] = pvalid[t] ? (nb * P.HTH + r * P.sh) * P.HTW + c * P.sw : 0;
-        oaddr[t] = ((long)(n0 + nb) * P.Cout * P.Hout + (ho0 + r)) * P.Wout + (wo0 + c);
+        oaddr[t] = ((long)(n0 + nb) * P.CoutS * P.Hout + (ho0 + r)) * P.Wout + (wo0 + c);
     }
 
     f32x16 acc[NTW][NACC];

@@ -63,6 +63,9 @@ struct Problem {
     FilterStrides fs;
     bool has_bias;
     bool real_input;  // x (and dx) are real-valued [n, ci, h, w]: imaginary components are zero and not stored
+    // Grouped convolution: ci / co above are one group's channels, the tensors hold ci_mem / co_mem channels per
+    // image and `groups` such slices side by side (ci_mem == ci, co_mem == co without groups)
+    int groups, ci_mem, co_mem;
 };
 
 static int out_size(int in, int k, int d, int s, int before, int after) {
@@ -84,17 +87,20 @@ static int problem_from_conv(const phx_qconv_desc* d, Problem& p) {
     if (d->real_input != 0 && d->real_input != 1) return PHX_ERR_INVALID_ARGUMENT;
     // "Bias addition is not supported for type0 inputs" (src/conv2d.hpp:125-127)
     if (d->real_input && d->has_bias) return PHX_ERR_INVALID_ARGUMENT;
+    const int groups = d->groups > 1 ? d->groups : 1;
+    if (d->ci % groups || d->co % groups) return PHX_ERR_INVALID_ARGUMENT;
     p.dtype = d->dtype;
     p.mode = d->product_mode;
     p.policy = d->fp16_policy;
-    p.n = d->n; p.ci = d->ci; p.co = d->co; p.h = d->h; p.w = d->w; p.kh = d->kh; p.kw = d->kw;
+    p.groups = groups; p.ci_mem = d->ci; p.co_mem = d->co;
+    p.n = d->n; p.ci = d->ci / groups; p.co = d->co / groups; p.h = d->h; p.w = d->w; p.kh = d->kh; p.kw = d->kw;
     p.sh = d->stride_h; p.sw = d->stride_w; p.dh = d->dilation_h; p.dw = d->dilation_w;
     p.pt = d->pad_top; p.pl = d->pad_left; p.pb = d->pad_bottom; p.pr = d->pad_right;
     p.ho = out_size(p.h, p.kh, p.dh, p.sh, p.pt, p.pb);
     p.wo = out_size(p.w, p.kw, p.dw, p.sw, p.pl, p.pr);
     if ((p.h > 0 && p.ho <= 0) || (p.w > 0 && p.wo <= 0)) return PHX_ERR_INVALID_ARGUMENT;
     const long taps = (long)p.kh * p.kw;
-    p.fs.wcs = (long)p.co * p.ci * taps;
+    p.fs.wcs = (long)p.co_mem * p.ci * taps;  // filter [4][co_mem][ci per group][kh][kw]
     if (d->filter_layout == PHX_OIHW) {
         p.fs.so = p.ci * taps; p.fs.si = taps; p.fs.skh = p.kw; p.fs.skw = 1;
     } else {  // OHWI
@@ -118,6 +124,7 @@ static int problem_from_dense(const phx_qdense_desc* d, Problem& p) {
     p.fs.wcs = (long)p.ci * p.co; p.fs.so = 1; p.fs.si = p.co; p.fs.skh = 0; p.fs.skw = 0;
     p.has_bias = d->has_bias != 0;
     p.real_input = false;
+    p.groups = 1; p.ci_mem = p.ci; p.co_mem = p.co;
     return PHX_OK;
 }
 
@@ -368,13 +375,15 @@ static int run_corr(const Problem& p, const Corr& creal, int map, hipStream_t st
     const int pack_blocks = (int)std::min<long>((pack_items + WG_THREADS - 1) / WG_THREADS, 4096);
 
     ConvArgs a;
-    a.in.base = in; a.in.comp_stride = (long)c.N * creal.Cin * c.Hin * c.Win;
+    // channels per image in memory on the input and output side of this correlation (grouped convolutions: slices)
+    const int cin_mem = (map == MAP_FWD) ? p.ci_mem : p.co_mem, cout_mem = (map == MAP_FWD) ? p.co_mem : p.ci_mem;
+    a.in.base = in; a.in.comp_stride = (long)c.N * cin_mem * c.Hin * c.Win; a.in.Cs = cin_mem;
     a.in.N = c.N; a.in.C = creal.Cin; a.in.Hd = c.Hin; a.in.Wd = c.Win; a.in.uh = c.uh; a.in.uw = c.uw; a.in.pw = pw;
     // real-valued input: the forward pass reads one component, the others are zero
     a.in.ncomp = (p.real_input && map == MAP_FWD) ? 1 : 4;
     a.wpk = ws; a.bias = bias; a.out = out;
-    a.out_cs = (long)c.N * c.Cout * c.Hout * c.Wout;
-    a.Cout = c.Cout; a.Hout = c.Hout; a.Wout = c.Wout;
+    a.out_cs = (long)c.N * cout_mem * c.Hout * c.Wout;
+    a.Cout = c.Cout; a.CoutS = cout_mem; a.Hout = c.Hout; a.Wout = c.Wout;
     a.taps = c.Kh * c.Kw; a.Kw = c.Kw; a.dh = c.dh; a.dw = c.dw; a.sh = c.sh; a.sw = c.sw; a.pt = c.pt; a.pl = c.pl;
     a.NB = pl.NB; a.TH = pl.TH; a.TW = pl.TW; a.HTH = pl.HTH; a.HTW = pl.HTW; a.HP = pl.HP; a.HPp = pl.HPp;
     a.tiles_n = pl.tiles_n; a.tiles_h = pl.tiles_h; a.tiles_w = pl.tiles_w; a.co_tiles = pl.co_tiles;
@@ -515,8 +524,8 @@ static bool plan_wgrad_f16(const Problem& p, WgPlan& best) {
 static bool wgrad_on_f16_mfma(const Problem& p) {
     // the kernel addresses one component with 32-bit element offsets
     const long lim = (1L << 31) - 64;
-    return use_f16_mfma(p, PHX_PASS_BWD_WEIGHTS) && (p.sw == 1 || p.sw == 2) && (long)p.n * p.ci * p.h * p.w < lim &&
-           (long)p.n * p.co * p.ho * p.wo < lim;
+    return use_f16_mfma(p, PHX_PASS_BWD_WEIGHTS) && (p.sw == 1 || p.sw == 2) && (long)p.n * p.ci_mem * p.h * p.w < lim &&
+           (long)p.n * p.co_mem * p.ho * p.wo < lim;
 }
 
 static bool plan_wgrad(const Problem& p, bool f16mfma, WgPlan& best) {
@@ -530,9 +539,9 @@ static int run_wgrad(const Problem& p, hipStream_t st, const void* x, const void
     if (!plan_wgrad(p, f16, pl)) return PHX_ERR_NOT_SUPPORTED;
     if (ws_bytes < pl.partial_bytes || !ws) return PHX_ERR_WORKSPACE;
     WgradArgs a;
-    a.x.base = x; a.x.comp_stride = (long)p.n * p.ci * p.h * p.w; a.x.N = p.n; a.x.C = p.ci; a.x.Hd = p.h; a.x.Wd = p.w;
+    a.x.base = x; a.x.comp_stride = (long)p.n * p.ci_mem * p.h * p.w; a.x.N = p.n; a.x.C = p.ci; a.x.Cs = p.ci_mem; a.x.Hd = p.h; a.x.Wd = p.w;
     a.x.uh = a.x.uw = 1; a.x.pw = 0; a.x.ncomp = p.real_input ? 1 : 4;
-    a.g.base = g; a.g.comp_stride = (long)p.n * p.co * p.ho * p.wo; a.g.N = p.n; a.g.C = p.co; a.g.Hd = p.ho; a.g.Wd = p.wo;
+    a.g.base = g; a.g.comp_stride = (long)p.n * p.co_mem * p.ho * p.wo; a.g.N = p.n; a.g.C = p.co; a.g.Cs = p.co_mem; a.g.Hd = p.ho; a.g.Wd = p.wo;
     a.g.uh = a.g.uw = 1; a.g.pw = 0; a.g.ncomp = 4;
     a.partial = static_cast<float*>(ws);
     a.Kh = p.kh; a.Kw = p.kw; a.sh = p.sh; a.sw = p.sw; a.dh = p.dh; a.dw = p.dw; a.pt = p.pt; a.pl = p.pl;
@@ -605,7 +614,7 @@ static PhaseAxis phase_axis(int a, int extent, int k, int d, int s, int pad_befo
 // (3x3 stride 2, 32-128 channels: 0.08-0.11 ms against 0.13-0.19 ms); PHX_TUNE_PHASE=1 sends every strided
 // input gradient through the phases, PHX_TUNE_PHASE=0 none.
 static bool dgrad_by_phases(const Problem& p) {
-    if ((p.sh == 1 && p.sw == 1) || p.sh * p.sw > 16 || is_empty(p)) return false;
+    if ((p.sh == 1 && p.sw == 1) || p.sh * p.sw > 16 || is_empty(p) || p.groups > 1) return false;
     if (const char* e = getenv("PHX_TUNE_PHASE")) return atoi(e) != 0;
     return p.kh == 1 && p.kw == 1;
 }
@@ -660,12 +669,13 @@ static int floordiv(int a, int b) { return a >= 0 ? a / b : -((-a + b - 1) / b);
 
 static bool s2d_view(const Problem& p, S2dView& v) {
     if (p.sh != 2 || p.sw != 2 || p.dh != 1 || p.dw != 1 || p.ci > 4 || (p.kh < 3 && p.kw < 3) || is_empty(p)) return false;
+    if (p.groups > 1) return false;  // the rearranged copies are laid out for whole tensors
     if (getenv("PHX_TUNE_NOS2D")) return false;
     const int aminh = floordiv(-p.pt, 2), amaxh = floordiv(p.kh - 1 - p.pt, 2);
     const int aminw = floordiv(-p.pl, 2), amaxw = floordiv(p.kw - 1 - p.pl, 2);
     Problem& q = v.q;
     q = p;
-    q.ci = 4 * p.ci;
+    q.ci = 4 * p.ci; q.ci_mem = q.ci;
     q.h = (p.h + 1) / 2; q.w = (p.w + 1) / 2;
     q.kh = amaxh - aminh + 1; q.kw = amaxw - aminw + 1;
     q.sh = q.sw = 1;
@@ -837,6 +847,25 @@ int phx_profile_collect(float* milliseconds, int max_count, int* count) {
     return PHX_OK;
 }
 
+// Grouped convolution (groups passed on to the scalar convolutions in the reference,
+// src/backend/onednn/conv2d.hpp:116-137): the groups are independent convolutions on channel slices of the
+// same tensors; each runs as a problem of its own whose tensors are views (byte offsets below) with the whole
+// tensors' image strides.  An empty problem runs once: it only zeroes the filter gradient, all of it.
+struct GroupOffsets {
+    size_t x, y, w, b;  // bytes from one group's slice to the next: input, output, filter, bias
+    int runs;
+    explicit GroupOffsets(const Problem& p) {
+        const size_t esize = p.dtype == PHX_F32 ? 4 : 2;
+        x = (size_t)p.ci * p.h * p.w * esize;
+        y = (size_t)p.co * p.ho * p.wo * esize;
+        w = (size_t)p.co * p.fs.so * esize;
+        b = (size_t)p.co * esize;
+        runs = is_empty(p) ? 1 : p.groups;
+    }
+    static const void* at(const void* ptr, size_t off) { return ptr ? static_cast<const char*>(ptr) + off : nullptr; }
+    static void* at(void* ptr, size_t off) { return ptr ? static_cast<char*>(ptr) + off : nullptr; }
+};
+
 int phx_qconv2d_output_hw(const phx_qconv_desc* desc, int32_t* ho, int32_t* wo) {
     Problem p;
     const int rc = problem_from_conv(desc, p);
@@ -863,7 +892,14 @@ int phx_qconv2d_fwd(const phx_qconv_desc* desc, phx_stream_t stream, const void*
     Problem p;
     const int rc = problem_from_conv(desc, p);
     if (rc != PHX_OK) return rc;
-    return do_fwd(p, static_cast<hipStream_t>(stream), x, w, bias_or_null, y, workspace, workspace_bytes);
+    const GroupOffsets o(p);
+    for (int g = 0; g < o.runs; ++g) {
+        const int grc = do_fwd(p, static_cast<hipStream_t>(stream), o.at(x, g * o.x), o.at(w, g * o.w),
+                               bias_or_null ? o.at(bias_or_null, g * o.b) : nullptr, o.at(y, g * o.y), workspace,
+                               workspace_bytes);
+        if (grc != PHX_OK) return grc;
+    }
+    return PHX_OK;
 }
 
 int phx_qconv2d_bwd_data(const phx_qconv_desc* desc, phx_stream_t stream, const void* grad, const void* w, void* dx,
@@ -874,7 +910,13 @@ int phx_qconv2d_bwd_data(const phx_qconv_desc* desc, phx_stream_t stream, const 
     // the gradient with respect to a real-valued input has imaginary parts that are stored nowhere;
     // the reference refuses the request likewise (src/conv2d.hpp:394-398)
     if (p.real_input) return PHX_ERR_INVALID_ARGUMENT;
-    return do_bwd_data(p, static_cast<hipStream_t>(stream), grad, w, dx, workspace, workspace_bytes);
+    const GroupOffsets o(p);
+    for (int g = 0; g < o.runs; ++g) {
+        const int grc = do_bwd_data(p, static_cast<hipStream_t>(stream), o.at(grad, g * o.y), o.at(w, g * o.w),
+                                    o.at(dx, g * o.x), workspace, workspace_bytes);
+        if (grc != PHX_OK) return grc;
+    }
+    return PHX_OK;
 }
 
 int phx_qconv2d_bwd_weights(const phx_qconv_desc* desc, phx_stream_t stream, const void* x, const void* grad, void* dw,
@@ -882,7 +924,13 @@ int phx_qconv2d_bwd_weights(const phx_qconv_desc* desc, phx_stream_t stream, con
     Problem p;
     const int rc = problem_from_conv(desc, p);
     if (rc != PHX_OK) return rc;
-    return do_bwd_weights(p, static_cast<hipStream_t>(stream), x, grad, dw, workspace, workspace_bytes);
+    const GroupOffsets o(p);
+    for (int g = 0; g < o.runs; ++g) {
+        const int grc = do_bwd_weights(p, static_cast<hipStream_t>(stream), o.at(x, g * o.x), o.at(grad, g * o.y),
+                                       o.at(dw, g * o.w), workspace, workspace_bytes);
+        if (grc != PHX_OK) return grc;
+    }
+    return PHX_OK;
 }
 
 int phx_qdense_fwd(const phx_qdense_desc* desc, phx_stream_t stream, const void* x, const void* w,

@@ -712,7 +712,6 @@ inline phx_qconv_desc makeConvDesc(const Conv2DDescriptor& d, Context& ctx, int 
     if (d.getAlgebra() != Algebra::QUATERNION)
         throw std::runtime_error("Only the quaternion algebra is built for device::HIP");
     if (d.getDataFormat() != DataFormat::NCHW) throw std::runtime_error("device::HIP runs NCHW tensors only");
-    if (d.getGroups() != 1) throw std::runtime_error("Grouped quaternion convolution is not built for device::HIP");
     const FilterLayout fl = d.getFilterLayout();
     if (fl != FilterLayout::OIHW && fl != FilterLayout::OHWI)
         throw std::runtime_error("device::HIP takes OIHW or OHWI filters");
@@ -723,7 +722,8 @@ inline phx_qconv_desc makeConvDesc(const Conv2DDescriptor& d, Context& ctx, int 
     c.dtype = dtype;
     const bool real = d.isRealValuedInput();  // [n, ci, h, w] without imaginary components
     c.n = real ? in[0] : in[0] / 4;
-    c.ci = filter.numInputChannels(w);
+    c.groups = d.getGroups();
+    c.ci = filter.numInputChannels(w) * c.groups;  // the filter holds one group's input channels
     c.co = filter.numOutputChannels(w);
     c.h = in[2];
     c.w = in[3];

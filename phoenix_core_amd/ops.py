@@ -95,8 +95,8 @@ class Conv2DDescriptor:
             raise ValueError("Five-dimensional filter tensor expected")
         if filter_shape[0] != 4:
             raise ValueError("First filter dimension mismatch, got %d" % filter_shape[0])
-        if groups != 1:
-            raise NotImplementedError("grouped quaternion convolution is not built")
+        if groups < 1:
+            raise ValueError("groups must be positive")
         if not real_valued_input and input_shape[0] % 4:
             raise ValueError("Cannot split %d onto 4 parts" % input_shape[0])
         if filter_layout == "OIHW":
@@ -105,8 +105,13 @@ class Conv2DDescriptor:
             _, co, kh, kw, ci = filter_shape
         else:
             raise ValueError("Unsupported Conv2D filter layout")
+        # grouped convolution: the filter holds the input channels of one group (src/backend/conv2d_descriptor.hpp)
+        ci *= groups
         if input_shape[1] != ci:
             raise ValueError("input channels %d do not match the filter's %d" % (input_shape[1], ci))
+        if co % groups:
+            raise ValueError("output channels %d are not a multiple of %d groups" % (co, groups))
+        self.groups = groups
         self.context = context or default_context()
         self.input_shape = tuple(input_shape)
         self.filter_shape = tuple(filter_shape)
@@ -135,7 +140,7 @@ class Conv2DDescriptor:
             _DTYPES[dtype], n4 // 4, ci, co, h, w, kh, kw, self.stride[0], self.stride[1], self.dilation[0],
             self.dilation[1], pt, pl, pb, pr, capi.PHX_OIHW if filter_layout == "OIHW" else capi.PHX_OHWI,
             self.context.product_mode, self.context.fp16_policy, int(self.use_bias and not self.real_valued_input),
-            int(self.real_valued_input))
+            int(self.real_valued_input), groups)
 
     def workspace_bytes(self, which):
         return capi.lib().phx_qconv2d_workspace_bytes(ctypes.byref(self.c), which)
