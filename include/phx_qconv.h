@@ -37,6 +37,11 @@ enum phx_dtype { PHX_F32 = 0, PHX_F16 = 1 };
 
 enum phx_filter_layout { PHX_OIHW = 0, PHX_OHWI = 1 };
 
+/* Layout of the activation tensors (DataFormat, src/backend/types.hpp:85; dimension numbers
+ * src/backend/tensor.hpp:17-31).  The kernels compute on channels-first planes; a channels-last call
+ * transposes its activations into the workspace on the way in and out (two extra passes over each tensor). */
+enum phx_data_format { PHX_NCHW = 0, PHX_NHWC = 1 };
+
 /* Which Hamilton-product formulation runs.
  * Mirrors Context::preferSpeedToMemory() (src/backend/backend.hpp:58): the reference's default is
  * the factorized 8-product path (src/conv2d.hpp:167-234), UPSTRIDE_MEMORY_OPTIMIZED=1 selects the
@@ -79,6 +84,8 @@ typedef struct phx_qconv_desc {
                               phx_qconv2d_bwd_data is refused as the reference refuses it (src/conv2d.hpp:394-398) */
     int32_t groups;        /* grouped convolution: ci and co are the totals, both multiples of groups; the filter is
                               [4, co, ci/groups, kh, kw] (OHWI: [4, co, kh, kw, ci/groups]); 0 or 1 = ungrouped */
+    int32_t data_format;   /* phx_data_format of x, y and their gradients: PHX_NCHW [4n, c, h, w] or PHX_NHWC
+                              [4n, h, w, c]; filters and bias are unaffected (filter_layout is separate) */
 } phx_qconv_desc;
 
 /* Quaternion Dense geometry (src/backend/dense_descriptor.hpp:11-59); filter layout is IO. */

@@ -12,6 +12,7 @@ PHX_OK = 0
 PHX_ERR_INVALID_ARGUMENT, PHX_ERR_NOT_SUPPORTED, PHX_ERR_WORKSPACE, PHX_ERR_RUNTIME = 1, 2, 3, 4
 PHX_F32, PHX_F16 = 0, 1
 PHX_OIHW, PHX_OHWI = 0, 1
+PHX_NCHW, PHX_NHWC = 0, 1
 PHX_PRODUCT_16, PHX_PRODUCT_8 = 16, 8
 PHX_FP16_FULL32, PHX_FP16_BACKWARD32, PHX_FP16_FULL16 = 0, 1, 2
 PHX_PASS_FWD, PHX_PASS_BWD_DATA, PHX_PASS_BWD_WEIGHTS = 0, 1, 2
@@ -40,7 +41,7 @@ class QConvDesc(ctypes.Structure):
     _fields_ = [(k, ctypes.c_int32) for k in (
         "dtype", "n", "ci", "co", "h", "w", "kh", "kw", "stride_h", "stride_w", "dilation_h", "dilation_w",
         "pad_top", "pad_left", "pad_bottom", "pad_right", "filter_layout", "product_mode", "fp16_policy", "has_bias",
-        "real_input", "groups")]
+        "real_input", "groups", "data_format")]
 
 
 class QDenseDesc(ctypes.Structure):

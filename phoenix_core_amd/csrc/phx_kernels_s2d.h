@@ -134,4 +134,45 @@ __global__ void __launch_bounds__(WG_THREADS) phase_merge_kernel(const PhaseMerg
     }
 }
 
+// Channels-last activations: [rows][H][W][C] <-> [rows][C][H][W], i.e. a batch of matrix transposes
+// src[b][R][Cc] -> dst[b][Cc][R] (R = H*W, Cc = C towards the kernels' layout; R = C, Cc = H*W back).
+struct TransposeArgs {
+    const void* src;
+    void* dst;
+    long batch;
+    int R, Cc;
+};
+
+// 64x64 tiles through LDS, coalesced along the contiguous axis on both sides; ragged edges are masked.
+// The tile pitch of 65 words (66 halves = 33 words) keeps the transposed reads on distinct banks.
+template <typename TS>
+__global__ void __launch_bounds__(WG_THREADS) transpose_kernel(const TransposeArgs A) {
+    constexpr int T = 64, PITCH = sizeof(TS) == 4 ? T + 1 : T + 2;
+    __shared__ TS tile[T * PITCH];
+    const TS* src = static_cast<const TS*>(A.src);
+    TS* dst = static_cast<TS*>(A.dst);
+    const int tr = (A.R + T - 1) / T, tc = (A.Cc + T - 1) / T;
+    const long tiles = A.batch * tr * tc;
+    const int lane = threadIdx.x % T, row0 = threadIdx.x / T;  // 256 threads: 4 tile rows per sweep
+    for (long t = blockIdx.x; t < tiles; t += gridDim.x) {
+        const long b = t / ((long)tr * tc);
+        const int rem = (int)(t - b * tr * tc);
+        const int r0 = (rem / tc) * T, c0 = (rem % tc) * T;
+        const TS* s = src + b * A.R * (long)A.Cc;
+        TS* d = dst + b * A.R * (long)A.Cc;
+        __syncthreads();  // the previous tile has been read out
+#pragma unroll 4
+        for (int i = row0; i < T; i += WG_THREADS / T) {
+            const int r = r0 + i, c = c0 + lane;
+            if (r < A.R && c < A.Cc) tile[i * PITCH + lane] = s[(long)r * A.Cc + c];
+        }
+        __syncthreads();
+#pragma unroll 4
+        for (int i = row0; i < T; i += WG_THREADS / T) {
+            const int c = c0 + i, r = r0 + lane;
+            if (c < A.Cc && r < A.R) d[(long)c * A.R + r] = tile[lane * PITCH + i];
+        }
+    }
+}
+
 }  // namespace phx

@@ -1,4 +1,4 @@
-// Launchers of the space-to-depth rearrangement kernels and of the zero fill.
+// Launchers of the rearrangement kernels (space-to-depth, phase merge, channels-last transposes) and of the zero fill.
 #include "phx_kernels_s2d.h"
 #include "phx_launch.h"
 
@@ -48,6 +48,15 @@ int launch_phase_merge(bool half_storage, const PhaseMergeArgs& a, hipStream_t s
     if (items == 0) return 0;
     if (half_storage) hipLaunchKernelGGL((phase_merge_kernel<_Float16>), dim3(blocks_for(items)), dim3(WG_THREADS), 0, st, a);
     else hipLaunchKernelGGL((phase_merge_kernel<float>), dim3(blocks_for(items)), dim3(WG_THREADS), 0, st, a);
+    return 0;
+}
+
+int launch_transpose(bool half_storage, const TransposeArgs& a, hipStream_t st) {
+    const long tiles = a.batch * ((a.R + 63) / 64) * ((a.Cc + 63) / 64);
+    if (tiles == 0) return 0;
+    const int blocks = (int)std::min<long>(tiles, 1 << 16);
+    if (half_storage) hipLaunchKernelGGL((transpose_kernel<_Float16>), dim3(blocks), dim3(WG_THREADS), 0, st, a);
+    else hipLaunchKernelGGL((transpose_kernel<float>), dim3(blocks), dim3(WG_THREADS), 0, st, a);
     return 0;
 }
 

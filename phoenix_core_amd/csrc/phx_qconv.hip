@@ -66,6 +66,7 @@ struct Problem {
     // Grouped convolution: ci / co above are one group's channels, the tensors hold ci_mem / co_mem channels per
     // image and `groups` such slices side by side (ci_mem == ci, co_mem == co without groups)
     int groups, ci_mem, co_mem;
+    bool nhwc;  // the caller's activation tensors are channels-last: [rows, h, w, channels]
 };
 
 static int out_size(int in, int k, int d, int s, int before, int after) {
@@ -87,6 +88,7 @@ static int problem_from_conv(const phx_qconv_desc* d, Problem& p) {
     if (d->real_input != 0 && d->real_input != 1) return PHX_ERR_INVALID_ARGUMENT;
     // "Bias addition is not supported for type0 inputs" (src/conv2d.hpp:125-127)
     if (d->real_input && d->has_bias) return PHX_ERR_INVALID_ARGUMENT;
+    if (d->data_format != PHX_NCHW && d->data_format != PHX_NHWC) return PHX_ERR_INVALID_ARGUMENT;
     const int groups = d->groups > 1 ? d->groups : 1;
     if (d->ci % groups || d->co % groups) return PHX_ERR_INVALID_ARGUMENT;
     p.dtype = d->dtype;
@@ -108,6 +110,7 @@ static int problem_from_conv(const phx_qconv_desc* d, Problem& p) {
     }
     p.has_bias = d->has_bias != 0;
     p.real_input = d->real_input != 0;
+    p.nhwc = d->data_format == PHX_NHWC;
     return PHX_OK;
 }
 
@@ -125,6 +128,7 @@ static int problem_from_dense(const phx_qdense_desc* d, Problem& p) {
     p.has_bias = d->has_bias != 0;
     p.real_input = false;
     p.groups = 1; p.ci_mem = p.ci; p.co_mem = p.co;
+    p.nhwc = false;
     return PHX_OK;
 }
 
@@ -866,6 +870,36 @@ struct GroupOffsets {
     static void* at(void* ptr, size_t off) { return ptr ? static_cast<char*>(ptr) + off : nullptr; }
 };
 
+// Channels-last activations (DataFormat::NHWC, src/backend/tensor.hpp:17-31): the kernels read and write
+// channels-first planes, so such a call keeps channels-first copies of its input-side and output-side activation
+// tensors at the front of the workspace and transposes on the way in and out.
+struct ChannelsLast {
+    size_t x_bytes = 0, y_bytes = 0;
+    long x_rows = 0, y_rows = 0;
+    explicit ChannelsLast(const Problem& p) {
+        if (!p.nhwc) return;
+        const size_t esize = p.dtype == PHX_F32 ? 4 : 2;
+        x_rows = (p.real_input ? 1L : 4L) * p.n;
+        y_rows = 4L * p.n;
+        x_bytes = ((size_t)x_rows * p.ci_mem * p.h * p.w * esize + 255) / 256 * 256;
+        y_bytes = ((size_t)y_rows * p.co_mem * p.ho * p.wo * esize + 255) / 256 * 256;
+    }
+    size_t bytes() const { return x_bytes + y_bytes; }
+    // caller's input-side tensor -> planes, and back
+    void x_in(const Problem& p, const void* x, void* planes, hipStream_t st) const {
+        launch_transpose(p.dtype == PHX_F16, TransposeArgs{x, planes, x_rows, p.h * p.w, p.ci_mem}, st);
+    }
+    void x_out(const Problem& p, const void* planes, void* x, hipStream_t st) const {
+        launch_transpose(p.dtype == PHX_F16, TransposeArgs{planes, x, x_rows, p.ci_mem, p.h * p.w}, st);
+    }
+    void y_in(const Problem& p, const void* y, void* planes, hipStream_t st) const {
+        launch_transpose(p.dtype == PHX_F16, TransposeArgs{y, planes, y_rows, p.ho * p.wo, p.co_mem}, st);
+    }
+    void y_out(const Problem& p, const void* planes, void* y, hipStream_t st) const {
+        launch_transpose(p.dtype == PHX_F16, TransposeArgs{planes, y, y_rows, p.co_mem, p.ho * p.wo}, st);
+    }
+};
+
 int phx_qconv2d_output_hw(const phx_qconv_desc* desc, int32_t* ho, int32_t* wo) {
     Problem p;
     const int rc = problem_from_conv(desc, p);
@@ -878,7 +912,7 @@ int phx_qconv2d_output_hw(const phx_qconv_desc* desc, int32_t* ho, int32_t* wo) 
 size_t phx_qconv2d_workspace_bytes(const phx_qconv_desc* desc, int pass) {
     Problem p;
     if (problem_from_conv(desc, p) != PHX_OK) return 0;
-    return workspace_for(p, pass);
+    return ChannelsLast(p).bytes() + workspace_for(p, pass);
 }
 
 size_t phx_qdense_workspace_bytes(const phx_qdense_desc* desc, int pass) {
@@ -893,12 +927,23 @@ int phx_qconv2d_fwd(const phx_qconv_desc* desc, phx_stream_t stream, const void*
     const int rc = problem_from_conv(desc, p);
     if (rc != PHX_OK) return rc;
     const GroupOffsets o(p);
+    const ChannelsLast cl(p);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (cl.bytes() > workspace_bytes || (cl.bytes() && !workspace)) return PHX_ERR_WORKSPACE;
+    char* ws = static_cast<char*>(workspace);
+    void* y_planes = y;
+    if (p.nhwc) {
+        cl.x_in(p, x, ws, st);
+        x = ws;
+        y_planes = ws + cl.x_bytes;
+    }
     for (int g = 0; g < o.runs; ++g) {
-        const int grc = do_fwd(p, static_cast<hipStream_t>(stream), o.at(x, g * o.x), o.at(w, g * o.w),
-                               bias_or_null ? o.at(bias_or_null, g * o.b) : nullptr, o.at(y, g * o.y), workspace,
-                               workspace_bytes);
+        const int grc = do_fwd(p, st, o.at(x, g * o.x), o.at(w, g * o.w),
+                               bias_or_null ? o.at(bias_or_null, g * o.b) : nullptr, o.at(y_planes, g * o.y),
+                               ws ? ws + cl.bytes() : nullptr, workspace_bytes - cl.bytes());
         if (grc != PHX_OK) return grc;
     }
+    if (p.nhwc) cl.y_out(p, y_planes, y, st);
     return PHX_OK;
 }
 
@@ -911,11 +956,22 @@ int phx_qconv2d_bwd_data(const phx_qconv_desc* desc, phx_stream_t stream, const 
     // the reference refuses the request likewise (src/conv2d.hpp:394-398)
     if (p.real_input) return PHX_ERR_INVALID_ARGUMENT;
     const GroupOffsets o(p);
+    const ChannelsLast cl(p);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (cl.bytes() > workspace_bytes || (cl.bytes() && !workspace)) return PHX_ERR_WORKSPACE;
+    char* ws = static_cast<char*>(workspace);
+    void* dx_planes = dx;
+    if (p.nhwc) {
+        cl.y_in(p, grad, ws + cl.x_bytes, st);
+        grad = ws + cl.x_bytes;
+        dx_planes = ws;
+    }
     for (int g = 0; g < o.runs; ++g) {
-        const int grc = do_bwd_data(p, static_cast<hipStream_t>(stream), o.at(grad, g * o.y), o.at(w, g * o.w),
-                                    o.at(dx, g * o.x), workspace, workspace_bytes);
+        const int grc = do_bwd_data(p, st, o.at(grad, g * o.y), o.at(w, g * o.w), o.at(dx_planes, g * o.x),
+                                    ws ? ws + cl.bytes() : nullptr, workspace_bytes - cl.bytes());
         if (grc != PHX_OK) return grc;
     }
+    if (p.nhwc) cl.x_out(p, dx_planes, dx, st);
     return PHX_OK;
 }
 
@@ -925,9 +981,19 @@ int phx_qconv2d_bwd_weights(const phx_qconv_desc* desc, phx_stream_t stream, con
     const int rc = problem_from_conv(desc, p);
     if (rc != PHX_OK) return rc;
     const GroupOffsets o(p);
+    const ChannelsLast cl(p);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (cl.bytes() > workspace_bytes || (cl.bytes() && !workspace)) return PHX_ERR_WORKSPACE;
+    char* ws = static_cast<char*>(workspace);
+    if (p.nhwc) {
+        cl.x_in(p, x, ws, st);
+        cl.y_in(p, grad, ws + cl.x_bytes, st);
+        x = ws;
+        grad = ws + cl.x_bytes;
+    }
     for (int g = 0; g < o.runs; ++g) {
-        const int grc = do_bwd_weights(p, static_cast<hipStream_t>(stream), o.at(x, g * o.x), o.at(grad, g * o.y),
-                                       o.at(dw, g * o.w), workspace, workspace_bytes);
+        const int grc = do_bwd_weights(p, st, o.at(x, g * o.x), o.at(grad, g * o.y), o.at(dw, g * o.w),
+                                       ws ? ws + cl.bytes() : nullptr, workspace_bytes - cl.bytes());
         if (grc != PHX_OK) return grc;
     }
     return PHX_OK;

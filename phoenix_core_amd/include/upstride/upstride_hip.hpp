@@ -711,7 +711,8 @@ namespace detail {
 inline phx_qconv_desc makeConvDesc(const Conv2DDescriptor& d, Context& ctx, int dtype, bool useBias) {
     if (d.getAlgebra() != Algebra::QUATERNION)
         throw std::runtime_error("Only the quaternion algebra is built for device::HIP");
-    if (d.getDataFormat() != DataFormat::NCHW) throw std::runtime_error("device::HIP runs NCHW tensors only");
+    const DataFormat df = d.getDataFormat();
+    if (df != DataFormat::NCHW && df != DataFormat::NHWC) throw std::runtime_error("device::HIP runs NCHW or NHWC tensors");
     const FilterLayout fl = d.getFilterLayout();
     if (fl != FilterLayout::OIHW && fl != FilterLayout::OHWI)
         throw std::runtime_error("device::HIP takes OIHW or OHWI filters");
@@ -725,8 +726,9 @@ inline phx_qconv_desc makeConvDesc(const Conv2DDescriptor& d, Context& ctx, int 
     c.groups = d.getGroups();
     c.ci = filter.numInputChannels(w) * c.groups;  // the filter holds one group's input channels
     c.co = filter.numOutputChannels(w);
-    c.h = in[2];
-    c.w = in[3];
+    c.h = in.height(df);
+    c.w = in.width(df);
+    c.data_format = df == DataFormat::NCHW ? PHX_NCHW : PHX_NHWC;
     c.kh = filter.height(w);
     c.kw = filter.width(w);
     c.stride_h = d.getStride().x; c.stride_w = d.getStride().y;
@@ -739,7 +741,7 @@ inline phx_qconv_desc makeConvDesc(const Conv2DDescriptor& d, Context& ctx, int 
     c.has_bias = (useBias && !real) ? 1 : 0;  // a bias given with a real-valued input is refused at call time
     c.real_input = real ? 1 : 0;
     if (!real && in[0] % 4 != 0) throw std::invalid_argument("Cannot split " + std::to_string(in[0]) + " onto 4 parts");
-    if (in[1] != c.ci) throw std::invalid_argument("Input channels do not match the filter");
+    if (in.depth(df) != c.ci) throw std::invalid_argument("Input channels do not match the filter");
     return c;
 }
 

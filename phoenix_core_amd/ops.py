@@ -82,11 +82,12 @@ _DTYPES = {torch.float32: capi.PHX_F32, torch.float16: capi.PHX_F16}
 
 class Conv2DDescriptor:
     """Geometry of one quaternion convolution (Conv2DFwdDescriptor / Conv2DBwdDescriptor of the
-    reference, restricted to NCHW activations and the quaternion algebra)."""
+    reference, restricted to the quaternion algebra).  data_format "NCHW" takes activations [4n, c, h, w],
+    "NHWC" [4n, h, w, c] (transposed inside the call: the kernels compute on channels-first planes)."""
 
     def __init__(self, input_shape, filter_shape, stride=1, dilation=1, padding="VALID", groups=1,
                  algebra=QUATERNION, filter_layout="OIHW", use_bias=False, dtype=torch.float32, context=None,
-                 require_input_grad=True, real_valued_input=False):
+                 require_input_grad=True, real_valued_input=False, data_format="NCHW"):
         if len(input_shape) != 4:
             raise ValueError("Four-dimensional input tensor expected")
         if algebra != QUATERNION:
@@ -107,8 +108,12 @@ class Conv2DDescriptor:
             raise ValueError("Unsupported Conv2D filter layout")
         # grouped convolution: the filter holds the input channels of one group (src/backend/conv2d_descriptor.hpp)
         ci *= groups
-        if input_shape[1] != ci:
-            raise ValueError("input channels %d do not match the filter's %d" % (input_shape[1], ci))
+        if data_format not in ("NCHW", "NHWC"):
+            raise ValueError("Unsupported data format")
+        self.data_format = data_format
+        n4, c_in, h, w = input_shape if data_format == "NCHW" else (input_shape[i] for i in (0, 3, 1, 2))
+        if c_in != ci:
+            raise ValueError("input channels %d do not match the filter's %d" % (c_in, ci))
         if co % groups:
             raise ValueError("output channels %d are not a multiple of %d groups" % (co, groups))
         self.groups = groups
@@ -123,7 +128,6 @@ class Conv2DDescriptor:
         # real-valued input (realValuedInput of the reference's descriptors): [n, ci, h, w] without imaginary
         # parts; the output still has the four components stacked on the batch axis
         self.real_valued_input = bool(real_valued_input)
-        n4, _, h, w = input_shape
         if self.real_valued_input:
             n4 *= 4
         if isinstance(padding, str):
@@ -134,13 +138,13 @@ class Conv2DDescriptor:
             ho = (h + pt + pb - ((kh - 1) * self.dilation[0] + 1) + self.stride[0]) // self.stride[0]
             wo = (w + pl + pr - ((kw - 1) * self.dilation[1] + 1) + self.stride[1]) // self.stride[1]
         self.pad_before, self.pad_after = (pt, pl), (pb, pr)
-        self.output_shape = (n4, co, ho, wo)
+        self.output_shape = (n4, co, ho, wo) if data_format == "NCHW" else (n4, ho, wo, co)
         self.bias_shape = (4, co) if use_bias else ()
         self.c = capi.QConvDesc(
             _DTYPES[dtype], n4 // 4, ci, co, h, w, kh, kw, self.stride[0], self.stride[1], self.dilation[0],
             self.dilation[1], pt, pl, pb, pr, capi.PHX_OIHW if filter_layout == "OIHW" else capi.PHX_OHWI,
             self.context.product_mode, self.context.fp16_policy, int(self.use_bias and not self.real_valued_input),
-            int(self.real_valued_input), groups)
+            int(self.real_valued_input), groups, capi.PHX_NCHW if data_format == "NCHW" else capi.PHX_NHWC)
 
     def workspace_bytes(self, which):
         return capi.lib().phx_qconv2d_workspace_bytes(ctypes.byref(self.c), which)

@@ -204,6 +204,29 @@ static void gpuQuaternionRealInput(Context& context) {  // tests/tests.cpp:317-3
     CHECK_THROWS((conv2DBwd<device::HIP, float>(device, device, input, kernel, g, dw, dx, need)), std::logic_error);
 }
 
+static void gpuChannelsLast(Context& context) {  // tests/tests.cpp:440-487
+    // the reference's real NHWC / OHWI case, run as the real part of a quaternion convolution: real-valued
+    // input, filter with zero imaginary components
+    device::HIP device(context);
+    AllocatedTensor<device::HIP, float> input(device, {1, 2, 2, 3});
+    input = {0, -1, 1,   0, 0, 2,   0, 0, 3,   1, 0, 4};
+    AllocatedTensor<device::HIP, float> kernel(device, {MULTIVECTOR_DIM[Algebra::QUATERNION], 2, 1, 1, 3});
+    std::vector<float> kv(24, 0.f);
+    const float real[6] = {1, 1, 1, 0, 0, 2};
+    for (int i = 0; i < 6; ++i) kv[i] = real[i];
+    kernel = kv;
+    AllocatedTensor<device::HIP, float> output(device, {MULTIVECTOR_DIM[Algebra::QUATERNION], 2, 2, 2});
+    Conv2DFwdDescriptor descriptor(input.getShape(), kernel.getShape(), 1, 1, Padding::VALID, {}, 1, Algebra::QUATERNION,
+                                   DataFormat::NHWC, FilterLayout::OHWI, false, true);
+    CHECK(descriptor.getOutputShape() == Shape({4, 2, 2, 2}));
+    conv2DFwd<device::HIP, float>(device, device, input, kernel, nullptr, output, descriptor);
+    std::vector<float> got = output;
+    std::vector<float> want(32, 0.f);
+    const float ref[8] = {0, 2, 2, 4, 3, 6, 5, 8};
+    for (int i = 0; i < 8; ++i) want[i] = ref[i];
+    CHECK(equalVectors(got, want));
+}
+
 static void gpuPointwiseKnownAnswer(Context& context) {
     // 2 pixels, 2 input channels, 1 output channel; y = sum_c x_c (x) w_c computed by hand:
     //   pixel 0: (1+2i)(3+k) + (j)(1-i)   = (3 + 6i - 2j + k) + (j + k)      = 3 + 6i - j + 2k
@@ -294,6 +317,7 @@ int main(int argc, char** argv) {
             Context context;
             gpuQuaternionOnes(context);
             gpuQuaternionRealInput(context);
+            gpuChannelsLast(context);
             gpuPointwiseKnownAnswer(context);
             gpuDenseAndEmpty(context);
             testTensorSplit(context);

@@ -3,6 +3,7 @@ inputs.  Tolerances are the ones the task states: relative error (max-norm and L
 fp32 tensors, <= 2e-2 for fp16 tensors under every fp16 policy; the yardstick is the oracle's
 fp64 closed-form quaternion convolution evaluated on the (fp16-rounded) inputs."""
 import ctypes
+import zlib
 
 import numpy as np
 import pytest
@@ -24,6 +25,11 @@ class Ctx(phx.Context):
             env["UPSTRIDE_MEMORY_OPTIMIZED"] = "1"
         env["UPSTRIDE_CONV_FP16_POLICY"] = policy
         super().__init__(env)
+
+
+def name_seed(name):
+    """Seed from a case name, the same in every process (hash() of a string is salted per process)."""
+    return zlib.crc32(name.encode()) % 1000
 
 
 def rel_errors(got, want):
@@ -77,7 +83,7 @@ CONV_CASES = [
 def test_conv_fp32(case, mode):
     name, n, ci, co, h, w, kh, kw, stride, dilation, padding = case
     dtype = torch.float32
-    g, x, wt, b, gr = make_inputs(hash(name) % 1000, n, ci, co, h, w, kh, kw, stride, dilation, padding, dtype)
+    g, x, wt, b, gr = make_inputs(name_seed(name), n, ci, co, h, w, kh, kw, stride, dilation, padding, dtype)
     print("case", name, "mode", mode, flush=True)
     desc = phx.Conv2DDescriptor(x.shape, wt.shape, stride, dilation, padding, use_bias=True, dtype=dtype,
                                 context=Ctx(mode))
@@ -155,7 +161,7 @@ def test_conv_real_valued_input(case, mode, dtype, policy):
     fp16 tensors it is the fp64 closed form on the input padded with zero imaginary parts."""
     name, n, ci, co, h, w, kh, kw, stride, dilation, padding = case
     scale = 1.0 if dtype == torch.float32 else 0.5
-    g, x, wt, b, gr = make_inputs(hash(name) % 1000 + 2, n, ci, co, h, w, kh, kw, stride, dilation, padding, dtype, scale)
+    g, x, wt, b, gr = make_inputs(name_seed(name) + 2, n, ci, co, h, w, kh, kw, stride, dilation, padding, dtype, scale)
     x = np.ascontiguousarray(x[:n])
     print("case", name, "mode", mode, dtype, policy, flush=True)
     ctx = Ctx(mode, policy)
@@ -243,7 +249,7 @@ def test_conv_fp16(case, mode, policy):
     fp64 closed form on the fp16-rounded inputs (the reference's CPU backend is float-only)."""
     name, n, ci, co, h, w, kh, kw, stride, dilation, padding = case
     dtype = torch.float16
-    g, x, wt, b, gr = make_inputs(hash(name) % 1000 + 1, n, ci, co, h, w, kh, kw, stride, dilation, padding, dtype, 0.5)
+    g, x, wt, b, gr = make_inputs(name_seed(name) + 1, n, ci, co, h, w, kh, kw, stride, dilation, padding, dtype, 0.5)
     print("case", name, "mode", mode, "policy", policy, flush=True)
     desc = phx.Conv2DDescriptor(x.shape, wt.shape, stride, dilation, padding, use_bias=True, dtype=dtype,
                                 context=Ctx(mode, policy))
@@ -278,7 +284,7 @@ def test_factorized_filter_gradient_on_fp16_matrix_cores(case, monkeypatch):
     one there); PHX_TUNE_WG8 selects the factorized 8-lane kernel, which must meet the same tolerance."""
     name, n, ci, co, h, w, kh, kw, stride, dilation, padding = case
     dtype = torch.float16
-    g, x, wt, b, gr = make_inputs(hash(name) % 1000 + 3, n, ci, co, h, w, kh, kw, stride, dilation, padding, dtype, 0.5)
+    g, x, wt, b, gr = make_inputs(name_seed(name) + 3, n, ci, co, h, w, kh, kw, stride, dilation, padding, dtype, 0.5)
     xd, wd, gd = (torch.from_numpy(a).cuda() for a in (x, wt, gr))
     desc = phx.Conv2DDescriptor(x.shape, wt.shape, stride, dilation, padding, dtype=dtype, context=Ctx(8, "full16"),
                                 require_input_grad=False)
@@ -300,7 +306,7 @@ def test_factorized_pointwise_on_fp16_matrix_cores(case, monkeypatch):
     beat the factorized kernel there); PHX_TUNE_PW8 selects the factorized kernel, same tolerance."""
     name, n, ci, co, h, w, kh, kw, stride, dilation, padding = case
     dtype = torch.float16
-    g, x, wt, b, gr = make_inputs(hash(name) % 1000 + 4, n, ci, co, h, w, kh, kw, stride, dilation, padding, dtype, 0.5)
+    g, x, wt, b, gr = make_inputs(name_seed(name) + 4, n, ci, co, h, w, kh, kw, stride, dilation, padding, dtype, 0.5)
     xd, wd, bd, gd = (torch.from_numpy(a).cuda() for a in (x, wt, b, gr))
     desc = phx.Conv2DDescriptor(x.shape, wt.shape, stride, dilation, padding, use_bias=True, dtype=dtype,
                                 context=Ctx(8, "full16"))
@@ -341,8 +347,8 @@ def test_grouped_convolution(case, mode, dtype, policy):
     name, G, n, ci, co, h, w, kh, kw, stride, dilation, padding = case
     cig, cog = ci // G, co // G
     scale = 1.0 if dtype == torch.float32 else 0.5
-    g, x, _, b, gr = make_inputs(hash(name) % 1000 + 6, n, ci, co, h, w, kh, kw, stride, dilation, padding, dtype, scale)
-    r = np.random.default_rng(hash(name) % 1000 + 7)
+    g, x, _, b, gr = make_inputs(name_seed(name) + 6, n, ci, co, h, w, kh, kw, stride, dilation, padding, dtype, scale)
+    r = np.random.default_rng(name_seed(name) + 7)
     npdt = np.float32 if dtype == torch.float32 else np.float16
     wt = (scale * r.standard_normal((4, co, cig, kh, kw)) * np.sqrt(2.0 / (cig * kh * kw))).astype(npdt)
     desc = phx.Conv2DDescriptor(x.shape, wt.shape, stride, dilation, padding, groups=G, use_bias=True, dtype=dtype,
@@ -364,6 +370,83 @@ def test_grouped_convolution(case, mode, dtype, policy):
     assert_close(dw.cpu().numpy(), want_dw, dtype, "grouped wgrad " + name)
 
 
+def test_reference_kat_channels_last():
+    """tests/tests.cpp:440-487 of the reference: a real 2x2 image with 3 channels, NHWC, through a real 1x1
+    OHWI filter with 2 output channels -> (0,2, 2,4, 3,6, 5,8).  A real convolution is the real part of a
+    quaternion convolution whose input and filter have no imaginary parts, which is how it runs here (real-valued
+    input, imaginary filter components zero); the imaginary outputs must be exact zeros."""
+    x = [0, -1, 1, 0, 0, 2, 0, 0, 3, 1, 0, 4]
+    k = [1, 1, 1, 0, 0, 2]
+    want = [0, 2, 2, 4, 3, 6, 5, 8]
+    for mode in (8, 16):
+        for dtype in (torch.float32, torch.float16):
+            xd = torch.tensor(x, dtype=dtype, device="cuda").reshape(1, 2, 2, 3)
+            wd = torch.zeros(4, 2, 1, 1, 3, dtype=dtype, device="cuda")
+            wd[0] = torch.tensor(k, dtype=dtype, device="cuda").reshape(2, 1, 1, 3)
+            desc = phx.Conv2DDescriptor(xd.shape, wd.shape, 1, 1, "VALID", filter_layout="OHWI", dtype=dtype,
+                                        context=Ctx(mode, "full16"), real_valued_input=True, data_format="NHWC")
+            assert desc.output_shape == (4, 2, 2, 2)
+            y = phx.conv2d_fwd(xd, wd, None, desc)
+            assert y[0].flatten().tolist() == [float(v) for v in want], (mode, dtype)
+            assert not y[1:].any()
+
+
+# name, groups, real input, OHWI filter, n, ci, co, h, w, kh, kw, stride, dilation, padding
+CHANNELS_LAST = [
+    ("nhwc_pw", 1, False, True, 2, 64, 64, 14, 14, 1, 1, 1, 1, "VALID"),
+    ("nhwc_k3", 1, False, True, 2, 24, 40, 13, 9, 3, 3, 1, 1, "SAME"),
+    ("nhwc_k3_s2_oihw", 1, False, False, 3, 5, 7, 17, 15, 3, 3, 2, 1, "SAME"),
+    ("nhwc_wide", 1, False, True, 1, 130, 70, 9, 11, 1, 1, 1, 1, "VALID"),
+    ("nhwc_plane_gt_tile", 1, False, True, 1, 3, 2, 20, 23, 5, 5, 1, 2, (2, 1, 3, 0)),
+    ("nhwc_stem_real", 1, True, True, 2, 3, 16, 32, 32, 7, 7, 2, 1, "SAME"),
+    ("nhwc_grouped", 4, False, True, 2, 16, 24, 10, 10, 3, 3, 1, 1, "SAME"),
+]
+
+
+@pytest.mark.parametrize("dtype,policy", [(torch.float32, "fp32"), (torch.float16, "full16"), (torch.float16, "backward32")],
+                         ids=["f32", "f16_full16", "f16_backward32"])
+@pytest.mark.parametrize("mode", [16, 8])
+@pytest.mark.parametrize("case", CHANNELS_LAST, ids=lambda c: c[0])
+def test_channels_last(case, mode, dtype, policy):
+    """Channels-last activations [4n, h, w, c] (DataFormat::NHWC, src/backend/tensor.hpp:17-31): a pure
+    permutation of the channels-first tensors, so the oracle runs on the permuted arrays."""
+    name, G, real, ohwi, n, ci, co, h, w, kh, kw, stride, dilation, padding = case
+    cig, cog = ci // G, co // G
+    scale = 1.0 if dtype == torch.float32 else 0.5
+    g, x, _, b, gr = make_inputs(name_seed(name) + 8, n, ci, co, h, w, kh, kw, stride, dilation, padding, dtype, scale)
+    r = np.random.default_rng(name_seed(name) + 9)
+    npdt = np.float32 if dtype == torch.float32 else np.float16
+    wt = (scale * r.standard_normal((4, co, cig, kh, kw)) * np.sqrt(2.0 / (cig * kh * kw))).astype(npdt)
+    bias = not real
+    if real:
+        x[n:] = 0
+    x_dev = np.ascontiguousarray((x[:n] if real else x).transpose(0, 2, 3, 1))
+    g_dev = np.ascontiguousarray(gr.transpose(0, 2, 3, 1))
+    w_dev = np.ascontiguousarray(wt.transpose(0, 1, 3, 4, 2)) if ohwi else wt
+    desc = phx.Conv2DDescriptor(x_dev.shape, w_dev.shape, stride, dilation, padding, groups=G, use_bias=bias, dtype=dtype,
+                                filter_layout="OHWI" if ohwi else "OIHW", context=Ctx(mode, policy),
+                                real_valued_input=real, require_input_grad=not real, data_format="NHWC")
+    assert desc.output_shape == (4 * n, g.ho, g.wo, co)
+    xd, wd, bd, gd = (torch.from_numpy(a).cuda() for a in (x_dev, w_dev, b, g_dev))
+    y = phx.conv2d_fwd(xd, wd, bd if bias else None, desc)
+    dw, dx = phx.conv2d_bwd(xd, wd, gd, desc)
+    gg = oracle.make_geom(n, cig, cog, h, w, kh, kw, stride, dilation, padding)
+    x64, w64, b64, g64 = (a.astype(np.float64) for a in (x, wt, b, gr))
+    want_y, want_dx, want_dw = np.empty(gr.shape), np.empty(x.shape), np.empty(wt.shape)
+    for k in range(G):
+        ic, oc = slice(k * cig, (k + 1) * cig), slice(k * cog, (k + 1) * cog)
+        xs, ws, bs, gs = (np.ascontiguousarray(a) for a in (x64[:, ic], w64[:, oc], b64[:, oc], g64[:, oc]))
+        want_y[:, oc] = oracle.conv2d_fwd(gg, xs, ws, bs if bias else None, "hamilton")
+        want_dw[:, oc], want_dx[:, ic] = oracle.conv2d_bwd(gg, xs, ws, gs, "hamilton")
+    assert_close(y.cpu().numpy().transpose(0, 3, 1, 2), want_y, dtype, "channels-last fwd " + name)
+    got_dw = dw.cpu().numpy()
+    assert_close(got_dw.transpose(0, 1, 4, 2, 3) if ohwi else got_dw, want_dw, dtype, "channels-last wgrad " + name)
+    if real:
+        assert dx is None
+    else:
+        assert_close(dx.cpu().numpy().transpose(0, 3, 1, 2), want_dx, dtype, "channels-last dgrad " + name)
+
+
 STRIDED = [c for c in FP16_CASES if c[0] in ("k3_s2", "pw_s2", "k7_s2", "k3_s2_c4", "k5_s2_valid", "k3_s3", "k32_s21")]
 
 
@@ -377,7 +460,7 @@ def test_strided_input_gradient_variants(case, mode, dtype, policy, variant, mon
     factorized one is forced); the planner picks by shape, the environment overrides select each."""
     name, n, ci, co, h, w, kh, kw, stride, dilation, padding = case
     scale = 1.0 if dtype == torch.float32 else 0.5
-    g, x, wt, b, gr = make_inputs(hash(name) % 1000 + 5, n, ci, co, h, w, kh, kw, stride, dilation, padding, dtype, scale)
+    g, x, wt, b, gr = make_inputs(name_seed(name) + 5, n, ci, co, h, w, kh, kw, stride, dilation, padding, dtype, scale)
     monkeypatch.setenv("PHX_TUNE_PHASE", "1" if variant == "phases" else "0")
     if variant == "zero_insertion_factorized":
         monkeypatch.setenv("PHX_TUNE_ZI8", "1")

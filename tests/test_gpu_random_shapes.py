@@ -1,6 +1,6 @@
 """GPU parity on seeded random problem geometries: batch, channel counts, image and filter sizes, strides,
-dilations, padding (SAME / VALID / explicit asymmetric), filter layout, bias, product mode, fp16 policy and
-real-valued input are all drawn at random, so that the host planner's corner cases (ragged tiles, windows
+dilations, padding (SAME / VALID / explicit asymmetric), filter layout, data format, bias, product mode, fp16
+policy and real-valued input are all drawn at random, so that the host planner's corner cases (ragged tiles, windows
 that leave the tensor, space-to-depth stems, virtual pointwise taps, zero-inserted strided gradients) meet
 the oracle on shapes nobody picked by hand.  Tolerances as in test_gpu_parity.py."""
 import numpy as np
@@ -53,6 +53,7 @@ def draw(seed):
                co=int(r.choice([1, 2, 3, 7, 8, 16, 33, 64, 72, 130])), h=h, w=w, kh=kh, kw=kw, stride=stride,
                dilation=dilation, padding=padding, mode=int(r.choice([8, 16])), ohwi=bool(r.random() < 0.25),
                bias=bool(r.random() < 0.5), real=bool(r.random() < 0.2), seed=seed)
+    cfg["nhwc"] = bool(r.random() < 0.25)
     return cfg, r
 
 
@@ -70,25 +71,30 @@ def run_case(cfg, r, dtype, policy):
         x[n:] = 0  # the oracle sees the same input with explicit zero imaginary parts
     w_dev = np.ascontiguousarray(wt.transpose(0, 1, 3, 4, 2)) if cfg["ohwi"] else wt
     x_dev = np.ascontiguousarray(x[:n]) if real else x
+    nhwc = cfg["nhwc"]
+    to_dev = (lambda a: np.ascontiguousarray(a.transpose(0, 2, 3, 1))) if nhwc else (lambda a: a)
+    from_dev = (lambda a: a.transpose(0, 3, 1, 2)) if nhwc else (lambda a: a)
+    x_dev, g_dev = to_dev(x_dev), to_dev(gr)
     ctx = Ctx(cfg["mode"], policy)
     desc = phx.Conv2DDescriptor(x_dev.shape, w_dev.shape, cfg["stride"], cfg["dilation"], cfg["padding"],
                                 filter_layout="OHWI" if cfg["ohwi"] else "OIHW", use_bias=bias, dtype=dtype, context=ctx,
-                                real_valued_input=real, require_input_grad=not real)
-    assert desc.output_shape == (4 * n, co, geom.ho, geom.wo), cfg
-    xd, wd, bd, gd = (torch.from_numpy(a).cuda() for a in (x_dev, w_dev, b, gr))
+                                real_valued_input=real, require_input_grad=not real,
+                                data_format="NHWC" if nhwc else "NCHW")
+    assert desc.output_shape == ((4 * n, geom.ho, geom.wo, co) if nhwc else (4 * n, co, geom.ho, geom.wo)), cfg
+    xd, wd, bd, gd = (torch.from_numpy(a).cuda() for a in (x_dev, w_dev, b, g_dev))
     y = phx.conv2d_fwd(xd, wd, bd if bias else None, desc)
     dw, dx = phx.conv2d_bwd(xd, wd, gd, desc)
     torch.cuda.synchronize()
     x64, w64, b64, g64 = (a.astype(np.float64) for a in (x, wt, b, gr))
     want_y = oracle.conv2d_fwd(geom, x64, w64, b64 if bias else None, "hamilton")
     want_dw, want_dx = oracle.conv2d_bwd(geom, x64, w64, g64, "hamilton")
-    close(y.cpu().numpy(), want_y, dtype, "fwd %s" % cfg)
+    close(from_dev(y.cpu().numpy()), want_y, dtype, "fwd %s" % cfg)
     got_dw = dw.cpu().numpy()
     close(got_dw.transpose(0, 1, 4, 2, 3) if cfg["ohwi"] else got_dw, want_dw, dtype, "wgrad %s" % cfg)
     if real:
         assert dx is None
     else:
-        close(dx.cpu().numpy(), want_dx, dtype, "dgrad %s" % cfg)
+        close(from_dev(dx.cpu().numpy()), want_dx, dtype, "dgrad %s" % cfg)
 
 
 @pytest.mark.parametrize("seed", range(CASES))
