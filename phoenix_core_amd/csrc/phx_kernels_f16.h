@@ -420,8 +420,12 @@ __device__ __forceinline__ void lane_step(const f16x8 (&x)[4], f16x8 (&L)[8], f1
     }
 }
 
-template <int MODE, int MAP, int WCO, int NTW, int P2LOG, bool CHUNKS>
+// EARLY (chunk staging, problems with one filter group per chunk, i.e. pointwise ones): only the products of one
+// group stand between the request for the next chunk's activations and their use, so the request goes out at the
+// start of the group, ahead of the filter copy (which the same wait then covers).
+template <int MODE, int MAP, int WCO, int NTW, int P2LOG, bool CHUNKS, bool EARLY = false>
 __global__ void __launch_bounds__(WG_THREADS, (MODE == 16 && NTW == 1) ? 2 : 1) qconv_fwd_f16_lds_kernel(const ConvArgs P) {
+    static_assert(!EARLY || CHUNKS, "early activation requests belong to chunk staging");
     constexpr int CK = F16_CK;
     constexpr int WPX = 4 / WCO;
     constexpr int TG = F16_TG;
@@ -596,7 +600,19 @@ __global__ void __launch_bounds__(WG_THREADS, (MODE == 16 && NTW == 1) ? 2 : 1) 
 #pragma unroll
             for (int blk = 0; blk < NBLK; ++blk) {
                 const int tg = blk / NTW, t = blk % NTW;
-                if (blk < DBLK) {
+                if constexpr (EARLY) {
+                    constexpr int EPB = NBLK > 1 ? (NSL + NBLK - 2) / (NBLK - 1) : NSL;  // filter slices per later block
+                    if (blk == 0 && more_chunks) {
+#pragma unroll
+                        for (int i = 0; i < 8; ++i) stage_chunk_load(stagec, P.in, sc, (chunk + 1) * CK, i);
+                    }
+                    if (more_groups && (blk > 0 || NBLK == 1)) {
+#pragma unroll
+                        for (int s = 0; s < NSL; ++s) {
+                            if (NBLK == 1 || s / EPB == blk - 1) copy_slice(wsrc_next, wdst_next, s);
+                        }
+                    }
+                } else if (blk < DBLK) {
                     if (more_groups) {
                         // (loops with constant bounds: they must unroll, the staging registers are indexed by them)
 #pragma unroll
@@ -667,7 +683,7 @@ __global__ void __launch_bounds__(WG_THREADS, (MODE == 16 && NTW == 1) ? 2 : 1) 
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
-            x_in_flight = CHUNKS && more_chunks;
+            x_in_flight = CHUNKS && !EARLY && more_chunks;
             carried = carry;
             PHX_STAMP(4)
         }
@@ -675,7 +691,9 @@ __global__ void __launch_bounds__(WG_THREADS, (MODE == 16 && NTW == 1) ? 2 : 1) 
     }
 
     conv_epilogue<_Float16, MODE, MAP, NTW, NW>(P, acc, (ct * WCO + wco) * 32 + 4 * kk, oaddr, pvalid);
-    __builtin_amdgcn_s_waitcnt(0x0F70);
+#ifdef PHX_PHASE_TIMING
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // (charge the stores to the epilogue; otherwise the wave ends with them in flight)
+#endif
     PHX_STAMP(5)
     PHX_PHASES_REPORT("fwd_f16_lds: barrier / store / wait+barrier / prefetch / mfma / epilogue", 6)
 }

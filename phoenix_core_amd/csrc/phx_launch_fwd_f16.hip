@@ -1,4 +1,6 @@
 // Instantiations of the fp16-MFMA forward / input-gradient kernels and their filter packing.
+#include <cstdlib>
+
 #include "phx_kernels_f16.h"
 #include "phx_launch.h"
 
@@ -38,6 +40,21 @@ static int launch_lds16(const FwdVariant& v, const ConvArgs& a, hipStream_t st) 
         hipLaunchKernelGGL((qconv_fwd_f16_lds_kernel<16, MAP_FWD, WCO_, NTW_, P2_, CHUNKS>), dim3(v.wgs), dim3(WG_THREADS), \
                            v.lds_bytes, st, a);                                                               \
         return 0;                                                                                             \
+    }
+    if constexpr (CHUNKS) {
+        // one filter group per chunk (pointwise problems): the variant that requests the next chunk first
+        if (v.ngroups == 1 && v.NTW == 1 && !getenv("PHX_TUNE_NOEARLY")) {
+            if (v.WCO == 1) {
+                hipLaunchKernelGGL((qconv_fwd_f16_lds_kernel<16, MAP_FWD, 1, 1, 8, true, true>), dim3(v.wgs), dim3(WG_THREADS),
+                                   v.lds_bytes, st, a);
+                return 0;
+            }
+            if (v.WCO == 2) {
+                hipLaunchKernelGGL((qconv_fwd_f16_lds_kernel<16, MAP_FWD, 2, 1, 8, true, true>), dim3(v.wgs), dim3(WG_THREADS),
+                                   v.lds_bytes, st, a);
+                return 0;
+            }
+        }
     }
     PHX_CASE(1, 1, P2A) PHX_CASE(1, 1, P2B) PHX_CASE(1, 2, P2A) PHX_CASE(1, 2, P2B)
     PHX_CASE(2, 1, P2A) PHX_CASE(2, 1, P2B) PHX_CASE(2, 2, P2A) PHX_CASE(2, 2, P2B)
