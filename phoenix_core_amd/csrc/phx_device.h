@@ -270,6 +270,7 @@ struct TileSrc {
     int uh, uw;        // zero-insertion factors (1 = none)
     int ncomp;         // components present in memory: 4, or 1 for a real-valued tensor (components 1..3 read as zero)
     int pw;            // pointwise trick: window row r holds channels (chunk*pw + r)*16.. of the single image row (0 = off)
+    int tall;          // flat tiling: the images are rows [n*tall, n*tall + Hd) of one tall image, zero rows between them (0 = off)
 };
 
 // Window staging, split so that global loads can be in flight while the previous chunk is being

@@ -331,14 +331,19 @@ __device__ __forceinline__ StageChunk make_stage_chunk(const TileSrc& s, int n0,
     // sub-chunks of the one (flattened) image row, so that a "filter column" of s.pw taps walks over
     // 16*s.pw channels per staged chunk
     sc.sub = s.pw ? hr : 0;
-    const int vh = s.pw ? 0 : h0 + hr, vw0 = w0 + cc * 8;
+    int vh = s.pw ? 0 : h0 + hr, img = n0 + nb;
+    const int vw0 = w0 + cc * 8;
+    if (s.tall) {  // h0 counts rows of the tall image; rows above it and between the images are zeros
+        img = vh >= 0 ? vh / s.tall : -1;
+        vh -= img * s.tall;
+    }
     const int p = u >> 1;
     sc.kp = u & 1;
-    sc.live = sc.task && p < s.ncomp && nb < NB && (n0 + nb) < s.N && vh >= 0 && vh < s.Hd;
+    sc.live = sc.task && p < s.ncomp && nb < NB && img >= 0 && img < s.N && vh >= 0 && vh < s.Hd;
     sc.bits = sc.live ? interval_bits(-vw0, s.Wd - vw0) : 0u;
     const _Float16* base = static_cast<const _Float16*>(s.base);
     const long plane = (long)s.Hd * s.Wd;
-    sc.ptr = base + p * s.comp_stride + ((long)(n0 + nb) * s.Cs * s.Hd + vh) * s.Wd + vw0;
+    sc.ptr = base + p * s.comp_stride + ((long)img * s.Cs * s.Hd + vh) * s.Wd + vw0;
     const _Float16* end = base + (long)(s.ncomp - 1) * s.comp_stride + ((long)(s.N - 1) * s.Cs + s.C) * plane;
     sc.careful = sc.live && (sc.ptr < base || sc.ptr + (long)(s.C - 1) * plane + 8 > end);
     const int e0 = row * HTW + cc * 8;
@@ -453,7 +458,13 @@ __global__ void __launch_bounds__(WG_THREADS, (MODE == 16 && NTW == 1) ? 2 : 1) 
     const int th = bid % P.tiles_h;
     const int tn = bid / P.tiles_h;
     const int n0 = tn * P.NB, ho0 = th * P.TH, wo0 = tw * P.TW;
-    const int h0 = ho0 * P.sh - P.pt, w0 = wo0 * P.sw - P.pl;
+    int h0 = ho0 * P.sh - P.pt;
+    const int w0 = wo0 * P.sw - P.pl;
+    // Flat tiling (P.in.tall > 0; unit stride, whole rows): the images form one tall image, P.in.tall rows apart
+    // with zero rows between them, and workgroup th takes the next WPX*NTW*32 output positions of it in row-major
+    // order -- every lane works whatever the image size; the window is every row those positions touch.
+    const int q0 = th * (WPX * NTW * 32), R0 = P.in.tall ? q0 / P.Wout : 0;
+    if (P.in.tall) h0 = R0 - P.pt;
 
     int poff[NTW];
     long oaddr[NTW];
@@ -462,11 +473,19 @@ __global__ void __launch_bounds__(WG_THREADS, (MODE == 16 && NTW == 1) ? 2 : 1) 
 #pragma unroll
     for (int t = 0; t < NTW; ++t) {
         const int pix = (wpx * NTW + t) * 32 + j;
-        const int nb = pix / thw, rem = pix - nb * thw;
-        const int r = rem / P.TW, c = rem - r * P.TW;
-        pvalid[t] = nb < P.NB && (n0 + nb) < P.in.N && (ho0 + r) < P.Hout && (wo0 + c) < P.Wout;
-        poff[t] = pvalid[t] ? (nb * P.HTH + r * P.sh) * P.HTW + c * P.sw : 0;
-        oaddr[t] = ((long)(n0 + nb) * P.CoutS * P.Hout + (ho0 + r)) * P.Wout + (wo0 + c);
+        if (P.in.tall) {
+            const int q = q0 + pix, R = q / P.Wout, c = q - R * P.Wout;
+            const int n = R / P.in.tall, ho = R - n * P.in.tall;
+            pvalid[t] = n < P.in.N && ho < P.Hout;
+            poff[t] = pvalid[t] ? (R - R0) * P.HTW + c : 0;
+            oaddr[t] = ((long)n * P.CoutS * P.Hout + ho) * P.Wout + c;
+        } else {
+            const int nb = pix / thw, rem = pix - nb * thw;
+            const int r = rem / P.TW, c = rem - r * P.TW;
+            pvalid[t] = nb < P.NB && (n0 + nb) < P.in.N && (ho0 + r) < P.Hout && (wo0 + c) < P.Wout;
+            poff[t] = pvalid[t] ? (nb * P.HTH + r * P.sh) * P.HTW + c * P.sw : 0;
+            oaddr[t] = ((long)(n0 + nb) * P.CoutS * P.Hout + (ho0 + r)) * P.Wout + (wo0 + c);
+        }
     }
 
     f32x16 acc[NTW][NW];

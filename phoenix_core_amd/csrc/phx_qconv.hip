@@ -190,6 +190,7 @@ struct FwdPlan {
     int tiles_n, tiles_h, tiles_w, co_tiles, nchunks;
     size_t lds_bytes, wpk_bytes;
     int wgs;
+    int tall;                // flat tiling (row distance of the images in the tall image), 0 = rectangular tiles
 };
 
 
@@ -210,6 +211,7 @@ static bool plan_forward(const Corr& c, int mode, bool f16mfma, FwdPlan& best, b
     // PHX_TUNE_TILE="wco,ntw" pins the workgroup shape (kernel tuning experiments)
     int force_wco = 0, force_ntw = 0;
     if (const char* t = std::getenv("PHX_TUNE_TILE")) sscanf(t, "%d,%d", &force_wco, &force_ntw);
+    const bool force_flat = getenv("PHX_TUNE_FLAT") != nullptr;
     for (int wi = 0; wi < 3; ++wi) {
         const int WCO = wcos[wi];
         if (force_wco && WCO != force_wco) continue;
@@ -219,6 +221,53 @@ static bool plan_forward(const Corr& c, int mode, bool f16mfma, FwdPlan& best, b
         for (int NTW = 1; NTW <= ((mode == 16 || ldsk) ? 2 : 1); ++NTW) {
             if (force_ntw && NTW != force_ntw) continue;
             const int BN = (4 / WCO) * NTW * 32;
+            const int cot = cdiv(c.Cout, 32 * WCO);
+            auto consider = [&](int NB, int TH, int TW, int HTH, int HTW, int tn, int th, int tw, int tall) {
+                const int HP = NB * HTH * HTW;
+                if (HP > 256) return;  // one staging position per thread
+                const long wgs = (long)tn * th * tw * cot;
+                const double eff = ((double)c.N * c.Hout * c.Wout * c.Cout) / ((double)wgs * BN * 32 * WCO);
+                const double fill = (double)wgs / ((double)cdiv((int)std::min<long>(wgs, 1 << 30), 512) * 512);
+                const double halo = (double)std::min(NB * TH * TW, BN) / HP;  // staged data actually used
+                double score = eff * (0.25 + 0.75 * fill) * (0.9 + 0.1 * halo) * (NTW == 2 ? 1.02 : 1.0);
+                // fp16 MFMA is operand-bandwidth hungry: two column tiles per wave and two filter
+                // sub-tiles per workgroup amortise LDS reads and activation staging (measured)
+                // (pointwise problems, 16-product: workgroups live for a few blocks only, and two of them
+                // per CU -- one column tile per wave, two filter sub-tiles -- hide each other's start and end)
+                if (ldsk && pointwise && mode == 16) score *= (NTW == 1 ? 1.25 : 1.0) * (WCO == 2 ? 1.2 : 1.0);
+                else if (ldsk) score *= (NTW == 2 ? 1.25 : 1.0) * (WCO == 2 ? 1.08 : 1.0);
+                else if (f16mfma && NTW == 2) score *= 0.8;  // that kernel drops to one workgroup per CU
+                if (tall && force_flat) score *= 100.0;  // (tests: flat tiling wherever it applies)
+                if (score > best_score) {
+                    best_score = score;
+                    best.WCO = WCO; best.NTW = NTW; best.BN = BN;
+                    best.NB = NB; best.TH = TH; best.TW = TW; best.HTH = HTH; best.HTW = HTW;
+                    best.HP = HP; best.HPp = HP;
+                    best.tiles_n = tn; best.tiles_h = th; best.tiles_w = tw; best.co_tiles = cot;
+                    best.wgs = (int)wgs;
+                    best.tall = tall;
+                }
+            };
+            // Flat tiling (chunk-staging kernels, unit stride): the images are stacked into one tall image, far
+            // enough apart that no window of one reaches the rows of another, and a workgroup takes BN consecutive
+            // output positions of it in row-major order: every lane works whatever the image size (a 28-wide
+            // image fills 112 of 128 lanes with rectangular tiles, a 14x14 one 98 or 126 of them on 14 of 18 rows).
+            // Measured: it pays where the matrix pipe is the bound (two column tiles per wave, long reductions:
+            // +4-7 % at 128 channels, 28x28) and costs where workgroups are short-lived and the larger window's
+            // staging shows (-7 % at 32 channels), so it is offered only to the former.
+            const bool flat_pays = NTW == 2 && (long)c.Cin * c.Kh * c.Kw >= 576;
+            if (chunks && !pointwise && c.sh == 1 && c.sw == 1 && (flat_pays || force_flat) &&
+                !getenv("PHX_TUNE_NOFLAT")) {
+                const int reach = (c.Hout - 1) - c.pt + (c.Kh - 1) * c.dh - (c.Hin - 1);  // rows read below the image
+                const int gap = std::max(0, std::max(c.pt, reach));
+                const long S = (long)c.Hin + gap;                          // row distance of the images
+                const long Q = ((long)(c.N - 1) * S + c.Hout) * c.Wout;    // output positions of the tall image
+                const int rows = (BN + c.Wout - 2) / c.Wout + 1;           // rows BN consecutive positions can touch
+                const int HTH = rows + (c.Kh - 1) * c.dh;
+                const int HTW = (c.Wout + (c.Kw - 1) * c.dw + 7) & ~7;
+                if (c.Hout <= S && Q < (1L << 30))
+                    consider(1, rows, c.Wout, HTH, HTW, 1, (int)cdiv((int)Q, BN), 1, (int)S);
+            }
             int cand[24];
             int nc = 0;
             for (int k = 1; k <= 8; ++k) cand[nc++] = cdiv(c.Wout, k);
@@ -236,31 +285,7 @@ static bool plan_forward(const Corr& c, int mode, bool f16mfma, FwdPlan& best, b
                     if (pairs) HTW = (HTW + 2) & ~1;  // room for the even start column, even pitch
                     if (chunks) HTW = (HTW + 7) & ~7;  // whole 8-position chunks
                     if (vstage) HTW = (HTW + 3) & ~3;  // whole 4-position groups
-                    const int HP = NB * HTH * HTW;
-                    const int HPp = HP;
-                    if (HP > 256) continue;  // one staging position per thread
-                    const int tn = cdiv(c.N, NB), th = cdiv(c.Hout, TH), tw = cdiv(c.Wout, TW);
-                    const int cot = cdiv(c.Cout, 32 * WCO);
-                    const long wgs = (long)tn * th * tw * cot;
-                    const double eff = ((double)c.N * c.Hout * c.Wout * c.Cout) / ((double)wgs * BN * 32 * WCO);
-                    const double fill = (double)wgs / ((double)cdiv((int)std::min<long>(wgs, 1 << 30), 512) * 512);
-                    const double halo = (double)(NB * TH * TW) / HP;  // staged data actually used
-                    double score = eff * (0.25 + 0.75 * fill) * (0.9 + 0.1 * halo) * (NTW == 2 ? 1.02 : 1.0);
-                    // fp16 MFMA is operand-bandwidth hungry: two column tiles per wave and two filter
-                    // sub-tiles per workgroup amortise LDS reads and activation staging (measured)
-                    // (pointwise problems, 16-product: workgroups live for a few blocks only, and two of them
-                    // per CU -- one column tile per wave, two filter sub-tiles -- hide each other's start and end)
-                    if (ldsk && pointwise && mode == 16) score *= (NTW == 1 ? 1.25 : 1.0) * (WCO == 2 ? 1.2 : 1.0);
-                    else if (ldsk) score *= (NTW == 2 ? 1.25 : 1.0) * (WCO == 2 ? 1.08 : 1.0);
-                    else if (f16mfma && NTW == 2) score *= 0.8;  // that kernel drops to one workgroup per CU
-                    if (score > best_score) {
-                        best_score = score;
-                        best.WCO = WCO; best.NTW = NTW; best.BN = BN;
-                        best.NB = NB; best.TH = TH; best.TW = TW; best.HTH = HTH; best.HTW = HTW;
-                        best.HP = HP; best.HPp = HPp;
-                        best.tiles_n = tn; best.tiles_h = th; best.tiles_w = tw; best.co_tiles = cot;
-                        best.wgs = (int)wgs;
-                    }
+                    consider(NB, TH, TW, HTH, HTW, cdiv(c.N, NB), cdiv(c.Hout, TH), cdiv(c.Wout, TW), 0);
                 }
             }
         }
@@ -382,7 +407,7 @@ static int run_corr(const Problem& p, const Corr& creal, int map, hipStream_t st
     // channels per image in memory on the input and output side of this correlation (grouped convolutions: slices)
     const int cin_mem = (map == MAP_FWD) ? p.ci_mem : p.co_mem, cout_mem = (map == MAP_FWD) ? p.co_mem : p.ci_mem;
     a.in.base = in; a.in.comp_stride = (long)c.N * cin_mem * c.Hin * c.Win; a.in.Cs = cin_mem;
-    a.in.N = c.N; a.in.C = creal.Cin; a.in.Hd = c.Hin; a.in.Wd = c.Win; a.in.uh = c.uh; a.in.uw = c.uw; a.in.pw = pw;
+    a.in.N = c.N; a.in.C = creal.Cin; a.in.Hd = c.Hin; a.in.Wd = c.Win; a.in.uh = c.uh; a.in.uw = c.uw; a.in.pw = pw; a.in.tall = pl.tall;
     // real-valued input: the forward pass reads one component, the others are zero
     a.in.ncomp = (p.real_input && map == MAP_FWD) ? 1 : 4;
     a.wpk = ws; a.bias = bias; a.out = out;
@@ -404,9 +429,9 @@ static int run_corr(const Problem& p, const Corr& creal, int map, hipStream_t st
     }
     if (rc != 0) return PHX_ERR_NOT_SUPPORTED;
     PHX_HIP(hipGetLastError());
-    snprintf(g_name_buf, sizeof(g_name_buf), "%sqconv_%s_%smfma%s_p%d_%s_wco%d_ntw%d_ck%d_tile%dx%dx%d", g_name_prefix,
+    snprintf(g_name_buf, sizeof(g_name_buf), "%sqconv_%s_%smfma%s_p%d_%s_wco%d_ntw%d_ck%d_%s%dx%dx%d", g_name_prefix,
              map == MAP_FWD ? "fwd" : "dgrad", f16 ? "f16" : "f32", pl.lds_filters ? (pw ? "ldspw" : pl.chunks ? "ldsc" : "lds") : "", pl.kmode, p.dtype == PHX_F32 ? "f32" : "f16", pl.WCO,
-             pl.NTW, pl.CK, pl.NB, pl.TH, pl.TW);
+             pl.NTW, pl.CK, pl.tall ? "flat" : "tile", pl.NB, pl.TH, pl.TW);
     g_last_kernel = g_name_buf;
     return PHX_OK;
 }
@@ -544,9 +569,9 @@ static int run_wgrad(const Problem& p, hipStream_t st, const void* x, const void
     if (ws_bytes < pl.partial_bytes || !ws) return PHX_ERR_WORKSPACE;
     WgradArgs a;
     a.x.base = x; a.x.comp_stride = (long)p.n * p.ci_mem * p.h * p.w; a.x.N = p.n; a.x.C = p.ci; a.x.Cs = p.ci_mem; a.x.Hd = p.h; a.x.Wd = p.w;
-    a.x.uh = a.x.uw = 1; a.x.pw = 0; a.x.ncomp = p.real_input ? 1 : 4;
+    a.x.uh = a.x.uw = 1; a.x.pw = 0; a.x.tall = 0; a.x.ncomp = p.real_input ? 1 : 4;
     a.g.base = g; a.g.comp_stride = (long)p.n * p.co_mem * p.ho * p.wo; a.g.N = p.n; a.g.C = p.co; a.g.Cs = p.co_mem; a.g.Hd = p.ho; a.g.Wd = p.wo;
-    a.g.uh = a.g.uw = 1; a.g.pw = 0; a.g.ncomp = 4;
+    a.g.uh = a.g.uw = 1; a.g.pw = 0; a.g.tall = 0; a.g.ncomp = 4;
     a.partial = static_cast<float*>(ws);
     a.Kh = p.kh; a.Kw = p.kw; a.sh = p.sh; a.sw = p.sw; a.dh = p.dh; a.dw = p.dw; a.pt = p.pt; a.pl = p.pl;
     a.NB = pl.NB; a.TH = pl.TH; a.TW = pl.TW; a.KP = pl.KP; a.KPp = pl.KPp; a.HPp = pl.HPp; a.HTH = pl.HTH;

@@ -447,6 +447,53 @@ def test_channels_last(case, mode, dtype, policy):
         assert_close(dx.cpu().numpy().transpose(0, 3, 1, 2), want_dx, dtype, "channels-last dgrad " + name)
 
 
+# name, n, ci, co, h, w, kh, kw, stride, dilation, padding -- unit stride, more than one tap
+FLAT = [c for c in FP16_CASES if c[0] in ("k3_same", "k3_ragged", "k3_valid", "k3_dil2", "k4_same", "k24_c40", "k3_128_28")] + [
+    ("k3_7x7_n9", 9, 40, 40, 7, 7, 3, 3, 1, 1, "SAME"),              # several images per workgroup
+    ("k3_14_n5", 5, 64, 64, 14, 14, 3, 3, 1, 1, "SAME"),
+    ("k5_asym_pad", 3, 8, 8, 9, 12, 5, 3, 1, 1, (3, 0, 1, 2)),       # more rows read below the image than above
+    ("k3_full_pad", 2, 4, 4, 6, 10, 3, 3, 1, 1, (2, 2, 2, 2)),       # output larger than the input
+    ("k3_w29", 2, 8, 8, 5, 29, 3, 3, 1, 1, "SAME"),                  # odd width: scalar stores
+]
+
+
+@pytest.mark.parametrize("mode", [16, 8])
+@pytest.mark.parametrize("case", FLAT, ids=lambda c: c[0])
+def test_flat_tiling(case, mode, monkeypatch):
+    """Flat tiling of the fp16 LDS kernels (images stacked into one tall image, a workgroup takes consecutive
+    output positions in row-major order): the planner offers it by shape; PHX_TUNE_FLAT offers it everywhere
+    it applies, PHX_TUNE_NOFLAT nowhere.  Forward and input gradient against the oracle, and the two tilings
+    against each other."""
+    name, n, ci, co, h, w, kh, kw, stride, dilation, padding = case
+    dtype = torch.float16
+    g, x, wt, b, gr = make_inputs(name_seed(name) + 11, n, ci, co, h, w, kh, kw, stride, dilation, padding, dtype, 0.5)
+    desc = phx.Conv2DDescriptor(x.shape, wt.shape, stride, dilation, padding, use_bias=True, dtype=dtype,
+                                context=Ctx(mode, "full16"))
+    xd, wd, bd, gd = (torch.from_numpy(a).cuda() for a in (x, wt, b, gr))
+    x64, w64, b64, g64 = (a.astype(np.float64) for a in (x, wt, b, gr))
+    want_y = oracle.conv2d_fwd(g, x64, w64, b64, "hamilton")
+    _, want_dx = oracle.conv2d_bwd(g, x64, w64, g64, "hamilton")
+    got, names = {}, {}
+    for variant, env in (("flat", "PHX_TUNE_FLAT"), ("tiles", "PHX_TUNE_NOFLAT")):
+        monkeypatch.delenv("PHX_TUNE_FLAT", raising=False)
+        monkeypatch.delenv("PHX_TUNE_NOFLAT", raising=False)
+        monkeypatch.setenv(env, "1")
+        y = phx.conv2d_fwd(xd, wd, bd, desc)
+        k_fwd = capi.last_kernel_name()
+        _, dx = phx.conv2d_bwd(xd, wd, gd, desc)
+        k_bwd = capi.last_kernel_name()
+        print(name, mode, variant, k_fwd, k_bwd, flush=True)
+        assert_close(y.cpu().numpy(), want_y, dtype, "fwd " + k_fwd)
+        assert_close(dx.cpu().numpy(), want_dx, dtype, "dgrad " + k_bwd)
+        got[variant], names[variant] = (y, dx), (k_fwd, k_bwd)
+    assert all("_flat" not in k for k in names["tiles"])
+    # (narrow images with few output channels leave no workgroup shape whose window fits the staging limit)
+    if name in ("k3_same", "k3_ragged", "k3_dil2", "k3_128_28", "k3_7x7_n9", "k3_14_n5"):
+        assert all("_flat" in k for k in names["flat"]), names["flat"]
+    # same products in the same order per output position: the tilings agree exactly
+    assert torch.equal(got["flat"][0], got["tiles"][0]) and torch.equal(got["flat"][1], got["tiles"][1])
+
+
 STRIDED = [c for c in FP16_CASES if c[0] in ("k3_s2", "pw_s2", "k7_s2", "k3_s2_c4", "k5_s2_valid", "k3_s3", "k32_s21")]
 
 
