@@ -41,10 +41,10 @@ MEASURED_TRAFFIC = {
                        "bwd_weights": (100555.4 * 2 + 32768.0) * KIB},
     ("c3_k3_f32", 8): {"fwd": (150715.1 * 2 + 244946.0) * KIB, "bwd_data": (161077.9 * 2 + 246386.3) * KIB,
                        "bwd_weights": (379051.4 * 2 + 32256.0) * KIB},
-    ("c4_k3_f16_128_28", 16): {"fwd": (83632.0 * 2 + 105213.6) * KIB, "bwd_data": (83632.0 * 2 + 105213.6) * KIB,
-                               "bwd_weights": (179991.1 * 2 + 48384.0) * KIB},
-    ("c4_k3_f16_128_28", 8): {"fwd": (119307.0 * 2 + 104913.6) * KIB, "bwd_data": (123061.4 * 2 + 115787.4) * KIB,
-                              "bwd_weights": (179991.6 * 2 + 48384.0) * KIB},
+    ("c4_k3_f16_128_28", 16): {"fwd": (86388.7 * 2 + 111692.5) * KIB, "bwd_data": (86388.7 * 2 + 111692.5) * KIB,
+                               "bwd_weights": (180024.9 * 2 + 48384.0) * KIB},
+    ("c4_k3_f16_128_28", 8): {"fwd": (122328.1 * 2 + 112062.2) * KIB, "bwd_data": (121113.6 * 2 + 112644.7) * KIB,
+                              "bwd_weights": (180008.1 * 2 + 48384.0) * KIB},
 }
 
 
