@@ -143,34 +143,52 @@ struct TransposeArgs {
     int R, Cc;
 };
 
-// 64x64 tiles through LDS, coalesced along the contiguous axis on both sides; ragged edges are masked.
-// The tile pitch of 65 words (66 halves = 33 words) keeps the transposed reads on distinct banks.
+// A lane owns a square block of 16-byte rows (8x8 halves, 4x4 floats): it loads the block's rows, transposes it in
+// registers (byte permutes for halves, plain register renaming for floats) and stores the transposed rows; the
+// 64 lanes of a wave form an 8x8 grid of blocks, so that each load instruction covers 128 contiguous bytes of
+// eight source rows and each store instruction 128 contiguous bytes of eight destination rows.  Rows start at
+// element alignment only, which the 16-byte accesses tolerate.  Blocks cut by the matrix edge go element by element.
 template <typename TS>
 __global__ void __launch_bounds__(WG_THREADS) transpose_kernel(const TransposeArgs A) {
-    constexpr int T = 64, PITCH = sizeof(TS) == 4 ? T + 1 : T + 2;
-    __shared__ TS tile[T * PITCH];
+    constexpr int V = 16 / sizeof(TS), T = 8 * V;
+    typedef const __attribute__((address_space(1))) u32x4_a2* gload;
+    typedef __attribute__((address_space(1))) u32x4_a2* gstore;
     const TS* src = static_cast<const TS*>(A.src);
     TS* dst = static_cast<TS*>(A.dst);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int rg = lane >> 3, cg = lane & 7;
     const int tr = (A.R + T - 1) / T, tc = (A.Cc + T - 1) / T;
     const long tiles = A.batch * tr * tc;
-    const int lane = threadIdx.x % T, row0 = threadIdx.x / T;  // 256 threads: 4 tile rows per sweep
-    for (long t = blockIdx.x; t < tiles; t += gridDim.x) {
+    constexpr int WAVES = WG_THREADS / 64;
+    for (long t = (long)blockIdx.x * WAVES + wave; t < tiles; t += (long)gridDim.x * WAVES) {
         const long b = t / ((long)tr * tc);
         const int rem = (int)(t - b * tr * tc);
-        const int r0 = (rem / tc) * T, c0 = (rem % tc) * T;
+        const int r0 = (rem / tc) * T + rg * V, c0 = (rem % tc) * T + cg * V;
         const TS* s = src + b * A.R * (long)A.Cc;
         TS* d = dst + b * A.R * (long)A.Cc;
-        __syncthreads();  // the previous tile has been read out
-#pragma unroll 4
-        for (int i = row0; i < T; i += WG_THREADS / T) {
-            const int r = r0 + i, c = c0 + lane;
-            if (r < A.R && c < A.Cc) tile[i * PITCH + lane] = s[(long)r * A.Cc + c];
-        }
-        __syncthreads();
-#pragma unroll 4
-        for (int i = row0; i < T; i += WG_THREADS / T) {
-            const int c = c0 + i, r = r0 + lane;
-            if (c < A.Cc && r < A.R) d[(long)c * A.R + r] = tile[lane * PITCH + i];
+        if (r0 + V <= A.R && c0 + V <= A.Cc) {
+            u32x4 in[V], out[V];
+#pragma unroll
+            for (int i = 0; i < V; ++i) in[i] = *(gload)(s + (long)(r0 + i) * A.Cc + c0);
+            if constexpr (sizeof(TS) == 4) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) out[j][i] = in[i][j];
+            } else {
+                // dword m of output row j: element j of input rows 2m and 2m+1
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+#pragma unroll
+                    for (int m = 0; m < 4; ++m)
+                        out[j][m] = __builtin_amdgcn_perm(in[2 * m + 1][j >> 1], in[2 * m][j >> 1],
+                                                          (j & 1) ? 0x07060302u : 0x05040100u);
+            }
+#pragma unroll
+            for (int j = 0; j < V; ++j) *(gstore)(d + (long)(c0 + j) * A.R + r0) = out[j];
+        } else if (r0 < A.R && c0 < A.Cc) {
+            for (int i = 0; i < V && r0 + i < A.R; ++i)
+                for (int j = 0; j < V && c0 + j < A.Cc; ++j) d[(long)(c0 + j) * A.R + r0 + i] = s[(long)(r0 + i) * A.Cc + c0 + j];
         }
     }
 }

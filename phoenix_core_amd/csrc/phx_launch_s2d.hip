@@ -52,9 +52,10 @@ int launch_phase_merge(bool half_storage, const PhaseMergeArgs& a, hipStream_t s
 }
 
 int launch_transpose(bool half_storage, const TransposeArgs& a, hipStream_t st) {
-    const long tiles = a.batch * ((a.R + 63) / 64) * ((a.Cc + 63) / 64);
+    const int T = half_storage ? 64 : 32;  // tile edge of one wave
+    const long tiles = a.batch * ((a.R + T - 1) / T) * ((a.Cc + T - 1) / T);
     if (tiles == 0) return 0;
-    const int blocks = (int)std::min<long>(tiles, 1 << 16);
+    const int blocks = (int)std::min<long>((tiles + 3) / 4, 1 << 16);
     if (half_storage) hipLaunchKernelGGL((transpose_kernel<_Float16>), dim3(blocks), dim3(WG_THREADS), 0, st, a);
     else hipLaunchKernelGGL((transpose_kernel<float>), dim3(blocks), dim3(WG_THREADS), 0, st, a);
     return 0;
