@@ -31,7 +31,10 @@ class _QConv2dFn(torch.autograd.Function):
         db = None
         if ctx.has_bias:  # bias enters every output component once: plain reduction
             n = grad.shape[0] // 4
-            db = grad.view(4, n, grad.shape[1], -1).float().sum(dim=(1, 3)).to(grad.dtype)
+            if ctx.bdesc.data_format == "NHWC":
+                db = grad.view(4, n, -1, grad.shape[3]).float().sum(dim=(1, 2)).to(grad.dtype)
+            else:
+                db = grad.view(4, n, grad.shape[1], -1).float().sum(dim=(1, 3)).to(grad.dtype)
         return dx, dw, db, None, None
 
 
@@ -59,12 +62,17 @@ class QConv2d(nn.Module):
     """Quaternion Conv2D: x [4N, Ci, H, W] -> y [4N, Co, Ho, Wo]; padding 'SAME' / 'VALID' as in
     the reference's descriptors (src/backend/conv2d_descriptor.hpp:132-174).  With real_input the
     layer takes a real tensor [N, Ci, H, W] (realValuedInput of the reference) and, as there, gives
-    no gradient for it."""
+    no gradient for it.  groups > 1: grouped convolution, filter [4, Co, Ci / groups, Kh, Kw].  data_format
+    "NHWC": activations [4N, H, W, C] (the filter stays OIHW)."""
 
     def __init__(self, in_channels, out_channels, kernel_size, stride=1, padding="SAME", dilation=1, bias=False,
-                 dtype=torch.float32, context=None, input_requires_grad=True, real_input=False):
+                 dtype=torch.float32, context=None, input_requires_grad=True, real_input=False, groups=1,
+                 data_format="NCHW"):
         super().__init__()
-        self.real_input = real_input
+        if in_channels % groups or out_channels % groups:
+            raise ValueError("channel counts must be multiples of groups")
+        self.real_input, self.groups, self.data_format = real_input, groups, data_format
+        in_channels //= groups  # per group from here on: fan-in and the filter's input-channel axis
         input_requires_grad = input_requires_grad and not real_input
         k = (kernel_size, kernel_size) if isinstance(kernel_size, int) else tuple(kernel_size)
         self.stride, self.padding, self.dilation = stride, padding, dilation
@@ -80,7 +88,8 @@ class QConv2d(nn.Module):
         key = (tuple(x.shape), x.dtype)
         if key not in self._descs:
             common = dict(stride=self.stride, dilation=self.dilation, padding=self.padding, dtype=x.dtype,
-                          context=self.context, real_valued_input=self.real_input)
+                          context=self.context, real_valued_input=self.real_input, groups=self.groups,
+                          data_format=self.data_format)
             fwd = ops.Conv2DDescriptor(x.shape, self.weight.shape, use_bias=self.bias is not None, **common)
             bwd = ops.Conv2DDescriptor(x.shape, self.weight.shape, require_input_grad=self.input_requires_grad, **common)
             self._descs[key] = (fwd, bwd)

@@ -41,6 +41,48 @@ def test_qconv2d_autograd_matches_oracle(mode):
         assert np.abs(got - want).max() / np.abs(want).max() < 1e-4
 
 
+def test_qconv2d_groups_and_channels_last():
+    """QConv2d(groups=G) is G ungrouped layers on channel slices; QConv2d(data_format="NHWC") is the NCHW layer on
+    permuted activations: outputs and all gradients must agree with those compositions."""
+    torch.manual_seed(1)
+    n, ci, co, h, G = 2, 8, 12, 10, 2
+    ref = phx.QConv2d(ci, co, 3, padding="SAME", bias=True, context=Ctx(8), groups=G).cuda()
+    assert tuple(ref.weight.shape) == (4, co, ci // G, 3, 3)
+    with torch.no_grad():
+        ref.bias.normal_()
+    x = torch.randn(4 * n, ci, h, h, device="cuda", requires_grad=True)
+    y = ref(x)
+    gr = torch.randn_like(y)
+    y.backward(gr)
+    # G ungrouped layers on the slices
+    cig, cog = ci // G, co // G
+    for k in range(G):
+        part = phx.QConv2d(cig, cog, 3, padding="SAME", bias=True, context=Ctx(8)).cuda()
+        with torch.no_grad():
+            part.weight.copy_(ref.weight[:, k * cog:(k + 1) * cog])
+            part.bias.copy_(ref.bias[:, k * cog:(k + 1) * cog])
+        xs = x.detach()[:, k * cig:(k + 1) * cig].contiguous().requires_grad_()
+        ys = part(xs)
+        ys.backward(gr[:, k * cog:(k + 1) * cog].contiguous())
+        torch.testing.assert_close(y[:, k * cog:(k + 1) * cog], ys, rtol=1e-4, atol=1e-4)
+        torch.testing.assert_close(x.grad[:, k * cig:(k + 1) * cig], xs.grad, rtol=1e-4, atol=1e-4)
+        torch.testing.assert_close(ref.weight.grad[:, k * cog:(k + 1) * cog], part.weight.grad, rtol=1e-4, atol=1e-4)
+        torch.testing.assert_close(ref.bias.grad[:, k * cog:(k + 1) * cog], part.bias.grad, rtol=1e-4, atol=1e-4)
+    # the same layer on channels-last activations
+    last = phx.QConv2d(ci, co, 3, padding="SAME", bias=True, context=Ctx(8), groups=G, data_format="NHWC").cuda()
+    with torch.no_grad():
+        last.weight.copy_(ref.weight)
+        last.bias.copy_(ref.bias)
+    xl = x.detach().permute(0, 2, 3, 1).contiguous().requires_grad_()
+    yl = last(xl)
+    assert tuple(yl.shape) == (4 * n, h, h, co)
+    yl.backward(gr.permute(0, 2, 3, 1).contiguous())
+    torch.testing.assert_close(yl.permute(0, 3, 1, 2), y, rtol=1e-4, atol=1e-4)
+    torch.testing.assert_close(xl.grad.permute(0, 3, 1, 2), x.grad, rtol=1e-4, atol=1e-4)
+    torch.testing.assert_close(last.weight.grad, ref.weight.grad, rtol=1e-4, atol=1e-4)
+    torch.testing.assert_close(last.bias.grad, ref.bias.grad, rtol=1e-4, atol=1e-4)
+
+
 def test_qlinear_autograd_matches_oracle():
     torch.manual_seed(1)
     lin = phx.QLinear(12, 7, bias=True, context=Ctx(8)).cuda()
