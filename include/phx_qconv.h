@@ -35,7 +35,12 @@ enum phx_status {
 
 enum phx_dtype { PHX_F32 = 0, PHX_F16 = 1 };
 
-enum phx_filter_layout { PHX_OIHW = 0, PHX_OHWI = 1 };
+/* Filter layouts (FilterLayout, src/backend/types.hpp:91-97; dimension order src/backend/conv2d_descriptor.hpp:14-37):
+ * the component index is outermost in all of them, [4, O, I, H, W] / [4, O, H, W, I] / [4, H, W, I, O]. */
+enum phx_filter_layout { PHX_OIHW = 0, PHX_OHWI = 1, PHX_HWIO = 2 };
+
+/* Dense filter layouts (src/backend/dense_descriptor.hpp:30-37): [4, in, out] or [4, out, in]. */
+enum phx_dense_layout { PHX_IO = 0, PHX_OI = 1 };
 
 /* Layout of the activation tensors (DataFormat, src/backend/types.hpp:85; dimension numbers
  * src/backend/tensor.hpp:17-31).  The kernels compute on channels-first planes; a channels-last call
@@ -83,12 +88,13 @@ typedef struct phx_qconv_desc {
                               must be 0 (src/conv2d.hpp:125-127) and
                               phx_qconv2d_bwd_data is refused as the reference refuses it (src/conv2d.hpp:394-398) */
     int32_t groups;        /* grouped convolution: ci and co are the totals, both multiples of groups; the filter is
-                              [4, co, ci/groups, kh, kw] (OHWI: [4, co, kh, kw, ci/groups]); 0 or 1 = ungrouped */
+                              [4, co, ci/groups, kh, kw] (OHWI: [4, co, kh, kw, ci/groups], HWIO: [4, kh, kw, ci/groups,
+                              co]); 0 or 1 = ungrouped */
     int32_t data_format;   /* phx_data_format of x, y and their gradients: PHX_NCHW [4n, c, h, w] or PHX_NHWC
                               [4n, h, w, c]; filters and bias are unaffected (filter_layout is separate) */
 } phx_qconv_desc;
 
-/* Quaternion Dense geometry (src/backend/dense_descriptor.hpp:11-59); filter layout is IO. */
+/* Quaternion Dense geometry (src/backend/dense_descriptor.hpp:11-59). */
 typedef struct phx_qdense_desc {
     int32_t dtype;
     int32_t n;             /* batch; activation tensors have 4*n rows */
@@ -96,6 +102,7 @@ typedef struct phx_qdense_desc {
     int32_t product_mode;
     int32_t fp16_policy;
     int32_t has_bias;
+    int32_t filter_layout; /* phx_dense_layout */
 } phx_qdense_desc;
 
 const char* phx_status_string(int status);

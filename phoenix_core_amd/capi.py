@@ -11,7 +11,8 @@ LIB_PATH = os.path.join(_HERE, "lib", "libphx_qconv.so")
 PHX_OK = 0
 PHX_ERR_INVALID_ARGUMENT, PHX_ERR_NOT_SUPPORTED, PHX_ERR_WORKSPACE, PHX_ERR_RUNTIME = 1, 2, 3, 4
 PHX_F32, PHX_F16 = 0, 1
-PHX_OIHW, PHX_OHWI = 0, 1
+PHX_OIHW, PHX_OHWI, PHX_HWIO = 0, 1, 2
+PHX_IO, PHX_OI = 0, 1
 PHX_NCHW, PHX_NHWC = 0, 1
 PHX_PRODUCT_16, PHX_PRODUCT_8 = 16, 8
 PHX_FP16_FULL32, PHX_FP16_BACKWARD32, PHX_FP16_FULL16 = 0, 1, 2
@@ -45,7 +46,8 @@ class QConvDesc(ctypes.Structure):
 
 
 class QDenseDesc(ctypes.Structure):
-    _fields_ = [(k, ctypes.c_int32) for k in ("dtype", "n", "ni", "no", "product_mode", "fp16_policy", "has_bias")]
+    _fields_ = [(k, ctypes.c_int32) for k in ("dtype", "n", "ni", "no", "product_mode", "fp16_policy", "has_bias",
+                                               "filter_layout")]
 
 
 class PhxError(RuntimeError):

@@ -79,7 +79,8 @@ static int problem_from_conv(const phx_qconv_desc* d, Problem& p) {
     if (d->dtype != PHX_F32 && d->dtype != PHX_F16) return PHX_ERR_INVALID_ARGUMENT;
     if (d->product_mode != PHX_PRODUCT_16 && d->product_mode != PHX_PRODUCT_8) return PHX_ERR_INVALID_ARGUMENT;
     if (d->fp16_policy < PHX_FP16_FULL32 || d->fp16_policy > PHX_FP16_FULL16) return PHX_ERR_INVALID_ARGUMENT;
-    if (d->filter_layout != PHX_OIHW && d->filter_layout != PHX_OHWI) return PHX_ERR_INVALID_ARGUMENT;
+    if (d->filter_layout != PHX_OIHW && d->filter_layout != PHX_OHWI && d->filter_layout != PHX_HWIO)
+        return PHX_ERR_INVALID_ARGUMENT;
     if (d->n < 0 || d->ci <= 0 || d->co <= 0 || d->h < 0 || d->w < 0 || d->kh <= 0 || d->kw <= 0)
         return PHX_ERR_INVALID_ARGUMENT;
     if (d->stride_h <= 0 || d->stride_w <= 0 || d->dilation_h <= 0 || d->dilation_w <= 0)
@@ -105,8 +106,10 @@ static int problem_from_conv(const phx_qconv_desc* d, Problem& p) {
     p.fs.wcs = (long)p.co_mem * p.ci * taps;  // filter [4][co_mem][ci per group][kh][kw]
     if (d->filter_layout == PHX_OIHW) {
         p.fs.so = p.ci * taps; p.fs.si = taps; p.fs.skh = p.kw; p.fs.skw = 1;
-    } else {  // OHWI
+    } else if (d->filter_layout == PHX_OHWI) {
         p.fs.so = taps * p.ci; p.fs.si = 1; p.fs.skh = (long)p.kw * p.ci; p.fs.skw = p.ci;
+    } else {  // HWIO: [kh][kw][ci per group][co_mem]
+        p.fs.so = 1; p.fs.si = p.co_mem; p.fs.skw = (long)p.ci * p.co_mem; p.fs.skh = (long)p.kw * p.ci * p.co_mem;
     }
     p.has_bias = d->has_bias != 0;
     p.real_input = d->real_input != 0;
@@ -120,11 +123,14 @@ static int problem_from_dense(const phx_qdense_desc* d, Problem& p) {
     if (d->product_mode != PHX_PRODUCT_16 && d->product_mode != PHX_PRODUCT_8) return PHX_ERR_INVALID_ARGUMENT;
     if (d->fp16_policy < PHX_FP16_FULL32 || d->fp16_policy > PHX_FP16_FULL16) return PHX_ERR_INVALID_ARGUMENT;
     if (d->n < 0 || d->ni <= 0 || d->no <= 0) return PHX_ERR_INVALID_ARGUMENT;
+    if (d->filter_layout != PHX_IO && d->filter_layout != PHX_OI) return PHX_ERR_INVALID_ARGUMENT;
     p.dtype = d->dtype; p.mode = d->product_mode; p.policy = d->fp16_policy;
     p.n = d->n; p.ci = d->ni; p.co = d->no; p.h = p.w = 1; p.kh = p.kw = 1;
     p.sh = p.sw = p.dh = p.dw = 1; p.pt = p.pl = p.pb = p.pr = 0; p.ho = p.wo = 1;
-    // layout IO: w[r][i][o]
-    p.fs.wcs = (long)p.ci * p.co; p.fs.so = 1; p.fs.si = p.co; p.fs.skh = 0; p.fs.skw = 0;
+    // layout IO: w[r][i][o]; OI: w[r][o][i]
+    p.fs.wcs = (long)p.ci * p.co; p.fs.skh = 0; p.fs.skw = 0;
+    if (d->filter_layout == PHX_IO) { p.fs.so = 1; p.fs.si = p.co; }
+    else { p.fs.so = p.ci; p.fs.si = 1; }
     p.has_bias = d->has_bias != 0;
     p.real_input = false;
     p.groups = 1; p.ci_mem = p.ci; p.co_mem = p.co;

@@ -714,8 +714,8 @@ inline phx_qconv_desc makeConvDesc(const Conv2DDescriptor& d, Context& ctx, int 
     const DataFormat df = d.getDataFormat();
     if (df != DataFormat::NCHW && df != DataFormat::NHWC) throw std::runtime_error("device::HIP runs NCHW or NHWC tensors");
     const FilterLayout fl = d.getFilterLayout();
-    if (fl != FilterLayout::OIHW && fl != FilterLayout::OHWI)
-        throw std::runtime_error("device::HIP takes OIHW or OHWI filters");
+    if (fl != FilterLayout::OIHW && fl != FilterLayout::OHWI && fl != FilterLayout::HWIO)
+        throw std::runtime_error("device::HIP takes OIHW, OHWI or HWIO filters");
     Conv2DFilterLayout filter(fl, Algebra::QUATERNION);
     const Shape& in = d.getInputShape();
     const Shape& w = d.getFilterShape();
@@ -735,7 +735,7 @@ inline phx_qconv_desc makeConvDesc(const Conv2DDescriptor& d, Context& ctx, int 
     c.dilation_h = d.getDilation().x; c.dilation_w = d.getDilation().y;
     c.pad_top = d.getPaddingBefore().x; c.pad_left = d.getPaddingBefore().y;
     c.pad_bottom = d.getPaddingAfter().x; c.pad_right = d.getPaddingAfter().y;
-    c.filter_layout = fl == FilterLayout::OIHW ? PHX_OIHW : PHX_OHWI;
+    c.filter_layout = fl == FilterLayout::OIHW ? PHX_OIHW : fl == FilterLayout::OHWI ? PHX_OHWI : PHX_HWIO;
     c.product_mode = ctx.phxProductMode();
     c.fp16_policy = ctx.phxFp16Policy();
     c.has_bias = (useBias && !real) ? 1 : 0;  // a bias given with a real-valued input is refused at call time
@@ -748,12 +748,14 @@ inline phx_qconv_desc makeConvDesc(const Conv2DDescriptor& d, Context& ctx, int 
 inline phx_qdense_desc makeDenseDesc(const DenseDescriptor& d, Context& ctx, int dtype, bool useBias) {
     if (d.getAlgebra() != Algebra::QUATERNION)
         throw std::runtime_error("Only the quaternion algebra is built for device::HIP");
-    if (d.getFilterLayout() != FilterLayout::IO) throw std::runtime_error("device::HIP takes dense filters in IO layout");
+    const bool io = d.getFilterLayout() == FilterLayout::IO;
+    if (!io && d.getFilterLayout() != FilterLayout::OI) throw std::runtime_error("device::HIP takes dense filters in IO or OI layout");
     const Shape in = d.getInputShape(), w = d.getFilterShape();
-    if (in.getSize() != 2 || w.getSize() != 3 || w[0] != 4 || in[0] % 4 != 0 || in[1] != w[1])
-        throw std::invalid_argument("Dense expects input [4n, in] and filter [4, in, out]");
+    if (in.getSize() != 2 || w.getSize() != 3 || w[0] != 4 || in[0] % 4 != 0 || in[1] != w[io ? 1 : 2])
+        throw std::invalid_argument("Dense expects input [4n, in] and filter [4, in, out] (IO) or [4, out, in] (OI)");
     phx_qdense_desc c;
-    c.dtype = dtype; c.n = in[0] / 4; c.ni = w[1]; c.no = w[2];
+    c.dtype = dtype; c.n = in[0] / 4; c.ni = w[io ? 1 : 2]; c.no = w[io ? 2 : 1];
+    c.filter_layout = io ? PHX_IO : PHX_OI;
     c.product_mode = ctx.phxProductMode(); c.fp16_policy = ctx.phxFp16Policy(); c.has_bias = useBias ? 1 : 0;
     return c;
 }

@@ -104,6 +104,8 @@ class Conv2DDescriptor:
             _, co, ci, kh, kw = filter_shape
         elif filter_layout == "OHWI":
             _, co, kh, kw, ci = filter_shape
+        elif filter_layout == "HWIO":
+            _, kh, kw, ci, co = filter_shape
         else:
             raise ValueError("Unsupported Conv2D filter layout")
         # grouped convolution: the filter holds the input channels of one group (src/backend/conv2d_descriptor.hpp)
@@ -142,7 +144,7 @@ class Conv2DDescriptor:
         self.bias_shape = (4, co) if use_bias else ()
         self.c = capi.QConvDesc(
             _DTYPES[dtype], n4 // 4, ci, co, h, w, kh, kw, self.stride[0], self.stride[1], self.dilation[0],
-            self.dilation[1], pt, pl, pb, pr, capi.PHX_OIHW if filter_layout == "OIHW" else capi.PHX_OHWI,
+            self.dilation[1], pt, pl, pb, pr, {"OIHW": capi.PHX_OIHW, "OHWI": capi.PHX_OHWI, "HWIO": capi.PHX_HWIO}[filter_layout],
             self.context.product_mode, self.context.fp16_policy, int(self.use_bias and not self.real_valued_input),
             int(self.real_valued_input), groups, capi.PHX_NCHW if data_format == "NCHW" else capi.PHX_NHWC)
 
@@ -151,27 +153,31 @@ class Conv2DDescriptor:
 
 
 class DenseDescriptor:
-    """DenseFwdDescriptor / DenseBwdDescriptor for the quaternion algebra, filter layout IO."""
+    """DenseFwdDescriptor / DenseBwdDescriptor for the quaternion algebra; filter [4, in, out] ("IO") or
+    [4, out, in] ("OI")."""
 
     def __init__(self, input_shape, filter_shape, algebra=QUATERNION, filter_layout="IO", use_bias=False,
                  dtype=torch.float32, context=None, require_input_grad=True):
         if algebra != QUATERNION:
             raise NotImplementedError("only the quaternion algebra is built on this device")
-        if filter_layout != "IO":
-            raise NotImplementedError("dense filters are taken in IO layout only")
+        if filter_layout not in ("IO", "OI"):
+            raise ValueError("Unsupported Dense filter layout")
         if len(input_shape) != 2 or len(filter_shape) != 3 or filter_shape[0] != 4:
-            raise ValueError("expected input [4n, in] and filter [4, in, out]")
+            raise ValueError("expected input [4n, in] and filter [4, in, out] (IO) or [4, out, in] (OI)")
+        n_in, n_out = filter_shape[1:] if filter_layout == "IO" else filter_shape[:0:-1]
+        self.filter_layout = filter_layout
         if input_shape[0] % 4:
             raise ValueError("Cannot split %d onto 4 parts" % input_shape[0])
-        if input_shape[1] != filter_shape[1]:
+        if input_shape[1] != n_in:
             raise ValueError("input features do not match the filter")
         self.context = context or default_context()
         self.input_shape, self.filter_shape = tuple(input_shape), tuple(filter_shape)
         self.use_bias, self.require_input_grad, self.dtype = bool(use_bias), bool(require_input_grad), dtype
-        self.output_shape = (input_shape[0], filter_shape[2])
-        self.bias_shape = (4, filter_shape[2]) if use_bias else ()
-        self.c = capi.QDenseDesc(_DTYPES[dtype], input_shape[0] // 4, filter_shape[1], filter_shape[2],
-                                 self.context.product_mode, self.context.fp16_policy, int(self.use_bias))
+        self.output_shape = (input_shape[0], n_out)
+        self.bias_shape = (4, n_out) if use_bias else ()
+        self.c = capi.QDenseDesc(_DTYPES[dtype], input_shape[0] // 4, n_in, n_out,
+                                 self.context.product_mode, self.context.fp16_policy, int(self.use_bias),
+                                 capi.PHX_IO if filter_layout == "IO" else capi.PHX_OI)
 
     def workspace_bytes(self, which):
         return capi.lib().phx_qdense_workspace_bytes(ctypes.byref(self.c), which)

@@ -391,6 +391,24 @@ def test_reference_kat_channels_last():
             assert not y[1:].any()
 
 
+def test_reference_kat_channels_last_hwio():
+    """tests/tests.cpp:492-547 of the reference (CPU only there): the same real NHWC image through the filter in
+    HWIO layout {1,0, 1,0, 1,2} -> (0,2, 2,4, 3,6, 5,8), run as the real part of a quaternion convolution."""
+    x = [0, -1, 1, 0, 0, 2, 0, 0, 3, 1, 0, 4]
+    k = [1, 0, 1, 0, 1, 2]
+    want = [0, 2, 2, 4, 3, 6, 5, 8]
+    for mode in (8, 16):
+        xd = torch.tensor(x, dtype=torch.float32, device="cuda").reshape(1, 2, 2, 3)
+        wd = torch.zeros(4, 1, 1, 3, 2, device="cuda")
+        wd[0] = torch.tensor(k, dtype=torch.float32, device="cuda").reshape(1, 1, 3, 2)
+        desc = phx.Conv2DDescriptor(xd.shape, wd.shape, 1, 1, "VALID", filter_layout="HWIO", context=Ctx(mode),
+                                    real_valued_input=True, data_format="NHWC")
+        assert desc.output_shape == (4, 2, 2, 2)
+        y = phx.conv2d_fwd(xd, wd, None, desc)
+        assert y[0].flatten().tolist() == [float(v) for v in want], mode
+        assert not y[1:].any()
+
+
 # name, groups, real input, OHWI filter, n, ci, co, h, w, kh, kw, stride, dilation, padding
 CHANNELS_LAST = [
     ("nhwc_pw", 1, False, True, 2, 64, 64, 14, 14, 1, 1, 1, 1, "VALID"),

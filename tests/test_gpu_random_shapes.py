@@ -54,6 +54,7 @@ def draw(seed):
                dilation=dilation, padding=padding, mode=int(r.choice([8, 16])), ohwi=bool(r.random() < 0.25),
                bias=bool(r.random() < 0.5), real=bool(r.random() < 0.2), seed=seed)
     cfg["nhwc"] = bool(r.random() < 0.25)
+    cfg["layout"] = "HWIO" if r.random() < 0.15 else ("OHWI" if cfg["ohwi"] else "OIHW")
     return cfg, r
 
 
@@ -69,7 +70,9 @@ def run_case(cfg, r, dtype, policy):
     real, bias = cfg["real"], cfg["bias"] and not cfg["real"]
     if real:
         x[n:] = 0  # the oracle sees the same input with explicit zero imaginary parts
-    w_dev = np.ascontiguousarray(wt.transpose(0, 1, 3, 4, 2)) if cfg["ohwi"] else wt
+    to_layout = {"OIHW": (0, 1, 2, 3, 4), "OHWI": (0, 1, 3, 4, 2), "HWIO": (0, 3, 4, 2, 1)}[cfg["layout"]]
+    from_layout = tuple(int(i) for i in np.argsort(to_layout))
+    w_dev = np.ascontiguousarray(wt.transpose(to_layout))
     x_dev = np.ascontiguousarray(x[:n]) if real else x
     nhwc = cfg["nhwc"]
     to_dev = (lambda a: np.ascontiguousarray(a.transpose(0, 2, 3, 1))) if nhwc else (lambda a: a)
@@ -77,7 +80,7 @@ def run_case(cfg, r, dtype, policy):
     x_dev, g_dev = to_dev(x_dev), to_dev(gr)
     ctx = Ctx(cfg["mode"], policy)
     desc = phx.Conv2DDescriptor(x_dev.shape, w_dev.shape, cfg["stride"], cfg["dilation"], cfg["padding"],
-                                filter_layout="OHWI" if cfg["ohwi"] else "OIHW", use_bias=bias, dtype=dtype, context=ctx,
+                                filter_layout=cfg["layout"], use_bias=bias, dtype=dtype, context=ctx,
                                 real_valued_input=real, require_input_grad=not real,
                                 data_format="NHWC" if nhwc else "NCHW")
     assert desc.output_shape == ((4 * n, geom.ho, geom.wo, co) if nhwc else (4 * n, co, geom.ho, geom.wo)), cfg
@@ -90,7 +93,7 @@ def run_case(cfg, r, dtype, policy):
     want_dw, want_dx = oracle.conv2d_bwd(geom, x64, w64, g64, "hamilton")
     close(from_dev(y.cpu().numpy()), want_y, dtype, "fwd %s" % cfg)
     got_dw = dw.cpu().numpy()
-    close(got_dw.transpose(0, 1, 4, 2, 3) if cfg["ohwi"] else got_dw, want_dw, dtype, "wgrad %s" % cfg)
+    close(got_dw.transpose(from_layout), want_dw, dtype, "wgrad %s" % cfg)
     if real:
         assert dx is None
     else:
@@ -128,8 +131,11 @@ def test_random_dense(seed):
     w = r.uniform(-lim, lim, (4, ni, no)).astype(npdt)
     b = (scale * r.standard_normal((4, no))).astype(npdt)
     gr = (scale * r.standard_normal((4 * n, no))).astype(npdt)
-    desc = phx.DenseDescriptor(x.shape, w.shape, use_bias=bias, dtype=dtype, context=Ctx(mode, policy))
-    xd, wd, bd, gd = (torch.from_numpy(a).cuda() for a in (x, w, b, gr))
+    oi = seed % 3 == 2  # filter [4, out, in]
+    w_dev = np.ascontiguousarray(w.transpose(0, 2, 1)) if oi else w
+    desc = phx.DenseDescriptor(x.shape, w_dev.shape, filter_layout="OI" if oi else "IO", use_bias=bias, dtype=dtype,
+                               context=Ctx(mode, policy))
+    xd, wd, bd, gd = (torch.from_numpy(a).cuda() for a in (x, w_dev, b, gr))
     y = phx.dense_fwd(xd, wd, bd if bias else None, desc)
     dw, dx = phx.dense_bwd(xd, wd, gd, desc)
     x64, w64, b64, g64 = (a.astype(np.float64) for a in (x, w, b, gr))
@@ -137,4 +143,5 @@ def test_random_dense(seed):
     want_dw, want_dx = oracle.dense_bwd(x64, w64, g64, "generic")
     close(y.cpu().numpy(), want_y, dtype, "dense fwd")
     close(dx.cpu().numpy(), want_dx, dtype, "dense dgrad")
-    close(dw.cpu().numpy(), want_dw, dtype, "dense wgrad")
+    got_dw = dw.cpu().numpy()
+    close(got_dw.transpose(0, 2, 1) if oi else got_dw, want_dw, dtype, "dense wgrad")
