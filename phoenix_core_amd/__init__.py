@@ -3,6 +3,6 @@
 The arithmetic lives in hand-written HIP kernels (csrc/) behind a C ABI (include/phx_qconv.h);
 `ops` is the Python host mirror of the reference's operator interface for this path."""
 from . import capi  # noqa: F401
-from .ops import (Context, Conv2DDescriptor, DenseDescriptor, conv2d_bwd, conv2d_fwd, default_context,  # noqa: F401
-                  dense_bwd, dense_fwd, windowed_output_size_and_padding)
+from .ops import (COMPLEX, GA_300, QUATERNION, REAL, Context, Conv2DDescriptor, DenseDescriptor, conv2d_bwd,  # noqa: F401
+                  conv2d_fwd, default_context, dense_bwd, dense_fwd, windowed_output_size_and_padding)
 from .nn import QBatchNorm2d, QConv2d, QLinear, QResNet50  # noqa: F401,E402

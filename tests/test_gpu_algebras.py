@@ -1,0 +1,127 @@
+"""GPU parity of the other algebras (REAL, COMPLEX, GA_300), which run as compositions on the quaternion kernels
+(phoenix_core_amd/algebras.py): the reference's known-answer vectors (tests/golden/reference_kats.json, from
+tests/tests.cpp:224-290, 371-423, 562-648) exactly, and forward / backward passes of random problems against the
+oracle's generic path, which walks the reference's sign tables.  Tolerances as in test_gpu_parity.py."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import phoenix_core_amd as phx
+from phoenix_core_amd import algebras
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.float32: 1e-4, torch.float16: 2e-2}
+KATS = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "reference_kats.json")))
+
+
+class Ctx(phx.Context):
+    def __init__(self, mode, policy="fp32"):
+        env = {"UPSTRIDE_CONV_FP16_POLICY": policy}
+        if mode == 16:
+            env["UPSTRIDE_MEMORY_OPTIMIZED"] = "1"
+        super().__init__(env)
+
+
+def close(got, want, dtype, what):
+    got = got.astype(np.float64)
+    assert got.shape == want.shape, what
+    d = np.abs(got - want)
+    e_max = d.max() / max(np.abs(want).max(), 1e-30)
+    e_l2 = np.sqrt((d ** 2).sum()) / max(np.sqrt((want ** 2).sum()), 1e-30)
+    assert np.isfinite(got).all(), what
+    assert e_max <= TOL[dtype] and e_l2 <= TOL[dtype], "%s: rel max %.3e, rel l2 %.3e" % (what, e_max, e_l2)
+
+
+@pytest.mark.parametrize("mode", [8, 16])
+@pytest.mark.parametrize("kat", [k for k in KATS["conv2d"] if k["algebra"] != phx.QUATERNION], ids=lambda k: k["name"])
+def test_reference_conv_vectors(kat, mode):
+    d = algebras.DIMS[kat["algebra"]]
+    x = torch.tensor(kat["input"], dtype=torch.float32, device="cuda").reshape(d * kat["n"], kat["ci"], kat["h"], kat["w"])
+    w = torch.tensor(kat["filter"], dtype=torch.float32, device="cuda").reshape(d, kat["co"], kat["ci"], kat["kh"], kat["kw"])
+    desc = phx.Conv2DDescriptor(x.shape, w.shape, 1, 1, kat["padding"], algebra=kat["algebra"], context=Ctx(mode))
+    y = phx.conv2d_fwd(x, w, None, desc)
+    assert y.flatten().tolist() == [float(v) for v in kat["output"]]
+
+
+@pytest.mark.parametrize("mode", [8, 16])
+@pytest.mark.parametrize("kat", KATS["dense"], ids=lambda k: k["name"])
+def test_reference_dense_vectors(kat, mode):
+    d = algebras.DIMS[kat["algebra"]]
+    x = torch.tensor(kat["input"], dtype=torch.float32, device="cuda").reshape(d * kat["n"], kat["ni"])
+    w = torch.tensor(kat["filter"], dtype=torch.float32, device="cuda").reshape(d, kat["ni"], kat["no"])
+    desc = phx.DenseDescriptor(x.shape, w.shape, algebra=kat["algebra"], context=Ctx(mode))
+    y = phx.dense_fwd(x, w, None, desc)
+    assert y.flatten().tolist() == [float(v) for v in kat["output"]]
+
+
+# n, ci, co, h, w, kh, kw, stride, dilation, padding
+SHAPES = [
+    (2, 5, 7, 9, 11, 1, 1, 1, 1, "VALID"),
+    (2, 6, 4, 10, 13, 3, 3, 1, 1, "SAME"),
+    (1, 3, 8, 15, 14, 3, 3, 2, 1, "SAME"),
+    (3, 4, 4, 8, 9, 3, 2, (1, 2), (2, 1), (2, 0, 1, 3)),
+]
+
+
+@pytest.mark.parametrize("dtype,policy", [(torch.float32, "fp32"), (torch.float16, "full16")], ids=["f32", "f16"])
+@pytest.mark.parametrize("mode", [8, 16])
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "k%dx%d_%dx%d" % (s[5], s[6], s[3], s[4]))
+@pytest.mark.parametrize("algebra", [phx.REAL, phx.COMPLEX, phx.GA_300], ids=["real", "complex", "ga300"])
+def test_conv_against_the_sign_tables(algebra, shape, mode, dtype, policy):
+    n, ci, co, h, w, kh, kw, stride, dilation, padding = shape
+    d = algebras.DIMS[algebra]
+    r = np.random.default_rng(100 * algebra + kh * kw + h)
+    npdt = np.float32 if dtype == torch.float32 else np.float16
+    scale = 1.0 if dtype == torch.float32 else 0.5
+    g = oracle.make_geom(n, ci, co, h, w, kh, kw, stride, dilation, padding)
+    x = (scale * r.standard_normal((d * n, ci, h, w))).astype(npdt)
+    wt = (scale * r.standard_normal((d, co, ci, kh, kw)) * np.sqrt(2.0 / (ci * kh * kw))).astype(npdt)
+    b = (scale * r.standard_normal((d, co))).astype(npdt)
+    gr = (scale * r.standard_normal((d * n, co, g.ho, g.wo))).astype(npdt)
+    real = algebra == phx.REAL  # a real filter / bias has no blade axis
+    w_dev, b_dev = (wt[0], b[0]) if real else (wt, b)
+    desc = phx.Conv2DDescriptor(x.shape, w_dev.shape, stride, dilation, padding, algebra=algebra, use_bias=True,
+                                dtype=dtype, context=Ctx(mode, policy))
+    assert desc.output_shape == gr.shape
+    xd, wd, bd, gd = (torch.from_numpy(np.ascontiguousarray(a)).cuda() for a in (x, w_dev, b_dev, gr))
+    y = phx.conv2d_fwd(xd, wd, bd, desc)
+    dw, dx = phx.conv2d_bwd(xd, wd, gd, desc)
+    x64, w64, b64, g64 = (a.astype(np.float64) for a in (x, wt, b, gr))
+    want_y = oracle.conv2d_fwd(g, x64, w64, b64, "generic", algebra=algebra)
+    want_dw, want_dx = oracle.conv2d_bwd(g, x64, w64, g64, "generic", algebra=algebra)
+    close(y.cpu().numpy(), want_y, dtype, "fwd")
+    close(dx.cpu().numpy(), want_dx, dtype, "dgrad")
+    got_dw = dw.cpu().numpy()
+    close(got_dw[None] if real else got_dw, want_dw, dtype, "wgrad")
+
+
+@pytest.mark.parametrize("dtype,policy", [(torch.float32, "fp32"), (torch.float16, "full16")], ids=["f32", "f16"])
+@pytest.mark.parametrize("algebra", [phx.REAL, phx.COMPLEX, phx.GA_300], ids=["real", "complex", "ga300"])
+def test_dense_against_the_sign_tables(algebra, dtype, policy):
+    d = algebras.DIMS[algebra]
+    r = np.random.default_rng(200 + algebra)
+    n, ni, no = 7, 33, 20
+    npdt = np.float32 if dtype == torch.float32 else np.float16
+    scale = 1.0 if dtype == torch.float32 else 0.5
+    x = (scale * r.standard_normal((d * n, ni))).astype(npdt)
+    wt = (r.uniform(-1, 1, (d, ni, no)) * np.sqrt(6.0 / (ni + no))).astype(npdt)
+    b = (scale * r.standard_normal((d, no))).astype(npdt)
+    gr = (scale * r.standard_normal((d * n, no))).astype(npdt)
+    real = algebra == phx.REAL
+    w_dev, b_dev = (wt[0], b[0]) if real else (wt, b)
+    desc = phx.DenseDescriptor(x.shape, w_dev.shape, algebra=algebra, use_bias=True, dtype=dtype, context=Ctx(8, policy))
+    xd, wd, bd, gd = (torch.from_numpy(np.ascontiguousarray(a)).cuda() for a in (x, w_dev, b_dev, gr))
+    y = phx.dense_fwd(xd, wd, bd, desc)
+    dw, dx = phx.dense_bwd(xd, wd, gd, desc)
+    x64, w64, b64, g64 = (a.astype(np.float64) for a in (x, wt, b, gr))
+    want_y = oracle.dense_fwd(x64, w64, b64, "generic", algebra=algebra)
+    want_dw, want_dx = oracle.dense_bwd(x64, w64, g64, "generic", algebra=algebra)
+    close(y.cpu().numpy(), want_y, dtype, "dense fwd")
+    close(dx.cpu().numpy(), want_dx, dtype, "dense dgrad")
+    got_dw = dw.cpu().numpy()
+    close(got_dw[None] if real else got_dw, want_dw, dtype, "dense wgrad")
