@@ -47,6 +47,16 @@ enum phx_dense_layout { PHX_IO = 0, PHX_OI = 1 };
  * transposes its activations into the workspace on the way in and out (two extra passes over each tensor). */
 enum phx_data_format { PHX_NCHW = 0, PHX_NHWC = 1 };
 
+/* Algebra of the tensors (Algebra, src/algebras.hpp:17-22; zero is the quaternions here, so that a descriptor filled
+ * without this field means what it always meant).  The quaternion algebra runs on the kernels directly.  REAL,
+ * COMPLEX and GA_300 run as one quaternion call on rearranged tensors: a GA_300 multivector (blades 1, e1, e2, e3,
+ * e12, e13, e23, e123; src/algebras.cc:58-131) is A + e123 B with quaternion-like A = (m0, m4, m5, -m6) and
+ * B = (m7, -m3, m2, m1), and (A1 + I B1)(A2 + I B2) = (A1 A2 - B1 B2) + I (A1 B2 + B1 A2), i.e. one quaternion
+ * convolution of twice the channel counts; COMPLEX and REAL are embedded with zero components.  For these
+ * algebras activations have dims * n batch rows (dims = 1, 2, 8), filters are [dims, co, ci, kh, kw] (Dense:
+ * [dims, ni, no]), bias [dims, co]; NCHW, OIHW / IO, no groups, no real-valued input. */
+enum phx_algebra { PHX_QUATERNION = 0, PHX_REAL = 1, PHX_COMPLEX = 2, PHX_GA_300 = 3 };
+
 /* Which Hamilton-product formulation runs.
  * Mirrors Context::preferSpeedToMemory() (src/backend/backend.hpp:58): the reference's default is
  * the factorized 8-product path (src/conv2d.hpp:167-234), UPSTRIDE_MEMORY_OPTIMIZED=1 selects the
@@ -92,6 +102,7 @@ typedef struct phx_qconv_desc {
                               co]); 0 or 1 = ungrouped */
     int32_t data_format;   /* phx_data_format of x, y and their gradients: PHX_NCHW [4n, c, h, w] or PHX_NHWC
                               [4n, h, w, c]; filters and bias are unaffected (filter_layout is separate) */
+    int32_t algebra;       /* phx_algebra */
 } phx_qconv_desc;
 
 /* Quaternion Dense geometry (src/backend/dense_descriptor.hpp:11-59). */
@@ -103,9 +114,16 @@ typedef struct phx_qdense_desc {
     int32_t fp16_policy;
     int32_t has_bias;
     int32_t filter_layout; /* phx_dense_layout */
+    int32_t algebra;       /* phx_algebra */
 } phx_qdense_desc;
 
 const char* phx_status_string(int status);
+
+/* The rearrangement that carries an algebra onto the quaternion kernels: `dims` blades, `halves` quaternion-like
+ * parts; quaternion component p of half h is sign[h * 4 + p] * blade[h * 4 + p] (blade -1: the component is zero).
+ * Host-only (no GPU work): lets a caller, or a test, check the map against the algebra's sign table
+ * (src/algebras.cc:5-145). */
+int phx_algebra_map(int algebra, int32_t* dims, int32_t* halves, int32_t blade[8], int32_t sign[8]);
 
 /* Output spatial size for the descriptor's explicit padding (src/utils.cc:42-51). */
 int phx_qconv2d_output_hw(const phx_qconv_desc* desc, int32_t* ho, int32_t* wo);

@@ -13,6 +13,7 @@ PHX_ERR_INVALID_ARGUMENT, PHX_ERR_NOT_SUPPORTED, PHX_ERR_WORKSPACE, PHX_ERR_RUNT
 PHX_F32, PHX_F16 = 0, 1
 PHX_OIHW, PHX_OHWI, PHX_HWIO = 0, 1, 2
 PHX_IO, PHX_OI = 0, 1
+PHX_QUATERNION, PHX_REAL, PHX_COMPLEX, PHX_GA_300 = 0, 1, 2, 3
 PHX_NCHW, PHX_NHWC = 0, 1
 PHX_PRODUCT_16, PHX_PRODUCT_8 = 16, 8
 PHX_FP16_FULL32, PHX_FP16_BACKWARD32, PHX_FP16_FULL16 = 0, 1, 2
@@ -25,7 +26,7 @@ EXPORTS = (
     "phx_qdense_fwd", "phx_qdense_bwd_data", "phx_qdense_bwd_weights",
     "phx_device_count", "phx_device_malloc", "phx_device_free", "phx_memcpy_h2d", "phx_memcpy_d2h",
     "phx_memset_zero", "phx_stream_create", "phx_stream_destroy", "phx_stream_synchronize",
-    "phx_last_kernel_name", "phx_profile_enable", "phx_profile_collect",
+    "phx_last_kernel_name", "phx_profile_enable", "phx_profile_collect", "phx_algebra_map",
 )
 
 
@@ -42,12 +43,12 @@ class QConvDesc(ctypes.Structure):
     _fields_ = [(k, ctypes.c_int32) for k in (
         "dtype", "n", "ci", "co", "h", "w", "kh", "kw", "stride_h", "stride_w", "dilation_h", "dilation_w",
         "pad_top", "pad_left", "pad_bottom", "pad_right", "filter_layout", "product_mode", "fp16_policy", "has_bias",
-        "real_input", "groups", "data_format")]
+        "real_input", "groups", "data_format", "algebra")]
 
 
 class QDenseDesc(ctypes.Structure):
     _fields_ = [(k, ctypes.c_int32) for k in ("dtype", "n", "ni", "no", "product_mode", "fp16_policy", "has_bias",
-                                               "filter_layout")]
+                                               "filter_layout", "algebra")]
 
 
 class PhxError(RuntimeError):
@@ -96,6 +97,7 @@ def lib():
         L.phx_stream_create.argtypes = [ctypes.POINTER(vp)]
         L.phx_stream_destroy.argtypes = [vp]
         L.phx_stream_synchronize.argtypes = [vp]
+        L.phx_algebra_map.argtypes = [ctypes.c_int, i32p, i32p, i32p, i32p]
         L.phx_profile_enable.argtypes = [ctypes.c_int]
         L.phx_profile_collect.argtypes = [ctypes.POINTER(ctypes.c_float), ctypes.c_int, i32p]
         _lib = L

@@ -1,0 +1,343 @@
+// Conv2D and Dense of the reference's other algebras -- REAL, COMPLEX, GA_300 (src/algebras.hpp:17-22, sign
+// tables src/algebras.cc:5-145) -- as compositions on the quaternion entry points.
+//
+// GA_300 has the blades 1, e1, e2, e3, e12, e13, e23, e123 (src/algebras.cc:58-131).  Its even part
+// {1, e12, e13, -e23} multiplies like the quaternion units {1, i, j, k}; the pseudoscalar I = e123 commutes with
+// every blade and squares to -1.  Every multivector is therefore M = A + I B with quaternion-like
+// A = (m0, m4, m5, -m6), B = (m7, -m3, m2, m1), and
+//     (A1 + I B1)(A2 + I B2) = (A1 A2 - B1 B2) + I (A1 B2 + B1 A2),
+// i.e. a GA_300 convolution of Ci -> Co channels is one quaternion convolution of 2 Ci -> 2 Co channels on the
+// activations [A | B] with the filter blocks [[A2, B2], [-B2, A2]] (input half x output half): 64 real products
+// per multivector product, as many as the algebra's own table holds.  COMPLEX and REAL are the sub-algebras
+// {1, i} and {1} of the quaternions; their tensors are embedded with zero components (correct, but the full
+// quaternion arithmetic runs: 4x / 16x the products these algebras need).
+//
+// The kernels here only rearrange (signed blade permutation, channel concatenation) into workspace buffers
+// around one call of the quaternion path; the backward passes use the transposes of the same maps.
+#include <algorithm>
+
+#include "../../include/phx_qconv.h"
+#include "phx_device.h"
+
+namespace phx {
+
+// quaternion component p of half h is sign * blade (blade < 0: zero)
+struct BladeMap {
+    int dims, halves;
+    int blade[8], sign[8];  // [h * 4 + p]
+    int slot[8];            // inverse: blade b sits in slot h * 4 + p
+};
+
+static bool blade_map(int algebra, BladeMap& m) {
+    auto fill = [&](int dims, int halves, const int (&blade)[8], const int (&sign)[8]) {
+        m.dims = dims; m.halves = halves;
+        for (int s = 0; s < 8; ++s) { m.blade[s] = blade[s]; m.sign[s] = sign[s]; m.slot[s] = -1; }
+        for (int s = 0; s < 4 * halves; ++s)
+            if (blade[s] >= 0) m.slot[blade[s]] = s;
+    };
+    switch (algebra) {
+        case PHX_REAL: fill(1, 1, {0, -1, -1, -1, -1, -1, -1, -1}, {1, 0, 0, 0, 0, 0, 0, 0}); return true;
+        case PHX_COMPLEX: fill(2, 1, {0, 1, -1, -1, -1, -1, -1, -1}, {1, 1, 0, 0, 0, 0, 0, 0}); return true;
+        case PHX_GA_300: fill(8, 2, {0, 4, 5, 6, 7, 3, 2, 1}, {1, 1, 1, -1, 1, -1, 1, 1}); return true;
+        default: return false;
+    }
+}
+
+struct BladeArgs {
+    const void* src;
+    void* dst;
+    BladeMap m;
+    long n;   // images (bias: 1)
+    int C;    // channels of the algebra's tensor
+    long hw;  // positions per plane
+};
+
+// algebra tensor [dims][n][C][hw] -> quaternion tensor [4][n][halves * C][hw]
+template <typename TS>
+__global__ void __launch_bounds__(WG_THREADS) blade_gather_kernel(const BladeArgs A) {
+    const TS* src = static_cast<const TS*>(A.src);
+    TS* dst = static_cast<TS*>(A.dst);
+    const long HC = (long)A.m.halves * A.C;
+    const long total = 4 * A.n * HC * A.hw;
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
+        const long pos = idx % A.hw;
+        long r = idx / A.hw;
+        const int hc = (int)(r % HC);
+        r /= HC;
+        const long nn = r % A.n;
+        const int p = (int)(r / A.n);
+        const int h = hc / A.C, c = hc - h * A.C;
+        const int b = A.m.blade[h * 4 + p];
+        float v = 0.f;
+        if (b >= 0) v = (float)A.m.sign[h * 4 + p] * (float)src[(((long)b * A.n + nn) * A.C + c) * A.hw + pos];
+        dst[idx] = (TS)v;
+    }
+}
+
+// quaternion tensor [4][n][halves * C][hw] -> algebra tensor [dims][n][C][hw]
+template <typename TS>
+__global__ void __launch_bounds__(WG_THREADS) blade_scatter_kernel(const BladeArgs A) {
+    const TS* src = static_cast<const TS*>(A.src);
+    TS* dst = static_cast<TS*>(A.dst);
+    const long HC = (long)A.m.halves * A.C;
+    const long total = (long)A.m.dims * A.n * A.C * A.hw;
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
+        const long pos = idx % A.hw;
+        long r = idx / A.hw;
+        const int c = (int)(r % A.C);
+        r /= A.C;
+        const long nn = r % A.n;
+        const int b = (int)(r / A.n);
+        const int s = A.m.slot[b], h = s >> 2, p = s & 3;
+        const float v = (float)src[(((long)p * A.n + nn) * HC + h * A.C + c) * A.hw + pos];
+        dst[idx] = (TS)((float)A.m.sign[s] * v);
+    }
+}
+
+struct BladeFilterArgs {
+    const void* w;   // algebra filter (forward: read; fold: written)
+    void* q;         // quaternion filter with halves * Co x halves * Ci channels
+    BladeMap m;
+    int Co, Ci, taps;
+    long wcs, so, si;     // algebra filter: elements between blades, output channels, input channels (taps contiguous)
+    long qcs, qso, qsi;   // the same for the quaternion filter
+};
+
+// filter blocks (input half x output half): [[A, B], [-B, A]]
+template <typename TS>
+__global__ void __launch_bounds__(WG_THREADS) blade_filter_build_kernel(const BladeFilterArgs A) {
+    const TS* w = static_cast<const TS*>(A.w);
+    TS* q = static_cast<TS*>(A.q);
+    const int H = A.m.halves;
+    const long HO = (long)H * A.Co, HI = (long)H * A.Ci;
+    const long total = 4 * HO * HI * A.taps;
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
+        const int tap = (int)(idx % A.taps);
+        long r = idx / A.taps;
+        const int i2 = (int)(r % HI);
+        r /= HI;
+        const int o2 = (int)(r % HO);
+        const int p = (int)(r / HO);
+        const int ho = o2 / A.Co, o = o2 - ho * A.Co, hi = i2 / A.Ci, i = i2 - hi * A.Ci;
+        const int part = (ho != hi) ? 1 : 0;
+        const float block_sign = (ho == 0 && hi == 1) ? -1.f : 1.f;
+        const int s = part * 4 + p, b = A.m.blade[s];
+        float v = 0.f;
+        if (b >= 0) v = block_sign * (float)A.m.sign[s] * (float)w[b * A.wcs + o * A.so + i * A.si + tap];
+        q[p * A.qcs + o2 * A.qso + i2 * A.qsi + tap] = (TS)v;
+    }
+}
+
+// transpose of the build: gradient of the quaternion filter -> gradient of the algebra filter
+template <typename TS>
+__global__ void __launch_bounds__(WG_THREADS) blade_filter_fold_kernel(const BladeFilterArgs A) {
+    TS* w = static_cast<TS*>(const_cast<void*>(A.w));
+    const TS* q = static_cast<const TS*>(A.q);
+    const long total = (long)A.m.dims * A.Co * A.Ci * A.taps;
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
+        const int tap = (int)(idx % A.taps);
+        long r = idx / A.taps;
+        const int i = (int)(r % A.Ci);
+        r /= A.Ci;
+        const int o = (int)(r % A.Co);
+        const int b = (int)(r / A.Co);
+        const int s = A.m.slot[b], part = s >> 2, p = s & 3;
+        auto at = [&](int ho, int hi) {
+            return (float)q[p * A.qcs + (long)(ho * A.Co + o) * A.qso + (long)(hi * A.Ci + i) * A.qsi + tap];
+        };
+        float v;
+        if (A.m.halves == 1) v = at(0, 0);
+        else if (part == 0) v = at(0, 0) + at(1, 1);
+        else v = at(1, 0) - at(0, 1);
+        w[b * A.wcs + o * A.so + i * A.si + tap] = (TS)((float)A.m.sign[s] * v);
+    }
+}
+
+static int blocks_for(long items) { return (int)std::max<long>(1, std::min<long>((items + WG_THREADS - 1) / WG_THREADS, 1 << 16)); }
+
+template <typename K32, typename K16, typename Args>
+static void launch(bool half_storage, K32 k32, K16 k16, long items, const Args& a, hipStream_t st) {
+    if (items <= 0) return;
+    if (half_storage) hipLaunchKernelGGL(k16, dim3(blocks_for(items)), dim3(WG_THREADS), 0, st, a);
+    else hipLaunchKernelGGL(k32, dim3(blocks_for(items)), dim3(WG_THREADS), 0, st, a);
+}
+
+static size_t align256(size_t b) { return (b + 255) / 256 * 256; }
+
+// Buffers of one composed call at the front of the workspace: quaternion forms of the input-side tensor, the
+// output-side tensor, the filter and the bias; the quaternion call's own workspace follows.
+struct Composition {
+    BladeMap m;
+    bool half;
+    size_t esize, x_bytes, y_bytes, w_bytes, b_bytes;
+    long n;
+    int ci, co, taps;
+    long hw_in, hw_out;
+    size_t buffers() const { return x_bytes + y_bytes + w_bytes + b_bytes; }
+    void init(int dtype, long n_, int ci_, int co_, long hw_in_, long hw_out_, int taps_) {
+        half = dtype == PHX_F16; esize = half ? 2 : 4;
+        n = n_; ci = ci_; co = co_; hw_in = hw_in_; hw_out = hw_out_; taps = taps_;
+        const size_t H = m.halves;
+        x_bytes = align256(4 * n * H * ci * hw_in * esize);
+        y_bytes = align256(4 * n * H * co * hw_out * esize);
+        w_bytes = align256(4 * H * co * H * ci * taps * esize);
+        b_bytes = align256(4 * H * co * esize);
+    }
+    void gather(const void* src, void* dst, long rows, int C, long hw, hipStream_t st) const {
+        BladeArgs a{src, dst, m, rows, C, hw};
+        launch(half, blade_gather_kernel<float>, blade_gather_kernel<_Float16>, 4 * rows * m.halves * C * hw, a, st);
+    }
+    void scatter(const void* src, void* dst, long rows, int C, long hw, hipStream_t st) const {
+        BladeArgs a{src, dst, m, rows, C, hw};
+        launch(half, blade_scatter_kernel<float>, blade_scatter_kernel<_Float16>, (long)m.dims * rows * C * hw, a, st);
+    }
+    // dense filters are [blade][in][out], convolution filters [blade][out][in][taps]
+    BladeFilterArgs filter_args(const void* w, void* q, bool dense) const {
+        BladeFilterArgs a;
+        a.w = w; a.q = q; a.m = m; a.Co = co; a.Ci = ci; a.taps = taps;
+        const long H = m.halves;
+        a.wcs = (long)co * ci * taps; a.qcs = H * co * H * ci * taps;
+        if (dense) { a.so = 1; a.si = co; a.qso = 1; a.qsi = H * co; }
+        else { a.so = (long)ci * taps; a.si = taps; a.qso = H * ci * taps; a.qsi = taps; }
+        return a;
+    }
+    void build_filter(const void* w, void* q, bool dense, hipStream_t st) const {
+        launch(half, blade_filter_build_kernel<float>, blade_filter_build_kernel<_Float16>,
+               4L * m.halves * co * m.halves * ci * taps, filter_args(w, q, dense), st);
+    }
+    void fold_filter(const void* q, void* w, bool dense, hipStream_t st) const {
+        launch(half, blade_filter_fold_kernel<float>, blade_filter_fold_kernel<_Float16>, (long)m.dims * co * ci * taps,
+               filter_args(w, const_cast<void*>(q), dense), st);
+    }
+};
+
+static int conv_composition(const phx_qconv_desc* d, Composition& c, phx_qconv_desc& inner) {
+    if (!d || !blade_map(d->algebra, c.m)) return PHX_ERR_INVALID_ARGUMENT;
+    if (d->groups > 1 || d->filter_layout != PHX_OIHW || d->data_format != PHX_NCHW || d->real_input)
+        return PHX_ERR_NOT_SUPPORTED;
+    inner = *d;
+    inner.algebra = PHX_QUATERNION;
+    inner.ci = d->ci * c.m.halves;
+    inner.co = d->co * c.m.halves;
+    int32_t ho = 0, wo = 0;
+    const int rc = phx_qconv2d_output_hw(&inner, &ho, &wo);
+    if (rc != PHX_OK) return rc;
+    c.init(d->dtype, d->n, d->ci, d->co, (long)d->h * d->w, (long)ho * wo, d->kh * d->kw);
+    return PHX_OK;
+}
+
+static int dense_composition(const phx_qdense_desc* d, Composition& c, phx_qdense_desc& inner) {
+    if (!d || !blade_map(d->algebra, c.m)) return PHX_ERR_INVALID_ARGUMENT;
+    if (d->filter_layout != PHX_IO) return PHX_ERR_NOT_SUPPORTED;
+    if (d->n < 0 || d->ni <= 0 || d->no <= 0 || (d->dtype != PHX_F32 && d->dtype != PHX_F16)) return PHX_ERR_INVALID_ARGUMENT;
+    inner = *d;
+    inner.algebra = PHX_QUATERNION;
+    inner.ni = d->ni * c.m.halves;
+    inner.no = d->no * c.m.halves;
+    c.init(d->dtype, d->n, d->ni, d->no, 1, 1, 1);
+    return PHX_OK;
+}
+
+// One composed pass.  `pass` picks which tensors are rearranged in and out; `run` is the quaternion call on the
+// buffers (x, y, w, bias, inner workspace).
+template <typename Run>
+static int composed_pass(const Composition& c, int pass, bool dense, hipStream_t st, const void* a, const void* b,
+                         const void* bias, void* out, void* ws, size_t ws_bytes, Run run) {
+    if (ws_bytes < c.buffers() || !ws) return PHX_ERR_WORKSPACE;
+    char* base = static_cast<char*>(ws);
+    void* xq = base;
+    void* yq = base + c.x_bytes;
+    void* wq = base + c.x_bytes + c.y_bytes;
+    void* bq = base + c.x_bytes + c.y_bytes + c.w_bytes;
+    void* inner_ws = base + c.buffers();
+    const size_t inner_bytes = ws_bytes - c.buffers();
+    int rc;
+    if (pass == PHX_PASS_FWD) {  // a = x, b = w
+        c.gather(a, xq, c.n, c.ci, c.hw_in, st);
+        c.build_filter(b, wq, dense, st);
+        if (bias) c.gather(bias, bq, 1, c.co, 1, st);
+        rc = run(xq, wq, bias ? bq : nullptr, yq, inner_ws, inner_bytes);
+        if (rc == PHX_OK) c.scatter(yq, out, c.n, c.co, c.hw_out, st);
+    } else if (pass == PHX_PASS_BWD_DATA) {  // a = grad, b = w
+        c.gather(a, yq, c.n, c.co, c.hw_out, st);
+        c.build_filter(b, wq, dense, st);
+        rc = run(yq, wq, nullptr, xq, inner_ws, inner_bytes);
+        if (rc == PHX_OK) c.scatter(xq, out, c.n, c.ci, c.hw_in, st);
+    } else {  // a = x, b = grad
+        c.gather(a, xq, c.n, c.ci, c.hw_in, st);
+        c.gather(b, yq, c.n, c.co, c.hw_out, st);
+        rc = run(xq, yq, nullptr, wq, inner_ws, inner_bytes);
+        if (rc == PHX_OK) c.fold_filter(wq, out, dense, st);
+    }
+    if (rc != PHX_OK) return rc;
+    return hipGetLastError() == hipSuccess ? PHX_OK : PHX_ERR_RUNTIME;
+}
+
+size_t algebra_conv_workspace_bytes(const phx_qconv_desc* d, int pass) {
+    Composition c;
+    phx_qconv_desc inner;
+    if (conv_composition(d, c, inner) != PHX_OK) return 0;
+    return c.buffers() + phx_qconv2d_workspace_bytes(&inner, pass);
+}
+
+size_t algebra_dense_workspace_bytes(const phx_qdense_desc* d, int pass) {
+    Composition c;
+    phx_qdense_desc inner;
+    if (dense_composition(d, c, inner) != PHX_OK) return 0;
+    return c.buffers() + phx_qdense_workspace_bytes(&inner, pass);
+}
+
+int algebra_conv_pass(const phx_qconv_desc* d, int pass, phx_stream_t stream, const void* a, const void* b, const void* bias,
+                      void* out, void* ws, size_t ws_bytes) {
+    Composition c;
+    phx_qconv_desc inner;
+    const int rc = conv_composition(d, c, inner);
+    if (rc != PHX_OK) return rc;
+    if (pass == PHX_PASS_FWD && d->has_bias && !bias) return PHX_ERR_INVALID_ARGUMENT;
+    if (pass != PHX_PASS_FWD || !d->has_bias) bias = nullptr;
+    return composed_pass(c, pass, false, static_cast<hipStream_t>(stream), a, b, bias, out, ws, ws_bytes,
+                         [&](const void* p0, const void* p1, const void* pb, void* po, void* iw, size_t ib) {
+                             if (pass == PHX_PASS_FWD) return phx_qconv2d_fwd(&inner, stream, p0, p1, pb, po, iw, ib);
+                             if (pass == PHX_PASS_BWD_DATA) return phx_qconv2d_bwd_data(&inner, stream, p0, p1, po, iw, ib);
+                             return phx_qconv2d_bwd_weights(&inner, stream, p0, p1, po, iw, ib);
+                         });
+}
+
+int algebra_dense_pass(const phx_qdense_desc* d, int pass, phx_stream_t stream, const void* a, const void* b, const void* bias,
+                       void* out, void* ws, size_t ws_bytes) {
+    Composition c;
+    phx_qdense_desc inner;
+    const int rc = dense_composition(d, c, inner);
+    if (rc != PHX_OK) return rc;
+    if (pass == PHX_PASS_FWD && d->has_bias && !bias) return PHX_ERR_INVALID_ARGUMENT;
+    if (pass != PHX_PASS_FWD || !d->has_bias) bias = nullptr;
+    return composed_pass(c, pass, true, static_cast<hipStream_t>(stream), a, b, bias, out, ws, ws_bytes,
+                         [&](const void* p0, const void* p1, const void* pb, void* po, void* iw, size_t ib) {
+                             if (pass == PHX_PASS_FWD) return phx_qdense_fwd(&inner, stream, p0, p1, pb, po, iw, ib);
+                             if (pass == PHX_PASS_BWD_DATA) return phx_qdense_bwd_data(&inner, stream, p0, p1, po, iw, ib);
+                             return phx_qdense_bwd_weights(&inner, stream, p0, p1, po, iw, ib);
+                         });
+}
+
+}  // namespace phx
+
+extern "C" int phx_algebra_map(int algebra, int32_t* dims, int32_t* halves, int32_t* blade, int32_t* sign) {
+    phx::BladeMap m;
+    if (algebra == PHX_QUATERNION) {
+        if (dims) *dims = 4;
+        if (halves) *halves = 1;
+        for (int s = 0; s < 8; ++s) {
+            if (blade) blade[s] = s < 4 ? s : -1;
+            if (sign) sign[s] = s < 4 ? 1 : 0;
+        }
+        return PHX_OK;
+    }
+    if (!phx::blade_map(algebra, m)) return PHX_ERR_INVALID_ARGUMENT;
+    if (dims) *dims = m.dims;
+    if (halves) *halves = m.halves;
+    for (int s = 0; s < 8; ++s) {
+        if (blade) blade[s] = m.blade[s];
+        if (sign) sign[s] = m.sign[s];
+    }
+    return PHX_OK;
+}

@@ -2,6 +2,7 @@
 // instantiate the kernel templates (split so that they compile in parallel).
 #pragma once
 
+#include "../../include/phx_qconv.h"
 #include "phx_kernels_f32.h"
 #include "phx_kernels_s2d.h"
 
@@ -46,5 +47,14 @@ int launch_phase_merge(bool half_storage, const PhaseMergeArgs& a, hipStream_t s
 // batched matrix transposes between channels-last tensors and the kernels' channels-first layout
 int launch_transpose(bool half_storage, const TransposeArgs& a, hipStream_t st);
 int launch_fill_zero(void* dst, size_t bytes, hipStream_t st);  // a kernel, so that it can be captured in a graph
+
+// REAL / COMPLEX / GA_300 as compositions on the quaternion entry points (phx_algebra.hip); pass = phx_pass,
+// (a, b) = (x, w) forward, (grad, w) input gradient, (x, grad) filter gradient
+size_t algebra_conv_workspace_bytes(const phx_qconv_desc* d, int pass);
+size_t algebra_dense_workspace_bytes(const phx_qdense_desc* d, int pass);
+int algebra_conv_pass(const phx_qconv_desc* d, int pass, phx_stream_t stream, const void* a, const void* b,
+                      const void* bias, void* out, void* ws, size_t ws_bytes);
+int algebra_dense_pass(const phx_qdense_desc* d, int pass, phx_stream_t stream, const void* a, const void* b,
+                       const void* bias, void* out, void* ws, size_t ws_bytes);
 
 }  // namespace phx

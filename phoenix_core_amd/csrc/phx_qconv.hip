@@ -90,6 +90,7 @@ static int problem_from_conv(const phx_qconv_desc* d, Problem& p) {
     // "Bias addition is not supported for type0 inputs" (src/conv2d.hpp:125-127)
     if (d->real_input && d->has_bias) return PHX_ERR_INVALID_ARGUMENT;
     if (d->data_format != PHX_NCHW && d->data_format != PHX_NHWC) return PHX_ERR_INVALID_ARGUMENT;
+    if (d->algebra < PHX_QUATERNION || d->algebra > PHX_GA_300) return PHX_ERR_INVALID_ARGUMENT;
     const int groups = d->groups > 1 ? d->groups : 1;
     if (d->ci % groups || d->co % groups) return PHX_ERR_INVALID_ARGUMENT;
     p.dtype = d->dtype;
@@ -124,6 +125,7 @@ static int problem_from_dense(const phx_qdense_desc* d, Problem& p) {
     if (d->fp16_policy < PHX_FP16_FULL32 || d->fp16_policy > PHX_FP16_FULL16) return PHX_ERR_INVALID_ARGUMENT;
     if (d->n < 0 || d->ni <= 0 || d->no <= 0) return PHX_ERR_INVALID_ARGUMENT;
     if (d->filter_layout != PHX_IO && d->filter_layout != PHX_OI) return PHX_ERR_INVALID_ARGUMENT;
+    if (d->algebra != PHX_QUATERNION) return PHX_ERR_INVALID_ARGUMENT;
     p.dtype = d->dtype; p.mode = d->product_mode; p.policy = d->fp16_policy;
     p.n = d->n; p.ci = d->ni; p.co = d->no; p.h = p.w = 1; p.kh = p.kw = 1;
     p.sh = p.sw = p.dh = p.dw = 1; p.pt = p.pl = p.pb = p.pr = 0; p.ho = p.wo = 1;
@@ -941,12 +943,14 @@ int phx_qconv2d_output_hw(const phx_qconv_desc* desc, int32_t* ho, int32_t* wo) 
 }
 
 size_t phx_qconv2d_workspace_bytes(const phx_qconv_desc* desc, int pass) {
+    if (desc && desc->algebra != PHX_QUATERNION) return algebra_conv_workspace_bytes(desc, pass);
     Problem p;
     if (problem_from_conv(desc, p) != PHX_OK) return 0;
     return ChannelsLast(p).bytes() + workspace_for(p, pass);
 }
 
 size_t phx_qdense_workspace_bytes(const phx_qdense_desc* desc, int pass) {
+    if (desc && desc->algebra != PHX_QUATERNION) return algebra_dense_workspace_bytes(desc, pass);
     Problem p;
     if (problem_from_dense(desc, p) != PHX_OK) return 0;
     return workspace_for(p, pass);
@@ -954,6 +958,8 @@ size_t phx_qdense_workspace_bytes(const phx_qdense_desc* desc, int pass) {
 
 int phx_qconv2d_fwd(const phx_qconv_desc* desc, phx_stream_t stream, const void* x, const void* w,
                     const void* bias_or_null, void* y, void* workspace, size_t workspace_bytes) {
+    if (desc && desc->algebra != PHX_QUATERNION)
+        return algebra_conv_pass(desc, PHX_PASS_FWD, stream, x, w, bias_or_null, y, workspace, workspace_bytes);
     Problem p;
     const int rc = problem_from_conv(desc, p);
     if (rc != PHX_OK) return rc;
@@ -980,6 +986,8 @@ int phx_qconv2d_fwd(const phx_qconv_desc* desc, phx_stream_t stream, const void*
 
 int phx_qconv2d_bwd_data(const phx_qconv_desc* desc, phx_stream_t stream, const void* grad, const void* w, void* dx,
                          void* workspace, size_t workspace_bytes) {
+    if (desc && desc->algebra != PHX_QUATERNION)
+        return algebra_conv_pass(desc, PHX_PASS_BWD_DATA, stream, grad, w, nullptr, dx, workspace, workspace_bytes);
     Problem p;
     const int rc = problem_from_conv(desc, p);
     if (rc != PHX_OK) return rc;
@@ -1008,6 +1016,8 @@ int phx_qconv2d_bwd_data(const phx_qconv_desc* desc, phx_stream_t stream, const 
 
 int phx_qconv2d_bwd_weights(const phx_qconv_desc* desc, phx_stream_t stream, const void* x, const void* grad, void* dw,
                             void* workspace, size_t workspace_bytes) {
+    if (desc && desc->algebra != PHX_QUATERNION)
+        return algebra_conv_pass(desc, PHX_PASS_BWD_WEIGHTS, stream, x, grad, nullptr, dw, workspace, workspace_bytes);
     Problem p;
     const int rc = problem_from_conv(desc, p);
     if (rc != PHX_OK) return rc;
@@ -1032,6 +1042,8 @@ int phx_qconv2d_bwd_weights(const phx_qconv_desc* desc, phx_stream_t stream, con
 
 int phx_qdense_fwd(const phx_qdense_desc* desc, phx_stream_t stream, const void* x, const void* w,
                    const void* bias_or_null, void* y, void* workspace, size_t workspace_bytes) {
+    if (desc && desc->algebra != PHX_QUATERNION)
+        return algebra_dense_pass(desc, PHX_PASS_FWD, stream, x, w, bias_or_null, y, workspace, workspace_bytes);
     Problem p;
     const int rc = problem_from_dense(desc, p);
     if (rc != PHX_OK) return rc;
@@ -1040,6 +1052,8 @@ int phx_qdense_fwd(const phx_qdense_desc* desc, phx_stream_t stream, const void*
 
 int phx_qdense_bwd_data(const phx_qdense_desc* desc, phx_stream_t stream, const void* grad, const void* w, void* dx,
                         void* workspace, size_t workspace_bytes) {
+    if (desc && desc->algebra != PHX_QUATERNION)
+        return algebra_dense_pass(desc, PHX_PASS_BWD_DATA, stream, grad, w, nullptr, dx, workspace, workspace_bytes);
     Problem p;
     const int rc = problem_from_dense(desc, p);
     if (rc != PHX_OK) return rc;
@@ -1048,6 +1062,8 @@ int phx_qdense_bwd_data(const phx_qdense_desc* desc, phx_stream_t stream, const 
 
 int phx_qdense_bwd_weights(const phx_qdense_desc* desc, phx_stream_t stream, const void* x, const void* grad, void* dw,
                            void* workspace, size_t workspace_bytes) {
+    if (desc && desc->algebra != PHX_QUATERNION)
+        return algebra_dense_pass(desc, PHX_PASS_BWD_WEIGHTS, stream, x, grad, nullptr, dw, workspace, workspace_bytes);
     Problem p;
     const int rc = problem_from_dense(desc, p);
     if (rc != PHX_OK) return rc;

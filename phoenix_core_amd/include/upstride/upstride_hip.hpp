@@ -704,25 +704,39 @@ class TensorSplit {
 // Operators (src/conv2d.hpp, src/dense.hpp).  The quaternion algebra runs on the fused HIP
 // kernels -- the seat the reference gives its custom quaternion kernels ahead of the factorized
 // and generic branches (src/conv2d.hpp:117-119, 380-382) -- with UPSTRIDE_MEMORY_OPTIMIZED
-// choosing the 8- or 16-product formulation inside them.  Other algebras are not built here.
+// choosing the 8- or 16-product formulation inside them.  The other algebras run inside the library
+// as one quaternion call on rearranged tensors (include/phx_qconv.h, phx_algebra).
 // ---------------------------------------------------------------------------------------------
 namespace detail {
 
+inline int phxAlgebra(Algebra a) {
+    switch (a) {
+        case Algebra::REAL: return PHX_REAL;
+        case Algebra::COMPLEX: return PHX_COMPLEX;
+        case Algebra::QUATERNION: return PHX_QUATERNION;
+        case Algebra::GA_300: return PHX_GA_300;
+    }
+    throw std::invalid_argument("Unknown algebra");
+}
+
 inline phx_qconv_desc makeConvDesc(const Conv2DDescriptor& d, Context& ctx, int dtype, bool useBias) {
-    if (d.getAlgebra() != Algebra::QUATERNION)
-        throw std::runtime_error("Only the quaternion algebra is built for device::HIP");
+    // the quaternion algebra runs on the kernels directly, the others as one quaternion call on rearranged
+    // tensors inside the library (NCHW, OIHW, no groups, no real-valued input: it reports anything else)
+    const Algebra algebra = d.getAlgebra();
+    const int dims = MULTIVECTOR_DIM[algebra];
     const DataFormat df = d.getDataFormat();
     if (df != DataFormat::NCHW && df != DataFormat::NHWC) throw std::runtime_error("device::HIP runs NCHW or NHWC tensors");
     const FilterLayout fl = d.getFilterLayout();
     if (fl != FilterLayout::OIHW && fl != FilterLayout::OHWI && fl != FilterLayout::HWIO)
         throw std::runtime_error("device::HIP takes OIHW, OHWI or HWIO filters");
-    Conv2DFilterLayout filter(fl, Algebra::QUATERNION);
+    Conv2DFilterLayout filter(fl, algebra);
     const Shape& in = d.getInputShape();
     const Shape& w = d.getFilterShape();
     phx_qconv_desc c;
     c.dtype = dtype;
     const bool real = d.isRealValuedInput();  // [n, ci, h, w] without imaginary components
-    c.n = real ? in[0] : in[0] / 4;
+    c.n = real ? in[0] : in[0] / dims;
+    c.algebra = phxAlgebra(algebra);
     c.groups = d.getGroups();
     c.ci = filter.numInputChannels(w) * c.groups;  // the filter holds one group's input channels
     c.co = filter.numOutputChannels(w);
@@ -740,21 +754,25 @@ inline phx_qconv_desc makeConvDesc(const Conv2DDescriptor& d, Context& ctx, int 
     c.fp16_policy = ctx.phxFp16Policy();
     c.has_bias = (useBias && !real) ? 1 : 0;  // a bias given with a real-valued input is refused at call time
     c.real_input = real ? 1 : 0;
-    if (!real && in[0] % 4 != 0) throw std::invalid_argument("Cannot split " + std::to_string(in[0]) + " onto 4 parts");
+    if (!real && in[0] % dims != 0)
+        throw std::invalid_argument("Cannot split " + std::to_string(in[0]) + " onto " + std::to_string(dims) + " parts");
     if (in.depth(df) != c.ci) throw std::invalid_argument("Input channels do not match the filter");
     return c;
 }
 
 inline phx_qdense_desc makeDenseDesc(const DenseDescriptor& d, Context& ctx, int dtype, bool useBias) {
-    if (d.getAlgebra() != Algebra::QUATERNION)
-        throw std::runtime_error("Only the quaternion algebra is built for device::HIP");
+    const Algebra algebra = d.getAlgebra();
+    const int dims = MULTIVECTOR_DIM[algebra];
     const bool io = d.getFilterLayout() == FilterLayout::IO;
     if (!io && d.getFilterLayout() != FilterLayout::OI) throw std::runtime_error("device::HIP takes dense filters in IO or OI layout");
-    const Shape in = d.getInputShape(), w = d.getFilterShape();
-    if (in.getSize() != 2 || w.getSize() != 3 || w[0] != 4 || in[0] % 4 != 0 || in[1] != w[io ? 1 : 2])
-        throw std::invalid_argument("Dense expects input [4n, in] and filter [4, in, out] (IO) or [4, out, in] (OI)");
+    const Shape in = d.getInputShape();
+    Shape w = d.getFilterShape();
+    if (algebra == Algebra::REAL && w.getSize() == 2) w = Shape{1, w[0], w[1]};  // a real filter has no blade axis
+    if (in.getSize() != 2 || w.getSize() != 3 || w[0] != dims || in[0] % dims != 0 || in[1] != w[io ? 1 : 2])
+        throw std::invalid_argument("Dense expects input [D n, in] and filter [D, in, out] (IO) or [D, out, in] (OI)");
     phx_qdense_desc c;
-    c.dtype = dtype; c.n = in[0] / 4; c.ni = w[io ? 1 : 2]; c.no = w[io ? 2 : 1];
+    c.dtype = dtype; c.n = in[0] / dims; c.ni = w[io ? 1 : 2]; c.no = w[io ? 2 : 1];
+    c.algebra = phxAlgebra(algebra);
     c.filter_layout = io ? PHX_IO : PHX_OI;
     c.product_mode = ctx.phxProductMode(); c.fp16_policy = ctx.phxFp16Policy(); c.has_bias = useBias ? 1 : 0;
     return c;

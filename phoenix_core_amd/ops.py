@@ -6,7 +6,7 @@ a Context that reads the UPSTRIDE_* switches once (src/backend/backend.cc:45-48)
 entry points conv2DFwd / conv2DBwd / denseFwd / denseBwd (src/upstride.hpp:18-86) -- on torch
 tensors, which serve only as device memory.  All arithmetic happens in the HIP library behind the
 C ABI; nothing here computes on the CPU.  The algebras other than the quaternions are carried onto
-the same kernels by tensor rearrangements (algebras.py).
+the same kernels by rearrangement kernels inside the library (csrc/phx_algebra.hip).
 """
 import ctypes
 import os
@@ -83,8 +83,8 @@ _DTYPES = {torch.float32: capi.PHX_F32, torch.float16: capi.PHX_F16}
 
 class Conv2DDescriptor:
     """Geometry of one convolution (Conv2DFwdDescriptor / Conv2DBwdDescriptor of the reference).  The quaternion
-    algebra runs on the HIP kernels directly; REAL, COMPLEX and GA_300 run as compositions on them
-    (phoenix_core_amd/algebras.py; NCHW, OIHW, no groups).  data_format "NCHW" takes activations [4n, c, h, w],
+    algebra runs on the HIP kernels directly; REAL, COMPLEX and GA_300 run inside the library as one
+    quaternion call on rearranged tensors (algebras.py resolves their shapes; NCHW, OIHW, no groups).  data_format "NCHW" takes activations [4n, c, h, w],
     "NHWC" [4n, h, w, c] (transposed inside the call: the kernels compute on channels-first planes)."""
 
     def __init__(self, input_shape, filter_shape, stride=1, dilation=1, padding="VALID", groups=1,
@@ -94,7 +94,7 @@ class Conv2DDescriptor:
             raise ValueError("Four-dimensional input tensor expected")
         self.algebra = algebra
         if algebra != QUATERNION:
-            # the other algebras run as compositions on the quaternion kernels (phoenix_core_amd/algebras.py)
+            # the other algebras: same entry points, the descriptor carries the algebra (algebras.py)
             from . import algebras
             algebras.init_conv_descriptor(self, input_shape, filter_shape, algebra, groups, filter_layout, data_format,
                                           real_valued_input, stride=stride, dilation=dilation, padding=padding,
@@ -158,8 +158,6 @@ class Conv2DDescriptor:
             int(self.real_valued_input), groups, capi.PHX_NCHW if data_format == "NCHW" else capi.PHX_NHWC)
 
     def workspace_bytes(self, which):
-        if self.algebra != QUATERNION:
-            return self.inner.workspace_bytes(which)
         return capi.lib().phx_qconv2d_workspace_bytes(ctypes.byref(self.c), which)
 
 
@@ -195,8 +193,6 @@ class DenseDescriptor:
                                  capi.PHX_IO if filter_layout == "IO" else capi.PHX_OI)
 
     def workspace_bytes(self, which):
-        if self.algebra != QUATERNION:
-            return self.inner.workspace_bytes(which)
         return capi.lib().phx_qdense_workspace_bytes(ctypes.byref(self.c), which)
 
 
@@ -251,9 +247,6 @@ def _stream():
 
 def conv2d_fwd(x, w, bias, desc, out=None):
     """conv2DFwd (src/upstride.hpp:18-33): y = x (x) w (+ bias)."""
-    if desc.algebra != QUATERNION:
-        from . import algebras
-        return algebras.conv2d_fwd(x, w, bias, desc)
     dev = _dev_check(x, w, bias)
     if tuple(x.shape) != desc.input_shape or tuple(w.shape) != desc.filter_shape or x.dtype != desc.dtype:
         raise ValueError("tensor shapes / dtype do not match the descriptor")
@@ -273,9 +266,6 @@ def conv2d_fwd(x, w, bias, desc, out=None):
 def conv2d_bwd(x, w, grad, desc):
     """conv2DBwd (src/upstride.hpp:35-51): returns (dw, dx); dx is None when the descriptor does
     not require the input gradient."""
-    if desc.algebra != QUATERNION:
-        from . import algebras
-        return algebras.conv2d_bwd(x, w, grad, desc)
     dev = _dev_check(x, w, grad)
     if tuple(x.shape) != desc.input_shape or tuple(w.shape) != desc.filter_shape or \
             tuple(grad.shape) != desc.output_shape:
@@ -299,9 +289,6 @@ def conv2d_bwd(x, w, grad, desc):
 
 def dense_fwd(x, w, bias, desc, out=None):
     """denseFwd (src/upstride.hpp:53-68)."""
-    if desc.algebra != QUATERNION:
-        from . import algebras
-        return algebras.dense_fwd(x, w, bias, desc)
     dev = _dev_check(x, w, bias)
     if tuple(x.shape) != desc.input_shape or tuple(w.shape) != desc.filter_shape or x.dtype != desc.dtype:
         raise ValueError("tensor shapes / dtype do not match the descriptor")
@@ -318,9 +305,6 @@ def dense_fwd(x, w, bias, desc, out=None):
 
 def dense_bwd(x, w, grad, desc):
     """denseBwd (src/upstride.hpp:70-86): returns (dw, dx)."""
-    if desc.algebra != QUATERNION:
-        from . import algebras
-        return algebras.dense_bwd(x, w, grad, desc)
     dev = _dev_check(x, w, grad)
     if tuple(x.shape) != desc.input_shape or tuple(w.shape) != desc.filter_shape or \
             tuple(grad.shape) != desc.output_shape:

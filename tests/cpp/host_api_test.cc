@@ -227,6 +227,54 @@ static void gpuChannelsLast(Context& context) {  // tests/tests.cpp:440-487
     CHECK(equalVectors(got, want));
 }
 
+static void gpuOtherAlgebras(Context& context) {
+    device::HIP device(context);
+    {  // tests/tests.cpp:224-290: complex 1x1 convolution, 3 -> 2 channels on a 2x2 image
+        AllocatedTensor<device::HIP, float> input(device, {2, 3, 2, 2}), kernel(device, {2, 2, 3, 1, 1}), output(device, {2, 2, 2, 2});
+        input = {0, 0, 0, 0,  -1, 0, 0, 0,  1, 2, 3, 4,    1, 1, 1, 1,  0, 0, 0, 0,  -1, -2, -3, -4};
+        kernel = {1, 1, 1,  0, 0, 2,    0, 0, 0,  -1, 0, 0};
+        Conv2DFwdDescriptor descriptor(input.getShape(), kernel.getShape(), 1, 1, Padding::VALID, {}, 1, Algebra::COMPLEX,
+                                       DataFormat::NCHW, FilterLayout::OIHW, false);
+        CHECK(descriptor.getOutputShape() == Shape({2, 2, 2, 2}));
+        conv2DFwd<device::HIP, float>(device, device, input, kernel, nullptr, output, descriptor);
+        std::vector<float> got = output;
+        CHECK(equalVectors(got, std::vector<float>{0, 2, 3, 4,  3, 5, 7, 9,    0, -1, -2, -3,  -2, -4, -6, -8}));
+    }
+    {  // tests/tests.cpp:371-423: GA(3,0,0) 1x1 convolution, 1 -> 2 channels on one pixel
+        AllocatedTensor<device::HIP, float> input(device, {8, 1, 1, 1}), kernel(device, {8, 2, 1, 1, 1}), output(device, {8, 2, 1, 1});
+        input = {1, 0, 0, 0, 2, 4, 3, 0};
+        kernel = {-1, 10,  0, 0,  0, 0,  0, 0,  -2, 0,  -4, 0,  -3, 0,  0, 0};
+        Conv2DFwdDescriptor descriptor(input.getShape(), kernel.getShape(), 1, 1, Padding::VALID, {}, 1, Algebra::GA_300,
+                                       DataFormat::NCHW, FilterLayout::OIHW, false);
+        conv2DFwd<device::HIP, float>(device, device, input, kernel, nullptr, output, descriptor);
+        std::vector<float> got = output;
+        CHECK(equalVectors(got, std::vector<float>{28, 10,  0, 0,  0, 0,  0, 0,  -4, 20,  -8, 40,  -6, 30,  0, 0}));
+        // backward through the same composition: with g = 1 on the scalar blade of output channel 0 the filter
+        // gradient of that channel is the reversed input (x -> <x w>_0 has gradient ~x: vectors and the scalar keep
+        // their sign, bivectors and the pseudoscalar change it) and the other channel's is zero
+        AllocatedTensor<device::HIP, float> g(device, {8, 2, 1, 1}), dw(device, {8, 2, 1, 1, 1}), dx(device, {8, 1, 1, 1});
+        std::vector<float> gv(16, 0.f);
+        gv[0] = 1.f;
+        g = gv;
+        Conv2DBwdDescriptor bd(input.getShape(), kernel.getShape(), 1, 1, Padding::VALID, {}, 1, Algebra::GA_300,
+                               DataFormat::NCHW, FilterLayout::OIHW, true);
+        conv2DBwd<device::HIP, float>(device, device, input, kernel, g, dw, dx, bd);
+        std::vector<float> gdw = dw;
+        CHECK(equalVectors(gdw, std::vector<float>{1, 0,  0, 0,  0, 0,  0, 0,  -2, 0,  -4, 0,  -3, 0,  0, 0}, 1e-5f));
+        std::vector<float> gdx = dx;  // likewise the reversed filter of channel 0
+        CHECK(equalVectors(gdx, std::vector<float>{-1, 0, 0, 0, 2, 4, 3, 0}, 1e-5f));
+    }
+    {  // tests/tests.cpp:605-648: GA(3,0,0) Dense, 1 -> 2 features
+        AllocatedTensor<device::HIP, float> input(device, {8, 1}), kernel(device, {8, 1, 2}), output(device, {8, 2});
+        input = {1, 0, 0, 0, 2, 4, 3, 0};
+        kernel = {-1, 10,  0, 0,  0, 0,  0, 0,  -2, 0,  -4, 0,  -3, 0,  0, 0};
+        DenseFwdDescriptor descriptor(input.getShape(), kernel.getShape(), Algebra::GA_300, FilterLayout::IO, false);
+        denseFwd<device::HIP, float>(device, device, input, kernel, nullptr, output, descriptor);
+        std::vector<float> got = output;
+        CHECK(equalVectors(got, std::vector<float>{28, 10,  0, 0,  0, 0,  0, 0,  -4, 20,  -8, 40,  -6, 30,  0, 0}));
+    }
+}
+
 static void gpuPointwiseKnownAnswer(Context& context) {
     // 2 pixels, 2 input channels, 1 output channel; y = sum_c x_c (x) w_c computed by hand:
     //   pixel 0: (1+2i)(3+k) + (j)(1-i)   = (3 + 6i - 2j + k) + (j + k)      = 3 + 6i - j + 2k
@@ -276,9 +324,9 @@ static void gpuDenseAndEmpty(Context& context) {
     conv2DBwd<device::HIP, float>(device, device, ex, ew, ey, edw, edx, ebd);
     std::vector<float> z = edw;
     CHECK(equalVectors(z, std::vector<float>(24, 0.f)));
-    // algebras that are not built raise instead of running something else
-    AllocatedTensor<device::HIP, float> cx(device, {2, 1, 1, 1}), cw(device, {2, 1, 1, 1, 1}), cy(device, {2, 1, 1, 1});
-    Conv2DFwdDescriptor cd(cx.getShape(), cw.getShape(), 1, 1, Padding::VALID, {}, 1, Algebra::COMPLEX,
+    // what the composed algebras do not cover raises instead of running something else (here: groups)
+    AllocatedTensor<device::HIP, float> cx(device, {2, 2, 1, 1}), cw(device, {2, 2, 1, 1, 1}), cy(device, {2, 2, 1, 1});
+    Conv2DFwdDescriptor cd(cx.getShape(), cw.getShape(), 1, 1, Padding::VALID, {}, 2, Algebra::COMPLEX,
                            DataFormat::NCHW, FilterLayout::OIHW, false);
     CHECK_THROWS((conv2DFwd<device::HIP, float>(device, device, cx, cw, nullptr, cy, cd)), std::runtime_error);
 }
@@ -318,6 +366,7 @@ int main(int argc, char** argv) {
             gpuQuaternionOnes(context);
             gpuQuaternionRealInput(context);
             gpuChannelsLast(context);
+            gpuOtherAlgebras(context);
             gpuPointwiseKnownAnswer(context);
             gpuDenseAndEmpty(context);
             testTensorSplit(context);

@@ -1,11 +1,11 @@
-"""The rearrangements that carry the other algebras onto the quaternion kernels (phoenix_core_amd/algebras.py),
-checked on the CPU against the reference's sign tables (through the oracle, which restates
-src/algebras.cc:5-145 and is pinned entry by entry against the reference's own object code): multiplying two
-multivectors blade by blade with the table must equal mapping both to their quaternion form, multiplying with
-the quaternion table, and mapping back.  No GPU, no kernels: tensors of shape [D] / [4, halves]."""
+"""The rearrangement that carries the other algebras onto the quaternion kernels (phx_algebra_map of the library,
+the table its rearrangement kernels use), checked on the CPU against the reference's sign tables (through the
+oracle, which restates src/algebras.cc:5-145 and is pinned entry by entry against the reference's own object
+code): multiplying two multivectors blade by blade with the algebra's table must equal mapping both to their
+quaternion-like halves, multiplying those with the quaternion table in the block form [[A, B], [-B, A]] (input half
+x output half), and mapping back.  Host-only: the library is loaded, no GPU call is made."""
 import numpy as np
 import pytest
-import torch
 
 import oracle
 from phoenix_core_amd import algebras, ops
@@ -19,12 +19,30 @@ def blade_terms(algebra):
 
 
 def table_product(algebra, a, b):
-    """Left-times-right product of two multivectors by the reference's table: entries (left, right, sign) grouped
-    by output blade."""
+    """Left-times-right product of two multivectors by the reference's table."""
     out = np.zeros(algebras.DIMS[algebra])
     for k, terms in enumerate(blade_terms(algebra)):
         for left, right, positive in terms:
             out[k] += (1.0 if positive else -1.0) * a[left] * b[right]
+    return out
+
+
+def halves_of(m, algebra):
+    """Multivector [D] -> its quaternion-like halves [halves, 4] by the library's map."""
+    dims, halves, blade, sign = algebras.blade_map(algebra)
+    assert dims == algebras.DIMS[algebra] == len(m)
+    return np.array([[sign[4 * h + p] * m[blade[4 * h + p]] if blade[4 * h + p] >= 0 else 0.0 for p in range(4)]
+                     for h in range(halves)])
+
+
+def from_halves(q, algebra):
+    dims, halves, blade, sign = algebras.blade_map(algebra)
+    out = np.full(dims, np.nan)
+    for h in range(halves):
+        for p in range(4):
+            if blade[4 * h + p] >= 0:
+                out[blade[4 * h + p]] = sign[4 * h + p] * q[h, p]
+    assert not np.isnan(out).any()  # every blade has a seat
     return out
 
 
@@ -35,31 +53,22 @@ def test_composition_equals_the_algebra(algebra):
     for _ in range(20):
         a, b = r.standard_normal(d), r.standard_normal(d)
         want = table_product(algebra, a, b)
-        # activations [D*1, C=1] and a Dense filter [D, in=1, out=1]
-        xq = algebras.to_quaternion(torch.from_numpy(a).reshape(d, 1), algebra)           # [4, halves]
-        wq = algebras.filter_to_quaternion(torch.from_numpy(b).reshape(d, 1, 1), algebra, 2, 1)  # [4, halves, halves]
-        halves = xq.shape[1]
-        yq = np.zeros((4, halves))
-        for k, terms in enumerate(blade_terms(ops.QUATERNION)):
-            for left, right, positive in terms:
-                for o in range(halves):
-                    for i in range(halves):
-                        yq[k, o] += (1.0 if positive else -1.0) * xq[left, i].item() * wq[right, i, o].item()
-        got = algebras.from_quaternion(torch.from_numpy(yq), algebra).reshape(d).numpy()
-        np.testing.assert_allclose(got, want, rtol=1e-12, atol=1e-12)
+        xa, wb = halves_of(a, algebra), halves_of(b, algebra)
+        halves = len(xa)
+        # filter blocks, input half x output half: [[A, B], [-B, A]]
+        block = (lambda i, o: wb[0]) if halves == 1 else (lambda i, o: wb[0] if i == o else (wb[1] if i == 0 else -wb[1]))
+        y = np.zeros((halves, 4))
+        for o in range(halves):
+            for i in range(halves):
+                y[o] += table_product(ops.QUATERNION, xa[i], block(i, o))
+        np.testing.assert_allclose(from_halves(y, algebra), want, rtol=1e-12, atol=1e-12)
+        # the embedded algebras stay inside their sub-algebra: components that are zero on the way in stay zero
+        _, _, blade, _ = algebras.blade_map(algebra)
+        for h in range(halves):
+            for p in range(4):
+                if blade[4 * h + p] < 0:
+                    assert abs(y[h, p]) < 1e-12
 
 
-@pytest.mark.parametrize("algebra", [ops.REAL, ops.COMPLEX, ops.GA_300])
-def test_maps_are_transposes_of_each_other(algebra):
-    """from_quaternion is the transpose of to_quaternion and filter_grad_from_quaternion the transpose of
-    filter_to_quaternion (what makes the composed backward pass the true gradient): <P a, q> = <a, P^T q>."""
-    g = torch.Generator().manual_seed(7 + algebra)
-    d, halves = algebras.DIMS[algebra], len(algebras._HALVES[algebra])
-    a = torch.randn(d * 3, 5, 2, 2, generator=g, dtype=torch.float64)
-    q = torch.randn(4 * 3, halves * 5, 2, 2, generator=g, dtype=torch.float64)
-    assert torch.allclose((algebras.to_quaternion(a, algebra) * q).sum(), (a * algebras.from_quaternion(q, algebra)).sum())
-    w = torch.randn(d, 6, 5, 3, 3, generator=g, dtype=torch.float64)
-    dq = torch.randn(4, halves * 6, halves * 5, 3, 3, generator=g, dtype=torch.float64)
-    lhs = (algebras.filter_to_quaternion(w, algebra, 1, 2) * dq).sum()
-    rhs = (w * algebras.filter_grad_from_quaternion(dq, algebra, 1, 2)).sum()
-    assert torch.allclose(lhs, rhs)
+def test_quaternion_map_is_the_identity():
+    assert algebras.blade_map(ops.QUATERNION) == (4, 1, [0, 1, 2, 3, -1, -1, -1, -1], [1, 1, 1, 1, 0, 0, 0, 0])
