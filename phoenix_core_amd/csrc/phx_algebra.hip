@@ -52,45 +52,63 @@ struct BladeArgs {
     long hw;  // positions per plane
 };
 
-// algebra tensor [dims][n][C][hw] -> quaternion tensor [4][n][halves * C][hw]
+// 16 bytes of one plane, sign applied (rows start at element alignment only, which 16-byte accesses tolerate)
 template <typename TS>
+__device__ __forceinline__ void copy_signed16(const TS* src, TS* dst, int sign) {
+    constexpr int V = 16 / sizeof(TS);
+    u32x4 raw = {0u, 0u, 0u, 0u};
+    if (src) raw = *reinterpret_cast<const __attribute__((address_space(1))) u32x4_a2*>((const __attribute__((address_space(1))) TS*)src);
+    if (sign < 0) {
+        const unsigned int flip = sizeof(TS) == 2 ? 0x80008000u : 0x80000000u;
+        raw = raw ^ u32x4{flip, flip, flip, flip};
+    }
+    (void)V;
+    *reinterpret_cast<__attribute__((address_space(1))) u32x4_a2*>((__attribute__((address_space(1))) TS*)dst) = raw;
+}
+
+// algebra tensor [dims][n][C][hw] -> quaternion tensor [4][n][halves * C][hw].  For a given blade and image the
+// C * hw elements are contiguous on both sides, so a thread moves V consecutive elements of such a block
+// (V = 16 bytes when C * hw allows, else 1).
+template <typename TS, int V>
 __global__ void __launch_bounds__(WG_THREADS) blade_gather_kernel(const BladeArgs A) {
     const TS* src = static_cast<const TS*>(A.src);
     TS* dst = static_cast<TS*>(A.dst);
-    const long HC = (long)A.m.halves * A.C;
-    const long total = 4 * A.n * HC * A.hw;
+    const long chw = (long)A.C * A.hw, per = chw / V;
+    const int H = A.m.halves;
+    const long total = 4 * A.n * H * per;
     for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
-        const long pos = idx % A.hw;
-        long r = idx / A.hw;
-        const int hc = (int)(r % HC);
-        r /= HC;
+        const long e = (idx % per) * V;
+        long r = idx / per;
+        const int h = (int)(r % H);
+        r /= H;
         const long nn = r % A.n;
         const int p = (int)(r / A.n);
-        const int h = hc / A.C, c = hc - h * A.C;
-        const int b = A.m.blade[h * 4 + p];
-        float v = 0.f;
-        if (b >= 0) v = (float)A.m.sign[h * 4 + p] * (float)src[(((long)b * A.n + nn) * A.C + c) * A.hw + pos];
-        dst[idx] = (TS)v;
+        const int b = A.m.blade[h * 4 + p], sg = A.m.sign[h * 4 + p];
+        const TS* s = b >= 0 ? src + ((long)b * A.n + nn) * chw + e : nullptr;
+        TS* d = dst + (((long)p * A.n + nn) * H + h) * chw + e;
+        if constexpr (V > 1) copy_signed16<TS>(s, d, sg);
+        else *d = s ? (TS)((float)sg * (float)*s) : (TS)0.f;
     }
 }
 
 // quaternion tensor [4][n][halves * C][hw] -> algebra tensor [dims][n][C][hw]
-template <typename TS>
+template <typename TS, int V>
 __global__ void __launch_bounds__(WG_THREADS) blade_scatter_kernel(const BladeArgs A) {
     const TS* src = static_cast<const TS*>(A.src);
     TS* dst = static_cast<TS*>(A.dst);
-    const long HC = (long)A.m.halves * A.C;
-    const long total = (long)A.m.dims * A.n * A.C * A.hw;
+    const long chw = (long)A.C * A.hw, per = chw / V;
+    const int H = A.m.halves;
+    const long total = (long)A.m.dims * A.n * per;
     for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
-        const long pos = idx % A.hw;
-        long r = idx / A.hw;
-        const int c = (int)(r % A.C);
-        r /= A.C;
+        const long e = (idx % per) * V;
+        long r = idx / per;
         const long nn = r % A.n;
         const int b = (int)(r / A.n);
-        const int s = A.m.slot[b], h = s >> 2, p = s & 3;
-        const float v = (float)src[(((long)p * A.n + nn) * HC + h * A.C + c) * A.hw + pos];
-        dst[idx] = (TS)((float)A.m.sign[s] * v);
+        const int sl = A.m.slot[b], h = sl >> 2, p = sl & 3;
+        const TS* s = src + (((long)p * A.n + nn) * H + h) * chw + e;
+        TS* d = dst + ((long)b * A.n + nn) * chw + e;
+        if constexpr (V > 1) copy_signed16<TS>(s, d, A.m.sign[sl]);
+        else *d = (TS)((float)A.m.sign[sl] * (float)*s);
     }
 }
 
@@ -185,11 +203,17 @@ struct Composition {
     }
     void gather(const void* src, void* dst, long rows, int C, long hw, hipStream_t st) const {
         BladeArgs a{src, dst, m, rows, C, hw};
-        launch(half, blade_gather_kernel<float>, blade_gather_kernel<_Float16>, 4 * rows * m.halves * C * hw, a, st);
+        const int V = half ? 8 : 4;
+        const long blocks = 4 * rows * m.halves, chw = C * hw;
+        if (chw % V == 0) launch(half, blade_gather_kernel<float, 4>, blade_gather_kernel<_Float16, 8>, blocks * (chw / V), a, st);
+        else launch(half, blade_gather_kernel<float, 1>, blade_gather_kernel<_Float16, 1>, blocks * chw, a, st);
     }
     void scatter(const void* src, void* dst, long rows, int C, long hw, hipStream_t st) const {
         BladeArgs a{src, dst, m, rows, C, hw};
-        launch(half, blade_scatter_kernel<float>, blade_scatter_kernel<_Float16>, (long)m.dims * rows * C * hw, a, st);
+        const int V = half ? 8 : 4;
+        const long blocks = (long)m.dims * rows, chw = C * hw;
+        if (chw % V == 0) launch(half, blade_scatter_kernel<float, 4>, blade_scatter_kernel<_Float16, 8>, blocks * (chw / V), a, st);
+        else launch(half, blade_scatter_kernel<float, 1>, blade_scatter_kernel<_Float16, 1>, blocks * chw, a, st);
     }
     // dense filters are [blade][in][out], convolution filters [blade][out][in][taps]
     BladeFilterArgs filter_args(const void* w, void* q, bool dense) const {
