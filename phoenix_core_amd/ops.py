@@ -207,17 +207,19 @@ def default_context():
 
 
 class _Workspace:
-    """Grow-only scratch buffer per device, shared by all operations (the reference's Device keeps
-    one workspace for all its operations, src/backend/device.hpp:75-84)."""
+    """Grow-only scratch buffer per device and stream, shared by the operations enqueued there (the reference's
+    Device keeps one workspace for all its operations, src/backend/device.hpp:75-84, and serializes them with a
+    mutex; here the stream's own order serializes them, and calls on different streams get different buffers)."""
 
     def __init__(self):
         self.buffers = {}
 
     def get(self, device, nbytes):
-        buf = self.buffers.get(device)
+        key = (device, torch.cuda.current_stream(device).cuda_stream)
+        buf = self.buffers.get(key)
         if buf is None or buf.numel() < nbytes:
             buf = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=device)
-            self.buffers[device] = buf
+            self.buffers[key] = buf
         return buf
 
 

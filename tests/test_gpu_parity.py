@@ -512,6 +512,30 @@ def test_flat_tiling(case, mode, monkeypatch):
     assert torch.equal(got["flat"][0], got["tiles"][0]) and torch.equal(got["flat"][1], got["tiles"][1])
 
 
+def test_two_streams_do_not_share_scratch():
+    """Calls enqueued on different streams may overlap on the GPU: each stream gets its own workspace from the
+    Python layer, so interleaved launches (filter packing and split-K partial sums live in the workspace) must give
+    the results of the serial run, bit for bit."""
+    torch.manual_seed(3)
+    n, c, h = 8, 64, 28
+    xs = [torch.randn(4 * n, c, h, h, device="cuda") for _ in range(2)]
+    ws = [torch.randn(4, c, c, 3, 3, device="cuda") * 0.05 for _ in range(2)]
+    gs = [torch.randn(4 * n, c, h, h, device="cuda") for _ in range(2)]
+    desc = phx.Conv2DDescriptor(xs[0].shape, ws[0].shape, 1, 1, "SAME", context=Ctx(8))
+    serial = [(phx.conv2d_fwd(x, w, None, desc),) + phx.conv2d_bwd(x, w, g, desc) for x, w, g in zip(xs, ws, gs)]
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream() for _ in range(2)]
+    results = [None, None]
+    for rep in range(4):  # several rounds of interleaved launches
+        for i, st in enumerate(streams):
+            with torch.cuda.stream(st):
+                results[i] = (phx.conv2d_fwd(xs[i], ws[i], None, desc),) + phx.conv2d_bwd(xs[i], ws[i], gs[i], desc)
+    torch.cuda.synchronize()
+    for want, got in zip(serial, results):
+        for a, b in zip(want, got):
+            assert torch.equal(a, b)
+
+
 STRIDED = [c for c in FP16_CASES if c[0] in ("k3_s2", "pw_s2", "k7_s2", "k3_s2_c4", "k5_s2_valid", "k3_s3", "k32_s21")]
 
 
