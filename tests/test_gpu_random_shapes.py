@@ -1,5 +1,5 @@
 """GPU parity on seeded random problem geometries: batch, channel counts, image and filter sizes, strides,
-dilations, padding (SAME / VALID / explicit asymmetric), filter layout, data format, bias, product mode, fp16
+dilations, padding (SAME / VALID / explicit asymmetric), filter layout, data format, groups, bias, product mode, fp16
 policy and real-valued input are all drawn at random, so that the host planner's corner cases (ragged tiles, windows
 that leave the tensor, space-to-depth stems, virtual pointwise taps, zero-inserted strided gradients) meet
 the oracle on shapes nobody picked by hand.  Tolerances as in test_gpu_parity.py."""
@@ -55,16 +55,20 @@ def draw(seed):
                bias=bool(r.random() < 0.5), real=bool(r.random() < 0.2), seed=seed)
     cfg["nhwc"] = bool(r.random() < 0.25)
     cfg["layout"] = "HWIO" if r.random() < 0.15 else ("OHWI" if cfg["ohwi"] else "OIHW")
+    # grouped convolution: the drawn channel counts become the channels of one group
+    cfg["groups"] = int(r.choice([1, 1, 1, 2, 3])) if cfg["ci"] <= 17 and cfg["co"] <= 33 else 1
     return cfg, r
 
 
 def run_case(cfg, r, dtype, policy):
-    n, ci, co, h, w, kh, kw = (cfg[k] for k in ("n", "ci", "co", "h", "w", "kh", "kw"))
-    geom = oracle.make_geom(n, ci, co, h, w, kh, kw, cfg["stride"], cfg["dilation"], cfg["padding"])
+    n, cig, cog, h, w, kh, kw = (cfg[k] for k in ("n", "ci", "co", "h", "w", "kh", "kw"))
+    G = cfg["groups"]
+    ci, co = cig * G, cog * G
+    geom = oracle.make_geom(n, cig, cog, h, w, kh, kw, cfg["stride"], cfg["dilation"], cfg["padding"])
     npdt = np.float32 if dtype == torch.float32 else np.float16
     scale = 1.0 if dtype == torch.float32 else 0.5
     x = (scale * r.standard_normal((4 * n, ci, h, w))).astype(npdt)
-    wt = (scale * r.standard_normal((4, co, ci, kh, kw)) * np.sqrt(2.0 / (ci * kh * kw))).astype(npdt)
+    wt = (scale * r.standard_normal((4, co, cig, kh, kw)) * np.sqrt(2.0 / (cig * kh * kw))).astype(npdt)
     b = (scale * r.standard_normal((4, co))).astype(npdt)
     gr = (scale * r.standard_normal((4 * n, co, geom.ho, geom.wo))).astype(npdt)
     real, bias = cfg["real"], cfg["bias"] and not cfg["real"]
@@ -81,7 +85,7 @@ def run_case(cfg, r, dtype, policy):
     ctx = Ctx(cfg["mode"], policy)
     desc = phx.Conv2DDescriptor(x_dev.shape, w_dev.shape, cfg["stride"], cfg["dilation"], cfg["padding"],
                                 filter_layout=cfg["layout"], use_bias=bias, dtype=dtype, context=ctx,
-                                real_valued_input=real, require_input_grad=not real,
+                                real_valued_input=real, require_input_grad=not real, groups=G,
                                 data_format="NHWC" if nhwc else "NCHW")
     assert desc.output_shape == ((4 * n, geom.ho, geom.wo, co) if nhwc else (4 * n, co, geom.ho, geom.wo)), cfg
     xd, wd, bd, gd = (torch.from_numpy(a).cuda() for a in (x_dev, w_dev, b, g_dev))
@@ -89,8 +93,13 @@ def run_case(cfg, r, dtype, policy):
     dw, dx = phx.conv2d_bwd(xd, wd, gd, desc)
     torch.cuda.synchronize()
     x64, w64, b64, g64 = (a.astype(np.float64) for a in (x, wt, b, gr))
-    want_y = oracle.conv2d_fwd(geom, x64, w64, b64 if bias else None, "hamilton")
-    want_dw, want_dx = oracle.conv2d_bwd(geom, x64, w64, g64, "hamilton")
+    # by definition G independent convolutions on channel slices
+    want_y, want_dx, want_dw = np.empty(gr.shape), np.empty(x.shape), np.empty(wt.shape)
+    for k in range(G):
+        ic, oc = slice(k * cig, (k + 1) * cig), slice(k * cog, (k + 1) * cog)
+        xs, ws, bs, gs = (np.ascontiguousarray(a) for a in (x64[:, ic], w64[:, oc], b64[:, oc], g64[:, oc]))
+        want_y[:, oc] = oracle.conv2d_fwd(geom, xs, ws, bs if bias else None, "hamilton")
+        want_dw[:, oc], want_dx[:, ic] = oracle.conv2d_bwd(geom, xs, ws, gs, "hamilton")
     close(from_dev(y.cpu().numpy()), want_y, dtype, "fwd %s" % cfg)
     got_dw = dw.cpu().numpy()
     close(got_dw.transpose(from_layout), want_dw, dtype, "wgrad %s" % cfg)
