@@ -13,7 +13,7 @@ import phoenix_core_amd as phx
 pytestmark = pytest.mark.gpu
 
 TOL = {torch.float32: 1e-4, torch.float16: 2e-2}
-CASES = 160
+CASES = 320
 
 
 class Ctx(phx.Context):
