@@ -124,6 +124,22 @@ def test_random_geometry_fp16(seed):
     run_case(cfg, r, torch.float16, policy)
 
 
+@pytest.mark.parametrize("seed", range(96))
+def test_random_wide(seed):
+    """Wider channels and images (64-136 channels, up to 30x30, mostly unit stride): the shapes on which the planner
+    picks flat tiling, two column tiles per wave, several channel chunks and multi-tap filter-gradient workgroups."""
+    r = np.random.default_rng(7000 + seed)
+    kh, kw = [(3, 3), (3, 3), (3, 1), (1, 3), (5, 5), (2, 2)][int(r.integers(0, 6))]
+    s = 1 if r.random() < 0.75 else 2
+    cfg = dict(n=int(r.integers(1, 4)), ci=int(r.choice([64, 80, 96, 130])), co=int(r.choice([64, 100, 128, 136])),
+               h=int(r.integers(12, 31)), w=int(r.integers(12, 31)), kh=kh, kw=kw, stride=(s, s), dilation=(1, 1),
+               padding=str(r.choice(["SAME", "VALID"])), mode=int(r.choice([8, 16])), ohwi=False, bias=bool(r.random() < 0.5),
+               real=False, seed=seed, nhwc=False, layout="OIHW", groups=1)
+    dtype, policy = [(torch.float16, "full16"), (torch.float32, "fp32"), (torch.float16, "backward32")][seed % 3]
+    print("case", cfg, dtype, policy, flush=True)
+    run_case(cfg, r, dtype, policy)
+
+
 @pytest.mark.parametrize("seed", range(48))
 def test_random_dense(seed):
     """Quaternion Dense on random batch / feature counts, both tensor types, every mode and policy, in fp64
