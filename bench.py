@@ -1,17 +1,24 @@
 #!/usr/bin/env python3
-"""Benchmark of the quaternion Conv2D hot path on one MI355X.
+"""Benchmark of the quaternion Conv2D / Dense hot path on one MI355X.
 
-A step is one pass of the hot path over one batch of synthetic input: forward, input-gradient and
-filter-gradient of one quaternion convolution, inputs resident in HBM.  The default workload is the
-pointwise fp32 configuration (N=32, 64->64 quaternion channels, 56x56); --workload selects the
-others.  Prints ONE JSON line: real-equivalent TFLOP/s (16 real multiply-adds per quaternion
-multiply-add, for either product mode), the roofline of the dominant kernel and the reference's CPU
-algorithm timed on the host cores of the same box.
+A step is one pass of the hot path over one batch of synthetic input, resident in HBM: forward,
+input gradient and filter gradient of one quaternion operator (or one forward+backward of the
+quaternion ResNet-50).  The default run prints ONE JSON line whose headline (`value`, `roofline`,
+`cpu_baseline`) is the largest convolution configuration -- 3x3, fp16 tensors, N=128, 128->128
+quaternion channels, 28x28, full16 policy -- and which carries, under `per_config`, the same figures
+for every other configuration (Dense fp32; 1x1 and 3x3 fp32; the four fp16 shapes under both fp16
+policies; each in both product modes) and, under `c5_qresnet50`, the ResNet-50 images/s.
+`--workload NAME` runs one configuration alone (used for profiling).
+
+Throughput is real-equivalent: 16 real multiply-adds per quaternion multiply-add whichever product
+formulation runs; the factorized (8-product) kernels execute half of them, which `executed_frac`
+reports next to the real-equivalent `frac`.
 """
 import argparse
 import ctypes
 import json
 import os
+import re
 import sys
 import time
 
@@ -20,51 +27,55 @@ sys.path.insert(0, ROOT)
 
 METRIC = "quaternion conv TFLOP/s (real-equiv, % MFMA peak) + q-ResNet-50 fwd+bwd img/s"
 PEAK_TFLOPS = {"f32": 157.3, "f16": 2500.0}  # MI355X dense MFMA peaks
+PEAK_HBM_GBS = 8000.0
 
-WORKLOADS = {
-    # name: (n, ci, co, h, w, k, padding, dtype, policy)
-    "c2_pw_f32": (32, 64, 64, 56, 56, 1, "VALID", "f32", "fp32"),
-    "c3_k3_f32": (64, 64, 64, 56, 56, 3, "SAME", "f32", "fp32"),
-    "c4_k3_f16_128_28": (128, 128, 128, 28, 28, 3, "SAME", "f16", "full16"),
-    "c4_k3_f16_256_14": (128, 256, 256, 14, 14, 3, "SAME", "f16", "full16"),
-    "c4_pw_f16_128_28": (128, 128, 128, 28, 28, 1, "VALID", "f16", "full16"),
-    "c4_pw_f16_256_14": (128, 256, 256, 14, 14, 1, "VALID", "f16", "full16"),
+CONVS = {
+    # name: (n, ci, co, h, w, k, padding, dtype)
+    "c2_pw_f32": (32, 64, 64, 56, 56, 1, "VALID", "f32"),
+    "c3_k3_f32": (64, 64, 64, 56, 56, 3, "SAME", "f32"),
+    "c4_k3_f16_128_28": (128, 128, 128, 28, 28, 3, "SAME", "f16"),
+    "c4_k3_f16_256_14": (128, 256, 256, 14, 14, 3, "SAME", "f16"),
+    "c4_pw_f16_128_28": (128, 128, 128, 28, 28, 1, "VALID", "f16"),
+    "c4_pw_f16_256_14": (128, 256, 256, 14, 14, 1, "VALID", "f16"),
 }
+DENSE = {"c1_dense_f32": (32, 128, 128, "f32")}  # name: (n, in, out, dtype)
 RESNET = "c5_qresnet50"  # quaternion ResNet-50 forward+backward, N=64, 224x224, fp16 full16 policy
-
-# HBM bytes per launch of the main kernel of each pass, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
-# this script (summaries under profiles/): (FETCH_SIZE * 2 KiB + WRITE_SIZE * 1 KiB), the unit sizes being
-# what the same counters read for a plain 256 MiB device copy.  Configurations not profiled report null.
-KIB = 1024.0
-MEASURED_TRAFFIC = {
-    ("c2_pw_f32", 8): {"fwd": (66673.9 * 2 + 131712.0) * KIB, "bwd_data": (66610.1 * 2 + 131712.0) * KIB,
-                       "bwd_weights": (100555.4 * 2 + 32768.0) * KIB},
-    ("c3_k3_f32", 8): {"fwd": (150715.1 * 2 + 244946.0) * KIB, "bwd_data": (161077.9 * 2 + 246386.3) * KIB,
-                       "bwd_weights": (379051.4 * 2 + 32256.0) * KIB},
-    ("c4_k3_f16_128_28", 16): {"fwd": (86388.7 * 2 + 111692.5) * KIB, "bwd_data": (86388.7 * 2 + 111692.5) * KIB,
-                               "bwd_weights": (180024.9 * 2 + 48384.0) * KIB},
-    ("c4_k3_f16_128_28", 8): {"fwd": (122328.1 * 2 + 112062.2) * KIB, "bwd_data": (121113.6 * 2 + 112644.7) * KIB,
-                              "bwd_weights": (180008.1 * 2 + 48384.0) * KIB},
-}
+HEADLINE = "c4_k3_f16_128_28"
+PASSES = ("fwd", "bwd_data", "bwd_weights")
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.md")
 
 
 def executed_share(kernel_name):
     """Executed / real-equivalent arithmetic of a kernel: the factorized (8-product) kernels run half the
-    multiplications.  The product mode asks for a formulation; on fp16 matrix cores the library runs the
-    pointwise passes and the filter gradient of the 8-product mode on 16-product kernels (faster there), so
-    the share is read off the kernel that actually ran."""
+    multiplications.  The product mode asks for a formulation; where the 16-product kernel is the faster one
+    the library runs that in either mode, so the share is read off the kernel that actually ran."""
     return 0.5 if "_p8_" in kernel_name else 1.0
+
+
+def measured_traffic():
+    """HBM bytes per launch from the rocprofv3 --pmc summaries, keyed by (workload, kernel variant name):
+    rows `| workload | kernel | fetched bytes | written bytes |` of profiles/hbm_traffic.md."""
+    table = {}
+    try:
+        with open(TRAFFIC_FILE) as f:
+            for line in f:
+                cells = [c.strip().strip("`") for c in line.strip().strip("|").split("|")]
+                if len(cells) == 4 and re.fullmatch(r"[0-9.e+]+", cells[2]) and re.fullmatch(r"[0-9.e+]+", cells[3]):
+                    table[(cells[0], cells[1])] = float(cells[2]) + float(cells[3])
+    except OSError:
+        pass
+    return table
 
 
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="c2_pw_f32", choices=sorted(WORKLOADS) + [RESNET])
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="all", choices=["all"] + sorted(CONVS) + sorted(DENSE) + [RESNET])
     ap.add_argument("--mode", type=int, default=0, choices=[0, 8, 16],
                     help="product formulation; 0 = from UPSTRIDE_MEMORY_OPTIMIZED like the reference (default 8)")
-    ap.add_argument("--policy", default=None, help="override UPSTRIDE_CONV_FP16_POLICY for fp16 workloads")
+    ap.add_argument("--policy", default=None, help="UPSTRIDE_CONV_FP16_POLICY for fp16 workloads (default full16)")
     ap.add_argument("--batch", type=int, default=64, help="images per step of the ResNet workload")
     ap.add_argument("--torch-bn", action="store_true",
                     help="ResNet workload: torch.nn.BatchNorm2d + ReLU (MIOpen) instead of the library's batch-norm kernels")
@@ -75,13 +86,28 @@ def parse():
     return ap.parse_args()
 
 
-def cpu_baseline(cfg, mode, seconds):
+def make_context(mode, policy):
+    import phoenix_core_amd as phx
+    env = {"UPSTRIDE_CONV_FP16_POLICY": policy}
+    if mode == 16:
+        env["UPSTRIDE_MEMORY_OPTIMIZED"] = "1"
+    return phx.Context(env)
+
+
+def default_mode(args):
+    import phoenix_core_amd as phx
+    if args.mode:
+        return args.mode
+    return 16 if phx.Context().memory_optimized else 8
+
+
+def cpu_baseline_conv(cfg, mode, seconds):
     """The reference's CPU algorithm (lane decomposition + scalar oneDNN convolutions through
     torch's CPU backend) on a bounded sample of the same workload."""
     import torch
     import oracle
     from oracle import torch_cpu_path as tcp
-    n, ci, co, h, w, k, padding, _, _ = cfg
+    n, ci, co, h, w, k, padding, _ = cfg
     threads = min(os.cpu_count() or 1, 16)
     torch.set_num_threads(threads)
     n_s = max(1, n // 8)
@@ -114,111 +140,104 @@ def cpu_baseline(cfg, mode, seconds):
     }
 
 
-def resnet_flops(n):
-    """Real-equivalent forward FLOPs of the 53 convolutions + head (2*16*N*Co*Ci*Ho*Wo*Kh*Kw each)."""
-    total, size = 0.0, 224
-    def conv(ci, co, k, s, hin):
-        ho = (hin + s - 1) // s
-        return 2.0 * 16 * n * co * ci * ho * ho * k * k, ho
-    f, size = conv(3, 16, 7, 2, size)
-    total += f
-    size = (size + 1) // 2  # max-pool
-    cin = 16
-    for width, cout, count, stride in ((16, 64, 3, 1), (32, 128, 4, 2), (64, 256, 6, 2), (128, 512, 3, 2)):
-        for i in range(count):
-            s = stride if i == 0 else 1
-            total += conv(cin, width, 1, 1, size)[0]
-            f, out = conv(width, width, 3, s, size)
-            total += f + conv(width, cout, 1, 1, out)[0]
-            if s != 1 or cin != cout:
-                total += conv(cin, cout, 1, s, size)[0]
-            size, cin = out, cout
-    return total + 2.0 * 16 * n * 250 * 512
-
-
-def bench_resnet(args):
-    import torch
-    import phoenix_core_amd as phx
-    from phoenix_core_amd import capi
-    policy = args.policy or "full16"
-    env = {"UPSTRIDE_CONV_FP16_POLICY": policy}
-    if args.mode == 16 or (args.mode == 0 and phx.Context().memory_optimized):
-        env["UPSTRIDE_MEMORY_OPTIMIZED"] = "1"
-    ctx = phx.Context(env)
-    mode = 16 if ctx.memory_optimized else 8
-    n = args.batch
-    dev = torch.device("cuda:0")
-    torch.manual_seed(0x5EED + 5)
-    model = phx.QResNet50(1000, dtype=torch.float16, context=ctx, fused_bn=not args.torch_bn).to(dev).train()
-    images = torch.randn(n, 3, 224, 224, device=dev).half()
-    labels = torch.randint(0, 1000, (n,), device=dev)
+def cpu_baseline_dense(cfg, mode, seconds):
+    """The reference's CPU Dense path restated in C (oracle/, float arithmetic, the factorized or generic
+    formulation), whole workload, single thread."""
+    import numpy as np
+    import oracle
+    n, ni, no, _ = cfg
+    r = np.random.default_rng(0x5EED + 1)
+    x = r.standard_normal((4 * n, ni)).astype(np.float32)
+    lim = (6.0 / (ni + no)) ** 0.5
+    w = r.uniform(-lim, lim, (4, ni, no)).astype(np.float32)
+    b = np.zeros((4, no), np.float32)
+    gr = r.standard_normal((4 * n, no)).astype(np.float32)
+    name = "factorized" if mode == 8 else "generic"
 
     def step():
-        model.zero_grad(set_to_none=True)
-        loss = torch.nn.functional.cross_entropy(model(images).float(), labels)
-        loss.backward()
-        return loss
+        oracle.dense_fwd(x, w, b, name, dtype=np.float32)
+        oracle.dense_bwd(x, w, gr, name, dtype=np.float32)
 
-    for _ in range(args.warmup):
+    step()
+    times = []
+    t_end = time.perf_counter() + min(seconds, 2.0)
+    while len(times) < 5 or (time.perf_counter() < t_end and len(times) < 200):
+        t0 = time.perf_counter()
         step()
-    torch.cuda.synchronize()
-    ncalls = 3 * 54
-    capi.profile_enable(ncalls * args.steps)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        loss = step()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    kernel_ms = capi.profile_collect(ncalls * args.steps)
-    capi.profile_enable(0)
-    ms_per_step = elapsed / args.steps * 1e3
-    fwd_flops = resnet_flops(n)
-    conv_ms = sum(kernel_ms) / args.steps
-    out = {
-        "metric": METRIC, "value": n / (ms_per_step * 1e-3), "unit": "img/s", "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "f16", "data": "synthetic",
-        "config": {"workload": "%s: quaternion ResNet-50 forward+backward (no optimizer step, as the metric names), "
-                               "N=%d real images (4N=%d quaternion rows after the real-input stem), 224x224, 53 quaternion convs + "
-                               "quaternion dense head; batch-norm (with the ReLU behind it) by %s, residual add, "
-                               "pooling and cross-entropy by PyTorch"
-                               % (RESNET, n, 4 * n, "torch.nn.BatchNorm2d (MIOpen)" if args.torch_bn else
-                                  "the library's streaming kernels (include/phx_bn.h)"),
-                   "product_mode": mode, "fp16_policy": policy, "batch_norm": "torch" if args.torch_bn else "library"},
-        "real_equiv_tflops": 3 * fwd_flops / (ms_per_step * 1e-3) / 1e12,
-        "quaternion_kernel_ms_per_step": conv_ms, "loss": float(loss.detach()),
-    }
-    print(json.dumps(out))
-    return 0
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    med = times[len(times) // 2]
+    flops = 3 * 2.0 * 16 * n * ni * no
+    return {"value": flops / med / 1e12, "unit": "TFLOP/s", "cores": 1, "kind": "port",
+            "sample": "whole workload, fwd+dgrad+wgrad, %s path, C restatement of the reference's CPU algorithm "
+                      "(scalar matmuls as plain loops, one thread), fp32, median of %d runs" % (name, len(times)),
+            "ms_per_step_sample": med * 1e3}
 
 
-def main():
-    args = parse()
-    if args.gpus != 1:
-        print("bench.py measures one GPU: this build has no multi-GPU path (--gpus %d refused)" % args.gpus,
-              file=sys.stderr)
-        return 2
-    if args.workload == RESNET:
-        return bench_resnet(args)
+class _Timed:
+    """Runs `step` (which makes ncalls library calls) warmup + steps times and returns wall-clock
+    milliseconds per step and, per call slot, the mean HIP-event duration of its dominant kernel."""
 
+    def __init__(self, step, ncalls, steps, warmup):
+        import torch
+        from phoenix_core_amd import capi
+        for _ in range(warmup):
+            step()
+        torch.cuda.synchronize()
+        capi.profile_enable(ncalls * steps)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step()
+        torch.cuda.synchronize()
+        self.ms_per_step = (time.perf_counter() - t0) / steps * 1e3
+        ms = capi.profile_collect(ncalls * steps)
+        capi.profile_enable(0)
+        self.kernel_ms = [sum(ms[i::ncalls]) / max(1, len(ms[i::ncalls])) for i in range(ncalls)]
+
+
+def roofline_of(pass_name, kernel, flops, nbytes, kernel_ms, compute, traffic):
+    """Roofline record of one kernel launch.  `bound` names the roof that applies by arithmetic
+    intensity (algorithmic FLOPs / algorithmic bytes against the ridge peak_flops / peak_bandwidth);
+    `regime` says "latency" when the kernel is below half of both roofs."""
+    peak = PEAK_TFLOPS[compute]
+    tflops = flops / (kernel_ms * 1e-3) / 1e12
+    gbs = nbytes / (kernel_ms * 1e-3) / 1e9
+    share = executed_share(kernel)
+    ridge = peak * 1e12 / (PEAK_HBM_GBS * 1e9)
+    ai = flops / nbytes
+    bound = "hbm" if ai < ridge else "mfma"
+    frac_mfma, frac_hbm = tflops / peak, gbs / PEAK_HBM_GBS
+    out = {"bound": bound, "pass": pass_name, "kernel": kernel, "kernel_ms": kernel_ms}
+    if bound == "mfma":
+        out.update({"achieved": tflops, "peak": peak, "unit": "TFLOP/s", "frac": frac_mfma})
+    else:
+        out.update({"achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": frac_hbm})
+    out.update({
+        "executed_frac": frac_mfma * share,  # executed FLOPs / MFMA peak (the factorized kernels run half)
+        "real_equiv_tflops": tflops, "frac_of_mfma_peak": frac_mfma, "algorithmic_gb_s": gbs, "frac_of_hbm_peak": frac_hbm,
+        "arithmetic_intensity": ai, "ridge": ridge,
+        "regime": "latency" if max(frac_mfma * share, frac_hbm) < 0.5 else bound,
+        "algorithmic_bytes": nbytes, "algorithmic_flops": flops,
+        "traffic": traffic,
+    })
+    if traffic is None:
+        out["traffic_note"] = "no rocprofv3 --pmc summary under profiles/ for this kernel variant on this workload"
+    return out
+
+
+def run_conv(name, mode, policy, args, traffic_table):
+    """fwd + input gradient + filter gradient of one convolution configuration through the C ABI."""
     import torch
     import phoenix_core_amd as phx
     from phoenix_core_amd import capi
-
-    cfg = WORKLOADS[args.workload]
-    n, ci, co, h, w, k, padding, dt, policy = cfg
-    if args.policy:
-        policy = args.policy
-    env = {"UPSTRIDE_CONV_FP16_POLICY": policy}
-    if args.mode == 16 or (args.mode == 0 and phx.Context().memory_optimized):
-        env["UPSTRIDE_MEMORY_OPTIMIZED"] = "1"
-    ctx = phx.Context(env)
-    mode = 16 if ctx.memory_optimized else 8
+    n, ci, co, h, w, k, padding, dt = CONVS[name]
+    if dt == "f32":
+        policy = "fp32"
+    ctx = make_context(mode, policy)
     dtype = torch.float32 if dt == "f32" else torch.float16
-
     dev = torch.device("cuda:0")
-    torch.manual_seed(0x5EED + sorted(WORKLOADS).index(args.workload))
+    torch.manual_seed(0x5EED + sorted(CONVS).index(name))
     scale = 1.0 if dt == "f32" else 0.5
     x = (scale * torch.randn(4 * n, ci, h, w, device=dev)).to(dtype)
     wt = (scale * torch.randn(4, co, ci, k, k, device=dev) * (2.0 / (ci * k * k)) ** 0.5).to(dtype)
@@ -230,7 +249,7 @@ def main():
     dw = torch.empty_like(wt)
     L = capi.lib()
     sizes = [desc.workspace_bytes(p) for p in (capi.PHX_PASS_FWD, capi.PHX_PASS_BWD_DATA, capi.PHX_PASS_BWD_WEIGHTS)]
-    ws = torch.empty(max(sizes), dtype=torch.uint8, device=dev)
+    ws = torch.empty(max(sizes + [1]), dtype=torch.uint8, device=dev)
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     P = lambda t: ctypes.c_void_p(t.data_ptr())
     d = ctypes.byref(desc.c)
@@ -250,29 +269,8 @@ def main():
         for _ in range(3):
             dst.copy_(src)  # reads 256 MiB, writes 256 MiB
         del src, dst
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    capi.profile_enable(3 * args.steps)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    kernel_ms = capi.profile_collect(3 * args.steps)
-    capi.profile_enable(0)
-
+    t = _Timed(step, 3, args.steps, args.warmup)
     flops_pass = 2.0 * 16 * n * co * ci * ho * wo * k * k
-    ms_per_step = elapsed / args.steps * 1e3
-    value = 3 * flops_pass / (ms_per_step * 1e-3) / 1e12
-    per_pass = {}
-    for i, key in enumerate(("fwd", "bwd_data", "bwd_weights")):
-        vals = kernel_ms[i::3]
-        per_pass[key] = sum(vals) / max(1, len(vals))
-    dominant = max(per_pass, key=per_pass.get)
-    compute = "f32" if (dt == "f32" or policy == "fp32" or (policy == "backward32" and dominant != "fwd")) else "f16"
-    achieved = flops_pass / (per_pass[dominant] * 1e-3) / 1e12
     esize = 4 if dt == "f32" else 2
     # algorithmic bytes of a pass: read the activations (or the gradient), read the filters, write the result
     bytes_pass = {
@@ -280,27 +278,210 @@ def main():
         "bwd_data": esize * (gr.numel() + wt.numel() + dx.numel()),
         "bwd_weights": esize * (x.numel() + gr.numel() + dw.numel()),
     }
-    traffic = MEASURED_TRAFFIC.get((args.workload, mode), {}).get(dominant)
-    out = {
-        "metric": METRIC, "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": dt, "data": "synthetic",
-        "config": {"workload": "%s: quaternion conv %dx%d stride 1, N=%d (4N=%d rows), %d->%d q-channels, %dx%d, "
-                               "fwd+input-grad+filter-grad" % (args.workload, k, k, n, 4 * n, ci, co, h, w),
-                   "product_mode": mode, "fp16_policy": policy, "padding": padding},
-        "images_per_s": n / (ms_per_step * 1e-3),
-        "frac_of_mfma_peak": value / PEAK_TFLOPS[compute],
-        "executed_tflops": value * sum(executed_share(names[k]) for k in names) / len(names),
+    per_pass = dict(zip(PASSES, t.kernel_ms))
+    compute = {p: "f32" if (dt == "f32" or policy == "fp32" or (policy == "backward32" and p != "fwd")) else "f16"
+               for p in PASSES}
+    roofs = {p: roofline_of(p, names[p], flops_pass, bytes_pass[p], per_pass[p], compute[p],
+                            traffic_table.get((name, names[p]))) for p in PASSES}
+    dominant = max(per_pass, key=per_pass.get)
+    value = 3 * flops_pass / (t.ms_per_step * 1e-3) / 1e12
+    del x, wt, gr, y, dx, dw, ws
+    torch.cuda.empty_cache()
+    return {
+        "workload": "%s: quaternion conv %dx%d stride 1, N=%d (4N=%d rows), %d->%d q-channels, %dx%d, "
+                    "fwd+input-grad+filter-grad" % (name, k, k, n, 4 * n, ci, co, h, w),
+        "product_mode": mode, "fp16_policy": policy, "padding": padding, "dtype": dt,
+        "value": value, "unit": "TFLOP/s", "ms_per_step": t.ms_per_step, "images_per_s": n / (t.ms_per_step * 1e-3),
         "kernel_ms": per_pass, "kernels": names,
-        "algorithmic_hbm_gb_s": {k: bytes_pass[k] / (per_pass[k] * 1e-3) / 1e9 for k in per_pass},
-        "roofline": {"bound": "mfma", "kernel": names[dominant], "achieved": achieved, "peak": PEAK_TFLOPS[compute],
-                     "unit": "TFLOP/s", "frac": achieved / PEAK_TFLOPS[compute], "traffic": traffic,
-                     "algorithmic_bytes": bytes_pass[dominant],
-                     "executed": achieved * executed_share(names[dominant])},
+        "real_equiv_tflops": {p: roofs[p]["real_equiv_tflops"] for p in PASSES},
+        "frac_of_mfma_peak": {p: roofs[p]["frac_of_mfma_peak"] for p in PASSES},
+        "executed_frac": {p: roofs[p]["executed_frac"] for p in PASSES},
+        "frac_of_hbm_peak": {p: roofs[p]["frac_of_hbm_peak"] for p in PASSES},
+        "roofline": roofs[dominant],
+    }
+
+
+def run_dense(name, mode, args, traffic_table):
+    """fwd + input gradient + filter gradient of the Dense configuration through the C ABI."""
+    import torch
+    import phoenix_core_amd as phx
+    from phoenix_core_amd import capi
+    n, ni, no, dt = DENSE[name]
+    ctx = make_context(mode, "fp32")
+    dev = torch.device("cuda:0")
+    torch.manual_seed(0x5EED + 1)
+    x = torch.randn(4 * n, ni, device=dev)
+    lim = (6.0 / (ni + no)) ** 0.5
+    wt = torch.empty(4, ni, no, device=dev).uniform_(-lim, lim)
+    b = torch.zeros(4, no, device=dev)
+    desc = phx.DenseDescriptor(x.shape, wt.shape, use_bias=True, context=ctx)
+    gr = torch.randn(desc.output_shape, device=dev)
+    y, dx, dw = torch.empty_like(gr), torch.empty_like(x), torch.empty_like(wt)
+    L = capi.lib()
+    sizes = [desc.workspace_bytes(p) for p in (capi.PHX_PASS_FWD, capi.PHX_PASS_BWD_DATA, capi.PHX_PASS_BWD_WEIGHTS)]
+    ws = torch.empty(max(sizes + [1]), dtype=torch.uint8, device=dev)
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+    d = ctypes.byref(desc.c)
+    names = {}
+
+    def step():
+        capi.check(L.phx_qdense_fwd(d, stream, P(x), P(wt), P(b), P(y), P(ws), sizes[0]), "fwd")
+        names.setdefault("fwd", capi.last_kernel_name())
+        capi.check(L.phx_qdense_bwd_data(d, stream, P(gr), P(wt), P(dx), P(ws), sizes[1]), "bwd_data")
+        names.setdefault("bwd_data", capi.last_kernel_name())
+        capi.check(L.phx_qdense_bwd_weights(d, stream, P(x), P(gr), P(dw), P(ws), sizes[2]), "bwd_weights")
+        names.setdefault("bwd_weights", capi.last_kernel_name())
+
+    t = _Timed(step, 3, args.steps, args.warmup)
+    flops_pass = 2.0 * 16 * n * ni * no
+    bytes_pass = {"fwd": 4 * (x.numel() + wt.numel() + b.numel() + y.numel()),
+                  "bwd_data": 4 * (gr.numel() + wt.numel() + dx.numel()),
+                  "bwd_weights": 4 * (x.numel() + gr.numel() + dw.numel())}
+    per_pass = dict(zip(PASSES, t.kernel_ms))
+    roofs = {p: roofline_of(p, names[p], flops_pass, bytes_pass[p], per_pass[p], "f32", traffic_table.get((name, names[p])))
+             for p in PASSES}
+    dominant = max(per_pass, key=per_pass.get)
+    out = {
+        "workload": "%s: quaternion Dense, N=%d (4N=%d rows), %d->%d quaternion units, bias, "
+                    "fwd+input-grad+filter-grad" % (name, n, 4 * n, ni, no),
+        "product_mode": mode, "fp16_policy": "fp32", "dtype": dt,
+        "value": 3 * flops_pass / (t.ms_per_step * 1e-3) / 1e12, "unit": "TFLOP/s", "ms_per_step": t.ms_per_step,
+        "kernel_ms": per_pass, "kernels": names,
+        "real_equiv_tflops": {p: roofs[p]["real_equiv_tflops"] for p in PASSES},
+        "roofline": roofs[dominant],
+        "note": "16.8 MFLOP per pass: three kernel launches of a few microseconds each, launch-latency bound",
     }
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(cfg, mode, args.cpu_seconds)
-    print(json.dumps(out))
+        out["cpu_baseline"] = cpu_baseline_dense(DENSE[name], mode, args.cpu_seconds)
+    return out
+
+
+def resnet_flops(n):
+    """Real-equivalent forward FLOPs of the 53 convolutions + head (2*16*N*Co*Ci*Ho*Wo*Kh*Kw each)."""
+    total, size = 0.0, 224
+
+    def conv(ci, co, k, s, hin):
+        ho = (hin + s - 1) // s
+        return 2.0 * 16 * n * co * ci * ho * ho * k * k, ho
+    f, size = conv(3, 16, 7, 2, size)
+    total += f
+    size = (size + 1) // 2  # max-pool
+    cin = 16
+    for width, cout, count, stride in ((16, 64, 3, 1), (32, 128, 4, 2), (64, 256, 6, 2), (128, 512, 3, 2)):
+        for i in range(count):
+            s = stride if i == 0 else 1
+            total += conv(cin, width, 1, 1, size)[0]
+            f, out = conv(width, width, 3, s, size)
+            total += f + conv(width, cout, 1, 1, out)[0]
+            if s != 1 or cin != cout:
+                total += conv(cin, cout, 1, s, size)[0]
+            size, cin = out, cout
+    return total + 2.0 * 16 * n * 250 * 512
+
+
+def run_resnet(mode, policy, args):
+    import torch
+    import phoenix_core_amd as phx
+    ctx = make_context(mode, policy)
+    n = args.batch
+    dev = torch.device("cuda:0")
+    torch.manual_seed(0x5EED + 5)
+    model = phx.QResNet50(1000, dtype=torch.float16, context=ctx, fused_bn=not args.torch_bn).to(dev).train()
+    images = torch.randn(n, 3, 224, 224, device=dev).half()
+    labels = torch.randint(0, 1000, (n,), device=dev)
+    last = {}
+
+    def step():
+        model.zero_grad(set_to_none=True)
+        loss = torch.nn.functional.cross_entropy(model(images).float(), labels)
+        loss.backward()
+        last["loss"] = loss
+
+    t = _Timed(step, 3 * 54, args.steps, max(args.warmup, 3))
+    fwd_flops = resnet_flops(n)
+    out = {
+        "workload": "%s: quaternion ResNet-50 forward+backward (no optimizer step, as the metric names), "
+                    "N=%d real images (4N=%d quaternion rows after the real-input stem), 224x224, 53 quaternion convs + "
+                    "quaternion dense head; batch-norm (with the ReLU behind it) by %s, residual add, "
+                    "pooling and cross-entropy by PyTorch"
+                    % (RESNET, n, 4 * n, "torch.nn.BatchNorm2d (MIOpen)" if args.torch_bn else
+                       "the library's streaming kernels (include/phx_bn.h)"),
+        "product_mode": mode, "fp16_policy": policy, "batch_norm": "torch" if args.torch_bn else "library", "dtype": "f16",
+        "value": n / (t.ms_per_step * 1e-3), "unit": "img/s", "images_per_s": n / (t.ms_per_step * 1e-3),
+        "ms_per_step": t.ms_per_step,
+        "real_equiv_tflops": 3 * fwd_flops / (t.ms_per_step * 1e-3) / 1e12,
+        "frac_of_mfma_peak": 3 * fwd_flops / (t.ms_per_step * 1e-3) / 1e12 / PEAK_TFLOPS["f16"],
+        "quaternion_kernel_ms_per_step": sum(t.kernel_ms), "loss": float(last["loss"].detach()),
+    }
+    del model, images, labels, last
+    torch.cuda.empty_cache()
+    return out
+
+
+def line(head, args, extra=None):
+    """The contract's JSON line around one workload record."""
+    out = {
+        "metric": METRIC, "value": head["value"], "unit": head["unit"], "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": head["ms_per_step"], "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": head["dtype"], "data": "synthetic",
+        "config": {k: head[k] for k in ("workload", "product_mode", "fp16_policy", "padding", "batch_norm") if k in head},
+    }
+    for k, v in head.items():
+        if k not in out and k not in out["config"]:
+            out[k] = v
+    if extra:
+        out.update(extra)
+    return out
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (--gpus %d refused)" % args.gpus,
+              file=sys.stderr)
+        return 2
+    import phoenix_core_amd  # noqa: F401  (fails loudly when the HIP library is missing)
+    mode = default_mode(args)
+    policy = args.policy or "full16"
+    traffic = measured_traffic()
+
+    if args.workload == RESNET:
+        print(json.dumps(line(run_resnet(mode, policy, args), args)))
+        return 0
+    if args.workload in DENSE:
+        print(json.dumps(line(run_dense(args.workload, mode, args, traffic), args)))
+        return 0
+    if args.workload in CONVS:
+        head = run_conv(args.workload, mode, policy, args, traffic)
+        if not args.no_cpu_baseline:
+            head["cpu_baseline"] = cpu_baseline_conv(CONVS[args.workload], mode, args.cpu_seconds)
+        print(json.dumps(line(head, args)))
+        return 0
+
+    # default: headline on the largest convolution configuration + every other configuration beside it
+    head = run_conv(HEADLINE, mode, policy, args, traffic)
+    per_config = {}
+    for name in sorted(DENSE):
+        per_config[name] = {"mode%d" % m: run_dense(name, m, args, traffic) for m in (8, 16)}
+    for name in sorted(CONVS):
+        policies = ("fp32",) if CONVS[name][7] == "f32" else ("full16", "backward32")
+        entry = {}
+        for pol in policies:
+            for m in (8, 16):
+                if name == HEADLINE and m == mode and pol == policy:
+                    rec = dict(head)
+                else:
+                    rec = run_conv(name, m, pol, args, traffic)
+                entry["%s_mode%d" % (pol, m)] = rec
+        per_config[name] = entry
+    c5 = {"mode%d" % m: run_resnet(m, "full16", args) for m in (mode, 24 - mode)}
+    extra = {"per_config": per_config, RESNET: c5,
+             "images_per_s_%s" % RESNET: c5["mode%d" % mode]["images_per_s"],
+             "ms_per_step_%s" % RESNET: c5["mode%d" % mode]["ms_per_step"]}
+    if not args.no_cpu_baseline:
+        head["cpu_baseline"] = cpu_baseline_conv(CONVS[HEADLINE], mode, args.cpu_seconds)
+    print(json.dumps(line(head, args, extra)))
     return 0
 
 

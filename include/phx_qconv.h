@@ -119,6 +119,19 @@ typedef struct phx_qdense_desc {
 
 const char* phx_status_string(int status);
 
+/* One-time set-up for the device that is current on the calling thread: opts every kernel variant that needs it
+ * into more than 64 KiB of dynamic LDS.  Every
+ * compute entry point does the same on its first call with a device current, so calling this is optional --
+ * except in front of a stream capture (HIP graphs), where it keeps the set-up calls out of the captured region.
+ * Plays the part of the reference's per-device context construction (src/backend/cudnn/context.hpp:57-66,
+ * src/backend/cudnn/device.hpp:55-73). */
+int phx_init(void);
+
+/* Developer hook: reads the PHX_TUNE_* planner overrides and UPSTRIDE_VERBOSE again (they are otherwise read once,
+ * on first use) and forgets the cached plans.  Not to be called while another thread is inside a compute entry
+ * point.  No counterpart in the reference, whose Context reads its switches once (src/backend/backend.cc:45-48). */
+int phx_tuning_reload(void);
+
 /* The rearrangement that carries an algebra onto the quaternion kernels: `dims` blades, `halves` quaternion-like
  * parts; quaternion component p of half h is sign[h * 4 + p] * blade[h * 4 + p] (blade -1: the component is zero).
  * Host-only (no GPU work): lets a caller, or a test, check the map against the algebra's sign table

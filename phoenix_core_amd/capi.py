@@ -27,6 +27,7 @@ EXPORTS = (
     "phx_device_count", "phx_device_malloc", "phx_device_free", "phx_memcpy_h2d", "phx_memcpy_d2h",
     "phx_memset_zero", "phx_stream_create", "phx_stream_destroy", "phx_stream_synchronize",
     "phx_last_kernel_name", "phx_profile_enable", "phx_profile_collect", "phx_algebra_map",
+    "phx_init", "phx_tuning_reload",
 )
 
 
@@ -115,6 +116,16 @@ def last_kernel_name():
 def check(status, what):
     if status != PHX_OK:
         raise PhxError(status, what)
+
+
+def init():
+    """Per-device set-up for the current device (optional, except in front of a stream capture)."""
+    check(lib().phx_init(), "phx_init")
+
+
+def tuning_reload():
+    """Re-read the PHX_TUNE_* overrides and UPSTRIDE_VERBOSE from the environment (tests)."""
+    check(lib().phx_tuning_reload(), "phx_tuning_reload")
 
 
 def profile_enable(capacity):

@@ -8,6 +8,18 @@
 
 namespace phx {
 
+// Kernels that need more dynamic LDS than the default 64 KiB must opt in with hipFuncSetAttribute.  That call does
+// not belong inside a launch (a launch may sit in a stream capture, and a first-use flag would be shared by
+// threads): every such kernel registers itself while the library loads, and the opt-in is applied to all of them
+// once per device by phx_init() or by the first compute call made with that device current.
+bool register_big_lds_kernel(const void* fn);
+template <auto Kernel>
+struct BigLds {
+    static inline const bool registered = register_big_lds_kernel(reinterpret_cast<const void*>(Kernel));
+};
+
+bool tuning_noearly();  // PHX_TUNE_NOEARLY, read once with the other planner overrides
+
 // which instantiation of the forward / input-gradient kernel to run
 struct FwdVariant {
     bool half_storage;  // tensors are fp16 (else fp32)

@@ -1,6 +1,4 @@
 // Instantiations of the fp16-MFMA forward / input-gradient kernels and their filter packing.
-#include <cstdlib>
-
 #include "phx_kernels_f16.h"
 #include "phx_launch.h"
 
@@ -37,21 +35,24 @@ static int launch_lds16(const FwdVariant& v, const ConvArgs& a, hipStream_t st) 
     constexpr int P2A = 8, P2B = CHUNKS ? 8 : 7;  // chunk staging has a single shape
 #define PHX_CASE(WCO_, NTW_, P2_)                                                                             \
     if (v.WCO == WCO_ && v.NTW == NTW_ && (CHUNKS || v.P2LOG == P2_)) {                                        \
-        hipLaunchKernelGGL((qconv_fwd_f16_lds_kernel<16, MAP_FWD, WCO_, NTW_, P2_, CHUNKS>), dim3(v.wgs), dim3(WG_THREADS), \
-                           v.lds_bytes, st, a);                                                               \
+        constexpr auto kernel = qconv_fwd_f16_lds_kernel<16, MAP_FWD, WCO_, NTW_, P2_, CHUNKS>;              \
+        if (!BigLds<kernel>::registered) return -1; /* dynamic LDS opt-in at set-up, see BigLds */            \
+        hipLaunchKernelGGL(kernel, dim3(v.wgs), dim3(WG_THREADS), v.lds_bytes, st, a);                        \
         return 0;                                                                                             \
     }
     if constexpr (CHUNKS) {
         // one filter group per chunk (pointwise problems): the variant that requests the next chunk first
-        if (v.ngroups == 1 && v.NTW == 1 && !getenv("PHX_TUNE_NOEARLY")) {
+        if (v.ngroups == 1 && v.NTW == 1 && !tuning_noearly()) {
             if (v.WCO == 1) {
-                hipLaunchKernelGGL((qconv_fwd_f16_lds_kernel<16, MAP_FWD, 1, 1, 8, true, true>), dim3(v.wgs), dim3(WG_THREADS),
-                                   v.lds_bytes, st, a);
+                constexpr auto kernel = qconv_fwd_f16_lds_kernel<16, MAP_FWD, 1, 1, 8, true, true>;
+                if (!BigLds<kernel>::registered) return -1;
+                hipLaunchKernelGGL(kernel, dim3(v.wgs), dim3(WG_THREADS), v.lds_bytes, st, a);
                 return 0;
             }
             if (v.WCO == 2) {
-                hipLaunchKernelGGL((qconv_fwd_f16_lds_kernel<16, MAP_FWD, 2, 1, 8, true, true>), dim3(v.wgs), dim3(WG_THREADS),
-                                   v.lds_bytes, st, a);
+                constexpr auto kernel = qconv_fwd_f16_lds_kernel<16, MAP_FWD, 2, 1, 8, true, true>;
+                if (!BigLds<kernel>::registered) return -1;
+                hipLaunchKernelGGL(kernel, dim3(v.wgs), dim3(WG_THREADS), v.lds_bytes, st, a);
                 return 0;
             }
         }

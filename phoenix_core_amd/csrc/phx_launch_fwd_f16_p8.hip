@@ -8,16 +8,9 @@ template <int MAP>
 static int launch_lds8(const FwdVariant& v, const ConvArgs& a, hipStream_t st) {
 #define PHX_CASE(WCO_, NTW_)                                                                                       \
     if (v.WCO == WCO_ && v.NTW == NTW_) {                                                                          \
-        auto kernel = qconv_fwd_f16_lds_kernel<8, MAP, WCO_, NTW_, 8, true>;                                       \
-        static bool raised = false; /* dynamic LDS above the default 64 KiB needs an explicit opt-in */           \
-        if (!raised && v.lds_bytes > 64 * 1024) {                                                                  \
-            if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, \
-                                    160 * 1024) != hipSuccess) {                                                   \
-                (void)hipGetLastError();                                                                           \
-                return -1;                                                                                         \
-            }                                                                                                      \
-            raised = true;                                                                                         \
-        }                                                                                                          \
+        constexpr auto kernel = qconv_fwd_f16_lds_kernel<8, MAP, WCO_, NTW_, 8, true>;                             \
+        /* more than 64 KiB of dynamic LDS: opted in per device at set-up, see BigLds */                           \
+        if (!BigLds<kernel>::registered) return -1;                                                                \
         hipLaunchKernelGGL(kernel, dim3(v.wgs), dim3(WG_THREADS), v.lds_bytes, st, a);                             \
         return 0;                                                                                                  \
     }

@@ -6,16 +6,8 @@ namespace phx {
 
 template <int MODE, int MT, int NT, int TPW, int SW>
 static int launch_one(const WgradArgs& a, int nblocks, size_t lds_bytes, hipStream_t st) {
-    auto kernel = qconv_wgrad_f16_kernel<MODE, MT, NT, TPW, SW>;
-    static bool raised = false;  // dynamic LDS above the default 64 KiB needs an explicit opt-in
-    if (!raised && lds_bytes > 64 * 1024) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                160 * 1024) != hipSuccess) {
-            (void)hipGetLastError();
-            return -1;
-        }
-        raised = true;
-    }
+    constexpr auto kernel = qconv_wgrad_f16_kernel<MODE, MT, NT, TPW, SW>;
+    if (!BigLds<kernel>::registered) return -1;  // (always true: naming the member makes the registration happen while the library loads)
     hipLaunchKernelGGL(kernel, dim3(nblocks), dim3(WG_THREADS), lds_bytes, st, a);
     return 0;
 }

@@ -3,15 +3,112 @@
 #include "../../include/phx_qconv.h"
 
 #include <algorithm>
+#include <atomic>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
 #include <mutex>
+#include <unordered_map>
 #include <vector>
 
 #include "phx_launch.h"
 
 namespace phx {
+
+// Developer overrides of the planner (kernel tuning experiments and the tests that pin a kernel variant), read
+// from the environment once; phx_tuning_reload() reads them again and forgets the cached plans.
+struct Tuning {
+    int tile_wco = 0, tile_ntw = 0;   // PHX_TUNE_TILE="wco,ntw"
+    bool flat = false, noflat = false, nopw = false, pw8 = false, zi8 = false, wg8 = false, nos2d = false, noearly = false;
+    bool nopwx = false;               // PHX_TUNE_NOPWX: pointwise fp16 problems stay on the staged-window kernels
+    int vec = 0;                      // PHX_TUNE_VEC (0 = unset)
+    int wgs = 0;                      // PHX_TUNE_WGS (0 = unset)
+    int wg_mt = 0, wg_nt = 0;         // PHX_TUNE_WG="mt,nt"
+    int phase = -1;                   // PHX_TUNE_PHASE (-1 = unset)
+    int verbose = 0;                  // UPSTRIDE_VERBOSE (src/backend/backend.cc:45-48)
+    void read() {
+        *this = Tuning();
+        if (const char* t = std::getenv("PHX_TUNE_TILE")) sscanf(t, "%d,%d", &tile_wco, &tile_ntw);
+        flat = getenv("PHX_TUNE_FLAT") != nullptr;
+        noflat = getenv("PHX_TUNE_NOFLAT") != nullptr;
+        nopw = getenv("PHX_TUNE_NOPW") != nullptr;
+        pw8 = getenv("PHX_TUNE_PW8") != nullptr;
+        zi8 = getenv("PHX_TUNE_ZI8") != nullptr;
+        wg8 = getenv("PHX_TUNE_WG8") != nullptr;
+        nos2d = getenv("PHX_TUNE_NOS2D") != nullptr;
+        noearly = getenv("PHX_TUNE_NOEARLY") != nullptr;
+        nopwx = getenv("PHX_TUNE_NOPWX") != nullptr;
+        if (const char* e = getenv("PHX_TUNE_VEC")) vec = atoi(e);
+        if (const char* e = getenv("PHX_TUNE_WGS")) wgs = atoi(e);
+        if (const char* e = getenv("PHX_TUNE_WG")) sscanf(e, "%d,%d", &wg_mt, &wg_nt);
+        if (const char* e = getenv("PHX_TUNE_PHASE")) phase = atoi(e) != 0;
+        if (const char* e = getenv("UPSTRIDE_VERBOSE")) verbose = (int)strtol(e, nullptr, 10);
+    }
+};
+static Tuning g_tune;
+static std::once_flag g_tune_once;
+static const Tuning& tune() {
+    std::call_once(g_tune_once, [] { g_tune.read(); });
+    return g_tune;
+}
+bool tuning_noearly() { return tune().noearly; }
+
+// Plans are pure functions of the problem and the tuning overrides; they are computed once per distinct
+// problem (the reference keeps its configured operations per descriptor, src/backend/op_collections.hpp:121-144).
+// (fixed-size keys: a lookup that hits allocates nothing)
+struct PlanKey {
+    int v[24];
+    bool operator==(const PlanKey& o) const { return std::memcmp(v, o.v, sizeof(v)) == 0; }
+};
+struct PlanKeyHash {
+    size_t operator()(const PlanKey& k) const {
+        size_t h = 1469598103934665603ull;
+        for (int x : k.v) h = (h ^ (unsigned)x) * 1099511628211ull;
+        return h;
+    }
+};
+static std::mutex g_plan_mutex;
+static unsigned g_plan_generation = 0;  // bumped (under g_plan_mutex) when the tuning overrides are read again
+// Kernels that need more dynamic LDS than the default 64 KiB (see phx_launch.h)
+static std::vector<const void*>& big_lds_kernels() {
+    static std::vector<const void*> v;
+    return v;
+}
+bool register_big_lds_kernel(const void* fn) {
+    big_lds_kernels().push_back(fn);
+    return true;
+}
+
+// Per-device set-up, done once per device by phx_init() or by the first compute call made with that device
+// current: the dynamic-LDS opt-in of every kernel variant that needs it (never done inside a launch, which may
+// sit in a stream capture).
+struct DeviceState {
+    std::atomic<int> ready{0};  // 0 = not set up, 1 = ready, -1 = set-up failed
+};
+constexpr int MAX_DEVICES = 64;
+static DeviceState g_devices[MAX_DEVICES];
+static std::mutex g_device_mutex;
+
+static int device_state(DeviceState** out) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) { (void)hipGetLastError(); return PHX_ERR_RUNTIME; }
+    DeviceState& d = g_devices[dev];
+    if (d.ready.load(std::memory_order_acquire) == 0) {
+        std::lock_guard<std::mutex> lock(g_device_mutex);
+        if (d.ready.load(std::memory_order_relaxed) == 0) {
+            int ok = 1;
+            for (const void* fn : big_lds_kernels())
+                if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess) {
+                    (void)hipGetLastError();
+                    ok = -1;
+                }
+            d.ready.store(ok, std::memory_order_release);
+        }
+    }
+    if (d.ready.load(std::memory_order_acquire) != 1) return PHX_ERR_RUNTIME;
+    if (out) *out = &d;
+    return PHX_OK;
+}
 
 static thread_local const char* g_last_kernel = "";
 static thread_local char g_name_buf[160];
@@ -31,6 +128,10 @@ struct KernelTimer {
     int slot;
     explicit KernelTimer(hipStream_t s) : st(s), slot(-1) {
         if (!g_prof.on) return;
+        // no event records into a stream capture: a captured graph would replay them against events of this run
+        hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(st, &cs) != hipSuccess) { (void)hipGetLastError(); return; }
+        if (cs != hipStreamCaptureStatusNone) return;
         std::lock_guard<std::mutex> lock(g_prof_mutex);
         if (2 * (g_prof.used + 1) <= (int)g_prof.ev.size()) {
             slot = g_prof.used++;
@@ -140,6 +241,15 @@ static int problem_from_dense(const phx_qdense_desc* d, Problem& p) {
     return PHX_OK;
 }
 
+// UPSTRIDE_VERBOSE > 0 (src/backend/backend.cc:45-62, the reference's UPSTRIDE_SAYS): one line per kernel
+// dispatch naming the product mode asked for, the fp16 policy and the kernel variant chosen
+static void say(const Problem& p, const char* pass) {
+    if (tune().verbose <= 0) return;
+    static const char* const policies[] = {"fp32", "backward32", "full16"};
+    fprintf(stderr, "[upstride] quaternion %s: product mode %d, fp16 policy %s, kernel %s\n", pass, p.mode,
+            p.dtype == PHX_F16 ? policies[p.policy] : "n/a (fp32 tensors)", g_last_kernel);
+}
+
 static bool is_empty(const Problem& p) { return p.n == 0 || p.h == 0 || p.w == 0; }
 
 static bool is_pointwise_unit(const Problem& p) {
@@ -217,9 +327,8 @@ static bool plan_forward(const Corr& c, int mode, bool f16mfma, FwdPlan& best, b
     best.pairs = pairs; best.chunks = chunks; best.vstage = vstage;
     const int wcos[3] = {1, 2, 4};
     // PHX_TUNE_TILE="wco,ntw" pins the workgroup shape (kernel tuning experiments)
-    int force_wco = 0, force_ntw = 0;
-    if (const char* t = std::getenv("PHX_TUNE_TILE")) sscanf(t, "%d,%d", &force_wco, &force_ntw);
-    const bool force_flat = getenv("PHX_TUNE_FLAT") != nullptr;
+    const int force_wco = tune().tile_wco, force_ntw = tune().tile_ntw;
+    const bool force_flat = tune().flat;
     for (int wi = 0; wi < 3; ++wi) {
         const int WCO = wcos[wi];
         if (force_wco && WCO != force_wco) continue;
@@ -265,7 +374,7 @@ static bool plan_forward(const Corr& c, int mode, bool f16mfma, FwdPlan& best, b
             // staging shows (-7 % at 32 channels), so it is offered only to the former.
             const bool flat_pays = NTW == 2 && (long)c.Cin * c.Kh * c.Kw >= 576;
             if (chunks && !pointwise && c.sh == 1 && c.sw == 1 && (flat_pays || force_flat) &&
-                !getenv("PHX_TUNE_NOFLAT")) {
+                !tune().noflat) {
                 const int reach = (c.Hout - 1) - c.pt + (c.Kh - 1) * c.dh - (c.Hin - 1);  // rows read below the image
                 const int gap = std::max(0, std::max(c.pt, reach));
                 const long S = (long)c.Hin + gap;                          // row distance of the images
@@ -352,7 +461,7 @@ static Corr virtual_pointwise(const Corr& c, bool f16mfma, int& pw) {
     if (!f16mfma || c.Kh * c.Kw != 1 || c.uh != 1 || c.uw != 1 || c.sh != 1 || c.sw != 1 || c.Hin != 1 || c.Hout != 1 ||
         c.pt != 0 || c.pl != 0 || c.Win != c.Wout)
         return c;
-    if (getenv("PHX_TUNE_NOPW")) return c;
+    if (tune().nopw) return c;
     pw = PW_TAPS;
     Corr v = c;
     v.Kh = PW_TAPS; v.Kw = 1; v.dh = 1;
@@ -368,10 +477,10 @@ static Corr virtual_pointwise(const Corr& c, bool f16mfma, int& pw) {
 // 16<->64-channel layers of a ResNet 37-75 against 64-112).  The 8-product mode means "prefer speed"
 // (src/backend/backend.hpp:36-66), so those problems run on the 16-product kernel; PHX_TUNE_PW8 keeps the
 // factorized one (tests exercise it).
-static bool plan_corr(const Corr& creal, int mode, bool f16mfma, Corr& c, FwdPlan& pl, int& pw) {
+static bool plan_corr_uncached(const Corr& creal, int mode, bool f16mfma, Corr& c, FwdPlan& pl, int& pw) {
     c = virtual_pointwise(creal, f16mfma, pw);
     if (pw) {
-        pl.kmode = (mode == 8 && !getenv("PHX_TUNE_PW8")) ? 16 : mode;
+        pl.kmode = (mode == 8 && !tune().pw8) ? 16 : mode;
         if (plan_forward(c, pl.kmode, f16mfma, pl, true) && pl.lds_filters && pl.chunks) return true;
     }
     pw = 0;
@@ -380,8 +489,35 @@ static bool plan_corr(const Corr& creal, int mode, bool f16mfma, Corr& c, FwdPla
     // the factorized kernel has no LDS-filter form for them, the 16-product kernel has (3x3 stride 2 at
     // 32-128 channels: 0.15-0.18 ms against 0.08-0.11 ms), so the 8-product mode takes that one here as well
     const bool zero_inserted = c.uh > 1 || c.uw > 1;
-    pl.kmode = (f16mfma && mode == 8 && zero_inserted && c.Kh * c.Kw > 1 && !getenv("PHX_TUNE_ZI8")) ? 16 : mode;
+    pl.kmode = (f16mfma && mode == 8 && zero_inserted && c.Kh * c.Kw > 1 && !tune().zi8) ? 16 : mode;
     return plan_forward(c, pl.kmode, f16mfma, pl);
+}
+
+struct CorrPlan {
+    Corr c;
+    FwdPlan pl;
+    int pw;
+    bool ok;
+};
+
+static bool plan_corr(const Corr& creal, int mode, bool f16mfma, Corr& c, FwdPlan& pl, int& pw) {
+    static std::unordered_map<PlanKey, CorrPlan, PlanKeyHash> memo;
+    static_assert(sizeof(Corr) == 21 * sizeof(int), "Corr is hashed as raw ints: no padding allowed");
+    PlanKey key{};
+    std::memcpy(key.v, &creal, sizeof(Corr));
+    key.v[21] = mode;
+    key.v[22] = f16mfma;
+    std::lock_guard<std::mutex> lock(g_plan_mutex);
+    static unsigned generation = 0;
+    if (generation != g_plan_generation) { memo.clear(); generation = g_plan_generation; }
+    auto it = memo.find(key);
+    if (it == memo.end()) {
+        CorrPlan cp{};
+        cp.ok = plan_corr_uncached(creal, mode, f16mfma, cp.c, cp.pl, cp.pw);
+        it = memo.emplace(key, cp).first;
+    }
+    c = it->second.c; pl = it->second.pl; pw = it->second.pw;
+    return it->second.ok;
 }
 
 static int run_corr(const Problem& p, const Corr& creal, int map, hipStream_t st, const void* in, const void* w,
@@ -427,7 +563,7 @@ static int run_corr(const Problem& p, const Corr& creal, int map, hipStream_t st
     a.nchunks = pl.nchunks;
     // pixels a lane may store as one word: the groups must not straddle tile rows or the image edge
     a.vec = (pl.TW % 4 == 0 && c.Wout % 4 == 0) ? 4 : (pl.TW % 2 == 0 && c.Wout % 2 == 0) ? 2 : 1;
-    if (const char* e = getenv("PHX_TUNE_VEC")) a.vec = std::min(a.vec, atoi(e));
+    if (tune().vec > 0) a.vec = std::min(a.vec, tune().vec);
 
     int rc = f16 ? launch_pack_filters_f16(v, pa, pack_blocks, st) : launch_pack_filters(v, pa, pack_blocks, st);
     if (rc != 0) return PHX_ERR_NOT_SUPPORTED;
@@ -441,6 +577,7 @@ static int run_corr(const Problem& p, const Corr& creal, int map, hipStream_t st
              map == MAP_FWD ? "fwd" : "dgrad", f16 ? "f16" : "f32", pl.lds_filters ? (pw ? "ldspw" : pl.chunks ? "ldsc" : "lds") : "", pl.kmode, p.dtype == PHX_F32 ? "f32" : "f16", pl.WCO,
              pl.NTW, pl.CK, pl.tall ? "flat" : "tile", pl.NB, pl.TH, pl.TW);
     g_last_kernel = g_name_buf;
+    say(p, map == MAP_FWD ? "forward" : "input gradient");
     return PHX_OK;
 }
 
@@ -464,7 +601,7 @@ static void finish_wgrad_plan(const Problem& p, int CoT, int CiT, WgPlan& best) 
     const int xy = best.co_tiles * best.ci_tiles * best.groups_per_row * p.kh;
     const int ntiles = best.tiles_n * best.tiles_h * best.tiles_w;
     int target = 512;  // two workgroups per CU: one round
-    if (const char* e = getenv("PHX_TUNE_WGS")) target = atoi(e);
+    if (tune().wgs > 0) target = tune().wgs;
     best.Z = std::max(1, std::min(ntiles, target / std::max(1, xy)));
     best.partial_bytes = (size_t)best.Z * p.kh * p.kw * 4 * best.CoP * best.CiP * sizeof(float);
 }
@@ -520,7 +657,7 @@ static bool plan_wgrad_f32(const Problem& p, WgPlan& best) {
 // speed" (src/backend/backend.hpp:36-66), so the 8-product mode runs this pass on the 16-product kernel;
 // PHX_TUNE_WG8 keeps the factorized kernel (tests exercise it).
 static int wgrad_f16_formulation(const Problem& p) {
-    return (p.mode == 8 && !getenv("PHX_TUNE_WG8")) ? 16 : p.mode;
+    return (p.mode == 8 && !tune().wg8) ? 16 : p.mode;
 }
 
 static bool plan_wgrad_f16(const Problem& p, WgPlan& best) {
@@ -529,7 +666,7 @@ static bool plan_wgrad_f16(const Problem& p, WgPlan& best) {
     best.kmode = wgrad_f16_formulation(p);
     best.MT = p.co > 32 ? 2 : 1;
     best.NT = p.ci > 32 ? 2 : 1;
-    if (const char* e = getenv("PHX_TUNE_WG")) sscanf(e, "%d,%d", &best.MT, &best.NT);
+    if (tune().wg_mt > 0 && tune().wg_nt > 0) { best.MT = tune().wg_mt; best.NT = tune().wg_nt; }
     // taps of one filter row that share a workgroup (and with it the staged gradient tile): three, or four
     // where the row has a multiple of four taps and the channel tile leaves the registers for it
     const bool shifts = best.kmode == 16 && p.sw == 1 && p.dw == 1;
@@ -551,7 +688,7 @@ static bool plan_wgrad_f16(const Problem& p, WgPlan& best) {
     const int xy = best.co_tiles * best.ci_tiles * best.groups_per_row * p.kh;
     const int per_cu = best.lds_bytes <= 80 * 1024 ? 2 : 1;
     int target = 256 * per_cu;
-    if (const char* e = getenv("PHX_TUNE_WGS")) target = atoi(e);
+    if (tune().wgs > 0) target = tune().wgs;
     best.Z = std::max(1, std::min(best.ntiles, target / std::max(1, xy)));
     best.partial_bytes = (size_t)best.Z * p.kh * p.kw * 4 * best.CoP * best.CiP * sizeof(float);
     return true;
@@ -566,7 +703,22 @@ static bool wgrad_on_f16_mfma(const Problem& p) {
 }
 
 static bool plan_wgrad(const Problem& p, bool f16mfma, WgPlan& best) {
-    return f16mfma ? plan_wgrad_f16(p, best) : plan_wgrad_f32(p, best);
+    struct Entry { WgPlan pl; bool ok; };
+    static std::unordered_map<PlanKey, Entry, PlanKeyHash> memo;
+    // everything the two planners read
+    const PlanKey key{{p.mode, p.n, p.ci, p.co, p.h, p.w, p.kh, p.kw, p.sh, p.sw, p.dh, p.dw, p.pt, p.pl, p.pb, p.pr,
+                       p.ho, p.wo, (int)f16mfma}};
+    std::lock_guard<std::mutex> lock(g_plan_mutex);
+    static unsigned generation = 0;
+    if (generation != g_plan_generation) { memo.clear(); generation = g_plan_generation; }
+    auto it = memo.find(key);
+    if (it == memo.end()) {
+        Entry e{};
+        e.ok = f16mfma ? plan_wgrad_f16(p, e.pl) : plan_wgrad_f32(p, e.pl);
+        it = memo.emplace(key, e).first;
+    }
+    best = it->second.pl;
+    return it->second.ok;
 }
 
 static int run_wgrad(const Problem& p, hipStream_t st, const void* x, const void* g, void* dw, void* ws,
@@ -615,6 +767,7 @@ static int run_wgrad(const Problem& p, hipStream_t st, const void* x, const void
         snprintf(g_name_buf, sizeof(g_name_buf), "%sqconv_wgrad_f32mfma%s_p%d_%s_tile%dx%dx%d_z%d", g_name_prefix, pl.vec ? "v" : "", p.mode,
                  p.dtype == PHX_F32 ? "f32" : "f16", pl.NB, pl.TH, pl.TW, pl.Z);
     g_last_kernel = g_name_buf;
+    say(p, "filter gradient");
     return PHX_OK;
 }
 
@@ -652,7 +805,7 @@ static PhaseAxis phase_axis(int a, int extent, int k, int d, int s, int pad_befo
 // input gradient through the phases, PHX_TUNE_PHASE=0 none.
 static bool dgrad_by_phases(const Problem& p) {
     if ((p.sh == 1 && p.sw == 1) || p.sh * p.sw > 16 || is_empty(p) || p.groups > 1) return false;
-    if (const char* e = getenv("PHX_TUNE_PHASE")) return atoi(e) != 0;
+    if (tune().phase >= 0) return tune().phase != 0;
     return p.kh == 1 && p.kw == 1;
 }
 
@@ -707,7 +860,7 @@ static int floordiv(int a, int b) { return a >= 0 ? a / b : -((-a + b - 1) / b);
 static bool s2d_view(const Problem& p, S2dView& v) {
     if (p.sh != 2 || p.sw != 2 || p.dh != 1 || p.dw != 1 || p.ci > 4 || (p.kh < 3 && p.kw < 3) || is_empty(p)) return false;
     if (p.groups > 1) return false;  // the rearranged copies are laid out for whole tensors
-    if (getenv("PHX_TUNE_NOS2D")) return false;
+    if (tune().nos2d) return false;
     const int aminh = floordiv(-p.pt, 2), amaxh = floordiv(p.kh - 1 - p.pt, 2);
     const int aminw = floordiv(-p.pl, 2), amaxw = floordiv(p.kw - 1 - p.pl, 2);
     Problem& q = v.q;
@@ -857,6 +1010,16 @@ const char* phx_status_string(int status) {
 
 const char* phx_last_kernel_name(void) { return g_last_kernel; }
 
+int phx_init(void) { return device_state(nullptr); }
+
+int phx_tuning_reload(void) {
+    std::lock_guard<std::mutex> lock(g_plan_mutex);
+    (void)tune();  // (so that a first read cannot race with this one)
+    g_tune.read();
+    ++g_plan_generation;
+    return PHX_OK;
+}
+
 int phx_profile_enable(int capacity) {
     std::lock_guard<std::mutex> lock(g_prof_mutex);
     g_prof.on = false;
@@ -958,6 +1121,7 @@ size_t phx_qdense_workspace_bytes(const phx_qdense_desc* desc, int pass) {
 
 int phx_qconv2d_fwd(const phx_qconv_desc* desc, phx_stream_t stream, const void* x, const void* w,
                     const void* bias_or_null, void* y, void* workspace, size_t workspace_bytes) {
+    if (const int init_rc = device_state(nullptr)) return init_rc;
     if (desc && desc->algebra != PHX_QUATERNION)
         return algebra_conv_pass(desc, PHX_PASS_FWD, stream, x, w, bias_or_null, y, workspace, workspace_bytes);
     Problem p;
@@ -986,6 +1150,7 @@ int phx_qconv2d_fwd(const phx_qconv_desc* desc, phx_stream_t stream, const void*
 
 int phx_qconv2d_bwd_data(const phx_qconv_desc* desc, phx_stream_t stream, const void* grad, const void* w, void* dx,
                          void* workspace, size_t workspace_bytes) {
+    if (const int init_rc = device_state(nullptr)) return init_rc;
     if (desc && desc->algebra != PHX_QUATERNION)
         return algebra_conv_pass(desc, PHX_PASS_BWD_DATA, stream, grad, w, nullptr, dx, workspace, workspace_bytes);
     Problem p;
@@ -1016,6 +1181,7 @@ int phx_qconv2d_bwd_data(const phx_qconv_desc* desc, phx_stream_t stream, const 
 
 int phx_qconv2d_bwd_weights(const phx_qconv_desc* desc, phx_stream_t stream, const void* x, const void* grad, void* dw,
                             void* workspace, size_t workspace_bytes) {
+    if (const int init_rc = device_state(nullptr)) return init_rc;
     if (desc && desc->algebra != PHX_QUATERNION)
         return algebra_conv_pass(desc, PHX_PASS_BWD_WEIGHTS, stream, x, grad, nullptr, dw, workspace, workspace_bytes);
     Problem p;
@@ -1042,6 +1208,7 @@ int phx_qconv2d_bwd_weights(const phx_qconv_desc* desc, phx_stream_t stream, con
 
 int phx_qdense_fwd(const phx_qdense_desc* desc, phx_stream_t stream, const void* x, const void* w,
                    const void* bias_or_null, void* y, void* workspace, size_t workspace_bytes) {
+    if (const int init_rc = device_state(nullptr)) return init_rc;
     if (desc && desc->algebra != PHX_QUATERNION)
         return algebra_dense_pass(desc, PHX_PASS_FWD, stream, x, w, bias_or_null, y, workspace, workspace_bytes);
     Problem p;
@@ -1052,6 +1219,7 @@ int phx_qdense_fwd(const phx_qdense_desc* desc, phx_stream_t stream, const void*
 
 int phx_qdense_bwd_data(const phx_qdense_desc* desc, phx_stream_t stream, const void* grad, const void* w, void* dx,
                         void* workspace, size_t workspace_bytes) {
+    if (const int init_rc = device_state(nullptr)) return init_rc;
     if (desc && desc->algebra != PHX_QUATERNION)
         return algebra_dense_pass(desc, PHX_PASS_BWD_DATA, stream, grad, w, nullptr, dx, workspace, workspace_bytes);
     Problem p;
@@ -1062,6 +1230,7 @@ int phx_qdense_bwd_data(const phx_qdense_desc* desc, phx_stream_t stream, const 
 
 int phx_qdense_bwd_weights(const phx_qdense_desc* desc, phx_stream_t stream, const void* x, const void* grad, void* dw,
                            void* workspace, size_t workspace_bytes) {
+    if (const int init_rc = device_state(nullptr)) return init_rc;
     if (desc && desc->algebra != PHX_QUATERNION)
         return algebra_dense_pass(desc, PHX_PASS_BWD_WEIGHTS, stream, x, grad, nullptr, dw, workspace, workspace_bytes);
     Problem p;

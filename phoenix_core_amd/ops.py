@@ -239,8 +239,25 @@ def _dev_check(*tensors):
     return dev
 
 
+def _expect(t, shape, dtype, what):
+    """The library reads raw device memory in the descriptor's type and shape: anything else is refused here."""
+    if t is None:
+        raise ValueError("%s tensor missing" % what)
+    if tuple(t.shape) != tuple(shape):
+        raise ValueError("%s has shape %s, the descriptor says %s" % (what, tuple(t.shape), tuple(shape)))
+    if t.dtype != dtype:
+        raise ValueError("%s has dtype %s, the descriptor says %s" % (what, t.dtype, dtype))
+
+
 def _ptr(t):
     return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def reserve_workspace(nbytes, device=None):
+    """Grows the scratch buffer of the current stream to at least nbytes ahead of time -- in front of a stream
+    capture, inside which the buffer must not be reallocated."""
+    device = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+    return _workspace.get(device, int(nbytes))
 
 
 def _stream():
@@ -249,13 +266,15 @@ def _stream():
 
 def conv2d_fwd(x, w, bias, desc, out=None):
     """conv2DFwd (src/upstride.hpp:18-33): y = x (x) w (+ bias)."""
-    dev = _dev_check(x, w, bias)
-    if tuple(x.shape) != desc.input_shape or tuple(w.shape) != desc.filter_shape or x.dtype != desc.dtype:
-        raise ValueError("tensor shapes / dtype do not match the descriptor")
-    if desc.use_bias and (bias is None or tuple(bias.shape) != desc.bias_shape):
-        raise ValueError("bias tensor missing or of wrong shape")
+    dev = _dev_check(x, w, bias, out)
+    _expect(x, desc.input_shape, desc.dtype, "input")
+    _expect(w, desc.filter_shape, desc.dtype, "filter")
+    if desc.use_bias:
+        _expect(bias, desc.bias_shape, desc.dtype, "bias")
     if desc.real_valued_input and desc.use_bias:  # src/conv2d.hpp:125-127
         raise RuntimeError("Bias addition is not supported for type0 inputs")
+    if out is not None:
+        _expect(out, desc.output_shape, desc.dtype, "output")
     y = out if out is not None else torch.empty(desc.output_shape, dtype=desc.dtype, device=dev)
     nbytes = desc.workspace_bytes(capi.PHX_PASS_FWD)
     ws = _workspace.get(dev, nbytes)
@@ -269,9 +288,9 @@ def conv2d_bwd(x, w, grad, desc):
     """conv2DBwd (src/upstride.hpp:35-51): returns (dw, dx); dx is None when the descriptor does
     not require the input gradient."""
     dev = _dev_check(x, w, grad)
-    if tuple(x.shape) != desc.input_shape or tuple(w.shape) != desc.filter_shape or \
-            tuple(grad.shape) != desc.output_shape:
-        raise ValueError("tensor shapes do not match the descriptor")
+    _expect(x, desc.input_shape, desc.dtype, "input")
+    _expect(w, desc.filter_shape, desc.dtype, "filter")
+    _expect(grad, desc.output_shape, desc.dtype, "output gradient")
     dw = torch.empty(desc.filter_shape, dtype=desc.dtype, device=dev)
     nbytes = desc.workspace_bytes(capi.PHX_PASS_BWD_WEIGHTS)
     ws = _workspace.get(dev, nbytes)
@@ -291,11 +310,13 @@ def conv2d_bwd(x, w, grad, desc):
 
 def dense_fwd(x, w, bias, desc, out=None):
     """denseFwd (src/upstride.hpp:53-68)."""
-    dev = _dev_check(x, w, bias)
-    if tuple(x.shape) != desc.input_shape or tuple(w.shape) != desc.filter_shape or x.dtype != desc.dtype:
-        raise ValueError("tensor shapes / dtype do not match the descriptor")
-    if desc.use_bias and (bias is None or tuple(bias.shape) != desc.bias_shape):
-        raise ValueError("bias tensor missing or of wrong shape")
+    dev = _dev_check(x, w, bias, out)
+    _expect(x, desc.input_shape, desc.dtype, "input")
+    _expect(w, desc.filter_shape, desc.dtype, "filter")
+    if desc.use_bias:
+        _expect(bias, desc.bias_shape, desc.dtype, "bias")
+    if out is not None:
+        _expect(out, desc.output_shape, desc.dtype, "output")
     y = out if out is not None else torch.empty(desc.output_shape, dtype=desc.dtype, device=dev)
     nbytes = desc.workspace_bytes(capi.PHX_PASS_FWD)
     ws = _workspace.get(dev, nbytes)
@@ -308,9 +329,9 @@ def dense_fwd(x, w, bias, desc, out=None):
 def dense_bwd(x, w, grad, desc):
     """denseBwd (src/upstride.hpp:70-86): returns (dw, dx)."""
     dev = _dev_check(x, w, grad)
-    if tuple(x.shape) != desc.input_shape or tuple(w.shape) != desc.filter_shape or \
-            tuple(grad.shape) != desc.output_shape:
-        raise ValueError("tensor shapes do not match the descriptor")
+    _expect(x, desc.input_shape, desc.dtype, "input")
+    _expect(w, desc.filter_shape, desc.dtype, "filter")
+    _expect(grad, desc.output_shape, desc.dtype, "output gradient")
     dw = torch.empty(desc.filter_shape, dtype=desc.dtype, device=dev)
     nbytes = desc.workspace_bytes(capi.PHX_PASS_BWD_WEIGHTS)
     ws = _workspace.get(dev, nbytes)
@@ -334,6 +355,11 @@ def batch_norm_fwd(x, gamma, beta, running_mean, running_var, eps, momentum, rel
     if residual is not None and (residual.shape != x.shape or residual.dtype != x.dtype):
         raise ValueError("the residual must have the shape and type of the input")
     rows, c = x.shape[0], x.shape[1]
+    if x.dtype not in _DTYPES:
+        raise ValueError("batch normalisation takes float32 or float16 activations")
+    for t, what in ((gamma, "gamma"), (beta, "beta"), (running_mean, "running_mean"), (running_var, "running_var")):
+        if t is not None:
+            _expect(t, (c,), torch.float32, what)
     hw = x.numel() // max(rows * c, 1)
     desc = capi.BnDesc(_DTYPES[x.dtype], rows, c, hw, eps, momentum, int(relu))
     y = torch.empty_like(x)
@@ -351,6 +377,13 @@ def batch_norm_bwd(x, dy, gamma, beta, mean, invstd, eps, relu, residual=None):
     """Returns (dx, dgamma, dbeta, dresidual) of batch_norm_fwd; dresidual is None without a residual."""
     dev = _dev_check(x, dy, gamma, beta, mean, invstd, residual)
     rows, c = x.shape[0], x.shape[1]
+    if x.dtype not in _DTYPES:
+        raise ValueError("batch normalisation takes float32 or float16 activations")
+    _expect(dy, x.shape, x.dtype, "output gradient")
+    if residual is not None:
+        _expect(residual, x.shape, x.dtype, "residual")
+    for t, what in ((gamma, "gamma"), (beta, "beta"), (mean, "mean"), (invstd, "invstd")):
+        _expect(t, (c,), torch.float32, what)
     hw = x.numel() // max(rows * c, 1)
     desc = capi.BnDesc(_DTYPES[x.dtype], rows, c, hw, eps, 0.0, int(relu))
     dx = torch.empty_like(x)

@@ -15,3 +15,22 @@ def pytest_configure(config):
 @pytest.fixture(scope="session")
 def golden_dir():
     return os.path.join(ROOT, "tests", "golden")
+
+
+@pytest.fixture
+def tune_env(monkeypatch):
+    """tune_env(NAME="1", OTHER=None) sets / deletes planner override variables and makes the library read them
+    again (it reads them once otherwise); the environment and the library's view of it are restored afterwards."""
+    from phoenix_core_amd import capi
+
+    def apply(**variables):
+        for key, value in variables.items():
+            if value is None:
+                monkeypatch.delenv(key, raising=False)
+            else:
+                monkeypatch.setenv(key, value)
+        capi.tuning_reload()
+
+    yield apply
+    monkeypatch.undo()
+    capi.tuning_reload()

@@ -32,6 +32,11 @@ FULL = [
     ("c4_k3_f16_128_28", 128, 128, 128, 28, 28, 3, "SAME", torch.float16, "full16"),
     ("c4_k3_f16_256_14", 128, 256, 256, 14, 14, 3, "SAME", torch.float16, "full16"),
     ("c4_pw_f16_128_28", 128, 128, 128, 28, 28, 1, "VALID", torch.float16, "full16"),
+    ("c4_pw_f16_256_14", 128, 256, 256, 14, 14, 1, "VALID", torch.float16, "full16"),
+    # fp16 MFMA forward, fp32 MFMA backward
+    ("c4_k3_f16_128_28", 128, 128, 128, 28, 28, 3, "SAME", torch.float16, "backward32"),
+    ("c4_k3_f16_256_14", 128, 256, 256, 14, 14, 3, "SAME", torch.float16, "backward32"),
+    ("c4_pw_f16_128_28", 128, 128, 128, 28, 28, 1, "VALID", torch.float16, "backward32"),
     ("c4_pw_f16_256_14", 128, 256, 256, 14, 14, 1, "VALID", torch.float16, "backward32"),
 ]
 
@@ -67,7 +72,7 @@ def norm(a):
 
 
 @pytest.mark.parametrize("mode", [8, 16])
-@pytest.mark.parametrize("cfg", FULL, ids=[c[0] for c in FULL])
+@pytest.mark.parametrize("cfg", FULL, ids=[c[0] + ("" if c[9] in ("fp32", "full16") else "_" + c[9]) for c in FULL])
 def test_full_size(cfg, mode):
     name, n, ci, co, h, w, k, padding, dtype, policy = cfg
     print("config", name, "mode", mode, flush=True)

@@ -238,6 +238,8 @@ FP16_CASES = [c for c in CONV_CASES if c[0] in ("pw_64", "pw_ragged", "pw_7x7img
     ("k24_c40", 3, 40, 24, 9, 21, 2, 4, 1, 1, "VALID"),
     ("k3_128_28", 2, 128, 128, 28, 28, 3, 3, 1, 1, "SAME"),
     ("pw_256_14", 3, 256, 256, 14, 14, 1, 1, 1, 1, "VALID"),
+    ("k3_256_14", 2, 256, 256, 14, 14, 3, 3, 1, 1, "SAME"),
+    ("pw_128_28", 2, 128, 128, 28, 28, 1, 1, 1, 1, "VALID"),
 ]
 
 
@@ -279,7 +281,7 @@ def test_conv_fp16(case, mode, policy):
 @pytest.mark.parametrize("case", [c for c in FP16_CASES if c[0] in ("pw_64", "pw_ragged", "k3_same", "k3_ragged", "k3_s2",
                                                                        "k7_s2", "k32_asym", "k3_128_28", "pw_256_14")],
                          ids=lambda c: c[0])
-def test_factorized_filter_gradient_on_fp16_matrix_cores(case, monkeypatch):
+def test_factorized_filter_gradient_on_fp16_matrix_cores(case, tune_env):
     """In 8-product mode the fp16 filter gradient runs on the 16-product kernel by default (it is the faster
     one there); PHX_TUNE_WG8 selects the factorized 8-lane kernel, which must meet the same tolerance."""
     name, n, ci, co, h, w, kh, kw, stride, dilation, padding = case
@@ -290,7 +292,7 @@ def test_factorized_filter_gradient_on_fp16_matrix_cores(case, monkeypatch):
                                 require_input_grad=False)
     dw16, _ = phx.conv2d_bwd(xd, wd, gd, desc)
     assert "f16mfma_p16" in capi.last_kernel_name()
-    monkeypatch.setenv("PHX_TUNE_WG8", "1")
+    tune_env(PHX_TUNE_WG8="1")
     dw8, _ = phx.conv2d_bwd(xd, wd, gd, desc)
     assert "f16mfma_p8" in capi.last_kernel_name()
     want_dw, _ = oracle.conv2d_bwd(g, x.astype(np.float64), wt.astype(np.float64), gr.astype(np.float64), "hamilton",
@@ -301,7 +303,7 @@ def test_factorized_filter_gradient_on_fp16_matrix_cores(case, monkeypatch):
 
 @pytest.mark.parametrize("case", [c for c in FP16_CASES if c[0] in ("pw_64", "pw_ragged", "pw_7x7img", "pw_256_14", "co_gt_128")],
                          ids=lambda c: c[0])
-def test_factorized_pointwise_on_fp16_matrix_cores(case, monkeypatch):
+def test_factorized_pointwise_on_fp16_matrix_cores(case, tune_env):
     """In 8-product mode pointwise fp16 problems run on the 16-product kernel by default (two workgroups per CU
     beat the factorized kernel there); PHX_TUNE_PW8 selects the factorized kernel, same tolerance."""
     name, n, ci, co, h, w, kh, kw, stride, dilation, padding = case
@@ -315,7 +317,7 @@ def test_factorized_pointwise_on_fp16_matrix_cores(case, monkeypatch):
     _, want_dx = oracle.conv2d_bwd(g, x64, w64, g64, "hamilton")
     for forced, tag in ((False, "ldspw_p16"), (True, "ldspw_p8")):
         if forced:
-            monkeypatch.setenv("PHX_TUNE_PW8", "1")
+            tune_env(PHX_TUNE_PW8="1")
         y = phx.conv2d_fwd(xd, wd, bd, desc)
         assert tag in capi.last_kernel_name(), capi.last_kernel_name()
         _, dx = phx.conv2d_bwd(xd, wd, gd, desc)
@@ -477,7 +479,7 @@ FLAT = [c for c in FP16_CASES if c[0] in ("k3_same", "k3_ragged", "k3_valid", "k
 
 @pytest.mark.parametrize("mode", [16, 8])
 @pytest.mark.parametrize("case", FLAT, ids=lambda c: c[0])
-def test_flat_tiling(case, mode, monkeypatch):
+def test_flat_tiling(case, mode, tune_env):
     """Flat tiling of the fp16 LDS kernels (images stacked into one tall image, a workgroup takes consecutive
     output positions in row-major order): the planner offers it by shape; PHX_TUNE_FLAT offers it everywhere
     it applies, PHX_TUNE_NOFLAT nowhere.  Forward and input gradient against the oracle, and the two tilings
@@ -493,9 +495,8 @@ def test_flat_tiling(case, mode, monkeypatch):
     _, want_dx = oracle.conv2d_bwd(g, x64, w64, g64, "hamilton")
     got, names = {}, {}
     for variant, env in (("flat", "PHX_TUNE_FLAT"), ("tiles", "PHX_TUNE_NOFLAT")):
-        monkeypatch.delenv("PHX_TUNE_FLAT", raising=False)
-        monkeypatch.delenv("PHX_TUNE_NOFLAT", raising=False)
-        monkeypatch.setenv(env, "1")
+        tune_env(**{"PHX_TUNE_FLAT": None, "PHX_TUNE_NOFLAT": None})
+        tune_env(**{env: "1"})
         y = phx.conv2d_fwd(xd, wd, bd, desc)
         k_fwd = capi.last_kernel_name()
         _, dx = phx.conv2d_bwd(xd, wd, gd, desc)
@@ -543,16 +544,15 @@ STRIDED = [c for c in FP16_CASES if c[0] in ("k3_s2", "pw_s2", "k7_s2", "k3_s2_c
 @pytest.mark.parametrize("dtype,policy", [(torch.float32, "fp32"), (torch.float16, "full16")], ids=["f32", "f16"])
 @pytest.mark.parametrize("mode", [16, 8])
 @pytest.mark.parametrize("case", STRIDED, ids=lambda c: c[0])
-def test_strided_input_gradient_variants(case, mode, dtype, policy, variant, monkeypatch):
+def test_strided_input_gradient_variants(case, mode, dtype, policy, variant, tune_env):
     """The input gradient of a strided convolution has two implementations, per-phase dense correlations merged
     into dx and zero insertion in the staged window (on fp16 matrix cores in 16-product form unless the
     factorized one is forced); the planner picks by shape, the environment overrides select each."""
     name, n, ci, co, h, w, kh, kw, stride, dilation, padding = case
     scale = 1.0 if dtype == torch.float32 else 0.5
     g, x, wt, b, gr = make_inputs(name_seed(name) + 5, n, ci, co, h, w, kh, kw, stride, dilation, padding, dtype, scale)
-    monkeypatch.setenv("PHX_TUNE_PHASE", "1" if variant == "phases" else "0")
-    if variant == "zero_insertion_factorized":
-        monkeypatch.setenv("PHX_TUNE_ZI8", "1")
+    tune_env(PHX_TUNE_PHASE="1" if variant == "phases" else "0",
+             PHX_TUNE_ZI8="1" if variant == "zero_insertion_factorized" else None)
     desc = phx.Conv2DDescriptor(x.shape, wt.shape, stride, dilation, padding, dtype=dtype, context=Ctx(mode, policy))
     xd, wd, gd = (torch.from_numpy(a).cuda() for a in (x, wt, gr))
     _, dx = phx.conv2d_bwd(xd, wd, gd, desc)
@@ -580,3 +580,27 @@ def test_dense_fp16(mode, policy):
     want_dw, want_dx = oracle.dense_bwd(x64, w64, g64, "generic")
     assert_close(dx.cpu().numpy(), want_dx, torch.float16, "dense dgrad")
     assert_close(dw.cpu().numpy(), want_dw, torch.float16, "dense wgrad")
+
+
+def test_mismatched_tensors_are_refused_before_the_library_reads_them():
+    """The library reads raw device memory in the descriptor's type: a tensor of another type or shape must be
+    refused by the host layer (a fp16 filter under a fp32 descriptor would be read past its end)."""
+    x = torch.randn(8, 4, 6, 6, device="cuda")
+    w = torch.randn(4, 4, 4, 3, 3, device="cuda")
+    desc = phx.Conv2DDescriptor(x.shape, w.shape, 1, 1, "SAME", use_bias=True, context=Ctx(8))
+    b = torch.zeros(4, 4, device="cuda")
+    g = torch.randn(desc.output_shape, device="cuda")
+    with pytest.raises(ValueError):
+        phx.conv2d_fwd(x, w.half(), b, desc)
+    with pytest.raises(ValueError):
+        phx.conv2d_fwd(x, w, b.half(), desc)
+    with pytest.raises(ValueError):
+        phx.conv2d_fwd(x, w, b, desc, out=torch.empty(desc.output_shape, dtype=torch.float16, device="cuda"))
+    with pytest.raises(ValueError):
+        phx.conv2d_bwd(x, w.half(), g, desc)
+    with pytest.raises(ValueError):
+        phx.conv2d_bwd(x, w, g.half(), desc)
+    with pytest.raises(ValueError):
+        phx.conv2d_bwd(x.half(), w, g, desc)
+    y = phx.conv2d_fwd(x, w, b, desc)
+    assert torch.isfinite(y).all()
