@@ -30,7 +30,8 @@ enum phx_status {
     PHX_ERR_INVALID_ARGUMENT = 1, /* malformed descriptor or null pointer */
     PHX_ERR_NOT_SUPPORTED = 2,    /* valid request outside what the kernels cover */
     PHX_ERR_WORKSPACE = 3,        /* workspace smaller than phx_*_workspace_bytes() */
-    PHX_ERR_RUNTIME = 4           /* HIP runtime reported an error */
+    PHX_ERR_RUNTIME = 4,          /* HIP runtime reported an error */
+    PHX_ERR_SCRATCH_LIMIT = 5     /* phx_qconv2d_fwd_noalloc: the call needs more than PHX_NOALLOC_SCRATCH_BYTES */
 };
 
 enum phx_dtype { PHX_F32 = 0, PHX_F16 = 1 };
@@ -120,7 +121,7 @@ typedef struct phx_qdense_desc {
 const char* phx_status_string(int status);
 
 /* One-time set-up for the device that is current on the calling thread: opts every kernel variant that needs it
- * into more than 64 KiB of dynamic LDS.  Every
+ * into more than 64 KiB of dynamic LDS and looks up the device address of the built-in scratch array.  Every
  * compute entry point does the same on its first call with a device current, so calling this is optional --
  * except in front of a stream capture (HIP graphs), where it keeps the set-up calls out of the captured region.
  * Plays the part of the reference's per-device context construction (src/backend/cudnn/context.hpp:57-66,
@@ -150,6 +151,21 @@ size_t phx_qdense_workspace_bytes(const phx_qdense_desc* desc, int pass);
  * QuatKernelPointwiseConvForwardFunctor::operator() (src/backend/backend.hpp:163-185). */
 int phx_qconv2d_fwd(const phx_qconv_desc* desc, phx_stream_t stream, const void* x, const void* w,
                     const void* bias_or_null, void* y, void* workspace, size_t workspace_bytes);
+
+/* The forward pass for callers that cannot allocate device memory or provide a workspace (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference, whose
+ * operations always draw their temporaries from the caller's allocator (src/backend/memory_request.hpp:73-114).
+ * Same arithmetic and kernels as phx_qconv2d_fwd; what that entry point stages in the caller's workspace (the
+ * packed filters; rearranged copies for channels-last, space-to-depth or non-quaternion calls) goes to an array of
+ * PHX_NOALLOC_SCRATCH_BYTES that is part of the library's code object: each GPU the library runs on holds its own
+ * copy until the process ends.  The call allocates nothing; a descriptor whose forward pass needs more than that
+ * (phx_qconv2d_workspace_bytes(desc, PHX_PASS_FWD)) is refused with PHX_ERR_SCRATCH_LIMIT and nothing is
+ * enqueued.  All calls on one GPU share that GPU's array, which keeps the previous call's contents (every byte a
+ * call reads it has written first): calls that overlap in time on one GPU -- different streams, or different
+ * threads -- race on it and must be serialized by the caller. */
+#define PHX_NOALLOC_SCRATCH_BYTES (16u << 20)
+int phx_qconv2d_fwd_noalloc(const phx_qconv_desc* desc, phx_stream_t stream, const void* x, const void* w,
+                            const void* bias_or_null, void* y);
 
 /* dx = g (x) conj(w), spatially transposed.  Replaces the input-gradient half of
  * UpstrideConv2DGradFunctor<Device,T>::operator() (src/conv2d.hpp:331-357, 433-562) and of

@@ -9,7 +9,8 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libphx_qconv.so")
 
 PHX_OK = 0
-PHX_ERR_INVALID_ARGUMENT, PHX_ERR_NOT_SUPPORTED, PHX_ERR_WORKSPACE, PHX_ERR_RUNTIME = 1, 2, 3, 4
+PHX_ERR_INVALID_ARGUMENT, PHX_ERR_NOT_SUPPORTED, PHX_ERR_WORKSPACE, PHX_ERR_RUNTIME, PHX_ERR_SCRATCH_LIMIT = 1, 2, 3, 4, 5
+PHX_NOALLOC_SCRATCH_BYTES = 16 << 20
 PHX_F32, PHX_F16 = 0, 1
 PHX_OIHW, PHX_OHWI, PHX_HWIO = 0, 1, 2
 PHX_IO, PHX_OI = 0, 1
@@ -27,7 +28,7 @@ EXPORTS = (
     "phx_device_count", "phx_device_malloc", "phx_device_free", "phx_memcpy_h2d", "phx_memcpy_d2h",
     "phx_memset_zero", "phx_stream_create", "phx_stream_destroy", "phx_stream_synchronize",
     "phx_last_kernel_name", "phx_profile_enable", "phx_profile_collect", "phx_algebra_map",
-    "phx_init", "phx_tuning_reload",
+    "phx_init", "phx_tuning_reload", "phx_qconv2d_fwd_noalloc",
 )
 
 
@@ -79,6 +80,7 @@ def lib():
         L.phx_qdense_workspace_bytes.restype = sz
         L.phx_qdense_workspace_bytes.argtypes = [dd, ctypes.c_int]
         L.phx_qconv2d_fwd.argtypes = [cd, vp, vp, vp, vp, vp, vp, sz]
+        L.phx_qconv2d_fwd_noalloc.argtypes = [cd, vp, vp, vp, vp, vp]
         L.phx_qconv2d_bwd_data.argtypes = [cd, vp, vp, vp, vp, vp, sz]
         L.phx_qconv2d_bwd_weights.argtypes = [cd, vp, vp, vp, vp, vp, sz]
         L.phx_qdense_fwd.argtypes = [dd, vp, vp, vp, vp, vp, vp, sz]

@@ -13,6 +13,12 @@
 
 #include "phx_launch.h"
 
+// Scratch memory of phx_qconv2d_fwd_noalloc: a device-resident array of the code object (every GPU the library
+// runs on holds its own copy until the process ends).  In host code this name is only a handle for
+// hipGetSymbolAddress; the device address it stands for is looked up once per device (device_state) and that
+// pointer, never the name, is what kernels and copies receive.
+static __device__ __align__(256) unsigned char scratch[PHX_NOALLOC_SCRATCH_BYTES];
+
 namespace phx {
 
 // Developer overrides of the planner (kernel tuning experiments and the tests that pin a kernel variant), read
@@ -81,9 +87,10 @@ bool register_big_lds_kernel(const void* fn) {
 
 // Per-device set-up, done once per device by phx_init() or by the first compute call made with that device
 // current: the dynamic-LDS opt-in of every kernel variant that needs it (never done inside a launch, which may
-// sit in a stream capture).
+// sit in a stream capture) and the device address of the built-in scratch array.
 struct DeviceState {
     std::atomic<int> ready{0};  // 0 = not set up, 1 = ready, -1 = set-up failed
+    void* scratch_ptr = nullptr;
 };
 constexpr int MAX_DEVICES = 64;
 static DeviceState g_devices[MAX_DEVICES];
@@ -102,6 +109,12 @@ static int device_state(DeviceState** out) {
                     (void)hipGetLastError();
                     ok = -1;
                 }
+            void* ptr = nullptr;
+            if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) {
+                (void)hipGetLastError();
+                ok = -1;
+            }
+            d.scratch_ptr = ptr;
             d.ready.store(ok, std::memory_order_release);
         }
     }
@@ -1004,6 +1017,7 @@ const char* phx_status_string(int status) {
         case PHX_ERR_NOT_SUPPORTED: return "not supported";
         case PHX_ERR_WORKSPACE: return "workspace too small";
         case PHX_ERR_RUNTIME: return "HIP runtime error";
+        case PHX_ERR_SCRATCH_LIMIT: return "request exceeds the built-in scratch buffer of the no-allocation entry point";
     }
     return "unknown status";
 }
@@ -1146,6 +1160,15 @@ int phx_qconv2d_fwd(const phx_qconv_desc* desc, phx_stream_t stream, const void*
     }
     if (p.nhwc) cl.y_out(p, y_planes, y, st);
     return PHX_OK;
+}
+
+int phx_qconv2d_fwd_noalloc(const phx_qconv_desc* desc, phx_stream_t stream, const void* x, const void* w,
+                            const void* bias_or_null, void* y) {
+    DeviceState* dev = nullptr;
+    if (const int init_rc = device_state(&dev)) return init_rc;
+    if (phx_qconv2d_workspace_bytes(desc, PHX_PASS_FWD) > (size_t)PHX_NOALLOC_SCRATCH_BYTES) return PHX_ERR_SCRATCH_LIMIT;
+    // the packed filters (and whatever else the forward pass stages) go to this device's copy of the scratch array
+    return phx_qconv2d_fwd(desc, stream, x, w, bias_or_null, y, dev->scratch_ptr, PHX_NOALLOC_SCRATCH_BYTES);
 }
 
 int phx_qconv2d_bwd_data(const phx_qconv_desc* desc, phx_stream_t stream, const void* grad, const void* w, void* dx,
