@@ -6,7 +6,8 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "libphx_qconv.so")
+# (PHX_QCONV_LIB: a developer's alternative build of the same library, e.g. one with in-kernel phase timing)
+LIB_PATH = os.environ.get("PHX_QCONV_LIB") or os.path.join(_HERE, "lib", "libphx_qconv.so")
 
 PHX_OK = 0
 PHX_ERR_INVALID_ARGUMENT, PHX_ERR_NOT_SUPPORTED, PHX_ERR_WORKSPACE, PHX_ERR_RUNTIME, PHX_ERR_SCRATCH_LIMIT = 1, 2, 3, 4, 5

@@ -42,6 +42,12 @@ int launch_fwd_f16(const FwdVariant& v, const ConvArgs& a, hipStream_t st);
 int launch_fwd_f16_lds8(const FwdVariant& v, const ConvArgs& a, hipStream_t st);  // 8-product, filters through LDS
 int launch_pack_filters_f16(const FwdVariant& v, const PackArgs& a, int blocks, hipStream_t st);
 
+// pointwise fp16-MFMA kernels with raw operand copies (phx_kernels_pw16.h); WCO = 32-channel sub-tiles per workgroup
+struct PwxArgs;
+int launch_pwx_f16(int WCO, const PwxArgs& a, int blocks, hipStream_t st);
+size_t pwx_packed_bytes(int WCO, int co_tiles, int nsteps);
+int launch_pack_filters_pwx(int map, int WCO, int nsteps, const PackArgs& a, hipStream_t st);
+
 int launch_wgrad_f32(bool half_storage, bool vec, int mode, const WgradArgs& a, dim3 grid, size_t lds_bytes,
                      hipStream_t st);  // vec: windows staged as groups of 4 positions
 // fp16-MFMA filter gradient: channel tile 32*MT x 32*NT, TPW taps per workgroup (1 or 3), stride SW along W (1 or 2)

@@ -12,6 +12,7 @@
 #include <vector>
 
 #include "phx_launch.h"
+#include "phx_kernels_pw16.h"
 
 // Scratch memory of phx_qconv2d_fwd_noalloc: a device-resident array of the code object (every GPU the library
 // runs on holds its own copy until the process ends).  In host code this name is only a handle for
@@ -90,6 +91,7 @@ bool register_big_lds_kernel(const void* fn) {
 // sit in a stream capture) and the device address of the built-in scratch array.
 struct DeviceState {
     std::atomic<int> ready{0};  // 0 = not set up, 1 = ready, -1 = set-up failed
+    int cu_count = 256;         // compute units (persistent kernels size their grids by it)
     void* scratch_ptr = nullptr;
 };
 constexpr int MAX_DEVICES = 64;
@@ -109,6 +111,9 @@ static int device_state(DeviceState** out) {
                     (void)hipGetLastError();
                     ok = -1;
                 }
+            int cus = 0;
+            if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && cus > 0) d.cu_count = cus;
+            else (void)hipGetLastError();
             void* ptr = nullptr;
             if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) {
                 (void)hipGetLastError();
@@ -289,6 +294,7 @@ struct Corr {
     // input gradient: tap (u, v) of the correlation is filter tap (khm - u*khs, kwm - v*kws); the plain mirrored
     // filter has khm = Kh-1, khs = 1
     int khm, khs, kwm, kws;
+    int ncomp;  // components of the input present in memory: 4, or 1 for the forward pass on a real-valued input
 };
 
 static Corr corr_forward(const Problem& p) {
@@ -296,6 +302,7 @@ static Corr corr_forward(const Problem& p) {
     if (p.kh == 1 && p.kw == 1 && p.sh == 1 && p.sw == 1 && !p.pt && !p.pl && !p.pb && !p.pr) {
         c.Win = p.h * p.w; c.Hin = 1; c.Wout = p.ho * p.wo; c.Hout = 1;  // pointwise: one long row per image
     }
+    c.ncomp = p.real_input ? 1 : 4;
     return c;
 }
 
@@ -305,6 +312,7 @@ static Corr corr_dgrad(const Problem& p) {
     if (p.kh == 1 && p.kw == 1 && p.sh == 1 && p.sw == 1 && !p.pt && !p.pl && !p.pb && !p.pr) {
         c.Win = p.ho * p.wo; c.Hin = 1; c.Wout = p.h * p.w; c.Hout = 1;
     }
+    c.ncomp = 4;
     return c;
 }
 
@@ -322,6 +330,8 @@ struct FwdPlan {
     size_t lds_bytes, wpk_bytes;
     int wgs;
     int tall;                // flat tiling (row distance of the images in the tall image), 0 = rectangular tiles
+    int pwx;                 // pointwise kernel with raw operand copies (phx_kernels_pw16.h): its WCO, 0 = not that kernel
+    int pwx_steps;           // ... its K steps of 16 channels
 };
 
 
@@ -490,7 +500,32 @@ static Corr virtual_pointwise(const Corr& c, bool f16mfma, int& pw) {
 // 16<->64-channel layers of a ResNet 37-75 against 64-112).  The 8-product mode means "prefer speed"
 // (src/backend/backend.hpp:36-66), so those problems run on the 16-product kernel; PHX_TUNE_PW8 keeps the
 // factorized one (tests exercise it).
+// Pointwise correlations on fp16 matrix cores whose planes have an even number (>= 8) of pixels run on the kernel
+// with raw operand copies, in 16-product form whatever the mode asks for (the 8-product mode means "prefer speed",
+// src/backend/backend.hpp:36-66, and this is the fastest pointwise kernel there is); PHX_TUNE_NOPWX keeps them on
+// the staged-window kernels.
+static bool pwx_applies(const Corr& c, bool f16mfma) {
+    return f16mfma && c.Kh * c.Kw == 1 && c.uh == 1 && c.uw == 1 && c.sh == 1 && c.sw == 1 && c.Hin == 1 && c.Hout == 1 &&
+           c.pt == 0 && c.pl == 0 && c.Win == c.Wout && c.Win % 2 == 0 && c.Win >= 8 && c.ncomp == 4 &&
+           (long)c.N * ((c.Win + 7) / 8) < (1L << 30) && !tune().nopwx && !tune().pw8;
+}
+
 static bool plan_corr_uncached(const Corr& creal, int mode, bool f16mfma, Corr& c, FwdPlan& pl, int& pw) {
+    pl.pwx = 0; pl.pwx_steps = 0;
+    if (pwx_applies(creal, f16mfma)) {
+        pw = 0;
+        c = creal;
+        pl = FwdPlan{};
+        pl.kmode = 16;
+        pl.pwx = creal.Cout > 64 ? 4 : creal.Cout > 32 ? 2 : 1;
+        if (tune().tile_wco == 1 || tune().tile_wco == 2 || tune().tile_wco == 4) pl.pwx = tune().tile_wco;
+        pl.WCO = pl.pwx; pl.NTW = 2; pl.CK = F16_CK;
+        pl.co_tiles = cdiv(creal.Cout, 32 * pl.pwx);
+        pl.pwx_steps = cdiv(creal.Cin, 16);
+        pl.nchunks = pl.pwx_steps;
+        pl.wpk_bytes = pwx_packed_bytes(pl.pwx, pl.co_tiles, pl.pwx_steps);
+        return true;
+    }
     c = virtual_pointwise(creal, f16mfma, pw);
     if (pw) {
         pl.kmode = (mode == 8 && !tune().pw8) ? 16 : mode;
@@ -515,11 +550,11 @@ struct CorrPlan {
 
 static bool plan_corr(const Corr& creal, int mode, bool f16mfma, Corr& c, FwdPlan& pl, int& pw) {
     static std::unordered_map<PlanKey, CorrPlan, PlanKeyHash> memo;
-    static_assert(sizeof(Corr) == 21 * sizeof(int), "Corr is hashed as raw ints: no padding allowed");
+    static_assert(sizeof(Corr) == 22 * sizeof(int), "Corr is hashed as raw ints: no padding allowed");
     PlanKey key{};
     std::memcpy(key.v, &creal, sizeof(Corr));
-    key.v[21] = mode;
-    key.v[22] = f16mfma;
+    key.v[22] = mode;
+    key.v[23] = f16mfma;
     std::lock_guard<std::mutex> lock(g_plan_mutex);
     static unsigned generation = 0;
     if (generation != g_plan_generation) { memo.clear(); generation = g_plan_generation; }
@@ -533,6 +568,42 @@ static bool plan_corr(const Corr& creal, int mode, bool f16mfma, Corr& c, FwdPla
     return it->second.ok;
 }
 
+static int run_pwx(const Problem& p, const Corr& c, const FwdPlan& pl, int map, hipStream_t st, const void* in, const void* w,
+                   const void* bias, void* out, void* ws) {
+    DeviceState* dev = nullptr;
+    if (const int rc = device_state(&dev)) return rc;
+    PackArgs pa{};
+    pa.w = w; pa.out = ws;
+    pa.wcs = p.fs.wcs; pa.so = p.fs.so; pa.si = p.fs.si; pa.skh = p.fs.skh; pa.skw = p.fs.skw;
+    pa.Co = p.co; pa.Ci = p.ci; pa.Kh = 1; pa.Kw = 1;
+    pa.khm = c.khm; pa.khs = c.khs; pa.kwm = c.kwm; pa.kws = c.kws;
+    pa.rows = c.Cout; pa.red = c.Cin; pa.row_tiles = pl.co_tiles; pa.nchunks = pl.pwx_steps;
+    if (launch_pack_filters_pwx(map, pl.pwx, pl.pwx_steps, pa, st) != 0) return PHX_ERR_NOT_SUPPORTED;
+    const int cin_mem = (map == MAP_FWD) ? p.ci_mem : p.co_mem, cout_mem = (map == MAP_FWD) ? p.co_mem : p.ci_mem;
+    PwxArgs a{};
+    a.in = static_cast<const _Float16*>(in); a.in_cs = (long)c.N * cin_mem * c.Win;
+    a.wpk = static_cast<const f16x8*>(ws); a.bias = static_cast<const _Float16*>(bias);
+    a.out = static_cast<_Float16*>(out); a.out_cs = (long)c.N * cout_mem * c.Wout;
+    a.N = c.N; a.Cin = c.Cin; a.CinS = cin_mem; a.Cout = c.Cout; a.CoutS = cout_mem; a.HW = c.Win;
+    a.GI = cdiv(c.Win, 8); a.TGp = c.N * a.GI;
+    a.co_tiles = pl.co_tiles; a.nsteps = pl.pwx_steps;
+    const int groups_per_tile = 8 * (4 / pl.pwx);
+    a.items = cdiv(a.TGp, groups_per_tile) * pl.co_tiles;
+    const int blocks = std::min(a.items, 2 * dev->cu_count);  // persistent workgroups, two per CU
+    int rc;
+    {
+        KernelTimer timer(st);
+        rc = launch_pwx_f16(pl.pwx, a, blocks, st);
+    }
+    if (rc != 0) return PHX_ERR_NOT_SUPPORTED;
+    PHX_HIP(hipGetLastError());
+    snprintf(g_name_buf, sizeof(g_name_buf), "%sqconv_%s_f16mfmapwx_p16_f16_wco%d_px%d_k%d_wgs%d", g_name_prefix,
+             map == MAP_FWD ? "fwd" : "dgrad", pl.pwx, 64 * (4 / pl.pwx), pl.pwx_steps, blocks);
+    g_last_kernel = g_name_buf;
+    say(p, map == MAP_FWD ? "forward" : "input gradient");
+    return PHX_OK;
+}
+
 static int run_corr(const Problem& p, const Corr& creal, int map, hipStream_t st, const void* in, const void* w,
                     const void* bias, void* out, void* ws, size_t ws_bytes) {
     const bool f16 = use_f16_mfma(p, map == MAP_FWD ? PHX_PASS_FWD : PHX_PASS_BWD_DATA);
@@ -541,6 +612,7 @@ static int run_corr(const Problem& p, const Corr& creal, int map, hipStream_t st
     FwdPlan pl;
     if (!plan_corr(creal, p.mode, f16, c, pl, pw)) return PHX_ERR_NOT_SUPPORTED;
     if (ws_bytes < pl.wpk_bytes || !ws) return PHX_ERR_WORKSPACE;
+    if (pl.pwx) return run_pwx(p, creal, pl, map, st, in, w, bias, out, ws);
 
     FwdVariant v;
     v.half_storage = p.dtype == PHX_F16; v.f16_mfma = f16; v.mode = pl.kmode; v.map = map;
@@ -829,6 +901,7 @@ static Corr phase_corr(const Problem& p, const PhaseAxis& ah, const PhaseAxis& a
     if (ah.taps == 1 && aw.taps == 1 && !ah.pad && !aw.pad && ah.size == p.ho && aw.size == p.wo) {
         c.Win = p.ho * p.wo; c.Hin = 1; c.Wout = c.Win; c.Hout = 1;
     }
+    c.ncomp = 4;
     return c;
 }
 

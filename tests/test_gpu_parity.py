@@ -301,11 +301,20 @@ def test_factorized_filter_gradient_on_fp16_matrix_cores(case, tune_env):
     assert_close(dw16.cpu().numpy(), want_dw, dtype, "16-product wgrad " + name)
 
 
-@pytest.mark.parametrize("case", [c for c in FP16_CASES if c[0] in ("pw_64", "pw_ragged", "pw_7x7img", "pw_256_14", "co_gt_128")],
-                         ids=lambda c: c[0])
-def test_factorized_pointwise_on_fp16_matrix_cores(case, tune_env):
-    """In 8-product mode pointwise fp16 problems run on the 16-product kernel by default (two workgroups per CU
-    beat the factorized kernel there); PHX_TUNE_PW8 selects the factorized kernel, same tolerance."""
+PW_CASES = [c for c in FP16_CASES if c[0] in ("pw_64", "pw_ragged", "pw_7x7img", "pw_256_14", "pw_128_28", "co_gt_128")] + [
+    ("pw_c40_10x10", 3, 40, 24, 10, 10, 1, 1, 1, 1, "VALID"),    # channels not multiples of 16 / 32, plane of 100 = 12.5 groups
+    ("pw_c200_2x4", 5, 72, 200, 2, 4, 1, 1, 1, 1, "VALID"),      # one 8-pixel group per image, two channel tiles
+    ("pw_c16_6x6_n33", 33, 16, 16, 6, 6, 1, 1, 1, 1, "VALID"),   # 32 output channels at most: one sub-tile per workgroup
+    ("pw_c64_n1_12x12", 1, 48, 64, 12, 12, 1, 1, 1, 1, "VALID"),
+]
+
+
+@pytest.mark.parametrize("case", PW_CASES, ids=lambda c: c[0])
+def test_pointwise_kernels_on_fp16_matrix_cores(case, tune_env):
+    """Pointwise fp16 problems have three kernels.  Planes with an even number (>= 8) of pixels run on the kernel
+    with raw operand copies ("pwx", 16-product form in either mode); PHX_TUNE_NOPWX sends them to the staged-window
+    kernel the other planes use ("ldspw", in 8-product mode the 16-product kernel by default, which beats the
+    factorized one there); PHX_TUNE_PW8 selects the factorized kernel.  All to the same tolerance."""
     name, n, ci, co, h, w, kh, kw, stride, dilation, padding = case
     dtype = torch.float16
     g, x, wt, b, gr = make_inputs(name_seed(name) + 4, n, ci, co, h, w, kh, kw, stride, dilation, padding, dtype, 0.5)
@@ -315,9 +324,10 @@ def test_factorized_pointwise_on_fp16_matrix_cores(case, tune_env):
     x64, w64, b64, g64 = (a.astype(np.float64) for a in (x, wt, b, gr))
     want_y = oracle.conv2d_fwd(g, x64, w64, b64, "hamilton")
     _, want_dx = oracle.conv2d_bwd(g, x64, w64, g64, "hamilton")
-    for forced, tag in ((False, "ldspw_p16"), (True, "ldspw_p8")):
-        if forced:
-            tune_env(PHX_TUNE_PW8="1")
+    raw_copies = (h * w) % 2 == 0 and h * w >= 8
+    for env, tag in (({}, "pwx_p16" if raw_copies else "ldspw_p16"), ({"PHX_TUNE_NOPWX": "1"}, "ldspw_p16"),
+                     ({"PHX_TUNE_NOPWX": None, "PHX_TUNE_PW8": "1"}, "ldspw_p8")):
+        tune_env(**env)
         y = phx.conv2d_fwd(xd, wd, bd, desc)
         assert tag in capi.last_kernel_name(), capi.last_kernel_name()
         _, dx = phx.conv2d_bwd(xd, wd, gd, desc)
