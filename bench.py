@@ -79,6 +79,7 @@ def parse():
     ap.add_argument("--batch", type=int, default=64, help="images per step of the ResNet workload")
     ap.add_argument("--torch-bn", action="store_true",
                     help="ResNet workload: torch.nn.BatchNorm2d + ReLU (MIOpen) instead of the library's batch-norm kernels")
+    ap.add_argument("--no-graph", action="store_true", help="ResNet workload: time the eager step only (no HIP graph replay)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch a plain 256 MiB device copy (untimed), the yardstick for HBM byte counters")
@@ -380,6 +381,50 @@ def resnet_flops(n):
     return total + 2.0 * 16 * n * 250 * 512
 
 
+def _graphed_step(step, eager_loss, args):
+    """The same step captured into a HIP graph (torch.cuda.graph) and replayed: the ~330 kernel launches of a step
+    then cost one graph launch.  The capture is trusted only if every one of three checked replays -- with eager
+    steps and synchronisations between them -- reproduces the eager loss exactly (the step is deterministic and
+    nothing it reads changes between steps); otherwise the eager timing stands."""
+    import torch
+    from phoenix_core_amd import capi
+    try:
+        capi.init()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(2):
+                step()  # sizes the scratch buffer of the capture stream, fills the plan cache
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            graph_loss = step()
+        losses = []
+        for _ in range(3):
+            graph_loss.fill_(float("nan"))
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            losses.append(float(graph_loss))
+            step()  # eager work of the program between the replays
+            torch.cuda.synchronize()
+        if any(v != eager_loss for v in losses):
+            return {"used": False, "note": "replays gave losses %s, the eager step %r" % (losses, eager_loss)}
+        for _ in range(max(args.warmup, 3)):
+            graph.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            graph.replay()
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) / args.steps * 1e3
+        return {"used": True, "ms_per_step": ms, "replays_checked": len(losses),
+                "note": "every checked replay reproduced the eager loss exactly"}
+    except Exception as exc:  # capture is an optimisation: any failure leaves the eager figure standing
+        return {"used": False, "note": "capture or replay failed: %s" % (str(exc)[:200],)}
+
+
 def run_resnet(mode, policy, args):
     import torch
     import phoenix_core_amd as phx
@@ -396,23 +441,28 @@ def run_resnet(mode, policy, args):
         model.zero_grad(set_to_none=True)
         loss = torch.nn.functional.cross_entropy(model(images).float(), labels)
         loss.backward()
-        last["loss"] = loss
+        return loss.detach()
 
-    t = _Timed(step, 3 * 54, args.steps, max(args.warmup, 3))
+    t = _Timed(lambda: last.__setitem__("loss", step()), 3 * 54, args.steps, max(args.warmup, 3))
+    eager_ms, eager_loss = t.ms_per_step, float(last["loss"])
+    graph = _graphed_step(step, eager_loss, args) if not args.no_graph else {"used": False, "note": "--no-graph"}
+    ms_per_step = graph["ms_per_step"] if graph["used"] else eager_ms
     fwd_flops = resnet_flops(n)
     out = {
         "workload": "%s: quaternion ResNet-50 forward+backward (no optimizer step, as the metric names), "
                     "N=%d real images (4N=%d quaternion rows after the real-input stem), 224x224, 53 quaternion convs + "
                     "quaternion dense head; batch-norm (with the ReLU behind it) by %s, residual add, "
-                    "pooling and cross-entropy by PyTorch"
+                    "pooling and cross-entropy by PyTorch; the step %s"
                     % (RESNET, n, 4 * n, "torch.nn.BatchNorm2d (MIOpen)" if args.torch_bn else
-                       "the library's streaming kernels (include/phx_bn.h)"),
+                       "the library's streaming kernels (include/phx_bn.h)",
+                       "is captured once into a HIP graph and replayed" if graph["used"] else "runs eagerly"),
         "product_mode": mode, "fp16_policy": policy, "batch_norm": "torch" if args.torch_bn else "library", "dtype": "f16",
-        "value": n / (t.ms_per_step * 1e-3), "unit": "img/s", "images_per_s": n / (t.ms_per_step * 1e-3),
-        "ms_per_step": t.ms_per_step,
-        "real_equiv_tflops": 3 * fwd_flops / (t.ms_per_step * 1e-3) / 1e12,
-        "frac_of_mfma_peak": 3 * fwd_flops / (t.ms_per_step * 1e-3) / 1e12 / PEAK_TFLOPS["f16"],
-        "quaternion_kernel_ms_per_step": sum(t.kernel_ms), "loss": float(last["loss"].detach()),
+        "value": n / (ms_per_step * 1e-3), "unit": "img/s", "images_per_s": n / (ms_per_step * 1e-3),
+        "ms_per_step": ms_per_step, "ms_per_step_eager": eager_ms, "images_per_s_eager": n / (eager_ms * 1e-3),
+        "hip_graph": graph,
+        "real_equiv_tflops": 3 * fwd_flops / (ms_per_step * 1e-3) / 1e12,
+        "frac_of_mfma_peak": 3 * fwd_flops / (ms_per_step * 1e-3) / 1e12 / PEAK_TFLOPS["f16"],
+        "quaternion_kernel_ms_per_step": sum(t.kernel_ms), "loss": eager_loss,
     }
     del model, images, labels, last
     torch.cuda.empty_cache()

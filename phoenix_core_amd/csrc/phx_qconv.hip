@@ -673,7 +673,7 @@ struct WgPlan {
     int TPW, NB, TH, TW, KP, KPp, HPp, HPx, HTH, HTWmax;
     int tiles_n, tiles_h, tiles_w, co_tiles, ci_tiles, CoP, CiP, groups_per_row, Z;
     int MT, NT;  // fp16 kernel: 32*MT x 32*NT channel tile
-    int kmode;   // fp16 kernel: product formulation the kernel runs in (see wgrad_f16_formulation)
+    int kmode;   // product formulation the kernel runs in (see wgrad_f16_formulation, wgrad_f32_formulation)
     bool vec;    // fp32 kernel: windows staged as groups of 4 positions
     int SW, cpr, nchunks, ntiles;  // fp16 kernel: stride along W, 8-pixel chunks per output row / in total, pixel tiles
     size_t lds_bytes, partial_bytes;
@@ -691,9 +691,21 @@ static void finish_wgrad_plan(const Problem& p, int CoT, int CiT, WgPlan& best) 
     best.partial_bytes = (size_t)best.Z * p.kh * p.kw * 4 * best.CoP * best.CiP * sizeof(float);
 }
 
+// The fp32-MFMA filter gradient in 8-product mode gives every tap a workgroup of its own (its 8 accumulator sets
+// leave no room for more), so the taps of a filter row each stage the same gradient tile; the 16-product kernel
+// shares it between three taps.  On small images, where a workgroup's tiles are short and staging weighs most, that
+// is worth more than the halved multiplications (measured on fp16 tensors under the backward32 policy, 3x3:
+// 128->128 @ 28x28 5.2 against 5.9 ms, 256->256 @ 14x14 6.8 against 9.8 ms; at 56x56 and for single-tap filters
+// the factorized kernel stays ahead).  The 8-product mode means "prefer speed" (src/backend/backend.hpp:36-66), so
+// those problems run the 16-product kernel; PHX_TUNE_WG8 keeps the factorized one.
+static int wgrad_f32_formulation(const Problem& p) {
+    return (p.mode == 8 && p.kw % 3 == 0 && p.wo <= 28 && !tune().wg8) ? 16 : p.mode;
+}
+
 // fp32-MFMA kernel: 64x64 channel tiles, pixel tile and input window of at most 32 positions
 static bool plan_wgrad_f32(const Problem& p, WgPlan& best) {
-    const int TPW = (p.mode == 16) ? 3 : 1;
+    best.kmode = wgrad_f32_formulation(p);
+    const int TPW = (best.kmode == 16) ? 3 : 1;
     const int nkw = std::min(TPW, p.kw);
     double best_score = -1.0;
     const int budget = LDS_FLOATS_MAX / (4 * 64);  // KPp + HPp (+ offsets) per staged channel
@@ -833,7 +845,7 @@ static int run_wgrad(const Problem& p, hipStream_t st, const void* x, const void
             if (launch_wgrad_f16(pl.kmode, pl.MT, pl.NT, pl.TPW, pl.SW, a, nblocks, pl.lds_bytes, st) != 0)
                 return PHX_ERR_RUNTIME;
         } else {
-            launch_wgrad_f32(half_storage, pl.vec, p.mode, a, dim3(nblocks), pl.lds_bytes, st);
+            launch_wgrad_f32(half_storage, pl.vec, pl.kmode, a, dim3(nblocks), pl.lds_bytes, st);
         }
     }
     PHX_HIP(hipGetLastError());
@@ -849,7 +861,7 @@ static int run_wgrad(const Problem& p, hipStream_t st, const void* x, const void
         snprintf(g_name_buf, sizeof(g_name_buf), "%sqconv_wgrad_f16mfma_p%d_f16_ch%dx%d_taps%d_sw%d_z%d", g_name_prefix, pl.kmode, 32 * pl.MT,
                  32 * pl.NT, pl.TPW, pl.SW, pl.Z);
     else
-        snprintf(g_name_buf, sizeof(g_name_buf), "%sqconv_wgrad_f32mfma%s_p%d_%s_tile%dx%dx%d_z%d", g_name_prefix, pl.vec ? "v" : "", p.mode,
+        snprintf(g_name_buf, sizeof(g_name_buf), "%sqconv_wgrad_f32mfma%s_p%d_%s_tile%dx%dx%d_z%d", g_name_prefix, pl.vec ? "v" : "", pl.kmode,
                  p.dtype == PHX_F32 ? "f32" : "f16", pl.NB, pl.TH, pl.TW, pl.Z);
     g_last_kernel = g_name_buf;
     say(p, "filter gradient");
