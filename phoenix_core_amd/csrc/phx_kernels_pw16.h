@@ -44,6 +44,7 @@ struct PwxArgs {
     int co_tiles;           // ceil(Cout / (32 * WCO))
     int nsteps;             // ceil(Cin / 16)
     int items;              // pixel tiles * co_tiles
+    int NP;                 // channels-last kernel: pixels in all, N * HW
 };
 
 template <int WCO>
@@ -257,6 +258,178 @@ __global__ void __launch_bounds__(WG_THREADS, 2) qconv_pwx_f16_kernel(const PwxA
                t_clk1 - t_clk0, t_wall1 - t_wall0, t_wall0 % 1000000);
 #endif
     PHX_PHASES_REPORT("pwx: copy wait / barrier / drain before stores / reads+products / stores", 5)
+}
+
+// ---------------------------------------------------------------------------------------------
+// The same pipeline for CHANNELS-LAST tensors, in[4][N][HW][CinS] -> out[4][N][HW][CoutS] (DataFormat::NHWC of the
+// reference, src/backend/tensor.hpp:17-31).  There the 8 consecutive channels of a pixel that the MFMA operand
+// wants ARE 16 contiguous bytes, so nothing is transposed anywhere: a copy lane moves (pixel, channel half) of
+// the K step to LDS, the B operand is one 16-byte LDS read, and the images need no telling apart (all N * HW
+// pixels form one uniformly strided array).  The filters are the A operand here (rows = output channels), so a
+// lane receives 4 consecutive output channels per register group at its pixel; one v_permlane32_swap per dword
+// between the two lane halves turns its four groups into 16 consecutive channels: two 16-byte stores per tile.
+// LDS slot of (pixel p of a 32-pixel block, half h): 2p + (h ^ (p / 8) % 2) -- neighbouring lanes still copy the two
+// halves of one pixel (32 contiguous bytes), and the 16 lanes the LDS serves together read 16 different bank groups.
+// Requirements (host): channel counts and channel strides multiples of 8.
+// ---------------------------------------------------------------------------------------------
+template <int WCO>
+__global__ void __launch_bounds__(WG_THREADS, 2) qconv_pwx_nhwc_f16_kernel(const PwxArgs P) {
+    using S = PwxShape<WCO>;
+    constexpr int WPX = S::WPX, WV = S::WV, SV = S::SV, R = S::R, D = R - 1;
+    constexpr int PXT = 64 * WPX;     // pixels per workgroup tile
+    constexpr int BLK = 2 * WPX;      // 32-pixel blocks per tile (one copy instruction per component each)
+    extern __shared__ f16x8 lds16[];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wco = wave % WCO, wpx = wave / WCO;
+    const int j = lane & 31, kk = lane >> 5;
+    const int wg = xcd_remap(blockIdx.x, gridDim.x);
+
+    // ---- copy side
+    const int c_pxl = lane >> 1, c_half = (lane & 1) ^ ((c_pxl >> 3) & 1);
+    int p_item = wg, p_k = 0, p_ct = 0, p_px0 = 0;
+    auto locate_copy = [&](int item) {
+        const int tile = item / P.co_tiles;
+        p_ct = item - tile * P.co_tiles;
+        p_px0 = item < P.items ? tile * PXT : P.NP;  // (past the last item: every pixel out of range)
+    };
+    auto issue_slot = [&](int buf, int slot) {
+        f16x8* sb = lds16 + buf * SV;
+        if (slot < S::NWI) {
+            const int t = wave + 4 * slot;
+            const f16x8* wsrc = P.wpk + ((long)p_ct * P.nsteps + p_k) * WV;
+            lds_dma_16(wsrc + t * 64 + lane, sb + t * 64);
+        } else {
+            const int t = wave + 4 * (slot - S::NWI);
+            const int p = t / BLK, b = t % BLK;
+            const int gp = p_px0 + b * 32 + c_pxl, ch = p_k * 16 + c_half * 8;
+            // channels past the tensor meet zero filters; they, and pixels past the last image, copy zeros
+            const _Float16* src = (gp < P.NP && ch < P.Cin) ? P.in + p * P.in_cs + (long)gp * P.CinS + ch : zero_ptr<_Float16>();
+            lds_dma_16(src, sb + WV + t * 64);
+        }
+        if (slot == S::NPS - 1 && ++p_k == P.nsteps) {
+            p_k = 0;
+            p_item += gridDim.x;
+            locate_copy(p_item);
+        }
+    };
+    auto issue = [&](int buf) {
+#pragma unroll
+        for (int slot = 0; slot < S::NPS; ++slot) issue_slot(buf, slot);
+    };
+
+    // ---- product side: lane (j, kk) is pixel j of the wave's two 32-pixel blocks m = 0, 1 and channels kk*8.. of a K step
+    int c_item = wg, c_k = 0, c_ct = 0, c_px0 = 0;
+    auto locate_out = [&](int item) {
+        const int tile = item / P.co_tiles;
+        c_ct = item - tile * P.co_tiles;
+        c_px0 = tile * PXT + wpx * 64 + j;
+    };
+    const int xslot = 2 * j + (kk ^ ((j >> 3) & 1));
+
+    f32x16 acc[4][2];
+    const int my_items = P.items > wg ? (P.items - wg + (int)gridDim.x - 1) / (int)gridDim.x : 0;
+    const int total_steps = my_items * P.nsteps;
+    locate_copy(p_item);
+    locate_out(c_item);
+#pragma unroll
+    for (int s = 0; s < D; ++s)
+        if (s < total_steps) issue(s);
+
+    auto products = [&](int buf, bool more, int nbuf, auto first_tag) {
+        constexpr bool FIRST = decltype(first_tag)::value;
+        const f16x8* wb = lds16 + buf * SV + (wco * 4) * 64 + lane;
+        const f16x8* xb = lds16 + buf * SV + WV + (wpx * 2) * 64 + xslot;
+        f16x8 w[4], nw[4], x[4][2];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) w[r] = wb[r * 64];
+#pragma unroll
+        for (int p = 0; p < 4; ++p)
+#pragma unroll
+            for (int m = 0; m < 2; ++m) x[p][m] = xb[(p * BLK + m) * 64];
+#pragma unroll
+        for (int r = 1; r < 4; ++r) nw[r] = neg8(w[r]);
+        nw[0] = w[0];
+        const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const f16x8 f = qneg(p, q) ? nw[p ^ q] : w[p ^ q];
+                acc[q][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(f, x[p][0], (FIRST && p == 0) ? zero : acc[q][0], 0, 0, 0);
+                acc[q][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(f, x[p][1], (FIRST && p == 0) ? zero : acc[q][1], 0, 0, 0);
+                constexpr int PAIRS = 16;
+                const int pair = p * 4 + q;
+                if (more) {
+#pragma unroll
+                    for (int slot = 0; slot < S::NPS; ++slot)
+                        if (pair == (slot * PAIRS) / S::NPS) {
+                            __builtin_amdgcn_sched_barrier(0);
+                            issue_slot(nbuf, slot);
+                            __builtin_amdgcn_sched_barrier(0);
+                        }
+                }
+            }
+        }
+    };
+
+    int covered = 0;  // (the waiting protocol of qconv_pwx_f16_kernel)
+    for (int gs = 0; gs < total_steps; ++gs) {
+        const int buf = gs % R;
+        if (covered > 0) --covered;
+        else if (D == 2 && gs + 1 < total_steps) __builtin_amdgcn_s_waitcnt(0x0F70 | S::NPS);
+        else wait_vmem_all();
+        __syncthreads();
+        const bool more = gs + D < total_steps;
+        const int nbuf = (gs + D) % R;
+        if (c_k == 0) products(buf, more, nbuf, std::true_type());
+        else products(buf, more, nbuf, std::false_type());
+        if (++c_k == P.nsteps) {
+            wait_vmem_all();
+            covered = D;
+            // register e of a tile: output channel 8*(e/4) + 4*kk + e%4 of the wave's 32, at this lane's pixel.  After
+            // the swaps the lower lane half holds channels 0..15 and the upper half 16..31, in order.
+            const int co = (c_ct * WCO + wco) * 32 + 16 * kk;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+#pragma unroll
+                for (int m = 0; m < 2; ++m) {
+                    unsigned int d[4][2];
+#pragma unroll
+                    for (int g = 0; g < 4; ++g)
+#pragma unroll
+                        for (int i = 0; i < 2; ++i) {
+                            float a = acc[q][m][4 * g + 2 * i], b = acc[q][m][4 * g + 2 * i + 1];
+                            if (P.bias) {
+                                const int cb = (c_ct * WCO + wco) * 32 + 8 * g + 4 * kk + 2 * i;
+                                a += cb < P.Cout ? (float)P.bias[q * P.CoutS + cb] : 0.f;
+                                b += cb + 1 < P.Cout ? (float)P.bias[q * P.CoutS + cb + 1] : 0.f;
+                            }
+                            f16x2 h;
+                            h[0] = (_Float16)a;
+                            h[1] = (_Float16)b;
+                            d[g][i] = __builtin_bit_cast(unsigned int, h);
+                        }
+                    u32x4 v0, v1;
+#pragma unroll
+                    for (int i = 0; i < 2; ++i) {
+                        const auto s02 = __builtin_amdgcn_permlane32_swap(d[0][i], d[2][i], false, false);
+                        const auto s13 = __builtin_amdgcn_permlane32_swap(d[1][i], d[3][i], false, false);
+                        v0[i] = s02[0]; v0[2 + i] = s02[1];
+                        v1[i] = s13[0]; v1[2 + i] = s13[1];
+                    }
+                    const int gp = c_px0 + 32 * m;
+                    _Float16* dst = P.out + q * P.out_cs + (long)gp * P.CoutS + co;
+                    if (gp < P.NP && co < P.Cout) *reinterpret_cast<u32x4_a2*>(dst) = v0;
+                    if (gp < P.NP && co + 8 < P.Cout) *reinterpret_cast<u32x4_a2*>(dst + 8) = v1;
+                }
+            }
+            c_k = 0;
+            c_item += gridDim.x;
+            locate_out(c_item);
+        }
+    }
 }
 
 // Filter packing for the kernel above: one 16-byte vector per (output-channel tile of 32*WCO, K step, sub-tile,

@@ -19,6 +19,21 @@ int launch_pwx_f16(int WCO, const PwxArgs& a, int blocks, hipStream_t st) {
     return -1;
 }
 
+template <int WCO>
+static int launch_pwx_nhwc_one(const PwxArgs& a, int blocks, hipStream_t st) {
+    constexpr auto kernel = qconv_pwx_nhwc_f16_kernel<WCO>;
+    if (!BigLds<kernel>::registered) return -1;
+    hipLaunchKernelGGL(kernel, dim3(blocks), dim3(WG_THREADS), PwxShape<WCO>::lds_bytes, st, a);
+    return 0;
+}
+
+int launch_pwx_nhwc_f16(int WCO, const PwxArgs& a, int blocks, hipStream_t st) {
+    if (WCO == 4) return launch_pwx_nhwc_one<4>(a, blocks, st);
+    if (WCO == 2) return launch_pwx_nhwc_one<2>(a, blocks, st);
+    if (WCO == 1) return launch_pwx_nhwc_one<1>(a, blocks, st);
+    return -1;
+}
+
 size_t pwx_packed_bytes(int WCO, int co_tiles, int nsteps) { return (size_t)co_tiles * nsteps * WCO * 4 * 64 * 16; }
 
 int launch_pack_filters_pwx(int map, int WCO, int nsteps, const PackArgs& a, hipStream_t st) {

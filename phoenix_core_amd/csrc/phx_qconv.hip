@@ -504,6 +504,7 @@ static Corr virtual_pointwise(const Corr& c, bool f16mfma, int& pw) {
 // with raw operand copies, in 16-product form whatever the mode asks for (the 8-product mode means "prefer speed",
 // src/backend/backend.hpp:36-66, and this is the fastest pointwise kernel there is); PHX_TUNE_NOPWX keeps them on
 // the staged-window kernels.
+static int pwx_wco(int cout);
 static bool pwx_applies(const Corr& c, bool f16mfma) {
     return f16mfma && c.Kh * c.Kw == 1 && c.uh == 1 && c.uw == 1 && c.sh == 1 && c.sw == 1 && c.Hin == 1 && c.Hout == 1 &&
            c.pt == 0 && c.pl == 0 && c.Win == c.Wout && c.Win % 2 == 0 && c.Win >= 8 && c.ncomp == 4 &&
@@ -517,8 +518,7 @@ static bool plan_corr_uncached(const Corr& creal, int mode, bool f16mfma, Corr& 
         c = creal;
         pl = FwdPlan{};
         pl.kmode = 16;
-        pl.pwx = creal.Cout > 64 ? 4 : creal.Cout > 32 ? 2 : 1;
-        if (tune().tile_wco == 1 || tune().tile_wco == 2 || tune().tile_wco == 4) pl.pwx = tune().tile_wco;
+        pl.pwx = pwx_wco(creal.Cout);
         pl.WCO = pl.pwx; pl.NTW = 2; pl.CK = F16_CK;
         pl.co_tiles = cdiv(creal.Cout, 32 * pl.pwx);
         pl.pwx_steps = cdiv(creal.Cin, 16);
@@ -601,6 +601,63 @@ static int run_pwx(const Problem& p, const Corr& c, const FwdPlan& pl, int map, 
              map == MAP_FWD ? "fwd" : "dgrad", pl.pwx, 64 * (4 / pl.pwx), pl.pwx_steps, blocks);
     g_last_kernel = g_name_buf;
     say(p, map == MAP_FWD ? "forward" : "input gradient");
+    return PHX_OK;
+}
+
+// Channels-last pointwise convolutions on fp16 matrix cores run natively on the channels-last form of that kernel
+// (forward and input gradient; the filter gradient and every other channels-last call go through the transposes
+// of ChannelsLast below).
+static int pwx_wco(int cout) {
+    if (tune().tile_wco == 1 || tune().tile_wco == 2 || tune().tile_wco == 4) return tune().tile_wco;
+    return cout > 64 ? 4 : cout > 32 ? 2 : 1;
+}
+
+static bool nhwc_native(const Problem& p, int pass) {
+    return p.nhwc && (pass == PHX_PASS_FWD || pass == PHX_PASS_BWD_DATA) && is_pointwise_unit(p) && !is_empty(p) &&
+           use_f16_mfma(p, pass) && !p.real_input && p.groups == 1 && p.ci % 8 == 0 && p.co % 8 == 0 &&
+           (long)p.n * p.h * p.w < (1L << 30) && !tune().nopwx;
+}
+
+static size_t nhwc_native_workspace(const Problem& p, int pass) {
+    const int cin = pass == PHX_PASS_FWD ? p.ci : p.co, cout = pass == PHX_PASS_FWD ? p.co : p.ci;
+    const int wco = pwx_wco(cout);
+    return align_up(pwx_packed_bytes(wco, cdiv(cout, 32 * wco), cdiv(cin, 16)), 256);
+}
+
+static int run_pwx_nhwc(const Problem& p, int map, hipStream_t st, const void* in, const void* w, const void* bias, void* out,
+                        void* ws, size_t ws_bytes) {
+    DeviceState* dev = nullptr;
+    if (const int rc = device_state(&dev)) return rc;
+    if (!in || !w || !out) return PHX_ERR_INVALID_ARGUMENT;
+    const int cin = map == MAP_FWD ? p.ci : p.co, cout = map == MAP_FWD ? p.co : p.ci;
+    const int wco = pwx_wco(cout), co_tiles = cdiv(cout, 32 * wco), nsteps = cdiv(cin, 16);
+    if (ws_bytes < pwx_packed_bytes(wco, co_tiles, nsteps) || !ws) return PHX_ERR_WORKSPACE;
+    PackArgs pa{};
+    pa.w = w; pa.out = ws;
+    pa.wcs = p.fs.wcs; pa.so = p.fs.so; pa.si = p.fs.si; pa.skh = p.fs.skh; pa.skw = p.fs.skw;
+    pa.Co = p.co; pa.Ci = p.ci; pa.Kh = 1; pa.Kw = 1; pa.khm = 0; pa.khs = 1; pa.kwm = 0; pa.kws = 1;
+    pa.rows = cout; pa.red = cin; pa.row_tiles = co_tiles; pa.nchunks = nsteps;
+    if (launch_pack_filters_pwx(map, wco, nsteps, pa, st) != 0) return PHX_ERR_NOT_SUPPORTED;
+    PwxArgs a{};
+    const long np = (long)p.n * p.h * p.w;
+    a.in = static_cast<const _Float16*>(in); a.in_cs = np * cin;
+    a.wpk = static_cast<const f16x8*>(ws); a.bias = static_cast<const _Float16*>(bias);
+    a.out = static_cast<_Float16*>(out); a.out_cs = np * cout;
+    a.N = p.n; a.Cin = cin; a.CinS = cin; a.Cout = cout; a.CoutS = cout; a.HW = p.h * p.w; a.NP = (int)np;
+    a.co_tiles = co_tiles; a.nsteps = nsteps;
+    a.items = cdiv((int)np, 64 * (4 / wco)) * co_tiles;
+    const int blocks = std::min(a.items, 2 * dev->cu_count);
+    int rc;
+    {
+        KernelTimer timer(st);
+        rc = launch_pwx_nhwc_f16(wco, a, blocks, st);
+    }
+    if (rc != 0) return PHX_ERR_NOT_SUPPORTED;
+    PHX_HIP(hipGetLastError());
+    snprintf(g_name_buf, sizeof(g_name_buf), "qconv_%s_f16mfmapwxcl_p16_f16_wco%d_px%d_k%d_wgs%d", map == MAP_FWD ? "fwd" : "dgrad",
+             wco, 64 * (4 / wco), nsteps, blocks);
+    g_last_kernel = g_name_buf;
+    say(p, map == MAP_FWD ? "forward (channels-last)" : "input gradient (channels-last)");
     return PHX_OK;
 }
 
@@ -1208,6 +1265,7 @@ size_t phx_qconv2d_workspace_bytes(const phx_qconv_desc* desc, int pass) {
     if (desc && desc->algebra != PHX_QUATERNION) return algebra_conv_workspace_bytes(desc, pass);
     Problem p;
     if (problem_from_conv(desc, p) != PHX_OK) return 0;
+    if (nhwc_native(p, pass)) return nhwc_native_workspace(p, pass);
     return ChannelsLast(p).bytes() + workspace_for(p, pass);
 }
 
@@ -1226,6 +1284,9 @@ int phx_qconv2d_fwd(const phx_qconv_desc* desc, phx_stream_t stream, const void*
     Problem p;
     const int rc = problem_from_conv(desc, p);
     if (rc != PHX_OK) return rc;
+    if (nhwc_native(p, PHX_PASS_FWD))
+        return run_pwx_nhwc(p, MAP_FWD, static_cast<hipStream_t>(stream), x, w, p.has_bias ? bias_or_null : nullptr, y, workspace,
+                            workspace_bytes);
     const GroupOffsets o(p);
     const ChannelsLast cl(p);
     hipStream_t st = static_cast<hipStream_t>(stream);
@@ -1267,6 +1328,8 @@ int phx_qconv2d_bwd_data(const phx_qconv_desc* desc, phx_stream_t stream, const 
     // the gradient with respect to a real-valued input has imaginary parts that are stored nowhere;
     // the reference refuses the request likewise (src/conv2d.hpp:394-398)
     if (p.real_input) return PHX_ERR_INVALID_ARGUMENT;
+    if (nhwc_native(p, PHX_PASS_BWD_DATA))
+        return run_pwx_nhwc(p, MAP_DGRAD, static_cast<hipStream_t>(stream), grad, w, nullptr, dx, workspace, workspace_bytes);
     const GroupOffsets o(p);
     const ChannelsLast cl(p);
     hipStream_t st = static_cast<hipStream_t>(stream);

@@ -430,6 +430,11 @@ CHANNELS_LAST = [
     ("nhwc_plane_gt_tile", 1, False, True, 1, 3, 2, 20, 23, 5, 5, 1, 2, (2, 1, 3, 0)),
     ("nhwc_stem_real", 1, True, True, 2, 3, 16, 32, 32, 7, 7, 2, 1, "SAME"),
     ("nhwc_grouped", 4, False, True, 2, 16, 24, 10, 10, 3, 3, 1, 1, "SAME"),
+    # pointwise, channel counts multiples of 8: the native channels-last kernel on fp16 matrix cores
+    ("nhwc_pw_c40_24", 1, False, True, 3, 40, 24, 10, 10, 1, 1, 1, 1, "VALID"),
+    ("nhwc_pw_c72_200", 1, False, False, 2, 72, 200, 6, 5, 1, 1, 1, 1, "VALID"),
+    ("nhwc_pw_63px", 1, False, True, 3, 16, 48, 7, 9, 1, 1, 1, 1, "VALID"),
+    ("nhwc_pw_128", 1, False, True, 2, 128, 128, 12, 12, 1, 1, 1, 1, "VALID"),
 ]
 
 
@@ -459,7 +464,11 @@ def test_channels_last(case, mode, dtype, policy):
     assert desc.output_shape == (4 * n, g.ho, g.wo, co)
     xd, wd, bd, gd = (torch.from_numpy(a).cuda() for a in (x_dev, w_dev, b, g_dev))
     y = phx.conv2d_fwd(xd, wd, bd if bias else None, desc)
+    native = (dtype == torch.float16 and policy != "fp32" and kh == 1 and kw == 1 and stride == 1 and G == 1 and not real
+              and ci % 8 == 0 and co % 8 == 0)
+    assert ("pwxcl" in capi.last_kernel_name()) == native, capi.last_kernel_name()
     dw, dx = phx.conv2d_bwd(xd, wd, gd, desc)
+    assert ("pwxcl" in capi.last_kernel_name()) == (native and policy == "full16"), capi.last_kernel_name()
     gg = oracle.make_geom(n, cig, cog, h, w, kh, kw, stride, dilation, padding)
     x64, w64, b64, g64 = (a.astype(np.float64) for a in (x, wt, b, gr))
     want_y, want_dx, want_dw = np.empty(gr.shape), np.empty(x.shape), np.empty(wt.shape)
