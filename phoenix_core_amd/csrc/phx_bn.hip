@@ -112,8 +112,11 @@ __device__ __forceinline__ void channel_totals(const BnArgs& P, int c, float& t0
     wg_sum2(t0, t1, red);
 }
 
-// MODE 0: sum x, sum x^2 (forward statistics).  MODE 1: sum dy', sum dy' * xhat with dy' the gradient
-// behind the optional ReLU (backward sums).
+// MODE 0: sum (x - K), sum (x - K)^2 (forward statistics) with the shift K = the channel's first element: the
+// variance is E[(x-K)^2] - E[x-K]^2 whatever K is, and with K inside the data's range the two terms are of the size
+// of the variance itself -- the plain E[x^2] - E[x]^2 loses every significant bit of a channel whose mean is large
+// against its spread (activations behind a ReLU or a residual add, in fp16).
+// MODE 1: sum dy', sum dy' * xhat with dy' the gradient behind the optional ReLU (backward sums).
 template <typename TS, int MODE>
 __global__ void __launch_bounds__(256) bn_sums_kernel(const BnArgs P) {
     constexpr int V = Vec<TS>::N;
@@ -126,6 +129,7 @@ __global__ void __launch_bounds__(256) bn_sums_kernel(const BnArgs P) {
     const TS* res = static_cast<const TS*>(P.res);
     float mean = 0.f, invstd = 0.f, g = 0.f, be = 0.f;
     if constexpr (MODE == 1) { mean = P.save_mean[c]; invstd = P.save_invstd[c]; g = P.gamma[c]; be = P.beta[c]; }
+    const float shift = (MODE == 0) ? (float)x[(long)c * P.hw] : 0.f;
     float a0 = 0.f, a1 = 0.f;
     const int total = nb * P.nchunk;
     for (int idx = threadIdx.x; idx < total; idx += 256) {
@@ -136,7 +140,11 @@ __global__ void __launch_bounds__(256) bn_sums_kernel(const BnArgs P) {
         load_chunk<TS>(x + off, n, xv);
         if constexpr (MODE == 0) {
 #pragma unroll
-            for (int i = 0; i < V; ++i) { a0 += xv[i]; a1 += xv[i] * xv[i]; }
+            for (int i = 0; i < V; ++i) {
+                const float d = i < n ? xv[i] - shift : 0.f;
+                a0 += d;
+                a1 += d * d;
+            }
         } else {
             float dv[V], rv[V];
             load_chunk<TS>(dy + off, n, dv);
@@ -172,8 +180,9 @@ __global__ void __launch_bounds__(256) bn_apply_kernel(const BnArgs P) {
     const float g = P.gamma[c], be = P.beta[c];
     float mean, invstd;
     if constexpr (MODE == 0) {
-        mean = t0 / m;
-        const float var = fmaxf(t1 / m - mean * mean, 0.f);
+        const float shifted = t0 / m;  // mean of x - K, K as in bn_sums_kernel
+        mean = (float)static_cast<const TS*>(P.x)[(long)c * P.hw] + shifted;
+        const float var = fmaxf(t1 / m - shifted * shifted, 0.f);
         invstd = 1.f / sqrtf(var + P.eps);
         if (s == 0 && threadIdx.x == 0) {
             P.save_mean[c] = mean;
