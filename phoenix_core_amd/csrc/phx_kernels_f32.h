@@ -166,61 +166,127 @@ __device__ __forceinline__ void conv_epilogue(const ConvArgs& P, const f32x16 (&
 // ---------------------------------------------------------------------------------------------
 struct StageVec {
     long goff;           // element offset of the group's first position from component 0, channel 0
+    long tbase;          // goff + the offset of the thread group's own (component, channel) plane
     int lpos;            // first window position of the group
     int group;
+    int c_room, p_room;  // channels / components from the thread group's own plane to the end of the tensor
     unsigned int bits;   // positions inside the image
     bool live, careful;
+    bool fast;           // live and every vector load stays inside the tensor
 };
 
-template <typename TS, int P2LOG>
-__device__ __forceinline__ StageVec make_stage_vec(const TileSrc& s, int n0, int h0, int w0, int NB, int HTH, int HTW,
-                                                   int HP) {
-    StageVec sv;
+// What a thread's position group is, apart from the window's origin: decoded once per kernel.
+struct StageVecLane {
+    int lpos, group, nb, hr, col;
+    bool inside;  // the group lies inside the window
+};
+
+template <int P2LOG>
+__device__ __forceinline__ StageVecLane make_stage_vec_lane(int NB, int HTH, int HTW, int HP) {
+    StageVecLane L;
     constexpr int NPC = 1 << (P2LOG - 2);
     const int pc = threadIdx.x & (NPC - 1);
-    sv.group = threadIdx.x >> (P2LOG - 2);
-    sv.lpos = pc * 4;
-    const int row = sv.lpos / HTW, col = sv.lpos - row * HTW;
-    const int nb = row / HTH, hr = row - nb * HTH;
-    const int vh = h0 + hr, vw0 = w0 + col;
-    sv.live = sv.lpos < HP && nb < NB && (n0 + nb) < s.N && vh >= 0 && vh < s.Hd;
+    L.group = threadIdx.x >> (P2LOG - 2);
+    L.lpos = pc * 4;
+    const int row = L.lpos / HTW;
+    L.col = L.lpos - row * HTW;
+    L.nb = row / HTH;
+    L.hr = row - L.nb * HTH;
+    L.inside = L.lpos < HP && L.nb < NB;
+    return L;
+}
+
+// NCH channels per chunk: thread group g takes planes g, g + G4, ... of the chunk's 4*NCH (component, channel)
+// planes; plane pc is (component pc / NCH, channel pc % NCH).  With G4 and NCH powers of two, the plane of load e
+// is (p_group + pe(e), c_group + ce(e)) with pe, ce the same for every thread.
+// vector loads per thread and chunk
+constexpr int stage_loads(int nch, int p2log, int nt) { return (4 * nch) / (nt >> (p2log - 2)); }
+
+template <int NCH, int P2LOG, int NT = WG_THREADS>
+struct StagePlanes {
+    static constexpr int G4 = NT >> (P2LOG - 2);   // thread groups
+    static constexpr int E = stage_loads(NCH, P2LOG, NT);
+    static __device__ __forceinline__ int p_group(int group) { return G4 >= NCH ? group / NCH : 0; }
+    static __device__ __forceinline__ int c_group(int group) { return G4 >= NCH ? group % NCH : group; }
+    static __device__ __forceinline__ int pe(int e) { return G4 >= NCH ? e * (G4 / NCH) : (e * G4) / NCH; }
+    static __device__ __forceinline__ int ce(int e) { return G4 >= NCH ? 0 : (e * G4) % NCH; }
+};
+
+template <typename TS, int NCH, int P2LOG, int NT = WG_THREADS>
+__device__ __forceinline__ StageVec place_stage_vec(const TileSrc& s, const StageVecLane& L, int n0, int h0, int w0) {
+    typedef StagePlanes<NCH, P2LOG, NT> PL;
+    StageVec sv;
+    sv.group = L.group;
+    sv.lpos = L.lpos;
+    const int vh = h0 + L.hr, vw0 = w0 + L.col;
+    sv.live = L.inside && (n0 + L.nb) < s.N && vh >= 0 && vh < s.Hd;
     sv.bits = sv.live ? interval_bits<4>(-vw0, s.Wd - vw0) : 0u;
-    sv.goff = ((long)(n0 + nb) * s.Cs * s.Hd + vh) * s.Wd + vw0;
+    sv.goff = ((long)(n0 + L.nb) * s.Cs * s.Hd + vh) * s.Wd + vw0;
     const long plane = (long)s.Hd * s.Wd;
     const long last = (long)(s.ncomp - 1) * s.comp_stride;  // offset of the last component in memory
     const long total = last + ((long)(s.N - 1) * s.Cs + s.C) * plane;
     sv.careful = sv.live && (sv.goff < 0 || sv.goff + last + (long)(s.C - 1) * plane + 4 > total);
+    sv.fast = sv.live && !sv.careful;
+    const int pg = PL::p_group(L.group), cg = PL::c_group(L.group);
+    sv.tbase = sv.goff + pg * s.comp_stride + cg * plane;
+    sv.c_room = s.C - cg;
+    sv.p_room = s.ncomp - pg;
     return sv;
 }
 
-// plane index e*G4 + group -> (component, channel of the chunk)
 template <typename TS, int NCH, int P2LOG>
-__device__ __forceinline__ void stage_vec_load(f32x4 (&v)[(NCH << P2LOG) >> 8], const TileSrc& s, const StageVec& sv,
-                                               int c0, int e) {
-    constexpr int G4 = (4 * WG_THREADS) >> P2LOG;
+__device__ __forceinline__ StageVec make_stage_vec(const TileSrc& s, int n0, int h0, int w0, int NB, int HTH, int HTW,
+                                                   int HP) {
+    return place_stage_vec<TS, NCH, P2LOG>(s, make_stage_vec_lane<P2LOG>(NB, HTH, HTW, HP), n0, h0, w0);
+}
+
+// load e of the chunk that starts at channel c0
+template <typename TS, int NCH, int P2LOG, int NT = WG_THREADS>
+__device__ __forceinline__ void stage_vec_load(f32x4 (&v)[stage_loads(NCH, P2LOG, NT)], const TileSrc& s,
+                                               const StageVec& sv, int c0, int e) {
+    typedef StagePlanes<NCH, P2LOG, NT> PL;
     const TS* origin = static_cast<const TS*>(s.base);
     const long plane = (long)s.Hd * s.Wd;
-    const int pc = e * G4 + sv.group;
-    const int p = pc / NCH, c = c0 + pc % NCH;
+    // the same for every thread: scalar arithmetic, one 64-bit add per load and thread
+    const long uoff = (long)PL::pe(e) * s.comp_stride + (long)(c0 + PL::ce(e)) * plane;
     // channels past the tensor meet zero filters: any finite value will do, the tensor's first bytes are safe
     // (components a real-valued tensor does not have are masked to zero by the store)
-    const TS* ptr =
-        (sv.live && !sv.careful && c < s.C && p < s.ncomp) ? origin + sv.goff + p * s.comp_stride + c * plane : origin;
+    const bool ok = sv.fast && (c0 + PL::ce(e)) < sv.c_room && PL::pe(e) < sv.p_room;
+    const TS* ptr = ok ? origin + (sv.tbase + uoff) : origin;
     if constexpr (sizeof(TS) == 4) {
         typedef f32x4 f32x4_a4 __attribute__((aligned(4)));
         v[e] = *reinterpret_cast<const f32x4_a4*>(ptr);
     } else {
+        // kept as loaded (8 bytes in the first two registers) and widened by staged_values() when it is stored:
+        // a conversion here would wait for the load where it is issued
         typedef _Float16 f16x4_a2 __attribute__((ext_vector_type(4), aligned(2)));
-        const f16x4_a2 h = *reinterpret_cast<const f16x4_a2*>(ptr);
-        v[e] = f32x4{(float)h[0], (float)h[1], (float)h[2], (float)h[3]};
+        typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+        typedef float f32x2 __attribute__((ext_vector_type(2)));
+        const f16x4 h = *reinterpret_cast<const f16x4_a2*>(ptr);
+        const f32x2 bits = __builtin_bit_cast(f32x2, h);
+        v[e] = f32x4{bits[0], bits[1], 0.f, 0.f};
     }
 }
 
-template <typename TS, int NCH, int P2LOG>
-__device__ __forceinline__ void stage_vec_store(float* lds, const f32x4 (&v)[(NCH << P2LOG) >> 8], const TileSrc& s,
-                                                const StageVec& sv, int c0, int HP, int HPp) {
-    constexpr int G4 = (4 * WG_THREADS) >> P2LOG;
-    constexpr int E = (NCH << P2LOG) >> 8;
+// the four fp32 values of a staged group
+template <typename TS>
+__device__ __forceinline__ f32x4 staged_values(const f32x4& raw) {
+    if constexpr (sizeof(TS) == 4) {
+        return raw;
+    } else {
+        // (the elements are copied out first: __builtin_bit_cast applied to a vector element reads element 0)
+        const float lo = raw[0], hi = raw[1];
+        const unsigned int a = __builtin_bit_cast(unsigned int, lo), b = __builtin_bit_cast(unsigned int, hi);
+        auto half_of = [](unsigned int bits) { return (float)__builtin_bit_cast(_Float16, (unsigned short)bits); };
+        return f32x4{half_of(a), half_of(a >> 16), half_of(b), half_of(b >> 16)};
+    }
+}
+
+template <typename TS, int NCH, int P2LOG, int NT = WG_THREADS>
+__device__ __forceinline__ void stage_vec_store(float* lds, const f32x4 (&v)[stage_loads(NCH, P2LOG, NT)],
+                                                const TileSrc& s, const StageVec& sv, int c0, int HP, int HPp) {
+    constexpr int G4 = StagePlanes<NCH, P2LOG, NT>::G4;
+    constexpr int E = StagePlanes<NCH, P2LOG, NT>::E;
     if (sv.lpos >= HP) return;
     const unsigned int keep = sv.careful ? 0u : sv.bits;
     u32x4 mk;
@@ -229,7 +295,7 @@ __device__ __forceinline__ void stage_vec_store(float* lds, const f32x4 (&v)[(NC
 #pragma unroll
     for (int e = 0; e < E; ++e) {
         const bool present = (e * G4 + sv.group) / NCH < s.ncomp;
-        const u32x4 w = present ? (__builtin_bit_cast(u32x4, v[e]) & mk) : u32x4{0u, 0u, 0u, 0u};
+        const u32x4 w = present ? (__builtin_bit_cast(u32x4, staged_values<TS>(v[e])) & mk) : u32x4{0u, 0u, 0u, 0u};
         *reinterpret_cast<u32x4*>(lds + (e * G4 + sv.group) * HPp + sv.lpos) = w;
     }
     if (sv.careful) {
@@ -252,19 +318,20 @@ __device__ __forceinline__ void stage_vec_store(float* lds, const f32x4 (&v)[(NC
 }
 
 // same, for LDS rows with an odd pitch (bank-conflict-free 4-byte reads down a column of rows): four 4-byte stores
-template <typename TS, int NCH, int P2LOG>
-__device__ __forceinline__ void stage_vec_store_scalar(float* lds, const f32x4 (&v)[(NCH << P2LOG) >> 8], const TileSrc& s,
-                                                       const StageVec& sv, int c0, int HP, int pitch) {
-    constexpr int G4 = (4 * WG_THREADS) >> P2LOG;
-    constexpr int E = (NCH << P2LOG) >> 8;
+template <typename TS, int NCH, int P2LOG, int NT = WG_THREADS>
+__device__ __forceinline__ void stage_vec_store_scalar(float* lds, const f32x4 (&v)[stage_loads(NCH, P2LOG, NT)],
+                                                       const TileSrc& s, const StageVec& sv, int c0, int HP, int pitch) {
+    constexpr int G4 = StagePlanes<NCH, P2LOG, NT>::G4;
+    constexpr int E = StagePlanes<NCH, P2LOG, NT>::E;
     if (sv.lpos >= HP) return;
     const unsigned int keep = sv.careful ? 0u : sv.bits;
 #pragma unroll
     for (int e = 0; e < E; ++e) {
         float* dst = lds + (e * G4 + sv.group) * pitch + sv.lpos;
         const bool present = (e * G4 + sv.group) / NCH < s.ncomp;
+        const f32x4 val = staged_values<TS>(v[e]);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) dst[i] = (present && ((keep >> i) & 1)) ? v[e][i] : 0.f;
+        for (int i = 0; i < 4; ++i) dst[i] = (present && ((keep >> i) & 1)) ? val[i] : 0.f;
     }
     if (sv.careful) {
         const TS* origin = static_cast<const TS*>(s.base);
@@ -350,7 +417,7 @@ __global__ void __launch_bounds__(WG_THREADS, (MODE == 8 || NTW == 1) ? 2 : 1) q
     const long cpitch = (long)CK * P.HPp;  // LDS floats between components
     // 2^P2LOG window positions, 256 >> P2LOG thread groups sharing the 4*CK planes of a chunk
     const StagePos sp = make_stage_pos<P2LOG>(P.in, n0, h0, w0, P.NB, P.HTH, P.HTW);
-    const StageVec sv = make_stage_vec<TS, P2LOG>(P.in, n0, h0, w0, P.NB, P.HTH, P.HTW, P.HP);
+    const StageVec sv = make_stage_vec<TS, CK, P2LOG>(P.in, n0, h0, w0, P.NB, P.HTH, P.HTW, P.HP);
     constexpr int EV = (CK << P2LOG) >> 8;  // vector loads per thread and chunk
     float stage[VSTG ? 1 : ((4 * CK) >> (8 - P2LOG))];
     f32x4 stagev[VSTG ? EV : 1];
@@ -524,16 +591,22 @@ struct WgradArgs {
     int cpr, nchunks, ntiles, zsplit;  // fp16 kernel: 8-pixel chunks per output row / in total, pixel tiles, reduction slices
 };
 
-template <typename TS, int MODE, int TPW, bool VEC>
-__global__ void __launch_bounds__(WG_THREADS) qconv_wgrad_f32_kernel(const WgradArgs P) {
+//   KSETS = 2: eight waves, two per SIMD (while one forms lanes or waits for LDS, the other's matrix
+//   instructions run); the second set of four takes the odd K steps of every tile into accumulators of its
+//   own, which go to a reduction slice of their own (slice z*KSETS + set).  Every thread stages half as much.
+template <typename TS, int MODE, int TPW, bool VEC, int KSETS>
+__global__ void __launch_bounds__(WG_THREADS * KSETS) qconv_wgrad_f32_kernel(const WgradArgs P) {
     constexpr int CT = 64;
+    constexpr int NT = WG_THREADS * KSETS;
+    constexpr int EV = 8 / KSETS;  // vector loads per thread, tile and operand
+    static_assert(KSETS == 1 || VEC, "the K split is written for the vector staging");
     constexpr int NACC = (MODE == 16) ? 4 : 8;
     extern __shared__ float lds[];
     float* gl = lds;                           // [4][CT][KPp]
     float* xl = lds + 4 * CT * P.KPp;          // [4][CT][HPp]
     int* poff = reinterpret_cast<int*>(xl + 4 * CT * P.HPp);  // [KP]
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, wave = (tid >> 6) & 3, kset = tid >> 8;
     const int wco = wave & 1, wci = wave >> 1;
     const int m = lane & 31, kk = lane >> 5;
     // workgroups that share a reduction slice read the same gradient / input tiles: keep them on one XCD
@@ -550,7 +623,7 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_wgrad_f32_kernel(const Wgrad
     const int HTW = VEC ? ((HTWx + 3) & ~3) : HTWx;  // vector staging: whole groups of 4 positions per window row
 
     const int thw = P.TH * P.TW;
-    for (int k = tid; k < P.KP; k += WG_THREADS) {
+    for (int k = tid; k < P.KP; k += NT) {
         const int nb = k / thw, rem = k - nb * thw;
         const int r = rem / P.TW, c = rem - r * P.TW;
         poff[k] = (nb < P.NB) ? (nb * P.HTH + r * P.sh) * HTW + c * P.sw : 0;
@@ -568,32 +641,40 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_wgrad_f32_kernel(const Wgrad
     const long gcp = (long)CT * P.KPp, xcp = (long)CT * P.HPp;
     constexpr int P2LOG = 5;  // 32 window positions x 8 plane groups (vector form: 8 groups of 4 x 32 plane groups)
     float sg[VEC ? 1 : 32], sx[VEC ? 1 : 32];
-    f32x4 vg[VEC ? 8 : 1], vx[VEC ? 8 : 1];
+    f32x4 vg[VEC ? EV : 1], vx[VEC ? EV : 1];
     StagePos spg, spx;
     StageVec svg, svx;
-    auto locate = [&](int tile) {
-        const int tw = tile % P.tiles_w;
-        const int th = (tile / P.tiles_w) % P.tiles_h;
-        const int tn = tile / (P.tiles_w * P.tiles_h);
+    // tiles zi, zi + zsplit, ... as (image group, row tile, column tile): stepped with carries, no division per tile
+    int tw = zi % P.tiles_w, th = (zi / P.tiles_w) % P.tiles_h, tn = zi / (P.tiles_w * P.tiles_h);
+    const int step_w = P.zsplit % P.tiles_w, step_h = (P.zsplit / P.tiles_w) % P.tiles_h;
+    const int step_n = P.zsplit / (P.tiles_w * P.tiles_h);
+    const StageVecLane lane_g = make_stage_vec_lane<P2LOG>(P.NB, P.TH, P.TW, P.NB * thw);
+    const StageVecLane lane_x = make_stage_vec_lane<P2LOG>(P.NB, P.HTH, HTW, P.NB * P.HTH * HTW);
+    auto locate = [&]() {  // the staging positions of tile (tn, th, tw); then steps to the workgroup's next tile
         const int n0 = tn * P.NB, ho0 = th * P.TH, wo0 = tw * P.TW;
         const int h0x = ho0 * P.sh - P.pt + kh * P.dh, w0x = wo0 * P.sw - P.pl + kw0 * P.dw;
         // gradient window: TH x TW output pixels, no halo; pixels beyond the tensor are zero and
         // therefore contribute nothing whatever the input window holds there
         if constexpr (VEC) {
-            svg = make_stage_vec<TS, P2LOG>(P.g, n0, ho0, wo0, P.NB, P.TH, P.TW, P.NB * thw);
-            svx = make_stage_vec<TS, P2LOG>(P.x, n0, h0x, w0x, P.NB, P.HTH, HTW, P.NB * P.HTH * HTW);
+            svg = place_stage_vec<TS, CT, P2LOG, NT>(P.g, lane_g, n0, ho0, wo0);
+            svx = place_stage_vec<TS, CT, P2LOG, NT>(P.x, lane_x, n0, h0x, w0x);
         } else {
             spg = make_stage_pos<P2LOG>(P.g, n0, ho0, wo0, P.NB, P.TH, P.TW);
             spx = make_stage_pos<P2LOG>(P.x, n0, h0x, w0x, P.NB, P.HTH, HTW);
         }
+        tw += step_w;
+        if (tw >= P.tiles_w) { tw -= P.tiles_w; ++th; }
+        th += step_h;
+        if (th >= P.tiles_h) { th -= P.tiles_h; ++tn; }
+        tn += step_n;
     };
-    auto issue = [&](int tile) {
-        locate(tile);
+    auto issue = [&]() {
+        locate();
         if constexpr (VEC) {
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                stage_vec_load<TS, CT, P2LOG>(vg, P.g, svg, cot * CT, e);
-                stage_vec_load<TS, CT, P2LOG>(vx, P.x, svx, cit * CT, e);
+            for (int e = 0; e < EV; ++e) {
+                stage_vec_load<TS, CT, P2LOG, NT>(vg, P.g, svg, cot * CT, e);
+                stage_vec_load<TS, CT, P2LOG, NT>(vx, P.x, svx, cit * CT, e);
             }
         } else {
             stage_load<TS, CT, P2LOG>(sg, P.g, spg, cot * CT);
@@ -601,78 +682,130 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_wgrad_f32_kernel(const Wgrad
         }
     };
     const int HPx = P.NB * P.HTH * HTW;
-    if (zi < ntiles) issue(zi);
+    if (zi < ntiles) issue();
+    PHX_PHASES_BEGIN(5)
     for (int tile = zi; tile < ntiles; tile += P.zsplit) {
+        PHX_STAMP(4)
         __syncthreads();
+        PHX_STAMP(0)
         if constexpr (VEC) {
-            stage_vec_store_scalar<TS, CT, P2LOG>(gl, vg, P.g, svg, cot * CT, P.NB * thw, P.KPp);
-            stage_vec_store_scalar<TS, CT, P2LOG>(xl, vx, P.x, svx, cit * CT, HPx, P.HPp);
+            stage_vec_store_scalar<TS, CT, P2LOG, NT>(gl, vg, P.g, svg, cot * CT, P.NB * thw, P.KPp);
+            stage_vec_store_scalar<TS, CT, P2LOG, NT>(xl, vx, P.x, svx, cit * CT, HPx, P.HPp);
         } else {
             stage_store<CT, P2LOG, float>(gl, sg, spg, P.NB * thw, P.KPp);
             stage_store<CT, P2LOG, float>(xl, sx, spx, HPx, P.HPp);
         }
         if (P.KP != P.NB * thw)  // odd pixel count: the padding column of the gradient window must be zero
-            for (int c = tid; c < 4 * CT; c += WG_THREADS) gl[c * P.KPp + P.KP - 1] = 0.f;
+            for (int c = tid; c < 4 * CT; c += NT) gl[c * P.KPp + P.KP - 1] = 0.f;
+        // Threads without a window position skip the stores and, with them, the waits for their loads.  Stated
+        // here for every path, it lets the next tile's loads be issued below without a wait in front of each
+        // (they reuse the staging registers).
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+        PHX_STAMP(1)
         __syncthreads();
+        PHX_STAMP(2)
         const bool more = tile + P.zsplit < ntiles;
         if constexpr (VEC) {
-            if (more) locate(tile + P.zsplit);
+            if (more) locate();
         } else {
-            if (more) issue(tile + P.zsplit);
+            if (more) issue();
         }
+        PHX_STAMP(3)
         const float* ga = gl + (wco * 32 + m) * P.KPp + kk;
         const float* xb = xl + (wci * 32 + m) * P.HPp;
-        // (vector form: at most 16 K steps, unrolled, so that the next tile's loads can be dealt over them --
-        // a wave that issues them back to back stalls until the memory pipeline has taken them all)
+        // one K step (two pixels): gradient values g of the wave's 32 output channels, input values x[t] of its
+        // 32 input channels under each tap
+        auto products = [&](const float (&g)[4], const float (&xs)[TPW][4]) {
+            float G[8];
+            if constexpr (MODE == 8) lanes_grad(g, G, 0.5f);
 #pragma unroll
-        for (int ksi = 0; ksi < (VEC ? 16 : 1); ++ksi) {
-            if constexpr (VEC) {
-                if (more && ksi < 8) {
-                    stage_vec_load<TS, CT, P2LOG>(vg, P.g, svg, cot * CT, ksi);
-                    stage_vec_load<TS, CT, P2LOG>(vx, P.x, svx, cit * CT, ksi);
-                }
-                if (2 * ksi >= P.KP) continue;
-            }
-            for (int ks = VEC ? 2 * ksi : 0; ks < (VEC ? 2 * ksi + 2 : P.KP); ks += 2) {
-                float g[4];
+            for (int t = 0; t < TPW; ++t) {
+                if (t < nkw) {
+                    const float(&x)[4] = xs[t];
+                    if constexpr (MODE == 16) {
+                        float nx[4];
 #pragma unroll
-                for (int q = 0; q < 4; ++q) g[q] = ga[q * gcp + ks];
-                const int po = poff[ks + kk];
-                float G[8];
-                if constexpr (MODE == 8) lanes_grad(g, G, 0.5f);
+                        for (int p = 0; p < 4; ++p) nx[p] = -x[p];
 #pragma unroll
-                for (int t = 0; t < TPW; ++t) {
-                    if (t < nkw) {
-                        float x[4];
+                        for (int p = 0; p < 4; ++p)
 #pragma unroll
-                        for (int p = 0; p < 4; ++p) x[p] = xb[p * xcp + po + t * P.dw];
-                        if constexpr (MODE == 16) {
-                            float nx[4];
+                            for (int q = 0; q < 4; ++q)
+                                acc[t][p ^ q] = __builtin_amdgcn_mfma_f32_32x32x2f32(g[q], qneg(p, q) ? nx[p] : x[p],
+                                                                                     acc[t][p ^ q], 0, 0, 0);
+                    } else {
+                        float L[8];
+                        lanes_left(x, L);
 #pragma unroll
-                            for (int p = 0; p < 4; ++p) nx[p] = -x[p];
-#pragma unroll
-                            for (int p = 0; p < 4; ++p)
-#pragma unroll
-                                for (int q = 0; q < 4; ++q)
-                                    acc[t][p ^ q] = __builtin_amdgcn_mfma_f32_32x32x2f32(g[q], qneg(p, q) ? nx[p] : x[p],
-                                                                                         acc[t][p ^ q], 0, 0, 0);
-                        } else {
-                            float L[8];
-                            lanes_left(x, L);
-#pragma unroll
-                            for (int i = 0; i < 8; ++i)
-                                acc[t][i] = __builtin_amdgcn_mfma_f32_32x32x2f32(G[i], L[i], acc[t][i], 0, 0, 0);
-                        }
+                        for (int i = 0; i < 8; ++i)
+                            acc[t][i] = __builtin_amdgcn_mfma_f32_32x32x2f32(G[i], L[i], acc[t][i], 0, 0, 0);
                     }
                 }
+            }
+        };
+        if constexpr (VEC) {
+            // At most 16 K steps, unrolled: the next tile's global loads are dealt over the first eight (a wave
+            // that issues them back to back stalls until the memory pipeline has taken them all), and each step's
+            // LDS reads (the pixel's window offset, then the values) are issued one step ahead of the matrix
+            // products that use them.
+            // (a wave of set s takes the steps s, s + KSETS, ...)
+            constexpr int NJ = 16 / KSETS;
+            auto fetch = [&](int j, float (&g)[4], float (&xs)[TPW][4]) {
+                const int ksi = j * KSETS + kset;
+                const int ks = (2 * ksi < P.KP) ? 2 * ksi : P.KP - 2;
+#pragma unroll
+                for (int q = 0; q < 4; ++q) g[q] = ga[q * gcp + ks];
+                const int pk = poff[ks + kk];
+#pragma unroll
+                for (int t = 0; t < TPW; ++t) {
+                    const int tt = (t < nkw) ? t : 0;
+#pragma unroll
+                    for (int p = 0; p < 4; ++p) xs[t][p] = xb[p * xcp + pk + tt * P.dw];
+                }
+            };
+            float gc[4], xc[TPW][4];
+            fetch(0, gc, xc);
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) {
+                if (j == NJ / 2) { PHX_STAMP(5) }
+                if (more && j < EV) {
+                    stage_vec_load<TS, CT, P2LOG, NT>(vg, P.g, svg, cot * CT, j);
+                    stage_vec_load<TS, CT, P2LOG, NT>(vx, P.x, svx, cit * CT, j);
+                }
+                float gn[4], xn[TPW][4];
+                if (j + 1 < NJ) fetch(j + 1, gn, xn);
+                if (2 * (j * KSETS + kset) < P.KP) products(gc, xc);
+                if (j + 1 < NJ) {
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) gc[q] = gn[q];
+#pragma unroll
+                    for (int t = 0; t < TPW; ++t)
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) xc[t][q] = xn[t][q];
+                }
+            }
+        } else {
+            for (int ks = 0; ks < P.KP; ks += 2) {
+                float g[4], xs[TPW][4];
+#pragma unroll
+                for (int q = 0; q < 4; ++q) g[q] = ga[q * gcp + ks];
+                const int pk = poff[ks + kk];
+#pragma unroll
+                for (int t = 0; t < TPW; ++t) {
+                    const int tt = (t < nkw) ? t : 0;
+#pragma unroll
+                    for (int p = 0; p < 4; ++p) xs[t][p] = xb[p * xcp + pk + tt * P.dw];
+                }
+                products(g, xs);
             }
         }
     }
 
+    PHX_STAMP(4)
+    PHX_PHASES_REPORT("wgrad_f32: barrier / store / barrier / locate / products, second half / products, first half", 6)
     // partial[z][tap][r][co][ci]
     const int taps = P.Kh * P.Kw;
     const long tap_stride = 4L * P.CoP * P.CiP;
-    float* dst = P.partial + (long)zi * taps * tap_stride;
+    float* dst = P.partial + ((long)zi * KSETS + kset) * taps * tap_stride;
     const int ci = cit * CT + wci * 32 + m;
     const int co_base = cot * CT + wco * 32 + 4 * kk;
 #pragma unroll

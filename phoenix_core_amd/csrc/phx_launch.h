@@ -49,6 +49,8 @@ int launch_pwx_nhwc_f16(int WCO, const PwxArgs& a, int blocks, hipStream_t st); 
 size_t pwx_packed_bytes(int WCO, int co_tiles, int nsteps);
 int launch_pack_filters_pwx(int map, int WCO, int nsteps, const PackArgs& a, hipStream_t st);
 
+// wave sets (reduction slices) per workgroup of the fp32-MFMA filter-gradient kernel
+constexpr int wgrad_f32_ksets(int mode, bool vec) { return (mode == 8 && vec) ? 2 : 1; }
 int launch_wgrad_f32(bool half_storage, bool vec, int mode, const WgradArgs& a, dim3 grid, size_t lds_bytes,
                      hipStream_t st);  // vec: windows staged as groups of 4 positions
 // fp16-MFMA filter gradient: channel tile 32*MT x 32*NT, TPW taps per workgroup (1 or 3), stride SW along W (1 or 2)

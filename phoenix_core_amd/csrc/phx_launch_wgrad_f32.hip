@@ -5,9 +5,9 @@ namespace phx {
 
 template <typename TS, bool VEC>
 static void launch_ts(int mode, const WgradArgs& a, dim3 grid, size_t lds_bytes, hipStream_t st) {
-    const dim3 b(WG_THREADS);
-    if (mode == 16) hipLaunchKernelGGL((qconv_wgrad_f32_kernel<TS, 16, 3, VEC>), grid, b, lds_bytes, st, a);
-    else hipLaunchKernelGGL((qconv_wgrad_f32_kernel<TS, 8, 1, VEC>), grid, b, lds_bytes, st, a);
+    constexpr int KSETS = wgrad_f32_ksets(8, VEC);
+    if (mode == 16) hipLaunchKernelGGL((qconv_wgrad_f32_kernel<TS, 16, 3, VEC, 1>), grid, dim3(WG_THREADS), lds_bytes, st, a);
+    else hipLaunchKernelGGL((qconv_wgrad_f32_kernel<TS, 8, 1, VEC, KSETS>), grid, dim3(WG_THREADS * KSETS), lds_bytes, st, a);
 }
 
 int launch_wgrad_f32(bool half_storage, bool vec, int mode, const WgradArgs& a, dim3 grid, size_t lds_bytes,

@@ -732,17 +732,18 @@ struct WgPlan {
     int MT, NT;  // fp16 kernel: 32*MT x 32*NT channel tile
     int kmode;   // product formulation the kernel runs in (see wgrad_f16_formulation, wgrad_f32_formulation)
     bool vec;    // fp32 kernel: windows staged as groups of 4 positions
+    int ksets;   // fp32 kernel: wave sets per workgroup, each with a reduction slice of its own
     int SW, cpr, nchunks, ntiles;  // fp16 kernel: stride along W, 8-pixel chunks per output row / in total, pixel tiles
     size_t lds_bytes, partial_bytes;
 };
 
-static void finish_wgrad_plan(const Problem& p, int CoT, int CiT, WgPlan& best) {
+static void finish_wgrad_plan(const Problem& p, int CoT, int CiT, int per_cu, WgPlan& best) {
     best.co_tiles = cdiv(p.co, CoT); best.ci_tiles = cdiv(p.ci, CiT);
     best.CoP = best.co_tiles * CoT; best.CiP = best.ci_tiles * CiT;
     best.groups_per_row = cdiv(p.kw, best.TPW);
     const int xy = best.co_tiles * best.ci_tiles * best.groups_per_row * p.kh;
     const int ntiles = best.tiles_n * best.tiles_h * best.tiles_w;
-    int target = 512;  // two workgroups per CU: one round
+    int target = 256 * per_cu;  // one round of workgroups
     if (tune().wgs > 0) target = tune().wgs;
     best.Z = std::max(1, std::min(ntiles, target / std::max(1, xy)));
     best.partial_bytes = (size_t)best.Z * p.kh * p.kw * 4 * best.CoP * best.CiP * sizeof(float);
@@ -750,13 +751,14 @@ static void finish_wgrad_plan(const Problem& p, int CoT, int CiT, WgPlan& best) 
 
 // The fp32-MFMA filter gradient in 8-product mode gives every tap a workgroup of its own (its 8 accumulator sets
 // leave no room for more), so the taps of a filter row each stage the same gradient tile; the 16-product kernel
-// shares it between three taps.  On small images, where a workgroup's tiles are short and staging weighs most, that
-// is worth more than the halved multiplications (measured on fp16 tensors under the backward32 policy, 3x3:
-// 128->128 @ 28x28 5.2 against 5.9 ms, 256->256 @ 14x14 6.8 against 9.8 ms; at 56x56 and for single-tap filters
-// the factorized kernel stays ahead).  The 8-product mode means "prefer speed" (src/backend/backend.hpp:36-66), so
-// those problems run the 16-product kernel; PHX_TUNE_WG8 keeps the factorized one.
+// shares it between three taps.  On the smallest images, where a workgroup's tiles are short, staging weighs most
+// and there are too few reduction slices to fill the CUs, that is worth more than the halved multiplications
+// (measured on fp16 tensors under the backward32 policy, 3x3: 256->256 @ 14x14 5.3 against 7.7 ms; 128->128 @
+// 28x28 the factorized kernel leads with 3.0 against 4.0 ms, as it does at 56x56 and for single-tap filters).  The
+// 8-product mode means "prefer speed" (src/backend/backend.hpp:36-66), so those problems run the 16-product
+// kernel; PHX_TUNE_WG8 keeps the factorized one.
 static int wgrad_f32_formulation(const Problem& p) {
-    return (p.mode == 8 && p.kw % 3 == 0 && p.wo <= 28 && !tune().wg8) ? 16 : p.mode;
+    return (p.mode == 8 && p.kw % 3 == 0 && p.wo <= 20 && !tune().wg8) ? 16 : p.mode;
 }
 
 // fp32-MFMA kernel: 64x64 channel tiles, pixel tile and input window of at most 32 positions
@@ -797,7 +799,9 @@ static bool plan_wgrad_f32(const Problem& p, WgPlan& best) {
     }
     if (best_score < 0) return false;
     best.MT = best.NT = 2;
-    finish_wgrad_plan(p, 64, 64, best);
+    best.ksets = wgrad_f32_ksets(best.kmode, best.vec);
+    finish_wgrad_plan(p, 64, 64, best.ksets == 2 ? 1 : 2, best);  // (eight waves of 256 registers fill a CU)
+    best.partial_bytes *= best.ksets;
     best.lds_bytes = ((size_t)4 * 64 * (best.KPp + best.HPp) + best.KP) * sizeof(float);
     return true;
 }
@@ -909,7 +913,7 @@ static int run_wgrad(const Problem& p, hipStream_t st, const void* x, const void
     ReduceArgs r;
     r.partial = a.partial; r.dw = dw;
     r.wcs = p.fs.wcs; r.so = p.fs.so; r.si = p.fs.si; r.skh = p.fs.skh; r.skw = p.fs.skw;
-    r.Z = pl.Z; r.Co = p.co; r.Ci = p.ci; r.Kh = p.kh; r.Kw = p.kw; r.CoP = pl.CoP; r.CiP = pl.CiP;
+    r.Z = f16 ? pl.Z : pl.Z * pl.ksets; r.Co = p.co; r.Ci = p.ci; r.Kh = p.kh; r.Kw = p.kw; r.CoP = pl.CoP; r.CiP = pl.CiP;
     const long items = 4L * p.kh * p.kw * p.co * p.ci;
     const int blocks = (int)((items + 31) / 32);
     launch_reduce_wgrad(half_storage, r, blocks, st);
