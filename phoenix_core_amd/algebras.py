@@ -4,7 +4,9 @@ sign tables src/algebras.cc:5-145).
 The library runs them as one quaternion call on rearranged tensors (csrc/phx_algebra.hip): a GA_300 multivector
 (blades 1, e1, e2, e3, e12, e13, e23, e123) is A + e123 B with quaternion-like A = (m0, m4, m5, -m6) and
 B = (m7, -m3, m2, m1), and (A1 + I B1)(A2 + I B2) = (A1 A2 - B1 B2) + I (A1 B2 + B1 A2), i.e. one quaternion
-convolution of twice the channel counts; COMPLEX and REAL are embedded with zero components.  This module only
+convolution of twice the channel counts; COMPLEX and REAL run in place as a quaternion problem on paired /
+quadrupled images (half / a quarter of the batch; batches that do not divide are embedded with zero components).
+This module only
 resolves shapes and fills the C descriptors with the algebra; the entry points of `ops` then take the tensors in
 the algebra's own layout: activations [D n, C, H, W], filters [D, Co, Ci, Kh, Kw] (REAL: no blade axis), bias
 [D, Co]; NCHW, OIHW / IO, no groups."""

@@ -8,9 +8,22 @@
 //     (A1 + I B1)(A2 + I B2) = (A1 A2 - B1 B2) + I (A1 B2 + B1 A2),
 // i.e. a GA_300 convolution of Ci -> Co channels is one quaternion convolution of 2 Ci -> 2 Co channels on the
 // activations [A | B] with the filter blocks [[A2, B2], [-B2, A2]] (input half x output half): 64 real products
-// per multivector product, as many as the algebra's own table holds.  COMPLEX and REAL are the sub-algebras
-// {1, i} and {1} of the quaternions; their tensors are embedded with zero components (correct, but the full
-// quaternion arithmetic runs: 4x / 16x the products these algebras need).
+// per multivector product, as many as the algebra's own table holds.
+//
+// COMPLEX and REAL are the sub-algebras {1, i} and {1} of the quaternions.  Embedding their tensors with zero
+// components is correct but runs the full quaternion arithmetic on zeros (4x / 16x the products these algebras
+// need); it remains the path for batches that cannot be paired.  With an even batch a COMPLEX problem is instead
+// run as a quaternion problem on HALF the batch, in place: images A (first half) and B (second half) form
+//     q = z_A + conj(z_B) j,      q (x) u = z_A u + conj(z_B u) j      for a complex filter u  (j u = conj(u) j),
+// so one quaternion product yields both complex products, and the factorized 8-product form spends 4 real
+// multiplications per complex product -- what a 2x2-block kernel of its own would.  The layout needs no copy: in
+// the basis (1, j, i, -k) the coefficients of q are (re A, re B, im A, im B), which is how a complex tensor
+// [re(0..N) | im(0..N)] lies in memory, and relabelling the units by i <-> j, k -> -k is an automorphism of the
+// quaternions, so the kernels' (1, i, j, k) arithmetic on those coefficients computes the same product provided the
+// filter is relabelled too: u = u0 + u1 i goes in as (u0, 0, u1, 0).  The output (z_A u, z_B u) comes out in the
+// complex layout, the input gradient g (x) conj(u) likewise, and the complex filter gradient is the (1, i) part
+// (components 0 and 2) of the quaternion one, conj(q) (x) g = conj(z_A) g_A + conj(z_B) g_B + (...) j.  A bias b
+// enters as (b0, b0, b1, b1).  REAL: four images per quaternion, filter (w, 0, 0, 0), bias (b, b, b, b).
 //
 // The kernels here only rearrange (signed blade permutation, channel concatenation) into workspace buffers
 // around one call of the quaternion path; the backward passes use the transposes of the same maps.
@@ -27,6 +40,19 @@ struct BladeMap {
     int blade[8], sign[8];  // [h * 4 + p]
     int slot[8];            // inverse: blade b sits in slot h * 4 + p
 };
+
+// the paired forms described at the top: filter map and bias map
+static bool packed_maps(int algebra, BladeMap& filter, BladeMap& bias, int& images) {
+    auto fill = [](BladeMap& m, int dims, const int (&blade)[4]) {
+        m.dims = dims; m.halves = 1;
+        for (int s = 0; s < 8; ++s) { m.blade[s] = s < 4 ? blade[s] : -1; m.sign[s] = (s < 4 && blade[s] >= 0) ? 1 : 0; m.slot[s] = -1; }
+        for (int s = 3; s >= 0; --s)
+            if (blade[s] >= 0) m.slot[blade[s]] = s;
+    };
+    if (algebra == PHX_COMPLEX) { fill(filter, 2, {0, -1, 1, -1}); fill(bias, 2, {0, 0, 1, 1}); images = 2; return true; }
+    if (algebra == PHX_REAL) { fill(filter, 1, {0, -1, -1, -1}); fill(bias, 1, {0, 0, 0, 0}); images = 4; return true; }
+    return false;
+}
 
 static bool blade_map(int algebra, BladeMap& m) {
     auto fill = [&](int dims, int halves, const int (&blade)[8], const int (&sign)[8]) {
@@ -186,6 +212,8 @@ static size_t align256(size_t b) { return (b + 255) / 256 * 256; }
 // output-side tensor, the filter and the bias; the quaternion call's own workspace follows.
 struct Composition {
     BladeMap m;
+    BladeMap bias_map;  // paired form only
+    bool packed = false;  // paired form: activations in place, `m` maps the filter
     bool half;
     size_t esize, x_bytes, y_bytes, w_bytes, b_bytes;
     long n;
@@ -196,13 +224,13 @@ struct Composition {
         half = dtype == PHX_F16; esize = half ? 2 : 4;
         n = n_; ci = ci_; co = co_; hw_in = hw_in_; hw_out = hw_out_; taps = taps_;
         const size_t H = m.halves;
-        x_bytes = align256(4 * n * H * ci * hw_in * esize);
-        y_bytes = align256(4 * n * H * co * hw_out * esize);
+        x_bytes = packed ? 0 : align256(4 * n * H * ci * hw_in * esize);
+        y_bytes = packed ? 0 : align256(4 * n * H * co * hw_out * esize);
         w_bytes = align256(4 * H * co * H * ci * taps * esize);
         b_bytes = align256(4 * H * co * esize);
     }
-    void gather(const void* src, void* dst, long rows, int C, long hw, hipStream_t st) const {
-        BladeArgs a{src, dst, m, rows, C, hw};
+    void gather(const void* src, void* dst, long rows, int C, long hw, hipStream_t st, const BladeMap* map = nullptr) const {
+        BladeArgs a{src, dst, map ? *map : m, rows, C, hw};
         const int V = half ? 8 : 4;
         const long blocks = 4 * rows * m.halves, chw = C * hw;
         if (chw % V == 0) launch(half, blade_gather_kernel<float, 4>, blade_gather_kernel<_Float16, 8>, blocks * (chw / V), a, st);
@@ -241,12 +269,18 @@ static int conv_composition(const phx_qconv_desc* d, Composition& c, phx_qconv_d
         return PHX_ERR_NOT_SUPPORTED;
     inner = *d;
     inner.algebra = PHX_QUATERNION;
+    int images = 1;
+    BladeMap fm, bm;
+    if (packed_maps(d->algebra, fm, bm, images) && d->n > 0 && d->n % images == 0) {
+        c.packed = true; c.m = fm; c.bias_map = bm;
+        inner.n = d->n / images;
+    }
     inner.ci = d->ci * c.m.halves;
     inner.co = d->co * c.m.halves;
     int32_t ho = 0, wo = 0;
     const int rc = phx_qconv2d_output_hw(&inner, &ho, &wo);
     if (rc != PHX_OK) return rc;
-    c.init(d->dtype, d->n, d->ci, d->co, (long)d->h * d->w, (long)ho * wo, d->kh * d->kw);
+    c.init(d->dtype, inner.n, d->ci, d->co, (long)d->h * d->w, (long)ho * wo, d->kh * d->kw);
     return PHX_OK;
 }
 
@@ -256,9 +290,15 @@ static int dense_composition(const phx_qdense_desc* d, Composition& c, phx_qdens
     if (d->n < 0 || d->ni <= 0 || d->no <= 0 || (d->dtype != PHX_F32 && d->dtype != PHX_F16)) return PHX_ERR_INVALID_ARGUMENT;
     inner = *d;
     inner.algebra = PHX_QUATERNION;
+    int images = 1;
+    BladeMap fm, bm;
+    if (packed_maps(d->algebra, fm, bm, images) && d->n > 0 && d->n % images == 0) {
+        c.packed = true; c.m = fm; c.bias_map = bm;
+        inner.n = d->n / images;
+    }
     inner.ni = d->ni * c.m.halves;
     inner.no = d->no * c.m.halves;
-    c.init(d->dtype, d->n, d->ni, d->no, 1, 1, 1);
+    c.init(d->dtype, inner.n, d->ni, d->no, 1, 1, 1);
     return PHX_OK;
 }
 
@@ -276,7 +316,19 @@ static int composed_pass(const Composition& c, int pass, bool dense, hipStream_t
     void* inner_ws = base + c.buffers();
     const size_t inner_bytes = ws_bytes - c.buffers();
     int rc;
-    if (pass == PHX_PASS_FWD) {  // a = x, b = w
+    if (c.packed) {  // activations and gradients are used where they lie
+        if (pass == PHX_PASS_FWD) {
+            c.build_filter(b, wq, dense, st);
+            if (bias) c.gather(bias, bq, 1, c.co, 1, st, &c.bias_map);
+            rc = run(a, wq, bias ? bq : nullptr, out, inner_ws, inner_bytes);
+        } else if (pass == PHX_PASS_BWD_DATA) {
+            c.build_filter(b, wq, dense, st);
+            rc = run(a, wq, nullptr, out, inner_ws, inner_bytes);
+        } else {
+            rc = run(a, b, nullptr, wq, inner_ws, inner_bytes);
+            if (rc == PHX_OK) c.fold_filter(wq, out, dense, st);
+        }
+    } else if (pass == PHX_PASS_FWD) {  // a = x, b = w
         c.gather(a, xq, c.n, c.ci, c.hw_in, st);
         c.build_filter(b, wq, dense, st);
         if (bias) c.gather(bias, bq, 1, c.co, 1, st);

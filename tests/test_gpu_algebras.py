@@ -65,12 +65,17 @@ SHAPES = [
     (2, 6, 4, 10, 13, 3, 3, 1, 1, "SAME"),
     (1, 3, 8, 15, 14, 3, 3, 2, 1, "SAME"),
     (3, 4, 4, 8, 9, 3, 2, (1, 2), (2, 1), (2, 0, 1, 3)),
+    # batches of 2 (above) and 4, 8: COMPLEX and REAL run in place on paired / quadrupled images (csrc/phx_algebra.hip);
+    # odd batches take the embedding with zero components
+    (4, 6, 4, 10, 13, 3, 3, 1, 1, "SAME"),
+    (8, 16, 24, 12, 12, 1, 1, 1, 1, "VALID"),
+    (4, 5, 9, 11, 9, 3, 3, 2, 1, "SAME"),
 ]
 
 
 @pytest.mark.parametrize("dtype,policy", [(torch.float32, "fp32"), (torch.float16, "full16")], ids=["f32", "f16"])
 @pytest.mark.parametrize("mode", [8, 16])
-@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "k%dx%d_%dx%d" % (s[5], s[6], s[3], s[4]))
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "n%d_k%dx%d_%dx%d" % (s[0], s[5], s[6], s[3], s[4]))
 @pytest.mark.parametrize("algebra", [phx.REAL, phx.COMPLEX, phx.GA_300], ids=["real", "complex", "ga300"])
 def test_conv_against_the_sign_tables(algebra, shape, mode, dtype, policy):
     n, ci, co, h, w, kh, kw, stride, dilation, padding = shape
@@ -101,11 +106,12 @@ def test_conv_against_the_sign_tables(algebra, shape, mode, dtype, policy):
 
 
 @pytest.mark.parametrize("dtype,policy", [(torch.float32, "fp32"), (torch.float16, "full16")], ids=["f32", "f16"])
+@pytest.mark.parametrize("n", [7, 8])
 @pytest.mark.parametrize("algebra", [phx.REAL, phx.COMPLEX, phx.GA_300], ids=["real", "complex", "ga300"])
-def test_dense_against_the_sign_tables(algebra, dtype, policy):
+def test_dense_against_the_sign_tables(algebra, n, dtype, policy):
     d = algebras.DIMS[algebra]
     r = np.random.default_rng(200 + algebra)
-    n, ni, no = 7, 33, 20
+    ni, no = 33, 20
     npdt = np.float32 if dtype == torch.float32 else np.float16
     scale = 1.0 if dtype == torch.float32 else 0.5
     x = (scale * r.standard_normal((d * n, ni))).astype(npdt)
