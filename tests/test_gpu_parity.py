@@ -623,3 +623,23 @@ def test_mismatched_tensors_are_refused_before_the_library_reads_them():
         phx.conv2d_bwd(x.half(), w, g, desc)
     y = phx.conv2d_fwd(x, w, b, desc)
     assert torch.isfinite(y).all()
+
+
+def test_verbose_names_mode_policy_and_kernel(tune_env, capfd):
+    """UPSTRIDE_VERBOSE (src/backend/backend.cc:50-62 switches the reference's debug log on): one line per call on
+    stderr with the product mode, the fp16 policy and the kernel variant that ran; silent without it."""
+    x = torch.randn(4 * 2, 16, 12, 12, device="cuda").half()
+    w = (0.1 * torch.randn(4, 16, 16, 3, 3, device="cuda")).half()
+    desc = phx.Conv2DDescriptor(x.shape, w.shape, 1, 1, "SAME", dtype=torch.float16, context=Ctx(8, "full16"))
+    phx.conv2d_fwd(x, w, None, desc)
+    torch.cuda.synchronize()
+    assert "[upstride]" not in capfd.readouterr().err
+    tune_env(UPSTRIDE_VERBOSE="1")
+    phx.conv2d_fwd(x, w, None, desc)
+    phx.conv2d_bwd(x, w, torch.randn_like(x), desc)
+    torch.cuda.synchronize()
+    lines = [l for l in capfd.readouterr().err.splitlines() if l.startswith("[upstride]")]
+    assert len(lines) == 3, lines
+    assert "forward" in lines[0] and "product mode 8" in lines[0] and "fp16 policy full16" in lines[0]
+    assert any("filter gradient" in l for l in lines[1:]) and any("input gradient" in l for l in lines[1:])
+    assert capi.last_kernel_name() in lines[2]
