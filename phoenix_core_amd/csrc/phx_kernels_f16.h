@@ -816,12 +816,18 @@ __global__ void __launch_bounds__(WG_THREADS) pack_filters_f16_lds_kernel(const 
 //   three copies shifted by 0/1/2 pixels with byte-align operations; each copy is written to its
 //   own LDS plane so every MFMA operand is one aligned 16-byte LDS read.
 //   SW == 2: the input chunk is 16 consecutive pixels of which the even ones are kept.
+//   Flat chunk list (P.flat; unit strides, output and input rows of the same length >= 7): a row of 28 or 14
+//   pixels fills its last chunk half, an eighth of all chunks' work multiplies zeros.  Here the whole image plane
+//   is cut into chunks of 8 consecutive pixels instead (row-major, so a chunk may run over a row end): the input
+//   pixel of output pixel q under tap (kh, kw) is the plane's pixel q + (kh*dh - pt)*W + (kw*dw - pl), again 8 (or
+//   10, 12) consecutive pixels of memory; which of them are padding depends on the pixel's own row and column,
+//   so the masks are per tap and pixel, built from the at most two row segments of a chunk.
 //   Partial sums go to workspace[z]; reduce_wgrad_kernel adds them in a fixed order.
 // ---------------------------------------------------------------------------------------------
 constexpr int WG16_KP = 64;         // reduction indices per pixel tile
 constexpr int WG16_PITCH = 64 + 8;  // LDS halves per staged channel row (16-byte skew against bank conflicts)
 
-struct WgChunk {  // where one 8-pixel chunk of the reduction space lies
+struct WgChunk {  // where one 8-pixel chunk of the reduction space lies (flat list: ho = 0, wo0 = pixel of the plane)
     bool live;    // inside the reduction space
     int n, ho, wo0;
     int gi;       // index in the chunk list
@@ -836,8 +842,8 @@ __device__ __forceinline__ WgStep wg_step(const WgradArgs& P) {
     s.dgi = 8 * P.zsplit;
     const int drow = s.dgi / P.cpr;
     s.dwo = (s.dgi - drow * P.cpr) * 8;
-    s.dn = drow / P.g.Hd;
-    s.dho = drow - s.dn * P.g.Hd;
+    s.dn = drow / P.rows;
+    s.dho = drow - s.dn * P.rows;
     return s;
 }
 
@@ -849,8 +855,8 @@ __device__ __forceinline__ void wg_advance(WgChunk& c, const WgStep& s, const Wg
     const bool c1 = c.wo0 >= P.cpr * 8;
     c.wo0 -= c1 ? P.cpr * 8 : 0;
     c.ho += s.dho + (c1 ? 1 : 0);
-    const bool c2 = c.ho >= P.g.Hd;
-    c.ho -= c2 ? P.g.Hd : 0;
+    const bool c2 = c.ho >= P.rows;
+    c.ho -= c2 ? P.rows : 0;
     c.n += s.dn + (c2 ? 1 : 0);
 }
 
@@ -860,8 +866,8 @@ __device__ __forceinline__ WgChunk wg_chunk(const WgradArgs& P, int tile, int j)
     c.live = gi < P.nchunks;
     const int row = gi / P.cpr;
     c.wo0 = (gi - row * P.cpr) * 8;
-    c.n = row / P.g.Hd;
-    c.ho = row - c.n * P.g.Hd;
+    c.n = row / P.rows;
+    c.ho = row - c.n * P.rows;
     c.gi = gi;
     return c;
 }
@@ -922,12 +928,17 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_wgrad_f16_kernel(const Wgrad
 
     u32x4 sg[GE];
     unsigned int sx[XE][XR];
-    u32x4 mg;                // keeps the gradient pixels that lie inside their row
-    unsigned int mx[XR];     // keeps the loaded input columns that lie inside the image
+    u32x4 mg;                // keeps the gradient pixels that lie inside their row (flat list: inside the plane)
+    u32x4 mx[TPW];           // per tap: keeps the pixels whose input pixel lies inside the image
+    unsigned int gbits = 0, xbits[TPW];  // the same as bit masks, whether or not the chunk is filled element by element
     bool careful = false;    // this thread's chunk of the tile in flight is filled element by element
 
     auto xcol0 = [&](const WgChunk& c) { return c.wo0 * SW + kw0 * P.dw - P.pl; };
     auto xrow = [&](const WgChunk& c) { return c.ho * P.sh + kh * P.dh - P.pt; };
+    // element offset of the chunk's first loaded input pixel from its plane's first pixel
+    auto xlin = [&](const WgChunk& c) {
+        return P.flat ? c.wo0 + (kh * P.dh - P.pt) * W + (kw0 * P.dw - P.pl) : xrow(c) * W + xcol0(c);
+    };
 
     // Loads of one tile: every address is (uniform component/plane-group base) + (one 32-bit element
     // offset per thread), so a tile costs a handful of address instructions.  Chunks outside the
@@ -946,28 +957,55 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_wgrad_f16_kernel(const Wgrad
 
     unsigned int lgoff[MT], lxoff[NT];  // load offsets of the tile being fetched
     auto prep = [&](const WgChunk& c) {
-        const int hi = xrow(c), wi0 = xcol0(c);
-        const bool rowok = c.live && hi >= 0 && hi < H;
-        const int grow = c.n * gimg + c.ho * Wo + c.wo0;
-        const int xrow_off = c.n * ximg + hi * W + wi0;
+        bool any_x;
+        if (P.flat) {
+            // pixels q0 .. q0+7 of the plane: a first segment in row r0 from column c0 on, the rest in row r0 + 1
+            const int q0 = c.wo0, r0 = q0 / Wo, c0 = q0 - r0 * Wo, iw = Wo - c0;
+            const int ra = r0 + kh * P.dh - P.pt;
+            const bool rowa = c.live && ra >= 0 && ra < H, rowb = c.live && ra + 1 >= 0 && ra + 1 < H;
+            const unsigned int inplane = interval_bits(0, (int)gplane - q0);
+            gbits = c.live ? inplane : 0u;
+            any_x = false;
+#pragma unroll
+            for (int t = 0; t < TPW; ++t) {
+                const int dc = (kw0 + t) * P.dw - P.pl;          // input column = output column + dc
+                const int lo = dc < 0 ? -dc : 0, hi = W - dc < Wo ? W - dc : Wo;  // valid output columns [lo, hi)
+                const unsigned int a = rowa ? interval_bits(lo - c0, hi - c0 < iw ? hi - c0 : iw) : 0u;
+                const unsigned int b = rowb ? interval_bits(lo + iw > iw ? lo + iw : iw, hi + iw) : 0u;
+                xbits[t] = (a | b) & inplane;
+                any_x = any_x || xbits[t] != 0u;
+            }
+        } else {
+            const int hi = xrow(c), wi0 = xcol0(c);
+            const bool rowok = c.live && hi >= 0 && hi < H;
+            gbits = c.live ? interval_bits(0, Wo - c.wo0) : 0u;
+            const unsigned int window = rowok ? interval_bits<2 * XR>(-wi0, W - wi0) : 0u;  // loaded columns inside the image
+            any_x = rowok;
+#pragma unroll
+            for (int t = 0; t < TPW; ++t) {
+                if constexpr (SW == 1) {
+                    xbits[t] = (window >> t) & 0xFFu;
+                } else {
+                    unsigned int b = 0u;
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) b |= ((window >> (i * SW + t)) & 1u) << i;
+                    xbits[t] = b;
+                }
+            }
+        }
+        const int grow = c.n * gimg + (P.flat ? c.wo0 : c.ho * Wo + c.wo0);
+        const int xrow_off = c.n * ximg + xlin(c);
         int goff[MT], xoff[NT];
 #pragma unroll
         for (int i = 0; i < MT; ++i) goff[i] = grow + gch[i];
 #pragma unroll
         for (int i = 0; i < NT; ++i) xoff[i] = xrow_off + xch[i];
         // would any of this thread's vector loads leave the tensors?
-        careful = (c.live && goff[MT - 1] + 8 > gcomp) || (rowok && (xoff[0] < 0 || xoff[NT - 1] + 2 * XR > xcomp));
-        const bool gok = c.live && !careful, xok = rowok && !careful;
-        mg = expand_half_mask(gok ? interval_bits(0, Wo - c.wo0) : 0u);
-        {
-            const unsigned int bits = xok ? interval_bits<2 * XR>(-wi0, W - wi0) : 0u;
+        careful = (c.live && goff[MT - 1] + 8 > gcomp) || (any_x && (xoff[0] < 0 || xoff[NT - 1] + 2 * XR > xcomp));
+        const bool gok = c.live && !careful, xok = any_x && !careful;
+        mg = expand_half_mask(gok ? gbits : 0u);
 #pragma unroll
-            for (int d = 0; d < XR; ++d) {
-                const unsigned int lo = (unsigned int)((int)(bits << (31 - 2 * d)) >> 31);
-                const unsigned int up = (unsigned int)((int)(bits << (30 - 2 * d)) >> 31);
-                mx[d] = (lo & 0x0000FFFFu) | (up & 0xFFFF0000u);
-            }
-        }
+        for (int t = 0; t < TPW; ++t) mx[t] = expand_half_mask(xok ? xbits[t] : 0u);
 #pragma unroll
         for (int i = 0; i < MT; ++i) lgoff[i] = (unsigned int)(gok ? goff[i] : 0);
 #pragma unroll
@@ -1001,18 +1039,17 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_wgrad_f16_kernel(const Wgrad
     // element-wise fill of this thread's chunk (only next to the ends of the tensors).  The loads of
     // one plane are independent of each other, so their latencies overlap.
     auto fill_careful = [&](int tile) {
-        constexpr int NEL = 7 * SW + TPW;  // input columns one chunk touches over all taps of the group
+        constexpr int NEL = 7 * SW + TPW;  // input pixels one chunk touches over all taps of the group
         const WgChunk c = wg_chunk(P, tile, j);
-        const int hi = xrow(c), wi0 = xcol0(c);
-        const bool rowok = c.live && hi >= 0 && hi < H;
+        const int glin = P.flat ? c.wo0 : c.ho * Wo + c.wo0, lin = xlin(c);
 #pragma unroll 2
         for (int e = 0; e < GE; ++e) {
             const int q = e / MT, cc = (e % MT) * 32;
             const int ch = co_first + cc < P.g.C ? co_first + cc : P.g.C - 1;
-            const _Float16* src = gbase + q * P.g.comp_stride + (((long)c.n * P.g.Cs + ch) * Ho + c.ho) * Wo + c.wo0;
+            const _Float16* src = gbase + q * P.g.comp_stride + ((long)c.n * P.g.Cs + ch) * gplane + glin;
             _Float16 v[8];
 #pragma unroll
-            for (int i = 0; i < 8; ++i) v[i] = (c.live && c.wo0 + i < Wo) ? src[i] : (_Float16)0;
+            for (int i = 0; i < 8; ++i) v[i] = ((gbits >> i) & 1u) ? src[i] : (_Float16)0;
 #pragma unroll
             for (int i = 0; i < 8; ++i) gl[(q * CoT + cc + pg) * KPp + j * 8 + i] = v[i];
         }
@@ -1020,17 +1057,21 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_wgrad_f16_kernel(const Wgrad
         for (int e = 0; e < XE; ++e) {
             const int q = e / NT, cc = (e % NT) * 32;
             const int ch = ci_first + cc < P.x.C ? ci_first + cc : P.x.C - 1;
-            const _Float16* src = xbase + q * P.x.comp_stride + (((long)c.n * P.x.Cs + ch) * H + hi) * W;
-            _Float16 w[NEL];
-#pragma unroll
-            for (int k = 0; k < NEL; ++k) {
-                const int col = wi0 + k;
-                w[k] = (rowok && q < xnc && col >= 0 && col < W) ? src[col] : (_Float16)0;
-            }
+            const _Float16* src = xbase + q * P.x.comp_stride + ((long)c.n * P.x.Cs + ch) * xplane + lin;
+            // a pixel that some tap keeps is a pixel of the image; the others are not read
+            unsigned int used = 0u;
 #pragma unroll
             for (int t = 0; t < TPW; ++t)
 #pragma unroll
-                for (int i = 0; i < 8; ++i) xl[((t * 4 + q) * CiT + cc + pg) * KPp + j * 8 + i] = w[i * SW + t];
+                for (int i = 0; i < 8; ++i) used |= ((xbits[t] >> i) & 1u) << (i * SW + t);
+            _Float16 w[NEL];
+#pragma unroll
+            for (int k = 0; k < NEL; ++k) w[k] = (q < xnc && ((used >> k) & 1u)) ? src[k] : (_Float16)0;
+#pragma unroll
+            for (int t = 0; t < TPW; ++t)
+#pragma unroll
+                for (int i = 0; i < 8; ++i)
+                    xl[((t * 4 + q) * CiT + cc + pg) * KPp + j * 8 + i] = ((xbits[t] >> i) & 1u) ? w[i * SW + t] : (_Float16)0;
         }
     };
 
@@ -1055,7 +1096,7 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_wgrad_f16_kernel(const Wgrad
                 const int q = e / NT, cc = (e % NT) * 32;
                 unsigned int w[XR];
 #pragma unroll
-                for (int d = 0; d < XR; ++d) w[d] = q < xnc ? (sx[e][d] & mx[d]) : 0u;
+                for (int d = 0; d < XR; ++d) w[d] = q < xnc ? sx[e][d] : 0u;
 #pragma unroll
                 for (int t = 0; t < TPW; ++t) {
                     u32x4 v;
@@ -1070,7 +1111,7 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_wgrad_f16_kernel(const Wgrad
 #pragma unroll
                         for (int d = 0; d < 4; ++d) v[d] = w[(d + (t >> 1)) % XR];
                     }
-                    *reinterpret_cast<u32x4*>(xl + ((t * 4 + q) * CiT + cc + pg) * KPp + j * 8) = v;
+                    *reinterpret_cast<u32x4*>(xl + ((t * 4 + q) * CiT + cc + pg) * KPp + j * 8) = v & mx[t];
                 }
             }
             if (careful) fill_careful(tile);

@@ -589,6 +589,7 @@ struct WgradArgs {
     int co_tiles, ci_tiles, CoP, CiP;
     int groups_per_row; // tap groups per filter row
     int cpr, nchunks, ntiles, zsplit;  // fp16 kernel: 8-pixel chunks per output row / in total, pixel tiles, reduction slices
+    int flat, rows;                    // fp16 kernel: chunk list over whole planes (rows = 1) or over the rows of an image
 };
 
 //   KSETS = 2: eight waves, two per SIMD (while one forms lanes or waits for LDS, the other's matrix

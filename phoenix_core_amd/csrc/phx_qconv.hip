@@ -734,6 +734,7 @@ struct WgPlan {
     bool vec;    // fp32 kernel: windows staged as groups of 4 positions
     int ksets;   // fp32 kernel: wave sets per workgroup, each with a reduction slice of its own
     int SW, cpr, nchunks, ntiles;  // fp16 kernel: stride along W, 8-pixel chunks per output row / in total, pixel tiles
+    bool flat;   // fp16 kernel: the chunk list runs over whole image planes (cpr = chunks per plane)
     size_t lds_bytes, partial_bytes;
 };
 
@@ -832,8 +833,10 @@ static bool plan_wgrad_f16(const Problem& p, WgPlan& best) {
     auto lds_need = [&](int tpw) { return (size_t)(4 * 32 * best.MT + tpw * 4 * 32 * best.NT) * 72 * 2; };
     if (lds_need(best.TPW) > 160 * 1024) best.TPW = 1;  // (four shifted copies of a 64-channel input tile do not fit)
     const int CoT = 32 * best.MT, CiT = 32 * best.NT;
-    best.cpr = cdiv(p.wo, 8);
-    const long nchunks = (long)p.n * p.ho * best.cpr;
+    // chunk list over whole planes where rows would leave their last chunk partly empty (see the kernel's header)
+    best.flat = p.sh == 1 && p.sw == 1 && p.w == p.wo && p.h > 1 && p.wo >= 7 && p.wo % 8 != 0 && !tune().noflat;
+    best.cpr = best.flat ? cdiv(p.ho * p.wo, 8) : cdiv(p.wo, 8);
+    const long nchunks = (long)p.n * (best.flat ? 1 : p.ho) * best.cpr;
     if (nchunks > (1L << 28)) return false;
     best.nchunks = (int)nchunks;
     best.ntiles = cdiv(best.nchunks, 8);
@@ -898,6 +901,7 @@ static int run_wgrad(const Problem& p, hipStream_t st, const void* x, const void
     a.co_tiles = pl.co_tiles; a.ci_tiles = pl.ci_tiles; a.CoP = pl.CoP; a.CiP = pl.CiP;
     a.groups_per_row = pl.groups_per_row;
     a.cpr = pl.cpr; a.nchunks = pl.nchunks; a.ntiles = pl.ntiles; a.zsplit = pl.Z;
+    a.flat = (f16 && pl.flat) ? 1 : 0; a.rows = a.flat ? 1 : p.ho;
     const int nblocks = pl.co_tiles * pl.ci_tiles * pl.groups_per_row * p.kh * pl.Z;
     const bool half_storage = p.dtype == PHX_F16;
     {
@@ -919,8 +923,8 @@ static int run_wgrad(const Problem& p, hipStream_t st, const void* x, const void
     launch_reduce_wgrad(half_storage, r, blocks, st);
     PHX_HIP(hipGetLastError());
     if (f16)
-        snprintf(g_name_buf, sizeof(g_name_buf), "%sqconv_wgrad_f16mfma_p%d_f16_ch%dx%d_taps%d_sw%d_z%d", g_name_prefix, pl.kmode, 32 * pl.MT,
-                 32 * pl.NT, pl.TPW, pl.SW, pl.Z);
+        snprintf(g_name_buf, sizeof(g_name_buf), "%sqconv_wgrad_f16mfma_p%d_f16_ch%dx%d_taps%d_sw%d%s_z%d", g_name_prefix, pl.kmode, 32 * pl.MT,
+                 32 * pl.NT, pl.TPW, pl.SW, pl.flat ? "_flat" : "", pl.Z);
     else
         snprintf(g_name_buf, sizeof(g_name_buf), "%sqconv_wgrad_f32mfma%s_p%d_%s_tile%dx%dx%d_z%d", g_name_prefix, pl.vec ? "v" : "", pl.kmode,
                  p.dtype == PHX_F32 ? "f32" : "f16", pl.NB, pl.TH, pl.TW, pl.Z);
