@@ -928,6 +928,39 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_wgrad_f16_kernel(const Wgrad
 
     u32x4 sg[GE];
     unsigned int sx[XE][XR];
+    // Flat chunk list: the masks of every chunk of a plane under this workgroup's taps, as the 16-byte AND masks the
+    // staging stores use ([chunk][gradient, tap 0, tap 1, ...]; entry P.cpr is all zeros, for chunks that are not
+    // staged by vector loads) and as bits ([chunk][taps packed 8 bits each, gradient]).  Pixels q0 .. q0+7 of the
+    // plane form a first segment in row r0 from column c0 on and a second one in row r0 + 1 (rows are at least 7
+    // pixels long).
+    u32x4* fmask = reinterpret_cast<u32x4*>(xl + TPW * 4 * CiT * KPp);
+    unsigned int* fbits = reinterpret_cast<unsigned int*>(fmask + (P.cpr + 1) * (TPW + 1));
+    if (P.flat) {
+        for (int ch = tid; ch <= P.cpr; ch += WG_THREADS) {
+            const int q0 = ch * 8, r0 = q0 / Wo, c0 = q0 - r0 * Wo, iw = Wo - c0;
+            const int ra = r0 + kh * P.dh - P.pt;
+            const bool rowa = ra >= 0 && ra < H, rowb = ra + 1 >= 0 && ra + 1 < H;
+            const unsigned int inplane = ch < P.cpr ? interval_bits(0, Ho * Wo - q0) : 0u;
+            unsigned int packed = 0u;
+            fmask[ch * (TPW + 1)] = expand_half_mask(inplane);
+#pragma unroll
+            for (int t = 0; t < TPW; ++t) {
+                const int dc = (kw0 + t) * P.dw - P.pl;          // input column = output column + dc
+                const int lo = dc < 0 ? -dc : 0, hi = W - dc < Wo ? W - dc : Wo;  // valid output columns [lo, hi)
+                const unsigned int a = rowa ? interval_bits(lo - c0, hi - c0 < iw ? hi - c0 : iw) : 0u;
+                const unsigned int b = rowb ? interval_bits(lo + iw, hi + iw) : 0u;
+                const unsigned int bits = (a | b) & inplane;
+                fmask[ch * (TPW + 1) + 1 + t] = expand_half_mask(bits);
+                packed |= bits << (8 * t);
+            }
+            if (ch < P.cpr) {
+                fbits[2 * ch] = packed;
+                fbits[2 * ch + 1] = inplane;
+            }
+        }
+        __syncthreads();
+    }
+
     u32x4 mg;                // keeps the gradient pixels that lie inside their row (flat list: inside the plane)
     u32x4 mx[TPW];           // per tap: keeps the pixels whose input pixel lies inside the image
     unsigned int gbits = 0, xbits[TPW];  // the same as bit masks, whether or not the chunk is filled element by element
@@ -957,25 +990,8 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_wgrad_f16_kernel(const Wgrad
 
     unsigned int lgoff[MT], lxoff[NT];  // load offsets of the tile being fetched
     auto prep = [&](const WgChunk& c) {
-        bool any_x;
-        if (P.flat) {
-            // pixels q0 .. q0+7 of the plane: a first segment in row r0 from column c0 on, the rest in row r0 + 1
-            const int q0 = c.wo0, r0 = q0 / Wo, c0 = q0 - r0 * Wo, iw = Wo - c0;
-            const int ra = r0 + kh * P.dh - P.pt;
-            const bool rowa = c.live && ra >= 0 && ra < H, rowb = c.live && ra + 1 >= 0 && ra + 1 < H;
-            const unsigned int inplane = interval_bits(0, (int)gplane - q0);
-            gbits = c.live ? inplane : 0u;
-            any_x = false;
-#pragma unroll
-            for (int t = 0; t < TPW; ++t) {
-                const int dc = (kw0 + t) * P.dw - P.pl;          // input column = output column + dc
-                const int lo = dc < 0 ? -dc : 0, hi = W - dc < Wo ? W - dc : Wo;  // valid output columns [lo, hi)
-                const unsigned int a = rowa ? interval_bits(lo - c0, hi - c0 < iw ? hi - c0 : iw) : 0u;
-                const unsigned int b = rowb ? interval_bits(lo + iw > iw ? lo + iw : iw, hi + iw) : 0u;
-                xbits[t] = (a | b) & inplane;
-                any_x = any_x || xbits[t] != 0u;
-            }
-        } else {
+        bool any_x = c.live;
+        if (!P.flat) {
             const int hi = xrow(c), wi0 = xcol0(c);
             const bool rowok = c.live && hi >= 0 && hi < H;
             gbits = c.live ? interval_bits(0, Wo - c.wo0) : 0u;
@@ -1003,9 +1019,16 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_wgrad_f16_kernel(const Wgrad
         // would any of this thread's vector loads leave the tensors?
         careful = (c.live && goff[MT - 1] + 8 > gcomp) || (any_x && (xoff[0] < 0 || xoff[NT - 1] + 2 * XR > xcomp));
         const bool gok = c.live && !careful, xok = any_x && !careful;
-        mg = expand_half_mask(gok ? gbits : 0u);
+        if (P.flat) {  // the masks of a chunk depend on its place in the plane only: looked up
+            const u32x4* entry = fmask + (gok ? (c.wo0 >> 3) : P.cpr) * (TPW + 1);
+            mg = entry[0];
 #pragma unroll
-        for (int t = 0; t < TPW; ++t) mx[t] = expand_half_mask(xok ? xbits[t] : 0u);
+            for (int t = 0; t < TPW; ++t) mx[t] = entry[1 + t];
+        } else {
+            mg = expand_half_mask(gok ? gbits : 0u);
+#pragma unroll
+            for (int t = 0; t < TPW; ++t) mx[t] = expand_half_mask(xok ? xbits[t] : 0u);
+        }
 #pragma unroll
         for (int i = 0; i < MT; ++i) lgoff[i] = (unsigned int)(gok ? goff[i] : 0);
 #pragma unroll
@@ -1042,6 +1065,12 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_wgrad_f16_kernel(const Wgrad
         constexpr int NEL = 7 * SW + TPW;  // input pixels one chunk touches over all taps of the group
         const WgChunk c = wg_chunk(P, tile, j);
         const int glin = P.flat ? c.wo0 : c.ho * Wo + c.wo0, lin = xlin(c);
+        if (P.flat) {
+            const u32x2 entry = *reinterpret_cast<const u32x2*>(fbits + 2 * (c.wo0 >> 3));
+            gbits = c.live ? entry[1] : 0u;
+#pragma unroll
+            for (int t = 0; t < TPW; ++t) xbits[t] = c.live ? (entry[0] >> (8 * t)) & 0xFFu : 0u;
+        }
 #pragma unroll 2
         for (int e = 0; e < GE; ++e) {
             const int q = e / MT, cc = (e % MT) * 32;

@@ -844,6 +844,17 @@ static bool plan_wgrad_f16(const Problem& p, WgPlan& best) {
     best.CoP = best.co_tiles * CoT; best.CiP = best.ci_tiles * CiT;
     best.groups_per_row = cdiv(p.kw, best.TPW);
     best.lds_bytes = (size_t)(4 * CoT + best.TPW * 4 * CiT) * 72 * 2;
+    if (best.flat) {  // the kernel keeps the masks of a plane's chunks in LDS: small planes only (large ones waste little)
+        const size_t tables = (size_t)(best.cpr + 1) * (best.TPW + 1) * 16 + (size_t)best.cpr * 8;
+        if (best.lds_bytes + tables <= 160 * 1024) {
+            best.lds_bytes += tables;
+        } else {
+            best.flat = false;
+            best.cpr = cdiv(p.wo, 8);
+            best.nchunks = (int)((long)p.n * p.ho * best.cpr);
+            best.ntiles = cdiv(best.nchunks, 8);
+        }
+    }
     // one round of workgroups: as many reduction slices as fill every CU once (twice where two workgroups fit),
     // which keeps the partial sums small and lets no CU wait for a straggler round
     const int xy = best.co_tiles * best.ci_tiles * best.groups_per_row * p.kh;
