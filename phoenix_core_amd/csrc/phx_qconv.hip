@@ -538,6 +538,12 @@ static bool plan_corr_uncached(const Corr& creal, int mode, bool f16mfma, Corr& 
     // 32-128 channels: 0.15-0.18 ms against 0.08-0.11 ms), so the 8-product mode takes that one here as well
     const bool zero_inserted = c.uh > 1 || c.uw > 1;
     pl.kmode = (f16mfma && mode == 8 && zero_inserted && c.Kh * c.Kw > 1 && !tune().zi8) ? 16 : mode;
+    // Real-valued input (one stored component) on fp16 matrix cores: the factorized kernel forms its lanes from one
+    // real and three zero components for nothing; the 16-product kernel is the faster one (q-ResNet-50 stem, 7x7
+    // stride 2 on 3 channels by space-to-depth: 0.19 against 0.30 ms).  Skipping the twelve products with the absent
+    // components as well would need a kernel variant of its own: a run-time branch around them slowed every
+    // 16-product convolution by 5-15 %.
+    if (f16mfma && mode == 8 && c.ncomp == 1 && !tune().zi8) pl.kmode = 16;
     return plan_forward(c, pl.kmode, f16mfma, pl);
 }
 
