@@ -643,3 +643,51 @@ def test_verbose_names_mode_policy_and_kernel(tune_env, capfd):
     assert "forward" in lines[0] and "product mode 8" in lines[0] and "fp16 policy full16" in lines[0]
     assert any("filter gradient" in l for l in lines[1:]) and any("input gradient" in l for l in lines[1:])
     assert capi.last_kernel_name() in lines[2]
+
+
+# name, n, ci, co, h, w, kh, kw, stride, dilation, padding -- unit strides, rows of equal length >= 7 in and out whose
+# length is not a multiple of 8
+FLAT_WGRAD = [
+    ("wg_7", 5, 24, 24, 7, 7, 3, 3, 1, 1, "SAME"),                 # a chunk always runs over a row end
+    ("wg_9x11", 3, 16, 40, 9, 11, 3, 3, 1, 1, "SAME"),
+    ("wg_14", 4, 64, 64, 14, 14, 3, 3, 1, 1, "SAME"),              # 64x64 channel tile
+    ("wg_28", 2, 64, 96, 28, 28, 3, 3, 1, 1, "SAME"),
+    ("wg_dil2", 2, 16, 16, 12, 13, 3, 3, 1, 2, "SAME"),            # one tap per workgroup, columns two apart
+    ("wg_asym", 2, 8, 8, 10, 15, 3, 3, 1, 1, (0, 2, 2, 0)),        # all padding on one side
+    ("wg_k5", 2, 8, 12, 9, 12, 5, 5, 1, 1, "SAME"),                # two rows of padding
+    ("wg_k4", 3, 12, 16, 11, 10, 4, 4, 1, 1, (1, 1, 2, 2)),        # four taps per workgroup
+]
+
+
+@pytest.mark.parametrize("real_input", [False, True], ids=["quat", "real"])
+@pytest.mark.parametrize("case", FLAT_WGRAD, ids=lambda c: c[0])
+def test_flat_chunk_list_of_the_filter_gradient(case, real_input, tune_env):
+    """The fp16 filter gradient cuts whole image planes, not rows, into its 8-pixel chunks where rows do not fill
+    their last chunk (csrc/phx_kernels_f16.h, WgradArgs::flat; PHX_TUNE_NOFLAT keeps the rows): per-tap pixel masks
+    stand in for the row structure.  Both chunk lists against the oracle and against each other."""
+    name, n, ci, co, h, w, kh, kw, stride, dilation, padding = case
+    dtype = torch.float16
+    g, x, wt, b, gr = make_inputs(name_seed(name) + 17, n, ci, co, h, w, kh, kw, stride, dilation, padding, dtype, 0.5)
+    assert (g.ho, g.wo) == (h, w)
+    if real_input:
+        x = np.ascontiguousarray(x[:n])
+    desc = phx.Conv2DDescriptor(x.shape, wt.shape, stride, dilation, padding, dtype=dtype, context=Ctx(8, "full16"),
+                                real_valued_input=real_input, require_input_grad=False)
+    xd, wd, gd = (torch.from_numpy(a).cuda() for a in (x, wt, gr))
+    x4 = np.zeros((4 * n,) + x.shape[1:], np.float64)
+    x4[:x.shape[0]] = x
+    want_dw, _ = oracle.conv2d_bwd(g, x4, wt.astype(np.float64), gr.astype(np.float64), "hamilton", need_dx=False)
+    got = {}
+    for variant, env in (("planes", None), ("rows", "PHX_TUNE_NOFLAT")):
+        tune_env(PHX_TUNE_NOFLAT=None)
+        if env:
+            tune_env(**{env: "1"})
+        dw, _ = phx.conv2d_bwd(xd, wd, gd, desc)
+        k = capi.last_kernel_name()
+        print(name, variant, k, flush=True)
+        assert ("_flat" in k) == (variant == "planes"), k
+        assert_close(dw.cpu().numpy(), want_dw, dtype, "wgrad " + k)
+        got[variant] = dw.double()
+    # the same products, summed over differently cut chunks: equal up to fp32 summation order
+    scale = got["rows"].abs().max().item()
+    assert (got["planes"] - got["rows"]).abs().max().item() <= 2e-3 * scale
