@@ -79,7 +79,7 @@ def parse():
     ap.add_argument("--batch", type=int, default=64, help="images per step of the ResNet workload")
     ap.add_argument("--torch-bn", action="store_true",
                     help="ResNet workload: torch.nn.BatchNorm2d + ReLU (MIOpen) instead of the library's batch-norm kernels")
-    ap.add_argument("--no-graph", action="store_true", help="ResNet workload: time the eager step only (no HIP graph replay)")
+    ap.add_argument("--no-graph", action="store_true", help="time the eager steps only (no HIP graph replay)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch a plain 256 MiB device copy (untimed), the yardstick for HBM byte counters")
@@ -176,25 +176,77 @@ def cpu_baseline_dense(cfg, mode, seconds):
 
 
 class _Timed:
-    """Runs `step` (which makes ncalls library calls) warmup + steps times and returns wall-clock
-    milliseconds per step and, per call slot, the mean HIP-event duration of its dominant kernel."""
+    """Runs `step` (which makes ncalls library calls) and returns wall-clock milliseconds per step and, per call
+    slot, the mean HIP-event duration of its dominant kernel.  Three passes of `steps` steps each: eager without
+    the library's event timer (its event records sit between the kernels), eager with it (kernel durations), and --
+    where `outputs` is given and graphs are not switched off -- the step replayed from a HIP graph, trusted only if
+    every checked replay reproduces the eager outputs bit for bit; `ms_per_step` is the faster of eager and replay."""
 
-    def __init__(self, step, ncalls, steps, warmup):
+    def __init__(self, step, ncalls, steps, warmup, outputs=None, use_graph=True):
         import torch
         from phoenix_core_amd import capi
         for _ in range(warmup):
             step()
         torch.cuda.synchronize()
-        capi.profile_enable(ncalls * steps)
-        torch.cuda.synchronize()
         t0 = time.perf_counter()
         for _ in range(steps):
             step()
         torch.cuda.synchronize()
-        self.ms_per_step = (time.perf_counter() - t0) / steps * 1e3
+        self.ms_per_step_eager = (time.perf_counter() - t0) / steps * 1e3
+        capi.profile_enable(ncalls * steps)
+        torch.cuda.synchronize()
+        for _ in range(steps):
+            step()
+        torch.cuda.synchronize()
         ms = capi.profile_collect(ncalls * steps)
         capi.profile_enable(0)
         self.kernel_ms = [sum(ms[i::ncalls]) / max(1, len(ms[i::ncalls])) for i in range(ncalls)]
+        self.ms_per_step = self.ms_per_step_eager
+        self.graph = {"used": False, "note": "not attempted"}
+        if outputs is not None and use_graph:
+            self.graph = self._replay(step, steps, warmup, outputs)
+            # (a step of a few launches can be faster eagerly: the figure reported is the faster of the two ways)
+            if self.graph["used"] and self.graph["ms_per_step"] < self.ms_per_step_eager:
+                self.ms_per_step = self.graph["ms_per_step"]
+            self.graph["reported"] = "hip_graph_replay" if self.ms_per_step != self.ms_per_step_eager else "eager"
+
+    @staticmethod
+    def _replay(step, steps, warmup, outputs):
+        import torch
+        from phoenix_core_amd import capi
+        try:
+            capi.init()
+            want = [t.clone() for t in outputs()]
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                step()
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=side):
+                step()
+            for _ in range(3):
+                for t in outputs():
+                    t.zero_()
+                torch.cuda.synchronize()
+                graph.replay()
+                torch.cuda.synchronize()
+                if not all(torch.equal(a, b) for a, b in zip(outputs(), want)):
+                    return {"used": False, "note": "a replay did not reproduce the eager outputs"}
+                step()  # eager work of the program between the replays
+                torch.cuda.synchronize()
+            for _ in range(max(warmup, 3)):
+                graph.replay()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                graph.replay()
+            torch.cuda.synchronize()
+            return {"used": True, "ms_per_step": (time.perf_counter() - t0) / steps * 1e3, "replays_checked": 3,
+                    "note": "every checked replay reproduced the eager outputs bit for bit"}
+        except Exception as exc:  # capture is an optimisation: any failure leaves the eager figure standing
+            return {"used": False, "note": "capture or replay failed: %s" % (str(exc)[:200],)}
 
 
 def roofline_of(pass_name, kernel, flops, nbytes, kernel_ms, compute, traffic):
@@ -251,12 +303,12 @@ def run_conv(name, mode, policy, args, traffic_table):
     L = capi.lib()
     sizes = [desc.workspace_bytes(p) for p in (capi.PHX_PASS_FWD, capi.PHX_PASS_BWD_DATA, capi.PHX_PASS_BWD_WEIGHTS)]
     ws = torch.empty(max(sizes + [1]), dtype=torch.uint8, device=dev)
-    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     P = lambda t: ctypes.c_void_p(t.data_ptr())
     d = ctypes.byref(desc.c)
     names = {}
 
     def step():
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)  # (the capture stream during a graph capture)
         capi.check(L.phx_qconv2d_fwd(d, stream, P(x), P(wt), None, P(y), P(ws), sizes[0]), "fwd")
         names.setdefault("fwd", capi.last_kernel_name())
         capi.check(L.phx_qconv2d_bwd_data(d, stream, P(gr), P(wt), P(dx), P(ws), sizes[1]), "bwd_data")
@@ -270,7 +322,7 @@ def run_conv(name, mode, policy, args, traffic_table):
         for _ in range(3):
             dst.copy_(src)  # reads 256 MiB, writes 256 MiB
         del src, dst
-    t = _Timed(step, 3, args.steps, args.warmup)
+    t = _Timed(step, 3, args.steps, args.warmup, outputs=lambda: (y, dx, dw), use_graph=not args.no_graph)
     flops_pass = 2.0 * 16 * n * co * ci * ho * wo * k * k
     esize = 4 if dt == "f32" else 2
     # algorithmic bytes of a pass: read the activations (or the gradient), read the filters, write the result
@@ -292,7 +344,8 @@ def run_conv(name, mode, policy, args, traffic_table):
         "workload": "%s: quaternion conv %dx%d stride 1, N=%d (4N=%d rows), %d->%d q-channels, %dx%d, "
                     "fwd+input-grad+filter-grad" % (name, k, k, n, 4 * n, ci, co, h, w),
         "product_mode": mode, "fp16_policy": policy, "padding": padding, "dtype": dt,
-        "value": value, "unit": "TFLOP/s", "ms_per_step": t.ms_per_step, "images_per_s": n / (t.ms_per_step * 1e-3),
+        "value": value, "unit": "TFLOP/s", "ms_per_step": t.ms_per_step, "ms_per_step_eager": t.ms_per_step_eager,
+        "hip_graph": t.graph, "images_per_s": n / (t.ms_per_step * 1e-3),
         "kernel_ms": per_pass, "kernels": names,
         "real_equiv_tflops": {p: roofs[p]["real_equiv_tflops"] for p in PASSES},
         "frac_of_mfma_peak": {p: roofs[p]["frac_of_mfma_peak"] for p in PASSES},
@@ -321,12 +374,12 @@ def run_dense(name, mode, args, traffic_table):
     L = capi.lib()
     sizes = [desc.workspace_bytes(p) for p in (capi.PHX_PASS_FWD, capi.PHX_PASS_BWD_DATA, capi.PHX_PASS_BWD_WEIGHTS)]
     ws = torch.empty(max(sizes + [1]), dtype=torch.uint8, device=dev)
-    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     P = lambda t: ctypes.c_void_p(t.data_ptr())
     d = ctypes.byref(desc.c)
     names = {}
 
     def step():
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)  # (the capture stream during a graph capture)
         capi.check(L.phx_qdense_fwd(d, stream, P(x), P(wt), P(b), P(y), P(ws), sizes[0]), "fwd")
         names.setdefault("fwd", capi.last_kernel_name())
         capi.check(L.phx_qdense_bwd_data(d, stream, P(gr), P(wt), P(dx), P(ws), sizes[1]), "bwd_data")
@@ -334,7 +387,7 @@ def run_dense(name, mode, args, traffic_table):
         capi.check(L.phx_qdense_bwd_weights(d, stream, P(x), P(gr), P(dw), P(ws), sizes[2]), "bwd_weights")
         names.setdefault("bwd_weights", capi.last_kernel_name())
 
-    t = _Timed(step, 3, args.steps, args.warmup)
+    t = _Timed(step, 3, args.steps, args.warmup, outputs=lambda: (y, dx, dw), use_graph=not args.no_graph)
     flops_pass = 2.0 * 16 * n * ni * no
     bytes_pass = {"fwd": 4 * (x.numel() + wt.numel() + b.numel() + y.numel()),
                   "bwd_data": 4 * (gr.numel() + wt.numel() + dx.numel()),
@@ -348,10 +401,11 @@ def run_dense(name, mode, args, traffic_table):
                     "fwd+input-grad+filter-grad" % (name, n, 4 * n, ni, no),
         "product_mode": mode, "fp16_policy": "fp32", "dtype": dt,
         "value": 3 * flops_pass / (t.ms_per_step * 1e-3) / 1e12, "unit": "TFLOP/s", "ms_per_step": t.ms_per_step,
+        "ms_per_step_eager": t.ms_per_step_eager, "hip_graph": t.graph,
         "kernel_ms": per_pass, "kernels": names,
         "real_equiv_tflops": {p: roofs[p]["real_equiv_tflops"] for p in PASSES},
         "roofline": roofs[dominant],
-        "note": "16.8 MFLOP per pass: three kernel launches of a few microseconds each, launch-latency bound",
+        "note": "16.8 MFLOP per pass: a handful of kernel launches of a few microseconds each, launch-latency bound",
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline_dense(DENSE[name], mode, args.cpu_seconds)
