@@ -15,6 +15,11 @@
 //     (columns = output channels), so a lane receives, for ONE output channel, eight consecutive pixels per group
 //     of four accumulator registers (the two pixels of its pair x four row registers interleave exactly so): one
 //     16-byte store per group, no cross-lane shuffle;
+//   * stored like that, the 64 lanes of a store instruction would write 32 channel rows x 32 bytes: four
+//     instructions to complete a 128-byte line, and the address path handles a line at a time.  So a wave passes
+//     each component's 4 KB through a small LDS buffer of its own ([channel][8-pixel piece], rows padded by one
+//     piece against bank conflicts) and reads it back with the lanes along the pixels: a store instruction then
+//     writes 8 channel rows x 128 bytes (WCO > 1; the 256-pixel tiles of WCO == 1 have no LDS to spare);
 //   * a wave owns 32 output channels x 64 pixels x 4 output components = 8 accumulator tiles (128 registers),
 //     so two workgroups fit a CU and one's stores and start-up run under the other's products;
 //   * pixels are addressed in groups of 8 (one 16-byte copy lane); an image whose plane is not a multiple of 8
@@ -60,13 +65,20 @@ struct PwxShape {
     static constexpr int NXI = 2 * WPX;          // activation copy instructions per wave and stage
     static constexpr int NPS = NWI + NXI;
     static constexpr size_t lds_bytes = (size_t)R * SV * 16;
+    // NCHW kernel: a ring of two stages does as well as three (a K step is bound by the copy instructions' issue
+    // and the barrier, not by the copies' latency), which leaves room for the store transposition below
+    static constexpr bool TSTORE = WCO > 1;      // stores regrouped through LDS into whole channel rows
+    static constexpr int RN = 2;
+    static constexpr int SCRV = 32 * 9;          // 16-byte vectors of a wave's transposition buffer: 32 channels x (8 + 1) pieces
+    static constexpr size_t lds_bytes_nchw = (size_t)RN * SV * 16 + (TSTORE ? 4 * SCRV * 16 : 0);
 };
 
 template <int WCO>
 __global__ void __launch_bounds__(WG_THREADS, 2) qconv_pwx_f16_kernel(const PwxArgs P) {
     using S = PwxShape<WCO>;
-    constexpr int WPX = S::WPX, GPT = S::GPT, ROWDW = S::ROWDW, WV = S::WV, SV = S::SV, R = S::R, D = R - 1;
+    constexpr int WPX = S::WPX, GPT = S::GPT, ROWDW = S::ROWDW, WV = S::WV, SV = S::SV, R = S::RN, D = R - 1;
     constexpr int RPI = 64 / GPT;  // activation rows one copy instruction covers
+    constexpr bool TSTORE = S::TSTORE;
     extern __shared__ f16x8 lds16[];
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -126,18 +138,23 @@ __global__ void __launch_bounds__(WG_THREADS, 2) qconv_pwx_f16_kernel(const PwxA
     // output channel j of the wave's 32, register e = pixel row 8*(e/4) + 4*kk + e%4, i.e. pixel 2*row + m.  The four
     // registers of a group e/4, for m = 0 and 1, are therefore EIGHT CONSECUTIVE pixels 16*(e/4) + 8*kk .. + 7 of one
     // output channel: one 16-byte store, no cross-lane traffic at all.
-    long oaddr[4] = {0, 0, 0, 0};  // per register group: element offset of its 8-pixel group in an output component
-    bool ovalid[4] = {false, false, false, false};
+    // (TSTORE: after the transposition a lane stores piece lane % 8 of the wave's 8 pixel groups, for channel
+    // 8*i + lane / 8 in its i-th store: one address)
+    constexpr int NOA = TSTORE ? 1 : 4;
+    long oaddr[NOA];    // per register group: element offset of its 8-pixel group in an output component
+    bool ovalid[NOA];
+#pragma unroll
+    for (int a = 0; a < NOA; ++a) { oaddr[a] = 0; ovalid[a] = false; }
     int c_item = wg, c_k = 0, c_ct = 0;
     auto locate_out = [&](int item) {
         const int tile = item / P.co_tiles;
         c_ct = item - tile * P.co_tiles;
 #pragma unroll
-        for (int g4 = 0; g4 < 4; ++g4) {
-            const int gg = tile * GPT + wpx * 8 + 2 * g4 + kk;
-            ovalid[g4] = gg < P.TGp;
+        for (int a = 0; a < NOA; ++a) {
+            const int gg = tile * GPT + wpx * 8 + (TSTORE ? (lane & 7) : 2 * a + kk);
+            ovalid[a] = gg < P.TGp;
             const int n = gg / P.GI, gi = gg - n * P.GI;
-            oaddr[g4] = ((long)n * P.CoutS) * HW + min(gi * 8, HW - 8);
+            oaddr[a] = ((long)n * P.CoutS) * HW + min(gi * 8, HW - 8);
         }
     };
 
@@ -226,8 +243,10 @@ __global__ void __launch_bounds__(WG_THREADS, 2) qconv_pwx_f16_kernel(const PwxA
             wait_vmem_all();  // this wave's copies of the next D stages: landed
             covered = D;
             PHX_STAMP(2)
-            const int co = (c_ct * WCO + wco) * 32 + j;
+            const int co0 = (c_ct * WCO + wco) * 32;
+            const int co = co0 + j;
             const bool co_ok = co < P.Cout;
+            u32x4* scr = reinterpret_cast<u32x4*>(lds16 + R * SV) + wave * S::SCRV;  // (TSTORE) this wave's own
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
                 const float bv = (P.bias && co_ok) ? (float)P.bias[q * P.CoutS + co] : 0.f;
@@ -242,7 +261,21 @@ __global__ void __launch_bounds__(WG_THREADS, 2) qconv_pwx_f16_kernel(const PwxA
                         h[1] = (_Float16)(acc[q][1][g4 * 4 + k] + bv);
                         v[k] = __builtin_bit_cast(unsigned int, h);
                     }
-                    if (ovalid[g4] && co_ok) *reinterpret_cast<u32x4_a2*>(dst + oaddr[g4]) = v;
+                    if constexpr (TSTORE) scr[j * 9 + 2 * g4 + kk] = v;  // channel j, piece 2*g4 + kk
+                    else if (ovalid[g4] && co_ok) *reinterpret_cast<u32x4_a2*>(dst + oaddr[g4]) = v;
+                }
+                if constexpr (TSTORE) {
+                    // (LDS serves a wave's accesses in order: the reads see the writes above, and the next
+                    // component's writes come after these reads)
+                    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const int c = 8 * i + (lane >> 3);
+                        const u32x4 t = scr[c * 9 + (lane & 7)];
+                        if (ovalid[0] && co0 + c < P.Cout)
+                            *reinterpret_cast<u32x4_a2*>(P.out + q * P.out_cs + (long)(co0 + c) * HW + oaddr[0]) = t;
+                    }
+                    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
                 }
             }
             c_k = 0;

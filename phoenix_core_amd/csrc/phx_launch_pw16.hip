@@ -7,8 +7,8 @@ namespace phx {
 template <int WCO>
 static int launch_pwx_one(const PwxArgs& a, int blocks, hipStream_t st) {
     constexpr auto kernel = qconv_pwx_f16_kernel<WCO>;
-    if (!BigLds<kernel>::registered) return -1;  // 72 KiB of dynamic LDS: opted in per device at set-up, see BigLds
-    hipLaunchKernelGGL(kernel, dim3(blocks), dim3(WG_THREADS), PwxShape<WCO>::lds_bytes, st, a);
+    if (!BigLds<kernel>::registered) return -1;  // more than 64 KiB of dynamic LDS: opted in per device at set-up, see BigLds
+    hipLaunchKernelGGL(kernel, dim3(blocks), dim3(WG_THREADS), PwxShape<WCO>::lds_bytes_nchw, st, a);
     return 0;
 }
 
