@@ -5,8 +5,8 @@
 // filter that is the same everywhere, so the kernel is built around the data path, not around a halo window:
 //   * both operands reach LDS by the register-less copy path (global_load_lds, 16 bytes per lane), activations
 //     exactly as they lie in NCHW memory -- rows of (component, channel) x consecutive pixels, no transposition,
-//     no masks, no staging registers; a ring of stages (one 16-channel K step each) keeps the copies two steps
-//     ahead of the matrix instructions, one barrier per step;
+//     no masks, no staging registers; a ring of stages (one 16-channel K step each) keeps the copies ahead of the
+//     matrix instructions (one step here, two in the channels-last kernel), one barrier per step;
 //   * the MFMA B operand wants 8 consecutive channels of one pixel per lane, NCHW has 8 consecutive pixels of one
 //     channel: the transposition happens on the way from LDS to the registers.  A lane owns TWO neighbouring
 //     pixels: it reads one dword (two pixels) per channel, and byte permutes split the eight dwords of a channel
@@ -60,7 +60,7 @@ struct PwxShape {
     static constexpr int WV = WCO * 4 * 64;      // 16-byte vectors of one filter stage
     static constexpr int XV = 64 * GPT;          // 16-byte vectors of one activation stage: 64 rows (4 components x 16 channels)
     static constexpr int SV = WV + XV;
-    static constexpr int R = (WCO == 1) ? 2 : 3; // ring stages (two workgroups per CU: at most 80 KiB each)
+    static constexpr int R = (WCO == 1) ? 2 : 3; // ring stages of the channels-last kernel (two workgroups per CU: at most 80 KiB each)
     static constexpr int NWI = WCO;              // filter copy instructions per wave and stage
     static constexpr int NXI = 2 * WPX;          // activation copy instructions per wave and stage
     static constexpr int NPS = NWI + NXI;
