@@ -159,15 +159,6 @@ __device__ __forceinline__ void merge_output(const V (&P)[8], V (&y)[4]) {
     y[3] = a5 - P[2] + P[7];
 }
 
-// 8 lane gradients -> left-operand (input) gradient
-template <typename V>
-__device__ __forceinline__ void merge_left_grad(const V (&d)[8], V (&y)[4]) {
-    y[0] = d[1] + d[2] + d[5] + d[6];
-    y[1] = d[0] - d[3] + d[5] - d[6];
-    y[2] = d[2] - d[1] - d[4] + d[7];
-    y[3] = d[0] + d[3] + d[4] + d[7];
-}
-
 // 8 lane gradients -> right-operand (filter) gradient
 template <typename V>
 __device__ __forceinline__ void merge_right_grad(const V (&d)[8], V (&y)[4]) {

@@ -116,7 +116,7 @@ __device__ __forceinline__ void stage_store16_pairs(f16x8* dst, const unsigned i
 //   MODE 16: 16 MFMAs per step and column tile, the four filter components reused across the
 //            4x4 block, negative entries by flipping the sign bits of the activation operand.
 //   MODE 8 : 8 MFMAs per step and column tile on lanes formed with packed fp16 adds.
-template <int MODE, int MAP, int WCO, int NTW, int P2LOG, bool PAIRS>
+template <int MODE, int WCO, int NTW, int P2LOG, bool PAIRS>
 __global__ void __launch_bounds__(WG_THREADS, (MODE == 8 || NTW == 1) ? 2 : 1) qconv_fwd_f16_kernel(const ConvArgs P) {
     constexpr int CK = F16_CK;
     constexpr int WPX = 4 / WCO;
@@ -211,8 +211,7 @@ __global__ void __launch_bounds__(WG_THREADS, (MODE == 8 || NTW == 1) ? 2 : 1) q
                                                                                acc[t][q], 0, 0, 0);
                 } else {
                     f16x8 L[8];
-                    if constexpr (MAP == MAP_FWD) lanes_left(x, L);
-                    else lanes_grad(x, L, (_Float16)0.5f);
+                    lanes_left(x, L);
 #pragma unroll
                     for (int i = 0; i < 8; ++i)
                         acc[t][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wcur[i], L[i], acc[t][i], 0, 0, 0);
@@ -225,13 +224,14 @@ __global__ void __launch_bounds__(WG_THREADS, (MODE == 8 || NTW == 1) ? 2 : 1) q
         }
     }
 
-    conv_epilogue<_Float16, MODE, MAP, NTW, NACC>(P, acc, (ct * WCO + wco) * 32 + 4 * kk, oaddr, pvalid);
+    conv_epilogue<_Float16, MODE, NTW, NACC>(P, acc, (ct * WCO + wco) * 32 + 4 * kk, oaddr, pvalid);
 }
 
 // Filter packing for the kernel above: one group of WC 16-byte vectors per (32-channel filter
 // tile, K step, lane); lane = (row = lane % 32, kk = lane / 32), K step = chunk*taps + tap,
 // vector element i = reduced channel chunk*16 + kk*8 + i.  MODE 16: the four filter components
-// (conjugated for MAP_DGRAD); MODE 8: the eight right-operand lanes, formed in fp32 and rounded once.
+// MODE 8: the eight right-operand lanes, formed in fp32 and rounded once (both of the conjugated filter for
+// MAP_DGRAD: dx = g (x) conj(w) is a forward product, and the forward kernel runs it).
 template <int MODE, int MAP>
 __global__ void __launch_bounds__(WG_THREADS) pack_filters_f16_kernel(const PackArgs P) {
     constexpr int WC = (MODE == 16) ? 4 : 8;
@@ -262,14 +262,11 @@ __global__ void __launch_bounds__(WG_THREADS) pack_filters_f16_kernel(const Pack
                 const int in = (MAP == MAP_DGRAD) ? row : red;
                 const long off = o * P.so + in * P.si + kh * P.skh + kw * P.skw;
 #pragma unroll
-                for (int r = 0; r < 4; ++r) wv[r] = (float)w[r * P.wcs + off];
+                for (int r = 0; r < 4; ++r) wv[r] = ((MAP == MAP_DGRAD && r > 0) ? -1.f : 1.f) * (float)w[r * P.wcs + off];
             }
             if constexpr (MODE == 16) {
-                const float sgn = (MAP == MAP_DGRAD) ? -1.f : 1.f;
-                vec[0][i] = (_Float16)wv[0];
-                vec[1][i] = (_Float16)(sgn * wv[1]);
-                vec[2][i] = (_Float16)(sgn * wv[2]);
-                vec[3][i] = (_Float16)(sgn * wv[3]);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) vec[r][i] = (_Float16)wv[r];
             } else {
                 float R[8];
                 lanes_right(wv, R);
@@ -393,42 +390,24 @@ __device__ __forceinline__ void stage_chunk_store(f16x8* xl, const u32x4 (&r)[8]
     }
 }
 
-// One eighth of the left-operand lane map of the factorized product: step i leaves lane i ready
-// (forward: lanes_left; input gradient: lanes_grad without the factor 1/2, which the packed filters
-// carry; T holds its four partial sums between steps).
-template <int MAP>
-__device__ __forceinline__ void lane_step(const f16x8 (&x)[4], f16x8 (&L)[8], f16x8 (&T)[4], int i) {
-    if constexpr (MAP == MAP_FWD) {
-        switch (i) {
-            case 0: L[0] = add8_pinned(x[3], x[1]); break;
-            case 1: L[1] = sub8_pinned(x[0], x[2]); break;
-            case 2: L[2] = add8_pinned(x[0], x[2]); break;
-            case 3: L[3] = sub8_pinned(x[3], x[1]); break;
-            case 4: L[4] = sub8_pinned(x[3], x[2]); break;
-            case 5: L[5] = add8_pinned(x[1], x[0]); break;
-            case 6: L[6] = sub8_pinned(x[0], x[1]); break;
-            default: L[7] = add8_pinned(x[3], x[2]); break;
-        }
-    } else {
-        // the plain copies (lanes 4..7) first: they free the component registers for the next request;
-        // T = {g0+g1, g2+g3, g0-g1, g2-g3}
-        switch (i) {
-            case 0: L[4] = x[0]; L[5] = x[1]; T[0] = add8_pinned(x[0], x[1]); break;
-            case 1: L[6] = x[2]; L[7] = x[3]; T[1] = add8_pinned(x[2], x[3]); break;
-            case 2: T[2] = sub8_pinned(x[0], x[1]); break;
-            case 3: T[3] = sub8_pinned(x[2], x[3]); break;
-            case 4: L[0] = sub8_pinned(T[1], T[0]); break;
-            case 5: L[1] = sub8_pinned(T[2], T[3]); break;
-            case 6: L[2] = add8_pinned(T[2], T[3]); break;
-            default: L[3] = add8_pinned(T[0], T[1]); break;
-        }
+// One eighth of the left-operand lane map of the factorized product (lanes_left): step i leaves lane i ready.
+__device__ __forceinline__ void lane_step(const f16x8 (&x)[4], f16x8 (&L)[8], int i) {
+    switch (i) {
+        case 0: L[0] = add8_pinned(x[3], x[1]); break;
+        case 1: L[1] = sub8_pinned(x[0], x[2]); break;
+        case 2: L[2] = add8_pinned(x[0], x[2]); break;
+        case 3: L[3] = sub8_pinned(x[3], x[1]); break;
+        case 4: L[4] = sub8_pinned(x[3], x[2]); break;
+        case 5: L[5] = add8_pinned(x[1], x[0]); break;
+        case 6: L[6] = sub8_pinned(x[0], x[1]); break;
+        default: L[7] = add8_pinned(x[3], x[2]); break;
     }
 }
 
 // EARLY (chunk staging, problems with one filter group per chunk, i.e. pointwise ones): only the products of one
 // group stand between the request for the next chunk's activations and their use, so the request goes out at the
 // start of the group, ahead of the filter copy (which the same wait then covers).
-template <int MODE, int MAP, int WCO, int NTW, int P2LOG, bool CHUNKS, bool EARLY = false>
+template <int MODE, int WCO, int NTW, int P2LOG, bool CHUNKS, bool EARLY = false>
 __global__ void __launch_bounds__(WG_THREADS, (MODE == 16 && NTW == 1) ? 2 : 1) qconv_fwd_f16_lds_kernel(const ConvArgs P) {
     static_assert(!EARLY || CHUNKS, "early activation requests belong to chunk staging");
     constexpr int CK = F16_CK;
@@ -536,7 +515,7 @@ __global__ void __launch_bounds__(WG_THREADS, (MODE == 16 && NTW == 1) ? 2 : 1) 
     // that pipeline runs on across the group boundary (CARRY; it needs an even number of blocks per group
     // so that the register double buffers keep their parity).
     constexpr bool CARRY = MODE == 8 && (TG * NTW) % 2 == 0;
-    f16x8 xf[2][4], Lf[MODE == 8 ? 2 : 1][8], Lt[4];
+    f16x8 xf[2][4], Lf[MODE == 8 ? 2 : 1][8];
     bool carried = false;      // the previous group left this group's first lanes and components in registers
     // one flat loop over (chunk, filter group) steps: a single loop keeps the accumulators in place
     for (int gs = 0; gs < total_groups; ++gs) {
@@ -606,7 +585,7 @@ __global__ void __launch_bounds__(WG_THREADS, (MODE == 16 && NTW == 1) ? 2 : 1) 
                     read_x(xf[0], 0);
                     if (NBLK > 1) read_x(xf[1], 1);
 #pragma unroll
-                    for (int i = 0; i < 8; ++i) lane_step<MAP>(xf[0], Lf[0], Lt, i);
+                    for (int i = 0; i < 8; ++i) lane_step(xf[0], Lf[0], i);
                 }
                 __builtin_amdgcn_sched_barrier(0);
                 if (NBLK > 2) read_x(xf[0], 2);
@@ -683,7 +662,7 @@ __global__ void __launch_bounds__(WG_THREADS, (MODE == 16 && NTW == 1) ? 2 : 1) 
 #pragma unroll
                     for (int i = 0; i < 8; ++i) {
                         acc[t][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(w[i], Lf[blk & 1][i], acc[t][i], 0, 0, 0);
-                        if (blk + 1 < NBLK || carry) lane_step<MAP>(xf[(blk + 1) & 1], Lf[(blk + 1) & 1], Lt, i);
+                        if (blk + 1 < NBLK || carry) lane_step(xf[(blk + 1) & 1], Lf[(blk + 1) & 1], i);
                         __builtin_amdgcn_sched_barrier(0);
                         // (last block: after the lane arithmetic, whose waits sit behind run-time branches there
                         // and are therefore complete ones)
@@ -709,7 +688,7 @@ __global__ void __launch_bounds__(WG_THREADS, (MODE == 16 && NTW == 1) ? 2 : 1) 
         if (++g == ngroups) { g = 0; ++chunk; }
     }
 
-    conv_epilogue<_Float16, MODE, MAP, NTW, NW>(P, acc, (ct * WCO + wco) * 32 + 4 * kk, oaddr, pvalid);
+    conv_epilogue<_Float16, MODE, NTW, NW>(P, acc, (ct * WCO + wco) * 32 + 4 * kk, oaddr, pvalid);
 #ifdef PHX_PHASE_TIMING
     __builtin_amdgcn_s_waitcnt(0x0F70);  // (charge the stores to the epilogue; otherwise the wave ends with them in flight)
 #endif
@@ -777,13 +756,15 @@ __global__ void __launch_bounds__(WG_THREADS) pack_filters_f16_lds_kernel(const 
                         const float sgn = (MAP == MAP_DGRAD && r > 0) ? -1.f : 1.f;  // conjugate
                         vec[0][i] = (_Float16)(sgn * (float)w[r * P.wcs + off]);
                     } else {
+                        // input gradient: dx = g (x) conj(w) is the forward product of the gradient with the
+                        // conjugated filter, so the forward kernel serves it and only the packing differs
                         float wv[4], R[8];
 #pragma unroll
-                        for (int c = 0; c < 4; ++c) wv[c] = (float)w[c * P.wcs + off];
+                        for (int c = 0; c < 4; ++c)
+                            wv[c] = ((MAP == MAP_DGRAD && c > 0) ? -1.f : 1.f) * (float)w[c * P.wcs + off];
                         lanes_right(wv, R);  // formed in fp32, rounded once
-                        // input gradient: the kernel forms the gradient lanes 0..3 without their factor 1/2
 #pragma unroll
-                        for (int q = 0; q < 8; ++q) vec[q][i] = (_Float16)((MAP == MAP_DGRAD && q < 4) ? 0.5f * R[q] : R[q]);
+                        for (int q = 0; q < 8; ++q) vec[q][i] = (_Float16)R[q];
                     }
                 }
             }

@@ -84,7 +84,7 @@ __device__ __forceinline__ void store_pixels(TS* ptr, const float (&v)[V]) {
     }
 }
 
-template <typename TS, int MODE, int MAP, int NTW, int NACC>
+template <typename TS, int MODE, int NTW, int NACC>
 __device__ __forceinline__ void conv_epilogue(const ConvArgs& P, const f32x16 (&acc)[NTW][NACC], int co_base,
                                               const long (&oaddr)[NTW], const bool (&pvalid)[NTW]) {
     TS* out = static_cast<TS*>(P.out);
@@ -99,8 +99,7 @@ __device__ __forceinline__ void conv_epilogue(const ConvArgs& P, const f32x16 (&
             float l[8];
 #pragma unroll
             for (int i = 0; i < 8; ++i) l[i] = acc[t][i][e];
-            if constexpr (MAP == MAP_FWD) merge_output(l, y);
-            else merge_left_grad(l, y);
+            merge_output(l, y);
         }
     };
 #pragma unroll
@@ -359,7 +358,7 @@ __device__ __forceinline__ void stage_vec_store_scalar(float* lds, const f32x4 (
 //   lane and K step, prefetched one step ahead); B operand = activations from the LDS halo window.
 //   MODE 16: acc[q] += W_{p^q} * (+-x_p), 16 MFMAs per K step, filters reused across the 4x4 block.
 //   MODE 8 : acc[i] += R_i * L_i with the 8 lanes L_i formed in registers, 8 MFMAs per K step.
-template <typename TS, int MODE, int MAP, int WCO, int NTW, int CK, int P2LOG, bool VSTG>
+template <typename TS, int MODE, int WCO, int NTW, int CK, int P2LOG, bool VSTG>
 __global__ void __launch_bounds__(WG_THREADS, (MODE == 8 || NTW == 1) ? 2 : 1) qconv_fwd_f32_kernel(const ConvArgs P) {
     constexpr int WPX = 4 / WCO;
     constexpr int NACC = (MODE == 16) ? 4 : 8;
@@ -478,8 +477,7 @@ __global__ void __launch_bounds__(WG_THREADS, (MODE == 8 || NTW == 1) ? 2 : 1) q
                                                                                  acc[t][q], 0, 0, 0);
                     } else {
                         float L[8];
-                        if constexpr (MAP == MAP_FWD) lanes_left(x, L);
-                        else lanes_grad(x, L, 0.5f);
+                        lanes_left(x, L);
 #pragma unroll
                         for (int i = 0; i < 8; ++i)
                             acc[t][i] = __builtin_amdgcn_mfma_f32_32x32x2f32(wcur[i >> 2][i & 3], L[i], acc[t][i], 0, 0, 0);
@@ -498,7 +496,7 @@ __global__ void __launch_bounds__(WG_THREADS, (MODE == 8 || NTW == 1) ? 2 : 1) q
     }
 
     // epilogue: fold lanes (8-product), add bias, store NCHW with components on the batch axis
-    conv_epilogue<TS, MODE, MAP, NTW, NACC>(P, acc, (ct * WCO + wco) * 32 + 4 * kk, oaddr, pvalid);
+    conv_epilogue<TS, MODE, NTW, NACC>(P, acc, (ct * WCO + wco) * 32 + 4 * kk, oaddr, pvalid);
     PHX_STAMP(5)
     PHX_PHASES_REPORT("fwd_f32: barrier / store / barrier / load issue / mfma / epilogue", 6)
 }
@@ -507,8 +505,8 @@ __global__ void __launch_bounds__(WG_THREADS, (MODE == 8 || NTW == 1) ? 2 : 1) q
 //   lane = (row = lane % 32, kk = lane / 32), output channel = tile*32 + row,
 //   K step = ((chunk * taps) + tap) * 4 + cp, input channel = chunk*8 + 2*cp + kk.
 //   MODE 16: the four filter components; MODE 8: the eight right-operand lanes R_i.
-//   MAP_DGRAD swaps the channel roles, mirrors the taps and (MODE 16) conjugates the filter, so
-//   that dx = g (x) conj(w) runs through the forward kernel.
+//   MAP_DGRAD swaps the channel roles, mirrors the taps and conjugates the filter (MODE 8: before its
+//   lanes are formed), so that dx = g (x) conj(w) runs through the forward kernel.
 // Filter element (r, o, i, kh, kw) lives at r*wcs + o*so + i*si + kh*skh + kw*skw.
 struct PackArgs {
     const void* w;
@@ -553,12 +551,13 @@ __global__ void __launch_bounds__(WG_THREADS) pack_filters_f32_kernel(const Pack
             for (int r = 0; r < 4; ++r) wv[r] = ldf<TS>(w + r * P.wcs + off);
         }
         float* dst = static_cast<float*>(P.out) + idx * WC;
+        if (MAP == MAP_DGRAD) {
+#pragma unroll
+            for (int r = 1; r < 4; ++r) wv[r] = -wv[r];
+        }
         if constexpr (MODE == 16) {
-            const float sgn = (MAP == MAP_DGRAD) ? -1.f : 1.f;
-            dst[0] = wv[0];
-            dst[1] = sgn * wv[1];
-            dst[2] = sgn * wv[2];
-            dst[3] = sgn * wv[3];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) dst[r] = wv[r];
         } else {
             float R[8];
             lanes_right(wv, R);

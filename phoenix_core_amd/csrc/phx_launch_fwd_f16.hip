@@ -4,12 +4,12 @@
 
 namespace phx {
 
-template <int MODE, int MAP, bool PAIRS>
+template <int MODE, bool PAIRS>
 static int launch_variant16(const FwdVariant& v, const ConvArgs& a, hipStream_t st) {
     constexpr int P2A = 8, P2B = PAIRS ? 8 : 7;  // the pair path has a single staging shape
 #define PHX_CASE(WCO_, NTW_, P2_)                                                                             \
     if (v.WCO == WCO_ && v.NTW == NTW_ && (PAIRS || v.P2LOG == P2_)) {                                        \
-        hipLaunchKernelGGL((qconv_fwd_f16_kernel<MODE, MAP, WCO_, NTW_, P2_, PAIRS>), dim3(v.wgs),            \
+        hipLaunchKernelGGL((qconv_fwd_f16_kernel<MODE, WCO_, NTW_, P2_, PAIRS>), dim3(v.wgs),                 \
                            dim3(WG_THREADS), v.lds_bytes, st, a);                                             \
         return 0;                                                                                             \
     }
@@ -25,9 +25,8 @@ static int launch_variant16(const FwdVariant& v, const ConvArgs& a, hipStream_t 
 
 template <bool PAIRS>
 static int launch_v1(const FwdVariant& v, const ConvArgs& a, hipStream_t st) {
-    if (v.mode == 16) return launch_variant16<16, MAP_FWD, PAIRS>(v, a, st);
-    if (v.map == MAP_FWD) return launch_variant16<8, MAP_FWD, PAIRS>(v, a, st);
-    return launch_variant16<8, MAP_DGRAD, PAIRS>(v, a, st);
+    if (v.mode == 16) return launch_variant16<16, PAIRS>(v, a, st);
+    return launch_variant16<8, PAIRS>(v, a, st);
 }
 
 template <bool CHUNKS>
@@ -35,7 +34,7 @@ static int launch_lds16(const FwdVariant& v, const ConvArgs& a, hipStream_t st) 
     constexpr int P2A = 8, P2B = CHUNKS ? 8 : 7;  // chunk staging has a single shape
 #define PHX_CASE(WCO_, NTW_, P2_)                                                                             \
     if (v.WCO == WCO_ && v.NTW == NTW_ && (CHUNKS || v.P2LOG == P2_)) {                                        \
-        constexpr auto kernel = qconv_fwd_f16_lds_kernel<16, MAP_FWD, WCO_, NTW_, P2_, CHUNKS>;              \
+        constexpr auto kernel = qconv_fwd_f16_lds_kernel<16, WCO_, NTW_, P2_, CHUNKS>;              \
         if (!BigLds<kernel>::registered) return -1; /* dynamic LDS opt-in at set-up, see BigLds */            \
         hipLaunchKernelGGL(kernel, dim3(v.wgs), dim3(WG_THREADS), v.lds_bytes, st, a);                        \
         return 0;                                                                                             \
@@ -44,13 +43,13 @@ static int launch_lds16(const FwdVariant& v, const ConvArgs& a, hipStream_t st) 
         // one filter group per chunk (pointwise problems): the variant that requests the next chunk first
         if (v.ngroups == 1 && v.NTW == 1 && !tuning_noearly()) {
             if (v.WCO == 1) {
-                constexpr auto kernel = qconv_fwd_f16_lds_kernel<16, MAP_FWD, 1, 1, 8, true, true>;
+                constexpr auto kernel = qconv_fwd_f16_lds_kernel<16, 1, 1, 8, true, true>;
                 if (!BigLds<kernel>::registered) return -1;
                 hipLaunchKernelGGL(kernel, dim3(v.wgs), dim3(WG_THREADS), v.lds_bytes, st, a);
                 return 0;
             }
             if (v.WCO == 2) {
-                constexpr auto kernel = qconv_fwd_f16_lds_kernel<16, MAP_FWD, 2, 1, 8, true, true>;
+                constexpr auto kernel = qconv_fwd_f16_lds_kernel<16, 2, 1, 8, true, true>;
                 if (!BigLds<kernel>::registered) return -1;
                 hipLaunchKernelGGL(kernel, dim3(v.wgs), dim3(WG_THREADS), v.lds_bytes, st, a);
                 return 0;

@@ -4,11 +4,10 @@
 
 namespace phx {
 
-template <int MAP>
-static int launch_lds8(const FwdVariant& v, const ConvArgs& a, hipStream_t st) {
+static int launch_lds8_impl(const FwdVariant& v, const ConvArgs& a, hipStream_t st) {
 #define PHX_CASE(WCO_, NTW_)                                                                                       \
     if (v.WCO == WCO_ && v.NTW == NTW_) {                                                                          \
-        constexpr auto kernel = qconv_fwd_f16_lds_kernel<8, MAP, WCO_, NTW_, 8, true>;                             \
+        constexpr auto kernel = qconv_fwd_f16_lds_kernel<8, WCO_, NTW_, 8, true>;                             \
         /* more than 64 KiB of dynamic LDS: opted in per device at set-up, see BigLds */                           \
         if (!BigLds<kernel>::registered) return -1;                                                                \
         hipLaunchKernelGGL(kernel, dim3(v.wgs), dim3(WG_THREADS), v.lds_bytes, st, a);                             \
@@ -20,7 +19,9 @@ static int launch_lds8(const FwdVariant& v, const ConvArgs& a, hipStream_t st) {
 }
 
 int launch_fwd_f16_lds8(const FwdVariant& v, const ConvArgs& a, hipStream_t st) {
-    return v.map == MAP_FWD ? launch_lds8<MAP_FWD>(v, a, st) : launch_lds8<MAP_DGRAD>(v, a, st);
+    // the input gradient is the forward product with the conjugated, mirrored, transposed filter: the packing
+    // kernel builds that filter's lanes and the same kernel instance runs both passes
+    return launch_lds8_impl(v, a, st);
 }
 
 }  // namespace phx

@@ -3,11 +3,11 @@
 
 namespace phx {
 
-template <typename TS, int MODE, int MAP>
+template <typename TS, int MODE>
 static int launch_variant(const FwdVariant& v, const ConvArgs& a, hipStream_t st) {
 #define PHX_CASE(WCO_, NTW_, CK_, P2_, VS_)                                                                   \
     if (v.WCO == WCO_ && v.NTW == NTW_ && v.CK == CK_ && v.P2LOG == P2_ && v.vstage == VS_) {                 \
-        hipLaunchKernelGGL((qconv_fwd_f32_kernel<TS, MODE, MAP, WCO_, NTW_, CK_, P2_, VS_>), dim3(v.wgs),     \
+        hipLaunchKernelGGL((qconv_fwd_f32_kernel<TS, MODE, WCO_, NTW_, CK_, P2_, VS_>), dim3(v.wgs),          \
                            dim3(WG_THREADS), v.lds_bytes, st, a);                                             \
         return 0;                                                                                             \
     }
@@ -26,10 +26,9 @@ static int launch_variant(const FwdVariant& v, const ConvArgs& a, hipStream_t st
 
 template <typename TS>
 static int launch_ts(const FwdVariant& v, const ConvArgs& a, hipStream_t st) {
-    // the 16-product input gradient is the forward kernel on conjugated, mirrored filters
-    if (v.mode == 16) return launch_variant<TS, 16, MAP_FWD>(v, a, st);
-    if (v.map == MAP_FWD) return launch_variant<TS, 8, MAP_FWD>(v, a, st);
-    return launch_variant<TS, 8, MAP_DGRAD>(v, a, st);
+    // one kernel for both passes: the input gradient differs only in how its filters are packed
+    if (v.mode == 16) return launch_variant<TS, 16>(v, a, st);
+    return launch_variant<TS, 8>(v, a, st);
 }
 
 int launch_fwd_f32(const FwdVariant& v, const ConvArgs& a, hipStream_t st) {
