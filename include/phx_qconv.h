@@ -142,7 +142,9 @@ int phx_algebra_map(int algebra, int32_t* dims, int32_t* halves, int32_t blade[8
 /* Output spatial size for the descriptor's explicit padding (src/utils.cc:42-51). */
 int phx_qconv2d_output_hw(const phx_qconv_desc* desc, int32_t* ho, int32_t* wo);
 
-/* Scratch bytes one call of the given pass needs (packed filters, split-K partial sums). */
+/* Scratch bytes one call of the given pass needs (packed filters, split-K partial sums).  The workspace a caller
+ * passes must be 16-byte aligned (any hipMalloc allocation is); a misaligned one is refused with
+ * PHX_ERR_INVALID_ARGUMENT. */
 size_t phx_qconv2d_workspace_bytes(const phx_qconv_desc* desc, int pass);
 size_t phx_qdense_workspace_bytes(const phx_qdense_desc* desc, int pass);
 

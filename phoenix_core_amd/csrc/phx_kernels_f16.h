@@ -696,9 +696,8 @@ __global__ void __launch_bounds__(WG_THREADS, (MODE == 16 && NTW == 1) ? 2 : 1) 
     PHX_PHASES_REPORT("fwd_f16_lds: barrier / store / wait+barrier / prefetch / mfma / epilogue", 6)
 }
 
-// Filter packing for qconv_fwd_f16_lds_kernel (16-product only; conjugated / mirrored / transposed
-// for MAP_DGRAD).  One thread per 16-byte vector of the image described above; taps beyond the
-// filter (last group of a chunk) and channels beyond the tensor are zero.
+// Filter packing for qconv_fwd_f16_lds_kernel (conjugated / mirrored / transposed for MAP_DGRAD) into the
+// image described above; taps beyond the filter (last group of a chunk) and channels beyond the tensor are zero.
 struct PackLdsArgs {
     PackArgs base;
     int WCO;       // filter sub-tiles per workgroup tile
@@ -711,17 +710,19 @@ __global__ void __launch_bounds__(WG_THREADS) pack_filters_f16_lds_kernel(const 
     const PackArgs& P = A.base;
     constexpr int TG = F16_TG;
     constexpr int NW = (MODE == 16) ? 4 : 8;
-    // 16-product: one thread per 16-byte vector (one component).  8-product: one thread per group of the
-    // eight lane vectors of a (tap, sub-tile, lane) slot, which all derive from the same 8 x 4 filter values.
+    // One thread per reduced channel (element i of a 16-byte vector).  16-product: of one vector (one component);
+    // 8-product: of the eight lane vectors of a (tap, sub-tile, lane) slot, which all derive from the same four
+    // filter values.  Neighbouring threads write neighbouring halves: every store instruction fills whole vectors.
     constexpr int PER = (MODE == 16) ? 1 : NW;
     const int taps = A.pw ? A.pw : P.Kh * P.Kw;
-    // vector index = ((((tile*nchunks + chunk)*ngroups + g)*TG + tg)*WCO + wco)*NW + r)*64 + lane
-    const long total = (long)P.row_tiles * P.nchunks * A.ngroups * TG * A.WCO * (NW / PER) * 64;
+    // element index = (((((tile*nchunks + chunk)*ngroups + g)*TG + tg)*WCO + wco)*NW + r)*64 + lane)*8 + i
+    const long total = (long)P.row_tiles * P.nchunks * A.ngroups * TG * A.WCO * (NW / PER) * 64 * 8;
     const _Float16* w = static_cast<const _Float16*>(P.w);
-    f16x8* outv = reinterpret_cast<f16x8*>(P.out);
+    _Float16* outh = static_cast<_Float16*>(P.out);
     for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
-        const int lane = idx & 63;
-        long s = idx >> 6;
+        const int i = idx & 7;
+        const int lane = (idx >> 3) & 63;
+        long s = idx >> 9;
         int r = 0;
         if constexpr (PER == 1) { r = s % NW; s /= NW; }
         const long slot = s;  // (tile, chunk, g, tg, wco)
@@ -732,48 +733,41 @@ __global__ void __launch_bounds__(WG_THREADS) pack_filters_f16_lds_kernel(const 
         const int tile = s / P.nchunks;
         const int tap = g * TG + tg;
         const int row = (tile * A.WCO + wco) * 32 + (lane & 31);
-        f16x8 vec[PER];
+        const int k16 = (lane >> 5) * 8 + i;
+        const int red = A.pw ? (chunk * A.pw + tap) * 16 + k16 : chunk * F16_CK + k16;
+        _Float16 val[PER];
 #pragma unroll
-        for (int q = 0; q < PER; ++q)
-#pragma unroll
-            for (int i = 0; i < 8; ++i) vec[q][i] = (_Float16)0;
-        if (tap < taps && row < P.rows) {
+        for (int q = 0; q < PER; ++q) val[q] = (_Float16)0;
+        if (tap < taps && row < P.rows && red < P.red) {
             int kh = tap / P.Kw, kw = tap - kh * P.Kw;
             if (MAP == MAP_DGRAD) { kh = P.khm - kh * P.khs; kw = P.kwm - kw * P.kws; }
             if (A.pw) {  // the one real tap (of a strided convolution's phase: the filter tap that reaches it)
                 kh = (MAP == MAP_DGRAD) ? P.khm : 0;
                 kw = (MAP == MAP_DGRAD) ? P.kwm : 0;
             }
+            const int o = (MAP == MAP_DGRAD) ? red : row;
+            const int in = (MAP == MAP_DGRAD) ? row : red;
+            const long off = o * P.so + in * P.si + kh * P.skh + kw * P.skw;
+            if constexpr (MODE == 16) {
+                const float sgn = (MAP == MAP_DGRAD && r > 0) ? -1.f : 1.f;  // conjugate
+                val[0] = (_Float16)(sgn * (float)w[r * P.wcs + off]);
+            } else {
+                // input gradient: dx = g (x) conj(w) is the forward product of the gradient with the
+                // conjugated filter, so the forward kernel serves it and only the packing differs
+                float wv[4], R[8];
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const int k16 = (lane >> 5) * 8 + i;
-                const int red = A.pw ? (chunk * A.pw + tap) * 16 + k16 : chunk * F16_CK + k16;
-                if (red < P.red) {
-                    const int o = (MAP == MAP_DGRAD) ? red : row;
-                    const int in = (MAP == MAP_DGRAD) ? row : red;
-                    const long off = o * P.so + in * P.si + kh * P.skh + kw * P.skw;
-                    if constexpr (MODE == 16) {
-                        const float sgn = (MAP == MAP_DGRAD && r > 0) ? -1.f : 1.f;  // conjugate
-                        vec[0][i] = (_Float16)(sgn * (float)w[r * P.wcs + off]);
-                    } else {
-                        // input gradient: dx = g (x) conj(w) is the forward product of the gradient with the
-                        // conjugated filter, so the forward kernel serves it and only the packing differs
-                        float wv[4], R[8];
+                for (int c = 0; c < 4; ++c)
+                    wv[c] = ((MAP == MAP_DGRAD && c > 0) ? -1.f : 1.f) * (float)w[c * P.wcs + off];
+                lanes_right(wv, R);  // formed in fp32, rounded once
 #pragma unroll
-                        for (int c = 0; c < 4; ++c)
-                            wv[c] = ((MAP == MAP_DGRAD && c > 0) ? -1.f : 1.f) * (float)w[c * P.wcs + off];
-                        lanes_right(wv, R);  // formed in fp32, rounded once
-#pragma unroll
-                        for (int q = 0; q < 8; ++q) vec[q][i] = (_Float16)R[q];
-                    }
-                }
+                for (int q = 0; q < 8; ++q) val[q] = (_Float16)R[q];
             }
         }
         if constexpr (PER == 1) {
-            outv[idx] = vec[0];
+            outh[idx] = val[0];
         } else {
 #pragma unroll
-            for (int q = 0; q < PER; ++q) outv[(slot * NW + q) * 64 + lane] = vec[q];
+            for (int q = 0; q < PER; ++q) outh[(((slot * NW + q) * 64 + lane) << 3) + i] = val[q];
         }
     }
 }

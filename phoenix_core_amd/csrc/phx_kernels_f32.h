@@ -838,47 +838,55 @@ struct ReduceArgs {
     int Z, Co, Ci, Kh, Kw, CoP, CiP;
 };
 
-// dw(r, co, ci, kh, kw) = sum_z partial[z][tap][r][co][ci].  A workgroup owns 32 consecutive
-// outputs; its 8 z-slices each add every 8th partial, then the slices are added in a fixed order,
-// so the result does not depend on scheduling.
+// dw(r, co, ci, kh, kw) = sum_z partial[z][tap][r][co][ci].  A thread owns four consecutive input channels of
+// one (tap, component, output channel) -- 16-byte loads, the padded row length CiP is a multiple of 4.  The
+// threads of a workgroup form nsl z-slices (8 where there are that many partials, else 4, 2 or 1) over
+// WG_THREADS / nsl such groups; slice s adds partials s, s + nsl, ..., then the slices are added in a fixed
+// order, so the result does not depend on scheduling.
+__host__ __device__ inline int reduce_slices(int Z) { return Z >= 7 ? 8 : Z >= 4 ? 4 : Z >= 2 ? 2 : 1; }
+
 template <typename TS>
 __global__ void __launch_bounds__(WG_THREADS) reduce_wgrad_kernel(const ReduceArgs P) {
-    __shared__ float part[8][33];
+    __shared__ f32x4 part[WG_THREADS];
     const int taps = P.Kh * P.Kw;
-    const long total = 4L * taps * P.Co * P.Ci;
+    const int ci4s = (P.Ci + 3) >> 2;
+    const long total = 4L * taps * P.Co * ci4s;
     const long zstride = 4L * taps * P.CoP * P.CiP;
     TS* dw = static_cast<TS*>(P.dw);
-    const int lane = threadIdx.x & 31, slice = threadIdx.x >> 5;
-    const long idx = (long)blockIdx.x * 32 + lane;
-    float sum = 0.f;
+    const int nsl = reduce_slices(P.Z), groups = WG_THREADS / nsl;
+    const int lane = threadIdx.x % groups, slice = threadIdx.x / groups;
+    const long idx = (long)blockIdx.x * groups + lane;
+    f32x4 sum = {0.f, 0.f, 0.f, 0.f};
     int ci = 0, co = 0, r = 0, tap = 0;
     if (idx < total) {
-        ci = idx % P.Ci;
-        long t = idx / P.Ci;
+        ci = (int)(idx % ci4s) * 4;
+        long t = idx / ci4s;
         co = t % P.Co;
         t /= P.Co;
         r = t & 3;
         tap = t >> 2;
         const float* src = P.partial + (((long)tap * 4 + r) * P.CoP + co) * P.CiP + ci;
-        float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+        f32x4 s0 = sum, s1 = sum, s2 = sum, s3 = sum;
         int z = slice;
-        for (; z + 24 < P.Z; z += 32) {
-            s0 += src[(long)z * zstride];
-            s1 += src[(long)(z + 8) * zstride];
-            s2 += src[(long)(z + 16) * zstride];
-            s3 += src[(long)(z + 24) * zstride];
+        for (; z + 3 * nsl < P.Z; z += 4 * nsl) {
+            s0 += *reinterpret_cast<const f32x4*>(src + (long)z * zstride);
+            s1 += *reinterpret_cast<const f32x4*>(src + (long)(z + nsl) * zstride);
+            s2 += *reinterpret_cast<const f32x4*>(src + (long)(z + 2 * nsl) * zstride);
+            s3 += *reinterpret_cast<const f32x4*>(src + (long)(z + 3 * nsl) * zstride);
         }
-        for (; z < P.Z; z += 8) s0 += src[(long)z * zstride];
+        for (; z < P.Z; z += nsl) s0 += *reinterpret_cast<const f32x4*>(src + (long)z * zstride);
         sum = (s0 + s1) + (s2 + s3);
     }
-    part[slice][lane] = sum;
+    part[threadIdx.x] = sum;
     __syncthreads();
     if (slice == 0 && idx < total) {
-        float v = part[0][lane];
-#pragma unroll
-        for (int k = 1; k < 8; ++k) v += part[k][lane];
+        f32x4 v = part[lane];
+        for (int k = 1; k < nsl; ++k) v += part[k * groups + lane];
         const int kh = tap / P.Kw, kw = tap - kh * P.Kw;
-        stf<TS>(dw + r * P.wcs + co * P.so + ci * P.si + kh * P.skh + kw * P.skw, v);
+        TS* dst = dw + r * P.wcs + co * P.so + ci * P.si + kh * P.skh + kw * P.skw;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            if (ci + e < P.Ci) stf<TS>(dst + e * P.si, v[e]);
     }
 }
 

@@ -59,7 +59,7 @@ int launch_wgrad_f16(int mode, int MT, int NT, int TPW, int SW, const WgradArgs&
 int launch_wgrad_f16_p16(int MT, int NT, int TPW, int SW, const WgradArgs& a, int nblocks, size_t lds_bytes, hipStream_t st);
 int launch_wgrad_f16_p16t3(int MT, int NT, const WgradArgs& a, int nblocks, size_t lds_bytes, hipStream_t st);
 int launch_wgrad_f16_p8(int MT, int NT, int SW, const WgradArgs& a, int nblocks, size_t lds_bytes, hipStream_t st);
-int launch_reduce_wgrad(bool half_storage, const ReduceArgs& a, int blocks, hipStream_t st);
+int launch_reduce_wgrad(bool half_storage, const ReduceArgs& a, hipStream_t st);
 
 // space-to-depth rearrangements (stride-2 convolutions with very few input channels)
 int launch_s2d_input(bool half_storage, const S2dArgs& a, hipStream_t st);

@@ -6,6 +6,7 @@
 #include <atomic>
 #include <cstdio>
 #include <cstdlib>
+#include <cstdint>
 #include <cstring>
 #include <mutex>
 #include <unordered_map>
@@ -97,6 +98,9 @@ struct DeviceState {
 constexpr int MAX_DEVICES = 64;
 static DeviceState g_devices[MAX_DEVICES];
 static std::mutex g_device_mutex;
+
+// packed filters, partial sums and rearranged tensors are read and written as 16-byte vectors
+static bool misaligned_workspace(const void* ws) { return (reinterpret_cast<uintptr_t>(ws) & 15) != 0; }
 
 static int device_state(DeviceState** out) {
     int dev = 0;
@@ -689,8 +693,8 @@ static int run_corr(const Problem& p, const Corr& creal, int map, hipStream_t st
     pa.khm = creal.khm; pa.khs = creal.khs; pa.kwm = creal.kwm; pa.kws = creal.kws;
     pa.rows = c.Cout; pa.red = creal.Cin; pa.row_tiles = pl.co_tiles * pl.WCO;
     pa.nchunks = f16 ? pl.nchunks : pl.nchunks * (pl.CK / F32_CK);
-    // (LDS images: one thread per 16-byte vector, in 8-product form one thread per eight lane vectors)
-    const long pack_items = pl.lds_filters ? (long)(pl.wpk_bytes / 16) / (pl.kmode == 8 ? 8 : 1)
+    // (LDS images: one thread per packed half, in 8-product form one thread per element of eight lane vectors)
+    const long pack_items = pl.lds_filters ? (long)(pl.wpk_bytes / 2) / (pl.kmode == 8 ? 8 : 1)
                                             : (long)pa.row_tiles * pa.nchunks * creal.Kh * creal.Kw * (f16 ? 1 : 4) * 64;
     if (pl.lds_filters) pa.row_tiles = pl.co_tiles;  // packed per workgroup tile of WCO*32 channels
     const int pack_blocks = (int)std::min<long>((pack_items + WG_THREADS - 1) / WG_THREADS, 4096);
@@ -935,9 +939,7 @@ static int run_wgrad(const Problem& p, hipStream_t st, const void* x, const void
     r.partial = a.partial; r.dw = dw;
     r.wcs = p.fs.wcs; r.so = p.fs.so; r.si = p.fs.si; r.skh = p.fs.skh; r.skw = p.fs.skw;
     r.Z = f16 ? pl.Z : pl.Z * pl.ksets; r.Co = p.co; r.Ci = p.ci; r.Kh = p.kh; r.Kw = p.kw; r.CoP = pl.CoP; r.CiP = pl.CiP;
-    const long items = 4L * p.kh * p.kw * p.co * p.ci;
-    const int blocks = (int)((items + 31) / 32);
-    launch_reduce_wgrad(half_storage, r, blocks, st);
+    launch_reduce_wgrad(half_storage, r, st);
     PHX_HIP(hipGetLastError());
     if (f16)
         snprintf(g_name_buf, sizeof(g_name_buf), "%sqconv_wgrad_f16mfma_p%d_f16_ch%dx%d_taps%d_sw%d%s_z%d", g_name_prefix, pl.kmode, 32 * pl.MT,
@@ -1304,6 +1306,7 @@ size_t phx_qdense_workspace_bytes(const phx_qdense_desc* desc, int pass) {
 int phx_qconv2d_fwd(const phx_qconv_desc* desc, phx_stream_t stream, const void* x, const void* w,
                     const void* bias_or_null, void* y, void* workspace, size_t workspace_bytes) {
     if (const int init_rc = device_state(nullptr)) return init_rc;
+    if (misaligned_workspace(workspace)) return PHX_ERR_INVALID_ARGUMENT;
     if (desc && desc->algebra != PHX_QUATERNION)
         return algebra_conv_pass(desc, PHX_PASS_FWD, stream, x, w, bias_or_null, y, workspace, workspace_bytes);
     Problem p;
@@ -1345,6 +1348,7 @@ int phx_qconv2d_fwd_noalloc(const phx_qconv_desc* desc, phx_stream_t stream, con
 int phx_qconv2d_bwd_data(const phx_qconv_desc* desc, phx_stream_t stream, const void* grad, const void* w, void* dx,
                          void* workspace, size_t workspace_bytes) {
     if (const int init_rc = device_state(nullptr)) return init_rc;
+    if (misaligned_workspace(workspace)) return PHX_ERR_INVALID_ARGUMENT;
     if (desc && desc->algebra != PHX_QUATERNION)
         return algebra_conv_pass(desc, PHX_PASS_BWD_DATA, stream, grad, w, nullptr, dx, workspace, workspace_bytes);
     Problem p;
@@ -1378,6 +1382,7 @@ int phx_qconv2d_bwd_data(const phx_qconv_desc* desc, phx_stream_t stream, const 
 int phx_qconv2d_bwd_weights(const phx_qconv_desc* desc, phx_stream_t stream, const void* x, const void* grad, void* dw,
                             void* workspace, size_t workspace_bytes) {
     if (const int init_rc = device_state(nullptr)) return init_rc;
+    if (misaligned_workspace(workspace)) return PHX_ERR_INVALID_ARGUMENT;
     if (desc && desc->algebra != PHX_QUATERNION)
         return algebra_conv_pass(desc, PHX_PASS_BWD_WEIGHTS, stream, x, grad, nullptr, dw, workspace, workspace_bytes);
     Problem p;
@@ -1405,6 +1410,7 @@ int phx_qconv2d_bwd_weights(const phx_qconv_desc* desc, phx_stream_t stream, con
 int phx_qdense_fwd(const phx_qdense_desc* desc, phx_stream_t stream, const void* x, const void* w,
                    const void* bias_or_null, void* y, void* workspace, size_t workspace_bytes) {
     if (const int init_rc = device_state(nullptr)) return init_rc;
+    if (misaligned_workspace(workspace)) return PHX_ERR_INVALID_ARGUMENT;
     if (desc && desc->algebra != PHX_QUATERNION)
         return algebra_dense_pass(desc, PHX_PASS_FWD, stream, x, w, bias_or_null, y, workspace, workspace_bytes);
     Problem p;
@@ -1416,6 +1422,7 @@ int phx_qdense_fwd(const phx_qdense_desc* desc, phx_stream_t stream, const void*
 int phx_qdense_bwd_data(const phx_qdense_desc* desc, phx_stream_t stream, const void* grad, const void* w, void* dx,
                         void* workspace, size_t workspace_bytes) {
     if (const int init_rc = device_state(nullptr)) return init_rc;
+    if (misaligned_workspace(workspace)) return PHX_ERR_INVALID_ARGUMENT;
     if (desc && desc->algebra != PHX_QUATERNION)
         return algebra_dense_pass(desc, PHX_PASS_BWD_DATA, stream, grad, w, nullptr, dx, workspace, workspace_bytes);
     Problem p;
@@ -1427,6 +1434,7 @@ int phx_qdense_bwd_data(const phx_qdense_desc* desc, phx_stream_t stream, const 
 int phx_qdense_bwd_weights(const phx_qdense_desc* desc, phx_stream_t stream, const void* x, const void* grad, void* dw,
                            void* workspace, size_t workspace_bytes) {
     if (const int init_rc = device_state(nullptr)) return init_rc;
+    if (misaligned_workspace(workspace)) return PHX_ERR_INVALID_ARGUMENT;
     if (desc && desc->algebra != PHX_QUATERNION)
         return algebra_dense_pass(desc, PHX_PASS_BWD_WEIGHTS, stream, x, grad, nullptr, dw, workspace, workspace_bytes);
     Problem p;

@@ -625,6 +625,31 @@ def test_mismatched_tensors_are_refused_before_the_library_reads_them():
     assert torch.isfinite(y).all()
 
 
+def test_misaligned_workspace_is_refused():
+    """Packed filters and partial sums are 16-byte vectors: a workspace that is not 16-byte aligned is an invalid
+    argument for every pass, and nothing is launched."""
+    import ctypes
+    from phoenix_core_amd import capi
+    x = torch.randn(8, 4, 6, 6, device="cuda")
+    w = torch.randn(4, 4, 4, 3, 3, device="cuda")
+    desc = phx.Conv2DDescriptor(x.shape, w.shape, 1, 1, "SAME", context=Ctx(8))
+    y = torch.full(desc.output_shape, 7.0, device="cuda")
+    dx, dw = torch.empty_like(x), torch.empty_like(w)
+    nbytes = max(desc.workspace_bytes(p) for p in range(3))
+    ws = torch.empty(nbytes + 16, dtype=torch.uint8, device="cuda")
+    L, d, st = capi.lib(), ctypes.byref(desc.c), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+    bad = ctypes.c_void_p(ws.data_ptr() + 4)
+    assert L.phx_qconv2d_fwd(d, st, P(x), P(w), None, P(y), bad, nbytes) == capi.PHX_ERR_INVALID_ARGUMENT
+    assert L.phx_qconv2d_bwd_data(d, st, P(y), P(w), P(dx), bad, nbytes) == capi.PHX_ERR_INVALID_ARGUMENT
+    assert L.phx_qconv2d_bwd_weights(d, st, P(x), P(y), P(dw), bad, nbytes) == capi.PHX_ERR_INVALID_ARGUMENT
+    torch.cuda.synchronize()
+    assert (y == 7.0).all()
+    assert L.phx_qconv2d_fwd(d, st, P(x), P(w), None, P(y), P(ws), nbytes) == 0
+    torch.cuda.synchronize()
+    assert torch.isfinite(y).all() and not (y == 7.0).all()
+
+
 def test_verbose_names_mode_policy_and_kernel(tune_env, capfd):
     """UPSTRIDE_VERBOSE (src/backend/backend.cc:50-62 switches the reference's debug log on): one line per call on
     stderr with the product mode, the fp16 policy and the kernel variant that ran; silent without it."""
