@@ -407,9 +407,13 @@ __device__ __forceinline__ void lane_step(const f16x8 (&x)[4], f16x8 (&L)[8], in
 // EARLY (chunk staging, problems with one filter group per chunk, i.e. pointwise ones): only the products of one
 // group stand between the request for the next chunk's activations and their use, so the request goes out at the
 // start of the group, ahead of the filter copy (which the same wait then covers).
-template <int MODE, int WCO, int NTW, int P2LOG, bool CHUNKS, bool EARLY = false>
+// XREAL (16-product, chunk staging): the input holds its real component only (P.in.ncomp == 1); the twelve
+// products with the absent components and their operand reads are left out at compile time.
+template <int MODE, int WCO, int NTW, int P2LOG, bool CHUNKS, bool EARLY = false, bool XREAL = false>
 __global__ void __launch_bounds__(WG_THREADS, (MODE == 16 && NTW == 1) ? 2 : 1) qconv_fwd_f16_lds_kernel(const ConvArgs P) {
     static_assert(!EARLY || CHUNKS, "early activation requests belong to chunk staging");
+    static_assert(!XREAL || (MODE == 16 && CHUNKS), "the real-input variant is a 16-product kernel with chunk staging");
+    constexpr int NP = XREAL ? 1 : 4;          // input components that take part
     constexpr int CK = F16_CK;
     constexpr int WPX = 4 / WCO;
     constexpr int TG = F16_TG;
@@ -575,7 +579,7 @@ __global__ void __launch_bounds__(WG_THREADS, (MODE == 16 && NTW == 1) ? 2 : 1) 
                 const int pos = tapoff[blk / NTW] + poff[blk % NTW];
                 const f16x8* xb = xl + kk * XP + (CHUNKS ? swizzle_entry(pos) : pos);
 #pragma unroll
-                for (int p = 0; p < 4; ++p) x[p] = xb[p * 2 * XP];
+                for (int p = 0; p < NP; ++p) x[p] = xb[p * 2 * XP];
             };
             read_w(wf[0], 0);
             if constexpr (MODE == 16) {
@@ -643,7 +647,7 @@ __global__ void __launch_bounds__(WG_THREADS, (MODE == 16 && NTW == 1) ? 2 : 1) 
 #pragma unroll
                     for (int r = 0; r < 4; ++r) nw[r] = neg8(w[r]);
 #pragma unroll
-                    for (int p = 0; p < 4; ++p) {
+                    for (int p = 0; p < NP; ++p) {
 #pragma unroll
                         for (int q = 0; q < 4; ++q)
                             acc[t][q] = __builtin_amdgcn_mfma_f32_32x32x16_f16(qneg(p, q) ? nw[p ^ q] : w[p ^ q], x[p],

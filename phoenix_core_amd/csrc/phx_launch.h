@@ -40,6 +40,7 @@ int launch_pack_filters(const FwdVariant& v, const PackArgs& a, int blocks, hipS
 int launch_fwd_f32(const FwdVariant& v, const ConvArgs& a, hipStream_t st);
 int launch_fwd_f16(const FwdVariant& v, const ConvArgs& a, hipStream_t st);
 int launch_fwd_f16_lds8(const FwdVariant& v, const ConvArgs& a, hipStream_t st);  // 8-product, filters through LDS
+int launch_fwd_f16_lds16_real(const FwdVariant& v, const ConvArgs& a, hipStream_t st);  // 16-product, chunk staging, real-valued input
 int launch_pack_filters_f16(const FwdVariant& v, const PackArgs& a, int blocks, hipStream_t st);
 
 // pointwise fp16-MFMA kernels with raw operand copies (phx_kernels_pw16.h); WCO = 32-channel sub-tiles per workgroup

@@ -65,6 +65,8 @@ static int launch_lds16(const FwdVariant& v, const ConvArgs& a, hipStream_t st) 
 
 int launch_fwd_f16(const FwdVariant& v, const ConvArgs& a, hipStream_t st) {
     if (v.lds_filters && v.mode == 8) return launch_fwd_f16_lds8(v, a, st);
+    // real-valued input (one stored component), several filter groups per chunk: the variant without the absent products
+    if (v.lds_filters && v.chunks && a.in.ncomp == 1 && !(v.ngroups == 1 && v.NTW == 1)) return launch_fwd_f16_lds16_real(v, a, st);
     if (v.lds_filters) return v.chunks ? launch_lds16<true>(v, a, st) : launch_lds16<false>(v, a, st);
     return v.pairs ? launch_v1<true>(v, a, st) : launch_v1<false>(v, a, st);
 }
