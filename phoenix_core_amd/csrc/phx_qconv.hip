@@ -4,6 +4,7 @@
 
 #include <algorithm>
 #include <atomic>
+#include <cmath>
 #include <cstdio>
 #include <cstdlib>
 #include <cstdint>
@@ -379,7 +380,19 @@ static bool plan_forward(const Corr& c, int mode, bool f16mfma, FwdPlan& best, b
                 // (pointwise problems, 16-product: workgroups live for a few blocks only, and two of them
                 // per CU -- one column tile per wave, two filter sub-tiles -- hide each other's start and end)
                 if (ldsk && pointwise && mode == 16) score *= (NTW == 1 ? 1.25 : 1.0) * (WCO == 2 ? 1.2 : 1.0);
-                else if (ldsk) score *= (NTW == 2 ? 1.25 : 1.0) * (WCO == 2 ? 1.08 : 1.0);
+                else if (ldsk && mode == 8) {
+                    // The factorized LDS kernels hold one workgroup per CU, so their time is counted out: rounds of
+                    // workgroups over the CUs (half by the whole rounds the last workgroup waits for, half by the
+                    // work there is -- a last round that is partly empty still frees power and memory bandwidth) times
+                    // the tile's area over the shape's throughput (measured at 128 channels, 28x28, per unit of tile
+                    // area: two column tiles per wave 1.0 / 1.04 with two / one filter sub-tile, one column tile
+                    // 0.79 / 0.85).  A small problem then takes the small tile that fills the CUs (64 channels at
+                    // 14x14, N=64: 0.041 -> 0.032 ms per pass).
+                    const double rate = NTW == 2 ? (WCO == 2 ? 1.0 : 1.04) : (WCO == 2 ? 0.79 : 0.85);
+                    const double cus = 256.0;
+                    const double rounds = 0.5 * std::ceil(wgs / cus) + 0.5 * (wgs / cus);
+                    score = 1e6 * rate / (rounds * BN * 32.0 * WCO) * (0.9 + 0.1 * halo);
+                } else if (ldsk) score *= (NTW == 2 ? 1.25 : 1.0) * (WCO == 2 ? 1.08 : 1.0);
                 else if (f16mfma && NTW == 2) score *= 0.8;  // that kernel drops to one workgroup per CU
                 if (tall && force_flat) score *= 100.0;  // (tests: flat tiling wherever it applies)
                 if (score > best_score) {
