@@ -4,6 +4,7 @@
 
 #include "../../include/phx_qconv.h"
 #include "phx_kernels_f32.h"
+#include "phx_kernels_realx.h"
 #include "phx_kernels_s2d.h"
 
 namespace phx {
@@ -59,6 +60,8 @@ int launch_wgrad_f16(int mode, int MT, int NT, int TPW, int SW, const WgradArgs&
                      hipStream_t st);
 int launch_wgrad_f16_p16(int MT, int NT, int TPW, int SW, const WgradArgs& a, int nblocks, size_t lds_bytes, hipStream_t st);
 int launch_wgrad_f16_p16t3(int MT, int NT, const WgradArgs& a, int nblocks, size_t lds_bytes, hipStream_t st);
+// real-valued input, few channels: the whole filter gradient as one matrix product (phx_kernels_realx.h)
+int launch_wgrad_f16_realx(const RealWgArgs& a, int nblocks, size_t lds_bytes, hipStream_t st);
 int launch_wgrad_f16_p8(int MT, int NT, int SW, const WgradArgs& a, int nblocks, size_t lds_bytes, hipStream_t st);
 int launch_reduce_wgrad(bool half_storage, const ReduceArgs& a, hipStream_t st);
 

@@ -28,7 +28,7 @@ namespace phx {
 // from the environment once; phx_tuning_reload() reads them again and forgets the cached plans.
 struct Tuning {
     int tile_wco = 0, tile_ntw = 0;   // PHX_TUNE_TILE="wco,ntw"
-    bool flat = false, noflat = false, nopw = false, pw8 = false, zi8 = false, wg8 = false, nos2d = false, noearly = false;
+    bool flat = false, noflat = false, nopw = false, pw8 = false, zi8 = false, wg8 = false, nos2d = false, noearly = false, norealx = false;
     bool nopwx = false;               // PHX_TUNE_NOPWX: pointwise fp16 problems stay on the staged-window kernels
     int vec = 0;                      // PHX_TUNE_VEC (0 = unset)
     int wgs = 0;                      // PHX_TUNE_WGS (0 = unset)
@@ -46,6 +46,7 @@ struct Tuning {
         wg8 = getenv("PHX_TUNE_WG8") != nullptr;
         nos2d = getenv("PHX_TUNE_NOS2D") != nullptr;
         noearly = getenv("PHX_TUNE_NOEARLY") != nullptr;
+        norealx = getenv("PHX_TUNE_NOREALX") != nullptr;
         nopwx = getenv("PHX_TUNE_NOPWX") != nullptr;
         if (const char* e = getenv("PHX_TUNE_VEC")) vec = atoi(e);
         if (const char* e = getenv("PHX_TUNE_WGS")) wgs = atoi(e);
@@ -758,6 +759,8 @@ struct WgPlan {
     int ksets;   // fp32 kernel: wave sets per workgroup, each with a reduction slice of its own
     int SW, cpr, nchunks, ntiles;  // fp16 kernel: stride along W, 8-pixel chunks per output row / in total, pixel tiles
     bool flat;   // fp16 kernel: the chunk list runs over whole image planes (cpr = chunks per plane)
+    bool realx;  // real-valued input, few channels: the one-product kernel of phx_kernels_realx.h
+    int rows_per_wg, pitch;  // ... its output rows per workgroup (Z workgroups) and LDS row pitch; ntiles = column tiles
     size_t lds_bytes, partial_bytes;
 };
 
@@ -842,7 +845,36 @@ static int wgrad_f16_formulation(const Problem& p) {
     return (p.mode == 8 && !tune().wg8) ? 16 : p.mode;
 }
 
+// Real-valued input with few channels (the first layer of a network on images): one matrix product holds the whole
+// filter gradient, see phx_kernels_realx.h.  q-ResNet-50 stem (7x7 stride 2 on 3 channels as 4x4 on 12 by
+// space-to-depth, 16 output channels, N=64): 0.47 ms on the general kernel.
+static bool plan_wgrad_realx(const Problem& p, WgPlan& best) {
+    if (!p.real_input || p.dtype != PHX_F16 || p.groups > 1 || p.nhwc || tune().norealx) return false;
+    if (p.sh != 1 || p.sw != 1 || p.dh != 1 || p.dw != 1 || p.kw > 4 || p.co > 16 || p.ci * p.kh * 4 > 192) return false;
+    if (p.wo % 8 != 0 || p.w < 8 || p.pt < 0 || p.pl < 0 || p.pl > 7 || p.pr > 7) return false;
+    const int cpr = p.wo / 8;
+    if (4 * p.co * cpr > REALX_GI * WG_THREADS || p.ci * p.kw * cpr > REALX_XI * WG_THREADS) return false;
+    if ((long)p.n * p.ci * p.h * p.w >= (1L << 31) || (long)p.n * p.co * p.ho * p.wo >= (1L << 31)) return false;
+    best = WgPlan{};
+    best.realx = true;
+    best.kmode = 16;
+    best.ntiles = cdiv(p.ci * p.kh * 4, 32);
+    int pitch = (p.wo + 15) & ~15;
+    while (pitch % 64 != 8) pitch += 8;
+    best.pitch = pitch;
+    best.lds_bytes = (size_t)(64 + 32 * best.ntiles) * pitch * 2;
+    if (best.lds_bytes > 160 * 1024) return false;
+    const int total_rows = p.n * p.ho;
+    const int target = tune().wgs > 0 ? tune().wgs : 512;  // two workgroups per CU
+    best.rows_per_wg = cdiv(total_rows, std::min(total_rows, target));
+    best.Z = cdiv(total_rows, best.rows_per_wg);
+    best.CoP = p.co; best.CiP = (p.ci + 3) & ~3;
+    best.partial_bytes = (size_t)best.Z * p.kh * p.kw * 4 * best.CoP * best.CiP * sizeof(float);
+    return true;
+}
+
 static bool plan_wgrad_f16(const Problem& p, WgPlan& best) {
+    if (plan_wgrad_realx(p, best)) return true;
     best = WgPlan{};
     best.SW = p.sw;
     best.kmode = wgrad_f16_formulation(p);
@@ -902,7 +934,7 @@ static bool plan_wgrad(const Problem& p, bool f16mfma, WgPlan& best) {
     static std::unordered_map<PlanKey, Entry, PlanKeyHash> memo;
     // everything the two planners read
     const PlanKey key{{p.mode, p.n, p.ci, p.co, p.h, p.w, p.kh, p.kw, p.sh, p.sw, p.dh, p.dw, p.pt, p.pl, p.pb, p.pr,
-                       p.ho, p.wo, (int)f16mfma}};
+                       p.ho, p.wo, (int)f16mfma, (int)p.real_input, (int)p.dtype, p.groups, (int)p.nhwc}};
     std::lock_guard<std::mutex> lock(g_plan_mutex);
     static unsigned generation = 0;
     if (generation != g_plan_generation) { memo.clear(); generation = g_plan_generation; }
@@ -922,6 +954,31 @@ static int run_wgrad(const Problem& p, hipStream_t st, const void* x, const void
     WgPlan pl;
     if (!plan_wgrad(p, f16, pl)) return PHX_ERR_NOT_SUPPORTED;
     if (ws_bytes < pl.partial_bytes || !ws) return PHX_ERR_WORKSPACE;
+    if (f16 && pl.realx) {
+        RealWgArgs ra{};
+        ra.x = static_cast<const _Float16*>(x); ra.g = static_cast<const _Float16*>(g);
+        ra.g_cs = (long)p.n * p.co * p.ho * p.wo;
+        ra.partial = static_cast<float*>(ws);
+        ra.N = p.n; ra.Ci = p.ci; ra.Co = p.co; ra.H = p.h; ra.W = p.w; ra.Ho = p.ho; ra.Wo = p.wo;
+        ra.Kh = p.kh; ra.Kw = p.kw; ra.pt = p.pt; ra.pl = p.pl;
+        ra.CoP = pl.CoP; ra.CiP = pl.CiP; ra.rows_per_wg = pl.rows_per_wg;
+        ra.ncol = p.ci * p.kh * 4; ra.ntiles = pl.ntiles; ra.pitch = pl.pitch;
+        {
+            KernelTimer timer(st);
+            if (launch_wgrad_f16_realx(ra, pl.Z, pl.lds_bytes, st) != 0) return PHX_ERR_RUNTIME;
+        }
+        PHX_HIP(hipGetLastError());
+        ReduceArgs r;
+        r.partial = ra.partial; r.dw = dw;
+        r.wcs = p.fs.wcs; r.so = p.fs.so; r.si = p.fs.si; r.skh = p.fs.skh; r.skw = p.fs.skw;
+        r.Z = pl.Z; r.Co = p.co; r.Ci = p.ci; r.Kh = p.kh; r.Kw = p.kw; r.CoP = pl.CoP; r.CiP = pl.CiP;
+        launch_reduce_wgrad(true, r, st);
+        PHX_HIP(hipGetLastError());
+        snprintf(g_name_buf, sizeof(g_name_buf), "%sqconv_wgrad_f16mfma_realx_f16_cols%d_rows%d_z%d", g_name_prefix, ra.ncol,
+                 pl.rows_per_wg, pl.Z);
+        say(p, "filter gradient (real-valued input)");
+        return PHX_OK;
+    }
     WgradArgs a;
     a.x.base = x; a.x.comp_stride = (long)p.n * p.ci_mem * p.h * p.w; a.x.N = p.n; a.x.C = p.ci; a.x.Cs = p.ci_mem; a.x.Hd = p.h; a.x.Wd = p.w;
     a.x.uh = a.x.uw = 1; a.x.pw = 0; a.x.tall = 0; a.x.ncomp = p.real_input ? 1 : 4;

@@ -147,7 +147,15 @@ def test_reference_kat_quaternion_real_input():
 REAL_INPUT_CASES = [c for c in CONV_CASES if c[0] in ("pw_ragged", "k3_same", "k3_ragged", "k3_s2", "k7_s2", "k3_s2_c4",
                                                       "k32_asym", "pw_64")] + [
     ("stem_7x7", 2, 3, 64, 64, 64, 7, 7, 2, 1, "SAME"),
+    # few channels and an output width that is a multiple of 8: on fp16 matrix cores the filter gradient of these
+    # is one matrix product (rows = component x output channel, columns = input channel x tap)
+    ("stem_7x7_co16", 3, 3, 16, 32, 32, 7, 7, 2, 1, "SAME"),      # by space-to-depth: 4x4 taps on 12 channels, 192 columns
+    ("stem_3x3_s1", 2, 3, 12, 10, 24, 3, 3, 1, 1, "SAME"),
+    ("stem_4x4_valid", 2, 1, 4, 12, 19, 4, 4, 1, 1, "VALID"),
+    ("stem_2x3_w40", 5, 2, 7, 6, 40, 2, 3, 1, 1, "SAME"),          # five 8-pixel chunks: the last K step is half empty
+    ("stem_5x2_many_rows", 9, 4, 16, 23, 8, 5, 2, 1, 1, "SAME"),    # 207 output rows: runs of rows cross image boundaries
 ]
+REALX_CASES = ("stem_7x7_co16", "stem_3x3_s1", "stem_4x4_valid", "stem_2x3_w40", "stem_5x2_many_rows")
 
 
 @pytest.mark.parametrize("dtype,policy", [(torch.float32, "fp32"), (torch.float16, "full16"), (torch.float16, "fp32")],
@@ -185,6 +193,8 @@ def test_conv_real_valued_input(case, mode, dtype, policy):
         want_dw, _ = oracle.conv2d_bwd(g, x4, w64, g64, "hamilton")
     assert_close(y.cpu().numpy(), want_y, dtype, "fwd " + k_fwd)
     assert_close(dw.cpu().numpy(), want_dw, dtype, "wgrad " + capi.last_kernel_name())
+    if name in REALX_CASES:
+        assert ("realx" in capi.last_kernel_name()) == (dtype == torch.float16 and policy == "full16"), capi.last_kernel_name()
     # neither a bias nor the input gradient can be asked for, as in the reference (src/conv2d.hpp:125-127, 394-398)
     with pytest.raises(RuntimeError):
         phx.conv2d_fwd(xd, wd, bd, phx.Conv2DDescriptor(x.shape, wt.shape, stride, dilation, padding, use_bias=True,
