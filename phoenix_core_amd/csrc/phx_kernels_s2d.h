@@ -52,6 +52,48 @@ __global__ void __launch_bounds__(WG_THREADS) s2d_input_kernel(const S2dArgs A) 
     }
 }
 
+// Strided pointwise convolutions read every sh-th row and sw-th column of their input and nothing else:
+// dst[plane][i][j] = src[plane][i * sh][j * sw] turns them into unit-stride pointwise convolutions, which have the
+// streaming kernels.  One thread per 8 destination columns (one 16-byte store).
+struct SubsampleArgs {
+    const void* src;
+    void* dst;
+    long planes;        // components x images x channels
+    int H, W, H2, W2;   // source and destination extent
+    int sh, sw;
+};
+
+template <typename TS>
+__global__ void __launch_bounds__(WG_THREADS) subsample_kernel(const SubsampleArgs A) {
+    const int wq = (A.W2 + 7) / 8;
+    const long total = A.planes * A.H2 * wq;
+    const TS* src = static_cast<const TS*>(A.src);
+    TS* dst = static_cast<TS*>(A.dst);
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
+        const int jq = idx % wq;
+        const long rest = idx / wq;
+        const int i = rest % A.H2;
+        const long plane = rest / A.H2;
+        const int j0 = jq * 8;
+        const TS* row = src + (plane * A.H + (long)i * A.sh) * A.W;
+        TS* out = dst + (plane * A.H2 + i) * A.W2 + j0;
+        TS v[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) v[k] = (j0 + k < A.W2) ? row[(long)(j0 + k) * A.sw] : (TS)0;
+        if (j0 + 8 <= A.W2 && (reinterpret_cast<size_t>(out) & (8 * sizeof(TS) - 1)) == 0) {
+            typedef TS vec8 __attribute__((ext_vector_type(8)));
+            vec8 o;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) o[k] = v[k];
+            *reinterpret_cast<vec8*>(out) = o;
+        } else {
+#pragma unroll
+            for (int k = 0; k < 8; ++k)
+                if (j0 + k < A.W2) out[k] = v[k];
+        }
+    }
+}
+
 struct S2dFilterArgs {
     const void* w;      // caller's filters, element (r, o, i, kh, kw) at r*wcs + o*so + i*si + kh*skh + kw*skw
     void* w2;           // rearranged filters [4][Co][4*Ci][K2h][K2w] (OIHW)

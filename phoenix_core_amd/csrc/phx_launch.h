@@ -67,6 +67,7 @@ int launch_reduce_wgrad(bool half_storage, const ReduceArgs& a, hipStream_t st);
 
 // space-to-depth rearrangements (stride-2 convolutions with very few input channels)
 int launch_s2d_input(bool half_storage, const S2dArgs& a, hipStream_t st);
+int launch_subsample(bool half_storage, const SubsampleArgs& a, hipStream_t st);
 int launch_s2d_filter(bool half_storage, const S2dFilterArgs& a, bool to_caller, hipStream_t st);
 int launch_phase_merge(bool half_storage, const PhaseMergeArgs& a, hipStream_t st);
 // batched matrix transposes between channels-last tensors and the kernels' channels-first layout

@@ -28,6 +28,13 @@ int launch_s2d_input(bool half_storage, const S2dArgs& a, hipStream_t st) {
     return 0;
 }
 
+int launch_subsample(bool half_storage, const SubsampleArgs& a, hipStream_t st) {
+    const long items = a.planes * a.H2 * ((a.W2 + 7) / 8);
+    if (half_storage) hipLaunchKernelGGL((subsample_kernel<_Float16>), dim3(blocks_for(items)), dim3(WG_THREADS), 0, st, a);
+    else hipLaunchKernelGGL((subsample_kernel<float>), dim3(blocks_for(items)), dim3(WG_THREADS), 0, st, a);
+    return 0;
+}
+
 int launch_s2d_filter(bool half_storage, const S2dFilterArgs& a, bool to_caller, hipStream_t st) {
     const long items = 4L * a.Co * 4 * a.Ci * a.K2h * a.K2w;
     if (half_storage)

@@ -28,7 +28,7 @@ namespace phx {
 // from the environment once; phx_tuning_reload() reads them again and forgets the cached plans.
 struct Tuning {
     int tile_wco = 0, tile_ntw = 0;   // PHX_TUNE_TILE="wco,ntw"
-    bool flat = false, noflat = false, nopw = false, pw8 = false, zi8 = false, wg8 = false, nos2d = false, noearly = false, norealx = false;
+    bool flat = false, noflat = false, nopw = false, pw8 = false, zi8 = false, wg8 = false, nos2d = false, noearly = false, norealx = false, nosub = false;
     bool nopwx = false;               // PHX_TUNE_NOPWX: pointwise fp16 problems stay on the staged-window kernels
     int vec = 0;                      // PHX_TUNE_VEC (0 = unset)
     int wgs = 0;                      // PHX_TUNE_WGS (0 = unset)
@@ -47,6 +47,7 @@ struct Tuning {
         nos2d = getenv("PHX_TUNE_NOS2D") != nullptr;
         noearly = getenv("PHX_TUNE_NOEARLY") != nullptr;
         norealx = getenv("PHX_TUNE_NOREALX") != nullptr;
+        nosub = getenv("PHX_TUNE_NOSUB") != nullptr;
         nopwx = getenv("PHX_TUNE_NOPWX") != nullptr;
         if (const char* e = getenv("PHX_TUNE_VEC")) vec = atoi(e);
         if (const char* e = getenv("PHX_TUNE_WGS")) wgs = atoi(e);
@@ -1140,9 +1141,31 @@ static bool s2d_view(const Problem& p, S2dView& v) {
     return true;
 }
 
+// A strided, unpadded pointwise convolution as the unit-stride one on the rows and columns it reads (forward and
+// filter gradient; the input gradient has its phases): the problem q on the subsampled input and that copy's size.
+// q-ResNet-50's three downsampling shortcuts, N=64: forward 0.07 ms on the general kernel.
+static bool subsample_view(const Problem& p, Problem& q, size_t& xs_bytes) {
+    if (p.kh != 1 || p.kw != 1 || (p.sh == 1 && p.sw == 1) || p.pt || p.pl || p.pb || p.pr || is_empty(p)) return false;
+    if (p.groups > 1 || p.nhwc || p.real_input || tune().nosub) return false;
+    q = p;
+    q.h = p.ho; q.w = p.wo; q.sh = q.sw = 1;
+    if (out_size(q.h, 1, 1, 1, 0, 0) != p.ho || out_size(q.w, 1, 1, 1, 0, 0) != p.wo) return false;
+    xs_bytes = align_up((size_t)4 * p.n * p.ci * p.ho * p.wo * (p.dtype == PHX_F32 ? 4 : 2), 256);
+    return true;
+}
+
+static void subsample_input(const Problem& p, const void* x, void* xs, hipStream_t st) {
+    SubsampleArgs a;
+    a.src = x; a.dst = xs; a.planes = 4L * p.n * p.ci; a.H = p.h; a.W = p.w; a.H2 = p.ho; a.W2 = p.wo; a.sh = p.sh; a.sw = p.sw;
+    launch_subsample(p.dtype == PHX_F16, a, st);
+}
+
 static size_t workspace_for(const Problem& p, int pass) {
     S2dView v;
     if (pass != PHX_PASS_BWD_DATA && s2d_view(p, v)) return v.x2_bytes + v.w2_bytes + workspace_plain(v.q, pass);
+    Problem q;
+    size_t xs_bytes = 0;
+    if (pass != PHX_PASS_BWD_DATA && subsample_view(p, q, xs_bytes)) return xs_bytes + workspace_plain(q, pass);
     return workspace_plain(p, pass);
 }
 
@@ -1170,6 +1193,17 @@ static int do_fwd(const Problem& p, hipStream_t st, const void* x, const void* w
         g_name_prefix = "s2d_";
         const int rc = run_corr(v.q, corr_forward(v.q), MAP_FWD, st, x2, w2, b, y, w2 + v.w2_bytes,
                                 wsb - v.x2_bytes - v.w2_bytes);
+        g_name_prefix = "";
+        return rc;
+    }
+    Problem q;
+    size_t xs_bytes = 0;
+    if (subsample_view(p, q, xs_bytes)) {
+        if (wsb < xs_bytes || !ws) return PHX_ERR_WORKSPACE;
+        subsample_input(p, x, ws, st);
+        PHX_HIP(hipGetLastError());
+        g_name_prefix = "sub_";
+        const int rc = run_corr(q, corr_forward(q), MAP_FWD, st, ws, w, b, y, static_cast<char*>(ws) + xs_bytes, wsb - xs_bytes);
         g_name_prefix = "";
         return rc;
     }
@@ -1238,6 +1272,17 @@ static int do_bwd_weights(const Problem& p, hipStream_t st, const void* x, const
         launch_s2d_filter(p.dtype == PHX_F16, fa, true, st);
         PHX_HIP(hipGetLastError());
         return PHX_OK;
+    }
+    Problem q;
+    size_t xs_bytes = 0;
+    if (subsample_view(p, q, xs_bytes)) {
+        if (wsb < xs_bytes || !ws) return PHX_ERR_WORKSPACE;
+        subsample_input(p, x, ws, st);
+        PHX_HIP(hipGetLastError());
+        g_name_prefix = "sub_";
+        const int rc = run_wgrad(flatten_pointwise(q), st, ws, g, dw, static_cast<char*>(ws) + xs_bytes, wsb - xs_bytes);
+        g_name_prefix = "";
+        return rc;
     }
     const Problem f = flatten_pointwise(p);
     return run_wgrad(f, st, x, g, dw, ws, wsb);
