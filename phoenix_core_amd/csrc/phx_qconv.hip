@@ -28,7 +28,7 @@ namespace phx {
 // from the environment once; phx_tuning_reload() reads them again and forgets the cached plans.
 struct Tuning {
     int tile_wco = 0, tile_ntw = 0;   // PHX_TUNE_TILE="wco,ntw"
-    bool flat = false, noflat = false, nopw = false, pw8 = false, zi8 = false, wg8 = false, nos2d = false, noearly = false, norealx = false, nosub = false;
+    bool flat = false, noflat = false, nopw = false, pw8 = false, zi8 = false, wg8 = false, nos2d = false, noearly = false, norealx = false, nosub = false, oldplan = false;
     bool nopwx = false;               // PHX_TUNE_NOPWX: pointwise fp16 problems stay on the staged-window kernels
     int vec = 0;                      // PHX_TUNE_VEC (0 = unset)
     int wgs = 0;                      // PHX_TUNE_WGS (0 = unset)
@@ -48,6 +48,7 @@ struct Tuning {
         noearly = getenv("PHX_TUNE_NOEARLY") != nullptr;
         norealx = getenv("PHX_TUNE_NOREALX") != nullptr;
         nosub = getenv("PHX_TUNE_NOSUB") != nullptr;
+        oldplan = getenv("PHX_TUNE_OLDPLAN") != nullptr;
         nopwx = getenv("PHX_TUNE_NOPWX") != nullptr;
         if (const char* e = getenv("PHX_TUNE_VEC")) vec = atoi(e);
         if (const char* e = getenv("PHX_TUNE_WGS")) wgs = atoi(e);
@@ -394,6 +395,14 @@ static bool plan_forward(const Corr& c, int mode, bool f16mfma, FwdPlan& best, b
                     const double cus = 256.0;
                     const double rounds = 0.5 * std::ceil(wgs / cus) + 0.5 * (wgs / cus);
                     score = 1e6 * rate / (rounds * BN * 32.0 * WCO) * (0.9 + 0.1 * halo);
+                } else if (ldsk && !pointwise && !tune().oldplan) {
+                    // the 16-product LDS kernels by the same count (one column tile per wave: two workgroups share a
+                    // CU at about half speed each, so the rounds are still rounds over the CUs)
+                    // (measured at 128 channels 28x28 and 256 channels 14x14, N=128, per unit of tile area)
+                    const double rate = NTW == 2 ? (WCO == 1 ? 1.05 : 1.0) : (WCO == 1 ? 1.05 : WCO == 2 ? 1.04 : 0.87);
+                    const double cus = 256.0;
+                    const double rounds = 0.5 * std::ceil(wgs / cus) + 0.5 * (wgs / cus);
+                    score = 1e6 * rate / (rounds * BN * 32.0 * WCO) * (0.9 + 0.1 * halo);
                 } else if (ldsk) score *= (NTW == 2 ? 1.25 : 1.0) * (WCO == 2 ? 1.08 : 1.0);
                 else if (f16mfma && NTW == 2) score *= 0.8;  // that kernel drops to one workgroup per CU
                 if (tall && force_flat) score *= 100.0;  // (tests: flat tiling wherever it applies)
@@ -563,6 +572,12 @@ static bool plan_corr_uncached(const Corr& creal, int mode, bool f16mfma, Corr& 
     // components as well would need a kernel variant of its own: a run-time branch around them slowed every
     // 16-product convolution by 5-15 %.
     if (f16mfma && mode == 8 && c.ncomp == 1 && !tune().zi8) pl.kmode = 16;
+    // One or two 16-channel chunks to reduce over: a workgroup is mostly its start and its epilogue, which the
+    // 16-product kernel has less of (four accumulators to write out instead of eight lanes to merge, two workgroups
+    // per CU with one column tile per wave).  3x3 on 16 channels at 56x56, N=64: 0.063 -> 0.047 ms; on 32 at 28x28:
+    // 0.029 -> 0.028; from 64 channels on the factorized kernel wins (14x14: 0.032 against 0.033).
+    // (with 25 taps the halved products count again: 5x5 on 24 channels 0.031 against 0.034 ms)
+    if (f16mfma && mode == 8 && c.Kh * c.Kw > 1 && c.Kh * c.Kw <= 9 && c.Cin <= 32 && !tune().zi8) pl.kmode = 16;
     return plan_forward(c, pl.kmode, f16mfma, pl);
 }
 
