@@ -67,6 +67,8 @@ CONV_CASES = [
     ("k3_valid", 1, 4, 4, 9, 9, 3, 3, 1, 1, "VALID"),
     ("k3_s2", 2, 8, 16, 15, 14, 3, 3, 2, 1, "SAME"),
     ("pw_s2", 2, 8, 16, 14, 14, 1, 1, 2, 1, "VALID"),
+    ("pw_s2_odd", 3, 10, 12, 15, 13, 1, 1, 2, 1, "VALID"),    # strided pointwise: runs on a subsampled copy of the input
+    ("pw_s31", 2, 6, 9, 10, 27, 1, 1, (3, 1), 1, "VALID"),
     ("k7_s2", 1, 3, 16, 30, 30, 7, 7, 2, 1, "SAME"),
     ("k3_s2_c4", 2, 4, 8, 15, 13, 3, 3, 2, 1, "SAME"),       # few input channels, stride 2: space-to-depth path
     ("k5_s2_valid", 1, 2, 8, 17, 16, 5, 5, 2, 1, "VALID"),
@@ -98,6 +100,8 @@ def test_conv_fp32(case, mode):
     assert_close(y.cpu().numpy(), want_y, dtype, "fwd " + kernel)
     assert_close(dx.cpu().numpy(), want_dx, dtype, "dgrad " + name)
     assert_close(dw.cpu().numpy(), want_dw, dtype, "wgrad " + name)
+    if name.startswith("pw_s"):  # a strided pointwise convolution runs forward (and its filter gradient) in the subsampled form
+        assert kernel.startswith("sub_"), kernel
 
 
 @pytest.mark.parametrize("mode", [16, 8])
@@ -241,7 +245,7 @@ def test_empty_input_is_a_no_op_and_zeroes_dw():
 
 
 FP16_CASES = [c for c in CONV_CASES if c[0] in ("pw_64", "pw_ragged", "pw_7x7img", "k3_same", "k3_same_56", "k3_ragged",
-                                                "k3_valid", "k3_s2", "pw_s2", "k7_s2", "k3_s2_c4", "k5_s2_valid", "k3_dil2", "k32_s21", "k32_asym",
+                                                "k3_valid", "k3_s2", "pw_s2", "pw_s2_odd", "pw_s31", "k7_s2", "k3_s2_c4", "k5_s2_valid", "k3_dil2", "k32_s21", "k32_asym",
                                                 "co_gt_128")] + [
     ("k3_s3", 2, 8, 8, 13, 13, 3, 3, 3, 1, "SAME"),
     ("k4_same", 2, 8, 16, 13, 15, 4, 4, 1, 1, "SAME"),        # four taps per filter row share a filter-gradient workgroup
