@@ -15,6 +15,33 @@ from torch import nn
 from . import ops
 
 
+# The two gradients of a convolution are independent of each other.  With OVERLAP_BACKWARD the filter gradient is
+# enqueued on a second stream (default priority) between two joins with the caller's stream, so that on layers too
+# small to fill the GPU the two kernels run side by side.
+OVERLAP_BACKWARD = True
+_side_streams = {}
+
+
+def _side_stream(device):
+    s = _side_streams.get(device)
+    if s is None:
+        s = _side_streams[device] = torch.cuda.Stream(device=device)
+    return s
+
+
+def _conv_backward(x, w, grad, bdesc):
+    if not (OVERLAP_BACKWARD and bdesc.require_input_grad):
+        return ops.conv2d_bwd(x, w, grad, bdesc)
+    main, side = torch.cuda.current_stream(x.device), _side_stream(x.device)
+    side.wait_stream(main)  # x and grad are complete where the side stream starts
+    with torch.cuda.stream(side):
+        dw = ops.conv2d_bwd_weights(x, grad, bdesc)
+    dx = ops.conv2d_bwd_data(w, grad, bdesc)
+    main.wait_stream(side)  # whatever follows on the caller's stream may read dw (and free x, grad)
+    dw.record_stream(main)
+    return dw, dx
+
+
 class _QConv2dFn(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, w, bias, fdesc, bdesc):
@@ -27,7 +54,7 @@ class _QConv2dFn(torch.autograd.Function):
     def backward(ctx, grad):
         x, w = ctx.saved_tensors
         grad = grad.contiguous()
-        dw, dx = ops.conv2d_bwd(x, w, grad, ctx.bdesc)
+        dw, dx = _conv_backward(x, w, grad, ctx.bdesc)
         db = None
         if ctx.has_bias:  # bias enters every output component once: plain reduction
             n = grad.shape[0] // 4

@@ -284,27 +284,41 @@ def conv2d_fwd(x, w, bias, desc, out=None):
     return y
 
 
-def conv2d_bwd(x, w, grad, desc):
-    """conv2DBwd (src/upstride.hpp:35-51): returns (dw, dx); dx is None when the descriptor does
-    not require the input gradient."""
-    dev = _dev_check(x, w, grad)
+def conv2d_bwd_weights(x, grad, desc):
+    """The filter-gradient half of conv2DBwd (src/conv2d.hpp:330-440): dw."""
+    dev = _dev_check(x, grad)
     _expect(x, desc.input_shape, desc.dtype, "input")
-    _expect(w, desc.filter_shape, desc.dtype, "filter")
     _expect(grad, desc.output_shape, desc.dtype, "output gradient")
     dw = torch.empty(desc.filter_shape, dtype=desc.dtype, device=dev)
     nbytes = desc.workspace_bytes(capi.PHX_PASS_BWD_WEIGHTS)
     ws = _workspace.get(dev, nbytes)
     capi.check(capi.lib().phx_qconv2d_bwd_weights(ctypes.byref(desc.c), _stream(), _ptr(x), _ptr(grad), _ptr(dw),
                                                   _ptr(ws), nbytes), "phx_qconv2d_bwd_weights")
-    dx = None
-    if desc.require_input_grad:
-        if desc.real_valued_input:  # src/conv2d.hpp:394-398
-            raise RuntimeError("Input gradient required for type0 input tensor")
-        dx = torch.empty(desc.input_shape, dtype=desc.dtype, device=dev)
-        nbytes = desc.workspace_bytes(capi.PHX_PASS_BWD_DATA)
-        ws = _workspace.get(dev, nbytes)
-        capi.check(capi.lib().phx_qconv2d_bwd_data(ctypes.byref(desc.c), _stream(), _ptr(grad), _ptr(w), _ptr(dx),
-                                                   _ptr(ws), nbytes), "phx_qconv2d_bwd_data")
+    return dw
+
+
+def conv2d_bwd_data(w, grad, desc):
+    """The input-gradient half of conv2DBwd: dx (the descriptor must ask for it)."""
+    dev = _dev_check(w, grad)
+    _expect(w, desc.filter_shape, desc.dtype, "filter")
+    _expect(grad, desc.output_shape, desc.dtype, "output gradient")
+    if desc.real_valued_input:  # src/conv2d.hpp:394-398
+        raise RuntimeError("Input gradient required for type0 input tensor")
+    dx = torch.empty(desc.input_shape, dtype=desc.dtype, device=dev)
+    nbytes = desc.workspace_bytes(capi.PHX_PASS_BWD_DATA)
+    ws = _workspace.get(dev, nbytes)
+    capi.check(capi.lib().phx_qconv2d_bwd_data(ctypes.byref(desc.c), _stream(), _ptr(grad), _ptr(w), _ptr(dx),
+                                               _ptr(ws), nbytes), "phx_qconv2d_bwd_data")
+    return dx
+
+
+def conv2d_bwd(x, w, grad, desc):
+    """conv2DBwd (src/upstride.hpp:35-51): returns (dw, dx); dx is None when the descriptor does
+    not require the input gradient."""
+    _dev_check(x, w, grad)
+    _expect(w, desc.filter_shape, desc.dtype, "filter")
+    dw = conv2d_bwd_weights(x, grad, desc)
+    dx = conv2d_bwd_data(w, grad, desc) if desc.require_input_grad else None
     return dw, dx
 
 

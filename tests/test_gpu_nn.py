@@ -41,6 +41,41 @@ def test_qconv2d_autograd_matches_oracle(mode):
         assert np.abs(got - want).max() / np.abs(want).max() < 1e-4
 
 
+def test_overlapped_backward_equals_the_sequential_one():
+    """The filter gradient on a second stream (nn.OVERLAP_BACKWARD) must give exactly what the one-stream backward
+    gives: a small stack of convolutions, stepped several times with fresh tensors each time (buffers of earlier
+    steps are recycled by the allocator while later kernels run), both ways, bit for bit."""
+    from phoenix_core_amd import nn as qnn
+    torch.manual_seed(3)
+    ctx = Ctx(8, "full16")
+    layers = torch.nn.ModuleList([phx.QConv2d(16, 32, 3, dtype=torch.float16, context=ctx), phx.QConv2d(32, 32, 1, dtype=torch.float16, context=ctx),
+                                  phx.QConv2d(32, 16, 3, stride=2, dtype=torch.float16, context=ctx)]).cuda()
+    xs = [torch.randn(8, 16, 20, 20, device="cuda").half() for _ in range(4)]
+
+    def run(overlap):
+        old, qnn.OVERLAP_BACKWARD = qnn.OVERLAP_BACKWARD, overlap
+        try:
+            out = []
+            for x0 in xs:
+                for m in layers:
+                    m.weight.grad = None
+                x = x0.clone().requires_grad_(True)
+                y = x
+                for m in layers:
+                    y = m(y)
+                y.float().square().mean().backward()
+                out.append([x.grad.clone()] + [m.weight.grad.clone() for m in layers])
+            torch.cuda.synchronize()
+            return out
+        finally:
+            qnn.OVERLAP_BACKWARD = old
+
+    want, got = run(False), run(True)
+    for a, b in zip(want, got):
+        for ta, tb in zip(a, b):
+            assert torch.equal(ta, tb)
+
+
 def test_qconv2d_groups_and_channels_last():
     """QConv2d(groups=G) is G ungrouped layers on channel slices; QConv2d(data_format="NHWC") is the NCHW layer on
     permuted activations: outputs and all gradients must agree with those compositions."""
