@@ -79,6 +79,8 @@ def parse():
     ap.add_argument("--batch", type=int, default=64, help="images per step of the ResNet workload")
     ap.add_argument("--torch-bn", action="store_true",
                     help="ResNet workload: torch.nn.BatchNorm2d + ReLU (MIOpen) instead of the library's batch-norm kernels")
+    ap.add_argument("--frozen-filters", action="store_true",
+                    help="ResNet workload: the filters do not change between steps, so no step packs them again")
     ap.add_argument("--no-graph", action="store_true", help="time the eager steps only (no HIP graph replay)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -491,8 +493,15 @@ def run_resnet(mode, policy, args):
     labels = torch.randint(0, 1000, (n,), device=dev)
     last = {}
 
+    convs = [m for m in model.modules() if isinstance(m, phx.QConv2d)]
+
     def step():
         model.zero_grad(set_to_none=True)
+        if not args.frozen_filters:
+            # a training step follows an optimizer update: every layer packs its filter anew (once, for the forward
+            # pass and the input gradient together); with frozen filters the packed images of the first step stay valid
+            for m in convs:
+                m.invalidate_packed_filters()
         loss = torch.nn.functional.cross_entropy(model(images).float(), labels)
         loss.backward()
         return loss.detach()
@@ -511,6 +520,8 @@ def run_resnet(mode, policy, args):
                        "the library's streaming kernels (include/phx_bn.h)",
                        "is captured once into a HIP graph and replayed" if graph["used"] else "runs eagerly"),
         "product_mode": mode, "fp16_policy": policy, "batch_norm": "torch" if args.torch_bn else "library", "dtype": "f16",
+        "filters": "frozen (packed once, before the timed steps)" if args.frozen_filters else
+                   "packed once per step and layer, for the forward pass and the input gradient together",
         "value": n / (ms_per_step * 1e-3), "unit": "img/s", "images_per_s": n / (ms_per_step * 1e-3),
         "ms_per_step": ms_per_step, "ms_per_step_eager": eager_ms, "images_per_s_eager": n / (eager_ms * 1e-3),
         "hip_graph": graph,

@@ -180,6 +180,31 @@ int phx_qconv2d_bwd_data(const phx_qconv_desc* desc, phx_stream_t stream, const 
 int phx_qconv2d_bwd_weights(const phx_qconv_desc* desc, phx_stream_t stream, const void* x, const void* grad,
                             void* dw, void* workspace, size_t workspace_bytes);
 
+/* Filters packed ahead of the passes that read them.  Every forward and input-gradient call above first rewrites
+ * the filter into the operand order of the kernel it runs (for the factorized product: into the eight right-hand
+ * lanes, the job of decomposeRightInput in the reference, src/backend/cudnn/kernels_quat.cu:34-49, which the
+ * reference likewise repeats in every call, src/conv2d.hpp:176-207, 442-495).  A caller whose filter changes once
+ * per training step, or never (inference), can do that once: phx_qconv2d_pack_filters writes the images of the
+ * forward pass and of the input gradient with ONE kernel launch, and the *_prepacked entry points run the same
+ * kernels on them without packing.  No counterpart in the reference's interface.
+ *   phx_qconv2d_packed_filter_bytes(desc, pass): bytes of the image for pass PHX_PASS_FWD or PHX_PASS_BWD_DATA;
+ *     0 = this descriptor has no prepacked form for that pass (non-quaternion algebra, empty input, the
+ *     space-to-depth forward path of strided convolutions with at most 4 input channels, the input gradient of a
+ *     real-valued input): use the plain entry point.
+ *   phx_qconv2d_pack_filters: either image pointer may be NULL (that image is not made); buffers 16-byte aligned.
+ *   An image is valid for the descriptor it was packed for (same sizes, dtype, policy and product mode), on any
+ *   stream ordered after the packing call, until the filter changes.  Results are bit-identical to the plain
+ *   entry points'.  The workspace of a prepacked call is that of the plain call (phx_qconv2d_workspace_bytes). */
+size_t phx_qconv2d_packed_filter_bytes(const phx_qconv_desc* desc, int pass);
+int phx_qconv2d_pack_filters(const phx_qconv_desc* desc, phx_stream_t stream, const void* w, void* packed_fwd,
+                             size_t packed_fwd_bytes, void* packed_bwd_data, size_t packed_bwd_data_bytes);
+int phx_qconv2d_fwd_prepacked(const phx_qconv_desc* desc, phx_stream_t stream, const void* x, const void* packed_fwd,
+                              size_t packed_fwd_bytes, const void* bias_or_null, void* y, void* workspace,
+                              size_t workspace_bytes);
+int phx_qconv2d_bwd_data_prepacked(const phx_qconv_desc* desc, phx_stream_t stream, const void* grad,
+                                   const void* packed_bwd_data, size_t packed_bwd_data_bytes, void* dx, void* workspace,
+                                   size_t workspace_bytes);
+
 /* Dense trio.  Replaces UpstrideDenseFunctor / UpstrideDenseGradFunctor for the quaternion
  * algebra (src/dense.hpp:52-62, 77-180, 223-237, 252-377). */
 int phx_qdense_fwd(const phx_qdense_desc* desc, phx_stream_t stream, const void* x, const void* w,

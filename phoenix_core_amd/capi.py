@@ -30,6 +30,8 @@ EXPORTS = (
     "phx_memset_zero", "phx_stream_create", "phx_stream_destroy", "phx_stream_synchronize",
     "phx_last_kernel_name", "phx_profile_enable", "phx_profile_collect", "phx_algebra_map",
     "phx_init", "phx_tuning_reload", "phx_qconv2d_fwd_noalloc",
+    "phx_qconv2d_packed_filter_bytes", "phx_qconv2d_pack_filters", "phx_qconv2d_fwd_prepacked",
+    "phx_qconv2d_bwd_data_prepacked",
 )
 
 
@@ -83,6 +85,11 @@ def lib():
         L.phx_qconv2d_fwd.argtypes = [cd, vp, vp, vp, vp, vp, vp, sz]
         L.phx_qconv2d_fwd_noalloc.argtypes = [cd, vp, vp, vp, vp, vp]
         L.phx_qconv2d_bwd_data.argtypes = [cd, vp, vp, vp, vp, vp, sz]
+        L.phx_qconv2d_packed_filter_bytes.restype = sz
+        L.phx_qconv2d_packed_filter_bytes.argtypes = [cd, ctypes.c_int]
+        L.phx_qconv2d_pack_filters.argtypes = [cd, vp, vp, vp, sz, vp, sz]
+        L.phx_qconv2d_fwd_prepacked.argtypes = [cd, vp, vp, vp, sz, vp, vp, vp, sz]
+        L.phx_qconv2d_bwd_data_prepacked.argtypes = [cd, vp, vp, vp, sz, vp, vp, sz]
         L.phx_qconv2d_bwd_weights.argtypes = [cd, vp, vp, vp, vp, vp, sz]
         L.phx_qdense_fwd.argtypes = [dd, vp, vp, vp, vp, vp, vp, sz]
         L.phx_qdense_bwd_data.argtypes = [dd, vp, vp, vp, vp, vp, sz]

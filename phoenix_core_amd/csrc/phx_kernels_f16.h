@@ -233,13 +233,13 @@ __global__ void __launch_bounds__(WG_THREADS, (MODE == 8 || NTW == 1) ? 2 : 1) q
 // MODE 8: the eight right-operand lanes, formed in fp32 and rounded once (both of the conjugated filter for
 // MAP_DGRAD: dx = g (x) conj(w) is a forward product, and the forward kernel runs it).
 template <int MODE, int MAP>
-__global__ void __launch_bounds__(WG_THREADS) pack_filters_f16_kernel(const PackArgs P) {
+__device__ __forceinline__ void pack_filters_f16_body(const PackArgs& P, long first, long stride) {
     constexpr int WC = (MODE == 16) ? 4 : 8;
     const int taps = P.Kh * P.Kw;
     const long total = (long)P.row_tiles * P.nchunks * taps * 64;
     const _Float16* w = static_cast<const _Float16*>(P.w);
     f16x8* outv = reinterpret_cast<f16x8*>(P.out);
-    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
+    for (long idx = first; idx < total; idx += stride) {
         const int lane = idx & 63;
         long s = idx >> 6;
         const int tap = s % taps;
@@ -277,6 +277,11 @@ __global__ void __launch_bounds__(WG_THREADS) pack_filters_f16_kernel(const Pack
 #pragma unroll
         for (int v = 0; v < WC; ++v) outv[idx * WC + v] = vec[v];
     }
+}
+
+template <int MODE, int MAP>
+__global__ void __launch_bounds__(WG_THREADS) pack_filters_f16_kernel(const PackArgs P) {
+    pack_filters_f16_body<MODE, MAP>(P, (long)blockIdx.x * blockDim.x + threadIdx.x, (long)gridDim.x * blockDim.x);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -710,7 +715,7 @@ struct PackLdsArgs {
 };
 
 template <int MODE, int MAP>
-__global__ void __launch_bounds__(WG_THREADS) pack_filters_f16_lds_kernel(const PackLdsArgs A) {
+__device__ __forceinline__ void pack_filters_f16_lds_body(const PackLdsArgs& A, long first, long stride) {
     const PackArgs& P = A.base;
     constexpr int TG = F16_TG;
     constexpr int NW = (MODE == 16) ? 4 : 8;
@@ -723,7 +728,7 @@ __global__ void __launch_bounds__(WG_THREADS) pack_filters_f16_lds_kernel(const 
     const long total = (long)P.row_tiles * P.nchunks * A.ngroups * TG * A.WCO * (NW / PER) * 64 * 8;
     const _Float16* w = static_cast<const _Float16*>(P.w);
     _Float16* outh = static_cast<_Float16*>(P.out);
-    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
+    for (long idx = first; idx < total; idx += stride) {
         const int i = idx & 7;
         const int lane = (idx >> 3) & 63;
         long s = idx >> 9;
@@ -774,6 +779,11 @@ __global__ void __launch_bounds__(WG_THREADS) pack_filters_f16_lds_kernel(const 
             for (int q = 0; q < PER; ++q) outh[(((slot * NW + q) * 64 + lane) << 3) + i] = val[q];
         }
     }
+}
+
+template <int MODE, int MAP>
+__global__ void __launch_bounds__(WG_THREADS) pack_filters_f16_lds_kernel(const PackLdsArgs A) {
+    pack_filters_f16_lds_body<MODE, MAP>(A, (long)blockIdx.x * blockDim.x + threadIdx.x, (long)gridDim.x * blockDim.x);
 }
 
 // ---------------------------------------------------------------------------------------------

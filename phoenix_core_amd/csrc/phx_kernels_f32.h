@@ -519,13 +519,15 @@ struct PackArgs {
     int row_tiles, nchunks;
 };
 
+// (the packing bodies take the thread's first index and the stride of its loop, so that one launch can also pack
+// several filter images side by side: pack_jobs_kernel)
 template <typename TS, int MODE, int MAP>
-__global__ void __launch_bounds__(WG_THREADS) pack_filters_f32_kernel(const PackArgs P) {
+__device__ __forceinline__ void pack_filters_f32_body(const PackArgs& P, long first, long stride) {
     constexpr int WC = (MODE == 16) ? 4 : 8;
     const int taps = P.Kh * P.Kw;
     const long total = (long)P.row_tiles * P.nchunks * taps * 4 * 64;
     const TS* w = static_cast<const TS*>(P.w);
-    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
+    for (long idx = first; idx < total; idx += stride) {
         const int lane = idx & 63;
         long s = idx >> 6;
         const int cp = s & 3;
@@ -565,6 +567,11 @@ __global__ void __launch_bounds__(WG_THREADS) pack_filters_f32_kernel(const Pack
             for (int i = 0; i < 8; ++i) dst[i] = R[i];
         }
     }
+}
+
+template <typename TS, int MODE, int MAP>
+__global__ void __launch_bounds__(WG_THREADS) pack_filters_f32_kernel(const PackArgs P) {
+    pack_filters_f32_body<TS, MODE, MAP>(P, (long)blockIdx.x * blockDim.x + threadIdx.x, (long)gridDim.x * blockDim.x);
 }
 
 // ---------------------------------------------------------------------------------------------

@@ -476,12 +476,12 @@ struct PackPwxArgs {
 };
 
 template <int MAP>
-__global__ void __launch_bounds__(WG_THREADS) pack_filters_pwx_kernel(const PackPwxArgs A) {
+__device__ __forceinline__ void pack_filters_pwx_body(const PackPwxArgs& A, long first, long stride) {
     const PackArgs& P = A.base;
     const long total = (long)P.row_tiles * A.nsteps * A.WCO * 4 * 64;
     const _Float16* w = static_cast<const _Float16*>(P.w);
     f16x8* outv = reinterpret_cast<f16x8*>(P.out);
-    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
+    for (long idx = first; idx < total; idx += stride) {
         const int lane = idx & 63;
         long s = idx >> 6;
         const int r = s & 3; s >>= 2;
@@ -505,6 +505,11 @@ __global__ void __launch_bounds__(WG_THREADS) pack_filters_pwx_kernel(const Pack
         }
         outv[idx] = vec;
     }
+}
+
+template <int MAP>
+__global__ void __launch_bounds__(WG_THREADS) pack_filters_pwx_kernel(const PackPwxArgs A) {
+    pack_filters_pwx_body<MAP>(A, (long)blockIdx.x * blockDim.x + threadIdx.x, (long)gridDim.x * blockDim.x);
 }
 
 }  // namespace phx

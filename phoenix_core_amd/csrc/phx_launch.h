@@ -51,6 +51,26 @@ int launch_pwx_nhwc_f16(int WCO, const PwxArgs& a, int blocks, hipStream_t st); 
 size_t pwx_packed_bytes(int WCO, int co_tiles, int nsteps);
 int launch_pack_filters_pwx(int map, int WCO, int nsteps, const PackArgs& a, hipStream_t st);
 
+// Several filter images packed by one launch (phx_launch_pack.hip): a convolution's forward and input-gradient
+// images, the sub-filters of a strided input gradient's phases, the groups of a grouped convolution.  A job is one
+// call of one of the packing kernels above; the workgroups of the launch are dealt to the jobs in order.
+enum PackKind { PACK_F32 = 0, PACK_F16 = 1, PACK_F16_LDS = 2, PACK_PWX = 3 };
+struct PackJob {
+    PackArgs a;
+    int kind;                    // PackKind
+    int half_storage;            // PACK_F32: the filter is stored as fp16
+    int mode, map;               // 16 / 8, MAP_FWD / MAP_DGRAD
+    int WCO, ngroups, pw;        // PACK_F16_LDS (PackLdsArgs), PACK_PWX (WCO)
+    int nsteps;                  // PACK_PWX
+    int block0, nblocks;         // this job's workgroups: [block0, block0 + nblocks)
+};
+constexpr int PACK_JOBS_MAX = 12;
+struct PackJobs {
+    int n;
+    PackJob job[PACK_JOBS_MAX];
+};
+int launch_pack_jobs(const PackJobs& jobs, hipStream_t st);
+
 // wave sets (reduction slices) per workgroup of the fp32-MFMA filter-gradient kernel
 constexpr int wgrad_f32_ksets(int mode, bool vec) { return (mode == 8 && vec) ? 2 : 1; }
 int launch_wgrad_f32(bool half_storage, bool vec, int mode, const WgradArgs& a, dim3 grid, size_t lds_bytes,

@@ -6,8 +6,16 @@ namespace phx {
 template <typename TS, bool VEC>
 static void launch_ts(int mode, const WgradArgs& a, dim3 grid, size_t lds_bytes, hipStream_t st) {
     constexpr int KSETS = wgrad_f32_ksets(8, VEC);
-    if (mode == 16) hipLaunchKernelGGL((qconv_wgrad_f32_kernel<TS, 16, 3, VEC, 1>), grid, dim3(WG_THREADS), lds_bytes, st, a);
-    else hipLaunchKernelGGL((qconv_wgrad_f32_kernel<TS, 8, 1, VEC, KSETS>), grid, dim3(WG_THREADS * KSETS), lds_bytes, st, a);
+    if (mode == 16) {
+        hipLaunchKernelGGL((qconv_wgrad_f32_kernel<TS, 16, 3, VEC, 1>), grid, dim3(WG_THREADS), lds_bytes, st, a);
+    } else {
+        // (eight waves: one workgroup per CU, which may then use more than 64 KiB of LDS -- opted in at set-up, see BigLds)
+        constexpr auto kernel = qconv_wgrad_f32_kernel<TS, 8, 1, VEC, KSETS>;
+        if constexpr (KSETS == 2) {
+            if (!BigLds<kernel>::registered) return;
+        }
+        hipLaunchKernelGGL(kernel, grid, dim3(WG_THREADS * KSETS), lds_bytes, st, a);
+    }
 }
 
 int launch_wgrad_f32(bool half_storage, bool vec, int mode, const WgradArgs& a, dim3 grid, size_t lds_bytes,

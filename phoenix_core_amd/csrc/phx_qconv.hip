@@ -140,6 +140,67 @@ static thread_local const char* g_last_kernel = "";
 static thread_local char g_name_buf[160];
 static thread_local const char* g_name_prefix = "";  // "s2d_" while a rewritten problem runs
 
+// Filters packed ahead of the passes that use them (phx_qconv2d_pack_filters and the *_prepacked entry points).
+// The forward and input-gradient code paths run as always, and this thread's session tells the places that pack
+// what to do instead: SIZE adds up the bytes the packed images take, RECORD notes every packing call as a job of one
+// combined launch (and launches nothing else), USE skips the packing and reads the images where RECORD put them.
+// The same descriptor walks the same path in all three, so the images are found by their running offset.
+struct PackSession {
+    enum Mode { OFF, SIZE, RECORD, USE };
+    Mode mode = OFF;
+    char* base = nullptr;
+    size_t capacity = 0, offset = 0;
+    hipStream_t st = nullptr;
+    PackJobs jobs{};
+    bool dry() const { return mode == SIZE || mode == RECORD; }
+};
+static thread_local PackSession g_pack;
+
+struct PackSessionScope {  // a session lasts for one entry-point call
+    PackSessionScope(PackSession::Mode m, void* base, size_t capacity, hipStream_t st) {
+        g_pack.mode = m; g_pack.base = static_cast<char*>(base); g_pack.capacity = capacity; g_pack.offset = 0; g_pack.st = st;
+    }
+    ~PackSessionScope() { g_pack.mode = PackSession::OFF; g_pack.base = nullptr; g_pack.capacity = g_pack.offset = 0; }
+};
+
+static int flush_pack_jobs() {
+    const int rc = launch_pack_jobs(g_pack.jobs, g_pack.st);
+    g_pack.jobs.n = 0;
+    return rc == 0 ? PHX_OK : PHX_ERR_NOT_SUPPORTED;
+}
+
+// Where a run's packed filters live and who packs them.  dst: the image's address (the workspace outside a
+// session); pack_now: the caller launches its packing kernel as usual; compute: the caller goes on to its kernels.
+struct PackSlot {
+    void* dst;
+    bool pack_now, compute;
+    int rc;
+};
+static PackSlot pack_slot(void* ws, size_t ws_bytes, size_t image_bytes) {
+    PackSession& s = g_pack;
+    if (s.mode == PackSession::OFF) {
+        if (ws_bytes < image_bytes || !ws) return {nullptr, false, false, PHX_ERR_WORKSPACE};
+        return {ws, true, true, PHX_OK};
+    }
+    const size_t off = s.offset;
+    s.offset += (image_bytes + 255) / 256 * 256;
+    if (s.mode == PackSession::SIZE) return {nullptr, false, false, PHX_OK};
+    if (s.offset > s.capacity || !s.base) return {nullptr, false, false, PHX_ERR_WORKSPACE};
+    return {s.base + off, false, s.mode == PackSession::USE, PHX_OK};
+}
+
+// RECORD: one more job for the combined launch (a full list is launched and started anew)
+static int record_pack_job(PackJob j, long items) {
+    PackSession& s = g_pack;
+    if (s.mode != PackSession::RECORD) return PHX_OK;
+    if (s.jobs.n == PACK_JOBS_MAX)
+        if (const int rc = flush_pack_jobs()) return rc;
+    j.block0 = s.jobs.n ? s.jobs.job[s.jobs.n - 1].block0 + s.jobs.job[s.jobs.n - 1].nblocks : 0;
+    j.nblocks = (int)std::max<long>(1, std::min<long>((items + WG_THREADS - 1) / WG_THREADS, 1024));
+    s.jobs.job[s.jobs.n++] = j;
+    return PHX_OK;
+}
+
 // optional event pairs around the dominant kernel of each call (see phx_profile_enable)
 struct ProfileState {
     std::vector<hipEvent_t> ev;  // 2 per slot
@@ -608,17 +669,28 @@ static bool plan_corr(const Corr& creal, int mode, bool f16mfma, Corr& c, FwdPla
     return it->second.ok;
 }
 
+static int record_pwx_job(const PackArgs& pa, int map, int wco, int nsteps) {
+    PackJob j{};
+    j.a = pa; j.kind = PACK_PWX; j.mode = 16; j.map = map; j.WCO = wco; j.nsteps = nsteps;
+    return record_pack_job(j, (long)pa.row_tiles * nsteps * wco * 4 * 64);
+}
+
 static int run_pwx(const Problem& p, const Corr& c, const FwdPlan& pl, int map, hipStream_t st, const void* in, const void* w,
-                   const void* bias, void* out, void* ws) {
-    DeviceState* dev = nullptr;
-    if (const int rc = device_state(&dev)) return rc;
+                   const void* bias, void* out, void* ws, size_t ws_bytes) {
+    const PackSlot slot = pack_slot(ws, ws_bytes, pl.wpk_bytes);
+    if (slot.rc != PHX_OK) return slot.rc;
+    ws = slot.dst;
     PackArgs pa{};
     pa.w = w; pa.out = ws;
     pa.wcs = p.fs.wcs; pa.so = p.fs.so; pa.si = p.fs.si; pa.skh = p.fs.skh; pa.skw = p.fs.skw;
     pa.Co = p.co; pa.Ci = p.ci; pa.Kh = 1; pa.Kw = 1;
     pa.khm = c.khm; pa.khs = c.khs; pa.kwm = c.kwm; pa.kws = c.kws;
     pa.rows = c.Cout; pa.red = c.Cin; pa.row_tiles = pl.co_tiles; pa.nchunks = pl.pwx_steps;
-    if (launch_pack_filters_pwx(map, pl.pwx, pl.pwx_steps, pa, st) != 0) return PHX_ERR_NOT_SUPPORTED;
+    if (slot.pack_now && launch_pack_filters_pwx(map, pl.pwx, pl.pwx_steps, pa, st) != 0) return PHX_ERR_NOT_SUPPORTED;
+    if (const int rrc = record_pwx_job(pa, map, pl.pwx, pl.pwx_steps)) return rrc;
+    if (!slot.compute) return PHX_OK;
+    DeviceState* dev = nullptr;
+    if (const int rc = device_state(&dev)) return rc;
     const int cin_mem = (map == MAP_FWD) ? p.ci_mem : p.co_mem, cout_mem = (map == MAP_FWD) ? p.co_mem : p.ci_mem;
     PwxArgs a{};
     a.in = static_cast<const _Float16*>(in); a.in_cs = (long)c.N * cin_mem * c.Win;
@@ -666,18 +738,22 @@ static size_t nhwc_native_workspace(const Problem& p, int pass) {
 
 static int run_pwx_nhwc(const Problem& p, int map, hipStream_t st, const void* in, const void* w, const void* bias, void* out,
                         void* ws, size_t ws_bytes) {
-    DeviceState* dev = nullptr;
-    if (const int rc = device_state(&dev)) return rc;
-    if (!in || !w || !out) return PHX_ERR_INVALID_ARGUMENT;
+    if (!g_pack.dry() && (!in || !w || !out)) return PHX_ERR_INVALID_ARGUMENT;
     const int cin = map == MAP_FWD ? p.ci : p.co, cout = map == MAP_FWD ? p.co : p.ci;
     const int wco = pwx_wco(cout), co_tiles = cdiv(cout, 32 * wco), nsteps = cdiv(cin, 16);
-    if (ws_bytes < pwx_packed_bytes(wco, co_tiles, nsteps) || !ws) return PHX_ERR_WORKSPACE;
+    const PackSlot slot = pack_slot(ws, ws_bytes, pwx_packed_bytes(wco, co_tiles, nsteps));
+    if (slot.rc != PHX_OK) return slot.rc;
+    ws = slot.dst;
     PackArgs pa{};
     pa.w = w; pa.out = ws;
     pa.wcs = p.fs.wcs; pa.so = p.fs.so; pa.si = p.fs.si; pa.skh = p.fs.skh; pa.skw = p.fs.skw;
     pa.Co = p.co; pa.Ci = p.ci; pa.Kh = 1; pa.Kw = 1; pa.khm = 0; pa.khs = 1; pa.kwm = 0; pa.kws = 1;
     pa.rows = cout; pa.red = cin; pa.row_tiles = co_tiles; pa.nchunks = nsteps;
-    if (launch_pack_filters_pwx(map, wco, nsteps, pa, st) != 0) return PHX_ERR_NOT_SUPPORTED;
+    if (slot.pack_now && launch_pack_filters_pwx(map, wco, nsteps, pa, st) != 0) return PHX_ERR_NOT_SUPPORTED;
+    if (const int rrc = record_pwx_job(pa, map, wco, nsteps)) return rrc;
+    if (!slot.compute) return PHX_OK;
+    DeviceState* dev = nullptr;
+    if (const int rc = device_state(&dev)) return rc;
     PwxArgs a{};
     const long np = (long)p.n * p.h * p.w;
     a.in = static_cast<const _Float16*>(in); a.in_cs = np * cin;
@@ -708,8 +784,10 @@ static int run_corr(const Problem& p, const Corr& creal, int map, hipStream_t st
     Corr c;
     FwdPlan pl;
     if (!plan_corr(creal, p.mode, f16, c, pl, pw)) return PHX_ERR_NOT_SUPPORTED;
-    if (ws_bytes < pl.wpk_bytes || !ws) return PHX_ERR_WORKSPACE;
-    if (pl.pwx) return run_pwx(p, creal, pl, map, st, in, w, bias, out, ws);
+    if (pl.pwx) return run_pwx(p, creal, pl, map, st, in, w, bias, out, ws, ws_bytes);
+    const PackSlot slot = pack_slot(ws, ws_bytes, pl.wpk_bytes);
+    if (slot.rc != PHX_OK) return slot.rc;
+    ws = slot.dst;
 
     FwdVariant v;
     v.half_storage = p.dtype == PHX_F16; v.f16_mfma = f16; v.mode = pl.kmode; v.map = map;
@@ -747,8 +825,16 @@ static int run_corr(const Problem& p, const Corr& creal, int map, hipStream_t st
     a.vec = (pl.TW % 4 == 0 && c.Wout % 4 == 0) ? 4 : (pl.TW % 2 == 0 && c.Wout % 2 == 0) ? 2 : 1;
     if (tune().vec > 0) a.vec = std::min(a.vec, tune().vec);
 
-    int rc = f16 ? launch_pack_filters_f16(v, pa, pack_blocks, st) : launch_pack_filters(v, pa, pack_blocks, st);
+    int rc = 0;
+    if (slot.pack_now) rc = f16 ? launch_pack_filters_f16(v, pa, pack_blocks, st) : launch_pack_filters(v, pa, pack_blocks, st);
     if (rc != 0) return PHX_ERR_NOT_SUPPORTED;
+    if (g_pack.mode == PackSession::RECORD) {
+        PackJob j{};
+        j.a = pa; j.kind = !f16 ? PACK_F32 : pl.lds_filters ? PACK_F16_LDS : PACK_F16;
+        j.half_storage = v.half_storage; j.mode = pl.kmode; j.map = map; j.WCO = pl.WCO; j.ngroups = pl.ngroups; j.pw = pw;
+        if (const int rrc = record_pack_job(j, pack_items)) return rrc;
+    }
+    if (!slot.compute) return PHX_OK;
     {
         KernelTimer timer(st);
         rc = f16 ? launch_fwd_f16(v, a, st) : launch_fwd_f32(v, a, st);
@@ -780,6 +866,30 @@ struct WgPlan {
     size_t lds_bytes, partial_bytes;
 };
 
+// Reduction slices of a filter gradient.  xy workgroups share a slice (channel tiles x tap groups), a slice walks
+// ceil(ntiles / Z) pixel tiles, `slots` workgroups run at a time.  With few workgroups per slice one round of
+// workgroups is best (Z = slots / xy: small partial sums, no straggler round) and is kept wherever it fills four
+// fifths of the slots; where xy alone is a good part of a round (large channel counts: 256 -> 256, 3x3, one tap per
+// workgroup = 144) it leaves CUs idle, and several rounds of shorter workgroups fill them.  The cost below is in units of one pixel tile of one workgroup: rounds x
+// (tiles per workgroup + one tile's worth of start-up and epilogue) + slices x the time to write and read back a
+// slice of partial sums (slice_bytes twice at 5 TB/s, against tile_flops at the rate one CU sustains).
+static int reduction_slices(int xy, int ntiles, int slots, double slice_bytes, double tile_flops, bool f16mfma) {
+    xy = std::max(1, xy);
+    const int one_round = std::max(1, std::min(ntiles, slots / xy));
+    if ((double)xy * one_round >= 0.8 * slots) return one_round;
+    const double tile_seconds = tile_flops / (f16mfma ? 4.5e12 : 0.45e12);
+    const double slice_cost = (2.0 * slice_bytes / 5e12) / tile_seconds;
+    const int zmax = std::max(1, std::min(ntiles, std::max(slots / xy, 32)));
+    int best_z = 1;
+    double best_cost = 1e300;
+    for (int z = 1; z <= zmax; ++z) {
+        const long rounds = ((long)xy * z + slots - 1) / slots;
+        const double cost = (double)rounds * ((ntiles + z - 1) / z + 1.0) + slice_cost * z;
+        if (cost < best_cost) { best_cost = cost; best_z = z; }
+    }
+    return best_z;
+}
+
 static void finish_wgrad_plan(const Problem& p, int CoT, int CiT, int per_cu, WgPlan& best) {
     best.co_tiles = cdiv(p.co, CoT); best.ci_tiles = cdiv(p.ci, CiT);
     best.CoP = best.co_tiles * CoT; best.CiP = best.ci_tiles * CiT;
@@ -788,20 +898,21 @@ static void finish_wgrad_plan(const Problem& p, int CoT, int CiT, int per_cu, Wg
     const int ntiles = best.tiles_n * best.tiles_h * best.tiles_w;
     int target = 256 * per_cu;  // one round of workgroups
     if (tune().wgs > 0) target = tune().wgs;
-    best.Z = std::max(1, std::min(ntiles, target / std::max(1, xy)));
+    const double slice_bytes = (double)std::max(1, best.ksets) * p.kh * p.kw * 4 * best.CoP * best.CiP * sizeof(float);
+    const double tile_flops = 2.0 * best.KP * CoT * CiT * best.kmode * std::min(best.TPW, p.kw);
+    best.Z = tune().oldplan ? std::max(1, std::min(ntiles, target / std::max(1, xy)))
+                            : reduction_slices(xy, ntiles, target, slice_bytes, tile_flops, false);
     best.partial_bytes = (size_t)best.Z * p.kh * p.kw * 4 * best.CoP * best.CiP * sizeof(float);
 }
 
-// The fp32-MFMA filter gradient in 8-product mode gives every tap a workgroup of its own (its 8 accumulator sets
-// leave no room for more), so the taps of a filter row each stage the same gradient tile; the 16-product kernel
-// shares it between three taps.  On the smallest images, where a workgroup's tiles are short, staging weighs most
-// and there are too few reduction slices to fill the CUs, that is worth more than the halved multiplications
-// (measured on fp16 tensors under the backward32 policy, 3x3: 256->256 @ 14x14 5.3 against 7.7 ms; 128->128 @
-// 28x28 the factorized kernel leads with 3.0 against 4.0 ms, as it does at 56x56 and for single-tap filters).  The
-// 8-product mode means "prefer speed" (src/backend/backend.hpp:36-66), so those problems run the 16-product
-// kernel; PHX_TUNE_WG8 keeps the factorized one.
+// The fp32-MFMA filter gradient runs in the product mode that was asked for.  In 8-product mode every tap has a
+// workgroup of its own (its 8 accumulator sets leave no room for more), so the taps of a filter row each stage the
+// same gradient tile, where the 16-product kernel shares it between three taps; with reduction slices that fill the
+// CUs (reduction_slices) and row-pair tiles of 32 positions the halved multiplications still win on the smallest
+// images (fp16 tensors under the backward32 policy, 3x3, 256 -> 256 @ 14x14: 3.2 ms factorized against 5.1 ms).
+// PHX_TUNE_OLDPLAN brings back the earlier choice (16-product kernel for rows of at most 20 positions).
 static int wgrad_f32_formulation(const Problem& p) {
-    return (p.mode == 8 && p.kw % 3 == 0 && p.wo <= 20 && !tune().wg8) ? 16 : p.mode;
+    return (p.mode == 8 && p.kw % 3 == 0 && p.wo <= 20 && !tune().wg8 && tune().oldplan) ? 16 : p.mode;
 }
 
 // fp32-MFMA kernel: 64x64 channel tiles, pixel tile and input window of at most 32 positions
@@ -810,9 +921,12 @@ static bool plan_wgrad_f32(const Problem& p, WgPlan& best) {
     const int TPW = (best.kmode == 16) ? 3 : 1;
     const int nkw = std::min(TPW, p.kw);
     double best_score = -1.0;
-    const int budget = LDS_FLOATS_MAX / (4 * 64);  // KPp + HPp (+ offsets) per staged channel
     for (int vec = 0; vec < 2; ++vec) {  // vec: windows staged as groups of 4 positions (16-byte loads)
-        for (int TW = vec ? 4 : 1; TW <= std::min(p.wo, 64); TW += vec ? 4 : 1) {
+        // KPp + HPp (+ offsets) per staged channel; the eight-wave workgroups have their CU, and its LDS, to themselves
+        const int budget = (wgrad_f32_ksets(best.kmode, vec != 0) == 2 && !tune().oldplan ? 72 * 1024 / 4 : LDS_FLOATS_MAX) / (4 * 64);
+        // (a vector tile may reach past the row end -- 16 columns for a row of 14 -- its last positions masked like
+        // those of any edge tile: one long tile per row pair instead of two short ones)
+        for (int TW = vec ? 4 : 1; TW <= std::min(vec && !tune().oldplan ? (p.wo + 3) & ~3 : p.wo, 64); TW += vec ? 4 : 1) {
             for (int TH = 1; TH <= p.ho; ++TH) {
                 for (int NB = 1; NB <= p.n; ++NB) {
                     if (NB > 1 && !(TH == p.ho && TW == p.wo)) break;
@@ -932,7 +1046,10 @@ static bool plan_wgrad_f16(const Problem& p, WgPlan& best) {
     const int per_cu = best.lds_bytes <= 80 * 1024 ? 2 : 1;
     int target = 256 * per_cu;
     if (tune().wgs > 0) target = tune().wgs;
-    best.Z = std::max(1, std::min(best.ntiles, target / std::max(1, xy)));
+    const double slice_bytes = (double)p.kh * p.kw * 4 * best.CoP * best.CiP * sizeof(float);
+    const double tile_flops = 2.0 * 64 * CoT * CiT * best.kmode * std::min(best.TPW, p.kw);  // a pixel tile: 8 chunks of 8
+    best.Z = tune().oldplan ? std::max(1, std::min(best.ntiles, target / std::max(1, xy)))
+                            : reduction_slices(xy, best.ntiles, target, slice_bytes, tile_flops, true);
     best.partial_bytes = (size_t)best.Z * p.kh * p.kw * 4 * best.CoP * best.CiP * sizeof(float);
     return true;
 }
@@ -1193,10 +1310,13 @@ static void s2d_rearrange_input(const Problem& p, const S2dView& v, const void* 
 static int do_fwd(const Problem& p, hipStream_t st, const void* x, const void* w, const void* bias, void* y, void* ws,
                   size_t wsb) {
     if (is_empty(p)) return PHX_OK;  // the reference returns silently on empty input (src/conv2d.hpp:81-82)
-    if (!x || !w || !y || (p.has_bias && !bias)) return PHX_ERR_INVALID_ARGUMENT;
+    const bool dry = g_pack.dry();
+    if (!dry && (!x || !w || !y || (p.has_bias && !bias))) return PHX_ERR_INVALID_ARGUMENT;
     const void* b = p.has_bias ? bias : nullptr;
     S2dView v;
     if (s2d_view(p, v)) {
+        // (the rearranged filter of this path is itself made per call: no prepacked form)
+        if (g_pack.mode != PackSession::OFF) return PHX_ERR_NOT_SUPPORTED;
         if (wsb < v.x2_bytes + v.w2_bytes || !ws) return PHX_ERR_WORKSPACE;
         char* x2 = static_cast<char*>(ws);
         char* w2 = x2 + v.x2_bytes;
@@ -1214,11 +1334,14 @@ static int do_fwd(const Problem& p, hipStream_t st, const void* x, const void* w
     Problem q;
     size_t xs_bytes = 0;
     if (subsample_view(p, q, xs_bytes)) {
-        if (wsb < xs_bytes || !ws) return PHX_ERR_WORKSPACE;
-        subsample_input(p, x, ws, st);
-        PHX_HIP(hipGetLastError());
+        if (!dry) {
+            if (wsb < xs_bytes || !ws) return PHX_ERR_WORKSPACE;
+            subsample_input(p, x, ws, st);
+            PHX_HIP(hipGetLastError());
+        }
         g_name_prefix = "sub_";
-        const int rc = run_corr(q, corr_forward(q), MAP_FWD, st, ws, w, b, y, static_cast<char*>(ws) + xs_bytes, wsb - xs_bytes);
+        const int rc = run_corr(q, corr_forward(q), MAP_FWD, st, ws, w, b, y, dry ? nullptr : static_cast<char*>(ws) + xs_bytes,
+                                dry ? 0 : wsb - xs_bytes);
         g_name_prefix = "";
         return rc;
     }
@@ -1228,7 +1351,8 @@ static int do_fwd(const Problem& p, hipStream_t st, const void* x, const void* w
 
 static int do_bwd_data(const Problem& p, hipStream_t st, const void* g, const void* w, void* dx, void* ws, size_t wsb) {
     if (is_empty(p)) return PHX_OK;
-    if (!g || !w || !dx) return PHX_ERR_INVALID_ARGUMENT;
+    const bool dry = g_pack.dry();
+    if (!dry && (!g || !w || !dx)) return PHX_ERR_INVALID_ARGUMENT;
     if (dgrad_by_phases(p)) {
         const size_t esize = p.dtype == PHX_F32 ? 4 : 2;
         PhaseMergeArgs m;
@@ -1242,7 +1366,8 @@ static int do_bwd_data(const Problem& p, hipStream_t st, const void* g, const vo
                 m.off[a * p.sw + b] = (long)(bufs / esize);
                 bufs += align_up((size_t)4 * p.n * p.ci * ah.size * aw.size * esize, 256);
             }
-        if (wsb < bufs || !ws) return PHX_ERR_WORKSPACE;
+        if (dry) { ws = nullptr; wsb = bufs = 0; }  // (only the packing calls of the phases matter)
+        else if (wsb < bufs || !ws) return PHX_ERR_WORKSPACE;
         char* base = static_cast<char*>(ws);
         g_name_prefix = "phase_";
         for (int a = 0; a < p.sh; ++a)
@@ -1250,10 +1375,11 @@ static int do_bwd_data(const Problem& p, hipStream_t st, const void* g, const vo
                 if (m.off[a * p.sw + b] < 0) continue;
                 const PhaseAxis ah = phase_axis(a, p.h, p.kh, p.dh, p.sh, p.pt), aw = phase_axis(b, p.w, p.kw, p.dw, p.sw, p.pl);
                 const int rc = run_corr(p, phase_corr(p, ah, aw), MAP_DGRAD, st, g, w, nullptr,
-                                        base + m.off[a * p.sw + b] * esize, base + bufs, wsb - bufs);
+                                        dry ? nullptr : base + m.off[a * p.sw + b] * esize, dry ? nullptr : base + bufs, wsb - bufs);
                 if (rc != PHX_OK) { g_name_prefix = ""; return rc; }
             }
         g_name_prefix = "";
+        if (dry) return PHX_OK;
         launch_phase_merge(p.dtype == PHX_F16, m, st);
         PHX_HIP(hipGetLastError());
         return PHX_OK;
@@ -1433,12 +1559,10 @@ size_t phx_qdense_workspace_bytes(const phx_qdense_desc* desc, int pass) {
     return workspace_for(p, pass);
 }
 
-int phx_qconv2d_fwd(const phx_qconv_desc* desc, phx_stream_t stream, const void* x, const void* w,
-                    const void* bias_or_null, void* y, void* workspace, size_t workspace_bytes) {
-    if (const int init_rc = device_state(nullptr)) return init_rc;
-    if (misaligned_workspace(workspace)) return PHX_ERR_INVALID_ARGUMENT;
-    if (desc && desc->algebra != PHX_QUATERNION)
-        return algebra_conv_pass(desc, PHX_PASS_FWD, stream, x, w, bias_or_null, y, workspace, workspace_bytes);
+// The forward pass of a quaternion convolution (also walked "dry" by the packing session, see PackSession)
+static int conv_fwd_quaternion(const phx_qconv_desc* desc, phx_stream_t stream, const void* x, const void* w,
+                               const void* bias_or_null, void* y, void* workspace, size_t workspace_bytes) {
+    const bool dry = g_pack.dry();
     Problem p;
     const int rc = problem_from_conv(desc, p);
     if (rc != PHX_OK) return rc;
@@ -1448,10 +1572,11 @@ int phx_qconv2d_fwd(const phx_qconv_desc* desc, phx_stream_t stream, const void*
     const GroupOffsets o(p);
     const ChannelsLast cl(p);
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (cl.bytes() > workspace_bytes || (cl.bytes() && !workspace)) return PHX_ERR_WORKSPACE;
+    if (dry) { workspace = nullptr; workspace_bytes = cl.bytes(); }
+    else if (cl.bytes() > workspace_bytes || (cl.bytes() && !workspace)) return PHX_ERR_WORKSPACE;
     char* ws = static_cast<char*>(workspace);
     void* y_planes = y;
-    if (p.nhwc) {
+    if (p.nhwc && !dry) {
         cl.x_in(p, x, ws, st);
         x = ws;
         y_planes = ws + cl.x_bytes;
@@ -1462,8 +1587,17 @@ int phx_qconv2d_fwd(const phx_qconv_desc* desc, phx_stream_t stream, const void*
                                ws ? ws + cl.bytes() : nullptr, workspace_bytes - cl.bytes());
         if (grc != PHX_OK) return grc;
     }
-    if (p.nhwc) cl.y_out(p, y_planes, y, st);
+    if (p.nhwc && !dry) cl.y_out(p, y_planes, y, st);
     return PHX_OK;
+}
+
+int phx_qconv2d_fwd(const phx_qconv_desc* desc, phx_stream_t stream, const void* x, const void* w,
+                    const void* bias_or_null, void* y, void* workspace, size_t workspace_bytes) {
+    if (const int init_rc = device_state(nullptr)) return init_rc;
+    if (misaligned_workspace(workspace)) return PHX_ERR_INVALID_ARGUMENT;
+    if (desc && desc->algebra != PHX_QUATERNION)
+        return algebra_conv_pass(desc, PHX_PASS_FWD, stream, x, w, bias_or_null, y, workspace, workspace_bytes);
+    return conv_fwd_quaternion(desc, stream, x, w, bias_or_null, y, workspace, workspace_bytes);
 }
 
 int phx_qconv2d_fwd_noalloc(const phx_qconv_desc* desc, phx_stream_t stream, const void* x, const void* w,
@@ -1475,12 +1609,9 @@ int phx_qconv2d_fwd_noalloc(const phx_qconv_desc* desc, phx_stream_t stream, con
     return phx_qconv2d_fwd(desc, stream, x, w, bias_or_null, y, dev->scratch_ptr, PHX_NOALLOC_SCRATCH_BYTES);
 }
 
-int phx_qconv2d_bwd_data(const phx_qconv_desc* desc, phx_stream_t stream, const void* grad, const void* w, void* dx,
-                         void* workspace, size_t workspace_bytes) {
-    if (const int init_rc = device_state(nullptr)) return init_rc;
-    if (misaligned_workspace(workspace)) return PHX_ERR_INVALID_ARGUMENT;
-    if (desc && desc->algebra != PHX_QUATERNION)
-        return algebra_conv_pass(desc, PHX_PASS_BWD_DATA, stream, grad, w, nullptr, dx, workspace, workspace_bytes);
+static int conv_bwd_data_quaternion(const phx_qconv_desc* desc, phx_stream_t stream, const void* grad, const void* w, void* dx,
+                                    void* workspace, size_t workspace_bytes) {
+    const bool dry = g_pack.dry();
     Problem p;
     const int rc = problem_from_conv(desc, p);
     if (rc != PHX_OK) return rc;
@@ -1492,10 +1623,11 @@ int phx_qconv2d_bwd_data(const phx_qconv_desc* desc, phx_stream_t stream, const 
     const GroupOffsets o(p);
     const ChannelsLast cl(p);
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (cl.bytes() > workspace_bytes || (cl.bytes() && !workspace)) return PHX_ERR_WORKSPACE;
+    if (dry) { workspace = nullptr; workspace_bytes = cl.bytes(); }
+    else if (cl.bytes() > workspace_bytes || (cl.bytes() && !workspace)) return PHX_ERR_WORKSPACE;
     char* ws = static_cast<char*>(workspace);
     void* dx_planes = dx;
-    if (p.nhwc) {
+    if (p.nhwc && !dry) {
         cl.y_in(p, grad, ws + cl.x_bytes, st);
         grad = ws + cl.x_bytes;
         dx_planes = ws;
@@ -1505,8 +1637,79 @@ int phx_qconv2d_bwd_data(const phx_qconv_desc* desc, phx_stream_t stream, const 
                                     ws ? ws + cl.bytes() : nullptr, workspace_bytes - cl.bytes());
         if (grc != PHX_OK) return grc;
     }
-    if (p.nhwc) cl.x_out(p, dx_planes, dx, st);
+    if (p.nhwc && !dry) cl.x_out(p, dx_planes, dx, st);
     return PHX_OK;
+}
+
+int phx_qconv2d_bwd_data(const phx_qconv_desc* desc, phx_stream_t stream, const void* grad, const void* w, void* dx,
+                         void* workspace, size_t workspace_bytes) {
+    if (const int init_rc = device_state(nullptr)) return init_rc;
+    if (misaligned_workspace(workspace)) return PHX_ERR_INVALID_ARGUMENT;
+    if (desc && desc->algebra != PHX_QUATERNION)
+        return algebra_conv_pass(desc, PHX_PASS_BWD_DATA, stream, grad, w, nullptr, dx, workspace, workspace_bytes);
+    return conv_bwd_data_quaternion(desc, stream, grad, w, dx, workspace, workspace_bytes);
+}
+
+// ---- filters packed ahead of the passes ----
+static bool prepack_pass_ok(int pass) { return pass == PHX_PASS_FWD || pass == PHX_PASS_BWD_DATA; }
+
+static int walk_pass(const phx_qconv_desc* desc, int pass, phx_stream_t stream, const void* in, const void* w,
+                     const void* bias, void* out, void* ws, size_t wsb) {
+    return pass == PHX_PASS_FWD ? conv_fwd_quaternion(desc, stream, in, w, bias, out, ws, wsb)
+                                : conv_bwd_data_quaternion(desc, stream, in, w, out, ws, wsb);
+}
+
+size_t phx_qconv2d_packed_filter_bytes(const phx_qconv_desc* desc, int pass) {
+    if (!desc || desc->algebra != PHX_QUATERNION || !prepack_pass_ok(pass)) return 0;
+    PackSessionScope scope(PackSession::SIZE, nullptr, 0, nullptr);
+    if (walk_pass(desc, pass, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0) != PHX_OK) return 0;
+    return g_pack.offset;
+}
+
+int phx_qconv2d_pack_filters(const phx_qconv_desc* desc, phx_stream_t stream, const void* w, void* packed_fwd,
+                             size_t packed_fwd_bytes, void* packed_bwd_data, size_t packed_bwd_data_bytes) {
+    if (const int init_rc = device_state(nullptr)) return init_rc;
+    if (!desc || desc->algebra != PHX_QUATERNION) return PHX_ERR_NOT_SUPPORTED;
+    if (!w || (!packed_fwd && !packed_bwd_data)) return PHX_ERR_INVALID_ARGUMENT;
+    if (misaligned_workspace(packed_fwd) || misaligned_workspace(packed_bwd_data)) return PHX_ERR_INVALID_ARGUMENT;
+    g_pack.jobs.n = 0;
+    void* const dst[2] = {packed_fwd, packed_bwd_data};
+    const size_t cap[2] = {packed_fwd_bytes, packed_bwd_data_bytes};
+    const int pass[2] = {PHX_PASS_FWD, PHX_PASS_BWD_DATA};
+    for (int i = 0; i < 2; ++i) {
+        if (!dst[i]) continue;
+        PackSessionScope scope(PackSession::RECORD, dst[i], cap[i], static_cast<hipStream_t>(stream));
+        const int rc = walk_pass(desc, pass[i], stream, nullptr, w, nullptr, nullptr, nullptr, 0);
+        if (rc != PHX_OK) { g_pack.jobs.n = 0; return rc; }
+        if (g_pack.offset == 0) { g_pack.jobs.n = 0; return PHX_ERR_NOT_SUPPORTED; }
+    }
+    g_pack.st = static_cast<hipStream_t>(stream);
+    const int rc = flush_pack_jobs();  // both passes' images by one launch
+    if (rc != PHX_OK) return rc;
+    PHX_HIP(hipGetLastError());
+    return PHX_OK;
+}
+
+int phx_qconv2d_fwd_prepacked(const phx_qconv_desc* desc, phx_stream_t stream, const void* x, const void* packed_fwd,
+                              size_t packed_fwd_bytes, const void* bias_or_null, void* y, void* workspace,
+                              size_t workspace_bytes) {
+    if (const int init_rc = device_state(nullptr)) return init_rc;
+    if (!desc || desc->algebra != PHX_QUATERNION) return PHX_ERR_NOT_SUPPORTED;
+    if (!packed_fwd || misaligned_workspace(workspace) || misaligned_workspace(packed_fwd)) return PHX_ERR_INVALID_ARGUMENT;
+    PackSessionScope scope(PackSession::USE, const_cast<void*>(packed_fwd), packed_fwd_bytes, static_cast<hipStream_t>(stream));
+    // (the filter argument of the walk only has to be non-null: nothing reads it)
+    return conv_fwd_quaternion(desc, stream, x, packed_fwd, bias_or_null, y, workspace, workspace_bytes);
+}
+
+int phx_qconv2d_bwd_data_prepacked(const phx_qconv_desc* desc, phx_stream_t stream, const void* grad,
+                                   const void* packed_bwd_data, size_t packed_bwd_data_bytes, void* dx, void* workspace,
+                                   size_t workspace_bytes) {
+    if (const int init_rc = device_state(nullptr)) return init_rc;
+    if (!desc || desc->algebra != PHX_QUATERNION) return PHX_ERR_NOT_SUPPORTED;
+    if (!packed_bwd_data || misaligned_workspace(workspace) || misaligned_workspace(packed_bwd_data)) return PHX_ERR_INVALID_ARGUMENT;
+    PackSessionScope scope(PackSession::USE, const_cast<void*>(packed_bwd_data), packed_bwd_data_bytes,
+                           static_cast<hipStream_t>(stream));
+    return conv_bwd_data_quaternion(desc, stream, grad, packed_bwd_data, dx, workspace, workspace_bytes);
 }
 
 int phx_qconv2d_bwd_weights(const phx_qconv_desc* desc, phx_stream_t stream, const void* x, const void* grad, void* dw,

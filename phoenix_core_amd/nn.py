@@ -8,6 +8,7 @@ the standard bottleneck stack with every channel count divided by four (quaterni
 batch-norm, ReLU, pooling and the loss are plain PyTorch (the reference has no model code).
 """
 import math
+import os
 
 import torch
 from torch import nn
@@ -29,14 +30,21 @@ def _side_stream(device):
     return s
 
 
-def _conv_backward(x, w, grad, bdesc):
+# QConv2d keeps its filter packed for the forward and input-gradient kernels (ops.PackedFilters) and packs again
+# only after the filter has changed -- once per optimizer step while training, never while serving -- instead of
+# in every forward and every backward call.
+PREPACK_FILTERS = os.environ.get("PHX_NO_PREPACK", "") in ("", "0")
+
+
+def _conv_backward(x, w, grad, bdesc, packed=None):
     if not (OVERLAP_BACKWARD and bdesc.require_input_grad):
-        return ops.conv2d_bwd(x, w, grad, bdesc)
+        dw = ops.conv2d_bwd_weights(x, grad, bdesc)
+        return dw, (ops.conv2d_bwd_data(w, grad, bdesc, packed=packed) if bdesc.require_input_grad else None)
     main, side = torch.cuda.current_stream(x.device), _side_stream(x.device)
     side.wait_stream(main)  # x and grad are complete where the side stream starts
     with torch.cuda.stream(side):
         dw = ops.conv2d_bwd_weights(x, grad, bdesc)
-    dx = ops.conv2d_bwd_data(w, grad, bdesc)
+    dx = ops.conv2d_bwd_data(w, grad, bdesc, packed=packed)
     main.wait_stream(side)  # whatever follows on the caller's stream may read dw (and free x, grad)
     dw.record_stream(main)
     return dw, dx
@@ -44,17 +52,18 @@ def _conv_backward(x, w, grad, bdesc):
 
 class _QConv2dFn(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, x, w, bias, fdesc, bdesc):
+    def forward(ctx, x, w, bias, fdesc, bdesc, packed=None):
         ctx.save_for_backward(x, w)
         ctx.bdesc = bdesc
         ctx.has_bias = bias is not None
-        return ops.conv2d_fwd(x, w, bias, fdesc)
+        ctx.packed = packed
+        return ops.conv2d_fwd(x, w, bias, fdesc, packed=packed)
 
     @staticmethod
     def backward(ctx, grad):
-        x, w = ctx.saved_tensors
+        x, w = ctx.saved_tensors  # (autograd refuses a filter modified since the forward pass: the packed images match it)
         grad = grad.contiguous()
-        dw, dx = _conv_backward(x, w, grad, ctx.bdesc)
+        dw, dx = _conv_backward(x, w, grad, ctx.bdesc, ctx.packed)
         db = None
         if ctx.has_bias:  # bias enters every output component once: plain reduction
             n = grad.shape[0] // 4
@@ -62,7 +71,7 @@ class _QConv2dFn(torch.autograd.Function):
                 db = grad.view(4, n, -1, grad.shape[3]).float().sum(dim=(1, 2)).to(grad.dtype)
             else:
                 db = grad.view(4, n, grad.shape[1], -1).float().sum(dim=(1, 3)).to(grad.dtype)
-        return dx, dw, db, None, None
+        return dx, dw, db, None, None, None
 
 
 class _QLinearFn(torch.autograd.Function):
@@ -110,6 +119,28 @@ class QConv2d(nn.Module):
         self.weight = nn.Parameter(w.to(dtype))
         self.bias = nn.Parameter(torch.zeros(4, out_channels, dtype=dtype)) if bias else None
         self._descs = {}
+        self._packed = {}  # per descriptor pair: [filter state the images were packed from, ops.PackedFilters or None]
+
+    def _packed_filters(self, key, fwd):
+        """The filter packed for this input shape, repacked (one launch, no allocation) if the filter has changed
+        since: in-place updates are seen by the tensor's version counter, replaced storage by its address."""
+        if not PREPACK_FILTERS:
+            return None
+        w = self.weight
+        state = (w._version, w.data_ptr())
+        ent = self._packed.get(key)
+        if ent is None:
+            ent = self._packed[key] = [state, ops.conv2d_pack_filters(w.detach(), fwd, bwd_data=self.input_requires_grad)]
+        elif ent[1] is not None and ent[0] != state:
+            ops.conv2d_pack_filters(w.detach(), fwd, into=ent[1])
+            ent[0] = state
+        return ent[1]
+
+    def invalidate_packed_filters(self):
+        """Forces the next forward call to pack again (for a filter changed behind the version counter's back,
+        e.g. through .data)."""
+        for ent in self._packed.values():
+            ent[0] = None
 
     def _descriptors(self, x):
         key = (tuple(x.shape), x.dtype)
@@ -124,7 +155,8 @@ class QConv2d(nn.Module):
 
     def forward(self, x):
         fwd, bwd = self._descriptors(x)
-        return _QConv2dFn.apply(x.contiguous(), self.weight, self.bias, fwd, bwd)
+        packed = self._packed_filters((tuple(x.shape), x.dtype), fwd)
+        return _QConv2dFn.apply(x.contiguous(), self.weight, self.bias, fwd, bwd, packed)
 
 
 class QLinear(nn.Module):

@@ -264,8 +264,47 @@ def _stream():
     return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
 
 
-def conv2d_fwd(x, w, bias, desc, out=None):
-    """conv2DFwd (src/upstride.hpp:18-33): y = x (x) w (+ bias)."""
+class PackedFilters:
+    """A convolution's filter in the operand order of its forward and input-gradient kernels
+    (phx_qconv2d_pack_filters): made once per filter update, read by conv2d_fwd / conv2d_bwd_data through their
+    `packed` argument instead of packing in every call.  Either image may be None (no prepacked form for that
+    pass, or not asked for)."""
+
+    def __init__(self, fwd, bwd_data, filter_shape, dtype):
+        self.fwd, self.bwd_data, self.filter_shape, self.dtype = fwd, bwd_data, tuple(filter_shape), dtype
+
+
+def conv2d_packed_filter_bytes(desc, which):
+    """Bytes of the packed filter image of a pass (0: that pass of this descriptor has no prepacked form)."""
+    if desc.algebra != QUATERNION:
+        return 0
+    return capi.lib().phx_qconv2d_packed_filter_bytes(ctypes.byref(desc.c), which)
+
+
+def conv2d_pack_filters(w, desc, bwd_data=True, into=None):
+    """Packs w for the forward pass and (bwd_data) the input gradient of desc with one kernel launch; `into`: a
+    PackedFilters of the same descriptor to overwrite (no allocation).  Returns None when neither pass has a
+    prepacked form."""
+    dev = _dev_check(w)
+    _expect(w, desc.filter_shape, desc.dtype, "filter")
+    if into is None:
+        nf = conv2d_packed_filter_bytes(desc, capi.PHX_PASS_FWD)
+        nb = conv2d_packed_filter_bytes(desc, capi.PHX_PASS_BWD_DATA) if bwd_data and not desc.real_valued_input else 0
+        if nf == 0 and nb == 0:
+            return None
+        into = PackedFilters(torch.empty(nf, dtype=torch.uint8, device=dev) if nf else None,
+                             torch.empty(nb, dtype=torch.uint8, device=dev) if nb else None, desc.filter_shape, desc.dtype)
+    elif into.filter_shape != tuple(desc.filter_shape) or into.dtype != desc.dtype:
+        raise ValueError("these packed filters belong to another descriptor")
+    f, b = into.fwd, into.bwd_data
+    capi.check(capi.lib().phx_qconv2d_pack_filters(ctypes.byref(desc.c), _stream(), _ptr(w), _ptr(f), f.numel() if f is not None else 0,
+                                                   _ptr(b), b.numel() if b is not None else 0), "phx_qconv2d_pack_filters")
+    return into
+
+
+def conv2d_fwd(x, w, bias, desc, out=None, packed=None):
+    """conv2DFwd (src/upstride.hpp:18-33): y = x (x) w (+ bias).  packed: PackedFilters of (w, desc) -- the call
+    then reads the packed image and not w."""
     dev = _dev_check(x, w, bias, out)
     _expect(x, desc.input_shape, desc.dtype, "input")
     _expect(w, desc.filter_shape, desc.dtype, "filter")
@@ -278,6 +317,13 @@ def conv2d_fwd(x, w, bias, desc, out=None):
     y = out if out is not None else torch.empty(desc.output_shape, dtype=desc.dtype, device=dev)
     nbytes = desc.workspace_bytes(capi.PHX_PASS_FWD)
     ws = _workspace.get(dev, nbytes)
+    if packed is not None and packed.fwd is not None:
+        if packed.filter_shape != tuple(desc.filter_shape) or packed.dtype != desc.dtype:
+            raise ValueError("these packed filters belong to another descriptor")
+        capi.check(capi.lib().phx_qconv2d_fwd_prepacked(ctypes.byref(desc.c), _stream(), _ptr(x), _ptr(packed.fwd),
+                                                        packed.fwd.numel(), _ptr(bias if desc.use_bias else None), _ptr(y),
+                                                        _ptr(ws), nbytes), "phx_qconv2d_fwd_prepacked")
+        return y
     capi.check(capi.lib().phx_qconv2d_fwd(ctypes.byref(desc.c), _stream(), _ptr(x), _ptr(w),
                                           _ptr(bias if desc.use_bias else None), _ptr(y), _ptr(ws), nbytes),
                "phx_qconv2d_fwd")
@@ -297,8 +343,8 @@ def conv2d_bwd_weights(x, grad, desc):
     return dw
 
 
-def conv2d_bwd_data(w, grad, desc):
-    """The input-gradient half of conv2DBwd: dx (the descriptor must ask for it)."""
+def conv2d_bwd_data(w, grad, desc, packed=None):
+    """The input-gradient half of conv2DBwd: dx (the descriptor must ask for it).  packed: as in conv2d_fwd."""
     dev = _dev_check(w, grad)
     _expect(w, desc.filter_shape, desc.dtype, "filter")
     _expect(grad, desc.output_shape, desc.dtype, "output gradient")
@@ -307,6 +353,13 @@ def conv2d_bwd_data(w, grad, desc):
     dx = torch.empty(desc.input_shape, dtype=desc.dtype, device=dev)
     nbytes = desc.workspace_bytes(capi.PHX_PASS_BWD_DATA)
     ws = _workspace.get(dev, nbytes)
+    if packed is not None and packed.bwd_data is not None:
+        if packed.filter_shape != tuple(desc.filter_shape) or packed.dtype != desc.dtype:
+            raise ValueError("these packed filters belong to another descriptor")
+        capi.check(capi.lib().phx_qconv2d_bwd_data_prepacked(ctypes.byref(desc.c), _stream(), _ptr(grad), _ptr(packed.bwd_data),
+                                                             packed.bwd_data.numel(), _ptr(dx), _ptr(ws), nbytes),
+                   "phx_qconv2d_bwd_data_prepacked")
+        return dx
     capi.check(capi.lib().phx_qconv2d_bwd_data(ctypes.byref(desc.c), _stream(), _ptr(grad), _ptr(w), _ptr(dx),
                                                _ptr(ws), nbytes), "phx_qconv2d_bwd_data")
     return dx

@@ -45,6 +45,27 @@ def test_status_strings_and_descriptor_validation():
         assert capi.lib().phx_qconv2d_workspace_bytes(ctypes.byref(good), which) > 0
 
 
+def test_packed_filter_sizes_need_no_gpu():
+    """phx_qconv2d_packed_filter_bytes only plans: an image no larger than the pass's workspace where the pass has
+    a prepacked form, 0 where it has none."""
+    L = capi.lib()
+    # fp16 full16, 3x3 on 32 -> 64 channels at 14x14, factorized mode
+    d = capi.QConvDesc(capi.PHX_F16, 2, 32, 64, 14, 14, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 0, 8, capi.PHX_FP16_FULL16, 0, 0, 1, 0, 0)
+    for which in (capi.PHX_PASS_FWD, capi.PHX_PASS_BWD_DATA):
+        n = L.phx_qconv2d_packed_filter_bytes(ctypes.byref(d), which)
+        assert 0 < n <= L.phx_qconv2d_workspace_bytes(ctypes.byref(d), which) and n % 256 == 0
+    assert L.phx_qconv2d_packed_filter_bytes(ctypes.byref(d), capi.PHX_PASS_BWD_WEIGHTS) == 0
+    # stride 2 on 3 input channels: the forward pass rearranges the filter per call (space-to-depth)
+    s2d = capi.QConvDesc(capi.PHX_F16, 2, 3, 16, 32, 32, 7, 7, 2, 2, 1, 1, 3, 3, 3, 3, 0, 8, capi.PHX_FP16_FULL16, 0, 0, 1, 0, 0)
+    assert L.phx_qconv2d_packed_filter_bytes(ctypes.byref(s2d), capi.PHX_PASS_FWD) == 0
+    assert L.phx_qconv2d_packed_filter_bytes(ctypes.byref(s2d), capi.PHX_PASS_BWD_DATA) > 0
+    # strided 3x3 (its input gradient runs as several phases with a sub-filter each, or with zero insertion)
+    s2 = capi.QConvDesc(capi.PHX_F16, 2, 32, 32, 14, 14, 3, 3, 2, 2, 1, 1, 1, 1, 1, 1, 0, 8, capi.PHX_FP16_FULL16, 0, 0, 1, 0, 0)
+    assert L.phx_qconv2d_packed_filter_bytes(ctypes.byref(s2), capi.PHX_PASS_BWD_DATA) > 0
+    bad = capi.QConvDesc(0, 1, 0, 4, 8, 8, 3, 3, 1, 1, 1, 1, 0, 0, 0, 0, 0, 8, 0, 0)
+    assert L.phx_qconv2d_packed_filter_bytes(ctypes.byref(bad), 0) == 0
+
+
 def test_python_descriptor_matches_oracle_padding():
     import oracle
     import torch

@@ -76,6 +76,61 @@ def test_overlapped_backward_equals_the_sequential_one():
             assert torch.equal(ta, tb)
 
 
+def test_layers_repack_their_filters_when_and_only_when_they_change():
+    """QConv2d keeps packed filters (nn.PREPACK_FILTERS): a training loop with in-place filter updates between the
+    steps must give, bit for bit, what the layers give when every call packs for itself; and a step without an
+    update must not pack at all."""
+    from phoenix_core_amd import nn as qnn, ops
+    ctx = Ctx(8, "full16")
+    xs = [torch.randn(8, 16, 20, 20, device="cuda", generator=torch.Generator("cuda").manual_seed(5 + i)).half() for i in range(3)]
+
+    def run(prepack):
+        old, qnn.PREPACK_FILTERS = qnn.PREPACK_FILTERS, prepack
+        torch.manual_seed(4)
+        layers = torch.nn.ModuleList([phx.QConv2d(16, 32, 3, dtype=torch.float16, context=ctx), phx.QConv2d(32, 32, 1, dtype=torch.float16, context=ctx),
+                                      phx.QConv2d(32, 16, 3, stride=2, dtype=torch.float16, context=ctx)]).cuda()
+        try:
+            out = []
+            for x0 in xs:
+                for m in layers:
+                    m.weight.grad = None
+                x = x0.clone().requires_grad_(True)
+                y = x
+                for m in layers:
+                    y = m(y)
+                y.float().square().mean().backward()
+                out.append([y.detach().clone(), x.grad.clone()] + [m.weight.grad.clone() for m in layers])
+                with torch.no_grad():
+                    for m in layers:
+                        m.weight.add_(m.weight.grad, alpha=-0.01)  # in place: bumps the version counter
+            torch.cuda.synchronize()
+            return out, layers
+        finally:
+            qnn.PREPACK_FILTERS = old
+
+    want, _ = run(False)
+    got, layers = run(True)
+    for a, b in zip(want, got):
+        for ta, tb in zip(a, b):
+            assert torch.equal(ta, tb)
+    # unchanged filters: no packing call at all; a change behind the counter's back needs invalidate_packed_filters()
+    calls = []
+    real_pack = ops.conv2d_pack_filters
+    ops.conv2d_pack_filters = lambda *a, **k: (calls.append(1), real_pack(*a, **k))[1]
+    try:
+        with torch.no_grad():
+            y1 = layers[0](xs[0])
+            assert len(calls) == 1  # (the update after the last step)
+            y2 = layers[0](xs[0])
+            assert len(calls) == 1 and torch.equal(y1, y2)
+            layers[0].weight.data.mul_(2.0)
+            layers[0].invalidate_packed_filters()
+            y3 = layers[0](xs[0])
+            assert len(calls) == 2 and not torch.equal(y3, y1)
+    finally:
+        ops.conv2d_pack_filters = real_pack
+
+
 def test_qconv2d_groups_and_channels_last():
     """QConv2d(groups=G) is G ungrouped layers on channel slices; QConv2d(data_format="NHWC") is the NCHW layer on
     permuted activations: outputs and all gradients must agree with those compositions."""

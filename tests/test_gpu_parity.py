@@ -11,7 +11,7 @@ import torch
 
 import oracle
 import phoenix_core_amd as phx
-from phoenix_core_amd import capi
+from phoenix_core_amd import capi, ops
 
 pytestmark = pytest.mark.gpu
 
@@ -730,3 +730,92 @@ def test_flat_chunk_list_of_the_filter_gradient(case, real_input, tune_env):
     # the same products, summed over differently cut chunks: equal up to fp32 summation order
     scale = got["rows"].abs().max().item()
     assert (got["planes"] - got["rows"]).abs().max().item() <= 2e-3 * scale
+
+
+# ---- filters packed ahead of the passes (phx_qconv2d_pack_filters and the *_prepacked entry points) ----
+S2D_FORWARD = ("k7_s2", "k3_s2_c4", "k5_s2_valid")  # at most 4 input channels, stride 2: the filter is rearranged per call
+
+
+@pytest.mark.parametrize("dtype,policy", [(torch.float32, "fp32"), (torch.float16, "full16"), (torch.float16, "backward32")],
+                         ids=["f32", "f16_full16", "f16_backward32"])
+@pytest.mark.parametrize("mode", [16, 8])
+@pytest.mark.parametrize("case", CONV_CASES, ids=[c[0] for c in CONV_CASES])
+def test_prepacked_filters_give_the_plain_result(case, mode, dtype, policy):
+    """The prepacked entry points run the kernels of the plain ones on images made by one combined packing
+    launch: results must be identical bit for bit (the plain ones are held against the oracle above)."""
+    name, n, ci, co, h, w, kh, kw, stride, dilation, padding = case
+    scale = 1.0 if dtype == torch.float32 else 0.5
+    g, x, wt, b, gr = make_inputs(name_seed(name) + 21, n, ci, co, h, w, kh, kw, stride, dilation, padding, dtype, scale)
+    desc = phx.Conv2DDescriptor(x.shape, wt.shape, stride, dilation, padding, use_bias=True, dtype=dtype, context=Ctx(mode, policy))
+    xd, wd, bd, gd = (torch.from_numpy(a).cuda() for a in (x, wt, b, gr))
+    y = phx.conv2d_fwd(xd, wd, bd, desc)
+    fwd_kernel = capi.last_kernel_name()
+    dx = ops.conv2d_bwd_data(wd, gd, desc)
+    packed = ops.conv2d_pack_filters(wd, desc)
+    assert packed is not None and packed.bwd_data is not None
+    assert (packed.fwd is None) == (name in S2D_FORWARD), fwd_kernel
+    wd.zero_()  # the prepacked calls must not read the filter itself
+    y2 = phx.conv2d_fwd(xd, wd, bd, desc, packed=packed)
+    if packed.fwd is not None:
+        assert capi.last_kernel_name() == fwd_kernel
+        assert torch.equal(y2, y), "prepacked fwd " + name
+    dx2 = ops.conv2d_bwd_data(wd, gd, desc, packed=packed)
+    assert torch.equal(dx2, dx), "prepacked dgrad " + name
+    # packing again into the same buffers after the filter has changed
+    wd.copy_(torch.from_numpy(wt).cuda() * 0.5)
+    assert ops.conv2d_pack_filters(wd, desc, into=packed) is packed
+    want = ops.conv2d_bwd_data(wd, gd, desc)
+    assert torch.equal(ops.conv2d_bwd_data(wd, gd, desc, packed=packed), want), "repacked dgrad " + name
+
+
+@pytest.mark.parametrize("mode", [16, 8])
+@pytest.mark.parametrize("case", [c for c in GROUPED if c[0] in ("g2_k3", "g4_pw", "g3_k3_s2", "depthwise_k3")] +
+                         [c[:1] + (1,) + c[4:] for c in CHANNELS_LAST if c[0] in ("nhwc_pw", "nhwc_k3", "nhwc_pw_c40_24")],
+                         ids=lambda c: c[0])
+def test_prepacked_filters_grouped_and_channels_last(case, mode):
+    """Groups (one packing job per group and pass -- more jobs than one launch holds for the depthwise case) and
+    channels-last activations, fp16."""
+    name, G, n, ci, co, h, w, kh, kw, stride, dilation, padding = case
+    nhwc = name.startswith("nhwc")
+    dtype = torch.float16
+    r = np.random.default_rng(name_seed(name) + 22)
+    geom = oracle.make_geom(n, ci // G, co // G, h, w, kh, kw, stride, dilation, padding)
+    xs = (4 * n, h, w, ci) if nhwc else (4 * n, ci, h, w)
+    gs = (4 * n, geom.ho, geom.wo, co) if nhwc else (4 * n, co, geom.ho, geom.wo)
+    xd = torch.from_numpy((0.5 * r.standard_normal(xs)).astype(np.float16)).cuda()
+    gd = torch.from_numpy((0.5 * r.standard_normal(gs)).astype(np.float16)).cuda()
+    wd = torch.from_numpy((0.2 * r.standard_normal((4, co, ci // G, kh, kw))).astype(np.float16)).cuda()
+    desc = phx.Conv2DDescriptor(xs, wd.shape, stride, dilation, padding, groups=G, dtype=dtype, context=Ctx(mode, "full16"),
+                                data_format="NHWC" if nhwc else "NCHW")
+    y = phx.conv2d_fwd(xd, wd, None, desc)
+    dx = ops.conv2d_bwd_data(wd, gd, desc)
+    packed = ops.conv2d_pack_filters(wd, desc)
+    assert packed is not None and packed.fwd is not None and packed.bwd_data is not None
+    wd.zero_()
+    assert torch.equal(phx.conv2d_fwd(xd, wd, None, desc, packed=packed), y), "prepacked fwd " + name
+    assert torch.equal(ops.conv2d_bwd_data(wd, gd, desc, packed=packed), dx), "prepacked dgrad " + name
+
+
+def test_prepacked_filters_are_refused_where_they_do_not_apply():
+    wd = torch.zeros(4, 8, 8, 3, 3, device="cuda")
+    desc = phx.Conv2DDescriptor((8, 8, 6, 6), wd.shape, 1, 1, "SAME", context=Ctx(8))
+    packed = ops.conv2d_pack_filters(wd, desc)
+    other = phx.Conv2DDescriptor((8, 8, 6, 6), (4, 8, 8, 1, 1), 1, 1, "SAME", context=Ctx(8))
+    with pytest.raises(ValueError):
+        phx.conv2d_fwd(torch.zeros(8, 8, 6, 6, device="cuda"), torch.zeros(4, 8, 8, 1, 1, device="cuda"), None, other, packed=packed)
+    # an image smaller than the descriptor needs
+    L = capi.lib()
+    x = torch.zeros(8, 8, 6, 6, device="cuda")
+    y = torch.empty(desc.output_shape, device="cuda")
+    nbytes = desc.workspace_bytes(capi.PHX_PASS_FWD)
+    ws = ops.reserve_workspace(nbytes)
+    rc = L.phx_qconv2d_fwd_prepacked(ctypes.byref(desc.c), None, x.data_ptr(), packed.fwd.data_ptr(), packed.fwd.numel() - 256, None,
+                                     y.data_ptr(), ws.data_ptr(), nbytes)
+    assert rc == capi.PHX_ERR_WORKSPACE
+    rc = L.phx_qconv2d_pack_filters(ctypes.byref(desc.c), None, wd.data_ptr(), packed.fwd.data_ptr(), packed.fwd.numel() - 256, None, 0)
+    assert rc == capi.PHX_ERR_WORKSPACE
+    # empty input: nothing to pack
+    empty = phx.Conv2DDescriptor((0, 8, 6, 6), wd.shape, 1, 1, "SAME", context=Ctx(8))
+    assert ops.conv2d_packed_filter_bytes(empty, capi.PHX_PASS_FWD) == 0
+    assert ops.conv2d_pack_filters(wd, empty) is None
+    torch.cuda.synchronize()
