@@ -866,18 +866,20 @@ struct WgPlan {
     size_t lds_bytes, partial_bytes;
 };
 
-// Reduction slices of a filter gradient.  xy workgroups share a slice (channel tiles x tap groups), a slice walks
+// Reduction slices of a filter gradient on the fp32 matrix cores.  xy workgroups share a slice (channel tiles x tap groups), a slice walks
 // ceil(ntiles / Z) pixel tiles, `slots` workgroups run at a time.  With few workgroups per slice one round of
 // workgroups is best (Z = slots / xy: small partial sums, no straggler round) and is kept wherever it fills four
 // fifths of the slots; where xy alone is a good part of a round (large channel counts: 256 -> 256, 3x3, one tap per
 // workgroup = 144) it leaves CUs idle, and several rounds of shorter workgroups fill them.  The cost below is in units of one pixel tile of one workgroup: rounds x
 // (tiles per workgroup + one tile's worth of start-up and epilogue) + slices x the time to write and read back a
-// slice of partial sums (slice_bytes twice at 5 TB/s, against tile_flops at the rate one CU sustains).
-static int reduction_slices(int xy, int ntiles, int slots, double slice_bytes, double tile_flops, bool f16mfma) {
+// slice of partial sums (slice_bytes twice at 5 TB/s, against tile_flops at the 0.45 TFLOP/s one CU sustains).
+// (The fp16 kernels keep the one-round rule: two of their workgroups share a CU, which this count of rounds does
+// not describe -- tried there, it cost the small layers of a ResNet 10-35 %.)
+static int reduction_slices(int xy, int ntiles, int slots, double slice_bytes, double tile_flops) {
     xy = std::max(1, xy);
     const int one_round = std::max(1, std::min(ntiles, slots / xy));
     if ((double)xy * one_round >= 0.8 * slots) return one_round;
-    const double tile_seconds = tile_flops / (f16mfma ? 4.5e12 : 0.45e12);
+    const double tile_seconds = tile_flops / 0.45e12;
     const double slice_cost = (2.0 * slice_bytes / 5e12) / tile_seconds;
     const int zmax = std::max(1, std::min(ntiles, std::max(slots / xy, 32)));
     int best_z = 1;
@@ -901,7 +903,7 @@ static void finish_wgrad_plan(const Problem& p, int CoT, int CiT, int per_cu, Wg
     const double slice_bytes = (double)std::max(1, best.ksets) * p.kh * p.kw * 4 * best.CoP * best.CiP * sizeof(float);
     const double tile_flops = 2.0 * best.KP * CoT * CiT * best.kmode * std::min(best.TPW, p.kw);
     best.Z = tune().oldplan ? std::max(1, std::min(ntiles, target / std::max(1, xy)))
-                            : reduction_slices(xy, ntiles, target, slice_bytes, tile_flops, false);
+                            : reduction_slices(xy, ntiles, target, slice_bytes, tile_flops);
     best.partial_bytes = (size_t)best.Z * p.kh * p.kw * 4 * best.CoP * best.CiP * sizeof(float);
 }
 
@@ -1046,10 +1048,7 @@ static bool plan_wgrad_f16(const Problem& p, WgPlan& best) {
     const int per_cu = best.lds_bytes <= 80 * 1024 ? 2 : 1;
     int target = 256 * per_cu;
     if (tune().wgs > 0) target = tune().wgs;
-    const double slice_bytes = (double)p.kh * p.kw * 4 * best.CoP * best.CiP * sizeof(float);
-    const double tile_flops = 2.0 * 64 * CoT * CiT * best.kmode * std::min(best.TPW, p.kw);  // a pixel tile: 8 chunks of 8
-    best.Z = tune().oldplan ? std::max(1, std::min(best.ntiles, target / std::max(1, xy)))
-                            : reduction_slices(xy, best.ntiles, target, slice_bytes, tile_flops, true);
+    best.Z = std::max(1, std::min(best.ntiles, target / std::max(1, xy)));
     best.partial_bytes = (size_t)best.Z * p.kh * p.kw * 4 * best.CoP * best.CiP * sizeof(float);
     return true;
 }
