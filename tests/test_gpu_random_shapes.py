@@ -9,6 +9,7 @@ import torch
 
 import oracle
 import phoenix_core_amd as phx
+from phoenix_core_amd import ops
 
 pytestmark = pytest.mark.gpu
 
@@ -91,6 +92,12 @@ def run_case(cfg, r, dtype, policy):
     xd, wd, bd, gd = (torch.from_numpy(a).cuda() for a in (x_dev, w_dev, b, g_dev))
     y = phx.conv2d_fwd(xd, wd, bd if bias else None, desc)
     dw, dx = phx.conv2d_bwd(xd, wd, gd, desc)
+    # the same passes on filters packed ahead of them (one packing launch for both images): bit-identical
+    packed = ops.conv2d_pack_filters(wd, desc, bwd_data=not real)
+    if packed is not None and packed.fwd is not None:
+        assert torch.equal(phx.conv2d_fwd(xd, wd, bd if bias else None, desc, packed=packed), y), "prepacked fwd %s" % cfg
+    if packed is not None and packed.bwd_data is not None:
+        assert torch.equal(ops.conv2d_bwd_data(wd, gd, desc, packed=packed), dx), "prepacked dgrad %s" % cfg
     torch.cuda.synchronize()
     x64, w64, b64, g64 = (a.astype(np.float64) for a in (x, wt, b, gr))
     # by definition G independent convolutions on channel slices
