@@ -514,10 +514,10 @@ def run_resnet(mode, policy, args):
     out = {
         "workload": "%s: quaternion ResNet-50 forward+backward (no optimizer step, as the metric names), "
                     "N=%d real images (4N=%d quaternion rows after the real-input stem), 224x224, 53 quaternion convs + "
-                    "quaternion dense head; batch-norm (with the ReLU behind it) by %s, residual add, "
-                    "pooling and cross-entropy by PyTorch; the step %s"
-                    % (RESNET, n, 4 * n, "torch.nn.BatchNorm2d (MIOpen)" if args.torch_bn else
-                       "the library's streaming kernels (include/phx_bn.h)",
+                    "quaternion dense head; batch-norm (with the ReLU behind it) and the stem's max-pool by %s, residual add, "
+                    "average pool and cross-entropy by PyTorch; the step %s"
+                    % (RESNET, n, 4 * n, "torch.nn.BatchNorm2d (MIOpen) and torch.nn.MaxPool2d" if args.torch_bn else
+                       "the library's streaming kernels (include/phx_bn.h, include/phx_pool.h)",
                        "is captured once into a HIP graph and replayed" if graph["used"] else "runs eagerly"),
         "product_mode": mode, "fp16_policy": policy, "batch_norm": "torch" if args.torch_bn else "library", "dtype": "f16",
         "filters": "frozen (packed once, before the timed steps)" if args.frozen_filters else

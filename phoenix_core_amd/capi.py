@@ -39,6 +39,10 @@ EXPORTS = (
 EXPORTS_BN = ("phx_bn_workspace_bytes", "phx_bn_fwd_train", "phx_bn_bwd")
 
 
+# every symbol include/phx_pool.h declares (max pooling for the same harness)
+EXPORTS_POOL = ("phx_maxpool3x3s2_fwd", "phx_maxpool3x3s2_bwd")
+
+
 class BnDesc(ctypes.Structure):
     _fields_ = [("dtype", ctypes.c_int32), ("rows", ctypes.c_int32), ("c", ctypes.c_int32), ("hw", ctypes.c_int32),
                 ("eps", ctypes.c_float), ("momentum", ctypes.c_float), ("relu", ctypes.c_int32)]
@@ -99,6 +103,8 @@ def lib():
         L.phx_bn_workspace_bytes.argtypes = [bd]
         L.phx_bn_fwd_train.argtypes = [bd, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, sz]
         L.phx_bn_bwd.argtypes = [bd, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, sz]
+        L.phx_maxpool3x3s2_fwd.argtypes = [ctypes.c_int32, ctypes.c_int64, ctypes.c_int32, ctypes.c_int32, vp, vp, vp, vp]
+        L.phx_maxpool3x3s2_bwd.argtypes = [ctypes.c_int32, ctypes.c_int64, ctypes.c_int32, ctypes.c_int32, vp, vp, vp, vp]
         L.phx_device_count.argtypes = [i32p]
         L.phx_device_malloc.argtypes = [ctypes.POINTER(vp), sz]
         L.phx_device_free.argtypes = [vp]

@@ -5,7 +5,8 @@ with gradients; this module plays that role for PyTorch.  QConv2d / QLinear hold
 tensor layouts (components stacked on the batch axis, filters [4, Co, Ci, Kh, Kw], dense filters
 [4, I, O]); every forward / backward call goes through the HIP library.  The ResNet-50 below is
 the standard bottleneck stack with every channel count divided by four (quaternion channels);
-batch-norm, ReLU, pooling and the loss are plain PyTorch (the reference has no model code).
+batch-norm with its ReLU and the stem's max-pool run on the library's streaming kernels (include/phx_bn.h,
+include/phx_pool.h) or on torch's modules; the loss is plain PyTorch (the reference has no model code).
 """
 import math
 import os
@@ -226,6 +227,28 @@ class QBatchNorm2d(nn.Module):
         return torch.relu(y) if self.relu else y
 
 
+class _QMaxPoolFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x):
+        y, index = ops.max_pool_3x3s2_fwd(x)
+        ctx.save_for_backward(index)
+        ctx.input_shape = tuple(x.shape)
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        (index,) = ctx.saved_tensors
+        return ops.max_pool_3x3s2_bwd(dy.contiguous(), index, ctx.input_shape)
+
+
+class QMaxPool3x3s2(nn.Module):
+    """torch.nn.MaxPool2d(3, 2, 1) on the library's streaming kernels (include/phx_pool.h): same outputs and
+    gradients, one byte of index per output element instead of eight."""
+
+    def forward(self, x):
+        return _QMaxPoolFn.apply(x.contiguous())
+
+
 class _Bottleneck(nn.Module):
     def __init__(self, cin, width, cout, stride, dtype, context, fused_bn):
         super().__init__()
@@ -268,7 +291,7 @@ class QResNet50(nn.Module):
         self.fused_bn = fused_bn
         self.bn = QBatchNorm2d(16, relu=True) if fused_bn else nn.BatchNorm2d(16)
         self.relu = nn.ReLU(inplace=True)
-        self.pool = nn.MaxPool2d(3, 2, 1)
+        self.pool = QMaxPool3x3s2() if fused_bn else nn.MaxPool2d(3, 2, 1)
         blocks, cin = [], 16
         for width, cout, count, stride in ((16, 64, 3, 1), (32, 128, 4, 2), (64, 256, 6, 2), (128, 512, 3, 2)):
             for i in range(count):

@@ -464,3 +464,33 @@ def batch_norm_bwd(x, dy, gamma, beta, mean, invstd, eps, relu, residual=None):
                                      _ptr(beta), _ptr(mean), _ptr(invstd), _ptr(dx), _ptr(dres), _ptr(dgamma), _ptr(dbeta),
                                      _ptr(ws), nbytes), "phx_bn_bwd")
     return dx, dgamma, dbeta, dres
+
+
+def max_pool_3x3s2_fwd(x):
+    """3x3 max pooling, stride 2, padding 1, of x [rows, C, H, W] (include/phx_pool.h): returns (y, index) with
+    index [rows, C, Ho, Wo] uint8 = the window position 0..8 that held the maximum (max_pool_3x3s2_bwd reads it)."""
+    dev = _dev_check(x)
+    if x.dtype not in _DTYPES or x.dim() != 4:
+        raise ValueError("max pooling takes a float32 or float16 tensor [rows, C, H, W]")
+    rows, c, h, w = x.shape
+    ho, wo = ((h - 1) // 2 + 1, (w - 1) // 2 + 1) if h and w else (0, 0)
+    y = torch.empty((rows, c, ho, wo), dtype=x.dtype, device=dev)
+    index = torch.empty((rows, c, ho, wo), dtype=torch.uint8, device=dev)
+    capi.check(capi.lib().phx_maxpool3x3s2_fwd(_DTYPES[x.dtype], rows * c, h, w, _stream(), _ptr(x), _ptr(y), _ptr(index)),
+               "phx_maxpool3x3s2_fwd")
+    return y, index
+
+
+def max_pool_3x3s2_bwd(dy, index, input_shape):
+    """Gradient of max_pool_3x3s2_fwd with respect to its input of shape input_shape."""
+    dev = _dev_check(dy, index)
+    rows, c, h, w = input_shape
+    ho, wo = ((h - 1) // 2 + 1, (w - 1) // 2 + 1) if h and w else (0, 0)
+    if dy.dtype not in _DTYPES:
+        raise ValueError("max pooling takes float32 or float16 gradients")
+    _expect(dy, (rows, c, ho, wo), dy.dtype, "output gradient")
+    _expect(index, (rows, c, ho, wo), torch.uint8, "index")
+    dx = torch.empty(tuple(input_shape), dtype=dy.dtype, device=dev)
+    capi.check(capi.lib().phx_maxpool3x3s2_bwd(_DTYPES[dy.dtype], rows * c, h, w, _stream(), _ptr(dy), _ptr(index), _ptr(dx)),
+               "phx_maxpool3x3s2_bwd")
+    return dx

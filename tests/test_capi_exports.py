@@ -31,6 +31,17 @@ def test_batch_norm_header_symbols_are_exported():
     assert lib.phx_bn_workspace_bytes(ctypes.byref(capi.BnDesc(7, 1, 1, 1, 1e-5, 0.1, 0))) == 0
 
 
+def test_pool_header_symbols_are_exported():
+    lib = capi.lib()
+    header = open(os.path.join(ROOT, "include", "phx_pool.h")).read()
+    declared = set(re.findall(r"\b(phx_maxpool[a-z0-9_]+)\s*\(", header))
+    assert declared == set(capi.EXPORTS_POOL)
+    assert all(hasattr(lib, s) for s in declared)
+    # argument checks need no GPU: an unknown dtype is refused, an empty tensor is a no-op
+    assert lib.phx_maxpool3x3s2_fwd(7, 1, 4, 4, None, None, None, None) == capi.PHX_ERR_INVALID_ARGUMENT
+    assert lib.phx_maxpool3x3s2_bwd(capi.PHX_F16, 0, 4, 4, None, None, None, None) == capi.PHX_OK
+
+
 def test_status_strings_and_descriptor_validation():
     assert capi.status_string(0) == "ok"
     assert "workspace" in capi.status_string(3)

@@ -228,7 +228,7 @@ def _cpu_forward(model, xq, storage=None):
         t.load_state_dict({k: v.detach().cpu().float() for k, v in m.state_dict().items() if k != "num_batches_tracked"},
                           strict=False)
         return t.train()
-    y = model.pool(rnd(model.relu(bn(model.bn)(conv(model.stem, xq)))))
+    y = torch.nn.functional.max_pool2d(rnd(model.relu(bn(model.bn)(conv(model.stem, xq)))), 3, 2, 1)
     for b in model.blocks:
         idt = y if b.down is None else rnd(bn(b.down[1])(conv(b.down[0], y)))
         z = rnd(torch.relu(bn(b.bn1)(conv(b.conv1, y))))
