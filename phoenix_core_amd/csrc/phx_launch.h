@@ -85,6 +85,18 @@ int launch_wgrad_f16_realx(const RealWgArgs& a, int nblocks, size_t lds_bytes, h
 int launch_wgrad_f16_p8(int MT, int NT, int SW, const WgradArgs& a, int nblocks, size_t lds_bytes, hipStream_t st);
 int launch_reduce_wgrad(bool half_storage, const ReduceArgs& a, hipStream_t st);
 
+// Dense on fp32 FMA threads for small problems (phx_launch_dense_small.hip); (a, b) = (x, w) forward, (grad, w) input
+// gradient, (x, grad) filter gradient; filter element (r, i, o) at r * wcs + o * so + i * si
+struct DenseSmallArgs {
+    const void* a;
+    const void* b;
+    const void* bias;  // forward only, or null
+    void* out;
+    long wcs, so, si;
+    int n, ni, no;
+};
+int launch_dense_small(bool half_storage, int pass, const DenseSmallArgs& a, hipStream_t st);
+
 // space-to-depth rearrangements (stride-2 convolutions with very few input channels)
 int launch_s2d_input(bool half_storage, const S2dArgs& a, hipStream_t st);
 int launch_subsample(bool half_storage, const SubsampleArgs& a, hipStream_t st);

@@ -30,6 +30,7 @@ struct Tuning {
     int tile_wco = 0, tile_ntw = 0;   // PHX_TUNE_TILE="wco,ntw"
     bool flat = false, noflat = false, nopw = false, pw8 = false, zi8 = false, wg8 = false, nos2d = false, noearly = false, norealx = false, nosub = false, oldplan = false;
     bool nopwx = false;               // PHX_TUNE_NOPWX: pointwise fp16 problems stay on the staged-window kernels
+    bool nosmalldense = false;        // PHX_TUNE_NOSMALLDENSE: small Dense problems stay on the matrix-core kernels
     int vec = 0;                      // PHX_TUNE_VEC (0 = unset)
     int wgs = 0;                      // PHX_TUNE_WGS (0 = unset)
     int wg_mt = 0, wg_nt = 0;         // PHX_TUNE_WG="mt,nt"
@@ -50,6 +51,7 @@ struct Tuning {
         nosub = getenv("PHX_TUNE_NOSUB") != nullptr;
         oldplan = getenv("PHX_TUNE_OLDPLAN") != nullptr;
         nopwx = getenv("PHX_TUNE_NOPWX") != nullptr;
+        nosmalldense = getenv("PHX_TUNE_NOSMALLDENSE") != nullptr;
         if (const char* e = getenv("PHX_TUNE_VEC")) vec = atoi(e);
         if (const char* e = getenv("PHX_TUNE_WGS")) wgs = atoi(e);
         if (const char* e = getenv("PHX_TUNE_WG")) sscanf(e, "%d,%d", &wg_mt, &wg_nt);
@@ -1551,10 +1553,36 @@ size_t phx_qconv2d_workspace_bytes(const phx_qconv_desc* desc, int pass) {
     return ChannelsLast(p).bytes() + workspace_for(p, pass);
 }
 
+// Small Dense problems (a classifier head, the reference's 128 -> 128 benchmark layer at batch 32) run on plain fp32
+// FMA threads: no packing, no workspace, one launch per pass (phx_launch_dense_small.hip).  Up to 16 M quaternion
+// products per pass; beyond that the matrix cores win.
+static bool dense_is_small(const Problem& p) {
+    return !tune().nosmalldense && (double)p.n * p.ci * p.co <= 16.0 * 1024 * 1024 && (long)p.n * std::max(p.ci, p.co) < (1L << 30) &&
+           (long)p.ci * p.co < (1L << 30);
+}
+
+static int run_dense_small(const Problem& p, int pass, hipStream_t st, const void* a, const void* b, const void* bias, void* out) {
+    if (!out || (p.n > 0 && (!a || !b)) || (pass == PHX_PASS_FWD && p.has_bias && !bias)) return PHX_ERR_INVALID_ARGUMENT;
+    DenseSmallArgs d{a, b, (pass == PHX_PASS_FWD && p.has_bias) ? bias : nullptr, out, p.fs.wcs, p.fs.so, p.fs.si, p.n, p.ci, p.co};
+    int rc;
+    {
+        KernelTimer timer(st);
+        rc = launch_dense_small(p.dtype == PHX_F16, pass, d, st);
+    }
+    if (rc != 0) return PHX_ERR_NOT_SUPPORTED;
+    PHX_HIP(hipGetLastError());
+    snprintf(g_name_buf, sizeof(g_name_buf), "qdense_%s_fma_%s_n%d_i%d_o%d",
+             pass == PHX_PASS_FWD ? "fwd" : pass == PHX_PASS_BWD_DATA ? "dgrad" : "wgrad", p.dtype == PHX_F32 ? "f32" : "f16", p.n, p.ci, p.co);
+    g_last_kernel = g_name_buf;
+    say(p, pass == PHX_PASS_FWD ? "forward (dense)" : pass == PHX_PASS_BWD_DATA ? "input gradient (dense)" : "filter gradient (dense)");
+    return PHX_OK;
+}
+
 size_t phx_qdense_workspace_bytes(const phx_qdense_desc* desc, int pass) {
     if (desc && desc->algebra != PHX_QUATERNION) return algebra_dense_workspace_bytes(desc, pass);
     Problem p;
     if (problem_from_dense(desc, p) != PHX_OK) return 0;
+    if (dense_is_small(p)) return 0;
     return workspace_for(p, pass);
 }
 
@@ -1748,6 +1776,7 @@ int phx_qdense_fwd(const phx_qdense_desc* desc, phx_stream_t stream, const void*
     Problem p;
     const int rc = problem_from_dense(desc, p);
     if (rc != PHX_OK) return rc;
+    if (dense_is_small(p)) return is_empty(p) ? PHX_OK : run_dense_small(p, PHX_PASS_FWD, static_cast<hipStream_t>(stream), x, w, bias_or_null, y);
     return do_fwd(p, static_cast<hipStream_t>(stream), x, w, bias_or_null, y, workspace, workspace_bytes);
 }
 
@@ -1760,6 +1789,7 @@ int phx_qdense_bwd_data(const phx_qdense_desc* desc, phx_stream_t stream, const 
     Problem p;
     const int rc = problem_from_dense(desc, p);
     if (rc != PHX_OK) return rc;
+    if (dense_is_small(p)) return is_empty(p) ? PHX_OK : run_dense_small(p, PHX_PASS_BWD_DATA, static_cast<hipStream_t>(stream), grad, w, nullptr, dx);
     return do_bwd_data(p, static_cast<hipStream_t>(stream), grad, w, dx, workspace, workspace_bytes);
 }
 
@@ -1772,6 +1802,7 @@ int phx_qdense_bwd_weights(const phx_qdense_desc* desc, phx_stream_t stream, con
     Problem p;
     const int rc = problem_from_dense(desc, p);
     if (rc != PHX_OK) return rc;
+    if (dense_is_small(p)) return run_dense_small(p, PHX_PASS_BWD_WEIGHTS, static_cast<hipStream_t>(stream), x, grad, nullptr, dw);
     return do_bwd_weights(p, static_cast<hipStream_t>(stream), x, grad, dw, workspace, workspace_bytes);
 }
 

@@ -210,9 +210,12 @@ def test_conv_real_valued_input(case, mode, dtype, policy):
         capi.PHX_ERR_INVALID_ARGUMENT
 
 
+# Dense problems this small run on plain FMA threads ("fma"); PHX_TUNE_NOSMALLDENSE keeps them on the matrix cores
+@pytest.mark.parametrize("kernels", ["fma", "mfma"])
 @pytest.mark.parametrize("mode", [16, 8])
 @pytest.mark.parametrize("shape", [(32, 128, 128), (3, 5, 7), (1, 1, 1), (70, 33, 130)])
-def test_dense_fp32(shape, mode):
+def test_dense_fp32(shape, mode, kernels, tune_env):
+    tune_env(PHX_TUNE_NOSMALLDENSE="1" if kernels == "mfma" else None)
     n, ni, no = shape
     r = np.random.default_rng(n * 1000 + ni)
     x = r.standard_normal((4 * n, ni)).astype(np.float32)
@@ -223,6 +226,7 @@ def test_dense_fp32(shape, mode):
     desc = phx.DenseDescriptor(x.shape, w.shape, use_bias=True, context=Ctx(mode))
     xd, wd, bd, gd = (torch.from_numpy(a).cuda() for a in (x, w, b, gr))
     y = phx.dense_fwd(xd, wd, bd, desc)
+    assert ("qdense_fwd_fma" in capi.last_kernel_name()) == (kernels == "fma"), capi.last_kernel_name()
     dw, dx = phx.dense_bwd(xd, wd, gd, desc)
     want_y = oracle.dense_fwd(x, w, b, "generic")
     want_dw, want_dx = oracle.dense_bwd(x, w, gr, "generic")
@@ -595,9 +599,11 @@ def test_strided_input_gradient_variants(case, mode, dtype, policy, variant, tun
     assert_close(dx.cpu().numpy(), want_dx, dtype, "dgrad " + k)
 
 
+@pytest.mark.parametrize("kernels", ["fma", "mfma"])
 @pytest.mark.parametrize("policy", ["full16", "fp32"])
 @pytest.mark.parametrize("mode", [16, 8])
-def test_dense_fp16(mode, policy):
+def test_dense_fp16(mode, policy, kernels, tune_env):
+    tune_env(PHX_TUNE_NOSMALLDENSE="1" if kernels == "mfma" else None)
     n, ni, no = 16, 96, 40
     r = np.random.default_rng(5)
     x = (0.5 * r.standard_normal((4 * n, ni))).astype(np.float16)

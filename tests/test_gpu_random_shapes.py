@@ -147,10 +147,13 @@ def test_random_wide(seed):
     run_case(cfg, r, dtype, policy)
 
 
+@pytest.mark.parametrize("kernels", ["fma", "mfma"])
 @pytest.mark.parametrize("seed", range(48))
-def test_random_dense(seed):
+def test_random_dense(seed, kernels, tune_env):
     """Quaternion Dense on random batch / feature counts, both tensor types, every mode and policy, in fp64
-    against the oracle's generic path."""
+    against the oracle's generic path -- on the FMA kernels that serve problems this small and, with
+    PHX_TUNE_NOSMALLDENSE, on the matrix-core kernels."""
+    tune_env(PHX_TUNE_NOSMALLDENSE="1" if kernels == "mfma" else None)
     r = np.random.default_rng(9000 + seed)
     n, ni, no = int(r.integers(1, 80)), int(r.integers(1, 200)), int(r.integers(1, 200))
     dtype = [torch.float32, torch.float16][seed % 2]
