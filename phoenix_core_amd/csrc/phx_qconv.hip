@@ -440,7 +440,10 @@ static bool plan_forward(const Corr& c, int mode, bool f16mfma, FwdPlan& best, b
                 const double eff = ((double)c.N * c.Hout * c.Wout * c.Cout) / ((double)wgs * BN * 32 * WCO);
                 const double fill = (double)wgs / ((double)cdiv((int)std::min<long>(wgs, 1 << 30), 512) * 512);
                 const double halo = (double)std::min(NB * TH * TW, BN) / HP;  // staged data actually used
-                double score = eff * (0.25 + 0.75 * fill) * (0.9 + 0.1 * halo) * (NTW == 2 ? 1.02 : 1.0);
+                // (fp32 matrix cores, 16-product: two column tiles per wave measured slower than any one-tile shape --
+                // 3x3, 256 channels at 14x14: 5.1 against 4.1-4.6 ms -- where only the count of workgroups favoured them)
+                double score = eff * (0.25 + 0.75 * fill) * (0.9 + 0.1 * halo) *
+                               (NTW == 2 ? ((!f16mfma && !tune().oldplan) ? 0.9 : 1.02) : 1.0);
                 // fp16 MFMA is operand-bandwidth hungry: two column tiles per wave and two filter
                 // sub-tiles per workgroup amortise LDS reads and activation staging (measured)
                 // (pointwise problems, 16-product: workgroups live for a few blocks only, and two of them
