@@ -134,14 +134,19 @@ __global__ void __launch_bounds__(256) bn_sums_kernel(const BnArgs P) {
     const int total = nb * P.nchunk;
     for (int idx = threadIdx.x; idx < total; idx += 256) {
         const int b = idx / P.nchunk, ch = idx - b * P.nchunk;
-        const long off = ((long)(b0 + b) * P.C + c) * P.hw + ch * V;
-        const int n = min(V, P.hw - ch * V);
+        long off = ((long)(b0 + b) * P.C + c) * P.hw + ch * V;
+        int n = min(V, P.hw - ch * V);
+        // The last chunk of a plane that is not a whole number of chunks is read as the full chunk that ENDS at the
+        // plane's end (one 16-byte load like the others, no element-wise path that every lane of the wave would walk
+        // through); its first `seen` elements belong to the chunk before and are left out of the sums.
+        int seen = 0;
+        if (n < V && P.hw >= V) { seen = V - n; off -= seen; n = V; }
         float xv[V];
         load_chunk<TS>(x + off, n, xv);
         if constexpr (MODE == 0) {
 #pragma unroll
             for (int i = 0; i < V; ++i) {
-                const float d = i < n ? xv[i] - shift : 0.f;
+                const float d = (i < n && i >= seen) ? xv[i] - shift : 0.f;
                 a0 += d;
                 a1 += d * d;
             }
@@ -152,7 +157,7 @@ __global__ void __launch_bounds__(256) bn_sums_kernel(const BnArgs P) {
 #pragma unroll
             for (int i = 0; i < V; ++i) {
                 const float xh = (xv[i] - mean) * invstd;
-                const float d = (P.relu && g * xh + be + (res ? rv[i] : 0.f) <= 0.f) ? 0.f : dv[i];
+                const float d = (i < seen || (P.relu && g * xh + be + (res ? rv[i] : 0.f) <= 0.f)) ? 0.f : dv[i];
                 a0 += d;
                 a1 += d * xh;  // (elements past the plane carry dy = 0)
             }
@@ -204,8 +209,11 @@ __global__ void __launch_bounds__(256) bn_apply_kernel(const BnArgs P) {
     const int total = nb * P.nchunk;
     for (int idx = threadIdx.x; idx < total; idx += 256) {
         const int b = idx / P.nchunk, ch = idx - b * P.nchunk;
-        const long off = ((long)(b0 + b) * P.C + c) * P.hw + ch * V;
-        const int n = min(V, P.hw - ch * V);
+        long off = ((long)(b0 + b) * P.C + c) * P.hw + ch * V;
+        int n = min(V, P.hw - ch * V);
+        // (a plane's last, partial chunk: the full chunk ending at the plane's end instead, as in bn_sums_kernel; the
+        // elements it shares with the chunk before are computed and stored twice, with the same values)
+        if (n < V && P.hw >= V) { off -= V - n; n = V; }
         float xv[V], ov[V], rv[V];
         load_chunk<TS>(x + off, n, xv);
         if (res) load_chunk<TS>(res + off, n, rv);
@@ -239,6 +247,7 @@ static int plan(const phx_bn_desc* d, BnArgs& a) {
     const int V = d->dtype == PHX_F16 ? 8 : 4;
     a.nchunk = (d->hw + V - 1) / V;
     // enough workgroups to fill the chip several times over, at most 256 splits (one partial per thread)
+    // (fewer, longer-lived workgroups on the small layers -- at least four chunks per thread -- measured slower)
     int S = (2048 + d->c - 1) / d->c;
     S = std::max(1, std::min(S, std::min(std::max(d->rows, 1), 256)));
     a.rows_per_split = (std::max(d->rows, 1) + S - 1) / S;
