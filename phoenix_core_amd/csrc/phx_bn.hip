@@ -157,10 +157,15 @@ __global__ void __launch_bounds__(256) bn_sums_kernel(const BnArgs P) {
 #pragma unroll
             for (int i = 0; i < V; ++i) {
                 const float xh = (xv[i] - mean) * invstd;
-                const float d = (i < seen || (P.relu && g * xh + be + (res ? rv[i] : 0.f) <= 0.f)) ? 0.f : dv[i];
+                const float dm = (P.relu && g * xh + be + (res ? rv[i] : 0.f) <= 0.f) ? 0.f : dv[i];
+                dv[i] = dm;
+                const float d = i < seen ? 0.f : dm;
                 a0 += d;
                 a1 += d * xh;  // (elements past the plane carry dy = 0)
             }
+            // With a residual, the gradient behind the ReLU is the residual's gradient: written here, it also saves
+            // the apply kernel the reads of dy and the residual and the mask.
+            if (P.dres) store_chunk<TS>(static_cast<TS*>(P.dres) + off, n, dv);
         }
     }
     wg_sum2(a0, a1, red);
@@ -216,7 +221,7 @@ __global__ void __launch_bounds__(256) bn_apply_kernel(const BnArgs P) {
         if (n < V && P.hw >= V) { off -= V - n; n = V; }
         float xv[V], ov[V], rv[V];
         load_chunk<TS>(x + off, n, xv);
-        if (res) load_chunk<TS>(res + off, n, rv);
+        if (res && (MODE == 0 || !dres)) load_chunk<TS>(res + off, n, rv);
         if constexpr (MODE == 0) {
 #pragma unroll
             for (int i = 0; i < V; ++i) {
@@ -225,15 +230,19 @@ __global__ void __launch_bounds__(256) bn_apply_kernel(const BnArgs P) {
             }
         } else {
             float dv[V];
-            load_chunk<TS>(dy + off, n, dv);
+            if (dres) {  // the masked gradient, as bn_sums_kernel left it
+                load_chunk<TS>(dres + off, n, dv);
 #pragma unroll
-            for (int i = 0; i < V; ++i) {
-                const float xh = (xv[i] - mean) * invstd;
-                const float d = (P.relu && g * xh + be + (res ? rv[i] : 0.f) <= 0.f) ? 0.f : dv[i];
-                ov[i] = scale * (d - k0 - xh * k1);
-                dv[i] = d;
+                for (int i = 0; i < V; ++i) ov[i] = scale * (dv[i] - k0 - (xv[i] - mean) * invstd * k1);
+            } else {
+                load_chunk<TS>(dy + off, n, dv);
+#pragma unroll
+                for (int i = 0; i < V; ++i) {
+                    const float xh = (xv[i] - mean) * invstd;
+                    const float d = (P.relu && g * xh + be + (res ? rv[i] : 0.f) <= 0.f) ? 0.f : dv[i];
+                    ov[i] = scale * (d - k0 - xh * k1);
+                }
             }
-            if (dres) store_chunk<TS>(dres + off, n, dv);
         }
         store_chunk<TS>(out + off, n, ov);
     }
