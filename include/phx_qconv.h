@@ -192,8 +192,9 @@ int phx_qconv2d_bwd_weights(const phx_qconv_desc* desc, phx_stream_t stream, con
  *     space-to-depth forward path of strided convolutions with at most 4 input channels, the input gradient of a
  *     real-valued input): use the plain entry point.
  *   phx_qconv2d_pack_filters: either image pointer may be NULL (that image is not made); buffers 16-byte aligned.
- *   An image is valid for the descriptor it was packed for (same sizes, dtype, policy and product mode), on any
- *   stream ordered after the packing call, until the filter changes.  Results are bit-identical to the plain
+ *   An image is valid for the descriptor it was packed for (same sizes, dtype, policy and product mode; and the
+ *   same PHX_TUNE_* developer overrides, which select kernels), on any stream ordered after the packing call, until
+ *   the filter changes.  Results are bit-identical to the plain
  *   entry points'.  The workspace of a prepacked call is that of the plain call (phx_qconv2d_workspace_bytes). */
 size_t phx_qconv2d_packed_filter_bytes(const phx_qconv_desc* desc, int pass);
 int phx_qconv2d_pack_filters(const phx_qconv_desc* desc, phx_stream_t stream, const void* w, void* packed_fwd,
