@@ -50,10 +50,59 @@ int launch_fill_zero(void* dst, size_t bytes, hipStream_t st) {
     return 0;
 }
 
+// phase_merge_kernel for fp16 tensors with two column phases and fewer than 2^31 16-byte words in dx (32-bit index
+// arithmetic): a word is four elements of each of the two phase rows that feed the dx row (two 8-byte runs of two
+// buffers instead of eight 2-byte loads), interleaved in registers.
+__global__ void __launch_bounds__(WG_THREADS) phase_merge_f16_sw2_kernel(const PhaseMergeArgs A) {
+    const _Float16* buf = static_cast<const _Float16*>(A.buf);
+    _Float16* dx = static_cast<_Float16*>(A.dx);
+    const unsigned int cpr = (unsigned int)(A.W + 7) / 8u;
+    const unsigned int total = (unsigned int)A.planes * (unsigned int)A.H * cpr;
+    const int Wp0 = (A.W + 1) >> 1, Wp1 = A.W >> 1;
+    for (unsigned int idx = blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += gridDim.x * blockDim.x) {
+        const unsigned int r = idx / cpr;
+        const int w0 = (int)(idx - r * cpr) * 8;
+        const unsigned int plane = r / (unsigned int)A.H;
+        const int h = (int)(r - plane * (unsigned int)A.H);
+        const int a = h % A.sh, hp = h / A.sh;
+        const int Hp = (A.H - a + A.sh - 1) / A.sh;
+        const long o0 = A.off[a * 2], o1 = A.off[a * 2 + 1];
+        const long row = (long)plane * Hp + hp;
+        _Float16 v[8];
+        if (w0 + 8 <= A.W) {
+            f16x2 e01{}, e23{}, o01{}, o23{};
+            if (o0 >= 0) {
+                const _Float16* p = buf + o0 + row * Wp0 + (w0 >> 1);
+                e01 = __builtin_bit_cast(f16x2, load4_a2(p));
+                e23 = __builtin_bit_cast(f16x2, load4_a2(p + 2));
+            }
+            if (o1 >= 0) {
+                const _Float16* p = buf + o1 + row * Wp1 + (w0 >> 1);
+                o01 = __builtin_bit_cast(f16x2, load4_a2(p));
+                o23 = __builtin_bit_cast(f16x2, load4_a2(p + 2));
+            }
+            v[0] = e01[0]; v[1] = o01[0]; v[2] = e01[1]; v[3] = o01[1];
+            v[4] = e23[0]; v[5] = o23[0]; v[6] = e23[1]; v[7] = o23[1];
+            u32x4 raw;
+            __builtin_memcpy(&raw, v, 16);
+            *reinterpret_cast<__attribute__((address_space(1))) u32x4_a2*>(
+                (__attribute__((address_space(1))) _Float16*)(dx + (long)r * A.W + w0)) = raw;
+        } else {
+            for (int i = 0; w0 + i < A.W; ++i) {
+                const int w = w0 + i, b = w & 1;
+                const long o = b ? o1 : o0;
+                dx[(long)r * A.W + w] = o >= 0 ? buf[o + row * (b ? Wp1 : Wp0) + (w >> 1)] : (_Float16)0;
+            }
+        }
+    }
+}
+
 int launch_phase_merge(bool half_storage, const PhaseMergeArgs& a, hipStream_t st) {
     const long items = a.planes * a.H * ((a.W + 3) / 4);  // at most: 16-byte words
     if (items == 0) return 0;
-    if (half_storage) hipLaunchKernelGGL((phase_merge_kernel<_Float16>), dim3(blocks_for(items)), dim3(WG_THREADS), 0, st, a);
+    if (half_storage && a.sw == 2 && items < (1L << 31))
+        hipLaunchKernelGGL(phase_merge_f16_sw2_kernel, dim3(blocks_for(a.planes * a.H * ((a.W + 7) / 8))), dim3(WG_THREADS), 0, st, a);
+    else if (half_storage) hipLaunchKernelGGL((phase_merge_kernel<_Float16>), dim3(blocks_for(items)), dim3(WG_THREADS), 0, st, a);
     else hipLaunchKernelGGL((phase_merge_kernel<float>), dim3(blocks_for(items)), dim3(WG_THREADS), 0, st, a);
     return 0;
 }
