@@ -64,16 +64,40 @@ def rows_of(images, n):
 
 
 def dot(a, b):
-    return (a.double() * b.double()).sum().item()
+    """Inner product accumulated in fp64, a slice of the leading dimension at a time."""
+    return sum((a[i].double() * b[i].double()).sum().item() for i in range(a.shape[0]))
 
 
 def norm(a):
-    return a.double().norm().item()
+    return dot(a, a) ** 0.5
+
+
+# tensors of more than 2^31 elements (4.6 GB each in fp16): every element offset must be computed in 64 bits, and the
+# kernels that address with 32-bit offsets must have handed such problems to the ones that do not.  The crops
+# of the last images and the sparse gradient in the last image lie beyond the 2^31-st element.
+BEYOND_2G = [
+    ("k3_f16_2g", 32, 64, 64, 528, 528, 3, "SAME", torch.float16, "full16"),
+    ("pw_f16_2g", 32, 64, 64, 528, 528, 1, "VALID", torch.float16, "full16"),
+    ("k3_f32_2g", 32, 64, 64, 528, 528, 3, "SAME", torch.float32, "fp32"),
+]
 
 
 @pytest.mark.parametrize("mode", [8, 16])
 @pytest.mark.parametrize("cfg", FULL, ids=[c[0] + ("" if c[9] in ("fp32", "full16") else "_" + c[9]) for c in FULL])
 def test_full_size(cfg, mode):
+    check_full_size(cfg, mode)
+
+
+@pytest.mark.parametrize("mode", [8, 16])
+@pytest.mark.parametrize("cfg", BEYOND_2G, ids=[c[0] for c in BEYOND_2G])
+def test_beyond_2g_elements(cfg, mode):
+    name, n, ci, co, h, w = cfg[:6]
+    assert 4 * n * ci * h * w > 2 ** 31 and 4 * n * co * h * w > 2 ** 31
+    check_full_size(cfg, mode)
+    torch.cuda.empty_cache()
+
+
+def check_full_size(cfg, mode):
     name, n, ci, co, h, w, k, padding, dtype, policy = cfg
     print("config", name, "mode", mode, flush=True)
     scale = 1.0 if dtype == torch.float32 else 0.5
