@@ -214,8 +214,8 @@ class _Workspace:
     def __init__(self):
         self.buffers = {}
 
-    def get(self, device, nbytes):
-        key = (device, torch.cuda.current_stream(device).cuda_stream)
+    def get(self, device, nbytes, stream=None):
+        key = (device, current_stream_handle(device) if stream is None else stream)
         buf = self.buffers.get(key)
         if buf is None or buf.numel() < nbytes:
             buf = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=device)
@@ -223,7 +223,24 @@ class _Workspace:
         return buf
 
 
+    def holds(self, device, stream, nbytes):
+        """Whether the buffer of that stream is already large enough (no allocation would happen)."""
+        buf = self.buffers.get((device, stream))
+        return buf is not None and buf.numel() >= nbytes
+
+
 _workspace = _Workspace()
+
+# torch.cuda.current_stream() builds a Stream object through several Python layers (6-7 us per call, twice per
+# operator call); the raw handle is all the library needs
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
+def current_stream_handle(device):
+    """The handle of the device's current stream, as an integer."""
+    if _raw_stream is not None and device.index is not None:
+        return _raw_stream(device.index)
+    return torch.cuda.current_stream(device).cuda_stream
 
 
 def _dev_check(*tensors):
@@ -253,6 +270,11 @@ def _ptr(t):
     return None if t is None else ctypes.c_void_p(t.data_ptr())
 
 
+def workspace_holds(device, stream, nbytes):
+    """Whether the scratch buffer of that stream (a handle) already has nbytes: a call on it then allocates nothing."""
+    return _workspace.holds(device, stream, int(nbytes))
+
+
 def reserve_workspace(nbytes, device=None):
     """Grows the scratch buffer of the current stream to at least nbytes ahead of time -- in front of a stream
     capture, inside which the buffer must not be reallocated."""
@@ -260,8 +282,8 @@ def reserve_workspace(nbytes, device=None):
     return _workspace.get(device, int(nbytes))
 
 
-def _stream():
-    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+def _stream(device, stream=None):
+    return ctypes.c_void_p(current_stream_handle(device) if stream is None else stream)
 
 
 class PackedFilters:
@@ -297,7 +319,7 @@ def conv2d_pack_filters(w, desc, bwd_data=True, into=None):
     elif into.filter_shape != tuple(desc.filter_shape) or into.dtype != desc.dtype:
         raise ValueError("these packed filters belong to another descriptor")
     f, b = into.fwd, into.bwd_data
-    capi.check(capi.lib().phx_qconv2d_pack_filters(ctypes.byref(desc.c), _stream(), _ptr(w), _ptr(f), f.numel() if f is not None else 0,
+    capi.check(capi.lib().phx_qconv2d_pack_filters(ctypes.byref(desc.c), _stream(dev), _ptr(w), _ptr(f), f.numel() if f is not None else 0,
                                                    _ptr(b), b.numel() if b is not None else 0), "phx_qconv2d_pack_filters")
     return into
 
@@ -320,25 +342,27 @@ def conv2d_fwd(x, w, bias, desc, out=None, packed=None):
     if packed is not None and packed.fwd is not None:
         if packed.filter_shape != tuple(desc.filter_shape) or packed.dtype != desc.dtype:
             raise ValueError("these packed filters belong to another descriptor")
-        capi.check(capi.lib().phx_qconv2d_fwd_prepacked(ctypes.byref(desc.c), _stream(), _ptr(x), _ptr(packed.fwd),
+        capi.check(capi.lib().phx_qconv2d_fwd_prepacked(ctypes.byref(desc.c), _stream(dev), _ptr(x), _ptr(packed.fwd),
                                                         packed.fwd.numel(), _ptr(bias if desc.use_bias else None), _ptr(y),
                                                         _ptr(ws), nbytes), "phx_qconv2d_fwd_prepacked")
         return y
-    capi.check(capi.lib().phx_qconv2d_fwd(ctypes.byref(desc.c), _stream(), _ptr(x), _ptr(w),
+    capi.check(capi.lib().phx_qconv2d_fwd(ctypes.byref(desc.c), _stream(dev), _ptr(x), _ptr(w),
                                           _ptr(bias if desc.use_bias else None), _ptr(y), _ptr(ws), nbytes),
                "phx_qconv2d_fwd")
     return y
 
 
-def conv2d_bwd_weights(x, grad, desc):
-    """The filter-gradient half of conv2DBwd (src/conv2d.hpp:330-440): dw."""
+def conv2d_bwd_weights(x, grad, desc, stream=None):
+    """The filter-gradient half of conv2DBwd (src/conv2d.hpp:330-440): dw.  stream: the handle of a stream to enqueue
+    on instead of the device's current one; the caller then orders that stream behind the producers of x and grad
+    and the consumers of dw behind it (dw itself is allocated on the current stream)."""
     dev = _dev_check(x, grad)
     _expect(x, desc.input_shape, desc.dtype, "input")
     _expect(grad, desc.output_shape, desc.dtype, "output gradient")
     dw = torch.empty(desc.filter_shape, dtype=desc.dtype, device=dev)
     nbytes = desc.workspace_bytes(capi.PHX_PASS_BWD_WEIGHTS)
-    ws = _workspace.get(dev, nbytes)
-    capi.check(capi.lib().phx_qconv2d_bwd_weights(ctypes.byref(desc.c), _stream(), _ptr(x), _ptr(grad), _ptr(dw),
+    ws = _workspace.get(dev, nbytes, stream)
+    capi.check(capi.lib().phx_qconv2d_bwd_weights(ctypes.byref(desc.c), _stream(dev, stream), _ptr(x), _ptr(grad), _ptr(dw),
                                                   _ptr(ws), nbytes), "phx_qconv2d_bwd_weights")
     return dw
 
@@ -356,11 +380,11 @@ def conv2d_bwd_data(w, grad, desc, packed=None):
     if packed is not None and packed.bwd_data is not None:
         if packed.filter_shape != tuple(desc.filter_shape) or packed.dtype != desc.dtype:
             raise ValueError("these packed filters belong to another descriptor")
-        capi.check(capi.lib().phx_qconv2d_bwd_data_prepacked(ctypes.byref(desc.c), _stream(), _ptr(grad), _ptr(packed.bwd_data),
+        capi.check(capi.lib().phx_qconv2d_bwd_data_prepacked(ctypes.byref(desc.c), _stream(dev), _ptr(grad), _ptr(packed.bwd_data),
                                                              packed.bwd_data.numel(), _ptr(dx), _ptr(ws), nbytes),
                    "phx_qconv2d_bwd_data_prepacked")
         return dx
-    capi.check(capi.lib().phx_qconv2d_bwd_data(ctypes.byref(desc.c), _stream(), _ptr(grad), _ptr(w), _ptr(dx),
+    capi.check(capi.lib().phx_qconv2d_bwd_data(ctypes.byref(desc.c), _stream(dev), _ptr(grad), _ptr(w), _ptr(dx),
                                                _ptr(ws), nbytes), "phx_qconv2d_bwd_data")
     return dx
 
@@ -387,7 +411,7 @@ def dense_fwd(x, w, bias, desc, out=None):
     y = out if out is not None else torch.empty(desc.output_shape, dtype=desc.dtype, device=dev)
     nbytes = desc.workspace_bytes(capi.PHX_PASS_FWD)
     ws = _workspace.get(dev, nbytes)
-    capi.check(capi.lib().phx_qdense_fwd(ctypes.byref(desc.c), _stream(), _ptr(x), _ptr(w),
+    capi.check(capi.lib().phx_qdense_fwd(ctypes.byref(desc.c), _stream(dev), _ptr(x), _ptr(w),
                                          _ptr(bias if desc.use_bias else None), _ptr(y), _ptr(ws), nbytes),
                "phx_qdense_fwd")
     return y
@@ -402,14 +426,14 @@ def dense_bwd(x, w, grad, desc):
     dw = torch.empty(desc.filter_shape, dtype=desc.dtype, device=dev)
     nbytes = desc.workspace_bytes(capi.PHX_PASS_BWD_WEIGHTS)
     ws = _workspace.get(dev, nbytes)
-    capi.check(capi.lib().phx_qdense_bwd_weights(ctypes.byref(desc.c), _stream(), _ptr(x), _ptr(grad), _ptr(dw),
+    capi.check(capi.lib().phx_qdense_bwd_weights(ctypes.byref(desc.c), _stream(dev), _ptr(x), _ptr(grad), _ptr(dw),
                                                  _ptr(ws), nbytes), "phx_qdense_bwd_weights")
     dx = None
     if desc.require_input_grad:
         dx = torch.empty(desc.input_shape, dtype=desc.dtype, device=dev)
         nbytes = desc.workspace_bytes(capi.PHX_PASS_BWD_DATA)
         ws = _workspace.get(dev, nbytes)
-        capi.check(capi.lib().phx_qdense_bwd_data(ctypes.byref(desc.c), _stream(), _ptr(grad), _ptr(w), _ptr(dx),
+        capi.check(capi.lib().phx_qdense_bwd_data(ctypes.byref(desc.c), _stream(dev), _ptr(grad), _ptr(w), _ptr(dx),
                                                   _ptr(ws), nbytes), "phx_qdense_bwd_data")
     return dw, dx
 
@@ -434,7 +458,7 @@ def batch_norm_fwd(x, gamma, beta, running_mean, running_var, eps, momentum, rel
     invstd = torch.empty(c, dtype=torch.float32, device=dev)
     nbytes = capi.lib().phx_bn_workspace_bytes(ctypes.byref(desc))
     ws = _workspace.get(dev, nbytes)
-    capi.check(capi.lib().phx_bn_fwd_train(ctypes.byref(desc), _stream(), _ptr(x), _ptr(residual), _ptr(gamma), _ptr(beta),
+    capi.check(capi.lib().phx_bn_fwd_train(ctypes.byref(desc), _stream(dev), _ptr(x), _ptr(residual), _ptr(gamma), _ptr(beta),
                                            _ptr(y), _ptr(mean), _ptr(invstd), _ptr(running_mean), _ptr(running_var),
                                            _ptr(ws), nbytes), "phx_bn_fwd_train")
     return y, mean, invstd
@@ -460,7 +484,7 @@ def batch_norm_bwd(x, dy, gamma, beta, mean, invstd, eps, relu, residual=None):
     dbeta = (torch.zeros if empty else torch.empty)(c, dtype=torch.float32, device=dev)
     nbytes = capi.lib().phx_bn_workspace_bytes(ctypes.byref(desc))
     ws = _workspace.get(dev, nbytes)
-    capi.check(capi.lib().phx_bn_bwd(ctypes.byref(desc), _stream(), _ptr(x), _ptr(residual), _ptr(dy), _ptr(gamma),
+    capi.check(capi.lib().phx_bn_bwd(ctypes.byref(desc), _stream(dev), _ptr(x), _ptr(residual), _ptr(dy), _ptr(gamma),
                                      _ptr(beta), _ptr(mean), _ptr(invstd), _ptr(dx), _ptr(dres), _ptr(dgamma), _ptr(dbeta),
                                      _ptr(ws), nbytes), "phx_bn_bwd")
     return dx, dgamma, dbeta, dres
@@ -476,7 +500,7 @@ def max_pool_3x3s2_fwd(x):
     ho, wo = ((h - 1) // 2 + 1, (w - 1) // 2 + 1) if h and w else (0, 0)
     y = torch.empty((rows, c, ho, wo), dtype=x.dtype, device=dev)
     index = torch.empty((rows, c, ho, wo), dtype=torch.uint8, device=dev)
-    capi.check(capi.lib().phx_maxpool3x3s2_fwd(_DTYPES[x.dtype], rows * c, h, w, _stream(), _ptr(x), _ptr(y), _ptr(index)),
+    capi.check(capi.lib().phx_maxpool3x3s2_fwd(_DTYPES[x.dtype], rows * c, h, w, _stream(dev), _ptr(x), _ptr(y), _ptr(index)),
                "phx_maxpool3x3s2_fwd")
     return y, index
 
@@ -491,6 +515,6 @@ def max_pool_3x3s2_bwd(dy, index, input_shape):
     _expect(dy, (rows, c, ho, wo), dy.dtype, "output gradient")
     _expect(index, (rows, c, ho, wo), torch.uint8, "index")
     dx = torch.empty(tuple(input_shape), dtype=dy.dtype, device=dev)
-    capi.check(capi.lib().phx_maxpool3x3s2_bwd(_DTYPES[dy.dtype], rows * c, h, w, _stream(), _ptr(dy), _ptr(index), _ptr(dx)),
+    capi.check(capi.lib().phx_maxpool3x3s2_bwd(_DTYPES[dy.dtype], rows * c, h, w, _stream(dev), _ptr(dy), _ptr(index), _ptr(dx)),
                "phx_maxpool3x3s2_bwd")
     return dx
