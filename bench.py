@@ -79,6 +79,9 @@ def parse():
     ap.add_argument("--batch", type=int, default=64, help="images per step of the ResNet workload")
     ap.add_argument("--torch-bn", action="store_true",
                     help="ResNet workload: torch.nn.BatchNorm2d + ReLU (MIOpen) instead of the library's batch-norm kernels")
+    ap.add_argument("--pack-in-forward", action="store_true",
+                    help="c5_qresnet50: every layer packs its changed filter in its own forward call (on the caller's "
+                         "stream) instead of all layers ahead of the forward pass on the second stream")
     ap.add_argument("--frozen-filters", action="store_true",
                     help="ResNet workload: the filters do not change between steps, so no step packs them again")
     ap.add_argument("--no-graph", action="store_true", help="time the eager steps only (no HIP graph replay)")
@@ -497,13 +500,19 @@ def run_resnet(mode, policy, args):
 
     def step():
         model.zero_grad(set_to_none=True)
+        packed = None
         if not args.frozen_filters:
             # a training step follows an optimizer update: every layer packs its filter anew (once, for the forward
             # pass and the input gradient together); with frozen filters the packed images of the first step stay valid
             for m in convs:
                 m.invalidate_packed_filters()
+            if not args.pack_in_forward:
+                # ... all of them here, on the library's second stream, instead of each in front of its convolution
+                packed = phx.repack_filters(model)
         loss = torch.nn.functional.cross_entropy(model(images).float(), labels)
         loss.backward()
+        if packed is not None:
+            torch.cuda.current_stream().wait_event(packed)
         return loss.detach()
 
     t = _Timed(lambda: last.__setitem__("loss", step()), 3 * 54, args.steps, max(args.warmup, 3))
@@ -521,7 +530,9 @@ def run_resnet(mode, policy, args):
                        "is captured once into a HIP graph and replayed" if graph["used"] else "runs eagerly"),
         "product_mode": mode, "fp16_policy": policy, "batch_norm": "torch" if args.torch_bn else "library", "dtype": "f16",
         "filters": "frozen (packed once, before the timed steps)" if args.frozen_filters else
-                   "packed once per step and layer, for the forward pass and the input gradient together",
+                   "packed once per step and layer, for the forward pass and the input gradient together, " +
+                   ("by each layer in its forward call" if args.pack_in_forward else
+                    "all at the top of the step on the library's second stream"),
         "value": n / (ms_per_step * 1e-3), "unit": "img/s", "images_per_s": n / (ms_per_step * 1e-3),
         "ms_per_step": ms_per_step, "ms_per_step_eager": eager_ms, "images_per_s_eager": n / (eager_ms * 1e-3),
         "hip_graph": graph,

@@ -5,4 +5,4 @@ The arithmetic lives in hand-written HIP kernels (csrc/) behind a C ABI (include
 from . import capi  # noqa: F401
 from .ops import (COMPLEX, GA_300, QUATERNION, REAL, Context, Conv2DDescriptor, DenseDescriptor, conv2d_bwd,  # noqa: F401
                   conv2d_fwd, default_context, dense_bwd, dense_fwd, windowed_output_size_and_padding)
-from .nn import QBatchNorm2d, QConv2d, QLinear, QResNet50  # noqa: F401,E402
+from .nn import QBatchNorm2d, QConv2d, QLinear, QResNet50, repack_filters  # noqa: F401,E402

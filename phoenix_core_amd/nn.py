@@ -162,12 +162,17 @@ class QConv2d(nn.Module):
         self.bias = nn.Parameter(torch.zeros(4, out_channels, dtype=dtype)) if bias else None
         self._descs = {}
         self._packed = {}  # per descriptor pair: [filter state the images were packed from, ops.PackedFilters or None]
+        self._pack_event = None    # kept per layer: marks the end of a pack enqueued on another stream (repack_filters)
+        self._pack_pending = False  # ... which the next forward call has to wait for
 
     def _packed_filters(self, key, fwd):
         """The filter packed for this input shape, repacked (one launch, no allocation) if the filter has changed
         since: in-place updates are seen by the tensor's version counter, replaced storage by its address."""
         if not PREPACK_FILTERS:
             return None
+        if self._pack_pending:
+            _current_stream(self.weight.device).wait_event(self._pack_event)
+            self._pack_pending = False
         w = self.weight
         state = (w._version, w.data_ptr())
         ent = self._packed.get(key)
@@ -177,6 +182,18 @@ class QConv2d(nn.Module):
             ops.conv2d_pack_filters(w.detach(), fwd, into=ent[1])
             ent[0] = state
         return ent[1]
+
+    def _repack_stale(self):
+        """Packs again, on the current stream, every image whose filter has changed; True if there was one."""
+        w = self.weight
+        state = (w._version, w.data_ptr())
+        packed = False
+        for key, ent in self._packed.items():
+            if ent[1] is not None and ent[0] != state:
+                ops.conv2d_pack_filters(w.detach(), self._descs[key][0], into=ent[1])
+                ent[0] = state
+                packed = True
+        return packed
 
     def invalidate_packed_filters(self):
         """Forces the next forward call to pack again (for a filter changed behind the version counter's back,
@@ -199,6 +216,32 @@ class QConv2d(nn.Module):
         fwd, bwd = self._descriptors(x)
         packed = self._packed_filters((tuple(x.shape), x.dtype), fwd)
         return _QConv2dFn.apply(x.contiguous(), self.weight, self.bias, fwd, bwd, packed)
+
+
+def repack_filters(module):
+    """For the top of a training step, after the optimizer has changed the filters: packs the filters of every
+    QConv2d below `module` again NOW, on the second stream, instead of each layer doing so in its forward call in
+    front of its convolution -- fifty small launches leave the caller's stream and run beside the first layers.
+    Each layer's next forward call waits for its own pack.  Returns an event behind the last pack (None if nothing
+    had to be packed); a caller that captures the step into a graph makes its stream wait for it before the capture
+    ends, in case a layer that was packed did not run.  Layers that have not run yet have nothing to repack and pack
+    in their first forward call as always."""
+    convs = [m for m in module.modules() if isinstance(m, QConv2d)]
+    if not convs or not PREPACK_FILTERS:
+        return None
+    dev = convs[0].weight.device
+    main, side = torch.cuda.current_stream(dev), _side_stream(dev)
+    side.wait_stream(main)  # the images are overwritten: every kernel enqueued so far that reads them comes first
+    last = None
+    with torch.cuda.stream(side):
+        for m in convs:
+            if m._repack_stale():
+                if m._pack_event is None:
+                    m._pack_event = torch.cuda.Event()
+                m._pack_event.record(side)
+                m._pack_pending = True
+                last = m._pack_event
+    return last
 
 
 class QLinear(nn.Module):

@@ -84,7 +84,7 @@ def test_layers_repack_their_filters_when_and_only_when_they_change():
     ctx = Ctx(8, "full16")
     xs = [torch.randn(8, 16, 20, 20, device="cuda", generator=torch.Generator("cuda").manual_seed(5 + i)).half() for i in range(3)]
 
-    def run(prepack):
+    def run(prepack, ahead=False):
         old, qnn.PREPACK_FILTERS = qnn.PREPACK_FILTERS, prepack
         torch.manual_seed(4)
         layers = torch.nn.ModuleList([phx.QConv2d(16, 32, 3, dtype=torch.float16, context=ctx), phx.QConv2d(32, 32, 1, dtype=torch.float16, context=ctx),
@@ -103,6 +103,9 @@ def test_layers_repack_their_filters_when_and_only_when_they_change():
                 with torch.no_grad():
                     for m in layers:
                         m.weight.add_(m.weight.grad, alpha=-0.01)  # in place: bumps the version counter
+                if ahead:  # all layers' packs now, on the second stream; the layers wait for them
+                    done = phx.repack_filters(layers)
+                    assert done is not None and all(m._pack_pending for m in layers)
             torch.cuda.synchronize()
             return out, layers
         finally:
@@ -113,6 +116,23 @@ def test_layers_repack_their_filters_when_and_only_when_they_change():
     for a, b in zip(want, got):
         for ta, tb in zip(a, b):
             assert torch.equal(ta, tb)
+    # the same with the filters packed ahead of the forward pass (repack_filters), which then packs nothing itself
+    got, ahead_layers = run(True, ahead=True)
+    for a, b in zip(want, got):
+        for ta, tb in zip(a, b):
+            assert torch.equal(ta, tb)
+    calls = []
+    real_pack = ops.conv2d_pack_filters
+    ops.conv2d_pack_filters = lambda *a, **k: (calls.append(1), real_pack(*a, **k))[1]
+    try:
+        with torch.no_grad():
+            y = xs[0]
+            for m in ahead_layers:
+                y = m(y)
+        assert not calls and not any(m._pack_pending for m in ahead_layers)
+        assert phx.repack_filters(ahead_layers) is None  # nothing has changed
+    finally:
+        ops.conv2d_pack_filters = real_pack
     # unchanged filters: no packing call at all; a change behind the counter's back needs invalidate_packed_filters()
     calls = []
     real_pack = ops.conv2d_pack_filters
