@@ -206,6 +206,17 @@ int phx_qconv2d_bwd_data_prepacked(const phx_qconv_desc* desc, phx_stream_t stre
                                    const void* packed_bwd_data, size_t packed_bwd_data_bytes, void* dx, void* workspace,
                                    size_t workspace_bytes);
 
+/* Input gradient plus a tensor: dx = conv2DBwd's dx + addend, addend shaped and typed like dx and not dx itself.  No
+ * counterpart in the reference's interface (src/upstride.hpp:35-51 returns the gradient alone); it is what a framework
+ * does next when the convolution's input has a second consumer -- the identity branch of a residual block -- and it
+ * saves that elementwise pass: the pointwise fp16 kernels add the tensor in their epilogue, every other path adds it
+ * in a pass of its own behind the kernel.  The sum is the tensor type's own addition of the rounded gradient and the
+ * addend (fp16: rounded once more), i.e. bit for bit what the separate addition gives.  packed_bwd_data_or_null: the
+ * image of phx_qconv2d_pack_filters (then w is not read) or NULL (then w is).  Workspace as phx_qconv2d_bwd_data. */
+int phx_qconv2d_bwd_data_add(const phx_qconv_desc* desc, phx_stream_t stream, const void* grad, const void* w,
+                             const void* packed_bwd_data_or_null, size_t packed_bwd_data_bytes, const void* addend, void* dx,
+                             void* workspace, size_t workspace_bytes);
+
 /* Dense trio.  Replaces UpstrideDenseFunctor / UpstrideDenseGradFunctor for the quaternion
  * algebra (src/dense.hpp:52-62, 77-180, 223-237, 252-377). */
 int phx_qdense_fwd(const phx_qdense_desc* desc, phx_stream_t stream, const void* x, const void* w,

@@ -32,6 +32,7 @@ EXPORTS = (
     "phx_init", "phx_tuning_reload", "phx_qconv2d_fwd_noalloc",
     "phx_qconv2d_packed_filter_bytes", "phx_qconv2d_pack_filters", "phx_qconv2d_fwd_prepacked",
     "phx_qconv2d_bwd_data_prepacked",
+    "phx_qconv2d_bwd_data_add",
 )
 
 
@@ -94,6 +95,7 @@ def lib():
         L.phx_qconv2d_pack_filters.argtypes = [cd, vp, vp, vp, sz, vp, sz]
         L.phx_qconv2d_fwd_prepacked.argtypes = [cd, vp, vp, vp, sz, vp, vp, vp, sz]
         L.phx_qconv2d_bwd_data_prepacked.argtypes = [cd, vp, vp, vp, sz, vp, vp, sz]
+        L.phx_qconv2d_bwd_data_add.argtypes = [cd, vp, vp, vp, vp, sz, vp, vp, vp, sz]
         L.phx_qconv2d_bwd_weights.argtypes = [cd, vp, vp, vp, vp, vp, sz]
         L.phx_qdense_fwd.argtypes = [dd, vp, vp, vp, vp, vp, vp, sz]
         L.phx_qdense_bwd_data.argtypes = [dd, vp, vp, vp, vp, vp, sz]

@@ -36,6 +36,12 @@
 
 namespace phx {
 
+// eight fp16 sums (each rounded once, as an fp16 addition is) of two 16-byte vectors of halves
+__device__ __forceinline__ u32x4 add_halves(const u32x4& a, const u32x4& b) {
+    const f16x8 s = __builtin_bit_cast(f16x8, a) + __builtin_bit_cast(f16x8, b);
+    return __builtin_bit_cast(u32x4, s);
+}
+
 struct PwxArgs {
     const _Float16* in;     // [4][N][CinS][HW]
     long in_cs;             // elements between input components
@@ -43,6 +49,7 @@ struct PwxArgs {
     const _Float16* bias;   // [4][CoutS] or null
     _Float16* out;          // [4][N][CoutS][HW]
     long out_cs;
+    const _Float16* addend; // NCHW kernel: a tensor laid out like out that is added to the result (fp16 add), or null
     int N, Cin, CinS, Cout, CoutS, HW;
     int GI;                 // 8-pixel groups per image plane: ceil(HW / 8)
     int TGp;                // groups in all: N * GI
@@ -262,7 +269,10 @@ __global__ void __launch_bounds__(WG_THREADS, 2) qconv_pwx_f16_kernel(const PwxA
                         v[k] = __builtin_bit_cast(unsigned int, h);
                     }
                     if constexpr (TSTORE) scr[j * 9 + 2 * g4 + kk] = v;  // channel j, piece 2*g4 + kk
-                    else if (ovalid[g4] && co_ok) *reinterpret_cast<u32x4_a2*>(dst + oaddr[g4]) = v;
+                    else if (ovalid[g4] && co_ok) {
+                        if (P.addend) v = add_halves(v, load16_a2(P.addend + q * P.out_cs + (long)co * HW + oaddr[g4]));
+                        *reinterpret_cast<u32x4_a2*>(dst + oaddr[g4]) = v;
+                    }
                 }
                 if constexpr (TSTORE) {
                     // (LDS serves a wave's accesses in order: the reads see the writes above, and the next
@@ -271,9 +281,12 @@ __global__ void __launch_bounds__(WG_THREADS, 2) qconv_pwx_f16_kernel(const PwxA
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
                         const int c = 8 * i + (lane >> 3);
-                        const u32x4 t = scr[c * 9 + (lane & 7)];
-                        if (ovalid[0] && co0 + c < P.Cout)
-                            *reinterpret_cast<u32x4_a2*>(P.out + q * P.out_cs + (long)(co0 + c) * HW + oaddr[0]) = t;
+                        u32x4 t = scr[c * 9 + (lane & 7)];
+                        if (ovalid[0] && co0 + c < P.Cout) {
+                            const long o = q * P.out_cs + (long)(co0 + c) * HW + oaddr[0];
+                            if (P.addend) t = add_halves(t, load16_a2(P.addend + o));
+                            *reinterpret_cast<u32x4_a2*>(P.out + o) = t;
+                        }
                     }
                     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
                 }

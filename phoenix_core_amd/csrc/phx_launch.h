@@ -105,6 +105,7 @@ int launch_phase_merge(bool half_storage, const PhaseMergeArgs& a, hipStream_t s
 // batched matrix transposes between channels-last tensors and the kernels' channels-first layout
 int launch_transpose(bool half_storage, const TransposeArgs& a, hipStream_t st);
 int launch_fill_zero(void* dst, size_t bytes, hipStream_t st);  // a kernel, so that it can be captured in a graph
+int launch_add_inplace(bool half_storage, void* dst, const void* src, long count, hipStream_t st);  // dst += src
 
 // REAL / COMPLEX / GA_300 as compositions on the quaternion entry points (phx_algebra.hip); pass = phx_pass,
 // (a, b) = (x, w) forward, (grad, w) input gradient, (x, grad) filter gradient

@@ -107,6 +107,37 @@ int launch_phase_merge(bool half_storage, const PhaseMergeArgs& a, hipStream_t s
     return 0;
 }
 
+// dst[i] += src[i] in the tensors' own arithmetic (an fp16 sum is rounded once, like the elementwise add of a
+// framework): what follows an input gradient that could not add its addend in its own epilogue.  16-byte words
+// where both pointers allow it, element by element otherwise and for the tail.
+template <typename TS>
+__global__ void __launch_bounds__(WG_THREADS) add_inplace_kernel(TS* dst, const TS* src, long count) {
+    constexpr int V = 16 / (int)sizeof(TS);
+    const long stride = (long)gridDim.x * blockDim.x, tid = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    const bool aligned = ((reinterpret_cast<size_t>(dst) | reinterpret_cast<size_t>(src)) & 15) == 0;
+    const long words = aligned ? count / V : 0;
+    for (long i = tid; i < words; i += stride) {
+        const u32x4 a = reinterpret_cast<const u32x4*>(dst)[i], b = reinterpret_cast<const u32x4*>(src)[i];
+        u32x4 r;
+        if constexpr (sizeof(TS) == 2) r = __builtin_bit_cast(u32x4, __builtin_bit_cast(f16x8, a) + __builtin_bit_cast(f16x8, b));
+        else r = __builtin_bit_cast(u32x4, __builtin_bit_cast(f32x4, a) + __builtin_bit_cast(f32x4, b));
+        reinterpret_cast<u32x4*>(dst)[i] = r;
+    }
+    for (long i = words * V + tid; i < count; i += stride) dst[i] = dst[i] + src[i];
+}
+
+int launch_add_inplace(bool half_storage, void* dst, const void* src, long count, hipStream_t st) {
+    if (count <= 0) return 0;
+    const int blocks = blocks_for((count + 7) / 8);
+    if (half_storage)
+        hipLaunchKernelGGL((add_inplace_kernel<_Float16>), dim3(blocks), dim3(WG_THREADS), 0, st, static_cast<_Float16*>(dst),
+                           static_cast<const _Float16*>(src), count);
+    else
+        hipLaunchKernelGGL((add_inplace_kernel<float>), dim3(blocks), dim3(WG_THREADS), 0, st, static_cast<float*>(dst),
+                           static_cast<const float*>(src), count);
+    return 0;
+}
+
 int launch_transpose(bool half_storage, const TransposeArgs& a, hipStream_t st) {
     const int T = half_storage ? 64 : 32;  // tile edge of one wave
     const long tiles = a.batch * ((a.R + T - 1) / T) * ((a.Cc + T - 1) / T);

@@ -165,6 +165,15 @@ struct PackSessionScope {  // a session lasts for one entry-point call
     ~PackSessionScope() { g_pack.mode = PackSession::OFF; g_pack.base = nullptr; g_pack.capacity = g_pack.offset = 0; }
 };
 
+// An input-gradient call that adds a tensor to its result (phx_qconv2d_bwd_data_add): the kernel that writes the
+// caller's dx adds it in its epilogue if it can and says so here; otherwise a separate pass adds it afterwards.
+struct Addend {
+    const void* ptr = nullptr;
+    const void* dx = nullptr;  // the tensor the addend belongs to: only the kernel that writes THAT may take it
+    bool fused = false;
+};
+static thread_local Addend g_addend;
+
 static int flush_pack_jobs() {
     const int rc = launch_pack_jobs(g_pack.jobs, g_pack.st);
     g_pack.jobs.n = 0;
@@ -704,6 +713,10 @@ static int run_pwx(const Problem& p, const Corr& c, const FwdPlan& pl, int map, 
     a.N = c.N; a.Cin = c.Cin; a.CinS = cin_mem; a.Cout = c.Cout; a.CoutS = cout_mem; a.HW = c.Win;
     a.GI = cdiv(c.Win, 8); a.TGp = c.N * a.GI;
     a.co_tiles = pl.co_tiles; a.nsteps = pl.pwx_steps;
+    if (map == MAP_DGRAD && g_addend.ptr && out == g_addend.dx && !g_addend.fused) {
+        a.addend = static_cast<const _Float16*>(g_addend.ptr);
+        g_addend.fused = true;
+    }
     const int groups_per_tile = 8 * (4 / pl.pwx);
     a.items = cdiv(a.TGp, groups_per_tile) * pl.co_tiles;
     const int blocks = std::min(a.items, 2 * dev->cu_count);  // persistent workgroups, two per CU
@@ -714,8 +727,8 @@ static int run_pwx(const Problem& p, const Corr& c, const FwdPlan& pl, int map, 
     }
     if (rc != 0) return PHX_ERR_NOT_SUPPORTED;
     PHX_HIP(hipGetLastError());
-    snprintf(g_name_buf, sizeof(g_name_buf), "%sqconv_%s_f16mfmapwx_p16_f16_wco%d_px%d_k%d_wgs%d", g_name_prefix,
-             map == MAP_FWD ? "fwd" : "dgrad", pl.pwx, 64 * (4 / pl.pwx), pl.pwx_steps, blocks);
+    snprintf(g_name_buf, sizeof(g_name_buf), "%sqconv_%s_f16mfmapwx_p16_f16_wco%d_px%d_k%d_wgs%d%s", g_name_prefix,
+             map == MAP_FWD ? "fwd" : "dgrad", pl.pwx, 64 * (4 / pl.pwx), pl.pwx_steps, blocks, a.addend ? "_add" : "");
     g_last_kernel = g_name_buf;
     say(p, map == MAP_FWD ? "forward" : "input gradient");
     return PHX_OK;
@@ -1740,6 +1753,27 @@ int phx_qconv2d_bwd_data_prepacked(const phx_qconv_desc* desc, phx_stream_t stre
     PackSessionScope scope(PackSession::USE, const_cast<void*>(packed_bwd_data), packed_bwd_data_bytes,
                            static_cast<hipStream_t>(stream));
     return conv_bwd_data_quaternion(desc, stream, grad, packed_bwd_data, dx, workspace, workspace_bytes);
+}
+
+int phx_qconv2d_bwd_data_add(const phx_qconv_desc* desc, phx_stream_t stream, const void* grad, const void* w,
+                             const void* packed_bwd_data_or_null, size_t packed_bwd_data_bytes, const void* addend, void* dx,
+                             void* workspace, size_t workspace_bytes) {
+    if (const int init_rc = device_state(nullptr)) return init_rc;
+    if (!desc || desc->algebra != PHX_QUATERNION) return PHX_ERR_NOT_SUPPORTED;
+    if (!addend || !dx || addend == dx) return PHX_ERR_INVALID_ARGUMENT;
+    Problem p;
+    if (const int prc = problem_from_conv(desc, p)) return prc;
+    g_addend.ptr = addend; g_addend.dx = dx; g_addend.fused = false;
+    const int rc = packed_bwd_data_or_null
+                       ? phx_qconv2d_bwd_data_prepacked(desc, stream, grad, packed_bwd_data_or_null, packed_bwd_data_bytes, dx,
+                                                        workspace, workspace_bytes)
+                       : phx_qconv2d_bwd_data(desc, stream, grad, w, dx, workspace, workspace_bytes);
+    const bool fused = g_addend.fused;
+    g_addend = Addend{};
+    if (rc != PHX_OK || fused || is_empty(p)) return rc;
+    launch_add_inplace(p.dtype == PHX_F16, dx, addend, 4L * p.n * p.ci_mem * p.h * p.w, static_cast<hipStream_t>(stream));
+    PHX_HIP(hipGetLastError());
+    return PHX_OK;
 }
 
 int phx_qconv2d_bwd_weights(const phx_qconv_desc* desc, phx_stream_t stream, const void* x, const void* grad, void* dw,

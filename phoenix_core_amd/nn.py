@@ -21,6 +21,8 @@ from . import capi, ops
 # enqueued on a second stream (default priority) between two joins with the caller's stream, so that on layers too
 # small to fill the GPU the two kernels run side by side.
 OVERLAP_BACKWARD = True
+# The bottleneck blocks' first convolution takes the identity branch's gradient into its own input gradient.
+FUSE_BRANCH_GRADIENT = True
 _side_streams = {}
 
 
@@ -60,10 +62,11 @@ def _fork_join_events(device):
 PREPACK_FILTERS = os.environ.get("PHX_NO_PREPACK", "") in ("", "0")
 
 
-def _conv_backward(x, w, grad, bdesc, packed=None):
+def _conv_backward(x, w, grad, bdesc, packed=None, addend=None):
+    """(dw, dx); addend: a second gradient of x (from another consumer of x) that the input gradient takes in."""
     if not (OVERLAP_BACKWARD and bdesc.require_input_grad):
         dw = ops.conv2d_bwd_weights(x, grad, bdesc)
-        return dw, (ops.conv2d_bwd_data(w, grad, bdesc, packed=packed) if bdesc.require_input_grad else None)
+        return dw, (ops.conv2d_bwd_data(w, grad, bdesc, packed=packed, addend=addend) if bdesc.require_input_grad else None)
     dev = x.device
     main, side = _current_stream(dev), _side_stream(dev)
     side_handle = side.cuda_stream
@@ -77,7 +80,7 @@ def _conv_backward(x, w, grad, bdesc, packed=None):
         fork.record(main)
         side.wait_event(fork)
         dw = ops.conv2d_bwd_weights(x, grad, bdesc, stream=side_handle)
-        dx = ops.conv2d_bwd_data(w, grad, bdesc, packed=packed)
+        dx = ops.conv2d_bwd_data(w, grad, bdesc, packed=packed, addend=addend)
         join.record(side)
         main.wait_event(join)
         return dw, dx
@@ -86,7 +89,7 @@ def _conv_backward(x, w, grad, bdesc, packed=None):
     side.wait_stream(main)  # x and grad are complete where the side stream starts
     with torch.cuda.stream(side):
         dw = ops.conv2d_bwd_weights(x, grad, bdesc)
-    dx = ops.conv2d_bwd_data(w, grad, bdesc, packed=packed)
+    dx = ops.conv2d_bwd_data(w, grad, bdesc, packed=packed, addend=addend)
     main.wait_stream(side)  # whatever follows on the caller's stream may read dw (and free x, grad)
     dw.record_stream(main)
     return dw, dx
@@ -94,18 +97,28 @@ def _conv_backward(x, w, grad, bdesc, packed=None):
 
 class _QConv2dFn(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, x, w, bias, fdesc, bdesc, packed=None):
+    def forward(ctx, x, w, bias, fdesc, bdesc, packed=None, passthrough=False):
         ctx.save_for_backward(x, w)
         ctx.bdesc = bdesc
         ctx.has_bias = bias is not None
         ctx.packed = packed
-        return ops.conv2d_fwd(x, w, bias, fdesc, packed=packed)
+        ctx.passthrough = passthrough
+        y = ops.conv2d_fwd(x, w, bias, fdesc, packed=packed)
+        if passthrough:
+            # x is handed on as a second output: whatever else consumes x consumes THAT, so its gradient arrives
+            # here with y's, and the input gradient adds it in its own kernel instead of autograd in a pass of its own
+            ctx.set_materialize_grads(False)
+            return y, x.view_as(x)
+        return y
 
     @staticmethod
-    def backward(ctx, grad):
+    def backward(ctx, grad, grad_through=None):
         x, w = ctx.saved_tensors  # (autograd refuses a filter modified since the forward pass: the packed images match it)
+        if grad is None:  # (only with passthrough: y had no consumer)
+            return grad_through, None, None, None, None, None, None
         grad = grad.contiguous()
-        dw, dx = _conv_backward(x, w, grad, ctx.bdesc, ctx.packed)
+        addend = grad_through.contiguous() if grad_through is not None and ctx.bdesc.require_input_grad else None
+        dw, dx = _conv_backward(x, w, grad, ctx.bdesc, ctx.packed, addend)
         db = None
         if ctx.has_bias:  # bias enters every output component once: plain reduction
             n = grad.shape[0] // 4
@@ -113,7 +126,7 @@ class _QConv2dFn(torch.autograd.Function):
                 db = grad.view(4, n, -1, grad.shape[3]).float().sum(dim=(1, 2)).to(grad.dtype)
             else:
                 db = grad.view(4, n, grad.shape[1], -1).float().sum(dim=(1, 3)).to(grad.dtype)
-        return dx, dw, db, None, None, None
+        return dx, dw, db, None, None, None, None
 
 
 class _QLinearFn(torch.autograd.Function):
@@ -212,10 +225,16 @@ class QConv2d(nn.Module):
             self._descs[key] = (fwd, bwd)
         return self._descs[key]
 
-    def forward(self, x):
+    def forward(self, x, passthrough=False):
+        """passthrough: returns (y, x') with x' an alias of x for the OTHER consumers of x (the identity branch of a
+        residual block): the gradient that comes back through x' is added to the input gradient inside the
+        convolution's backward call (ops.conv2d_bwd_data(addend=...)) instead of by autograd's accumulation."""
         fwd, bwd = self._descriptors(x)
         packed = self._packed_filters((tuple(x.shape), x.dtype), fwd)
-        return _QConv2dFn.apply(x.contiguous(), self.weight, self.bias, fwd, bwd, packed)
+        if passthrough and self.input_requires_grad:
+            return _QConv2dFn.apply(x.contiguous(), self.weight, self.bias, fwd, bwd, packed, True)
+        y = _QConv2dFn.apply(x.contiguous(), self.weight, self.bias, fwd, bwd, packed)
+        return (y, x) if passthrough else y
 
 
 def repack_filters(module):
@@ -349,11 +368,14 @@ class _Bottleneck(nn.Module):
         self.relu = nn.ReLU(inplace=True)
 
     def forward(self, x):
-        idt = x if self.down is None else self.down(x)
         if self.fused_bn:
-            y = self.bn1(self.conv1(x))
+            # (conv1 hands x on to the identity branch, see QConv2d.forward: one elementwise pass less per block)
+            y, x = self.conv1(x, passthrough=True) if FUSE_BRANCH_GRADIENT else (self.conv1(x), x)
+            idt = x if self.down is None else self.down(x)
+            y = self.bn1(y)
             y = self.bn2(self.conv2(y))
             return self.bn3(self.conv3(y), idt)
+        idt = x if self.down is None else self.down(x)
         y = self.relu(self.bn1(self.conv1(x)))
         y = self.relu(self.bn2(self.conv2(y)))
         y = self.bn3(self.conv3(y))

@@ -367,9 +367,11 @@ def conv2d_bwd_weights(x, grad, desc, stream=None):
     return dw
 
 
-def conv2d_bwd_data(w, grad, desc, packed=None):
-    """The input-gradient half of conv2DBwd: dx (the descriptor must ask for it).  packed: as in conv2d_fwd."""
-    dev = _dev_check(w, grad)
+def conv2d_bwd_data(w, grad, desc, packed=None, addend=None):
+    """The input-gradient half of conv2DBwd: dx (the descriptor must ask for it).  packed: as in conv2d_fwd.
+    addend: a tensor like dx that is added to it (phx_qconv2d_bwd_data_add: in the kernel's epilogue where it can,
+    the same values as dx + addend either way); quaternion descriptors only."""
+    dev = _dev_check(w, grad, addend)
     _expect(w, desc.filter_shape, desc.dtype, "filter")
     _expect(grad, desc.output_shape, desc.dtype, "output gradient")
     if desc.real_valued_input:  # src/conv2d.hpp:394-398
@@ -377,6 +379,15 @@ def conv2d_bwd_data(w, grad, desc, packed=None):
     dx = torch.empty(desc.input_shape, dtype=desc.dtype, device=dev)
     nbytes = desc.workspace_bytes(capi.PHX_PASS_BWD_DATA)
     ws = _workspace.get(dev, nbytes)
+    if addend is not None:
+        _expect(addend, desc.input_shape, desc.dtype, "addend")
+        image = packed.bwd_data if packed is not None else None
+        if image is not None and (packed.filter_shape != tuple(desc.filter_shape) or packed.dtype != desc.dtype):
+            raise ValueError("these packed filters belong to another descriptor")
+        capi.check(capi.lib().phx_qconv2d_bwd_data_add(ctypes.byref(desc.c), _stream(dev), _ptr(grad), _ptr(w), _ptr(image),
+                                                       image.numel() if image is not None else 0, _ptr(addend), _ptr(dx),
+                                                       _ptr(ws), nbytes), "phx_qconv2d_bwd_data_add")
+        return dx
     if packed is not None and packed.bwd_data is not None:
         if packed.filter_shape != tuple(desc.filter_shape) or packed.dtype != desc.dtype:
             raise ValueError("these packed filters belong to another descriptor")

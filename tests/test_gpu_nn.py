@@ -151,6 +151,35 @@ def test_layers_repack_their_filters_when_and_only_when_they_change():
         ops.conv2d_pack_filters = real_pack
 
 
+@pytest.mark.parametrize("stride,cin", [(1, 32), (2, 16)], ids=["identity", "downsample"])
+def test_bottleneck_branch_gradient_inside_the_convolution(stride, cin):
+    """The first convolution of a bottleneck hands its input on to the identity branch (QConv2d passthrough) and adds
+    that branch's gradient inside its own input-gradient call: outputs and every gradient must equal, bit for bit,
+    those of the block whose branch gradient autograd adds in a pass of its own."""
+    from phoenix_core_amd import nn as qnn
+    ctx = Ctx(8, "full16")
+    torch.manual_seed(11)
+    block = qnn._Bottleneck(cin, 8, 32, stride, torch.float16, ctx, True).cuda()
+    x0 = torch.randn(8, cin, 12, 12, device="cuda").half()
+
+    def run(fuse):
+        old, qnn.FUSE_BRANCH_GRADIENT = qnn.FUSE_BRANCH_GRADIENT, fuse
+        try:
+            block.zero_grad(set_to_none=True)
+            x = x0.clone().requires_grad_(True)
+            y = block(x * 1.0)  # (a non-leaf input, as inside a network)
+            y.float().square().mean().backward()
+            torch.cuda.synchronize()
+            return [y.detach().clone(), x.grad.clone()] + [p.grad.clone() for p in block.parameters()]
+        finally:
+            qnn.FUSE_BRANCH_GRADIENT = old
+
+    want, got = run(False), run(True)
+    assert len(want) == len(got) > 10
+    for a, b in zip(want, got):
+        assert torch.equal(a, b)
+
+
 def test_qconv2d_groups_and_channels_last():
     """QConv2d(groups=G) is G ungrouped layers on channel slices; QConv2d(data_format="NHWC") is the NCHW layer on
     permuted activations: outputs and all gradients must agree with those compositions."""
@@ -319,7 +348,8 @@ def test_qresnet50_fp16_full16_matches_cpu_restatement(mode):
     def hook(idx):
         def fn(module, inputs, output):
             seen[idx] = [inputs[0].detach(), None]
-            output.register_hook(lambda g: seen[idx].__setitem__(1, g.detach()))
+            y = output[0] if isinstance(output, tuple) else output  # (a block's first convolution also hands its input on)
+            y.register_hook(lambda g: seen[idx].__setitem__(1, g.detach()))
         return fn
     handles = [m.register_forward_hook(hook(i)) for i, m in enumerate(convs)]
     images = torch.randn(4, 3, 64, 64).half()
@@ -383,7 +413,7 @@ def test_qresnet50_full_size_step_and_layer_crops():
 
     def hook(idx):
         def fn(module, inputs, output):
-            seen[idx] = (inputs[0].detach(), output.detach())
+            seen[idx] = (inputs[0].detach(), (output[0] if isinstance(output, tuple) else output).detach())
         return fn
     handles = [convs[i].register_forward_hook(hook(i)) for i in picked]
     images = torch.randn(n, 3, 224, 224, device="cuda").half()

@@ -767,11 +767,15 @@ def test_prepacked_filters_give_the_plain_result(case, mode, dtype, policy):
         assert torch.equal(y2, y), "prepacked fwd " + name
     dx2 = ops.conv2d_bwd_data(wd, gd, desc, packed=packed)
     assert torch.equal(dx2, dx), "prepacked dgrad " + name
+    # the input gradient that takes a second tensor in (phx_qconv2d_bwd_data_add) against the separate addition
+    addend = torch.from_numpy(x).cuda().flip(0) * 0.75
+    assert torch.equal(ops.conv2d_bwd_data(wd, gd, desc, packed=packed, addend=addend), dx + addend), "dgrad + addend " + name
     # packing again into the same buffers after the filter has changed
     wd.copy_(torch.from_numpy(wt).cuda() * 0.5)
     assert ops.conv2d_pack_filters(wd, desc, into=packed) is packed
     want = ops.conv2d_bwd_data(wd, gd, desc)
     assert torch.equal(ops.conv2d_bwd_data(wd, gd, desc, packed=packed), want), "repacked dgrad " + name
+    assert torch.equal(ops.conv2d_bwd_data(wd, gd, desc, addend=addend), want + addend), "dgrad + addend, plain " + name
 
 
 @pytest.mark.parametrize("mode", [16, 8])
@@ -800,6 +804,42 @@ def test_prepacked_filters_grouped_and_channels_last(case, mode):
     wd.zero_()
     assert torch.equal(phx.conv2d_fwd(xd, wd, None, desc, packed=packed), y), "prepacked fwd " + name
     assert torch.equal(ops.conv2d_bwd_data(wd, gd, desc, packed=packed), dx), "prepacked dgrad " + name
+    addend = xd.flip(0) * 0.75
+    assert torch.equal(ops.conv2d_bwd_data(wd, gd, desc, packed=packed, addend=addend), dx + addend), "dgrad + addend " + name
+
+
+@pytest.mark.parametrize("mode", [16, 8])
+@pytest.mark.parametrize("shape", [(3, 40, 24, 6, 6), (2, 128, 128, 14, 14), (5, 16, 64, 7, 8), (2, 64, 16, 28, 28)],
+                         ids=lambda s: "n%d_%dto%d_%dx%d" % s)
+def test_pointwise_input_gradient_adds_in_its_epilogue(shape, mode):
+    """Pointwise fp16 input gradients on even planes run the streaming kernel, which adds the tensor while it stores
+    (one launch, no pass of its own): same kernel as without the addend, the values of dx + addend bit for bit."""
+    n, ci, co, h, w = shape
+    r = np.random.default_rng(n * 1000 + ci + co)
+    gd = torch.from_numpy((0.5 * r.standard_normal((4 * n, co, h, w))).astype(np.float16)).cuda()
+    wd = torch.from_numpy((0.2 * r.standard_normal((4, co, ci, 1, 1))).astype(np.float16)).cuda()
+    addend = torch.from_numpy((2.0 * r.standard_normal((4 * n, ci, h, w))).astype(np.float16)).cuda()
+    desc = phx.Conv2DDescriptor((4 * n, ci, h, w), wd.shape, 1, 1, "VALID", dtype=torch.float16, context=Ctx(mode, "full16"))
+    dx = ops.conv2d_bwd_data(wd, gd, desc)
+    kernel = capi.last_kernel_name()
+    assert "pwx" in kernel, kernel
+    got = ops.conv2d_bwd_data(wd, gd, desc, addend=addend)
+    assert capi.last_kernel_name() == kernel + "_add"
+    assert torch.equal(got, dx + addend)
+    packed = ops.conv2d_pack_filters(wd, desc)
+    assert torch.equal(ops.conv2d_bwd_data(wd, gd, desc, packed=packed, addend=addend), dx + addend)
+    assert capi.last_kernel_name() == kernel + "_add"
+    # refused: the addend must not be dx itself, nor missing
+    L = capi.lib()
+    nbytes = desc.workspace_bytes(capi.PHX_PASS_BWD_DATA)
+    ws = ops.reserve_workspace(nbytes)
+    rc = L.phx_qconv2d_bwd_data_add(ctypes.byref(desc.c), None, gd.data_ptr(), wd.data_ptr(), None, 0, got.data_ptr(), got.data_ptr(),
+                                    ws.data_ptr(), nbytes)
+    assert rc == capi.PHX_ERR_INVALID_ARGUMENT
+    rc = L.phx_qconv2d_bwd_data_add(ctypes.byref(desc.c), None, gd.data_ptr(), wd.data_ptr(), None, 0, None, got.data_ptr(),
+                                    ws.data_ptr(), nbytes)
+    assert rc == capi.PHX_ERR_INVALID_ARGUMENT
+    torch.cuda.synchronize()
 
 
 def test_prepacked_filters_are_refused_where_they_do_not_apply():
