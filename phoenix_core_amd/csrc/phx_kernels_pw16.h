@@ -80,7 +80,9 @@ struct PwxShape {
     static constexpr size_t lds_bytes_nchw = (size_t)RN * SV * 16 + (TSTORE ? 4 * SCRV * 16 : 0);
 };
 
-template <int WCO>
+// ADD: the instance that adds P.addend to what it stores (the plain instance carries none of that code: the extra
+// registers of the addend's prefetch cost the plain kernel 4 % where both were one)
+template <int WCO, bool ADD = false>
 __global__ void __launch_bounds__(WG_THREADS, 2) qconv_pwx_f16_kernel(const PwxArgs P) {
     using S = PwxShape<WCO>;
     constexpr int WPX = S::WPX, GPT = S::GPT, ROWDW = S::ROWDW, WV = S::WV, SV = S::SV, R = S::RN, D = R - 1;
@@ -247,10 +249,23 @@ __global__ void __launch_bounds__(WG_THREADS, 2) qconv_pwx_f16_kernel(const PwxA
         PHX_STAMP(3)
         if (++c_k == P.nsteps) {
             // the item is complete (see above for who holds what)
+            const int co0 = (c_ct * WCO + wco) * 32;
+            // (TSTORE) the addend's vectors of a component are requested a component ahead -- the first here, in
+            // front of the drain, which then covers their latency; the others in front of the stores of the component
+            // before -- so that no store waits for a load of its own
+            u32x4 ad[4];
+            auto request_addend = [&](int q, u32x4 (&dst)[4]) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int c = 8 * i + (lane >> 3);
+                    const bool ok = ovalid[0] && co0 + c < P.Cout;
+                    dst[i] = ok ? load16_a2(P.addend + q * P.out_cs + (long)(co0 + c) * HW + oaddr[0]) : u32x4{0u, 0u, 0u, 0u};
+                }
+            };
+            if constexpr (TSTORE && ADD) request_addend(0, ad);
             wait_vmem_all();  // this wave's copies of the next D stages: landed
             covered = D;
             PHX_STAMP(2)
-            const int co0 = (c_ct * WCO + wco) * 32;
             const int co = co0 + j;
             const bool co_ok = co < P.Cout;
             u32x4* scr = reinterpret_cast<u32x4*>(lds16 + R * SV) + wave * S::SCRV;  // (TSTORE) this wave's own
@@ -270,7 +285,7 @@ __global__ void __launch_bounds__(WG_THREADS, 2) qconv_pwx_f16_kernel(const PwxA
                     }
                     if constexpr (TSTORE) scr[j * 9 + 2 * g4 + kk] = v;  // channel j, piece 2*g4 + kk
                     else if (ovalid[g4] && co_ok) {
-                        if (P.addend) v = add_halves(v, load16_a2(P.addend + q * P.out_cs + (long)co * HW + oaddr[g4]));
+                        if constexpr (ADD) v = add_halves(v, load16_a2(P.addend + q * P.out_cs + (long)co * HW + oaddr[g4]));
                         *reinterpret_cast<u32x4_a2*>(dst + oaddr[g4]) = v;
                     }
                 }
@@ -278,15 +293,20 @@ __global__ void __launch_bounds__(WG_THREADS, 2) qconv_pwx_f16_kernel(const PwxA
                     // (LDS serves a wave's accesses in order: the reads see the writes above, and the next
                     // component's writes come after these reads)
                     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                    u32x4 t[4];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        t[i] = scr[(8 * i + (lane >> 3)) * 9 + (lane & 7)];
+                        if constexpr (ADD) t[i] = add_halves(t[i], ad[i]);
+                    }
+                    if constexpr (ADD) {
+                        if (q < 3) request_addend(q + 1, ad);  // (in front of this component's stores)
+                    }
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
                         const int c = 8 * i + (lane >> 3);
-                        u32x4 t = scr[c * 9 + (lane & 7)];
-                        if (ovalid[0] && co0 + c < P.Cout) {
-                            const long o = q * P.out_cs + (long)(co0 + c) * HW + oaddr[0];
-                            if (P.addend) t = add_halves(t, load16_a2(P.addend + o));
-                            *reinterpret_cast<u32x4_a2*>(P.out + o) = t;
-                        }
+                        if (ovalid[0] && co0 + c < P.Cout)
+                            *reinterpret_cast<u32x4_a2*>(P.out + q * P.out_cs + (long)(co0 + c) * HW + oaddr[0]) = t[i];
                     }
                     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
                 }

@@ -4,18 +4,24 @@
 
 namespace phx {
 
-template <int WCO>
+template <int WCO, bool ADD>
 static int launch_pwx_one(const PwxArgs& a, int blocks, hipStream_t st) {
-    constexpr auto kernel = qconv_pwx_f16_kernel<WCO>;
+    constexpr auto kernel = qconv_pwx_f16_kernel<WCO, ADD>;
     if (!BigLds<kernel>::registered) return -1;  // more than 64 KiB of dynamic LDS: opted in per device at set-up, see BigLds
     hipLaunchKernelGGL(kernel, dim3(blocks), dim3(WG_THREADS), PwxShape<WCO>::lds_bytes_nchw, st, a);
     return 0;
 }
 
 int launch_pwx_f16(int WCO, const PwxArgs& a, int blocks, hipStream_t st) {
-    if (WCO == 4) return launch_pwx_one<4>(a, blocks, st);
-    if (WCO == 2) return launch_pwx_one<2>(a, blocks, st);
-    if (WCO == 1) return launch_pwx_one<1>(a, blocks, st);
+    if (a.addend) {  // the instance that adds a tensor to what it stores
+        if (WCO == 4) return launch_pwx_one<4, true>(a, blocks, st);
+        if (WCO == 2) return launch_pwx_one<2, true>(a, blocks, st);
+        if (WCO == 1) return launch_pwx_one<1, true>(a, blocks, st);
+        return -1;
+    }
+    if (WCO == 4) return launch_pwx_one<4, false>(a, blocks, st);
+    if (WCO == 2) return launch_pwx_one<2, false>(a, blocks, st);
+    if (WCO == 1) return launch_pwx_one<1, false>(a, blocks, st);
     return -1;
 }
 
