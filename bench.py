@@ -3,12 +3,13 @@
 
 A step is one pass of the hot path over one batch of synthetic input, resident in HBM: forward,
 input gradient and filter gradient of one quaternion operator (or one forward+backward of the
-quaternion ResNet-50).  The default run prints ONE JSON line whose headline (`value`, `roofline`,
-`cpu_baseline`) is the largest convolution configuration -- 3x3, fp16 tensors, N=128, 128->128
-quaternion channels, 28x28, full16 policy -- and which carries, under `per_config`, the same figures
-for every other configuration (Dense fp32; 1x1 and 3x3 fp32; the four fp16 shapes under both fp16
-policies; each in both product modes) and, under `c5_qresnet50`, the ResNet-50 images/s.
-`--workload NAME` runs one configuration alone (used for profiling).
+quaternion ResNet-50).  The default run measures every configuration (Dense fp32; 1x1 and 3x3 fp32; the
+four fp16 shapes under both fp16 policies; each in both product modes; the ResNet-50) and prints one
+full JSON record per configuration as a line of its own (`{"record": ...}`), then -- LAST -- the one
+short JSON line of the contract (under 1800 characters): headline (`value`, `roofline`, `cpu_baseline`)
+= the largest convolution configuration -- 3x3, fp16 tensors, N=128, 128->128 quaternion channels,
+28x28, full16 policy --, `per_config` as workload -> policy -> mode -> [ms per step, TFLOP/s] and `c5`
+= the ResNet-50's images/s.  `--workload NAME` runs one configuration alone (used for profiling).
 
 Throughput is real-equivalent: 16 real multiply-adds per quaternion multiply-add whichever product
 formulation runs; the factorized (8-product) kernels execute half of them, which `executed_frac`
@@ -53,18 +54,45 @@ def executed_share(kernel_name):
 
 
 def measured_traffic():
-    """HBM bytes per launch from the rocprofv3 --pmc summaries, keyed by (workload, kernel variant name):
-    rows `| workload | kernel | fetched bytes | written bytes |` of profiles/hbm_traffic.md."""
+    """Counter figures per launch from the rocprofv3 --pmc summaries, keyed by (workload, kernel variant name):
+    rows `| workload | kernel | fetched bytes | written bytes | MFMA busy |` of profiles/hbm_traffic.md
+    -> {"bytes": fetched + written, "mfma_busy": fraction or None}."""
     table = {}
+    num = r"[0-9.e+]+"
     try:
         with open(TRAFFIC_FILE) as f:
             for line in f:
                 cells = [c.strip().strip("`") for c in line.strip().strip("|").split("|")]
-                if len(cells) == 4 and re.fullmatch(r"[0-9.e+]+", cells[2]) and re.fullmatch(r"[0-9.e+]+", cells[3]):
-                    table[(cells[0], cells[1])] = float(cells[2]) + float(cells[3])
+                if len(cells) in (4, 5) and re.fullmatch(num, cells[2]) and re.fullmatch(num, cells[3]):
+                    busy = None
+                    if len(cells) == 5 and re.fullmatch(num, cells[4].rstrip(" %")):
+                        busy = float(cells[4].rstrip(" %")) / 100.0
+                    table[(cells[0], cells[1])] = {"bytes": float(cells[2]) + float(cells[3]), "mfma_busy": busy}
     except OSError:
         pass
     return table
+
+
+def host_info():
+    """What the CPU baselines ran on: CPU model, the threads used, torch's version and its oneDNN."""
+    import torch
+    model = "unknown"
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    model = line.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
+    try:
+        threads = int(os.environ.get("OMP_NUM_THREADS", "0"))
+    except ValueError:
+        threads = 0
+    if threads <= 0:
+        threads = min(os.cpu_count() or 1, 16)  # a one-GPU box's share of its host is 16 cores
+    return {"cpu_model": model, "threads": threads, "torch": torch.__version__,
+            "onednn": bool(torch.backends.mkldnn.is_available())}
 
 
 def parse():
@@ -107,16 +135,28 @@ def default_mode(args):
     return 16 if phx.Context().memory_optimized else 8
 
 
-def cpu_baseline_conv(cfg, mode, seconds):
+def _median_time(step, seconds, least, most):
+    step()  # warm-up (primitive creation)
+    times = []
+    t_end = time.perf_counter() + seconds
+    while len(times) < least or (time.perf_counter() < t_end and len(times) < most):
+        t0 = time.perf_counter()
+        step()
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    return times[len(times) // 2], len(times)
+
+
+def cpu_baseline_conv(cfg, mode, seconds, images=None):
     """The reference's CPU algorithm (lane decomposition + scalar oneDNN convolutions through
-    torch's CPU backend) on a bounded sample of the same workload."""
+    torch's CPU backend) on a bounded sample of the same workload: `images` of its N images."""
     import torch
     import oracle
     from oracle import torch_cpu_path as tcp
     n, ci, co, h, w, k, padding, _ = cfg
-    threads = min(os.cpu_count() or 1, 16)
-    torch.set_num_threads(threads)
-    n_s = max(1, n // 8)
+    host = host_info()
+    torch.set_num_threads(host["threads"])
+    n_s = images or max(1, n // 8)
     g = oracle.make_geom(n_s, ci, co, h, w, k, k, 1, 1, padding)
     gen = torch.Generator().manual_seed(0x5EED)
     x = torch.randn(4 * n_s, ci, h, w, generator=gen)
@@ -129,29 +169,27 @@ def cpu_baseline_conv(cfg, mode, seconds):
         tcp.conv2d_fwd(g, x, wt, None, name)
         tcp.conv2d_bwd(g, x, wt, gr, name)
 
-    step()  # warm-up (primitive creation)
-    times = []
-    t_end = time.perf_counter() + seconds
-    while len(times) < 3 or (time.perf_counter() < t_end and len(times) < 50):
-        t0 = time.perf_counter()
-        step()
-        times.append(time.perf_counter() - t0)
-    times.sort()
-    med = times[len(times) // 2]
+    med, runs = _median_time(step, seconds, 3, 50)
     return {
-        "value": flops / med / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
-        "sample": "%d of %d images of the same workload, fwd+dgrad+wgrad, %s path, scalar convs by torch %s CPU "
-                  "(oneDNN), fp32, median of %d runs" % (n_s, n, name, torch.__version__, len(times)),
+        "value": flops / med / 1e12, "unit": "TFLOP/s", "cores": host["threads"], "cpu_model": host["cpu_model"],
+        "kind": "port",
+        "sample": "%d/%d images, fwd+bwd, %s path, torch %s CPU (oneDNN) convs, fp32, "
+                  "median of %d" % (n_s, n, name, host["torch"], runs),
         "ms_per_step_sample": med * 1e3,
     }
 
 
 def cpu_baseline_dense(cfg, mode, seconds):
-    """The reference's CPU Dense path restated in C (oracle/, float arithmetic, the factorized or generic
-    formulation), whole workload, single thread."""
+    """The reference's CPU Dense path (lane decomposition + 8 or 16 scalar matmuls, src/dense.hpp:77-180, 252-377
+    over src/backend/onednn/dense.hpp:53-93) with the matmuls by torch's CPU backend, whole workload, all threads;
+    the single-threaded C restatement of the same algorithm is timed beside it."""
     import numpy as np
+    import torch
     import oracle
+    from oracle import torch_cpu_path as tcp
     n, ni, no, _ = cfg
+    host = host_info()
+    torch.set_num_threads(host["threads"])
     r = np.random.default_rng(0x5EED + 1)
     x = r.standard_normal((4 * n, ni)).astype(np.float32)
     lim = (6.0 / (ni + no)) ** 0.5
@@ -159,25 +197,25 @@ def cpu_baseline_dense(cfg, mode, seconds):
     b = np.zeros((4, no), np.float32)
     gr = r.standard_normal((4 * n, no)).astype(np.float32)
     name = "factorized" if mode == 8 else "generic"
+    tx, tw, tb, tg = (torch.from_numpy(a) for a in (x, w, b, gr))
 
     def step():
+        tcp.dense_fwd(tx, tw, tb, name)
+        tcp.dense_bwd(tx, tw, tg, name)
+
+    def step_c():
         oracle.dense_fwd(x, w, b, name, dtype=np.float32)
         oracle.dense_bwd(x, w, gr, name, dtype=np.float32)
 
-    step()
-    times = []
-    t_end = time.perf_counter() + min(seconds, 2.0)
-    while len(times) < 5 or (time.perf_counter() < t_end and len(times) < 200):
-        t0 = time.perf_counter()
-        step()
-        times.append(time.perf_counter() - t0)
-    times.sort()
-    med = times[len(times) // 2]
+    med, runs = _median_time(step, min(seconds, 2.0), 5, 500)
+    med_c, _ = _median_time(step_c, min(seconds, 1.0), 5, 200)
     flops = 3 * 2.0 * 16 * n * ni * no
-    return {"value": flops / med / 1e12, "unit": "TFLOP/s", "cores": 1, "kind": "port",
-            "sample": "whole workload, fwd+dgrad+wgrad, %s path, C restatement of the reference's CPU algorithm "
-                      "(scalar matmuls as plain loops, one thread), fp32, median of %d runs" % (name, len(times)),
-            "ms_per_step_sample": med * 1e3}
+    return {"value": flops / med / 1e12, "unit": "TFLOP/s", "cores": host["threads"], "cpu_model": host["cpu_model"],
+            "kind": "port",
+            "sample": "whole workload, fwd+dgrad+wgrad, %s path, scalar matmuls by torch %s CPU (oneDNN), fp32, "
+                      "median of %d" % (name, host["torch"], runs),
+            "ms_per_step_sample": med * 1e3,
+            "c_restatement_one_thread_ms": med_c * 1e3}
 
 
 class _Timed:
@@ -185,7 +223,8 @@ class _Timed:
     slot, the mean HIP-event duration of its dominant kernel.  Three passes of `steps` steps each: eager without
     the library's event timer (its event records sit between the kernels), eager with it (kernel durations), and --
     where `outputs` is given and graphs are not switched off -- the step replayed from a HIP graph, trusted only if
-    every checked replay reproduces the eager outputs bit for bit; `ms_per_step` is the faster of eager and replay."""
+    every checked replay reproduces the eager outputs bit for bit.  One rule for `ms_per_step`: the verified replay
+    where there is one, the eager figure otherwise (both are kept in the record)."""
 
     def __init__(self, step, ncalls, steps, warmup, outputs=None, use_graph=True):
         import torch
@@ -210,10 +249,9 @@ class _Timed:
         self.graph = {"used": False, "note": "not attempted"}
         if outputs is not None and use_graph:
             self.graph = self._replay(step, steps, warmup, outputs)
-            # (a step of a few launches can be faster eagerly: the figure reported is the faster of the two ways)
-            if self.graph["used"] and self.graph["ms_per_step"] < self.ms_per_step_eager:
+            if self.graph["used"]:
                 self.ms_per_step = self.graph["ms_per_step"]
-            self.graph["reported"] = "hip_graph_replay" if self.ms_per_step != self.ms_per_step_eager else "eager"
+            self.graph["reported"] = "hip_graph_replay" if self.graph["used"] else "eager"
 
     @staticmethod
     def _replay(step, steps, warmup, outputs):
@@ -254,10 +292,13 @@ class _Timed:
             return {"used": False, "note": "capture or replay failed: %s" % (str(exc)[:200],)}
 
 
-def roofline_of(pass_name, kernel, flops, nbytes, kernel_ms, compute, traffic):
+def roofline_of(pass_name, kernel, flops, nbytes, kernel_ms, compute, counters):
     """Roofline record of one kernel launch.  `bound` names the roof that applies by arithmetic
-    intensity (algorithmic FLOPs / algorithmic bytes against the ridge peak_flops / peak_bandwidth);
-    `regime` says "latency" when the kernel is below half of both roofs."""
+    intensity (algorithmic FLOPs / algorithmic bytes against the ridge peak_flops / peak_bandwidth) and
+    `frac` is algorithmic work over that roof.  `regime` is what the counters of the committed rocprofv3
+    run of this kernel variant say it is held by: "mfma" when the matrix pipe is busy at least half the
+    time, "hbm" when the measured traffic moves at half of peak bandwidth or more, otherwise "issue/latency";
+    null when the variant has no counter row."""
     peak = PEAK_TFLOPS[compute]
     tflops = flops / (kernel_ms * 1e-3) / 1e12
     gbs = nbytes / (kernel_ms * 1e-3) / 1e9
@@ -266,16 +307,26 @@ def roofline_of(pass_name, kernel, flops, nbytes, kernel_ms, compute, traffic):
     ai = flops / nbytes
     bound = "hbm" if ai < ridge else "mfma"
     frac_mfma, frac_hbm = tflops / peak, gbs / PEAK_HBM_GBS
+    traffic = counters["bytes"] if counters else None
+    busy = counters["mfma_busy"] if counters else None
     out = {"bound": bound, "pass": pass_name, "kernel": kernel, "kernel_ms": kernel_ms}
     if bound == "mfma":
         out.update({"achieved": tflops, "peak": peak, "unit": "TFLOP/s", "frac": frac_mfma})
     else:
         out.update({"achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": frac_hbm})
+    regime = None
+    if counters:
+        traffic_frac = traffic / (kernel_ms * 1e-3) / 1e9 / PEAK_HBM_GBS
+        if busy is not None and busy >= 0.5:
+            regime = "mfma"
+        elif traffic_frac >= 0.5:
+            regime = "hbm"
+        elif busy is not None:
+            regime = "issue/latency"
     out.update({
         "executed_frac": frac_mfma * share,  # executed FLOPs / MFMA peak (the factorized kernels run half)
         "real_equiv_tflops": tflops, "frac_of_mfma_peak": frac_mfma, "algorithmic_gb_s": gbs, "frac_of_hbm_peak": frac_hbm,
-        "arithmetic_intensity": ai, "ridge": ridge,
-        "regime": "latency" if max(frac_mfma * share, frac_hbm) < 0.5 else bound,
+        "arithmetic_intensity": ai, "ridge": ridge, "regime": regime, "mfma_busy": busy,
         "algorithmic_bytes": nbytes, "algorithmic_flops": flops,
         "traffic": traffic,
     })
@@ -348,7 +399,7 @@ def run_conv(name, mode, policy, args, traffic_table):
     return {
         "workload": "%s: quaternion conv %dx%d stride 1, N=%d (4N=%d rows), %d->%d q-channels, %dx%d, "
                     "fwd+input-grad+filter-grad" % (name, k, k, n, 4 * n, ci, co, h, w),
-        "product_mode": mode, "fp16_policy": policy, "padding": padding, "dtype": dt,
+        "n": n, "product_mode": mode, "fp16_policy": policy, "padding": padding, "dtype": dt,
         "value": value, "unit": "TFLOP/s", "ms_per_step": t.ms_per_step, "ms_per_step_eager": t.ms_per_step_eager,
         "hip_graph": t.graph, "images_per_s": n / (t.ms_per_step * 1e-3),
         "kernel_ms": per_pass, "kernels": names,
@@ -357,6 +408,7 @@ def run_conv(name, mode, policy, args, traffic_table):
         "executed_frac": {p: roofs[p]["executed_frac"] for p in PASSES},
         "frac_of_hbm_peak": {p: roofs[p]["frac_of_hbm_peak"] for p in PASSES},
         "roofline": roofs[dominant],
+        "unprofiled_kernels": sorted({names[p] for p in PASSES if (name, names[p]) not in traffic_table}),
     }
 
 
@@ -410,6 +462,7 @@ def run_dense(name, mode, args, traffic_table):
         "kernel_ms": per_pass, "kernels": names,
         "real_equiv_tflops": {p: roofs[p]["real_equiv_tflops"] for p in PASSES},
         "roofline": roofs[dominant],
+        "unprofiled_kernels": sorted({names[p] for p in PASSES if (name, names[p]) not in traffic_table}),
         "note": "16.8 MFLOP per pass: a handful of kernel launches of a few microseconds each, launch-latency bound",
     }
     if not args.no_cpu_baseline:
@@ -545,20 +598,57 @@ def run_resnet(mode, policy, args):
     return out
 
 
+def sig(v, digits=4):
+    """Floats rounded to `digits` significant digits, recursively (the contract's line has to stay short)."""
+    if isinstance(v, float):
+        if v != v or abs(v) == float("inf"):
+            return None
+        r = float("%.*g" % (digits, v))
+        return int(r) if abs(r) >= 10 ** (digits - 1) else r  # (no digits behind the point are significant there)
+    if isinstance(v, dict):
+        return {k: sig(x, digits) for k, x in v.items()}
+    if isinstance(v, (list, tuple)):
+        return [sig(x, digits) for x in v]
+    return v
+
+
+LINE_LIMIT = 1800  # characters; the driver keeps the last 2000 of the output for parsing
+
+
 def line(head, args, extra=None):
-    """The contract's JSON line around one workload record."""
+    """The contract's JSON line around one workload record: the keys the contract names, a trimmed `roofline`
+    and `cpu_baseline`, and whatever short `extra` the caller adds; the full record goes out on a line before it."""
     out = {
         "metric": METRIC, "value": head["value"], "unit": head["unit"], "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": head["ms_per_step"], "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": head["dtype"], "data": "synthetic",
         "config": {k: head[k] for k in ("workload", "product_mode", "fp16_policy", "padding", "batch_norm") if k in head},
     }
-    for k, v in head.items():
-        if k not in out and k not in out["config"]:
-            out[k] = v
+    out["config"]["workload"] = out["config"]["workload"].split(", fwd+")[0].replace(" (4N=%d rows)" % (4 * head.get("n", 0)), "")[:120]
+    if "roofline" in head:
+        keep = ("bound", "pass", "kernel", "kernel_ms", "achieved", "peak", "unit", "frac", "executed_frac",
+                "algorithmic_bytes", "traffic", "regime")
+        out["roofline"] = {k: head["roofline"].get(k) for k in keep}
+    if "cpu_baseline" in head:
+        keep = ("value", "unit", "cores", "cpu_model", "kind", "sample", "ms_per_step_sample")
+        out["cpu_baseline"] = {k: head["cpu_baseline"].get(k) for k in keep}
+        out["cpu_baseline"]["cpu_model"] = str(out["cpu_baseline"]["cpu_model"])[:40]
     if extra:
         out.update(extra)
-    return out
+    out = sig(out)
+    text = json.dumps(out, separators=(",", ":"))
+    if len(text) > LINE_LIMIT and "per_config" in out:  # keep the headline parseable whatever the table's size
+        out["per_config"] = sig(out["per_config"], 2)
+        text = json.dumps(out, separators=(",", ":"))
+        if len(text) > LINE_LIMIT:
+            out["per_config"] = "see the record lines above"
+            text = json.dumps(out, separators=(",", ":"))
+    return text
+
+
+def emit(record, name, key=None):
+    """One full record as a line of its own, ahead of the contract's line."""
+    print(json.dumps({"record": name if key is None else "%s/%s" % (name, key), **sig(record, 6)}), flush=True)
 
 
 def main():
@@ -573,41 +663,68 @@ def main():
     traffic = measured_traffic()
 
     if args.workload == RESNET:
-        print(json.dumps(line(run_resnet(mode, policy, args), args)))
+        head = run_resnet(mode, policy, args)
+        emit(head, RESNET)
+        print(line(head, args, {"c5": {"images_per_s": head["images_per_s"], "ms_per_step": head["ms_per_step"]}}))
         return 0
     if args.workload in DENSE:
-        print(json.dumps(line(run_dense(args.workload, mode, args, traffic), args)))
+        head = run_dense(args.workload, mode, args, traffic)
+        emit(head, args.workload)
+        print(line(head, args))
         return 0
     if args.workload in CONVS:
         head = run_conv(args.workload, mode, policy, args, traffic)
         if not args.no_cpu_baseline:
             head["cpu_baseline"] = cpu_baseline_conv(CONVS[args.workload], mode, args.cpu_seconds)
-        print(json.dumps(line(head, args)))
+        emit(head, args.workload)
+        print(line(head, args))
         return 0
 
-    # default: headline on the largest convolution configuration + every other configuration beside it
-    head = run_conv(HEADLINE, mode, policy, args, traffic)
-    per_config = {}
+    # default: every configuration as a record line of its own, the headline's short line last
+    short, stale = {}, set()
+
+    def note(name, pol, m, rec):
+        emit(rec, name, "%s_mode%d" % (pol, m))
+        short.setdefault(name, {}).setdefault(pol, {})[str(m)] = sig([rec["ms_per_step"], rec["value"]], 3)
+        stale.update("%s:%s" % (name, k) for k in rec.get("unprofiled_kernels", ()))
+
+    sampled = {"c4_pw_f16_128_28": 4, "c2_pw_f32": 8, "c3_k3_f32": 4}  # images of the 1-2 s CPU samples
+    c5 = {}
+    for m in (mode, 24 - mode):
+        c5[m] = run_resnet(m, "full16", args)
+        emit(c5[m], RESNET, "full16_mode%d" % m)
     for name in sorted(DENSE):
-        per_config[name] = {"mode%d" % m: run_dense(name, m, args, traffic) for m in (8, 16)}
-    for name in sorted(CONVS):
-        policies = ("fp32",) if CONVS[name][7] == "f32" else ("full16", "backward32")
-        entry = {}
-        for pol in policies:
+        for m in (8, 16):
+            note(name, "fp32", m, run_dense(name, m, args, traffic))
+    # the longest-running records last: the tail of the output is what a log keeps
+    order = [n for n in sorted(CONVS) if "pw" in n and CONVS[n][7] == "f16"] + \
+            [n for n in sorted(CONVS) if "k3" in n and CONVS[n][7] == "f16"] + \
+            [n for n in sorted(CONVS) if CONVS[n][7] == "f32"]
+    head = None
+    for pol_pick in ("full16", "backward32", "fp32"):
+        for name in order:
+            if (CONVS[name][7] == "f32") != (pol_pick == "fp32"):
+                continue
             for m in (8, 16):
-                if name == HEADLINE and m == mode and pol == policy:
-                    rec = dict(head)
-                else:
-                    rec = run_conv(name, m, pol, args, traffic)
-                entry["%s_mode%d" % (pol, m)] = rec
-        per_config[name] = entry
-    c5 = {"mode%d" % m: run_resnet(m, "full16", args) for m in (mode, 24 - mode)}
-    extra = {"per_config": per_config, RESNET: c5,
-             "images_per_s_%s" % RESNET: c5["mode%d" % mode]["images_per_s"],
-             "ms_per_step_%s" % RESNET: c5["mode%d" % mode]["ms_per_step"]}
-    if not args.no_cpu_baseline:
-        head["cpu_baseline"] = cpu_baseline_conv(CONVS[HEADLINE], mode, args.cpu_seconds)
-    print(json.dumps(line(head, args, extra)))
+                rec = run_conv(name, m, pol_pick, args, traffic)
+                if name in sampled and m == mode and pol_pick in ("full16", "fp32") and not args.no_cpu_baseline:
+                    rec["cpu_baseline"] = cpu_baseline_conv(CONVS[name], m, 1.5, images=sampled[name])
+                if name == HEADLINE and m == mode and pol_pick == policy:
+                    head = rec
+                    if not args.no_cpu_baseline:
+                        head["cpu_baseline"] = cpu_baseline_conv(CONVS[HEADLINE], mode, args.cpu_seconds)
+                note(name, pol_pick, m, rec)
+    if head is None:  # a policy outside the table was asked for
+        head = run_conv(HEADLINE, mode, policy, args, traffic)
+        if not args.no_cpu_baseline:
+            head["cpu_baseline"] = cpu_baseline_conv(CONVS[HEADLINE], mode, args.cpu_seconds)
+        emit(head, HEADLINE, "%s_mode%d" % (policy, mode))
+    print(json.dumps({"record": "stale_profiles", "note": "kernel variants that ran without a row in "
+                      "profiles/hbm_traffic.md", "kernels": sorted(stale)}), flush=True)
+    extra = {"c5": {"images_per_s": c5[mode]["images_per_s"], "ms_per_step": c5[mode]["ms_per_step"],
+                    "images_per_s_other_mode": c5[24 - mode]["images_per_s"]},
+             "per_config": short, "stale_profiles": len(stale)}
+    print(line(head, args, extra))
     return 0
 
 

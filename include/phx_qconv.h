@@ -53,7 +53,10 @@ enum phx_data_format { PHX_NCHW = 0, PHX_NHWC = 1 };
  * COMPLEX and GA_300 run as one quaternion call on rearranged tensors: a GA_300 multivector (blades 1, e1, e2, e3,
  * e12, e13, e23, e123; src/algebras.cc:58-131) is A + e123 B with quaternion-like A = (m0, m4, m5, -m6) and
  * B = (m7, -m3, m2, m1), and (A1 + I B1)(A2 + I B2) = (A1 A2 - B1 B2) + I (A1 B2 + B1 A2), i.e. one quaternion
- * convolution of twice the channel counts; COMPLEX and REAL are embedded with zero components.  For these
+ * convolution of twice the channel counts.  COMPLEX and REAL run in place on grouped images -- two (four) images
+ * of the batch read as one quaternion image, q = z_A + conj(z_B) j, the filter relabelled to (u0, 0, u1, 0) /
+ * (w, 0, 0, 0) -- and fall back to an embedding with zero components only for batches that cannot be grouped
+ * (odd n; n not a multiple of 4 for REAL).  For these
  * algebras activations have dims * n batch rows (dims = 1, 2, 8), filters are [dims, co, ci, kh, kw] (Dense:
  * [dims, ni, no]), bias [dims, co]; NCHW, OIHW / IO, no groups, no real-valued input. */
 enum phx_algebra { PHX_QUATERNION = 0, PHX_REAL = 1, PHX_COMPLEX = 2, PHX_GA_300 = 3 };
@@ -132,6 +135,13 @@ int phx_init(void);
  * on first use) and forgets the cached plans.  Not to be called while another thread is inside a compute entry
  * point.  No counterpart in the reference, whose Context reads its switches once (src/backend/backend.cc:45-48). */
 int phx_tuning_reload(void);
+
+/* The plans (tile choice, reduction slices, packed-image sizes) are kept per distinct problem in a bounded,
+ * process-wide cache: a miss that finds more than 200 entries drops all but the 100 most recently used -- the
+ * policy of the reference's per-device operation cache (KEEP_TOP_100, src/backend/op_collections.cc:21-59;
+ * looked up per descriptor in src/backend/op_collections.hpp:121-144).  Reports the entries held now and the
+ * entries dropped so far; either pointer may be null.  Host-only. */
+int phx_plan_cache_stats(long* entries, long* evictions);
 
 /* The rearrangement that carries an algebra onto the quaternion kernels: `dims` blades, `halves` quaternion-like
  * parts; quaternion component p of half h is sign[h * 4 + p] * blade[h * 4 + p] (blade -1: the component is zero).

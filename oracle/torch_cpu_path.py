@@ -102,3 +102,73 @@ def conv2d_bwd(geom, x, w, grad, mode="factorized", need_dx=True):
             if need_dx:
                 dxs[left] -= bx
     return torch.stack(dws), (torch.cat(dxs) if need_dx else None)
+
+
+def _dense(x, w, b):
+    """Scalar Dense of the CPU backend: one matmul Y[N,O] = X[N,I] . W[I,O] (+ bias)
+    (src/backend/onednn/dense.hpp:53-93); torch.nn.functional.linear takes the filter as [O,I]."""
+    return F.linear(x, w.t(), b)
+
+
+def _dense_bwd(x, w, gr, need_dx):
+    """dW = X^T . G and dX = G . W^T through transposed views (src/backend/onednn/dense.hpp:166-181, 203-210)."""
+    dw = F.linear(x.t(), gr.t())
+    dx = F.linear(gr, w) if need_dx else None
+    return dw, dx
+
+
+def dense_fwd(x, w, bias=None, mode="factorized"):
+    """Quaternion Dense forward (src/dense.hpp:77-140 factorized, :143-180 generic).
+    x [4n,i], w [4,i,o] (layout IO), bias [4,o] or None (CPU float32 tensors)."""
+    n = x.shape[0] // 4
+    xs = [x[p * n:(p + 1) * n] for p in range(4)]
+    ws = [w[p] for p in range(4)]
+    if mode == "factorized":
+        L, R = decompose_left(xs), decompose_right(ws)
+        P = [_dense(L[i], R[i], bias[i - 4] if (bias is not None and i >= 4) else None) for i in range(8)]
+        a2 = P[0] + P[1] + P[2]
+        a5 = 0.5 * (a2 + P[3])
+        return torch.cat([a5 - P[0] + P[4], a5 - a2 + P[5], a5 - P[1] + P[6], a5 - P[2] + P[7]])
+    y = [None] * 4
+    for left, right, dim, positive, fill in product_terms(QUATERNION):
+        if fill:
+            y[dim] = _dense(xs[left], ws[right], bias[dim] if bias is not None else None)
+        else:
+            buf = _dense(xs[left], ws[right], None)
+            if positive:
+                y[dim] += buf
+            else:
+                y[dim] -= buf
+    return torch.cat(y)
+
+
+def dense_bwd(x, w, grad, mode="factorized", need_dx=True):
+    """Quaternion Dense backward (src/dense.hpp:252-335 factorized, :338-377 generic): returns (dw, dx)."""
+    n = x.shape[0] // 4
+    xs = [x[p * n:(p + 1) * n] for p in range(4)]
+    ws = [w[p] for p in range(4)]
+    gs = [grad[p * n:(p + 1) * n] for p in range(4)]
+    if mode == "factorized":
+        L, R, G = decompose_left(xs), decompose_right(ws), decompose_grad(gs)
+        dR, dL = zip(*[_dense_bwd(L[i], R[i], G[i], need_dx) for i in range(8)])
+        dw = torch.stack([dR[1] + dR[2] + dR[5] + dR[7], dR[0] + dR[3] + dR[5] - dR[7],
+                          dR[0] - dR[3] + dR[4] + dR[6], dR[1] - dR[2] - dR[4] + dR[6]])
+        dx = None
+        if need_dx:
+            dx = torch.cat([dL[1] + dL[2] + dL[5] + dL[6], dL[0] - dL[3] + dL[5] - dL[6],
+                            dL[2] - dL[1] - dL[4] + dL[7], dL[0] + dL[3] + dL[4] + dL[7]])
+        return dw, dx
+    dws, dxs = [None] * 4, [None] * 4
+    for left, right, dim, positive, fill in product_terms(QUATERNION, backprop=True):
+        bw, bx = _dense_bwd(xs[left], ws[right], gs[dim], need_dx)
+        if fill:
+            dws[right], dxs[left] = bw, bx
+        elif positive:
+            dws[right] += bw
+            if need_dx:
+                dxs[left] += bx
+        else:
+            dws[right] -= bw
+            if need_dx:
+                dxs[left] -= bx
+    return torch.stack(dws), (torch.cat(dxs) if need_dx else None)

@@ -29,7 +29,7 @@ EXPORTS = (
     "phx_device_count", "phx_device_malloc", "phx_device_free", "phx_memcpy_h2d", "phx_memcpy_d2h",
     "phx_memset_zero", "phx_stream_create", "phx_stream_destroy", "phx_stream_synchronize",
     "phx_last_kernel_name", "phx_profile_enable", "phx_profile_collect", "phx_algebra_map",
-    "phx_init", "phx_tuning_reload", "phx_qconv2d_fwd_noalloc",
+    "phx_init", "phx_tuning_reload", "phx_plan_cache_stats", "phx_qconv2d_fwd_noalloc",
     "phx_qconv2d_packed_filter_bytes", "phx_qconv2d_pack_filters", "phx_qconv2d_fwd_prepacked",
     "phx_qconv2d_bwd_data_prepacked",
     "phx_qconv2d_bwd_data_add",
@@ -141,9 +141,14 @@ def init():
     check(lib().phx_init(), "phx_init")
 
 
+tuning_generation = 0  # counts tuning_reload() calls: plans, and so packed filter layouts, may differ across one
+
+
 def tuning_reload():
     """Re-read the PHX_TUNE_* overrides and UPSTRIDE_VERBOSE from the environment (tests)."""
+    global tuning_generation
     check(lib().phx_tuning_reload(), "phx_tuning_reload")
+    tuning_generation += 1
 
 
 def profile_enable(capacity):

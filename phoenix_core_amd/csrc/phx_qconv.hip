@@ -68,7 +68,9 @@ static const Tuning& tune() {
 bool tuning_noearly() { return tune().noearly; }
 
 // Plans are pure functions of the problem and the tuning overrides; they are computed once per distinct
-// problem (the reference keeps its configured operations per descriptor, src/backend/op_collections.hpp:121-144).
+// problem (the reference keeps its configured operations per descriptor, src/backend/op_collections.hpp:121-144)
+// and kept in bounded memos: when a miss finds more than PLAN_MEMO_LIMIT entries, all but the PLAN_MEMO_KEEP most
+// recently used ones are dropped (the reference's KEEP_TOP_100 policy, src/backend/op_collections.cc:21-59).
 // (fixed-size keys: a lookup that hits allocates nothing)
 struct PlanKey {
     int v[24];
@@ -83,6 +85,46 @@ struct PlanKeyHash {
 };
 static std::mutex g_plan_mutex;
 static unsigned g_plan_generation = 0;  // bumped (under g_plan_mutex) when the tuning overrides are read again
+constexpr size_t PLAN_MEMO_LIMIT = 200, PLAN_MEMO_KEEP = 100;
+static std::atomic<long> g_plan_evictions{0};
+static long g_plan_memo_sizes[2] = {0, 0};  // entries of the forward / input-gradient and of the filter-gradient memo
+
+// One memo; every method is called with g_plan_mutex held.
+template <typename V>
+class PlanMemo {
+    struct Slot { V value; unsigned long used; };
+    std::unordered_map<PlanKey, Slot, PlanKeyHash> map_;
+    unsigned long clock_ = 0;
+    unsigned generation_ = 0;
+
+    void collect() {
+        if (map_.size() <= PLAN_MEMO_LIMIT) return;
+        std::vector<unsigned long> stamps;
+        stamps.reserve(map_.size());
+        for (const auto& kv : map_) stamps.push_back(kv.second.used);
+        std::nth_element(stamps.begin(), stamps.end() - PLAN_MEMO_KEEP, stamps.end());
+        const unsigned long oldest_kept = *(stamps.end() - PLAN_MEMO_KEEP);
+        for (auto it = map_.begin(); it != map_.end();) {
+            if (it->second.used < oldest_kept) { it = map_.erase(it); ++g_plan_evictions; }
+            else ++it;
+        }
+    }
+
+public:
+    // The entry of `key`, made by `make()` on a miss.
+    template <typename Make>
+    const V& get(const PlanKey& key, Make make) {
+        if (generation_ != g_plan_generation) { map_.clear(); generation_ = g_plan_generation; }
+        auto it = map_.find(key);
+        if (it == map_.end()) {
+            collect();
+            it = map_.emplace(key, Slot{make(), 0}).first;
+        }
+        it->second.used = ++clock_;
+        return it->second.value;
+    }
+    size_t size() const { return map_.size(); }
+};
 // Kernels that need more dynamic LDS than the default 64 KiB (see phx_launch.h)
 static std::vector<const void*>& big_lds_kernels() {
     static std::vector<const void*> v;
@@ -664,23 +706,21 @@ struct CorrPlan {
 };
 
 static bool plan_corr(const Corr& creal, int mode, bool f16mfma, Corr& c, FwdPlan& pl, int& pw) {
-    static std::unordered_map<PlanKey, CorrPlan, PlanKeyHash> memo;
+    static PlanMemo<CorrPlan> memo;
     static_assert(sizeof(Corr) == 22 * sizeof(int), "Corr is hashed as raw ints: no padding allowed");
     PlanKey key{};
     std::memcpy(key.v, &creal, sizeof(Corr));
     key.v[22] = mode;
     key.v[23] = f16mfma;
     std::lock_guard<std::mutex> lock(g_plan_mutex);
-    static unsigned generation = 0;
-    if (generation != g_plan_generation) { memo.clear(); generation = g_plan_generation; }
-    auto it = memo.find(key);
-    if (it == memo.end()) {
+    const CorrPlan& hit = memo.get(key, [&] {
         CorrPlan cp{};
         cp.ok = plan_corr_uncached(creal, mode, f16mfma, cp.c, cp.pl, cp.pw);
-        it = memo.emplace(key, cp).first;
-    }
-    c = it->second.c; pl = it->second.pl; pw = it->second.pw;
-    return it->second.ok;
+        return cp;
+    });
+    g_plan_memo_sizes[0] = (long)memo.size();
+    c = hit.c; pl = hit.pl; pw = hit.pw;
+    return hit.ok;
 }
 
 static int record_pwx_job(const PackArgs& pa, int map, int wco, int nsteps) {
@@ -713,7 +753,9 @@ static int run_pwx(const Problem& p, const Corr& c, const FwdPlan& pl, int map, 
     a.N = c.N; a.Cin = c.Cin; a.CinS = cin_mem; a.Cout = c.Cout; a.CoutS = cout_mem; a.HW = c.Win;
     a.GI = cdiv(c.Win, 8); a.TGp = c.N * a.GI;
     a.co_tiles = pl.co_tiles; a.nsteps = pl.pwx_steps;
-    if (map == MAP_DGRAD && g_addend.ptr && out == g_addend.dx && !g_addend.fused) {
+    // (a grouped convolution runs this once per group on a channel slice: only an ungrouped call covers the whole
+    // addend with one launch, the groups leave it to the separate pass)
+    if (map == MAP_DGRAD && g_addend.ptr && out == g_addend.dx && !g_addend.fused && p.groups == 1) {
         a.addend = static_cast<const _Float16*>(g_addend.ptr);
         g_addend.fused = true;
     }
@@ -1081,21 +1123,19 @@ static bool wgrad_on_f16_mfma(const Problem& p) {
 
 static bool plan_wgrad(const Problem& p, bool f16mfma, WgPlan& best) {
     struct Entry { WgPlan pl; bool ok; };
-    static std::unordered_map<PlanKey, Entry, PlanKeyHash> memo;
+    static PlanMemo<Entry> memo;
     // everything the two planners read
     const PlanKey key{{p.mode, p.n, p.ci, p.co, p.h, p.w, p.kh, p.kw, p.sh, p.sw, p.dh, p.dw, p.pt, p.pl, p.pb, p.pr,
                        p.ho, p.wo, (int)f16mfma, (int)p.real_input, (int)p.dtype, p.groups, (int)p.nhwc}};
     std::lock_guard<std::mutex> lock(g_plan_mutex);
-    static unsigned generation = 0;
-    if (generation != g_plan_generation) { memo.clear(); generation = g_plan_generation; }
-    auto it = memo.find(key);
-    if (it == memo.end()) {
+    const Entry& hit = memo.get(key, [&] {
         Entry e{};
         e.ok = f16mfma ? plan_wgrad_f16(p, e.pl) : plan_wgrad_f32(p, e.pl);
-        it = memo.emplace(key, e).first;
-    }
-    best = it->second.pl;
-    return it->second.ok;
+        return e;
+    });
+    g_plan_memo_sizes[1] = (long)memo.size();
+    best = hit.pl;
+    return hit.ok;
 }
 
 static int run_wgrad(const Problem& p, hipStream_t st, const void* x, const void* g, void* dw, void* ws,
@@ -1467,6 +1507,13 @@ const char* phx_status_string(int status) {
 const char* phx_last_kernel_name(void) { return g_last_kernel; }
 
 int phx_init(void) { return device_state(nullptr); }
+
+int phx_plan_cache_stats(long* entries, long* evictions) {
+    std::lock_guard<std::mutex> lock(g_plan_mutex);
+    if (entries) *entries = g_plan_memo_sizes[0] + g_plan_memo_sizes[1];
+    if (evictions) *evictions = g_plan_evictions.load();
+    return PHX_OK;
+}
 
 int phx_tuning_reload(void) {
     std::lock_guard<std::mutex> lock(g_plan_mutex);

@@ -46,6 +46,10 @@ def _current_stream(device):
     return s
 
 
+def _capturing():
+    return torch.cuda.is_current_stream_capturing()
+
+
 _events = {}
 
 
@@ -183,6 +187,7 @@ class QConv2d(nn.Module):
         since: in-place updates are seen by the tensor's version counter, replaced storage by its address."""
         if not PREPACK_FILTERS:
             return None
+        packed_ahead = self._pack_pending  # repack_filters() has packed this step's images on the second stream
         if self._pack_pending:
             _current_stream(self.weight.device).wait_event(self._pack_event)
             self._pack_pending = False
@@ -191,7 +196,10 @@ class QConv2d(nn.Module):
         ent = self._packed.get(key)
         if ent is None:
             ent = self._packed[key] = [state, ops.conv2d_pack_filters(w.detach(), fwd, bwd_data=self.input_requires_grad)]
-        elif ent[1] is not None and ent[0] != state:
+        elif ent[1] is not None and (ent[0] != state or (_capturing() and not packed_ahead)):
+            # Under stream capture the check above runs once, at capture time, while the graph is replayed after
+            # every later update of the filter: the packing launch has to be part of the graph whether or not the
+            # filter has changed since the last call.
             ops.conv2d_pack_filters(w.detach(), fwd, into=ent[1])
             ent[0] = state
         return ent[1]
@@ -201,8 +209,9 @@ class QConv2d(nn.Module):
         w = self.weight
         state = (w._version, w.data_ptr())
         packed = False
+        capturing = _capturing()  # (a captured step packs unconditionally: see _packed_filters)
         for key, ent in self._packed.items():
-            if ent[1] is not None and ent[0] != state:
+            if ent[1] is not None and (ent[0] != state or capturing):
                 ops.conv2d_pack_filters(w.detach(), self._descs[key][0], into=ent[1])
                 ent[0] = state
                 packed = True

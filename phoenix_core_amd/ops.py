@@ -292,8 +292,24 @@ class PackedFilters:
     `packed` argument instead of packing in every call.  Either image may be None (no prepacked form for that
     pass, or not asked for)."""
 
-    def __init__(self, fwd, bwd_data, filter_shape, dtype):
+    def __init__(self, fwd, bwd_data, filter_shape, dtype, layout_key=None):
         self.fwd, self.bwd_data, self.filter_shape, self.dtype = fwd, bwd_data, tuple(filter_shape), dtype
+        self.layout_key = layout_key
+
+    def check(self, desc):
+        """The images' layout follows the plan of the descriptor they were packed for (sizes, strides, padding,
+        product mode, policy, groups, data format) under the tuning in force then: any other descriptor is refused."""
+        if self.filter_shape != tuple(desc.filter_shape) or self.dtype != desc.dtype or \
+                (self.layout_key is not None and self.layout_key != _layout_key(desc)):
+            raise ValueError("these packed filters belong to another descriptor")
+
+
+def _layout_key(desc):
+    """Everything of a descriptor that a packed image depends on: its C struct without the bias flag (the forward
+    and backward descriptors of one layer differ in it and share their images) + the tuning generation."""
+    c = capi.QConvDesc.from_buffer_copy(bytes(desc.c))
+    c.has_bias = 0
+    return bytes(c), capi.tuning_generation
 
 
 def conv2d_packed_filter_bytes(desc, which):
@@ -315,9 +331,10 @@ def conv2d_pack_filters(w, desc, bwd_data=True, into=None):
         if nf == 0 and nb == 0:
             return None
         into = PackedFilters(torch.empty(nf, dtype=torch.uint8, device=dev) if nf else None,
-                             torch.empty(nb, dtype=torch.uint8, device=dev) if nb else None, desc.filter_shape, desc.dtype)
-    elif into.filter_shape != tuple(desc.filter_shape) or into.dtype != desc.dtype:
-        raise ValueError("these packed filters belong to another descriptor")
+                             torch.empty(nb, dtype=torch.uint8, device=dev) if nb else None, desc.filter_shape, desc.dtype,
+                             _layout_key(desc))
+    else:
+        into.check(desc)
     f, b = into.fwd, into.bwd_data
     capi.check(capi.lib().phx_qconv2d_pack_filters(ctypes.byref(desc.c), _stream(dev), _ptr(w), _ptr(f), f.numel() if f is not None else 0,
                                                    _ptr(b), b.numel() if b is not None else 0), "phx_qconv2d_pack_filters")
@@ -340,8 +357,7 @@ def conv2d_fwd(x, w, bias, desc, out=None, packed=None):
     nbytes = desc.workspace_bytes(capi.PHX_PASS_FWD)
     ws = _workspace.get(dev, nbytes)
     if packed is not None and packed.fwd is not None:
-        if packed.filter_shape != tuple(desc.filter_shape) or packed.dtype != desc.dtype:
-            raise ValueError("these packed filters belong to another descriptor")
+        packed.check(desc)
         capi.check(capi.lib().phx_qconv2d_fwd_prepacked(ctypes.byref(desc.c), _stream(dev), _ptr(x), _ptr(packed.fwd),
                                                         packed.fwd.numel(), _ptr(bias if desc.use_bias else None), _ptr(y),
                                                         _ptr(ws), nbytes), "phx_qconv2d_fwd_prepacked")
@@ -382,15 +398,14 @@ def conv2d_bwd_data(w, grad, desc, packed=None, addend=None):
     if addend is not None:
         _expect(addend, desc.input_shape, desc.dtype, "addend")
         image = packed.bwd_data if packed is not None else None
-        if image is not None and (packed.filter_shape != tuple(desc.filter_shape) or packed.dtype != desc.dtype):
-            raise ValueError("these packed filters belong to another descriptor")
+        if image is not None:
+            packed.check(desc)
         capi.check(capi.lib().phx_qconv2d_bwd_data_add(ctypes.byref(desc.c), _stream(dev), _ptr(grad), _ptr(w), _ptr(image),
                                                        image.numel() if image is not None else 0, _ptr(addend), _ptr(dx),
                                                        _ptr(ws), nbytes), "phx_qconv2d_bwd_data_add")
         return dx
     if packed is not None and packed.bwd_data is not None:
-        if packed.filter_shape != tuple(desc.filter_shape) or packed.dtype != desc.dtype:
-            raise ValueError("these packed filters belong to another descriptor")
+        packed.check(desc)
         capi.check(capi.lib().phx_qconv2d_bwd_data_prepacked(ctypes.byref(desc.c), _stream(dev), _ptr(grad), _ptr(packed.bwd_data),
                                                              packed.bwd_data.numel(), _ptr(dx), _ptr(ws), nbytes),
                    "phx_qconv2d_bwd_data_prepacked")

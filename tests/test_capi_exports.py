@@ -103,3 +103,26 @@ def test_python_context_matches_oracle_env_rules():
             want = oracle.env_fp16_policy(pol)
             assert ctx.is_fp16_conv_forward_allowed() == (want in ("full16", "backward32"))
             assert ctx.is_fp16_conv_backward_allowed() == (want == "full16")
+
+
+def test_plan_cache_is_bounded():
+    """Plans are memoized per distinct problem; the memo drops all but the 100 most recently used entries once a miss
+    finds more than 200 (the reference's operation cache does the same, src/backend/op_collections.cc:21-59), and a
+    problem that was dropped is simply planned again with the same result."""
+    L = capi.lib()
+    L.phx_plan_cache_stats.argtypes = [ctypes.POINTER(ctypes.c_long), ctypes.POINTER(ctypes.c_long)]
+    entries, evictions = ctypes.c_long(), ctypes.c_long()
+    first = capi.QConvDesc(1, 2, 16, 16, 20, 20, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 0, 8, 2, 0)
+    want = [L.phx_qconv2d_workspace_bytes(ctypes.byref(first), which) for which in (0, 1, 2)]
+    assert all(v > 0 for v in want)
+    assert L.phx_plan_cache_stats(ctypes.byref(entries), ctypes.byref(evictions)) == 0
+    dropped_before = evictions.value
+    for h in range(8, 8 + 700):
+        d = capi.QConvDesc(1, 2, 16, 16, h, 24, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 0, 8, 2, 0)
+        for which in (0, 1, 2):
+            assert L.phx_qconv2d_workspace_bytes(ctypes.byref(d), which) > 0
+        L.phx_plan_cache_stats(ctypes.byref(entries), None)
+        assert entries.value <= 2 * 201, entries.value  # two memos (forward / input gradient, filter gradient)
+    L.phx_plan_cache_stats(ctypes.byref(entries), ctypes.byref(evictions))
+    assert evictions.value > dropped_before
+    assert [L.phx_qconv2d_workspace_bytes(ctypes.byref(first), which) for which in (0, 1, 2)] == want

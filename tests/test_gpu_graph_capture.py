@@ -55,3 +55,45 @@ def test_captured_conv_replays_match_eager(dtype, policy):
         y1 = phx.conv2d_fwd(x, w, None, desc)
         torch.cuda.synchronize()
         assert torch.equal(y1, y0)
+
+
+def test_captured_layer_packs_its_filter_inside_the_graph():
+    """nn.QConv2d keeps its filter packed and repacks when the tensor has changed -- a host-side check made at call
+    time.  A captured step is replayed after every later update, so the packing launch must be in the graph even
+    when the filter had not changed between warm-up and capture: replays after in-place updates of the weights
+    are held against an eager layer on the same weights."""
+    capi.init()
+    torch.manual_seed(5)
+    ctx = Ctx(8, "full16")
+    layer = phx.QConv2d(16, 32, 3, padding="SAME", dtype=torch.float16, context=ctx).cuda()
+    x = (0.5 * torch.randn(8, 16, 14, 14, device="cuda")).half().requires_grad_(True)
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        for _ in range(2):  # warm-up: packs once, the second call finds the filter unchanged
+            layer(x).float().sum().backward()
+    side.synchronize()
+    x.grad = None
+    layer.zero_grad(set_to_none=True)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        y = layer(x)
+        y.float().square().sum().backward()
+    dx, dw = x.grad, layer.weight.grad
+    for replay in range(3):
+        with torch.no_grad():
+            layer.weight.mul_(0.5).add_(0.01 * (replay + 1))  # "optimizer step" between replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in (y, dx, dw)]
+        # eager layer with the same, current weights (prepacked images bypassed)
+        desc = phx.Conv2DDescriptor(x.shape, layer.weight.shape, 1, 1, "SAME", dtype=torch.float16, context=ctx)
+        y1 = phx.conv2d_fwd(x.detach(), layer.weight.detach(), layer.bias.detach() if layer.bias is not None else None,
+                            phx.Conv2DDescriptor(x.shape, layer.weight.shape, 1, 1, "SAME", dtype=torch.float16, context=ctx,
+                                                 use_bias=layer.bias is not None))
+        gy = (2.0 * y1.float()).half()
+        dw1, dx1 = phx.conv2d_bwd(x.detach(), layer.weight.detach(), gy, desc)
+        torch.cuda.synchronize()
+        assert torch.equal(got[0], y1), "forward of replay %d ran on a stale packed filter" % replay
+        assert torch.equal(got[1], dx1), "input gradient of replay %d ran on a stale packed filter" % replay
+        assert torch.equal(got[2], dw1)

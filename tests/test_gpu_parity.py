@@ -362,6 +362,7 @@ GROUPED = [
     ("g2_k5_ragged", 2, 1, 10, 6, 11, 12, 5, 5, 1, 2, (2, 1, 3, 0)),
     ("depthwise_k3", 8, 2, 8, 8, 10, 10, 3, 3, 1, 1, "SAME"),
     ("g2_wide", 2, 1, 96, 160, 7, 7, 1, 1, 1, 1, "VALID"),
+    ("g2_pw_even", 2, 2, 32, 32, 8, 8, 1, 1, 1, 1, "VALID"),  # even planes: the fp16 streaming kernel, once per group
 ]
 
 
@@ -779,7 +780,7 @@ def test_prepacked_filters_give_the_plain_result(case, mode, dtype, policy):
 
 
 @pytest.mark.parametrize("mode", [16, 8])
-@pytest.mark.parametrize("case", [c for c in GROUPED if c[0] in ("g2_k3", "g4_pw", "g3_k3_s2", "depthwise_k3")] +
+@pytest.mark.parametrize("case", [c for c in GROUPED if c[0] in ("g2_k3", "g4_pw", "g3_k3_s2", "depthwise_k3", "g2_pw_even")] +
                          [c[:1] + (1,) + c[4:] for c in CHANNELS_LAST if c[0] in ("nhwc_pw", "nhwc_k3", "nhwc_pw_c40_24")],
                          ids=lambda c: c[0])
 def test_prepacked_filters_grouped_and_channels_last(case, mode):
@@ -806,6 +807,10 @@ def test_prepacked_filters_grouped_and_channels_last(case, mode):
     assert torch.equal(ops.conv2d_bwd_data(wd, gd, desc, packed=packed), dx), "prepacked dgrad " + name
     addend = xd.flip(0) * 0.75
     assert torch.equal(ops.conv2d_bwd_data(wd, gd, desc, packed=packed, addend=addend), dx + addend), "dgrad + addend " + name
+    if name == "g2_pw_even":
+        # every group's slice of the addend must arrive: the streaming kernel runs per group and none of its launches
+        # covers the whole tensor, so the addition is the separate pass
+        assert "pwx" in capi.last_kernel_name() and not capi.last_kernel_name().endswith("_add"), capi.last_kernel_name()
 
 
 @pytest.mark.parametrize("mode", [16, 8])
@@ -849,6 +854,22 @@ def test_prepacked_filters_are_refused_where_they_do_not_apply():
     other = phx.Conv2DDescriptor((8, 8, 6, 6), (4, 8, 8, 1, 1), 1, 1, "SAME", context=Ctx(8))
     with pytest.raises(ValueError):
         phx.conv2d_fwd(torch.zeros(8, 8, 6, 6, device="cuda"), torch.zeros(4, 8, 8, 1, 1, device="cuda"), None, other, packed=packed)
+    # the same filter shape under another descriptor: another input size, stride, product mode or policy may mean
+    # another plan and so another image layout -- refused whatever the plans turn out to be
+    for args, kw in ((((8, 8, 12, 12), wd.shape, 1, 1, "SAME"), dict(context=Ctx(8))),
+                     (((8, 8, 6, 6), wd.shape, 2, 1, "SAME"), dict(context=Ctx(8))),
+                     (((8, 8, 6, 6), wd.shape, 1, 1, "SAME"), dict(context=Ctx(16))),
+                     (((8, 8, 6, 6), wd.shape, 1, 1, "VALID"), dict(context=Ctx(8)))):
+        d2 = phx.Conv2DDescriptor(*args, **kw)
+        with pytest.raises(ValueError):
+            phx.conv2d_fwd(torch.zeros(d2.input_shape, device="cuda"), wd, None, d2, packed=packed)
+        with pytest.raises(ValueError):
+            ops.conv2d_bwd_data(wd, torch.zeros(d2.output_shape, device="cuda"), d2, packed=packed)
+        with pytest.raises(ValueError):
+            ops.conv2d_pack_filters(wd, d2, into=packed)
+    # ... while the backward descriptor of the same layer (no bias flag) shares the images of the forward one
+    with_bias = phx.Conv2DDescriptor((8, 8, 6, 6), wd.shape, 1, 1, "SAME", use_bias=True, context=Ctx(8))
+    ops.conv2d_bwd_data(wd, torch.zeros(desc.output_shape, device="cuda"), desc, packed=ops.conv2d_pack_filters(wd, with_bias))
     # an image smaller than the descriptor needs
     L = capi.lib()
     x = torch.zeros(8, 8, 6, 6, device="cuda")

@@ -27,3 +27,27 @@ def test_torch_cpu_path_matches_oracle(cfg, mode):
     want_dw, want_dx = oracle.conv2d_bwd(g, x, w, gr, "hamilton")
     for got, want in ((y, want_y), (dw.numpy(), want_dw), (dx.numpy(), want_dx)):
         assert np.abs(got - want).max() / np.abs(want).max() < 1e-5
+
+
+@pytest.mark.parametrize("mode", ["factorized", "generic"])
+@pytest.mark.parametrize("shape", [(3, 5, 7), (32, 128, 128)])
+@pytest.mark.parametrize("use_bias", [False, True])
+def test_torch_cpu_dense_path_matches_oracle(shape, mode, use_bias):
+    """The Dense port (8 / 16 scalar matmuls by torch's CPU backend + lane maps) against the C oracle in fp64,
+    ragged sizes and the benchmark's 32 x 128 -> 128 layer."""
+    n, ni, no = shape
+    r = np.random.default_rng(11)
+    x = r.standard_normal((4 * n, ni)).astype(np.float32)
+    w = r.standard_normal((4, ni, no)).astype(np.float32)
+    b = r.standard_normal((4, no)).astype(np.float32) if use_bias else None
+    gr = r.standard_normal((4 * n, no)).astype(np.float32)
+    tb = torch.from_numpy(b) if use_bias else None
+    y = tcp.dense_fwd(torch.from_numpy(x), torch.from_numpy(w), tb, mode).numpy()
+    dw, dx = tcp.dense_bwd(torch.from_numpy(x), torch.from_numpy(w), torch.from_numpy(gr), mode)
+    want_y = oracle.dense_fwd(x, w, b, "generic")
+    want_dw, want_dx = oracle.dense_bwd(x, w, gr, "generic")
+    for got, want in ((y, want_y), (dw.numpy(), want_dw), (dx.numpy(), want_dx)):
+        assert got.shape == want.shape
+        assert np.abs(got - want).max() / np.abs(want).max() < 2e-5
+    dw2, dx2 = tcp.dense_bwd(torch.from_numpy(x), torch.from_numpy(w), torch.from_numpy(gr), mode, need_dx=False)
+    assert dx2 is None and torch.equal(dw2, dw)
