@@ -300,6 +300,26 @@ __device__ __forceinline__ void lds_dma_16(const void* gsrc, void* ldst) {
 
 __device__ __forceinline__ void wait_vmem_all() { __builtin_amdgcn_s_waitcnt(0x0F70); }  // vmcnt(0)
 
+// The copies into LDS and the workgroup barrier of the kernels that keep copies in flight across barriers, kept out of the compiler's memory model.
+// __syncthreads() carries workgroup-scope fences, in front of which the compiler waits for EVERY outstanding
+// vector memory operation (s_waitcnt vmcnt(0)), and it puts the same wait in front of LDS reads that may alias an
+// LDS write by a global_load_lds it knows of -- either way the copies of the steps ahead, which a ring of stages
+// exists to keep in flight across the barrier, would be drained at every step.  So the copy is issued from inline
+// assembly (the compiler then counts nothing for it: the kernels wait for their copies with explicit s_waitcnt
+// vmcnt(n); the compiler's own waits for the loads it does know of stay correct, extra operations in flight can
+// only make them longer), and the barrier is the bare instruction behind a wait for this wave's LDS operations.
+__device__ __forceinline__ void lds_dma_16_untracked(const void* gsrc, void* ldst) {
+    const unsigned int lds_addr = (unsigned int)(unsigned long)(__attribute__((address_space(3))) void*)ldst;
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                 :
+                 : "v"(gsrc), "s"(lds_addr)
+                 : "memory");  // (m0 is a reserved register: it cannot be named as clobbered, and nothing else here uses it)
+}
+__device__ __forceinline__ void wg_barrier_no_vmem_wait() {
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+
 // Chunk staging of the activation window (CHUNKS): the window is NB*HTH rows of HTW positions, HTW a
 // multiple of 8.  One task = (component, 8-channel pack, 8 consecutive positions of a row): eight
 // 16-byte loads (one per channel, 2-byte aligned), an 8x8 transpose with byte permutes, eight 16-byte

@@ -7,26 +7,30 @@
 //     exactly as they lie in NCHW memory -- rows of (component, channel) x consecutive pixels, no transposition,
 //     no masks, no staging registers; a ring of stages (one 16-channel K step each) keeps the copies ahead of the
 //     matrix instructions (one step here, two in the channels-last kernel), one barrier per step;
-//   * the MFMA B operand wants 8 consecutive channels of one pixel per lane, NCHW has 8 consecutive pixels of one
-//     channel: the transposition happens on the way from LDS to the registers.  A lane owns TWO neighbouring
-//     pixels: it reads one dword (two pixels) per channel, and byte permutes split the eight dwords of a channel
-//     pack into the two operands (one v_perm per matrix instruction);
+//   * the MFMA A operand wants 8 consecutive channels of one pixel per lane, NCHW has consecutive pixels of one
+//     channel: the transposition happens on the way from LDS to the registers, by the transposing LDS read of
+//     gfx950 (ds_read_b64_tr_b16): sixteen lanes hand in the addresses of sixteen 8-byte runs -- four pixel quads
+//     of each of four channel rows -- and lane i receives pixel i of the sixteen with its four channels.  Two
+//     such reads are one matrix operand: no vector arithmetic touches the data on its way in.  The 16-byte pieces
+//     of a staged row are stored XOR-swizzled by the row number (the copy lanes choose which piece of global
+//     memory they fetch), so that the four rows of a read fall into four different bank groups;
 //   * the activations are the A operand of the matrix instruction (rows = pixels) and the filters the B operand
-//     (columns = output channels), so a lane receives, for ONE output channel, eight consecutive pixels per group
-//     of four accumulator registers (the two pixels of its pair x four row registers interleave exactly so): one
-//     16-byte store per group, no cross-lane shuffle;
-//   * stored like that, the 64 lanes of a store instruction would write 32 channel rows x 32 bytes: four
-//     instructions to complete a 128-byte line, and the address path handles a line at a time.  So a wave passes
-//     each component's 4 KB through a small LDS buffer of its own ([channel][8-pixel piece], rows padded by one
-//     piece against bank conflicts) and reads it back with the lanes along the pixels: a store instruction then
-//     writes 8 channel rows x 128 bytes (WCO > 1; the 256-pixel tiles of WCO == 1 have no LDS to spare);
+//     (columns = output channels), so a lane receives, for ONE output channel, four consecutive pixels per group
+//     of four accumulator registers;
+//   * stored like that, the 64 lanes of a store instruction would write 32 channel rows x 16 bytes.  So a wave
+//     passes each component's 4 KB through a small LDS buffer of its own ([channel][8-pixel piece], rows padded by
+//     one piece against bank conflicts) and reads it back with the lanes along the pixels: a store instruction then
+//     writes 8 channel rows x 128 bytes (WCO > 1; the 256-pixel tiles of WCO == 1 have no LDS to spare and store
+//     their quads directly);
 //   * a wave owns 32 output channels x 64 pixels x 4 output components = 8 accumulator tiles (128 registers),
 //     so two workgroups fit a CU and one's stores and start-up run under the other's products;
 //   * pixels are addressed in groups of 8 (one 16-byte copy lane); an image whose plane is not a multiple of 8
 //     pixels has its last group moved back to end at the plane's end (a few pixels are computed twice, with the
 //     same result), so no copy ever leaves its row and no lane needs a mask;
 //   * workgroups are persistent: each walks over (pixel tile, output-channel tile) items, the copy ring running on
-//     across item boundaries.
+//     across item boundaries.  Where the items do not divide among the workgroups and the last round would keep
+//     at most half of them busy, the items of that round are cut in two along the pixels (half items: one of the
+//     two 32-pixel column tiles of every wave), so that the round costs half an item instead of a whole one.
 // Requirements (checked on the host): fp16 tensors, all four components present, plane size even and >= 8.
 #pragma once
 
@@ -40,6 +44,19 @@ namespace phx {
 __device__ __forceinline__ u32x4 add_halves(const u32x4& a, const u32x4& b) {
     const f16x8 s = __builtin_bit_cast(f16x8, a) + __builtin_bit_cast(f16x8, b);
     return __builtin_bit_cast(u32x4, s);
+}
+__device__ __forceinline__ u32x2 add_halves4(const u32x2& a, const u32x2& b) {
+    const f16x4 s = __builtin_bit_cast(f16x4, a) + __builtin_bit_cast(f16x4, b);
+    return __builtin_bit_cast(u32x2, s);
+}
+
+// The transposing LDS read (ds_read_b64_tr_b16).  Within each group of sixteen lanes, lane s hands in the address
+// of four consecutive halves M[s][0..3]; lane i receives M[4r + i/4][i%4] for r = 0..3.
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ f16x4 lds_read_tr16(const void* lds_base, unsigned int byte_offset) {
+    const auto p = reinterpret_cast<__attribute__((address_space(3))) s16x4*>(
+        (__attribute__((address_space(3))) char*)lds_base + byte_offset);
+    return __builtin_bit_cast(f16x4, __builtin_amdgcn_ds_read_tr16_b64_v4i16(p));
 }
 
 struct PwxArgs {
@@ -55,7 +72,8 @@ struct PwxArgs {
     int TGp;                // groups in all: N * GI
     int co_tiles;           // ceil(Cout / (32 * WCO))
     int nsteps;             // ceil(Cin / 16)
-    int items;              // pixel tiles * co_tiles
+    int items;              // work items: whole items (pixel tiles * co_tiles), the last ones possibly as pairs of half items
+    int items_whole;        // NCHW kernel: work items below this index are whole items, the others half items
     int NP;                 // channels-last kernel: pixels in all, N * HW
 };
 
@@ -72,12 +90,17 @@ struct PwxShape {
     static constexpr int NXI = 2 * WPX;          // activation copy instructions per wave and stage
     static constexpr int NPS = NWI + NXI;
     static constexpr size_t lds_bytes = (size_t)R * SV * 16;
-    // NCHW kernel: a ring of two stages does as well as three (a K step is bound by the copy instructions' issue
-    // and the barrier, not by the copies' latency), which leaves room for the store transposition below
+    // NCHW kernel: the filters (from L2: short latency) go through a ring of two stages, one K step ahead of the
+    // products; the activations (from HBM) through a ring of their own, two steps ahead where LDS has the room
+    // (WCO == 4: 32 + 24 KiB of rings + 18 KiB of store transposition, two workgroups per CU)
     static constexpr bool TSTORE = WCO > 1;      // stores regrouped through LDS into whole channel rows
-    static constexpr int RN = 2;
+    static constexpr int RF = 2;                 // filter stages
+    static constexpr int RA = (WCO == 4) ? 3 : 2;  // activation stages
     static constexpr int SCRV = 32 * 9;          // 16-byte vectors of a wave's transposition buffer: 32 channels x (8 + 1) pieces
-    static constexpr size_t lds_bytes_nchw = (size_t)RN * SV * 16 + (TSTORE ? 4 * SCRV * 16 : 0);
+    static constexpr size_t lds_bytes_nchw = ((size_t)RF * WV + (size_t)RA * XV + (TSTORE ? 4 * SCRV : 0)) * 16;
+    // swizzle of the 16-byte pieces of staged activation row `row`: slot s of the row holds piece s ^ swz(row)
+    // (four consecutive rows, read together by sixteen lanes, then lie in four different quarters of the 64 banks)
+    __host__ __device__ static constexpr int swz(int row) { return WPX == 1 ? 4 * ((row >> 1) & 1) : 4 * (row & 3); }
 };
 
 // ADD: the instance that adds P.addend to what it stores (the plain instance carries none of that code: the extra
@@ -85,8 +108,10 @@ struct PwxShape {
 template <int WCO, bool ADD = false>
 __global__ void __launch_bounds__(WG_THREADS, 2) qconv_pwx_f16_kernel(const PwxArgs P) {
     using S = PwxShape<WCO>;
-    constexpr int WPX = S::WPX, GPT = S::GPT, ROWDW = S::ROWDW, WV = S::WV, SV = S::SV, R = S::RN, D = R - 1;
-    constexpr int RPI = 64 / GPT;  // activation rows one copy instruction covers
+    constexpr int WPX = S::WPX, GPT = S::GPT, ROWDW = S::ROWDW, WV = S::WV, XV = S::XV, RF = S::RF, RA = S::RA;
+    constexpr int DF = RF - 1, DA = RA - 1;  // steps the filter / activation copies run ahead of the products
+    constexpr int RPI = 64 / GPT;      // activation rows one copy instruction covers
+    constexpr int PITCH = ROWDW * 4;   // bytes of a staged activation row
     constexpr bool TSTORE = S::TSTORE;
     extern __shared__ f16x8 lds16[];
 
@@ -100,223 +125,301 @@ __global__ void __launch_bounds__(WG_THREADS, 2) qconv_pwx_f16_kernel(const PwxA
     // tiles of one pixel tile read the same activations -- both should meet in one L2.
     const int wg = xcd_remap(blockIdx.x, gridDim.x);
 
-    // ---- copy side: a lane always copies the same pixel group of the tile (64 % GPT == 0)
-    const int g_l = lane % GPT, rl = lane / GPT;
+    // work item i -> (whole item index, half): half < 0 for a whole item, else the column tile (0 / 1) it is cut down to
+    auto decode = [&](int i, int& item, int& half) {
+        if (i < P.items_whole) { item = i; half = -1; }
+        else { item = P.items_whole + ((i - P.items_whole) >> 1); half = (i - P.items_whole) & 1; }
+    };
+
+    // ---- copy side: a lane always fills the same slot (row rl of its instruction's rows, slot s_l of that row), i.e.
+    // copies the same pixel group of the tile: piece s_l ^ swz(row), and row % 4 does not depend on the instruction.
+    // Two cursors run ahead of the products: the filters' (DF steps ahead) and the activations' (DA steps).
+    f16x8* const fring = lds16;
+    f16x8* const aring = lds16 + RF * WV;
+    const int rl = lane / GPT;
+    const int g_l = (lane % GPT) ^ S::swz(wave * RPI + rl);
     long xoff = 0;       // element offset of this lane's group inside a component (channel 0)
     bool xok = false;
-    int p_item = wg, p_k = 0, p_ct = 0;  // item / K step / channel tile the next copy belongs to
-    auto locate_copy = [&](int item) {
+    int pa_item = wg, pa_k = 0;            // work item / K step of the next activation copies
+    int pf_item = wg, pf_k = 0, pf_ct = 0; // ... of the next filter copies, and their channel tile
+    auto locate_act = [&](int i) {
+        int item, half;
+        decode(i, item, half);
         const int tile = item / P.co_tiles;
-        p_ct = item - tile * P.co_tiles;
         const int gg = tile * GPT + g_l;
-        xok = item < P.items && gg < P.TGp;
+        xok = i < P.items && gg < P.TGp;
         const int n = gg / P.GI, gi = gg - n * P.GI;
         const int off = min(gi * 8, HW - 8);  // the last group of a plane ends at the plane's end
         xoff = xok ? ((long)n * P.CinS) * HW + off : 0;
     };
-    // The copies of one stage, (p_item, p_k) -> ring buffer buf, as NPS separate "slots": a wave that issues its
-    // copies back to back stalls until the memory pipeline has taken them all, so the product loop deals them out
-    // between its matrix instructions.  The last slot moves on to the next K step / item.
-    auto issue_slot = [&](int buf, int slot) {
-        f16x8* sb = lds16 + buf * SV;
+    auto locate_filter = [&](int i) {
+        int item, half;
+        decode(i, item, half);
+        pf_ct = item % P.co_tiles;
+    };
+    // The copies of one step as NPS separate "slots" -- filters of the step DF ahead into filter stage fbuf, then
+    // activations of the step DA ahead into activation stage abuf: a wave that issues its copies back to back stalls
+    // until the memory pipeline has taken them all, so the product loop deals them out between its matrix
+    // instructions.  The last slot of each kind moves its cursor on.  (A half item copies the whole tile: its twin
+    // reads the other half of the same stage in another workgroup.)  The cursors run on past the last item -- filters
+    // of some valid tile, zeros for activations, into stages nobody reads again -- so that every step issues the same
+    // copies, without branches between the matrix instructions, and the waits can count them.
+    auto issue_slot = [&](int fbuf, int abuf, int slot) {
         if (slot < S::NWI) {
             const int t = wave + 4 * slot;
-            const f16x8* wsrc = P.wpk + ((long)p_ct * P.nsteps + p_k) * WV;
-            lds_dma_16(wsrc + t * 64 + lane, sb + t * 64);
+            const f16x8* wsrc = P.wpk + ((long)pf_ct * P.nsteps + pf_k) * WV;
+            lds_dma_16_untracked(wsrc + t * 64 + lane, fring + fbuf * WV + t * 64);
+            if (slot == S::NWI - 1 && ++pf_k == P.nsteps) {
+                pf_k = 0;
+                pf_item += gridDim.x;
+                locate_filter(pf_item);
+            }
         } else {
             const int t = wave + 4 * (slot - S::NWI);
-            const int r = t * RPI + rl, p = r >> 4, ch = p_k * 16 + (r & 15);
+            const int r = t * RPI + rl, p = r >> 4, ch = pa_k * 16 + (r & 15);
             // channels past the tensor meet zero filters; they, and groups past the last image, copy zeros
             const _Float16* src = (xok && ch < P.Cin) ? P.in + p * P.in_cs + xoff + (long)ch * HW : zero_ptr<_Float16>();
-            lds_dma_16(src, sb + WV + t * 64);
+            lds_dma_16_untracked(src, aring + abuf * XV + t * 64);
+            if (slot == S::NPS - 1 && ++pa_k == P.nsteps) {
+                pa_k = 0;
+                pa_item += gridDim.x;
+                locate_act(pa_item);
+            }
         }
-        if (slot == S::NPS - 1 && ++p_k == P.nsteps) {
-            p_k = 0;
-            p_item += gridDim.x;
-            locate_copy(p_item);
-        }
-    };
-    auto issue = [&](int buf) {
-#pragma unroll
-        for (int slot = 0; slot < S::NPS; ++slot) issue_slot(buf, slot);
     };
 
     // ---- product side.  The activations are the MFMA A operand (rows = pixels), the filters the B operand (columns
-    // = output channels): lane (j, kk) feeds pixels 2j + m (m = 0, 1: two matrix instructions) and channels kk*8.. of
-    // the K step on the A side, filter row j on the B side, and receives D[pixel row][channel column]: column =
-    // output channel j of the wave's 32, register e = pixel row 8*(e/4) + 4*kk + e%4, i.e. pixel 2*row + m.  The four
-    // registers of a group e/4, for m = 0 and 1, are therefore EIGHT CONSECUTIVE pixels 16*(e/4) + 8*kk .. + 7 of one
-    // output channel: one 16-byte store, no cross-lane traffic at all.
+    // = output channels).  Lane l of a transposing read: sixteen-lane group G = l / 16 reads channels kk*8 + 4h .. + 3
+    // (kk = G / 2; h = first / second read of an operand) for pixels 32m + 16 (G % 2) .. + 15 of the wave's 64;
+    // as a source lane it points at channel row (l % 16) / 4 of those four and pixel quad l % 4.  The lane receives
+    // D[pixel row][channel column]: column = output channel j of the wave's 32, register e = pixel
+    // 32m + 8 (e / 4) + 4 kk + e % 4: four consecutive pixels per register group.
+    const int rr = (lane >> 2) & 3, qd = lane & 3;
+    const int piece0 = wpx * 8 + 2 * ((lane >> 4) & 1) + (qd >> 1);
+    unsigned int xrd[2];  // byte offsets of this lane's source run in a stage's activations, per column tile m
+#pragma unroll
+    for (int m = 0; m < 2; ++m)
+        xrd[m] = (unsigned int)((kk * 8 + rr) * PITCH + (((piece0 + 4 * m) ^ S::swz(rr)) * 16) + (qd & 1) * 8);
+
     // (TSTORE: after the transposition a lane stores piece lane % 8 of the wave's 8 pixel groups, for channel
-    // 8*i + lane / 8 in its i-th store: one address)
-    constexpr int NOA = TSTORE ? 1 : 4;
-    long oaddr[NOA];    // per register group: element offset of its 8-pixel group in an output component
+    // 8*i + lane / 8 in its i-th store: one address; else a lane stores the quads of all eight groups itself)
+    constexpr int NOA = TSTORE ? 1 : 8;
+    long oaddr[NOA];    // element offset of an 8-pixel group in an output component
     bool ovalid[NOA];
 #pragma unroll
     for (int a = 0; a < NOA; ++a) { oaddr[a] = 0; ovalid[a] = false; }
-    int c_item = wg, c_k = 0, c_ct = 0;
-    auto locate_out = [&](int item) {
+    int c_item = wg, c_k = 0, c_ct = 0, c_half = -1;
+    auto locate_out = [&](int i) {
+        int item;
+        decode(i, item, c_half);
         const int tile = item / P.co_tiles;
         c_ct = item - tile * P.co_tiles;
 #pragma unroll
         for (int a = 0; a < NOA; ++a) {
-            const int gg = tile * GPT + wpx * 8 + (TSTORE ? (lane & 7) : 2 * a + kk);
-            ovalid[a] = gg < P.TGp;
+            const int piece = TSTORE ? (lane & 7) : a;
+            const int gg = tile * GPT + wpx * 8 + piece;
+            ovalid[a] = gg < P.TGp && (c_half < 0 || (piece >> 2) == c_half);
             const int n = gg / P.GI, gi = gg - n * P.GI;
             oaddr[a] = ((long)n * P.CoutS) * HW + min(gi * 8, HW - 8);
         }
     };
 
     f32x16 acc[4][2];
+    PHX_PHASES_BEGIN(5)
     const int my_items = P.items > wg ? (P.items - wg + (int)gridDim.x - 1) / (int)gridDim.x : 0;
     const int total_steps = my_items * P.nsteps;
-    locate_copy(p_item);
+    // this workgroup's whole items come first, its half item (at most one: half items are the last round) last
+    const int my_whole = P.items_whole > wg ? (P.items_whole - wg + (int)gridDim.x - 1) / (int)gridDim.x : 0;
+    const int whole_steps = my_whole * P.nsteps;
+    locate_act(pa_item);
+    locate_filter(pf_item);
     locate_out(c_item);
+    // start-up, in the order the waits below count on: filters of the first DF steps, activations of the first DA
 #pragma unroll
-    for (int s = 0; s < D; ++s)
-        if (s < total_steps) issue(s);
+    for (int st = 0; st < DF; ++st)
+#pragma unroll
+        for (int slot = 0; slot < S::NWI; ++slot) issue_slot(st, 0, slot);
+#pragma unroll
+    for (int st = 0; st < DA; ++st)
+#pragma unroll
+        for (int slot = S::NWI; slot < S::NPS; ++slot) issue_slot(0, st, slot);
+    int fcur = 0, acur = 0;  // filter / activation stage of the current step
 
-    // One K step: operands from ring buffer buf, the copies of stage gs + D dealt out between the matrix
-    // instructions.  FIRST: the accumulators start from zero (first step of an item).
-    auto products = [&](int buf, bool more, int nbuf, auto first_tag) {
-        constexpr bool FIRST = decltype(first_tag)::value;
-        const f16x8* wb = lds16 + buf * SV + (wco * 4) * 64 + lane;
-        const unsigned int* xb = reinterpret_cast<const unsigned int*>(lds16 + buf * SV + WV) + (kk * 8) * ROWDW + wpx * 32 + j;
-        f16x8 w[4], nw[4];
+    // One K step: operands from filter stage fcur and activation stage acur, the copies of the steps ahead dealt out
+    // between the matrix instructions.  FIRST: the accumulators start from zero (first step of an item).  HALF: a
+    // half item -- only column tile mh is multiplied, into acc[.][0].
+    auto products = [&](int mh, auto first_tag, auto half_tag) {
+        constexpr bool FIRST = decltype(first_tag)::value, HALF = decltype(half_tag)::value;
+        constexpr int NM = HALF ? 1 : 2;
+        const int fnext = fcur ^ 1, anext = acur == 0 ? RA - 1 : acur - 1;  // (DF = 1, DA = RA - 1 stages ahead)
+        const f16x8* wb = fring + fcur * WV + (wco * 4) * 64 + lane;
+        const f16x8* xs = aring + acur * XV;
+        f16x8 w[4];
 #pragma unroll
         for (int r = 0; r < 4; ++r) w[r] = wb[r * 64];
-        unsigned int raw[4][8];
+        f16x8 x[4][NM];
 #pragma unroll
         for (int p = 0; p < 4; ++p)
 #pragma unroll
-            for (int i = 0; i < 8; ++i) raw[p][i] = xb[(p * 16 + i) * ROWDW];
-#pragma unroll
-        for (int r = 1; r < 4; ++r) nw[r] = neg8(w[r]);  // the negative blocks of the Hamilton matrix use -w1, -w2, -w3 only
-        nw[0] = w[0];
+            for (int m = 0; m < NM; ++m) {
+                const unsigned int at = (HALF ? (mh ? xrd[1] : xrd[0]) : xrd[m]) + (unsigned int)(p * 16 * PITCH);
+                const f16x4 lo = lds_read_tr16(xs, at), hi = lds_read_tr16(xs, at + 4 * PITCH);
+                x[p][m] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+            }
         const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int p = 0; p < 4; ++p) {
-            u32x4 lo, hi;
+            // (the negative blocks of the Hamilton matrix negate the ACTIVATION operand: a value that lives for one
+            // component's products, where negated filters would be twelve registers held across the whole step)
+            f16x8 nx[NM];
 #pragma unroll
-            for (int d = 0; d < 4; ++d) {
-                lo[d] = __builtin_amdgcn_perm(raw[p][2 * d + 1], raw[p][2 * d], 0x05040100u);
-                hi[d] = __builtin_amdgcn_perm(raw[p][2 * d + 1], raw[p][2 * d], 0x07060302u);
-            }
-            const f16x8 x0 = __builtin_bit_cast(f16x8, lo), x1 = __builtin_bit_cast(f16x8, hi);
+            for (int m = 0; m < NM; ++m) nx[m] = neg8(x[p][m]);
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
-                const f16x8 f = qneg(p, q) ? nw[p ^ q] : w[p ^ q];
-                acc[q][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(x0, f, (FIRST && p == 0) ? zero : acc[q][0], 0, 0, 0);
-                acc[q][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(x1, f, (FIRST && p == 0) ? zero : acc[q][1], 0, 0, 0);
-                // one copy of the stage after next behind every few pairs of matrix instructions
+#pragma unroll
+                for (int m = 0; m < NM; ++m) {
+                    acc[q][m] = __builtin_amdgcn_mfma_f32_32x32x16_f16(qneg(p, q) ? nx[m] : x[p][m], w[p ^ q],
+                                                                       (FIRST && p == 0) ? zero : acc[q][m], 0, 0, 0);
+                }
+                // one copy of the steps ahead behind every few (pairs of) matrix instructions
                 constexpr int PAIRS = 16;
                 const int pair = p * 4 + q;
-                if (more) {
 #pragma unroll
-                    for (int slot = 0; slot < S::NPS; ++slot)
-                        if (pair == (slot * PAIRS) / S::NPS) {
-                            __builtin_amdgcn_sched_barrier(0);
-                            issue_slot(nbuf, slot);
-                            __builtin_amdgcn_sched_barrier(0);
+                for (int slot = 0; slot < S::NPS; ++slot)
+                    if (pair == (slot * PAIRS) / S::NPS) {
+                        __builtin_amdgcn_sched_barrier(0);
+                        issue_slot(fnext, anext, slot);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+            }
+        }
+        fcur ^= 1;
+        acur = acur == RA - 1 ? 0 : acur + 1;
+    };
+
+    // An item is complete: convert, add the bias (BIAS), regroup and store.  HALF: the results of column tile
+    // c_half sit in acc[.][0].
+    auto store_item = [&](auto bias_tag, auto half_tag) {
+        constexpr bool BIAS = decltype(bias_tag)::value, HALF = decltype(half_tag)::value;
+        const int co0 = (c_ct * WCO + wco) * 32;
+        // (TSTORE) the addend's vectors of a component are requested a component ahead -- the first here, in
+        // front of the drain, which then covers their latency; the others in front of the stores of the component
+        // before -- so that no store waits for a load of its own
+        u32x4 ad[4];
+        auto request_addend = [&](int q, u32x4 (&dst)[4]) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int c = 8 * i + (lane >> 3);
+                const bool ok = ovalid[0] && co0 + c < P.Cout;
+                dst[i] = ok ? load16_a2(P.addend + q * P.out_cs + (long)(co0 + c) * HW + oaddr[0]) : u32x4{0u, 0u, 0u, 0u};
+            }
+        };
+        if constexpr (TSTORE && ADD) request_addend(0, ad);
+        wait_vmem_all();  // this wave's copies of the steps ahead: landed
+        PHX_STAMP(2)
+        const int co = co0 + j;
+        const bool co_ok = co < P.Cout;
+        char* scr = reinterpret_cast<char*>(lds16 + RF * WV + RA * XV) + wave * (S::SCRV * 16);  // (TSTORE) this wave's own
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            float bv = 0.f;
+            if constexpr (BIAS) bv = co_ok ? (float)P.bias[q * P.CoutS + co] : 0.f;
+            _Float16* dst = P.out + q * P.out_cs + (long)co * HW;
+#pragma unroll
+            for (int m = 0; m < (HALF ? 1 : 2); ++m) {
+                const int mt = HALF ? c_half : m;  // the column tile these registers belong to
+#pragma unroll
+                for (int g4 = 0; g4 < 4; ++g4) {
+                    u32x2 v;
+#pragma unroll
+                    for (int k2 = 0; k2 < 2; ++k2) {
+                        f16x2 h;
+                        if constexpr (BIAS) {
+                            h[0] = (_Float16)(acc[q][m][g4 * 4 + 2 * k2] + bv);
+                            h[1] = (_Float16)(acc[q][m][g4 * 4 + 2 * k2 + 1] + bv);
+                        } else {
+                            h[0] = (_Float16)acc[q][m][g4 * 4 + 2 * k2];
+                            h[1] = (_Float16)acc[q][m][g4 * 4 + 2 * k2 + 1];
                         }
+                        v[k2] = __builtin_bit_cast(unsigned int, h);
+                    }
+                    // pixels 32 mt + 8 g4 + 4 kk .. + 3 of channel j: half kk of piece 4 mt + g4
+                    if constexpr (TSTORE) {
+                        *reinterpret_cast<u32x2*>(scr + (j * 9 + 4 * mt + g4) * 16 + kk * 8) = v;
+                    } else {
+                        // (HALF: mt is not a compile-time index; the eight addresses are, so pick among them)
+                        long oa = 0;
+                        bool ov = false;
+#pragma unroll
+                        for (int a = 0; a < NOA; ++a)
+                            if (a == 4 * mt + g4) { oa = oaddr[a]; ov = ovalid[a]; }
+                        if (ov && co_ok) {
+                            if constexpr (ADD) v = add_halves4(v, load8_a2(P.addend + q * P.out_cs + (long)co * HW + oa + 4 * kk));
+                            *reinterpret_cast<u32x2_a2*>(dst + oa + 4 * kk) = v;
+                        }
+                    }
                 }
+            }
+            if constexpr (TSTORE) {
+                // (LDS serves a wave's accesses in order: the reads see the writes above, and the next
+                // component's writes come after these reads)
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                u32x4 t[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    t[i] = *reinterpret_cast<const u32x4*>(scr + ((8 * i + (lane >> 3)) * 9 + (lane & 7)) * 16);
+                    if constexpr (ADD) t[i] = add_halves(t[i], ad[i]);
+                }
+                if constexpr (ADD) {
+                    if (q < 3) request_addend(q + 1, ad);  // (in front of this component's stores)
+                }
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int c = 8 * i + (lane >> 3);
+                    if (ovalid[0] && co0 + c < P.Cout)
+                        *reinterpret_cast<u32x4_a2*>(P.out + q * P.out_cs + (long)(co0 + c) * HW + oaddr[0]) = t[i];
+                }
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
             }
         }
     };
 
-    // Waiting for a stage's copies.  A wave's copies complete in order among themselves, so in steady state the
-    // copies of (at most D - 1) younger stages may stay in flight.  Output stores share the counter and complete
-    // in no fixed order relative to the copies: a wave therefore drains its copies BEFORE it issues an item's
-    // stores -- cheap, they were requested one and two steps earlier -- and then needs no wait at all for the next
-    // D steps, whose stages that drain has covered; by the time it counts again the stores are long gone.
+    // Waiting for a step's copies.  A wave's copies complete in the order of their issue, which is, step by step,
+    // filters (of the step DF ahead) then activations (DA ahead): at the top of a step everything but the activation
+    // copies issued during the step before has to have landed.  Output stores share the counter and complete in no
+    // fixed order relative to the copies: a wave therefore drains its copies BEFORE it issues an item's stores --
+    // cheap, they were requested one and two steps earlier -- and then needs no wait for the next step, whose
+    // stages that drain has covered; a store still in flight a step later only makes that step's wait longer.
     int covered = 0;  // steps ahead whose copies are known to have landed
 #ifdef PHX_PHASE_TIMING
     const long long t_wall0 = wall_clock64(), t_clk0 = clock64();
 #endif
-    PHX_PHASES_BEGIN(5)
-    for (int gs = 0; gs < total_steps; ++gs) {
-        const int buf = gs % R;
-        if (covered > 0) --covered;
-        else if (D == 2 && gs + 1 < total_steps) __builtin_amdgcn_s_waitcnt(0x0F70 | S::NPS);
-        else wait_vmem_all();
-        PHX_STAMP(0)
-        __syncthreads();  // ... for every wave; and every wave is done with the buffer the next copies overwrite
-        PHX_STAMP(1)
-        const bool more = gs + D < total_steps;
-        const int nbuf = (gs + D) % R;
-        if (c_k == 0) products(buf, more, nbuf, std::true_type());
-        else products(buf, more, nbuf, std::false_type());
-        PHX_STAMP(3)
-        if (++c_k == P.nsteps) {
-            // the item is complete (see above for who holds what)
-            const int co0 = (c_ct * WCO + wco) * 32;
-            // (TSTORE) the addend's vectors of a component are requested a component ahead -- the first here, in
-            // front of the drain, which then covers their latency; the others in front of the stores of the component
-            // before -- so that no store waits for a load of its own
-            u32x4 ad[4];
-            auto request_addend = [&](int q, u32x4 (&dst)[4]) {
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int c = 8 * i + (lane >> 3);
-                    const bool ok = ovalid[0] && co0 + c < P.Cout;
-                    dst[i] = ok ? load16_a2(P.addend + q * P.out_cs + (long)(co0 + c) * HW + oaddr[0]) : u32x4{0u, 0u, 0u, 0u};
-                }
-            };
-            if constexpr (TSTORE && ADD) request_addend(0, ad);
-            wait_vmem_all();  // this wave's copies of the next D stages: landed
-            covered = D;
-            PHX_STAMP(2)
-            const int co = co0 + j;
-            const bool co_ok = co < P.Cout;
-            u32x4* scr = reinterpret_cast<u32x4*>(lds16 + R * SV) + wave * S::SCRV;  // (TSTORE) this wave's own
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const float bv = (P.bias && co_ok) ? (float)P.bias[q * P.CoutS + co] : 0.f;
-                _Float16* dst = P.out + q * P.out_cs + (long)co * HW;
-#pragma unroll
-                for (int g4 = 0; g4 < 4; ++g4) {
-                    u32x4 v;
-#pragma unroll
-                    for (int k = 0; k < 4; ++k) {
-                        f16x2 h;
-                        h[0] = (_Float16)(acc[q][0][g4 * 4 + k] + bv);
-                        h[1] = (_Float16)(acc[q][1][g4 * 4 + k] + bv);
-                        v[k] = __builtin_bit_cast(unsigned int, h);
-                    }
-                    if constexpr (TSTORE) scr[j * 9 + 2 * g4 + kk] = v;  // channel j, piece 2*g4 + kk
-                    else if (ovalid[g4] && co_ok) {
-                        if constexpr (ADD) v = add_halves(v, load16_a2(P.addend + q * P.out_cs + (long)co * HW + oaddr[g4]));
-                        *reinterpret_cast<u32x4_a2*>(dst + oaddr[g4]) = v;
-                    }
-                }
-                if constexpr (TSTORE) {
-                    // (LDS serves a wave's accesses in order: the reads see the writes above, and the next
-                    // component's writes come after these reads)
-                    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-                    u32x4 t[4];
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        t[i] = scr[(8 * i + (lane >> 3)) * 9 + (lane & 7)];
-                        if constexpr (ADD) t[i] = add_halves(t[i], ad[i]);
-                    }
-                    if constexpr (ADD) {
-                        if (q < 3) request_addend(q + 1, ad);  // (in front of this component's stores)
-                    }
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        const int c = 8 * i + (lane >> 3);
-                        if (ovalid[0] && co0 + c < P.Cout)
-                            *reinterpret_cast<u32x4_a2*>(P.out + q * P.out_cs + (long)(co0 + c) * HW + oaddr[0]) = t[i];
-                    }
-                    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-                }
+    auto step_loop = [&](int gs0, int gs1, auto half_tag) {
+        for (int gs = gs0; gs < gs1; ++gs) {
+            if (covered > 0) --covered;
+            else if (DA >= 2 && gs + 1 < total_steps) __builtin_amdgcn_s_waitcnt(0x0F70 | S::NXI);  // (all but the youngest activation copies)
+            else wait_vmem_all();
+            PHX_STAMP(0)
+            wg_barrier_no_vmem_wait();  // ... for every wave; and every wave is done with the stages the next copies overwrite
+            PHX_STAMP(1)
+            if (c_k == 0) products(c_half, std::true_type(), half_tag);
+            else products(c_half, std::false_type(), half_tag);
+            PHX_STAMP(3)
+            if (++c_k == P.nsteps) {
+                // the item is complete (see above for who holds what)
+                if (P.bias) store_item(std::true_type(), half_tag);
+                else store_item(std::false_type(), half_tag);
+                covered = 1;
+                c_k = 0;
+                c_item += gridDim.x;
+                locate_out(c_item);
+                PHX_STAMP(4)
             }
-            c_k = 0;
-            c_item += gridDim.x;
-            locate_out(c_item);
-            PHX_STAMP(4)
         }
-    }
+    };
+    step_loop(0, whole_steps, std::false_type());
+    step_loop(whole_steps, total_steps, std::true_type());
+    wait_vmem_all();  // (the copies issued past the last item)
 #ifdef PHX_PHASE_TIMING
     const long long t_clk1 = clock64(), t_wall1 = wall_clock64();
     if ((blockIdx.x % 61) == 0 && (threadIdx.x & 63) == 0)
@@ -365,14 +468,14 @@ __global__ void __launch_bounds__(WG_THREADS, 2) qconv_pwx_nhwc_f16_kernel(const
         if (slot < S::NWI) {
             const int t = wave + 4 * slot;
             const f16x8* wsrc = P.wpk + ((long)p_ct * P.nsteps + p_k) * WV;
-            lds_dma_16(wsrc + t * 64 + lane, sb + t * 64);
+            lds_dma_16_untracked(wsrc + t * 64 + lane, sb + t * 64);
         } else {
             const int t = wave + 4 * (slot - S::NWI);
             const int p = t / BLK, b = t % BLK;
             const int gp = p_px0 + b * 32 + c_pxl, ch = p_k * 16 + c_half * 8;
             // channels past the tensor meet zero filters; they, and pixels past the last image, copy zeros
             const _Float16* src = (gp < P.NP && ch < P.Cin) ? P.in + p * P.in_cs + (long)gp * P.CinS + ch : zero_ptr<_Float16>();
-            lds_dma_16(src, sb + WV + t * 64);
+            lds_dma_16_untracked(src, sb + WV + t * 64);
         }
         if (slot == S::NPS - 1 && ++p_k == P.nsteps) {
             p_k = 0;
@@ -446,7 +549,7 @@ __global__ void __launch_bounds__(WG_THREADS, 2) qconv_pwx_nhwc_f16_kernel(const
         if (covered > 0) --covered;
         else if (D == 2 && gs + 1 < total_steps) __builtin_amdgcn_s_waitcnt(0x0F70 | S::NPS);
         else wait_vmem_all();
-        __syncthreads();
+        wg_barrier_no_vmem_wait();
         const bool more = gs + D < total_steps;
         const int nbuf = (gs + D) % R;
         if (c_k == 0) products(buf, more, nbuf, std::true_type());

@@ -30,6 +30,7 @@ struct Tuning {
     int tile_wco = 0, tile_ntw = 0;   // PHX_TUNE_TILE="wco,ntw"
     bool flat = false, noflat = false, nopw = false, pw8 = false, zi8 = false, wg8 = false, nos2d = false, noearly = false, norealx = false, nosub = false, oldplan = false;
     bool nopwx = false;               // PHX_TUNE_NOPWX: pointwise fp16 problems stay on the staged-window kernels
+    bool nohalf = false;              // PHX_TUNE_NOHALF: the pointwise streaming kernel never cuts items in two
     bool nosmalldense = false;        // PHX_TUNE_NOSMALLDENSE: small Dense problems stay on the matrix-core kernels
     int vec = 0;                      // PHX_TUNE_VEC (0 = unset)
     int wgs = 0;                      // PHX_TUNE_WGS (0 = unset)
@@ -51,6 +52,7 @@ struct Tuning {
         nosub = getenv("PHX_TUNE_NOSUB") != nullptr;
         oldplan = getenv("PHX_TUNE_OLDPLAN") != nullptr;
         nopwx = getenv("PHX_TUNE_NOPWX") != nullptr;
+        nohalf = getenv("PHX_TUNE_NOHALF") != nullptr;
         nosmalldense = getenv("PHX_TUNE_NOSMALLDENSE") != nullptr;
         if (const char* e = getenv("PHX_TUNE_VEC")) vec = atoi(e);
         if (const char* e = getenv("PHX_TUNE_WGS")) wgs = atoi(e);
@@ -760,8 +762,17 @@ static int run_pwx(const Problem& p, const Corr& c, const FwdPlan& pl, int map, 
         g_addend.fused = true;
     }
     const int groups_per_tile = 8 * (4 / pl.pwx);
-    a.items = cdiv(a.TGp, groups_per_tile) * pl.co_tiles;
-    const int blocks = std::min(a.items, 2 * dev->cu_count);  // persistent workgroups, two per CU
+    const int whole = cdiv(a.TGp, groups_per_tile) * pl.co_tiles;
+    const int slots = 2 * dev->cu_count;  // persistent workgroups, two per CU
+    int blocks = std::min(whole, slots);
+    a.items = a.items_whole = whole;
+    // A last round that keeps at most half of the workgroups busy runs as half items (one of a wave's two column
+    // tiles each): it then costs half an item's time.  With 1568 items on 512 workgroups that is 3.5 rounds for 4.
+    const int rem = whole % blocks;
+    if (!tune().nohalf) {
+        if (2 * whole <= slots) { a.items_whole = 0; a.items = blocks = 2 * whole; }
+        else if (rem > 0 && 2 * rem <= blocks) { a.items_whole = whole - rem; a.items = whole + rem; }
+    }
     int rc;
     {
         KernelTimer timer(st);
@@ -769,8 +780,9 @@ static int run_pwx(const Problem& p, const Corr& c, const FwdPlan& pl, int map, 
     }
     if (rc != 0) return PHX_ERR_NOT_SUPPORTED;
     PHX_HIP(hipGetLastError());
-    snprintf(g_name_buf, sizeof(g_name_buf), "%sqconv_%s_f16mfmapwx_p16_f16_wco%d_px%d_k%d_wgs%d%s", g_name_prefix,
-             map == MAP_FWD ? "fwd" : "dgrad", pl.pwx, 64 * (4 / pl.pwx), pl.pwx_steps, blocks, a.addend ? "_add" : "");
+    snprintf(g_name_buf, sizeof(g_name_buf), "%sqconv_%s_f16mfmapwx_p16_f16_wco%d_px%d_k%d_wgs%d_half%d%s", g_name_prefix,
+             map == MAP_FWD ? "fwd" : "dgrad", pl.pwx, 64 * (4 / pl.pwx), pl.pwx_steps, blocks, a.items - a.items_whole,
+             a.addend ? "_add" : "");
     g_last_kernel = g_name_buf;
     say(p, map == MAP_FWD ? "forward" : "input gradient");
     return PHX_OK;
