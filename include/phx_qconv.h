@@ -58,7 +58,8 @@ enum phx_data_format { PHX_NCHW = 0, PHX_NHWC = 1 };
  * (w, 0, 0, 0) -- and fall back to an embedding with zero components only for batches that cannot be grouped
  * (odd n; n not a multiple of 4 for REAL).  For these
  * algebras activations have dims * n batch rows (dims = 1, 2, 8), filters are [dims, co, ci, kh, kw] (Dense:
- * [dims, ni, no]), bias [dims, co]; NCHW, OIHW / IO, no groups, no real-valued input. */
+ * [dims, ni, no]), bias [dims, co]; every data format, filter layout and group count of the quaternion path (the
+ * reference's generic path is algebra-agnostic in these, src/conv2d.hpp:237-275), no real-valued input. */
 enum phx_algebra { PHX_QUATERNION = 0, PHX_REAL = 1, PHX_COMPLEX = 2, PHX_GA_300 = 3 };
 
 /* Which Hamilton-product formulation runs.

@@ -138,22 +138,77 @@ __global__ void __launch_bounds__(WG_THREADS) blade_scatter_kernel(const BladeAr
     }
 }
 
-struct BladeFilterArgs {
-    const void* w;   // algebra filter (forward: read; fold: written)
-    void* q;         // quaternion filter with halves * Co x halves * Ci channels
+// The same two maps for channels-last tensors, [dims][n][hw][C] <-> [4][n][hw][halves * C] (and channel groups, see
+// Composition): the channel axis is the contiguous one and the halves interleave along it, so these go element by
+// element.  A.C is the channel count per group here, A.G the number of groups.
+struct BladeLastArgs {
+    const void* src;
+    void* dst;
     BladeMap m;
-    int Co, Ci, taps;
-    long wcs, so, si;     // algebra filter: elements between blades, output channels, input channels (taps contiguous)
-    long qcs, qso, qsi;   // the same for the quaternion filter
+    long n, hw;
+    int Cg, G;
 };
 
-// filter blocks (input half x output half): [[A, B], [-B, A]]
+template <typename TS>
+__global__ void __launch_bounds__(WG_THREADS) blade_gather_last_kernel(const BladeLastArgs A) {
+    const TS* src = static_cast<const TS*>(A.src);
+    TS* dst = static_cast<TS*>(A.dst);
+    const int H = A.m.halves;
+    const long C = (long)A.Cg * A.G, C2 = C * H;
+    const long total = 4 * A.n * A.hw * C2;
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
+        const long c2 = idx % C2;
+        long r = idx / C2;
+        const long pos = r % A.hw;
+        r /= A.hw;
+        const long nn = r % A.n;
+        const int p = (int)(r / A.n);
+        const int g = (int)(c2 / ((long)H * A.Cg)), h = (int)((c2 / A.Cg) % H), cin = (int)(c2 % A.Cg);
+        const int b = A.m.blade[h * 4 + p], sg = A.m.sign[h * 4 + p];
+        float v = 0.f;
+        if (b >= 0) v = (float)sg * (float)src[(((long)b * A.n + nn) * A.hw + pos) * C + (long)g * A.Cg + cin];
+        dst[idx] = (TS)v;
+    }
+}
+
+template <typename TS>
+__global__ void __launch_bounds__(WG_THREADS) blade_scatter_last_kernel(const BladeLastArgs A) {
+    const TS* src = static_cast<const TS*>(A.src);
+    TS* dst = static_cast<TS*>(A.dst);
+    const int H = A.m.halves;
+    const long C = (long)A.Cg * A.G, C2 = C * H;
+    const long total = (long)A.m.dims * A.n * A.hw * C;
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
+        const long c = idx % C;
+        long r = idx / C;
+        const long pos = r % A.hw;
+        r /= A.hw;
+        const long nn = r % A.n;
+        const int b = (int)(r / A.n);
+        const int sl = A.m.slot[b], h = sl >> 2, p = sl & 3;
+        const long g = c / A.Cg, cin = c % A.Cg;
+        const long c2 = (g * H + h) * A.Cg + cin;
+        dst[idx] = (TS)((float)A.m.sign[sl] * (float)src[(((long)p * A.n + nn) * A.hw + pos) * C2 + c2]);
+    }
+}
+
+struct BladeFilterArgs {
+    const void* w;   // algebra filter (forward: read; fold: written)
+    void* q;         // quaternion filter with halves * Co x halves * Cig channels
+    BladeMap m;
+    int Co, Cog, Cig, taps;    // output channels in all and per group, input channels per group (the filter's own axis)
+    long wcs, wso, wsi, wst;   // algebra filter: elements between blades, output channels, input channels, taps
+    long qcs, qso, qsi, qst;   // the same for the quaternion filter
+};
+
+// filter blocks (input half x output half): [[A, B], [-B, A]]; with channel groups, group g of the quaternion
+// problem holds the two halves of the algebra's group g side by side: output channel (g * halves + ho) * Cog + o
 template <typename TS>
 __global__ void __launch_bounds__(WG_THREADS) blade_filter_build_kernel(const BladeFilterArgs A) {
     const TS* w = static_cast<const TS*>(A.w);
     TS* q = static_cast<TS*>(A.q);
     const int H = A.m.halves;
-    const long HO = (long)H * A.Co, HI = (long)H * A.Ci;
+    const long HO = (long)H * A.Co, HI = (long)H * A.Cig;
     const long total = 4 * HO * HI * A.taps;
     for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
         const int tap = (int)(idx % A.taps);
@@ -162,13 +217,14 @@ __global__ void __launch_bounds__(WG_THREADS) blade_filter_build_kernel(const Bl
         r /= HI;
         const int o2 = (int)(r % HO);
         const int p = (int)(r / HO);
-        const int ho = o2 / A.Co, o = o2 - ho * A.Co, hi = i2 / A.Ci, i = i2 - hi * A.Ci;
+        const int g = o2 / (H * A.Cog), ho = (o2 / A.Cog) % H, o = g * A.Cog + o2 % A.Cog;
+        const int hi = i2 / A.Cig, i = i2 - hi * A.Cig;
         const int part = (ho != hi) ? 1 : 0;
         const float block_sign = (ho == 0 && hi == 1) ? -1.f : 1.f;
         const int s = part * 4 + p, b = A.m.blade[s];
         float v = 0.f;
-        if (b >= 0) v = block_sign * (float)A.m.sign[s] * (float)w[b * A.wcs + o * A.so + i * A.si + tap];
-        q[p * A.qcs + o2 * A.qso + i2 * A.qsi + tap] = (TS)v;
+        if (b >= 0) v = block_sign * (float)A.m.sign[s] * (float)w[b * A.wcs + o * A.wso + i * A.wsi + tap * A.wst];
+        q[p * A.qcs + o2 * A.qso + i2 * A.qsi + tap * A.qst] = (TS)v;
     }
 }
 
@@ -177,23 +233,25 @@ template <typename TS>
 __global__ void __launch_bounds__(WG_THREADS) blade_filter_fold_kernel(const BladeFilterArgs A) {
     TS* w = static_cast<TS*>(const_cast<void*>(A.w));
     const TS* q = static_cast<const TS*>(A.q);
-    const long total = (long)A.m.dims * A.Co * A.Ci * A.taps;
+    const int H = A.m.halves;
+    const long total = (long)A.m.dims * A.Co * A.Cig * A.taps;
     for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
         const int tap = (int)(idx % A.taps);
         long r = idx / A.taps;
-        const int i = (int)(r % A.Ci);
-        r /= A.Ci;
+        const int i = (int)(r % A.Cig);
+        r /= A.Cig;
         const int o = (int)(r % A.Co);
         const int b = (int)(r / A.Co);
         const int s = A.m.slot[b], part = s >> 2, p = s & 3;
+        const int g = o / A.Cog, oin = o - g * A.Cog;
         auto at = [&](int ho, int hi) {
-            return (float)q[p * A.qcs + (long)(ho * A.Co + o) * A.qso + (long)(hi * A.Ci + i) * A.qsi + tap];
+            return (float)q[p * A.qcs + (long)((g * H + ho) * A.Cog + oin) * A.qso + (long)(hi * A.Cig + i) * A.qsi + tap * A.qst];
         };
         float v;
-        if (A.m.halves == 1) v = at(0, 0);
+        if (H == 1) v = at(0, 0);
         else if (part == 0) v = at(0, 0) + at(1, 1);
         else v = at(1, 0) - at(0, 1);
-        w[b * A.wcs + o * A.so + i * A.si + tap] = (TS)((float)A.m.sign[s] * v);
+        w[b * A.wcs + o * A.wso + i * A.wsi + tap * A.wst] = (TS)((float)A.m.sign[s] * v);
     }
 }
 
@@ -210,11 +268,22 @@ static size_t align256(size_t b) { return (b + 255) / 256 * 256; }
 
 // Buffers of one composed call at the front of the workspace: quaternion forms of the input-side tensor, the
 // output-side tensor, the filter and the bias; the quaternion call's own workspace follows.
+// Filter element strides (output channel, input channel, tap) of a layout with the given extents
+struct FilterStep { long so, si, st; };
+static FilterStep conv_filter_step(int layout, long O, long I, long taps) {
+    if (layout == PHX_OHWI) return {taps * I, 1, I};
+    if (layout == PHX_HWIO) return {1, O, I * O};
+    return {I * taps, taps, 1};  // OIHW
+}
+
 struct Composition {
     BladeMap m;
     BladeMap bias_map;  // paired form only
     bool packed = false;  // paired form: activations in place, `m` maps the filter
     bool half;
+    bool nhwc = false;    // channels-last activations
+    int groups = 1;
+    int layout = PHX_OIHW;  // filter layout (Dense: phx_dense_layout, see filter_args)
     size_t esize, x_bytes, y_bytes, w_bytes, b_bytes;
     long n;
     int ci, co, taps;
@@ -226,10 +295,21 @@ struct Composition {
         const size_t H = m.halves;
         x_bytes = packed ? 0 : align256(4 * n * H * ci * hw_in * esize);
         y_bytes = packed ? 0 : align256(4 * n * H * co * hw_out * esize);
-        w_bytes = align256(4 * H * co * H * ci * taps * esize);
+        w_bytes = align256(4 * H * co * H * (ci / groups) * taps * esize);
         b_bytes = align256(4 * H * co * esize);
     }
-    void gather(const void* src, void* dst, long rows, int C, long hw, hipStream_t st, const BladeMap* map = nullptr) const {
+    // Activations [blade][rows][C][hw] (or [blade][rows][hw][C], channels-last) -> quaternion form.  With channel
+    // groups the two halves interleave per group, [g][half][C / groups]: in the channels-first layout that is the
+    // ungrouped map on rows * groups "images" of C / groups channels.
+    void gather(const void* src, void* dst, long rows, int C, long hw, hipStream_t st, const BladeMap* map = nullptr,
+                bool grouped = true) const {
+        const int G = grouped ? groups : 1;
+        if (nhwc && hw > 1) {
+            BladeLastArgs a{src, dst, map ? *map : m, rows, hw, C / G, G};
+            launch(half, blade_gather_last_kernel<float>, blade_gather_last_kernel<_Float16>, 4 * rows * hw * m.halves * C, a, st);
+            return;
+        }
+        rows *= G; C /= G;
         BladeArgs a{src, dst, map ? *map : m, rows, C, hw};
         const int V = half ? 8 : 4;
         const long blocks = 4 * rows * m.halves, chw = C * hw;
@@ -237,36 +317,55 @@ struct Composition {
         else launch(half, blade_gather_kernel<float, 1>, blade_gather_kernel<_Float16, 1>, blocks * chw, a, st);
     }
     void scatter(const void* src, void* dst, long rows, int C, long hw, hipStream_t st) const {
+        if (nhwc && hw > 1) {
+            BladeLastArgs a{src, dst, m, rows, hw, C / groups, groups};
+            launch(half, blade_scatter_last_kernel<float>, blade_scatter_last_kernel<_Float16>, (long)m.dims * rows * hw * C, a, st);
+            return;
+        }
+        rows *= groups; C /= groups;
         BladeArgs a{src, dst, m, rows, C, hw};
         const int V = half ? 8 : 4;
         const long blocks = (long)m.dims * rows, chw = C * hw;
         if (chw % V == 0) launch(half, blade_scatter_kernel<float, 4>, blade_scatter_kernel<_Float16, 8>, blocks * (chw / V), a, st);
         else launch(half, blade_scatter_kernel<float, 1>, blade_scatter_kernel<_Float16, 1>, blocks * chw, a, st);
     }
-    // dense filters are [blade][in][out], convolution filters [blade][out][in][taps]
+    // dense filters are [blade][in][out] (IO) or [blade][out][in] (OI), convolution filters [blade] x the layout's axes;
+    // the quaternion filter is built in the same layout with halves * the channel counts
     BladeFilterArgs filter_args(const void* w, void* q, bool dense) const {
         BladeFilterArgs a;
-        a.w = w; a.q = q; a.m = m; a.Co = co; a.Ci = ci; a.taps = taps;
-        const long H = m.halves;
-        a.wcs = (long)co * ci * taps; a.qcs = H * co * H * ci * taps;
-        if (dense) { a.so = 1; a.si = co; a.qso = 1; a.qsi = H * co; }
-        else { a.so = (long)ci * taps; a.si = taps; a.qso = H * ci * taps; a.qsi = taps; }
+        a.w = w; a.q = q; a.m = m; a.Co = co; a.Cog = co / groups; a.Cig = ci / groups; a.taps = taps;
+        const long H = m.halves, O = co, I = ci / groups;
+        a.wcs = O * I * taps; a.qcs = H * O * H * I * taps;
+        FilterStep ws, qs;
+        if (dense) {
+            ws = layout == PHX_OI ? FilterStep{I, 1, 1} : FilterStep{1, O, 1};
+            qs = layout == PHX_OI ? FilterStep{H * I, 1, 1} : FilterStep{1, H * O, 1};
+        } else {
+            ws = conv_filter_step(layout, O, I, taps);
+            qs = conv_filter_step(layout, H * O, H * I, taps);
+        }
+        a.wso = ws.so; a.wsi = ws.si; a.wst = ws.st;
+        a.qso = qs.so; a.qsi = qs.si; a.qst = qs.st;
         return a;
     }
     void build_filter(const void* w, void* q, bool dense, hipStream_t st) const {
         launch(half, blade_filter_build_kernel<float>, blade_filter_build_kernel<_Float16>,
-               4L * m.halves * co * m.halves * ci * taps, filter_args(w, q, dense), st);
+               4L * m.halves * co * m.halves * (ci / groups) * taps, filter_args(w, q, dense), st);
     }
     void fold_filter(const void* q, void* w, bool dense, hipStream_t st) const {
-        launch(half, blade_filter_fold_kernel<float>, blade_filter_fold_kernel<_Float16>, (long)m.dims * co * ci * taps,
+        launch(half, blade_filter_fold_kernel<float>, blade_filter_fold_kernel<_Float16>, (long)m.dims * co * (ci / groups) * taps,
                filter_args(w, const_cast<void*>(q), dense), st);
     }
 };
 
 static int conv_composition(const phx_qconv_desc* d, Composition& c, phx_qconv_desc& inner) {
     if (!d || !blade_map(d->algebra, c.m)) return PHX_ERR_INVALID_ARGUMENT;
-    if (d->groups > 1 || d->filter_layout != PHX_OIHW || d->data_format != PHX_NCHW || d->real_input)
-        return PHX_ERR_NOT_SUPPORTED;
+    // (the reference's generic path is algebra-agnostic in layouts and groups, src/conv2d.hpp:237-275; a real-valued
+    // input is taken by the quaternion algebra only here)
+    if (d->real_input) return PHX_ERR_NOT_SUPPORTED;
+    const int groups = d->groups > 1 ? d->groups : 1;
+    if (d->ci % groups || d->co % groups) return PHX_ERR_INVALID_ARGUMENT;
+    c.groups = groups; c.layout = d->filter_layout; c.nhwc = d->data_format == PHX_NHWC;
     inner = *d;
     inner.algebra = PHX_QUATERNION;
     int images = 1;
@@ -286,7 +385,7 @@ static int conv_composition(const phx_qconv_desc* d, Composition& c, phx_qconv_d
 
 static int dense_composition(const phx_qdense_desc* d, Composition& c, phx_qdense_desc& inner) {
     if (!d || !blade_map(d->algebra, c.m)) return PHX_ERR_INVALID_ARGUMENT;
-    if (d->filter_layout != PHX_IO) return PHX_ERR_NOT_SUPPORTED;
+    c.layout = d->filter_layout;
     if (d->n < 0 || d->ni <= 0 || d->no <= 0 || (d->dtype != PHX_F32 && d->dtype != PHX_F16)) return PHX_ERR_INVALID_ARGUMENT;
     inner = *d;
     inner.algebra = PHX_QUATERNION;

@@ -721,7 +721,7 @@ inline int phxAlgebra(Algebra a) {
 
 inline phx_qconv_desc makeConvDesc(const Conv2DDescriptor& d, Context& ctx, int dtype, bool useBias) {
     // the quaternion algebra runs on the kernels directly, the others as one quaternion call on rearranged
-    // tensors inside the library (NCHW, OIHW, no groups, no real-valued input: it reports anything else)
+    // tensors inside the library (any data format, filter layout and group count; no real-valued input: the library reports that)
     const Algebra algebra = d.getAlgebra();
     const int dims = MULTIVECTOR_DIM[algebra];
     const DataFormat df = d.getDataFormat();

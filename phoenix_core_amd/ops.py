@@ -84,7 +84,7 @@ _DTYPES = {torch.float32: capi.PHX_F32, torch.float16: capi.PHX_F16}
 class Conv2DDescriptor:
     """Geometry of one convolution (Conv2DFwdDescriptor / Conv2DBwdDescriptor of the reference).  The quaternion
     algebra runs on the HIP kernels directly; REAL, COMPLEX and GA_300 run inside the library as one
-    quaternion call on rearranged tensors (algebras.py resolves their shapes; NCHW, OIHW, no groups).  data_format "NCHW" takes activations [4n, c, h, w],
+    quaternion call on rearranged tensors (algebras.py resolves their shapes).  data_format "NCHW" takes activations [4n, c, h, w],
     "NHWC" [4n, h, w, c] (transposed inside the call: the kernels compute on channels-first planes)."""
 
     def __init__(self, input_shape, filter_shape, stride=1, dilation=1, padding="VALID", groups=1,

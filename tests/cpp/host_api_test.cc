@@ -324,11 +324,40 @@ static void gpuDenseAndEmpty(Context& context) {
     conv2DBwd<device::HIP, float>(device, device, ex, ew, ey, edw, edx, ebd);
     std::vector<float> z = edw;
     CHECK(equalVectors(z, std::vector<float>(24, 0.f)));
-    // what the composed algebras do not cover raises instead of running something else (here: groups)
+    // the composed algebras take groups and layouts like the quaternions: a grouped complex 1x1 convolution is a
+    // complex product per channel, (1+2i)(2+i) = 5i and (3-i)(-i) = -1-3i
     AllocatedTensor<device::HIP, float> cx(device, {2, 2, 1, 1}), cw(device, {2, 2, 1, 1, 1}), cy(device, {2, 2, 1, 1});
+    cx = {1, 3, 2, -1};
+    cw = {2, 0, 1, -1};
     Conv2DFwdDescriptor cd(cx.getShape(), cw.getShape(), 1, 1, Padding::VALID, {}, 2, Algebra::COMPLEX,
                            DataFormat::NCHW, FilterLayout::OIHW, false);
-    CHECK_THROWS((conv2DFwd<device::HIP, float>(device, device, cx, cw, nullptr, cy, cd)), std::runtime_error);
+    conv2DFwd<device::HIP, float>(device, device, cx, cw, nullptr, cy, cd);
+    std::vector<float> cgot = cy;
+    CHECK(equalVectors(cgot, std::vector<float>{0, -1, 5, -3}, 1e-5f));
+    // tests/tests.cpp:440-487 and :492-547 as written: Algebra::REAL, NHWC, OHWI / HWIO
+    {
+        AllocatedTensor<device::HIP, float> rx(device, {1, 2, 2, 3}), rw(device, {2, 1, 1, 3}), rw2(device, {1, 1, 3, 2});
+        AllocatedTensor<device::HIP, float> ry(device, {1, 2, 2, 2});
+        rx = {0, -1, 1,  0, 0, 2,  0, 0, 3,  1, 0, 4};
+        rw = {1, 1, 1,  0, 0, 2};
+        rw2 = {1, 0,  1, 0,  1, 2};
+        Conv2DFwdDescriptor rd(rx.getShape(), rw.getShape(), 1, 1, Padding::VALID, {}, 1, Algebra::REAL, DataFormat::NHWC,
+                               FilterLayout::OHWI, false);
+        conv2DFwd<device::HIP, float>(device, device, rx, rw, nullptr, ry, rd);
+        std::vector<float> rgot = ry;
+        CHECK(equalVectors(rgot, std::vector<float>{0, 2, 2, 4, 3, 6, 5, 8}));
+        ry = std::vector<float>(8, -1.f);
+        Conv2DFwdDescriptor rd2(rx.getShape(), rw2.getShape(), 1, 1, Padding::VALID, {}, 1, Algebra::REAL, DataFormat::NHWC,
+                                FilterLayout::HWIO, false);
+        conv2DFwd<device::HIP, float>(device, device, rx, rw2, nullptr, ry, rd2);
+        rgot = ry;
+        CHECK(equalVectors(rgot, std::vector<float>{0, 2, 2, 4, 3, 6, 5, 8}));
+    }
+    // what the composed algebras do not cover raises instead of running something else: a real-valued input
+    AllocatedTensor<device::HIP, float> vx(device, {1, 2, 1, 1}), vw(device, {2, 2, 2, 1, 1}), vy(device, {2, 2, 1, 1});
+    Conv2DFwdDescriptor vd(vx.getShape(), vw.getShape(), 1, 1, Padding::VALID, {}, 1, Algebra::COMPLEX,
+                           DataFormat::NCHW, FilterLayout::OIHW, false, true);
+    CHECK_THROWS((conv2DFwd<device::HIP, float>(device, device, vx, vw, nullptr, vy, vd)), std::runtime_error);
 }
 
 static void testTensorSplit(Context& context) {  // tests/tests.cpp:729-760
