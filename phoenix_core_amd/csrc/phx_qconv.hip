@@ -156,28 +156,27 @@ static int device_state(DeviceState** out) {
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) { (void)hipGetLastError(); return PHX_ERR_RUNTIME; }
     DeviceState& d = g_devices[dev];
-    if (d.ready.load(std::memory_order_acquire) == 0) {
+    if (d.ready.load(std::memory_order_acquire) != 1) {
         std::lock_guard<std::mutex> lock(g_device_mutex);
-        if (d.ready.load(std::memory_order_relaxed) == 0) {
-            int ok = 1;
+        if (d.ready.load(std::memory_order_relaxed) != 1) {
+            // A kernel whose opt-in fails (a device with less LDS) is the only one affected: its launch reports the
+            // error, every other path runs.  Nothing is latched on failure: the next call tries again.
+            bool all = true;
             for (const void* fn : big_lds_kernels())
                 if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess) {
                     (void)hipGetLastError();
-                    ok = -1;
+                    all = false;
                 }
             int cus = 0;
             if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && cus > 0) d.cu_count = cus;
             else (void)hipGetLastError();
+            // (the built-in scratch array serves phx_qconv2d_fwd_noalloc alone, which reports a missing address itself)
             void* ptr = nullptr;
-            if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) {
-                (void)hipGetLastError();
-                ok = -1;
-            }
+            if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess) { (void)hipGetLastError(); ptr = nullptr; }
             d.scratch_ptr = ptr;
-            d.ready.store(ok, std::memory_order_release);
+            if (all && ptr) d.ready.store(1, std::memory_order_release);
         }
     }
-    if (d.ready.load(std::memory_order_acquire) != 1) return PHX_ERR_RUNTIME;
     if (out) *out = &d;
     return PHX_OK;
 }
@@ -1611,6 +1610,23 @@ struct ChannelsLast {
     }
 };
 
+// Entry points check their descriptor before they touch the device: an invalid descriptor is an invalid argument
+// whether or not a device is present.
+static int conv_desc_status(const phx_qconv_desc* desc) {
+    if (!desc) return PHX_ERR_INVALID_ARGUMENT;
+    phx_qconv_desc q = *desc;
+    q.algebra = PHX_QUATERNION;  // (the geometry rules are the same for every algebra)
+    Problem p;
+    return problem_from_conv(&q, p);
+}
+static int dense_desc_status(const phx_qdense_desc* desc) {
+    if (!desc) return PHX_ERR_INVALID_ARGUMENT;
+    phx_qdense_desc q = *desc;
+    q.algebra = PHX_QUATERNION;
+    Problem p;
+    return problem_from_dense(&q, p);
+}
+
 int phx_qconv2d_output_hw(const phx_qconv_desc* desc, int32_t* ho, int32_t* wo) {
     Problem p;
     const int rc = problem_from_conv(desc, p);
@@ -1695,6 +1711,7 @@ static int conv_fwd_quaternion(const phx_qconv_desc* desc, phx_stream_t stream, 
 
 int phx_qconv2d_fwd(const phx_qconv_desc* desc, phx_stream_t stream, const void* x, const void* w,
                     const void* bias_or_null, void* y, void* workspace, size_t workspace_bytes) {
+    if (const int desc_rc = conv_desc_status(desc)) return desc_rc;
     if (const int init_rc = device_state(nullptr)) return init_rc;
     if (misaligned_workspace(workspace)) return PHX_ERR_INVALID_ARGUMENT;
     if (desc && desc->algebra != PHX_QUATERNION)
@@ -1704,8 +1721,10 @@ int phx_qconv2d_fwd(const phx_qconv_desc* desc, phx_stream_t stream, const void*
 
 int phx_qconv2d_fwd_noalloc(const phx_qconv_desc* desc, phx_stream_t stream, const void* x, const void* w,
                             const void* bias_or_null, void* y) {
+    if (const int desc_rc = conv_desc_status(desc)) return desc_rc;
     DeviceState* dev = nullptr;
     if (const int init_rc = device_state(&dev)) return init_rc;
+    if (!dev->scratch_ptr) return PHX_ERR_RUNTIME;  // (the array's address could not be looked up on this device)
     if (phx_qconv2d_workspace_bytes(desc, PHX_PASS_FWD) > (size_t)PHX_NOALLOC_SCRATCH_BYTES) return PHX_ERR_SCRATCH_LIMIT;
     // the packed filters (and whatever else the forward pass stages) go to this device's copy of the scratch array
     return phx_qconv2d_fwd(desc, stream, x, w, bias_or_null, y, dev->scratch_ptr, PHX_NOALLOC_SCRATCH_BYTES);
@@ -1745,6 +1764,7 @@ static int conv_bwd_data_quaternion(const phx_qconv_desc* desc, phx_stream_t str
 
 int phx_qconv2d_bwd_data(const phx_qconv_desc* desc, phx_stream_t stream, const void* grad, const void* w, void* dx,
                          void* workspace, size_t workspace_bytes) {
+    if (const int desc_rc = conv_desc_status(desc)) return desc_rc;
     if (const int init_rc = device_state(nullptr)) return init_rc;
     if (misaligned_workspace(workspace)) return PHX_ERR_INVALID_ARGUMENT;
     if (desc && desc->algebra != PHX_QUATERNION)
@@ -1770,6 +1790,7 @@ size_t phx_qconv2d_packed_filter_bytes(const phx_qconv_desc* desc, int pass) {
 
 int phx_qconv2d_pack_filters(const phx_qconv_desc* desc, phx_stream_t stream, const void* w, void* packed_fwd,
                              size_t packed_fwd_bytes, void* packed_bwd_data, size_t packed_bwd_data_bytes) {
+    if (const int desc_rc = conv_desc_status(desc)) return desc_rc;
     if (const int init_rc = device_state(nullptr)) return init_rc;
     if (!desc || desc->algebra != PHX_QUATERNION) return PHX_ERR_NOT_SUPPORTED;
     if (!w || (!packed_fwd && !packed_bwd_data)) return PHX_ERR_INVALID_ARGUMENT;
@@ -1795,6 +1816,7 @@ int phx_qconv2d_pack_filters(const phx_qconv_desc* desc, phx_stream_t stream, co
 int phx_qconv2d_fwd_prepacked(const phx_qconv_desc* desc, phx_stream_t stream, const void* x, const void* packed_fwd,
                               size_t packed_fwd_bytes, const void* bias_or_null, void* y, void* workspace,
                               size_t workspace_bytes) {
+    if (const int desc_rc = conv_desc_status(desc)) return desc_rc;
     if (const int init_rc = device_state(nullptr)) return init_rc;
     if (!desc || desc->algebra != PHX_QUATERNION) return PHX_ERR_NOT_SUPPORTED;
     if (!packed_fwd || misaligned_workspace(workspace) || misaligned_workspace(packed_fwd)) return PHX_ERR_INVALID_ARGUMENT;
@@ -1806,6 +1828,7 @@ int phx_qconv2d_fwd_prepacked(const phx_qconv_desc* desc, phx_stream_t stream, c
 int phx_qconv2d_bwd_data_prepacked(const phx_qconv_desc* desc, phx_stream_t stream, const void* grad,
                                    const void* packed_bwd_data, size_t packed_bwd_data_bytes, void* dx, void* workspace,
                                    size_t workspace_bytes) {
+    if (const int desc_rc = conv_desc_status(desc)) return desc_rc;
     if (const int init_rc = device_state(nullptr)) return init_rc;
     if (!desc || desc->algebra != PHX_QUATERNION) return PHX_ERR_NOT_SUPPORTED;
     if (!packed_bwd_data || misaligned_workspace(workspace) || misaligned_workspace(packed_bwd_data)) return PHX_ERR_INVALID_ARGUMENT;
@@ -1817,6 +1840,7 @@ int phx_qconv2d_bwd_data_prepacked(const phx_qconv_desc* desc, phx_stream_t stre
 int phx_qconv2d_bwd_data_add(const phx_qconv_desc* desc, phx_stream_t stream, const void* grad, const void* w,
                              const void* packed_bwd_data_or_null, size_t packed_bwd_data_bytes, const void* addend, void* dx,
                              void* workspace, size_t workspace_bytes) {
+    if (const int desc_rc = conv_desc_status(desc)) return desc_rc;
     if (const int init_rc = device_state(nullptr)) return init_rc;
     if (!desc || desc->algebra != PHX_QUATERNION) return PHX_ERR_NOT_SUPPORTED;
     if (!addend || !dx || addend == dx) return PHX_ERR_INVALID_ARGUMENT;
@@ -1837,6 +1861,7 @@ int phx_qconv2d_bwd_data_add(const phx_qconv_desc* desc, phx_stream_t stream, co
 
 int phx_qconv2d_bwd_weights(const phx_qconv_desc* desc, phx_stream_t stream, const void* x, const void* grad, void* dw,
                             void* workspace, size_t workspace_bytes) {
+    if (const int desc_rc = conv_desc_status(desc)) return desc_rc;
     if (const int init_rc = device_state(nullptr)) return init_rc;
     if (misaligned_workspace(workspace)) return PHX_ERR_INVALID_ARGUMENT;
     if (desc && desc->algebra != PHX_QUATERNION)
@@ -1865,6 +1890,7 @@ int phx_qconv2d_bwd_weights(const phx_qconv_desc* desc, phx_stream_t stream, con
 
 int phx_qdense_fwd(const phx_qdense_desc* desc, phx_stream_t stream, const void* x, const void* w,
                    const void* bias_or_null, void* y, void* workspace, size_t workspace_bytes) {
+    if (const int desc_rc = dense_desc_status(desc)) return desc_rc;
     if (const int init_rc = device_state(nullptr)) return init_rc;
     if (misaligned_workspace(workspace)) return PHX_ERR_INVALID_ARGUMENT;
     if (desc && desc->algebra != PHX_QUATERNION)
@@ -1878,6 +1904,7 @@ int phx_qdense_fwd(const phx_qdense_desc* desc, phx_stream_t stream, const void*
 
 int phx_qdense_bwd_data(const phx_qdense_desc* desc, phx_stream_t stream, const void* grad, const void* w, void* dx,
                         void* workspace, size_t workspace_bytes) {
+    if (const int desc_rc = dense_desc_status(desc)) return desc_rc;
     if (const int init_rc = device_state(nullptr)) return init_rc;
     if (misaligned_workspace(workspace)) return PHX_ERR_INVALID_ARGUMENT;
     if (desc && desc->algebra != PHX_QUATERNION)
@@ -1891,6 +1918,7 @@ int phx_qdense_bwd_data(const phx_qdense_desc* desc, phx_stream_t stream, const 
 
 int phx_qdense_bwd_weights(const phx_qdense_desc* desc, phx_stream_t stream, const void* x, const void* grad, void* dw,
                            void* workspace, size_t workspace_bytes) {
+    if (const int desc_rc = dense_desc_status(desc)) return desc_rc;
     if (const int init_rc = device_state(nullptr)) return init_rc;
     if (misaligned_workspace(workspace)) return PHX_ERR_INVALID_ARGUMENT;
     if (desc && desc->algebra != PHX_QUATERNION)

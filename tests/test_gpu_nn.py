@@ -396,7 +396,8 @@ def test_qresnet50_fp16_full16_matches_cpu_restatement(mode):
     assert worst < 2e-2, worst
 
 
-def test_qresnet50_full_size_step_and_layer_crops():
+@pytest.mark.parametrize("mode", [8, 16])
+def test_qresnet50_full_size_step_and_layer_crops(mode):
     """The benchmark's own configuration: N=64 images of 224x224, fp16 tensors, full16 policy, one forward+backward
     step.  The loss and every gradient must be finite, and the outputs of a handful of convolutions across the
     network (captured by hooks during that step) must agree with the oracle on a top-left crop of two images:
@@ -404,7 +405,7 @@ def test_qresnet50_full_size_step_and_layer_crops():
     only, where the true top / left padding applies."""
     torch.manual_seed(4)
     n = 64
-    model = phx.QResNet50(num_classes=1000, dtype=torch.float16, context=Ctx(8, "full16"), real_input=True,
+    model = phx.QResNet50(num_classes=1000, dtype=torch.float16, context=Ctx(mode, "full16"), real_input=True,
                           fused_bn=True).cuda().train()
     convs = model.conv_layers()
     picked = {1: "1x1 16->16 @56", 2: "3x3 16->16 @56", 12: "3x3 s2 32->32 @56->28", 13: "1x1 32->128 @28",

@@ -39,9 +39,13 @@ def _both(desc, x, w, b):
     got = torch.full(desc.output_shape, float("nan"), dtype=x.dtype, device=x.device)
     capi.check(L.phx_qconv2d_fwd(ctypes.byref(desc.c), stream, _ptr(x), _ptr(w), _ptr(b), _ptr(want), _ptr(ws), nbytes),
                "phx_qconv2d_fwd")
+    # the call allocates nothing: neither the device's free memory nor torch's own books move across it
+    torch.cuda.synchronize()
+    free_before, held_before = torch.cuda.mem_get_info()[0], torch.cuda.memory_allocated()
     capi.check(L.phx_qconv2d_fwd_noalloc(ctypes.byref(desc.c), stream, _ptr(x), _ptr(w), _ptr(b), _ptr(got)),
                "phx_qconv2d_fwd_noalloc")
     torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before and torch.cuda.memory_allocated() == held_before
     return want, got
 
 
@@ -74,6 +78,32 @@ def test_no_alloc_forward_matches_workspace_forward(pair, mode, dtype, policy):
     desc = phx.Conv2DDescriptor(x.shape, wt.shape, 1, 1, padding, dtype=dtype, context=Ctx(mode, policy))
     want, got = _both(desc, x, wt, None)
     assert torch.equal(want, got)
+
+
+STAGED = [
+    # paths that stage more than packed filters through the built-in array, all under its 16 MiB
+    ("nhwc_k3", dict(shape=(8, 10, 12, 24), wshape=(4, 16, 24, 3, 3), stride=1, padding="SAME", data_format="NHWC")),
+    ("stem_7x7_s2_real", dict(shape=(2, 3, 32, 32), wshape=(4, 16, 3, 7, 7), stride=2, padding="SAME", real_valued_input=True)),
+    ("strided_pw", dict(shape=(8, 32, 14, 14), wshape=(4, 48, 32, 1, 1), stride=2, padding="VALID")),
+    ("complex_k3", dict(shape=(6, 8, 9, 9), wshape=(2, 12, 8, 3, 3), stride=1, padding="SAME", algebra=phx.COMPLEX)),
+]
+
+
+@pytest.mark.parametrize("dtype,policy", [(torch.float32, "fp32"), (torch.float16, "full16")], ids=["f32", "f16"])
+@pytest.mark.parametrize("case", STAGED, ids=lambda c: c[0])
+def test_no_alloc_forward_with_staged_tensors(case, dtype, policy):
+    """Channels-last transposes, the space-to-depth stem, a subsampled strided pointwise convolution and another
+    algebra's rearranged tensors all go through the built-in array: bit for bit the workspace entry point's result."""
+    name, kw = case
+    kw = dict(kw)
+    torch.manual_seed(3)
+    scale = 1.0 if dtype == torch.float32 else 0.5
+    x = (scale * torch.randn(kw.pop("shape"), device="cuda")).to(dtype)
+    wt = (scale * 0.3 * torch.randn(kw.pop("wshape"), device="cuda")).to(dtype)
+    desc = phx.Conv2DDescriptor(x.shape, wt.shape, kw.pop("stride"), 1, kw.pop("padding"), dtype=dtype, context=Ctx(8, policy), **kw)
+    want, got = _both(desc, x, wt, None)
+    assert torch.isfinite(want.float()).all()
+    assert torch.equal(want, got), name
 
 
 def test_no_alloc_forward_refuses_what_does_not_fit():
