@@ -262,6 +262,7 @@ struct TileSrc {
     int ncomp;         // components present in memory: 4, or 1 for a real-valued tensor (components 1..3 read as zero)
     int pw;            // pointwise trick: window row r holds channels (chunk*pw + r)*16.. of the single image row (0 = off)
     int tall;          // flat tiling: the images are rows [n*tall, n*tall + Hd) of one tall image, zero rows between them (0 = off)
+    int nhwc;          // channels-last memory, t[4][N][Hd][Wd][Cs] (chunk staging of the fp16 LDS kernels only; 0 = planes)
 };
 
 // Window staging, split so that global loads can be in flight while the previous chunk is being

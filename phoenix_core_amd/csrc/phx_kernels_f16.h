@@ -335,6 +335,7 @@ struct StageChunk {
     unsigned int bits;    // positions inside the image
     int kp;
     int sub;              // pointwise trick: 16-channel sub-chunk this window row stands for
+    int cpr;              // channels-last: tasks per window row = positions between two of a task's entries
     bool task, live, careful;
 };
 
@@ -362,12 +363,32 @@ __device__ __forceinline__ StageChunk make_stage_chunk(const TileSrc& s, int n0,
     const int p = u >> 1;
     sc.kp = u & 1;
     sc.live = sc.task && p < s.ncomp && nb < NB && img >= 0 && img < s.N && vh >= 0 && vh < s.Hd;
-    sc.bits = sc.live ? interval_bits(-vw0, s.Wd - vw0) : 0u;
     const _Float16* base = static_cast<const _Float16*>(s.base);
     const long plane = (long)s.Hd * s.Wd;
-    sc.ptr = base + p * s.comp_stride + ((long)img * s.Cs * s.Hd + vh) * s.Wd + vw0;
-    const _Float16* end = base + (long)(s.ncomp - 1) * s.comp_stride + ((long)(s.N - 1) * s.Cs + s.C) * plane;
-    sc.careful = sc.live && (sc.ptr < base || sc.ptr + (long)(s.C - 1) * plane + 8 > end);
+    sc.cpr = cpr;
+    if (s.nhwc) {
+        // channels-last: the entry of a position (8 consecutive channels) is 16 contiguous bytes of memory, loaded and
+        // stored as it is.  A task takes positions cc, cc + cpr, ... of its window row rather than 8 neighbours:
+        // the lanes of a load then read neighbouring positions (Cs elements apart) instead of every eighth -- with a
+        // power-of-two channel count those would all sit 4 or 8 KiB apart, on one memory channel.
+        const int vw = w0 + cc;
+        sc.bits = 0u;
+        if (sc.live) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) sc.bits |= (unsigned int)(vw + j * cpr >= 0 && vw + j * cpr < s.Wd) << j;
+        }
+        sc.ptr = base + p * s.comp_stride + (((long)img * s.Hd + vh) * s.Wd + vw) * s.Cs;
+        const _Float16* end = base + (long)(s.ncomp - 1) * s.comp_stride + (long)s.N * plane * s.Cs;
+        sc.careful = sc.live && (sc.ptr < base || sc.ptr + 7L * cpr * s.Cs + ((s.C + 15) & ~15) > end);
+        sc.ent = (sc.task ? u : 0) * HPp;  // unit base; the entries are row * HTW + cc + j * cpr, swizzled one by one
+        sc.swz = row * HTW + cc;
+        return sc;
+    } else {
+        sc.bits = sc.live ? interval_bits(-vw0, s.Wd - vw0) : 0u;
+        sc.ptr = base + p * s.comp_stride + ((long)img * s.Cs * s.Hd + vh) * s.Wd + vw0;
+        const _Float16* end = base + (long)(s.ncomp - 1) * s.comp_stride + ((long)(s.N - 1) * s.Cs + s.C) * plane;
+        sc.careful = sc.live && (sc.ptr < base || sc.ptr + (long)(s.C - 1) * plane + 8 > end);
+    }
     const int e0 = row * HTW + cc * 8;
     sc.ent = (sc.task ? u : 0) * HPp + e0;
     sc.swz = (e0 >> 3) & 7;
@@ -375,6 +396,12 @@ __device__ __forceinline__ StageChunk make_stage_chunk(const TileSrc& s, int n0,
 }
 
 __device__ __forceinline__ void stage_chunk_load(u32x4 (&r)[8], const TileSrc& s, const StageChunk& sc, int c0, int i) {
+    if (s.nhwc) {  // position i of the task: channels c0 + 8 kp .. + 7
+        const int c = c0 + sc.kp * 8;
+        const _Float16* ptr = (sc.live && !sc.careful && c < s.C) ? sc.ptr + (long)i * sc.cpr * s.Cs + c : static_cast<const _Float16*>(s.base);
+        r[i] = load16_a2(ptr);
+        return;
+    }
     const long plane = (long)s.Hd * s.Wd;
     const int cv = c0 + sc.kp * 8 + i;
     const int c = s.pw ? ((cv >> 4) * s.pw + sc.sub) * 16 + (cv & 15) : cv;
@@ -387,6 +414,28 @@ __device__ __forceinline__ void stage_chunk_load(u32x4 (&r)[8], const TileSrc& s
 __device__ __forceinline__ void stage_chunk_store(f16x8* xl, const u32x4 (&r)[8], const TileSrc& s, const StageChunk& sc,
                                                   int c0) {
     if (!sc.task) return;
+    if (s.nhwc) {
+        // entries as loaded (the host takes this path only when C is a multiple of 8: a pack of 8 channels is inside
+        // the tensor or outside it as a whole); positions outside the image and packs outside the tensor are cleared
+        const int c = c0 + sc.kp * 8;
+        const unsigned int bits = (sc.careful || c >= s.C) ? 0u : sc.bits;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const u32x4 v = ((bits >> j) & 1) ? r[j] : u32x4{0u, 0u, 0u, 0u};
+            xl[sc.ent + swizzle_entry(sc.swz + j * sc.cpr)] = __builtin_bit_cast(f16x8, v);
+        }
+        if (sc.careful) {
+            _Float16* xh = reinterpret_cast<_Float16*>(xl);
+#pragma unroll 2
+            for (int j = 0; j < 8; ++j) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i)
+                    xh[(sc.ent + swizzle_entry(sc.swz + j * sc.cpr)) * 8 + i] =
+                        (c + i < s.C && ((sc.bits >> j) & 1)) ? sc.ptr[(long)j * sc.cpr * s.Cs + c + i] : (_Float16)0;
+            }
+        }
+        return;
+    }
     const u32x4 mk = expand_half_mask(sc.careful ? 0u : sc.bits);
     u32x4 rm[8];
 #pragma unroll
@@ -411,6 +460,69 @@ __device__ __forceinline__ void stage_chunk_store(f16x8* xl, const u32x4 (&r)[8]
             for (int j = 0; j < 8; ++j) v[j] = (c < s.C && ((sc.bits >> j) & 1)) ? sc.ptr[c * plane + j] : (_Float16)0;
 #pragma unroll
             for (int j = 0; j < 8; ++j) xh[(sc.ent + (j ^ sc.swz)) * 8 + i] = v[j];
+        }
+    }
+}
+
+// Epilogue for a channels-last output, out[4][N][Hout][Wout][CoutS] with oaddr = pixel index * CoutS.  Register e of an
+// accumulator is output channel 8*(e/4) + 4*kk + e%4 of the wave's 32 at this lane's pixel: four groups of 4
+// consecutive channels.  One v_permlane32_swap per packed dword between the two lane halves (which hold the same
+// pixels) turns them into 16 consecutive channels per lane -- the lower half 0..15, the upper half 16..31 -- stored as
+// two 16-byte words.  The host takes this path only when Cout and CoutS are multiples of 8.
+template <int MODE, int NTW, int NACC>
+__device__ __forceinline__ void conv_epilogue_cl(const ConvArgs& P, const f32x16 (&acc)[NTW][NACC], int co_wave,
+                                                 const long (&oaddr)[NTW], const bool (&pvalid)[NTW]) {
+    _Float16* out = static_cast<_Float16*>(P.out);
+    const _Float16* bias = static_cast<const _Float16*>(P.bias);
+    const int kk = (threadIdx.x >> 5) & 1;
+#pragma unroll
+    for (int t = 0; t < NTW; ++t) {
+        unsigned int d[4][4][2];  // [component][register group][packed pair]
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                float y[2][4];
+#pragma unroll
+                for (int k = 0; k < 2; ++k) {
+                    const int e = 4 * g + 2 * i + k;
+                    if constexpr (MODE == 16) {
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) y[k][q] = acc[t][q][e];
+                    } else {
+                        float l[8];
+#pragma unroll
+                        for (int a = 0; a < 8; ++a) l[a] = acc[t][a][e];
+                        merge_output(l, y[k]);
+                    }
+                    const int co = co_wave + 8 * g + 4 * kk + 2 * i + k;
+                    if (bias && co < P.Cout) {
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) y[k][q] += (float)bias[q * P.CoutS + co];
+                    }
+                }
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    f16x2 h;
+                    h[0] = (_Float16)y[0][q];
+                    h[1] = (_Float16)y[1][q];
+                    d[q][g][i] = __builtin_bit_cast(unsigned int, h);
+                }
+            }
+        const int co = co_wave + 16 * kk;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            u32x4 v0, v1;
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {  // (every lane takes part in the swaps, whatever its pixel)
+                const auto s02 = __builtin_amdgcn_permlane32_swap(d[q][0][i], d[q][2][i], false, false);
+                const auto s13 = __builtin_amdgcn_permlane32_swap(d[q][1][i], d[q][3][i], false, false);
+                v0[i] = s02[0]; v0[2 + i] = s02[1];
+                v1[i] = s13[0]; v1[2 + i] = s13[1];
+            }
+            _Float16* dst = out + q * P.out_cs + oaddr[t] + co;
+            if (pvalid[t] && co < P.Cout) *reinterpret_cast<u32x4_a2*>(dst) = v0;
+            if (pvalid[t] && co + 8 < P.Cout) *reinterpret_cast<u32x4_a2*>(dst + 8) = v1;
         }
     }
 }
@@ -486,13 +598,14 @@ __global__ void __launch_bounds__(WG_THREADS, (MODE == 16 && NTW == 1) ? 2 : 1) 
             const int n = R / P.in.tall, ho = R - n * P.in.tall;
             pvalid[t] = n < P.in.N && ho < P.Hout;
             poff[t] = pvalid[t] ? (R - R0) * P.HTW + c : 0;
-            oaddr[t] = ((long)n * P.CoutS * P.Hout + ho) * P.Wout + c;
+            oaddr[t] = P.nhwc ? (((long)n * P.Hout + ho) * P.Wout + c) * P.CoutS : ((long)n * P.CoutS * P.Hout + ho) * P.Wout + c;
         } else {
             const int nb = pix / thw, rem = pix - nb * thw;
             const int r = rem / P.TW, c = rem - r * P.TW;
             pvalid[t] = nb < P.NB && (n0 + nb) < P.in.N && (ho0 + r) < P.Hout && (wo0 + c) < P.Wout;
             poff[t] = pvalid[t] ? (nb * P.HTH + r * P.sh) * P.HTW + c * P.sw : 0;
-            oaddr[t] = ((long)(n0 + nb) * P.CoutS * P.Hout + (ho0 + r)) * P.Wout + (wo0 + c);
+            oaddr[t] = P.nhwc ? (((long)(n0 + nb) * P.Hout + (ho0 + r)) * P.Wout + (wo0 + c)) * P.CoutS
+                              : ((long)(n0 + nb) * P.CoutS * P.Hout + (ho0 + r)) * P.Wout + (wo0 + c);
         }
     }
 
@@ -717,7 +830,8 @@ __global__ void __launch_bounds__(WG_THREADS, (MODE == 16 && NTW == 1) ? 2 : 1) 
         if (++g == ngroups) { g = 0; ++chunk; }
     }
 
-    conv_epilogue<_Float16, MODE, NTW, NW>(P, acc, (ct * WCO + wco) * 32 + 4 * kk, oaddr, pvalid);
+    if (CHUNKS && P.nhwc) conv_epilogue_cl<MODE, NTW, NW>(P, acc, (ct * WCO + wco) * 32, oaddr, pvalid);
+    else conv_epilogue<_Float16, MODE, NTW, NW>(P, acc, (ct * WCO + wco) * 32 + 4 * kk, oaddr, pvalid);
 #ifdef PHX_PHASE_TIMING
     __builtin_amdgcn_s_waitcnt(0x0F70);  // (charge the stores to the epilogue; otherwise the wave ends with them in flight)
 #endif
@@ -832,6 +946,12 @@ __global__ void __launch_bounds__(WG_THREADS) pack_filters_f16_lds_kernel(const 
 //   10, 12) consecutive pixels of memory; which of them are padding depends on the pixel's own row and column,
 //   so the masks are per tap and pixel, built from the at most two row segments of a chunk.
 //   Partial sums go to workspace[z]; reduce_wgrad_kernel adds them in a fixed order.
+//   Channels-last tensors (CL; 64x64 channel tiles, unit stride, one or three taps): the reduction index is no
+//   longer the contiguous one, 8 consecutive CHANNELS of a pixel are.  A thread then stages (chunk of 8 pixels) x
+//   (component, 8 channels): one 16-byte load per pixel -- 8 for the gradient, 8 + TPW - 1 for the input, whose taps
+//   are shifts by whole pixels -- and an 8x8 transposition in registers (byte permutes) on the way to the same LDS
+//   rows of 8 pixels per channel, under the same pixel masks.  Load and store counts per thread are those of the
+//   channels-first form; the multiplications and the epilogue do not know the difference.
 // ---------------------------------------------------------------------------------------------
 constexpr int WG16_KP = 64;         // reduction indices per pixel tile
 constexpr int WG16_PITCH = 64 + 8;  // LDS halves per staged channel row (16-byte skew against bank conflicts)
@@ -881,9 +1001,10 @@ __device__ __forceinline__ WgChunk wg_chunk(const WgradArgs& P, int tile, int j)
     return c;
 }
 
-template <int MODE, int MT, int NT, int TPW, int SW>
+template <int MODE, int MT, int NT, int TPW, int SW, bool CL = false>
 __global__ void __launch_bounds__(WG_THREADS) qconv_wgrad_f16_kernel(const WgradArgs P) {
     static_assert(TPW == 1 || ((TPW == 3 || TPW == 4) && SW == 1), "shifted copies need unit stride");
+    static_assert(!CL || (MT == 2 && NT == 2 && SW == 1 && (TPW == 1 || TPW == 3)), "channels-last staging: 64x64 tiles, unit stride");
     constexpr int CoT = 32 * MT, CiT = 32 * NT;
     constexpr int NL = (MODE == 16) ? 4 : 8;  // accumulators per (tap, tile): components or lanes
     constexpr int KPp = WG16_PITCH;
@@ -914,6 +1035,9 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_wgrad_f16_kernel(const Wgrad
     const _Float16* gbase = static_cast<const _Float16*>(P.g.base);
     const _Float16* xbase = static_cast<const _Float16*>(P.x.base);
     const int co_first = cot * CoT + pg, ci_first = cit * CiT + pg;
+    // channels-last staging role: chunk j, component clq, channels clo*8 .. clo*8 + 7 of both channel tiles
+    const int clq = pg >> 3, clo = pg & 7;
+    constexpr int NXP = 8 + TPW - 1;  // input pixels a chunk touches over the taps of the group (unit stride)
 
     // 64x64 channel tiles: one 32x32 MFMA tile per wave (v_mfma_f32_32x32x16_f16 sustains its full rate from a
     // single wave per SIMD, the 16x16 shape does not); smaller tiles: MT x NT tiles of 16x16 per wave
@@ -936,7 +1060,8 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_wgrad_f16_kernel(const Wgrad
             for (int r = 0; r < 16; ++r) accb[t][a][r] = 0.f;
 
     u32x4 sg[GE];
-    unsigned int sx[XE][XR];
+    unsigned int sx[CL ? 1 : XE][XR];
+    u32x4 cx[CL ? NXP : 1];  // channels-last: the 8 channels of input pixel k of the chunk
     // Flat chunk list: the masks of every chunk of a plane under this workgroup's taps, as the 16-byte AND masks the
     // staging stores use ([chunk][gradient, tap 0, tap 1, ...]; entry P.cpr is all zeros, for chunks that are not
     // staged by vector loads) and as bits ([chunk][taps packed 8 bits each, gradient]).  Pixels q0 .. q0+7 of the
@@ -998,6 +1123,13 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_wgrad_f16_kernel(const Wgrad
     for (int i = 0; i < NT; ++i) xch[i] = (ci_first + 32 * i < P.x.C ? ci_first + 32 * i : P.x.C - 1) * (int)xplane;
 
     unsigned int lgoff[MT], lxoff[NT];  // load offsets of the tile being fetched
+    // channels-last: first channel of this thread's octets (octets beyond the tensor re-read its last one), elements
+    // per component, and the distance between two pixels of the tile being fetched (0 where everything is masked:
+    // such loads all read the tensor's first bytes)
+    const int gch0 = cot * CoT + clo * 8 < P.g.C ? cot * CoT + clo * 8 : P.g.C - 8;
+    const int xch0 = cit * CiT + clo * 8 < P.x.C ? cit * CiT + clo * 8 : P.x.C - 8;
+    const int gcomp_cl = P.g.N * (int)gplane * P.g.Cs, xcomp_cl = P.x.N * (int)xplane * P.x.Cs;
+    int lgstep = 0, lxstep = 0;
     auto prep = [&](const WgChunk& c) {
         bool any_x = c.live;
         if (!P.flat) {
@@ -1018,16 +1150,28 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_wgrad_f16_kernel(const Wgrad
                 }
             }
         }
-        const int grow = c.n * gimg + (P.flat ? c.wo0 : c.ho * Wo + c.wo0);
-        const int xrow_off = c.n * ximg + xlin(c);
         int goff[MT], xoff[NT];
+        if constexpr (CL) {
+            // element offsets of the chunk's first pixel (gradient) / first loaded pixel (input) at the thread's octet
+            goff[0] = (c.n * (int)gplane + (P.flat ? c.wo0 : c.ho * Wo + c.wo0)) * P.g.Cs + gch0;
+            xoff[0] = (c.n * (int)xplane + xlin(c)) * P.x.Cs + xch0;
+            careful = (c.live && goff[0] + 7 * P.g.Cs + 8 > gcomp_cl) ||
+                      (any_x && (xoff[0] < 0 || xoff[0] + (NXP - 1) * P.x.Cs + 8 > xcomp_cl));
+        } else {
+            const int grow = c.n * gimg + (P.flat ? c.wo0 : c.ho * Wo + c.wo0);
+            const int xrow_off = c.n * ximg + xlin(c);
 #pragma unroll
-        for (int i = 0; i < MT; ++i) goff[i] = grow + gch[i];
+            for (int i = 0; i < MT; ++i) goff[i] = grow + gch[i];
 #pragma unroll
-        for (int i = 0; i < NT; ++i) xoff[i] = xrow_off + xch[i];
-        // would any of this thread's vector loads leave the tensors?
-        careful = (c.live && goff[MT - 1] + 8 > gcomp) || (any_x && (xoff[0] < 0 || xoff[NT - 1] + 2 * XR > xcomp));
+            for (int i = 0; i < NT; ++i) xoff[i] = xrow_off + xch[i];
+            // would any of this thread's vector loads leave the tensors?
+            careful = (c.live && goff[MT - 1] + 8 > gcomp) || (any_x && (xoff[0] < 0 || xoff[NT - 1] + 2 * XR > xcomp));
+        }
         const bool gok = c.live && !careful, xok = any_x && !careful;
+        if constexpr (CL) {
+            lgstep = gok ? P.g.Cs : 0;
+            lxstep = xok ? P.x.Cs : 0;
+        }
         if (P.flat) {  // the masks of a chunk depend on its place in the plane only: looked up
             const u32x4* entry = fmask + (gok ? (c.wo0 >> 3) : P.cpr) * (TPW + 1);
             mg = entry[0];
@@ -1039,16 +1183,21 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_wgrad_f16_kernel(const Wgrad
             for (int t = 0; t < TPW; ++t) mx[t] = expand_half_mask(xok ? xbits[t] : 0u);
         }
 #pragma unroll
-        for (int i = 0; i < MT; ++i) lgoff[i] = (unsigned int)(gok ? goff[i] : 0);
+        for (int i = 0; i < (CL ? 1 : MT); ++i) lgoff[i] = (unsigned int)(gok ? goff[i] : 0);
 #pragma unroll
-        for (int i = 0; i < NT; ++i) lxoff[i] = (unsigned int)(xok ? xoff[i] : 0);
+        for (int i = 0; i < (CL ? 1 : NT); ++i) lxoff[i] = (unsigned int)(xok ? xoff[i] : 0);
     };
     // the load instructions of a tile, one "slot" each, so that they can be spread over the MFMA blocks:
     // a wave that issues them back to back stalls until the memory pipeline has taken them all
     constexpr int XL = (XR == 4) ? 1 : 2;          // load instructions per input chunk
-    constexpr int NLOADS = GE + XE * XL;
+    constexpr int NLOADS = CL ? 8 + NXP : GE + XE * XL;
+    const _Float16* gbase_cl = gbase + clq * P.g.comp_stride;
+    const _Float16* xbase_cl = xbase + clq * P.x.comp_stride;
     auto load_slot = [&](int sl) {
-        if (sl < GE) {
+        if constexpr (CL) {  // one pixel per slot: the gradient's 8, then the input's
+            if (sl < 8) sg[sl] = load16_a2(gbase_cl + lgoff[0] + sl * lgstep);
+            else if (sl < NLOADS) cx[sl - 8] = load16_a2(xbase_cl + lxoff[0] + (sl - 8) * lxstep);
+        } else if (sl < GE) {
             sg[sl] = load16_a2(gbase + (sl / MT) * P.g.comp_stride + lgoff[sl % MT]);
         } else if (sl < NLOADS) {
             const int e = (sl - GE) / XL, part = (sl - GE) % XL;
@@ -1079,6 +1228,27 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_wgrad_f16_kernel(const Wgrad
             gbits = c.live ? entry[1] : 0u;
 #pragma unroll
             for (int t = 0; t < TPW; ++t) xbits[t] = c.live ? (entry[0] >> (8 * t)) & 0xFFu : 0u;
+        }
+        if constexpr (CL) {
+            const _Float16* gsrc = gbase_cl + ((long)c.n * gplane + glin) * P.g.Cs + gch0;
+            const _Float16* xsrc = xbase_cl + ((long)c.n * xplane + lin) * P.x.Cs + xch0;  // (before the tensor where lin < 0: read under its bits only)
+#pragma unroll 2
+            for (int i = 0; i < 8; ++i) {
+#pragma unroll
+                for (int c8 = 0; c8 < 8; ++c8)
+                    gl[(clq * CoT + clo * 8 + c8) * KPp + j * 8 + i] = ((gbits >> i) & 1u) ? gsrc[(long)i * P.g.Cs + c8] : (_Float16)0;
+            }
+#pragma unroll
+            for (int t = 0; t < TPW; ++t) {
+#pragma unroll 2
+                for (int i = 0; i < 8; ++i) {
+#pragma unroll
+                    for (int c8 = 0; c8 < 8; ++c8)
+                        xl[((t * 4 + clq) * CiT + clo * 8 + c8) * KPp + j * 8 + i] =
+                            ((xbits[t] >> i) & 1u) ? xsrc[(long)(i + t) * P.x.Cs + c8] : (_Float16)0;
+                }
+            }
+            return;
         }
 #pragma unroll 2
         for (int e = 0; e < GE; ++e) {
@@ -1123,7 +1293,30 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_wgrad_f16_kernel(const Wgrad
     for (int tile = zi; tile < ntiles; tile += P.zsplit) {
         __syncthreads();
         PHX_STAMP(0)
-        {
+        if constexpr (CL) {
+            // 8 pixels x 8 channels -> 8 channel rows of 8 pixels: dword m of a row pairs pixels 2m and 2m + 1
+#pragma unroll
+            for (int c8 = 0; c8 < 8; ++c8) {
+                u32x4 v;
+#pragma unroll
+                for (int d = 0; d < 4; ++d)
+                    v[d] = __builtin_amdgcn_perm(sg[2 * d + 1][c8 >> 1], sg[2 * d][c8 >> 1], (c8 & 1) ? 0x07060302u : 0x05040100u);
+                *reinterpret_cast<u32x4*>(gl + (clq * CoT + clo * 8 + c8) * KPp + j * 8) = v & mg;
+            }
+#pragma unroll
+            for (int t = 0; t < TPW; ++t) {
+#pragma unroll
+                for (int c8 = 0; c8 < 8; ++c8) {
+                    u32x4 v;
+#pragma unroll
+                    for (int d = 0; d < 4; ++d)
+                        v[d] = __builtin_amdgcn_perm(cx[t + 2 * d + 1][c8 >> 1], cx[t + 2 * d][c8 >> 1],
+                                                     (c8 & 1) ? 0x07060302u : 0x05040100u);
+                    *reinterpret_cast<u32x4*>(xl + ((t * 4 + clq) * CiT + clo * 8 + c8) * KPp + j * 8) = v & mx[t];
+                }
+            }
+            if (careful) fill_careful(tile);
+        } else {
 #pragma unroll
             for (int e = 0; e < GE; ++e) {
                 const int q = e / MT, cc = (e % MT) * 32;

@@ -30,6 +30,7 @@ struct ConvArgs {
     int tiles_n, tiles_h, tiles_w, co_tiles;
     int nchunks;        // ceil(Cin / CK) for the kernel's chunk size CK
     int vec;            // output pixels a lane stores at once (4, 2 or 1): divides TW and Wout
+    int nhwc;           // the output is channels-last, out[4][N][Hout][Wout][CoutS] (fp16 chunk-staging kernel only)
 };
 
 // ---------------------------------------------------------------------------------------------

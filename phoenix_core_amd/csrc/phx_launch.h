@@ -81,6 +81,7 @@ int launch_wgrad_f16(int mode, int MT, int NT, int TPW, int SW, const WgradArgs&
 int launch_wgrad_f16_p16(int MT, int NT, int TPW, int SW, const WgradArgs& a, int nblocks, size_t lds_bytes, hipStream_t st);
 int launch_wgrad_f16_p16t3(int MT, int NT, const WgradArgs& a, int nblocks, size_t lds_bytes, hipStream_t st);
 // real-valued input, few channels: the whole filter gradient as one matrix product (phx_kernels_realx.h)
+int launch_wgrad_f16_cl(int TPW, const WgradArgs& a, int nblocks, size_t lds_bytes, hipStream_t st);  // channels-last tensors
 int launch_wgrad_f16_realx(const RealWgArgs& a, int nblocks, size_t lds_bytes, hipStream_t st);
 int launch_wgrad_f16_p8(int MT, int NT, int SW, const WgradArgs& a, int nblocks, size_t lds_bytes, hipStream_t st);
 int launch_reduce_wgrad(bool half_storage, const ReduceArgs& a, hipStream_t st);

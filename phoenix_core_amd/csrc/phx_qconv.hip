@@ -31,6 +31,8 @@ struct Tuning {
     bool flat = false, noflat = false, nopw = false, pw8 = false, zi8 = false, wg8 = false, nos2d = false, noearly = false, norealx = false, nosub = false, oldplan = false;
     bool nopwx = false;               // PHX_TUNE_NOPWX: pointwise fp16 problems stay on the staged-window kernels
     bool nohalf = false;              // PHX_TUNE_NOHALF: the pointwise streaming kernel never cuts items in two
+    bool nowincl = false;             // PHX_TUNE_NOWINCL: channels-last windowed problems go through the transposes
+    int wincl_max = 3072;             // PHX_TUNE_WINCL_MAX: largest channels x taps that runs on channels-last tensors directly
     bool nosmalldense = false;        // PHX_TUNE_NOSMALLDENSE: small Dense problems stay on the matrix-core kernels
     int vec = 0;                      // PHX_TUNE_VEC (0 = unset)
     int wgs = 0;                      // PHX_TUNE_WGS (0 = unset)
@@ -53,6 +55,8 @@ struct Tuning {
         oldplan = getenv("PHX_TUNE_OLDPLAN") != nullptr;
         nopwx = getenv("PHX_TUNE_NOPWX") != nullptr;
         nohalf = getenv("PHX_TUNE_NOHALF") != nullptr;
+        nowincl = getenv("PHX_TUNE_NOWINCL") != nullptr;
+        if (const char* e = getenv("PHX_TUNE_WINCL_MAX")) wincl_max = atoi(e);
         nosmalldense = getenv("PHX_TUNE_NOSMALLDENSE") != nullptr;
         if (const char* e = getenv("PHX_TUNE_VEC")) vec = atoi(e);
         if (const char* e = getenv("PHX_TUNE_WGS")) wgs = atoi(e);
@@ -184,6 +188,7 @@ static int device_state(DeviceState** out) {
 static thread_local const char* g_last_kernel = "";
 static thread_local char g_name_buf[160];
 static thread_local const char* g_name_prefix = "";  // "s2d_" while a rewritten problem runs
+static thread_local bool g_window_cl = false;        // run_corr reads and writes channels-last tensors (see nhwc_window_native)
 
 // Filters packed ahead of the passes that use them (phx_qconv2d_pack_filters and the *_prepacked entry points).
 // The forward and input-gradient code paths run as always, and this thread's session tells the places that pack
@@ -883,6 +888,10 @@ static int run_corr(const Problem& p, const Corr& creal, int map, hipStream_t st
     const int cin_mem = (map == MAP_FWD) ? p.ci_mem : p.co_mem, cout_mem = (map == MAP_FWD) ? p.co_mem : p.ci_mem;
     a.in.base = in; a.in.comp_stride = (long)c.N * cin_mem * c.Hin * c.Win; a.in.Cs = cin_mem;
     a.in.N = c.N; a.in.C = creal.Cin; a.in.Hd = c.Hin; a.in.Wd = c.Win; a.in.uh = c.uh; a.in.uw = c.uw; a.in.pw = pw; a.in.tall = pl.tall;
+    // channels-last tensors on both sides: only the chunk-staging fp16 kernel reads them (nhwc_window_native holds)
+    const bool cl = g_window_cl;
+    if (cl && !(f16 && pl.lds_filters && pl.chunks && !pw)) return PHX_ERR_RUNTIME;
+    a.in.nhwc = cl; a.nhwc = cl;
     // real-valued input: the forward pass reads one component, the others are zero
     a.in.ncomp = (p.real_input && map == MAP_FWD) ? 1 : 4;
     a.wpk = ws; a.bias = bias; a.out = out;
@@ -912,9 +921,9 @@ static int run_corr(const Problem& p, const Corr& creal, int map, hipStream_t st
     }
     if (rc != 0) return PHX_ERR_NOT_SUPPORTED;
     PHX_HIP(hipGetLastError());
-    snprintf(g_name_buf, sizeof(g_name_buf), "%sqconv_%s_%smfma%s_p%d_%s_wco%d_ntw%d_ck%d_%s%dx%dx%d", g_name_prefix,
-             map == MAP_FWD ? "fwd" : "dgrad", f16 ? "f16" : "f32", pl.lds_filters ? (pw ? "ldspw" : pl.chunks ? "ldsc" : "lds") : "", pl.kmode, p.dtype == PHX_F32 ? "f32" : "f16", pl.WCO,
-             pl.NTW, pl.CK, pl.tall ? "flat" : "tile", pl.NB, pl.TH, pl.TW);
+    snprintf(g_name_buf, sizeof(g_name_buf), "%sqconv_%s_%smfma%s%s_p%d_%s_wco%d_ntw%d_ck%d_%s%dx%dx%d", g_name_prefix,
+             map == MAP_FWD ? "fwd" : "dgrad", f16 ? "f16" : "f32", pl.lds_filters ? (pw ? "ldspw" : pl.chunks ? "ldsc" : "lds") : "",
+             cl ? "cl" : "", pl.kmode, p.dtype == PHX_F32 ? "f32" : "f16", pl.WCO, pl.NTW, pl.CK, pl.tall ? "flat" : "tile", pl.NB, pl.TH, pl.TW);
     g_last_kernel = g_name_buf;
     say(p, map == MAP_FWD ? "forward" : "input gradient");
     return PHX_OK;
@@ -1182,9 +1191,12 @@ static int run_wgrad(const Problem& p, hipStream_t st, const void* x, const void
     }
     WgradArgs a;
     a.x.base = x; a.x.comp_stride = (long)p.n * p.ci_mem * p.h * p.w; a.x.N = p.n; a.x.C = p.ci; a.x.Cs = p.ci_mem; a.x.Hd = p.h; a.x.Wd = p.w;
-    a.x.uh = a.x.uw = 1; a.x.pw = 0; a.x.tall = 0; a.x.ncomp = p.real_input ? 1 : 4;
+    // channels-last tensors on both sides: only the 64x64-tile fp16 kernel stages them (nhwc_wgrad_native holds)
+    const bool cl = g_window_cl;
+    if (cl && !(f16 && pl.kmode == 16 && pl.MT == 2 && pl.NT == 2 && pl.SW == 1 && (pl.TPW == 1 || pl.TPW == 3))) return PHX_ERR_RUNTIME;
+    a.x.uh = a.x.uw = 1; a.x.pw = 0; a.x.tall = 0; a.x.nhwc = cl; a.x.ncomp = p.real_input ? 1 : 4;
     a.g.base = g; a.g.comp_stride = (long)p.n * p.co_mem * p.ho * p.wo; a.g.N = p.n; a.g.C = p.co; a.g.Cs = p.co_mem; a.g.Hd = p.ho; a.g.Wd = p.wo;
-    a.g.uh = a.g.uw = 1; a.g.pw = 0; a.g.tall = 0; a.g.ncomp = 4;
+    a.g.uh = a.g.uw = 1; a.g.pw = 0; a.g.tall = 0; a.g.nhwc = cl; a.g.ncomp = 4;
     a.partial = static_cast<float*>(ws);
     a.Kh = p.kh; a.Kw = p.kw; a.sh = p.sh; a.sw = p.sw; a.dh = p.dh; a.dw = p.dw; a.pt = p.pt; a.pl = p.pl;
     a.NB = pl.NB; a.TH = pl.TH; a.TW = pl.TW; a.KP = pl.KP; a.KPp = pl.KPp; a.HPp = pl.HPp; a.HTH = pl.HTH;
@@ -1199,7 +1211,8 @@ static int run_wgrad(const Problem& p, hipStream_t st, const void* x, const void
     {
         KernelTimer timer(st);
         if (f16) {
-            if (launch_wgrad_f16(pl.kmode, pl.MT, pl.NT, pl.TPW, pl.SW, a, nblocks, pl.lds_bytes, st) != 0)
+            if ((cl ? launch_wgrad_f16_cl(pl.TPW, a, nblocks, pl.lds_bytes, st)
+                    : launch_wgrad_f16(pl.kmode, pl.MT, pl.NT, pl.TPW, pl.SW, a, nblocks, pl.lds_bytes, st)) != 0)
                 return PHX_ERR_RUNTIME;
         } else {
             launch_wgrad_f32(half_storage, pl.vec, pl.kmode, a, dim3(nblocks), pl.lds_bytes, st);
@@ -1213,8 +1226,8 @@ static int run_wgrad(const Problem& p, hipStream_t st, const void* x, const void
     launch_reduce_wgrad(half_storage, r, st);
     PHX_HIP(hipGetLastError());
     if (f16)
-        snprintf(g_name_buf, sizeof(g_name_buf), "%sqconv_wgrad_f16mfma_p%d_f16_ch%dx%d_taps%d_sw%d%s_z%d", g_name_prefix, pl.kmode, 32 * pl.MT,
-                 32 * pl.NT, pl.TPW, pl.SW, pl.flat ? "_flat" : "", pl.Z);
+        snprintf(g_name_buf, sizeof(g_name_buf), "%sqconv_wgrad_f16mfma%s_p%d_f16_ch%dx%d_taps%d_sw%d%s_z%d", g_name_prefix, cl ? "cl" : "",
+                 pl.kmode, 32 * pl.MT, 32 * pl.NT, pl.TPW, pl.SW, pl.flat ? "_flat" : "", pl.Z);
     else
         snprintf(g_name_buf, sizeof(g_name_buf), "%sqconv_wgrad_f32mfma%s_p%d_%s_tile%dx%dx%d_z%d", g_name_prefix, pl.vec ? "v" : "", pl.kmode,
                  p.dtype == PHX_F32 ? "f32" : "f16", pl.NB, pl.TH, pl.TW, pl.Z);
@@ -1610,6 +1623,45 @@ struct ChannelsLast {
     }
 };
 
+// Channels-last windowed convolutions (3x3 and other multi-tap filters, unit stride) whose forward / input-gradient
+// plan is the chunk-staging fp16 kernel run on the caller's tensors as they are: that kernel's LDS layout is
+// [position][8 channels], which IS the channels-last order, so its staging copies 16-byte entries without the
+// channel transpose the channels-first form needs, and the epilogue stores 16 consecutive channels of a pixel per
+// lane.  Everything else channels-last (the filter gradient, strides, groups, fp32) keeps the transposes.
+// A chunk of 16 channels is only 32 contiguous bytes per position, so the staging loads of this form touch many more
+// cache lines per instruction than the channels-first ones; the kernel is 0-5 % faster than the channels-first one
+// at 64 and 128 channels and 5-12 % slower at 256 and 512 (3x3; 56x56 .. 7x7 images), while the two transposes it
+// saves cost in proportion to the tensors, not to the arithmetic.  Calls whose arithmetic per tensor byte
+// (channels x taps) is beyond what was measured to pay (256 channels, 3x3) keep the transposes;
+// PHX_TUNE_WINCL_MAX moves that bound, PHX_TUNE_NOWINCL switches the direct form off.
+static bool nhwc_window_native(const Problem& p, int pass) {
+    if (!p.nhwc || (pass != PHX_PASS_FWD && pass != PHX_PASS_BWD_DATA) || is_empty(p) || is_pointwise_unit(p)) return false;
+    if (p.real_input || p.groups != 1 || p.sh != 1 || p.sw != 1 || tune().nowincl || !use_f16_mfma(p, pass)) return false;
+    if ((long)std::max(p.ci, p.co) * p.kh * p.kw > tune().wincl_max) return false;
+    if (p.ci % 8 != 0 || p.co % 8 != 0 || p.ci_mem != p.ci || p.co_mem != p.co) return false;  // whole 16-byte entries, 8-byte stores
+    S2dView v;
+    if (pass == PHX_PASS_FWD && s2d_view(p, v)) return false;
+    if (pass == PHX_PASS_BWD_DATA && dgrad_by_phases(p)) return false;
+    Corr c;
+    FwdPlan pl;
+    int pw = 0;
+    if (!plan_corr(pass == PHX_PASS_FWD ? corr_forward(p) : corr_dgrad(p), p.mode, true, c, pl, pw)) return false;
+    return pl.lds_filters && pl.chunks && !pl.pwx && pw == 0;
+}
+
+// The filter gradient of a channels-last call runs on the caller's tensors where its plan is the fp16 kernel with
+// 64x64 channel tiles, unit stride and one or three taps per workgroup (more than 32 channels on either side): that
+// kernel's channels-last staging transposes 8x8 blocks in registers on the way to LDS (qconv_wgrad_f16_kernel, CL).
+static bool nhwc_wgrad_native(const Problem& p) {
+    if (!p.nhwc || is_empty(p) || p.real_input || p.groups != 1 || p.sh != 1 || p.sw != 1 || tune().nowincl) return false;
+    if (p.ci % 8 != 0 || p.co % 8 != 0 || p.ci_mem != p.ci || p.co_mem != p.co) return false;
+    const Problem f = flatten_pointwise(p);
+    if (!wgrad_on_f16_mfma(f)) return false;
+    WgPlan pl;
+    if (!plan_wgrad(f, true, pl)) return false;
+    return !pl.realx && pl.kmode == 16 && pl.MT == 2 && pl.NT == 2 && pl.SW == 1 && (pl.TPW == 1 || pl.TPW == 3);
+}
+
 // Entry points check their descriptor before they touch the device: an invalid descriptor is an invalid argument
 // whether or not a device is present.
 static int conv_desc_status(const phx_qconv_desc* desc) {
@@ -1641,6 +1693,8 @@ size_t phx_qconv2d_workspace_bytes(const phx_qconv_desc* desc, int pass) {
     Problem p;
     if (problem_from_conv(desc, p) != PHX_OK) return 0;
     if (nhwc_native(p, pass)) return nhwc_native_workspace(p, pass);
+    if (nhwc_window_native(p, pass)) return workspace_for(p, pass);
+    if (pass == PHX_PASS_BWD_WEIGHTS && nhwc_wgrad_native(p)) return workspace_for(p, pass);
     return ChannelsLast(p).bytes() + workspace_for(p, pass);
 }
 
@@ -1688,8 +1742,14 @@ static int conv_fwd_quaternion(const phx_qconv_desc* desc, phx_stream_t stream, 
         return run_pwx_nhwc(p, MAP_FWD, static_cast<hipStream_t>(stream), x, w, p.has_bias ? bias_or_null : nullptr, y, workspace,
                             workspace_bytes);
     const GroupOffsets o(p);
-    const ChannelsLast cl(p);
     hipStream_t st = static_cast<hipStream_t>(stream);
+    if (nhwc_window_native(p, PHX_PASS_FWD)) {
+        g_window_cl = true;
+        const int nrc = do_fwd(p, st, x, w, bias_or_null, y, dry ? nullptr : workspace, dry ? 0 : workspace_bytes);
+        g_window_cl = false;
+        return nrc;
+    }
+    const ChannelsLast cl(p);
     if (dry) { workspace = nullptr; workspace_bytes = cl.bytes(); }
     else if (cl.bytes() > workspace_bytes || (cl.bytes() && !workspace)) return PHX_ERR_WORKSPACE;
     char* ws = static_cast<char*>(workspace);
@@ -1742,8 +1802,14 @@ static int conv_bwd_data_quaternion(const phx_qconv_desc* desc, phx_stream_t str
     if (nhwc_native(p, PHX_PASS_BWD_DATA))
         return run_pwx_nhwc(p, MAP_DGRAD, static_cast<hipStream_t>(stream), grad, w, nullptr, dx, workspace, workspace_bytes);
     const GroupOffsets o(p);
-    const ChannelsLast cl(p);
     hipStream_t st = static_cast<hipStream_t>(stream);
+    if (nhwc_window_native(p, PHX_PASS_BWD_DATA)) {
+        g_window_cl = true;
+        const int nrc = do_bwd_data(p, st, grad, w, dx, dry ? nullptr : workspace, dry ? 0 : workspace_bytes);
+        g_window_cl = false;
+        return nrc;
+    }
+    const ChannelsLast cl(p);
     if (dry) { workspace = nullptr; workspace_bytes = cl.bytes(); }
     else if (cl.bytes() > workspace_bytes || (cl.bytes() && !workspace)) return PHX_ERR_WORKSPACE;
     char* ws = static_cast<char*>(workspace);
@@ -1870,8 +1936,14 @@ int phx_qconv2d_bwd_weights(const phx_qconv_desc* desc, phx_stream_t stream, con
     const int rc = problem_from_conv(desc, p);
     if (rc != PHX_OK) return rc;
     const GroupOffsets o(p);
-    const ChannelsLast cl(p);
     hipStream_t st = static_cast<hipStream_t>(stream);
+    if (nhwc_wgrad_native(p)) {
+        g_window_cl = true;
+        const int nrc = do_bwd_weights(p, st, x, grad, dw, workspace, workspace_bytes);
+        g_window_cl = false;
+        return nrc;
+    }
+    const ChannelsLast cl(p);
     if (cl.bytes() > workspace_bytes || (cl.bytes() && !workspace)) return PHX_ERR_WORKSPACE;
     char* ws = static_cast<char*>(workspace);
     if (p.nhwc) {

@@ -505,6 +505,71 @@ def test_channels_last(case, mode, dtype, policy):
         assert_close(dx.cpu().numpy().transpose(0, 3, 1, 2), want_dx, dtype, "channels-last dgrad " + name)
 
 
+# name, n, ci, co, h, w, kh, kw, dilation, padding -- unit stride, more than one tap, channel counts multiples of 8
+CHANNELS_LAST_WINDOWS = [
+    ("clw_k3_24_40", 2, 24, 40, 13, 9, 3, 3, 1, "SAME"),           # half-filled last chunk on both sides
+    ("clw_k3_64_14_n5", 5, 64, 64, 14, 14, 3, 3, 1, "SAME"),       # images stacked into one tall image
+    ("clw_k3_128_28", 2, 128, 128, 28, 28, 3, 3, 1, "SAME"),
+    ("clw_k3_7x7_n9", 9, 40, 40, 7, 7, 3, 3, 1, "SAME"),           # several images per workgroup
+    ("clw_k3_dil2", 2, 16, 32, 12, 12, 3, 3, 2, "SAME"),
+    ("clw_k5_asym_pad", 3, 8, 8, 9, 12, 5, 3, 1, (3, 0, 1, 2)),    # more rows read below the image than above
+    ("clw_k3_full_pad", 2, 8, 8, 6, 10, 3, 3, 1, (2, 2, 2, 2)),    # output larger than the input
+    ("clw_k3_w29", 2, 8, 16, 5, 29, 3, 3, 1, "SAME"),              # odd width
+    ("clw_k3_valid_c72_200", 1, 72, 200, 9, 11, 3, 3, 1, "VALID"),
+    ("clw_k2_1px", 1, 8, 8, 2, 2, 2, 2, 1, "VALID"),               # one output position: every window load is near an end of the tensor
+    ("clw_k1x3_c40_72", 2, 40, 72, 6, 17, 1, 3, 1, "SAME"),        # filter gradient: half-filled channel tiles, rows of 17
+    ("clw_k2_c64", 1, 64, 64, 3, 3, 2, 2, 1, (1, 1, 1, 1)),        # tiny planes: most chunk loads are next to an end of the tensors
+    ("clw_k3x2_c136", 1, 136, 64, 9, 8, 3, 2, 1, "SAME"),          # one tap per workgroup (two-tap rows), three input-channel tiles
+]
+
+
+@pytest.mark.parametrize("mode", [16, 8])
+@pytest.mark.parametrize("case", CHANNELS_LAST_WINDOWS, ids=lambda c: c[0])
+def test_channels_last_windows_run_on_the_tensors_as_they_are(case, mode, tune_env):
+    """Multi-tap, unit-stride channels-last convolutions on fp16 matrix cores: forward, input gradient and (from 33
+    channels on either side) filter gradient read and write the caller's [4n, h, w, c] tensors directly (kernel names
+    carry "cl"), no transposed copies.  Held against the oracle, and bit for bit against the same call through the
+    transposes (PHX_TUNE_NOWINCL): both run the same products in the same order."""
+    name, n, ci, co, h, w, kh, kw, dilation, padding = case
+    dtype = torch.float16
+    g, x, wt, b, gr = make_inputs(name_seed(name) + 13, n, ci, co, h, w, kh, kw, 1, dilation, padding, dtype, 0.5)
+    x_dev = np.ascontiguousarray(x.transpose(0, 2, 3, 1))
+    g_dev = np.ascontiguousarray(gr.transpose(0, 2, 3, 1))
+    w_dev = np.ascontiguousarray(wt.transpose(0, 1, 3, 4, 2))
+    desc = phx.Conv2DDescriptor(x_dev.shape, w_dev.shape, 1, dilation, padding, use_bias=True, dtype=dtype, filter_layout="OHWI",
+                                context=Ctx(mode, "full16"), data_format="NHWC")
+    xd, wd, bd, gd = (torch.from_numpy(a).cuda() for a in (x_dev, w_dev, b, g_dev))
+    x64, w64, b64, g64 = (a.astype(np.float64) for a in (x, wt, b, gr))
+    want_y = oracle.conv2d_fwd(g, x64, w64, b64, "hamilton")
+    want_dw, want_dx = oracle.conv2d_bwd(g, x64, w64, g64, "hamilton")
+    got = {}
+    for variant in ("direct", "transposed"):
+        tune_env(PHX_TUNE_NOWINCL=None if variant == "direct" else "1")
+        ws = [desc.workspace_bytes(p) for p in range(3)]
+        y = phx.conv2d_fwd(xd, wd, bd, desc)
+        k_fwd = capi.last_kernel_name()
+        dx = ops.conv2d_bwd_data(wd, gd, desc)
+        k_bwd = capi.last_kernel_name()
+        dw = ops.conv2d_bwd_weights(xd, gd, desc)
+        k_wg = capi.last_kernel_name()
+        print(name, mode, variant, k_fwd, k_bwd, k_wg, ws, flush=True)
+        assert_close(y.cpu().numpy().transpose(0, 3, 1, 2), want_y, dtype, "fwd " + k_fwd)
+        assert_close(dx.cpu().numpy().transpose(0, 3, 1, 2), want_dx, dtype, "dgrad " + k_bwd)
+        assert_close(dw.cpu().numpy().transpose(0, 1, 4, 2, 3), want_dw, dtype, "wgrad " + k_wg)
+        got[variant] = dict(y=y, dx=dx, dw=dw, names=(k_fwd, k_bwd, k_wg), ws=ws)
+    direct, transposed = got["direct"], got["transposed"]
+    assert not any("cl_" in k for k in transposed["names"]), transposed["names"]
+    planes = 2 * 4 * n * (ci * h * w + co * g.ho * g.wo)  # bytes of the channels-first copies
+    if name != "clw_k2_1px":  # (the planner keeps so small a problem off the chunk-staging kernel)
+        assert "ldsccl_" in direct["names"][0] and "ldsccl_" in direct["names"][1], direct["names"]
+        assert direct["ws"][0] <= transposed["ws"][0] - planes and direct["ws"][1] <= transposed["ws"][1] - planes
+    if ci > 32 and co > 32:
+        assert "mfmacl_" in direct["names"][2], direct["names"]
+        assert direct["ws"][2] <= transposed["ws"][2] - planes
+    for key in ("y", "dx", "dw"):
+        assert torch.equal(direct[key], transposed[key]), key
+
+
 # name, n, ci, co, h, w, kh, kw, stride, dilation, padding -- unit stride, more than one tap
 FLAT = [c for c in FP16_CASES if c[0] in ("k3_same", "k3_ragged", "k3_valid", "k3_dil2", "k4_same", "k24_c40", "k3_128_28")] + [
     ("k3_7x7_n9", 9, 40, 40, 7, 7, 3, 3, 1, 1, "SAME"),              # several images per workgroup
