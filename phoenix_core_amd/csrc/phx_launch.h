@@ -47,6 +47,8 @@ int launch_pack_filters_f16(const FwdVariant& v, const PackArgs& a, int blocks, 
 // pointwise fp16-MFMA kernels with raw operand copies (phx_kernels_pw16.h); WCO = 32-channel sub-tiles per workgroup
 struct PwxArgs;
 int launch_pwx_f16(int WCO, const PwxArgs& a, int blocks, hipStream_t st);
+int launch_pwr_f16(int WCO, const PwxArgs& a, int blocks, hipStream_t st);  // packed filter resident in LDS
+size_t pwr_lds_bytes(int WCO, int nsteps);
 int launch_pwx_nhwc_f16(int WCO, const PwxArgs& a, int blocks, hipStream_t st);  // channels-last tensors
 size_t pwx_packed_bytes(int WCO, int co_tiles, int nsteps);
 int launch_pack_filters_pwx(int map, int WCO, int nsteps, const PackArgs& a, hipStream_t st);

@@ -31,12 +31,15 @@ struct Tuning {
     bool flat = false, noflat = false, nopw = false, pw8 = false, zi8 = false, wg8 = false, nos2d = false, noearly = false, norealx = false, nosub = false, oldplan = false;
     bool nopwx = false;               // PHX_TUNE_NOPWX: pointwise fp16 problems stay on the staged-window kernels
     bool nohalf = false;              // PHX_TUNE_NOHALF: the pointwise streaming kernel never cuts items in two
+    bool nopwr = false;               // PHX_TUNE_NOPWR: pointwise fp16 problems with small filters stay on the streaming kernel
+    bool pwrall = false;              // PHX_TUNE_PWRALL: ... and every problem that kernel can run goes to it (not only those of at most 32 output channels)
     bool nowincl = false;             // PHX_TUNE_NOWINCL: channels-last windowed problems go through the transposes
     int wincl_max = 3072;             // PHX_TUNE_WINCL_MAX: largest channels x taps that runs on channels-last tensors directly
     bool nosmalldense = false;        // PHX_TUNE_NOSMALLDENSE: small Dense problems stay on the matrix-core kernels
     int vec = 0;                      // PHX_TUNE_VEC (0 = unset)
     int wgs = 0;                      // PHX_TUNE_WGS (0 = unset)
     int wg_mt = 0, wg_nt = 0;         // PHX_TUNE_WG="mt,nt"
+    int wg_tpw = 0;                   // PHX_TUNE_WGTPW: taps per workgroup of the fp16 filter gradient (1 = no shared gradient tile)
     int phase = -1;                   // PHX_TUNE_PHASE (-1 = unset)
     int verbose = 0;                  // UPSTRIDE_VERBOSE (src/backend/backend.cc:45-48)
     void read() {
@@ -55,12 +58,15 @@ struct Tuning {
         oldplan = getenv("PHX_TUNE_OLDPLAN") != nullptr;
         nopwx = getenv("PHX_TUNE_NOPWX") != nullptr;
         nohalf = getenv("PHX_TUNE_NOHALF") != nullptr;
+        nopwr = getenv("PHX_TUNE_NOPWR") != nullptr;
+        pwrall = getenv("PHX_TUNE_PWRALL") != nullptr;
         nowincl = getenv("PHX_TUNE_NOWINCL") != nullptr;
         if (const char* e = getenv("PHX_TUNE_WINCL_MAX")) wincl_max = atoi(e);
         nosmalldense = getenv("PHX_TUNE_NOSMALLDENSE") != nullptr;
         if (const char* e = getenv("PHX_TUNE_VEC")) vec = atoi(e);
         if (const char* e = getenv("PHX_TUNE_WGS")) wgs = atoi(e);
         if (const char* e = getenv("PHX_TUNE_WG")) sscanf(e, "%d,%d", &wg_mt, &wg_nt);
+        if (const char* e = getenv("PHX_TUNE_WGTPW")) wg_tpw = atoi(e);
         if (const char* e = getenv("PHX_TUNE_PHASE")) phase = atoi(e) != 0;
         if (const char* e = getenv("UPSTRIDE_VERBOSE")) verbose = (int)strtol(e, nullptr, 10);
     }
@@ -765,6 +771,45 @@ static int run_pwx(const Problem& p, const Corr& c, const FwdPlan& pl, int map, 
         a.addend = static_cast<const _Float16*>(g_addend.ptr);
         g_addend.fused = true;
     }
+    // Small filters (the packed image and the waves' copy rings fit 160 KiB of LDS, one output-channel tile, whole K
+    // steps, at least two, plane size a multiple of 8) can run on the kernel that keeps the filter resident and never
+    // synchronises its waves (phx_kernels_pwr16.h); it reads the packed image the streaming kernel reads, so
+    // prepacked filters serve both.  Measured against the streaming kernel (N=64; forward, us): at most 32 output
+    // channels 64->32 @56x56 42 against 56, 32->32 @56x56 24 against 36, 64->16 @56x56 29 against 37, 128->32 @28x28 19
+    // against 23 -- there the streaming kernel's workgroup tile is 256 pixels wide and stores its quads directly;
+    // wider outputs 64->64 @56x56 54 against 50-62, 128->64 @28x28 26 against 24, 64->128 @28x28 37 against 29,
+    // 128->128 @28x28 (N=128) 78-81 against 76-79.  So it takes the problems of at most 32 output channels;
+    // PHX_TUNE_PWRALL sends it everything it can run.
+    if (!tune().nopwr && (pl.pwx == 1 || tune().pwrall) && pl.co_tiles == 1 && pwr_lds_bytes(pl.pwx, pl.pwx_steps) <= 160 * 1024 &&
+        pl.pwx_steps >= 2 && c.Cin == 16 * pl.pwx_steps && c.Win % 8 == 0) {
+        const int tiles = cdiv(a.TGp, 4);                            // 32 pixels x all output channels per wave
+        // persistent workgroups of four waves: as many per CU as LDS and registers allow (16 accumulator tiles fill a
+        // SIMD's register file, 8 leave room for a second wave, 4 for a third)
+        const size_t lds = pwr_lds_bytes(pl.pwx, pl.pwx_steps);
+        int per_cu = std::min((int)(160 * 1024 / lds), pl.pwx == 4 ? 1 : pl.pwx == 2 ? 2 : 3);
+        if (tune().wgs > 0) per_cu = std::min(per_cu, tune().wgs);
+        const int wgs = std::min(per_cu * dev->cu_count, cdiv(tiles, 4));
+        const int waves = 4 * wgs, rem = tiles % waves;
+        a.items = a.items_whole = tiles;
+        // a last round that not every wave takes part in is cut into sub-tiles of 32 output channels where that
+        // makes it shorter
+        if (rem > 0 && pl.pwx > 1 && cdiv(rem * pl.pwx, waves) < pl.pwx && !tune().nohalf) {
+            a.items_whole = tiles - rem;
+            a.items = a.items_whole + rem * pl.pwx;
+        }
+        int prc;
+        {
+            KernelTimer timer(st);
+            prc = launch_pwr_f16(pl.pwx, a, wgs, st);
+        }
+        if (prc != 0) return PHX_ERR_NOT_SUPPORTED;
+        PHX_HIP(hipGetLastError());
+        snprintf(g_name_buf, sizeof(g_name_buf), "%sqconv_%s_f16mfmapwr_p16_f16_wco%d_k%d_wgs%d_sub%d%s", g_name_prefix,
+                 map == MAP_FWD ? "fwd" : "dgrad", pl.pwx, pl.pwx_steps, wgs, a.items - a.items_whole, a.addend ? "_add" : "");
+        g_last_kernel = g_name_buf;
+        say(p, map == MAP_FWD ? "forward" : "input gradient");
+        return PHX_OK;
+    }
     const int groups_per_tile = 8 * (4 / pl.pwx);
     const int whole = cdiv(a.TGp, groups_per_tile) * pl.co_tiles;
     const int slots = 2 * dev->cu_count;  // persistent workgroups, two per CU
@@ -1099,6 +1144,7 @@ static bool plan_wgrad_f16(const Problem& p, WgPlan& best) {
     best.TPW = (shifts && p.kw % 3 == 0) ? 3 : (shifts && p.kw % 4 == 0 && !(best.MT == 2 && best.NT == 2)) ? 4 : 1;
     auto lds_need = [&](int tpw) { return (size_t)(4 * 32 * best.MT + tpw * 4 * 32 * best.NT) * 72 * 2; };
     if (lds_need(best.TPW) > 160 * 1024) best.TPW = 1;  // (four shifted copies of a 64-channel input tile do not fit)
+    if (tune().wg_tpw == 1) best.TPW = 1;
     const int CoT = 32 * best.MT, CiT = 32 * best.NT;
     // chunk list over whole planes where rows would leave their last chunk partly empty (see the kernel's header)
     best.flat = p.sh == 1 && p.sw == 1 && p.w == p.wo && p.h > 1 && p.wo >= 7 && p.wo % 8 != 0 && !tune().noflat;

@@ -324,13 +324,31 @@ PW_CASES = [c for c in FP16_CASES if c[0] in ("pw_64", "pw_ragged", "pw_7x7img",
     ("pw_c200_2x4", 5, 72, 200, 2, 4, 1, 1, 1, 1, "VALID"),      # one 8-pixel group per image, two channel tiles
     ("pw_c16_6x6_n33", 33, 16, 16, 6, 6, 1, 1, 1, 1, "VALID"),   # 32 output channels at most: one sub-tile per workgroup
     ("pw_c64_n1_12x12", 1, 48, 64, 12, 12, 1, 1, 1, 1, "VALID"),
+    # small filters (input channels a multiple of 16 from 32 on, at most 128 output channels, planes a multiple of 8):
+    # the kernel that keeps the packed filter in LDS
+    ("pwr_128_128_28", 2, 128, 128, 28, 28, 1, 1, 1, 1, "VALID"),       # fewer tiles than waves: every item one sub-tile
+    ("pwr_64_32_12x14_n3", 3, 64, 32, 12, 14, 1, 1, 1, 1, "VALID"),     # plane of 168 = 5.25 tiles: tiles straddle images
+    ("pwr_48_32_4x4_n7", 7, 48, 32, 4, 4, 1, 1, 1, 1, "VALID"),         # three K steps, two images per tile
+    ("pwr_96_64_6x4_n5", 5, 96, 64, 6, 4, 1, 1, 1, 1, "VALID"),         # six K steps, two sub-tiles, tiles straddle images
+    ("pwr_128_100_8x8_n9", 9, 128, 100, 8, 8, 1, 1, 1, 1, "VALID"),     # last sub-tile partly beyond the output channels
+    ("pwr_64_40_28_n48", 48, 64, 40, 28, 28, 1, 1, 1, 1, "VALID"),      # more tiles than waves: whole items, then a round of sub-tiles
+    ("pwr_64_8_10x4_n3", 3, 64, 8, 10, 4, 1, 1, 1, 1, "VALID"),         # one sub-tile, last tile partly beyond the last pixel
 ]
+
+
+def resident_filter_kernel(ci, co, hw, everything=False):
+    """The host's rule for the pointwise kernel with the filter resident in LDS (run_pwx in csrc/phx_qconv.hip): by
+    default the problems of at most 32 output channels that it can run, with PHX_TUNE_PWRALL (everything) all of them."""
+    sub_tiles = 4 if co > 64 else 2 if co > 32 else 1
+    can = ci % 16 == 0 and ci >= 32 and co <= 32 * sub_tiles and (ci // 16) * sub_tiles * 4096 + 32768 <= 160 * 1024 and hw % 8 == 0
+    return can and (everything or sub_tiles == 1)
 
 
 @pytest.mark.parametrize("case", PW_CASES, ids=lambda c: c[0])
 def test_pointwise_kernels_on_fp16_matrix_cores(case, tune_env):
-    """Pointwise fp16 problems have three kernels.  Planes with an even number (>= 8) of pixels run on the kernel
-    with raw operand copies ("pwx", 16-product form in either mode); PHX_TUNE_NOPWX sends them to the staged-window
+    """Pointwise fp16 problems have four kernels.  Planes with an even number (>= 8) of pixels run on the kernel
+    with raw operand copies ("pwx", 16-product form in either mode) or, where the packed filter fits LDS, on the one
+    that keeps it there ("pwr"; PHX_TUNE_NOPWR sends those to "pwx" too); PHX_TUNE_NOPWX sends them to the staged-window
     kernel the other planes use ("ldspw", in 8-product mode the 16-product kernel by default, which beats the
     factorized one there); PHX_TUNE_PW8 selects the factorized kernel.  All to the same tolerance."""
     name, n, ci, co, h, w, kh, kw, stride, dilation, padding = case
@@ -343,15 +361,22 @@ def test_pointwise_kernels_on_fp16_matrix_cores(case, tune_env):
     want_y = oracle.conv2d_fwd(g, x64, w64, b64, "hamilton")
     _, want_dx = oracle.conv2d_bwd(g, x64, w64, g64, "hamilton")
     raw_copies = (h * w) % 2 == 0 and h * w >= 8
-    for env, tag in (({}, "pwx_p16" if raw_copies else "ldspw_p16"), ({"PHX_TUNE_NOPWX": "1"}, "ldspw_p16"),
-                     ({"PHX_TUNE_NOPWX": None, "PHX_TUNE_PW8": "1"}, "ldspw_p8")):
+    # (the input gradient is the same kind of problem with the channel counts exchanged)
+    def tags(everything):
+        resident = [raw_copies and resident_filter_kernel(ci, co, h * w, everything), raw_copies and resident_filter_kernel(co, ci, h * w, everything)]
+        return ["pwr_p16" if r else "pwx_p16" if raw_copies else "ldspw_p16" for r in resident]
+    variants = [({}, tags(False)), ({"PHX_TUNE_NOPWX": "1"}, ["ldspw_p16"] * 2), ({"PHX_TUNE_NOPWX": None, "PHX_TUNE_PW8": "1"}, ["ldspw_p8"] * 2)]
+    if "pwr_p16" in tags(True):
+        variants.append(({"PHX_TUNE_PW8": None, "PHX_TUNE_PWRALL": "1"}, tags(True)))
+        variants.append(({"PHX_TUNE_PWRALL": None, "PHX_TUNE_NOPWR": "1"}, ["pwx_p16"] * 2))
+    for env, tags in variants:
         tune_env(**env)
         y = phx.conv2d_fwd(xd, wd, bd, desc)
-        assert tag in capi.last_kernel_name(), capi.last_kernel_name()
+        assert tags[0] in capi.last_kernel_name(), capi.last_kernel_name()
         _, dx = phx.conv2d_bwd(xd, wd, gd, desc)
-        assert tag in capi.last_kernel_name(), capi.last_kernel_name()
-        assert_close(y.cpu().numpy(), want_y, dtype, "fwd " + tag)
-        assert_close(dx.cpu().numpy(), want_dx, dtype, "dgrad " + tag)
+        assert tags[1] in capi.last_kernel_name(), capi.last_kernel_name()
+        assert_close(y.cpu().numpy(), want_y, dtype, "fwd " + tags[0])
+        assert_close(dx.cpu().numpy(), want_dx, dtype, "dgrad " + tags[1])
 
 
 GROUPED = [
@@ -879,11 +904,12 @@ def test_prepacked_filters_grouped_and_channels_last(case, mode):
 
 
 @pytest.mark.parametrize("mode", [16, 8])
-@pytest.mark.parametrize("shape", [(3, 40, 24, 6, 6), (2, 128, 128, 14, 14), (5, 16, 64, 7, 8), (2, 64, 16, 28, 28)],
-                         ids=lambda s: "n%d_%dto%d_%dx%d" % s)
+@pytest.mark.parametrize("shape", [(3, 40, 24, 6, 6), (2, 128, 128, 14, 14), (5, 16, 64, 7, 8), (2, 64, 16, 28, 28), (3, 32, 96, 6, 4),
+                                   (40, 16, 64, 28, 28)], ids=lambda s: "n%d_%dto%d_%dx%d" % s)
 def test_pointwise_input_gradient_adds_in_its_epilogue(shape, mode):
-    """Pointwise fp16 input gradients on even planes run the streaming kernel, which adds the tensor while it stores
-    (one launch, no pass of its own): same kernel as without the addend, the values of dx + addend bit for bit."""
+    """Pointwise fp16 input gradients on even planes run the streaming kernel or the one with the filter resident in
+    LDS; both add the tensor while they store (one launch, no pass of its own): same kernel as without the addend, the
+    values of dx + addend bit for bit."""
     n, ci, co, h, w = shape
     r = np.random.default_rng(n * 1000 + ci + co)
     gd = torch.from_numpy((0.5 * r.standard_normal((4 * n, co, h, w))).astype(np.float16)).cuda()
@@ -892,7 +918,7 @@ def test_pointwise_input_gradient_adds_in_its_epilogue(shape, mode):
     desc = phx.Conv2DDescriptor((4 * n, ci, h, w), wd.shape, 1, 1, "VALID", dtype=torch.float16, context=Ctx(mode, "full16"))
     dx = ops.conv2d_bwd_data(wd, gd, desc)
     kernel = capi.last_kernel_name()
-    assert "pwx" in kernel, kernel
+    assert ("pwr" if resident_filter_kernel(co, ci, h * w) else "pwx") in kernel, kernel
     got = ops.conv2d_bwd_data(wd, gd, desc, addend=addend)
     assert capi.last_kernel_name() == kernel + "_add"
     assert torch.equal(got, dx + addend)
