@@ -113,6 +113,8 @@ def parse():
     ap.add_argument("--frozen-filters", action="store_true",
                     help="ResNet workload: the filters do not change between steps, so no step packs them again")
     ap.add_argument("--no-graph", action="store_true", help="time the eager steps only (no HIP graph replay)")
+    ap.add_argument("--channels-last", action="store_true",
+                    help="one convolution workload on channels-last activations [4N, H, W, C] (needs --workload)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch a plain 256 MiB device copy (untimed), the yardstick for HBM byte counters")
@@ -348,11 +350,12 @@ def run_conv(name, mode, policy, args, traffic_table):
     dev = torch.device("cuda:0")
     torch.manual_seed(0x5EED + sorted(CONVS).index(name))
     scale = 1.0 if dt == "f32" else 0.5
-    x = (scale * torch.randn(4 * n, ci, h, w, device=dev)).to(dtype)
+    cl = bool(getattr(args, "channels_last", False))
+    x = (scale * torch.randn((4 * n, h, w, ci) if cl else (4 * n, ci, h, w), device=dev)).to(dtype)
     wt = (scale * torch.randn(4, co, ci, k, k, device=dev) * (2.0 / (ci * k * k)) ** 0.5).to(dtype)
-    desc = phx.Conv2DDescriptor(x.shape, wt.shape, 1, 1, padding, dtype=dtype, context=ctx)
+    desc = phx.Conv2DDescriptor(x.shape, wt.shape, 1, 1, padding, dtype=dtype, context=ctx, data_format="NHWC" if cl else "NCHW")
     gr = (scale * torch.randn(desc.output_shape, device=dev)).to(dtype)
-    ho, wo = desc.output_shape[2:]
+    ho, wo = desc.output_shape[1:3] if cl else desc.output_shape[2:]
     y = torch.empty(desc.output_shape, dtype=dtype, device=dev)
     dx = torch.empty_like(x)
     dw = torch.empty_like(wt)
@@ -398,7 +401,8 @@ def run_conv(name, mode, policy, args, traffic_table):
     torch.cuda.empty_cache()
     return {
         "workload": "%s: quaternion conv %dx%d stride 1, N=%d (4N=%d rows), %d->%d q-channels, %dx%d, "
-                    "fwd+input-grad+filter-grad" % (name, k, k, n, 4 * n, ci, co, h, w),
+                    "fwd+input-grad+filter-grad%s" % (name, k, k, n, 4 * n, ci, co, h, w, ", channels-last activations" if cl else ""),
+        "data_format": "NHWC" if cl else "NCHW",
         "n": n, "product_mode": mode, "fp16_policy": policy, "padding": padding, "dtype": dt,
         "value": value, "unit": "TFLOP/s", "ms_per_step": t.ms_per_step, "ms_per_step_eager": t.ms_per_step_eager,
         "hip_graph": t.graph, "images_per_s": n / (t.ms_per_step * 1e-3),
@@ -656,6 +660,9 @@ def main():
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (--gpus %d refused)" % args.gpus,
               file=sys.stderr)
+        return 2
+    if args.channels_last and args.workload not in CONVS:
+        print("--channels-last takes one convolution workload (--workload c2_.. / c3_.. / c4_..)", file=sys.stderr)
         return 2
     import phoenix_core_amd  # noqa: F401  (fails loudly when the HIP library is missing)
     mode = default_mode(args)

@@ -72,3 +72,9 @@ def test_more_than_one_gpu_is_refused(capsys, monkeypatch):
     monkeypatch.setattr(sys, "argv", ["bench.py", "--gpus", "2"])
     assert bench.main() == 2
     assert "one GPU" in capsys.readouterr().err
+
+
+def test_channels_last_needs_one_convolution_workload(capsys, monkeypatch):
+    monkeypatch.setattr(sys, "argv", ["bench.py", "--channels-last"])
+    assert bench.main() == 2
+    assert "--workload" in capsys.readouterr().err
