@@ -253,6 +253,15 @@ __device__ __forceinline__ const T* zero_ptr() {
 
 // A rectangular window of a component-stacked NCHW tensor t[4][N][C][Hd][Wd], seen through an
 // optional zero-insertion (virtual coordinate v maps to stored v/u when v % u == 0, else zero).
+// One launch for all groups of a grouped convolution: the workgroups of grid row blockIdx.y work on group blockIdx.y,
+// whose tensors lie blockIdx.y times a byte step behind group 0's (a grid of one row, i.e. no shift, otherwise).
+__device__ __forceinline__ const void* group_shift(const void* p, long step) {
+    return p ? static_cast<const char*>(p) + (long)blockIdx.y * step : nullptr;
+}
+__device__ __forceinline__ void* group_shift(void* p, long step) {
+    return p ? static_cast<char*>(p) + (long)blockIdx.y * step : nullptr;
+}
+
 struct TileSrc {
     const void* base;
     long comp_stride;  // elements between components

@@ -117,7 +117,8 @@ __device__ __forceinline__ void stage_store16_pairs(f16x8* dst, const unsigned i
 //            4x4 block, negative entries by flipping the sign bits of the activation operand.
 //   MODE 8 : 8 MFMAs per step and column tile on lanes formed with packed fp16 adds.
 template <int MODE, int WCO, int NTW, int P2LOG, bool PAIRS>
-__global__ void __launch_bounds__(WG_THREADS, (MODE == 8 || NTW == 1) ? 2 : 1) qconv_fwd_f16_kernel(const ConvArgs P) {
+__global__ void __launch_bounds__(WG_THREADS, (MODE == 8 || NTW == 1) ? 2 : 1) qconv_fwd_f16_kernel(const ConvArgs P0) {
+    const ConvArgs P = group_view(P0);
     constexpr int CK = F16_CK;
     constexpr int WPX = 4 / WCO;
     constexpr int NACC = (MODE == 16) ? 4 : 8;
@@ -280,7 +281,8 @@ __device__ __forceinline__ void pack_filters_f16_body(const PackArgs& P, long fi
 }
 
 template <int MODE, int MAP>
-__global__ void __launch_bounds__(WG_THREADS) pack_filters_f16_kernel(const PackArgs P) {
+__global__ void __launch_bounds__(WG_THREADS) pack_filters_f16_kernel(const PackArgs P0) {
+    const PackArgs P = group_view(P0);
     pack_filters_f16_body<MODE, MAP>(P, (long)blockIdx.x * blockDim.x + threadIdx.x, (long)gridDim.x * blockDim.x);
 }
 
@@ -547,7 +549,8 @@ __device__ __forceinline__ void lane_step(const f16x8 (&x)[4], f16x8 (&L)[8], in
 // XREAL (16-product, chunk staging): the input holds its real component only (P.in.ncomp == 1); the twelve
 // products with the absent components and their operand reads are left out at compile time.
 template <int MODE, int WCO, int NTW, int P2LOG, bool CHUNKS, bool EARLY = false, bool XREAL = false>
-__global__ void __launch_bounds__(WG_THREADS, (MODE == 16 && NTW == 1) ? 2 : 1) qconv_fwd_f16_lds_kernel(const ConvArgs P) {
+__global__ void __launch_bounds__(WG_THREADS, (MODE == 16 && NTW == 1) ? 2 : 1) qconv_fwd_f16_lds_kernel(const ConvArgs P0) {
+    const ConvArgs P = group_view(P0);
     static_assert(!EARLY || CHUNKS, "early activation requests belong to chunk staging");
     static_assert(!XREAL || (MODE == 16 && CHUNKS), "the real-input variant is a 16-product kernel with chunk staging");
     constexpr int NP = XREAL ? 1 : 4;          // input components that take part
@@ -916,7 +919,9 @@ __device__ __forceinline__ void pack_filters_f16_lds_body(const PackLdsArgs& A, 
 }
 
 template <int MODE, int MAP>
-__global__ void __launch_bounds__(WG_THREADS) pack_filters_f16_lds_kernel(const PackLdsArgs A) {
+__global__ void __launch_bounds__(WG_THREADS) pack_filters_f16_lds_kernel(const PackLdsArgs A0) {
+    PackLdsArgs A = A0;
+    A.base = group_view(A0.base);
     pack_filters_f16_lds_body<MODE, MAP>(A, (long)blockIdx.x * blockDim.x + threadIdx.x, (long)gridDim.x * blockDim.x);
 }
 
@@ -1002,7 +1007,8 @@ __device__ __forceinline__ WgChunk wg_chunk(const WgradArgs& P, int tile, int j)
 }
 
 template <int MODE, int MT, int NT, int TPW, int SW, bool CL = false>
-__global__ void __launch_bounds__(WG_THREADS) qconv_wgrad_f16_kernel(const WgradArgs P) {
+__global__ void __launch_bounds__(WG_THREADS) qconv_wgrad_f16_kernel(const WgradArgs P0) {
+    const WgradArgs P = group_view(P0);
     static_assert(TPW == 1 || ((TPW == 3 || TPW == 4) && SW == 1), "shifted copies need unit stride");
     static_assert(!CL || (MT == 2 && NT == 2 && SW == 1 && (TPW == 1 || TPW == 3)), "channels-last staging: 64x64 tiles, unit stride");
     constexpr int CoT = 32 * MT, CiT = 32 * NT;

@@ -31,7 +31,19 @@ struct ConvArgs {
     int nchunks;        // ceil(Cin / CK) for the kernel's chunk size CK
     int vec;            // output pixels a lane stores at once (4, 2 or 1): divides TW and Wout
     int nhwc;           // the output is channels-last, out[4][N][Hout][Wout][CoutS] (fp16 chunk-staging kernel only)
+    int groups;         // grid rows: the groups of a grouped convolution run by this one launch (1 otherwise)
+    long g_in, g_w, g_bias, g_out;  // bytes from one group's input / packed filters / bias / output to the next group's
 };
+
+// the arguments as group blockIdx.y sees them
+__device__ __forceinline__ ConvArgs group_view(const ConvArgs& P0) {
+    ConvArgs P = P0;
+    P.in.base = group_shift(P0.in.base, P0.g_in);
+    P.wpk = group_shift(P0.wpk, P0.g_w);
+    P.bias = group_shift(P0.bias, P0.g_bias);
+    P.out = group_shift(P0.out, P0.g_out);
+    return P;
+}
 
 // ---------------------------------------------------------------------------------------------
 // Epilogue shared by the forward / input-gradient kernels (32x32 MFMA tiles: a lane holds one pixel
@@ -360,7 +372,8 @@ __device__ __forceinline__ void stage_vec_store_scalar(float* lds, const f32x4 (
 //   MODE 16: acc[q] += W_{p^q} * (+-x_p), 16 MFMAs per K step, filters reused across the 4x4 block.
 //   MODE 8 : acc[i] += R_i * L_i with the 8 lanes L_i formed in registers, 8 MFMAs per K step.
 template <typename TS, int MODE, int WCO, int NTW, int CK, int P2LOG, bool VSTG>
-__global__ void __launch_bounds__(WG_THREADS, (MODE == 8 || NTW == 1) ? 2 : 1) qconv_fwd_f32_kernel(const ConvArgs P) {
+__global__ void __launch_bounds__(WG_THREADS, (MODE == 8 || NTW == 1) ? 2 : 1) qconv_fwd_f32_kernel(const ConvArgs P0) {
+    const ConvArgs P = group_view(P0);
     constexpr int WPX = 4 / WCO;
     constexpr int NACC = (MODE == 16) ? 4 : 8;
     constexpr int WC = (MODE == 16) ? 4 : 8;  // packed filter values per lane and K step
@@ -518,7 +531,16 @@ struct PackArgs {
     int khm, khs, kwm, kws;  // input gradient: tap (u, v) of the correlation is filter tap (khm - u*khs, kwm - v*kws)
     int rows, red;    // correlation: output channels (rows) and reduced channels
     int row_tiles, nchunks;
+    int groups;       // grid rows: the groups packed by this one launch (1 otherwise)
+    long g_w, g_out;  // bytes from one group's filter / packed image to the next group's
 };
+
+__device__ __forceinline__ PackArgs group_view(const PackArgs& P0) {
+    PackArgs P = P0;
+    P.w = group_shift(P0.w, P0.g_w);
+    P.out = group_shift(P0.out, P0.g_out);
+    return P;
+}
 
 // (the packing bodies take the thread's first index and the stride of its loop, so that one launch can also pack
 // several filter images side by side: pack_jobs_kernel)
@@ -571,7 +593,8 @@ __device__ __forceinline__ void pack_filters_f32_body(const PackArgs& P, long fi
 }
 
 template <typename TS, int MODE, int MAP>
-__global__ void __launch_bounds__(WG_THREADS) pack_filters_f32_kernel(const PackArgs P) {
+__global__ void __launch_bounds__(WG_THREADS) pack_filters_f32_kernel(const PackArgs P0) {
+    const PackArgs P = group_view(P0);
     pack_filters_f32_body<TS, MODE, MAP>(P, (long)blockIdx.x * blockDim.x + threadIdx.x, (long)gridDim.x * blockDim.x);
 }
 
@@ -597,13 +620,24 @@ struct WgradArgs {
     int groups_per_row; // tap groups per filter row
     int cpr, nchunks, ntiles, zsplit;  // fp16 kernel: 8-pixel chunks per output row / in total, pixel tiles, reduction slices
     int flat, rows;                    // fp16 kernel: chunk list over whole planes (rows = 1) or over the rows of an image
+    int groups;                        // grid rows: the groups of a grouped convolution run by this one launch (1 otherwise)
+    long g_x, g_g, g_partial;          // bytes from one group's input / gradient / partial sums to the next group's
 };
+
+__device__ __forceinline__ WgradArgs group_view(const WgradArgs& P0) {
+    WgradArgs P = P0;
+    P.x.base = group_shift(P0.x.base, P0.g_x);
+    P.g.base = group_shift(P0.g.base, P0.g_g);
+    P.partial = static_cast<float*>(group_shift(static_cast<void*>(P0.partial), P0.g_partial));
+    return P;
+}
 
 //   KSETS = 2: eight waves, two per SIMD (while one forms lanes or waits for LDS, the other's matrix
 //   instructions run); the second set of four takes the odd K steps of every tile into accumulators of its
 //   own, which go to a reduction slice of their own (slice z*KSETS + set).  Every thread stages half as much.
 template <typename TS, int MODE, int TPW, bool VEC, int KSETS>
-__global__ void __launch_bounds__(WG_THREADS * KSETS) qconv_wgrad_f32_kernel(const WgradArgs P) {
+__global__ void __launch_bounds__(WG_THREADS * KSETS) qconv_wgrad_f32_kernel(const WgradArgs P0) {
+    const WgradArgs P = group_view(P0);
     constexpr int CT = 64;
     constexpr int NT = WG_THREADS * KSETS;
     constexpr int EV = 8 / KSETS;  // vector loads per thread, tile and operand
@@ -844,7 +878,16 @@ struct ReduceArgs {
     void* dw;
     long wcs, so, si, skh, skw;
     int Z, Co, Ci, Kh, Kw, CoP, CiP;
+    int groups;              // grid rows: the groups reduced by this one launch (1 otherwise)
+    long g_partial, g_dw;    // bytes from one group's partial sums / filter gradient to the next group's
 };
+
+__device__ __forceinline__ ReduceArgs group_view(const ReduceArgs& P0) {
+    ReduceArgs P = P0;
+    P.partial = static_cast<const float*>(group_shift(static_cast<const void*>(P0.partial), P0.g_partial));
+    P.dw = group_shift(P0.dw, P0.g_dw);
+    return P;
+}
 
 // dw(r, co, ci, kh, kw) = sum_z partial[z][tap][r][co][ci].  A thread owns four consecutive input channels of
 // one (tap, component, output channel) -- 16-byte loads, the padded row length CiP is a multiple of 4.  The
@@ -854,7 +897,8 @@ struct ReduceArgs {
 __host__ __device__ inline int reduce_slices(int Z) { return Z >= 7 ? 8 : Z >= 4 ? 4 : Z >= 2 ? 2 : 1; }
 
 template <typename TS>
-__global__ void __launch_bounds__(WG_THREADS) reduce_wgrad_kernel(const ReduceArgs P) {
+__global__ void __launch_bounds__(WG_THREADS) reduce_wgrad_kernel(const ReduceArgs P0) {
+    const ReduceArgs P = group_view(P0);
     __shared__ f32x4 part[WG_THREADS];
     const int taps = P.Kh * P.Kw;
     const int ci4s = (P.Ci + 3) >> 2;

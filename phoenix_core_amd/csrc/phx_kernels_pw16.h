@@ -75,7 +75,20 @@ struct PwxArgs {
     int items;              // work items: whole items (pixel tiles * co_tiles), the last ones possibly as pairs of half items
     int items_whole;        // NCHW kernel: work items below this index are whole items, the others half items
     int NP;                 // channels-last kernel: pixels in all, N * HW
+    int groups;             // grid rows: the groups of a grouped convolution run by this one launch (1 otherwise)
+    long g_in, g_w, g_bias, g_out;  // bytes from one group's input / packed filters / bias / output (and addend) to the next group's
 };
+
+// the arguments as group blockIdx.y sees them
+__device__ __forceinline__ PwxArgs group_view(const PwxArgs& P0) {
+    PwxArgs P = P0;
+    P.in = static_cast<const _Float16*>(group_shift(static_cast<const void*>(P0.in), P0.g_in));
+    P.wpk = static_cast<const f16x8*>(group_shift(static_cast<const void*>(P0.wpk), P0.g_w));
+    P.bias = static_cast<const _Float16*>(group_shift(static_cast<const void*>(P0.bias), P0.g_bias));
+    P.out = static_cast<_Float16*>(group_shift(static_cast<void*>(P0.out), P0.g_out));
+    P.addend = static_cast<const _Float16*>(group_shift(static_cast<const void*>(P0.addend), P0.g_out));
+    return P;
+}
 
 template <int WCO>
 struct PwxShape {
@@ -106,7 +119,8 @@ struct PwxShape {
 // ADD: the instance that adds P.addend to what it stores (the plain instance carries none of that code: the extra
 // registers of the addend's prefetch cost the plain kernel 4 % where both were one)
 template <int WCO, bool ADD = false>
-__global__ void __launch_bounds__(WG_THREADS, 2) qconv_pwx_f16_kernel(const PwxArgs P) {
+__global__ void __launch_bounds__(WG_THREADS, 2) qconv_pwx_f16_kernel(const PwxArgs P0) {
+    const PwxArgs P = group_view(P0);
     using S = PwxShape<WCO>;
     constexpr int WPX = S::WPX, GPT = S::GPT, ROWDW = S::ROWDW, WV = S::WV, XV = S::XV, RF = S::RF, RA = S::RA;
     constexpr int DF = RF - 1, DA = RA - 1;  // steps the filter / activation copies run ahead of the products
@@ -644,7 +658,9 @@ __device__ __forceinline__ void pack_filters_pwx_body(const PackPwxArgs& A, long
 }
 
 template <int MAP>
-__global__ void __launch_bounds__(WG_THREADS) pack_filters_pwx_kernel(const PackPwxArgs A) {
+__global__ void __launch_bounds__(WG_THREADS) pack_filters_pwx_kernel(const PackPwxArgs A0) {
+    PackPwxArgs A = A0;
+    A.base = group_view(A0.base);
     pack_filters_pwx_body<MAP>(A, (long)blockIdx.x * blockDim.x + threadIdx.x, (long)gridDim.x * blockDim.x);
 }
 

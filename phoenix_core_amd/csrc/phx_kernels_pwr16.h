@@ -48,7 +48,8 @@ __device__ __forceinline__ float agpr_value(float a) {
 // ADD: the instance that adds P.addend (a tensor laid out like the output; an fp16 addition to the rounded result)
 // to what it stores.
 template <int WCO, bool ADD = false>
-__global__ void __launch_bounds__(WG_THREADS, 1) qconv_pwr_f16_kernel(const PwxArgs P) {
+__global__ void __launch_bounds__(WG_THREADS, 1) qconv_pwr_f16_kernel(const PwxArgs P0) {
+    const PwxArgs P = group_view(P0);
     extern __shared__ f16x8 lds16[];  // filters [K step][sub-tile][component][lane], then the waves' rings
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);

@@ -19,6 +19,9 @@ struct BigLds {
     static inline const bool registered = register_big_lds_kernel(reinterpret_cast<const void*>(Kernel));
 };
 
+// grid rows of a launch that runs every group of a grouped convolution (one row otherwise)
+inline unsigned int grid_rows(int groups) { return groups > 1 ? (unsigned int)groups : 1u; }
+
 bool tuning_noearly();  // PHX_TUNE_NOEARLY, read once with the other planner overrides
 
 // which instantiation of the forward / input-gradient kernel to run

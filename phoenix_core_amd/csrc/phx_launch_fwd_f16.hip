@@ -9,7 +9,7 @@ static int launch_variant16(const FwdVariant& v, const ConvArgs& a, hipStream_t 
     constexpr int P2A = 8, P2B = PAIRS ? 8 : 7;  // the pair path has a single staging shape
 #define PHX_CASE(WCO_, NTW_, P2_)                                                                             \
     if (v.WCO == WCO_ && v.NTW == NTW_ && (PAIRS || v.P2LOG == P2_)) {                                        \
-        hipLaunchKernelGGL((qconv_fwd_f16_kernel<MODE, WCO_, NTW_, P2_, PAIRS>), dim3(v.wgs),                 \
+        hipLaunchKernelGGL((qconv_fwd_f16_kernel<MODE, WCO_, NTW_, P2_, PAIRS>), dim3(v.wgs, grid_rows(a.groups)),                 \
                            dim3(WG_THREADS), v.lds_bytes, st, a);                                             \
         return 0;                                                                                             \
     }
@@ -36,7 +36,7 @@ static int launch_lds16(const FwdVariant& v, const ConvArgs& a, hipStream_t st) 
     if (v.WCO == WCO_ && v.NTW == NTW_ && (CHUNKS || v.P2LOG == P2_)) {                                        \
         constexpr auto kernel = qconv_fwd_f16_lds_kernel<16, WCO_, NTW_, P2_, CHUNKS>;              \
         if (!BigLds<kernel>::registered) return -1; /* dynamic LDS opt-in at set-up, see BigLds */            \
-        hipLaunchKernelGGL(kernel, dim3(v.wgs), dim3(WG_THREADS), v.lds_bytes, st, a);                        \
+        hipLaunchKernelGGL(kernel, dim3(v.wgs, grid_rows(a.groups)), dim3(WG_THREADS), v.lds_bytes, st, a);                        \
         return 0;                                                                                             \
     }
     if constexpr (CHUNKS) {
@@ -45,13 +45,13 @@ static int launch_lds16(const FwdVariant& v, const ConvArgs& a, hipStream_t st) 
             if (v.WCO == 1) {
                 constexpr auto kernel = qconv_fwd_f16_lds_kernel<16, 1, 1, 8, true, true>;
                 if (!BigLds<kernel>::registered) return -1;
-                hipLaunchKernelGGL(kernel, dim3(v.wgs), dim3(WG_THREADS), v.lds_bytes, st, a);
+                hipLaunchKernelGGL(kernel, dim3(v.wgs, grid_rows(a.groups)), dim3(WG_THREADS), v.lds_bytes, st, a);
                 return 0;
             }
             if (v.WCO == 2) {
                 constexpr auto kernel = qconv_fwd_f16_lds_kernel<16, 2, 1, 8, true, true>;
                 if (!BigLds<kernel>::registered) return -1;
-                hipLaunchKernelGGL(kernel, dim3(v.wgs), dim3(WG_THREADS), v.lds_bytes, st, a);
+                hipLaunchKernelGGL(kernel, dim3(v.wgs, grid_rows(a.groups)), dim3(WG_THREADS), v.lds_bytes, st, a);
                 return 0;
             }
         }
@@ -72,7 +72,7 @@ int launch_fwd_f16(const FwdVariant& v, const ConvArgs& a, hipStream_t st) {
 }
 
 int launch_pack_filters_f16(const FwdVariant& v, const PackArgs& a, int blocks, hipStream_t st) {
-    const dim3 g(blocks), b(WG_THREADS);
+    const dim3 g(blocks, grid_rows(a.groups)), b(WG_THREADS);
     if (v.lds_filters) {
         PackLdsArgs la{a, v.WCO, v.ngroups, v.pw};
         if (v.mode == 16 && v.map == MAP_FWD) hipLaunchKernelGGL((pack_filters_f16_lds_kernel<16, MAP_FWD>), g, b, 0, st, la);

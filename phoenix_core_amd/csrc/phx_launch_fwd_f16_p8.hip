@@ -10,7 +10,7 @@ static int launch_lds8_impl(const FwdVariant& v, const ConvArgs& a, hipStream_t 
         constexpr auto kernel = qconv_fwd_f16_lds_kernel<8, WCO_, NTW_, 8, true>;                             \
         /* more than 64 KiB of dynamic LDS: opted in per device at set-up, see BigLds */                           \
         if (!BigLds<kernel>::registered) return -1;                                                                \
-        hipLaunchKernelGGL(kernel, dim3(v.wgs), dim3(WG_THREADS), v.lds_bytes, st, a);                             \
+        hipLaunchKernelGGL(kernel, dim3(v.wgs, grid_rows(a.groups)), dim3(WG_THREADS), v.lds_bytes, st, a);                             \
         return 0;                                                                                                  \
     }
     PHX_CASE(1, 1) PHX_CASE(1, 2) PHX_CASE(2, 1) PHX_CASE(2, 2)

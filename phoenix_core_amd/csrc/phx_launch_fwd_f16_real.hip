@@ -10,7 +10,7 @@ int launch_fwd_f16_lds16_real(const FwdVariant& v, const ConvArgs& a, hipStream_
     if (v.WCO == WCO_ && v.NTW == NTW_) {                                                                      \
         constexpr auto kernel = qconv_fwd_f16_lds_kernel<16, WCO_, NTW_, 8, true, false, true>;                \
         if (!BigLds<kernel>::registered) return -1; /* dynamic LDS opt-in at set-up, see BigLds */             \
-        hipLaunchKernelGGL(kernel, dim3(v.wgs), dim3(WG_THREADS), v.lds_bytes, st, a);                         \
+        hipLaunchKernelGGL(kernel, dim3(v.wgs, grid_rows(a.groups)), dim3(WG_THREADS), v.lds_bytes, st, a);                         \
         return 0;                                                                                              \
     }
     PHX_CASE(1, 1) PHX_CASE(1, 2) PHX_CASE(2, 1) PHX_CASE(2, 2) PHX_CASE(4, 1) PHX_CASE(4, 2)

@@ -7,7 +7,7 @@ template <typename TS, int MODE>
 static int launch_variant(const FwdVariant& v, const ConvArgs& a, hipStream_t st) {
 #define PHX_CASE(WCO_, NTW_, CK_, P2_, VS_)                                                                   \
     if (v.WCO == WCO_ && v.NTW == NTW_ && v.CK == CK_ && v.P2LOG == P2_ && v.vstage == VS_) {                 \
-        hipLaunchKernelGGL((qconv_fwd_f32_kernel<TS, MODE, WCO_, NTW_, CK_, P2_, VS_>), dim3(v.wgs),          \
+        hipLaunchKernelGGL((qconv_fwd_f32_kernel<TS, MODE, WCO_, NTW_, CK_, P2_, VS_>), dim3(v.wgs, grid_rows(a.groups)),          \
                            dim3(WG_THREADS), v.lds_bytes, st, a);                                             \
         return 0;                                                                                             \
     }
@@ -37,7 +37,7 @@ int launch_fwd_f32(const FwdVariant& v, const ConvArgs& a, hipStream_t st) {
 
 template <typename TS>
 static int pack_ts(const FwdVariant& v, const PackArgs& a, int blocks, hipStream_t st) {
-    const dim3 g(blocks), b(WG_THREADS);
+    const dim3 g(blocks, grid_rows(a.groups)), b(WG_THREADS);
     if (v.mode == 16 && v.map == MAP_FWD) hipLaunchKernelGGL((pack_filters_f32_kernel<TS, 16, MAP_FWD>), g, b, 0, st, a);
     else if (v.mode == 16) hipLaunchKernelGGL((pack_filters_f32_kernel<TS, 16, MAP_DGRAD>), g, b, 0, st, a);
     else if (v.map == MAP_FWD) hipLaunchKernelGGL((pack_filters_f32_kernel<TS, 8, MAP_FWD>), g, b, 0, st, a);

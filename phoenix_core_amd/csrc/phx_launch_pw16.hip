@@ -8,7 +8,7 @@ template <int WCO, bool ADD>
 static int launch_pwx_one(const PwxArgs& a, int blocks, hipStream_t st) {
     constexpr auto kernel = qconv_pwx_f16_kernel<WCO, ADD>;
     if (!BigLds<kernel>::registered) return -1;  // more than 64 KiB of dynamic LDS: opted in per device at set-up, see BigLds
-    hipLaunchKernelGGL(kernel, dim3(blocks), dim3(WG_THREADS), PwxShape<WCO>::lds_bytes_nchw, st, a);
+    hipLaunchKernelGGL(kernel, dim3(blocks, grid_rows(a.groups)), dim3(WG_THREADS), PwxShape<WCO>::lds_bytes_nchw, st, a);
     return 0;
 }
 
@@ -46,8 +46,9 @@ int launch_pack_filters_pwx(int map, int WCO, int nsteps, const PackArgs& a, hip
     PackPwxArgs pa{a, WCO, nsteps};
     const long total = (long)a.row_tiles * nsteps * WCO * 4 * 64;
     const int blocks = (int)std::min<long>((total + WG_THREADS - 1) / WG_THREADS, 4096);
-    if (map == MAP_FWD) hipLaunchKernelGGL((pack_filters_pwx_kernel<MAP_FWD>), dim3(blocks), dim3(WG_THREADS), 0, st, pa);
-    else hipLaunchKernelGGL((pack_filters_pwx_kernel<MAP_DGRAD>), dim3(blocks), dim3(WG_THREADS), 0, st, pa);
+    const dim3 grid(blocks, grid_rows(a.groups));
+    if (map == MAP_FWD) hipLaunchKernelGGL((pack_filters_pwx_kernel<MAP_FWD>), grid, dim3(WG_THREADS), 0, st, pa);
+    else hipLaunchKernelGGL((pack_filters_pwx_kernel<MAP_DGRAD>), grid, dim3(WG_THREADS), 0, st, pa);
     return 0;
 }
 

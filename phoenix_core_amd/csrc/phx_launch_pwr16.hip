@@ -8,7 +8,7 @@ template <int WCO, bool ADD>
 static int launch_pwr_one(const PwxArgs& a, int blocks, size_t lds_bytes, hipStream_t st) {
     constexpr auto kernel = qconv_pwr_f16_kernel<WCO, ADD>;
     if (!BigLds<kernel>::registered) return -1;  // more than 64 KiB of dynamic LDS: opted in per device at set-up, see BigLds
-    hipLaunchKernelGGL(kernel, dim3(blocks), dim3(WG_THREADS), lds_bytes, st, a);
+    hipLaunchKernelGGL(kernel, dim3(blocks, grid_rows(a.groups)), dim3(WG_THREADS), lds_bytes, st, a);
     return 0;
 }
 

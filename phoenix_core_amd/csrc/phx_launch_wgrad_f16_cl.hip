@@ -8,7 +8,7 @@ template <int TPW>
 static int launch_one(const WgradArgs& a, int nblocks, size_t lds_bytes, hipStream_t st) {
     constexpr auto kernel = qconv_wgrad_f16_kernel<16, 2, 2, TPW, 1, true>;
     if (!BigLds<kernel>::registered) return -1;  // (always true: naming the member makes the registration happen while the library loads)
-    hipLaunchKernelGGL(kernel, dim3(nblocks), dim3(WG_THREADS), lds_bytes, st, a);
+    hipLaunchKernelGGL(kernel, dim3(nblocks, grid_rows(a.groups)), dim3(WG_THREADS), lds_bytes, st, a);
     return 0;
 }
 

@@ -29,8 +29,8 @@ int launch_reduce_wgrad(bool half_storage, const ReduceArgs& a, hipStream_t st) 
     const long groups = 4L * a.Kh * a.Kw * a.Co * ((a.Ci + 3) / 4);
     const int per_wg = WG_THREADS / reduce_slices(a.Z);
     const int blocks = (int)((groups + per_wg - 1) / per_wg);
-    if (half_storage) hipLaunchKernelGGL((reduce_wgrad_kernel<_Float16>), dim3(blocks), dim3(WG_THREADS), 0, st, a);
-    else hipLaunchKernelGGL((reduce_wgrad_kernel<float>), dim3(blocks), dim3(WG_THREADS), 0, st, a);
+    if (half_storage) hipLaunchKernelGGL((reduce_wgrad_kernel<_Float16>), dim3(blocks, grid_rows(a.groups)), dim3(WG_THREADS), 0, st, a);
+    else hipLaunchKernelGGL((reduce_wgrad_kernel<float>), dim3(blocks, grid_rows(a.groups)), dim3(WG_THREADS), 0, st, a);
     return 0;
 }
 

@@ -34,6 +34,7 @@ struct Tuning {
     bool nopwr = false;               // PHX_TUNE_NOPWR: pointwise fp16 problems with small filters stay on the streaming kernel
     bool pwrall = false;              // PHX_TUNE_PWRALL: ... and every problem that kernel can run goes to it (not only those of at most 32 output channels)
     bool nowincl = false;             // PHX_TUNE_NOWINCL: channels-last windowed problems go through the transposes
+    bool nogroupbatch = false;        // PHX_TUNE_NOGROUPBATCH: a grouped convolution runs group after group
     int wincl_max = 3072;             // PHX_TUNE_WINCL_MAX: largest channels x taps that runs on channels-last tensors directly
     bool nosmalldense = false;        // PHX_TUNE_NOSMALLDENSE: small Dense problems stay on the matrix-core kernels
     int vec = 0;                      // PHX_TUNE_VEC (0 = unset)
@@ -61,6 +62,7 @@ struct Tuning {
         nopwr = getenv("PHX_TUNE_NOPWR") != nullptr;
         pwrall = getenv("PHX_TUNE_PWRALL") != nullptr;
         nowincl = getenv("PHX_TUNE_NOWINCL") != nullptr;
+        nogroupbatch = getenv("PHX_TUNE_NOGROUPBATCH") != nullptr;
         if (const char* e = getenv("PHX_TUNE_WINCL_MAX")) wincl_max = atoi(e);
         nosmalldense = getenv("PHX_TUNE_NOSMALLDENSE") != nullptr;
         if (const char* e = getenv("PHX_TUNE_VEC")) vec = atoi(e);
@@ -195,6 +197,22 @@ static thread_local const char* g_last_kernel = "";
 static thread_local char g_name_buf[160];
 static thread_local const char* g_name_prefix = "";  // "s2d_" while a rewritten problem runs
 static thread_local bool g_window_cl = false;        // run_corr reads and writes channels-last tensors (see nhwc_window_native)
+// All groups of a grouped convolution in one launch per kernel (see group_batchable): the number of groups and the
+// bytes from one group's slice of the caller's tensors to the next group's.  The runners below give every kernel a
+// grid row per group and these steps (their own packed images and partial sums lie group after group in the workspace).
+struct GroupBatch {
+    int n = 1;
+    size_t x = 0, y = 0, w = 0, b = 0;
+};
+static thread_local GroupBatch g_batch;
+// (kernel labels of launches that run every group carry the number of groups)
+static void label_groups(int groups) {
+    if (groups <= 1) return;
+    const size_t len = strlen(g_name_buf);
+    if (len < sizeof(g_name_buf)) snprintf(g_name_buf + len, sizeof(g_name_buf) - len, "_groups%d", groups);
+}
+static const void* at_bytes(const void* ptr, size_t off) { return ptr ? static_cast<const char*>(ptr) + off : nullptr; }
+static void* at_bytes(void* ptr, size_t off) { return ptr ? static_cast<char*>(ptr) + off : nullptr; }
 
 // Filters packed ahead of the passes that use them (phx_qconv2d_pack_filters and the *_prepacked entry points).
 // The forward and input-gradient code paths run as always, and this thread's session tells the places that pack
@@ -743,17 +761,26 @@ static int record_pwx_job(const PackArgs& pa, int map, int wco, int nsteps) {
 
 static int run_pwx(const Problem& p, const Corr& c, const FwdPlan& pl, int map, hipStream_t st, const void* in, const void* w,
                    const void* bias, void* out, void* ws, size_t ws_bytes) {
-    const PackSlot slot = pack_slot(ws, ws_bytes, pl.wpk_bytes);
+    const GroupBatch gb = g_batch;
+    const size_t image = align_up(pl.wpk_bytes, 256);  // (group after group where one launch runs them all)
+    const PackSlot slot = pack_slot(ws, ws_bytes, gb.n > 1 ? image * gb.n : pl.wpk_bytes);
     if (slot.rc != PHX_OK) return slot.rc;
     ws = slot.dst;
     PackArgs pa{};
+    pa.groups = gb.n; pa.g_w = (long)gb.w; pa.g_out = (long)image;
     pa.w = w; pa.out = ws;
     pa.wcs = p.fs.wcs; pa.so = p.fs.so; pa.si = p.fs.si; pa.skh = p.fs.skh; pa.skw = p.fs.skw;
     pa.Co = p.co; pa.Ci = p.ci; pa.Kh = 1; pa.Kw = 1;
     pa.khm = c.khm; pa.khs = c.khs; pa.kwm = c.kwm; pa.kws = c.kws;
     pa.rows = c.Cout; pa.red = c.Cin; pa.row_tiles = pl.co_tiles; pa.nchunks = pl.pwx_steps;
     if (slot.pack_now && launch_pack_filters_pwx(map, pl.pwx, pl.pwx_steps, pa, st) != 0) return PHX_ERR_NOT_SUPPORTED;
-    if (const int rrc = record_pwx_job(pa, map, pl.pwx, pl.pwx_steps)) return rrc;
+    for (int g = 0; g < gb.n; ++g) {  // (the combined packing launch takes one job per image)
+        PackArgs one = pa;
+        one.groups = 1;
+        one.w = at_bytes(pa.w, g * gb.w);
+        one.out = at_bytes(pa.out, g * image);
+        if (const int rrc = record_pwx_job(one, map, pl.pwx, pl.pwx_steps)) return rrc;
+    }
     if (!slot.compute) return PHX_OK;
     DeviceState* dev = nullptr;
     if (const int rc = device_state(&dev)) return rc;
@@ -765,6 +792,8 @@ static int run_pwx(const Problem& p, const Corr& c, const FwdPlan& pl, int map, 
     a.N = c.N; a.Cin = c.Cin; a.CinS = cin_mem; a.Cout = c.Cout; a.CoutS = cout_mem; a.HW = c.Win;
     a.GI = cdiv(c.Win, 8); a.TGp = c.N * a.GI;
     a.co_tiles = pl.co_tiles; a.nsteps = pl.pwx_steps;
+    a.groups = gb.n; a.g_in = (long)(map == MAP_FWD ? gb.x : gb.y); a.g_w = (long)image; a.g_bias = (long)gb.b;
+    a.g_out = (long)(map == MAP_FWD ? gb.y : gb.x);
     // (a grouped convolution runs this once per group on a channel slice: only an ungrouped call covers the whole
     // addend with one launch, the groups leave it to the separate pass)
     if (map == MAP_DGRAD && g_addend.ptr && out == g_addend.dx && !g_addend.fused && p.groups == 1) {
@@ -806,6 +835,7 @@ static int run_pwx(const Problem& p, const Corr& c, const FwdPlan& pl, int map, 
         PHX_HIP(hipGetLastError());
         snprintf(g_name_buf, sizeof(g_name_buf), "%sqconv_%s_f16mfmapwr_p16_f16_wco%d_k%d_wgs%d_sub%d%s", g_name_prefix,
                  map == MAP_FWD ? "fwd" : "dgrad", pl.pwx, pl.pwx_steps, wgs, a.items - a.items_whole, a.addend ? "_add" : "");
+        label_groups(gb.n);
         g_last_kernel = g_name_buf;
         say(p, map == MAP_FWD ? "forward" : "input gradient");
         return PHX_OK;
@@ -832,6 +862,7 @@ static int run_pwx(const Problem& p, const Corr& c, const FwdPlan& pl, int map, 
     snprintf(g_name_buf, sizeof(g_name_buf), "%sqconv_%s_f16mfmapwx_p16_f16_wco%d_px%d_k%d_wgs%d_half%d%s", g_name_prefix,
              map == MAP_FWD ? "fwd" : "dgrad", pl.pwx, 64 * (4 / pl.pwx), pl.pwx_steps, blocks, a.items - a.items_whole,
              a.addend ? "_add" : "");
+    label_groups(gb.n);
     g_last_kernel = g_name_buf;
     say(p, map == MAP_FWD ? "forward" : "input gradient");
     return PHX_OK;
@@ -906,7 +937,9 @@ static int run_corr(const Problem& p, const Corr& creal, int map, hipStream_t st
     FwdPlan pl;
     if (!plan_corr(creal, p.mode, f16, c, pl, pw)) return PHX_ERR_NOT_SUPPORTED;
     if (pl.pwx) return run_pwx(p, creal, pl, map, st, in, w, bias, out, ws, ws_bytes);
-    const PackSlot slot = pack_slot(ws, ws_bytes, pl.wpk_bytes);
+    const GroupBatch gb = g_batch;
+    const size_t image = align_up(pl.wpk_bytes, 256);  // (group after group where one launch runs them all)
+    const PackSlot slot = pack_slot(ws, ws_bytes, gb.n > 1 ? image * gb.n : pl.wpk_bytes);
     if (slot.rc != PHX_OK) return slot.rc;
     ws = slot.dst;
 
@@ -915,7 +948,8 @@ static int run_corr(const Problem& p, const Corr& creal, int map, hipStream_t st
     v.WCO = pl.WCO; v.NTW = pl.NTW; v.CK = pl.CK; v.P2LOG = pl.P2LOG; v.wgs = pl.wgs; v.lds_bytes = pl.lds_bytes;
     v.lds_filters = pl.lds_filters; v.ngroups = pl.ngroups; v.pairs = pl.pairs; v.chunks = pl.chunks; v.pw = pw; v.vstage = pl.vstage;
 
-    PackArgs pa;
+    PackArgs pa{};
+    pa.groups = gb.n; pa.g_w = (long)gb.w; pa.g_out = (long)image;
     pa.w = w; pa.out = ws;
     pa.wcs = p.fs.wcs; pa.so = p.fs.so; pa.si = p.fs.si; pa.skh = p.fs.skh; pa.skw = p.fs.skw;
     pa.Co = p.co; pa.Ci = p.ci; pa.Kh = creal.Kh; pa.Kw = creal.Kw;
@@ -928,7 +962,9 @@ static int run_corr(const Problem& p, const Corr& creal, int map, hipStream_t st
     if (pl.lds_filters) pa.row_tiles = pl.co_tiles;  // packed per workgroup tile of WCO*32 channels
     const int pack_blocks = (int)std::min<long>((pack_items + WG_THREADS - 1) / WG_THREADS, 4096);
 
-    ConvArgs a;
+    ConvArgs a{};
+    a.groups = gb.n; a.g_in = (long)(map == MAP_FWD ? gb.x : gb.y); a.g_w = (long)image; a.g_bias = (long)gb.b;
+    a.g_out = (long)(map == MAP_FWD ? gb.y : gb.x);
     // channels per image in memory on the input and output side of this correlation (grouped convolutions: slices)
     const int cin_mem = (map == MAP_FWD) ? p.ci_mem : p.co_mem, cout_mem = (map == MAP_FWD) ? p.co_mem : p.ci_mem;
     a.in.base = in; a.in.comp_stride = (long)c.N * cin_mem * c.Hin * c.Win; a.in.Cs = cin_mem;
@@ -954,10 +990,15 @@ static int run_corr(const Problem& p, const Corr& creal, int map, hipStream_t st
     if (slot.pack_now) rc = f16 ? launch_pack_filters_f16(v, pa, pack_blocks, st) : launch_pack_filters(v, pa, pack_blocks, st);
     if (rc != 0) return PHX_ERR_NOT_SUPPORTED;
     if (g_pack.mode == PackSession::RECORD) {
-        PackJob j{};
-        j.a = pa; j.kind = !f16 ? PACK_F32 : pl.lds_filters ? PACK_F16_LDS : PACK_F16;
-        j.half_storage = v.half_storage; j.mode = pl.kmode; j.map = map; j.WCO = pl.WCO; j.ngroups = pl.ngroups; j.pw = pw;
-        if (const int rrc = record_pack_job(j, pack_items)) return rrc;
+        for (int g = 0; g < gb.n; ++g) {  // (the combined packing launch takes one job per image)
+            PackJob j{};
+            j.a = pa; j.a.groups = 1;
+            j.a.w = at_bytes(pa.w, g * gb.w);
+            j.a.out = at_bytes(pa.out, g * image);
+            j.kind = !f16 ? PACK_F32 : pl.lds_filters ? PACK_F16_LDS : PACK_F16;
+            j.half_storage = v.half_storage; j.mode = pl.kmode; j.map = map; j.WCO = pl.WCO; j.ngroups = pl.ngroups; j.pw = pw;
+            if (const int rrc = record_pack_job(j, pack_items)) return rrc;
+        }
     }
     if (!slot.compute) return PHX_OK;
     {
@@ -969,6 +1010,7 @@ static int run_corr(const Problem& p, const Corr& creal, int map, hipStream_t st
     snprintf(g_name_buf, sizeof(g_name_buf), "%sqconv_%s_%smfma%s%s_p%d_%s_wco%d_ntw%d_ck%d_%s%dx%dx%d", g_name_prefix,
              map == MAP_FWD ? "fwd" : "dgrad", f16 ? "f16" : "f32", pl.lds_filters ? (pw ? "ldspw" : pl.chunks ? "ldsc" : "lds") : "",
              cl ? "cl" : "", pl.kmode, p.dtype == PHX_F32 ? "f32" : "f16", pl.WCO, pl.NTW, pl.CK, pl.tall ? "flat" : "tile", pl.NB, pl.TH, pl.TW);
+    label_groups(gb.n);
     g_last_kernel = g_name_buf;
     say(p, map == MAP_FWD ? "forward" : "input gradient");
     return PHX_OK;
@@ -1017,13 +1059,18 @@ static int reduction_slices(int xy, int ntiles, int slots, double slice_bytes, d
     return best_z;
 }
 
+static bool group_batchable(const Problem& p, int pass);
+
+// the groups that share the GPU with one group's filter-gradient launch: its reduction slices fill that share
+static int wgrad_group_share(const Problem& p) { return group_batchable(p, PHX_PASS_BWD_WEIGHTS) ? p.groups : 1; }
+
 static void finish_wgrad_plan(const Problem& p, int CoT, int CiT, int per_cu, WgPlan& best) {
     best.co_tiles = cdiv(p.co, CoT); best.ci_tiles = cdiv(p.ci, CiT);
     best.CoP = best.co_tiles * CoT; best.CiP = best.ci_tiles * CiT;
     best.groups_per_row = cdiv(p.kw, best.TPW);
     const int xy = best.co_tiles * best.ci_tiles * best.groups_per_row * p.kh;
     const int ntiles = best.tiles_n * best.tiles_h * best.tiles_w;
-    int target = 256 * per_cu;  // one round of workgroups
+    int target = std::max(1, 256 * per_cu / wgrad_group_share(p));  // one round of workgroups
     if (tune().wgs > 0) target = tune().wgs;
     const double slice_bytes = (double)std::max(1, best.ksets) * p.kh * p.kw * 4 * best.CoP * best.CiP * sizeof(float);
     const double tile_flops = 2.0 * best.KP * CoT * CiT * best.kmode * std::min(best.TPW, p.kw);
@@ -1172,7 +1219,7 @@ static bool plan_wgrad_f16(const Problem& p, WgPlan& best) {
     // which keeps the partial sums small and lets no CU wait for a straggler round
     const int xy = best.co_tiles * best.ci_tiles * best.groups_per_row * p.kh;
     const int per_cu = best.lds_bytes <= 80 * 1024 ? 2 : 1;
-    int target = 256 * per_cu;
+    int target = std::max(1, 256 * per_cu / wgrad_group_share(p));
     if (tune().wgs > 0) target = tune().wgs;
     best.Z = std::max(1, std::min(best.ntiles, target / std::max(1, xy)));
     best.partial_bytes = (size_t)best.Z * p.kh * p.kw * 4 * best.CoP * best.CiP * sizeof(float);
@@ -1209,7 +1256,10 @@ static int run_wgrad(const Problem& p, hipStream_t st, const void* x, const void
     const bool f16 = wgrad_on_f16_mfma(p);
     WgPlan pl;
     if (!plan_wgrad(p, f16, pl)) return PHX_ERR_NOT_SUPPORTED;
-    if (ws_bytes < pl.partial_bytes || !ws) return PHX_ERR_WORKSPACE;
+    const GroupBatch gb = g_batch;
+    const size_t slab = align_up(pl.partial_bytes, 256);  // partial sums, group after group where one launch runs them all
+    if (ws_bytes < (gb.n > 1 ? slab * gb.n : pl.partial_bytes) || !ws) return PHX_ERR_WORKSPACE;
+    if (gb.n > 1 && f16 && pl.realx) return PHX_ERR_RUNTIME;  // (group_batchable keeps real-valued input out)
     if (f16 && pl.realx) {
         RealWgArgs ra{};
         ra.x = static_cast<const _Float16*>(x); ra.g = static_cast<const _Float16*>(g);
@@ -1224,7 +1274,7 @@ static int run_wgrad(const Problem& p, hipStream_t st, const void* x, const void
             if (launch_wgrad_f16_realx(ra, pl.Z, pl.lds_bytes, st) != 0) return PHX_ERR_RUNTIME;
         }
         PHX_HIP(hipGetLastError());
-        ReduceArgs r;
+        ReduceArgs r{};
         r.partial = ra.partial; r.dw = dw;
         r.wcs = p.fs.wcs; r.so = p.fs.so; r.si = p.fs.si; r.skh = p.fs.skh; r.skw = p.fs.skw;
         r.Z = pl.Z; r.Co = p.co; r.Ci = p.ci; r.Kh = p.kh; r.Kw = p.kw; r.CoP = pl.CoP; r.CiP = pl.CiP;
@@ -1235,7 +1285,8 @@ static int run_wgrad(const Problem& p, hipStream_t st, const void* x, const void
         say(p, "filter gradient (real-valued input)");
         return PHX_OK;
     }
-    WgradArgs a;
+    WgradArgs a{};
+    a.groups = gb.n; a.g_x = (long)gb.x; a.g_g = (long)gb.y; a.g_partial = (long)slab;
     a.x.base = x; a.x.comp_stride = (long)p.n * p.ci_mem * p.h * p.w; a.x.N = p.n; a.x.C = p.ci; a.x.Cs = p.ci_mem; a.x.Hd = p.h; a.x.Wd = p.w;
     // channels-last tensors on both sides: only the 64x64-tile fp16 kernel stages them (nhwc_wgrad_native holds)
     const bool cl = g_window_cl;
@@ -1261,11 +1312,12 @@ static int run_wgrad(const Problem& p, hipStream_t st, const void* x, const void
                     : launch_wgrad_f16(pl.kmode, pl.MT, pl.NT, pl.TPW, pl.SW, a, nblocks, pl.lds_bytes, st)) != 0)
                 return PHX_ERR_RUNTIME;
         } else {
-            launch_wgrad_f32(half_storage, pl.vec, pl.kmode, a, dim3(nblocks), pl.lds_bytes, st);
+            launch_wgrad_f32(half_storage, pl.vec, pl.kmode, a, dim3(nblocks, grid_rows(gb.n)), pl.lds_bytes, st);
         }
     }
     PHX_HIP(hipGetLastError());
-    ReduceArgs r;
+    ReduceArgs r{};
+    r.groups = gb.n; r.g_partial = (long)slab; r.g_dw = (long)gb.w;
     r.partial = a.partial; r.dw = dw;
     r.wcs = p.fs.wcs; r.so = p.fs.so; r.si = p.fs.si; r.skh = p.fs.skh; r.skw = p.fs.skw;
     r.Z = f16 ? pl.Z : pl.Z * pl.ksets; r.Co = p.co; r.Ci = p.ci; r.Kh = p.kh; r.Kw = p.kw; r.CoP = pl.CoP; r.CiP = pl.CiP;
@@ -1277,6 +1329,7 @@ static int run_wgrad(const Problem& p, hipStream_t st, const void* x, const void
     else
         snprintf(g_name_buf, sizeof(g_name_buf), "%sqconv_wgrad_f32mfma%s_p%d_%s_tile%dx%dx%d_z%d", g_name_prefix, pl.vec ? "v" : "", pl.kmode,
                  p.dtype == PHX_F32 ? "f32" : "f16", pl.NB, pl.TH, pl.TW, pl.Z);
+    label_groups(gb.n);
     g_last_kernel = g_name_buf;
     say(p, "filter gradient");
     return PHX_OK;
@@ -1639,6 +1692,14 @@ struct GroupOffsets {
     static void* at(void* ptr, size_t off) { return ptr ? static_cast<char*>(ptr) + off : nullptr; }
 };
 
+struct GroupBatchScope {  // all groups in one launch per kernel (see group_batchable); lasts for one run of a pass
+    explicit GroupBatchScope(const Problem& p) {
+        const GroupOffsets o(p);
+        g_batch.n = o.runs; g_batch.x = o.x; g_batch.y = o.y; g_batch.w = o.w; g_batch.b = o.b;
+    }
+    ~GroupBatchScope() { g_batch = GroupBatch{}; }
+};
+
 // Channels-last activations (DataFormat::NHWC, src/backend/tensor.hpp:17-31): the kernels read and write
 // channels-first planes, so such a call keeps channels-first copies of its input-side and output-side activation
 // tensors at the front of the workspace and transposes on the way in and out.
@@ -1708,6 +1769,24 @@ static bool nhwc_wgrad_native(const Problem& p) {
     return !pl.realx && pl.kmode == 16 && pl.MT == 2 && pl.NT == 2 && pl.SW == 1 && (pl.TPW == 1 || pl.TPW == 3);
 }
 
+namespace phx {
+// A grouped convolution runs ALL its groups in one launch per kernel -- grid rows = groups, every kernel shifting its
+// tensors by its row's byte steps (group_view) -- the way the reference hands `groups` to one primitive
+// (src/backend/onednn/conv2d.hpp:116-137), wherever the pass is a plain run of the kernels on channel-slice views:
+// channels-first tensors, all components present, none of the rewritten forms (space-to-depth, subsampled strided
+// pointwise, input gradient by phases), whose rearrangement kernels work on one group's tensors.  Everything else
+// runs group after group.  The plans are those of one group, so the results are the same either way.
+static bool group_batchable(const Problem& p, int pass) {
+    if (p.groups <= 1 || is_empty(p) || p.nhwc || p.real_input || tune().nogroupbatch) return false;
+    S2dView v;
+    Problem q;
+    size_t xs_bytes = 0;
+    if (pass != PHX_PASS_BWD_DATA && (s2d_view(p, v) || subsample_view(p, q, xs_bytes))) return false;
+    if (pass == PHX_PASS_BWD_DATA && dgrad_by_phases(p)) return false;
+    return true;
+}
+}  // namespace phx
+
 // Entry points check their descriptor before they touch the device: an invalid descriptor is an invalid argument
 // whether or not a device is present.
 static int conv_desc_status(const phx_qconv_desc* desc) {
@@ -1741,6 +1820,8 @@ size_t phx_qconv2d_workspace_bytes(const phx_qconv_desc* desc, int pass) {
     if (nhwc_native(p, pass)) return nhwc_native_workspace(p, pass);
     if (nhwc_window_native(p, pass)) return workspace_for(p, pass);
     if (pass == PHX_PASS_BWD_WEIGHTS && nhwc_wgrad_native(p)) return workspace_for(p, pass);
+    // (packed images / partial sums of all groups side by side where one launch runs them)
+    if (group_batchable(p, pass)) return (size_t)p.groups * workspace_for(p, pass);
     return ChannelsLast(p).bytes() + workspace_for(p, pass);
 }
 
@@ -1794,6 +1875,10 @@ static int conv_fwd_quaternion(const phx_qconv_desc* desc, phx_stream_t stream, 
         const int nrc = do_fwd(p, st, x, w, bias_or_null, y, dry ? nullptr : workspace, dry ? 0 : workspace_bytes);
         g_window_cl = false;
         return nrc;
+    }
+    if (group_batchable(p, PHX_PASS_FWD)) {
+        const GroupBatchScope batch(p);
+        return do_fwd(p, st, x, w, bias_or_null, y, dry ? nullptr : workspace, dry ? 0 : workspace_bytes);
     }
     const ChannelsLast cl(p);
     if (dry) { workspace = nullptr; workspace_bytes = cl.bytes(); }
@@ -1854,6 +1939,10 @@ static int conv_bwd_data_quaternion(const phx_qconv_desc* desc, phx_stream_t str
         const int nrc = do_bwd_data(p, st, grad, w, dx, dry ? nullptr : workspace, dry ? 0 : workspace_bytes);
         g_window_cl = false;
         return nrc;
+    }
+    if (group_batchable(p, PHX_PASS_BWD_DATA)) {
+        const GroupBatchScope batch(p);
+        return do_bwd_data(p, st, grad, w, dx, dry ? nullptr : workspace, dry ? 0 : workspace_bytes);
     }
     const ChannelsLast cl(p);
     if (dry) { workspace = nullptr; workspace_bytes = cl.bytes(); }
@@ -1988,6 +2077,10 @@ int phx_qconv2d_bwd_weights(const phx_qconv_desc* desc, phx_stream_t stream, con
         const int nrc = do_bwd_weights(p, st, x, grad, dw, workspace, workspace_bytes);
         g_window_cl = false;
         return nrc;
+    }
+    if (group_batchable(p, PHX_PASS_BWD_WEIGHTS)) {
+        const GroupBatchScope batch(p);
+        return do_bwd_weights(p, st, x, grad, dw, workspace, workspace_bytes);
     }
     const ChannelsLast cl(p);
     if (cl.bytes() > workspace_bytes || (cl.bytes() && !workspace)) return PHX_ERR_WORKSPACE;

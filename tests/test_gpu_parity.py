@@ -426,6 +426,55 @@ def test_grouped_convolution(case, mode, dtype, policy):
     assert_close(dw.cpu().numpy(), want_dw, dtype, "grouped wgrad " + name)
 
 
+@pytest.mark.parametrize("dtype,policy", [(torch.float32, "fp32"), (torch.float16, "full16"), (torch.float16, "backward32")],
+                         ids=["f32", "f16_full16", "f16_backward32"])
+@pytest.mark.parametrize("mode", [16, 8])
+@pytest.mark.parametrize("case", [c for c in GROUPED if c[0] != "g3_k3_s2"] + [("depthwise_k3_g32", 32, 3, 32, 32, 12, 12, 3, 3, 1, 1, "SAME")],
+                         ids=lambda c: c[0])
+def test_groups_run_in_one_launch_per_kernel(case, mode, dtype, policy, tune_env):
+    """A grouped convolution on channels-first tensors whose passes are plain runs of the kernels (no space-to-depth,
+    subsampling or phases) runs every kernel once, with a grid row per group (the reference hands `groups` to one
+    primitive, src/backend/onednn/conv2d.hpp:116-137): the kernel label says so, and forward and input gradient are bit
+    for bit those of the same call run group after group (PHX_TUNE_NOGROUPBATCH), plain and through prepacked filters."""
+    name, G, n, ci, co, h, w, kh, kw, stride, dilation, padding = case
+    r = np.random.default_rng(name_seed(name) + 31)
+    npdt = np.float32 if dtype == torch.float32 else np.float16
+    geom = oracle.make_geom(n, ci // G, co // G, h, w, kh, kw, stride, dilation, padding)
+    xd = torch.from_numpy((0.5 * r.standard_normal((4 * n, ci, h, w))).astype(npdt)).cuda()
+    gd = torch.from_numpy((0.5 * r.standard_normal((4 * n, co, geom.ho, geom.wo))).astype(npdt)).cuda()
+    wd = torch.from_numpy((0.3 * r.standard_normal((4, co, ci // G, kh, kw))).astype(npdt)).cuda()
+    bd = torch.from_numpy(r.standard_normal((4, co)).astype(npdt)).cuda()
+    desc = phx.Conv2DDescriptor(xd.shape, wd.shape, stride, dilation, padding, groups=G, use_bias=True, dtype=dtype,
+                                context=Ctx(mode, policy))
+    got = {}
+    for variant in ("one launch", "group after group"):
+        tune_env(PHX_TUNE_NOGROUPBATCH=None if variant == "one launch" else "1")
+        y = phx.conv2d_fwd(xd, wd, bd, desc)
+        k_fwd = capi.last_kernel_name()
+        dx = ops.conv2d_bwd_data(wd, gd, desc)
+        k_bwd = capi.last_kernel_name()
+        dw = ops.conv2d_bwd_weights(xd, gd, desc)
+        k_wg = capi.last_kernel_name()
+        outs = [y, dx, dw]
+        if dtype == torch.float16:
+            packed = ops.conv2d_pack_filters(wd, desc)
+            outs += [phx.conv2d_fwd(xd, torch.zeros_like(wd), bd, desc, packed=packed),
+                     ops.conv2d_bwd_data(torch.zeros_like(wd), gd, desc, packed=packed)]
+        got[variant] = (outs, (k_fwd, k_bwd, k_wg))
+        tag = "_groups%d" % G
+        assert all(k.endswith(tag) == (variant == "one launch") for k in (k_fwd, k_bwd, k_wg)), (variant, k_fwd, k_bwd, k_wg)
+    for i, (a, b) in enumerate(zip(got["one launch"][0], got["group after group"][0])):
+        if i == 2:
+            # the filter gradient: a launch that runs all groups gives every group its share of the reduction slices,
+            # so its partial sums are added in another order than those of a launch that has the GPU to itself
+            scale = b.float().abs().max().item()
+            assert (a.float() - b.float()).abs().max().item() <= (2e-6 if dtype == torch.float32 else 2e-3) * scale
+        else:
+            assert torch.equal(a, b)
+    if dtype == torch.float16:
+        assert torch.equal(got["one launch"][0][3], got["one launch"][0][0]) and torch.equal(got["one launch"][0][4], got["one launch"][0][1])
+
+
 def test_reference_kat_channels_last():
     """tests/tests.cpp:440-487 of the reference: a real 2x2 image with 3 channels, NHWC, through a real 1x1
     OHWI filter with 2 output channels -> (0,2, 2,4, 3,6, 5,8).  A real convolution is the real part of a
