@@ -1730,8 +1730,8 @@ struct ChannelsLast {
     }
 };
 
-// Channels-last windowed convolutions (3x3 and other multi-tap filters, unit stride) whose forward / input-gradient
-// plan is the chunk-staging fp16 kernel run on the caller's tensors as they are: that kernel's LDS layout is
+// Channels-last windowed convolutions (3x3 and other multi-tap filters; any stride forward, unit stride backward) whose
+// forward / input-gradient plan is the chunk-staging fp16 kernel run on the caller's tensors as they are: that kernel's LDS layout is
 // [position][8 channels], which IS the channels-last order, so its staging copies 16-byte entries without the
 // channel transpose the channels-first form needs, and the epilogue stores 16 consecutive channels of a pixel per
 // lane.  Everything else channels-last (the filter gradient, strides, groups, fp32) keeps the transposes.
@@ -1743,7 +1743,10 @@ struct ChannelsLast {
 // PHX_TUNE_WINCL_MAX moves that bound, PHX_TUNE_NOWINCL switches the direct form off.
 static bool nhwc_window_native(const Problem& p, int pass) {
     if (!p.nhwc || (pass != PHX_PASS_FWD && pass != PHX_PASS_BWD_DATA) || is_empty(p) || is_pointwise_unit(p)) return false;
-    if (p.real_input || p.groups != 1 || p.sh != 1 || p.sw != 1 || tune().nowincl || !use_f16_mfma(p, pass)) return false;
+    if (p.real_input || p.groups != 1 || tune().nowincl || !use_f16_mfma(p, pass)) return false;
+    // (a strided forward pass reads its staged window with the stride, whatever the memory order; a strided input
+    // gradient runs by phases or on zero-inserted windows, neither of which is staged in chunks)
+    if ((p.sh != 1 || p.sw != 1) && pass != PHX_PASS_FWD) return false;
     if ((long)std::max(p.ci, p.co) * p.kh * p.kw > tune().wincl_max) return false;
     if (p.ci % 8 != 0 || p.co % 8 != 0 || p.ci_mem != p.ci || p.co_mem != p.co) return false;  // whole 16-byte entries, 8-byte stores
     S2dView v;

@@ -644,6 +644,42 @@ def test_channels_last_windows_run_on_the_tensors_as_they_are(case, mode, tune_e
         assert torch.equal(direct[key], transposed[key]), key
 
 
+@pytest.mark.parametrize("mode", [16, 8])
+@pytest.mark.parametrize("case", [("clw_k3_s2", 2, 32, 64, 15, 13, 3, 3, 2, "SAME"), ("clw_k3_s2_128", 2, 128, 128, 28, 28, 3, 3, 2, "SAME"),
+                                  ("clw_k5_s1x2", 3, 16, 24, 11, 14, 5, 5, (1, 2), "VALID"), ("clw_k1_s2", 2, 64, 128, 14, 14, 1, 1, 2, "VALID")],
+                         ids=lambda c: c[0])
+def test_channels_last_strided_forward_runs_on_the_tensors_as_they_are(case, mode, tune_env):
+    """The forward pass of a strided channels-last convolution on fp16 matrix cores reads and writes the caller's
+    tensors directly as well (the staged window is read with the stride); its backward passes keep the transposes.
+    Against the oracle, and forward bit for bit against the transposed path."""
+    name, n, ci, co, h, w, kh, kw, stride, padding = case
+    dtype = torch.float16
+    g, x, wt, b, gr = make_inputs(name_seed(name) + 14, n, ci, co, h, w, kh, kw, stride, 1, padding, dtype, 0.5)
+    x_dev, g_dev = (np.ascontiguousarray(a.transpose(0, 2, 3, 1)) for a in (x, gr))
+    w_dev = np.ascontiguousarray(wt.transpose(0, 1, 3, 4, 2))
+    desc = phx.Conv2DDescriptor(x_dev.shape, w_dev.shape, stride, 1, padding, use_bias=True, dtype=dtype, filter_layout="OHWI",
+                                context=Ctx(mode, "full16"), data_format="NHWC")
+    xd, wd, bd, gd = (torch.from_numpy(a).cuda() for a in (x_dev, w_dev, b, g_dev))
+    x64, w64, b64, g64 = (a.astype(np.float64) for a in (x, wt, b, gr))
+    want_y = oracle.conv2d_fwd(g, x64, w64, b64, "hamilton")
+    want_dw, want_dx = oracle.conv2d_bwd(g, x64, w64, g64, "hamilton")
+    ys, names = [], []
+    for variant in ("direct", "transposed"):
+        tune_env(PHX_TUNE_NOWINCL=None if variant == "direct" else "1")
+        y = phx.conv2d_fwd(xd, wd, bd, desc)
+        names.append(capi.last_kernel_name())
+        dw, dx = phx.conv2d_bwd(xd, wd, gd, desc)
+        assert "cl_" not in capi.last_kernel_name(), capi.last_kernel_name()
+        assert_close(y.cpu().numpy().transpose(0, 3, 1, 2), want_y, dtype, "fwd " + names[-1])
+        assert_close(dx.cpu().numpy().transpose(0, 3, 1, 2), want_dx, dtype, "dgrad " + name)
+        assert_close(dw.cpu().numpy().transpose(0, 1, 4, 2, 3), want_dw, dtype, "wgrad " + name)
+        ys.append(y)
+    print(name, mode, names, flush=True)
+    if name != "clw_k1_s2":  # (a strided pointwise convolution has no chunk-staged plan)
+        assert "ldsccl_" in names[0] and "ldsccl_" not in names[1], names
+    assert torch.equal(ys[0], ys[1])
+
+
 # name, n, ci, co, h, w, kh, kw, stride, dilation, padding -- unit stride, more than one tap
 FLAT = [c for c in FP16_CASES if c[0] in ("k3_same", "k3_ragged", "k3_valid", "k3_dil2", "k4_same", "k24_c40", "k3_128_28")] + [
     ("k3_7x7_n9", 9, 40, 40, 7, 7, 3, 3, 1, 1, "SAME"),              # several images per workgroup
