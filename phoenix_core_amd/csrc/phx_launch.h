@@ -103,6 +103,26 @@ struct DenseSmallArgs {
 };
 int launch_dense_small(bool half_storage, int pass, const DenseSmallArgs& a, hipStream_t st);
 
+// Grouped convolutions with very few channels per group (depthwise and the like) on fp32 FMA threads, on the caller's
+// channels-first tensors and filter (phx_launch_thin.hip).  in = x (forward, filter gradient) or the output gradient
+// (input gradient); out = y, dx or dw.  Filter element (r, co, i, kh, kw), co over all groups and i inside its group,
+// at r * wcs + co * so + i * si + kh * skh + kw * skw.
+struct ThinArgs {
+    const void* in;
+    const void* w;
+    const void* bias;  // forward: [4][all output channels] or null
+    void* out;
+    const void* grad;  // filter gradient: the output gradient
+    float* partial;    // filter gradient: [Z][output channel x input channel of its group][tap][4] partial sums
+    long wcs, so, si, skh, skw;
+    int N, groups, cig, cog;  // images, groups, input / output channels of one group
+    int H, W, Ho, Wo;         // input and output image of the forward pass
+    int Kh, Kw, sh, sw, dh, dw, pt, pl;
+    int Z;                    // filter gradient: slices of the images summed by separate workgroups
+    unsigned int mh, mw;      // strided input gradient: ceil(2^32 / sh), ceil(2^32 / sw); 0 for a unit stride
+};
+int launch_thin(bool half_storage, int pass, const ThinArgs& a, hipStream_t st);
+
 // space-to-depth rearrangements (stride-2 convolutions with very few input channels)
 int launch_s2d_input(bool half_storage, const S2dArgs& a, hipStream_t st);
 int launch_subsample(bool half_storage, const SubsampleArgs& a, hipStream_t st);

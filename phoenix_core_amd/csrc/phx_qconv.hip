@@ -35,6 +35,7 @@ struct Tuning {
     bool pwrall = false;              // PHX_TUNE_PWRALL: ... and every problem that kernel can run goes to it (not only those of at most 32 output channels)
     bool nowincl = false;             // PHX_TUNE_NOWINCL: channels-last windowed problems go through the transposes
     bool nogroupbatch = false;        // PHX_TUNE_NOGROUPBATCH: a grouped convolution runs group after group
+    int thin_max = 4;                 // PHX_TUNE_THIN_MAX: most channels per group that run on the FMA kernels for thin groups (0 = never)
     int wincl_max = 3072;             // PHX_TUNE_WINCL_MAX: largest channels x taps that runs on channels-last tensors directly
     bool nosmalldense = false;        // PHX_TUNE_NOSMALLDENSE: small Dense problems stay on the matrix-core kernels
     int vec = 0;                      // PHX_TUNE_VEC (0 = unset)
@@ -64,6 +65,7 @@ struct Tuning {
         nowincl = getenv("PHX_TUNE_NOWINCL") != nullptr;
         nogroupbatch = getenv("PHX_TUNE_NOGROUPBATCH") != nullptr;
         if (const char* e = getenv("PHX_TUNE_WINCL_MAX")) wincl_max = atoi(e);
+        if (const char* e = getenv("PHX_TUNE_THIN_MAX")) thin_max = atoi(e);
         nosmalldense = getenv("PHX_TUNE_NOSMALLDENSE") != nullptr;
         if (const char* e = getenv("PHX_TUNE_VEC")) vec = atoi(e);
         if (const char* e = getenv("PHX_TUNE_WGS")) wgs = atoi(e);
@@ -1772,6 +1774,69 @@ static bool nhwc_wgrad_native(const Problem& p) {
     return !pl.realx && pl.kmode == 16 && pl.MT == 2 && pl.NT == 2 && pl.SW == 1 && (pl.TPW == 1 || pl.TPW == 3);
 }
 
+// Grouped convolutions whose groups hold at most a few channels on either side (depthwise convolutions first of all)
+// run on the fp32 FMA kernels of phx_launch_thin.hip, all groups by one launch per pass, straight on the caller's
+// channels-first tensors and filter: a 32 x 32 matrix-core tile per group would be nearly empty (1.6 % full at 4
+// channels per group), and measured per pass the FMA threads are 6-30x faster there.  PHX_TUNE_THIN_MAX moves the bound.
+static bool thin_groups(const Problem& p) {
+    if (p.groups <= 1 || is_empty(p) || p.real_input || p.ho <= 0 || p.wo <= 0) return false;
+    if (std::max(p.ci, p.co) > tune().thin_max) return false;
+    return (long)std::max(p.ci, p.co) * p.kh * p.kw * 16 <= 48 * 1024 && std::max(p.ci_mem, p.co_mem) <= 65535;
+}
+
+// reduction slices of the thin-group filter gradient: enough workgroups to fill the GPU, each with at least a few
+// pixels per thread
+static int thin_wgrad_slices(const Problem& p) {
+    const long taps = (long)p.kh * p.kw;
+    const long columns = (long)p.co_mem * p.ci * (taps == 1 ? 1 : cdiv((int)taps, 9));
+    const long want = (2048 + columns - 1) / columns, fit = std::max(1L, (long)p.n * p.ho * p.wo / (4 * WG_THREADS));
+    return (int)std::max(1L, std::min({want, fit, (long)p.n, 65535L}));
+}
+static size_t thin_workspace(const Problem& p, int pass) {
+    if (pass != PHX_PASS_BWD_WEIGHTS) return 0;
+    return align_up((size_t)thin_wgrad_slices(p) * p.co_mem * p.ci * p.kh * p.kw * 4 * sizeof(float), 256);
+}
+
+// (a, b) = (x, w) forward, (grad, w) input gradient, (x, grad) filter gradient; channels-first tensors of all groups
+static int run_thin(const Problem& p, int pass, hipStream_t st, const void* a, const void* b, const void* bias, void* out, void* ws,
+                    size_t wsb) {
+    if (!a || !b || !out || (pass == PHX_PASS_FWD && p.has_bias && !bias)) return PHX_ERR_INVALID_ARGUMENT;
+    ThinArgs t{};
+    t.in = a; t.out = out;
+    t.wcs = p.fs.wcs; t.so = p.fs.so; t.si = p.fs.si; t.skh = p.fs.skh; t.skw = p.fs.skw;
+    t.N = p.n; t.groups = p.groups; t.cig = p.ci; t.cog = p.co;
+    t.H = p.h; t.W = p.w; t.Ho = p.ho; t.Wo = p.wo;
+    t.Kh = p.kh; t.Kw = p.kw; t.sh = p.sh; t.sw = p.sw; t.dh = p.dh; t.dw = p.dw; t.pt = p.pt; t.pl = p.pl;
+    t.Z = 1;
+    t.mh = p.sh > 1 ? (unsigned int)(((1ULL << 32) + p.sh - 1) / p.sh) : 0u;
+    t.mw = p.sw > 1 ? (unsigned int)(((1ULL << 32) + p.sw - 1) / p.sw) : 0u;
+    if (pass == PHX_PASS_BWD_WEIGHTS) {
+        t.grad = b;
+        t.Z = thin_wgrad_slices(p);
+        if (thin_workspace(p, pass) > wsb || !ws) return PHX_ERR_WORKSPACE;
+        t.partial = static_cast<float*>(ws);
+    } else {
+        t.w = b;
+        t.bias = (pass == PHX_PASS_FWD && p.has_bias) ? bias : nullptr;
+    }
+    int rc;
+    {
+        KernelTimer timer(st);
+        rc = launch_thin(p.dtype == PHX_F16, pass, t, st);
+    }
+    if (rc != 0) return PHX_ERR_NOT_SUPPORTED;
+    PHX_HIP(hipGetLastError());
+    if (pass == PHX_PASS_BWD_WEIGHTS)
+        snprintf(g_name_buf, sizeof(g_name_buf), "qconv_wgrad_fma_thin_%s_g%dx%dx%d_k%dx%d_z%d", p.dtype == PHX_F32 ? "f32" : "f16", p.groups,
+                 p.ci, p.co, p.kh, p.kw, t.Z);
+    else
+        snprintf(g_name_buf, sizeof(g_name_buf), "qconv_%s_fma_thin_%s_g%dx%dx%d_k%dx%d", pass == PHX_PASS_FWD ? "fwd" : "dgrad",
+                 p.dtype == PHX_F32 ? "f32" : "f16", p.groups, p.ci, p.co, p.kh, p.kw);
+    g_last_kernel = g_name_buf;
+    say(p, pass == PHX_PASS_FWD ? "forward (thin groups)" : pass == PHX_PASS_BWD_DATA ? "input gradient (thin groups)" : "filter gradient (thin groups)");
+    return PHX_OK;
+}
+
 namespace phx {
 // A grouped convolution runs ALL its groups in one launch per kernel -- grid rows = groups, every kernel shifting its
 // tensors by its row's byte steps (group_view) -- the way the reference hands `groups` to one primitive
@@ -1780,7 +1845,7 @@ namespace phx {
 // pointwise, input gradient by phases), whose rearrangement kernels work on one group's tensors.  Everything else
 // runs group after group.  The plans are those of one group, so the results are the same either way.
 static bool group_batchable(const Problem& p, int pass) {
-    if (p.groups <= 1 || is_empty(p) || p.nhwc || p.real_input || tune().nogroupbatch) return false;
+    if (p.groups <= 1 || is_empty(p) || p.nhwc || p.real_input || tune().nogroupbatch || thin_groups(p)) return false;
     S2dView v;
     Problem q;
     size_t xs_bytes = 0;
@@ -1825,7 +1890,7 @@ size_t phx_qconv2d_workspace_bytes(const phx_qconv_desc* desc, int pass) {
     if (pass == PHX_PASS_BWD_WEIGHTS && nhwc_wgrad_native(p)) return workspace_for(p, pass);
     // (packed images / partial sums of all groups side by side where one launch runs them)
     if (group_batchable(p, pass)) return (size_t)p.groups * workspace_for(p, pass);
-    return ChannelsLast(p).bytes() + workspace_for(p, pass);
+    return ChannelsLast(p).bytes() + (thin_groups(p) ? thin_workspace(p, pass) : workspace_for(p, pass));
 }
 
 // Small Dense problems (a classifier head, the reference's 128 -> 128 benchmark layer at batch 32) run on plain fp32
@@ -1893,6 +1958,11 @@ static int conv_fwd_quaternion(const phx_qconv_desc* desc, phx_stream_t stream, 
         x = ws;
         y_planes = ws + cl.x_bytes;
     }
+    if (thin_groups(p)) {  // (no packed form: a packing session finds nothing to pack)
+        if (g_pack.mode == PackSession::USE) return PHX_ERR_NOT_SUPPORTED;
+        if (!dry)
+            if (const int trc = run_thin(p, PHX_PASS_FWD, st, x, w, bias_or_null, y_planes, nullptr, 0)) return trc;
+    } else
     for (int g = 0; g < o.runs; ++g) {
         const int grc = do_fwd(p, st, o.at(x, g * o.x), o.at(w, g * o.w),
                                bias_or_null ? o.at(bias_or_null, g * o.b) : nullptr, o.at(y_planes, g * o.y),
@@ -1957,6 +2027,11 @@ static int conv_bwd_data_quaternion(const phx_qconv_desc* desc, phx_stream_t str
         grad = ws + cl.x_bytes;
         dx_planes = ws;
     }
+    if (thin_groups(p)) {
+        if (g_pack.mode == PackSession::USE) return PHX_ERR_NOT_SUPPORTED;
+        if (!dry)
+            if (const int trc = run_thin(p, PHX_PASS_BWD_DATA, st, grad, w, nullptr, dx_planes, nullptr, 0)) return trc;
+    } else
     for (int g = 0; g < o.runs; ++g) {
         const int grc = do_bwd_data(p, st, o.at(grad, g * o.y), o.at(w, g * o.w), o.at(dx_planes, g * o.x),
                                     ws ? ws + cl.bytes() : nullptr, workspace_bytes - cl.bytes());
@@ -2094,6 +2169,8 @@ int phx_qconv2d_bwd_weights(const phx_qconv_desc* desc, phx_stream_t stream, con
         x = ws;
         grad = ws + cl.x_bytes;
     }
+    if (thin_groups(p))
+        return run_thin(p, PHX_PASS_BWD_WEIGHTS, st, x, grad, nullptr, dw, ws ? ws + cl.bytes() : nullptr, workspace_bytes - cl.bytes());
     for (int g = 0; g < o.runs; ++g) {
         const int grc = do_bwd_weights(p, st, o.at(x, g * o.x), o.at(grad, g * o.y), o.at(dw, g * o.w),
                                        ws ? ws + cl.bytes() : nullptr, workspace_bytes - cl.bytes());

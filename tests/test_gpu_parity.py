@@ -448,7 +448,8 @@ def test_groups_run_in_one_launch_per_kernel(case, mode, dtype, policy, tune_env
                                 context=Ctx(mode, policy))
     got = {}
     for variant in ("one launch", "group after group"):
-        tune_env(PHX_TUNE_NOGROUPBATCH=None if variant == "one launch" else "1")
+        # (THIN_MAX=0: the depthwise cases stay on the matrix-core kernels this test is about)
+        tune_env(PHX_TUNE_NOGROUPBATCH=None if variant == "one launch" else "1", PHX_TUNE_THIN_MAX="0")
         y = phx.conv2d_fwd(xd, wd, bd, desc)
         k_fwd = capi.last_kernel_name()
         dx = ops.conv2d_bwd_data(wd, gd, desc)
@@ -473,6 +474,82 @@ def test_groups_run_in_one_launch_per_kernel(case, mode, dtype, policy, tune_env
             assert torch.equal(a, b)
     if dtype == torch.float16:
         assert torch.equal(got["one launch"][0][3], got["one launch"][0][0]) and torch.equal(got["one launch"][0][4], got["one launch"][0][1])
+
+
+THIN_GROUPS = [
+    # name, groups, channels-last, n, ci, co, h, w, kh, kw, stride, dilation, padding
+    ("dw_k3", 8, False, 2, 8, 8, 10, 10, 3, 3, 1, 1, "SAME"),
+    ("dw_k3_s2", 6, False, 3, 6, 6, 15, 13, 3, 3, 2, 1, "SAME"),
+    ("dw_mult2_k5_dil2", 4, False, 2, 4, 8, 11, 12, 5, 5, 1, 2, (2, 1, 3, 0)),   # two output channels per input channel
+    ("g3_4to3_k3_s2", 3, False, 2, 12, 9, 15, 13, 3, 3, 2, 1, "SAME"),
+    ("g5_2to4_k3", 5, False, 2, 10, 20, 9, 12, 3, 3, 1, 1, "SAME"),
+    ("dw_pw", 16, False, 3, 16, 16, 9, 7, 1, 1, 1, 1, "VALID"),
+    ("dw_k7_s3_valid", 4, False, 2, 4, 4, 23, 20, 7, 7, 3, 1, "VALID"),         # rows and columns behind the last window: their gradient is zero
+    ("dw_k3_s2_dil2", 5, False, 2, 5, 10, 14, 17, 3, 3, 2, 2, "SAME"),          # strided and dilated
+    ("dw_k32_s21", 4, False, 2, 4, 4, 13, 19, 3, 2, (2, 1), 1, "SAME"),         # stride along H only
+    ("dw_k3_n40", 4, False, 40, 4, 4, 14, 14, 3, 3, 1, 1, "SAME"),              # filter gradient summed over several slices of the images
+    ("dw_k5_n9", 3, False, 9, 3, 3, 12, 11, 5, 5, 1, 1, "SAME"),                # 25 taps: three workgroups of nine per channel pair
+    ("dw_k3_1px", 2, False, 1, 2, 2, 3, 3, 3, 3, 1, 1, "VALID"),                # one output position
+    ("dw_k3_nhwc", 8, True, 2, 8, 8, 10, 9, 3, 3, 1, 1, "SAME"),
+    ("dw_k3_s2_nhwc", 6, True, 3, 6, 12, 15, 13, 3, 3, 2, 1, "SAME"),
+]
+
+
+@pytest.mark.parametrize("dtype,policy", [(torch.float32, "fp32"), (torch.float16, "full16"), (torch.float16, "backward32")],
+                         ids=["f32", "f16_full16", "f16_backward32"])
+@pytest.mark.parametrize("mode", [16, 8])
+@pytest.mark.parametrize("case", THIN_GROUPS, ids=lambda c: c[0])
+def test_thin_groups_run_on_fma_threads(case, mode, dtype, policy):
+    """Grouped convolutions with at most four channels per group on either side (depthwise convolutions first of all; the
+    reference hands `groups` to its scalar convolutions, src/backend/onednn/conv2d.hpp:116-137, and has no vector for
+    them) run on the FMA kernels for thin groups, every pass by one launch on the caller's filter: the kernel label says
+    so, the filter gradient asks for its partial sums only, and the results are those of G independent convolutions on
+    channel slices, which is how the oracle's result is assembled here.  OIHW filter on channels-first tensors, OHWI on
+    channels-last ones (which run through channels-first copies)."""
+    name, G, cl, n, ci, co, h, w, kh, kw, stride, dilation, padding = case
+    cig, cog = ci // G, co // G
+    scale = 1.0 if dtype == torch.float32 else 0.5
+    g, x, _, b, gr = make_inputs(name_seed(name) + 40, n, ci, co, h, w, kh, kw, stride, dilation, padding, dtype, scale)
+    r = np.random.default_rng(name_seed(name) + 41)
+    npdt = np.float32 if dtype == torch.float32 else np.float16
+    wt = (scale * r.standard_normal((4, co, cig, kh, kw)) * np.sqrt(2.0 / (cig * kh * kw))).astype(npdt)
+    to_dev = (lambda a: np.ascontiguousarray(a.transpose(0, 2, 3, 1))) if cl else (lambda a: a)
+    from_dev = (lambda a: a.transpose(0, 3, 1, 2)) if cl else (lambda a: a)
+    x_dev, g_dev = to_dev(x), to_dev(gr)
+    w_dev = np.ascontiguousarray(wt.transpose(0, 1, 3, 4, 2)) if cl else wt
+    desc = phx.Conv2DDescriptor(x_dev.shape, w_dev.shape, stride, dilation, padding, groups=G, use_bias=True, dtype=dtype,
+                                filter_layout="OHWI" if cl else "OIHW", context=Ctx(mode, policy),
+                                data_format="NHWC" if cl else "NCHW")
+    xd, wd, bd, gd = (torch.from_numpy(a).cuda() for a in (x_dev, w_dev, b, g_dev))
+    y = phx.conv2d_fwd(xd, wd, bd, desc)
+    names = [capi.last_kernel_name()]
+    dx = ops.conv2d_bwd_data(wd, gd, desc)
+    names.append(capi.last_kernel_name())
+    dw = ops.conv2d_bwd_weights(xd, gd, desc)
+    names.append(capi.last_kernel_name())
+    assert all("_fma_thin_" in k for k in names), names
+    esize = 4 if dtype == torch.float32 else 2
+    planes = (x.nbytes + 255) // 256 * 256 + (gr.nbytes + 255) // 256 * 256 if cl else 0
+    assert desc.workspace_bytes(capi.PHX_PASS_FWD) == planes
+    assert desc.workspace_bytes(capi.PHX_PASS_BWD_DATA) == planes
+    slices = int(names[2].rsplit("_z", 1)[1])
+    assert desc.workspace_bytes(capi.PHX_PASS_BWD_WEIGHTS) == planes + (slices * co * cig * kh * kw * 16 + 255) // 256 * 256
+    # nothing to pack: the kernels read the caller's filter
+    assert ops.conv2d_packed_filter_bytes(desc, capi.PHX_PASS_FWD) == 0 and ops.conv2d_pack_filters(wd, desc) is None
+    gg = oracle.make_geom(n, cig, cog, h, w, kh, kw, stride, dilation, padding)
+    x64, w64, b64, g64 = (a.astype(np.float64) for a in (x, wt, b, gr))
+    want_y, want_dx, want_dw = np.empty(gr.shape), np.empty(x.shape), np.empty(wt.shape)
+    for k in range(G):
+        ic, oc = slice(k * cig, (k + 1) * cig), slice(k * cog, (k + 1) * cog)
+        xs, ws, bs, gs = (np.ascontiguousarray(a) for a in (x64[:, ic], w64[:, oc], b64[:, oc], g64[:, oc]))
+        want_y[:, oc] = oracle.conv2d_fwd(gg, xs, ws, bs, "hamilton")
+        want_dw[:, oc], want_dx[:, ic] = oracle.conv2d_bwd(gg, xs, ws, gs, "hamilton")
+    assert_close(from_dev(y.cpu().numpy()), want_y, dtype, "thin groups fwd " + name)
+    assert_close(from_dev(dx.cpu().numpy()), want_dx, dtype, "thin groups dgrad " + name)
+    got_dw = dw.cpu().numpy()
+    assert_close(got_dw.transpose(0, 1, 4, 2, 3) if cl else got_dw, want_dw, dtype, "thin groups wgrad " + name)
+    # the same filter gradient twice: no atomics, so bit for bit
+    assert torch.equal(dw, ops.conv2d_bwd_weights(xd, gd, desc))
 
 
 def test_reference_kat_channels_last():
@@ -958,10 +1035,11 @@ def test_prepacked_filters_give_the_plain_result(case, mode, dtype, policy):
 @pytest.mark.parametrize("case", [c for c in GROUPED if c[0] in ("g2_k3", "g4_pw", "g3_k3_s2", "depthwise_k3", "g2_pw_even")] +
                          [c[:1] + (1,) + c[4:] for c in CHANNELS_LAST if c[0] in ("nhwc_pw", "nhwc_k3", "nhwc_pw_c40_24")],
                          ids=lambda c: c[0])
-def test_prepacked_filters_grouped_and_channels_last(case, mode):
+def test_prepacked_filters_grouped_and_channels_last(case, mode, tune_env):
     """Groups (one packing job per group and pass -- more jobs than one launch holds for the depthwise case) and
     channels-last activations, fp16."""
     name, G, n, ci, co, h, w, kh, kw, stride, dilation, padding = case
+    tune_env(PHX_TUNE_THIN_MAX="0")  # (groups of few channels on the matrix-core kernels: the FMA kernels pack nothing)
     nhwc = name.startswith("nhwc")
     dtype = torch.float16
     r = np.random.default_rng(name_seed(name) + 22)
