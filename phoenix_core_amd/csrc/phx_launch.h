@@ -23,6 +23,7 @@ struct BigLds {
 inline unsigned int grid_rows(int groups) { return groups > 1 ? (unsigned int)groups : 1u; }
 
 bool tuning_noearly();  // PHX_TUNE_NOEARLY, read once with the other planner overrides
+bool tuning_thin_notile();  // PHX_TUNE_THIN_NOTILE
 
 // which instantiation of the forward / input-gradient kernel to run
 struct FwdVariant {
@@ -107,6 +108,9 @@ int launch_dense_small(bool half_storage, int pass, const DenseSmallArgs& a, hip
 // channels-first tensors and filter (phx_launch_thin.hip).  in = x (forward, filter gradient) or the output gradient
 // (input gradient); out = y, dx or dw.  Filter element (r, co, i, kh, kw), co over all groups and i inside its group,
 // at r * wcs + co * so + i * si + kh * skh + kw * skw.
+struct ThinDiv {  // t / d == umulhi(t, m) + (t & one): m = ceil(2^32 / d), one = 0, or m = 0, one = ~0 for d == 1; exact while t * d < 2^32
+    unsigned int m, one;
+};
 struct ThinArgs {
     const void* in;
     const void* w;
@@ -120,8 +124,14 @@ struct ThinArgs {
     int Kh, Kw, sh, sw, dh, dw, pt, pl;
     int Z;                    // filter gradient: slices of the images summed by separate workgroups
     unsigned int mh, mw;      // strided input gradient: ceil(2^32 / sh), ceil(2^32 / sw); 0 for a unit stride
+    // the tiled kernels (set by launch_thin): a workgroup works on R output rows of J images from a window tile of
+    // J x rows x cols entries in LDS; bands = such tiles per image group; d_* = the divisions they make
+    int tile_R, tile_J, tile_rows, tile_cols, tile_bands;
+    ThinDiv d_cols, d_rows, d_wout, d_R;
 };
+// < 0: not launched; 1: ran on the kernel that stages window tiles in LDS; 0 otherwise
 int launch_thin(bool half_storage, int pass, const ThinArgs& a, hipStream_t st);
+int thin_wgrad_slices(bool half_storage, const ThinArgs& a);  // Z of the filter gradient (sizes `partial`)
 
 // space-to-depth rearrangements (stride-2 convolutions with very few input channels)
 int launch_s2d_input(bool half_storage, const S2dArgs& a, hipStream_t st);

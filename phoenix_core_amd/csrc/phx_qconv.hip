@@ -35,7 +35,8 @@ struct Tuning {
     bool pwrall = false;              // PHX_TUNE_PWRALL: ... and every problem that kernel can run goes to it (not only those of at most 32 output channels)
     bool nowincl = false;             // PHX_TUNE_NOWINCL: channels-last windowed problems go through the transposes
     bool nogroupbatch = false;        // PHX_TUNE_NOGROUPBATCH: a grouped convolution runs group after group
-    int thin_max = 4;                 // PHX_TUNE_THIN_MAX: most channels per group that run on the FMA kernels for thin groups (0 = never)
+    int thin_max = 16;                // PHX_TUNE_THIN_MAX: most input x output channels per group that run on the FMA kernels for thin groups (0 = never)
+    bool thin_notile = false;         // PHX_TUNE_THIN_NOTILE: ... and never on the kernel that stages window tiles in LDS
     int wincl_max = 3072;             // PHX_TUNE_WINCL_MAX: largest channels x taps that runs on channels-last tensors directly
     bool nosmalldense = false;        // PHX_TUNE_NOSMALLDENSE: small Dense problems stay on the matrix-core kernels
     int vec = 0;                      // PHX_TUNE_VEC (0 = unset)
@@ -66,6 +67,7 @@ struct Tuning {
         nogroupbatch = getenv("PHX_TUNE_NOGROUPBATCH") != nullptr;
         if (const char* e = getenv("PHX_TUNE_WINCL_MAX")) wincl_max = atoi(e);
         if (const char* e = getenv("PHX_TUNE_THIN_MAX")) thin_max = atoi(e);
+        thin_notile = getenv("PHX_TUNE_THIN_NOTILE") != nullptr;
         nosmalldense = getenv("PHX_TUNE_NOSMALLDENSE") != nullptr;
         if (const char* e = getenv("PHX_TUNE_VEC")) vec = atoi(e);
         if (const char* e = getenv("PHX_TUNE_WGS")) wgs = atoi(e);
@@ -82,6 +84,7 @@ static const Tuning& tune() {
     return g_tune;
 }
 bool tuning_noearly() { return tune().noearly; }
+bool tuning_thin_notile() { return tune().thin_notile; }
 
 // Plans are pure functions of the problem and the tuning overrides; they are computed once per distinct
 // problem (the reference keeps its configured operations per descriptor, src/backend/op_collections.hpp:121-144)
@@ -1774,35 +1777,20 @@ static bool nhwc_wgrad_native(const Problem& p) {
     return !pl.realx && pl.kmode == 16 && pl.MT == 2 && pl.NT == 2 && pl.SW == 1 && (pl.TPW == 1 || pl.TPW == 3);
 }
 
-// Grouped convolutions whose groups hold at most a few channels on either side (depthwise convolutions first of all)
-// run on the fp32 FMA kernels of phx_launch_thin.hip, all groups by one launch per pass, straight on the caller's
-// channels-first tensors and filter: a 32 x 32 matrix-core tile per group would be nearly empty (1.6 % full at 4
-// channels per group), and measured per pass the FMA threads are 6-30x faster there.  PHX_TUNE_THIN_MAX moves the bound.
+// Grouped convolutions whose groups hold only a few channels (depthwise convolutions first of all) run on the FMA
+// kernels of phx_launch_thin.hip, all groups by one launch per pass, straight on the caller's channels-first tensors
+// and filter: a 32 x 32 matrix-core tile per group would be nearly empty (1.6 % full at 4 x 4 channels per group).
+// The matrix-core path costs a tile per group whatever it holds, the FMA threads cost in proportion to the channel
+// pairs of a group (input x output channels): measured at 3x3, 28x28, they are 15x faster at one pair, 1.7x at 16
+// (4 x 4) and 1.6x slower at 64 (8 x 8).  PHX_TUNE_THIN_MAX moves the bound.
 static bool thin_groups(const Problem& p) {
     if (p.groups <= 1 || is_empty(p) || p.real_input || p.ho <= 0 || p.wo <= 0) return false;
-    if (std::max(p.ci, p.co) > tune().thin_max) return false;
-    return (long)std::max(p.ci, p.co) * p.kh * p.kw * 16 <= 48 * 1024 && std::max(p.ci_mem, p.co_mem) <= 65535;
+    if ((long)p.ci * p.co > tune().thin_max) return false;
+    return (long)std::max(p.ci, p.co) * p.kh * p.kw * 32 <= 32 * 1024 && std::max(p.ci_mem, p.co_mem) <= 65535;
 }
 
-// reduction slices of the thin-group filter gradient: enough workgroups to fill the GPU, each with at least a few
-// pixels per thread
-static int thin_wgrad_slices(const Problem& p) {
-    const long taps = (long)p.kh * p.kw;
-    const long columns = (long)p.co_mem * p.ci * (taps == 1 ? 1 : cdiv((int)taps, 9));
-    const long want = (2048 + columns - 1) / columns, fit = std::max(1L, (long)p.n * p.ho * p.wo / (4 * WG_THREADS));
-    return (int)std::max(1L, std::min({want, fit, (long)p.n, 65535L}));
-}
-static size_t thin_workspace(const Problem& p, int pass) {
-    if (pass != PHX_PASS_BWD_WEIGHTS) return 0;
-    return align_up((size_t)thin_wgrad_slices(p) * p.co_mem * p.ci * p.kh * p.kw * 4 * sizeof(float), 256);
-}
-
-// (a, b) = (x, w) forward, (grad, w) input gradient, (x, grad) filter gradient; channels-first tensors of all groups
-static int run_thin(const Problem& p, int pass, hipStream_t st, const void* a, const void* b, const void* bias, void* out, void* ws,
-                    size_t wsb) {
-    if (!a || !b || !out || (pass == PHX_PASS_FWD && p.has_bias && !bias)) return PHX_ERR_INVALID_ARGUMENT;
+static ThinArgs thin_args(const Problem& p) {
     ThinArgs t{};
-    t.in = a; t.out = out;
     t.wcs = p.fs.wcs; t.so = p.fs.so; t.si = p.fs.si; t.skh = p.fs.skh; t.skw = p.fs.skw;
     t.N = p.n; t.groups = p.groups; t.cig = p.ci; t.cog = p.co;
     t.H = p.h; t.W = p.w; t.Ho = p.ho; t.Wo = p.wo;
@@ -1810,9 +1798,23 @@ static int run_thin(const Problem& p, int pass, hipStream_t st, const void* a, c
     t.Z = 1;
     t.mh = p.sh > 1 ? (unsigned int)(((1ULL << 32) + p.sh - 1) / p.sh) : 0u;
     t.mw = p.sw > 1 ? (unsigned int)(((1ULL << 32) + p.sw - 1) / p.sw) : 0u;
+    return t;
+}
+// the filter gradient's partial sums: [slices][output channel x input channel of its group][tap][4]
+static size_t thin_workspace(const Problem& p, int pass) {
+    if (pass != PHX_PASS_BWD_WEIGHTS) return 0;
+    return align_up((size_t)thin_wgrad_slices(p.dtype == PHX_F16, thin_args(p)) * p.co_mem * p.ci * p.kh * p.kw * 4 * sizeof(float), 256);
+}
+
+// (a, b) = (x, w) forward, (grad, w) input gradient, (x, grad) filter gradient; channels-first tensors of all groups
+static int run_thin(const Problem& p, int pass, hipStream_t st, const void* a, const void* b, const void* bias, void* out, void* ws,
+                    size_t wsb) {
+    if (!a || !b || !out || (pass == PHX_PASS_FWD && p.has_bias && !bias)) return PHX_ERR_INVALID_ARGUMENT;
+    ThinArgs t = thin_args(p);
+    t.in = a; t.out = out;
     if (pass == PHX_PASS_BWD_WEIGHTS) {
         t.grad = b;
-        t.Z = thin_wgrad_slices(p);
+        t.Z = thin_wgrad_slices(p.dtype == PHX_F16, t);
         if (thin_workspace(p, pass) > wsb || !ws) return PHX_ERR_WORKSPACE;
         t.partial = static_cast<float*>(ws);
     } else {
@@ -1824,14 +1826,14 @@ static int run_thin(const Problem& p, int pass, hipStream_t st, const void* a, c
         KernelTimer timer(st);
         rc = launch_thin(p.dtype == PHX_F16, pass, t, st);
     }
-    if (rc != 0) return PHX_ERR_NOT_SUPPORTED;
+    if (rc < 0) return PHX_ERR_NOT_SUPPORTED;
     PHX_HIP(hipGetLastError());
     if (pass == PHX_PASS_BWD_WEIGHTS)
-        snprintf(g_name_buf, sizeof(g_name_buf), "qconv_wgrad_fma_thin_%s_g%dx%dx%d_k%dx%d_z%d", p.dtype == PHX_F32 ? "f32" : "f16", p.groups,
-                 p.ci, p.co, p.kh, p.kw, t.Z);
+        snprintf(g_name_buf, sizeof(g_name_buf), "qconv_wgrad_fma_thin_%s_g%dx%dx%d_k%dx%d%s_z%d", p.dtype == PHX_F32 ? "f32" : "f16", p.groups,
+                 p.ci, p.co, p.kh, p.kw, rc == 1 ? "_tile" : "", t.Z);
     else
-        snprintf(g_name_buf, sizeof(g_name_buf), "qconv_%s_fma_thin_%s_g%dx%dx%d_k%dx%d", pass == PHX_PASS_FWD ? "fwd" : "dgrad",
-                 p.dtype == PHX_F32 ? "f32" : "f16", p.groups, p.ci, p.co, p.kh, p.kw);
+        snprintf(g_name_buf, sizeof(g_name_buf), "qconv_%s_fma_thin_%s_g%dx%dx%d_k%dx%d%s", pass == PHX_PASS_FWD ? "fwd" : "dgrad",
+                 p.dtype == PHX_F32 ? "f32" : "f16", p.groups, p.ci, p.co, p.kh, p.kw, rc == 1 ? "_tile" : "");
     g_last_kernel = g_name_buf;
     say(p, pass == PHX_PASS_FWD ? "forward (thin groups)" : pass == PHX_PASS_BWD_DATA ? "input gradient (thin groups)" : "filter gradient (thin groups)");
     return PHX_OK;

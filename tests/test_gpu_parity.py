@@ -490,6 +490,12 @@ THIN_GROUPS = [
     ("dw_k3_n40", 4, False, 40, 4, 4, 14, 14, 3, 3, 1, 1, "SAME"),              # filter gradient summed over several slices of the images
     ("dw_k5_n9", 3, False, 9, 3, 3, 12, 11, 5, 5, 1, 1, "SAME"),                # 25 taps: three workgroups of nine per channel pair
     ("dw_k3_1px", 2, False, 1, 2, 2, 3, 3, 3, 3, 1, 1, "VALID"),                # one output position
+    ("dw_mult16_k3", 2, False, 2, 2, 32, 8, 9, 3, 3, 1, 1, "SAME"),             # sixteen output channels per input channel
+    ("g2_4x4_k3", 2, False, 3, 8, 8, 7, 8, 3, 3, 1, 1, "SAME"),                 # sixteen channel pairs per group: the most that runs here
+    ("dw_k3_wide", 2, False, 1, 2, 2, 3, 1100, 3, 3, 1, 1, "SAME"),             # rows wider than a workgroup's outputs: no window tiles
+    ("dw_k3_28_n5", 3, False, 5, 3, 3, 28, 28, 3, 3, 1, 1, "SAME"),             # 784 outputs per tile: a last slot that one wave runs alone
+    ("dw_k3_7x7_n23", 2, False, 23, 2, 2, 7, 7, 3, 3, 1, 1, "SAME"),            # twenty images per tile, the last tile with three
+    ("dw_k3_s2_56", 2, False, 2, 2, 2, 56, 56, 3, 3, 2, 1, "SAME"),             # strided windows: tiles of several row bands
     ("dw_k3_nhwc", 8, True, 2, 8, 8, 10, 9, 3, 3, 1, 1, "SAME"),
     ("dw_k3_s2_nhwc", 6, True, 3, 6, 12, 15, 13, 3, 3, 2, 1, "SAME"),
 ]
@@ -497,16 +503,19 @@ THIN_GROUPS = [
 
 @pytest.mark.parametrize("dtype,policy", [(torch.float32, "fp32"), (torch.float16, "full16"), (torch.float16, "backward32")],
                          ids=["f32", "f16_full16", "f16_backward32"])
-@pytest.mark.parametrize("mode", [16, 8])
+@pytest.mark.parametrize("mode,tiles", [(16, True), (8, True), (16, False)], ids=["p16", "p8", "p16_notile"])
 @pytest.mark.parametrize("case", THIN_GROUPS, ids=lambda c: c[0])
-def test_thin_groups_run_on_fma_threads(case, mode, dtype, policy):
-    """Grouped convolutions with at most four channels per group on either side (depthwise convolutions first of all; the
+def test_thin_groups_run_on_fma_threads(case, mode, tiles, dtype, policy, tune_env):
+    """Grouped convolutions with at most sixteen channel pairs (input x output channels) per group (depthwise convolutions first of all; the
     reference hands `groups` to its scalar convolutions, src/backend/onednn/conv2d.hpp:116-137, and has no vector for
     them) run on the FMA kernels for thin groups, every pass by one launch on the caller's filter: the kernel label says
     so, the filter gradient asks for its partial sums only, and the results are those of G independent convolutions on
     channel slices, which is how the oracle's result is assembled here.  OIHW filter on channels-first tensors, OHWI on
-    channels-last ones (which run through channels-first copies)."""
+    channels-last ones (which run through channels-first copies).  The kernels that stage window tiles in LDS run
+    wherever an output row fits a workgroup (the input gradient: at unit stride); PHX_TUNE_THIN_NOTILE keeps every
+    case on the kernels that read global memory per tap."""
     name, G, cl, n, ci, co, h, w, kh, kw, stride, dilation, padding = case
+    tune_env(PHX_TUNE_THIN_NOTILE=None if tiles else "1")
     cig, cog = ci // G, co // G
     scale = 1.0 if dtype == torch.float32 else 0.5
     g, x, _, b, gr = make_inputs(name_seed(name) + 40, n, ci, co, h, w, kh, kw, stride, dilation, padding, dtype, scale)
@@ -528,6 +537,9 @@ def test_thin_groups_run_on_fma_threads(case, mode, dtype, policy):
     dw = ops.conv2d_bwd_weights(xd, gd, desc)
     names.append(capi.last_kernel_name())
     assert all("_fma_thin_" in k for k in names), names
+    unit_stride = stride == 1 or stride == (1, 1)
+    want_tiles = [tiles and g.wo <= 1024, tiles and unit_stride and w <= 1024, tiles and g.wo <= 1024]
+    assert ["_tile" in k for k in names] == want_tiles, names
     esize = 4 if dtype == torch.float32 else 2
     planes = (x.nbytes + 255) // 256 * 256 + (gr.nbytes + 255) // 256 * 256 if cl else 0
     assert desc.workspace_bytes(capi.PHX_PASS_FWD) == planes
