@@ -39,6 +39,12 @@ CONVS = {
     "c4_pw_f16_128_28": (128, 128, 128, 28, 28, 1, "VALID", "f16"),
     "c4_pw_f16_256_14": (128, 256, 256, 14, 14, 1, "VALID", "f16"),
 }
+# grouped convolutions (run by name only, not part of the default table): name: (..., groups)
+GROUPED = {
+    "x_depthwise_k3_f16_128_28": (32, 128, 128, 28, 28, 3, "SAME", "f16", 128),
+    "x_depthwise_k3_f16_256_14": (64, 256, 256, 14, 14, 3, "SAME", "f16", 256),
+    "x_groups32_k3_f16_128_28": (32, 128, 128, 28, 28, 3, "SAME", "f16", 32),
+}
 DENSE = {"c1_dense_f32": (32, 128, 128, "f32")}  # name: (n, in, out, dtype)
 RESNET = "c5_qresnet50"  # quaternion ResNet-50 forward+backward, N=64, 224x224, fp16 full16 policy
 HEADLINE = "c4_k3_f16_128_28"
@@ -100,7 +106,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="all", choices=["all"] + sorted(CONVS) + sorted(DENSE) + [RESNET])
+    ap.add_argument("--workload", default="all", choices=["all"] + sorted(CONVS) + sorted(GROUPED) + sorted(DENSE) + [RESNET])
     ap.add_argument("--mode", type=int, default=0, choices=[0, 8, 16],
                     help="product formulation; 0 = from UPSTRIDE_MEMORY_OPTIMIZED like the reference (default 8)")
     ap.add_argument("--policy", default=None, help="UPSTRIDE_CONV_FP16_POLICY for fp16 workloads (default full16)")
@@ -342,18 +348,20 @@ def run_conv(name, mode, policy, args, traffic_table):
     import torch
     import phoenix_core_amd as phx
     from phoenix_core_amd import capi
-    n, ci, co, h, w, k, padding, dt = CONVS[name]
+    n, ci, co, h, w, k, padding, dt = (CONVS.get(name) or GROUPED[name])[:8]
+    groups = GROUPED[name][8] if name in GROUPED else 1
     if dt == "f32":
         policy = "fp32"
     ctx = make_context(mode, policy)
     dtype = torch.float32 if dt == "f32" else torch.float16
     dev = torch.device("cuda:0")
-    torch.manual_seed(0x5EED + sorted(CONVS).index(name))
+    torch.manual_seed(0x5EED + sorted(list(CONVS) + list(GROUPED)).index(name))
     scale = 1.0 if dt == "f32" else 0.5
     cl = bool(getattr(args, "channels_last", False))
     x = (scale * torch.randn((4 * n, h, w, ci) if cl else (4 * n, ci, h, w), device=dev)).to(dtype)
-    wt = (scale * torch.randn(4, co, ci, k, k, device=dev) * (2.0 / (ci * k * k)) ** 0.5).to(dtype)
-    desc = phx.Conv2DDescriptor(x.shape, wt.shape, 1, 1, padding, dtype=dtype, context=ctx, data_format="NHWC" if cl else "NCHW")
+    wt = (scale * torch.randn(4, co, ci // groups, k, k, device=dev) * (2.0 / (ci // groups * k * k)) ** 0.5).to(dtype)
+    desc = phx.Conv2DDescriptor(x.shape, wt.shape, 1, 1, padding, groups=groups, dtype=dtype, context=ctx,
+                                data_format="NHWC" if cl else "NCHW")
     gr = (scale * torch.randn(desc.output_shape, device=dev)).to(dtype)
     ho, wo = desc.output_shape[1:3] if cl else desc.output_shape[2:]
     y = torch.empty(desc.output_shape, dtype=dtype, device=dev)
@@ -382,7 +390,7 @@ def run_conv(name, mode, policy, args, traffic_table):
             dst.copy_(src)  # reads 256 MiB, writes 256 MiB
         del src, dst
     t = _Timed(step, 3, args.steps, args.warmup, outputs=lambda: (y, dx, dw), use_graph=not args.no_graph)
-    flops_pass = 2.0 * 16 * n * co * ci * ho * wo * k * k
+    flops_pass = 2.0 * 16 * n * co * (ci // groups) * ho * wo * k * k
     esize = 4 if dt == "f32" else 2
     # algorithmic bytes of a pass: read the activations (or the gradient), read the filters, write the result
     bytes_pass = {
@@ -400,8 +408,9 @@ def run_conv(name, mode, policy, args, traffic_table):
     del x, wt, gr, y, dx, dw, ws
     torch.cuda.empty_cache()
     return {
-        "workload": "%s: quaternion conv %dx%d stride 1, N=%d (4N=%d rows), %d->%d q-channels, %dx%d, "
-                    "fwd+input-grad+filter-grad%s" % (name, k, k, n, 4 * n, ci, co, h, w, ", channels-last activations" if cl else ""),
+        "workload": "%s: quaternion conv %dx%d stride 1, N=%d (4N=%d rows), %d->%d q-channels%s, %dx%d, "
+                    "fwd+input-grad+filter-grad%s" % (name, k, k, n, 4 * n, ci, co, " in %d groups" % groups if groups > 1 else "", h, w,
+                                                      ", channels-last activations" if cl else ""),
         "data_format": "NHWC" if cl else "NCHW",
         "n": n, "product_mode": mode, "fp16_policy": policy, "padding": padding, "dtype": dt,
         "value": value, "unit": "TFLOP/s", "ms_per_step": t.ms_per_step, "ms_per_step_eager": t.ms_per_step_eager,
@@ -679,9 +688,9 @@ def main():
         emit(head, args.workload)
         print(line(head, args))
         return 0
-    if args.workload in CONVS:
+    if args.workload in CONVS or args.workload in GROUPED:
         head = run_conv(args.workload, mode, policy, args, traffic)
-        if not args.no_cpu_baseline:
+        if not args.no_cpu_baseline and args.workload in CONVS:  # (the CPU restatement has no grouped form)
             head["cpu_baseline"] = cpu_baseline_conv(CONVS[args.workload], mode, args.cpu_seconds)
         emit(head, args.workload)
         print(line(head, args))
