@@ -180,11 +180,13 @@ def test_bottleneck_branch_gradient_inside_the_convolution(stride, cin):
         assert torch.equal(a, b)
 
 
-def test_qconv2d_groups_and_channels_last():
+@pytest.mark.parametrize("ci,co,G", [(8, 12, 2), (8, 16, 8)], ids=["two_groups", "depthwise_two_outputs_per_input"])
+def test_qconv2d_groups_and_channels_last(ci, co, G):
     """QConv2d(groups=G) is G ungrouped layers on channel slices; QConv2d(data_format="NHWC") is the NCHW layer on
-    permuted activations: outputs and all gradients must agree with those compositions."""
+    permuted activations: outputs and all gradients must agree with those compositions.  (The depthwise case runs the
+    layer on the vector-ALU kernels for thin groups and its slices on the matrix-core / fp32 kernels.)"""
     torch.manual_seed(1)
-    n, ci, co, h, G = 2, 8, 12, 10, 2
+    n, h = 2, 10
     ref = phx.QConv2d(ci, co, 3, padding="SAME", bias=True, context=Ctx(8), groups=G).cuda()
     assert tuple(ref.weight.shape) == (4, co, ci // G, 3, 3)
     with torch.no_grad():
