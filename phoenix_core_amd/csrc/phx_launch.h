@@ -127,9 +127,11 @@ struct ThinArgs {
     // the tiled kernels (set by launch_thin): a workgroup works on R output rows of J images from a window tile of
     // J x rows x cols entries in LDS; bands = such tiles per image group; d_* = the divisions they make
     int tile_R, tile_J, tile_rows, tile_cols, tile_bands;
+    int tile_row0, tile_col0;  // strided input gradient by phases: the tile's first row / column relative to its first output block
     ThinDiv d_cols, d_rows, d_wout, d_R;
 };
-// < 0: not launched; 1: ran on the kernel that stages window tiles in LDS; 0 otherwise
+// < 0: not launched; 1: ran on the kernel that stages window tiles in LDS, 2: the strided input gradient by phases from
+// such tiles; 0 otherwise
 int launch_thin(bool half_storage, int pass, const ThinArgs& a, hipStream_t st);
 int thin_wgrad_slices(bool half_storage, const ThinArgs& a);  // Z of the filter gradient (sizes `partial`)
 

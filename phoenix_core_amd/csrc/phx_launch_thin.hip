@@ -313,6 +313,142 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_thin_tile_kernel(const ThinA
         }
 }
 
+// The input gradient of a convolution with stride 2 (along either axis or both) from window tiles: a window entry
+// (kh, kw) reaches the input positions of ONE phase (h mod sh, w mod sw) only -- ph(kh) = (kh dh - pt) mod sh -- and
+// there it reads the gradient at block row + (ph + pt - kh dh) / sh.  So a thread takes whole sh x sw blocks of input
+// positions (two of them), a tile holds the gradient window of R block rows, and every entry is applied once, to the
+// accumulators of its phase: no divisibility tests and none of the entries that do not apply (three in four at
+// stride 2 x 2) are touched.  The per-entry tile offset and phase are tabled in LDS next to the filter.
+constexpr int THIN_PH_SLOTS = 2;  // blocks of input positions per thread
+
+template <int N, typename Body>
+__device__ __forceinline__ void thin_dispatch_phase(int phase, const Body& body) {
+    if constexpr (N == 1) {
+        body(std::integral_constant<int, 0>());
+    } else {
+        if (phase == N - 1) body(std::integral_constant<int, N - 1>());
+        else thin_dispatch_phase<N - 1>(phase, body);
+    }
+}
+
+template <typename TS, int SH, int SW>
+__global__ void __launch_bounds__(WG_THREADS) qconv_thin_dgrad_phase_kernel(const ThinArgs P) {
+    using T = ThinTile<TS>;
+    using Entry = typename T::Entry;
+    using Filter = typename T::Filter;
+    constexpr int PHASES = SH * SW;
+    extern __shared__ __align__(16) unsigned char thin_lds[];
+    const int taps = P.Kh * P.Kw;
+    const int c = blockIdx.y;  // input channel, over all groups
+    const int K = P.cog, g = c / P.cig, c_in_group = c - g * P.cig;
+    Filter* filt = reinterpret_cast<Filter*>(thin_lds);                                    // [output channel of the group][entry]
+    int2* table = reinterpret_cast<int2*>(thin_lds + (size_t)K * taps * sizeof(Filter));   // [entry]: tile offset, phase
+    Entry* tile = reinterpret_cast<Entry*>(thin_lds + (size_t)K * taps * sizeof(Filter) + (size_t)((taps + 1) & ~1) * sizeof(int2));
+    const TS* W = static_cast<const TS*>(P.w);
+    for (int e = threadIdx.x; e < K * taps; e += WG_THREADS) {
+        const int k = e / taps, t = e - k * taps, kh = t / P.Kw, kw = t - kh * P.Kw;
+        const TS* at = W + ((long)g * P.cog + k) * P.so + c_in_group * P.si + kh * P.skh + kw * P.skw;
+        float w[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const float v = ldf<TS>(at + r * P.wcs);
+            w[r] = r ? -v : v;  // conjugate
+        }
+        filt[e] = T::filter(w);
+        if (k == 0) {
+            const int ph = ((kh * P.dh - P.pt) % SH + SH) % SH, pw = ((kw * P.dw - P.pl) % SW + SW) % SW;
+            const int oh = (ph + P.pt - kh * P.dh) / SH, ow = (pw + P.pl - kw * P.dw) / SW;  // (exact divisions)
+            table[t] = make_int2((oh - P.tile_row0) * P.tile_cols + (ow - P.tile_col0), ph * SW + pw);
+        }
+    }
+    const int Hb = (P.H + SH - 1) / SH, Wb = (P.W + SW - 1) / SW;  // blocks of input positions
+    const long opix = (long)P.H * P.W, ipix = (long)P.Ho * P.Wo;
+    const long Cin_all = (long)P.groups * K, Cout_all = (long)P.groups * P.cig;
+    const long in_cs = P.N * Cin_all * ipix, out_cs = P.N * Cout_all * opix;
+    const int ng = blockIdx.x / P.tile_bands, band = blockIdx.x - ng * P.tile_bands;
+    const int n0 = ng * P.tile_J, r0 = band * P.tile_R;
+    const int ih0 = r0 + P.tile_row0, iw0 = P.tile_col0;
+    const int entries = P.tile_J * P.tile_rows * P.tile_cols;
+    const int image_in = (int)(Cin_all * ipix), image_out = (int)(Cout_all * opix);
+
+    int tbase[THIN_PH_SLOTS], oh0[THIN_PH_SLOTS], ow0[THIN_PH_SLOTS];
+    unsigned int oaddr[THIN_PH_SLOTS];
+    bool live[THIN_PH_SLOTS];
+    float acc[THIN_PH_SLOTS][PHASES][4];
+#pragma unroll
+    for (int s = 0; s < THIN_PH_SLOTS; ++s) {
+        const int pix = threadIdx.x + s * WG_THREADS;
+        const int prow = thin_div(pix, P.d_wout), bw = pix - prow * Wb;
+        const int j = thin_div(prow, P.d_R), r = prow - j * P.tile_R;
+        live[s] = j < P.tile_J && n0 + j < P.N && r0 + r < Hb;
+        tbase[s] = live[s] ? (j * P.tile_rows + r) * P.tile_cols + bw : 0;
+        oh0[s] = (r0 + r) * SH;
+        ow0[s] = bw * SW;
+        oaddr[s] = (unsigned int)(j * image_out + r * SH * P.W + bw * SW);
+#pragma unroll
+        for (int ph = 0; ph < PHASES; ++ph)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) acc[s][ph][q] = 0.f;
+    }
+    const int wave_first = __builtin_amdgcn_readfirstlane(threadIdx.x & ~63);
+    const int total = P.tile_J * P.tile_R * Wb;
+    const int wave_slots = total <= wave_first ? 0 : std::min(THIN_PH_SLOTS, (total - wave_first + WG_THREADS - 1) / WG_THREADS);
+
+    const TS* in = static_cast<const TS*>(P.in) + ((long)n0 * Cin_all + (long)g * K) * ipix;
+    for (int k = 0; k < K; ++k, in += ipix) {
+        if (k) __syncthreads();
+        const __amdgpu_buffer_rsrc_t planes[4] = {thin_buffer(in), thin_buffer(in + in_cs), thin_buffer(in + 2 * in_cs),
+                                                  thin_buffer(in + 3 * in_cs)};
+#pragma unroll 2
+        for (int e = threadIdx.x; e < entries; e += WG_THREADS) {
+            const int row = thin_div(e, P.d_cols), tc = e - row * P.tile_cols;
+            const int j = thin_div(row, P.d_rows), tr = row - j * P.tile_rows;
+            const int ih = ih0 + tr, iw = iw0 + tc;
+            const bool ok = n0 + j < P.N && (unsigned)ih < (unsigned)P.Ho && (unsigned)iw < (unsigned)P.Wo;
+            const unsigned int at = ok ? (unsigned int)(j * image_in + ih * P.Wo + iw) * (unsigned int)sizeof(TS) : THIN_NOWHERE;
+            float v[4];
+#pragma unroll
+            for (int p = 0; p < 4; ++p) v[p] = thin_load<TS>(planes[p], at);
+            tile[e] = T::entry(v);
+        }
+        __syncthreads();
+        const auto run_taps = [&](auto slots) {
+            constexpr int NS = decltype(slots)::value;
+            for (int t = 0; t < taps; ++t) {
+                const int2 where = table[t];
+                const int toff = __builtin_amdgcn_readfirstlane(where.x), phase = __builtin_amdgcn_readfirstlane(where.y);
+                const Filter f = filt[k * taps + t];
+                Entry x[NS > 0 ? NS : 1];
+#pragma unroll
+                for (int s = 0; s < NS; ++s) x[s] = tile[tbase[s] + toff];
+                thin_dispatch_phase<PHASES>(phase, [&](auto which) {
+                    constexpr int PH = decltype(which)::value;
+#pragma unroll
+                    for (int s = 0; s < NS; ++s) T::mac(acc[s][PH], x[s], f);
+                    // (keeps the phases' instances apart: merged, they would index the accumulators by a variable,
+                    // which puts them into scratch memory)
+                    asm volatile("; phase %0" ::"n"(PH));
+                });
+            }
+        };
+        thin_dispatch_slots<THIN_PH_SLOTS>(wave_slots, run_taps);
+    }
+    TS* out = static_cast<TS*>(P.out) + ((long)n0 * Cout_all + c) * opix + (long)r0 * SH * P.W;
+    const __amdgpu_buffer_rsrc_t oplanes[4] = {thin_buffer(out), thin_buffer(out + out_cs), thin_buffer(out + 2 * out_cs),
+                                               thin_buffer(out + 3 * out_cs)};
+#pragma unroll
+    for (int s = 0; s < THIN_PH_SLOTS; ++s)
+#pragma unroll
+        for (int ph = 0; ph < SH; ++ph)
+#pragma unroll
+            for (int pw = 0; pw < SW; ++pw)
+                if (live[s] && oh0[s] + ph < P.H && ow0[s] + pw < P.W) {
+#pragma unroll
+                    for (int q = 0; q < 4; ++q)
+                        thin_store(oplanes[q], (oaddr[s] + ph * P.W + pw) * (unsigned int)sizeof(TS), (TS)acc[s][ph * SW + pw][q]);
+                }
+}
+
 static ThinDiv thin_magic(int d) { return d > 1 ? ThinDiv{(unsigned int)(((1ULL << 32) + d - 1) / d), 0u} : ThinDiv{0u, ~0u}; }
 
 // Fills the tile fields of `a` for the forward pass / unit-stride input gradient; false where the tiled kernel does not
@@ -557,6 +693,42 @@ __global__ void __launch_bounds__(WG_THREADS) thin_wgrad_reduce_kernel(const Thi
     static_cast<TS*>(P.out)[q * P.wcs + co * P.so + i * P.si + kh * P.skh + kw * P.skw] = (TS)sum;
 }
 
+// The plan of the strided input gradient by phases (strides 1 or 2 per axis): blocks of sh x sw input positions play
+// the part of the outputs, the tile is the gradient window of R block rows.
+static bool thin_phase_plan(bool half_storage, ThinArgs& a, size_t& lds) {
+    if (a.sh > 2 || a.sw > 2 || (a.sh == 1 && a.sw == 1)) return false;
+    const int Hb = (a.H + a.sh - 1) / a.sh, Wb = (a.W + a.sw - 1) / a.sw, taps = a.Kh * a.Kw;
+    const int tile_pixels = THIN_PH_SLOTS * WG_THREADS;
+    if (Wb > tile_pixels) return false;
+    const auto span = [](int k, int d, int pad, int s, int& lo, int& hi) {  // block offsets that the window entries read
+        lo = 1 << 30; hi = -(1 << 30);
+        for (int i = 0; i < k; ++i) {
+            const int ph = ((i * d - pad) % s + s) % s, o = (ph + pad - i * d) / s;
+            lo = std::min(lo, o); hi = std::max(hi, o);
+        }
+    };
+    int rlo, rhi, clo, chi;
+    span(a.Kh, a.dh, a.pt, a.sh, rlo, rhi);
+    span(a.Kw, a.dw, a.pl, a.sw, clo, chi);
+    const size_t entry = half_storage ? 8 : 16;
+    const size_t fixed = (size_t)a.cog * taps * (half_storage ? 32 : 16) + (size_t)((taps + 1) & ~1) * 8;
+    const long cols = (long)Wb + chi - clo;
+    int R = std::min(Hb, std::max(1, tile_pixels / Wb));
+    int J = R == Hb ? std::min(a.N, std::max(1, tile_pixels / (Hb * Wb))) : 1;
+    const auto bytes_of = [&](int r, int j) { return fixed + (size_t)j * (r + rhi - rlo) * cols * entry; };
+    while (J > 1 && bytes_of(R, J) > THIN_TILE_LDS) --J;
+    while (R > 1 && bytes_of(R, J) > THIN_TILE_LDS) R = (R + 1) / 2;
+    if (bytes_of(R, J) > THIN_TILE_LDS) return false;
+    const long image = (long)a.groups * std::max((long)a.cig * a.H * a.W, (long)a.cog * a.Ho * a.Wo);
+    if ((J + 1) * image * (half_storage ? 2 : 4) >= (1L << 32)) return false;
+    a.tile_R = R; a.tile_J = J; a.tile_rows = R + rhi - rlo; a.tile_cols = (int)cols;
+    a.tile_bands = (Hb + R - 1) / R;
+    a.tile_row0 = rlo; a.tile_col0 = clo;
+    a.d_cols = thin_magic(a.tile_cols); a.d_rows = thin_magic(a.tile_rows); a.d_wout = thin_magic(Wb); a.d_R = thin_magic(R);
+    lds = bytes_of(R, J);
+    return true;
+}
+
 static int thin_wgrad_taps_per_block(int taps) { return taps == 1 ? 1 : 9; }
 
 // The filter gradient's plan: tiled kernel or not (tile fields of `a`, LDS bytes), and the number of slices Z of the
@@ -631,6 +803,22 @@ int launch_thin(bool half_storage, int pass, const ThinArgs& a, hipStream_t st) 
             else hipLaunchKernelGGL((qconv_thin_tile_kernel<float, false>), grid, block, tile_lds, st, t);
         }
         return 1;
+    }
+    if (!tuning_thin_notile() && dgrad && thin_phase_plan(half_storage, t, tile_lds)) {
+        const long blocks = (long)((a.N + t.tile_J - 1) / t.tile_J) * t.tile_bands;
+        if (blocks >= (1L << 31)) return -1;
+        const dim3 grid((unsigned int)blocks, (unsigned int)channels), block(WG_THREADS);
+        const int key = t.sh * 10 + t.sw;
+        if (half_storage) {
+            if (key == 22) hipLaunchKernelGGL((qconv_thin_dgrad_phase_kernel<_Float16, 2, 2>), grid, block, tile_lds, st, t);
+            else if (key == 21) hipLaunchKernelGGL((qconv_thin_dgrad_phase_kernel<_Float16, 2, 1>), grid, block, tile_lds, st, t);
+            else hipLaunchKernelGGL((qconv_thin_dgrad_phase_kernel<_Float16, 1, 2>), grid, block, tile_lds, st, t);
+        } else {
+            if (key == 22) hipLaunchKernelGGL((qconv_thin_dgrad_phase_kernel<float, 2, 2>), grid, block, tile_lds, st, t);
+            else if (key == 21) hipLaunchKernelGGL((qconv_thin_dgrad_phase_kernel<float, 2, 1>), grid, block, tile_lds, st, t);
+            else hipLaunchKernelGGL((qconv_thin_dgrad_phase_kernel<float, 1, 2>), grid, block, tile_lds, st, t);
+        }
+        return 2;
     }
     const long pixels = (long)a.N * (dgrad ? (long)a.H * a.W : (long)a.Ho * a.Wo);
     const long blocks = (pixels + WG_THREADS - 1) / WG_THREADS;

@@ -1833,7 +1833,7 @@ static int run_thin(const Problem& p, int pass, hipStream_t st, const void* a, c
                  p.ci, p.co, p.kh, p.kw, rc == 1 ? "_tile" : "", t.Z);
     else
         snprintf(g_name_buf, sizeof(g_name_buf), "qconv_%s_fma_thin_%s_g%dx%dx%d_k%dx%d%s", pass == PHX_PASS_FWD ? "fwd" : "dgrad",
-                 p.dtype == PHX_F32 ? "f32" : "f16", p.groups, p.ci, p.co, p.kh, p.kw, rc == 1 ? "_tile" : "");
+                 p.dtype == PHX_F32 ? "f32" : "f16", p.groups, p.ci, p.co, p.kh, p.kw, rc == 1 ? "_tile" : rc == 2 ? "_phasetile" : "");
     g_last_kernel = g_name_buf;
     say(p, pass == PHX_PASS_FWD ? "forward (thin groups)" : pass == PHX_PASS_BWD_DATA ? "input gradient (thin groups)" : "filter gradient (thin groups)");
     return PHX_OK;

@@ -496,6 +496,10 @@ THIN_GROUPS = [
     ("dw_k3_28_n5", 3, False, 5, 3, 3, 28, 28, 3, 3, 1, 1, "SAME"),             # 784 outputs per tile: a last slot that one wave runs alone
     ("dw_k3_7x7_n23", 2, False, 23, 2, 2, 7, 7, 3, 3, 1, 1, "SAME"),            # twenty images per tile, the last tile with three
     ("dw_k3_s2_56", 2, False, 2, 2, 2, 56, 56, 3, 3, 2, 1, "SAME"),             # strided windows: tiles of several row bands
+    ("dw_k5_s2_dil2_odd", 3, False, 2, 3, 6, 17, 21, 5, 5, 2, 2, "SAME"),         # stride 2 with dilation 2: every entry on one phase
+    ("dw_k3_s12", 4, False, 2, 4, 4, 9, 22, 3, 3, (1, 2), 1, "SAME"),           # stride along W only
+    ("dw_k4_s2_valid_56", 2, False, 3, 2, 2, 56, 57, 4, 4, 2, 1, "VALID"),      # even filter, odd width, several row bands
+    ("dw_k3_s2_7x7_n30", 2, False, 30, 2, 4, 7, 7, 3, 3, 2, 1, "SAME"),         # many images per tile
     ("dw_k3_nhwc", 8, True, 2, 8, 8, 10, 9, 3, 3, 1, 1, "SAME"),
     ("dw_k3_s2_nhwc", 6, True, 3, 6, 12, 15, 13, 3, 3, 2, 1, "SAME"),
 ]
@@ -537,9 +541,13 @@ def test_thin_groups_run_on_fma_threads(case, mode, tiles, dtype, policy, tune_e
     dw = ops.conv2d_bwd_weights(xd, gd, desc)
     names.append(capi.last_kernel_name())
     assert all("_fma_thin_" in k for k in names), names
-    unit_stride = stride == 1 or stride == (1, 1)
-    want_tiles = [tiles and g.wo <= 1024, tiles and unit_stride and w <= 1024, tiles and g.wo <= 1024]
-    assert ["_tile" in k for k in names] == want_tiles, names
+    sh, sw = stride if isinstance(stride, tuple) else (stride, stride)
+    # the input gradient: window tiles at unit stride, tiles walked by phases at stride 2, per-tap loads beyond that
+    dgrad_kind = "" if not tiles else "_tile" if (sh, sw) == (1, 1) and w <= 1024 else \
+        "_phasetile" if max(sh, sw) == 2 and -(-w // sw) <= 512 else ""
+    want_kinds = ["_tile" if tiles and g.wo <= 1024 else "", dgrad_kind, "_tile" if tiles and g.wo <= 1024 else ""]
+    got_kinds = ["_phasetile" if "_phasetile" in k else "_tile" if "_tile" in k else "" for k in names]
+    assert got_kinds == want_kinds, names
     esize = 4 if dtype == torch.float32 else 2
     planes = (x.nbytes + 255) // 256 * 256 + (gr.nbytes + 255) // 256 * 256 if cl else 0
     assert desc.workspace_bytes(capi.PHX_PASS_FWD) == planes
