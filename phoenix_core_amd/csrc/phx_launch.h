@@ -124,6 +124,7 @@ struct ThinArgs {
     int Kh, Kw, sh, sw, dh, dw, pt, pl;
     int Z;                    // filter gradient: slices of the images summed by separate workgroups
     unsigned int mh, mw;      // strided input gradient: ceil(2^32 / sh), ceil(2^32 / sw); 0 for a unit stride
+    int kchunk;               // per-tap forward / input gradient (set by launch_thin): filters per LDS chunk
     // the tiled kernels (set by launch_thin): a workgroup works on R output rows of J images from a window tile of
     // J x rows x cols entries in LDS; bands = such tiles per image group; d_* = the divisions they make
     int tile_R, tile_J, tile_rows, tile_cols, tile_bands;

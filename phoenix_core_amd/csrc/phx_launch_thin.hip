@@ -20,30 +20,18 @@ namespace phx {
 // consecutive threads take consecutive pixels of a row, i.e. consecutive addresses of every plane they read.
 template <typename TS, bool DGRAD>
 __global__ void __launch_bounds__(WG_THREADS) qconv_thin_kernel(const ThinArgs P) {
-    extern __shared__ float4 thin_filter[];  // [other-side channel][tap]
+    extern __shared__ float4 thin_filter[];  // [other-side channel of the chunk][tap]
     const int taps = P.Kh * P.Kw;
     const int c = blockIdx.y;  // channel of the written tensor, over all groups
     const int cside = DGRAD ? P.cig : P.cog, K = DGRAD ? P.cog : P.cig;
     const int g = c / cside, c_in_group = c - g * cside;
     const TS* W = static_cast<const TS*>(P.w);
-    for (int e = threadIdx.x; e < K * taps; e += WG_THREADS) {
-        const int k = e / taps, t = e - k * taps, kh = t / P.Kw, kw = t - kh * P.Kw;
-        const long co = DGRAD ? g * P.cog + k : c, ci = DGRAD ? c_in_group : k;
-        const TS* at = W + co * P.so + ci * P.si + kh * P.skh + kw * P.skw;
-        float4 v;
-        v.x = ldf<TS>(at);
-        v.y = ldf<TS>(at + P.wcs);
-        v.z = ldf<TS>(at + 2 * P.wcs);
-        v.w = ldf<TS>(at + 3 * P.wcs);
-        if (DGRAD) { v.y = -v.y; v.z = -v.z; v.w = -v.w; }  // conjugate
-        thin_filter[e] = v;
-    }
-    __syncthreads();
     const int Hin = DGRAD ? P.Ho : P.H, Win = DGRAD ? P.Wo : P.W;    // the tensor read
     const int Hout = DGRAD ? P.H : P.Ho, Wout = DGRAD ? P.W : P.Wo;  // the tensor written
     const long opix = (long)Hout * Wout, ipix = (long)Hin * Win;
-    const long idx = (long)blockIdx.x * WG_THREADS + threadIdx.x;
-    if (idx >= P.N * opix) return;
+    const long idx_all = (long)blockIdx.x * WG_THREADS + threadIdx.x;
+    const bool live = idx_all < P.N * opix;
+    const long idx = live ? idx_all : 0;  // (a thread past the end computes the first output again and stores nothing)
     const int n = (int)(idx / opix), rem = (int)(idx - n * opix);
     const int oh = rem / Wout, ow = rem - oh * Wout;
     const long Cin_all = (long)P.groups * K, Cout_all = (long)P.groups * cside;
@@ -68,40 +56,60 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_thin_kernel(const ThinArgs P
 #pragma unroll
             for (int q = 0; q < 4; ++q) acc[q] += (qneg(p, q) ? -v[p] : v[p]) * wv[p ^ q];
     };
-    if (!DGRAD || (P.sh == 1 && P.sw == 1)) {
-        // no branches around the loads: a tap outside the image reads the plane's first element and counts as zero, so
-        // the loads of several taps are in flight together
-        for (int k = 0; k < K; ++k, in += ipix) {
-            int kh = 0, kw = 0;
-#pragma unroll 3
-            for (int t = 0; t < taps; ++t) {
-                const int ih = DGRAD ? oh + P.pt - kh * P.dh : oh * P.sh - P.pt + kh * P.dh;
-                const int iw = DGRAD ? ow + P.pl - kw * P.dw : ow * P.sw - P.pl + kw * P.dw;
-                const bool ok = (unsigned)ih < (unsigned)Hin && (unsigned)iw < (unsigned)Win;
-                tap(in + (ok ? (long)ih * Win + iw : 0L), ok, k * taps + t);
-                if (++kw == P.Kw) { kw = 0; ++kh; }
-            }
+    // exact division by multiplication: m = ceil(2^32 / s) (0: s == 1)
+    const auto divide = [](int t, int s, unsigned int m, int& quotient) {
+        quotient = m ? (int)__umulhi((unsigned int)t, m) : t;
+        return t >= 0 && quotient * s == t;
+    };
+    // the other side's channels go through LDS in chunks of P.kchunk filters (all of them at once for thin groups)
+    for (int k0 = 0; k0 < K; k0 += P.kchunk) {
+        const int kn = K - k0 < P.kchunk ? K - k0 : P.kchunk;
+        if (k0) __syncthreads();  // (everyone has read the previous chunk)
+        for (int e = threadIdx.x; e < kn * taps; e += WG_THREADS) {
+            const int k = e / taps, t = e - k * taps, kh = t / P.Kw, kw = t - kh * P.Kw;
+            const long co = DGRAD ? g * P.cog + k0 + k : c, ci = DGRAD ? c_in_group : k0 + k;
+            const TS* at = W + co * P.so + ci * P.si + kh * P.skh + kw * P.skw;
+            float4 v;
+            v.x = ldf<TS>(at);
+            v.y = ldf<TS>(at + P.wcs);
+            v.z = ldf<TS>(at + 2 * P.wcs);
+            v.w = ldf<TS>(at + 3 * P.wcs);
+            if (DGRAD) { v.y = -v.y; v.z = -v.z; v.w = -v.w; }  // conjugate
+            thin_filter[e] = v;
         }
-    } else {
-        // strided input gradient: a window entry (kh, kw) reaches this input position from the output position
-        // ((h + pt - kh dh) / sh, (w + pl - kw dw) / sw) where both divisions leave no remainder; one entry in sh * sw
-        // does, the others are skipped.  Exact division by multiplication: mh = ceil(2^32 / sh) (0: sh == 1).
-        const auto divide = [](int t, int s, unsigned int m, int& quotient) {
-            quotient = m ? (int)__umulhi((unsigned int)t, m) : t;
-            return t >= 0 && quotient * s == t;
-        };
-        for (int k = 0; k < K; ++k, in += ipix) {
-            for (int kh = 0; kh < P.Kh; ++kh) {
-                int ih;
-                if (!divide(oh + P.pt - kh * P.dh, P.sh, P.mh, ih) || ih >= Hin) continue;
-                for (int kw = 0; kw < P.Kw; ++kw) {
-                    int iw;
-                    if (!divide(ow + P.pl - kw * P.dw, P.sw, P.mw, iw) || iw >= Win) continue;
-                    tap(in + (long)ih * Win + iw, true, (k * P.Kh + kh) * P.Kw + kw);
+        __syncthreads();
+        if (!DGRAD || (P.sh == 1 && P.sw == 1)) {
+            // no branches around the loads: a tap outside the image reads the plane's first element and counts as zero,
+            // so the loads of several taps are in flight together
+            for (int k = 0; k < kn; ++k, in += ipix) {
+                int kh = 0, kw = 0;
+#pragma unroll 3
+                for (int t = 0; t < taps; ++t) {
+                    const int ih = DGRAD ? oh + P.pt - kh * P.dh : oh * P.sh - P.pt + kh * P.dh;
+                    const int iw = DGRAD ? ow + P.pl - kw * P.dw : ow * P.sw - P.pl + kw * P.dw;
+                    const bool ok = (unsigned)ih < (unsigned)Hin && (unsigned)iw < (unsigned)Win;
+                    tap(in + (ok ? (long)ih * Win + iw : 0L), ok, k * taps + t);
+                    if (++kw == P.Kw) { kw = 0; ++kh; }
+                }
+            }
+        } else {
+            // strided input gradient: a window entry (kh, kw) reaches this input position from the output position
+            // ((h + pt - kh dh) / sh, (w + pl - kw dw) / sw) where both divisions leave no remainder; one entry in
+            // sh * sw does, the others are skipped
+            for (int k = 0; k < kn; ++k, in += ipix) {
+                for (int kh = 0; kh < P.Kh; ++kh) {
+                    int ih;
+                    if (!divide(oh + P.pt - kh * P.dh, P.sh, P.mh, ih) || ih >= Hin) continue;
+                    for (int kw = 0; kw < P.Kw; ++kw) {
+                        int iw;
+                        if (!divide(ow + P.pl - kw * P.dw, P.sw, P.mw, iw) || iw >= Win) continue;
+                        tap(in + (long)ih * Win + iw, true, (k * P.Kh + kh) * P.Kw + kw);
+                    }
                 }
             }
         }
     }
+    if (!live) return;
     TS* out = static_cast<TS*>(P.out) + (n * Cout_all + c) * opix + rem;
 #pragma unroll
     for (int q = 0; q < 4; ++q) out[q * out_cs] = (TS)acc[q];
@@ -165,6 +173,7 @@ struct ThinTile<_Float16> {
 constexpr int THIN_PXT = 4;                          // outputs per thread
 constexpr int THIN_TILE_PIXELS = THIN_PXT * WG_THREADS;
 constexpr size_t THIN_TILE_LDS = 64 * 1024;
+constexpr size_t THIN_FILTER_LDS = 32 * 1024;  // the per-tap kernel's filter chunk
 
 __device__ __forceinline__ int thin_div(int t, const ThinDiv& d) { return (int)(__umulhi((unsigned int)t, d.m) + ((unsigned int)t & d.one)); }
 
@@ -822,15 +831,17 @@ int launch_thin(bool half_storage, int pass, const ThinArgs& a, hipStream_t st) 
     }
     const long pixels = (long)a.N * (dgrad ? (long)a.H * a.W : (long)a.Ho * a.Wo);
     const long blocks = (pixels + WG_THREADS - 1) / WG_THREADS;
-    const size_t lds = (size_t)(dgrad ? a.cog : a.cig) * taps * sizeof(float4);
-    if (blocks >= (1L << 31) || lds > 48 * 1024) return -1;
+    const int K = dgrad ? a.cog : a.cig;
+    t.kchunk = std::min(K, (int)(THIN_FILTER_LDS / (taps * sizeof(float4))));
+    if (blocks >= (1L << 31) || t.kchunk < 1) return -1;
+    const size_t lds = (size_t)t.kchunk * taps * sizeof(float4);
     const dim3 grid((unsigned int)blocks, (unsigned int)channels), block(WG_THREADS);
     if (dgrad) {
-        if (half_storage) hipLaunchKernelGGL((qconv_thin_kernel<_Float16, true>), grid, block, lds, st, a);
-        else hipLaunchKernelGGL((qconv_thin_kernel<float, true>), grid, block, lds, st, a);
+        if (half_storage) hipLaunchKernelGGL((qconv_thin_kernel<_Float16, true>), grid, block, lds, st, t);
+        else hipLaunchKernelGGL((qconv_thin_kernel<float, true>), grid, block, lds, st, t);
     } else {
-        if (half_storage) hipLaunchKernelGGL((qconv_thin_kernel<_Float16, false>), grid, block, lds, st, a);
-        else hipLaunchKernelGGL((qconv_thin_kernel<float, false>), grid, block, lds, st, a);
+        if (half_storage) hipLaunchKernelGGL((qconv_thin_kernel<_Float16, false>), grid, block, lds, st, t);
+        else hipLaunchKernelGGL((qconv_thin_kernel<float, false>), grid, block, lds, st, t);
     }
     return 0;
 }

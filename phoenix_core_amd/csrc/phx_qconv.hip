@@ -36,6 +36,7 @@ struct Tuning {
     bool nowincl = false;             // PHX_TUNE_NOWINCL: channels-last windowed problems go through the transposes
     bool nogroupbatch = false;        // PHX_TUNE_NOGROUPBATCH: a grouped convolution runs group after group
     int thin_max = 16;                // PHX_TUNE_THIN_MAX: most input x output channels per group that run on the FMA kernels for thin groups (0 = never)
+    bool direct = false;              // PHX_TUNE_DIRECT: every convolution those kernels can run goes to them (an independent path to check the matrix-core kernels against)
     bool thin_notile = false;         // PHX_TUNE_THIN_NOTILE: ... and never on the kernel that stages window tiles in LDS
     int wincl_max = 3072;             // PHX_TUNE_WINCL_MAX: largest channels x taps that runs on channels-last tensors directly
     bool nosmalldense = false;        // PHX_TUNE_NOSMALLDENSE: small Dense problems stay on the matrix-core kernels
@@ -68,6 +69,7 @@ struct Tuning {
         if (const char* e = getenv("PHX_TUNE_WINCL_MAX")) wincl_max = atoi(e);
         if (const char* e = getenv("PHX_TUNE_THIN_MAX")) thin_max = atoi(e);
         thin_notile = getenv("PHX_TUNE_THIN_NOTILE") != nullptr;
+        direct = getenv("PHX_TUNE_DIRECT") != nullptr;
         nosmalldense = getenv("PHX_TUNE_NOSMALLDENSE") != nullptr;
         if (const char* e = getenv("PHX_TUNE_VEC")) vec = atoi(e);
         if (const char* e = getenv("PHX_TUNE_WGS")) wgs = atoi(e);
@@ -594,6 +596,7 @@ static bool plan_forward(const Corr& c, int mode, bool f16mfma, FwdPlan& best, b
             cand[nc++] = 8; cand[nc++] = 16; cand[nc++] = 32; cand[nc++] = BN;
             // (long rows whose window must stay within the staging limit: fractions of the workgroup's pixels)
             cand[nc++] = BN / 2; cand[nc++] = (3 * BN) / 4; cand[nc++] = 48; cand[nc++] = 80;
+            cand[nc++] = 1; cand[nc++] = 2; cand[nc++] = 3;  // (windows that take most of the staging limit by themselves)
             for (int a = 0; a < nc; ++a) {
                 const int TW = std::min(cand[a], std::min(c.Wout, BN));
                 if (TW <= 0) continue;
@@ -605,6 +608,7 @@ static bool plan_forward(const Corr& c, int mode, bool f16mfma, FwdPlan& best, b
                     if (pairs) HTW = (HTW + 2) & ~1;  // room for the even start column, even pitch
                     if (chunks) HTW = (HTW + 7) & ~7;  // whole 8-position chunks
                     if (vstage) HTW = (HTW + 3) & ~3;  // whole 4-position groups
+                    NB = std::max(1, std::min(NB, 256 / (HTH * HTW)));  // (as many whole images as the staging limit holds)
                     consider(NB, TH, TW, HTH, HTW, cdiv(c.N, NB), cdiv(c.Hout, TH), cdiv(c.Wout, TW), 0);
                 }
             }
@@ -1783,10 +1787,19 @@ static bool nhwc_wgrad_native(const Problem& p) {
 // The matrix-core path costs a tile per group whatever it holds, the FMA threads cost in proportion to the channel
 // pairs of a group (input x output channels): measured at 3x3, 28x28, they are 15x faster at one pair, 1.7x at 16
 // (4 x 4) and 1.6x slower at 64 (8 x 8).  PHX_TUNE_THIN_MAX moves the bound.
+//
+// The same kernels are the way out for filters whose window does not fit the matrix-core kernels' staging: those
+// stage one window position per thread, so the window of a single output position -- ((kh-1) dh + 1) rows of
+// ((kw-1) dw + 1) columns, rounded up to whole 8-position chunks -- must not exceed 256 positions (a 7x7 filter at
+// dilation 3, a 17x17 one).  Such convolutions, grouped or not, run here at vector-ALU speed rather than not at all.
+static bool window_beyond_staging(const Problem& p) {
+    return ((long)(p.kh - 1) * p.dh + 1) * ((((long)(p.kw - 1) * p.dw + 1) + 7) & ~7L) > WG_THREADS;
+}
 static bool thin_groups(const Problem& p) {
-    if (p.groups <= 1 || is_empty(p) || p.real_input || p.ho <= 0 || p.wo <= 0) return false;
-    if ((long)p.ci * p.co > tune().thin_max) return false;
-    return (long)std::max(p.ci, p.co) * p.kh * p.kw * 32 <= 32 * 1024 && std::max(p.ci_mem, p.co_mem) <= 65535;
+    if (is_empty(p) || p.real_input || p.ho <= 0 || p.wo <= 0) return false;
+    if ((long)p.kh * p.kw > 2048 || std::max(p.ci_mem, p.co_mem) > 65535) return false;  // (a filter chunk in LDS; grid rows)
+    if (tune().direct || window_beyond_staging(p)) return true;
+    return p.groups > 1 && (long)p.ci * p.co <= tune().thin_max;
 }
 
 static ThinArgs thin_args(const Problem& p) {
@@ -1847,7 +1860,7 @@ namespace phx {
 // pointwise, input gradient by phases), whose rearrangement kernels work on one group's tensors.  Everything else
 // runs group after group.  The plans are those of one group, so the results are the same either way.
 static bool group_batchable(const Problem& p, int pass) {
-    if (p.groups <= 1 || is_empty(p) || p.nhwc || p.real_input || tune().nogroupbatch || thin_groups(p)) return false;
+    if (p.groups <= 1 || is_empty(p) || p.nhwc || p.real_input || tune().nogroupbatch) return false;
     S2dView v;
     Problem q;
     size_t xs_bytes = 0;
@@ -1887,12 +1900,13 @@ size_t phx_qconv2d_workspace_bytes(const phx_qconv_desc* desc, int pass) {
     if (desc && desc->algebra != PHX_QUATERNION) return algebra_conv_workspace_bytes(desc, pass);
     Problem p;
     if (problem_from_conv(desc, p) != PHX_OK) return 0;
+    if (thin_groups(p)) return ChannelsLast(p).bytes() + thin_workspace(p, pass);
     if (nhwc_native(p, pass)) return nhwc_native_workspace(p, pass);
     if (nhwc_window_native(p, pass)) return workspace_for(p, pass);
     if (pass == PHX_PASS_BWD_WEIGHTS && nhwc_wgrad_native(p)) return workspace_for(p, pass);
     // (packed images / partial sums of all groups side by side where one launch runs them)
     if (group_batchable(p, pass)) return (size_t)p.groups * workspace_for(p, pass);
-    return ChannelsLast(p).bytes() + (thin_groups(p) ? thin_workspace(p, pass) : workspace_for(p, pass));
+    return ChannelsLast(p).bytes() + workspace_for(p, pass);
 }
 
 // Small Dense problems (a classifier head, the reference's 128 -> 128 benchmark layer at batch 32) run on plain fp32
@@ -1935,18 +1949,19 @@ static int conv_fwd_quaternion(const phx_qconv_desc* desc, phx_stream_t stream, 
     Problem p;
     const int rc = problem_from_conv(desc, p);
     if (rc != PHX_OK) return rc;
-    if (nhwc_native(p, PHX_PASS_FWD))
+    const bool direct = thin_groups(p);  // the vector-ALU kernels: groups of few channels, windows beyond the staging limit
+    if (!direct && nhwc_native(p, PHX_PASS_FWD))
         return run_pwx_nhwc(p, MAP_FWD, static_cast<hipStream_t>(stream), x, w, p.has_bias ? bias_or_null : nullptr, y, workspace,
                             workspace_bytes);
     const GroupOffsets o(p);
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (nhwc_window_native(p, PHX_PASS_FWD)) {
+    if (!direct && nhwc_window_native(p, PHX_PASS_FWD)) {
         g_window_cl = true;
         const int nrc = do_fwd(p, st, x, w, bias_or_null, y, dry ? nullptr : workspace, dry ? 0 : workspace_bytes);
         g_window_cl = false;
         return nrc;
     }
-    if (group_batchable(p, PHX_PASS_FWD)) {
+    if (!direct && group_batchable(p, PHX_PASS_FWD)) {
         const GroupBatchScope batch(p);
         return do_fwd(p, st, x, w, bias_or_null, y, dry ? nullptr : workspace, dry ? 0 : workspace_bytes);
     }
@@ -1960,7 +1975,7 @@ static int conv_fwd_quaternion(const phx_qconv_desc* desc, phx_stream_t stream, 
         x = ws;
         y_planes = ws + cl.x_bytes;
     }
-    if (thin_groups(p)) {  // (no packed form: a packing session finds nothing to pack)
+    if (direct) {  // (no packed form: a packing session finds nothing to pack)
         if (g_pack.mode == PackSession::USE) return PHX_ERR_NOT_SUPPORTED;
         if (!dry)
             if (const int trc = run_thin(p, PHX_PASS_FWD, st, x, w, bias_or_null, y_planes, nullptr, 0)) return trc;
@@ -2005,17 +2020,18 @@ static int conv_bwd_data_quaternion(const phx_qconv_desc* desc, phx_stream_t str
     // the gradient with respect to a real-valued input has imaginary parts that are stored nowhere;
     // the reference refuses the request likewise (src/conv2d.hpp:394-398)
     if (p.real_input) return PHX_ERR_INVALID_ARGUMENT;
-    if (nhwc_native(p, PHX_PASS_BWD_DATA))
+    const bool direct = thin_groups(p);
+    if (!direct && nhwc_native(p, PHX_PASS_BWD_DATA))
         return run_pwx_nhwc(p, MAP_DGRAD, static_cast<hipStream_t>(stream), grad, w, nullptr, dx, workspace, workspace_bytes);
     const GroupOffsets o(p);
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (nhwc_window_native(p, PHX_PASS_BWD_DATA)) {
+    if (!direct && nhwc_window_native(p, PHX_PASS_BWD_DATA)) {
         g_window_cl = true;
         const int nrc = do_bwd_data(p, st, grad, w, dx, dry ? nullptr : workspace, dry ? 0 : workspace_bytes);
         g_window_cl = false;
         return nrc;
     }
-    if (group_batchable(p, PHX_PASS_BWD_DATA)) {
+    if (!direct && group_batchable(p, PHX_PASS_BWD_DATA)) {
         const GroupBatchScope batch(p);
         return do_bwd_data(p, st, grad, w, dx, dry ? nullptr : workspace, dry ? 0 : workspace_bytes);
     }
@@ -2029,7 +2045,7 @@ static int conv_bwd_data_quaternion(const phx_qconv_desc* desc, phx_stream_t str
         grad = ws + cl.x_bytes;
         dx_planes = ws;
     }
-    if (thin_groups(p)) {
+    if (direct) {
         if (g_pack.mode == PackSession::USE) return PHX_ERR_NOT_SUPPORTED;
         if (!dry)
             if (const int trc = run_thin(p, PHX_PASS_BWD_DATA, st, grad, w, nullptr, dx_planes, nullptr, 0)) return trc;
@@ -2152,13 +2168,14 @@ int phx_qconv2d_bwd_weights(const phx_qconv_desc* desc, phx_stream_t stream, con
     if (rc != PHX_OK) return rc;
     const GroupOffsets o(p);
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (nhwc_wgrad_native(p)) {
+    const bool direct = thin_groups(p);
+    if (!direct && nhwc_wgrad_native(p)) {
         g_window_cl = true;
         const int nrc = do_bwd_weights(p, st, x, grad, dw, workspace, workspace_bytes);
         g_window_cl = false;
         return nrc;
     }
-    if (group_batchable(p, PHX_PASS_BWD_WEIGHTS)) {
+    if (!direct && group_batchable(p, PHX_PASS_BWD_WEIGHTS)) {
         const GroupBatchScope batch(p);
         return do_bwd_weights(p, st, x, grad, dw, workspace, workspace_bytes);
     }
@@ -2171,7 +2188,7 @@ int phx_qconv2d_bwd_weights(const phx_qconv_desc* desc, phx_stream_t stream, con
         x = ws;
         grad = ws + cl.x_bytes;
     }
-    if (thin_groups(p))
+    if (direct)
         return run_thin(p, PHX_PASS_BWD_WEIGHTS, st, x, grad, nullptr, dw, ws ? ws + cl.bytes() : nullptr, workspace_bytes - cl.bytes());
     for (int g = 0; g < o.runs; ++g) {
         const int grc = do_bwd_weights(p, st, o.at(x, g * o.x), o.at(grad, g * o.y), o.at(dw, g * o.w),

@@ -75,6 +75,8 @@ CONV_CASES = [
     ("k3_dil2", 1, 4, 6, 12, 12, 3, 3, 1, 2, "SAME"),
     ("k32_s21", 2, 8, 8, 13, 19, 3, 2, (2, 1), 1, "SAME"),    # stride along H only: zero insertion in rows, dense columns
     ("k32_asym", 1, 4, 4, 8, 9, 3, 2, (1, 2), (2, 1), (2, 0, 1, 3)),
+    ("k7_s2_dil2", 1, 3, 4, 22, 50, 7, 7, 2, 2, "SAME"),      # a 13x13 window: fits the staging limit with tiles of 1..3 columns only
+    ("k7x2_dil54_s2", 2, 8, 8, 31, 6, 7, 2, 2, (5, 4), "VALID"),   # one output position per image, a window of 248 staged positions: one image per tile
     ("single_pixel", 4, 6, 6, 1, 1, 1, 1, 1, 1, "VALID"),
     ("co_gt_128", 1, 8, 136, 7, 7, 1, 1, 1, 1, "VALID"),
 ]
@@ -250,7 +252,7 @@ def test_empty_input_is_a_no_op_and_zeroes_dw():
 
 FP16_CASES = [c for c in CONV_CASES if c[0] in ("pw_64", "pw_ragged", "pw_7x7img", "k3_same", "k3_same_56", "k3_ragged",
                                                 "k3_valid", "k3_s2", "pw_s2", "pw_s2_odd", "pw_s31", "k7_s2", "k3_s2_c4", "k5_s2_valid", "k3_dil2", "k32_s21", "k32_asym",
-                                                "co_gt_128")] + [
+                                                "co_gt_128", "k7_s2_dil2", "k7x2_dil54_s2")] + [
     ("k3_s3", 2, 8, 8, 13, 13, 3, 3, 3, 1, "SAME"),
     ("k4_same", 2, 8, 16, 13, 15, 4, 4, 1, 1, "SAME"),        # four taps per filter row share a filter-gradient workgroup
     ("k24_c40", 3, 40, 24, 9, 21, 2, 4, 1, 1, "VALID"),
@@ -474,6 +476,75 @@ def test_groups_run_in_one_launch_per_kernel(case, mode, dtype, policy, tune_env
             assert torch.equal(a, b)
     if dtype == torch.float16:
         assert torch.equal(got["one launch"][0][3], got["one launch"][0][0]) and torch.equal(got["one launch"][0][4], got["one launch"][0][1])
+
+
+BIG_WINDOWS = [
+    # name, n, ci, co, h, w, kh, kw, stride, dilation, padding
+    ("k7_dil3", 2, 3, 5, 24, 25, 7, 7, 1, 3, "SAME"),               # a 19x19 window
+    ("k17_valid", 1, 2, 3, 20, 21, 17, 17, 1, 1, "VALID"),
+    ("k7_dil3_s2", 1, 4, 4, 30, 27, 7, 7, 2, 3, "SAME"),            # input gradient by phases, every entry on its own phase pattern
+    ("k9x5_dil4_s3", 2, 5, 2, 40, 30, 9, 5, 3, 4, (5, 2, 0, 7)),    # stride 3: the per-tap input gradient
+    ("k17_c40_24", 1, 40, 24, 18, 19, 17, 17, 1, 1, "SAME"),        # more filter entries than LDS holds: chunks of channels
+]
+
+
+@pytest.mark.parametrize("dtype,policy", [(torch.float32, "fp32"), (torch.float16, "full16")], ids=["f32", "f16_full16"])
+@pytest.mark.parametrize("mode", [16, 8])
+@pytest.mark.parametrize("case", BIG_WINDOWS, ids=lambda c: c[0])
+def test_windows_beyond_the_staging_limit(case, mode, dtype, policy):
+    """The matrix-core kernels stage one window position per thread: a filter whose window for a single output
+    position -- ((kh-1) dh + 1) x ((kw-1) dw + 1), columns in whole chunks of 8 -- exceeds 256 positions runs on the
+    vector-ALU kernels instead (any filter size and dilation is valid at the reference's boundary,
+    src/backend/onednn/conv2d.hpp:116-210).  Against the oracle; no packed form, partial sums as the only workspace."""
+    name, n, ci, co, h, w, kh, kw, stride, dilation, padding = case
+    scale = 1.0 if dtype == torch.float32 else 0.5
+    g, x, wt, b, gr = make_inputs(name_seed(name) + 50, n, ci, co, h, w, kh, kw, stride, dilation, padding, dtype, scale)
+    desc = phx.Conv2DDescriptor(x.shape, wt.shape, stride, dilation, padding, use_bias=True, dtype=dtype, context=Ctx(mode, policy))
+    xd, wd, bd, gd = (torch.from_numpy(a).cuda() for a in (x, wt, b, gr))
+    y = phx.conv2d_fwd(xd, wd, bd, desc)
+    names = [capi.last_kernel_name()]
+    dx = ops.conv2d_bwd_data(wd, gd, desc)
+    names.append(capi.last_kernel_name())
+    dw = ops.conv2d_bwd_weights(xd, gd, desc)
+    names.append(capi.last_kernel_name())
+    assert all("_fma_thin_" in k for k in names), names
+    assert desc.workspace_bytes(capi.PHX_PASS_FWD) == 0 and desc.workspace_bytes(capi.PHX_PASS_BWD_DATA) == 0
+    assert ops.conv2d_pack_filters(wd, desc) is None
+    x64, w64, b64, g64 = (a.astype(np.float64) for a in (x, wt, b, gr))
+    want_y = oracle.conv2d_fwd(g, x64, w64, b64, "hamilton")
+    want_dw, want_dx = oracle.conv2d_bwd(g, x64, w64, g64, "hamilton")
+    assert_close(y.cpu().numpy(), want_y, dtype, "fwd " + names[0])
+    assert_close(dx.cpu().numpy(), want_dx, dtype, "dgrad " + names[1])
+    assert_close(dw.cpu().numpy(), want_dw, dtype, "wgrad " + names[2])
+
+
+DIRECT_CASES = ("pw_ragged", "k3_same", "k3_ragged", "k3_s2", "pw_s31", "k7_s2", "k5_s2_valid", "k3_dil2", "k32_asym", "k7_s2_dil2")
+
+
+@pytest.mark.parametrize("dtype,policy", [(torch.float32, "fp32"), (torch.float16, "full16")], ids=["f32", "f16_full16"])
+@pytest.mark.parametrize("tiles", [True, False], ids=["tiles", "per_tap"])
+@pytest.mark.parametrize("case", [c for c in CONV_CASES if c[0] in DIRECT_CASES], ids=lambda c: c[0])
+def test_vector_alu_kernels_agree_with_the_matrix_core_kernels(case, tiles, dtype, policy, tune_env):
+    """PHX_TUNE_DIRECT sends ordinary (ungrouped) convolutions to the vector-ALU kernels as well: two implementations
+    that share no device code, on the same tensors."""
+    name, n, ci, co, h, w, kh, kw, stride, dilation, padding = case
+    scale = 1.0 if dtype == torch.float32 else 0.5
+    g, x, wt, b, gr = make_inputs(name_seed(name) + 51, n, ci, co, h, w, kh, kw, stride, dilation, padding, dtype, scale)
+    desc = phx.Conv2DDescriptor(x.shape, wt.shape, stride, dilation, padding, use_bias=True, dtype=dtype, context=Ctx(8, policy))
+    xd, wd, bd, gd = (torch.from_numpy(a).cuda() for a in (x, wt, b, gr))
+    got = {}
+    for direct in (False, True):
+        tune_env(PHX_TUNE_DIRECT="1" if direct else None, PHX_TUNE_THIN_NOTILE=None if tiles else "1")
+        outs = [phx.conv2d_fwd(xd, wd, bd, desc)]
+        names = [capi.last_kernel_name()]
+        outs.append(ops.conv2d_bwd_data(wd, gd, desc))
+        names.append(capi.last_kernel_name())
+        outs.append(ops.conv2d_bwd_weights(xd, gd, desc))
+        names.append(capi.last_kernel_name())
+        assert all(("_fma_thin_" in k) == direct for k in names), names
+        got[direct] = outs
+    for a, r, what in zip(got[True], got[False], ("fwd", "dgrad", "wgrad")):
+        assert_close(a.cpu().numpy(), r.cpu().numpy().astype(np.float64), dtype, "%s %s" % (what, name))
 
 
 THIN_GROUPS = [
