@@ -170,8 +170,9 @@ struct ThinTile<_Float16> {
     }
 };
 
+constexpr int THIN_TILE_THREADS = 256;  // workgroup of the forward / unit-stride input-gradient tile kernel (64 / 128 measured 10-25 % slower at 3x3)
 constexpr int THIN_PXT = 4;                          // outputs per thread
-constexpr int THIN_TILE_PIXELS = THIN_PXT * WG_THREADS;
+constexpr int THIN_TILE_PIXELS = THIN_PXT * THIN_TILE_THREADS;
 constexpr size_t THIN_TILE_LDS = 64 * 1024;
 constexpr size_t THIN_FILTER_LDS = 32 * 1024;  // the per-tap kernel's filter chunk
 
@@ -213,7 +214,7 @@ __device__ __forceinline__ void thin_dispatch_slots(int slots, const Body& body)
 }
 
 template <typename TS, bool DGRAD>
-__global__ void __launch_bounds__(WG_THREADS) qconv_thin_tile_kernel(const ThinArgs P) {
+__global__ void __launch_bounds__(THIN_TILE_THREADS) qconv_thin_tile_kernel(const ThinArgs P) {
     using T = ThinTile<TS>;
     using Entry = typename T::Entry;
     using Filter = typename T::Filter;
@@ -225,7 +226,7 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_thin_tile_kernel(const ThinA
     Filter* filt = reinterpret_cast<Filter*>(thin_lds);                          // [other-side channel][tap]
     Entry* tile = reinterpret_cast<Entry*>(thin_lds + (size_t)K * taps * sizeof(Filter));  // [image][window row][window column]
     const TS* W = static_cast<const TS*>(P.w);
-    for (int e = threadIdx.x; e < K * taps; e += WG_THREADS) {
+    for (int e = threadIdx.x; e < K * taps; e += THIN_TILE_THREADS) {
         const int k = e / taps, t = e - k * taps, kh = t / P.Kw, kw = t - kh * P.Kw;
         const long co = DGRAD ? g * P.cog + k : c, ci = DGRAD ? c_in_group : k;
         const TS* at = W + co * P.so + ci * P.si + kh * P.skh + kw * P.skw;
@@ -258,7 +259,7 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_thin_tile_kernel(const ThinA
     float acc[THIN_PXT][4];
 #pragma unroll
     for (int s = 0; s < THIN_PXT; ++s) {
-        const int pix = threadIdx.x + s * WG_THREADS;
+        const int pix = threadIdx.x + s * THIN_TILE_THREADS;
         const int prow = thin_div(pix, P.d_wout), ow = pix - prow * Wout;
         const int j = thin_div(prow, P.d_R), r = prow - j * P.tile_R;
         live[s] = j < P.tile_J && n0 + j < P.N && r0 + r < Hout;
@@ -272,7 +273,7 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_thin_tile_kernel(const ThinA
     // would leave idle (784 outputs of a 28 x 28 image: the fourth slot is run by the first wave alone)
     const int wave_first = __builtin_amdgcn_readfirstlane(threadIdx.x & ~63);
     const int total = P.tile_J * P.tile_R * Wout;
-    const int wave_slots = total <= wave_first ? 0 : std::min(THIN_PXT, (total - wave_first + WG_THREADS - 1) / WG_THREADS);
+    const int wave_slots = total <= wave_first ? 0 : std::min(THIN_PXT, (total - wave_first + THIN_TILE_THREADS - 1) / THIN_TILE_THREADS);
 
     const TS* in = static_cast<const TS*>(P.in) + ((long)n0 * Cin_all + (long)g * K) * ipix;
     for (int k = 0; k < K; ++k, in += ipix) {
@@ -280,7 +281,7 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_thin_tile_kernel(const ThinA
         const __amdgpu_buffer_rsrc_t planes[4] = {thin_buffer(in), thin_buffer(in + in_cs), thin_buffer(in + 2 * in_cs),
                                                   thin_buffer(in + 3 * in_cs)};
 #pragma unroll 2
-        for (int e = threadIdx.x; e < entries; e += WG_THREADS) {
+        for (int e = threadIdx.x; e < entries; e += THIN_TILE_THREADS) {
             const int row = thin_div(e, P.d_cols), tc = e - row * P.tile_cols;
             const int j = thin_div(row, P.d_rows), tr = row - j * P.tile_rows;
             const int ih = ih0 + tr, iw = iw0 + tc;
@@ -803,7 +804,7 @@ int launch_thin(bool half_storage, int pass, const ThinArgs& a, hipStream_t st) 
     if (!tuning_thin_notile() && thin_tile_plan(half_storage, dgrad, (dgrad ? a.cog : a.cig) * taps, THIN_TILE_PIXELS, t, tile_lds)) {
         const long blocks = (long)((a.N + t.tile_J - 1) / t.tile_J) * t.tile_bands;
         if (blocks >= (1L << 31)) return -1;
-        const dim3 grid((unsigned int)blocks, (unsigned int)channels), block(WG_THREADS);
+        const dim3 grid((unsigned int)blocks, (unsigned int)channels), block(THIN_TILE_THREADS);
         if (dgrad) {
             if (half_storage) hipLaunchKernelGGL((qconv_thin_tile_kernel<_Float16, true>), grid, block, tile_lds, st, t);
             else hipLaunchKernelGGL((qconv_thin_tile_kernel<float, true>), grid, block, tile_lds, st, t);
