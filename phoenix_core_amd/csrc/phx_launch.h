@@ -123,6 +123,7 @@ struct ThinArgs {
     int H, W, Ho, Wo;         // input and output image of the forward pass
     int Kh, Kw, sh, sw, dh, dw, pt, pl;
     int Z;                    // filter gradient: slices of the images summed by separate workgroups
+    int real_x;               // x is real-valued: [N][channels][H][W], its imaginary components are zero and not stored
     unsigned int mh, mw;      // strided input gradient: ceil(2^32 / sh), ceil(2^32 / sw); 0 for a unit stride
     int kchunk;               // per-tap forward / input gradient (set by launch_thin): filters per LDS chunk
     // the tiled kernels (set by launch_thin): a workgroup works on R output rows of J images from a window tile of

@@ -35,7 +35,9 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_thin_kernel(const ThinArgs P
     const int n = (int)(idx / opix), rem = (int)(idx - n * opix);
     const int oh = rem / Wout, ow = rem - oh * Wout;
     const long Cin_all = (long)P.groups * K, Cout_all = (long)P.groups * cside;
-    const long in_cs = P.N * Cin_all * ipix, out_cs = P.N * Cout_all * opix;
+    // (real-valued input: one stored component; the loads of the absent ones go to the stored one and count as zero)
+    const bool real_x = !DGRAD && P.real_x;
+    const long in_cs = real_x ? 0 : P.N * Cin_all * ipix, out_cs = P.N * Cout_all * opix;
     const TS* in = static_cast<const TS*>(P.in) + (n * Cin_all + (long)g * K) * ipix;
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
     if (!DGRAD && P.bias) {
@@ -47,7 +49,7 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_thin_kernel(const ThinArgs P
 #pragma unroll
         for (int p = 0; p < 4; ++p) {
             const float f = ldf<TS>(px + p * in_cs);
-            v[p] = ok ? f : 0.f;
+            v[p] = (ok && !(p && real_x)) ? f : 0.f;
         }
         const float4 w4 = thin_filter[e];
         const float wv[4] = {w4.x, w4.y, w4.z, w4.w};
@@ -243,7 +245,8 @@ __global__ void __launch_bounds__(THIN_TILE_THREADS) qconv_thin_tile_kernel(cons
     const int rstep = DGRAD ? 1 : P.sh, cstep = DGRAD ? 1 : P.sw;    // window rows / columns per output row / column
     const long opix = (long)Hout * Wout, ipix = (long)Hin * Win;
     const long Cin_all = (long)P.groups * K, Cout_all = (long)P.groups * cside;
-    const long in_cs = P.N * Cin_all * ipix, out_cs = P.N * Cout_all * opix;
+    const bool real_x = !DGRAD && P.real_x;  // real-valued input: one stored component, the others read as zero
+    const long in_cs = real_x ? 0 : P.N * Cin_all * ipix, out_cs = P.N * Cout_all * opix;
     const int ng = blockIdx.x / P.tile_bands, band = blockIdx.x - ng * P.tile_bands;
     const int n0 = ng * P.tile_J, r0 = band * P.tile_R;
     // the tile's first row and column in the tensor read
@@ -289,7 +292,7 @@ __global__ void __launch_bounds__(THIN_TILE_THREADS) qconv_thin_tile_kernel(cons
             const unsigned int at = ok ? (unsigned int)(j * image_in + ih * Win + iw) * (unsigned int)sizeof(TS) : THIN_NOWHERE;
             float v[4];
 #pragma unroll
-            for (int p = 0; p < 4; ++p) v[p] = thin_load<TS>(planes[p], at);
+            for (int p = 0; p < 4; ++p) v[p] = thin_load<TS>(planes[p], (p && real_x) ? THIN_NOWHERE : at);
             tile[e] = T::entry(v);
         }
         __syncthreads();
@@ -500,7 +503,7 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_thin_wgrad_kernel(const Thin
     const int n0 = (int)((long)blockIdx.z * P.N / P.Z), n1 = (int)((long)(blockIdx.z + 1) * P.N / P.Z);
     const long Ci_all = (long)P.groups * P.cig, Co_all = (long)P.groups * P.cog;
     const long xpix = (long)P.H * P.W, gpix = (long)P.Ho * P.Wo;
-    const long x_cs = P.N * Ci_all * xpix, g_cs = P.N * Co_all * gpix;
+    const long x_cs = P.real_x ? 0 : P.N * Ci_all * xpix, g_cs = P.N * Co_all * gpix;  // (real-valued x: one stored component)
     const TS* x = static_cast<const TS*>(P.in) + ((long)g * P.cig + i) * xpix;
     const TS* gr = static_cast<const TS*>(P.grad) + (long)co * gpix;
     int th[TB], tw[TB];  // window offsets of this workgroup's taps
@@ -532,7 +535,7 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_thin_wgrad_kernel(const Thin
 #pragma unroll
             for (int p = 0; p < 4; ++p) {
                 const float v = ldf<TS>(px + p * x_cs);
-                cx[p] = !ok ? 0.f : p ? -v : v;  // conjugate
+                cx[p] = (!ok || (p && P.real_x)) ? 0.f : p ? -v : v;  // conjugate
             }
 #pragma unroll
             for (int p = 0; p < 4; ++p)
@@ -582,7 +585,7 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_thin_wgrad_tile_kernel(const
     const int taps = P.Kh * P.Kw, tap0 = blockIdx.y * TB;
     const long Ci_all = (long)P.groups * P.cig, Co_all = (long)P.groups * P.cog;
     const long xpix = (long)P.H * P.W, gpix = (long)P.Ho * P.Wo;
-    const long x_cs = P.N * Ci_all * xpix, g_cs = P.N * Co_all * gpix;
+    const long x_cs = P.real_x ? 0 : P.N * Ci_all * xpix, g_cs = P.N * Co_all * gpix;  // (real-valued x: one stored component)
     const TS* x = static_cast<const TS*>(P.in) + ((long)g * P.cig + i) * xpix;
     const TS* gr = static_cast<const TS*>(P.grad) + (long)co * gpix;
     int toff[TB];  // tile offsets of this workgroup's taps
@@ -647,7 +650,7 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_thin_wgrad_tile_kernel(const
                 float v[4];
 #pragma unroll
                 for (int p = 0; p < 4; ++p) {
-                    const float f = thin_load<TS>(xplanes[p], at);
+                    const float f = thin_load<TS>(xplanes[p], (p && P.real_x) ? THIN_NOWHERE : at);
                     v[p] = p ? -f : f;  // conjugate
                 }
                 tile[e] = T::entry(v);

@@ -1796,7 +1796,7 @@ static bool window_beyond_staging(const Problem& p) {
     return ((long)(p.kh - 1) * p.dh + 1) * ((((long)(p.kw - 1) * p.dw + 1) + 7) & ~7L) > WG_THREADS;
 }
 static bool thin_groups(const Problem& p) {
-    if (is_empty(p) || p.real_input || p.ho <= 0 || p.wo <= 0) return false;
+    if (is_empty(p) || p.ho <= 0 || p.wo <= 0) return false;
     if ((long)p.kh * p.kw > 2048 || std::max(p.ci_mem, p.co_mem) > 65535) return false;  // (a filter chunk in LDS; grid rows)
     if (tune().direct || window_beyond_staging(p)) return true;
     return p.groups > 1 && (long)p.ci * p.co <= tune().thin_max;
@@ -1809,6 +1809,7 @@ static ThinArgs thin_args(const Problem& p) {
     t.H = p.h; t.W = p.w; t.Ho = p.ho; t.Wo = p.wo;
     t.Kh = p.kh; t.Kw = p.kw; t.sh = p.sh; t.sw = p.sw; t.dh = p.dh; t.dw = p.dw; t.pt = p.pt; t.pl = p.pl;
     t.Z = 1;
+    t.real_x = p.real_input ? 1 : 0;
     t.mh = p.sh > 1 ? (unsigned int)(((1ULL << 32) + p.sh - 1) / p.sh) : 0u;
     t.mw = p.sw > 1 ? (unsigned int)(((1ULL << 32) + p.sw - 1) / p.sw) : 0u;
     return t;

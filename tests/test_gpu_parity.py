@@ -547,6 +547,56 @@ def test_vector_alu_kernels_agree_with_the_matrix_core_kernels(case, tiles, dtyp
         assert_close(a.cpu().numpy(), r.cpu().numpy().astype(np.float64), dtype, "%s %s" % (what, name))
 
 
+# name, groups, channels-last, n, ci, co, h, w, kh, kw, stride, dilation, padding
+REAL_INPUT_ON_VECTOR_ALUS = [
+    ("real_dw_k3_s2", 3, False, 2, 3, 6, 15, 13, 3, 3, 2, 1, "SAME"),          # depthwise first layer, two outputs per colour
+    ("real_k17", 1, False, 1, 3, 5, 24, 21, 17, 17, 1, 1, "SAME"),             # a window beyond the staging limit
+    ("real_k7_dil3_s2", 1, False, 2, 3, 4, 30, 27, 7, 7, 2, 3, "VALID"),
+    ("real_dw_k5_nhwc", 3, True, 2, 3, 3, 12, 11, 5, 5, 1, 1, "SAME"),
+]
+
+
+@pytest.mark.parametrize("dtype,policy", [(torch.float32, "fp32"), (torch.float16, "full16")], ids=["f32", "f16_full16"])
+@pytest.mark.parametrize("tiles", [True, False], ids=["tiles", "per_tap"])
+@pytest.mark.parametrize("case", REAL_INPUT_ON_VECTOR_ALUS, ids=lambda c: c[0])
+def test_vector_alu_kernels_take_real_valued_input(case, tiles, dtype, policy, tune_env):
+    """Real-valued input (src/conv2d.hpp:122-164, 384-430) through the vector-ALU kernels -- groups of few channels,
+    windows beyond the staging limit: x is [n, ci, h, w], its absent imaginary components count as zero.  Against
+    the fp64 closed form on the input padded with zero imaginary parts, group by group."""
+    name, G, cl, n, ci, co, h, w, kh, kw, stride, dilation, padding = case
+    tune_env(PHX_TUNE_THIN_NOTILE=None if tiles else "1")
+    cig, cog = ci // G, co // G
+    scale = 1.0 if dtype == torch.float32 else 0.5
+    g, x, _, b, gr = make_inputs(name_seed(name) + 60, n, ci, co, h, w, kh, kw, stride, dilation, padding, dtype, scale)
+    r = np.random.default_rng(name_seed(name) + 61)
+    npdt = np.float32 if dtype == torch.float32 else np.float16
+    wt = (scale * r.standard_normal((4, co, cig, kh, kw)) * np.sqrt(2.0 / (cig * kh * kw))).astype(npdt)
+    x[n:] = 0
+    to_dev = (lambda a: np.ascontiguousarray(a.transpose(0, 2, 3, 1))) if cl else (lambda a: np.ascontiguousarray(a))
+    x_dev, g_dev = to_dev(x[:n]), to_dev(gr)
+    w_dev = np.ascontiguousarray(wt.transpose(0, 1, 3, 4, 2)) if cl else wt
+    desc = phx.Conv2DDescriptor(x_dev.shape, w_dev.shape, stride, dilation, padding, groups=G, dtype=dtype, context=Ctx(8, policy),
+                                filter_layout="OHWI" if cl else "OIHW", data_format="NHWC" if cl else "NCHW",
+                                real_valued_input=True, require_input_grad=False)
+    xd, wd, gd = (torch.from_numpy(a).cuda() for a in (x_dev, w_dev, g_dev))
+    y = phx.conv2d_fwd(xd, wd, None, desc)
+    k_fwd = capi.last_kernel_name()
+    dw, dx = phx.conv2d_bwd(xd, wd, gd, desc)
+    k_wg = capi.last_kernel_name()
+    assert dx is None and "_fma_thin_" in k_fwd and "_fma_thin_" in k_wg, (k_fwd, k_wg)
+    gg = oracle.make_geom(n, cig, cog, h, w, kh, kw, stride, dilation, padding)
+    x64, w64, g64 = (a.astype(np.float64) for a in (x, wt, gr))
+    want_y, want_dw = np.empty(gr.shape), np.empty(wt.shape)
+    for k in range(G):
+        ic, oc = slice(k * cig, (k + 1) * cig), slice(k * cog, (k + 1) * cog)
+        xs, ws, gs = (np.ascontiguousarray(a) for a in (x64[:, ic], w64[:, oc], g64[:, oc]))
+        want_y[:, oc] = oracle.conv2d_fwd(gg, xs, ws, None, "hamilton")
+        want_dw[:, oc], _ = oracle.conv2d_bwd(gg, xs, ws, gs, "hamilton")
+    got_y, got_dw = y.cpu().numpy(), dw.cpu().numpy()
+    assert_close(got_y.transpose(0, 3, 1, 2) if cl else got_y, want_y, dtype, "fwd " + k_fwd)
+    assert_close(got_dw.transpose(0, 1, 4, 2, 3) if cl else got_dw, want_dw, dtype, "wgrad " + k_wg)
+
+
 THIN_GROUPS = [
     # name, groups, channels-last, n, ci, co, h, w, kh, kw, stride, dilation, padding
     ("dw_k3", 8, False, 2, 8, 8, 10, 10, 3, 3, 1, 1, "SAME"),
