@@ -235,4 +235,36 @@ __global__ void __launch_bounds__(WG_THREADS) transpose_kernel(const TransposeAr
     }
 }
 
+// Merged groups (see merged_groups in phx_qconv.hip): m consecutive groups of a grouped convolution run as one group of
+// m * ci -> m * co channels whose filter is block-diagonal.  to_caller == false: w -> w2, the merged filter
+// [4][Co][m * ci][Kh][Kw] with zeros off the diagonal blocks; to_caller == true: the diagonal blocks of dw2 -> dw.
+struct MergeFilterArgs {
+    const void* w;  // caller's filter (or its gradient): element (r, o, i, kh, kw) at r*wcs + o*so + i*si + kh*skh + kw*skw
+    void* w2;       // merged filter (or its gradient), OIHW
+    long wcs, so, si, skh, skw;
+    int Co, ci, co, m, Kh, Kw;  // all output channels; channels of one original group; groups merged into one
+};
+
+template <typename TS>
+__global__ void __launch_bounds__(WG_THREADS) merge_filter_kernel(const MergeFilterArgs A, bool to_caller) {
+    const int taps = A.Kh * A.Kw, cim = A.m * A.ci;
+    const long total = 4L * A.Co * cim * taps;
+    for (long e = (long)blockIdx.x * WG_THREADS + threadIdx.x; e < total; e += (long)gridDim.x * WG_THREADS) {
+        const int t = (int)(e % taps);
+        long rest = e / taps;
+        const int im = (int)(rest % cim);
+        rest /= cim;
+        const int o = (int)(rest % A.Co), r = (int)(rest / A.Co);
+        const int j = im / A.ci, i = im - j * A.ci;
+        const bool diagonal = j == (o / A.co) % A.m;
+        const int kh = t / A.Kw, kw = t - kh * A.Kw;
+        const long at = r * A.wcs + o * A.so + i * A.si + kh * A.skh + kw * A.skw;
+        if (to_caller) {
+            if (diagonal) static_cast<TS*>(const_cast<void*>(A.w))[at] = static_cast<const TS*>(A.w2)[e];
+        } else {
+            static_cast<TS*>(A.w2)[e] = diagonal ? static_cast<const TS*>(A.w)[at] : (TS)0.f;
+        }
+    }
+}
+
 }  // namespace phx

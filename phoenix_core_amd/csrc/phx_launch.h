@@ -142,6 +142,7 @@ int launch_s2d_input(bool half_storage, const S2dArgs& a, hipStream_t st);
 int launch_subsample(bool half_storage, const SubsampleArgs& a, hipStream_t st);
 int launch_s2d_filter(bool half_storage, const S2dFilterArgs& a, bool to_caller, hipStream_t st);
 int launch_phase_merge(bool half_storage, const PhaseMergeArgs& a, hipStream_t st);
+int launch_merge_filter(bool half_storage, const MergeFilterArgs& a, bool to_caller, hipStream_t st);  // block-diagonal filters of merged groups
 // batched matrix transposes between channels-last tensors and the kernels' channels-first layout
 int launch_transpose(bool half_storage, const TransposeArgs& a, hipStream_t st);
 int launch_fill_zero(void* dst, size_t bytes, hipStream_t st);  // a kernel, so that it can be captured in a graph

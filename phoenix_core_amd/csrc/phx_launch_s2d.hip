@@ -43,6 +43,15 @@ int launch_s2d_filter(bool half_storage, const S2dFilterArgs& a, bool to_caller,
     return 0;
 }
 
+int launch_merge_filter(bool half_storage, const MergeFilterArgs& a, bool to_caller, hipStream_t st) {
+    const long items = 4L * a.Co * a.m * a.ci * a.Kh * a.Kw;
+    if (items == 0) return 0;
+    if (half_storage)
+        hipLaunchKernelGGL((merge_filter_kernel<_Float16>), dim3(blocks_for(items)), dim3(WG_THREADS), 0, st, a, to_caller);
+    else hipLaunchKernelGGL((merge_filter_kernel<float>), dim3(blocks_for(items)), dim3(WG_THREADS), 0, st, a, to_caller);
+    return 0;
+}
+
 int launch_fill_zero(void* dst, size_t bytes, hipStream_t st) {
     if (bytes == 0) return 0;
     hipLaunchKernelGGL(fill_zero_kernel, dim3(blocks_for((long)((bytes + 15) / 16))), dim3(WG_THREADS), 0, st,

@@ -35,7 +35,8 @@ struct Tuning {
     bool pwrall = false;              // PHX_TUNE_PWRALL: ... and every problem that kernel can run goes to it (not only those of at most 32 output channels)
     bool nowincl = false;             // PHX_TUNE_NOWINCL: channels-last windowed problems go through the transposes
     bool nogroupbatch = false;        // PHX_TUNE_NOGROUPBATCH: a grouped convolution runs group after group
-    int thin_max = 16;                // PHX_TUNE_THIN_MAX: most input x output channels per group that run on the FMA kernels for thin groups (0 = never)
+    int thin_max = 4;                 // PHX_TUNE_THIN_MAX: most input x output channels per group that run on the vector-ALU kernels for thin groups (0 = never)
+    bool nomerge = false;             // PHX_TUNE_NOMERGE: groups are never merged into block-diagonal ones
     bool direct = false;              // PHX_TUNE_DIRECT: every convolution those kernels can run goes to them (an independent path to check the matrix-core kernels against)
     bool thin_notile = false;         // PHX_TUNE_THIN_NOTILE: ... and never on the kernel that stages window tiles in LDS
     int wincl_max = 3072;             // PHX_TUNE_WINCL_MAX: largest channels x taps that runs on channels-last tensors directly
@@ -70,6 +71,7 @@ struct Tuning {
         if (const char* e = getenv("PHX_TUNE_THIN_MAX")) thin_max = atoi(e);
         thin_notile = getenv("PHX_TUNE_THIN_NOTILE") != nullptr;
         direct = getenv("PHX_TUNE_DIRECT") != nullptr;
+        nomerge = getenv("PHX_TUNE_NOMERGE") != nullptr;
         nosmalldense = getenv("PHX_TUNE_NOSMALLDENSE") != nullptr;
         if (const char* e = getenv("PHX_TUNE_VEC")) vec = atoi(e);
         if (const char* e = getenv("PHX_TUNE_WGS")) wgs = atoi(e);
@@ -213,10 +215,13 @@ struct GroupBatch {
 };
 static thread_local GroupBatch g_batch;
 // (kernel labels of launches that run every group carry the number of groups)
+static thread_local int g_name_suffix_merged = 0;  // m while groups merged m at a time run (see merged_groups)
 static void label_groups(int groups) {
-    if (groups <= 1) return;
-    const size_t len = strlen(g_name_buf);
-    if (len < sizeof(g_name_buf)) snprintf(g_name_buf + len, sizeof(g_name_buf) - len, "_groups%d", groups);
+    size_t len = strlen(g_name_buf);
+    if (groups > 1 && len < sizeof(g_name_buf)) snprintf(g_name_buf + len, sizeof(g_name_buf) - len, "_groups%d", groups);
+    len = strlen(g_name_buf);
+    if (g_name_suffix_merged && len < sizeof(g_name_buf))
+        snprintf(g_name_buf + len, sizeof(g_name_buf) - len, "_merged%d", g_name_suffix_merged);
 }
 static const void* at_bytes(const void* ptr, size_t off) { return ptr ? static_cast<const char*>(ptr) + off : nullptr; }
 static void* at_bytes(void* ptr, size_t off) { return ptr ? static_cast<char*>(ptr) + off : nullptr; }
@@ -1781,12 +1786,14 @@ static bool nhwc_wgrad_native(const Problem& p) {
     return !pl.realx && pl.kmode == 16 && pl.MT == 2 && pl.NT == 2 && pl.SW == 1 && (pl.TPW == 1 || pl.TPW == 3);
 }
 
-// Grouped convolutions whose groups hold only a few channels (depthwise convolutions first of all) run on the FMA
+// Grouped convolutions whose groups hold very few channels (depthwise convolutions first of all) run on the vector-ALU
 // kernels of phx_launch_thin.hip, all groups by one launch per pass, straight on the caller's channels-first tensors
-// and filter: a 32 x 32 matrix-core tile per group would be nearly empty (1.6 % full at 4 x 4 channels per group).
-// The matrix-core path costs a tile per group whatever it holds, the FMA threads cost in proportion to the channel
-// pairs of a group (input x output channels): measured at 3x3, 28x28, they are 15x faster at one pair, 1.7x at 16
-// (4 x 4) and 1.6x slower at 64 (8 x 8).  PHX_TUNE_THIN_MAX moves the bound.
+// and filter.  A matrix-core tile spans 32 x 32 channels of one group and costs the same whatever it holds; the
+// vector-ALU threads cost in proportion to the channel pairs of a group (input x output channels).  Measured against
+// the matrix-core path with merged groups (merged_groups below; 128 channels, 28x28, N=32, fwd / dgrad / wgrad us):
+// depthwise 3x3 29 / 28 / 54 against 49 / 50 / 54, 5x5 (96 channels, 56x56) 128 / 122 / 231 against 261 / 263 / 610,
+// 2 x 2 channels per group 45 / 42 / 73 against 48 / 47 / 53, 4 x 4 71 / 67 / 111 against 46 / 45 / 51: up to four
+// pairs per group run here.  PHX_TUNE_THIN_MAX moves the bound.
 //
 // The same kernels are the way out for filters whose window does not fit the matrix-core kernels' staging: those
 // stage one window position per thread, so the window of a single output position -- ((kh-1) dh + 1) rows of
@@ -1871,6 +1878,89 @@ static bool group_batchable(const Problem& p, int pass) {
 }
 }  // namespace phx
 
+// One pass of a grouped convolution on channels-first tensors of all groups: by one launch per kernel where the pass
+// is a plain run of the kernels (group_batchable), group after group otherwise.  (a, b) = (x, w) forward,
+// (grad, w) input gradient, (x, grad) filter gradient.
+static int groups_pass(const Problem& p, int pass, hipStream_t st, const void* a, const void* b, const void* bias, void* out, void* ws,
+                       size_t wsb) {
+    const auto one = [&](const void* a_, const void* b_, const void* bias_, void* out_) {
+        return pass == PHX_PASS_FWD ? do_fwd(p, st, a_, b_, bias_, out_, ws, wsb)
+               : pass == PHX_PASS_BWD_DATA ? do_bwd_data(p, st, a_, b_, out_, ws, wsb) : do_bwd_weights(p, st, a_, b_, out_, ws, wsb);
+    };
+    if (group_batchable(p, pass)) {
+        const GroupBatchScope batch(p);
+        return one(a, b, bias, out);
+    }
+    const GroupOffsets o(p);
+    // bytes from a group to the next in the three tensors of the pass
+    const size_t sa = pass == PHX_PASS_BWD_DATA ? o.y : o.x, sb = pass == PHX_PASS_BWD_WEIGHTS ? o.y : o.w;
+    const size_t so = pass == PHX_PASS_FWD ? o.y : pass == PHX_PASS_BWD_DATA ? o.x : o.w;
+    for (int g = 0; g < o.runs; ++g) {
+        const int rc = one(o.at(a, g * sa), o.at(b, g * sb), bias ? o.at(bias, g * o.b) : nullptr, o.at(out, g * so));
+        if (rc != PHX_OK) return rc;
+    }
+    return PHX_OK;
+}
+static size_t groups_workspace(const Problem& p, int pass) {
+    return (group_batchable(p, pass) ? (size_t)p.groups : (size_t)1) * workspace_for(p, pass);
+}
+
+// Merged groups: a matrix-core tile spans 32 x 32 channels of one group, so groups of fewer channels leave most of
+// it empty and still cost a tile each.  m consecutive groups (m the largest divisor of the group count with
+// m x channels <= 32) are run as ONE group of m * ci -> m * co channels whose filter is block-diagonal: the
+// activation tensors are the same memory, the filter is expanded with zeros per call (merge_filter_kernel: a few KB),
+// the filter gradient's diagonal blocks are copied out.  The tile then does m times the arithmetic it needs to, which
+// the matrix cores have to spare: 32 groups of 4 x 4 channels (3x3, 28x28, N=32) take the time of 4 groups of 32 x 32.
+static int merged_groups(const Problem& p) {
+    if (p.groups <= 1 || is_empty(p) || p.real_input || tune().nomerge) return 0;
+    const int widest = std::max(p.ci, p.co);
+    int m = 0;
+    for (int d = 2; d <= p.groups && d * widest <= 32; ++d)
+        if (p.groups % d == 0) m = d;
+    return m;
+}
+struct MergedGroups {
+    Problem q;            // the merged problem: groups / m groups of m * ci -> m * co channels, channels-first
+    size_t filter_bytes;  // the block-diagonal filter (or its gradient), OIHW, at the front of the workspace
+    MergeFilterArgs fa;
+    MergedGroups(const Problem& p, int m) {
+        q = p;
+        q.groups = p.groups / m; q.ci = p.ci * m; q.co = p.co * m; q.nhwc = false;
+        const long taps = (long)p.kh * p.kw;
+        q.fs.skw = 1; q.fs.skh = p.kw; q.fs.si = taps; q.fs.so = (long)q.ci * taps; q.fs.wcs = (long)p.co_mem * q.fs.so;
+        filter_bytes = align_up((size_t)4 * q.fs.wcs * (p.dtype == PHX_F32 ? 4 : 2), 256);
+        fa = MergeFilterArgs{nullptr, nullptr, p.fs.wcs, p.fs.so, p.fs.si, p.fs.skh, p.fs.skw, p.co_mem, p.ci, p.co, m, p.kh, p.kw};
+    }
+    size_t workspace(int pass) const { return filter_bytes + groups_workspace(q, pass); }
+};
+// (a, b) as in groups_pass, on channels-first tensors
+static int run_merged(const Problem& p, int m, int pass, hipStream_t st, const void* a, const void* b, const void* bias, void* out,
+                      void* ws, size_t wsb) {
+    const MergedGroups mg(p, m);
+    if (!ws || wsb < mg.filter_bytes) return PHX_ERR_WORKSPACE;
+    char* inner = static_cast<char*>(ws) + mg.filter_bytes;
+    const size_t inner_bytes = wsb - mg.filter_bytes;
+    MergeFilterArgs fa = mg.fa;
+    fa.w2 = ws;
+    g_name_suffix_merged = m;
+    int rc;
+    if (pass == PHX_PASS_BWD_WEIGHTS) {
+        rc = groups_pass(mg.q, pass, st, a, b, nullptr, ws, inner, inner_bytes);  // the merged filter gradient, then its diagonal blocks
+        if (rc == PHX_OK) {
+            fa.w = out;
+            launch_merge_filter(p.dtype == PHX_F16, fa, true, st);
+        }
+    } else {
+        fa.w = b;
+        launch_merge_filter(p.dtype == PHX_F16, fa, false, st);
+        rc = groups_pass(mg.q, pass, st, a, ws, bias, out, inner, inner_bytes);
+    }
+    g_name_suffix_merged = 0;
+    if (rc != PHX_OK) return rc;
+    PHX_HIP(hipGetLastError());
+    return PHX_OK;
+}
+
 // Entry points check their descriptor before they touch the device: an invalid descriptor is an invalid argument
 // whether or not a device is present.
 static int conv_desc_status(const phx_qconv_desc* desc) {
@@ -1905,6 +1995,7 @@ size_t phx_qconv2d_workspace_bytes(const phx_qconv_desc* desc, int pass) {
     if (nhwc_native(p, pass)) return nhwc_native_workspace(p, pass);
     if (nhwc_window_native(p, pass)) return workspace_for(p, pass);
     if (pass == PHX_PASS_BWD_WEIGHTS && nhwc_wgrad_native(p)) return workspace_for(p, pass);
+    if (const int m = merged_groups(p)) return ChannelsLast(p).bytes() + MergedGroups(p, m).workspace(pass);
     // (packed images / partial sums of all groups side by side where one launch runs them)
     if (group_batchable(p, pass)) return (size_t)p.groups * workspace_for(p, pass);
     return ChannelsLast(p).bytes() + workspace_for(p, pass);
@@ -1962,7 +2053,8 @@ static int conv_fwd_quaternion(const phx_qconv_desc* desc, phx_stream_t stream, 
         g_window_cl = false;
         return nrc;
     }
-    if (!direct && group_batchable(p, PHX_PASS_FWD)) {
+    const int merged = direct ? 0 : merged_groups(p);
+    if (!direct && !merged && group_batchable(p, PHX_PASS_FWD)) {
         const GroupBatchScope batch(p);
         return do_fwd(p, st, x, w, bias_or_null, y, dry ? nullptr : workspace, dry ? 0 : workspace_bytes);
     }
@@ -1980,6 +2072,12 @@ static int conv_fwd_quaternion(const phx_qconv_desc* desc, phx_stream_t stream, 
         if (g_pack.mode == PackSession::USE) return PHX_ERR_NOT_SUPPORTED;
         if (!dry)
             if (const int trc = run_thin(p, PHX_PASS_FWD, st, x, w, bias_or_null, y_planes, nullptr, 0)) return trc;
+    } else if (merged) {  // (the block-diagonal filter is made per call: no packed form either)
+        if (g_pack.mode == PackSession::USE) return PHX_ERR_NOT_SUPPORTED;
+        if (!dry)
+            if (const int mrc = run_merged(p, merged, PHX_PASS_FWD, st, x, w, bias_or_null, y_planes, ws ? ws + cl.bytes() : nullptr,
+                                           workspace_bytes - cl.bytes()))
+                return mrc;
     } else
     for (int g = 0; g < o.runs; ++g) {
         const int grc = do_fwd(p, st, o.at(x, g * o.x), o.at(w, g * o.w),
@@ -2032,7 +2130,8 @@ static int conv_bwd_data_quaternion(const phx_qconv_desc* desc, phx_stream_t str
         g_window_cl = false;
         return nrc;
     }
-    if (!direct && group_batchable(p, PHX_PASS_BWD_DATA)) {
+    const int merged = direct ? 0 : merged_groups(p);
+    if (!direct && !merged && group_batchable(p, PHX_PASS_BWD_DATA)) {
         const GroupBatchScope batch(p);
         return do_bwd_data(p, st, grad, w, dx, dry ? nullptr : workspace, dry ? 0 : workspace_bytes);
     }
@@ -2050,6 +2149,12 @@ static int conv_bwd_data_quaternion(const phx_qconv_desc* desc, phx_stream_t str
         if (g_pack.mode == PackSession::USE) return PHX_ERR_NOT_SUPPORTED;
         if (!dry)
             if (const int trc = run_thin(p, PHX_PASS_BWD_DATA, st, grad, w, nullptr, dx_planes, nullptr, 0)) return trc;
+    } else if (merged) {
+        if (g_pack.mode == PackSession::USE) return PHX_ERR_NOT_SUPPORTED;
+        if (!dry)
+            if (const int mrc = run_merged(p, merged, PHX_PASS_BWD_DATA, st, grad, w, nullptr, dx_planes, ws ? ws + cl.bytes() : nullptr,
+                                           workspace_bytes - cl.bytes()))
+                return mrc;
     } else
     for (int g = 0; g < o.runs; ++g) {
         const int grc = do_bwd_data(p, st, o.at(grad, g * o.y), o.at(w, g * o.w), o.at(dx_planes, g * o.x),
@@ -2176,7 +2281,8 @@ int phx_qconv2d_bwd_weights(const phx_qconv_desc* desc, phx_stream_t stream, con
         g_window_cl = false;
         return nrc;
     }
-    if (!direct && group_batchable(p, PHX_PASS_BWD_WEIGHTS)) {
+    const int merged = direct ? 0 : merged_groups(p);
+    if (!direct && !merged && group_batchable(p, PHX_PASS_BWD_WEIGHTS)) {
         const GroupBatchScope batch(p);
         return do_bwd_weights(p, st, x, grad, dw, workspace, workspace_bytes);
     }
@@ -2189,6 +2295,9 @@ int phx_qconv2d_bwd_weights(const phx_qconv_desc* desc, phx_stream_t stream, con
         x = ws;
         grad = ws + cl.x_bytes;
     }
+    if (merged)
+        return run_merged(p, merged, PHX_PASS_BWD_WEIGHTS, st, x, grad, nullptr, dw, ws ? ws + cl.bytes() : nullptr,
+                          workspace_bytes - cl.bytes());
     if (direct)
         return run_thin(p, PHX_PASS_BWD_WEIGHTS, st, x, grad, nullptr, dw, ws ? ws + cl.bytes() : nullptr, workspace_bytes - cl.bytes());
     for (int g = 0; g < o.runs; ++g) {

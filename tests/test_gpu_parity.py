@@ -450,8 +450,8 @@ def test_groups_run_in_one_launch_per_kernel(case, mode, dtype, policy, tune_env
                                 context=Ctx(mode, policy))
     got = {}
     for variant in ("one launch", "group after group"):
-        # (THIN_MAX=0: the depthwise cases stay on the matrix-core kernels this test is about)
-        tune_env(PHX_TUNE_NOGROUPBATCH=None if variant == "one launch" else "1", PHX_TUNE_THIN_MAX="0")
+        # (THIN_MAX=0, NOMERGE: small groups stay one group per matrix-core tile, which this test is about)
+        tune_env(PHX_TUNE_NOGROUPBATCH=None if variant == "one launch" else "1", PHX_TUNE_THIN_MAX="0", PHX_TUNE_NOMERGE="1")
         y = phx.conv2d_fwd(xd, wd, bd, desc)
         k_fwd = capi.last_kernel_name()
         dx = ops.conv2d_bwd_data(wd, gd, desc)
@@ -597,6 +597,71 @@ def test_vector_alu_kernels_take_real_valued_input(case, tiles, dtype, policy, t
     assert_close(got_dw.transpose(0, 1, 4, 2, 3) if cl else got_dw, want_dw, dtype, "wgrad " + k_wg)
 
 
+MERGED_GROUPS = [
+    # name, groups, channels-last, n, ci, co, h, w, kh, kw, stride, dilation, padding -> groups merged at a time
+    ("g32_4x4_k3", 32, False, 2, 128, 128, 9, 10, 3, 3, 1, 1, "SAME", 8),
+    ("g16_8x8_k3", 16, False, 2, 128, 128, 7, 9, 3, 3, 1, 1, "SAME", 4),
+    ("g6_5to3_k3", 6, False, 3, 30, 18, 10, 11, 3, 3, 1, 1, "SAME", 6),             # all groups in one block-diagonal filter
+    ("g4_16to8_k3_s2", 4, False, 2, 64, 32, 15, 13, 3, 3, 2, 1, "SAME", 2),          # the strided input gradient of the merged problem
+    ("g8_4x4_pw", 8, False, 3, 32, 32, 8, 8, 1, 1, 1, 1, "VALID", 8),                # pointwise: the streaming kernel on the merged channels
+    ("g10_3to6_k5_dil2", 10, False, 2, 30, 60, 11, 12, 5, 5, 1, 2, (2, 1, 3, 0), 5),
+    ("g12_2x4_k3_s2_c4", 12, False, 2, 24, 48, 15, 14, 3, 3, 2, 1, "SAME", 6),
+    ("g8_4x4_k3_nhwc", 8, True, 2, 32, 32, 10, 9, 3, 3, 1, 1, "SAME", 8),
+    ("g3_16x16_k3", 3, False, 2, 48, 48, 9, 9, 3, 3, 1, 1, "SAME", 0),               # three groups of 16: two do not divide them, three are too wide
+]
+
+
+@pytest.mark.parametrize("dtype,policy", [(torch.float32, "fp32"), (torch.float16, "full16"), (torch.float16, "backward32")],
+                         ids=["f32", "f16_full16", "f16_backward32"])
+@pytest.mark.parametrize("mode", [16, 8])
+@pytest.mark.parametrize("case", MERGED_GROUPS, ids=lambda c: c[0])
+def test_small_groups_run_merged_on_the_matrix_cores(case, mode, dtype, policy):
+    """Groups of fewer than 32 channels would leave most of a 32 x 32 matrix-core tile empty: m consecutive groups (the
+    largest divisor of the group count with m x channels <= 32) run as one group with a block-diagonal filter (the
+    reference hands `groups` to its scalar convolutions, src/backend/onednn/conv2d.hpp:116-137; how they are run is
+    the backend's business).  The kernel labels say `_merged<m>`; results are those of G independent convolutions on
+    channel slices through the oracle -- the off-diagonal zeros must not leak into outputs or gradients."""
+    name, G, cl, n, ci, co, h, w, kh, kw, stride, dilation, padding, m = case
+    cig, cog = ci // G, co // G
+    scale = 1.0 if dtype == torch.float32 else 0.5
+    g, x, _, b, gr = make_inputs(name_seed(name) + 70, n, ci, co, h, w, kh, kw, stride, dilation, padding, dtype, scale)
+    r = np.random.default_rng(name_seed(name) + 71)
+    npdt = np.float32 if dtype == torch.float32 else np.float16
+    wt = (scale * r.standard_normal((4, co, cig, kh, kw)) * np.sqrt(2.0 / (cig * kh * kw))).astype(npdt)
+    to_dev = (lambda a: np.ascontiguousarray(a.transpose(0, 2, 3, 1))) if cl else (lambda a: a)
+    from_dev = (lambda a: a.transpose(0, 3, 1, 2)) if cl else (lambda a: a)
+    x_dev, g_dev = to_dev(x), to_dev(gr)
+    w_dev = np.ascontiguousarray(wt.transpose(0, 1, 3, 4, 2)) if cl else wt
+    desc = phx.Conv2DDescriptor(x_dev.shape, w_dev.shape, stride, dilation, padding, groups=G, use_bias=True, dtype=dtype,
+                                filter_layout="OHWI" if cl else "OIHW", context=Ctx(mode, policy),
+                                data_format="NHWC" if cl else "NCHW")
+    xd, wd, bd, gd = (torch.from_numpy(a).cuda() for a in (x_dev, w_dev, b, g_dev))
+    dw_before = torch.full(wd.shape, 7.0, dtype=dtype, device="cuda")  # (the filter gradient's blocks are copied into the caller's tensor: all of it must be written)
+    y = phx.conv2d_fwd(xd, wd, bd, desc)
+    names = [capi.last_kernel_name()]
+    dx = ops.conv2d_bwd_data(wd, gd, desc)
+    names.append(capi.last_kernel_name())
+    dw = ops.conv2d_bwd_weights(xd, gd, desc)
+    names.append(capi.last_kernel_name())
+    tag = "_merged%d" % m
+    assert all((tag in k) if m else ("_merged" not in k) for k in names), names
+    if m:
+        assert ops.conv2d_pack_filters(wd, desc) is None  # (the block-diagonal filter is made per call)
+    gg = oracle.make_geom(n, cig, cog, h, w, kh, kw, stride, dilation, padding)
+    x64, w64, b64, g64 = (a.astype(np.float64) for a in (x, wt, b, gr))
+    want_y, want_dx, want_dw = np.empty(gr.shape), np.empty(x.shape), np.empty(wt.shape)
+    for k in range(G):
+        ic, oc = slice(k * cig, (k + 1) * cig), slice(k * cog, (k + 1) * cog)
+        xs, ws, bs, gs = (np.ascontiguousarray(a) for a in (x64[:, ic], w64[:, oc], b64[:, oc], g64[:, oc]))
+        want_y[:, oc] = oracle.conv2d_fwd(gg, xs, ws, bs, "hamilton")
+        want_dw[:, oc], want_dx[:, ic] = oracle.conv2d_bwd(gg, xs, ws, gs, "hamilton")
+    assert_close(from_dev(y.cpu().numpy()), want_y, dtype, "merged groups fwd " + name)
+    assert_close(from_dev(dx.cpu().numpy()), want_dx, dtype, "merged groups dgrad " + name)
+    got_dw = dw.cpu().numpy()
+    assert_close(got_dw.transpose(0, 1, 4, 2, 3) if cl else got_dw, want_dw, dtype, "merged groups wgrad " + name)
+    del dw_before
+
+
 THIN_GROUPS = [
     # name, groups, channels-last, n, ci, co, h, w, kh, kw, stride, dilation, padding
     ("dw_k3", 8, False, 2, 8, 8, 10, 10, 3, 3, 1, 1, "SAME"),
@@ -631,7 +696,7 @@ THIN_GROUPS = [
 @pytest.mark.parametrize("mode,tiles", [(16, True), (8, True), (16, False)], ids=["p16", "p8", "p16_notile"])
 @pytest.mark.parametrize("case", THIN_GROUPS, ids=lambda c: c[0])
 def test_thin_groups_run_on_fma_threads(case, mode, tiles, dtype, policy, tune_env):
-    """Grouped convolutions with at most sixteen channel pairs (input x output channels) per group (depthwise convolutions first of all; the
+    """Grouped convolutions with few channel pairs (input x output channels) per group (depthwise convolutions first of all; the
     reference hands `groups` to its scalar convolutions, src/backend/onednn/conv2d.hpp:116-137, and has no vector for
     them) run on the FMA kernels for thin groups, every pass by one launch on the caller's filter: the kernel label says
     so, the filter gradient asks for its partial sums only, and the results are those of G independent convolutions on
@@ -640,7 +705,8 @@ def test_thin_groups_run_on_fma_threads(case, mode, tiles, dtype, policy, tune_e
     wherever an output row fits a workgroup (the input gradient: at unit stride); PHX_TUNE_THIN_NOTILE keeps every
     case on the kernels that read global memory per tap."""
     name, G, cl, n, ci, co, h, w, kh, kw, stride, dilation, padding = case
-    tune_env(PHX_TUNE_THIN_NOTILE=None if tiles else "1")
+    # (up to sixteen channel pairs per group here; by default groups of more than four pairs run merged on the matrix cores)
+    tune_env(PHX_TUNE_THIN_NOTILE=None if tiles else "1", PHX_TUNE_THIN_MAX="16")
     cig, cog = ci // G, co // G
     scale = 1.0 if dtype == torch.float32 else 0.5
     g, x, _, b, gr = make_inputs(name_seed(name) + 40, n, ci, co, h, w, kh, kw, stride, dilation, padding, dtype, scale)
@@ -1180,7 +1246,8 @@ def test_prepacked_filters_grouped_and_channels_last(case, mode, tune_env):
     """Groups (one packing job per group and pass -- more jobs than one launch holds for the depthwise case) and
     channels-last activations, fp16."""
     name, G, n, ci, co, h, w, kh, kw, stride, dilation, padding = case
-    tune_env(PHX_TUNE_THIN_MAX="0")  # (groups of few channels on the matrix-core kernels: the FMA kernels pack nothing)
+    # (groups of few channels stay a group per matrix-core tile: the vector-ALU kernels and merged groups pack nothing ahead)
+    tune_env(PHX_TUNE_THIN_MAX="0", PHX_TUNE_NOMERGE="1")
     nhwc = name.startswith("nhwc")
     dtype = torch.float16
     r = np.random.default_rng(name_seed(name) + 22)
