@@ -1908,7 +1908,7 @@ static size_t groups_workspace(const Problem& p, int pass) {
 // Merged groups: a matrix-core tile spans 32 x 32 channels of one group, so groups of fewer channels leave most of
 // it empty and still cost a tile each.  m consecutive groups (m the largest divisor of the group count with
 // m x channels <= 32) are run as ONE group of m * ci -> m * co channels whose filter is block-diagonal: the
-// activation tensors are the same memory, the filter is expanded with zeros per call (merge_filter_kernel: a few KB),
+// activation tensors are the same memory, the filter is expanded with zeros (merge_filter_kernel: a few KB; per call, or once with the packed images),
 // the filter gradient's diagonal blocks are copied out.  The tile then does m times the arithmetic it needs to, which
 // the matrix cores have to spare: 32 groups of 4 x 4 channels (3x3, 28x28, N=32) take the time of 4 groups of 32 x 32.
 static int merged_groups(const Problem& p) {
@@ -1933,31 +1933,44 @@ struct MergedGroups {
     }
     size_t workspace(int pass) const { return filter_bytes + groups_workspace(q, pass); }
 };
-// (a, b) as in groups_pass, on channels-first tensors
+// (a, b) as in groups_pass, on channels-first tensors.  In a packing session (PackSession) the block-diagonal filter is
+// an image like the packed ones: SIZE counts it, RECORD makes it (on the session's stream, ahead of the combined
+// packing launch that reads it), USE finds it where RECORD put it.
 static int run_merged(const Problem& p, int m, int pass, hipStream_t st, const void* a, const void* b, const void* bias, void* out,
                       void* ws, size_t wsb) {
     const MergedGroups mg(p, m);
-    if (!ws || wsb < mg.filter_bytes) return PHX_ERR_WORKSPACE;
-    char* inner = static_cast<char*>(ws) + mg.filter_bytes;
-    const size_t inner_bytes = wsb - mg.filter_bytes;
+    const PackSession::Mode session = g_pack.mode;
+    void* merged_filter = ws;
+    char* inner = static_cast<char*>(ws);
+    size_t inner_bytes = wsb;
+    if (session == PackSession::OFF || pass == PHX_PASS_BWD_WEIGHTS) {
+        if (!ws || wsb < mg.filter_bytes) return PHX_ERR_WORKSPACE;
+        inner += mg.filter_bytes;
+        inner_bytes -= mg.filter_bytes;
+    } else {
+        const PackSlot slot = pack_slot(nullptr, 0, mg.filter_bytes);
+        if (slot.rc != PHX_OK) return slot.rc;
+        merged_filter = slot.dst;  // (null while SIZE only counts)
+    }
     MergeFilterArgs fa = mg.fa;
-    fa.w2 = ws;
+    fa.w2 = merged_filter;
     g_name_suffix_merged = m;
     int rc;
     if (pass == PHX_PASS_BWD_WEIGHTS) {
-        rc = groups_pass(mg.q, pass, st, a, b, nullptr, ws, inner, inner_bytes);  // the merged filter gradient, then its diagonal blocks
+        rc = groups_pass(mg.q, pass, st, a, b, nullptr, merged_filter, inner, inner_bytes);  // the merged filter gradient, then its diagonal blocks
         if (rc == PHX_OK) {
             fa.w = out;
             launch_merge_filter(p.dtype == PHX_F16, fa, true, st);
         }
     } else {
         fa.w = b;
-        launch_merge_filter(p.dtype == PHX_F16, fa, false, st);
-        rc = groups_pass(mg.q, pass, st, a, ws, bias, out, inner, inner_bytes);
+        if (session == PackSession::OFF) launch_merge_filter(p.dtype == PHX_F16, fa, false, st);
+        else if (session == PackSession::RECORD) launch_merge_filter(p.dtype == PHX_F16, fa, false, g_pack.st);
+        rc = groups_pass(mg.q, pass, st, a, merged_filter, bias, out, inner, inner_bytes);
     }
     g_name_suffix_merged = 0;
     if (rc != PHX_OK) return rc;
-    PHX_HIP(hipGetLastError());
+    if (session != PackSession::SIZE) PHX_HIP(hipGetLastError());
     return PHX_OK;
 }
 
@@ -2072,12 +2085,10 @@ static int conv_fwd_quaternion(const phx_qconv_desc* desc, phx_stream_t stream, 
         if (g_pack.mode == PackSession::USE) return PHX_ERR_NOT_SUPPORTED;
         if (!dry)
             if (const int trc = run_thin(p, PHX_PASS_FWD, st, x, w, bias_or_null, y_planes, nullptr, 0)) return trc;
-    } else if (merged) {  // (the block-diagonal filter is made per call: no packed form either)
-        if (g_pack.mode == PackSession::USE) return PHX_ERR_NOT_SUPPORTED;
-        if (!dry)
-            if (const int mrc = run_merged(p, merged, PHX_PASS_FWD, st, x, w, bias_or_null, y_planes, ws ? ws + cl.bytes() : nullptr,
-                                           workspace_bytes - cl.bytes()))
-                return mrc;
+    } else if (merged) {
+        if (const int mrc = run_merged(p, merged, PHX_PASS_FWD, st, x, w, bias_or_null, y_planes, ws ? ws + cl.bytes() : nullptr,
+                                       workspace_bytes - cl.bytes()))
+            return mrc;
     } else
     for (int g = 0; g < o.runs; ++g) {
         const int grc = do_fwd(p, st, o.at(x, g * o.x), o.at(w, g * o.w),
@@ -2150,11 +2161,9 @@ static int conv_bwd_data_quaternion(const phx_qconv_desc* desc, phx_stream_t str
         if (!dry)
             if (const int trc = run_thin(p, PHX_PASS_BWD_DATA, st, grad, w, nullptr, dx_planes, nullptr, 0)) return trc;
     } else if (merged) {
-        if (g_pack.mode == PackSession::USE) return PHX_ERR_NOT_SUPPORTED;
-        if (!dry)
-            if (const int mrc = run_merged(p, merged, PHX_PASS_BWD_DATA, st, grad, w, nullptr, dx_planes, ws ? ws + cl.bytes() : nullptr,
-                                           workspace_bytes - cl.bytes()))
-                return mrc;
+        if (const int mrc = run_merged(p, merged, PHX_PASS_BWD_DATA, st, grad, w, nullptr, dx_planes, ws ? ws + cl.bytes() : nullptr,
+                                       workspace_bytes - cl.bytes()))
+            return mrc;
     } else
     for (int g = 0; g < o.runs; ++g) {
         const int grc = do_bwd_data(p, st, o.at(grad, g * o.y), o.at(w, g * o.w), o.at(dx_planes, g * o.x),

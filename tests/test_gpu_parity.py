@@ -636,7 +636,6 @@ def test_small_groups_run_merged_on_the_matrix_cores(case, mode, dtype, policy):
                                 filter_layout="OHWI" if cl else "OIHW", context=Ctx(mode, policy),
                                 data_format="NHWC" if cl else "NCHW")
     xd, wd, bd, gd = (torch.from_numpy(a).cuda() for a in (x_dev, w_dev, b, g_dev))
-    dw_before = torch.full(wd.shape, 7.0, dtype=dtype, device="cuda")  # (the filter gradient's blocks are copied into the caller's tensor: all of it must be written)
     y = phx.conv2d_fwd(xd, wd, bd, desc)
     names = [capi.last_kernel_name()]
     dx = ops.conv2d_bwd_data(wd, gd, desc)
@@ -645,8 +644,15 @@ def test_small_groups_run_merged_on_the_matrix_cores(case, mode, dtype, policy):
     names.append(capi.last_kernel_name())
     tag = "_merged%d" % m
     assert all((tag in k) if m else ("_merged" not in k) for k in names), names
-    if m:
-        assert ops.conv2d_pack_filters(wd, desc) is None  # (the block-diagonal filter is made per call)
+    # packed ahead of the passes, the block-diagonal filter is one more image: same kernels, same results
+    packed = ops.conv2d_pack_filters(wd, desc)
+    assert packed is not None and packed.fwd is not None and packed.bwd_data is not None
+    zero = torch.zeros_like(wd)
+    assert torch.equal(phx.conv2d_fwd(xd, zero, bd, desc, packed=packed), y), "prepacked fwd " + name
+    assert tag in capi.last_kernel_name() or not m
+    assert torch.equal(ops.conv2d_bwd_data(zero, gd, desc, packed=packed), dx), "prepacked dgrad " + name
+    addend = xd.flip(0) * 0.75
+    assert torch.equal(ops.conv2d_bwd_data(zero, gd, desc, packed=packed, addend=addend), dx + addend), "prepacked dgrad + addend " + name
     gg = oracle.make_geom(n, cig, cog, h, w, kh, kw, stride, dilation, padding)
     x64, w64, b64, g64 = (a.astype(np.float64) for a in (x, wt, b, gr))
     want_y, want_dx, want_dw = np.empty(gr.shape), np.empty(x.shape), np.empty(wt.shape)
@@ -659,7 +665,6 @@ def test_small_groups_run_merged_on_the_matrix_cores(case, mode, dtype, policy):
     assert_close(from_dev(dx.cpu().numpy()), want_dx, dtype, "merged groups dgrad " + name)
     got_dw = dw.cpu().numpy()
     assert_close(got_dw.transpose(0, 1, 4, 2, 3) if cl else got_dw, want_dw, dtype, "merged groups wgrad " + name)
-    del dw_before
 
 
 THIN_GROUPS = [
