@@ -120,7 +120,6 @@ template <int MODE, int WCO, int NTW, int P2LOG, bool PAIRS>
 __global__ void __launch_bounds__(WG_THREADS, (MODE == 8 || NTW == 1) ? 2 : 1) qconv_fwd_f16_kernel(const ConvArgs P0) {
     const ConvArgs P = group_view(P0);
     constexpr int CK = F16_CK;
-    constexpr int WPX = 4 / WCO;
     constexpr int NACC = (MODE == 16) ? 4 : 8;
     constexpr int WC = (MODE == 16) ? 4 : 8;  // packed 16-byte filter vectors per lane and K step
     extern __shared__ f16x8 lds16[];
@@ -1032,7 +1031,6 @@ __global__ void __launch_bounds__(WG_THREADS) qconv_wgrad_f16_kernel(const Wgrad
     const int zi = bid / ngroups;
     const int kh = grp / P.groups_per_row;
     const int kw0 = (grp % P.groups_per_row) * TPW;
-    constexpr int nkw = TPW;  // tap groups are always full
 
     // staging role: chunk j of the tile, planes pg + 32*i of every component
     const int j = tid & 7, pg = tid >> 3;

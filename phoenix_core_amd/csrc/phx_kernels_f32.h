@@ -81,7 +81,6 @@ __device__ __forceinline__ void quad_transpose(const float (&a)[4], float (&o)[4
 
 template <typename TS, int V>
 __device__ __forceinline__ void store_pixels(TS* ptr, const float (&v)[V]) {
-    typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
     if constexpr (sizeof(TS) == 4) {
         typedef float fv __attribute__((ext_vector_type(V), aligned(4)));
         fv w;
@@ -374,7 +373,6 @@ __device__ __forceinline__ void stage_vec_store_scalar(float* lds, const f32x4 (
 template <typename TS, int MODE, int WCO, int NTW, int CK, int P2LOG, bool VSTG>
 __global__ void __launch_bounds__(WG_THREADS, (MODE == 8 || NTW == 1) ? 2 : 1) qconv_fwd_f32_kernel(const ConvArgs P0) {
     const ConvArgs P = group_view(P0);
-    constexpr int WPX = 4 / WCO;
     constexpr int NACC = (MODE == 16) ? 4 : 8;
     constexpr int WC = (MODE == 16) ? 4 : 8;  // packed filter values per lane and K step
     extern __shared__ float lds[];

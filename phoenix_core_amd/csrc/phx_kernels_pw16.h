@@ -122,7 +122,7 @@ template <int WCO, bool ADD = false>
 __global__ void __launch_bounds__(WG_THREADS, 2) qconv_pwx_f16_kernel(const PwxArgs P0) {
     const PwxArgs P = group_view(P0);
     using S = PwxShape<WCO>;
-    constexpr int WPX = S::WPX, GPT = S::GPT, ROWDW = S::ROWDW, WV = S::WV, XV = S::XV, RF = S::RF, RA = S::RA;
+    constexpr int GPT = S::GPT, ROWDW = S::ROWDW, WV = S::WV, XV = S::XV, RF = S::RF, RA = S::RA;
     constexpr int DF = RF - 1, DA = RA - 1;  // steps the filter / activation copies run ahead of the products
     constexpr int RPI = 64 / GPT;      // activation rows one copy instruction covers
     constexpr int PITCH = ROWDW * 4;   // bytes of a staged activation row
