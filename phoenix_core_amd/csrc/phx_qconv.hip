@@ -433,6 +433,9 @@ static void say(const Problem& p, const char* pass) {
 }
 
 static bool is_empty(const Problem& p) { return p.n == 0 || p.h == 0 || p.w == 0; }
+// the problem works on a slice of its tensors' channels (one of several groups, or what is left of them): the paths
+// that rearrange whole tensors do not apply
+static bool channel_slices(const Problem& p) { return p.groups > 1 || p.ci_mem != p.ci || p.co_mem != p.co; }
 
 static bool is_pointwise_unit(const Problem& p) {
     return p.kh == 1 && p.kw == 1 && p.sh == 1 && p.sw == 1 && !p.pt && !p.pl && !p.pb && !p.pr;
@@ -1167,7 +1170,7 @@ static int wgrad_f16_formulation(const Problem& p) {
 // filter gradient, see phx_kernels_realx.h.  q-ResNet-50 stem (7x7 stride 2 on 3 channels as 4x4 on 12 by
 // space-to-depth, 16 output channels, N=64): 0.47 ms on the general kernel.
 static bool plan_wgrad_realx(const Problem& p, WgPlan& best) {
-    if (!p.real_input || p.dtype != PHX_F16 || p.groups > 1 || p.nhwc || tune().norealx) return false;
+    if (!p.real_input || p.dtype != PHX_F16 || channel_slices(p) || p.nhwc || tune().norealx) return false;
     if (p.sh != 1 || p.sw != 1 || p.dh != 1 || p.dw != 1 || p.kw > 4 || p.co > 16 || p.ci * p.kh * 4 > 192) return false;
     if (p.wo % 8 != 0 || p.w < 8 || p.pt < 0 || p.pl < 0 || p.pl > 7 || p.pr > 7) return false;
     const int cpr = p.wo / 8;
@@ -1382,7 +1385,7 @@ static PhaseAxis phase_axis(int a, int extent, int k, int d, int s, int pad_befo
 // (3x3 stride 2, 32-128 channels: 0.08-0.11 ms against 0.13-0.19 ms); PHX_TUNE_PHASE=1 sends every strided
 // input gradient through the phases, PHX_TUNE_PHASE=0 none.
 static bool dgrad_by_phases(const Problem& p) {
-    if ((p.sh == 1 && p.sw == 1) || p.sh * p.sw > 16 || is_empty(p) || p.groups > 1) return false;
+    if ((p.sh == 1 && p.sw == 1) || p.sh * p.sw > 16 || is_empty(p) || channel_slices(p)) return false;
     if (tune().phase >= 0) return tune().phase != 0;
     return p.kh == 1 && p.kw == 1;
 }
@@ -1438,7 +1441,7 @@ static int floordiv(int a, int b) { return a >= 0 ? a / b : -((-a + b - 1) / b);
 
 static bool s2d_view(const Problem& p, S2dView& v) {
     if (p.sh != 2 || p.sw != 2 || p.dh != 1 || p.dw != 1 || p.ci > 4 || (p.kh < 3 && p.kw < 3) || is_empty(p)) return false;
-    if (p.groups > 1) return false;  // the rearranged copies are laid out for whole tensors
+    if (channel_slices(p)) return false;  // the rearranged copies are laid out for whole tensors
     if (tune().nos2d) return false;
     const int aminh = floordiv(-p.pt, 2), amaxh = floordiv(p.kh - 1 - p.pt, 2);
     const int aminw = floordiv(-p.pl, 2), amaxw = floordiv(p.kw - 1 - p.pl, 2);
@@ -1472,7 +1475,7 @@ static bool s2d_view(const Problem& p, S2dView& v) {
 // q-ResNet-50's three downsampling shortcuts, N=64: forward 0.07 ms on the general kernel.
 static bool subsample_view(const Problem& p, Problem& q, size_t& xs_bytes) {
     if (p.kh != 1 || p.kw != 1 || (p.sh == 1 && p.sw == 1) || p.pt || p.pl || p.pb || p.pr || is_empty(p)) return false;
-    if (p.groups > 1 || p.nhwc || p.real_input || tune().nosub) return false;
+    if (channel_slices(p) || p.nhwc || p.real_input || tune().nosub) return false;
     q = p;
     q.h = p.ho; q.w = p.wo; q.sh = q.sw = 1;
     if (out_size(q.h, 1, 1, 1, 0, 0) != p.ho || out_size(q.w, 1, 1, 1, 0, 0) != p.wo) return false;
@@ -1911,13 +1914,16 @@ static size_t groups_workspace(const Problem& p, int pass) {
 // activation tensors are the same memory, the filter is expanded with zeros (merge_filter_kernel: a few KB; per call, or once with the packed images),
 // the filter gradient's diagonal blocks are copied out.  The tile then does m times the arithmetic it needs to, which
 // the matrix cores have to spare: 32 groups of 4 x 4 channels (3x3, 28x28, N=32) take the time of 4 groups of 32 x 32.
+// Returns m (0: no merging).  Where the group count has no divisor that fills the tile as well, the first
+// groups - groups % m groups are merged m at a time and the remaining groups % m as one more (run_merged).
 static int merged_groups(const Problem& p) {
     if (p.groups <= 1 || is_empty(p) || p.real_input || tune().nomerge) return 0;
-    const int widest = std::max(p.ci, p.co);
-    int m = 0;
-    for (int d = 2; d <= p.groups && d * widest <= 32; ++d)
-        if (p.groups % d == 0) m = d;
-    return m;
+    const int most = std::min(p.groups, 32 / std::max(p.ci, p.co));  // groups that fit a tile
+    if (most < 2) return 0;
+    int divisor = 1;
+    for (int d = 2; d <= most; ++d)
+        if (p.groups % d == 0) divisor = d;
+    return (divisor > 1 && p.groups / divisor == cdiv(p.groups, most)) ? divisor : most;
 }
 struct MergedGroups {
     Problem q;            // the merged problem: groups / m groups of m * ci -> m * co channels, channels-first
@@ -1927,17 +1933,17 @@ struct MergedGroups {
         q = p;
         q.groups = p.groups / m; q.ci = p.ci * m; q.co = p.co * m; q.nhwc = false;
         const long taps = (long)p.kh * p.kw;
-        q.fs.skw = 1; q.fs.skh = p.kw; q.fs.si = taps; q.fs.so = (long)q.ci * taps; q.fs.wcs = (long)p.co_mem * q.fs.so;
+        q.fs.skw = 1; q.fs.skh = p.kw; q.fs.si = taps; q.fs.so = (long)q.ci * taps; q.fs.wcs = (long)p.groups * p.co * q.fs.so;
         filter_bytes = align_up((size_t)4 * q.fs.wcs * (p.dtype == PHX_F32 ? 4 : 2), 256);
-        fa = MergeFilterArgs{nullptr, nullptr, p.fs.wcs, p.fs.so, p.fs.si, p.fs.skh, p.fs.skw, p.co_mem, p.ci, p.co, m, p.kh, p.kw};
+        fa = MergeFilterArgs{nullptr, nullptr, p.fs.wcs, p.fs.so, p.fs.si, p.fs.skh, p.fs.skw, p.groups * p.co, p.ci, p.co, m, p.kh, p.kw};
     }
     size_t workspace(int pass) const { return filter_bytes + groups_workspace(q, pass); }
 };
 // (a, b) as in groups_pass, on channels-first tensors.  In a packing session (PackSession) the block-diagonal filter is
 // an image like the packed ones: SIZE counts it, RECORD makes it (on the session's stream, ahead of the combined
 // packing launch that reads it), USE finds it where RECORD put it.
-static int run_merged(const Problem& p, int m, int pass, hipStream_t st, const void* a, const void* b, const void* bias, void* out,
-                      void* ws, size_t wsb) {
+static int run_merged_part(const Problem& p, int m, int pass, hipStream_t st, const void* a, const void* b, const void* bias, void* out,
+                           void* ws, size_t wsb) {
     const MergedGroups mg(p, m);
     const PackSession::Mode session = g_pack.mode;
     void* merged_filter = ws;
@@ -1974,6 +1980,39 @@ static int run_merged(const Problem& p, int m, int pass, hipStream_t st, const v
     return PHX_OK;
 }
 
+// The parts of a merged run: `first` groups merged m at a time, then the `rest` (fewer than m) as one group more.
+struct MergedParts {
+    Problem head, tail;
+    int first, rest;
+    MergedParts(const Problem& p, int m) : head(p), tail(p), first(p.groups - p.groups % m), rest(p.groups % m) {
+        head.groups = first;
+        tail.groups = rest;
+    }
+};
+static size_t merged_workspace(const Problem& p, int m, int pass) {
+    const MergedParts parts(p, m);
+    size_t bytes = MergedGroups(parts.head, m).workspace(pass);
+    if (parts.rest > 1) bytes = std::max(bytes, MergedGroups(parts.tail, parts.rest).workspace(pass));
+    if (parts.rest == 1) bytes = std::max(bytes, groups_workspace(parts.tail, pass));
+    return bytes;
+}
+static int run_merged(const Problem& p, int m, int pass, hipStream_t st, const void* a, const void* b, const void* bias, void* out,
+                      void* ws, size_t wsb) {
+    const MergedParts parts(p, m);
+    if (const int rc = run_merged_part(parts.head, m, pass, st, a, b, bias, out, ws, wsb)) return rc;
+    if (parts.rest == 0) return PHX_OK;
+    // the remaining groups' slices of the three tensors (and of the bias)
+    const GroupOffsets o(p);
+    const size_t sa = pass == PHX_PASS_BWD_DATA ? o.y : o.x, sb = pass == PHX_PASS_BWD_WEIGHTS ? o.y : o.w;
+    const size_t so = pass == PHX_PASS_FWD ? o.y : pass == PHX_PASS_BWD_DATA ? o.x : o.w;
+    const void* a2 = o.at(a, parts.first * sa);
+    const void* b2 = o.at(b, parts.first * sb);
+    const void* bias2 = bias ? o.at(bias, parts.first * o.b) : nullptr;
+    void* out2 = o.at(out, parts.first * so);
+    if (parts.rest == 1) return groups_pass(parts.tail, pass, st, a2, b2, bias2, out2, ws, wsb);
+    return run_merged_part(parts.tail, parts.rest, pass, st, a2, b2, bias2, out2, ws, wsb);
+}
+
 // Entry points check their descriptor before they touch the device: an invalid descriptor is an invalid argument
 // whether or not a device is present.
 static int conv_desc_status(const phx_qconv_desc* desc) {
@@ -2008,7 +2047,7 @@ size_t phx_qconv2d_workspace_bytes(const phx_qconv_desc* desc, int pass) {
     if (nhwc_native(p, pass)) return nhwc_native_workspace(p, pass);
     if (nhwc_window_native(p, pass)) return workspace_for(p, pass);
     if (pass == PHX_PASS_BWD_WEIGHTS && nhwc_wgrad_native(p)) return workspace_for(p, pass);
-    if (const int m = merged_groups(p)) return ChannelsLast(p).bytes() + MergedGroups(p, m).workspace(pass);
+    if (const int m = merged_groups(p)) return ChannelsLast(p).bytes() + merged_workspace(p, m, pass);
     // (packed images / partial sums of all groups side by side where one launch runs them)
     if (group_batchable(p, pass)) return (size_t)p.groups * workspace_for(p, pass);
     return ChannelsLast(p).bytes() + workspace_for(p, pass);
