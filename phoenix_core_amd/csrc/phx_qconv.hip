@@ -35,6 +35,8 @@ struct Tuning {
     bool pwrall = false;              // PHX_TUNE_PWRALL: ... and every problem that kernel can run goes to it (not only those of at most 32 output channels)
     bool nowincl = false;             // PHX_TUNE_NOWINCL: channels-last windowed problems go through the transposes
     bool nogroupbatch = false;        // PHX_TUNE_NOGROUPBATCH: a grouped convolution runs group after group
+    double wg_kpw = 0.01;             // PHX_TUNE_WGKPW: how much the fp32 filter-gradient planner favours larger pixel tiles (see plan_wgrad_f32)
+    int thin_max32 = 64;              // PHX_TUNE_THIN_MAX32: the same bound for passes in fp32 arithmetic (x4 for the filter gradient); PHX_TUNE_THIN_MAX=0 zeroes it too
     int thin_max = 4;                 // PHX_TUNE_THIN_MAX: most input x output channels per group that run on the vector-ALU kernels for thin groups (0 = never)
     bool nomerge = false;             // PHX_TUNE_NOMERGE: groups are never merged into block-diagonal ones
     bool direct = false;              // PHX_TUNE_DIRECT: every convolution those kernels can run goes to them (an independent path to check the matrix-core kernels against)
@@ -68,7 +70,9 @@ struct Tuning {
         nowincl = getenv("PHX_TUNE_NOWINCL") != nullptr;
         nogroupbatch = getenv("PHX_TUNE_NOGROUPBATCH") != nullptr;
         if (const char* e = getenv("PHX_TUNE_WINCL_MAX")) wincl_max = atoi(e);
-        if (const char* e = getenv("PHX_TUNE_THIN_MAX")) thin_max = atoi(e);
+        if (const char* e = getenv("PHX_TUNE_THIN_MAX")) { thin_max = atoi(e); if (thin_max == 0) thin_max32 = 0; }
+        if (const char* e = getenv("PHX_TUNE_THIN_MAX32")) thin_max32 = atoi(e);
+        if (const char* e = getenv("PHX_TUNE_WGKPW")) wg_kpw = atof(e);
         thin_notile = getenv("PHX_TUNE_THIN_NOTILE") != nullptr;
         direct = getenv("PHX_TUNE_DIRECT") != nullptr;
         nomerge = getenv("PHX_TUNE_NOMERGE") != nullptr;
@@ -1132,8 +1136,11 @@ static bool plan_wgrad_f32(const Problem& p, WgPlan& best) {
                     if (KPp + HPp + (KP + 255) / 256 > budget) break;
                     const int tn = cdiv(p.n, NB), th = cdiv(p.ho, TH), tw = cdiv(p.wo, TW);
                     const double eff = ((double)p.n * p.ho * p.wo) / ((double)tn * th * tw * KP);
+                    // (a tile is a barrier pair and a staging round whatever its size: on 7x7 images four rows of 8 at 77 %
+                    // fill beat one row of 8 at 88 % -- 512 channels, N=64: 2.46 against 4.32 ms, 128 channels 0.14 against
+                    // 0.23 ms -- which the weight on the tile's positions expresses; larger images are not affected)
                     const double score =
-                        eff * (1.0 + 0.002 * KP) * (TW >= std::min(p.wo, 8) ? 1.0 : 0.5) * (vec ? 1.25 : 1.0);
+                        eff * (1.0 + tune().wg_kpw * KP) * (TW >= std::min(p.wo, 8) ? 1.0 : 0.5) * (vec ? 1.25 : 1.0);
                     if (score > best_score) {
                         best_score = score;
                         best.vec = vec != 0;
@@ -1805,11 +1812,18 @@ static bool nhwc_wgrad_native(const Problem& p) {
 static bool window_beyond_staging(const Problem& p) {
     return ((long)(p.kh - 1) * p.dh + 1) * ((((long)(p.kw - 1) * p.dw + 1) + 7) & ~7L) > WG_THREADS;
 }
-static bool thin_groups(const Problem& p) {
+static bool thin_groups(const Problem& p, int pass) {
     if (is_empty(p) || p.ho <= 0 || p.wo <= 0) return false;
     if ((long)p.kh * p.kw > 2048 || std::max(p.ci_mem, p.co_mem) > 65535) return false;  // (a filter chunk in LDS; grid rows)
     if (tune().direct || window_beyond_staging(p)) return true;
-    return p.groups > 1 && (long)p.ci * p.co <= tune().thin_max;
+    if (p.groups <= 1) return false;
+    // Passes in fp32 arithmetic (fp32 tensors, fp16 tensors where the policy says so) have a sixteenth of the fp16
+    // matrix-core rate to lose against, and their filter gradient works on 64 x 64 channel tiles: measured like above,
+    // 8 x 8 channels per group 159 / 149 / 206 us here against 194 / 193 / 742 merged, 16 x 16 260 / 254 / 346 against
+    // 192 / 193 / 745 -- up to 64 pairs per group run here, the filter gradient up to 256.
+    const long pairs = (long)p.ci * p.co;
+    if (use_f16_mfma(p, pass)) return pairs <= tune().thin_max;
+    return pairs <= (long)tune().thin_max32 * (pass == PHX_PASS_BWD_WEIGHTS ? 4 : 1);
 }
 
 static ThinArgs thin_args(const Problem& p) {
@@ -1916,9 +1930,11 @@ static size_t groups_workspace(const Problem& p, int pass) {
 // the matrix cores have to spare: 32 groups of 4 x 4 channels (3x3, 28x28, N=32) take the time of 4 groups of 32 x 32.
 // Returns m (0: no merging).  Where the group count has no divisor that fills the tile as well, the first
 // groups - groups % m groups are merged m at a time and the remaining groups % m as one more (run_merged).
-static int merged_groups(const Problem& p) {
+static int merged_groups(const Problem& p, int pass) {
     if (p.groups <= 1 || is_empty(p) || p.real_input || tune().nomerge) return 0;
-    const int most = std::min(p.groups, 32 / std::max(p.ci, p.co));  // groups that fit a tile
+    // (the filter gradient in fp32 arithmetic works on 64 x 64 channel tiles)
+    const int tile = (pass == PHX_PASS_BWD_WEIGHTS && !wgrad_on_f16_mfma(flatten_pointwise(p))) ? 64 : 32;
+    const int most = std::min(p.groups, tile / std::max(p.ci, p.co));  // groups that fit a tile
     if (most < 2) return 0;
     int divisor = 1;
     for (int d = 2; d <= most; ++d)
@@ -2043,11 +2059,11 @@ size_t phx_qconv2d_workspace_bytes(const phx_qconv_desc* desc, int pass) {
     if (desc && desc->algebra != PHX_QUATERNION) return algebra_conv_workspace_bytes(desc, pass);
     Problem p;
     if (problem_from_conv(desc, p) != PHX_OK) return 0;
-    if (thin_groups(p)) return ChannelsLast(p).bytes() + thin_workspace(p, pass);
+    if (thin_groups(p, pass)) return ChannelsLast(p).bytes() + thin_workspace(p, pass);
     if (nhwc_native(p, pass)) return nhwc_native_workspace(p, pass);
     if (nhwc_window_native(p, pass)) return workspace_for(p, pass);
     if (pass == PHX_PASS_BWD_WEIGHTS && nhwc_wgrad_native(p)) return workspace_for(p, pass);
-    if (const int m = merged_groups(p)) return ChannelsLast(p).bytes() + merged_workspace(p, m, pass);
+    if (const int m = merged_groups(p, pass)) return ChannelsLast(p).bytes() + merged_workspace(p, m, pass);
     // (packed images / partial sums of all groups side by side where one launch runs them)
     if (group_batchable(p, pass)) return (size_t)p.groups * workspace_for(p, pass);
     return ChannelsLast(p).bytes() + workspace_for(p, pass);
@@ -2093,7 +2109,7 @@ static int conv_fwd_quaternion(const phx_qconv_desc* desc, phx_stream_t stream, 
     Problem p;
     const int rc = problem_from_conv(desc, p);
     if (rc != PHX_OK) return rc;
-    const bool direct = thin_groups(p);  // the vector-ALU kernels: groups of few channels, windows beyond the staging limit
+    const bool direct = thin_groups(p, PHX_PASS_FWD);  // the vector-ALU kernels: groups of few channels, windows beyond the staging limit
     if (!direct && nhwc_native(p, PHX_PASS_FWD))
         return run_pwx_nhwc(p, MAP_FWD, static_cast<hipStream_t>(stream), x, w, p.has_bias ? bias_or_null : nullptr, y, workspace,
                             workspace_bytes);
@@ -2105,7 +2121,7 @@ static int conv_fwd_quaternion(const phx_qconv_desc* desc, phx_stream_t stream, 
         g_window_cl = false;
         return nrc;
     }
-    const int merged = direct ? 0 : merged_groups(p);
+    const int merged = direct ? 0 : merged_groups(p, PHX_PASS_FWD);
     if (!direct && !merged && group_batchable(p, PHX_PASS_FWD)) {
         const GroupBatchScope batch(p);
         return do_fwd(p, st, x, w, bias_or_null, y, dry ? nullptr : workspace, dry ? 0 : workspace_bytes);
@@ -2169,7 +2185,7 @@ static int conv_bwd_data_quaternion(const phx_qconv_desc* desc, phx_stream_t str
     // the gradient with respect to a real-valued input has imaginary parts that are stored nowhere;
     // the reference refuses the request likewise (src/conv2d.hpp:394-398)
     if (p.real_input) return PHX_ERR_INVALID_ARGUMENT;
-    const bool direct = thin_groups(p);
+    const bool direct = thin_groups(p, PHX_PASS_BWD_DATA);
     if (!direct && nhwc_native(p, PHX_PASS_BWD_DATA))
         return run_pwx_nhwc(p, MAP_DGRAD, static_cast<hipStream_t>(stream), grad, w, nullptr, dx, workspace, workspace_bytes);
     const GroupOffsets o(p);
@@ -2180,7 +2196,7 @@ static int conv_bwd_data_quaternion(const phx_qconv_desc* desc, phx_stream_t str
         g_window_cl = false;
         return nrc;
     }
-    const int merged = direct ? 0 : merged_groups(p);
+    const int merged = direct ? 0 : merged_groups(p, PHX_PASS_BWD_DATA);
     if (!direct && !merged && group_batchable(p, PHX_PASS_BWD_DATA)) {
         const GroupBatchScope batch(p);
         return do_bwd_data(p, st, grad, w, dx, dry ? nullptr : workspace, dry ? 0 : workspace_bytes);
@@ -2322,14 +2338,14 @@ int phx_qconv2d_bwd_weights(const phx_qconv_desc* desc, phx_stream_t stream, con
     if (rc != PHX_OK) return rc;
     const GroupOffsets o(p);
     hipStream_t st = static_cast<hipStream_t>(stream);
-    const bool direct = thin_groups(p);
+    const bool direct = thin_groups(p, PHX_PASS_BWD_WEIGHTS);
     if (!direct && nhwc_wgrad_native(p)) {
         g_window_cl = true;
         const int nrc = do_bwd_weights(p, st, x, grad, dw, workspace, workspace_bytes);
         g_window_cl = false;
         return nrc;
     }
-    const int merged = direct ? 0 : merged_groups(p);
+    const int merged = direct ? 0 : merged_groups(p, PHX_PASS_BWD_WEIGHTS);
     if (!direct && !merged && group_batchable(p, PHX_PASS_BWD_WEIGHTS)) {
         const GroupBatchScope batch(p);
         return do_bwd_weights(p, st, x, grad, dw, workspace, workspace_bytes);

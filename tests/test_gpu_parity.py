@@ -620,13 +620,16 @@ MERGED_GROUPS = [
                          ids=["f32", "f16_full16", "f16_backward32"])
 @pytest.mark.parametrize("mode", [16, 8])
 @pytest.mark.parametrize("case", MERGED_GROUPS, ids=lambda c: c[0])
-def test_small_groups_run_merged_on_the_matrix_cores(case, mode, dtype, policy):
+def test_small_groups_run_merged_on_the_matrix_cores(case, mode, dtype, policy, tune_env):
     """Groups of fewer than 32 channels would leave most of a 32 x 32 matrix-core tile empty: m consecutive groups (the
     largest divisor of the group count with m x channels <= 32) run as one group with a block-diagonal filter (the
     reference hands `groups` to its scalar convolutions, src/backend/onednn/conv2d.hpp:116-137; how they are run is
     the backend's business).  The kernel labels say `_merged<m>`; results are those of G independent convolutions on
     channel slices through the oracle -- the off-diagonal zeros must not leak into outputs or gradients."""
     name, G, cl, n, ci, co, h, w, kh, kw, stride, dilation, padding, m = case
+    # (passes in fp32 arithmetic would take groups of up to 64 / 256 channel pairs to the vector-ALU kernels: here they
+    # stay on the matrix cores like the fp16 ones, so that merging is tested in every arithmetic)
+    tune_env(PHX_TUNE_THIN_MAX32="1")
     cig, cog = ci // G, co // G
     scale = 1.0 if dtype == torch.float32 else 0.5
     g, x, _, b, gr = make_inputs(name_seed(name) + 70, n, ci, co, h, w, kh, kw, stride, dilation, padding, dtype, scale)
@@ -649,7 +652,20 @@ def test_small_groups_run_merged_on_the_matrix_cores(case, mode, dtype, policy):
     names.append(capi.last_kernel_name())
     # the label of the last launch: the groups merged there (0: a single remaining group, which runs as it is)
     tag = "_merged%d" % m
-    assert all((tag in k) if m > 0 else ("_merged" not in k) for k in names), names
+    assert all((tag in k) if m > 0 else ("_merged" not in k) for k in names[:2]), names
+
+    def last_merged(tile):  # the planner's rule, for tiles of `tile` channels
+        most = min(G, tile // max(cig, cog))
+        if most < 2:
+            return 0
+        divisor = max(d for d in range(1, most + 1) if G % d == 0)
+        per = divisor if divisor > 1 and G // divisor == -(-G // most) else most
+        return per if G % per == 0 else (G % per if G % per > 1 else 0)
+
+    assert last_merged(32) == max(m, 0)
+    # the filter gradient in fp32 arithmetic works on 64 x 64 channel tiles: twice as many groups fit
+    m_wgrad = last_merged(32 if (dtype == torch.float16 and policy == "full16") else 64)
+    assert ("_merged%d" % m_wgrad in names[2]) if m_wgrad else ("_merged" not in names[2]), names
     # packed ahead of the passes, the block-diagonal filter is one more image: same kernels, same results
     packed = ops.conv2d_pack_filters(wd, desc)
     # (a remaining single group of four channels at stride 2 runs by space-to-depth, whose forward filter is rearranged per call)
