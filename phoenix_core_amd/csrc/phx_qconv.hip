@@ -1394,7 +1394,16 @@ static PhaseAxis phase_axis(int a, int extent, int k, int d, int s, int pad_befo
 static bool dgrad_by_phases(const Problem& p) {
     if ((p.sh == 1 && p.sw == 1) || p.sh * p.sw > 16 || is_empty(p) || channel_slices(p)) return false;
     if (tune().phase >= 0) return tune().phase != 0;
-    return p.kh == 1 && p.kw == 1;
+    if (p.kh == 1 && p.kw == 1) return true;
+    // Large problems: zero insertion multiplies the arithmetic by sh * sw, which the launches of the phases cost less
+    // than once there is enough of it and the phases' images are not tiny (fp16, N=64, 3x3 stride 2, zero insertion
+    // against phases: 128 channels at 28x28 261 / 197 us, 256 at 28x28 967 / 509, 512 at 14x14 1064 / 611, 5x5 256 at
+    // 28x28 2174 / 789; but 64 at 28x28 83 / 103, 128 at 14x14 78 / 153, 512 at 7x7 346 / 463)
+    // In fp32 arithmetic the phases win at every size measured (N=64, 3x3: 16 channels at 56x56 359 / 125 us, 128 at
+    // 14x14 622 / 353, 512 at 7x7 2967 / 1281, 256 at 28x28 10325 / 1809).
+    if (!use_f16_mfma(p, PHX_PASS_BWD_DATA)) return true;
+    const double flops = 32.0 * p.n * p.ci * p.co * p.ho * p.wo * p.kh * p.kw;
+    return flops >= 40e9 && (long)p.h * p.w >= 196;
 }
 
 static Corr phase_corr(const Problem& p, const PhaseAxis& ah, const PhaseAxis& aw) {
