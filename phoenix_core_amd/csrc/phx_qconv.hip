@@ -1825,12 +1825,18 @@ static bool thin_groups(const Problem& p, int pass) {
     if (is_empty(p) || p.ho <= 0 || p.wo <= 0) return false;
     if ((long)p.kh * p.kw > 2048 || std::max(p.ci_mem, p.co_mem) > 65535) return false;  // (a filter chunk in LDS; grid rows)
     if (tune().direct || window_beyond_staging(p)) return true;
+    const long pairs = (long)p.ci * p.co;
+    // The filter gradient in fp32 arithmetic works on 64 x 64 channel tiles whatever the layer holds: its time follows
+    // the pixels and taps alone (3x3, 56x56, N=64: 1.39 ms from 8 to 64 channels), that of the vector-ALU kernel the
+    // channel pairs too -- 8 -> 8 channels 0.11 ms, 16 -> 16 0.35, 3 -> 64 0.29, 24 -> 24 0.77, 32 -> 32 1.20; a
+    // single tap: 16 -> 16 0.18 against 0.17.  Layers of few channels, grouped or not, run it here.
+    if (pass == PHX_PASS_BWD_WEIGHTS && p.groups <= 1 && tune().thin_max32 > 0 && !wgrad_on_f16_mfma(flatten_pointwise(p)))
+        return pairs <= (p.kh * p.kw > 1 ? 512 : 128);
     if (p.groups <= 1) return false;
     // Passes in fp32 arithmetic (fp32 tensors, fp16 tensors where the policy says so) have a sixteenth of the fp16
     // matrix-core rate to lose against, and their filter gradient works on 64 x 64 channel tiles: measured like above,
     // 8 x 8 channels per group 159 / 149 / 206 us here against 194 / 193 / 742 merged, 16 x 16 260 / 254 / 346 against
     // 192 / 193 / 745 -- up to 64 pairs per group run here, the filter gradient up to 256.
-    const long pairs = (long)p.ci * p.co;
     if (use_f16_mfma(p, pass)) return pairs <= tune().thin_max;
     return pairs <= (long)tune().thin_max32 * (pass == PHX_PASS_BWD_WEIGHTS ? 4 : 1);
 }
