@@ -35,7 +35,7 @@ struct Tuning {
     bool pwrall = false;              // PHX_TUNE_PWRALL: ... and every problem that kernel can run goes to it (not only those of at most 32 output channels)
     bool nowincl = false;             // PHX_TUNE_NOWINCL: channels-last windowed problems go through the transposes
     bool nogroupbatch = false;        // PHX_TUNE_NOGROUPBATCH: a grouped convolution runs group after group
-    double wg_kpw = 0.01;             // PHX_TUNE_WGKPW: how much the fp32 filter-gradient planner favours larger pixel tiles (see plan_wgrad_f32)
+    double wg_kpw = 0.01;             // PHX_TUNE_WGKPW: how much the fp32 filter-gradient planner favours larger pixel tiles on small images (see plan_wgrad_f32)
     int thin_max32 = 64;              // PHX_TUNE_THIN_MAX32: the same bound for passes in fp32 arithmetic (x4 for the filter gradient); PHX_TUNE_THIN_MAX=0 zeroes it too
     int thin_max = 4;                 // PHX_TUNE_THIN_MAX: most input x output channels per group that run on the vector-ALU kernels for thin groups (0 = never)
     bool nomerge = false;             // PHX_TUNE_NOMERGE: groups are never merged into block-diagonal ones
@@ -1116,6 +1116,7 @@ static bool plan_wgrad_f32(const Problem& p, WgPlan& best) {
     const int TPW = (best.kmode == 16) ? 3 : 1;
     const int nkw = std::min(TPW, p.kw);
     double best_score = -1.0;
+    const bool small_image = p.ho * p.wo < 100;
     for (int vec = 0; vec < 2; ++vec) {  // vec: windows staged as groups of 4 positions (16-byte loads)
         // KPp + HPp (+ offsets) per staged channel; the eight-wave workgroups have their CU, and its LDS, to themselves
         const int budget = (wgrad_f32_ksets(best.kmode, vec != 0) == 2 && !tune().oldplan ? 72 * 1024 / 4 : LDS_FLOATS_MAX) / (4 * 64);
@@ -1138,9 +1139,9 @@ static bool plan_wgrad_f32(const Problem& p, WgPlan& best) {
                     const double eff = ((double)p.n * p.ho * p.wo) / ((double)tn * th * tw * KP);
                     // (a tile is a barrier pair and a staging round whatever its size: on 7x7 images four rows of 8 at 77 %
                     // fill beat one row of 8 at 88 % -- 512 channels, N=64: 2.46 against 4.32 ms, 128 channels 0.14 against
-                    // 0.23 ms -- which the weight on the tile's positions expresses; larger images are not affected)
+                    // 0.23 ms -- which the weight on the tile's positions expresses for images below 10x10)
                     const double score =
-                        eff * (1.0 + tune().wg_kpw * KP) * (TW >= std::min(p.wo, 8) ? 1.0 : 0.5) * (vec ? 1.25 : 1.0);
+                        eff * (1.0 + (small_image ? tune().wg_kpw : 0.002) * KP) * (TW >= std::min(p.wo, 8) ? 1.0 : 0.5) * (vec ? 1.25 : 1.0);
                     if (score > best_score) {
                         best_score = score;
                         best.vec = vec != 0;
