@@ -224,6 +224,51 @@ def test_qconv2d_groups_and_channels_last(ci, co, G):
     torch.testing.assert_close(last.bias.grad, ref.bias.grad, rtol=1e-4, atol=1e-4)
 
 
+def test_grouped_layers_replay_from_a_captured_graph():
+    """Depthwise layers (vector-ALU kernels), groups merged into block-diagonal ones and a strided depthwise layer in one
+    captured forward + backward pass: three replays, each with an eager step between them, reproduce the eager loss,
+    input gradient and filter gradients bit for bit (no memset nodes, no allocation inside the captured calls)."""
+    ctx = Ctx(8, "full16")
+    torch.manual_seed(0)
+    layers = [phx.QConv2d(32, 32, 3, padding="SAME", bias=True, context=ctx, groups=32, dtype=torch.float16).cuda(),
+              phx.QConv2d(32, 64, 3, padding="SAME", bias=True, context=ctx, groups=8, dtype=torch.float16).cuda(),
+              phx.QConv2d(64, 64, 3, stride=2, padding="SAME", bias=False, context=ctx, groups=64, dtype=torch.float16).cuda(),
+              phx.QConv2d(64, 32, 1, padding="VALID", bias=True, context=ctx, groups=4, dtype=torch.float16).cuda()]
+    x = (0.5 * torch.randn(8, 32, 20, 20, device="cuda")).half().requires_grad_()
+
+    def run():
+        for layer in layers:
+            layer.weight.grad = None
+        x.grad = None
+        y = x
+        for layer in layers:
+            y = layer(y)
+        loss = (y.float() ** 2).mean()
+        loss.backward()
+        return loss, x.grad, [layer.weight.grad for layer in layers]
+
+    def snapshot(out):
+        return out[0].detach().clone(), out[1].detach().clone(), [g.detach().clone() for g in out[2]]
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            run()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static = run()
+    for _ in range(3):
+        graph.replay()
+        torch.cuda.synchronize()
+        got = snapshot(static)
+        want = snapshot(run())
+        torch.cuda.synchronize()
+        assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1])
+        assert all(torch.equal(a, b) for a, b in zip(got[2], want[2]))
+
+
 def test_qlinear_autograd_matches_oracle():
     torch.manual_seed(1)
     lin = phx.QLinear(12, 7, bias=True, context=Ctx(8)).cuda()
