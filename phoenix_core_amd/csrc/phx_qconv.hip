@@ -38,6 +38,7 @@ struct Tuning {
     double wg_kpw = 0.01;             // PHX_TUNE_WGKPW: how much the fp32 filter-gradient planner favours larger pixel tiles on small images (see plan_wgrad_f32)
     int thin_max32 = 64;              // PHX_TUNE_THIN_MAX32: the same bound for passes in fp32 arithmetic (x4 for the filter gradient); PHX_TUNE_THIN_MAX=0 zeroes it too
     int thin_max = 4;                 // PHX_TUNE_THIN_MAX: most input x output channels per group that run on the vector-ALU kernels for thin groups (0 = never)
+    bool nodensecl = false;           // PHX_TUNE_NODENSECL: Dense never runs as a channels-last pointwise convolution
     bool nomerge = false;             // PHX_TUNE_NOMERGE: groups are never merged into block-diagonal ones
     bool direct = false;              // PHX_TUNE_DIRECT: every convolution those kernels can run goes to them (an independent path to check the matrix-core kernels against)
     bool thin_notile = false;         // PHX_TUNE_THIN_NOTILE: ... and never on the kernel that stages window tiles in LDS
@@ -76,6 +77,7 @@ struct Tuning {
         thin_notile = getenv("PHX_TUNE_THIN_NOTILE") != nullptr;
         direct = getenv("PHX_TUNE_DIRECT") != nullptr;
         nomerge = getenv("PHX_TUNE_NOMERGE") != nullptr;
+        nodensecl = getenv("PHX_TUNE_NODENSECL") != nullptr;
         nosmalldense = getenv("PHX_TUNE_NOSMALLDENSE") != nullptr;
         if (const char* e = getenv("PHX_TUNE_VEC")) vec = atoi(e);
         if (const char* e = getenv("PHX_TUNE_WGS")) wgs = atoi(e);
@@ -2110,11 +2112,30 @@ static int run_dense_small(const Problem& p, int pass, hipStream_t st, const voi
     return PHX_OK;
 }
 
+// A Dense layer's tensors [4n, units] are those of a channels-last pointwise convolution on ONE image of n x 1
+// positions, so the larger fp16 problems run on the channels-last pointwise kernels (streaming operand copies, no
+// staged windows) instead of a 1 x 1 convolution on n images of one position each.  PHX_TUNE_NODENSECL keeps the latter.
+static bool dense_as_channels_last(const Problem& p, int pass, Problem& q) {
+    if (tune().nodensecl || is_empty(p)) return false;
+    q = p;
+    q.n = 1; q.h = p.n; q.w = 1; q.ho = p.n; q.wo = 1; q.nhwc = true;
+    return pass == PHX_PASS_BWD_WEIGHTS ? nhwc_wgrad_native(q) : nhwc_native(q, pass);
+}
+
+// The FMA kernels' filter gradient is one thread per filter quaternion walking the batch: beyond 128 rows the
+// channels-last matrix-core kernel wins where it applies (64 -> 64 units, 1024 rows: 24 against 197 us for both gradients).
+static bool dense_runs_small(const Problem& p, int pass) {
+    if (!dense_is_small(p)) return false;
+    Problem q;
+    return !(pass == PHX_PASS_BWD_WEIGHTS && p.n > 128 && dense_as_channels_last(p, pass, q));
+}
+
 size_t phx_qdense_workspace_bytes(const phx_qdense_desc* desc, int pass) {
     if (desc && desc->algebra != PHX_QUATERNION) return algebra_dense_workspace_bytes(desc, pass);
-    Problem p;
+    Problem p, q;
     if (problem_from_dense(desc, p) != PHX_OK) return 0;
-    if (dense_is_small(p)) return 0;
+    if (dense_runs_small(p, pass)) return 0;
+    if (dense_as_channels_last(p, pass, q)) return pass == PHX_PASS_BWD_WEIGHTS ? workspace_for(q, pass) : nhwc_native_workspace(q, pass);
     return workspace_for(p, pass);
 }
 
@@ -2398,7 +2419,10 @@ int phx_qdense_fwd(const phx_qdense_desc* desc, phx_stream_t stream, const void*
     Problem p;
     const int rc = problem_from_dense(desc, p);
     if (rc != PHX_OK) return rc;
-    if (dense_is_small(p)) return is_empty(p) ? PHX_OK : run_dense_small(p, PHX_PASS_FWD, static_cast<hipStream_t>(stream), x, w, bias_or_null, y);
+    if (dense_runs_small(p, PHX_PASS_FWD)) return is_empty(p) ? PHX_OK : run_dense_small(p, PHX_PASS_FWD, static_cast<hipStream_t>(stream), x, w, bias_or_null, y);
+    Problem q;
+    if (dense_as_channels_last(p, PHX_PASS_FWD, q))
+        return run_pwx_nhwc(q, MAP_FWD, static_cast<hipStream_t>(stream), x, w, q.has_bias ? bias_or_null : nullptr, y, workspace, workspace_bytes);
     return do_fwd(p, static_cast<hipStream_t>(stream), x, w, bias_or_null, y, workspace, workspace_bytes);
 }
 
@@ -2412,7 +2436,10 @@ int phx_qdense_bwd_data(const phx_qdense_desc* desc, phx_stream_t stream, const 
     Problem p;
     const int rc = problem_from_dense(desc, p);
     if (rc != PHX_OK) return rc;
-    if (dense_is_small(p)) return is_empty(p) ? PHX_OK : run_dense_small(p, PHX_PASS_BWD_DATA, static_cast<hipStream_t>(stream), grad, w, nullptr, dx);
+    if (dense_runs_small(p, PHX_PASS_BWD_DATA)) return is_empty(p) ? PHX_OK : run_dense_small(p, PHX_PASS_BWD_DATA, static_cast<hipStream_t>(stream), grad, w, nullptr, dx);
+    Problem q;
+    if (dense_as_channels_last(p, PHX_PASS_BWD_DATA, q))
+        return run_pwx_nhwc(q, MAP_DGRAD, static_cast<hipStream_t>(stream), grad, w, nullptr, dx, workspace, workspace_bytes);
     return do_bwd_data(p, static_cast<hipStream_t>(stream), grad, w, dx, workspace, workspace_bytes);
 }
 
@@ -2426,7 +2453,14 @@ int phx_qdense_bwd_weights(const phx_qdense_desc* desc, phx_stream_t stream, con
     Problem p;
     const int rc = problem_from_dense(desc, p);
     if (rc != PHX_OK) return rc;
-    if (dense_is_small(p)) return run_dense_small(p, PHX_PASS_BWD_WEIGHTS, static_cast<hipStream_t>(stream), x, grad, nullptr, dw);
+    if (dense_runs_small(p, PHX_PASS_BWD_WEIGHTS)) return run_dense_small(p, PHX_PASS_BWD_WEIGHTS, static_cast<hipStream_t>(stream), x, grad, nullptr, dw);
+    Problem q;
+    if (dense_as_channels_last(p, PHX_PASS_BWD_WEIGHTS, q)) {
+        g_window_cl = true;
+        const int qrc = do_bwd_weights(q, static_cast<hipStream_t>(stream), x, grad, dw, workspace, workspace_bytes);
+        g_window_cl = false;
+        return qrc;
+    }
     return do_bwd_weights(p, static_cast<hipStream_t>(stream), x, grad, dw, workspace, workspace_bytes);
 }
 

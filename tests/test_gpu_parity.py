@@ -1112,6 +1112,47 @@ def test_dense_fp16(mode, policy, kernels, tune_env):
     assert_close(dw.cpu().numpy(), want_dw, torch.float16, "dense wgrad")
 
 
+@pytest.mark.parametrize("layout", ["IO", "OI"])
+@pytest.mark.parametrize("policy", ["full16", "backward32"])
+@pytest.mark.parametrize("shape", [(3000, 128, 72), (8192, 64, 64), (177, 512, 256), (1024, 96, 250), (1024, 64, 64)], ids=lambda s: "n%d_%dto%d" % s)
+def test_larger_dense_runs_as_a_channels_last_pointwise_convolution(shape, policy, layout, tune_env):
+    """A Dense layer's tensors [4n, units] are those of a channels-last pointwise convolution on one image of n x 1
+    positions (denseFwd / denseBwd, src/upstride.hpp:53-86): beyond the sizes of the FMA kernels, fp16 problems whose
+    unit counts are multiples of 8 run on the channels-last pointwise kernels -- the passes that the policy leaves on
+    fp16 matrix cores -- and agree with the 1 x 1 convolution on n images they ran as before (PHX_TUNE_NODENSECL)
+    and with the oracle."""
+    n, ni, no = shape
+    r = np.random.default_rng(n + ni)
+    x = (0.5 * r.standard_normal((4 * n, ni))).astype(np.float16)
+    w = (0.5 * r.standard_normal((4, ni, no)) * np.sqrt(2.0 / ni)).astype(np.float16)
+    b = (0.5 * r.standard_normal((4, no))).astype(np.float16)
+    gr = (0.5 * r.standard_normal((4 * n, no))).astype(np.float16)
+    w_dev = w if layout == "IO" else np.ascontiguousarray(w.transpose(0, 2, 1))
+    desc = phx.DenseDescriptor(x.shape, w_dev.shape, filter_layout=layout, use_bias=True, dtype=torch.float16, context=Ctx(8, policy))
+    xd, wd, bd, gd = (torch.from_numpy(a).cuda() for a in (x, w_dev, b, gr))
+    got = {}
+    for direct in (True, False):
+        tune_env(PHX_TUNE_NODENSECL=None if direct else "1")
+        y = phx.dense_fwd(xd, wd, bd, desc)
+        k_fwd = capi.last_kernel_name()
+        dw, dx = phx.dense_bwd(xd, wd, gd, desc)
+        k_dx = capi.last_kernel_name()  # (the input gradient runs last)
+        # (up to 16 M products forward and input gradient stay on the FMA kernels; of such a problem only the filter
+        # gradient of a batch beyond 128 rows moves to the matrix cores: the last shape)
+        eligible = direct and no % 8 == 0 and n * ni * no > 16 << 20
+        assert ("pwxcl" in k_fwd) == eligible and ("pwxcl" in k_dx) == (eligible and policy == "full16"), (k_fwd, k_dx)
+        got[direct] = (y, dx, dw)
+    x64, w64, b64, g64 = (a.astype(np.float64) for a in (x, w, b, gr))
+    want_y = oracle.dense_fwd(x64, w64, b64, "generic")
+    want_dw, want_dx = oracle.dense_bwd(x64, w64, g64, "generic")
+    for direct in (True, False):
+        y, dx, dw = got[direct]
+        got_dw = dw.cpu().numpy()
+        assert_close(y.cpu().numpy(), want_y, torch.float16, "dense fwd")
+        assert_close(dx.cpu().numpy(), want_dx, torch.float16, "dense dgrad")
+        assert_close(got_dw if layout == "IO" else got_dw.transpose(0, 2, 1), want_dw, torch.float16, "dense wgrad")
+
+
 def test_mismatched_tensors_are_refused_before_the_library_reads_them():
     """The library reads raw device memory in the descriptor's type: a tensor of another type or shape must be
     refused by the host layer (a fp16 filter under a fp32 descriptor would be read past its end)."""
