@@ -147,6 +147,10 @@ int launch_merge_filter(bool half_storage, const MergeFilterArgs& a, bool to_cal
 int launch_transpose(bool half_storage, const TransposeArgs& a, hipStream_t st);
 int launch_fill_zero(void* dst, size_t bytes, hipStream_t st);  // a kernel, so that it can be captured in a graph
 int launch_add_inplace(bool half_storage, void* dst, const void* src, long count, hipStream_t st);  // dst += src
+// dst = the sum of `slices` partial tensors of `count` elements (+ bias of the element's channel, + addend); partial results
+// of a pass whose channel reduction was cut into slices
+int launch_slice_sum(bool half_storage, const void* partial, int slices, long count, void* dst, const void* bias, const void* addend,
+                     int plane, int channels, long comp_count, hipStream_t st);
 
 // REAL / COMPLEX / GA_300 as compositions on the quaternion entry points (phx_algebra.hip); pass = phx_pass,
 // (a, b) = (x, w) forward, (grad, w) input gradient, (x, grad) filter gradient

@@ -147,6 +147,37 @@ int launch_add_inplace(bool half_storage, void* dst, const void* src, long count
     return 0;
 }
 
+// dst = sum of `slices` tensors of `count` elements each lying `count` elements apart (+ bias per channel: element e
+// belongs to channel (e / plane) % channels of component e / comp_count; + addend, element by element): what closes a
+// forward / input-gradient pass whose reduction over the channels was cut into slices.  fp32 sums, one rounding.
+template <typename TS>
+__global__ void __launch_bounds__(WG_THREADS) slice_sum_kernel(const TS* partial, int slices, long count, TS* dst, const TS* bias,
+                                                               const TS* addend, int plane, int channels, long comp_count) {
+    const long stride = (long)gridDim.x * blockDim.x;
+    for (long e = (long)blockIdx.x * blockDim.x + threadIdx.x; e < count; e += stride) {
+        float acc = 0.0f;
+        for (int z = 0; z < slices; ++z) acc += (float)partial[z * count + e];
+        if (bias) acc += (float)bias[(e / comp_count) * channels + (e / plane) % channels];
+        if (addend) acc += (float)addend[e];
+        dst[e] = (TS)acc;
+    }
+}
+
+int launch_slice_sum(bool half_storage, const void* partial, int slices, long count, void* dst, const void* bias, const void* addend,
+                     int plane, int channels, long comp_count, hipStream_t st) {
+    if (count <= 0) return 0;
+    const int blocks = blocks_for(count);
+    if (half_storage)
+        hipLaunchKernelGGL((slice_sum_kernel<_Float16>), dim3(blocks), dim3(WG_THREADS), 0, st, static_cast<const _Float16*>(partial),
+                           slices, count, static_cast<_Float16*>(dst), static_cast<const _Float16*>(bias),
+                           static_cast<const _Float16*>(addend), plane, channels, comp_count);
+    else
+        hipLaunchKernelGGL((slice_sum_kernel<float>), dim3(blocks), dim3(WG_THREADS), 0, st, static_cast<const float*>(partial), slices,
+                           count, static_cast<float*>(dst), static_cast<const float*>(bias), static_cast<const float*>(addend), plane,
+                           channels, comp_count);
+    return 0;
+}
+
 int launch_transpose(bool half_storage, const TransposeArgs& a, hipStream_t st) {
     const int T = half_storage ? 64 : 32;  // tile edge of one wave
     const long tiles = a.batch * ((a.R + T - 1) / T) * ((a.Cc + T - 1) / T);

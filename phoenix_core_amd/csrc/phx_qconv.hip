@@ -38,6 +38,7 @@ struct Tuning {
     double wg_kpw = 0.01;             // PHX_TUNE_WGKPW: how much the fp32 filter-gradient planner favours larger pixel tiles on small images (see plan_wgrad_f32)
     int thin_max32 = 64;              // PHX_TUNE_THIN_MAX32: the same bound for passes in fp32 arithmetic (x4 for the filter gradient); PHX_TUNE_THIN_MAX=0 zeroes it too
     int thin_max = 4;                 // PHX_TUNE_THIN_MAX: most input x output channels per group that run on the vector-ALU kernels for thin groups (0 = never)
+    int kslices = -1;                 // PHX_TUNE_KSLICES: reduction slices of a forward / input-gradient pass (0 = never, unset = by the rule of corr_slices)
     bool nodensecl = false;           // PHX_TUNE_NODENSECL: Dense never runs as a channels-last pointwise convolution
     bool nomerge = false;             // PHX_TUNE_NOMERGE: groups are never merged into block-diagonal ones
     bool direct = false;              // PHX_TUNE_DIRECT: every convolution those kernels can run goes to them (an independent path to check the matrix-core kernels against)
@@ -78,6 +79,7 @@ struct Tuning {
         direct = getenv("PHX_TUNE_DIRECT") != nullptr;
         nomerge = getenv("PHX_TUNE_NOMERGE") != nullptr;
         nodensecl = getenv("PHX_TUNE_NODENSECL") != nullptr;
+        if (const char* e = getenv("PHX_TUNE_KSLICES")) kslices = atoi(e);
         nosmalldense = getenv("PHX_TUNE_NOSMALLDENSE") != nullptr;
         if (const char* e = getenv("PHX_TUNE_VEC")) vec = atoi(e);
         if (const char* e = getenv("PHX_TUNE_WGS")) wgs = atoi(e);
@@ -1508,12 +1510,121 @@ static void subsample_input(const Problem& p, const void* x, void* xs, hipStream
     launch_subsample(p.dtype == PHX_F16, a, st);
 }
 
+// Reduction slices of a forward / input-gradient pass.  Those kernels give a workgroup an output tile and the whole
+// reduction over channels and taps, so a pass with few output tiles and many channels (small batches on deep
+// layers: 512 channels at 7x7, N=1 is 16 workgroups of 288 steps) leaves most of the GPU idle however long it
+// takes.  Such a pass runs as Z passes over Z slices of the reduced channels in ONE launch per kernel (the grid rows
+// that run the groups of a grouped convolution: slice z reads its channels of the input-side tensor and of the
+// filter and writes a partial result tensor of its own in the workspace), and a streaming kernel adds the partial
+// tensors (and the bias) into the caller's tensor, in fp32 with one rounding.
+// Z = the largest power of two that keeps at least 32 channels (a multiple of 16) and 8 reduction steps per slice
+// and at most two workgroups per CU in flight; 0 = the pass runs unsliced (enough workgroups already, or a rewritten
+// problem: groups, channels-last, real-valued input, space-to-depth, subsampling, phases).
+static int slices_rule(const Problem& p, int pass, const Corr& creal) {
+    Corr c;
+    FwdPlan pl;
+    int pw = 0;
+    const bool f16 = use_f16_mfma(p, pass);
+    if (!plan_corr(creal, p.mode, f16, c, pl, pw)) return 0;
+    const int red = creal.Cin;
+    const auto fits = [&](int z) { return red % z == 0 && (red / z) % 16 == 0 && red / z >= 32; };
+    if (tune().kslices > 1) return fits(tune().kslices) ? tune().kslices : 0;
+    const int cus = 256;  // (a constant, as in plan_forward: the workspace query answers without a device)
+    // workgroups (items of the pointwise streaming kernel, which runs at most two per CU and needs longer slices) and
+    // reduction steps of the unsliced pass
+    const long wgs = pl.pwx ? (long)cdiv(creal.N * cdiv(creal.Hin * creal.Win, 8), 8 * (4 / pl.pwx)) * pl.co_tiles : pl.wgs;
+    const long steps = pl.pwx ? pl.pwx_steps : (long)pl.nchunks * c.Kh * c.Kw;  // (c: a pointwise problem may run as a column of virtual taps)
+    const long most = pl.pwx ? cus : 2L * cus;
+    int Z = 1;
+    while (fits(2 * Z) && wgs * 2 * Z <= most && steps / (2 * Z) >= 8) Z *= 2;
+    // (two slices do not pay for the extra pass over the result on the fp16 matrix cores: 256 -> 256 3x3 at 14x14, N=16
+    // 107 -> 115 us; in fp32 arithmetic they do: 570 -> 410)
+    return Z >= (f16 ? 4 : 2) ? Z : 0;
+}
+
+static int corr_slices(const Problem& p, int pass) {
+    if (tune().kslices == 0 || pass == PHX_PASS_BWD_WEIGHTS || is_empty(p)) return 0;
+    if (channel_slices(p) || p.nhwc || p.real_input || g_batch.n > 1 || g_window_cl) return 0;
+    if (pass == PHX_PASS_BWD_DATA && dgrad_by_phases(p)) return 0;  // (see phase_slices)
+    if (pass == PHX_PASS_FWD) {
+        S2dView v;
+        Problem q;
+        size_t xs_bytes = 0;
+        if (s2d_view(p, v) || subsample_view(p, q, xs_bytes)) return 0;
+    }
+    return slices_rule(p, pass, pass == PHX_PASS_FWD ? corr_forward(p) : corr_dgrad(p));
+}
+
+// A strided input gradient that runs by phases (dgrad_by_phases): every phase is a pass of its own and is sliced like
+// one, all by the Z that the rule gives for the phase with the most taps.
+static int phase_slices(const Problem& p) {
+    if (tune().kslices == 0 || !dgrad_by_phases(p) || p.nhwc || g_batch.n > 1 || g_window_cl) return 0;
+    PhaseAxis bh{}, bw{};
+    for (int a = 0; a < p.sh; ++a)
+        for (int b = 0; b < p.sw; ++b) {
+            const PhaseAxis ah = phase_axis(a, p.h, p.kh, p.dh, p.sh, p.pt), aw = phase_axis(b, p.w, p.kw, p.dw, p.sw, p.pl);
+            if (!ah.taps || !aw.taps || !ah.size || !aw.size) continue;
+            if (ah.taps * aw.taps > bh.taps * bw.taps) { bh = ah; bw = aw; }
+        }
+    return bh.taps * bw.taps ? slices_rule(p, PHX_PASS_BWD_DATA, phase_corr(p, bh, bw)) : 0;
+}
+
+// the problem of one slice, and the steps from a slice to the next in the tensors of the pass
+struct SlicedCorr {
+    Problem q;
+    GroupBatch steps;
+    size_t partial_bytes;  // Z partial result tensors
+    long count;            // elements of one
+    // (plane: positions per channel of the result tensor; 0 = the whole image, else those of one phase)
+    SlicedCorr(const Problem& p, int pass, int Z, long plane = 0) : q(p) {
+        const size_t esize = p.dtype == PHX_F32 ? 4 : 2;
+        q.has_bias = false;
+        steps.n = Z;
+        if (pass == PHX_PASS_FWD) {
+            q.ci = p.ci / Z;
+            count = 4L * p.n * p.co * p.ho * p.wo;
+            steps.x = (size_t)q.ci * p.h * p.w * esize;
+            steps.y = (size_t)count * esize;
+            steps.w = (size_t)q.ci * p.fs.si * esize;
+        } else {
+            q.co = p.co / Z;
+            count = 4L * p.n * p.ci * (plane ? plane : (long)p.h * p.w);
+            steps.y = (size_t)q.co * p.ho * p.wo * esize;
+            steps.x = (size_t)count * esize;
+            steps.w = (size_t)q.co * p.fs.so * esize;
+        }
+        partial_bytes = align_up((size_t)Z * count * esize, 256);
+    }
+};
+
 static size_t workspace_for(const Problem& p, int pass) {
     S2dView v;
     if (pass != PHX_PASS_BWD_DATA && s2d_view(p, v)) return v.x2_bytes + v.w2_bytes + workspace_plain(v.q, pass);
     Problem q;
     size_t xs_bytes = 0;
     if (pass != PHX_PASS_BWD_DATA && subsample_view(p, q, xs_bytes)) return xs_bytes + workspace_plain(q, pass);
+    if (const int Z = corr_slices(p, pass)) {
+        const SlicedCorr sc(p, pass, Z);
+        return sc.partial_bytes + (size_t)Z * workspace_plain(sc.q, pass);
+    }
+    if (const int Z = pass == PHX_PASS_BWD_DATA ? phase_slices(p) : 0) {
+        // phase buffers + the most that a phase takes for its partial tensors and the packed sub-filters of its slices
+        const size_t esize = p.dtype == PHX_F32 ? 4 : 2;
+        size_t bufs = 0, most = 0;
+        for (int a = 0; a < p.sh; ++a)
+            for (int b = 0; b < p.sw; ++b) {
+                const PhaseAxis ah = phase_axis(a, p.h, p.kh, p.dh, p.sh, p.pt), aw = phase_axis(b, p.w, p.kw, p.dw, p.sw, p.pl);
+                if (!ah.taps || !aw.taps || !ah.size || !aw.size) continue;
+                bufs += align_up((size_t)4 * p.n * p.ci * ah.size * aw.size * esize, 256);
+                const SlicedCorr sc(p, pass, Z, (long)ah.size * aw.size);
+                Corr c;
+                FwdPlan pl;
+                int pw = 0;
+                if (!plan_corr(phase_corr(sc.q, ah, aw), p.mode, use_f16_mfma(p, pass), c, pl, pw)) return 0;
+                most = std::max(most, sc.partial_bytes + (size_t)Z * align_up(pl.wpk_bytes, 256));
+            }
+        return bufs + most;
+    }
     return workspace_plain(p, pass);
 }
 
@@ -1521,6 +1632,31 @@ static void s2d_rearrange_input(const Problem& p, const S2dView& v, const void* 
     S2dArgs a;
     a.src = x; a.dst = x2; a.planes = (p.real_input ? 1L : 4L) * p.n * p.ci; a.H = p.h; a.W = p.w; a.H2 = v.q.h; a.W2 = v.q.w;
     launch_s2d_input(p.dtype == PHX_F16, a, st);
+}
+
+// One forward (map == MAP_FWD: in = x) or input-gradient pass in Z reduction slices (see corr_slices)
+// (ah, aw: one phase of a strided input gradient, out = that phase's buffer)
+static int run_sliced(const Problem& p, int Z, int map, hipStream_t st, const void* in, const void* w, const void* bias, void* out,
+                      void* ws, size_t wsb, const PhaseAxis* ah = nullptr, const PhaseAxis* aw = nullptr) {
+    const int pass = map == MAP_FWD ? PHX_PASS_FWD : PHX_PASS_BWD_DATA;
+    const long plane = ah ? (long)ah->size * aw->size : map == MAP_FWD ? (long)p.ho * p.wo : (long)p.h * p.w;
+    const SlicedCorr sc(p, pass, Z, ah ? plane : 0);
+    const bool dry = g_pack.dry();
+    if (!dry && (wsb < sc.partial_bytes || !ws)) return PHX_ERR_WORKSPACE;
+    char* partial = static_cast<char*>(ws);
+    g_batch = sc.steps;
+    const int rc = run_corr(sc.q, ah ? phase_corr(sc.q, *ah, *aw) : map == MAP_FWD ? corr_forward(sc.q) : corr_dgrad(sc.q), map, st, in, w, nullptr, dry ? nullptr : partial,
+                            dry ? nullptr : partial + sc.partial_bytes, dry ? 0 : wsb - sc.partial_bytes);
+    g_batch = GroupBatch{};
+    if (rc != PHX_OK || dry) return rc;
+    const bool add = map == MAP_DGRAD && g_addend.dx == out && g_addend.ptr && !g_addend.fused;
+    launch_slice_sum(p.dtype == PHX_F16, partial, Z, sc.count, out, bias, add ? g_addend.ptr : nullptr,
+                     (int)plane, map == MAP_FWD ? p.co : p.ci, sc.count / 4, st);
+    PHX_HIP(hipGetLastError());
+    if (add) g_addend.fused = true;
+    const size_t len = strlen(g_name_buf);
+    if (g_last_kernel == g_name_buf && len < sizeof(g_name_buf)) snprintf(g_name_buf + len, sizeof(g_name_buf) - len, "_kslices%d", Z);
+    return PHX_OK;
 }
 
 static int do_fwd(const Problem& p, hipStream_t st, const void* x, const void* w, const void* bias, void* y, void* ws,
@@ -1561,6 +1697,7 @@ static int do_fwd(const Problem& p, hipStream_t st, const void* x, const void* w
         g_name_prefix = "";
         return rc;
     }
+    if (const int Z = corr_slices(p, PHX_PASS_FWD)) return run_sliced(p, Z, MAP_FWD, st, x, w, b, y, ws, wsb);
     const Corr c = corr_forward(p);
     return run_corr(p, c, MAP_FWD, st, x, w, b, y, ws, wsb);
 }
@@ -1585,13 +1722,16 @@ static int do_bwd_data(const Problem& p, hipStream_t st, const void* g, const vo
         if (dry) { ws = nullptr; wsb = bufs = 0; }  // (only the packing calls of the phases matter)
         else if (wsb < bufs || !ws) return PHX_ERR_WORKSPACE;
         char* base = static_cast<char*>(ws);
+        const int Z = phase_slices(p);
         g_name_prefix = "phase_";
         for (int a = 0; a < p.sh; ++a)
             for (int b = 0; b < p.sw; ++b) {
                 if (m.off[a * p.sw + b] < 0) continue;
                 const PhaseAxis ah = phase_axis(a, p.h, p.kh, p.dh, p.sh, p.pt), aw = phase_axis(b, p.w, p.kw, p.dw, p.sw, p.pl);
-                const int rc = run_corr(p, phase_corr(p, ah, aw), MAP_DGRAD, st, g, w, nullptr,
-                                        dry ? nullptr : base + m.off[a * p.sw + b] * esize, dry ? nullptr : base + bufs, wsb - bufs);
+                void* phase_out = dry ? nullptr : base + m.off[a * p.sw + b] * esize;
+                const int rc = Z ? run_sliced(p, Z, MAP_DGRAD, st, g, w, nullptr, phase_out, dry ? nullptr : base + bufs, wsb - bufs, &ah, &aw)
+                                 : run_corr(p, phase_corr(p, ah, aw), MAP_DGRAD, st, g, w, nullptr, phase_out, dry ? nullptr : base + bufs,
+                                            wsb - bufs);
                 if (rc != PHX_OK) { g_name_prefix = ""; return rc; }
             }
         g_name_prefix = "";
@@ -1600,6 +1740,7 @@ static int do_bwd_data(const Problem& p, hipStream_t st, const void* g, const vo
         PHX_HIP(hipGetLastError());
         return PHX_OK;
     }
+    if (const int Z = corr_slices(p, PHX_PASS_BWD_DATA)) return run_sliced(p, Z, MAP_DGRAD, st, g, w, nullptr, dx, ws, wsb);
     const Corr c = corr_dgrad(p);
     return run_corr(p, c, MAP_DGRAD, st, g, w, nullptr, dx, ws, wsb);
 }

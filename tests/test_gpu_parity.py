@@ -518,6 +518,63 @@ def test_windows_beyond_the_staging_limit(case, mode, dtype, policy):
     assert_close(dw.cpu().numpy(), want_dw, dtype, "wgrad " + names[2])
 
 
+SLICED = [
+    # name, n, ci, co, h, w, kh, kw, stride, dilation, padding, passes sliced by the default rule: fp32 (fwd, dgrad), fp16 (fwd, dgrad)
+    ("k3_128_7x7", 1, 128, 128, 7, 7, 3, 3, 1, 1, "SAME", (1, 1), (1, 1)),
+    ("k3_192_96_9x6", 2, 192, 96, 9, 6, 3, 3, 1, 1, "SAME", (1, 1), (1, 0)),            # 96 channels: two slices, fp32 arithmetic only
+    ("k3_dil2_160_64", 1, 160, 64, 10, 11, 3, 3, 1, 2, "SAME", (1, 1), (0, 0)),         # 160 = 2 x 80: no four slices of whole chunks
+    ("pw_512_64_8x8", 1, 512, 64, 8, 8, 1, 1, 1, 1, "VALID", (1, 0), (1, 0)),           # the pointwise streaming kernel
+    ("pw_256_96_7x7", 3, 256, 96, 7, 7, 1, 1, 1, 1, "VALID", (1, 0), (0, 0)),           # 16 steps: too few for four slices
+    ("k3_s2_128_14x14", 1, 128, 128, 14, 14, 3, 3, 2, 1, "SAME", (1, 1), (1, 1)),       # fp32: input gradient by phases, each sliced
+    ("pw_s2_128_512_14x14", 2, 128, 512, 14, 14, 1, 1, 2, 1, "VALID", (0, 1), (0, 1)),  # forward on a subsampled copy (unsliced), gradient by phases
+    ("k5x3_s21_128_96", 1, 128, 96, 12, 9, 5, 3, (2, 1), 1, (2, 1, 2, 1), (1, 1), (1, 0)),
+]
+
+
+@pytest.mark.parametrize("dtype,policy", [(torch.float32, "fp32"), (torch.float16, "full16"), (torch.float16, "backward32")],
+                         ids=["f32", "f16_full16", "f16_backward32"])
+@pytest.mark.parametrize("mode", [16, 8])
+@pytest.mark.parametrize("case", SLICED, ids=lambda c: c[0])
+def test_small_batches_cut_the_channel_reduction_into_slices(case, mode, dtype, policy, tune_env):
+    """The forward / input-gradient kernels give a workgroup an output tile and the whole reduction over channels and
+    taps: a small batch on a deep layer is a handful of long workgroups.  Such passes run as Z slices of the reduced
+    channels in one launch (a partial result tensor each, in the workspace) and a kernel that adds the partial
+    tensors and the bias.  Against the oracle, against the unsliced pass (PHX_TUNE_KSLICES=0), with another slice
+    count forced, with prepacked filters and with an addend on the input gradient."""
+    name, n, ci, co, h, w, kh, kw, stride, dilation, padding, sliced32, sliced16 = case
+    scale = 1.0 if dtype == torch.float32 else 0.5
+    g, x, wt, b, gr = make_inputs(name_seed(name) + 77, n, ci, co, h, w, kh, kw, stride, dilation, padding, dtype, scale)
+    desc = phx.Conv2DDescriptor(x.shape, wt.shape, stride, dilation, padding, use_bias=True, dtype=dtype, context=Ctx(mode, policy))
+    xd, wd, bd, gd = (torch.from_numpy(a).cuda() for a in (x, wt, b, gr))
+    x64, w64, b64, g64 = (a.astype(np.float64) for a in (x, wt, b, gr))
+    want_y = oracle.conv2d_fwd(g, x64, w64, b64, "hamilton")
+    _, want_dx = oracle.conv2d_bwd(g, x64, w64, g64, "hamilton")
+    addend = torch.from_numpy((scale * np.random.default_rng(5).standard_normal(x.shape)).astype(x.dtype)).cuda()
+    # (backward32: the input gradient runs in fp32 arithmetic on fp16 tensors)
+    expect = (bool(sliced32[0] if dtype == torch.float32 else sliced16[0]),
+              bool(sliced16[1] if policy == "full16" else sliced32[1]))
+    for setting in (None, "0", "2", "8"):
+        tune_env(PHX_TUNE_KSLICES=setting)
+        y = phx.conv2d_fwd(xd, wd, bd, desc)
+        k_fwd = capi.last_kernel_name()
+        dx = ops.conv2d_bwd_data(wd, gd, desc)
+        k_dx = capi.last_kernel_name()
+        if setting is None:
+            assert ("_kslices" in k_fwd, "_kslices" in k_dx) == expect, (k_fwd, k_dx)
+        elif setting == "0":
+            assert "_kslices" not in k_fwd and "_kslices" not in k_dx, (k_fwd, k_dx)
+        assert_close(y.cpu().numpy(), want_y, dtype, "fwd %s %s" % (setting, k_fwd))
+        assert_close(dx.cpu().numpy(), want_dx, dtype, "dgrad %s %s" % (setting, k_dx))
+        with_addend = ops.conv2d_bwd_data(wd, gd, desc, addend=addend)
+        assert_close(with_addend.cpu().numpy(), want_dx + addend.cpu().numpy().astype(np.float64), dtype, "dgrad + addend %s" % setting)
+        packed = ops.conv2d_pack_filters(wd, desc)
+        if packed is not None:
+            zero = torch.zeros_like(wd)
+            if ops.conv2d_packed_filter_bytes(desc, capi.PHX_PASS_FWD):
+                assert torch.equal(phx.conv2d_fwd(xd, zero, bd, desc, packed=packed), y), "prepacked fwd %s" % setting
+            assert torch.equal(ops.conv2d_bwd_data(zero, gd, desc, packed=packed), dx), "prepacked dgrad %s" % setting
+
+
 DIRECT_CASES = ("pw_ragged", "k3_same", "k3_ragged", "k3_s2", "pw_s31", "k7_s2", "k5_s2_valid", "k3_dil2", "k32_asym", "k7_s2_dil2")
 
 
