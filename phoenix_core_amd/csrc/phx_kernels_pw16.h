@@ -456,7 +456,8 @@ __global__ void __launch_bounds__(WG_THREADS, 2) qconv_pwx_f16_kernel(const PwxA
 // Requirements (host): channel counts and channel strides multiples of 8.
 // ---------------------------------------------------------------------------------------------
 template <int WCO>
-__global__ void __launch_bounds__(WG_THREADS, 2) qconv_pwx_nhwc_f16_kernel(const PwxArgs P) {
+__global__ void __launch_bounds__(WG_THREADS, 2) qconv_pwx_nhwc_f16_kernel(const PwxArgs P0) {
+    const PwxArgs P = group_view(P0);  // (grid rows: the reduction slices of a sliced pass)
     using S = PwxShape<WCO>;
     constexpr int WPX = S::WPX, WV = S::WV, SV = S::SV, R = S::R, D = R - 1;
     constexpr int PXT = 64 * WPX;     // pixels per workgroup tile

@@ -29,7 +29,7 @@ template <int WCO>
 static int launch_pwx_nhwc_one(const PwxArgs& a, int blocks, hipStream_t st) {
     constexpr auto kernel = qconv_pwx_nhwc_f16_kernel<WCO>;
     if (!BigLds<kernel>::registered) return -1;
-    hipLaunchKernelGGL(kernel, dim3(blocks), dim3(WG_THREADS), PwxShape<WCO>::lds_bytes, st, a);
+    hipLaunchKernelGGL(kernel, dim3(blocks, grid_rows(a.groups)), dim3(WG_THREADS), PwxShape<WCO>::lds_bytes, st, a);
     return 0;
 }
 

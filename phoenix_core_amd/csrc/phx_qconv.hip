@@ -907,38 +907,80 @@ static bool nhwc_native(const Problem& p, int pass) {
            (long)p.n * p.h * p.w < (1L << 30) && !tune().nopwx;
 }
 
+// Reduction slices of a channels-last pointwise pass (see corr_slices for the idea): few work items and a long
+// reduction -- Dense layers on a few hundred rows, deep pointwise layers on small batches -- run as Z slices of the
+// reduced channels in one launch and a pass that adds the partial tensors.  Z = the largest power of two that keeps at
+// least 32 channels (a multiple of 16) and 8 steps of 16 channels per slice and at most one item per CU; at least 4.
+static int nhwc_slices(const Problem& p, int map) {
+    if (tune().kslices == 0) return 0;
+    const int cin = map == MAP_FWD ? p.ci : p.co, cout = map == MAP_FWD ? p.co : p.ci;
+    const auto fits = [&](int z) { return cin % z == 0 && (cin / z) % 16 == 0 && cin / z >= 32; };
+    if (tune().kslices > 1) return fits(tune().kslices) ? tune().kslices : 0;
+    const int wco = pwx_wco(cout);
+    const long items = (long)cdiv((int)((long)p.n * p.h * p.w), 64 * (4 / wco)) * cdiv(cout, 32 * wco);
+    const int steps = cdiv(cin, 16);
+    int Z = 1;
+    while (fits(2 * Z) && items * 2 * Z <= 256 && steps / (2 * Z) >= 8) Z *= 2;
+    return Z >= 4 ? Z : 0;
+}
+
 static size_t nhwc_native_workspace(const Problem& p, int pass) {
+    const int map = pass == PHX_PASS_FWD ? MAP_FWD : MAP_DGRAD;
     const int cin = pass == PHX_PASS_FWD ? p.ci : p.co, cout = pass == PHX_PASS_FWD ? p.co : p.ci;
     const int wco = pwx_wco(cout);
+    if (const int Z = nhwc_slices(p, map))  // Z partial result tensors, then Z packed images
+        return align_up((size_t)Z * 4 * p.n * p.h * p.w * cout * 2, 256) +
+               (size_t)Z * align_up(pwx_packed_bytes(wco, cdiv(cout, 32 * wco), cdiv(cin / Z, 16)), 256);
     return align_up(pwx_packed_bytes(wco, cdiv(cout, 32 * wco), cdiv(cin, 16)), 256);
 }
 
 static int run_pwx_nhwc(const Problem& p, int map, hipStream_t st, const void* in, const void* w, const void* bias, void* out,
                         void* ws, size_t ws_bytes) {
-    if (!g_pack.dry() && (!in || !w || !out)) return PHX_ERR_INVALID_ARGUMENT;
-    const int cin = map == MAP_FWD ? p.ci : p.co, cout = map == MAP_FWD ? p.co : p.ci;
+    const bool dry = g_pack.dry();
+    if (!dry && (!in || !w || !out)) return PHX_ERR_INVALID_ARGUMENT;
+    const int Z = nhwc_slices(p, map), slices = Z ? Z : 1;
+    const int cin_all = map == MAP_FWD ? p.ci : p.co, cin = cin_all / slices, cout = map == MAP_FWD ? p.co : p.ci;
     const int wco = pwx_wco(cout), co_tiles = cdiv(cout, 32 * wco), nsteps = cdiv(cin, 16);
-    const PackSlot slot = pack_slot(ws, ws_bytes, pwx_packed_bytes(wco, co_tiles, nsteps));
+    const long np = (long)p.n * p.h * p.w;
+    // sliced: the partial tensors lie at the front of the workspace, the packed images of the slices behind them
+    const long count = 4L * np * cout;
+    const size_t partial_bytes = Z ? align_up((size_t)Z * count * 2, 256) : 0;
+    char* partial = static_cast<char*>(ws);
+    if (Z && !dry) {
+        if (ws_bytes < partial_bytes || !ws) return PHX_ERR_WORKSPACE;
+        ws = partial + partial_bytes; ws_bytes -= partial_bytes;
+    }
+    const size_t image = align_up(pwx_packed_bytes(wco, co_tiles, nsteps), 256);
+    const PackSlot slot = pack_slot(ws, ws_bytes, Z ? image * Z : pwx_packed_bytes(wco, co_tiles, nsteps));
     if (slot.rc != PHX_OK) return slot.rc;
     ws = slot.dst;
+    // bytes from a slice's reduced channels to the next slice's in the filter: input channels forward, output channels backward
+    const long w_step = (long)cin * (map == MAP_FWD ? p.fs.si : p.fs.so) * 2;
     PackArgs pa{};
+    pa.groups = slices; pa.g_w = w_step; pa.g_out = (long)image;
     pa.w = w; pa.out = ws;
     pa.wcs = p.fs.wcs; pa.so = p.fs.so; pa.si = p.fs.si; pa.skh = p.fs.skh; pa.skw = p.fs.skw;
-    pa.Co = p.co; pa.Ci = p.ci; pa.Kh = 1; pa.Kw = 1; pa.khm = 0; pa.khs = 1; pa.kwm = 0; pa.kws = 1;
+    pa.Co = map == MAP_FWD ? p.co : cin; pa.Ci = map == MAP_FWD ? cin : p.ci; pa.Kh = 1; pa.Kw = 1; pa.khm = 0; pa.khs = 1; pa.kwm = 0; pa.kws = 1;
     pa.rows = cout; pa.red = cin; pa.row_tiles = co_tiles; pa.nchunks = nsteps;
     if (slot.pack_now && launch_pack_filters_pwx(map, wco, nsteps, pa, st) != 0) return PHX_ERR_NOT_SUPPORTED;
-    if (const int rrc = record_pwx_job(pa, map, wco, nsteps)) return rrc;
+    for (int z = 0; z < slices; ++z) {  // (the combined packing launch takes one job per image)
+        PackArgs one = pa;
+        one.groups = 1;
+        one.w = at_bytes(pa.w, z * w_step);
+        one.out = at_bytes(pa.out, z * image);
+        if (const int rrc = record_pwx_job(one, map, wco, nsteps)) return rrc;
+    }
     if (!slot.compute) return PHX_OK;
     DeviceState* dev = nullptr;
     if (const int rc = device_state(&dev)) return rc;
     PwxArgs a{};
-    const long np = (long)p.n * p.h * p.w;
-    a.in = static_cast<const _Float16*>(in); a.in_cs = np * cin;
-    a.wpk = static_cast<const f16x8*>(ws); a.bias = static_cast<const _Float16*>(bias);
-    a.out = static_cast<_Float16*>(out); a.out_cs = np * cout;
-    a.N = p.n; a.Cin = cin; a.CinS = cin; a.Cout = cout; a.CoutS = cout; a.HW = p.h * p.w; a.NP = (int)np;
+    a.in = static_cast<const _Float16*>(in); a.in_cs = np * cin_all;
+    a.wpk = static_cast<const f16x8*>(ws); a.bias = Z ? nullptr : static_cast<const _Float16*>(bias);
+    a.out = Z ? reinterpret_cast<_Float16*>(partial) : static_cast<_Float16*>(out); a.out_cs = np * cout;
+    a.N = p.n; a.Cin = cin; a.CinS = cin_all; a.Cout = cout; a.CoutS = cout; a.HW = p.h * p.w; a.NP = (int)np;
     a.co_tiles = co_tiles; a.nsteps = nsteps;
     a.items = cdiv((int)np, 64 * (4 / wco)) * co_tiles;
+    a.groups = slices; a.g_in = (long)cin * 2; a.g_w = (long)image; a.g_bias = 0; a.g_out = count * 2;
     const int blocks = std::min(a.items, 2 * dev->cu_count);
     int rc;
     {
@@ -947,8 +989,15 @@ static int run_pwx_nhwc(const Problem& p, int map, hipStream_t st, const void* i
     }
     if (rc != 0) return PHX_ERR_NOT_SUPPORTED;
     PHX_HIP(hipGetLastError());
+    if (Z) {
+        const bool add = map == MAP_DGRAD && g_addend.dx == out && g_addend.ptr && !g_addend.fused;
+        launch_slice_sum(true, partial, Z, count, out, bias, add ? g_addend.ptr : nullptr, 1, cout, count / 4, st);
+        PHX_HIP(hipGetLastError());
+        if (add) g_addend.fused = true;
+    }
     snprintf(g_name_buf, sizeof(g_name_buf), "qconv_%s_f16mfmapwxcl_p16_f16_wco%d_px%d_k%d_wgs%d", map == MAP_FWD ? "fwd" : "dgrad",
              wco, 64 * (4 / wco), nsteps, blocks);
+    if (Z) snprintf(g_name_buf + strlen(g_name_buf), sizeof(g_name_buf) - strlen(g_name_buf), "_kslices%d", Z);
     g_last_kernel = g_name_buf;
     say(p, map == MAP_FWD ? "forward (channels-last)" : "input gradient (channels-last)");
     return PHX_OK;

@@ -575,6 +575,47 @@ def test_small_batches_cut_the_channel_reduction_into_slices(case, mode, dtype, 
             assert torch.equal(ops.conv2d_bwd_data(zero, gd, desc, packed=packed), dx), "prepacked dgrad %s" % setting
 
 
+@pytest.mark.parametrize("forced", [None, "2", "16"], ids=["rule", "z2", "z16"])
+@pytest.mark.parametrize("shape", [(1, 512, 64, 8, 8), (3, 256, 136, 5, 7), (2, 1024, 32, 4, 4)], ids=lambda s: "n%d_%dto%d_%dx%d" % s)
+def test_channels_last_pointwise_passes_are_sliced_too(shape, forced, tune_env):
+    """The channels-last pointwise kernel (fp16 matrix cores, channel counts multiples of 8) runs few-item passes in
+    reduction slices as well: the slices are grid rows reading their channels of every pixel.  Oracle, unsliced
+    pass, prepacked filters, addend."""
+    n, ci, co, h, w = shape
+    dtype = torch.float16
+    g, x, wt, b, gr = make_inputs(n * ci + co, n, ci, co, h, w, 1, 1, 1, 1, "VALID", dtype, 0.5)
+    x_dev = np.ascontiguousarray(x.transpose(0, 2, 3, 1))
+    g_dev = np.ascontiguousarray(gr.transpose(0, 2, 3, 1))
+    w_dev = np.ascontiguousarray(wt.transpose(0, 1, 3, 4, 2))
+    desc = phx.Conv2DDescriptor(x_dev.shape, w_dev.shape, 1, 1, "VALID", use_bias=True, dtype=dtype, filter_layout="OHWI",
+                                context=Ctx(8, "full16"), data_format="NHWC")
+    xd, wd, bd, gd = (torch.from_numpy(a).cuda() for a in (x_dev, w_dev, b, g_dev))
+    addend = torch.from_numpy((0.5 * np.random.default_rng(6).standard_normal(x_dev.shape)).astype(np.float16)).cuda()
+    x64, w64, b64, g64 = (a.astype(np.float64) for a in (x, wt, b, gr))
+    want_y = oracle.conv2d_fwd(g, x64, w64, b64, "hamilton")
+    _, want_dx = oracle.conv2d_bwd(g, x64, w64, g64, "hamilton")
+    for setting in (forced, "0"):
+        tune_env(PHX_TUNE_KSLICES=setting)
+        y = phx.conv2d_fwd(xd, wd, bd, desc)
+        k_fwd = capi.last_kernel_name()
+        dx = ops.conv2d_bwd_data(wd, gd, desc)
+        k_dx = capi.last_kernel_name()
+        assert "pwxcl" in k_fwd and "pwxcl" in k_dx, (k_fwd, k_dx)
+        # by the rule the forward passes that reduce over 512 channels and more are sliced; forced counts wherever they divide
+        want_sliced = (ci >= 512, False) if setting is None else (setting != "0" and ci % (16 * int(setting)) == 0 and ci // int(setting) >= 32,
+                                                                        setting != "0" and co % (16 * int(setting)) == 0 and co // int(setting) >= 32)
+        assert ("_kslices" in k_fwd, "_kslices" in k_dx) == want_sliced, (setting, k_fwd, k_dx)
+        assert_close(y.cpu().numpy().transpose(0, 3, 1, 2), want_y, dtype, "fwd " + k_fwd)
+        assert_close(dx.cpu().numpy().transpose(0, 3, 1, 2), want_dx, dtype, "dgrad " + k_dx)
+        with_addend = ops.conv2d_bwd_data(wd, gd, desc, addend=addend)
+        assert_close(with_addend.cpu().numpy().transpose(0, 3, 1, 2), want_dx + addend.cpu().numpy().astype(np.float64).transpose(0, 3, 1, 2),
+                     dtype, "dgrad + addend")
+        packed = ops.conv2d_pack_filters(wd, desc)
+        zero = torch.zeros_like(wd)
+        assert torch.equal(phx.conv2d_fwd(xd, zero, bd, desc, packed=packed), y), "prepacked fwd"
+        assert torch.equal(ops.conv2d_bwd_data(zero, gd, desc, packed=packed), dx), "prepacked dgrad"
+
+
 DIRECT_CASES = ("pw_ragged", "k3_same", "k3_ragged", "k3_s2", "pw_s31", "k7_s2", "k5_s2_valid", "k3_dil2", "k32_asym", "k7_s2_dil2")
 
 
@@ -1171,7 +1212,8 @@ def test_dense_fp16(mode, policy, kernels, tune_env):
 
 @pytest.mark.parametrize("layout", ["IO", "OI"])
 @pytest.mark.parametrize("policy", ["full16", "backward32"])
-@pytest.mark.parametrize("shape", [(3000, 128, 72), (8192, 64, 64), (177, 512, 256), (1024, 96, 250), (1024, 64, 64)], ids=lambda s: "n%d_%dto%d" % s)
+@pytest.mark.parametrize("shape", [(3000, 128, 72), (8192, 64, 64), (177, 512, 256), (1024, 96, 250), (1024, 64, 64), (64, 1024, 512), (40, 2048, 264)],
+                         ids=lambda s: "n%d_%dto%d" % s)
 def test_larger_dense_runs_as_a_channels_last_pointwise_convolution(shape, policy, layout, tune_env):
     """A Dense layer's tensors [4n, units] are those of a channels-last pointwise convolution on one image of n x 1
     positions (denseFwd / denseBwd, src/upstride.hpp:53-86): beyond the sizes of the FMA kernels, fp16 problems whose
@@ -1198,6 +1240,9 @@ def test_larger_dense_runs_as_a_channels_last_pointwise_convolution(shape, polic
         # gradient of a batch beyond 128 rows moves to the matrix cores: the last shape)
         eligible = direct and no % 8 == 0 and n * ni * no > 16 << 20
         assert ("pwxcl" in k_fwd) == eligible and ("pwxcl" in k_dx) == (eligible and policy == "full16"), (k_fwd, k_dx)
+        # (few rows and a long reduction: the forward pass runs in reduction slices)
+        if direct and n <= 64:
+            assert "_kslices" in k_fwd, k_fwd
         got[direct] = (y, dx, dw)
     x64, w64, b64, g64 = (a.astype(np.float64) for a in (x, w, b, gr))
     want_y = oracle.dense_fwd(x64, w64, b64, "generic")
