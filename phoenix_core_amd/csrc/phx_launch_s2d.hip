@@ -148,8 +148,9 @@ int launch_add_inplace(bool half_storage, void* dst, const void* src, long count
 }
 
 // dst = sum of `slices` tensors of `count` elements each lying `count` elements apart (+ bias per channel: element e
-// belongs to channel (e / plane) % channels of component e / comp_count; + addend, element by element): what closes a
-// forward / input-gradient pass whose reduction over the channels was cut into slices.  fp32 sums, one rounding.
+// belongs to channel (e / plane) % channels of component e / comp_count; then + addend, element by element, in the storage
+// type): what closes a forward / input-gradient pass whose reduction over the channels was cut into slices.  fp32 sums,
+// one rounding.
 template <typename TS>
 __global__ void __launch_bounds__(WG_THREADS) slice_sum_kernel(const TS* partial, int slices, long count, TS* dst, const TS* bias,
                                                                const TS* addend, int plane, int channels, long comp_count) {
@@ -158,8 +159,9 @@ __global__ void __launch_bounds__(WG_THREADS) slice_sum_kernel(const TS* partial
         float acc = 0.0f;
         for (int z = 0; z < slices; ++z) acc += (float)partial[z * count + e];
         if (bias) acc += (float)bias[(e / comp_count) * channels + (e / plane) % channels];
-        if (addend) acc += (float)addend[e];
-        dst[e] = (TS)acc;
+        TS r = (TS)acc;
+        if (addend) r = (TS)((float)r + (float)addend[e]);  // (as the separate in-place pass would: the rounded result plus the addend)
+        dst[e] = r;
     }
 }
 
