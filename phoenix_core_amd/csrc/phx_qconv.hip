@@ -1651,7 +1651,12 @@ static size_t workspace_for(const Problem& p, int pass) {
     if (pass != PHX_PASS_BWD_DATA && s2d_view(p, v)) return v.x2_bytes + v.w2_bytes + workspace_plain(v.q, pass);
     Problem q;
     size_t xs_bytes = 0;
-    if (pass != PHX_PASS_BWD_DATA && subsample_view(p, q, xs_bytes)) return xs_bytes + workspace_plain(q, pass);
+    if (pass != PHX_PASS_BWD_DATA && subsample_view(p, q, xs_bytes)) {
+        const int Z = pass == PHX_PASS_FWD ? corr_slices(q, pass) : 0;  // (the unit-stride problem on the subsampled copy is sliced like any other)
+        if (!Z) return xs_bytes + workspace_plain(q, pass);
+        const SlicedCorr sc(q, pass, Z);
+        return xs_bytes + sc.partial_bytes + (size_t)Z * workspace_plain(sc.q, pass);
+    }
     if (const int Z = corr_slices(p, pass)) {
         const SlicedCorr sc(p, pass, Z);
         return sc.partial_bytes + (size_t)Z * workspace_plain(sc.q, pass);
@@ -1741,8 +1746,10 @@ static int do_fwd(const Problem& p, hipStream_t st, const void* x, const void* w
             PHX_HIP(hipGetLastError());
         }
         g_name_prefix = "sub_";
-        const int rc = run_corr(q, corr_forward(q), MAP_FWD, st, ws, w, b, y, dry ? nullptr : static_cast<char*>(ws) + xs_bytes,
-                                dry ? 0 : wsb - xs_bytes);
+        void* rest = dry ? nullptr : static_cast<char*>(ws) + xs_bytes;
+        const int Z = corr_slices(q, PHX_PASS_FWD);
+        const int rc = Z ? run_sliced(q, Z, MAP_FWD, st, ws, w, b, y, rest, dry ? 0 : wsb - xs_bytes)
+                         : run_corr(q, corr_forward(q), MAP_FWD, st, ws, w, b, y, rest, dry ? 0 : wsb - xs_bytes);
         g_name_prefix = "";
         return rc;
     }

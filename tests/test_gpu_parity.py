@@ -528,6 +528,7 @@ SLICED = [
     ("k3_s2_128_14x14", 1, 128, 128, 14, 14, 3, 3, 2, 1, "SAME", (1, 1), (1, 1)),       # fp32: input gradient by phases, each sliced
     ("pw_s2_128_512_14x14", 2, 128, 512, 14, 14, 1, 1, 2, 1, "VALID", (0, 1), (0, 1)),  # forward on a subsampled copy (unsliced), gradient by phases
     ("k5x3_s21_128_96", 1, 128, 96, 12, 9, 5, 3, (2, 1), 1, (2, 1, 2, 1), (1, 1), (1, 0)),
+    ("pw_s2_512_96_14x14", 1, 512, 96, 14, 14, 1, 1, 2, 1, "VALID", (1, 0), (1, 0)),      # the forward pass on the subsampled copy, sliced
 ]
 
 
