@@ -1591,9 +1591,13 @@ static int slices_rule(const Problem& p, int pass, const Corr& creal) {
     return Z >= (f16 ? 4 : 2) ? Z : 0;
 }
 
+static bool nhwc_window_native(const Problem& p, int pass);
 static int corr_slices(const Problem& p, int pass) {
     if (tune().kslices == 0 || pass == PHX_PASS_BWD_WEIGHTS || is_empty(p)) return 0;
-    if (channel_slices(p) || p.nhwc || p.real_input || g_batch.n > 1 || g_window_cl) return 0;
+    if (channel_slices(p) || p.real_input || g_batch.n > 1 || g_window_cl) return 0;
+    // (channels-last tensors: a call that goes through channels-first copies is sliced on those; one that runs on the
+    // caller's tensors is not -- nhwc_window_native leaves the passes that would be sliced to the copies)
+    if (p.nhwc && nhwc_window_native(p, pass)) return 0;
     if (pass == PHX_PASS_BWD_DATA && dgrad_by_phases(p)) return 0;  // (see phase_slices)
     if (pass == PHX_PASS_FWD) {
         S2dView v;
@@ -1607,7 +1611,7 @@ static int corr_slices(const Problem& p, int pass) {
 // A strided input gradient that runs by phases (dgrad_by_phases): every phase is a pass of its own and is sliced like
 // one, all by the Z that the rule gives for the phase with the most taps.
 static int phase_slices(const Problem& p) {
-    if (tune().kslices == 0 || !dgrad_by_phases(p) || p.nhwc || g_batch.n > 1 || g_window_cl) return 0;
+    if (tune().kslices == 0 || !dgrad_by_phases(p) || g_batch.n > 1 || g_window_cl) return 0;
     PhaseAxis bh{}, bw{};
     for (int a = 0; a < p.sh; ++a)
         for (int b = 0; b < p.sw; ++b) {
@@ -1974,6 +1978,7 @@ struct ChannelsLast {
 // saves cost in proportion to the tensors, not to the arithmetic.  Calls whose arithmetic per tensor byte
 // (channels x taps) is beyond what was measured to pay (256 channels, 3x3) keep the transposes;
 // PHX_TUNE_WINCL_MAX moves that bound, PHX_TUNE_NOWINCL switches the direct form off.
+namespace phx {
 static bool nhwc_window_native(const Problem& p, int pass) {
     if (!p.nhwc || (pass != PHX_PASS_FWD && pass != PHX_PASS_BWD_DATA) || is_empty(p) || is_pointwise_unit(p)) return false;
     if (p.real_input || p.groups != 1 || tune().nowincl || !use_f16_mfma(p, pass)) return false;
@@ -1989,8 +1994,14 @@ static bool nhwc_window_native(const Problem& p, int pass) {
     FwdPlan pl;
     int pw = 0;
     if (!plan_corr(pass == PHX_PASS_FWD ? corr_forward(p) : corr_dgrad(p), p.mode, true, c, pl, pw)) return false;
-    return pl.lds_filters && pl.chunks && !pl.pwx && pw == 0;
+    if (!(pl.lds_filters && pl.chunks && !pl.pwx && pw == 0)) return false;
+    // a small batch on a deep layer gains more from reduction slices (corr_slices), which run on channels-first copies:
+    // the copies of so small a problem cost next to nothing
+    Problem planes = p;
+    planes.nhwc = false;
+    return corr_slices(planes, pass) == 0;
 }
+}  // namespace phx
 
 // The filter gradient of a channels-last call runs on the caller's tensors where its plan is the fp16 kernel with
 // 64x64 channel tiles, unit stride and one or three taps per workgroup (more than 32 channels on either side): that

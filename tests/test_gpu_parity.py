@@ -614,6 +614,36 @@ def test_channels_last_pointwise_passes_are_sliced_too(shape, forced, tune_env):
         assert torch.equal(ops.conv2d_bwd_data(zero, gd, desc, packed=packed), dx), "prepacked dgrad"
 
 
+@pytest.mark.parametrize("dtype,policy", [(torch.float32, "fp32"), (torch.float16, "full16")], ids=["f32", "f16_full16"])
+@pytest.mark.parametrize("case", [c for c in SLICED if c[0] in ("k3_128_7x7", "k3_s2_128_14x14", "pw_256_96_7x7")], ids=lambda c: c[0])
+def test_small_channels_last_batches_are_sliced_on_their_channels_first_copies(case, dtype, policy, tune_env):
+    """Channels-last calls that go through channels-first copies (fp32 arithmetic, strides) run their passes in reduction
+    slices on those copies; the multi-tap fp16 passes that would otherwise run on the caller's tensors do the same
+    where the slices apply (the copies of so small a problem cost next to nothing)."""
+    name, n, ci, co, h, w, kh, kw, stride, dilation, padding, sliced32, sliced16 = case
+    scale = 1.0 if dtype == torch.float32 else 0.5
+    g, x, wt, b, gr = make_inputs(name_seed(name) + 78, n, ci, co, h, w, kh, kw, stride, dilation, padding, dtype, scale)
+    x_dev = np.ascontiguousarray(x.transpose(0, 2, 3, 1))
+    g_dev = np.ascontiguousarray(gr.transpose(0, 2, 3, 1))
+    desc = phx.Conv2DDescriptor(x_dev.shape, wt.shape, stride, dilation, padding, use_bias=True, dtype=dtype, context=Ctx(8, policy),
+                                data_format="NHWC")
+    xd, wd, bd, gd = (torch.from_numpy(a).cuda() for a in (x_dev, wt, b, g_dev))
+    x64, w64, b64, g64 = (a.astype(np.float64) for a in (x, wt, b, gr))
+    want_y = oracle.conv2d_fwd(g, x64, w64, b64, "hamilton")
+    _, want_dx = oracle.conv2d_bwd(g, x64, w64, g64, "hamilton")
+    expect = tuple(bool(e) for e in (sliced32 if dtype == torch.float32 else sliced16))
+    for setting in (None, "0"):
+        tune_env(PHX_TUNE_KSLICES=setting)
+        y = phx.conv2d_fwd(xd, wd, bd, desc)
+        k_fwd = capi.last_kernel_name()
+        dx = ops.conv2d_bwd_data(wd, gd, desc)
+        k_dx = capi.last_kernel_name()
+        if name != "pw_256_96_7x7" or dtype == torch.float32:  # (the fp16 pointwise case runs on the channels-last pointwise kernel, by its own rule)
+            assert ("_kslices" in k_fwd, "_kslices" in k_dx) == (expect if setting is None else (False, False)), (k_fwd, k_dx)
+        assert_close(y.cpu().numpy().transpose(0, 3, 1, 2), want_y, dtype, "fwd " + k_fwd)
+        assert_close(dx.cpu().numpy().transpose(0, 3, 1, 2), want_dx, dtype, "dgrad " + k_dx)
+
+
 DIRECT_CASES = ("pw_ragged", "k3_same", "k3_ragged", "k3_s2", "pw_s31", "k7_s2", "k5_s2_valid", "k3_dil2", "k32_asym", "k7_s2_dil2")
 
 
@@ -1029,7 +1059,8 @@ def test_channels_last_windows_run_on_the_tensors_as_they_are(case, mode, tune_e
     want_dw, want_dx = oracle.conv2d_bwd(g, x64, w64, g64, "hamilton")
     got = {}
     for variant in ("direct", "transposed"):
-        tune_env(PHX_TUNE_NOWINCL=None if variant == "direct" else "1")
+        # (KSLICES=0: the test's small batches would otherwise run in reduction slices on channels-first copies)
+        tune_env(PHX_TUNE_NOWINCL=None if variant == "direct" else "1", PHX_TUNE_KSLICES="0")
         ws = [desc.workspace_bytes(p) for p in range(3)]
         y = phx.conv2d_fwd(xd, wd, bd, desc)
         k_fwd = capi.last_kernel_name()
@@ -1076,7 +1107,7 @@ def test_channels_last_strided_forward_runs_on_the_tensors_as_they_are(case, mod
     want_dw, want_dx = oracle.conv2d_bwd(g, x64, w64, g64, "hamilton")
     ys, names = [], []
     for variant in ("direct", "transposed"):
-        tune_env(PHX_TUNE_NOWINCL=None if variant == "direct" else "1")
+        tune_env(PHX_TUNE_NOWINCL=None if variant == "direct" else "1", PHX_TUNE_KSLICES="0")  # (see above)
         y = phx.conv2d_fwd(xd, wd, bd, desc)
         names.append(capi.last_kernel_name())
         dw, dx = phx.conv2d_bwd(xd, wd, gd, desc)
