@@ -21,11 +21,14 @@ def Ctx(mode, policy):
     return phx.Context(env)
 
 
+# (the second shape is a small batch on a deep layer: forward and input gradient run in reduction slices, partial
+# tensors in the workspace and the pass that adds them inside the graph)
+@pytest.mark.parametrize("shape", [(4, 32, 64, 14), (1, 256, 128, 7)], ids=lambda s: "n%d_%dto%d_%dx%d" % (s + s[-1:]))
 @pytest.mark.parametrize("dtype,policy", [(torch.float16, "full16"), (torch.float32, "fp32")], ids=["f16", "f32"])
-def test_captured_conv_replays_match_eager(dtype, policy):
+def test_captured_conv_replays_match_eager(dtype, policy, shape):
     capi.init()
     torch.manual_seed(11)
-    n, ci, co, h = 4, 32, 64, 14
+    n, ci, co, h = shape
     scale = 1.0 if dtype == torch.float32 else 0.5
     x = (scale * torch.randn(4 * n, ci, h, h, device="cuda")).to(dtype)
     w = (scale * torch.randn(4, co, ci, 3, 3, device="cuda") * (2.0 / (9 * ci)) ** 0.5).to(dtype)
@@ -36,6 +39,7 @@ def test_captured_conv_replays_match_eager(dtype, policy):
         ops.reserve_workspace(max(desc.workspace_bytes(p) for p in range(3)))
         # eager reference and warm-up on the capture stream (fills the plan cache, sizes the scratch buffer)
         y0 = phx.conv2d_fwd(x, w, None, desc)
+        assert ("_kslices" in capi.last_kernel_name()) == (n == 1)
         dw0, dx0 = phx.conv2d_bwd(x, w, g, desc)
     side.synchronize()
     graph = torch.cuda.CUDAGraph()
