@@ -1567,8 +1567,9 @@ static void subsample_input(const Problem& p, const void* x, void* xs, hipStream
 // filter and writes a partial result tensor of its own in the workspace), and a streaming kernel adds the partial
 // tensors (and the bias) into the caller's tensor, in fp32 with one rounding.
 // Z = the largest power of two that keeps at least 32 channels (a multiple of 16) and 8 reduction steps per slice
-// and at most two workgroups per CU in flight; 0 = the pass runs unsliced (enough workgroups already, or a rewritten
-// problem: groups, channels-last, real-valued input, space-to-depth, subsampling, phases).
+// and at most two workgroups per CU in flight; 0 = the pass runs unsliced (enough workgroups already; groups and
+// real-valued input are never sliced).  The unit-stride problem on a subsampled copy (strided pointwise forward) and
+// the phases of a strided input gradient are passes of their own and sliced as such (do_fwd, phase_slices).
 static int slices_rule(const Problem& p, int pass, const Corr& creal) {
     Corr c;
     FwdPlan pl;
