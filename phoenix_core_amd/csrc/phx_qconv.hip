@@ -1587,8 +1587,11 @@ static int slices_rule(const Problem& p, int pass, const Corr& creal) {
     const long most = pl.pwx ? cus : 2L * cus;
     int Z = 1;
     while (fits(2 * Z) && wgs * 2 * Z <= most && steps / (2 * Z) >= 8) Z *= 2;
-    // (two slices do not pay for the extra pass over the result on the fp16 matrix cores: 256 -> 256 3x3 at 14x14, N=16
-    // 107 -> 115 us; in fp32 arithmetic they do: 570 -> 410)
+    // (on the fp16 matrix cores two slices pay for the extra pass over the result only where the unsliced pass leaves
+    // half of the CUs without a workgroup: 64 -> 64 3x3 at 14x14, N=32, 128 workgroups 27 -> 23 us, at 56x56, N=1
+    // 31 -> 24; but 256 -> 256 at 14x14, N=16, 256 workgroups 107 -> 115, 64 -> 64 at 56x56, N=4, 200 workgroups
+    // 35 -> 43; in fp32 arithmetic they always do: 570 -> 410)
+    if (f16 && !pl.pwx && Z == 2 && wgs <= cus / 2) return 2;
     return Z >= (f16 ? 4 : 2) ? Z : 0;
 }
 

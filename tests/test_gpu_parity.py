@@ -521,13 +521,13 @@ def test_windows_beyond_the_staging_limit(case, mode, dtype, policy):
 SLICED = [
     # name, n, ci, co, h, w, kh, kw, stride, dilation, padding, passes sliced by the default rule: fp32 (fwd, dgrad), fp16 (fwd, dgrad)
     ("k3_128_7x7", 1, 128, 128, 7, 7, 3, 3, 1, 1, "SAME", (1, 1), (1, 1)),
-    ("k3_192_96_9x6", 2, 192, 96, 9, 6, 3, 3, 1, 1, "SAME", (1, 1), (1, 0)),            # 96 channels: two slices, fp32 arithmetic only
-    ("k3_dil2_160_64", 1, 160, 64, 10, 11, 3, 3, 1, 2, "SAME", (1, 1), (0, 0)),         # 160 = 2 x 80: no four slices of whole chunks
+    ("k3_192_96_9x6", 2, 192, 96, 9, 6, 3, 3, 1, 1, "SAME", (1, 1), (1, 1)),            # 96 channels: two slices (fp16: few workgroups)
+    ("k3_dil2_160_64", 1, 160, 64, 10, 11, 3, 3, 1, 2, "SAME", (1, 1), (1, 1)),         # 160 = 2 x 80: two slices of whole chunks
     ("pw_512_64_8x8", 1, 512, 64, 8, 8, 1, 1, 1, 1, "VALID", (1, 0), (1, 0)),           # the pointwise streaming kernel
-    ("pw_256_96_7x7", 3, 256, 96, 7, 7, 1, 1, 1, 1, "VALID", (1, 0), (0, 0)),           # 16 steps: too few for four slices
+    ("pw_256_96_7x7", 3, 256, 96, 7, 7, 1, 1, 1, 1, "VALID", (1, 0), (1, 0)),           # 16 steps: two slices
     ("k3_s2_128_14x14", 1, 128, 128, 14, 14, 3, 3, 2, 1, "SAME", (1, 1), (1, 1)),       # fp32: input gradient by phases, each sliced
     ("pw_s2_128_512_14x14", 2, 128, 512, 14, 14, 1, 1, 2, 1, "VALID", (0, 1), (0, 1)),  # forward on a subsampled copy (unsliced), gradient by phases
-    ("k5x3_s21_128_96", 1, 128, 96, 12, 9, 5, 3, (2, 1), 1, (2, 1, 2, 1), (1, 1), (1, 0)),
+    ("k5x3_s21_128_96", 1, 128, 96, 12, 9, 5, 3, (2, 1), 1, (2, 1, 2, 1), (1, 1), (1, 1)),
     ("pw_s2_512_96_14x14", 1, 512, 96, 14, 14, 1, 1, 2, 1, "VALID", (1, 0), (1, 0)),      # the forward pass on the subsampled copy, sliced
 ]
 
