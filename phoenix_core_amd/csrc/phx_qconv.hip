@@ -901,6 +901,15 @@ static int pwx_wco(int cout) {
     return cout > 64 ? 4 : cout > 32 ? 2 : 1;
 }
 
+// The channels-last kernel reads a K step as 32 bytes of every pixel's channel vector, so the steps of a work item
+// come back to the same cache lines; with one output sub-tile the item is 256 pixels wide and the items in flight
+// on an XCD hold more lines than its L2 keeps (64 -> 16 channels at 56x56, N=64: 78 us, where 16 -> 64 takes 25).
+// From two K steps on, narrow outputs take the 128-pixel item of two sub-tiles, half of it empty rows: 39 us.
+static int pwx_wco_nhwc(int cin, int cout) {
+    const int wco = pwx_wco(cout);
+    return (wco == 1 && cin > 16 && !tune().tile_wco) ? 2 : wco;
+}
+
 static bool nhwc_native(const Problem& p, int pass) {
     return p.nhwc && (pass == PHX_PASS_FWD || pass == PHX_PASS_BWD_DATA) && is_pointwise_unit(p) && !is_empty(p) &&
            use_f16_mfma(p, pass) && !p.real_input && p.groups == 1 && p.ci % 8 == 0 && p.co % 8 == 0 &&
@@ -916,7 +925,7 @@ static int nhwc_slices(const Problem& p, int map) {
     const int cin = map == MAP_FWD ? p.ci : p.co, cout = map == MAP_FWD ? p.co : p.ci;
     const auto fits = [&](int z) { return cin % z == 0 && (cin / z) % 16 == 0 && cin / z >= 32; };
     if (tune().kslices > 1) return fits(tune().kslices) ? tune().kslices : 0;
-    const int wco = pwx_wco(cout);
+    const int wco = pwx_wco_nhwc(cin, cout);
     const long items = (long)cdiv((int)((long)p.n * p.h * p.w), 64 * (4 / wco)) * cdiv(cout, 32 * wco);
     const int steps = cdiv(cin, 16);
     int Z = 1;
@@ -927,7 +936,7 @@ static int nhwc_slices(const Problem& p, int map) {
 static size_t nhwc_native_workspace(const Problem& p, int pass) {
     const int map = pass == PHX_PASS_FWD ? MAP_FWD : MAP_DGRAD;
     const int cin = pass == PHX_PASS_FWD ? p.ci : p.co, cout = pass == PHX_PASS_FWD ? p.co : p.ci;
-    const int wco = pwx_wco(cout);
+    const int wco = pwx_wco_nhwc(cin, cout);
     if (const int Z = nhwc_slices(p, map))  // Z partial result tensors, then Z packed images
         return align_up((size_t)Z * 4 * p.n * p.h * p.w * cout * 2, 256) +
                (size_t)Z * align_up(pwx_packed_bytes(wco, cdiv(cout, 32 * wco), cdiv(cin / Z, 16)), 256);
@@ -940,7 +949,7 @@ static int run_pwx_nhwc(const Problem& p, int map, hipStream_t st, const void* i
     if (!dry && (!in || !w || !out)) return PHX_ERR_INVALID_ARGUMENT;
     const int Z = nhwc_slices(p, map), slices = Z ? Z : 1;
     const int cin_all = map == MAP_FWD ? p.ci : p.co, cin = cin_all / slices, cout = map == MAP_FWD ? p.co : p.ci;
-    const int wco = pwx_wco(cout), co_tiles = cdiv(cout, 32 * wco), nsteps = cdiv(cin, 16);
+    const int wco = pwx_wco_nhwc(cin_all, cout), co_tiles = cdiv(cout, 32 * wco), nsteps = cdiv(cin, 16);
     const long np = (long)p.n * p.h * p.w;
     // sliced: the partial tensors lie at the front of the workspace, the packed images of the slices behind them
     const long count = 4L * np * cout;
