@@ -52,6 +52,55 @@ __global__ void __launch_bounds__(WG_THREADS) s2d_input_kernel(const S2dArgs A) 
     }
 }
 
+// Dilation phases.  With unit stride, an output position and every input position it reads lie dh rows and dw columns
+// apart: they share their row modulo dh and their column modulo dw (where the padding before the image is a multiple
+// of the dilation).  The convolution is then dh x dw independent UNDILATED convolutions on the phase images
+// x[a::dh, b::dw], which run as one convolution on a batch dh x dw times as long:
+//   phases[(row * dh + a) * dw + b][c][i][j] = x[row][c][i * dh + a][j * dw + b]   (zero beyond the image)
+// to_caller copies the other way (positions of the phase images beyond the caller's image are dropped).
+struct DilationPhaseArgs {
+    const void* src;
+    void* dst;
+    long rows;          // components x images of the caller's tensor
+    int C, H, W;        // channels and extent of the caller's tensor
+    int Hp, Wp;         // extent of a phase image: at least ceil(H / dh), ceil(W / dw)
+    int dh, dw;
+};
+
+template <typename TS>
+__global__ void __launch_bounds__(WG_THREADS) dilation_phase_kernel(const DilationPhaseArgs A, int to_caller) {
+    const long stride = (long)gridDim.x * blockDim.x, first = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (!to_caller) {
+        const TS* x = static_cast<const TS*>(A.src);
+        TS* ph = static_cast<TS*>(A.dst);
+        const long total = A.rows * A.dh * A.dw * A.C * A.Hp * A.Wp;
+        for (long idx = first; idx < total; idx += stride) {
+            const int j = idx % A.Wp;
+            long rest = idx / A.Wp;
+            const int i = rest % A.Hp; rest /= A.Hp;
+            const int c = rest % A.C; rest /= A.C;
+            const int b = rest % A.dw; rest /= A.dw;
+            const int a = rest % A.dh;
+            const long row = rest / A.dh;
+            const int yi = i * A.dh + a, xj = j * A.dw + b;
+            ph[idx] = (yi < A.H && xj < A.W) ? x[((row * A.C + c) * A.H + yi) * A.W + xj] : (TS)0;
+        }
+    } else {
+        const TS* ph = static_cast<const TS*>(A.src);
+        TS* x = static_cast<TS*>(A.dst);
+        const long total = A.rows * A.C * A.H * A.W;
+        for (long idx = first; idx < total; idx += stride) {
+            const int xj = idx % A.W;
+            long rest = idx / A.W;
+            const int yi = rest % A.H; rest /= A.H;
+            const int c = rest % A.C;
+            const long row = rest / A.C;
+            const int a = yi % A.dh, i = yi / A.dh, b = xj % A.dw, j = xj / A.dw;
+            x[idx] = ph[((((row * A.dh + a) * A.dw + b) * A.C + c) * A.Hp + i) * A.Wp + j];
+        }
+    }
+}
+
 // Strided pointwise convolutions read every sh-th row and sw-th column of their input and nothing else:
 // dst[plane][i][j] = src[plane][i * sh][j * sw] turns them into unit-stride pointwise convolutions, which have the
 // streaming kernels.  One thread per 8 destination columns (one 16-byte store).

@@ -38,6 +38,8 @@ struct Tuning {
     double wg_kpw = 0.01;             // PHX_TUNE_WGKPW: how much the fp32 filter-gradient planner favours larger pixel tiles on small images (see plan_wgrad_f32)
     int thin_max32 = 64;              // PHX_TUNE_THIN_MAX32: the same bound for passes in fp32 arithmetic (x4 for the filter gradient); PHX_TUNE_THIN_MAX=0 zeroes it too
     int thin_max = 4;                 // PHX_TUNE_THIN_MAX: most input x output channels per group that run on the vector-ALU kernels for thin groups (0 = never)
+    int dilphase_min = 160;           // PHX_TUNE_DILPHASE_MIN: forward / input-gradient passes whose dilated window has more positions than this run by dilation phases
+    bool nodilphase = false;          // PHX_TUNE_NODILPHASE: dilated convolutions beyond the staging limit stay on the vector-ALU kernels
     int kslices = -1;                 // PHX_TUNE_KSLICES: reduction slices of a forward / input-gradient pass (0 = never, unset = by the rule of corr_slices)
     bool nodensecl = false;           // PHX_TUNE_NODENSECL: Dense never runs as a channels-last pointwise convolution
     bool nomerge = false;             // PHX_TUNE_NOMERGE: groups are never merged into block-diagonal ones
@@ -80,6 +82,8 @@ struct Tuning {
         nomerge = getenv("PHX_TUNE_NOMERGE") != nullptr;
         nodensecl = getenv("PHX_TUNE_NODENSECL") != nullptr;
         if (const char* e = getenv("PHX_TUNE_KSLICES")) kslices = atoi(e);
+        nodilphase = getenv("PHX_TUNE_NODILPHASE") != nullptr;
+        if (const char* e = getenv("PHX_TUNE_DILPHASE_MIN")) dilphase_min = atoi(e);
         nosmalldense = getenv("PHX_TUNE_NOSMALLDENSE") != nullptr;
         if (const char* e = getenv("PHX_TUNE_VEC")) vec = atoi(e);
         if (const char* e = getenv("PHX_TUNE_WGS")) wgs = atoi(e);
@@ -1568,6 +1572,52 @@ static void subsample_input(const Problem& p, const void* x, void* xs, hipStream
     launch_subsample(p.dtype == PHX_F16, a, st);
 }
 
+// the window of one output position -- ((kh-1) dh + 1) rows of ((kw-1) dw + 1) columns in whole 8-position chunks --
+// exceeds what the matrix-core kernels stage (one position per thread)
+static long window_positions(const Problem& p) { return ((long)(p.kh - 1) * p.dh + 1) * ((((long)(p.kw - 1) * p.dw + 1) + 7) & ~7L); }
+static bool window_beyond_staging(const Problem& p) { return window_positions(p) > WG_THREADS; }
+
+// Dilated convolutions beyond that limit (a 3x3 filter from dilation 8 on: the atrous pyramids of segmentation
+// networks use 12, 18, 24, 36) with unit stride and padding before the image that is a multiple of the dilation
+// (SAME padding of odd filters, VALID): an output position and every input position it reads share their row modulo
+// dh and their column modulo dw, so the convolution is dh x dw independent undilated convolutions on the phase
+// images x[a::dh, b::dw] (see dilation_phase_kernel).  They run as ONE undilated convolution q on a batch dh x dw
+// times as long, between a pass that gathers the phase images of the input-side tensor and one that scatters the
+// result's; the filter is used as it is, so the filter gradient comes out of q directly.  Phase images are padded
+// with zeros to one size (rows beyond the image are what the padding behind it holds anyway); the padding behind
+// the phase images is what gives q the output extent ceil(ho / dh) x ceil(wo / dw).
+struct DilationView {
+    Problem q;
+    int Hp, Wp, Hop, Wop;      // extent of the input-side and output-side phase images
+    size_t x_bytes, y_bytes;   // the two phase tensors
+};
+static bool dilation_view(const Problem& p, int pass, DilationView& v) {
+    if (tune().nodilphase || tune().direct || is_empty(p) || (p.dh == 1 && p.dw == 1) || p.sh != 1 || p.sw != 1) return false;
+    // (the filter gradient stages no halo window around its tiles: it takes the rewrite only where it has to)
+    const long most = pass == PHX_PASS_BWD_WEIGHTS ? WG_THREADS : std::min<long>(tune().dilphase_min, WG_THREADS);
+    if (window_positions(p) <= most || channel_slices(p) || p.nhwc || p.real_input) return false;
+    if (p.pt % p.dh || p.pl % p.dw || (long)p.n * p.dh * p.dw > (1L << 22)) return false;
+    v.Hp = cdiv(p.h, p.dh); v.Wp = cdiv(p.w, p.dw); v.Hop = cdiv(p.ho, p.dh); v.Wop = cdiv(p.wo, p.dw);
+    Problem& q = v.q;
+    q = p;
+    q.n = p.n * p.dh * p.dw; q.h = v.Hp; q.w = v.Wp; q.ho = v.Hop; q.wo = v.Wop; q.dh = q.dw = 1;
+    q.pt = p.pt / p.dh; q.pl = p.pl / p.dw;
+    q.pb = v.Hop + (p.kh - 1) - v.Hp - q.pt; q.pr = v.Wop + (p.kw - 1) - v.Wp - q.pl;
+    if (q.pb < 0 || q.pr < 0 || window_beyond_staging(q)) return false;
+    if (out_size(q.h, q.kh, 1, 1, q.pt, q.pb) != q.ho || out_size(q.w, q.kw, 1, 1, q.pl, q.pr) != q.wo) return false;
+    const size_t esize = p.dtype == PHX_F32 ? 4 : 2;
+    v.x_bytes = align_up((size_t)4 * q.n * p.ci * v.Hp * v.Wp * esize, 256);
+    v.y_bytes = align_up((size_t)4 * q.n * p.co * v.Hop * v.Wop * esize, 256);
+    return true;
+}
+// the phase images of the input-side (input = true) or output-side tensor of p, or the tensor back from them
+static void dilation_phases(const Problem& p, const DilationView& v, bool input, const void* src, void* dst, bool to_caller, hipStream_t st) {
+    DilationPhaseArgs a;
+    a.src = src; a.dst = dst; a.rows = 4L * p.n; a.C = input ? p.ci : p.co; a.H = input ? p.h : p.ho; a.W = input ? p.w : p.wo;
+    a.Hp = input ? v.Hp : v.Hop; a.Wp = input ? v.Wp : v.Wop; a.dh = p.dh; a.dw = p.dw;
+    launch_dilation_phases(p.dtype == PHX_F16, a, to_caller, st);
+}
+
 // Reduction slices of a forward / input-gradient pass.  Those kernels give a workgroup an output tile and the whole
 // reduction over channels and taps, so a pass with few output tiles and many channels (small batches on deep
 // layers: 512 channels at 7x7, N=1 is 16 workgroups of 288 steps) leaves most of the GPU idle however long it
@@ -1664,6 +1714,8 @@ struct SlicedCorr {
 };
 
 static size_t workspace_for(const Problem& p, int pass) {
+    DilationView dilated;
+    if (dilation_view(p, pass, dilated)) return dilated.x_bytes + dilated.y_bytes + workspace_for(dilated.q, pass);
     S2dView v;
     if (pass != PHX_PASS_BWD_DATA && s2d_view(p, v)) return v.x2_bytes + v.w2_bytes + workspace_plain(v.q, pass);
     Problem q;
@@ -1736,6 +1788,24 @@ static int do_fwd(const Problem& p, hipStream_t st, const void* x, const void* w
     const bool dry = g_pack.dry();
     if (!dry && (!x || !w || !y || (p.has_bias && !bias))) return PHX_ERR_INVALID_ARGUMENT;
     const void* b = p.has_bias ? bias : nullptr;
+    DilationView dilated;
+    if (dilation_view(p, PHX_PASS_FWD, dilated)) {
+        const size_t tensors = dilated.x_bytes + dilated.y_bytes;
+        if (!dry && (wsb < tensors || !ws)) return PHX_ERR_WORKSPACE;
+        char* x2 = static_cast<char*>(ws);
+        char* y2 = dry ? nullptr : x2 + dilated.x_bytes;
+        if (!dry) {
+            dilation_phases(p, dilated, true, x, x2, false, st);
+            PHX_HIP(hipGetLastError());
+        }
+        g_name_prefix = "dil_";
+        const int rc = do_fwd(dilated.q, st, x2, w, b, y2, dry ? nullptr : y2 + dilated.y_bytes, dry ? 0 : wsb - tensors);
+        g_name_prefix = "";
+        if (rc != PHX_OK || dry) return rc;
+        dilation_phases(p, dilated, false, y2, y, true, st);
+        PHX_HIP(hipGetLastError());
+        return PHX_OK;
+    }
     S2dView v;
     if (s2d_view(p, v)) {
         // (the rearranged filter of this path is itself made per call: no prepacked form)
@@ -1779,6 +1849,24 @@ static int do_bwd_data(const Problem& p, hipStream_t st, const void* g, const vo
     if (is_empty(p)) return PHX_OK;
     const bool dry = g_pack.dry();
     if (!dry && (!g || !w || !dx)) return PHX_ERR_INVALID_ARGUMENT;
+    DilationView dilated;
+    if (dilation_view(p, PHX_PASS_BWD_DATA, dilated)) {
+        const size_t tensors = dilated.x_bytes + dilated.y_bytes;
+        if (!dry && (wsb < tensors || !ws)) return PHX_ERR_WORKSPACE;
+        char* dx2 = static_cast<char*>(ws);
+        char* g2 = dry ? nullptr : dx2 + dilated.x_bytes;
+        if (!dry) {
+            dilation_phases(p, dilated, false, g, g2, false, st);
+            PHX_HIP(hipGetLastError());
+        }
+        g_name_prefix = "dil_";
+        const int rc = do_bwd_data(dilated.q, st, g2, w, dx2, dry ? nullptr : g2 + dilated.y_bytes, dry ? 0 : wsb - tensors);
+        g_name_prefix = "";
+        if (rc != PHX_OK || dry) return rc;
+        dilation_phases(p, dilated, true, dx2, dx, true, st);
+        PHX_HIP(hipGetLastError());
+        return PHX_OK;
+    }
     if (dgrad_by_phases(p)) {
         const size_t esize = p.dtype == PHX_F32 ? 4 : 2;
         PhaseMergeArgs m;
@@ -1828,6 +1916,20 @@ static int do_bwd_weights(const Problem& p, hipStream_t st, const void* x, const
         return PHX_OK;
     }
     if (!x || !g) return PHX_ERR_INVALID_ARGUMENT;
+    DilationView dilated;
+    if (dilation_view(p, PHX_PASS_BWD_WEIGHTS, dilated)) {
+        const size_t tensors = dilated.x_bytes + dilated.y_bytes;
+        if (wsb < tensors || !ws) return PHX_ERR_WORKSPACE;
+        char* x2 = static_cast<char*>(ws);
+        char* g2 = x2 + dilated.x_bytes;
+        dilation_phases(p, dilated, true, x, x2, false, st);
+        dilation_phases(p, dilated, false, g, g2, false, st);
+        PHX_HIP(hipGetLastError());
+        g_name_prefix = "dil_";
+        const int rc = do_bwd_weights(dilated.q, st, x2, g2, dw, g2 + dilated.y_bytes, wsb - tensors);
+        g_name_prefix = "";
+        return rc;
+    }
     S2dView v;
     if (s2d_view(p, v)) {
         if (wsb < v.x2_bytes + v.w2_bytes || !ws) return PHX_ERR_WORKSPACE;
@@ -2042,13 +2144,13 @@ static bool nhwc_wgrad_native(const Problem& p) {
 // stage one window position per thread, so the window of a single output position -- ((kh-1) dh + 1) rows of
 // ((kw-1) dw + 1) columns, rounded up to whole 8-position chunks -- must not exceed 256 positions (a 7x7 filter at
 // dilation 3, a 17x17 one).  Such convolutions, grouped or not, run here at vector-ALU speed rather than not at all.
-static bool window_beyond_staging(const Problem& p) {
-    return ((long)(p.kh - 1) * p.dh + 1) * ((((long)(p.kw - 1) * p.dw + 1) + 7) & ~7L) > WG_THREADS;
-}
+// (window_beyond_staging; dilated ones that dilation_view can rewrite run as undilated convolutions instead)
 static bool thin_groups(const Problem& p, int pass) {
     if (is_empty(p) || p.ho <= 0 || p.wo <= 0) return false;
     if ((long)p.kh * p.kw > 2048 || std::max(p.ci_mem, p.co_mem) > 65535) return false;  // (a filter chunk in LDS; grid rows)
-    if (tune().direct || window_beyond_staging(p)) return true;
+    if (tune().direct) return true;
+    DilationView dilated;
+    if (window_beyond_staging(p)) return !dilation_view(p, pass, dilated);
     const long pairs = (long)p.ci * p.co;
     // The filter gradient in fp32 arithmetic works on 64 x 64 channel tiles whatever the layer holds: its time follows
     // the pixels and taps alone (3x3, 56x56, N=64: 1.39 ms from 8 to 64 channels), that of the vector-ALU kernel the

@@ -507,9 +507,12 @@ def test_windows_beyond_the_staging_limit(case, mode, dtype, policy):
     names.append(capi.last_kernel_name())
     dw = ops.conv2d_bwd_weights(xd, gd, desc)
     names.append(capi.last_kernel_name())
-    assert all("_fma_thin_" in k for k in names), names
-    assert desc.workspace_bytes(capi.PHX_PASS_FWD) == 0 and desc.workspace_bytes(capi.PHX_PASS_BWD_DATA) == 0
-    assert ops.conv2d_pack_filters(wd, desc) is None
+    if name == "k7_dil3":  # (unit stride, padding a multiple of the dilation: undilated on its dilation phases, see below)
+        assert all(k.startswith("dil_") and "mfma" in k for k in names), names
+    else:
+        assert all("_fma_thin_" in k for k in names), names
+        assert desc.workspace_bytes(capi.PHX_PASS_FWD) == 0 and desc.workspace_bytes(capi.PHX_PASS_BWD_DATA) == 0
+        assert ops.conv2d_pack_filters(wd, desc) is None
     x64, w64, b64, g64 = (a.astype(np.float64) for a in (x, wt, b, gr))
     want_y = oracle.conv2d_fwd(g, x64, w64, b64, "hamilton")
     want_dw, want_dx = oracle.conv2d_bwd(g, x64, w64, g64, "hamilton")
@@ -642,6 +645,74 @@ def test_small_channels_last_batches_are_sliced_on_their_channels_first_copies(c
             assert ("_kslices" in k_fwd, "_kslices" in k_dx) == (expect if setting is None else (False, False)), (k_fwd, k_dx)
         assert_close(y.cpu().numpy().transpose(0, 3, 1, 2), want_y, dtype, "fwd " + k_fwd)
         assert_close(dx.cpu().numpy().transpose(0, 3, 1, 2), want_dx, dtype, "dgrad " + k_dx)
+
+
+LARGE_DILATIONS = [
+    # name, n, ci, co, h, w, kh, kw, dilation, padding, runs by phases
+    ("aspp_k3_d12", 2, 24, 40, 33, 33, 3, 3, 12, "SAME", True),                  # an atrous-pyramid branch
+    ("aspp_k3_d18_17x21", 1, 16, 16, 17, 21, 3, 3, 18, "SAME", True),            # dilation beyond the image: most phases are one pixel
+    ("k3_d8x9_valid", 2, 8, 24, 30, 41, 3, 3, (8, 9), "VALID", True),            # extents that the dilation does not divide
+    ("k3x1_d40x1", 1, 16, 8, 90, 9, 3, 1, (40, 1), "SAME", True),                # rows only
+    ("k5_d6_pad", 1, 8, 8, 29, 31, 5, 5, 6, (12, 6, 7, 20), True),               # explicit padding: multiples before the image, anything behind
+    ("k3_d12_pad_odd", 1, 8, 8, 30, 30, 3, 3, 12, (5, 12, 12, 12), False),       # 5 rows before the image: not a multiple, vector-ALU kernels
+    ("k3_d16_128", 1, 128, 128, 20, 20, 3, 3, 16, "SAME", True),                 # deep and small: the undilated problem runs in reduction slices
+    # windows that the matrix-core kernels can stage, but with a halo that leaves next to nothing of a tile: forward and
+    # input gradient by phases, the filter gradient (no halo) as it is
+    ("k3_d6", 2, 16, 24, 27, 25, 3, 3, 6, "SAME", "fd"),
+    ("k5_d3_valid", 2, 8, 16, 30, 31, 5, 5, 3, "VALID", "fd"),
+    ("k7x3_d2x5", 1, 16, 8, 26, 40, 7, 3, (2, 5), "SAME", "fd"),
+    ("k3_d4", 2, 16, 16, 20, 20, 3, 3, 4, "SAME", None),                         # 9 x 16 positions: the dilated kernels keep it
+]
+
+
+@pytest.mark.parametrize("dtype,policy", [(torch.float32, "fp32"), (torch.float16, "full16"), (torch.float16, "backward32")],
+                         ids=["f32", "f16_full16", "f16_backward32"])
+@pytest.mark.parametrize("mode", [16, 8])
+@pytest.mark.parametrize("case", LARGE_DILATIONS, ids=lambda c: c[0])
+def test_large_dilations_run_as_undilated_convolutions_on_their_phases(case, mode, dtype, policy, tune_env):
+    """With unit stride an output position and all the input positions it reads share their row modulo dh and column
+    modulo dw: a dilated convolution whose window is beyond the matrix-core kernels' staging (3x3 from dilation 8
+    on) runs as one undilated convolution on the dh x dw phase images of its tensors, the batch that much longer,
+    where the padding before the image is a multiple of the dilation.  Forward and input gradient take the same route
+    from 161 window positions on (3x3 at dilation 5, 5x5 at 3, 7x7 at 2), where the halo of the dilated window leaves
+    their tiles next to no output positions.  Against the oracle and against the kernels that run such windows
+    otherwise (PHX_TUNE_NODILPHASE); prepacked filters and the addend bit for bit."""
+    # by_phases: True = all three passes, "fd" = forward and input gradient, None = no pass (matrix-core kernels as they
+    # are), False = no pass (vector-ALU kernels)
+    name, n, ci, co, h, w, kh, kw, dilation, padding, by_phases = case
+    scale = 1.0 if dtype == torch.float32 else 0.5
+    g, x, wt, b, gr = make_inputs(name_seed(name) + 91, n, ci, co, h, w, kh, kw, 1, dilation, padding, dtype, scale)
+    desc = phx.Conv2DDescriptor(x.shape, wt.shape, 1, dilation, padding, use_bias=True, dtype=dtype, context=Ctx(mode, policy))
+    xd, wd, bd, gd = (torch.from_numpy(a).cuda() for a in (x, wt, b, gr))
+    x64, w64, b64, g64 = (a.astype(np.float64) for a in (x, wt, b, gr))
+    want_y = oracle.conv2d_fwd(g, x64, w64, b64, "hamilton")
+    want_dw, want_dx = oracle.conv2d_bwd(g, x64, w64, g64, "hamilton")
+    addend = torch.from_numpy((scale * np.random.default_rng(7).standard_normal(x.shape)).astype(x.dtype)).cuda()
+    for phases in (True, False):
+        # (THIN_MAX32=0: filter gradients of few channels in fp32 arithmetic stay off the vector-ALU kernels)
+        tune_env(PHX_TUNE_NODILPHASE=None if phases else "1", PHX_TUNE_THIN_MAX32="0")
+        y = phx.conv2d_fwd(xd, wd, bd, desc)
+        names = [capi.last_kernel_name()]
+        dx = ops.conv2d_bwd_data(wd, gd, desc)
+        names.append(capi.last_kernel_name())
+        dw = ops.conv2d_bwd_weights(xd, gd, desc)
+        names.append(capi.last_kernel_name())
+        rewritten = [phases and bool(by_phases)] * 2 + [phases and by_phases is True]
+        assert [k.startswith("dil_") for k in names] == rewritten, names
+        # (what is not rewritten runs on the vector-ALU kernels if the window is beyond the staging limit)
+        assert ["_fma_thin_" in k for k in names] == [not r and by_phases in (True, False) for r in rewritten], names
+        if phases and name == "k3_d16_128":
+            assert "_kslices" in names[0] and "_kslices" in names[1], names
+        assert_close(y.cpu().numpy(), want_y, dtype, "fwd " + names[0])
+        assert_close(dx.cpu().numpy(), want_dx, dtype, "dgrad " + names[1])
+        assert_close(dw.cpu().numpy(), want_dw, dtype, "wgrad " + names[2])
+        assert torch.equal(ops.conv2d_bwd_data(wd, gd, desc, addend=addend), dx + addend), "dgrad + addend"
+        packed = ops.conv2d_pack_filters(wd, desc)
+        assert (packed is not None) == ((phases and bool(by_phases)) or by_phases in ("fd", None))
+        if packed is not None:
+            zero = torch.zeros_like(wd)
+            assert torch.equal(phx.conv2d_fwd(xd, zero, bd, desc, packed=packed), y), "prepacked fwd"
+            assert torch.equal(ops.conv2d_bwd_data(zero, gd, desc, packed=packed), dx), "prepacked dgrad"
 
 
 DIRECT_CASES = ("pw_ragged", "k3_same", "k3_ragged", "k3_s2", "pw_s31", "k7_s2", "k5_s2_valid", "k3_dil2", "k32_asym", "k7_s2_dil2")
