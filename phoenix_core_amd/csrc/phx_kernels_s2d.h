@@ -53,18 +53,20 @@ __global__ void __launch_bounds__(WG_THREADS) s2d_input_kernel(const S2dArgs A) 
 }
 
 // Dilation phases.  With unit stride, an output position and every input position it reads lie dh rows and dw columns
-// apart: they share their row modulo dh and their column modulo dw (where the padding before the image is a multiple
-// of the dilation).  The convolution is then dh x dw independent UNDILATED convolutions on the phase images
-// x[a::dh, b::dw], which run as one convolution on a batch dh x dw times as long:
-//   phases[(row * dh + a) * dw + b][c][i][j] = x[row][c][i * dh + a][j * dw + b]   (zero beyond the image)
-// to_caller copies the other way (positions of the phase images beyond the caller's image are dropped).
+// apart: counted from an origin (oh, ow) = padding before the image modulo the dilation in front of the input (from
+// the first position of the output), they share their row modulo dh and their column modulo dw.  The convolution is
+// then dh x dw independent UNDILATED convolutions on the phase images, which run as one convolution on a batch
+// dh x dw times as long:
+//   phases[(row * dh + a) * dw + b][c][i][j] = x[row][c][i * dh + a - oh][j * dw + b - ow]   (zero outside the image)
+// to_caller copies the other way (positions of the phase images outside the caller's image are dropped).
 struct DilationPhaseArgs {
     const void* src;
     void* dst;
     long rows;          // components x images of the caller's tensor
     int C, H, W;        // channels and extent of the caller's tensor
-    int Hp, Wp;         // extent of a phase image: at least ceil(H / dh), ceil(W / dw)
+    int Hp, Wp;         // extent of a phase image: at least ceil((H + oh) / dh), ceil((W + ow) / dw)
     int dh, dw;
+    int oh, ow;         // rows / columns of the origin in front of the tensor's first
 };
 
 template <typename TS>
@@ -82,8 +84,8 @@ __global__ void __launch_bounds__(WG_THREADS) dilation_phase_kernel(const Dilati
             const int b = rest % A.dw; rest /= A.dw;
             const int a = rest % A.dh;
             const long row = rest / A.dh;
-            const int yi = i * A.dh + a, xj = j * A.dw + b;
-            ph[idx] = (yi < A.H && xj < A.W) ? x[((row * A.C + c) * A.H + yi) * A.W + xj] : (TS)0;
+            const int yi = i * A.dh + a - A.oh, xj = j * A.dw + b - A.ow;
+            ph[idx] = (yi >= 0 && yi < A.H && xj >= 0 && xj < A.W) ? x[((row * A.C + c) * A.H + yi) * A.W + xj] : (TS)0;
         }
     } else {
         const TS* ph = static_cast<const TS*>(A.src);
@@ -95,7 +97,7 @@ __global__ void __launch_bounds__(WG_THREADS) dilation_phase_kernel(const Dilati
             const int yi = rest % A.H; rest /= A.H;
             const int c = rest % A.C;
             const long row = rest / A.C;
-            const int a = yi % A.dh, i = yi / A.dh, b = xj % A.dw, j = xj / A.dw;
+            const int a = (yi + A.oh) % A.dh, i = (yi + A.oh) / A.dh, b = (xj + A.ow) % A.dw, j = (xj + A.ow) / A.dw;
             x[idx] = ph[((((row * A.dh + a) * A.dw + b) * A.C + c) * A.Hp + i) * A.Wp + j];
         }
     }

@@ -1578,10 +1578,10 @@ static long window_positions(const Problem& p) { return ((long)(p.kh - 1) * p.dh
 static bool window_beyond_staging(const Problem& p) { return window_positions(p) > WG_THREADS; }
 
 // Dilated convolutions beyond that limit (a 3x3 filter from dilation 8 on: the atrous pyramids of segmentation
-// networks use 12, 18, 24, 36) with unit stride and padding before the image that is a multiple of the dilation
-// (SAME padding of odd filters, VALID): an output position and every input position it reads share their row modulo
-// dh and their column modulo dw, so the convolution is dh x dw independent undilated convolutions on the phase
-// images x[a::dh, b::dw] (see dilation_phase_kernel).  They run as ONE undilated convolution q on a batch dh x dw
+// networks use 12, 18, 24, 36) with unit stride: an output position and every input position it reads lie whole
+// dilations apart, so the convolution is dh x dw independent undilated convolutions on the phase images of its
+// tensors (see dilation_phase_kernel; the input side counts its phases from pt % dh rows, pl % dw columns in front
+// of the image, which leaves q whole rows and columns of padding).  They run as ONE undilated convolution q on a batch dh x dw
 // times as long, between a pass that gathers the phase images of the input-side tensor and one that scatters the
 // result's; the filter is used as it is, so the filter gradient comes out of q directly.  Phase images are padded
 // with zeros to one size (rows beyond the image are what the padding behind it holds anyway); the padding behind
@@ -1596,8 +1596,8 @@ static bool dilation_view(const Problem& p, int pass, DilationView& v) {
     // (the filter gradient stages no halo window around its tiles: it takes the rewrite only where it has to)
     const long most = pass == PHX_PASS_BWD_WEIGHTS ? WG_THREADS : std::min<long>(tune().dilphase_min, WG_THREADS);
     if (window_positions(p) <= most || channel_slices(p) || p.nhwc || p.real_input) return false;
-    if (p.pt % p.dh || p.pl % p.dw || (long)p.n * p.dh * p.dw > (1L << 22)) return false;
-    v.Hp = cdiv(p.h, p.dh); v.Wp = cdiv(p.w, p.dw); v.Hop = cdiv(p.ho, p.dh); v.Wop = cdiv(p.wo, p.dw);
+    if ((long)p.n * p.dh * p.dw > (1L << 22)) return false;
+    v.Hp = cdiv(p.h + p.pt % p.dh, p.dh); v.Wp = cdiv(p.w + p.pl % p.dw, p.dw); v.Hop = cdiv(p.ho, p.dh); v.Wop = cdiv(p.wo, p.dw);
     Problem& q = v.q;
     q = p;
     q.n = p.n * p.dh * p.dw; q.h = v.Hp; q.w = v.Wp; q.ho = v.Hop; q.wo = v.Wop; q.dh = q.dw = 1;
@@ -1615,6 +1615,7 @@ static void dilation_phases(const Problem& p, const DilationView& v, bool input,
     DilationPhaseArgs a;
     a.src = src; a.dst = dst; a.rows = 4L * p.n; a.C = input ? p.ci : p.co; a.H = input ? p.h : p.ho; a.W = input ? p.w : p.wo;
     a.Hp = input ? v.Hp : v.Hop; a.Wp = input ? v.Wp : v.Wop; a.dh = p.dh; a.dw = p.dw;
+    a.oh = input ? p.pt % p.dh : 0; a.ow = input ? p.pl % p.dw : 0;
     launch_dilation_phases(p.dtype == PHX_F16, a, to_caller, st);
 }
 

@@ -507,7 +507,7 @@ def test_windows_beyond_the_staging_limit(case, mode, dtype, policy):
     names.append(capi.last_kernel_name())
     dw = ops.conv2d_bwd_weights(xd, gd, desc)
     names.append(capi.last_kernel_name())
-    if name == "k7_dil3":  # (unit stride, padding a multiple of the dilation: undilated on its dilation phases, see below)
+    if name == "k7_dil3":  # (unit stride: undilated on its dilation phases, see below)
         assert all(k.startswith("dil_") and "mfma" in k for k in names), names
     else:
         assert all("_fma_thin_" in k for k in names), names
@@ -653,8 +653,10 @@ LARGE_DILATIONS = [
     ("aspp_k3_d18_17x21", 1, 16, 16, 17, 21, 3, 3, 18, "SAME", True),            # dilation beyond the image: most phases are one pixel
     ("k3_d8x9_valid", 2, 8, 24, 30, 41, 3, 3, (8, 9), "VALID", True),            # extents that the dilation does not divide
     ("k3x1_d40x1", 1, 16, 8, 90, 9, 3, 1, (40, 1), "SAME", True),                # rows only
-    ("k5_d6_pad", 1, 8, 8, 29, 31, 5, 5, 6, (12, 6, 7, 20), True),               # explicit padding: multiples before the image, anything behind
-    ("k3_d12_pad_odd", 1, 8, 8, 30, 30, 3, 3, 12, (5, 12, 12, 12), False),       # 5 rows before the image: not a multiple, vector-ALU kernels
+    ("k5_d6_pad", 1, 8, 8, 29, 31, 5, 5, 6, (12, 6, 7, 20), True),               # explicit padding: whole dilations before the image
+    ("k3_d12_pad_odd", 1, 8, 8, 30, 30, 3, 3, 12, (5, 12, 31, 0), True),         # 5 rows before the image: the input's phases count from 5 rows above it
+    ("k2_d9x31_pad", 2, 8, 16, 14, 39, 2, 2, (9, 31), (3, 40, 8, 13), True),     # more padding than a dilation: 40 = 31 + 9 columns
+    ("k3_d12_s2", 1, 8, 8, 40, 40, 3, 3, 12, "SAME", False, 2),                  # stride 2: vector-ALU kernels
     ("k3_d16_128", 1, 128, 128, 20, 20, 3, 3, 16, "SAME", True),                 # deep and small: the undilated problem runs in reduction slices
     # windows that the matrix-core kernels can stage, but with a halo that leaves next to nothing of a tile: forward and
     # input gradient by phases, the filter gradient (no halo) as it is
@@ -673,16 +675,17 @@ def test_large_dilations_run_as_undilated_convolutions_on_their_phases(case, mod
     """With unit stride an output position and all the input positions it reads share their row modulo dh and column
     modulo dw: a dilated convolution whose window is beyond the matrix-core kernels' staging (3x3 from dilation 8
     on) runs as one undilated convolution on the dh x dw phase images of its tensors, the batch that much longer,
-    where the padding before the image is a multiple of the dilation.  Forward and input gradient take the same route
+    whatever the padding (the input's phases count from the padding's remainder above the image).  Forward and input gradient take the same route
     from 161 window positions on (3x3 at dilation 5, 5x5 at 3, 7x7 at 2), where the halo of the dilated window leaves
     their tiles next to no output positions.  Against the oracle and against the kernels that run such windows
     otherwise (PHX_TUNE_NODILPHASE); prepacked filters and the addend bit for bit."""
     # by_phases: True = all three passes, "fd" = forward and input gradient, None = no pass (matrix-core kernels as they
     # are), False = no pass (vector-ALU kernels)
-    name, n, ci, co, h, w, kh, kw, dilation, padding, by_phases = case
+    name, n, ci, co, h, w, kh, kw, dilation, padding, by_phases = case[:11]
+    stride = case[11] if len(case) > 11 else 1
     scale = 1.0 if dtype == torch.float32 else 0.5
-    g, x, wt, b, gr = make_inputs(name_seed(name) + 91, n, ci, co, h, w, kh, kw, 1, dilation, padding, dtype, scale)
-    desc = phx.Conv2DDescriptor(x.shape, wt.shape, 1, dilation, padding, use_bias=True, dtype=dtype, context=Ctx(mode, policy))
+    g, x, wt, b, gr = make_inputs(name_seed(name) + 91, n, ci, co, h, w, kh, kw, stride, dilation, padding, dtype, scale)
+    desc = phx.Conv2DDescriptor(x.shape, wt.shape, stride, dilation, padding, use_bias=True, dtype=dtype, context=Ctx(mode, policy))
     xd, wd, bd, gd = (torch.from_numpy(a).cuda() for a in (x, wt, b, gr))
     x64, w64, b64, g64 = (a.astype(np.float64) for a in (x, wt, b, gr))
     want_y = oracle.conv2d_fwd(g, x64, w64, b64, "hamilton")
