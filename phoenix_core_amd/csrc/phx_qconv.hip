@@ -1595,11 +1595,14 @@ static bool dilation_view(const Problem& p, int pass, DilationView& v) {
     if (tune().nodilphase || tune().direct || is_empty(p) || (p.dh == 1 && p.dw == 1) || p.sh != 1 || p.sw != 1) return false;
     // (the filter gradient stages no halo window around its tiles: it takes the rewrite only where it has to)
     const long most = pass == PHX_PASS_BWD_WEIGHTS ? WG_THREADS : std::min<long>(tune().dilphase_min, WG_THREADS);
-    if (window_positions(p) <= most || channel_slices(p) || p.nhwc || p.real_input) return false;
+    // (channels-last calls: the rewrite works on the channels-first copies such a call goes through -- nhwc_window_native
+    // and nhwc_wgrad_native leave these problems to the copies -- never on the caller's tensors)
+    if (window_positions(p) <= most || channel_slices(p) || g_window_cl || p.real_input) return false;
     if ((long)p.n * p.dh * p.dw > (1L << 22)) return false;
     v.Hp = cdiv(p.h + p.pt % p.dh, p.dh); v.Wp = cdiv(p.w + p.pl % p.dw, p.dw); v.Hop = cdiv(p.ho, p.dh); v.Wop = cdiv(p.wo, p.dw);
     Problem& q = v.q;
     q = p;
+    q.nhwc = false;  // (the phase tensors are channels-first)
     q.n = p.n * p.dh * p.dw; q.h = v.Hp; q.w = v.Wp; q.ho = v.Hop; q.wo = v.Wop; q.dh = q.dw = 1;
     q.pt = p.pt / p.dh; q.pl = p.pl / p.dw;
     q.pb = v.Hop + (p.kh - 1) - v.Hp - q.pt; q.pr = v.Wop + (p.kw - 1) - v.Wp - q.pl;
@@ -2112,10 +2115,11 @@ static bool nhwc_window_native(const Problem& p, int pass) {
     if (!plan_corr(pass == PHX_PASS_FWD ? corr_forward(p) : corr_dgrad(p), p.mode, true, c, pl, pw)) return false;
     if (!(pl.lds_filters && pl.chunks && !pl.pwx && pw == 0)) return false;
     // a small batch on a deep layer gains more from reduction slices (corr_slices), which run on channels-first copies:
-    // the copies of so small a problem cost next to nothing
+    // the copies of so small a problem cost next to nothing; so do dilated windows from their dilation phases
     Problem planes = p;
     planes.nhwc = false;
-    return corr_slices(planes, pass) == 0;
+    DilationView dilated;
+    return corr_slices(planes, pass) == 0 && !dilation_view(planes, pass, dilated);
 }
 }  // namespace phx
 
@@ -2124,6 +2128,7 @@ static bool nhwc_window_native(const Problem& p, int pass) {
 // kernel's channels-last staging transposes 8x8 blocks in registers on the way to LDS (qconv_wgrad_f16_kernel, CL).
 static bool nhwc_wgrad_native(const Problem& p) {
     if (!p.nhwc || is_empty(p) || p.real_input || p.groups != 1 || p.sh != 1 || p.sw != 1 || tune().nowincl) return false;
+    if (window_beyond_staging(p)) return false;  // (the vector-ALU kernels, or the dilation phases of channels-first copies)
     if (p.ci % 8 != 0 || p.co % 8 != 0 || p.ci_mem != p.ci || p.co_mem != p.co) return false;
     const Problem f = flatten_pointwise(p);
     if (!wgrad_on_f16_mfma(f)) return false;

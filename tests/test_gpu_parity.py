@@ -718,6 +718,36 @@ def test_large_dilations_run_as_undilated_convolutions_on_their_phases(case, mod
             assert torch.equal(ops.conv2d_bwd_data(zero, gd, desc, packed=packed), dx), "prepacked dgrad"
 
 
+@pytest.mark.parametrize("dtype,policy", [(torch.float32, "fp32"), (torch.float16, "full16")], ids=["f32", "f16_full16"])
+@pytest.mark.parametrize("case", [c for c in LARGE_DILATIONS if c[0] in ("aspp_k3_d12", "k3_d12_pad_odd", "k3_d6", "k7x3_d2x5")], ids=lambda c: c[0])
+def test_large_dilations_on_channels_last_tensors(case, dtype, policy, tune_env):
+    """Channels-last calls take the same rewrite on the channels-first copies they go through (also where the window is
+    one that the channels-last kernels could have staged on the caller's tensors: the halo is the same there)."""
+    name, n, ci, co, h, w, kh, kw, dilation, padding, by_phases = case[:11]
+    scale = 1.0 if dtype == torch.float32 else 0.5
+    g, x, wt, b, gr = make_inputs(name_seed(name) + 92, n, ci, co, h, w, kh, kw, 1, dilation, padding, dtype, scale)
+    x_dev = np.ascontiguousarray(x.transpose(0, 2, 3, 1))
+    g_dev = np.ascontiguousarray(gr.transpose(0, 2, 3, 1))
+    w_dev = np.ascontiguousarray(wt.transpose(0, 1, 3, 4, 2))
+    desc = phx.Conv2DDescriptor(x_dev.shape, w_dev.shape, 1, dilation, padding, use_bias=True, dtype=dtype, filter_layout="OHWI",
+                                context=Ctx(8, policy), data_format="NHWC")
+    xd, wd, bd, gd = (torch.from_numpy(a).cuda() for a in (x_dev, w_dev, b, g_dev))
+    x64, w64, b64, g64 = (a.astype(np.float64) for a in (x, wt, b, gr))
+    want_y = oracle.conv2d_fwd(g, x64, w64, b64, "hamilton")
+    want_dw, want_dx = oracle.conv2d_bwd(g, x64, w64, g64, "hamilton")
+    tune_env(PHX_TUNE_THIN_MAX32="0")
+    y = phx.conv2d_fwd(xd, wd, bd, desc)
+    names = [capi.last_kernel_name()]
+    dx = ops.conv2d_bwd_data(wd, gd, desc)
+    names.append(capi.last_kernel_name())
+    dw = ops.conv2d_bwd_weights(xd, gd, desc)
+    names.append(capi.last_kernel_name())
+    assert [k.startswith("dil_") for k in names] == [True, True, by_phases is True], names
+    assert_close(y.cpu().numpy().transpose(0, 3, 1, 2), want_y, dtype, "fwd " + names[0])
+    assert_close(dx.cpu().numpy().transpose(0, 3, 1, 2), want_dx, dtype, "dgrad " + names[1])
+    assert_close(dw.cpu().numpy().transpose(0, 1, 4, 2, 3), want_dw, dtype, "wgrad " + names[2])
+
+
 DIRECT_CASES = ("pw_ragged", "k3_same", "k3_ragged", "k3_s2", "pw_s31", "k7_s2", "k5_s2_valid", "k3_dil2", "k32_asym", "k7_s2_dil2")
 
 
