@@ -52,6 +52,31 @@ __global__ void __launch_bounds__(WG_THREADS) s2d_input_kernel(const S2dArgs A) 
     }
 }
 
+// dst[plane][i][j] = src[plane][i * sh + oh][j * sw + ow], zero where that lies outside the source: the input rows and
+// columns that one residue class of filter taps reads in a strided convolution (the origin may lie in the padding).
+struct StridedGatherArgs {
+    const void* src;
+    void* dst;
+    long planes;        // components x images x channels
+    int H, W, H2, W2;   // source and destination extent
+    int sh, sw, oh, ow;
+};
+
+template <typename TS>
+__global__ void __launch_bounds__(WG_THREADS) strided_gather_kernel(const StridedGatherArgs A) {
+    const TS* src = static_cast<const TS*>(A.src);
+    TS* dst = static_cast<TS*>(A.dst);
+    const long total = A.planes * A.H2 * A.W2;
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
+        const int j = idx % A.W2;
+        const long rest = idx / A.W2;
+        const int i = rest % A.H2;
+        const long plane = rest / A.H2;
+        const long yi = (long)i * A.sh + A.oh, xj = (long)j * A.sw + A.ow;
+        dst[idx] = (yi >= 0 && yi < A.H && xj >= 0 && xj < A.W) ? src[(plane * A.H + yi) * A.W + xj] : (TS)0;
+    }
+}
+
 // Dilation phases.  With unit stride, an output position and every input position it reads lie dh rows and dw columns
 // apart: counted from an origin (oh, ow) = padding before the image modulo the dilation in front of the input (from
 // the first position of the output), they share their row modulo dh and their column modulo dw.  The convolution is

@@ -28,6 +28,14 @@ int launch_s2d_input(bool half_storage, const S2dArgs& a, hipStream_t st) {
     return 0;
 }
 
+int launch_strided_gather(bool half_storage, const StridedGatherArgs& a, hipStream_t st) {
+    const long items = a.planes * a.H2 * a.W2;
+    if (items <= 0) return 0;
+    if (half_storage) hipLaunchKernelGGL((strided_gather_kernel<_Float16>), dim3(blocks_for(items)), dim3(WG_THREADS), 0, st, a);
+    else hipLaunchKernelGGL((strided_gather_kernel<float>), dim3(blocks_for(items)), dim3(WG_THREADS), 0, st, a);
+    return 0;
+}
+
 int launch_dilation_phases(bool half_storage, const DilationPhaseArgs& a, bool to_caller, hipStream_t st) {
     const long items = to_caller ? a.rows * a.C * a.H * a.W : a.rows * a.dh * a.dw * a.C * a.Hp * a.Wp;
     if (items <= 0) return 0;

@@ -39,6 +39,7 @@ struct Tuning {
     int thin_max32 = 64;              // PHX_TUNE_THIN_MAX32: the same bound for passes in fp32 arithmetic (x4 for the filter gradient); PHX_TUNE_THIN_MAX=0 zeroes it too
     int thin_max = 4;                 // PHX_TUNE_THIN_MAX: most input x output channels per group that run on the vector-ALU kernels for thin groups (0 = never)
     int dilphase_min = 160;           // PHX_TUNE_DILPHASE_MIN: forward / input-gradient passes whose dilated window has more positions than this run by dilation phases
+    int wgphase = -1;                 // PHX_TUNE_WGPHASE: 1 = every strided filter gradient with several taps runs by tap classes, 0 = none (unset: wgrad_by_classes)
     bool nodilphase = false;          // PHX_TUNE_NODILPHASE: dilated convolutions beyond the staging limit stay on the vector-ALU kernels
     int kslices = -1;                 // PHX_TUNE_KSLICES: reduction slices of a forward / input-gradient pass (0 = never, unset = by the rule of corr_slices)
     bool nodensecl = false;           // PHX_TUNE_NODENSECL: Dense never runs as a channels-last pointwise convolution
@@ -83,6 +84,7 @@ struct Tuning {
         nodensecl = getenv("PHX_TUNE_NODENSECL") != nullptr;
         if (const char* e = getenv("PHX_TUNE_KSLICES")) kslices = atoi(e);
         nodilphase = getenv("PHX_TUNE_NODILPHASE") != nullptr;
+        if (const char* e = getenv("PHX_TUNE_WGPHASE")) wgphase = atoi(e) != 0;
         if (const char* e = getenv("PHX_TUNE_DILPHASE_MIN")) dilphase_min = atoi(e);
         nosmalldense = getenv("PHX_TUNE_NOSMALLDENSE") != nullptr;
         if (const char* e = getenv("PHX_TUNE_VEC")) vec = atoi(e);
@@ -1622,6 +1624,61 @@ static void dilation_phases(const Problem& p, const DilationView& v, bool input,
     launch_dilation_phases(p.dtype == PHX_F16, a, to_caller, st);
 }
 
+// Filter gradient of a strided convolution by tap classes.  Along an axis the taps whose input rows kh * d - pt share
+// a residue modulo the stride form an arithmetic progression k0, k0 + T, ... (T = s / gcd(s, d)), and for them
+//   x[s * i + kh * d - pt] = xg[i + m * (T * d / s)],   xg[i] = x[s * i + k0 * d - pt]  (zero outside the image):
+// a unit-stride, unpadded correlation of `taps` taps and dilation T * d / s on the gathered rows xg, of which
+// out + (taps - 1) * dilation are read.  The filter gradient of class (ch, cw) is therefore a unit-stride filter
+// gradient between xg and the output gradient, written to its own taps of dw through filter strides T times as
+// long: the strided problem runs as (at most sh x sw) unit-stride ones on the fast kernels, each behind one gather.
+// (3x3 stride 2: classes of 2x2, 2x1, 1x2 and 1x1 taps, nine taps' work in all.)
+struct TapClass {
+    int taps, k0, kstep, dil, origin, size;
+};
+static int tap_classes(int k, int d, int s, int pad_before, int out, TapClass* cls) {
+    const int period = s / std::__gcd(s, d);
+    int n = 0;
+    for (int k0 = 0; k0 < std::min(k, period); ++k0) {
+        TapClass c;
+        c.k0 = k0; c.kstep = period; c.taps = (k - 1 - k0) / period + 1;
+        c.dil = c.taps > 1 ? period * d / s : 1;
+        c.origin = k0 * d - pad_before;
+        c.size = out + (c.taps - 1) * c.dil;
+        cls[n++] = c;
+    }
+    return n;
+}
+constexpr int TAP_CLASSES_MAX = 8;  // strides up to 8 along an axis
+
+// Which strided filter gradients run that way: those that would otherwise fall to fp32 arithmetic although the
+// policy allows fp16 matrix cores (strides beyond 2 along W have no fp16 kernel: 3x3 stride 3, 128 channels at
+// 28x28, N=32 570 -> 204 us), and large ones, where the strided kernels' one tap per workgroup costs more than the
+// gathers, the launches and the classes' own reductions.  3x3 stride 2, strided kernel against classes (us):
+// fp16 matrix cores 512 channels at 28x28, N=32 1144 / 818, 512 at 14x14, N=64 772 / 521, 256 at 28x28 558 / 508, but
+// 256 at 14x14 197 / 219, 128 at 28x28 139 / 229, 64 at 56x56 131 / 289; fp32 arithmetic 512 at 28x28 5708 / 3396,
+// 512 at 14x14 4260 / 1973, 256 at 28x28 2169 / 1802, but 128 at 28x28 544 / 536, 64 at 28x28 151 / 223.
+static bool wgrad_by_classes(const Problem& p) {
+    if ((p.sh == 1 && p.sw == 1) || p.kh * p.kw == 1 || is_empty(p) || channel_slices(p) || p.real_input || g_window_cl) return false;
+    if (p.sh > TAP_CLASSES_MAX || p.sw > TAP_CLASSES_MAX) return false;
+    S2dView v;
+    if (s2d_view(p, v)) return false;
+    if (tune().wgphase >= 0) return tune().wgphase != 0;
+    if (use_f16_mfma(p, PHX_PASS_BWD_WEIGHTS) && !wgrad_on_f16_mfma(p)) return true;
+    const double flops = 32.0 * p.n * p.ci * p.co * p.ho * p.wo * p.kh * p.kw;
+    return flops >= 200e9;
+}
+
+// the unit-stride problem of one class, its gathered input extent and the first tap's offset in the filter (elements)
+static Problem wgrad_class_problem(const Problem& p, const TapClass& ch, const TapClass& cw, long& tap_offset) {
+    Problem q = p;
+    q.nhwc = false;
+    q.h = ch.size; q.w = cw.size; q.kh = ch.taps; q.kw = cw.taps; q.sh = q.sw = 1; q.dh = ch.dil; q.dw = cw.dil;
+    q.pt = q.pl = q.pb = q.pr = 0;
+    q.fs.skh = p.fs.skh * ch.kstep; q.fs.skw = p.fs.skw * cw.kstep;
+    tap_offset = ch.k0 * p.fs.skh + cw.k0 * p.fs.skw;
+    return q;
+}
+
 // Reduction slices of a forward / input-gradient pass.  Those kernels give a workgroup an output tile and the whole
 // reduction over channels and taps, so a pass with few output tiles and many channels (small batches on deep
 // layers: 512 channels at 7x7, N=1 is 16 workgroups of 288 steps) leaves most of the GPU idle however long it
@@ -1720,6 +1777,19 @@ struct SlicedCorr {
 static size_t workspace_for(const Problem& p, int pass) {
     DilationView dilated;
     if (dilation_view(p, pass, dilated)) return dilated.x_bytes + dilated.y_bytes + workspace_for(dilated.q, pass);
+    if (pass == PHX_PASS_BWD_WEIGHTS && wgrad_by_classes(p)) {  // the largest class: its gathered input + its own workspace
+        TapClass ch[TAP_CLASSES_MAX], cw[TAP_CLASSES_MAX];
+        const int nh = tap_classes(p.kh, p.dh, p.sh, p.pt, p.ho, ch), nw = tap_classes(p.kw, p.dw, p.sw, p.pl, p.wo, cw);
+        const size_t esize = p.dtype == PHX_F32 ? 4 : 2;
+        size_t most = 0;
+        for (int a = 0; a < nh; ++a)
+            for (int b = 0; b < nw; ++b) {
+                long tap_offset = 0;
+                const Problem q = wgrad_class_problem(p, ch[a], cw[b], tap_offset);
+                most = std::max(most, align_up((size_t)4 * p.n * p.ci * q.h * q.w * esize, 256) + workspace_for(q, pass));
+            }
+        return most;
+    }
     S2dView v;
     if (pass != PHX_PASS_BWD_DATA && s2d_view(p, v)) return v.x2_bytes + v.w2_bytes + workspace_plain(v.q, pass);
     Problem q;
@@ -1933,6 +2003,29 @@ static int do_bwd_weights(const Problem& p, hipStream_t st, const void* x, const
         const int rc = do_bwd_weights(dilated.q, st, x2, g2, dw, g2 + dilated.y_bytes, wsb - tensors);
         g_name_prefix = "";
         return rc;
+    }
+    if (wgrad_by_classes(p)) {
+        TapClass ch[TAP_CLASSES_MAX], cw[TAP_CLASSES_MAX];
+        const int nh = tap_classes(p.kh, p.dh, p.sh, p.pt, p.ho, ch), nw = tap_classes(p.kw, p.dw, p.sw, p.pl, p.wo, cw);
+        const size_t esize = p.dtype == PHX_F32 ? 4 : 2;
+        for (int a = 0; a < nh; ++a)
+            for (int b = 0; b < nw; ++b) {
+                long tap_offset = 0;
+                const Problem q = wgrad_class_problem(p, ch[a], cw[b], tap_offset);
+                const size_t xg_bytes = align_up((size_t)4 * p.n * p.ci * q.h * q.w * esize, 256);
+                if (wsb < xg_bytes || !ws) return PHX_ERR_WORKSPACE;
+                StridedGatherArgs ga;
+                ga.src = x; ga.dst = ws; ga.planes = 4L * p.n * p.ci; ga.H = p.h; ga.W = p.w; ga.H2 = q.h; ga.W2 = q.w;
+                ga.sh = p.sh; ga.sw = p.sw; ga.oh = ch[a].origin; ga.ow = cw[b].origin;
+                launch_strided_gather(p.dtype == PHX_F16, ga, st);
+                PHX_HIP(hipGetLastError());
+                g_name_prefix = "class_";
+                const int rc = do_bwd_weights(q, st, ws, g, static_cast<char*>(dw) + tap_offset * (long)esize, static_cast<char*>(ws) + xg_bytes,
+                                              wsb - xg_bytes);
+                g_name_prefix = "";
+                if (rc != PHX_OK) return rc;
+            }
+        return PHX_OK;
     }
     S2dView v;
     if (s2d_view(p, v)) {

@@ -748,6 +748,50 @@ def test_large_dilations_on_channels_last_tensors(case, dtype, policy, tune_env)
     assert_close(dw.cpu().numpy().transpose(0, 1, 4, 2, 3), want_dw, dtype, "wgrad " + names[2])
 
 
+TAP_CLASSES = [
+    # name, n, ci, co, h, w, kh, kw, stride, dilation, padding
+    ("k3_s2", 2, 40, 72, 15, 18, 3, 3, 2, 1, "SAME"),                      # classes of 2x2, 2x1, 1x2 and 1x1 taps
+    ("k3_s3", 2, 16, 24, 20, 19, 3, 3, 3, 1, "SAME"),                      # every tap a class of its own
+    ("k5_s2_valid", 1, 8, 16, 17, 16, 5, 5, 2, 1, "VALID"),                # 3x3, 3x2, 2x3, 2x2
+    ("k4_s2x1", 2, 8, 8, 13, 11, 4, 4, (2, 1), 1, (1, 2, 2, 1)),           # one strided axis
+    ("k3_s3x2_d2", 1, 8, 16, 25, 22, 3, 3, (3, 2), 2, "SAME"),             # dilation 2 under stride 2: all taps of a row in one class, dilation 1
+    ("k7_s4", 1, 4, 8, 40, 37, 7, 7, 4, 1, (3, 0, 2, 5)),                  # classes of two and of one tap; the origin in the padding
+    ("k2_s2", 2, 16, 16, 12, 12, 2, 2, 2, 1, "VALID"),                     # four classes of one tap
+    ("k3_s5", 1, 8, 8, 23, 23, 3, 3, 5, 1, "SAME"),                        # the stride beyond the filter
+    ("k3x5_s2_d3", 1, 8, 8, 26, 31, 3, 5, 2, 3, "SAME"),                   # odd dilation under stride 2: classes alternate, dilation 3 inside
+]
+
+
+@pytest.mark.parametrize("dtype,policy", [(torch.float32, "fp32"), (torch.float16, "full16"), (torch.float16, "backward32")],
+                         ids=["f32", "f16_full16", "f16_backward32"])
+@pytest.mark.parametrize("mode", [16, 8])
+@pytest.mark.parametrize("case", TAP_CLASSES, ids=lambda c: c[0])
+def test_strided_filter_gradients_run_by_tap_classes(case, mode, dtype, policy, tune_env):
+    """Along an axis, the taps whose input rows share a residue modulo the stride read a subsampled copy of the input
+    with unit stride: the filter gradient of a strided convolution is at most sh x sw unit-stride filter gradients,
+    each behind one gather, each written to its own taps of dw.  Forced for every case (PHX_TUNE_WGPHASE=1) and off
+    (=0), against the oracle; by default for strides along W beyond 2 on fp16 matrix cores, which have no strided kernel."""
+    name, n, ci, co, h, w, kh, kw, stride, dilation, padding = case
+    scale = 1.0 if dtype == torch.float32 else 0.5
+    g, x, wt, b, gr = make_inputs(name_seed(name) + 95, n, ci, co, h, w, kh, kw, stride, dilation, padding, dtype, scale)
+    desc = phx.Conv2DDescriptor(x.shape, wt.shape, stride, dilation, padding, dtype=dtype, context=Ctx(mode, policy))
+    xd, gd = (torch.from_numpy(a).cuda() for a in (x, gr))
+    want_dw, _ = oracle.conv2d_bwd(g, x.astype(np.float64), wt.astype(np.float64), gr.astype(np.float64), "hamilton")
+    sw = stride[1] if isinstance(stride, tuple) else stride
+    for setting in ("1", "0", None):
+        tune_env(PHX_TUNE_WGPHASE=setting, PHX_TUNE_THIN_MAX32="0")
+        # (every tap must be written by its class: the block that the result is about to be allocated from holds NaNs)
+        poison = torch.full(wt.shape, float("nan"), dtype=dtype, device="cuda")
+        del poison
+        got = ops.conv2d_bwd_weights(xd, gd, desc)
+        k_wg = capi.last_kernel_name()
+        by_default = policy == "full16" and sw > 2
+        assert k_wg.startswith("class_") == (setting == "1" or (setting is None and by_default)), (setting, k_wg)
+        if by_default and setting != "0":
+            assert "f16mfma" in k_wg, k_wg  # (not the fp32 arithmetic the strided problem falls to)
+        assert_close(got.cpu().numpy(), want_dw, dtype, "wgrad %s %s" % (setting, k_wg))
+
+
 DIRECT_CASES = ("pw_ragged", "k3_same", "k3_ragged", "k3_s2", "pw_s31", "k7_s2", "k5_s2_valid", "k3_dil2", "k32_asym", "k7_s2_dil2")
 
 
