@@ -2008,12 +2008,13 @@ static int do_bwd_weights(const Problem& p, hipStream_t st, const void* x, const
         TapClass ch[TAP_CLASSES_MAX], cw[TAP_CLASSES_MAX];
         const int nh = tap_classes(p.kh, p.dh, p.sh, p.pt, p.ho, ch), nw = tap_classes(p.kw, p.dw, p.sw, p.pl, p.wo, cw);
         const size_t esize = p.dtype == PHX_F32 ? 4 : 2;
+        // (refused as a whole: a class that ran would have written its taps of dw)
+        if (wsb < workspace_for(p, PHX_PASS_BWD_WEIGHTS) || !ws) return PHX_ERR_WORKSPACE;
         for (int a = 0; a < nh; ++a)
             for (int b = 0; b < nw; ++b) {
                 long tap_offset = 0;
                 const Problem q = wgrad_class_problem(p, ch[a], cw[b], tap_offset);
                 const size_t xg_bytes = align_up((size_t)4 * p.n * p.ci * q.h * q.w * esize, 256);
-                if (wsb < xg_bytes || !ws) return PHX_ERR_WORKSPACE;
                 StridedGatherArgs ga;
                 ga.src = x; ga.dst = ws; ga.planes = 4L * p.n * p.ci; ga.H = p.h; ga.W = p.w; ga.H2 = q.h; ga.W2 = q.w;
                 ga.sh = p.sh; ga.sw = p.sw; ga.oh = ch[a].origin; ga.ow = cw[b].origin;

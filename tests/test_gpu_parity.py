@@ -792,6 +792,53 @@ def test_strided_filter_gradients_run_by_tap_classes(case, mode, dtype, policy, 
         assert_close(got.cpu().numpy(), want_dw, dtype, "wgrad %s %s" % (setting, k_wg))
 
 
+REWRITTEN = [
+    # what, n, ci, co, h, w, k, stride, dilation, channels-last
+    ("reduction slices", 1, 128, 128, 7, 7, 3, 1, 1, False),
+    ("reduction slices on the channels-last pointwise kernel", 1, 512, 64, 8, 8, 1, 1, 1, True),
+    ("dilation phases", 2, 24, 40, 33, 33, 3, 1, 12, False),
+    ("dilation phases of a channels-last call", 1, 16, 16, 20, 20, 3, 1, 9, True),
+    ("tap classes", 1, 16, 24, 20, 19, 3, 3, 1, False),
+    ("phases of a strided input gradient, sliced", 1, 128, 128, 14, 14, 3, 2, 1, False),
+]
+
+
+@pytest.mark.parametrize("dtype,policy", [(torch.float32, "fp32"), (torch.float16, "full16")], ids=["f32", "f16_full16"])
+@pytest.mark.parametrize("case", REWRITTEN, ids=lambda c: c[0].replace(" ", "_").replace(",", ""))
+def test_rewritten_problems_refuse_a_workspace_that_is_too_small(case, dtype, policy):
+    """The rewritten problems keep partial results, phase images or gathered inputs in the caller's workspace: with
+    256 bytes less than phx_qconv2d_workspace_bytes answers, each pass is refused (PHX_ERR_WORKSPACE) before anything
+    that would write past the end runs, and the outputs stay as they were; with the full size it runs."""
+    what, n, ci, co, h, w, k, stride, dilation, cl = case
+    xs = (4 * n, h, w, ci) if cl else (4 * n, ci, h, w)
+    desc = phx.Conv2DDescriptor(xs, (4, co, ci, k, k), stride, dilation, "SAME", dtype=dtype, context=Ctx(8, policy),
+                                data_format="NHWC" if cl else "NCHW")
+    x = torch.randn(xs, device="cuda").to(dtype)
+    wt = torch.randn(4, co, ci, k, k, device="cuda").to(dtype)
+    g = torch.randn(desc.output_shape, device="cuda").to(dtype)
+    L = capi.lib()
+    d = ctypes.byref(desc.c)
+    calls = {
+        capi.PHX_PASS_FWD: (desc.output_shape, lambda out, ws, nb: L.phx_qconv2d_fwd(d, None, x.data_ptr(), wt.data_ptr(), None, out.data_ptr(), ws.data_ptr(), nb)),
+        capi.PHX_PASS_BWD_DATA: (xs, lambda out, ws, nb: L.phx_qconv2d_bwd_data(d, None, g.data_ptr(), wt.data_ptr(), out.data_ptr(), ws.data_ptr(), nb)),
+        capi.PHX_PASS_BWD_WEIGHTS: (wt.shape, lambda out, ws, nb: L.phx_qconv2d_bwd_weights(d, None, x.data_ptr(), g.data_ptr(), out.data_ptr(), ws.data_ptr(), nb)),
+    }
+    grown = 0
+    for which, (shape, call) in calls.items():
+        need = desc.workspace_bytes(which)
+        ws = torch.empty(max(need, 256), dtype=torch.uint8, device="cuda")
+        out = torch.full(shape, 7.0, dtype=dtype, device="cuda")
+        if need >= 512:
+            assert call(out, ws, need - 256) == capi.PHX_ERR_WORKSPACE, (what, which)
+            torch.cuda.synchronize()
+            assert bool((out == 7.0).all()), (what, which)
+        assert call(out, ws, need) == capi.PHX_OK, (what, which)
+        torch.cuda.synchronize()
+        assert bool(torch.isfinite(out.float()).all()) and not bool((out == 7.0).all())
+        grown += need
+    assert grown > 0
+
+
 DIRECT_CASES = ("pw_ragged", "k3_same", "k3_ragged", "k3_s2", "pw_s31", "k7_s2", "k5_s2_valid", "k3_dil2", "k32_asym", "k7_s2_dil2")
 
 
