@@ -44,6 +44,10 @@ GROUPED = {
     "x_depthwise_k3_f16_128_28": (32, 128, 128, 28, 28, 3, "SAME", "f16", 128),
     "x_depthwise_k3_f16_256_14": (64, 256, 256, 14, 14, 3, "SAME", "f16", 256),
     "x_groups32_k3_f16_128_28": (32, 128, 128, 28, 28, 3, "SAME", "f16", 32),
+    # (..., groups, stride, dilation): shapes that run as rewritten problems
+    "x_smallbatch_k3_f16_512_7": (1, 512, 512, 7, 7, 3, "SAME", "f16", 1, 1, 1),       # reduction slices
+    "x_atrous_k3_d12_f16_512_64_33": (8, 512, 64, 33, 33, 3, "SAME", "f16", 1, 1, 12),  # dilation phases
+    "x_stride3_k3_f16_128_28": (32, 128, 128, 28, 28, 3, "SAME", "f16", 1, 3, 1),       # filter gradient by tap classes
 }
 DENSE = {"c1_dense_f32": (32, 128, 128, "f32")}  # name: (n, in, out, dtype)
 RESNET = "c5_qresnet50"  # quaternion ResNet-50 forward+backward, N=64, 224x224, fp16 full16 policy
@@ -350,6 +354,7 @@ def run_conv(name, mode, policy, args, traffic_table):
     from phoenix_core_amd import capi
     n, ci, co, h, w, k, padding, dt = (CONVS.get(name) or GROUPED[name])[:8]
     groups = GROUPED[name][8] if name in GROUPED else 1
+    stride, dilation = GROUPED[name][9:11] if name in GROUPED and len(GROUPED[name]) > 9 else (1, 1)
     if dt == "f32":
         policy = "fp32"
     ctx = make_context(mode, policy)
@@ -360,7 +365,7 @@ def run_conv(name, mode, policy, args, traffic_table):
     cl = bool(getattr(args, "channels_last", False))
     x = (scale * torch.randn((4 * n, h, w, ci) if cl else (4 * n, ci, h, w), device=dev)).to(dtype)
     wt = (scale * torch.randn(4, co, ci // groups, k, k, device=dev) * (2.0 / (ci // groups * k * k)) ** 0.5).to(dtype)
-    desc = phx.Conv2DDescriptor(x.shape, wt.shape, 1, 1, padding, groups=groups, dtype=dtype, context=ctx,
+    desc = phx.Conv2DDescriptor(x.shape, wt.shape, stride, dilation, padding, groups=groups, dtype=dtype, context=ctx,
                                 data_format="NHWC" if cl else "NCHW")
     gr = (scale * torch.randn(desc.output_shape, device=dev)).to(dtype)
     ho, wo = desc.output_shape[1:3] if cl else desc.output_shape[2:]
@@ -408,8 +413,9 @@ def run_conv(name, mode, policy, args, traffic_table):
     del x, wt, gr, y, dx, dw, ws
     torch.cuda.empty_cache()
     return {
-        "workload": "%s: quaternion conv %dx%d stride 1, N=%d (4N=%d rows), %d->%d q-channels%s, %dx%d, "
-                    "fwd+input-grad+filter-grad%s" % (name, k, k, n, 4 * n, ci, co, " in %d groups" % groups if groups > 1 else "", h, w,
+        "workload": "%s: quaternion conv %dx%d stride %d%s, N=%d (4N=%d rows), %d->%d q-channels%s, %dx%d, "
+                    "fwd+input-grad+filter-grad%s" % (name, k, k, stride, " dilation %d" % dilation if dilation > 1 else "", n, 4 * n, ci, co,
+                                                      " in %d groups" % groups if groups > 1 else "", h, w,
                                                       ", channels-last activations" if cl else ""),
         "data_format": "NHWC" if cl else "NCHW",
         "n": n, "product_mode": mode, "fp16_policy": policy, "padding": padding, "dtype": dt,
