@@ -77,6 +77,82 @@ __global__ void __launch_bounds__(WG_THREADS) strided_gather_kernel(const Stride
     }
 }
 
+// Patches to depth.  A convolution whose stride equals its filter extent (patch embeddings, 2x2 / stride 2
+// downsampling) reads every input position once, for one output position: with the kh x kw positions of a patch
+// laid out as channels,
+//   patches[row][q][i][j] = x[row][c][i * kh + a][j * kw + b]   (zero outside the image),
+//   q = (c * kh + a) * kw + b (tap_major == 0) or (a * kw + b) * C + c (tap_major == 1),
+// it is a pointwise convolution over C * kh * kw channels.  to_caller copies the other way and zeroes the positions
+// of the caller's tensor that no patch holds (rows and columns behind the last whole patch).
+struct PatchArgs {
+    const void* src;
+    void* dst;
+    long rows;          // components x images
+    int C, H, W;        // channels and extent of the caller's tensor
+    int Ho, Wo;         // patches per column / row
+    int kh, kw;
+    int tap_major;
+};
+
+// (a workgroup works on whole planes -- one patch channel of one row, or one channel of the caller's tensor -- so that
+// the channel and tap of a plane are decoded once and a position costs one division)
+template <typename TS>
+__global__ void __launch_bounds__(WG_THREADS) patch_depth_kernel(const PatchArgs A, int to_caller) {
+    const int Cq = A.C * A.kh * A.kw;
+    if (!to_caller && (long)A.Ho * A.Wo < 512) {  // small patch planes: one position per thread, whatever its plane
+        const TS* x = static_cast<const TS*>(A.src);
+        TS* pt = static_cast<TS*>(A.dst);
+        const long total = A.rows * Cq * A.Ho * A.Wo;
+        for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
+            const int j = idx % A.Wo;
+            long rest = idx / A.Wo;
+            const int i = rest % A.Ho; rest /= A.Ho;
+            const int q = rest % Cq;
+            const long row = rest / Cq;
+            int c, a, b;
+            if (A.tap_major) { c = q % A.C; b = (q / A.C) % A.kw; a = q / (A.C * A.kw); }
+            else { b = q % A.kw; a = (q / A.kw) % A.kh; c = q / (A.kw * A.kh); }
+            const int yi = i * A.kh + a, xj = j * A.kw + b;
+            pt[idx] = (yi < A.H && xj < A.W) ? x[((row * A.C + c) * A.H + yi) * A.W + xj] : (TS)0;
+        }
+    } else if (!to_caller) {
+        const TS* x = static_cast<const TS*>(A.src);
+        TS* pt = static_cast<TS*>(A.dst);
+        const int plane = A.Ho * A.Wo;
+        for (long pl = blockIdx.x; pl < A.rows * Cq; pl += gridDim.x) {
+            const int q = pl % Cq;
+            const long row = pl / Cq;
+            int c, a, b;
+            if (A.tap_major) { c = q % A.C; b = (q / A.C) % A.kw; a = q / (A.C * A.kw); }
+            else { b = q % A.kw; a = (q / A.kw) % A.kh; c = q / (A.kw * A.kh); }
+            const TS* src = x + (row * A.C + c) * (long)A.H * A.W;
+            TS* dst = pt + pl * plane;
+            for (int t = threadIdx.x; t < plane; t += blockDim.x) {
+                const int i = t / A.Wo, j = t - i * A.Wo;
+                const int yi = i * A.kh + a, xj = j * A.kw + b;
+                dst[t] = (yi < A.H && xj < A.W) ? src[(long)yi * A.W + xj] : (TS)0;
+            }
+        }
+    } else {
+        const TS* pt = static_cast<const TS*>(A.src);
+        TS* x = static_cast<TS*>(A.dst);
+        const int plane = A.H * A.W;
+        const long patch_plane = (long)A.Ho * A.Wo;
+        for (long pl = blockIdx.x; pl < A.rows * A.C; pl += gridDim.x) {
+            const int c = pl % A.C;
+            const long row = pl / A.C;
+            const TS* src = pt + row * Cq * patch_plane;
+            TS* dst = x + pl * plane;
+            for (int t = threadIdx.x; t < plane; t += blockDim.x) {
+                const int yi = t / A.W, xj = t - yi * A.W;
+                const int i = yi / A.kh, a = yi - i * A.kh, j = xj / A.kw, b = xj - j * A.kw;
+                const int q = A.tap_major ? (a * A.kw + b) * A.C + c : (c * A.kh + a) * A.kw + b;
+                dst[t] = (i < A.Ho && j < A.Wo) ? src[(q * (long)A.Ho + i) * A.Wo + j] : (TS)0;
+            }
+        }
+    }
+}
+
 // Dilation phases.  With unit stride, an output position and every input position it reads lie dh rows and dw columns
 // apart: counted from an origin (oh, ow) = padding before the image modulo the dilation in front of the input (from
 // the first position of the output), they share their row modulo dh and their column modulo dw.  The convolution is

@@ -140,6 +140,7 @@ int thin_wgrad_slices(bool half_storage, const ThinArgs& a);  // Z of the filter
 // space-to-depth rearrangements (stride-2 convolutions with very few input channels)
 int launch_s2d_input(bool half_storage, const S2dArgs& a, hipStream_t st);
 int launch_subsample(bool half_storage, const SubsampleArgs& a, hipStream_t st);
+int launch_patch_depth(bool half_storage, const PatchArgs& a, bool to_caller, hipStream_t st);  // the patches of a stride == filter convolution as channels
 int launch_strided_gather(bool half_storage, const StridedGatherArgs& a, hipStream_t st);  // the input positions of one residue class of taps
 int launch_dilation_phases(bool half_storage, const DilationPhaseArgs& a, bool to_caller, hipStream_t st);  // phase images of a dilated convolution
 int launch_s2d_filter(bool half_storage, const S2dFilterArgs& a, bool to_caller, hipStream_t st);

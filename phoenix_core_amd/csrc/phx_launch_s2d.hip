@@ -28,6 +28,16 @@ int launch_s2d_input(bool half_storage, const S2dArgs& a, hipStream_t st) {
     return 0;
 }
 
+int launch_patch_depth(bool half_storage, const PatchArgs& a, bool to_caller, hipStream_t st) {
+    const long planes = to_caller ? a.rows * a.C : a.rows * a.C * a.kh * a.kw;  // one workgroup each (the surplus in turns)
+    if (planes <= 0 || (long)a.H * a.W <= 0) return 0;
+    const bool per_position = !to_caller && (long)a.Ho * a.Wo < 512;  // (the kernel's rule)
+    const dim3 grid(per_position ? (unsigned int)blocks_for(planes * a.Ho * a.Wo) : (unsigned int)std::min<long>(planes, 1 << 18));
+    if (half_storage) hipLaunchKernelGGL((patch_depth_kernel<_Float16>), grid, dim3(WG_THREADS), 0, st, a, (int)to_caller);
+    else hipLaunchKernelGGL((patch_depth_kernel<float>), grid, dim3(WG_THREADS), 0, st, a, (int)to_caller);
+    return 0;
+}
+
 int launch_strided_gather(bool half_storage, const StridedGatherArgs& a, hipStream_t st) {
     const long items = a.planes * a.H2 * a.W2;
     if (items <= 0) return 0;

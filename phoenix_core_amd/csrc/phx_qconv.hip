@@ -40,6 +40,8 @@ struct Tuning {
     int thin_max = 4;                 // PHX_TUNE_THIN_MAX: most input x output channels per group that run on the vector-ALU kernels for thin groups (0 = never)
     int dilphase_min = 160;           // PHX_TUNE_DILPHASE_MIN: forward / input-gradient passes whose dilated window has more positions than this run by dilation phases
     int wgphase = -1;                 // PHX_TUNE_WGPHASE: 1 = every strided filter gradient with several taps runs by tap classes, 0 = none (unset: wgrad_by_classes)
+    bool nopatch = false;             // PHX_TUNE_NOPATCH: convolutions whose stride equals their filter extent stay on the windowed kernels
+    bool patchall = false;            // PHX_TUNE_PATCHALL: every pass of every such convolution runs on patches (not only where that was measured to gain)
     bool nodilphase = false;          // PHX_TUNE_NODILPHASE: dilated convolutions beyond the staging limit stay on the vector-ALU kernels
     int kslices = -1;                 // PHX_TUNE_KSLICES: reduction slices of a forward / input-gradient pass (0 = never, unset = by the rule of corr_slices)
     bool nodensecl = false;           // PHX_TUNE_NODENSECL: Dense never runs as a channels-last pointwise convolution
@@ -84,6 +86,8 @@ struct Tuning {
         nodensecl = getenv("PHX_TUNE_NODENSECL") != nullptr;
         if (const char* e = getenv("PHX_TUNE_KSLICES")) kslices = atoi(e);
         nodilphase = getenv("PHX_TUNE_NODILPHASE") != nullptr;
+        nopatch = getenv("PHX_TUNE_NOPATCH") != nullptr;
+        patchall = getenv("PHX_TUNE_PATCHALL") != nullptr;
         if (const char* e = getenv("PHX_TUNE_WGPHASE")) wgphase = atoi(e) != 0;
         if (const char* e = getenv("PHX_TUNE_DILPHASE_MIN")) dilphase_min = atoi(e);
         nosmalldense = getenv("PHX_TUNE_NOSMALLDENSE") != nullptr;
@@ -1579,6 +1583,53 @@ static void subsample_input(const Problem& p, const void* x, void* xs, hipStream
 static long window_positions(const Problem& p) { return ((long)(p.kh - 1) * p.dh + 1) * ((((long)(p.kw - 1) * p.dw + 1) + 7) & ~7L); }
 static bool window_beyond_staging(const Problem& p) { return window_positions(p) > WG_THREADS; }
 
+// Convolutions whose stride equals their filter extent (patch embeddings: 16x16 stride 16; 2x2 stride 2 and 4x4
+// stride 4 downsampling), undilated, with no padding in front of the image: every input position belongs to one
+// output position, so with the positions of a patch laid out as channels (patch_depth_kernel) the convolution is a
+// POINTWISE one over ci * kh * kw channels on the ho x wo grid of patches -- all three passes, on the streaming
+// kernels, where the windowed kernels spend a window's worth of staging per output position and the input gradient
+// would multiply sh * sw - 1 inserted zeros for every value (16x16 stride 16 on 224x224 images: seconds).  The filter
+// is used as it lies: its taps and input channels form one channel index with one stride -- (c, kh, kw) in OIHW,
+// (kh, kw, c) in OHWI and HWIO -- and the filter gradient of the pointwise problem is written straight to it.
+// One gather in front of the forward pass and the filter gradient, one scatter behind the input gradient.
+struct PatchView {
+    Problem q;
+    int tap_major;
+    size_t x_bytes;  // the input-side tensor as patches
+};
+static bool patch_view(const Problem& p, int pass, PatchView& v) {
+    if (tune().nopatch || tune().direct || is_empty(p) || p.kh != p.sh || p.kw != p.sw || p.kh * p.kw == 1) return false;
+    if (p.dh != 1 || p.dw != 1 || p.pt || p.pl || channel_slices(p) || g_window_cl) return false;
+    // Patches of fewer than nine positions (2x2 stride 2): the windowed kernels' forward pass and fp16 filter gradient
+    // beat a gather plus the pointwise kernels (N=64, fp16, windowed / patches, us: 24 -> 48 channels at 56x56 forward
+    // 39 / 68, filter gradient 38 / 75; 128 -> 256 at 28x28 145 / 177, 118 / 190); the input gradient (zero insertion or
+    // four phases against one pointwise pass and a scatter: 99 / 71, 102 / 53) and the filter gradient in fp32 arithmetic
+    // (267 / 148) do not.  From 3x3 on every pass gains (4x4 stride 4, 32 -> 64 at 56x56: 45 / 141 / 258 -> 97 / 57 / 93).
+    if (p.kh * p.kw < 9 && !tune().patchall &&
+        (pass == PHX_PASS_FWD || (pass == PHX_PASS_BWD_WEIGHTS && use_f16_mfma(p, PHX_PASS_BWD_WEIGHTS) && wgrad_on_f16_mfma(p))))
+        return false;
+    const FilterStrides& f = p.fs;
+    long si = 0;
+    if (f.skh == p.kw * f.skw && f.si == (long)p.kh * p.kw * f.skw) { v.tap_major = 0; si = f.skw; }
+    else if (f.skw == p.ci * f.si && f.skh == (long)p.kw * p.ci * f.si) { v.tap_major = 1; si = f.si; }
+    else return false;
+    if ((long)p.ci * p.kh * p.kw > (1L << 20)) return false;
+    Problem& q = v.q;
+    q = p;
+    q.nhwc = false;  // (the patch tensor is channels-first)
+    q.ci = q.ci_mem = p.ci * p.kh * p.kw;
+    q.h = p.ho; q.w = p.wo; q.kh = q.kw = 1; q.sh = q.sw = 1; q.pt = q.pl = q.pb = q.pr = 0;
+    q.fs.si = si; q.fs.skh = q.fs.skw = 0;
+    v.x_bytes = align_up((size_t)(p.real_input ? 1 : 4) * p.n * q.ci * p.ho * p.wo * (p.dtype == PHX_F32 ? 4 : 2), 256);
+    return true;
+}
+static void patch_depth(const Problem& p, const PatchView& v, const void* src, void* dst, bool to_caller, hipStream_t st) {
+    PatchArgs a;
+    a.src = src; a.dst = dst; a.rows = (p.real_input ? 1L : 4L) * p.n; a.C = p.ci; a.H = p.h; a.W = p.w; a.Ho = p.ho; a.Wo = p.wo;
+    a.kh = p.kh; a.kw = p.kw; a.tap_major = v.tap_major;
+    launch_patch_depth(p.dtype == PHX_F16, a, to_caller, st);
+}
+
 // Dilated convolutions beyond that limit (a 3x3 filter from dilation 8 on: the atrous pyramids of segmentation
 // networks use 12, 18, 24, 36) with unit stride: an output position and every input position it reads lie whole
 // dilations apart, so the convolution is dh x dw independent undilated convolutions on the phase images of its
@@ -1775,6 +1826,8 @@ struct SlicedCorr {
 };
 
 static size_t workspace_for(const Problem& p, int pass) {
+    PatchView patches;
+    if (patch_view(p, pass, patches)) return patches.x_bytes + workspace_for(patches.q, pass);
     DilationView dilated;
     if (dilation_view(p, pass, dilated)) return dilated.x_bytes + dilated.y_bytes + workspace_for(dilated.q, pass);
     if (pass == PHX_PASS_BWD_WEIGHTS && wgrad_by_classes(p)) {  // the largest class: its gathered input + its own workspace
@@ -1862,6 +1915,18 @@ static int do_fwd(const Problem& p, hipStream_t st, const void* x, const void* w
     const bool dry = g_pack.dry();
     if (!dry && (!x || !w || !y || (p.has_bias && !bias))) return PHX_ERR_INVALID_ARGUMENT;
     const void* b = p.has_bias ? bias : nullptr;
+    PatchView patches;
+    if (patch_view(p, PHX_PASS_FWD, patches)) {
+        if (!dry && (wsb < patches.x_bytes || !ws)) return PHX_ERR_WORKSPACE;
+        if (!dry) {
+            patch_depth(p, patches, x, ws, false, st);
+            PHX_HIP(hipGetLastError());
+        }
+        g_name_prefix = "patch_";
+        const int rc = do_fwd(patches.q, st, ws, w, b, y, dry ? nullptr : static_cast<char*>(ws) + patches.x_bytes, dry ? 0 : wsb - patches.x_bytes);
+        g_name_prefix = "";
+        return rc;
+    }
     DilationView dilated;
     if (dilation_view(p, PHX_PASS_FWD, dilated)) {
         const size_t tensors = dilated.x_bytes + dilated.y_bytes;
@@ -1923,6 +1988,17 @@ static int do_bwd_data(const Problem& p, hipStream_t st, const void* g, const vo
     if (is_empty(p)) return PHX_OK;
     const bool dry = g_pack.dry();
     if (!dry && (!g || !w || !dx)) return PHX_ERR_INVALID_ARGUMENT;
+    PatchView patches;
+    if (patch_view(p, PHX_PASS_BWD_DATA, patches)) {
+        if (!dry && (wsb < patches.x_bytes || !ws)) return PHX_ERR_WORKSPACE;
+        g_name_prefix = "patch_";
+        const int rc = do_bwd_data(patches.q, st, g, w, ws, dry ? nullptr : static_cast<char*>(ws) + patches.x_bytes, dry ? 0 : wsb - patches.x_bytes);
+        g_name_prefix = "";
+        if (rc != PHX_OK || dry) return rc;
+        patch_depth(p, patches, ws, dx, true, st);
+        PHX_HIP(hipGetLastError());
+        return PHX_OK;
+    }
     DilationView dilated;
     if (dilation_view(p, PHX_PASS_BWD_DATA, dilated)) {
         const size_t tensors = dilated.x_bytes + dilated.y_bytes;
@@ -1990,6 +2066,16 @@ static int do_bwd_weights(const Problem& p, hipStream_t st, const void* x, const
         return PHX_OK;
     }
     if (!x || !g) return PHX_ERR_INVALID_ARGUMENT;
+    PatchView patches;
+    if (patch_view(p, PHX_PASS_BWD_WEIGHTS, patches)) {
+        if (wsb < patches.x_bytes || !ws) return PHX_ERR_WORKSPACE;
+        patch_depth(p, patches, x, ws, false, st);
+        PHX_HIP(hipGetLastError());
+        g_name_prefix = "patch_";
+        const int rc = do_bwd_weights(patches.q, st, ws, g, dw, static_cast<char*>(ws) + patches.x_bytes, wsb - patches.x_bytes);
+        g_name_prefix = "";
+        return rc;
+    }
     DilationView dilated;
     if (dilation_view(p, PHX_PASS_BWD_WEIGHTS, dilated)) {
         const size_t tensors = dilated.x_bytes + dilated.y_bytes;
@@ -2213,7 +2299,8 @@ static bool nhwc_window_native(const Problem& p, int pass) {
     Problem planes = p;
     planes.nhwc = false;
     DilationView dilated;
-    return corr_slices(planes, pass) == 0 && !dilation_view(planes, pass, dilated);
+    PatchView patches;
+    return corr_slices(planes, pass) == 0 && !dilation_view(planes, pass, dilated) && !patch_view(planes, pass, patches);
 }
 }  // namespace phx
 
@@ -2250,7 +2337,8 @@ static bool thin_groups(const Problem& p, int pass) {
     if ((long)p.kh * p.kw > 2048 || std::max(p.ci_mem, p.co_mem) > 65535) return false;  // (a filter chunk in LDS; grid rows)
     if (tune().direct) return true;
     DilationView dilated;
-    if (window_beyond_staging(p)) return !dilation_view(p, pass, dilated);
+    PatchView patches;
+    if (window_beyond_staging(p)) return !dilation_view(p, pass, dilated) && !patch_view(p, pass, patches);
     const long pairs = (long)p.ci * p.co;
     // The filter gradient in fp32 arithmetic works on 64 x 64 channel tiles whatever the layer holds: its time follows
     // the pixels and taps alone (3x3, 56x56, N=64: 1.39 ms from 8 to 64 channels), that of the vector-ALU kernel the

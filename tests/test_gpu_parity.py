@@ -779,7 +779,8 @@ def test_strided_filter_gradients_run_by_tap_classes(case, mode, dtype, policy, 
     want_dw, _ = oracle.conv2d_bwd(g, x.astype(np.float64), wt.astype(np.float64), gr.astype(np.float64), "hamilton")
     sw = stride[1] if isinstance(stride, tuple) else stride
     for setting in ("1", "0", None):
-        tune_env(PHX_TUNE_WGPHASE=setting, PHX_TUNE_THIN_MAX32="0")
+        # (NOPATCH: a stride equal to the filter extent would otherwise run on patches)
+        tune_env(PHX_TUNE_WGPHASE=setting, PHX_TUNE_THIN_MAX32="0", PHX_TUNE_NOPATCH="1")
         # (every tap must be written by its class: the block that the result is about to be allocated from holds NaNs)
         poison = torch.full(wt.shape, float("nan"), dtype=dtype, device="cuda")
         del poison
@@ -837,6 +838,80 @@ def test_rewritten_problems_refuse_a_workspace_that_is_too_small(case, dtype, po
         assert bool(torch.isfinite(out.float()).all()) and not bool((out == 7.0).all())
         grown += need
     assert grown > 0
+
+
+PATCHES = [
+    # name, n, ci, co, h, w, kh, kw, padding, filter layout, channels-last, real-valued input
+    ("down_k2", 2, 24, 40, 14, 18, 2, 2, "VALID", "OIHW", False, False),
+    ("down_k2_odd", 2, 16, 16, 15, 13, 2, 2, "VALID", "OIHW", False, False),          # a row and a column that no patch holds
+    ("down_k4_ohwi", 1, 8, 24, 16, 20, 4, 4, "VALID", "OHWI", False, False),
+    ("down_k3x2_hwio", 2, 8, 16, 12, 10, 3, 2, "VALID", "HWIO", False, False),
+    ("embed_k16_real", 1, 3, 24, 64, 48, 16, 16, "VALID", "OIHW", False, True),       # a patch embedding of real images
+    ("embed_k8", 1, 4, 16, 40, 40, 8, 8, "VALID", "OIHW", False, False),
+    ("down_k2_behind", 2, 8, 8, 9, 11, 2, 2, (0, 0, 1, 1), "OIHW", False, False),     # padding behind the image completes the last patches
+    ("down_k2_nhwc", 2, 16, 24, 12, 12, 2, 2, "VALID", "OHWI", True, False),
+    ("embed_k32", 1, 2, 8, 64, 96, 32, 32, "VALID", "OIHW", False, False),            # a window beyond the matrix-core kernels' staging
+]
+
+
+@pytest.mark.parametrize("dtype,policy", [(torch.float32, "fp32"), (torch.float16, "full16"), (torch.float16, "backward32")],
+                         ids=["f32", "f16_full16", "f16_backward32"])
+@pytest.mark.parametrize("mode", [16, 8])
+@pytest.mark.parametrize("case", PATCHES, ids=lambda c: c[0])
+def test_stride_equal_to_the_filter_runs_as_a_pointwise_convolution_on_patches(case, mode, dtype, policy, tune_env):
+    """Every input position of such a convolution belongs to one output position: with a patch's positions laid out
+    as channels it is a pointwise convolution (all three passes), the filter used as it lies.  Against the oracle, with
+    every pass on patches (PHX_TUNE_PATCHALL), with the passes that the rule sends there and with none
+    (PHX_TUNE_NOPATCH: the windowed kernels); prepacked filters bit for bit."""
+    name, n, ci, co, h, w, kh, kw, padding, layout, cl, real = case
+    scale = 1.0 if dtype == torch.float32 else 0.5
+    g, x, wt, b, gr = make_inputs(name_seed(name) + 97, n, ci, co, h, w, kh, kw, (kh, kw), 1, padding, dtype, scale)
+    if real:
+        x[n:] = 0
+    w_dev = wt if layout == "OIHW" else np.ascontiguousarray(wt.transpose(0, 1, 3, 4, 2)) if layout == "OHWI" else np.ascontiguousarray(wt.transpose(0, 3, 4, 2, 1))
+    x_dev = x[:n] if real else x
+    x_dev = np.ascontiguousarray(x_dev.transpose(0, 2, 3, 1)) if cl else np.ascontiguousarray(x_dev)
+    g_dev = np.ascontiguousarray(gr.transpose(0, 2, 3, 1)) if cl else gr
+    desc = phx.Conv2DDescriptor(x_dev.shape, w_dev.shape, (kh, kw), 1, padding, use_bias=not real, dtype=dtype, filter_layout=layout,
+                                context=Ctx(mode, policy), data_format="NHWC" if cl else "NCHW", real_valued_input=real,
+                                require_input_grad=not real)
+    xd, wd, bd, gd = (torch.from_numpy(a).cuda() for a in (x_dev, w_dev, b, g_dev))
+    x64, w64, b64, g64 = (a.astype(np.float64) for a in (x, wt, b, gr))
+    want_y = oracle.conv2d_fwd(g, x64, w64, None if real else b64, "hamilton")
+    want_dw, want_dx = oracle.conv2d_bwd(g, x64, w64, g64, "hamilton")
+    back = (lambda a: a.transpose(0, 3, 1, 2)) if cl else (lambda a: a)
+    w_back = (lambda a: a) if layout == "OIHW" else (lambda a: a.transpose(0, 1, 4, 2, 3)) if layout == "OHWI" else (lambda a: a.transpose(0, 4, 3, 1, 2))
+    for setting in ("all", "rule", "off"):
+        patches = setting == "all"
+        tune_env(PHX_TUNE_NOPATCH="1" if setting == "off" else None, PHX_TUNE_PATCHALL="1" if patches else None, PHX_TUNE_THIN_MAX32="0")
+        y = phx.conv2d_fwd(xd, wd, None if real else bd, desc)
+        names = [capi.last_kernel_name()]
+        assert_close(back(y.cpu().numpy()), want_y, dtype, "fwd " + names[0])
+        if not real:
+            dx = ops.conv2d_bwd_data(wd, gd, desc)
+            names.append(capi.last_kernel_name())
+            assert_close(back(dx.cpu().numpy()), want_dx, dtype, "dgrad " + names[1])
+        poison = torch.full(wd.shape, float("nan"), dtype=dtype, device="cuda")
+        del poison
+        dw = ops.conv2d_bwd_weights(xd, gd, desc)
+        names.append(capi.last_kernel_name())
+        assert_close(w_back(dw.cpu().numpy()), want_dw, dtype, "wgrad " + names[-1])
+        if setting == "rule":
+            # patches of at least nine positions: every pass; smaller ones: the input gradient, and the filter gradient
+            # where it runs in fp32 arithmetic
+            big = kh * kw >= 9
+            fp32_wgrad = dtype == torch.float32 or policy == "backward32"
+            want = [big] + ([] if real else [True]) + [big or fp32_wgrad]
+            assert [k.startswith("patch_") for k in names] == want, names
+        else:
+            assert all(k.startswith("patch_") == patches for k in names), names
+        if patches:
+            packed = ops.conv2d_pack_filters(wd, desc, bwd_data=not real)
+            if packed is not None:
+                zero = torch.zeros_like(wd)
+                assert torch.equal(phx.conv2d_fwd(xd, zero, None if real else bd, desc, packed=packed), y), "prepacked fwd"
+                if not real:
+                    assert torch.equal(ops.conv2d_bwd_data(zero, gd, desc, packed=packed), dx), "prepacked dgrad"
 
 
 DIRECT_CASES = ("pw_ragged", "k3_same", "k3_ragged", "k3_s2", "pw_s31", "k7_s2", "k5_s2_valid", "k3_dil2", "k32_asym", "k7_s2_dil2")
