@@ -287,7 +287,7 @@ __global__ void __launch_bounds__(WG_THREADS) s2d_filter_kernel(const S2dFilterA
 struct PhaseMergeArgs {
     const void* buf;      // start of the phase buffers
     void* dx;
-    long off[16];         // element offset of each phase buffer, -1 = all zero
+    long off[64];         // element offset of each phase buffer (a * sw + b), -1 = all zero
     long planes;          // 4N * C
     int H, W, sh, sw;
 };

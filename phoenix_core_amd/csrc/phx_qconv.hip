@@ -1464,10 +1464,17 @@ static PhaseAxis phase_axis(int a, int extent, int k, int d, int s, int pad_befo
 // each, and the zero-insertion form on the LDS kernel is the faster one at the sizes measured
 // (3x3 stride 2, 32-128 channels: 0.08-0.11 ms against 0.13-0.19 ms); PHX_TUNE_PHASE=1 sends every strided
 // input gradient through the phases, PHX_TUNE_PHASE=0 none.
+constexpr int PHASES_MAX = 64;  // strides up to 8 x 8 (PhaseMergeArgs::off)
 static bool dgrad_by_phases(const Problem& p) {
-    if ((p.sh == 1 && p.sw == 1) || p.sh * p.sw > 16 || is_empty(p) || channel_slices(p)) return false;
+    if ((p.sh == 1 && p.sw == 1) || p.sh * p.sw > PHASES_MAX || is_empty(p) || channel_slices(p)) return false;
     if (tune().phase >= 0) return tune().phase != 0;
     if (p.kh == 1 && p.kw == 1) return true;
+    // The largest windows (overlapping patch embeddings: 16x16 stride 8): the zero-inserted form stages the whole filter
+    // window around every output position, and at the staging limit a tile is next to no outputs, while a phase has
+    // ceil(k / s) taps per axis: 8 -> 32 channels at 64x64, N=2 4.65 ms against 1.09 ms for 64 launches of a 2x2 filter.
+    // (Smaller windows keep the zero insertion at such sizes: 12x12 stride 6 0.34 against 0.59 ms, 11x11 stride 4 0.10
+    // against 0.29 -- a phase is a packing and a convolution launch of some 8 us each.)
+    if (((long)(p.kh - 1) * p.dh + 1) * ((((long)(p.kw - 1) * p.dw + 1) + 7) & ~7L) > 224) return true;
     // Large problems: zero insertion multiplies the arithmetic by sh * sw, which the launches of the phases cost less
     // than once there is enough of it and the phases' images are not tiny (fp16, N=64, 3x3 stride 2, zero insertion
     // against phases: 128 channels at 28x28 261 / 197 us, 256 at 28x28 967 / 509, 512 at 14x14 1064 / 611, 5x5 256 at
@@ -2022,7 +2029,7 @@ static int do_bwd_data(const Problem& p, hipStream_t st, const void* g, const vo
         PhaseMergeArgs m;
         m.buf = ws; m.dx = dx; m.planes = 4L * p.n * p.ci; m.H = p.h; m.W = p.w; m.sh = p.sh; m.sw = p.sw;
         size_t bufs = 0;
-        for (int i = 0; i < 16; ++i) m.off[i] = -1;
+        for (int i = 0; i < PHASES_MAX; ++i) m.off[i] = -1;
         for (int a = 0; a < p.sh; ++a)
             for (int b = 0; b < p.sw; ++b) {
                 const PhaseAxis ah = phase_axis(a, p.h, p.kh, p.dh, p.sh, p.pt), aw = phase_axis(b, p.w, p.kw, p.dw, p.sw, p.pl);

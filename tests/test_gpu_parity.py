@@ -68,6 +68,8 @@ CONV_CASES = [
     ("k3_s2", 2, 8, 16, 15, 14, 3, 3, 2, 1, "SAME"),
     ("pw_s2", 2, 8, 16, 14, 14, 1, 1, 2, 1, "VALID"),
     ("pw_s2_odd", 3, 10, 12, 15, 13, 1, 1, 2, 1, "VALID"),    # strided pointwise: runs on a subsampled copy of the input
+    ("k16_s8", 1, 4, 8, 40, 44, 16, 16, 8, 1, "SAME"),        # an overlapping patch embedding: the input gradient by 64 phases of 2x2 taps
+    ("k15x3_s6x7", 1, 4, 4, 50, 30, 15, 3, (6, 7), 1, "VALID"),  # 42 phases, some of them without a tap
     ("pw_s31", 2, 6, 9, 10, 27, 1, 1, (3, 1), 1, "VALID"),
     ("k7_s2", 1, 3, 16, 30, 30, 7, 7, 2, 1, "SAME"),
     ("k3_s2_c4", 2, 4, 8, 15, 13, 3, 3, 2, 1, "SAME"),       # few input channels, stride 2: space-to-depth path
