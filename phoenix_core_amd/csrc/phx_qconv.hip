@@ -40,6 +40,7 @@ struct Tuning {
     int thin_max = 4;                 // PHX_TUNE_THIN_MAX: most input x output channels per group that run on the vector-ALU kernels for thin groups (0 = never)
     int dilphase_min = 160;           // PHX_TUNE_DILPHASE_MIN: forward / input-gradient passes whose dilated window has more positions than this run by dilation phases
     int wgphase = -1;                 // PHX_TUNE_WGPHASE: 1 = every strided filter gradient with several taps runs by tap classes, 0 = none (unset: wgrad_by_classes)
+    bool nobands = false;             // PHX_TUNE_NOBANDS: large filter windows are not cut into tap bands
     bool nopatch = false;             // PHX_TUNE_NOPATCH: convolutions whose stride equals their filter extent stay on the windowed kernels
     bool patchall = false;            // PHX_TUNE_PATCHALL: every pass of every such convolution runs on patches (not only where that was measured to gain)
     bool nodilphase = false;          // PHX_TUNE_NODILPHASE: dilated convolutions beyond the staging limit stay on the vector-ALU kernels
@@ -87,6 +88,7 @@ struct Tuning {
         if (const char* e = getenv("PHX_TUNE_KSLICES")) kslices = atoi(e);
         nodilphase = getenv("PHX_TUNE_NODILPHASE") != nullptr;
         nopatch = getenv("PHX_TUNE_NOPATCH") != nullptr;
+        nobands = getenv("PHX_TUNE_NOBANDS") != nullptr;
         patchall = getenv("PHX_TUNE_PATCHALL") != nullptr;
         if (const char* e = getenv("PHX_TUNE_WGPHASE")) wgphase = atoi(e) != 0;
         if (const char* e = getenv("PHX_TUNE_DILPHASE_MIN")) dilphase_min = atoi(e);
@@ -368,6 +370,7 @@ struct Problem {
     // image and `groups` such slices side by side (ci_mem == ci, co_mem == co without groups)
     int groups, ci_mem, co_mem;
     bool nhwc;  // the caller's activation tensors are channels-last: [rows, h, w, channels]
+    bool banded = false;  // a band of a larger filter's taps (see tap_bands): pads may be negative, and no rewrite applies
 };
 
 static int out_size(int in, int k, int d, int s, int before, int after) {
@@ -1466,6 +1469,7 @@ static PhaseAxis phase_axis(int a, int extent, int k, int d, int s, int pad_befo
 // input gradient through the phases, PHX_TUNE_PHASE=0 none.
 constexpr int PHASES_MAX = 64;  // strides up to 8 x 8 (PhaseMergeArgs::off)
 static bool dgrad_by_phases(const Problem& p) {
+    if (p.banded) return false;
     if ((p.sh == 1 && p.sw == 1) || p.sh * p.sw > PHASES_MAX || is_empty(p) || channel_slices(p)) return false;
     if (tune().phase >= 0) return tune().phase != 0;
     if (p.kh == 1 && p.kw == 1) return true;
@@ -1536,6 +1540,7 @@ struct S2dView {
 static int floordiv(int a, int b) { return a >= 0 ? a / b : -((-a + b - 1) / b); }
 
 static bool s2d_view(const Problem& p, S2dView& v) {
+    if (p.banded) return false;
     if (p.sh != 2 || p.sw != 2 || p.dh != 1 || p.dw != 1 || p.ci > 4 || (p.kh < 3 && p.kw < 3) || is_empty(p)) return false;
     if (channel_slices(p)) return false;  // the rearranged copies are laid out for whole tensors
     if (tune().nos2d) return false;
@@ -1570,6 +1575,7 @@ static bool s2d_view(const Problem& p, S2dView& v) {
 // filter gradient; the input gradient has its phases): the problem q on the subsampled input and that copy's size.
 // q-ResNet-50's three downsampling shortcuts, N=64: forward 0.07 ms on the general kernel.
 static bool subsample_view(const Problem& p, Problem& q, size_t& xs_bytes) {
+    if (p.banded) return false;
     if (p.kh != 1 || p.kw != 1 || (p.sh == 1 && p.sw == 1) || p.pt || p.pl || p.pb || p.pr || is_empty(p)) return false;
     if (channel_slices(p) || p.nhwc || p.real_input || tune().nosub) return false;
     q = p;
@@ -1605,6 +1611,7 @@ struct PatchView {
     size_t x_bytes;  // the input-side tensor as patches
 };
 static bool patch_view(const Problem& p, int pass, PatchView& v) {
+    if (p.banded) return false;
     if (tune().nopatch || tune().direct || is_empty(p) || p.kh != p.sh || p.kw != p.sw || p.kh * p.kw == 1) return false;
     if (p.dh != 1 || p.dw != 1 || p.pt || p.pl || channel_slices(p) || g_window_cl) return false;
     // Patches of fewer than nine positions (2x2 stride 2): the windowed kernels' forward pass and fp16 filter gradient
@@ -1652,6 +1659,7 @@ struct DilationView {
     size_t x_bytes, y_bytes;   // the two phase tensors
 };
 static bool dilation_view(const Problem& p, int pass, DilationView& v) {
+    if (p.banded) return false;
     if (tune().nodilphase || tune().direct || is_empty(p) || (p.dh == 1 && p.dw == 1) || p.sh != 1 || p.sw != 1) return false;
     // (the filter gradient stages no halo window around its tiles: it takes the rewrite only where it has to)
     const long most = pass == PHX_PASS_BWD_WEIGHTS ? WG_THREADS : std::min<long>(tune().dilphase_min, WG_THREADS);
@@ -1716,6 +1724,7 @@ constexpr int TAP_CLASSES_MAX = 8;  // strides up to 8 along an axis
 // 256 at 14x14 197 / 219, 128 at 28x28 139 / 229, 64 at 56x56 131 / 289; fp32 arithmetic 512 at 28x28 5708 / 3396,
 // 512 at 14x14 4260 / 1973, 256 at 28x28 2169 / 1802, but 128 at 28x28 544 / 536, 64 at 28x28 151 / 223.
 static bool wgrad_by_classes(const Problem& p) {
+    if (p.banded) return false;
     if ((p.sh == 1 && p.sw == 1) || p.kh * p.kw == 1 || is_empty(p) || channel_slices(p) || p.real_input || g_window_cl) return false;
     if (p.sh > TAP_CLASSES_MAX || p.sw > TAP_CLASSES_MAX) return false;
     S2dView v;
@@ -1734,6 +1743,50 @@ static Problem wgrad_class_problem(const Problem& p, const TapClass& ch, const T
     q.pt = q.pl = q.pb = q.pr = 0;
     q.fs.skh = p.fs.skh * ch.kstep; q.fs.skw = p.fs.skw * cw.kstep;
     tap_offset = ch.k0 * p.fs.skh + cw.k0 * p.fs.skw;
+    return q;
+}
+
+// Tap bands.  The windowed kernels stage, for every output tile, the window of the WHOLE filter around it: at the
+// staging limit (a 16x16 filter: 256 positions) a tile is a single output position and a pass takes 10-20 times what
+// a 13x13 filter takes; beyond it nothing fits (vector-ALU kernels).  A convolution is the sum of the convolutions
+// with the bands of its filter -- blocks of at most 8 window columns and 20 window rows, at most 160 positions --
+// each an ordinary problem on the same tensors whose padding is the original one minus the band's offset (negative
+// where the band starts inside the window), its filter the block's taps through the same strides.  Forward and
+// input gradient run one pass per band into partial tensors and add them (slice_sum_kernel, with the bias); the
+// filter gradient of a band IS that band's block of dw.  Used from 225 window positions on where no other rewrite
+// (patches, dilation phases) applies; groups and real-valued input keep the vector-ALU kernels.
+struct TapBand {
+    int r0, rows, c0, cols;
+};
+constexpr int TAP_BANDS_MAX = 32;
+static int tap_bands(const Problem& p, int pass, TapBand* bands) {
+    if (p.banded || tune().nobands || tune().direct || is_empty(p) || channel_slices(p) || p.real_input || g_window_cl) return 0;
+    if (window_positions(p) <= (pass == PHX_PASS_BWD_WEIGHTS ? WG_THREADS : 224)) return 0;
+    // (a strided input gradient by phases has ceil(k / s) taps per axis and phase: small windows already; windows
+    // beyond the staging limit do not get that far -- they would go to the vector-ALU kernels -- and take the bands)
+    if (pass == PHX_PASS_BWD_DATA && !window_beyond_staging(p) && dgrad_by_phases(p)) return 0;
+    const int bw = 7 / p.dw + 1, bh = 19 / p.dh + 1;  // ((bw-1) dw + 1 <= 8 columns, (bh-1) dh + 1 <= 20 rows
+    const int nh = cdiv(p.kh, bh), nw = cdiv(p.kw, bw);
+    if (nh * nw > TAP_BANDS_MAX || nh * nw < 2) return 0;
+    int n = 0;
+    for (int a = 0; a < nh; ++a)
+        for (int b = 0; b < nw; ++b) {
+            // (bands of even size: 16 columns as 8 + 8, 13 as 7 + 6)
+            const int r0 = (int)((long)a * p.kh / nh), r1 = (int)((long)(a + 1) * p.kh / nh);
+            const int c0 = (int)((long)b * p.kw / nw), c1 = (int)((long)(b + 1) * p.kw / nw);
+            bands[n++] = TapBand{r0, r1 - r0, c0, c1 - c0};
+        }
+    return n;
+}
+static Problem band_problem(const Problem& p, const TapBand& t, long& tap_offset) {
+    Problem q = p;
+    q.banded = true;
+    q.nhwc = false;
+    q.has_bias = false;
+    q.kh = t.rows; q.kw = t.cols;
+    q.pt = p.pt - t.r0 * p.dh; q.pl = p.pl - t.c0 * p.dw;
+    q.pb = p.pb - (p.kh - t.r0 - t.rows) * p.dh; q.pr = p.pr - (p.kw - t.c0 - t.cols) * p.dw;
+    tap_offset = t.r0 * p.fs.skh + t.c0 * p.fs.skw;
     return q;
 }
 
@@ -1775,6 +1828,7 @@ static int slices_rule(const Problem& p, int pass, const Corr& creal) {
 
 static bool nhwc_window_native(const Problem& p, int pass);
 static int corr_slices(const Problem& p, int pass) {
+    if (p.banded) return 0;
     if (tune().kslices == 0 || pass == PHX_PASS_BWD_WEIGHTS || is_empty(p)) return 0;
     if (channel_slices(p) || p.real_input || g_batch.n > 1 || g_window_cl) return 0;
     // (channels-last tensors: a call that goes through channels-first copies is sliced on those; one that runs on the
@@ -1793,6 +1847,7 @@ static int corr_slices(const Problem& p, int pass) {
 // A strided input gradient that runs by phases (dgrad_by_phases): every phase is a pass of its own and is sliced like
 // one, all by the Z that the rule gives for the phase with the most taps.
 static int phase_slices(const Problem& p) {
+    if (p.banded) return 0;
     if (tune().kslices == 0 || !dgrad_by_phases(p) || g_batch.n > 1 || g_window_cl) return 0;
     PhaseAxis bh{}, bw{};
     for (int a = 0; a < p.sh; ++a)
@@ -1837,6 +1892,17 @@ static size_t workspace_for(const Problem& p, int pass) {
     if (patch_view(p, pass, patches)) return patches.x_bytes + workspace_for(patches.q, pass);
     DilationView dilated;
     if (dilation_view(p, pass, dilated)) return dilated.x_bytes + dilated.y_bytes + workspace_for(dilated.q, pass);
+    TapBand bands[TAP_BANDS_MAX];
+    if (const int nb = tap_bands(p, pass, bands)) {  // partial results of every band (forward, input gradient) + the most a band needs
+        const size_t esize = p.dtype == PHX_F32 ? 4 : 2;
+        const size_t count = pass == PHX_PASS_FWD ? (size_t)4 * p.n * p.co * p.ho * p.wo : (size_t)4 * p.n * p.ci * p.h * p.w;
+        size_t most = 0;
+        for (int b = 0; b < nb; ++b) {
+            long tap_offset = 0;
+            most = std::max(most, workspace_for(band_problem(p, bands[b], tap_offset), pass));
+        }
+        return (pass == PHX_PASS_BWD_WEIGHTS ? 0 : align_up(nb * count * esize, 256)) + most;
+    }
     if (pass == PHX_PASS_BWD_WEIGHTS && wgrad_by_classes(p)) {  // the largest class: its gathered input + its own workspace
         TapClass ch[TAP_CLASSES_MAX], cw[TAP_CLASSES_MAX];
         const int nh = tap_classes(p.kh, p.dh, p.sh, p.pt, p.ho, ch), nw = tap_classes(p.kw, p.dw, p.sw, p.pl, p.wo, cw);
@@ -1889,6 +1955,38 @@ static void s2d_rearrange_input(const Problem& p, const S2dView& v, const void* 
     S2dArgs a;
     a.src = x; a.dst = x2; a.planes = (p.real_input ? 1L : 4L) * p.n * p.ci; a.H = p.h; a.W = p.w; a.H2 = v.q.h; a.W2 = v.q.w;
     launch_s2d_input(p.dtype == PHX_F16, a, st);
+}
+
+static int do_fwd(const Problem& p, hipStream_t st, const void* x, const void* w, const void* bias, void* y, void* ws, size_t wsb);
+static int do_bwd_data(const Problem& p, hipStream_t st, const void* g, const void* w, void* dx, void* ws, size_t wsb);
+// Forward (map == MAP_FWD: in = x) or input gradient by tap bands: a pass per band into its partial tensor, then their sum
+static int run_banded(const Problem& p, const TapBand* bands, int nb, int map, hipStream_t st, const void* in, const void* w, const void* bias,
+                      void* out, void* ws, size_t wsb) {
+    const bool dry = g_pack.dry();
+    const size_t esize = p.dtype == PHX_F32 ? 4 : 2;
+    const long count = map == MAP_FWD ? 4L * p.n * p.co * p.ho * p.wo : 4L * p.n * p.ci * p.h * p.w;
+    const size_t partial_bytes = align_up((size_t)nb * count * esize, 256);
+    if (!dry && (wsb < partial_bytes || !ws)) return PHX_ERR_WORKSPACE;
+    char* partial = static_cast<char*>(ws);
+    g_name_prefix = "band_";
+    for (int b = 0; b < nb; ++b) {
+        long tap_offset = 0;
+        const Problem q = band_problem(p, bands[b], tap_offset);
+        const void* wb = at_bytes(w, (size_t)tap_offset * esize);
+        void* part = dry ? nullptr : partial + (size_t)b * count * esize;
+        void* rest = dry ? nullptr : partial + partial_bytes;
+        const int rc = map == MAP_FWD ? do_fwd(q, st, in, wb, nullptr, part, rest, dry ? 0 : wsb - partial_bytes)
+                                      : do_bwd_data(q, st, in, wb, part, rest, dry ? 0 : wsb - partial_bytes);
+        if (rc != PHX_OK) { g_name_prefix = ""; return rc; }
+    }
+    g_name_prefix = "";
+    if (dry) return PHX_OK;
+    const bool add = map == MAP_DGRAD && g_addend.dx == out && g_addend.ptr && !g_addend.fused;
+    launch_slice_sum(p.dtype == PHX_F16, partial, nb, count, out, bias, add ? g_addend.ptr : nullptr,
+                     map == MAP_FWD ? p.ho * p.wo : p.h * p.w, map == MAP_FWD ? p.co : p.ci, count / 4, st);
+    PHX_HIP(hipGetLastError());
+    if (add) g_addend.fused = true;
+    return PHX_OK;
 }
 
 // One forward (map == MAP_FWD: in = x) or input-gradient pass in Z reduction slices (see corr_slices)
@@ -1952,6 +2050,8 @@ static int do_fwd(const Problem& p, hipStream_t st, const void* x, const void* w
         PHX_HIP(hipGetLastError());
         return PHX_OK;
     }
+    TapBand bands[TAP_BANDS_MAX];
+    if (const int nb = tap_bands(p, PHX_PASS_FWD, bands)) return run_banded(p, bands, nb, MAP_FWD, st, x, w, b, y, ws, wsb);
     S2dView v;
     if (s2d_view(p, v)) {
         // (the rearranged filter of this path is itself made per call: no prepacked form)
@@ -2024,6 +2124,8 @@ static int do_bwd_data(const Problem& p, hipStream_t st, const void* g, const vo
         PHX_HIP(hipGetLastError());
         return PHX_OK;
     }
+    TapBand bands[TAP_BANDS_MAX];
+    if (const int nb = tap_bands(p, PHX_PASS_BWD_DATA, bands)) return run_banded(p, bands, nb, MAP_DGRAD, st, g, w, nullptr, dx, ws, wsb);
     if (dgrad_by_phases(p)) {
         const size_t esize = p.dtype == PHX_F32 ? 4 : 2;
         PhaseMergeArgs m;
@@ -2096,6 +2198,20 @@ static int do_bwd_weights(const Problem& p, hipStream_t st, const void* x, const
         const int rc = do_bwd_weights(dilated.q, st, x2, g2, dw, g2 + dilated.y_bytes, wsb - tensors);
         g_name_prefix = "";
         return rc;
+    }
+    TapBand bands[TAP_BANDS_MAX];
+    if (const int nb = tap_bands(p, PHX_PASS_BWD_WEIGHTS, bands)) {  // a band's filter gradient is its block of dw
+        if (wsb < workspace_for(p, PHX_PASS_BWD_WEIGHTS) || (!ws && wsb)) return PHX_ERR_WORKSPACE;  // (refused as a whole)
+        const size_t esize = p.dtype == PHX_F32 ? 4 : 2;
+        g_name_prefix = "band_";
+        for (int b = 0; b < nb; ++b) {
+            long tap_offset = 0;
+            const Problem q = band_problem(p, bands[b], tap_offset);
+            const int rc = do_bwd_weights(q, st, x, g, static_cast<char*>(dw) + (size_t)tap_offset * esize, ws, wsb);
+            if (rc != PHX_OK) { g_name_prefix = ""; return rc; }
+        }
+        g_name_prefix = "";
+        return PHX_OK;
     }
     if (wgrad_by_classes(p)) {
         TapClass ch[TAP_CLASSES_MAX], cw[TAP_CLASSES_MAX];
@@ -2307,7 +2423,8 @@ static bool nhwc_window_native(const Problem& p, int pass) {
     planes.nhwc = false;
     DilationView dilated;
     PatchView patches;
-    return corr_slices(planes, pass) == 0 && !dilation_view(planes, pass, dilated) && !patch_view(planes, pass, patches);
+    TapBand bands[TAP_BANDS_MAX];
+    return corr_slices(planes, pass) == 0 && !dilation_view(planes, pass, dilated) && !patch_view(planes, pass, patches) && !tap_bands(planes, pass, bands);
 }
 }  // namespace phx
 
@@ -2345,7 +2462,8 @@ static bool thin_groups(const Problem& p, int pass) {
     if (tune().direct) return true;
     DilationView dilated;
     PatchView patches;
-    if (window_beyond_staging(p)) return !dilation_view(p, pass, dilated) && !patch_view(p, pass, patches);
+    TapBand bands[TAP_BANDS_MAX];
+    if (window_beyond_staging(p)) return !dilation_view(p, pass, dilated) && !patch_view(p, pass, patches) && !tap_bands(p, pass, bands);
     const long pairs = (long)p.ci * p.co;
     // The filter gradient in fp32 arithmetic works on 64 x 64 channel tiles whatever the layer holds: its time follows
     // the pixels and taps alone (3x3, 56x56, N=64: 1.39 ms from 8 to 64 channels), that of the vector-ALU kernel the

@@ -487,40 +487,61 @@ BIG_WINDOWS = [
     ("k7_dil3_s2", 1, 4, 4, 30, 27, 7, 7, 2, 3, "SAME"),            # input gradient by phases, every entry on its own phase pattern
     ("k9x5_dil4_s3", 2, 5, 2, 40, 30, 9, 5, 3, 4, (5, 2, 0, 7)),    # stride 3: the per-tap input gradient
     ("k17_c40_24", 1, 40, 24, 18, 19, 17, 17, 1, 1, "SAME"),        # more filter entries than LDS holds: chunks of channels
+    ("k16_same", 2, 8, 8, 20, 23, 16, 16, 1, 1, "SAME"),             # exactly the staging limit: two bands of 16 x 8
+    ("k31x3_s2", 1, 4, 8, 70, 20, 31, 3, 2, 1, (15, 1, 9, 0)),       # bands of rows only
+    ("k25_valid", 1, 2, 4, 40, 44, 25, 25, 1, 1, "VALID"),           # 2 x 4 bands
 ]
 
 
 @pytest.mark.parametrize("dtype,policy", [(torch.float32, "fp32"), (torch.float16, "full16")], ids=["f32", "f16_full16"])
 @pytest.mark.parametrize("mode", [16, 8])
 @pytest.mark.parametrize("case", BIG_WINDOWS, ids=lambda c: c[0])
-def test_windows_beyond_the_staging_limit(case, mode, dtype, policy):
+def test_windows_beyond_the_staging_limit(case, mode, dtype, policy, tune_env):
     """The matrix-core kernels stage one window position per thread: a filter whose window for a single output
-    position -- ((kh-1) dh + 1) x ((kw-1) dw + 1), columns in whole chunks of 8 -- exceeds 256 positions runs on the
-    vector-ALU kernels instead (any filter size and dilation is valid at the reference's boundary,
-    src/backend/onednn/conv2d.hpp:116-210).  Against the oracle; no packed form, partial sums as the only workspace."""
+    position -- ((kh-1) dh + 1) x ((kw-1) dw + 1), columns in whole chunks of 8 -- exceeds 256 positions cannot run
+    on them as it is (any filter size and dilation is valid at the reference's boundary,
+    src/backend/onednn/conv2d.hpp:116-210).  Such a convolution runs as the sum of the convolutions with the bands of
+    its filter (blocks of at most 20 x 8 window positions; the filter gradient of a band is its block of dw), as an
+    undilated convolution on its dilation phases where it is dilated with unit stride, or -- PHX_TUNE_NOBANDS,
+    PHX_TUNE_NODILPHASE, and always for groups -- on the vector-ALU kernels.  Against the oracle."""
     name, n, ci, co, h, w, kh, kw, stride, dilation, padding = case
     scale = 1.0 if dtype == torch.float32 else 0.5
     g, x, wt, b, gr = make_inputs(name_seed(name) + 50, n, ci, co, h, w, kh, kw, stride, dilation, padding, dtype, scale)
     desc = phx.Conv2DDescriptor(x.shape, wt.shape, stride, dilation, padding, use_bias=True, dtype=dtype, context=Ctx(mode, policy))
     xd, wd, bd, gd = (torch.from_numpy(a).cuda() for a in (x, wt, b, gr))
-    y = phx.conv2d_fwd(xd, wd, bd, desc)
-    names = [capi.last_kernel_name()]
-    dx = ops.conv2d_bwd_data(wd, gd, desc)
-    names.append(capi.last_kernel_name())
-    dw = ops.conv2d_bwd_weights(xd, gd, desc)
-    names.append(capi.last_kernel_name())
-    if name == "k7_dil3":  # (unit stride: undilated on its dilation phases, see below)
-        assert all(k.startswith("dil_") and "mfma" in k for k in names), names
-    else:
-        assert all("_fma_thin_" in k for k in names), names
-        assert desc.workspace_bytes(capi.PHX_PASS_FWD) == 0 and desc.workspace_bytes(capi.PHX_PASS_BWD_DATA) == 0
-        assert ops.conv2d_pack_filters(wd, desc) is None
     x64, w64, b64, g64 = (a.astype(np.float64) for a in (x, wt, b, gr))
     want_y = oracle.conv2d_fwd(g, x64, w64, b64, "hamilton")
     want_dw, want_dx = oracle.conv2d_bwd(g, x64, w64, g64, "hamilton")
-    assert_close(y.cpu().numpy(), want_y, dtype, "fwd " + names[0])
-    assert_close(dx.cpu().numpy(), want_dx, dtype, "dgrad " + names[1])
-    assert_close(dw.cpu().numpy(), want_dw, dtype, "wgrad " + names[2])
+    addend = torch.from_numpy((scale * np.random.default_rng(8).standard_normal(x.shape)).astype(x.dtype)).cuda()
+    for rewritten in (True, False):
+        tune_env(PHX_TUNE_NOBANDS=None if rewritten else "1", PHX_TUNE_NODILPHASE=None if rewritten else "1")
+        y = phx.conv2d_fwd(xd, wd, bd, desc)
+        names = [capi.last_kernel_name()]
+        dx = ops.conv2d_bwd_data(wd, gd, desc)
+        names.append(capi.last_kernel_name())
+        poison = torch.full(wd.shape, float("nan"), dtype=dtype, device="cuda")  # (every band must write its block of dw)
+        del poison
+        dw = ops.conv2d_bwd_weights(xd, gd, desc)
+        names.append(capi.last_kernel_name())
+        dil = dilation if isinstance(dilation, tuple) else (dilation, dilation)
+        beyond = ((kh - 1) * dil[0] + 1) * (((kw - 1) * dil[1] + 1 + 7) // 8 * 8) > 256  # (at 225-256 positions the filter gradient keeps its kernel)
+        if not rewritten:
+            if beyond:
+                assert all("_fma_thin_" in k for k in names), names
+                assert desc.workspace_bytes(capi.PHX_PASS_FWD) == 0 and desc.workspace_bytes(capi.PHX_PASS_BWD_DATA) == 0
+                assert ops.conv2d_pack_filters(wd, desc) is None
+        else:  # (unit stride and dilated: dilation phases; otherwise tap bands)
+            prefix = "dil_" if name == "k7_dil3" else "band_"
+            # (at 225-256 positions a strided input gradient goes by phases, the filter gradient keeps its kernel)
+            assert all(k.startswith(prefix) and "mfma" in k for k in (names if beyond else names[:1])), names
+            packed = ops.conv2d_pack_filters(wd, desc)
+            zero = torch.zeros_like(wd)
+            assert torch.equal(phx.conv2d_fwd(xd, zero, bd, desc, packed=packed), y), "prepacked fwd"
+            assert torch.equal(ops.conv2d_bwd_data(zero, gd, desc, packed=packed), dx), "prepacked dgrad"
+            assert torch.equal(ops.conv2d_bwd_data(wd, gd, desc, addend=addend), dx + addend), "dgrad + addend"
+        assert_close(y.cpu().numpy(), want_y, dtype, "fwd " + names[0])
+        assert_close(dx.cpu().numpy(), want_dx, dtype, "dgrad " + names[1])
+        assert_close(dw.cpu().numpy(), want_dw, dtype, "wgrad " + names[2])
 
 
 SLICED = [
@@ -695,7 +716,8 @@ def test_large_dilations_run_as_undilated_convolutions_on_their_phases(case, mod
     addend = torch.from_numpy((scale * np.random.default_rng(7).standard_normal(x.shape)).astype(x.dtype)).cuda()
     for phases in (True, False):
         # (THIN_MAX32=0: filter gradients of few channels in fp32 arithmetic stay off the vector-ALU kernels)
-        tune_env(PHX_TUNE_NODILPHASE=None if phases else "1", PHX_TUNE_THIN_MAX32="0")
+        # (NOBANDS: what is not rewritten here would otherwise run by tap bands, see test_windows_beyond_the_staging_limit)
+        tune_env(PHX_TUNE_NODILPHASE=None if phases else "1", PHX_TUNE_THIN_MAX32="0", PHX_TUNE_NOBANDS="1")
         y = phx.conv2d_fwd(xd, wd, bd, desc)
         names = [capi.last_kernel_name()]
         dx = ops.conv2d_bwd_data(wd, gd, desc)
