@@ -2463,14 +2463,22 @@ static bool thin_groups(const Problem& p, int pass) {
     DilationView dilated;
     PatchView patches;
     TapBand bands[TAP_BANDS_MAX];
-    if (window_beyond_staging(p)) return !dilation_view(p, pass, dilated) && !patch_view(p, pass, patches) && !tap_bands(p, pass, bands);
     const long pairs = (long)p.ci * p.co;
+    // (the rule for filter gradients of few channels in fp32 arithmetic, see below)
+    const bool few_fp32 = pass == PHX_PASS_BWD_WEIGHTS && p.groups <= 1 && tune().thin_max32 > 0 && !wgrad_on_f16_mfma(flatten_pointwise(p)) &&
+                          pairs <= (p.kh * p.kw > 1 ? 512 : 128);
+    if (window_beyond_staging(p))
+        return few_fp32 || (!dilation_view(p, pass, dilated) && !patch_view(p, pass, patches) && !tap_bands(p, pass, bands));
+    // at their staging limit the matrix-core kernels work on tiles of a single output position (a grouped 16x16 filter,
+    // 8 groups of 32 channels: 1.1 s for an input gradient): what the tap bands do not take runs here as well
+    if (window_positions(p) > 224 && (p.groups > 1 || p.real_input))
+        return !dilation_view(p, pass, dilated) && !patch_view(p, pass, patches);
     // The filter gradient in fp32 arithmetic works on 64 x 64 channel tiles whatever the layer holds: its time follows
     // the pixels and taps alone (3x3, 56x56, N=64: 1.39 ms from 8 to 64 channels), that of the vector-ALU kernel the
     // channel pairs too -- 8 -> 8 channels 0.11 ms, 16 -> 16 0.35, 3 -> 64 0.29, 24 -> 24 0.77, 32 -> 32 1.20; a
     // single tap: 16 -> 16 0.18 against 0.17.  Layers of few channels, grouped or not, run it here.
     if (pass == PHX_PASS_BWD_WEIGHTS && p.groups <= 1 && tune().thin_max32 > 0 && !wgrad_on_f16_mfma(flatten_pointwise(p)))
-        return pairs <= (p.kh * p.kw > 1 ? 512 : 128);
+        return few_fp32;
     if (p.groups <= 1) return false;
     // Passes in fp32 arithmetic (fp32 tensors, fp16 tensors where the policy says so) have a sixteenth of the fp16
     // matrix-core rate to lose against, and their filter gradient works on 64 x 64 channel tiles: measured like above,

@@ -514,7 +514,9 @@ def test_windows_beyond_the_staging_limit(case, mode, dtype, policy, tune_env):
     want_dw, want_dx = oracle.conv2d_bwd(g, x64, w64, g64, "hamilton")
     addend = torch.from_numpy((scale * np.random.default_rng(8).standard_normal(x.shape)).astype(x.dtype)).cuda()
     for rewritten in (True, False):
-        tune_env(PHX_TUNE_NOBANDS=None if rewritten else "1", PHX_TUNE_NODILPHASE=None if rewritten else "1")
+        # (THIN_MAX32=0: filter gradients of few channels in fp32 arithmetic would run on the vector-ALU kernels either way)
+        tune_env(PHX_TUNE_NOBANDS=None if rewritten else "1", PHX_TUNE_NODILPHASE=None if rewritten else "1",
+                 PHX_TUNE_THIN_MAX32="0" if rewritten else None)
         y = phx.conv2d_fwd(xd, wd, bd, desc)
         names = [capi.last_kernel_name()]
         dx = ops.conv2d_bwd_data(wd, gd, desc)
