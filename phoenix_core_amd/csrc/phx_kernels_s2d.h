@@ -168,38 +168,49 @@ struct DilationPhaseArgs {
     int Hp, Wp;         // extent of a phase image: at least ceil((H + oh) / dh), ceil((W + ow) / dw)
     int dh, dw;
     int oh, ow;         // rows / columns of the origin in front of the tensor's first
+    int CB;             // channels per workgroup item (divides C; set by launch_dilation_phases)
 };
 
+// A workgroup takes one (component x image, block of CB channels, row phase a) at a time: the rows of the caller's
+// tensor that it touches are shared by all dw column phases, so each of their cache lines is fetched once, and the
+// phase images it touches are runs of CB * Hp * Wp consecutive elements.  Index arithmetic per element is 32-bit.
 template <typename TS>
 __global__ void __launch_bounds__(WG_THREADS) dilation_phase_kernel(const DilationPhaseArgs A, int to_caller) {
-    const long stride = (long)gridDim.x * blockDim.x, first = (long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (!to_caller) {
-        const TS* x = static_cast<const TS*>(A.src);
-        TS* ph = static_cast<TS*>(A.dst);
-        const long total = A.rows * A.dh * A.dw * A.C * A.Hp * A.Wp;
-        for (long idx = first; idx < total; idx += stride) {
-            const int j = idx % A.Wp;
-            long rest = idx / A.Wp;
-            const int i = rest % A.Hp; rest /= A.Hp;
-            const int c = rest % A.C; rest /= A.C;
-            const int b = rest % A.dw; rest /= A.dw;
-            const int a = rest % A.dh;
-            const long row = rest / A.dh;
-            const int yi = i * A.dh + a - A.oh, xj = j * A.dw + b - A.ow;
-            ph[idx] = (yi >= 0 && yi < A.H && xj >= 0 && xj < A.W) ? x[((row * A.C + c) * A.H + yi) * A.W + xj] : (TS)0;
-        }
-    } else {
-        const TS* ph = static_cast<const TS*>(A.src);
-        TS* x = static_cast<TS*>(A.dst);
-        const long total = A.rows * A.C * A.H * A.W;
-        for (long idx = first; idx < total; idx += stride) {
-            const int xj = idx % A.W;
-            long rest = idx / A.W;
-            const int yi = rest % A.H; rest /= A.H;
-            const int c = rest % A.C;
-            const long row = rest / A.C;
-            const int a = (yi + A.oh) % A.dh, i = (yi + A.oh) / A.dh, b = (xj + A.ow) % A.dw, j = (xj + A.ow) / A.dw;
-            x[idx] = ph[((((row * A.dh + a) * A.dw + b) * A.C + c) * A.Hp + i) * A.Wp + j];
+    const int cblocks = A.C / A.CB;
+    const long items = A.rows * cblocks * A.dh;
+    const unsigned int plane = (unsigned int)A.Hp * A.Wp;
+    for (long item = blockIdx.x; item < items; item += gridDim.x) {
+        const int a = (int)(item % A.dh);
+        const long rest = item / A.dh;
+        const int c0 = (int)(rest % cblocks) * A.CB;
+        const long row = rest / cblocks;
+        const long caller0 = (row * A.C + c0) * A.H * A.W;                       // channel c0 of this row in the caller's tensor
+        const long phase0 = (row * A.dh + a) * A.dw * A.C * (long)plane + (long)c0 * plane;  // column phase 0, channel c0
+        const long phase_b = (long)A.C * plane;                                  // from one column phase to the next
+        if (!to_caller) {
+            const TS* x = static_cast<const TS*>(A.src) + caller0;
+            TS* ph = static_cast<TS*>(A.dst) + phase0;
+            const unsigned int per_b = (unsigned int)A.CB * plane, count = per_b * A.dw;
+            for (unsigned int e = threadIdx.x; e < count; e += WG_THREADS) {
+                const unsigned int b = e / per_b, in_b = e - b * per_b;          // in_b = (channel, i, j) of the phase image
+                const unsigned int cin = in_b / plane, ij = in_b - cin * plane;
+                const unsigned int i = ij / A.Wp, j = ij - i * A.Wp;
+                const int yi = (int)i * A.dh + a - A.oh, xj = (int)j * A.dw + (int)b - A.ow;
+                ph[b * phase_b + in_b] =
+                    (yi >= 0 && yi < A.H && xj >= 0 && xj < A.W) ? x[((long)cin * A.H + yi) * A.W + xj] : (TS)0;
+            }
+        } else {
+            const TS* ph = static_cast<const TS*>(A.src) + phase0;
+            TS* x = static_cast<TS*>(A.dst) + caller0;
+            const unsigned int per_c = (unsigned int)A.Hp * A.W, count = per_c * A.CB;
+            for (unsigned int e = threadIdx.x; e < count; e += WG_THREADS) {
+                const unsigned int cin = e / per_c, ix = e - cin * per_c;
+                const unsigned int i = ix / A.W, xj = ix - i * A.W;
+                const int yi = (int)i * A.dh + a - A.oh;
+                if (yi < 0 || yi >= A.H) continue;
+                const unsigned int xo = xj + A.ow, j = xo / A.dw, b = xo - j * A.dw;
+                x[((long)cin * A.H + yi) * A.W + xj] = ph[b * phase_b + (long)cin * plane + i * A.Wp + j];
+            }
         }
     }
 }

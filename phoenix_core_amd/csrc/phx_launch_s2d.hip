@@ -46,13 +46,21 @@ int launch_strided_gather(bool half_storage, const StridedGatherArgs& a, hipStre
     return 0;
 }
 
-int launch_dilation_phases(bool half_storage, const DilationPhaseArgs& a, bool to_caller, hipStream_t st) {
-    const long items = to_caller ? a.rows * a.C * a.H * a.W : a.rows * a.dh * a.dw * a.C * a.Hp * a.Wp;
-    if (items <= 0) return 0;
+int launch_dilation_phases(bool half_storage, const DilationPhaseArgs& a0, bool to_caller, hipStream_t st) {
+    if (a0.rows <= 0 || a0.C <= 0 || a0.H <= 0 || a0.W <= 0) return 0;
+    DilationPhaseArgs a = a0;
+    // channels per item: a power of two that divides C, for items of a few thousand elements
+    const long per_channel = (long)a.Hp * a.Wp * a.dw;
+    a.CB = 1;
+    while (a.C % (a.CB * 2) == 0 && per_channel * a.CB * 2 <= 4096) a.CB *= 2;
+    // a workgroup's 32-bit element count: (Hp * max(Wp * dw, W)) * CB
+    if (per_channel * a.CB >= (1L << 31) || (long)a.Hp * a.W * a.CB >= (1L << 31)) return -1;
+    const long items = a.rows * (a.C / a.CB) * a.dh;
+    const unsigned int blocks = (unsigned int)(items < (1L << 20) ? items : (1L << 20));
     if (half_storage)
-        hipLaunchKernelGGL((dilation_phase_kernel<_Float16>), dim3(blocks_for(items)), dim3(WG_THREADS), 0, st, a, (int)to_caller);
+        hipLaunchKernelGGL((dilation_phase_kernel<_Float16>), dim3(blocks), dim3(WG_THREADS), 0, st, a, (int)to_caller);
     else
-        hipLaunchKernelGGL((dilation_phase_kernel<float>), dim3(blocks_for(items)), dim3(WG_THREADS), 0, st, a, (int)to_caller);
+        hipLaunchKernelGGL((dilation_phase_kernel<float>), dim3(blocks), dim3(WG_THREADS), 0, st, a, (int)to_caller);
     return 0;
 }
 

@@ -1676,6 +1676,8 @@ static bool dilation_view(const Problem& p, int pass, DilationView& v) {
     q.pb = v.Hop + (p.kh - 1) - v.Hp - q.pt; q.pr = v.Wop + (p.kw - 1) - v.Wp - q.pl;
     if (q.pb < 0 || q.pr < 0 || window_beyond_staging(q)) return false;
     if (out_size(q.h, q.kh, 1, 1, q.pt, q.pb) != q.ho || out_size(q.w, q.kw, 1, 1, q.pl, q.pr) != q.wo) return false;
+    // the phase kernels index one channel's phase images with 32 bits
+    if ((long)v.Hp * v.Wp * p.dw >= (1L << 31) || (long)v.Hop * v.Wop * p.dw >= (1L << 31)) return false;
     const size_t esize = p.dtype == PHX_F32 ? 4 : 2;
     v.x_bytes = align_up((size_t)4 * q.n * p.ci * v.Hp * v.Wp * esize, 256);
     v.y_bytes = align_up((size_t)4 * q.n * p.co * v.Hop * v.Wop * esize, 256);
