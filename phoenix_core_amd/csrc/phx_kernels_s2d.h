@@ -77,6 +77,15 @@ __global__ void __launch_bounds__(WG_THREADS) strided_gather_kernel(const Stride
     }
 }
 
+// e / d for e < 2^24 (exact in fp32), rd = 1.0f / d: the rounded quotient is off by one at most, which the remainder shows
+__device__ __forceinline__ unsigned int div24(unsigned int e, unsigned int d, float rd) {
+    unsigned int q = (unsigned int)((float)e * rd);
+    const int r = (int)(e - q * d);
+    if (r < 0) --q;
+    else if (r >= (int)d) ++q;
+    return q;
+}
+
 // Patches to depth.  A convolution whose stride equals its filter extent (patch embeddings, 2x2 / stride 2
 // downsampling) reads every input position once, for one output position: with the kh x kw positions of a patch
 // laid out as channels,
@@ -92,62 +101,83 @@ struct PatchArgs {
     int Ho, Wo;         // patches per column / row
     int kh, kw;
     int tap_major;
+    int CB;             // channels per workgroup item (divides C; set by launch_patch_depth)
 };
 
-// (a workgroup works on whole planes -- one patch channel of one row, or one channel of the caller's tensor -- so that
-// the channel and tap of a plane are decoded once and a position costs one division)
+// 8 consecutive elements of a tensor, stored as one vector where the run is whole and its address aligned
+template <typename TS>
+struct alignas(8 * sizeof(TS)) PatchRun {
+    TS v[8];
+};
+template <typename TS>
+__device__ __forceinline__ void store_run(TS* dst, const PatchRun<TS>& run, unsigned int n) {
+    if (n == 8 && (reinterpret_cast<unsigned long>(dst) & (sizeof(PatchRun<TS>) - 1)) == 0) {
+        *reinterpret_cast<PatchRun<TS>*>(dst) = run;
+    } else {
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            if ((unsigned int)u < n) dst[u] = run.v[u];
+    }
+}
+
+// A workgroup takes one (component x image, block of CB channels, row a of the patch) at a time: the rows of the
+// caller's tensor that hold it serve all kw columns of the patch at once, so each of their cache lines is fetched (or
+// written) once, and on the patches' side it touches whole planes.  Index arithmetic is 32-bit, its divisions by fp32 reciprocal (an item has fewer than 2^24 elements).
 template <typename TS>
 __global__ void __launch_bounds__(WG_THREADS) patch_depth_kernel(const PatchArgs A, int to_caller) {
-    const int Cq = A.C * A.kh * A.kw;
-    if (!to_caller && (long)A.Ho * A.Wo < 512) {  // small patch planes: one position per thread, whatever its plane
-        const TS* x = static_cast<const TS*>(A.src);
-        TS* pt = static_cast<TS*>(A.dst);
-        const long total = A.rows * Cq * A.Ho * A.Wo;
-        for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
-            const int j = idx % A.Wo;
-            long rest = idx / A.Wo;
-            const int i = rest % A.Ho; rest /= A.Ho;
-            const int q = rest % Cq;
-            const long row = rest / Cq;
-            int c, a, b;
-            if (A.tap_major) { c = q % A.C; b = (q / A.C) % A.kw; a = q / (A.C * A.kw); }
-            else { b = q % A.kw; a = (q / A.kw) % A.kh; c = q / (A.kw * A.kh); }
-            const int yi = i * A.kh + a, xj = j * A.kw + b;
-            pt[idx] = (yi < A.H && xj < A.W) ? x[((row * A.C + c) * A.H + yi) * A.W + xj] : (TS)0;
-        }
-    } else if (!to_caller) {
-        const TS* x = static_cast<const TS*>(A.src);
-        TS* pt = static_cast<TS*>(A.dst);
-        const int plane = A.Ho * A.Wo;
-        for (long pl = blockIdx.x; pl < A.rows * Cq; pl += gridDim.x) {
-            const int q = pl % Cq;
-            const long row = pl / Cq;
-            int c, a, b;
-            if (A.tap_major) { c = q % A.C; b = (q / A.C) % A.kw; a = q / (A.C * A.kw); }
-            else { b = q % A.kw; a = (q / A.kw) % A.kh; c = q / (A.kw * A.kh); }
-            const TS* src = x + (row * A.C + c) * (long)A.H * A.W;
-            TS* dst = pt + pl * plane;
-            for (int t = threadIdx.x; t < plane; t += blockDim.x) {
-                const int i = t / A.Wo, j = t - i * A.Wo;
-                const int yi = i * A.kh + a, xj = j * A.kw + b;
-                dst[t] = (yi < A.H && xj < A.W) ? src[(long)yi * A.W + xj] : (TS)0;
+    const int cblocks = A.C / A.CB;
+    const long items = A.rows * cblocks * A.kh;
+    const unsigned int plane = (unsigned int)A.Ho * A.Wo;
+    const long Cq = (long)A.C * A.kh * A.kw;
+    // from one patch column to the next, and from one channel to the next, in planes of the patches' tensor
+    const long plane_b = A.tap_major ? A.C : 1, plane_c = A.tap_major ? 1 : A.kh * A.kw;
+    for (long item = blockIdx.x; item < items; item += gridDim.x) {
+        const int a = (int)(item % A.kh);
+        const long rest = item / A.kh;
+        const int c0 = (int)(rest % cblocks) * A.CB;
+        const long row = rest / cblocks;
+        const long caller0 = (row * A.C + c0) * A.H * A.W;
+        const long q0 = A.tap_major ? (long)a * A.kw * A.C + c0 : ((long)c0 * A.kh + a) * A.kw;  // plane of (c0, a, column 0)
+        const long patch0 = (row * Cq + q0) * plane;
+        if (!to_caller) {  // every position of the patches is written: those outside the caller's image are zero
+            // (one element per thread: neighbouring threads read kw elements apart, from lines that the workgroup's other
+            // patch columns use; runs of 8 per thread, as below, spread a wave's reads over 64 lines and measured slower)
+            const TS* x = static_cast<const TS*>(A.src) + caller0;
+            TS* pt = static_cast<TS*>(A.dst) + patch0;
+            const unsigned int per_c = (unsigned int)A.kw * plane, count = per_c * A.CB;
+            const float r_per_c = 1.0f / per_c, r_plane = 1.0f / plane, r_Wo = 1.0f / A.Wo;
+            for (unsigned int e = threadIdx.x; e < count; e += WG_THREADS) {
+                const unsigned int cin = div24(e, per_c, r_per_c), r = e - cin * per_c;
+                const unsigned int b = div24(r, plane, r_plane), ij = r - b * plane;
+                const unsigned int i = div24(ij, A.Wo, r_Wo), j = ij - i * A.Wo;
+                const unsigned int yi = i * A.kh + a, xj = j * A.kw + b;
+                pt[(cin * plane_c + b * plane_b) * plane + ij] =
+                    (yi < (unsigned int)A.H && xj < (unsigned int)A.W) ? x[((long)cin * A.H + yi) * A.W + xj] : (TS)0;
             }
-        }
-    } else {
-        const TS* pt = static_cast<const TS*>(A.src);
-        TS* x = static_cast<TS*>(A.dst);
-        const int plane = A.H * A.W;
-        const long patch_plane = (long)A.Ho * A.Wo;
-        for (long pl = blockIdx.x; pl < A.rows * A.C; pl += gridDim.x) {
-            const int c = pl % A.C;
-            const long row = pl / A.C;
-            const TS* src = pt + row * Cq * patch_plane;
-            TS* dst = x + pl * plane;
-            for (int t = threadIdx.x; t < plane; t += blockDim.x) {
-                const int yi = t / A.W, xj = t - yi * A.W;
-                const int i = yi / A.kh, a = yi - i * A.kh, j = xj / A.kw, b = xj - j * A.kw;
-                const int q = A.tap_major ? (a * A.kw + b) * A.C + c : (c * A.kh + a) * A.kw + b;
-                dst[t] = (i < A.Ho && j < A.Wo) ? src[(q * (long)A.Ho + i) * A.Wo + j] : (TS)0;
+        } else {  // every position of the caller's tensor is written: those outside the patches are zero
+            // (a thread works on 8 consecutive elements of a row -- one division set for the first, increments for the
+            // rest -- and stores them as one vector where the run is whole and aligned)
+            const TS* pt = static_cast<const TS*>(A.src) + patch0;
+            TS* x = static_cast<TS*>(A.dst) + caller0;
+            const unsigned int Hi = (A.H + A.kh - 1) / A.kh;                // patch rows that touch the caller's image
+            const unsigned int gpr = ((unsigned int)A.W + 7) / 8;           // groups of 8 per row of the caller's image
+            const unsigned int count = gpr * Hi * A.CB;
+            const float r_gpr = 1.0f / gpr, r_Hi = 1.0f / Hi, r_kw = 1.0f / A.kw;
+            for (unsigned int g = threadIdx.x; g < count; g += WG_THREADS) {
+                const unsigned int rowid = div24(g, gpr, r_gpr), xj0 = (g - rowid * gpr) * 8;
+                const unsigned int cin = div24(rowid, Hi, r_Hi), i = rowid - cin * Hi;
+                const unsigned int yi = i * A.kh + a;
+                if (yi >= (unsigned int)A.H) continue;
+                unsigned int j = div24(xj0, A.kw, r_kw), b = xj0 - j * A.kw;
+                const unsigned int n = min(8u, (unsigned int)A.W - xj0);
+                const TS* src = pt + cin * plane_c * plane + (long)i * A.Wo;
+                PatchRun<TS> run;
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    run.v[u] = ((unsigned int)u < n && i < (unsigned int)A.Ho && j < (unsigned int)A.Wo) ? src[b * plane_b * plane + j] : (TS)0;
+                    if (++b == (unsigned int)A.kw) { b = 0; ++j; }
+                }
+                store_run(x + ((long)cin * A.H + yi) * A.W + xj0, run, n);
             }
         }
     }
@@ -173,7 +203,7 @@ struct DilationPhaseArgs {
 
 // A workgroup takes one (component x image, block of CB channels, row phase a) at a time: the rows of the caller's
 // tensor that it touches are shared by all dw column phases, so each of their cache lines is fetched once, and the
-// phase images it touches are runs of CB * Hp * Wp consecutive elements.  Index arithmetic per element is 32-bit.
+// phase images it touches are runs of CB * Hp * Wp consecutive elements.  Index arithmetic per element is 32-bit, its divisions by fp32 reciprocal (an item has fewer than 2^24 elements).
 template <typename TS>
 __global__ void __launch_bounds__(WG_THREADS) dilation_phase_kernel(const DilationPhaseArgs A, int to_caller) {
     const int cblocks = A.C / A.CB;
@@ -191,10 +221,11 @@ __global__ void __launch_bounds__(WG_THREADS) dilation_phase_kernel(const Dilati
             const TS* x = static_cast<const TS*>(A.src) + caller0;
             TS* ph = static_cast<TS*>(A.dst) + phase0;
             const unsigned int per_b = (unsigned int)A.CB * plane, count = per_b * A.dw;
+            const float r_per_b = 1.0f / per_b, r_plane = 1.0f / plane, r_Wp = 1.0f / A.Wp;
             for (unsigned int e = threadIdx.x; e < count; e += WG_THREADS) {
-                const unsigned int b = e / per_b, in_b = e - b * per_b;          // in_b = (channel, i, j) of the phase image
-                const unsigned int cin = in_b / plane, ij = in_b - cin * plane;
-                const unsigned int i = ij / A.Wp, j = ij - i * A.Wp;
+                const unsigned int b = div24(e, per_b, r_per_b), in_b = e - b * per_b;  // in_b = (channel, i, j) of the phase image
+                const unsigned int cin = div24(in_b, plane, r_plane), ij = in_b - cin * plane;
+                const unsigned int i = div24(ij, A.Wp, r_Wp), j = ij - i * A.Wp;
                 const int yi = (int)i * A.dh + a - A.oh, xj = (int)j * A.dw + (int)b - A.ow;
                 ph[b * phase_b + in_b] =
                     (yi >= 0 && yi < A.H && xj >= 0 && xj < A.W) ? x[((long)cin * A.H + yi) * A.W + xj] : (TS)0;
@@ -202,13 +233,16 @@ __global__ void __launch_bounds__(WG_THREADS) dilation_phase_kernel(const Dilati
         } else {
             const TS* ph = static_cast<const TS*>(A.src) + phase0;
             TS* x = static_cast<TS*>(A.dst) + caller0;
+            // (one element per thread: the rows of atrous layers' images are short and odd -- 33, 65, 129 -- so runs of 8
+            // per thread, as in patch_depth_kernel, rarely store a vector and measured no faster)
             const unsigned int per_c = (unsigned int)A.Hp * A.W, count = per_c * A.CB;
+            const float r_per_c = 1.0f / per_c, r_W = 1.0f / A.W, r_dw = 1.0f / A.dw;
             for (unsigned int e = threadIdx.x; e < count; e += WG_THREADS) {
-                const unsigned int cin = e / per_c, ix = e - cin * per_c;
-                const unsigned int i = ix / A.W, xj = ix - i * A.W;
+                const unsigned int cin = div24(e, per_c, r_per_c), ix = e - cin * per_c;
+                const unsigned int i = div24(ix, A.W, r_W), xj = ix - i * A.W;
                 const int yi = (int)i * A.dh + a - A.oh;
                 if (yi < 0 || yi >= A.H) continue;
-                const unsigned int xo = xj + A.ow, j = xo / A.dw, b = xo - j * A.dw;
+                const unsigned int xo = xj + A.ow, j = div24(xo, A.dw, r_dw), b = xo - j * A.dw;
                 x[((long)cin * A.H + yi) * A.W + xj] = ph[b * phase_b + (long)cin * plane + i * A.Wp + j];
             }
         }

@@ -28,11 +28,16 @@ int launch_s2d_input(bool half_storage, const S2dArgs& a, hipStream_t st) {
     return 0;
 }
 
-int launch_patch_depth(bool half_storage, const PatchArgs& a, bool to_caller, hipStream_t st) {
-    const long planes = to_caller ? a.rows * a.C : a.rows * a.C * a.kh * a.kw;  // one workgroup each (the surplus in turns)
-    if (planes <= 0 || (long)a.H * a.W <= 0) return 0;
-    const bool per_position = !to_caller && (long)a.Ho * a.Wo < 512;  // (the kernel's rule)
-    const dim3 grid(per_position ? (unsigned int)blocks_for(planes * a.Ho * a.Wo) : (unsigned int)std::min<long>(planes, 1 << 18));
+int launch_patch_depth(bool half_storage, const PatchArgs& a0, bool to_caller, hipStream_t st) {
+    if (a0.rows <= 0 || a0.C <= 0 || (long)a0.H * a0.W <= 0) return 0;
+    PatchArgs a = a0;
+    // channels per item: a power of two that divides C, for items of a few thousand elements
+    const long per_channel = std::max((long)a.kw * a.Ho * a.Wo, (long)((a.H + a.kh - 1) / a.kh) * a.W);
+    a.CB = 1;
+    while (a.C % (a.CB * 2) == 0 && per_channel * a.CB * 2 <= 4096) a.CB *= 2;
+    if (per_channel * a.CB >= (1L << 24)) return -1;  // the kernel divides an item's element counts in fp32
+    const long items = a.rows * (a.C / a.CB) * a.kh;
+    const dim3 grid((unsigned int)std::min<long>(items, 1L << 20));
     if (half_storage) hipLaunchKernelGGL((patch_depth_kernel<_Float16>), grid, dim3(WG_THREADS), 0, st, a, (int)to_caller);
     else hipLaunchKernelGGL((patch_depth_kernel<float>), grid, dim3(WG_THREADS), 0, st, a, (int)to_caller);
     return 0;
@@ -53,8 +58,8 @@ int launch_dilation_phases(bool half_storage, const DilationPhaseArgs& a0, bool 
     const long per_channel = (long)a.Hp * a.Wp * a.dw;
     a.CB = 1;
     while (a.C % (a.CB * 2) == 0 && per_channel * a.CB * 2 <= 4096) a.CB *= 2;
-    // a workgroup's 32-bit element count: (Hp * max(Wp * dw, W)) * CB
-    if (per_channel * a.CB >= (1L << 31) || (long)a.Hp * a.W * a.CB >= (1L << 31)) return -1;
+    // a workgroup's element count, divided in fp32: (Hp * max(Wp * dw, W)) * CB
+    if (per_channel * a.CB >= (1L << 24) || (long)a.Hp * a.W * a.CB >= (1L << 24)) return -1;
     const long items = a.rows * (a.C / a.CB) * a.dh;
     const unsigned int blocks = (unsigned int)(items < (1L << 20) ? items : (1L << 20));
     if (half_storage)

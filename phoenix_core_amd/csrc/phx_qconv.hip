@@ -1628,6 +1628,8 @@ static bool patch_view(const Problem& p, int pass, PatchView& v) {
     else if (f.skw == p.ci * f.si && f.skh == (long)p.kw * p.ci * f.si) { v.tap_major = 1; si = f.si; }
     else return false;
     if ((long)p.ci * p.kh * p.kw > (1L << 20)) return false;
+    // the patch kernel's index arithmetic on one channel's image or patches is exact below that
+    if ((long)p.h * p.w >= (1L << 24) || (long)p.kw * p.ho * p.wo >= (1L << 24)) return false;
     Problem& q = v.q;
     q = p;
     q.nhwc = false;  // (the patch tensor is channels-first)
@@ -1676,8 +1678,8 @@ static bool dilation_view(const Problem& p, int pass, DilationView& v) {
     q.pb = v.Hop + (p.kh - 1) - v.Hp - q.pt; q.pr = v.Wop + (p.kw - 1) - v.Wp - q.pl;
     if (q.pb < 0 || q.pr < 0 || window_beyond_staging(q)) return false;
     if (out_size(q.h, q.kh, 1, 1, q.pt, q.pb) != q.ho || out_size(q.w, q.kw, 1, 1, q.pl, q.pr) != q.wo) return false;
-    // the phase kernels index one channel's phase images with 32 bits
-    if ((long)v.Hp * v.Wp * p.dw >= (1L << 31) || (long)v.Hop * v.Wop * p.dw >= (1L << 31)) return false;
+    // the phase kernels' index arithmetic on one channel's phase images is exact below that
+    if ((long)v.Hp * v.Wp * p.dw >= (1L << 24) || (long)v.Hop * v.Wop * p.dw >= (1L << 24)) return false;
     const size_t esize = p.dtype == PHX_F32 ? 4 : 2;
     v.x_bytes = align_up((size_t)4 * q.n * p.ci * v.Hp * v.Wp * esize, 256);
     v.y_bytes = align_up((size_t)4 * q.n * p.co * v.Hop * v.Wop * esize, 256);
