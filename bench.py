@@ -48,6 +48,7 @@ GROUPED = {
     "x_smallbatch_k3_f16_512_7": (1, 512, 512, 7, 7, 3, "SAME", "f16", 1, 1, 1),       # reduction slices
     "x_atrous_k3_d12_f16_512_64_33": (8, 512, 64, 33, 33, 3, "SAME", "f16", 1, 1, 12),  # dilation phases
     "x_stride3_k3_f16_128_28": (32, 128, 128, 28, 28, 3, "SAME", "f16", 1, 3, 1),       # filter gradient by tap classes
+    "x_patch_k16_s16_f16_16_192_224": (16, 16, 192, 224, 224, 16, "VALID", "f16", 1, 16, 1),  # patches as channels
 }
 DENSE = {"c1_dense_f32": (32, 128, 128, "f32")}  # name: (n, in, out, dtype)
 RESNET = "c5_qresnet50"  # quaternion ResNet-50 forward+backward, N=64, 224x224, fp16 full16 policy
